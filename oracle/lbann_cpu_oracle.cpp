@@ -1,0 +1,532 @@
+// CPU oracle: a restatement of LBANN's CPU (OpenMP) implementation of the
+// forward/backward compute of five layers.  TEST INFRASTRUCTURE ONLY: this file
+// is the checker that the HIP kernels are compared against and the timed CPU
+// baseline of the benchmark; nothing in the product path may call it.
+//
+// Every function keeps the reference's loop order, accumulation type and
+// operation order (sequential accumulation in the tensor data type, the same
+// clamps, reciprocal-vs-divide choices), so that its rounding pattern is the
+// reference's when built with -ffp-contract=off.  The `_f64` instantiations
+// are the same code with TensorDataType=double (a data type the reference can
+// also be built with) and serve as the "exact" answer where the fp32 reference
+// is itself noisy.
+//
+// Matrices are column-major, element (r,c) at buf[r + c*ld], one column per
+// sample, exactly like El::Matrix<T,CPU>.
+//
+// Pinning status (see tests/test_oracle_*.py): every function below is pinned
+// by float64 closed forms taken from the reference's own unit tests, by
+// invariants, by finite differences or by torch library routines; none is
+// "parity unpinned".
+//
+// Followed reference code (file:line in LBANN v0.105.0):
+//   layer norm      src/layers/regularizers/layer_norm.cpp:41-136 (fwd), :139-258 (bwd)
+//   batch norm      src/layers/regularizers/batch_normalization.cpp:37-175 (fwd), :178-329 (bwd)
+//   softmax         include/lbann/utils/dnn_lib/openmp/softmax.hpp:39-117 (fwd), :119-181 (bwd)
+//   log-softmax     src/layers/activations/log_softmax.cpp:35-93 (fwd), :95-136 (bwd)
+//   channelwise sm  src/layers/misc/channelwise_softmax.cpp:41-99 (fwd), :121-169 (bwd)
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <limits>
+#include <vector>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+namespace {
+
+using idx = std::int64_t;
+
+template <typename T>
+struct CMat {  // const column-major view
+  const T* p;
+  idx ld;
+  const T& operator()(idx r, idx c) const { return p[r + c * ld]; }
+};
+template <typename T>
+struct Mat {  // mutable column-major view
+  T* p;
+  idx ld;
+  T& operator()(idx r, idx c) const { return p[r + c * ld]; }
+};
+
+// ---------------------------------------------------------------- layer norm
+// layer_norm.cpp:41-136.  stats is (2G x w): rows [0,G) means, [G,2G) variances.
+template <typename T>
+void ln_fwd(idx G, idx n, idx stride, idx w, T eps, CMat<T> x, Mat<T> y,
+            Mat<T> stats, const T* gamma, const T* beta)
+{
+  // layer_norm.cpp:76  El::Zero(statistics)
+  for (idx i = 0; i < w; ++i)
+    for (idx j = 0; j < 2 * G; ++j) stats(j, i) = T(0);
+
+  // layer_norm.cpp:77-88  running sums, accumulated in place in the stats matrix
+#pragma omp parallel for collapse(2)
+  for (idx i = 0; i < w; ++i) {
+    for (idx j = 0; j < G; ++j) {
+      T& sum = stats(j, i);
+      T& sqsum = stats(G + j, i);
+      for (idx k = 0; k < n; ++k) {
+        const T v = x(k + j * stride, i);
+        sum += v;
+        sqsum += v * v;
+      }
+    }
+  }
+
+  // layer_norm.cpp:94-113
+  if (n <= 1) {
+    for (idx i = 0; i < w; ++i)
+      for (idx j = 0; j < G; ++j) stats(G + j, i) = T(1);
+  }
+  else {
+#pragma omp parallel for collapse(2)
+    for (idx i = 0; i < w; ++i) {
+      for (idx j = 0; j < G; ++j) {
+        const T sum = stats(j, i);
+        const T sqsum = stats(G + j, i);
+        const T nn = static_cast<T>(n);
+        const T mean = sum / nn;
+        const T sqmean = sqsum / nn;
+        const T var = sqmean - mean * mean;
+        stats(j, i) = mean;
+        stats(G + j, i) = std::max(var, T(0));
+      }
+    }
+  }
+
+  // layer_norm.cpp:117-135
+#pragma omp parallel for collapse(2)
+  for (idx i = 0; i < w; ++i) {
+    for (idx j = 0; j < G; ++j) {
+      const T mean = stats(j, i);
+      const T var = stats(G + j, i);
+      const T inv_stdev = T(1) / std::sqrt(var + eps);
+      for (idx k = 0; k < n; ++k) {
+        const T v = x(k + j * stride, i);
+        T r = (v - mean) * inv_stdev;
+        if (gamma) r *= gamma[k];
+        if (beta) r += beta[k];
+        y(k + j * stride, i) = r;
+      }
+    }
+  }
+}
+
+// layer_norm.cpp:139-258 plus the zeroing of the weight-gradient buffers done by
+// bp_compute (:300-309).  stats_grad is (2G x w): rows [0,G) dmean, [G,2G) dvar.
+template <typename T>
+void ln_bwd(idx G, idx n, idx stride, idx w, idx h, T eps, CMat<T> x, CMat<T> dy,
+            Mat<T> dx, CMat<T> stats, Mat<T> sgrad, const T* gamma, T* dgamma,
+            T* dbeta)
+{
+  if (dgamma) std::fill(dgamma, dgamma + n, T(0));
+  if (dbeta) std::fill(dbeta, dbeta + n, T(0));
+
+  // layer_norm.cpp:189-192
+  if (n <= 1) {
+    for (idx i = 0; i < w; ++i)
+      for (idx r = 0; r < h; ++r) dx(r, i) = T(0);
+    return;
+  }
+
+  for (idx i = 0; i < w; ++i)
+    for (idx j = 0; j < 2 * G; ++j) sgrad(j, i) = T(0);
+
+  // layer_norm.cpp:198-227
+#pragma omp parallel for collapse(2)
+  for (idx i = 0; i < w; ++i) {
+    for (idx j = 0; j < G; ++j) {
+      const T mean = stats(j, i);
+      const T var = stats(G + j, i);
+      const T inv_stdev = T(1) / std::sqrt(var + eps);
+      T& dmean = sgrad(j, i);
+      T& dvar = sgrad(G + j, i);
+      for (idx k = 0; k < n; ++k) {
+        const T v = x(k + j * stride, i);
+        T g = dy(k + j * stride, i);
+        if (dbeta) {
+#pragma omp atomic
+          dbeta[k] += g;
+        }
+        if (dgamma) {
+          const T contrib = g * (v - mean) * inv_stdev;
+#pragma omp atomic
+          dgamma[k] += contrib;
+          g *= gamma[k];
+        }
+        dmean += g;
+        dvar += g * (v - mean);
+      }
+      dmean *= -inv_stdev;
+      dvar *= -inv_stdev * inv_stdev * inv_stdev / 2;
+    }
+  }
+
+  // layer_norm.cpp:236-257  (the code divides by n, not n-1)
+#pragma omp parallel for collapse(2)
+  for (idx i = 0; i < w; ++i) {
+    for (idx j = 0; j < G; ++j) {
+      const T mean = stats(j, i);
+      const T var = stats(G + j, i);
+      const T inv_stdev = T(1) / std::sqrt(var + eps);
+      const T dmean = sgrad(j, i);
+      const T dvar = sgrad(G + j, i);
+      for (idx k = 0; k < n; ++k) {
+        const T v = x(k + j * stride, i);
+        T g = dy(k + j * stride, i);
+        if (gamma) g *= gamma[k];
+        dx(k + j * stride, i) =
+          g * inv_stdev + dmean / n + dvar * (v - mean) * 2 / n;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- batch norm
+// batch_normalization.cpp:37-175, local statistics (statistics_group_size==1), so
+// num_per_sum = channel_size * local_width (:94-97).
+template <typename T>
+void bn_fwd(idx C, idx cs, idx w, int bessel, T eps, T decay, int training,
+            CMat<T> x, Mat<T> y, T* mean_out, T* var_out, const T* gamma,
+            const T* beta, T* running_mean, T* running_var)
+{
+  const int correction = bessel ? 1 : 0;
+  if (training) {
+    // :70-85
+#pragma omp parallel for
+    for (idx c = 0; c < C; ++c) {
+      T sum = T(0), sqsum = T(0);
+      const idx r0 = c * cs, r1 = (c + 1) * cs;
+      for (idx col = 0; col < w; ++col) {
+        for (idx r = r0; r < r1; ++r) {
+          const T v = x(r, col);
+          sum += v;
+          sqsum += v * v;
+        }
+      }
+      mean_out[c] = sum;
+      var_out[c] = sqsum;
+    }
+    const idx num_per_sum = cs * w;
+    // :118-138
+    if (num_per_sum <= 1) {
+      for (idx c = 0; c < C; ++c) var_out[c] = T(1);
+    }
+    else {
+#pragma omp parallel for
+      for (idx c = 0; c < C; ++c) {
+        const T nn = static_cast<T>(num_per_sum);
+        const T mean = mean_out[c] / nn;
+        const T sqmean = var_out[c] / nn;
+        T var = nn * (sqmean - mean * mean) / (nn - correction);
+        var = std::max(var, eps);
+        mean_out[c] = mean;
+        var_out[c] = var;
+        running_mean[c] = decay * running_mean[c] + (T(1) - decay) * mean;
+        running_var[c] = decay * running_var[c] + (T(1) - decay) * var;
+      }
+    }
+  }
+  // :141-174  training uses the batch statistics, otherwise the running ones
+  const T* use_mean = training ? mean_out : running_mean;
+  const T* use_var = training ? var_out : running_var;
+#pragma omp parallel for
+  for (idx c = 0; c < C; ++c) {
+    const T mean = use_mean[c];
+    const T var = use_var[c];
+    const T inv_stdev = static_cast<T>(1 / std::sqrt(var + eps));
+    const T scale = gamma[c];
+    const T bias = beta[c];
+    const idx r0 = c * cs, r1 = (c + 1) * cs;
+    for (idx col = 0; col < w; ++col) {
+      for (idx r = r0; r < r1; ++r) {
+        const T xhat = (x(r, col) - mean) * inv_stdev;
+        y(r, col) = scale * xhat + bias;
+      }
+    }
+  }
+}
+
+// batch_normalization.cpp:178-329.
+template <typename T>
+void bn_bwd(idx C, idx cs, idx w, int bessel, T eps, int training, CMat<T> x,
+            CMat<T> dy, Mat<T> dx, const T* mean_in, const T* var_in,
+            const T* running_mean, const T* running_var, const T* gamma,
+            T* dgamma, T* dbeta, T* dmean_out, T* dvar_out)
+{
+  const int correction = bessel ? 1 : 0;
+  const T* use_mean = training ? mean_in : running_mean;
+  const T* use_var = training ? var_in : running_var;
+  // :211-245
+#pragma omp parallel for
+  for (idx c = 0; c < C; ++c) {
+    const T mean = use_mean[c];
+    const T var = use_var[c];
+    const T scale = gamma[c];
+    const T inv_stdev = static_cast<T>(1 / std::sqrt(var + eps));
+    const T dvar_factor = inv_stdev * inv_stdev * inv_stdev / 2;
+    T dmean = T(0), dvar = T(0), dscale = T(0), dbias = T(0);
+    const idx r0 = c * cs, r1 = (c + 1) * cs;
+    for (idx col = 0; col < w; ++col) {
+      for (idx r = r0; r < r1; ++r) {
+        const T v = x(r, col);
+        const T xhat = (v - mean) * inv_stdev;
+        const T g = dy(r, col);
+        dscale += g * xhat;
+        dbias += g;
+        const T dxhat = g * scale;
+        dmean += -dxhat * inv_stdev;
+        dvar += -dxhat * (v - mean) * dvar_factor;
+      }
+    }
+    dmean_out[c] = dmean;
+    dvar_out[c] = dvar;
+    dgamma[c] = dscale;
+    dbeta[c] = dbias;
+  }
+  // :248-267  outside training the statistics gradients are dropped
+  if (!training) {
+    for (idx c = 0; c < C; ++c) {
+      dmean_out[c] = T(0);
+      dvar_out[c] = T(0);
+    }
+  }
+  // :282-328
+  const idx num_per_sum = cs * w;
+  if (num_per_sum <= 1) {
+    for (idx col = 0; col < w; ++col)
+      for (idx r = 0; r < C * cs; ++r) dx(r, col) = T(0);
+    return;
+  }
+#pragma omp parallel for
+  for (idx c = 0; c < C; ++c) {
+    const T mean = use_mean[c];
+    const T var = use_var[c];
+    const T scale = gamma[c];
+    const T dmean = dmean_out[c];
+    const T dvar = dvar_out[c];
+    const T inv_stdev = static_cast<T>(1 / std::sqrt(var + eps));
+    const T dmean_term = dmean / num_per_sum;
+    const T dvar_term = dvar * 2 / (num_per_sum - correction);
+    const idx r0 = c * cs, r1 = (c + 1) * cs;
+    for (idx col = 0; col < w; ++col) {
+      for (idx r = r0; r < r1; ++r) {
+        const T dxhat = dy(r, col) * scale;
+        dx(r, col) = dxhat * inv_stdev + dmean_term + dvar_term * (x(r, col) - mean);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------- softmax
+// openmp/softmax.hpp:39-117
+template <typename T>
+void sm_fwd(idx h, idx w, CMat<T> x, Mat<T> y)
+{
+  std::vector<T> work(static_cast<size_t>(w), std::numeric_limits<T>::lowest());
+  T* ws = work.data();
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    T& m = ws[c];
+    for (idx r = 0; r < h; ++r) m = std::max(m, x(r, c));
+  }
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    const T shift = ws[c];
+    T sum = T(0);
+    for (idx r = 0; r < h; ++r) {
+      const T e = std::exp(x(r, c) - shift);
+      y(r, c) = e;
+      sum += e;
+    }
+    ws[c] = sum;
+  }
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    const T scale = 1 / ws[c];
+    for (idx r = 0; r < h; ++r) {
+      const T t = scale * y(r, c);
+      y(r, c) = std::isnormal(t) ? t : T(0);
+    }
+  }
+}
+
+// openmp/softmax.hpp:119-181
+template <typename T>
+void sm_bwd(idx h, idx w, CMat<T> y, CMat<T> dy, Mat<T> dx)
+{
+  std::vector<T> work(static_cast<size_t>(w), T(0));
+  T* ws = work.data();
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    T& d = ws[c];
+    for (idx r = 0; r < h; ++r) d += y(r, c) * dy(r, c);
+  }
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    const T d = ws[c];
+    for (idx r = 0; r < h; ++r) dx(r, c) = y(r, c) * (dy(r, c) - d);
+  }
+}
+
+// --------------------------------------------------------------- log-softmax
+// log_softmax.cpp:35-93
+template <typename T>
+void lsm_fwd(idx h, idx w, CMat<T> x, Mat<T> y)
+{
+  std::vector<T> work(static_cast<size_t>(w), std::numeric_limits<T>::lowest());
+  T* ws = work.data();
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    T& m = ws[c];
+    for (idx r = 0; r < h; ++r) m = std::max(m, x(r, c));
+  }
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    const T shift = ws[c];
+    T sum{0};
+    for (idx r = 0; r < h; ++r) {
+      const T v = x(r, c) - shift;
+      y(r, c) = v;
+      sum += std::exp(v);
+    }
+    ws[c] = sum;
+  }
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    const T lse = static_cast<T>(std::log(ws[c]));
+    for (idx r = 0; r < h; ++r) y(r, c) -= lse;
+  }
+}
+
+// log_softmax.cpp:95-136
+template <typename T>
+void lsm_bwd(idx h, idx w, CMat<T> y, CMat<T> dy, Mat<T> dx)
+{
+  std::vector<T> work(static_cast<size_t>(w), T(0));
+  T* ws = work.data();
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    T& s = ws[c];
+    for (idx r = 0; r < h; ++r) s += dy(r, c);
+  }
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    const T s = ws[c];
+    for (idx r = 0; r < h; ++r) dx(r, c) = dy(r, c) - std::exp(y(r, c)) * s;
+  }
+}
+
+// -------------------------------------------------------- channelwise softmax
+// channelwise_softmax.cpp:41-99.  Only the max loop is parallel in the
+// reference; the denominator and output loops (:75, :88) carry no pragma.
+template <typename T>
+void cws_fwd(idx C, idx cs, idx stride, idx w, CMat<T> x, Mat<T> y)
+{
+  std::vector<T> shifts(static_cast<size_t>(C * w), std::numeric_limits<T>::lowest());
+  std::vector<T> denoms(static_cast<size_t>(C * w), T(0));
+  T* sh = shifts.data();
+  T* dn = denoms.data();
+#pragma omp parallel for collapse(2)
+  for (idx k = 0; k < w; ++k) {
+    for (idx j = 0; j < C; ++j) {
+      T& m = sh[j + k * C];
+      for (idx i = 0; i < cs; ++i) m = std::max(m, x(i + j * stride, k));
+    }
+  }
+  for (idx k = 0; k < w; ++k) {
+    for (idx j = 0; j < C; ++j) {
+      const T shift = sh[j + k * C];
+      T& d = dn[j + k * C];
+      for (idx i = 0; i < cs; ++i) d += std::exp(x(i + j * stride, k) - shift);
+    }
+  }
+  for (idx k = 0; k < w; ++k) {
+    for (idx j = 0; j < C; ++j) {
+      const T shift = sh[j + k * C];
+      const T d = dn[j + k * C];
+      for (idx i = 0; i < cs; ++i)
+        y(i + j * stride, k) = std::exp(x(i + j * stride, k) - shift) / d;
+    }
+  }
+}
+
+// channelwise_softmax.cpp:121-169
+template <typename T>
+void cws_bwd(idx C, idx cs, idx stride, idx w, CMat<T> y, CMat<T> dy, Mat<T> dx)
+{
+  std::vector<T> dots(static_cast<size_t>(C * w), T(0));
+  T* dt = dots.data();
+#pragma omp parallel for collapse(2)
+  for (idx k = 0; k < w; ++k) {
+    for (idx j = 0; j < C; ++j) {
+      T& d = dt[j + k * C];
+      for (idx i = 0; i < cs; ++i) d += y(i + j * stride, k) * dy(i + j * stride, k);
+    }
+  }
+#pragma omp parallel for collapse(2)
+  for (idx k = 0; k < w; ++k) {
+    for (idx j = 0; j < C; ++j) {
+      const T d = dt[j + k * C];
+      for (idx i = 0; i < cs; ++i)
+        dx(i + j * stride, k) = y(i + j * stride, k) * (dy(i + j * stride, k) - d);
+    }
+  }
+}
+
+}  // namespace
+
+// C interface (one _f32 and one _f64 entry per function), bound by oracle/cpu_oracle.py.
+#define ORC_INSTANTIATE(SUF, T)                                                          \
+  extern "C" void orc_layer_norm_fwd_##SUF(idx G, idx n, idx stride, idx w, T eps,       \
+      const T* x, idx ldx, T* y, idx ldy, T* stats, idx lds, const T* gamma,             \
+      const T* beta)                                                                     \
+  { ln_fwd<T>(G, n, stride, w, eps, {x, ldx}, {y, ldy}, {stats, lds}, gamma, beta); }    \
+  extern "C" void orc_layer_norm_bwd_##SUF(idx G, idx n, idx stride, idx w, idx h,       \
+      T eps, const T* x, idx ldx, const T* dy, idx lddy, T* dx, idx lddx,                \
+      const T* stats, idx lds, T* sgrad, idx ldsg, const T* gamma, T* dgamma, T* dbeta)  \
+  { ln_bwd<T>(G, n, stride, w, h, eps, {x, ldx}, {dy, lddy}, {dx, lddx}, {stats, lds},   \
+              {sgrad, ldsg}, gamma, dgamma, dbeta); }                                    \
+  extern "C" void orc_batch_norm_fwd_##SUF(idx C, idx cs, idx w, int bessel, T eps,      \
+      T decay, int training, const T* x, idx ldx, T* y, idx ldy, T* mean, T* var,        \
+      const T* gamma, const T* beta, T* rmean, T* rvar)                                  \
+  { bn_fwd<T>(C, cs, w, bessel, eps, decay, training, {x, ldx}, {y, ldy}, mean, var,     \
+              gamma, beta, rmean, rvar); }                                               \
+  extern "C" void orc_batch_norm_bwd_##SUF(idx C, idx cs, idx w, int bessel, T eps,      \
+      int training, const T* x, idx ldx, const T* dy, idx lddy, T* dx, idx lddx,         \
+      const T* mean, const T* var, const T* rmean, const T* rvar, const T* gamma,        \
+      T* dgamma, T* dbeta, T* dmean, T* dvar)                                            \
+  { bn_bwd<T>(C, cs, w, bessel, eps, training, {x, ldx}, {dy, lddy}, {dx, lddx}, mean,   \
+              var, rmean, rvar, gamma, dgamma, dbeta, dmean, dvar); }                    \
+  extern "C" void orc_softmax_fwd_##SUF(idx h, idx w, const T* x, idx ldx, T* y, idx ldy)\
+  { sm_fwd<T>(h, w, {x, ldx}, {y, ldy}); }                                               \
+  extern "C" void orc_softmax_bwd_##SUF(idx h, idx w, const T* y, idx ldy, const T* dy,  \
+      idx lddy, T* dx, idx lddx)                                                         \
+  { sm_bwd<T>(h, w, {y, ldy}, {dy, lddy}, {dx, lddx}); }                                 \
+  extern "C" void orc_log_softmax_fwd_##SUF(idx h, idx w, const T* x, idx ldx, T* y,     \
+      idx ldy)                                                                           \
+  { lsm_fwd<T>(h, w, {x, ldx}, {y, ldy}); }                                              \
+  extern "C" void orc_log_softmax_bwd_##SUF(idx h, idx w, const T* y, idx ldy,           \
+      const T* dy, idx lddy, T* dx, idx lddx)                                            \
+  { lsm_bwd<T>(h, w, {y, ldy}, {dy, lddy}, {dx, lddx}); }                                \
+  extern "C" void orc_channelwise_softmax_fwd_##SUF(idx C, idx cs, idx stride, idx w,    \
+      const T* x, idx ldx, T* y, idx ldy)                                                \
+  { cws_fwd<T>(C, cs, stride, w, {x, ldx}, {y, ldy}); }                                  \
+  extern "C" void orc_channelwise_softmax_bwd_##SUF(idx C, idx cs, idx stride, idx w,    \
+      const T* y, idx ldy, const T* dy, idx lddy, T* dx, idx lddx)                       \
+  { cws_bwd<T>(C, cs, stride, w, {y, ldy}, {dy, lddy}, {dx, lddx}); }
+
+ORC_INSTANTIATE(f32, float)
+ORC_INSTANTIATE(f64, double)
+
+extern "C" int orc_max_threads()
+{
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}

@@ -1,0 +1,139 @@
+"""Regenerates tests/golden/reference_unit_tests.npz.
+
+The reference holds no golden files for the normalization / softmax layers: each of
+its layer tests draws a seeded NumPy dataset inside the test file, evaluates a
+float64 NumPy closed form, and lets the framework's forward result deviate from
+it by a stated tolerance.  This script re-creates those datasets (same legacy
+`np.random.seed` stream, same draw order, same shapes) and stores, for each,
+the inputs and the float64 closed-form expectation together with the tolerance
+the reference test states.  Nothing from the reference is imported or run;
+the formulas below are the textbook definitions the reference tests also use.
+
+Datasets and tolerances (reference file:line):
+  layer_norm            ci_test/unit_tests/test_unit_layer_layer_norm.py:21-24, :38-43, :107-113
+  layer_norm (affine)   ci_test/unit_tests/test_unit_layer_layernorm_affine.py:7-15, :67-104
+  layer_norm (multidim) ci_test/unit_tests/test_unit_layer_layernorm_affine.py:40-61
+  batch_normalization   ci_test/unit_tests/test_unit_layer_batch_normalization.py:21-25 (no forward pin there)
+  softmax               ci_test/unit_tests/test_unit_layer_softmax.py:21-24, :38-48
+  log_softmax           ci_test/unit_tests/test_unit_layer_log_softmax.py:21-24, :38-48
+  channelwise_softmax   ci_test/unit_tests/test_unit_layer_channelwise_softmax.py:21-26, :47-54, :109-137
+
+Run:  python tests/golden/make_reference_fixtures.py
+"""
+import os
+
+import numpy as np
+
+OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_unit_tests.npz")
+
+
+def l2norm2_metric(y):
+    """Mean over samples (axis 0) of the squared L2 norm, float64."""
+    y = np.asarray(y, dtype=np.float64).reshape(y.shape[0], -1)
+    return float(np.mean(np.sum(y * y, axis=1)))
+
+
+def main():
+    fx = {}
+
+    # ---- layer norm, whole sample, no affine, eps 1e-5
+    np.random.seed(20191114)
+    x = np.random.normal(size=(31, 31)).astype(np.float32)
+    xd = x.astype(np.float64)
+    mu = xd.mean(axis=1, keepdims=True)
+    var = xd.var(axis=1, ddof=0, keepdims=True)
+    y = (xd - mu) / np.sqrt(var + 1e-5)
+    fx["ln_x"] = x
+    fx["ln_y"] = y
+    fx["ln_metric"] = np.float64(l2norm2_metric(y))
+
+    # ---- layer norm with scale / bias.  The reference's NumPy expectation divides by
+    # (std + eps) instead of sqrt(var + eps); its test accepts a mean squared error of
+    # 1e-8, so both expectations are stored: the exact one and the one the test holds.
+    np.random.seed(20230814)
+    x = np.random.normal(size=(31, 31)).astype(np.float32)
+    scale = np.random.rand(31).astype(np.float32)
+    bias = np.random.rand(31).astype(np.float32)
+    xd = x.astype(np.float64)
+    mu = xd.mean(axis=1, keepdims=True)
+    var = xd.var(axis=1, ddof=0, keepdims=True)
+    fx["lna_x"] = x
+    fx["lna_scale"] = scale
+    fx["lna_bias"] = bias
+    fx["lna_y_exact"] = (xd - mu) / np.sqrt(var + 1e-5) * scale.astype(np.float64) + bias.astype(np.float64)
+    x32mu = x.mean(axis=-1, keepdims=True)
+    x32sd = x.std(axis=-1, ddof=0, keepdims=True)
+    fx["lna_y_test_scaled_bias"] = (x - x32mu) / (x32sd + 1e-5) * scale + bias
+    fx["lna_y_test_scaled"] = (x - x32mu) / (x32sd + 1e-5) * scale
+    fx["lna_y_test_plain"] = (x - x32mu) / (x32sd + 1e-5)
+
+    # ---- layer norm over trailing dims of a (31,2,5) sample, start_dim in {-1, 1, 0}
+    np.random.seed(20230814)
+    x = np.random.rand(31, 31, 2, 5).astype(np.float32)
+    fx["lnm_x"] = x
+    for start_dim, axes in ((-1, (3,)), (1, (2, 3)), (0, (1, 2, 3))):
+        m = x.mean(axis=axes, keepdims=True)
+        s = x.std(axis=axes, ddof=0, keepdims=True)
+        fx[f"lnm_y_test_sd{start_dim}"] = (x - m) / (s + 1e-5)
+        xd = x.astype(np.float64)
+        md = xd.mean(axis=axes, keepdims=True)
+        vd = xd.var(axis=axes, ddof=0, keepdims=True)
+        fx[f"lnm_y_exact_sd{start_dim}"] = (xd - md) / np.sqrt(vd + 1e-5)
+
+    # ---- batch norm dataset (the reference pins only gradients on it); the stored
+    # expectation is the training-mode definition in float64: per-channel statistics
+    # over batch and spatial positions, variance scaled by n/(n-1), clamped below at
+    # eps and then eps added again under the square root, gamma=1, beta=0.
+    np.random.seed(20200827)
+    x = np.random.normal(size=(29, 7 * 5 * 3)).astype(np.float32)
+    fx["bn_x"] = x
+    for tag, batch in (("mb14", x[:14]), ("all29", x)):
+        xd = batch.astype(np.float64).reshape(batch.shape[0], 7, 15)
+        n = xd.shape[0] * 15
+        mean = xd.mean(axis=(0, 2))
+        var_b = xd.var(axis=(0, 2), ddof=0)
+        for bessel in (0, 1):
+            var = np.maximum(var_b * n / (n - bessel), 1e-5)
+            yb = (xd - mean[None, :, None]) / np.sqrt(var[None, :, None] + 1e-5)
+            fx[f"bn_{tag}_b{bessel}_mean"] = mean
+            fx[f"bn_{tag}_b{bessel}_var"] = var
+            fx[f"bn_{tag}_b{bessel}_y"] = yb.reshape(batch.shape[0], -1)
+
+    # ---- softmax
+    np.random.seed(201910142)
+    x = np.random.normal(size=(19, 7)).astype(np.float32)
+    xd = x.astype(np.float64)
+    e = np.exp(xd - xd.max(axis=1, keepdims=True))
+    y = e / e.sum(axis=1, keepdims=True)
+    fx["sm_x"] = x
+    fx["sm_y"] = y
+    fx["sm_metric"] = np.float64(l2norm2_metric(y))
+
+    # ---- log-softmax
+    np.random.seed(201910213)
+    x = np.random.normal(size=(15, 11)).astype(np.float32)
+    xd = x.astype(np.float64)
+    sh = xd - xd.max(axis=1, keepdims=True)
+    y = sh - np.log(np.exp(sh).sum(axis=1, keepdims=True))
+    fx["lsm_x"] = x
+    fx["lsm_y"] = y
+    fx["lsm_metric"] = np.float64(l2norm2_metric(y))
+
+    # ---- channelwise softmax on (5,2,7) samples: default mode (softmax over the
+    # trailing (2,7) slab of each of 5 channels) and single-dim mode on the last axis.
+    np.random.seed(20200115)
+    x = np.random.normal(loc=0.5, size=(15, 5 * 2 * 7)).astype(np.float32)
+    fx["cws_x"] = x
+    xd = x.astype(np.float64).reshape(15, 5, 2, 7)
+    for tag, axes in (("default", (2, 3)), ("lastdim", (3,))):
+        e = np.exp(xd - xd.max(axis=axes, keepdims=True))
+        y = e / e.sum(axis=axes, keepdims=True)
+        fx[f"cws_y_{tag}"] = y.reshape(15, -1)
+        fx[f"cws_metric_{tag}"] = np.float64(l2norm2_metric(y))
+
+    np.savez_compressed(OUT, **fx)
+    print(OUT, os.path.getsize(OUT), "bytes,", len(fx), "arrays")
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,53 @@
+"""Error metric and pass/fail gates shared by the parity tests.
+
+`rel_err(a, b)` is the largest element-wise error of `a` against `b`, each
+element's error divided by max(|b_i|, rms(b)): a plain element-wise relative
+error is meaningless where the expected value crosses zero, a plain absolute
+one hides errors in small tensors.
+
+`check(...)` applies the gate used everywhere: the candidate must agree with the
+fp32 reference restatement within `tol`; where the fp32 reference is itself
+further than `tol` from the float64 evaluation of the same algorithm (long
+sequential fp32 sums, E[x^2]-mean^2 cancellation), a candidate is also accepted
+when it is at least as close to the float64 answer as the reference is.
+"""
+import numpy as np
+
+TOL_F32 = 1e-5   # fp32 storage and arithmetic
+TOL_F16 = 2e-3   # fp16 storage, fp32 accumulation
+
+
+def rel_err(a, b):
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    assert a.shape == b.shape, (a.shape, b.shape)
+    if a.size == 0:
+        return 0.0
+    bad = ~np.isfinite(a) | ~np.isfinite(b)
+    if bad.any():
+        # non-finite entries must match exactly (same NaN positions, same infinities)
+        same = (np.isnan(a) & np.isnan(b)) | (a == b)
+        if not same[bad].all():
+            return float("inf")
+        a = np.where(bad, 0.0, a)
+        b = np.where(bad, 0.0, b)
+    rms = float(np.sqrt(np.mean(b * b)))
+    denom = np.maximum(np.abs(b), rms)
+    denom = np.where(denom == 0.0, 1.0, denom)
+    return float(np.max(np.abs(a - b) / denom))
+
+
+def check(name, got, ref32, exact64=None, tol=TOL_F32, slack=1.0):
+    """Returns the dict of measured errors; raises AssertionError when the gate fails."""
+    e_ref = rel_err(got, ref32)
+    out = {"name": name, "vs_ref": e_ref}
+    if e_ref <= tol:
+        return out
+    assert exact64 is not None, f"{name}: err vs fp32 reference {e_ref:.3e} > {tol:.1e}"
+    e_exact = rel_err(got, exact64)
+    e_ref_exact = rel_err(ref32, exact64)
+    out.update(vs_exact=e_exact, ref_vs_exact=e_ref_exact)
+    assert e_exact <= max(tol, slack * e_ref_exact), (
+        f"{name}: err vs fp32 reference {e_ref:.3e} > {tol:.1e} and err vs float64 "
+        f"{e_exact:.3e} > reference's own {e_ref_exact:.3e}")
+    return out

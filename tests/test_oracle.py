@@ -1,0 +1,387 @@
+"""Pins the CPU oracle (oracle/lbann_cpu_oracle.cpp) before anything is compared with it.
+
+Each oracle function is checked against something that does not share its code:
+the float64 closed forms and tolerances of the reference's own layer tests
+(tests/golden), torch's library routines and autograd in float64, central finite
+differences, and invariants.  The checks are chosen so that a dropped term, a
+wrong sign, a wrong divisor (n vs n-1), a transposed operand or a misplaced
+epsilon fails at least one of them.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu_oracle as orc
+from tests.parity import rel_err
+
+F32_EPS = np.finfo(np.float32).eps
+
+
+def F(a, dtype=None):
+    """Column-major copy (samples become columns): input is (samples, features)."""
+    a = np.asarray(a)
+    return np.asfortranarray(a.T.astype(dtype or a.dtype))
+
+
+def metric(y_cols):
+    y = np.asarray(y_cols, dtype=np.float64)
+    return float(np.mean(np.sum(y * y, axis=0)))
+
+
+# =============================================================== golden: forward
+@pytest.mark.parametrize("dt,tol", [(np.float32, 2e-6), (np.float64, 1e-12)])
+def test_layer_norm_golden(golden, dt, tol):
+    x = F(golden["ln_x"], dt)
+    y, stats = orc.layer_norm_fwd(x, 1, 31, 31, 1e-5)
+    assert rel_err(y.T, golden["ln_y"]) < tol
+    # the reference's own acceptance band on the L2Norm2 metric
+    val = float(golden["ln_metric"])
+    assert abs(metric(y) - val) <= 8 * val * F32_EPS
+    xd = golden["ln_x"].astype(np.float64)
+    assert rel_err(stats[0], xd.mean(axis=1)) < 10 * tol
+    assert rel_err(stats[1], xd.var(axis=1)) < 10 * tol
+
+
+def test_layer_norm_affine_golden(golden):
+    x = F(golden["lna_x"])
+    g, b = golden["lna_scale"], golden["lna_bias"]
+    y, _ = orc.layer_norm_fwd(x, 1, 31, 31, 1e-5, g, b)
+    assert rel_err(y.T, golden["lna_y_exact"]) < 3e-6
+    # the tolerance the reference test states: mean squared error <= 1e-8
+    assert np.mean((y.T - golden["lna_y_test_scaled_bias"]) ** 2) <= 1e-8
+    y, _ = orc.layer_norm_fwd(x, 1, 31, 31, 1e-5, g, None)
+    assert np.mean((y.T - golden["lna_y_test_scaled"]) ** 2) <= 1e-8
+    y, _ = orc.layer_norm_fwd(x, 1, 31, 31, 1e-5, None, None)
+    assert np.mean((y.T - golden["lna_y_test_plain"]) ** 2) <= 1e-8
+    # default weights (scale 1, bias 0) equal the plain layer
+    y1, _ = orc.layer_norm_fwd(x, 1, 31, 31, 1e-5, np.ones(31, np.float32), np.zeros(31, np.float32))
+    assert np.array_equal(y, y1)
+
+
+@pytest.mark.parametrize("start_dim,G,n", [(-1, 62, 5), (1, 31, 10), (0, 1, 310)])
+def test_layer_norm_multidim_golden(golden, start_dim, G, n):
+    xs = golden["lnm_x"]
+    x = F(xs.reshape(31, -1))
+    y, _ = orc.layer_norm_fwd(x, G, n, n, 1e-5)
+    assert np.mean((y.T - golden[f"lnm_y_test_sd{start_dim}"].reshape(31, -1)) ** 2) <= 1e-7
+    # fp32 E[x^2]-mean^2 on 5 uniform draws cancels a few digits: the reference's own noise
+    assert rel_err(y.T, golden[f"lnm_y_exact_sd{start_dim}"].reshape(31, -1)) < 1e-4
+    yd, _ = orc.layer_norm_fwd(F(xs.reshape(31, -1), np.float64), G, n, n, 1e-5)
+    assert rel_err(yd.T, golden[f"lnm_y_exact_sd{start_dim}"].reshape(31, -1)) < 1e-11
+
+
+@pytest.mark.parametrize("tag,rows", [("mb14", 14), ("all29", 29)])
+@pytest.mark.parametrize("bessel", [0, 1])
+def test_batch_norm_golden(golden, tag, rows, bessel):
+    xs = golden["bn_x"][:rows]
+    for dt, tol in ((np.float32, 3e-6), (np.float64, 1e-12)):
+        x = F(xs, dt)
+        C, cs = 7, 15
+        gamma, beta = np.ones(C, dt), np.zeros(C, dt)
+        rm, rv = np.zeros(C, dt), np.ones(C, dt)
+        y, mean, var = orc.batch_norm_fwd(x, C, cs, 1e-5, 0.9, gamma, beta, rm, rv, bessel=bool(bessel))
+        assert rel_err(y.T, golden[f"bn_{tag}_b{bessel}_y"]) < tol
+        assert rel_err(mean, golden[f"bn_{tag}_b{bessel}_mean"]) < tol
+        assert rel_err(var, golden[f"bn_{tag}_b{bessel}_var"]) < tol
+        # running statistics: one exponential-moving-average step from (0, 1)
+        assert rel_err(rm, 0.1 * golden[f"bn_{tag}_b{bessel}_mean"]) < 10 * tol
+        assert rel_err(rv, 0.9 + 0.1 * golden[f"bn_{tag}_b{bessel}_var"]) < tol
+
+
+@pytest.mark.parametrize("dt,tol", [(np.float32, 1e-6), (np.float64, 1e-13)])
+def test_softmax_golden(golden, dt, tol):
+    y = orc.softmax_fwd(F(golden["sm_x"], dt))
+    assert rel_err(y.T, golden["sm_y"]) < tol
+    val = float(golden["sm_metric"])
+    assert abs(metric(y) - val) <= 8 * val * F32_EPS
+    assert np.allclose(y.sum(axis=0), 1.0, atol=10 * tol)
+
+
+@pytest.mark.parametrize("dt,tol", [(np.float32, 1e-6), (np.float64, 1e-13)])
+def test_log_softmax_golden(golden, dt, tol):
+    y = orc.log_softmax_fwd(F(golden["lsm_x"], dt))
+    assert rel_err(y.T, golden["lsm_y"]) < tol
+    val = float(golden["lsm_metric"])
+    assert abs(metric(y) - val) <= 8 * val * F32_EPS
+    assert np.allclose(np.exp(y.astype(np.float64)).sum(axis=0), 1.0, atol=20 * tol)
+
+
+@pytest.mark.parametrize("tag,C,cs", [("default", 5, 14), ("lastdim", 10, 7)])
+def test_channelwise_softmax_golden(golden, tag, C, cs):
+    for dt, tol in ((np.float32, 1e-6), (np.float64, 1e-13)):
+        x = F(golden["cws_x"], dt)
+        y = orc.channelwise_softmax_fwd(x, C, cs, cs)
+        assert rel_err(y.T, golden[f"cws_y_{tag}"]) < tol
+        val = float(golden[f"cws_metric_{tag}"])
+        assert abs(metric(y) - val) <= 8 * val * F32_EPS
+        # same numbers as a plain softmax over the (cs, C*w) reshaping
+        plain = orc.softmax_fwd(np.asfortranarray(x.reshape(cs, -1, order="F")))
+        assert rel_err(y.reshape(cs, -1, order="F"), plain) < 4 * tol
+
+
+# ============================================================ library routines
+def test_layer_norm_matches_torch():
+    rng = np.random.default_rng(1)
+    xs = rng.normal(1.5, 2.0, size=(6, 4, 10))
+    g, b = rng.normal(1, 0.3, size=10), rng.normal(0, 0.3, size=10)
+    # start_dim=-1: normalise the trailing 10 entries, 4 groups per sample
+    y, stats = orc.layer_norm_fwd(F(xs.reshape(6, -1)), 4, 10, 10, 1e-5, g, b)
+    t = torch.nn.functional.layer_norm(torch.tensor(xs), (10,), torch.tensor(g), torch.tensor(b), 1e-5)
+    assert rel_err(y.T.reshape(6, 4, 10), t.numpy()) < 1e-12
+    assert rel_err(stats[:4].T, xs.mean(axis=2)) < 1e-12
+    assert rel_err(stats[4:].T, xs.var(axis=2)) < 1e-11
+
+
+def test_batch_norm_matches_torch_without_bessel():
+    rng = np.random.default_rng(2)
+    N, C, H, W = 5, 3, 4, 6
+    xs = rng.normal(2.0, 3.0, size=(N, C, H, W))
+    g, b = rng.uniform(0.5, 1.5, C), rng.normal(0, 0.1, C)
+    rm, rv = np.zeros(C), np.ones(C)
+    y, mean, var = orc.batch_norm_fwd(F(xs.reshape(N, -1)), C, H * W, 1e-5, 0.9, g, b, rm, rv, bessel=False)
+    trm, trv = torch.zeros(C, dtype=torch.float64), torch.ones(C, dtype=torch.float64)
+    t = torch.nn.functional.batch_norm(torch.tensor(xs), trm, trv, torch.tensor(g), torch.tensor(b),
+                                       training=True, momentum=0.1, eps=1e-5)
+    assert rel_err(y.T.reshape(xs.shape), t.numpy()) < 1e-12
+    assert rel_err(rm, trm.numpy()) < 1e-12
+    # torch's running variance always carries n/(n-1); the layer's follows its own flag
+    n = N * H * W
+    assert rel_err(rv, 0.9 + 0.1 * xs.var(axis=(0, 2, 3))) < 1e-12
+    _, _, var_b = orc.batch_norm_fwd(F(xs.reshape(N, -1)), C, H * W, 1e-5, 0.9, g, b, rm.copy(), rv.copy(), bessel=True)
+    assert rel_err(var_b, xs.var(axis=(0, 2, 3)) * n / (n - 1)) < 1e-12
+
+
+def test_batch_norm_inference_uses_running_stats():
+    rng = np.random.default_rng(3)
+    xs = rng.normal(size=(4, 2 * 5))
+    g, b = rng.uniform(0.5, 1.5, 2), rng.normal(0, 0.1, 2)
+    rm, rv = rng.normal(size=2), rng.uniform(0.5, 2, 2)
+    rm0, rv0 = rm.copy(), rv.copy()
+    y, _, _ = orc.batch_norm_fwd(F(xs), 2, 5, 1e-5, 0.9, g, b, rm, rv, training=False)
+    assert np.array_equal(rm, rm0) and np.array_equal(rv, rv0)
+    exp = (xs.reshape(4, 2, 5) - rm0[None, :, None]) / np.sqrt(rv0[None, :, None] + 1e-5) * g[None, :, None] + b[None, :, None]
+    assert rel_err(y.T.reshape(4, 2, 5), exp) < 1e-13
+
+
+def test_batch_norm_variance_floor_and_tiny_batches():
+    # constant channel: variance 0 is raised to eps, then eps is added again
+    x = np.full((6, 1), 3.0, dtype=np.float64, order="F")
+    g, b = np.array([2.0]), np.array([0.5])
+    rm, rv = np.zeros(1), np.ones(1)
+    y, mean, var = orc.batch_norm_fwd(x, 1, 6, 1e-3, 0.9, g, b, rm, rv)
+    assert var[0] == 1e-3 and mean[0] == 3.0
+    assert np.allclose(y, 0.5)
+    # a single value per channel: variance is set to one, running stats untouched
+    x = np.array([[4.0], [7.0]], order="F")
+    rm, rv = np.zeros(2), np.ones(2)
+    y, mean, var = orc.batch_norm_fwd(x, 2, 1, 1e-5, 0.9, np.ones(2), np.zeros(2), rm, rv)
+    assert np.array_equal(var, [1.0, 1.0]) and np.array_equal(mean, [4.0, 7.0])
+    assert np.array_equal(rm, [0, 0]) and np.array_equal(rv, [1, 1])
+    assert np.allclose(y, 0)
+    dx, *_ = orc.batch_norm_bwd(x, np.ones_like(x), 2, 1, 1e-5, mean, var, np.ones(2))
+    assert np.array_equal(dx, np.zeros_like(x))
+
+
+def test_layer_norm_single_entry_groups():
+    x = F(np.arange(6, dtype=np.float64).reshape(2, 3))
+    y, stats = orc.layer_norm_fwd(x, 3, 1, 1, 1e-5)
+    assert np.array_equal(stats[:3], x) and np.all(stats[3:] == 1.0) and np.all(y == 0)
+    dx, *_ = orc.layer_norm_bwd(x, np.ones_like(x), stats, 3, 1, 1, 1e-5)
+    assert np.all(dx == 0)
+
+
+def test_softmax_flushes_non_normal_outputs_to_zero():
+    # exp(-95) is a denormal float: kept by exp, flushed by the isnormal() test.
+    x = np.zeros((4, 3), dtype=np.float32, order="F")
+    x[1, 0] = -95.0      # denormal result -> 0
+    x[2, 0] = -200.0     # underflows to 0 anyway
+    x[:, 1] = [50, -45, 50, -41]   # 2 maxima: exp(-95)/2, exp(-91)/2
+    x[:, 2] = np.nan     # a NaN column: every entry fails isnormal -> 0
+    y = orc.softmax_fwd(x)
+    assert y[1, 0] == 0.0 and y[2, 0] == 0.0 and abs(y[0, 0] - 0.5) < 1e-7
+    assert y[1, 1] == 0.0 and y[3, 1] == 0.0
+    assert np.all(y[:, 2] == 0.0)
+    # the channelwise layer has no such flush: the denormal survives
+    yc = orc.channelwise_softmax_fwd(np.asfortranarray(x[:, :1]), 1, 4, 4)
+    assert 0 < yc[1, 0] < np.finfo(np.float32).tiny
+
+
+def test_softmax_shift_invariance_and_log_relation():
+    rng = np.random.default_rng(4)
+    x = np.asfortranarray(rng.normal(0, 2, size=(40, 6)))
+    y = orc.softmax_fwd(x)
+    assert rel_err(orc.softmax_fwd(x + 7.25), y) < 1e-13
+    assert rel_err(orc.log_softmax_fwd(x), np.log(y)) < 1e-13
+    t = torch.softmax(torch.tensor(x), dim=0).numpy()
+    assert rel_err(y, t) < 1e-14
+
+
+# ================================================================== backward
+def _fd(f, x, h=1e-5):
+    """5-point central difference of scalar f at every entry of x (float64)."""
+    g = np.zeros_like(x)
+    it = np.nditer(x, flags=["multi_index"])
+    for _ in it:
+        i = it.multi_index
+        x0 = x[i]
+        v = []
+        for k in (-2, -1, 1, 2):
+            x[i] = x0 + k * h
+            v.append(f())
+        x[i] = x0
+        g[i] = (v[0] - 8 * v[1] + 8 * v[2] - v[3]) / (12 * h)
+    return g
+
+
+@pytest.mark.parametrize("affine", [False, True])
+@pytest.mark.parametrize("G,n", [(1, 12), (3, 4)])
+def test_layer_norm_bwd_finite_difference(affine, G, n):
+    rng = np.random.default_rng(10 + G)
+    h, w = G * n, 3
+    x = np.asfortranarray(rng.normal(0.3, 1.5, size=(h, w)))
+    dy = np.asfortranarray(rng.normal(size=(h, w)))
+    gamma = rng.normal(1, 0.4, size=n) if affine else None
+    beta = rng.normal(0, 0.4, size=n) if affine else None
+    eps = 1e-3
+
+    def loss():
+        y, _ = orc.layer_norm_fwd(x, G, n, n, eps, gamma, beta)
+        return float(np.sum(y * dy))
+
+    _, stats = orc.layer_norm_fwd(x, G, n, n, eps, gamma, beta)
+    dx, sgrad, dg, db = orc.layer_norm_bwd(x, dy, stats, G, n, n, eps, gamma, affine, affine)
+    assert rel_err(dx, _fd(loss, x)) < 1e-7
+    # every group's input gradient sums to zero (output is shift invariant)
+    assert np.abs(dx.reshape(n, -1, order="F").sum(axis=0)).max() < 1e-12
+    if affine:
+        assert rel_err(dg, _fd(loss, gamma)) < 1e-8
+        assert rel_err(db, _fd(loss, beta)) < 1e-8
+    # statistics gradients: derivative of the loss with mean and variance treated as
+    # free variables of y = (x-mean)/sqrt(var+eps)*gamma+beta
+    mean, var = stats[:G].copy(), stats[G:].copy()
+    xr = x.reshape(n, G, w, order="F")
+    dyr = dy.reshape(n, G, w, order="F")
+    gam = (gamma if affine else np.ones(n))[:, None, None]
+
+    def loss_mv():
+        return float(np.sum((xr - mean[None]) / np.sqrt(var[None] + eps) * gam * dyr))
+
+    assert rel_err(sgrad[:G], _fd(loss_mv, mean)) < 1e-7
+    assert rel_err(sgrad[G:], _fd(loss_mv, var, h=1e-6)) < 1e-6
+
+
+def test_layer_norm_bwd_matches_torch_autograd():
+    rng = np.random.default_rng(11)
+    xs, dys = rng.normal(size=(5, 3, 8)), rng.normal(size=(5, 3, 8))
+    g, b = rng.normal(1, 0.3, 8), rng.normal(0, 0.3, 8)
+    tx = torch.tensor(xs, requires_grad=True)
+    tg, tb = torch.tensor(g, requires_grad=True), torch.tensor(b, requires_grad=True)
+    torch.nn.functional.layer_norm(tx, (8,), tg, tb, 1e-5).backward(torch.tensor(dys))
+    x, dy = F(xs.reshape(5, -1)), F(dys.reshape(5, -1))
+    _, stats = orc.layer_norm_fwd(x, 3, 8, 8, 1e-5, g, b)
+    dx, _, dg, db = orc.layer_norm_bwd(x, dy, stats, 3, 8, 8, 1e-5, g, True, True)
+    assert rel_err(dx.T.reshape(xs.shape), tx.grad.numpy()) < 1e-11
+    assert rel_err(dg, tg.grad.numpy()) < 1e-12
+    assert rel_err(db, tb.grad.numpy()) < 1e-12
+
+
+@pytest.mark.parametrize("bessel", [False, True])
+def test_batch_norm_bwd_finite_difference(bessel):
+    rng = np.random.default_rng(12)
+    C, cs, w = 3, 4, 5
+    x = np.asfortranarray(rng.normal(2, 3, size=(C * cs, w)))
+    dy = np.asfortranarray(rng.normal(size=(C * cs, w)))
+    gamma, beta = rng.uniform(0.5, 1.5, C), rng.normal(0, 0.1, C)
+    eps = 1e-3
+
+    def fwd():
+        return orc.batch_norm_fwd(x, C, cs, eps, 0.9, gamma, beta, np.zeros(C), np.ones(C), bessel=bessel)
+
+    def loss():
+        return float(np.sum(fwd()[0] * dy))
+
+    _, mean, var = fwd()
+    dx, dg, db, dmean, dvar = orc.batch_norm_bwd(x, dy, C, cs, eps, mean, var, gamma, bessel=bessel)
+    assert rel_err(dx, _fd(loss, x)) < 1e-7
+    assert rel_err(dg, _fd(loss, gamma)) < 1e-8
+    assert rel_err(db, _fd(loss, beta)) < 1e-8
+    assert np.abs(dx.reshape(cs, C, w, order="F").sum(axis=(0, 2))).max() < 1e-12
+    m, v = mean.copy(), var.copy()
+    xr, dyr = x.reshape(cs, C, w, order="F"), dy.reshape(cs, C, w, order="F")
+
+    def loss_mv():
+        return float(np.sum(((xr - m[None, :, None]) / np.sqrt(v[None, :, None] + eps) * gamma[None, :, None]) * dyr))
+
+    assert rel_err(dmean, _fd(loss_mv, m)) < 1e-7
+    assert rel_err(dvar, _fd(loss_mv, v, h=1e-6)) < 1e-6
+    # inference mode: statistics are constants; their gradients are reported as zero
+    rm, rv = rng.normal(size=C), rng.uniform(0.5, 2, C)
+    dxi, dgi, dbi, dmi, dvi = orc.batch_norm_bwd(x, dy, C, cs, eps, mean, var, gamma, rm, rv,
+                                                 bessel=bessel, training=False)
+    assert np.all(dmi == 0) and np.all(dvi == 0)
+    assert rel_err(dbi, dyr.sum(axis=(0, 2))) < 1e-13
+
+
+def test_batch_norm_bwd_matches_torch_autograd():
+    rng = np.random.default_rng(13)
+    N, C, H, W = 4, 3, 2, 5
+    xs, dys = rng.normal(2, 3, size=(N, C, H, W)), rng.normal(size=(N, C, H, W))
+    g, b = rng.uniform(0.5, 1.5, C), rng.normal(0, 0.1, C)
+    tx = torch.tensor(xs, requires_grad=True)
+    tg, tb = torch.tensor(g, requires_grad=True), torch.tensor(b, requires_grad=True)
+    torch.nn.functional.batch_norm(tx, None, None, tg, tb, training=True, eps=1e-5).backward(torch.tensor(dys))
+    x, dy = F(xs.reshape(N, -1)), F(dys.reshape(N, -1))
+    _, mean, var = orc.batch_norm_fwd(x, C, H * W, 1e-5, 0.9, g, b, np.zeros(C), np.ones(C), bessel=False)
+    dx, dg, db, _, _ = orc.batch_norm_bwd(x, dy, C, H * W, 1e-5, mean, var, g, bessel=False)
+    assert rel_err(dx.T.reshape(xs.shape), tx.grad.numpy()) < 1e-11
+    assert rel_err(dg, tg.grad.numpy()) < 1e-12
+    assert rel_err(db, tb.grad.numpy()) < 1e-12
+
+
+@pytest.mark.parametrize("kind", ["softmax", "log_softmax", "channelwise"])
+def test_softmax_family_bwd(kind):
+    rng = np.random.default_rng(14)
+    h, w = 12, 4
+    x = np.asfortranarray(rng.normal(0, 2, size=(h, w)))
+    dy = np.asfortranarray(rng.normal(size=(h, w)))
+    tx = torch.tensor(x, requires_grad=True)
+    if kind == "softmax":
+        y = orc.softmax_fwd(x)
+        dx = orc.softmax_bwd(y, dy)
+        torch.softmax(tx, dim=0).backward(torch.tensor(dy))
+        loss = lambda: float(np.sum(orc.softmax_fwd(x) * dy))
+    elif kind == "log_softmax":
+        y = orc.log_softmax_fwd(x)
+        dx = orc.log_softmax_bwd(y, dy)
+        torch.log_softmax(tx, dim=0).backward(torch.tensor(dy))
+        loss = lambda: float(np.sum(orc.log_softmax_fwd(x) * dy))
+    else:
+        y = orc.channelwise_softmax_fwd(x, 3, 4, 4)
+        dx = orc.channelwise_softmax_bwd(y, dy, 3, 4, 4)
+        torch.softmax(tx.reshape(3, 4, w), dim=1).reshape(h, w).backward(torch.tensor(dy))
+        loss = lambda: float(np.sum(orc.channelwise_softmax_fwd(x, 3, 4, 4) * dy))
+    assert rel_err(dx, tx.grad.numpy()) < 1e-12
+    assert rel_err(dx, _fd(loss, x)) < 1e-7
+    if kind == "softmax":
+        assert np.abs(dx.sum(axis=0)).max() < 1e-13
+    if kind == "channelwise":
+        assert np.abs(dx.reshape(4, -1, order="F").sum(axis=0)).max() < 1e-13
+
+
+def test_leading_dimension_and_f32_f64_agreement():
+    """Views with ld > height must give the same numbers as packed matrices."""
+    rng = np.random.default_rng(15)
+    big = np.asfortranarray(rng.normal(size=(40, 6)).astype(np.float32))
+    view = big[4:28, :]
+    packed = np.asfortranarray(view.copy())
+    assert view.strides[1] // 4 == 40
+    assert np.array_equal(orc.softmax_fwd(view), orc.softmax_fwd(packed))
+    assert np.array_equal(orc.log_softmax_fwd(view), orc.log_softmax_fwd(packed))
+    assert np.array_equal(orc.layer_norm_fwd(view, 2, 12, 12, 1e-5)[0], orc.layer_norm_fwd(packed, 2, 12, 12, 1e-5)[0])
+    assert np.array_equal(orc.channelwise_softmax_fwd(view, 4, 6, 6), orc.channelwise_softmax_fwd(packed, 4, 6, 6))
+    g, b = np.ones(3, np.float32), np.zeros(3, np.float32)
+    a = orc.batch_norm_fwd(view, 3, 8, 1e-5, 0.9, g, b, np.zeros(3, np.float32), np.ones(3, np.float32))[0]
+    c = orc.batch_norm_fwd(packed, 3, 8, 1e-5, 0.9, g, b, np.zeros(3, np.float32), np.ones(3, np.float32))[0]
+    assert np.array_equal(a, c)
+    y64 = orc.softmax_fwd(packed.astype(np.float64, order="F"))
+    assert rel_err(orc.softmax_fwd(packed), y64) < 1e-6
