@@ -1,0 +1,202 @@
+/* lbnorm.h — C ABI of the MI355X (gfx950) normalization and softmax kernels.
+ *
+ * Each entry point is the device compute of one LBANN layer's fp_compute() or
+ * bp_compute() on LOCAL matrices: column-major, element (r,c) at buf[r + c*ld],
+ * one column per mini-batch sample (El::Matrix<T,Device>: Height/Width/LDim/Buffer).
+ * A call only enqueues work on `stream`: it never synchronises the device,
+ * allocates or frees memory, or reads results back.  All pointers are device
+ * pointers that must stay valid until the stream work completes.  Every output
+ * element is overwritten (outputs may be uninitialised on entry); nothing is
+ * accumulated into.  Calls with width == 0 or an empty sample return LBN_OK
+ * without launching.
+ *
+ * Return value: LBN_OK, a negative LBN_ERR_* code for a rejected argument, or a
+ * positive hipError_t from the launch.  No C++ exception crosses this boundary.
+ *
+ * Scratch memory ("workspace") is always caller-provided.  The matching
+ * *_workspace_bytes() function returns the size needed for a given shape
+ * (possibly 0, in which case NULL may be passed).  A workspace only carries data
+ * between the kernels of one call.
+ */
+#ifndef LBNORM_H_INCLUDED
+#define LBNORM_H_INCLUDED
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* lbn_stream_t; /* a hipStream_t; NULL is the default stream */
+
+#define LBN_OK 0
+#define LBN_ERR_INVALID_ARGUMENT (-1) /* negative size, ld < height, NULL matrix, ... */
+#define LBN_ERR_WORKSPACE (-2)        /* workspace NULL or smaller than *_workspace_bytes() */
+#define LBN_ERR_UNSUPPORTED (-3)      /* shape outside what the kernels index (e.g. > 2^31 rows) */
+
+/* Statistics formula selector for the `flags` argument of the normalization forwards.
+ * LBN_STATS_TWO_PASS (default): mean first, then the mean of squared deviations.
+ * LBN_STATS_SUMSQ: E[x^2] - mean^2 from running sums, the formula of the reference
+ * CPU code (layer_norm.cpp:99-112, batch_normalization.cpp:124-128), including its
+ * cancellation error. */
+#define LBN_STATS_TWO_PASS 0
+#define LBN_STATS_SUMSQ 1
+
+int lbn_version(void);
+const char* lbn_status_string(int status);
+
+/* ------------------------------------------------------------------ layer norm
+ * Replaces layer_norm_layer::fp_compute / bp_compute
+ * (src/layers/regularizers/layer_norm.cpp:263-290, :292-348; math :41-136, :139-258).
+ * A sample holds `num_groups` groups (get_normdims, layer_norm.hpp:362-405: product
+ * of dims before start_dim) of `norm_size` contiguous entries, group g starting at
+ * row g*norm_stride.  stats is (2*num_groups x width): rows [0,G) mean, [G,2G)
+ * variance (biased, clamped at 0; 1 when norm_size <= 1); stats_grad likewise holds
+ * dL/dmean and dL/dvar.  scale/bias (length norm_size, fp32) may be NULL.
+ * Backward overwrites dscale/dbias (length norm_size) when they are non-NULL;
+ * dscale != NULL requires scale != NULL.  The _f16 variants store x, y, dy, dx as
+ * IEEE binary16 and compute in fp32; statistics, scale, bias and their gradients
+ * stay fp32. */
+int lbn_layer_norm_fwd_f32(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
+                           int64_t norm_stride, int64_t width, float epsilon,
+                           const float* x, int64_t ldx, float* y, int64_t ldy,
+                           float* stats, int64_t ld_stats,
+                           const float* scale, const float* bias, int flags);
+int lbn_layer_norm_fwd_f16(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
+                           int64_t norm_stride, int64_t width, float epsilon,
+                           const void* x, int64_t ldx, void* y, int64_t ldy,
+                           float* stats, int64_t ld_stats,
+                           const float* scale, const float* bias, int flags);
+size_t lbn_layer_norm_bwd_workspace_bytes(int64_t num_groups, int64_t norm_size,
+                                          int64_t width, int has_weight_grads,
+                                          int elem_bytes);
+int lbn_layer_norm_bwd_f32(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
+                           int64_t norm_stride, int64_t width, float epsilon,
+                           const float* x, int64_t ldx, const float* dy, int64_t lddy,
+                           float* dx, int64_t lddx,
+                           const float* stats, int64_t ld_stats,
+                           float* stats_grad, int64_t ld_stats_grad,
+                           const float* scale, float* dscale, float* dbias,
+                           void* workspace, size_t workspace_bytes);
+int lbn_layer_norm_bwd_f16(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
+                           int64_t norm_stride, int64_t width, float epsilon,
+                           const void* x, int64_t ldx, const void* dy, int64_t lddy,
+                           void* dx, int64_t lddx,
+                           const float* stats, int64_t ld_stats,
+                           float* stats_grad, int64_t ld_stats_grad,
+                           const float* scale, float* dscale, float* dbias,
+                           void* workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------ batch norm
+ * Replaces batch_normalization_layer::fp_compute / bp_compute
+ * (src/layers/regularizers/batch_normalization.cpp:37-175, :178-329).
+ * A sample is `channels` contiguous slabs of `channel_size` entries (NCHW flattened:
+ * channel c = rows [c*cs,(c+1)*cs) of every column).  mean/var (length channels) are
+ * the layer's m_mean_and_var columns; scale, bias, running_mean, running_var are
+ * weights 0..3.  training != 0 computes batch statistics over channel_size*width
+ * values (local statistics, statistics_group_size == 1), writes mean/var and updates
+ * the running statistics with `decay`; training == 0 normalises with the running
+ * statistics and leaves mean/var untouched.  bessel != 0 scales the variance by
+ * n/(n-1) (the reference default).  The variance is clamped below at epsilon and
+ * epsilon is added again under the square root, as the reference does. */
+size_t lbn_batch_norm_workspace_bytes(int64_t channels, int64_t channel_size, int64_t width);
+int lbn_batch_norm_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                           int64_t width, int bessel, float epsilon, float decay,
+                           int training, const float* x, int64_t ldx, float* y, int64_t ldy,
+                           float* mean, float* var, const float* scale, const float* bias,
+                           float* running_mean, float* running_var,
+                           void* workspace, size_t workspace_bytes, int flags);
+int lbn_batch_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                           int64_t width, int bessel, float epsilon, int training,
+                           const float* x, int64_t ldx, const float* dy, int64_t lddy,
+                           float* dx, int64_t lddx, const float* mean, const float* var,
+                           const float* running_mean, const float* running_var,
+                           const float* scale, float* dscale, float* dbias,
+                           float* dmean, float* dvar,
+                           void* workspace, size_t workspace_bytes);
+
+/* The same computation cut where the reference places its all-reduces, for callers
+ * that aggregate statistics over several ranks (batch_normalization.cpp:87-115 and
+ * :248-263): local sums -> [caller's all-reduce] -> statistics -> apply.
+ * fwd_sums writes per-channel sum(x) into `mean` and sum(x^2) into `var`;
+ * fwd_stats turns those sums over `num_per_sum` values into mean/variance in place
+ * and updates the running statistics; fwd_apply normalises.  bwd_sums writes dscale,
+ * dbias and the local parts of dmean, dvar; bwd_apply forms dx from the (reduced)
+ * dmean, dvar and the global `num_per_sum`. */
+int lbn_batch_norm_fwd_sums_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                int64_t width, const float* x, int64_t ldx,
+                                float* mean, float* var,
+                                void* workspace, size_t workspace_bytes);
+int lbn_batch_norm_fwd_stats_f32(lbn_stream_t stream, int64_t channels, int64_t num_per_sum,
+                                 int bessel, float epsilon, float decay,
+                                 float* mean, float* var,
+                                 float* running_mean, float* running_var);
+int lbn_batch_norm_fwd_apply_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                 int64_t width, float epsilon, const float* x, int64_t ldx,
+                                 float* y, int64_t ldy, const float* mean, const float* var,
+                                 const float* scale, const float* bias);
+int lbn_batch_norm_bwd_sums_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                int64_t width, float epsilon,
+                                const float* x, int64_t ldx, const float* dy, int64_t lddy,
+                                const float* mean, const float* var, const float* scale,
+                                float* dscale, float* dbias, float* dmean, float* dvar,
+                                void* workspace, size_t workspace_bytes);
+int lbn_batch_norm_bwd_apply_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                 int64_t width, int64_t num_per_sum, int bessel, float epsilon,
+                                 const float* x, int64_t ldx, const float* dy, int64_t lddy,
+                                 float* dx, int64_t lddx, const float* mean, const float* var,
+                                 const float* scale, const float* dmean, const float* dvar);
+
+/* --------------------------------------------------------------------- softmax
+ * Replaces softmax_layer::fp_compute / bp_compute on the data-parallel layout
+ * (src/layers/activations/softmax.cpp:157-234), whose CPU arithmetic is
+ * openmp_backend::softmax_forward / softmax_backward
+ * (include/lbann/utils/dnn_lib/openmp/softmax.hpp:39-117, :119-181), mode INSTANCE:
+ * softmax over each column.  Results that are not normal floats (zero, denormal, NaN)
+ * are written as 0, as that code does.  y may alias x and dx may alias dy (the layer
+ * can run in place, softmax.hpp:134). */
+size_t lbn_softmax_workspace_bytes(int64_t height, int64_t width);
+int lbn_softmax_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                        const float* x, int64_t ldx, float* y, int64_t ldy,
+                        void* workspace, size_t workspace_bytes);
+int lbn_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                        const float* y, int64_t ldy, const float* dy, int64_t lddy,
+                        float* dx, int64_t lddx, void* workspace, size_t workspace_bytes);
+
+/* ----------------------------------------------------------------- log-softmax
+ * Replaces log_softmax_layer::fp_compute / bp_compute
+ * (src/layers/activations/log_softmax.cpp:35-93, :95-136, :140-156).
+ * y = x - max - log(sum(exp(x - max))); dx = dy - exp(y) * sum(dy).  In place allowed
+ * (log_softmax.hpp:101).  Shares lbn_softmax_workspace_bytes(). */
+int lbn_log_softmax_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                            const float* x, int64_t ldx, float* y, int64_t ldy,
+                            void* workspace, size_t workspace_bytes);
+int lbn_log_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                            const float* y, int64_t ldy, const float* dy, int64_t lddy,
+                            float* dx, int64_t lddx, void* workspace, size_t workspace_bytes);
+
+/* --------------------------------------------------------- channelwise softmax
+ * Replaces channelwise_softmax_layer::fp_compute / bp_compute
+ * (src/layers/misc/channelwise_softmax.cpp:41-113, :121-184).  Each sample holds
+ * `channels` windows of `channel_size` contiguous entries, window j starting at row
+ * j*channel_stride (get_channel_size_and_stride, channelwise_softmax_impl.hpp:58-104);
+ * a softmax is taken inside every window.  No flush of denormal results.  In place
+ * allowed (channelwise_softmax.hpp:78) when windows do not overlap. */
+size_t lbn_channelwise_softmax_workspace_bytes(int64_t channels, int64_t channel_size,
+                                               int64_t width);
+int lbn_channelwise_softmax_fwd_f32(lbn_stream_t stream, int64_t channels,
+                                    int64_t channel_size, int64_t channel_stride,
+                                    int64_t width, const float* x, int64_t ldx,
+                                    float* y, int64_t ldy,
+                                    void* workspace, size_t workspace_bytes);
+int lbn_channelwise_softmax_bwd_f32(lbn_stream_t stream, int64_t channels,
+                                    int64_t channel_size, int64_t channel_stride,
+                                    int64_t width, const float* y, int64_t ldy,
+                                    const float* dy, int64_t lddy, float* dx, int64_t lddx,
+                                    void* workspace, size_t workspace_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LBNORM_H_INCLUDED */

@@ -1,0 +1,38 @@
+"""Builds lbann_amd/liblbnorm.so: the HIP kernels and their C ABI, for gfx950 only.
+
+    python -m lbann_amd.build
+
+hipcc cross-compiles without a GPU.  The library depends on the HIP runtime only
+(no torch, no MPI).  Packed-fp32 VALU instructions are switched off for every
+translation unit.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "liblbnorm.so")
+SOURCES = ["capi_common.hip", "softmax.hip", "layer_norm.hip", "batch_norm.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _compile(src):
+    obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+    subprocess.run([HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj], check=True)
+    return obj
+
+
+def build(jobs: int = 4) -> str:
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(_compile, SOURCES))
+    subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], check=True)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build())
+    sys.exit(0)

@@ -1,0 +1,174 @@
+// Device-side building blocks shared by every kernel: 128-bit coalesced row I/O,
+// wave64 shuffle reductions, LDS cross-wave reductions, and the row -> address map
+// of LBANN's column-major local matrices.  gfx950 only (64-wide wavefronts).
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+#include <cstdint>
+
+namespace lbn {
+
+constexpr int kWave = 64;
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int64_t imin64(int64_t a, int64_t b) { return a < b ? a : b; }
+
+// ---------------------------------------------------------------------------
+// A "row" is one contiguous run of n entries that is normalised on its own: a
+// whole matrix column (softmax), one group of a column (layer norm with
+// start_dim > 0) or one channel window (channelwise softmax).  Row r lives at
+// (r % groups) * stride + (r / groups) * ld.
+struct RowMap {
+  int64_t groups;
+  int64_t stride;
+  __device__ __forceinline__ int64_t offset(int64_t row, int64_t ld) const
+  {
+    const int64_t col = row / groups;
+    const int64_t g = row - col * groups;
+    return g * stride + col * ld;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// 16-byte vector access for the two storage types.  Values are always widened to
+// fp32 registers.
+template <typename T>
+struct Vec16;
+
+template <>
+struct Vec16<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4])
+  {
+    const v4f r = *reinterpret_cast<const v4f*>(p);
+    v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4])
+  {
+    v4f r;
+    r.x = v[0]; r.y = v[1]; r.z = v[2]; r.w = v[3];
+    *reinterpret_cast<v4f*>(p) = r;
+  }
+  static __device__ __forceinline__ float load1(const float* p) { return *p; }
+  static __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
+};
+
+template <>
+struct Vec16<__half> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void load(const __half* p, float (&v)[8])
+  {
+    const v4u r = *reinterpret_cast<const v4u*>(p);
+    const unsigned int w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __half2 h;
+      __builtin_memcpy(&h, &w[i], 4);
+      const float2 f = __half22float2(h);
+      v[2 * i] = f.x;
+      v[2 * i + 1] = f.y;
+    }
+  }
+  static __device__ __forceinline__ void store(__half* p, const float (&v)[8])
+  {
+    unsigned int w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const __half2 h = __floats2half2_rn(v[2 * i], v[2 * i + 1]);
+      __builtin_memcpy(&w[i], &h, 4);
+    }
+    v4u r;
+    r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
+    *reinterpret_cast<v4u*>(p) = r;
+  }
+  static __device__ __forceinline__ float load1(const __half* p) { return __half2float(*p); }
+  static __device__ __forceinline__ void store1(__half* p, float v) { *p = __float2half_rn(v); }
+};
+
+// ---------------------------------------------------------------------------
+// Wave64 butterfly reductions: every lane ends with the result.
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+// Reductions over a team of NW waves (NW*64 consecutive threads of the block).
+// `slot` must point to NW floats (2*NW for the pair version) of LDS that no other
+// reduction touches before the next block-wide barrier; every thread of the block
+// must make the call when NW > 1.  The summation order is fixed, so results are
+// bitwise reproducible run to run.
+template <int NW>
+__device__ __forceinline__ float team_sum(float v, float* slot, int wave_in_team, int lane)
+{
+  v = wave_sum(v);
+  if constexpr (NW == 1) return v;
+  if (lane == 0) slot[wave_in_team] = v;
+  __syncthreads();
+  float r = slot[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) r += slot[i];
+  return r;
+}
+
+template <int NW>
+__device__ __forceinline__ float team_max(float v, float* slot, int wave_in_team, int lane)
+{
+  v = wave_max(v);
+  if constexpr (NW == 1) return v;
+  if (lane == 0) slot[wave_in_team] = v;
+  __syncthreads();
+  float r = slot[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) r = fmaxf(r, slot[i]);
+  return r;
+}
+
+template <int NW>
+__device__ __forceinline__ void team_sum2(float& a, float& b, float* slot, int wave_in_team,
+                                          int lane)
+{
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if constexpr (NW == 1) return;
+  if (lane == 0) {
+    slot[2 * wave_in_team] = a;
+    slot[2 * wave_in_team + 1] = b;
+  }
+  __syncthreads();
+  float ra = slot[0], rb = slot[1];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) {
+    ra += slot[2 * i];
+    rb += slot[2 * i + 1];
+  }
+  a = ra;
+  b = rb;
+}
+
+// Thread-block shape used by the register-resident row kernels: a row is owned by a
+// team of TPR threads (64, 256 or 1024) and a block holds TEAMS teams.  By default
+// blocks have at least 256 threads, so a block covers 4 rows when one wave owns a
+// row.  Reductions of multi-wave teams use block-wide barriers, so all teams of a
+// block must make the same sequence of reduction calls.
+template <int TPR, int TEAMS = (TPR < 256 ? 256 / TPR : 1)>
+struct RowBlock {
+  static constexpr int kTeams = TEAMS;
+  static constexpr int kThreads = TPR * TEAMS;
+  static constexpr int kWavesPerTeam = TPR / kWave;
+  static_assert(kThreads <= 1024, "block too large");
+};
+
+}  // namespace lbn

@@ -1,0 +1,85 @@
+// Host-side helpers shared by the entry points: argument checks, alignment tests,
+// launch-shape selection for the register-resident row kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdlib>
+
+#include "../../include/lbnorm.h"
+
+namespace lbn {
+
+inline hipStream_t as_stream(lbn_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Status of the launches issued so far by this thread: 0 or the hipError_t.
+inline int launch_status()
+{
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? LBN_OK : static_cast<int>(e);
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// True when every row start of a matrix walked with (stride, ld) keeps 16-byte
+// alignment for elements of `esize` bytes.
+inline bool rows_aligned16(const void* base, int64_t stride, int64_t ld, int64_t groups,
+                           int64_t width, int esize)
+{
+  const int64_t per = 16 / esize;
+  if (!aligned16(base)) return false;
+  if (groups > 1 && stride % per != 0) return false;
+  if (width > 1 && ld % per != 0) return false;
+  return true;
+}
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Shape of a register-resident row kernel: `tpr` threads own a row and each keeps
+// `v` 16-byte vectors of it in registers.  tpr == 0: the row does not fit.
+struct RowConfig {
+  int tpr;
+  int v;
+};
+
+inline int round_up_pow2_le8(int64_t v)
+{
+  if (v <= 1) return 1;
+  if (v <= 2) return 2;
+  if (v <= 4) return 4;
+  if (v <= 8) return 8;
+  return 0;
+}
+
+// nvec: 16-byte vectors per row; rows: number of independent rows.
+// Prefers <= 4 vectors per thread with the fewest threads per row, and widens the
+// team when the launch would otherwise leave most of the 256 compute units without
+// work (small problems are latency bound, so more threads per row helps there).
+inline RowConfig pick_row_config(int64_t nvec, int64_t rows, int max_v = 8)
+{
+  static const int force_tpr = std::getenv("LBN_ROW_TPR") ? std::atoi(std::getenv("LBN_ROW_TPR")) : 0;
+  const int tprs[3] = {64, 256, 1024};
+  int vs[3];
+  for (int i = 0; i < 3; ++i) {
+    vs[i] = round_up_pow2_le8(ceil_div(nvec, tprs[i]));
+    if (vs[i] > max_v) vs[i] = 0;
+  }
+  if (force_tpr) {
+    for (int i = 0; i < 3; ++i)
+      if (tprs[i] == force_tpr && vs[i]) return {tprs[i], vs[i]};
+  }
+  int pick = -1;
+  for (int i = 0; i < 3; ++i) {
+    if (vs[i] == 0) continue;
+    pick = i;
+    if (vs[i] <= 4) break;
+  }
+  if (pick < 0) return {0, 0};
+  const int64_t want_waves = 2048;
+  while (pick < 2 && vs[pick] > 1 && rows * (tprs[pick] / 64) < want_waves && vs[pick + 1] != 0)
+    ++pick;
+  return {tprs[pick], vs[pick]};
+}
+
+}  // namespace lbn

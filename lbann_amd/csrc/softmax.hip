@@ -1,0 +1,517 @@
+// Softmax, log-softmax and channelwise softmax, forward and backward, for gfx950.
+//
+// All three layers reduce over independent contiguous rows (a matrix column, or a
+// channel window of a column).  Two kernel families cover every shape:
+//
+//  * register-resident row kernels: TPR threads (one wave, 256 or 1024 threads)
+//    load a whole row with 128-bit coalesced loads, keep it in registers, reduce
+//    with wave64 shuffles (+ one LDS hop across waves), and store the result.
+//    Each tensor is read once and written once.  Used when rows are 16-byte
+//    aligned, a multiple of 4 long and at most 32768 entries.
+//  * split ("chunked") kernels for very long or unaligned rows: a row is cut into
+//    S chunks, one workgroup each.  Kernel 1 leaves one partial reduction per chunk
+//    in the workspace (for softmax an online (max, sum) pair), kernel 2 merges the
+//    S partials and writes its chunk.  Kernel 1 reads everything before kernel 2
+//    writes anything, so in-place operation stays safe with many workgroups per row.
+//
+// Numerics follow the reference CPU code: max-subtraction, expf/logf at <= 1 ulp,
+// reciprocal-then-multiply, and softmax (only) writes 0 for results that are not
+// normal floats (include/lbann/utils/dnn_lib/openmp/softmax.hpp:107-116).
+#include "device_utils.hpp"
+#include "host_utils.hpp"
+
+namespace lbn {
+
+enum SmKind : int { kSoftmax = 0, kLogSoftmax = 1, kChannelwise = 2 };
+
+constexpr int kMaxChunks = 64;  // S <= one wave, so a wave merges the partials of a row
+
+// ======================================================= register-resident rows
+template <int TPR, int V, int KIND>
+__global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
+sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
+            int nvec)
+{
+  using B = RowBlock<TPR>;
+  constexpr int NW = B::kWavesPerTeam;
+  __shared__ float red[2][NW];
+  const int tid = threadIdx.x;
+  const int team = tid / TPR;
+  const int t = tid - team * TPR;
+  const int lane = tid & (kWave - 1);
+  const int wv = t / kWave;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * B::kTeams + team;
+  if (B::kTeams > 1 && row >= rows) return;  // whole waves leave; no barrier below in that case
+
+  const float* xr = x + map.offset(row, ldx);
+  float v[V][4];
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const int idx = t + i * TPR;
+    if (idx < nvec) {
+      Vec16<float>::load(xr + 4 * idx, v[i]);
+    }
+    else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[i][k] = -FLT_MAX;
+    }
+  }
+
+  // column maximum, starting from the lowest finite float like the reference
+  float m = -FLT_MAX;
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m = fmaxf(m, v[i][k]);
+  m = team_max<NW>(m, red[0], wv, lane);
+
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const bool ok = (t + i * TPR) < nvec;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float d = v[i][k] - m;
+      const float e = ok ? expf(d) : 0.f;
+      s += e;
+      v[i][k] = (KIND == kLogSoftmax) ? d : e;
+    }
+  }
+  s = team_sum<NW>(s, red[1], wv, lane);
+
+  float* yr = y + map.offset(row, ldy);
+  const float scale = 1.0f / s;
+  const float lse = (KIND == kLogSoftmax) ? logf(s) : 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const int idx = t + i * TPR;
+    if (idx < nvec) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (KIND == kSoftmax) {
+          const float r = scale * v[i][k];
+          v[i][k] = __builtin_isnormal(r) ? r : 0.f;
+        }
+        else if (KIND == kLogSoftmax) {
+          v[i][k] -= lse;
+        }
+        else {
+          v[i][k] *= scale;
+        }
+      }
+      Vec16<float>::store(yr + 4 * idx, v[i]);
+    }
+  }
+}
+
+// softmax / channelwise: dx = y * (dy - dot(y, dy));  log-softmax: dx = dy - exp(y) * sum(dy)
+template <int TPR, int V, int KIND>
+__global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
+sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
+            RowMap map, int64_t rows, int nvec)
+{
+  using B = RowBlock<TPR>;
+  constexpr int NW = B::kWavesPerTeam;
+  __shared__ float red[NW];
+  const int tid = threadIdx.x;
+  const int team = tid / TPR;
+  const int t = tid - team * TPR;
+  const int lane = tid & (kWave - 1);
+  const int wv = t / kWave;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * B::kTeams + team;
+  if (B::kTeams > 1 && row >= rows) return;
+
+  const float* yr = y + map.offset(row, ldy);
+  const float* gr = dy + map.offset(row, lddy);
+  float a[V][4], g[V][4];
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const int idx = t + i * TPR;
+    if (idx < nvec) {
+      Vec16<float>::load(yr + 4 * idx, a[i]);
+      Vec16<float>::load(gr + 4 * idx, g[i]);
+    }
+    else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) a[i][k] = g[i][k] = 0.f;
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) s += (KIND == kLogSoftmax) ? g[i][k] : a[i][k] * g[i][k];
+  s = team_sum<NW>(s, red, wv, lane);
+
+  float* dr = dx + map.offset(row, lddx);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const int idx = t + i * TPR;
+    if (idx < nvec) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (KIND == kLogSoftmax) g[i][k] = g[i][k] - expf(a[i][k]) * s;
+        else g[i][k] = a[i][k] * (g[i][k] - s);
+      }
+      Vec16<float>::store(dr + 4 * idx, g[i]);
+    }
+  }
+}
+
+// ================================================================ split rows
+// Block b handles chunk (b % S) of row (b / S); 256 threads per block.
+constexpr int kChunkThreads = 256;
+
+// Merges the online-softmax pairs (m, acc) of the 256 threads; every thread gets the result.
+__device__ __forceinline__ void block_merge_max_sum(float& m, float& acc, float (*slot)[2])
+{
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wv = threadIdx.x / kWave;
+  const float wm = wave_max(m);
+  acc = wave_sum(acc * expf(m - wm));
+  if (lane == 0) {
+    slot[wv][0] = wm;
+    slot[wv][1] = acc;
+  }
+  __syncthreads();
+  float bm = slot[0][0];
+#pragma unroll
+  for (int i = 1; i < kChunkThreads / kWave; ++i) bm = fmaxf(bm, slot[i][0]);
+  float bs = 0.f;
+#pragma unroll
+  for (int i = 0; i < kChunkThreads / kWave; ++i) bs += slot[i][1] * expf(slot[i][0] - bm);
+  m = bm;
+  acc = bs;
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_fwd_partial(const float* x, int64_t ldx, RowMap map, int64_t n, int64_t chunk, int S,
+               float2* part)
+{
+  __shared__ float slot[kChunkThreads / kWave][2];
+  const int64_t row = blockIdx.x / S;
+  const int s = blockIdx.x - row * S;
+  const int64_t begin = s * chunk;
+  const int64_t end = imin64(n, begin + chunk);
+  const float* xr = x + map.offset(row, ldx);
+  float m = -FLT_MAX, acc = 0.f;
+  if (VEC) {
+    for (int64_t i = begin / 4 + threadIdx.x; i < end / 4; i += kChunkThreads) {
+      float v[4];
+      Vec16<float>::load(xr + 4 * i, v);
+      const float mn = fmaxf(fmaxf(fmaxf(m, v[0]), fmaxf(v[1], v[2])), v[3]);
+      acc = acc * expf(m - mn) + ((expf(v[0] - mn) + expf(v[1] - mn)) + (expf(v[2] - mn) + expf(v[3] - mn)));
+      m = mn;
+    }
+  }
+  else {
+    for (int64_t i = begin + threadIdx.x; i < end; i += kChunkThreads) {
+      const float v = xr[i];
+      const float mn = fmaxf(m, v);
+      acc = acc * expf(m - mn) + expf(v - mn);
+      m = mn;
+    }
+  }
+  block_merge_max_sum(m, acc, slot);
+  if (threadIdx.x == 0) part[blockIdx.x] = make_float2(m, acc);
+}
+
+template <bool VEC, int KIND>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_fwd_apply(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t n,
+             int64_t chunk, int S, const float2* part)
+{
+  const int64_t row = blockIdx.x / S;
+  const int s = blockIdx.x - row * S;
+  const int64_t begin = s * chunk;
+  const int64_t end = imin64(n, begin + chunk);
+  const int lane = threadIdx.x & (kWave - 1);
+  // every wave merges the S <= 64 partials of the row on its own
+  float pm = -FLT_MAX, ps = 0.f;
+  if (lane < S) {
+    const float2 p = part[row * S + lane];
+    pm = p.x;
+    ps = p.y;
+  }
+  const float m = wave_max(pm);
+  const float sum = wave_sum(ps * expf(pm - m));
+  const float scale = 1.0f / sum;
+  const float lse = (KIND == kLogSoftmax) ? logf(sum) : 0.f;
+  const float* xr = x + map.offset(row, ldx);
+  float* yr = y + map.offset(row, ldy);
+  auto f = [&](float v) -> float {
+    const float d = v - m;
+    if (KIND == kLogSoftmax) return d - lse;
+    const float r = scale * expf(d);
+    if (KIND == kSoftmax) return __builtin_isnormal(r) ? r : 0.f;
+    return r;
+  };
+  if (VEC) {
+    for (int64_t i = begin / 4 + threadIdx.x; i < end / 4; i += kChunkThreads) {
+      float v[4];
+      Vec16<float>::load(xr + 4 * i, v);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = f(v[k]);
+      Vec16<float>::store(yr + 4 * i, v);
+    }
+  }
+  else {
+    for (int64_t i = begin + threadIdx.x; i < end; i += kChunkThreads) yr[i] = f(xr[i]);
+  }
+}
+
+template <bool VEC, int KIND>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_bwd_partial(const float* y, const float* dy, int64_t ldy, int64_t lddy, RowMap map, int64_t n,
+               int64_t chunk, int S, float* part)
+{
+  __shared__ float slot[kChunkThreads / kWave];
+  const int64_t row = blockIdx.x / S;
+  const int s = blockIdx.x - row * S;
+  const int64_t begin = s * chunk;
+  const int64_t end = imin64(n, begin + chunk);
+  const float* yr = y + map.offset(row, ldy);
+  const float* gr = dy + map.offset(row, lddy);
+  float acc = 0.f;
+  if (VEC) {
+    for (int64_t i = begin / 4 + threadIdx.x; i < end / 4; i += kChunkThreads) {
+      float g[4];
+      Vec16<float>::load(gr + 4 * i, g);
+      if (KIND == kLogSoftmax) {
+        acc += (g[0] + g[1]) + (g[2] + g[3]);
+      }
+      else {
+        float a[4];
+        Vec16<float>::load(yr + 4 * i, a);
+        acc += (a[0] * g[0] + a[1] * g[1]) + (a[2] * g[2] + a[3] * g[3]);
+      }
+    }
+  }
+  else {
+    for (int64_t i = begin + threadIdx.x; i < end; i += kChunkThreads)
+      acc += (KIND == kLogSoftmax) ? gr[i] : yr[i] * gr[i];
+  }
+  acc = team_sum<kChunkThreads / kWave>(acc, slot, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+  if (threadIdx.x == 0) part[blockIdx.x] = acc;
+}
+
+template <bool VEC, int KIND>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_bwd_apply(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
+             RowMap map, int64_t n, int64_t chunk, int S, const float* part)
+{
+  const int64_t row = blockIdx.x / S;
+  const int s = blockIdx.x - row * S;
+  const int64_t begin = s * chunk;
+  const int64_t end = imin64(n, begin + chunk);
+  const int lane = threadIdx.x & (kWave - 1);
+  const float sum = wave_sum(lane < S ? part[row * S + lane] : 0.f);
+  const float* yr = y + map.offset(row, ldy);
+  const float* gr = dy + map.offset(row, lddy);
+  float* dr = dx + map.offset(row, lddx);
+  auto f = [&](float a, float g) -> float {
+    return (KIND == kLogSoftmax) ? g - expf(a) * sum : a * (g - sum);
+  };
+  if (VEC) {
+    for (int64_t i = begin / 4 + threadIdx.x; i < end / 4; i += kChunkThreads) {
+      float a[4], g[4];
+      Vec16<float>::load(yr + 4 * i, a);
+      Vec16<float>::load(gr + 4 * i, g);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) g[k] = f(a[k], g[k]);
+      Vec16<float>::store(dr + 4 * i, g);
+    }
+  }
+  else {
+    for (int64_t i = begin + threadIdx.x; i < end; i += kChunkThreads) dr[i] = f(yr[i], gr[i]);
+  }
+}
+
+// ==================================================================== host side
+struct ChunkPlan {
+  int S;
+  int64_t chunk;
+};
+
+// Chunks per row for the split kernels: enough workgroups to occupy the device
+// (about 4 per compute unit) without cutting rows into pieces shorter than 2048
+// entries; chunk lengths are multiples of 4 so vector access stays aligned.
+static ChunkPlan plan_chunks(int64_t n, int64_t rows)
+{
+  int64_t S = ceil_div(1024, rows);
+  const int64_t by_len = ceil_div(n, 2048);
+  if (S > by_len) S = by_len;
+  if (S > kMaxChunks) S = kMaxChunks;
+  if (S < 1) S = 1;
+  int64_t chunk = ceil_div(ceil_div(n, S), 4) * 4;
+  S = ceil_div(n, chunk);
+  return {static_cast<int>(S), chunk};
+}
+
+static size_t sm_workspace_bytes(int64_t n, int64_t rows)
+{
+  if (n <= 0 || rows <= 0) return 0;
+  return static_cast<size_t>(rows) * plan_chunks(n, rows).S * sizeof(float2);
+}
+
+#define LBN_ROW_CASES(X)                                                                     \
+  X(64, 1) X(64, 2) X(64, 4) X(64, 8) X(256, 1) X(256, 2) X(256, 4) X(256, 8) X(1024, 1)      \
+  X(1024, 2) X(1024, 4) X(1024, 8)
+
+template <int KIND>
+static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int64_t w,
+                  const float* x, int64_t ldx, float* y, int64_t ldy, void* ws, size_t ws_bytes)
+{
+  if (groups < 0 || n < 0 || w < 0 || stride < 0) return LBN_ERR_INVALID_ARGUMENT;
+  if (groups == 0 || n == 0 || w == 0) return LBN_OK;
+  if (!x || !y) return LBN_ERR_INVALID_ARGUMENT;
+  const int64_t height = (groups - 1) * stride + n;
+  if (w > 1 && (ldx < height || ldy < height)) return LBN_ERR_INVALID_ARGUMENT;
+  const int64_t rows = groups * w;
+  if (rows > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+  const RowMap map{groups, stride};
+  const bool vec = (n % 4 == 0) && rows_aligned16(x, stride, ldx, groups, w, 4) &&
+                   rows_aligned16(y, stride, ldy, groups, w, 4);
+  if (vec) {
+    const RowConfig c = pick_row_config(n / 4, rows);
+    if (c.tpr) {
+      const int nvec = static_cast<int>(n / 4);
+#define X(TPR, V)                                                                            \
+  if (c.tpr == TPR && c.v == V) {                                                            \
+    using B = RowBlock<TPR>;                                                                 \
+    const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
+    hipLaunchKernelGGL((sm_fwd_rows<TPR, V, KIND>), dim3(grid), dim3(B::kThreads), 0, st, x, \
+                       y, ldx, ldy, map, rows, nvec);                                        \
+    return launch_status();                                                                  \
+  }
+      LBN_ROW_CASES(X)
+#undef X
+    }
+  }
+  const ChunkPlan p = plan_chunks(n, rows);
+  if (rows * p.S > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+  if (!ws || ws_bytes < static_cast<size_t>(rows) * p.S * sizeof(float2)) return LBN_ERR_WORKSPACE;
+  float2* part = static_cast<float2*>(ws);
+  const dim3 grid(static_cast<unsigned>(rows * p.S)), block(kChunkThreads);
+  if (vec) {
+    hipLaunchKernelGGL((sm_fwd_partial<true>), grid, block, 0, st, x, ldx, map, n, p.chunk, p.S, part);
+    hipLaunchKernelGGL((sm_fwd_apply<true, KIND>), grid, block, 0, st, x, y, ldx, ldy, map, n, p.chunk, p.S, part);
+  }
+  else {
+    hipLaunchKernelGGL((sm_fwd_partial<false>), grid, block, 0, st, x, ldx, map, n, p.chunk, p.S, part);
+    hipLaunchKernelGGL((sm_fwd_apply<false, KIND>), grid, block, 0, st, x, y, ldx, ldy, map, n, p.chunk, p.S, part);
+  }
+  return launch_status();
+}
+
+template <int KIND>
+static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int64_t w,
+                  const float* y, int64_t ldy, const float* dy, int64_t lddy, float* dx,
+                  int64_t lddx, void* ws, size_t ws_bytes)
+{
+  if (groups < 0 || n < 0 || w < 0 || stride < 0) return LBN_ERR_INVALID_ARGUMENT;
+  if (groups == 0 || n == 0 || w == 0) return LBN_OK;
+  if (!y || !dy || !dx) return LBN_ERR_INVALID_ARGUMENT;
+  const int64_t height = (groups - 1) * stride + n;
+  if (w > 1 && (ldy < height || lddy < height || lddx < height)) return LBN_ERR_INVALID_ARGUMENT;
+  const int64_t rows = groups * w;
+  if (rows > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+  const RowMap map{groups, stride};
+  const bool vec = (n % 4 == 0) && rows_aligned16(y, stride, ldy, groups, w, 4) &&
+                   rows_aligned16(dy, stride, lddy, groups, w, 4) &&
+                   rows_aligned16(dx, stride, lddx, groups, w, 4);
+  if (vec) {
+    // two tensors live in registers: cap each at 4 vectors per thread when a row
+    // still fits, so 1024-thread blocks keep two blocks per compute unit
+    const RowConfig c = pick_row_config(n / 4, rows);
+    if (c.tpr) {
+      const int nvec = static_cast<int>(n / 4);
+#define X(TPR, V)                                                                            \
+  if (c.tpr == TPR && c.v == V) {                                                            \
+    using B = RowBlock<TPR>;                                                                 \
+    const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
+    hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND>), dim3(grid), dim3(B::kThreads), 0, st, y, \
+                       dy, dx, ldy, lddy, lddx, map, rows, nvec);                            \
+    return launch_status();                                                                  \
+  }
+      LBN_ROW_CASES(X)
+#undef X
+    }
+  }
+  const ChunkPlan p = plan_chunks(n, rows);
+  if (rows * p.S > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+  if (!ws || ws_bytes < static_cast<size_t>(rows) * p.S * sizeof(float2)) return LBN_ERR_WORKSPACE;
+  float* part = static_cast<float*>(ws);
+  const dim3 grid(static_cast<unsigned>(rows * p.S)), block(kChunkThreads);
+  if (vec) {
+    hipLaunchKernelGGL((sm_bwd_partial<true, KIND>), grid, block, 0, st, y, dy, ldy, lddy, map, n, p.chunk, p.S, part);
+    hipLaunchKernelGGL((sm_bwd_apply<true, KIND>), grid, block, 0, st, y, dy, dx, ldy, lddy, lddx, map, n, p.chunk, p.S, part);
+  }
+  else {
+    hipLaunchKernelGGL((sm_bwd_partial<false, KIND>), grid, block, 0, st, y, dy, ldy, lddy, map, n, p.chunk, p.S, part);
+    hipLaunchKernelGGL((sm_bwd_apply<false, KIND>), grid, block, 0, st, y, dy, dx, ldy, lddy, lddx, map, n, p.chunk, p.S, part);
+  }
+  return launch_status();
+}
+
+}  // namespace lbn
+
+using namespace lbn;
+
+extern "C" {
+
+size_t lbn_softmax_workspace_bytes(int64_t height, int64_t width)
+{
+  return sm_workspace_bytes(height, width);
+}
+
+size_t lbn_channelwise_softmax_workspace_bytes(int64_t channels, int64_t channel_size, int64_t width)
+{
+  if (channels <= 0 || width <= 0) return 0;
+  return sm_workspace_bytes(channel_size, channels * width);
+}
+
+int lbn_softmax_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* x,
+                        int64_t ldx, float* y, int64_t ldy, void* workspace, size_t workspace_bytes)
+{
+  return sm_fwd<kSoftmax>(as_stream(stream), 1, height, height, width, x, ldx, y, ldy, workspace, workspace_bytes);
+}
+
+int lbn_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* y,
+                        int64_t ldy, const float* dy, int64_t lddy, float* dx, int64_t lddx,
+                        void* workspace, size_t workspace_bytes)
+{
+  return sm_bwd<kSoftmax>(as_stream(stream), 1, height, height, width, y, ldy, dy, lddy, dx, lddx, workspace, workspace_bytes);
+}
+
+int lbn_log_softmax_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* x,
+                            int64_t ldx, float* y, int64_t ldy, void* workspace, size_t workspace_bytes)
+{
+  return sm_fwd<kLogSoftmax>(as_stream(stream), 1, height, height, width, x, ldx, y, ldy, workspace, workspace_bytes);
+}
+
+int lbn_log_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* y,
+                            int64_t ldy, const float* dy, int64_t lddy, float* dx, int64_t lddx,
+                            void* workspace, size_t workspace_bytes)
+{
+  return sm_bwd<kLogSoftmax>(as_stream(stream), 1, height, height, width, y, ldy, dy, lddy, dx, lddx, workspace, workspace_bytes);
+}
+
+int lbn_channelwise_softmax_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                    int64_t channel_stride, int64_t width, const float* x,
+                                    int64_t ldx, float* y, int64_t ldy, void* workspace,
+                                    size_t workspace_bytes)
+{
+  return sm_fwd<kChannelwise>(as_stream(stream), channels, channel_size, channel_stride, width, x, ldx, y, ldy, workspace, workspace_bytes);
+}
+
+int lbn_channelwise_softmax_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                    int64_t channel_stride, int64_t width, const float* y,
+                                    int64_t ldy, const float* dy, int64_t lddy, float* dx,
+                                    int64_t lddx, void* workspace, size_t workspace_bytes)
+{
+  return sm_bwd<kChannelwise>(as_stream(stream), channels, channel_size, channel_stride, width, y, ldy, dy, lddy, dx, lddx, workspace, workspace_bytes);
+}
+
+}  // extern "C"

@@ -1,0 +1,355 @@
+"""Host-side mirror of the five LBANN layer classes, over the C ABI.
+
+Each class keeps the reference layer's constructor parameters, its member
+matrices and its two compute hooks, `fp_compute()` and `bp_compute()`
+(include/lbann/layers/layer.hpp:835,852), and forwards them to liblbnorm.so.
+A harness plays the role of data_type_layer::forward_prop / back_prop_impl_
+(src/layers/data_type_layer.cpp:170-275, :292-376): it binds the input
+matrices, sizes the outputs (left uninitialised, as the reference does) and
+calls the hooks.
+
+PyTorch is used for device memory and the HIP stream only; no arithmetic on the
+path is done by torch, and there is no fallback when the library is missing.
+"""
+import functools
+import operator
+
+import numpy as np
+import torch
+
+from . import capi
+from .capi import LBN_STATS_SUMSQ, LBN_STATS_TWO_PASS, LbnError, call  # noqa: F401
+
+
+def _prod(xs):
+    return functools.reduce(operator.mul, xs, 1)
+
+
+class DeviceMatrix:
+    """Column-major matrix in device memory: Height/Width/LDim/Buffer of El::Matrix<T,GPU>.
+
+    Backed by a torch tensor of shape (width, ldim); element (r, c) is tensor[c, r].
+    """
+
+    def __init__(self, height, width, dtype=torch.float32, ldim=None, device="cuda", fill=None):
+        self.height, self.width = int(height), int(width)
+        self.ldim = int(ldim) if ldim is not None else max(self.height, 1)
+        assert self.ldim >= self.height
+        self.tensor = torch.empty((max(self.width, 1), self.ldim), dtype=dtype, device=device)
+        if fill is not None:
+            self.tensor.fill_(fill)
+
+    # El::Matrix vocabulary
+    def Height(self):
+        return self.height
+
+    def Width(self):
+        return self.width
+
+    def LDim(self):
+        return self.ldim
+
+    def Buffer(self):
+        return capi.vp(self.tensor.data_ptr())
+
+    LockedBuffer = Buffer
+
+    @property
+    def dtype(self):
+        return self.tensor.dtype
+
+    @classmethod
+    def from_numpy(cls, a, dtype=None, ldim=None, device="cuda"):
+        """`a` has shape (height, width) (any memory order)."""
+        a = np.asarray(a)
+        h, w = a.shape
+        tdt = dtype or {np.dtype("float32"): torch.float32, np.dtype("float16"): torch.float16,
+                        np.dtype("float64"): torch.float64}[a.dtype]
+        m = cls(h, w, dtype=tdt, ldim=ldim, device=device)
+        if ldim is not None and ldim > h:
+            m.tensor.fill_(float("nan"))  # padding rows must never be read or matter
+        if w > 0 and h > 0:
+            m.tensor[:w, :h] = torch.from_numpy(np.ascontiguousarray(a.T)).to(device=device, dtype=tdt)
+        return m
+
+    def to_numpy(self):
+        """Returns an (height, width) array."""
+        t = self.tensor[: self.width, : self.height]
+        if t.dtype == torch.float16:
+            t = t.float()
+        return np.asfortranarray(t.cpu().numpy().T)
+
+
+class _Vector:
+    """Weights / gradient vector in device memory (fp32)."""
+
+    def __init__(self, n, device="cuda", values=None):
+        if values is None:
+            self.tensor = torch.empty(max(int(n), 1), dtype=torch.float32, device=device)
+        else:
+            self.tensor = torch.as_tensor(np.asarray(values, dtype=np.float32)).to(device).contiguous()
+        self.n = int(n)
+
+    def Buffer(self):
+        return capi.vp(self.tensor.data_ptr())
+
+    def to_numpy(self):
+        return self.tensor[: self.n].cpu().numpy()
+
+
+def _stream():
+    return capi.vp(torch.cuda.current_stream().cuda_stream)
+
+
+def _null():
+    return capi.vp(None)
+
+
+class _Workspace:
+    """Scratch memory owned by a layer, grown on demand (never shrunk)."""
+
+    def __init__(self):
+        self.buf = None
+
+    def get(self, nbytes, device):
+        nbytes = int(nbytes)
+        if nbytes == 0:
+            return _null(), 0
+        if self.buf is None or self.buf.numel() < nbytes:
+            self.buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        return capi.vp(self.buf.data_ptr()), nbytes
+
+
+class _Layer:
+    """Members every data_type_layer hands to its compute hooks."""
+
+    def __init__(self, device="cuda"):
+        self.device = device
+        self.prev_activations = None    # input x
+        self.activations = None         # output y
+        self.prev_error_signals = None  # dL/dy
+        self.error_signals = None       # dL/dx
+        self._ws = _Workspace()
+
+    # what fp_setup_inputs/outputs and bp_setup_gradient_wrt_inputs do
+    def bind_forward(self, x, in_place=False):
+        self.prev_activations = x
+        if in_place:
+            self.activations = x
+        else:
+            self.activations = DeviceMatrix(x.height, x.width, dtype=x.dtype, device=self.device)
+
+    def bind_backward(self, dy, in_place=False):
+        self.prev_error_signals = dy
+        if in_place:
+            self.error_signals = dy
+        else:
+            self.error_signals = DeviceMatrix(dy.height, dy.width, dtype=dy.dtype, device=self.device)
+
+    # fp_call()/bp_call() return (entry point name, argument tuple) of the C-ABI call
+    # that is the body of the reference's fp_compute()/bp_compute().
+    def fp_compute(self):
+        name, args = self.fp_call()
+        call(name, *args)
+
+    def bp_compute(self):
+        name, args = self.bp_call()
+        call(name, *args)
+
+    def forward(self, x, in_place=False):
+        self.bind_forward(x, in_place)
+        self.fp_compute()
+        return self.activations
+
+    def backward(self, dy, in_place=False):
+        self.bind_backward(dy, in_place)
+        self.bp_compute()
+        return self.error_signals
+
+
+class layer_norm_layer(_Layer):
+    """lbann::layer_norm_layer (include/lbann/layers/regularizers/layer_norm.hpp:53-143)."""
+
+    def __init__(self, dims, epsilon=1e-5, scale=False, bias=False, start_dim=0,
+                 scale_values=None, bias_values=None, stats_mode=LBN_STATS_TWO_PASS, device="cuda"):
+        super().__init__(device)
+        self.dims = tuple(int(d) for d in dims)
+        self.m_epsilon, self.m_scale, self.m_bias, self.m_start_dim = float(epsilon), bool(scale), bool(bias), int(start_dim)
+        sd = self.m_start_dim if self.m_start_dim >= 0 else len(self.dims) + self.m_start_dim
+        if sd < 0 or sd >= len(self.dims):
+            raise ValueError(f"layer norm start dimension {start_dim} does not match tensor dimensionality {len(self.dims)}")
+        # get_normdims (layer_norm.hpp:362-405)
+        self.num_normalized = _prod(self.dims[:sd])
+        self.normalization_size = _prod(self.dims[sd:])
+        self.normalization_stride = self.normalization_size
+        n = self.normalization_size
+        self.weights = []
+        if self.m_scale:
+            self.weights.append(_Vector(n, device, scale_values if scale_values is not None else np.ones(n)))
+        if self.m_bias:
+            self.weights.append(_Vector(n, device, bias_values if bias_values is not None else np.zeros(n)))
+        self.m_scale_gradient = _Vector(n, device) if self.m_scale else None
+        self.m_bias_gradient = _Vector(n, device) if self.m_bias else None
+        self.m_statistics = None
+        self.m_statistics_gradient = None
+        self.stats_mode = stats_mode
+
+    def _suffix(self):
+        return "f16" if self.prev_activations.dtype == torch.float16 else "f32"
+
+    def fp_call(self):
+        x, y = self.prev_activations, self.activations
+        G, n = self.num_normalized, self.normalization_size
+        if self.m_statistics is None or self.m_statistics.width != x.width:
+            self.m_statistics = DeviceMatrix(2 * G, x.width, device=self.device)
+        scale = self.weights[0].Buffer() if self.m_scale else _null()
+        bias = self.weights[-1].Buffer() if self.m_bias else _null()
+        return (f"lbn_layer_norm_fwd_{self._suffix()}",
+                (_stream(), G, n, self.normalization_stride, x.width,
+                 self.m_epsilon, x.Buffer(), x.ldim, y.Buffer(), y.ldim, self.m_statistics.Buffer(),
+                 self.m_statistics.ldim, scale, bias, self.stats_mode))
+
+    def bp_call(self):
+        x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
+        G, n = self.num_normalized, self.normalization_size
+        if self.m_statistics_gradient is None or self.m_statistics_gradient.width != x.width:
+            self.m_statistics_gradient = DeviceMatrix(2 * G, x.width, device=self.device)
+        scale = self.weights[0].Buffer() if self.m_scale else _null()
+        dscale = self.m_scale_gradient.Buffer() if self.m_scale else _null()
+        dbias = self.m_bias_gradient.Buffer() if self.m_bias else _null()
+        wgrad = int(self.m_scale or self.m_bias)
+        esize = 2 if x.dtype == torch.float16 else 4
+        ws, nb = self._ws.get(capi.lib().lbn_layer_norm_bwd_workspace_bytes(G, n, x.width, wgrad, esize), self.device)
+        return (f"lbn_layer_norm_bwd_{self._suffix()}",
+                (_stream(), G, n, self.normalization_stride, x.width,
+                 self.m_epsilon, x.Buffer(), x.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim,
+                 self.m_statistics.Buffer(), self.m_statistics.ldim, self.m_statistics_gradient.Buffer(),
+                 self.m_statistics_gradient.ldim, scale, dscale, dbias, ws, nb))
+
+
+class batch_normalization_layer(_Layer):
+    """lbann::batch_normalization_layer (include/lbann/layers/regularizers/batch_normalization.hpp:130-199),
+    local statistics (statistics_group_size == 1)."""
+
+    def __init__(self, dims, decay=0.9, epsilon=1e-5, bessel_correction=True, scale_values=None,
+                 bias_values=None, stats_mode=LBN_STATS_TWO_PASS, device="cuda"):
+        super().__init__(device)
+        self.dims = tuple(int(d) for d in dims)
+        self.m_decay, self.m_epsilon, self.m_bessel_correction = float(decay), float(epsilon), bool(bessel_correction)
+        self.num_channels = self.dims[0]
+        self.channel_size = _prod(self.dims[1:])
+        C = self.num_channels
+        # weights 0..3: scale, bias, running mean, running variance (defaults 1, 0, 0, 1)
+        self.weights = [
+            _Vector(C, device, scale_values if scale_values is not None else np.ones(C)),
+            _Vector(C, device, bias_values if bias_values is not None else np.zeros(C)),
+            _Vector(C, device, np.zeros(C)),
+            _Vector(C, device, np.ones(C)),
+        ]
+        # m_mean_and_var / m_mean_and_var_gradient: C x 2, column 0 mean, column 1 variance
+        self.m_mean_and_var = DeviceMatrix(C, 2, device=device)
+        self.m_mean_and_var_gradient = DeviceMatrix(C, 2, device=device)
+        self.m_scale_gradient = _Vector(C, device)
+        self.m_bias_gradient = _Vector(C, device)
+        self.training = True
+        self.stats_mode = stats_mode
+
+    def _col(self, m, j):
+        return capi.vp(m.tensor.data_ptr() + 4 * j * m.ldim)
+
+    def fp_call(self):
+        x, y = self.prev_activations, self.activations
+        C, cs = self.num_channels, self.channel_size
+        ws, nb = self._ws.get(capi.lib().lbn_batch_norm_workspace_bytes(C, cs, x.width), self.device)
+        return ("lbn_batch_norm_fwd_f32",
+                (_stream(), C, cs, x.width, int(self.m_bessel_correction),
+                 self.m_epsilon, self.m_decay, int(self.training), x.Buffer(), x.ldim, y.Buffer(), y.ldim,
+                 self._col(self.m_mean_and_var, 0), self._col(self.m_mean_and_var, 1),
+                 self.weights[0].Buffer(), self.weights[1].Buffer(), self.weights[2].Buffer(),
+                 self.weights[3].Buffer(), ws, nb, self.stats_mode))
+
+    def bp_call(self):
+        x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
+        C, cs = self.num_channels, self.channel_size
+        ws, nb = self._ws.get(capi.lib().lbn_batch_norm_workspace_bytes(C, cs, x.width), self.device)
+        return ("lbn_batch_norm_bwd_f32",
+                (_stream(), C, cs, x.width, int(self.m_bessel_correction),
+                 self.m_epsilon, int(self.training), x.Buffer(), x.ldim, dy.Buffer(), dy.ldim, dx.Buffer(),
+                 dx.ldim, self._col(self.m_mean_and_var, 0), self._col(self.m_mean_and_var, 1),
+                 self.weights[2].Buffer(), self.weights[3].Buffer(), self.weights[0].Buffer(),
+                 self.m_scale_gradient.Buffer(), self.m_bias_gradient.Buffer(),
+                 self._col(self.m_mean_and_var_gradient, 0), self._col(self.m_mean_and_var_gradient, 1), ws, nb))
+
+
+class _softmax_like(_Layer):
+    _name = None
+
+    def fp_call(self):
+        x, y = self.prev_activations, self.activations
+        ws, nb = self._ws.get(capi.lib().lbn_softmax_workspace_bytes(x.height, x.width), self.device)
+        return (f"lbn_{self._name}_fwd_f32",
+                (_stream(), x.height, x.width, x.Buffer(), x.ldim, y.Buffer(), y.ldim, ws, nb))
+
+    def bp_call(self):
+        y, dy, dx = self.activations, self.prev_error_signals, self.error_signals
+        ws, nb = self._ws.get(capi.lib().lbn_softmax_workspace_bytes(y.height, y.width), self.device)
+        return (f"lbn_{self._name}_bwd_f32",
+                (_stream(), y.height, y.width, y.Buffer(), y.ldim, dy.Buffer(), dy.ldim, dx.Buffer(),
+                 dx.ldim, ws, nb))
+
+
+class softmax_layer(_softmax_like):
+    """lbann::softmax_layer, data-parallel layout, softmax_mode::INSTANCE
+    (include/lbann/layers/activations/softmax.hpp:85-262)."""
+    _name = "softmax"
+
+    def __init__(self, mode="instance", device="cuda"):
+        super().__init__(device)
+        if mode != "instance":
+            # the reference's CPU path rejects every other mode (openmp/softmax.hpp:61-63)
+            raise ValueError("Unsupported softmax mode")
+
+
+class log_softmax_layer(_softmax_like):
+    """lbann::log_softmax_layer (include/lbann/layers/activations/log_softmax.hpp)."""
+    _name = "log_softmax"
+
+
+class channelwise_softmax_layer(_Layer):
+    """lbann::channelwise_softmax_layer (include/lbann/layers/misc/channelwise_softmax.hpp:50-107)."""
+
+    def __init__(self, dims, dim=0, single_dim_mode=False, device="cuda"):
+        super().__init__(device)
+        self.dims = tuple(int(d) for d in dims)
+        nd = len(self.dims)
+        if dim < -nd or dim >= nd:
+            raise ValueError(f"Dimension {dim} is out of bounds for Channelwise Softmax layer on tensor with {nd} dimensions.")
+        if not single_dim_mode and dim not in (0, -nd, nd - 1, -1):
+            raise ValueError("Channelwise softmax with all dimensions is only supported for the first or last tensor dimensions.")
+        self.m_dim, self.m_single_dim_mode = int(dim), bool(single_dim_mode)
+
+    def get_channel_size_and_stride(self):
+        """(channel_size, channel_stride, num_channels), channelwise_softmax_impl.hpp:58-104."""
+        dims = self.dims
+        d = self.m_dim + len(dims) if self.m_dim < 0 else self.m_dim
+        total = _prod(dims)
+        if self.m_single_dim_mode:
+            cs = dims[d]
+            return cs, _prod(dims[d:]), total // cs
+        cs = total // dims[d]
+        return cs, (cs if d == 0 else 1), dims[d]
+
+    def fp_call(self):
+        x, y = self.prev_activations, self.activations
+        cs, stride, C = self.get_channel_size_and_stride()
+        ws, nb = self._ws.get(capi.lib().lbn_channelwise_softmax_workspace_bytes(C, cs, x.width), self.device)
+        return ("lbn_channelwise_softmax_fwd_f32",
+                (_stream(), C, cs, stride, x.width, x.Buffer(), x.ldim, y.Buffer(), y.ldim, ws, nb))
+
+    def bp_call(self):
+        y, dy, dx = self.activations, self.prev_error_signals, self.error_signals
+        cs, stride, C = self.get_channel_size_and_stride()
+        ws, nb = self._ws.get(capi.lib().lbn_channelwise_softmax_workspace_bytes(C, cs, y.width), self.device)
+        return ("lbn_channelwise_softmax_bwd_f32",
+                (_stream(), C, cs, stride, y.width, y.Buffer(), y.ldim, dy.Buffer(), dy.ldim, dx.Buffer(),
+                 dx.ldim, ws, nb))

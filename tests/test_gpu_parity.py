@@ -1,0 +1,415 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle.
+
+Tolerances (max relative error per tensor, tests/parity.py): 1e-5 for fp32,
+2e-3 for fp16 storage with fp32 accumulation.  Where the fp32 reference is itself
+further than that from the float64 evaluation of the same algorithm, a result at
+least as close to float64 as the reference is also accepted (parity.check).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu_oracle as orc
+from tests.parity import TOL_F16, TOL_F32, check, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def L():
+    from lbann_amd import layers
+    layers.capi.lib()  # fail loudly if the library is missing
+    assert torch.cuda.is_available()
+    return layers
+
+
+def f64(a):
+    return np.asfortranarray(np.asarray(a, dtype=np.float64))
+
+
+def f32(a):
+    return np.asfortranarray(np.asarray(a, dtype=np.float32))
+
+
+def rand(rng, h, w, mean=0.0, std=1.0):
+    return np.asfortranarray((rng.standard_normal((w, h)) * std + mean).astype(np.float32).T)
+
+
+# ===================================================================== softmax family
+SM_SHAPES = [
+    # (h, w, ld_pad)   register path: one wave / 256 / 1024 threads per row, all vector counts
+    (64, 5, 0), (256, 9, 0), (1000, 7, 0), (1024, 33, 0), (2048, 6, 0), (4096, 10, 0),
+    (8192, 4, 0), (12288, 3, 0), (32768, 3, 0), (20000, 2, 0),
+    (512, 7, 64),          # ld > height (a view into a taller matrix), still 16-byte aligned
+    (7, 19, 0), (31, 5, 0), (1001, 4, 0), (130, 3, 3),   # unaligned / odd heights: scalar split kernels
+    (32772, 2, 0), (70000, 3, 0), (262144, 2, 0),        # longer than the register path: split kernels
+    (1, 6, 0),
+]
+
+
+def _sm_oracle(kind):
+    return {"softmax": (orc.softmax_fwd, orc.softmax_bwd),
+            "log_softmax": (orc.log_softmax_fwd, orc.log_softmax_bwd)}[kind]
+
+
+@pytest.mark.parametrize("kind", ["softmax", "log_softmax"])
+@pytest.mark.parametrize("h,w,pad", SM_SHAPES)
+def test_softmax_family(L, kind, h, w, pad):
+    rng = np.random.default_rng(h * 1000 + w)
+    x, dy = rand(rng, h, w, 0, 2), rand(rng, h, w)
+    if h > 8:
+        x[rng.integers(0, h, size=max(1, h // 100)), :] = 30.0
+    fwd, bwd = _sm_oracle(kind)
+    layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
+    ld = h + pad
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=ld)).to_numpy()
+    y_ref, y_ex = fwd(x), fwd(f64(x))
+    check(f"{kind} y {h}x{w}", y, y_ref, y_ex)
+    # backward consumes the layer's own output, as in the framework
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=ld)).to_numpy()
+    check(f"{kind} dx {h}x{w}", dx, bwd(f32(y), dy), bwd(f64(y), f64(dy)))
+
+
+@pytest.mark.parametrize("kind", ["softmax", "log_softmax", "channelwise"])
+@pytest.mark.parametrize("h,w", [(4096, 6), (777, 5), (70000, 2)])
+def test_softmax_family_in_place(L, kind, h, w):
+    rng = np.random.default_rng(h + w)
+    x, dy = rand(rng, h, w, 0, 2), rand(rng, h, w)
+    if kind == "channelwise":
+        C = 7 if h == 777 else 4
+        layer = L.channelwise_softmax_layer((C, h // C))
+        y_ref = orc.channelwise_softmax_fwd(x, C, h // C, h // C)
+        bwd = lambda y, g: orc.channelwise_softmax_bwd(y, g, C, h // C, h // C)
+    else:
+        layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
+        y_ref = _sm_oracle(kind)[0](x)
+        bwd = _sm_oracle(kind)[1]
+    xm = L.DeviceMatrix.from_numpy(x)
+    ym = layer.forward(xm, in_place=True)
+    assert ym is xm
+    y = ym.to_numpy()
+    check(f"{kind} in-place y", y, y_ref, None, tol=TOL_F32)
+    gm = L.DeviceMatrix.from_numpy(dy)
+    dm = layer.backward(gm, in_place=True)
+    assert dm is gm
+    check(f"{kind} in-place dx", dm.to_numpy(), bwd(f32(y), dy), bwd(f64(y), f64(dy)))
+
+
+def test_softmax_special_values(L):
+    x = np.zeros((8, 5), dtype=np.float32, order="F")
+    x[1, 0] = -95.0                       # denormal after exp -> flushed to 0 by softmax
+    x[2, 0] = -200.0
+    x[:, 1] = [50, -45, 50, -41, 0, 0, 0, 0]
+    x[:, 2] = np.nan                      # NaN column -> all zeros (nothing is a normal float)
+    x[:, 3] = -np.inf                     # max stays at -FLT_MAX, exp(-inf) = 0, 0 * inf = NaN -> 0
+    x[3, 4] = np.inf                      # inf - inf = NaN at the maximum itself
+    for kind, layer in (("softmax", L.softmax_layer()), ("log_softmax", L.log_softmax_layer())):
+        y = layer.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+        ref = _sm_oracle(kind)[0](x)
+        assert rel_err(y, ref) <= TOL_F32, kind
+    # channelwise keeps denormals (no flush)
+    xc = np.asfortranarray(x[:, :1])
+    y = L.channelwise_softmax_layer((1, 8)).forward(L.DeviceMatrix.from_numpy(xc)).to_numpy()
+    ref = orc.channelwise_softmax_fwd(xc, 1, 8, 8)
+    assert 0 < y[1, 0] < np.finfo(np.float32).tiny
+    assert rel_err(y, ref) <= TOL_F32
+
+
+CWS_CASES = [
+    # dims, dim, single_dim_mode, width
+    ((5, 2, 7), 0, False, 15), ((5, 2, 7), -1, True, 15), ((64, 256), 0, False, 9),
+    ((4, 8, 128), -1, True, 3), ((16, 4096), 0, False, 3), ((3, 40000), 0, False, 2),
+    ((6, 10), 0, False, 4),
+]
+
+
+@pytest.mark.parametrize("dims,dim,single,w", CWS_CASES)
+def test_channelwise_softmax(L, dims, dim, single, w):
+    rng = np.random.default_rng(sum(dims) + w)
+    h = int(np.prod(dims))
+    x, dy = rand(rng, h, w, 0.5, 1.0), rand(rng, h, w)
+    layer = L.channelwise_softmax_layer(dims, dim=dim, single_dim_mode=single)
+    cs, stride, C = layer.get_channel_size_and_stride()
+    y = layer.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    check("cws y", y, orc.channelwise_softmax_fwd(x, C, cs, stride), orc.channelwise_softmax_fwd(f64(x), C, cs, stride))
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+    check("cws dx", dx, orc.channelwise_softmax_bwd(f32(y), dy, C, cs, stride),
+          orc.channelwise_softmax_bwd(f64(y), f64(dy), C, cs, stride))
+
+
+# ===================================================================== layer norm
+LN_CASES = [
+    # dims, start_dim, width, affine, ld_pad
+    ((1024,), 0, 128, True, 0), ((1024,), 0, 128, False, 0), ((256,), 0, 7, True, 0),
+    ((64,), 0, 300, True, 0), ((4096,), 0, 40, True, 0), ((8192,), 0, 5, True, 0),
+    ((16384,), 0, 3, True, 0), ((32768,), 0, 2, False, 0), ((40000,), 0, 2, True, 0),
+    ((31,), 0, 15, True, 0), ((31, 2, 5), -1, 9, True, 0), ((31, 2, 5), 1, 9, True, 0),
+    ((8, 512), -1, 33, True, 0), ((8, 512), 0, 6, True, 0), ((16, 64), 1, 700, True, 0),
+    ((512,), 0, 6, True, 32), ((100,), 0, 6, True, 3), ((2048,), 0, 2000, True, 0),
+    ((5, 1), -1, 4, False, 0),
+]
+
+
+def _ln_run(L, x, dy, dims, start_dim, affine, pad, scale, bias, mode=None, tol=TOL_F32, half=False):
+    h, w = x.shape
+    kw = dict(scale_values=scale, bias_values=bias) if affine else {}
+    if mode is not None:
+        kw["stats_mode"] = mode
+    layer = L.layer_norm_layer(dims, 1e-5, affine, affine, start_dim, **kw)
+    G, n = layer.num_normalized, layer.normalization_size
+    tdt = torch.float16 if half else torch.float32
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, dtype=tdt, ldim=h + pad)).to_numpy()
+    stats = layer.m_statistics.to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, dtype=tdt, ldim=h + pad)).to_numpy()
+    sgrad = layer.m_statistics_gradient.to_numpy()
+    out = dict(y=y, stats=stats, dx=dx, sgrad=sgrad)
+    if affine:
+        out["dscale"] = layer.m_scale_gradient.to_numpy()
+        out["dbias"] = layer.m_bias_gradient.to_numpy()
+    g = scale if affine else None
+    b = bias if affine else None
+    ref, ex = {}, {}
+    for dst, conv in ((ref, f32), (ex, f64)):
+        xx, gg = conv(x), conv(dy)
+        sc = None if g is None else conv(g)
+        bi = None if b is None else conv(b)
+        dst["y"], dst["stats"] = orc.layer_norm_fwd(xx, G, n, n, 1e-5, sc, bi)
+        dst["dx"], dst["sgrad"], dst["dscale"], dst["dbias"] = orc.layer_norm_bwd(
+            xx, gg, dst["stats"], G, n, n, 1e-5, sc, affine, affine)
+    if n <= 1:
+        out.pop("sgrad"); ref.pop("sgrad")   # left untouched by the reference in this case
+    res = {}
+    for k in out:
+        res[k] = check(f"layer_norm {k} dims={dims} w={w}", out[k], ref[k], ex[k], tol=tol)
+    return res
+
+
+@pytest.mark.parametrize("dims,start_dim,w,affine,pad", LN_CASES)
+def test_layer_norm_f32(L, dims, start_dim, w, affine, pad):
+    rng = np.random.default_rng(int(np.prod(dims)) + w)
+    h = int(np.prod(dims))
+    x, dy = rand(rng, h, w, 0.3, 1.5), rand(rng, h, w)
+    n = int(np.prod(dims[(start_dim if start_dim >= 0 else len(dims) + start_dim):]))
+    scale = (1 + 0.3 * rng.standard_normal(n)).astype(np.float32)
+    bias = (0.3 * rng.standard_normal(n)).astype(np.float32)
+    _ln_run(L, x, dy, dims, start_dim, affine, pad, scale, bias)
+
+
+@pytest.mark.parametrize("dims,start_dim,w", [((1024,), 0, 64), ((31,), 0, 15), ((8, 512), -1, 9)])
+def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
+    """E[x^2]-mean^2 mode reproduces the reference's variance, clamp included."""
+    rng = np.random.default_rng(5)
+    h = int(np.prod(dims))
+    x, dy = rand(rng, h, w, 3.0, 0.5), rand(rng, h, w)
+    x[:, 0] = 7.0   # constant column: the clamp at zero decides the variance
+    _ln_run(L, x, dy, dims, start_dim, False, 0, None, None, mode=L.LBN_STATS_SUMSQ)
+
+
+@pytest.mark.parametrize("dims,start_dim,w,pad", [((4096,), 0, 64, 0), ((512,), 0, 100, 0), ((64,), 0, 9, 0),
+                                                   ((8, 1024), -1, 5, 0), ((100,), 0, 7, 0), ((2048,), 0, 600, 8),
+                                                   ((16384,), 0, 3, 0)])
+def test_layer_norm_f16(L, dims, start_dim, w, pad):
+    rng = np.random.default_rng(int(np.prod(dims)) * 3 + w)
+    h = int(np.prod(dims))
+    x = rand(rng, h, w, 0.3, 1.5).astype(np.float16).astype(np.float32)
+    dy = rand(rng, h, w).astype(np.float16).astype(np.float32)
+    n = int(np.prod(dims[(start_dim if start_dim >= 0 else len(dims) + start_dim):]))
+    scale = (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(n)).astype(np.float32)
+    _ln_run(L, x, dy, dims, start_dim, True, pad, scale, bias, tol=TOL_F16, half=True)
+
+
+# ===================================================================== batch norm
+BN_CASES = [
+    # dims (C, ...), width, bessel, ld_pad
+    ((7, 5, 3), 14, True, 0), ((7, 5, 3), 29, False, 0), ((8, 16, 16), 12, True, 0),
+    ((256, 4, 4), 32, True, 0), ((3, 56, 56), 16, True, 0), ((16, 28, 28), 8, False, 0),
+    ((5, 12), 10, True, 4), ((5, 13), 10, True, 0), ((2, 1), 1, True, 0), ((1, 100000), 3, True, 0),
+    ((70, 1), 50, True, 0),
+]
+
+
+def _bn_run(L, x, dy, dims, bessel, pad, scale, bias, mode=None, training=True):
+    h, w = x.shape
+    C = dims[0]
+    cs = h // C
+    kw = {} if mode is None else {"stats_mode": mode}
+    layer = L.batch_normalization_layer(dims, 0.9, 1e-5, bessel, scale, bias, **kw)
+    layer.training = training
+    rm0 = (0.1 * np.arange(C)).astype(np.float32)
+    rv0 = (1.0 + 0.05 * np.arange(C)).astype(np.float32)
+    layer.weights[2].tensor[:C] = torch.from_numpy(rm0).cuda()
+    layer.weights[3].tensor[:C] = torch.from_numpy(rv0).cuda()
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    mv = layer.m_mean_and_var.to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    mvg = layer.m_mean_and_var_gradient.to_numpy()
+    out = dict(y=y, dx=dx, dscale=layer.m_scale_gradient.to_numpy(), dbias=layer.m_bias_gradient.to_numpy(),
+               dmean=mvg[:, 0], dvar=mvg[:, 1], rmean=layer.weights[2].to_numpy(), rvar=layer.weights[3].to_numpy())
+    if training:
+        out.update(mean=mv[:, 0], var=mv[:, 1])
+    ref, ex = {}, {}
+    for dst, conv in ((ref, f32), (ex, f64)):
+        xx, gg, sc, bi = conv(x), conv(dy), conv(scale), conv(bias)
+        rm, rv = conv(rm0).copy(), conv(rv0).copy()
+        dst["y"], dst["mean"], dst["var"] = orc.batch_norm_fwd(xx, C, cs, 1e-5, 0.9, sc, bi, rm, rv, bessel, training)
+        dst["rmean"], dst["rvar"] = rm, rv
+        dst["dx"], dst["dscale"], dst["dbias"], dst["dmean"], dst["dvar"] = orc.batch_norm_bwd(
+            xx, gg, C, cs, 1e-5, dst["mean"], dst["var"], sc, rm, rv, bessel, training)
+    return {k: check(f"batch_norm {k} dims={dims} w={w}", out[k], ref[k], ex[k]) for k in out}
+
+
+@pytest.mark.parametrize("dims,w,bessel,pad", BN_CASES)
+def test_batch_norm(L, dims, w, bessel, pad):
+    rng = np.random.default_rng(int(np.prod(dims)) + w)
+    h = int(np.prod(dims))
+    x, dy = rand(rng, h, w, 2.0, 3.0), rand(rng, h, w)
+    C = dims[0]
+    scale = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    _bn_run(L, x, dy, dims, bessel, pad, scale, bias)
+
+
+def test_batch_norm_inference_and_reference_formula(L):
+    rng = np.random.default_rng(77)
+    dims, w = (6, 10, 10), 9
+    h = int(np.prod(dims))
+    x, dy = rand(rng, h, w, 2.0, 3.0), rand(rng, h, w)
+    x[:100, :] = 4.0    # constant channel: variance is lifted to epsilon
+    scale = rng.uniform(0.5, 1.5, 6).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(6)).astype(np.float32)
+    _bn_run(L, x, dy, dims, True, 0, scale, bias, training=False)
+    _bn_run(L, x, dy, dims, True, 0, scale, bias, mode=L.LBN_STATS_SUMSQ)
+    _bn_run(L, x, dy, dims, True, 0, scale, bias)
+
+
+def test_batch_norm_split_entry_points(L):
+    """sums -> stats -> apply (the cut where a caller all-reduces) equals the fused call."""
+    from lbann_amd import capi
+    rng = np.random.default_rng(78)
+    C, cs, w = 12, 64, 10
+    h = C * cs
+    x, dy = rand(rng, h, w, 2.0, 3.0), rand(rng, h, w)
+    scale = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    xm, gm = L.DeviceMatrix.from_numpy(x), L.DeviceMatrix.from_numpy(dy)
+    ym, dm = L.DeviceMatrix(h, w), L.DeviceMatrix(h, w)
+    dev = lambda a: torch.from_numpy(np.asarray(a, np.float32)).cuda()
+    p = lambda t: capi.vp(t.data_ptr())
+    mean, var, rm, rv = torch.empty(C).cuda(), torch.empty(C).cuda(), torch.zeros(C).cuda(), torch.ones(C).cuda()
+    sc, bi = dev(scale), dev(bias)
+    nb = capi.lib().lbn_batch_norm_workspace_bytes(C, cs, w)
+    ws = torch.empty(max(nb, 1), dtype=torch.uint8, device="cuda")
+    st = capi.vp(torch.cuda.current_stream().cuda_stream)
+    capi.call("lbn_batch_norm_fwd_sums_f32", st, C, cs, w, xm.Buffer(), xm.ldim, p(mean), p(var), p(ws), nb)
+    sums = mean.cpu().numpy().copy()
+    assert rel_err(sums, x.astype(np.float64).reshape(cs, C, w, order="F").sum(axis=(0, 2))) < 1e-5
+    capi.call("lbn_batch_norm_fwd_stats_f32", st, C, cs * w, 1, 1e-5, 0.9, p(mean), p(var), p(rm), p(rv))
+    capi.call("lbn_batch_norm_fwd_apply_f32", st, C, cs, w, 1e-5, xm.Buffer(), xm.ldim, ym.Buffer(), ym.ldim,
+              p(mean), p(var), p(sc), p(bi))
+    rm0, rv0 = np.zeros(C, np.float32), np.ones(C, np.float32)
+    y_ref, mean_ref, var_ref = orc.batch_norm_fwd(x, C, cs, 1e-5, 0.9, scale, bias, rm0, rv0)
+    check("split y", ym.to_numpy(), y_ref, None)
+    check("split mean", mean.cpu().numpy(), mean_ref, None)
+    check("split var", var.cpu().numpy(), var_ref, None)
+    check("split rmean", rm.cpu().numpy(), rm0, None)
+    check("split rvar", rv.cpu().numpy(), rv0, None)
+    ds, db, dmn, dvr = (torch.empty(C).cuda() for _ in range(4))
+    capi.call("lbn_batch_norm_bwd_sums_f32", st, C, cs, w, 1e-5, xm.Buffer(), xm.ldim, gm.Buffer(), gm.ldim,
+              p(mean), p(var), p(sc), p(ds), p(db), p(dmn), p(dvr), p(ws), nb)
+    capi.call("lbn_batch_norm_bwd_apply_f32", st, C, cs, w, cs * w, 1, 1e-5, xm.Buffer(), xm.ldim, gm.Buffer(),
+              gm.ldim, dm.Buffer(), dm.ldim, p(mean), p(var), p(sc), p(dmn), p(dvr))
+    dx_ref, dg_ref, db_ref, dm_ref, dv_ref = orc.batch_norm_bwd(x, dy, C, cs, 1e-5, mean_ref, var_ref, scale)
+    ex = orc.batch_norm_bwd(f64(x), f64(dy), C, cs, 1e-5, f64(mean_ref), f64(var_ref), f64(scale))
+    check("split dx", dm.to_numpy(), dx_ref, ex[0])
+    check("split dscale", ds.cpu().numpy(), dg_ref, ex[1])
+    check("split dbias", db.cpu().numpy(), db_ref, ex[2])
+    check("split dmean", dmn.cpu().numpy(), dm_ref, ex[3])
+    check("split dvar", dvr.cpu().numpy(), dv_ref, ex[4])
+
+
+# ===================================================================== golden fixtures on the GPU
+def test_reference_fixtures_on_gpu(L, golden):
+    F32_EPS = np.finfo(np.float32).eps
+    met = lambda y: float(np.mean(np.sum(np.asarray(y, np.float64) ** 2, axis=0)))
+    T = lambda a: np.asfortranarray(np.asarray(a).T)
+    y = L.layer_norm_layer((31,)).forward(L.DeviceMatrix.from_numpy(T(golden["ln_x"]))).to_numpy()
+    assert abs(met(y) - float(golden["ln_metric"])) <= 8 * float(golden["ln_metric"]) * F32_EPS
+    assert rel_err(y.T, golden["ln_y"]) < TOL_F32
+    ln = L.layer_norm_layer((31,), scale=True, bias=True, scale_values=golden["lna_scale"], bias_values=golden["lna_bias"])
+    y = ln.forward(L.DeviceMatrix.from_numpy(T(golden["lna_x"]))).to_numpy()
+    assert np.mean((y.T - golden["lna_y_test_scaled_bias"]) ** 2) <= 1e-8
+    assert rel_err(y.T, golden["lna_y_exact"]) < TOL_F32
+    for sd in (-1, 1, 0):
+        y = L.layer_norm_layer((31, 2, 5), start_dim=sd).forward(
+            L.DeviceMatrix.from_numpy(T(golden["lnm_x"].reshape(31, -1)))).to_numpy()
+        assert np.mean((y.T - golden[f"lnm_y_test_sd{sd}"].reshape(31, -1)) ** 2) <= 1e-7
+        assert rel_err(y.T, golden[f"lnm_y_exact_sd{sd}"].reshape(31, -1)) < TOL_F32
+    for tag, rows in (("mb14", 14), ("all29", 29)):
+        for bessel in (0, 1):
+            bn = L.batch_normalization_layer((7, 5, 3), bessel_correction=bool(bessel))
+            y = bn.forward(L.DeviceMatrix.from_numpy(T(golden["bn_x"][:rows]))).to_numpy()
+            assert rel_err(y.T, golden[f"bn_{tag}_b{bessel}_y"]) < TOL_F32
+            mv = bn.m_mean_and_var.to_numpy()
+            assert rel_err(mv[:, 0], golden[f"bn_{tag}_b{bessel}_mean"]) < TOL_F32
+            assert rel_err(mv[:, 1], golden[f"bn_{tag}_b{bessel}_var"]) < TOL_F32
+    y = L.softmax_layer().forward(L.DeviceMatrix.from_numpy(T(golden["sm_x"]))).to_numpy()
+    assert abs(met(y) - float(golden["sm_metric"])) <= 8 * float(golden["sm_metric"]) * F32_EPS
+    assert rel_err(y.T, golden["sm_y"]) < TOL_F32
+    y = L.log_softmax_layer().forward(L.DeviceMatrix.from_numpy(T(golden["lsm_x"]))).to_numpy()
+    assert abs(met(y) - float(golden["lsm_metric"])) <= 8 * float(golden["lsm_metric"]) * F32_EPS
+    assert rel_err(y.T, golden["lsm_y"]) < TOL_F32
+    for tag, kw in (("default", {}), ("lastdim", dict(dim=-1, single_dim_mode=True))):
+        y = L.channelwise_softmax_layer((5, 2, 7), **kw).forward(L.DeviceMatrix.from_numpy(T(golden["cws_x"]))).to_numpy()
+        assert abs(met(y) - float(golden[f"cws_metric_{tag}"])) <= 8 * float(golden[f"cws_metric_{tag}"]) * F32_EPS
+        assert rel_err(y.T, golden[f"cws_y_{tag}"]) < TOL_F32
+
+
+# ===================================================================== boundary behaviour
+def test_empty_and_rejected_arguments(L):
+    from lbann_amd import capi
+    st = capi.vp(torch.cuda.current_stream().cuda_stream)
+    null = capi.vp(None)
+    lib = capi.lib()
+    buf = torch.zeros(64, device="cuda")
+    p = capi.vp(buf.data_ptr())
+    # empty inputs: success, nothing launched, no pointer touched
+    assert lib.lbn_softmax_fwd_f32(st, 0, 5, null, 0, null, 0, null, 0) == 0
+    assert lib.lbn_softmax_fwd_f32(st, 8, 0, null, 8, null, 8, null, 0) == 0
+    assert lib.lbn_layer_norm_fwd_f32(st, 1, 8, 8, 0, 1e-5, null, 8, null, 8, null, 2, null, null, 0) == 0
+    assert lib.lbn_batch_norm_fwd_f32(st, 0, 4, 4, 1, 1e-5, 0.9, 1, null, 0, null, 0, null, null, null, null, null, null, null, 0, 0) == 0
+    assert lib.lbn_channelwise_softmax_bwd_f32(st, 4, 0, 0, 3, null, 0, null, 0, null, 0, null, 0) == 0
+    # rejected arguments come back as negative status codes, never as a fault
+    assert lib.lbn_softmax_fwd_f32(st, -1, 5, p, 8, p, 8, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_softmax_fwd_f32(st, 8, 2, p, 4, p, 8, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT   # ld < height
+    assert lib.lbn_softmax_fwd_f32(st, 8, 2, null, 8, p, 8, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_softmax_fwd_f32(st, 7, 2, p, 7, p, 7, null, 0) == capi.LBN_ERR_WORKSPACE          # split path needs scratch
+    assert lib.lbn_batch_norm_fwd_f32(st, 2, 4, 2, 1, 1e-5, 0.9, 1, p, 8, p, 8, p, p, p, p, p, p, null, 0, 0) == capi.LBN_ERR_WORKSPACE
+    assert lib.lbn_layer_norm_bwd_f32(st, 1, 8, 8, 2, 1e-5, p, 8, p, 8, p, 8, p, 2, p, 2, null, p, null, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert b"workspace" in lib.lbn_status_string(capi.LBN_ERR_WORKSPACE)
+    with pytest.raises(L.LbnError):
+        capi.call("lbn_softmax_fwd_f32", st, -1, 5, p, 8, p, 8, null, 0)
+    with pytest.raises(ValueError):
+        L.softmax_layer(mode="channel")
+    with pytest.raises(ValueError):
+        L.layer_norm_layer((4, 4), start_dim=2)
+    torch.cuda.synchronize()
+
+
+def test_results_are_bitwise_reproducible(L):
+    """No atomics anywhere: two runs give identical bits (also a cheap race detector)."""
+    rng = np.random.default_rng(99)
+    x, dy = rand(rng, 4096, 300), rand(rng, 4096, 300)
+    scale = (1 + 0.1 * rng.standard_normal(4096)).astype(np.float32)
+    outs = []
+    for _ in range(2):
+        ln = L.layer_norm_layer((4096,), scale=True, bias=True, scale_values=scale, bias_values=scale)
+        ln.forward(L.DeviceMatrix.from_numpy(x))
+        ln.backward(L.DeviceMatrix.from_numpy(dy))
+        bn = L.batch_normalization_layer((16, 256))
+        yb = bn.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+        db = bn.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+        outs.append([ln.error_signals.to_numpy(), ln.m_scale_gradient.to_numpy(), ln.m_bias_gradient.to_numpy(),
+                     yb, db, bn.m_scale_gradient.to_numpy()])
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b)
