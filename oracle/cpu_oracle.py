@@ -47,8 +47,9 @@ def _suffix(a):
 
 def _mat(a):
     """(pointer, leading dimension) of a column-major 2-D array."""
-    assert a.ndim == 2 and a.strides[0] == a.itemsize, "matrix must be column-major"
+    assert a.ndim == 2 and (a.strides[0] == a.itemsize or a.shape[0] <= 1), "matrix must be column-major"
     ld = a.strides[1] // a.itemsize if a.shape[1] > 1 else max(a.shape[0], 1)
+    assert ld >= a.shape[0]
     return _vp(a.ctypes.data), _i64(ld)
 
 
