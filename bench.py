@@ -31,6 +31,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", default="all", help="all | headline | comma list of cfg names")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also time a plain elementwise copy of 256 MiB (torch kernel): the practical "
+                         "streaming ceiling, and the known-size kernel that scales the rocprof byte counters")
     return ap.parse_args()
 
 
@@ -206,6 +209,24 @@ def main():
         del layer
         torch.cuda.empty_cache()
 
+    copy_cal = None
+    if args.copy_calibration:
+        n = 64 * 1024 * 1024
+        src = torch.randn(n, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        evs = [(ev(), ev()) for _ in range(20)]
+        for a, b in evs:
+            a.record()
+            torch.mul(src, 1.0, out=dst)
+            b.record()
+        torch.cuda.synchronize()
+        ms = statistics.mean(a.elapsed_time(b) for a, b in evs)
+        copy_cal = {"bytes_read": 4 * n, "bytes_written": 4 * n, "ms": ms, "gbs": 8 * n / (ms * 1e-3) / 1e9}
+        print(f"# copy 256 MiB -> 256 MiB: {ms*1e3:.1f} us, {copy_cal['gbs']:.0f} GB/s", file=sys.stderr)
+
     h = results[headline]
     # dominant kernel of the headline step: the backward row kernel (3 tensors vs 2)
     dom_bytes = h["algorithmic_bytes"]["bwd"]
@@ -230,6 +251,8 @@ def main():
                      "bytes_per_launch": dom_bytes, "avg_launch_ms": h["bwd_ms"], "traffic": None},
         "layers": results,
     }
+    if copy_cal:
+        out["copy_calibration"] = copy_cal
     if "cpu" in h:
         out["cpu_baseline"] = {"value": h["cpu"]["gbs"], "unit": "GB/s", "cores": h["cpu"]["threads"],
                                "kind": "port",

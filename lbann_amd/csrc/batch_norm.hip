@@ -13,6 +13,7 @@
 // entry), sum(x-K) and sum((x-K)^2), which removes the cancellation of
 // E[x^2]-mean^2 when |mean| >> stdev at no extra cost; LBN_STATS_SUMSQ selects
 // K = 0, the reference's formula (batch_normalization.cpp:70-85, :124-128).
+#include "cluster_sync.hpp"
 #include "device_utils.hpp"
 #include "host_utils.hpp"
 
@@ -332,6 +333,334 @@ bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ dy, float* _
   }
 }
 
+
+// ===================================================== register-resident clusters
+// A channel (E = cs/4 * w vectors) is shared by a cluster of M workgroups of T
+// threads; workgroup k keeps vectors [k*T*V, (k+1)*T*V) in registers.  The grid is
+// persistent: cluster cl handles channels cl, cl + nclusters, ...
+//
+// The loop rotates three register tiles so that nothing waits on something issued
+// in the same step: in step s a workgroup (1) reduces tile s+1, whose loads were
+// issued a step earlier, and publishes its partial sums, (2) issues the loads of
+// tile s+2, (3) collects the cluster's partials of tile s, published a step
+// earlier, and finishes tile s from registers.  Loads, the rendezvous latency and
+// stores of different channels overlap; every tensor crosses HBM once.
+template <int V>
+struct BnIndex {
+  unsigned col[V], pos[V];
+  bool ok[V];
+};
+
+template <int T, int V>
+__device__ __forceinline__ BnIndex<V> bn_make_index(int k, unsigned seg, unsigned E)
+{
+  BnIndex<V> ix;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned e = static_cast<unsigned>(k) * (T * V) + i * T + threadIdx.x;
+    ix.ok[i] = e < E;
+    ix.col[i] = e / seg;
+    ix.pos[i] = e - ix.col[i] * seg;
+  }
+  return ix;
+}
+
+template <int V>
+__device__ __forceinline__ void bn_tile_load(float (&t)[V][4], const float* base, int64_t ld,
+                                             const BnIndex<V>& ix)
+{
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    if (ix.ok[i]) {
+      Vec16<float>::load(base + static_cast<int64_t>(ix.col[i]) * ld + 4 * static_cast<int64_t>(ix.pos[i]), t[i]);
+    }
+    else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t[i][j] = 0.f;
+    }
+  }
+}
+
+template <int V>
+__device__ __forceinline__ void bn_tile_store(const float (&t)[V][4], float* base, int64_t ld,
+                                              const BnIndex<V>& ix)
+{
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+    if (ix.ok[i])
+      Vec16<float>::store(base + static_cast<int64_t>(ix.col[i]) * ld + 4 * static_cast<int64_t>(ix.pos[i]), t[i]);
+}
+
+struct BnFwdArgs {
+  const float* x;
+  float* y;
+  int64_t ldx, ldy, cs;
+  int C, M, use_pivot, bessel;
+  float eps, decay;
+  int64_t n;
+  ClusterWorkspace cw;
+  float* mean_out;
+  float* var_out;
+  const float* gamma;
+  const float* beta;
+  float* rmean;
+  float* rvar;
+};
+
+// A register tile: a workgroup's share of one channel plus the channel's scalars,
+// all loaded at the same point of the pipeline so that no step waits on a load it
+// issued itself.
+template <int V>
+struct BnFwdTile {
+  float v[V][4];
+  float K, scale, bias;
+};
+
+template <int V>
+__device__ __forceinline__ void bn_fwd_load(BnFwdTile<V>& t, const BnFwdArgs& a, int ch,
+                                            const BnIndex<V>& ix)
+{
+  const float* xc = a.x + static_cast<int64_t>(ch) * a.cs;
+  bn_tile_load<V>(t.v, xc, a.ldx, ix);
+  t.K = a.use_pivot ? xc[0] : 0.f;
+  t.scale = a.gamma[ch];
+  t.bias = a.beta[ch];
+}
+
+// (1) of a step: partial sums of channel `ch` from tile `t`, published for the cluster.
+template <int T, int V>
+__device__ __forceinline__ void bn_fwd_reduce(const BnFwdArgs& a, const BnIndex<V>& ix, int ch, int k,
+                                              const BnFwdTile<V>& t, float* red)
+{
+  const unsigned tid = threadIdx.x;
+  const float K = t.K;
+  float s = 0.f, q = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float d = ix.ok[i] ? t.v[i][j] - K : 0.f;
+      s += d;
+      q += d * d;
+    }
+  }
+  team_sum2<T / kWave>(s, q, red, tid / kWave, tid & (kWave - 1));
+  if (tid == 0) cluster_publish(s, q, a.cw.slots + static_cast<int64_t>(ch) * a.M, k);
+}
+
+// (3) of a step: statistics of channel `ch` from the cluster's partials, output from tile `t`.
+template <int T, int V>
+__device__ __forceinline__ void bn_fwd_finish(const BnFwdArgs& a, const BnIndex<V>& ix, int ch, int k,
+                                              BnFwdTile<V>& t, float* bc)
+{
+  const unsigned tid = threadIdx.x;
+  if (tid < kWave) {
+    float ts, tq;
+    cluster_collect(a.cw.slots + static_cast<int64_t>(ch) * a.M, a.M, a.cw.error, 0.f, 0.f, ts, tq);
+    ts = wave_sum(ts);
+    tq = wave_sum(tq);
+    if (tid == 0) {
+      float mean, var;
+      stats_from_sums(ts, tq, t.K, a.n, a.bessel, a.eps, mean, var);
+      bc[0] = mean;
+      bc[1] = 1.0f / sqrtf(var + a.eps);
+      if (k == 0) {
+        a.mean_out[ch] = mean;
+        a.var_out[ch] = var;
+        a.rmean[ch] = a.decay * a.rmean[ch] + (1.f - a.decay) * mean;
+        a.rvar[ch] = a.decay * a.rvar[ch] + (1.f - a.decay) * var;
+      }
+    }
+  }
+  __syncthreads();
+  const float mean = bc[0];
+  const float inv_stdev = bc[1];
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t.v[i][j] = t.scale * ((t.v[i][j] - mean) * inv_stdev) + t.bias;
+  bn_tile_store<V>(t.v, a.y + static_cast<int64_t>(ch) * a.cs, a.ldy, ix);
+}
+
+// One step of the rotation: F finishes channel ch, R holds channel ch + nc, L
+// receives channel ch + 2 nc.
+template <int T, int V>
+__device__ __forceinline__ void bn_fwd_step(const BnFwdArgs& a, const BnIndex<V>& ix, int ch, int nc, int k,
+                                            BnFwdTile<V>& F, BnFwdTile<V>& R, BnFwdTile<V>& L,
+                                            float* red, float* bc)
+{
+  if (ch + nc < a.C) bn_fwd_reduce<T, V>(a, ix, ch + nc, k, R, red);
+  if (ch + 2 * nc < a.C) bn_fwd_load<V>(L, a, ch + 2 * nc, ix);
+  asm volatile("" ::: "memory");  // keep the loads above the wait below
+  bn_fwd_finish<T, V>(a, ix, ch, k, F, bc);
+}
+
+template <int T, int V>
+__global__ void __launch_bounds__(T)
+bn_fwd_cluster(BnFwdArgs a, unsigned seg, unsigned E)
+{
+  __shared__ float red[2 * (T / kWave)];
+  __shared__ float bc[2];
+  const int nc = gridDim.x / a.M;
+  const int cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - cl * a.M;
+  const BnIndex<V> ix = bn_make_index<T, V>(k, seg, E);
+  BnFwdTile<V> t0, t1, t2;
+  if (cl >= a.C) return;
+  bn_fwd_load<V>(t0, a, cl, ix);
+  if (cl + nc < a.C) bn_fwd_load<V>(t1, a, cl + nc, ix);
+  bn_fwd_reduce<T, V>(a, ix, cl, k, t0, red);
+  for (int ch = cl; ch < a.C; ch += 3 * nc) {
+    bn_fwd_step<T, V>(a, ix, ch, nc, k, t0, t1, t2, red, bc);
+    if (ch + nc < a.C) bn_fwd_step<T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, red, bc);
+    if (ch + 2 * nc < a.C) bn_fwd_step<T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, red, bc);
+  }
+}
+
+struct BnBwdArgs {
+  const float* x;
+  const float* dy;
+  float* dx;
+  int64_t ldx, lddy, lddx, cs;
+  int C, M, bessel;
+  float eps;
+  int64_t n;
+  ClusterWorkspace cw;
+  const float* mean_in;
+  const float* var_in;
+  const float* gamma;
+  float* dscale;
+  float* dbias;
+  float* dmean_out;
+  float* dvar_out;
+};
+
+template <int V>
+struct BnBwdTile {
+  float x[V][4];
+  float g[V][4];
+  float mean, var, scale;
+};
+
+template <int V>
+__device__ __forceinline__ void bn_bwd_load(BnBwdTile<V>& t, const BnBwdArgs& a, int ch,
+                                            const BnIndex<V>& ix)
+{
+  bn_tile_load<V>(t.x, a.x + static_cast<int64_t>(ch) * a.cs, a.ldx, ix);
+  bn_tile_load<V>(t.g, a.dy + static_cast<int64_t>(ch) * a.cs, a.lddy, ix);
+  t.mean = a.mean_in[ch];
+  t.var = a.var_in[ch];
+  t.scale = a.gamma[ch];
+}
+
+// Centres x in place (the finish step needs x - mean) and publishes
+// A = sum(dy), B = sum(dy * (x - mean)).
+template <int T, int V>
+__device__ __forceinline__ void bn_bwd_reduce(const BnBwdArgs& a, const BnIndex<V>& ix, int ch, int k,
+                                              BnBwdTile<V>& t, float* red)
+{
+  const unsigned tid = threadIdx.x;
+  const float mean = t.mean;
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      t.x[i][j] = ix.ok[i] ? t.x[i][j] - mean : 0.f;
+      sa += t.g[i][j];
+      sb += t.g[i][j] * t.x[i][j];
+    }
+  }
+  team_sum2<T / kWave>(sa, sb, red, tid / kWave, tid & (kWave - 1));
+  if (tid == 0) cluster_publish(sa, sb, a.cw.slots + static_cast<int64_t>(ch) * a.M, k);
+}
+
+template <int T, int V>
+__device__ __forceinline__ void bn_bwd_finish(const BnBwdArgs& a, const BnIndex<V>& ix, int ch, int k,
+                                              BnBwdTile<V>& t, float* bc)
+{
+  const unsigned tid = threadIdx.x;
+  const float inv_stdev = 1.0f / sqrtf(t.var + a.eps);
+  const float scale = t.scale;
+  if (tid < kWave) {
+    float ta, tb;
+    cluster_collect(a.cw.slots + static_cast<int64_t>(ch) * a.M, a.M, a.cw.error, 0.f, 0.f, ta, tb);
+    ta = wave_sum(ta);
+    tb = wave_sum(tb);
+    if (tid == 0) {
+      float ds, db, dmean, dvar;
+      grads_from_sums(ta, tb, scale, inv_stdev, ds, db, dmean, dvar);
+      bc[0] = dmean / static_cast<float>(a.n);
+      bc[1] = dvar * 2.f / static_cast<float>(a.n - (a.bessel ? 1 : 0));
+      if (k == 0) {
+        a.dscale[ch] = ds;
+        a.dbias[ch] = db;
+        a.dmean_out[ch] = dmean;
+        a.dvar_out[ch] = dvar;
+      }
+    }
+  }
+  __syncthreads();
+  const float dmean_term = bc[0];
+  const float dvar_term = bc[1];
+  const float k0 = scale * inv_stdev;
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t.g[i][j] = t.g[i][j] * k0 + dmean_term + dvar_term * t.x[i][j];
+  bn_tile_store<V>(t.g, a.dx + static_cast<int64_t>(ch) * a.cs, a.lddx, ix);
+}
+
+template <int T, int V>
+__device__ __forceinline__ void bn_bwd_step(const BnBwdArgs& a, const BnIndex<V>& ix, int ch, int nc, int k,
+                                            BnBwdTile<V>& F, BnBwdTile<V>& R, BnBwdTile<V>& L, float* red,
+                                            float* bc)
+{
+  if (ch + nc < a.C) bn_bwd_reduce<T, V>(a, ix, ch + nc, k, R, red);
+  if (ch + 2 * nc < a.C) bn_bwd_load<V>(L, a, ch + 2 * nc, ix);
+  asm volatile("" ::: "memory");
+  bn_bwd_finish<T, V>(a, ix, ch, k, F, bc);
+}
+
+// Backward in training mode: x and dy are read once, dx written once.
+template <int T, int V>
+__global__ void __launch_bounds__(T)
+bn_bwd_cluster(BnBwdArgs a, unsigned seg, unsigned E)
+{
+  __shared__ float red[2 * (T / kWave)];
+  __shared__ float bc[2];
+  const int nc = gridDim.x / a.M;
+  const int cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - cl * a.M;
+  const BnIndex<V> ix = bn_make_index<T, V>(k, seg, E);
+  BnBwdTile<V> t0, t1, t2;
+  if (cl >= a.C) return;
+  bn_bwd_load<V>(t0, a, cl, ix);
+  if (cl + nc < a.C) bn_bwd_load<V>(t1, a, cl + nc, ix);
+  bn_bwd_reduce<T, V>(a, ix, cl, k, t0, red);
+  for (int ch = cl; ch < a.C; ch += 3 * nc) {
+    bn_bwd_step<T, V>(a, ix, ch, nc, k, t0, t1, t2, red, bc);
+    if (ch + nc < a.C) bn_bwd_step<T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, red, bc);
+    if (ch + 2 * nc < a.C) bn_bwd_step<T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, red, bc);
+  }
+}
+
+// Workgroup size and vectors per thread of a cluster launch for channels of E vectors.
+struct BnClusterShape {
+  int T, V, M;
+};
+
+static BnClusterShape bn_cluster_shape(int64_t E, int max_v, int first_t)
+{
+  static const int force_t = std::getenv("LBN_BN_CLUSTER_T") ? std::atoi(std::getenv("LBN_BN_CLUSTER_T")) : 0;
+  for (int T = force_t ? force_t : first_t; T <= 1024; T *= 2) {
+    const ClusterPlan p = plan_cluster(E, max_v, T);
+    if (p.M) return {T, p.V, p.M};
+    if (force_t) break;
+  }
+  return {0, 0, 0};
+}
+
 // ==================================================================== host side
 // Workgroups per channel: about 4096 workgroups in total, each with at least four
 // accesses per thread, at most one wave's worth so a wave can merge the partials.
@@ -348,7 +677,79 @@ static int bn_split(int64_t C, int64_t cs, int64_t w)
 static size_t bn_workspace(int64_t C, int64_t cs, int64_t w)
 {
   if (C <= 0 || cs <= 0 || w <= 0) return 0;
-  return static_cast<size_t>(C) * bn_split(C, cs, w) * sizeof(float2);
+  const size_t split = static_cast<size_t>(C) * bn_split(C, cs, w) * sizeof(float2);
+  const size_t cluster = cluster_workspace_bytes(C);
+  return split > cluster ? split : cluster;
+}
+
+// Launches the register-resident forward when the shape allows it.  Returns false
+// when the caller must use the two-kernel path.
+template <int T, int V>
+static bool bn_launch_fwd_cluster(hipStream_t st, const BnFwdArgs& a, int64_t C, unsigned seg, unsigned E)
+{
+  const int cap = cluster_capacity(bn_fwd_cluster<T, V>, T);
+  const int64_t ncl = cap / a.M < C ? cap / a.M : C;
+  if (ncl < 1) return false;
+  launch_cluster_reset(st, a.cw, C * a.M);
+  hipLaunchKernelGGL((bn_fwd_cluster<T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
+  return true;
+}
+
+template <int T, int V>
+static bool bn_launch_bwd_cluster(hipStream_t st, const BnBwdArgs& a, int64_t C, unsigned seg, unsigned E)
+{
+  const int cap = cluster_capacity(bn_bwd_cluster<T, V>, T);
+  const int64_t ncl = cap / a.M < C ? cap / a.M : C;
+  if (ncl < 1) return false;
+  launch_cluster_reset(st, a.cw, C * a.M);
+  hipLaunchKernelGGL((bn_bwd_cluster<T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
+  return true;
+}
+
+static bool bn_cluster_usable(int64_t C, int64_t cs, int64_t w, const void* ws)
+{
+  static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
+  const int64_t E = cs / 4 * w;
+  return !disabled && E < (int64_t(1) << 31) - 8192 && cs * w > 1 && C <= (1 << 24) && aligned16(ws);
+}
+
+static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w, int pivot, int bessel,
+                               float eps, float decay, const float* x, int64_t ldx, float* y,
+                               int64_t ldy, float* mean, float* var, const float* scale,
+                               const float* bias, float* rmean, float* rvar, void* ws)
+{
+  if (!bn_cluster_usable(C, cs, w, ws)) return false;
+  const int64_t E = cs / 4 * w;
+  const BnClusterShape p = bn_cluster_shape(E, 4, 256);
+  if (!p.T) return false;
+  const BnFwdArgs a{x, y, ldx, ldy, cs, static_cast<int>(C), p.M, pivot, bessel, eps, decay, cs * w,
+                    cluster_workspace(ws), mean, var, scale, bias, rmean, rvar};
+  const unsigned seg = static_cast<unsigned>(cs / 4), Eu = static_cast<unsigned>(E);
+#define X(TT, VV) \
+  if (p.T == TT && p.V == VV) return bn_launch_fwd_cluster<TT, VV>(st, a, C, seg, Eu);
+  X(256, 1) X(256, 2) X(256, 3) X(256, 4) X(512, 1) X(512, 2) X(512, 3) X(512, 4) X(1024, 1) X(1024, 2)
+  X(1024, 3) X(1024, 4)
+#undef X
+  return false;
+}
+
+static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bessel, float eps,
+                               const float* x, int64_t ldx, const float* dy, int64_t lddy, float* dx,
+                               int64_t lddx, const float* mean, const float* var, const float* scale,
+                               float* dscale, float* dbias, float* dmean, float* dvar, void* ws)
+{
+  if (!bn_cluster_usable(C, cs, w, ws)) return false;
+  const int64_t E = cs / 4 * w;
+  const BnClusterShape p = bn_cluster_shape(E, 2, 256);
+  if (!p.T) return false;
+  const BnBwdArgs a{x, dy, dx, ldx, lddy, lddx, cs, static_cast<int>(C), p.M, bessel, eps, cs * w,
+                    cluster_workspace(ws), mean, var, scale, dscale, dbias, dmean, dvar};
+  const unsigned seg = static_cast<unsigned>(cs / 4), Eu = static_cast<unsigned>(E);
+#define X(TT, VV) \
+  if (p.T == TT && p.V == VV) return bn_launch_bwd_cluster<TT, VV>(st, a, C, seg, Eu);
+  X(256, 1) X(256, 2) X(512, 1) X(512, 2) X(1024, 1) X(1024, 2)
+#undef X
+  return false;
 }
 
 struct BnShape {
@@ -461,6 +862,10 @@ int lbn_batch_norm_fwd_f32(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
   const dim3 grid(P, static_cast<unsigned>(C));
   hipStream_t st = as_stream(stream);
   const int pivot = (flags & LBN_STATS_SUMSQ) ? 0 : 1;
+  if (bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, y, ldy) &&
+      bn_try_fwd_cluster(st, C, cs, w, pivot, bessel, epsilon, decay, x, ldx, y, ldy, mean, var, scale,
+                         bias, running_mean, running_var, workspace))
+    return launch_status();
   if (bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, y, ldy)) {
     hipLaunchKernelGGL((bn_fwd_sums<true>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, pivot, part);
     hipLaunchKernelGGL((bn_fwd_apply<true, true>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs, w,
@@ -548,6 +953,10 @@ int lbn_batch_norm_bwd_f32(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
   const dim3 grid(P, static_cast<unsigned>(C));
   hipStream_t st = as_stream(stream);
   const int64_t n = cs * w;
+  if (training && bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, dy, lddy) && bn_vec_ok(cs, w, dx, lddx) &&
+      bn_try_bwd_cluster(st, C, cs, w, bessel, epsilon, x, ldx, dy, lddy, dx, lddx, use_mean, use_var,
+                         scale, dscale, dbias, dmean, dvar, workspace))
+    return launch_status();
   if (bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, dy, lddy) && bn_vec_ok(cs, w, dx, lddx)) {
     hipLaunchKernelGGL((bn_bwd_sums<true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean, part);
     hipLaunchKernelGGL((bn_bwd_apply<true, true>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,

@@ -91,6 +91,34 @@ struct Vec16<__half> {
 };
 
 // ---------------------------------------------------------------------------
+// exp(x) for x <= ~0 (softmax arguments after max-subtraction) in 6 VALU operations
+// and one v_exp_f32: exp(x) = 2^t * 2^r with t = fl(x*log2e) and r the exact
+// rounding error of that product plus x*(log2e - fl(log2e)), 2^r ~ 1 + r*ln2.
+// Error stays below 2 ulp for x <= 88, against ~20 operations for the library expf.
+// Results below the smallest normal float come out as 0 (v_exp_f32 has no denormal
+// support); exp_keep_denormals() rescales to keep them.
+__device__ __forceinline__ float exp_fast(float x)
+{
+  constexpr float kLog2e = 1.44269502162933349609375f;        // fl(log2(e))
+  constexpr float kLog2eLo = 1.925963033500011e-08f;          // log2(e) - fl(log2(e))
+  constexpr float kLn2 = 0.693147182464599609375f;
+  x = x < -104.0f ? -104.0f : x;  // exp underflows to 0 there; keeps t finite and NaN a NaN
+  const float t = x * kLog2e;
+  float r = __builtin_fmaf(x, kLog2e, -t);
+  r = __builtin_fmaf(x, kLog2eLo, r);
+  const float e = __builtin_amdgcn_exp2f(t);
+  return __builtin_fmaf(e, r * kLn2, e);
+}
+
+__device__ __forceinline__ float exp_keep_denormals(float x)
+{
+  // below exp(-87.3) the result is denormal: evaluate 2^64 times larger, scale back
+  const bool tiny = x < -87.0f;
+  const float e = exp_fast(tiny ? x + 44.3614196f : x);       // 64*ln2
+  return tiny ? e * 5.42101086e-20f : e;                      // 2^-64
+}
+
+// ---------------------------------------------------------------------------
 // Wave64 butterfly reductions: every lane ends with the result.
 __device__ __forceinline__ float wave_sum(float v)
 {

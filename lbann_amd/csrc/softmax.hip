@@ -14,9 +14,10 @@
 //    S partials and writes its chunk.  Kernel 1 reads everything before kernel 2
 //    writes anything, so in-place operation stays safe with many workgroups per row.
 //
-// Numerics follow the reference CPU code: max-subtraction, expf/logf at <= 1 ulp,
+// Numerics follow the reference CPU code: max-subtraction, exp at <= 2 ulp (exp_fast),
 // reciprocal-then-multiply, and softmax (only) writes 0 for results that are not
 // normal floats (include/lbann/utils/dnn_lib/openmp/softmax.hpp:107-116).
+#include "cluster_sync.hpp"
 #include "device_utils.hpp"
 #include "host_utils.hpp"
 
@@ -72,7 +73,7 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const float d = v[i][k] - m;
-      const float e = ok ? expf(d) : 0.f;
+      const float e = ok ? (KIND == kChannelwise ? exp_keep_denormals(d) : exp_fast(d)) : 0.f;
       s += e;
       v[i][k] = (KIND == kLogSoftmax) ? d : e;
     }
@@ -150,10 +151,164 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
     if (idx < nvec) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        if (KIND == kLogSoftmax) g[i][k] = g[i][k] - expf(a[i][k]) * s;
+        if (KIND == kLogSoftmax) g[i][k] = g[i][k] - exp_fast(a[i][k]) * s;
         else g[i][k] = a[i][k] * (g[i][k] - s);
       }
       Vec16<float>::store(dr + 4 * idx, g[i]);
+    }
+  }
+}
+
+
+// ================================================ register-resident row clusters
+// Rows too long for one workgroup's registers: a cluster of M workgroups shares a
+// row, workgroup k keeps vectors [k*256*V, (k+1)*256*V) in registers, the cluster
+// exchanges one (max, sum) pair per workgroup and every workgroup finishes from its
+// registers.  One read and one write per element, and safe in place: a workgroup
+// has read its whole share before it writes any of it, and shares are disjoint.
+template <int V, int KIND>
+__global__ void __launch_bounds__(kClusterThreads)
+sm_fwd_cluster(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
+               unsigned nvec, int M, ClusterWorkspace cw)
+{
+  constexpr int NW = kClusterThreads / kWave;
+  __shared__ float red[2][NW];
+  __shared__ float bc[2];
+  const int nclusters = gridDim.x / M;
+  const int cl = blockIdx.x / M;
+  const int k = blockIdx.x - cl * M;
+  const unsigned tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wv = tid / kWave;
+  const unsigned base = static_cast<unsigned>(k) * (kClusterThreads * V) + tid;
+  for (int64_t row = cl; row < rows; row += nclusters) {
+    const float* xr = x + map.offset(row, ldx);
+    float v[V][4];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = base + i * kClusterThreads;
+      if (idx < nvec) {
+        Vec16<float>::load(xr + 4 * static_cast<int64_t>(idx), v[i]);
+      }
+      else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[i][j] = -FLT_MAX;
+      }
+    }
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) m = fmaxf(m, v[i][j]);
+    m = team_max<NW>(m, red[0], wv, lane);
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const bool ok = base + i * kClusterThreads < nvec;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float d = v[i][j] - m;
+        const float e = ok ? (KIND == kChannelwise ? exp_keep_denormals(d) : exp_fast(d)) : 0.f;
+        s += e;
+        v[i][j] = (KIND == kLogSoftmax) ? d : e;
+      }
+    }
+    s = team_sum<NW>(s, red[1], wv, lane);
+    if (tid < kWave) {
+      float pm, ps;
+      cluster_exchange(m, s, cw.slots + row * M, k, M, cw.error, -FLT_MAX, 0.f, pm, ps);
+      const float gmax = wave_max(pm);
+      const float gsum = wave_sum(ps * exp_fast(pm - gmax));
+      if (tid == 0) {
+        bc[0] = gmax;
+        bc[1] = gsum;
+      }
+    }
+    __syncthreads();
+    const float gm = bc[0];
+    const float gs = bc[1];
+    float* yr = y + map.offset(row, ldy);
+    const float shift = m - gm;                       // <= 0: this share's maximum against the row's
+    const float f = exp_fast(shift) * (1.0f / gs);    // rescales exp(x - m) to exp(x - gm) / sum
+    const float lse = (KIND == kLogSoftmax) ? logf(gs) : 0.f;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = base + i * kClusterThreads;
+      if (idx < nvec) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (KIND == kSoftmax) {
+            const float r = f * v[i][j];
+            v[i][j] = __builtin_isnormal(r) ? r : 0.f;
+          }
+          else if (KIND == kLogSoftmax) {
+            v[i][j] = (v[i][j] + shift) - lse;
+          }
+          else {
+            v[i][j] *= f;
+          }
+        }
+        Vec16<float>::store(yr + 4 * static_cast<int64_t>(idx), v[i]);
+      }
+    }
+  }
+}
+
+template <int V, int KIND>
+__global__ void __launch_bounds__(kClusterThreads)
+sm_bwd_cluster(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
+               RowMap map, int64_t rows, unsigned nvec, int M, ClusterWorkspace cw)
+{
+  constexpr int NW = kClusterThreads / kWave;
+  __shared__ float red[NW];
+  __shared__ float bc[1];
+  const int nclusters = gridDim.x / M;
+  const int cl = blockIdx.x / M;
+  const int k = blockIdx.x - cl * M;
+  const unsigned tid = threadIdx.x;
+  const unsigned base = static_cast<unsigned>(k) * (kClusterThreads * V) + tid;
+  for (int64_t row = cl; row < rows; row += nclusters) {
+    const float* yr = y + map.offset(row, ldy);
+    const float* gr = dy + map.offset(row, lddy);
+    float a[V][4], g[V][4];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = base + i * kClusterThreads;
+      if (idx < nvec) {
+        Vec16<float>::load(yr + 4 * static_cast<int64_t>(idx), a[i]);
+        Vec16<float>::load(gr + 4 * static_cast<int64_t>(idx), g[i]);
+      }
+      else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[i][j] = g[i][j] = 0.f;
+      }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s += (KIND == kLogSoftmax) ? g[i][j] : a[i][j] * g[i][j];
+    s = team_sum<NW>(s, red, tid / kWave, tid & (kWave - 1));
+    if (tid < kWave) {
+      float pt, unused;
+      cluster_exchange(s, 0.f, cw.slots + row * M, k, M, cw.error, 0.f, 0.f, pt, unused);
+      pt = wave_sum(pt);
+      if (tid == 0) bc[0] = pt;
+    }
+    __syncthreads();
+    const float tot = bc[0];
+    float* dr = dx + map.offset(row, lddx);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = base + i * kClusterThreads;
+      if (idx < nvec) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (KIND == kLogSoftmax) g[i][j] = g[i][j] - exp_fast(a[i][j]) * tot;
+          else g[i][j] = a[i][j] * (g[i][j] - tot);
+        }
+        Vec16<float>::store(dr + 4 * static_cast<int64_t>(idx), g[i]);
+      }
     }
   }
 }
@@ -168,7 +323,7 @@ __device__ __forceinline__ void block_merge_max_sum(float& m, float& acc, float 
   const int lane = threadIdx.x & (kWave - 1);
   const int wv = threadIdx.x / kWave;
   const float wm = wave_max(m);
-  acc = wave_sum(acc * expf(m - wm));
+  acc = wave_sum(acc * exp_fast(m - wm));
   if (lane == 0) {
     slot[wv][0] = wm;
     slot[wv][1] = acc;
@@ -179,7 +334,7 @@ __device__ __forceinline__ void block_merge_max_sum(float& m, float& acc, float 
   for (int i = 1; i < kChunkThreads / kWave; ++i) bm = fmaxf(bm, slot[i][0]);
   float bs = 0.f;
 #pragma unroll
-  for (int i = 0; i < kChunkThreads / kWave; ++i) bs += slot[i][1] * expf(slot[i][0] - bm);
+  for (int i = 0; i < kChunkThreads / kWave; ++i) bs += slot[i][1] * exp_fast(slot[i][0] - bm);
   m = bm;
   acc = bs;
 }
@@ -201,7 +356,7 @@ sm_fwd_partial(const float* x, int64_t ldx, RowMap map, int64_t n, int64_t chunk
       float v[4];
       Vec16<float>::load(xr + 4 * i, v);
       const float mn = fmaxf(fmaxf(fmaxf(m, v[0]), fmaxf(v[1], v[2])), v[3]);
-      acc = acc * expf(m - mn) + ((expf(v[0] - mn) + expf(v[1] - mn)) + (expf(v[2] - mn) + expf(v[3] - mn)));
+      acc = acc * exp_fast(m - mn) + ((exp_fast(v[0] - mn) + exp_fast(v[1] - mn)) + (exp_fast(v[2] - mn) + exp_fast(v[3] - mn)));
       m = mn;
     }
   }
@@ -209,7 +364,7 @@ sm_fwd_partial(const float* x, int64_t ldx, RowMap map, int64_t n, int64_t chunk
     for (int64_t i = begin + threadIdx.x; i < end; i += kChunkThreads) {
       const float v = xr[i];
       const float mn = fmaxf(m, v);
-      acc = acc * expf(m - mn) + expf(v - mn);
+      acc = acc * exp_fast(m - mn) + exp_fast(v - mn);
       m = mn;
     }
   }
@@ -235,7 +390,7 @@ sm_fwd_apply(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int
     ps = p.y;
   }
   const float m = wave_max(pm);
-  const float sum = wave_sum(ps * expf(pm - m));
+  const float sum = wave_sum(ps * exp_fast(pm - m));
   const float scale = 1.0f / sum;
   const float lse = (KIND == kLogSoftmax) ? logf(sum) : 0.f;
   const float* xr = x + map.offset(row, ldx);
@@ -243,7 +398,7 @@ sm_fwd_apply(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int
   auto f = [&](float v) -> float {
     const float d = v - m;
     if (KIND == kLogSoftmax) return d - lse;
-    const float r = scale * expf(d);
+    const float r = scale * (KIND == kChannelwise ? exp_keep_denormals(d) : exp_fast(d));
     if (KIND == kSoftmax) return __builtin_isnormal(r) ? r : 0.f;
     return r;
   };
@@ -311,7 +466,7 @@ sm_bwd_apply(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ld
   const float* gr = dy + map.offset(row, lddy);
   float* dr = dx + map.offset(row, lddx);
   auto f = [&](float a, float g) -> float {
-    return (KIND == kLogSoftmax) ? g - expf(a) * sum : a * (g - sum);
+    return (KIND == kLogSoftmax) ? g - exp_fast(a) * sum : a * (g - sum);
   };
   if (VEC) {
     for (int64_t i = begin / 4 + threadIdx.x; i < end / 4; i += kChunkThreads) {
@@ -349,10 +504,20 @@ static ChunkPlan plan_chunks(int64_t n, int64_t rows)
   return {static_cast<int>(S), chunk};
 }
 
+constexpr int64_t kMaxRowVectors = 8192;  // longest row the one-workgroup register kernels hold
+
 static size_t sm_workspace_bytes(int64_t n, int64_t rows)
 {
   if (n <= 0 || rows <= 0) return 0;
-  return static_cast<size_t>(rows) * plan_chunks(n, rows).S * sizeof(float2);
+  const size_t chunked = static_cast<size_t>(rows) * plan_chunks(n, rows).S * sizeof(float2);
+  const size_t cluster = (n / 4 > kMaxRowVectors) ? cluster_workspace_bytes(rows) : 0;
+  return chunked > cluster ? chunked : cluster;
+}
+
+static bool cluster_enabled()
+{
+  static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
+  return !disabled;
 }
 
 #define LBN_ROW_CASES(X)                                                                     \
@@ -386,6 +551,27 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     return launch_status();                                                                  \
   }
       LBN_ROW_CASES(X)
+#undef X
+    }
+  }
+  if (vec && cluster_enabled() && n / 4 < (int64_t(1) << 30)) {
+    const ClusterPlan cp = plan_cluster(n / 4, 8);
+    if (cp.M) {
+      if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
+      const ClusterWorkspace cw = cluster_workspace(ws);
+#define X(VV)                                                                                    \
+  if (cp.V == VV) {                                                                              \
+    const int cap = cluster_capacity(sm_fwd_cluster<VV, KIND>, kClusterThreads);                 \
+    const int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                   \
+    if (ncl >= 1) {                                                                              \
+      launch_cluster_reset(st, cw, rows * cp.M);                                                 \
+      hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND>), dim3(static_cast<unsigned>(ncl * cp.M)),    \
+                         dim3(kClusterThreads), 0, st, x, y, ldx, ldy, map, rows,                \
+                         static_cast<unsigned>(n / 4), cp.M, cw);                                \
+      return launch_status();                                                                    \
+    }                                                                                            \
+  }
+      X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8)
 #undef X
     }
   }
@@ -436,6 +622,27 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     return launch_status();                                                                  \
   }
       LBN_ROW_CASES(X)
+#undef X
+    }
+  }
+  if (vec && cluster_enabled() && n / 4 < (int64_t(1) << 30)) {
+    const ClusterPlan cp = plan_cluster(n / 4, 4);
+    if (cp.M) {
+      if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
+      const ClusterWorkspace cw = cluster_workspace(ws);
+#define X(VV)                                                                                    \
+  if (cp.V == VV) {                                                                              \
+    const int cap = cluster_capacity(sm_bwd_cluster<VV, KIND>, kClusterThreads);                 \
+    const int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                   \
+    if (ncl >= 1) {                                                                              \
+      launch_cluster_reset(st, cw, rows * cp.M);                                                 \
+      hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND>), dim3(static_cast<unsigned>(ncl * cp.M)),    \
+                         dim3(kClusterThreads), 0, st, y, dy, dx, ldy, lddy, lddx, map, rows,    \
+                         static_cast<unsigned>(n / 4), cp.M, cw);                                \
+      return launch_status();                                                                    \
+    }                                                                                            \
+  }
+      X(1) X(2) X(3) X(4)
 #undef X
     }
   }

@@ -78,17 +78,17 @@ def test_softmax_family_in_place(L, kind, h, w):
     if kind == "channelwise":
         C = 7 if h == 777 else 4
         layer = L.channelwise_softmax_layer((C, h // C))
-        y_ref = orc.channelwise_softmax_fwd(x, C, h // C, h // C)
+        fwd = lambda a: orc.channelwise_softmax_fwd(a, C, h // C, h // C)
         bwd = lambda y, g: orc.channelwise_softmax_bwd(y, g, C, h // C, h // C)
     else:
         layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
-        y_ref = _sm_oracle(kind)[0](x)
-        bwd = _sm_oracle(kind)[1]
+        fwd, bwd = _sm_oracle(kind)
+    y_ref, y_ex = fwd(x), fwd(f64(x))
     xm = L.DeviceMatrix.from_numpy(x)
     ym = layer.forward(xm, in_place=True)
     assert ym is xm
     y = ym.to_numpy()
-    check(f"{kind} in-place y", y, y_ref, None, tol=TOL_F32)
+    check(f"{kind} in-place y", y, y_ref, y_ex, tol=TOL_F32)
     gm = L.DeviceMatrix.from_numpy(dy)
     dm = layer.backward(gm, in_place=True)
     assert dm is gm
