@@ -1,0 +1,470 @@
+// Header-only C++ adapter: the five LBANN layer classes' fp_compute()/bp_compute()
+// bodies, written against the C ABI of include/lbnorm.h.
+//
+// The classes keep the reference's names, constructor parameters, member matrices
+// and error behaviour (a thrown exception where the reference calls LBANN_ERROR), so
+// that each body can replace the corresponding GPU specialisation in LBANN:
+//   layer_norm_layer            src/layers/regularizers/layer_norm.cu  (fp_compute/bp_compute)
+//   batch_normalization_layer   src/layers/regularizers/batch_normalization.cu
+//   softmax_layer               src/layers/activations/softmax.cu      (data-parallel branch)
+//   log_softmax_layer           src/layers/activations/log_softmax.cu
+//   channelwise_softmax_layer   src/layers/misc/channelwise_softmax.cu
+//
+// `Mat` is any local-matrix type with the El::Matrix<T, El::Device::GPU> accessors
+//   Height(), Width(), LDim(), Buffer(), LockedBuffer()
+// (El::Matrix itself inside LBANN; lbnorm::device_matrix below elsewhere).  The
+// adapter never touches matrix contents on the host and never synchronises.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <functional>
+#include <numeric>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+#include <vector>
+
+#include "../../include/lbnorm.h"
+
+namespace lbnorm {
+
+/// Thrown where the reference throws lbann::exception through LBANN_ERROR.
+struct exception : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+
+inline void check_status(int status, const char* where)
+{
+  if (status != LBN_OK)
+    throw exception(std::string(where) + ": " + lbn_status_string(status) + " (status " +
+                    std::to_string(status) + ")");
+}
+
+inline void check_hip(hipError_t e, const char* where)
+{
+  if (e != hipSuccess) throw exception(std::string(where) + ": " + hipGetErrorString(e));
+}
+
+/// Column-major device matrix with El::Matrix's accessor names.  Owns its memory
+/// unless attached to an existing buffer.
+template <typename T>
+class device_matrix {
+public:
+  device_matrix() = default;
+  device_matrix(int64_t height, int64_t width) { Resize(height, width); }
+  device_matrix(const device_matrix&) = delete;
+  device_matrix& operator=(const device_matrix&) = delete;
+  ~device_matrix() { release(); }
+
+  /// View of memory owned by someone else (El::Matrix::Attach / LockedAttach).
+  void Attach(int64_t height, int64_t width, T* buffer, int64_t ldim)
+  {
+    release();
+    m_h = height; m_w = width; m_ld = ldim; m_buf = buffer; m_owned = false;
+  }
+  void Resize(int64_t height, int64_t width)
+  {
+    if (m_owned && m_buf && height * width <= m_capacity) {
+      m_h = height; m_w = width; m_ld = height > 0 ? height : 1;
+      return;
+    }
+    release();
+    m_h = height; m_w = width; m_ld = height > 0 ? height : 1;
+    m_capacity = height * width;
+    if (m_capacity > 0) {
+      void* p = nullptr;
+      check_hip(hipMalloc(&p, static_cast<size_t>(m_capacity) * sizeof(T)), "device_matrix::Resize");
+      m_buf = static_cast<T*>(p);
+      m_owned = true;
+    }
+  }
+  int64_t Height() const { return m_h; }
+  int64_t Width() const { return m_w; }
+  int64_t LDim() const { return m_ld; }
+  T* Buffer() { return m_buf; }
+  const T* LockedBuffer() const { return m_buf; }
+  bool IsEmpty() const { return m_h < 1 || m_w < 1; }
+
+private:
+  void release()
+  {
+    if (m_owned && m_buf) (void)hipFree(m_buf);
+    m_buf = nullptr; m_owned = false; m_capacity = 0;
+  }
+  int64_t m_h = 0, m_w = 0, m_ld = 1, m_capacity = 0;
+  T* m_buf = nullptr;
+  bool m_owned = false;
+};
+
+/// Scratch buffer a layer owns (the role of the reference's m_workspace members).
+class workspace {
+public:
+  workspace() = default;
+  workspace(const workspace&) = delete;
+  workspace& operator=(const workspace&) = delete;
+  ~workspace() { if (m_buf) (void)hipFree(m_buf); }
+  void* reserve(size_t bytes)
+  {
+    if (bytes > m_bytes) {
+      if (m_buf) (void)hipFree(m_buf);
+      m_buf = nullptr;
+      check_hip(hipMalloc(&m_buf, bytes), "workspace::reserve");
+      m_bytes = bytes;
+    }
+    return m_buf;
+  }
+  size_t bytes() const { return m_bytes; }
+private:
+  void* m_buf = nullptr;
+  size_t m_bytes = 0;
+};
+
+/// What data_type_layer hands to the compute hooks: the four local matrices and the
+/// stream of their SyncInfo.
+template <typename Mat>
+struct layer_io {
+  const Mat* prev_activations = nullptr;    // get_prev_activations().LockedMatrix()
+  Mat* activations = nullptr;               // get_activations().Matrix()
+  const Mat* prev_error_signals = nullptr;  // get_prev_error_signals().LockedMatrix()
+  Mat* error_signals = nullptr;             // get_error_signals().Matrix()
+  hipStream_t stream = nullptr;
+};
+
+namespace detail {
+inline int64_t product(const std::vector<int64_t>& d, size_t from, size_t to)
+{
+  int64_t p = 1;
+  for (size_t i = from; i < to; ++i) p *= d[i];
+  return p;
+}
+template <typename T> struct is_half : std::false_type {};
+}  // namespace detail
+
+// ------------------------------------------------------------------ layer norm
+/// include/lbann/layers/regularizers/layer_norm.hpp:53-143.  T is float, or a 16-bit
+/// storage type (any 2-byte IEEE binary16 type) for the fp16-storage kernels.
+template <typename T, typename Mat = device_matrix<T>>
+class layer_norm_layer {
+public:
+  layer_norm_layer(double epsilon = 1e-5, bool scale = false, bool bias = false, int start_dim = 0)
+    : m_epsilon(static_cast<float>(epsilon)), m_scale(scale), m_bias(bias), m_start_dim(start_dim) {}
+
+  /// setup_dims + setup_data: fixes the normalised dimensions (layer_norm.hpp:259-290).
+  void setup(const std::vector<int64_t>& dims)
+  {
+    m_dims = dims;
+    const int nd = static_cast<int>(dims.size());
+    const int sd = m_start_dim >= 0 ? m_start_dim : nd + m_start_dim;
+    if (sd < 0 || sd >= nd)
+      throw exception("Layer normalization start dimension " + std::to_string(m_start_dim) +
+                      " does not match the input tensor dimensionality of " + std::to_string(nd));
+    m_sd = sd;
+  }
+  /// get_normdims (layer_norm.hpp:362-405), data-parallel layout.
+  void get_normdims(int64_t& normalization_size, int64_t& global_normalization_size,
+                    int64_t& num_normalized, int64_t& normalization_stride) const
+  {
+    num_normalized = detail::product(m_dims, 0, m_sd);
+    normalization_size = detail::product(m_dims, m_sd, m_dims.size());
+    normalization_stride = normalization_size;
+    global_normalization_size = normalization_size;
+  }
+  /// Weight values (weights_values(i).LockedMatrix().LockedBuffer()) and gradient sinks.
+  void set_weights(const float* scale, const float* bias) { m_scale_w = scale; m_bias_w = bias; }
+  void set_weight_gradients(float* dscale, float* dbias) { m_scale_grad = dscale; m_bias_grad = dbias; }
+
+  layer_io<Mat> io;
+  device_matrix<float> m_statistics;           // 2*num_normalized x width: means, then variances
+  device_matrix<float> m_statistics_gradient;  // same shape: dL/dmean, dL/dvar
+  int stats_mode = LBN_STATS_TWO_PASS;
+
+  /// layer_norm.cpp:263-290 / layer_norm.cu fp_compute.
+  void fp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    Mat& y = *io.activations;
+    int64_t n, gn, G, stride;
+    get_normdims(n, gn, G, stride);
+    m_statistics.Resize(2 * G, x.Width());
+    const float* sw = m_scale ? m_scale_w : nullptr;
+    const float* bw = m_bias ? m_bias_w : nullptr;
+    int st;
+    if (sizeof(T) == 2)
+      st = lbn_layer_norm_fwd_f16(io.stream, G, n, stride, x.Width(), m_epsilon, x.LockedBuffer(), x.LDim(),
+                                  y.Buffer(), y.LDim(), m_statistics.Buffer(), m_statistics.LDim(), sw, bw,
+                                  stats_mode);
+    else
+      st = lbn_layer_norm_fwd_f32(io.stream, G, n, stride, x.Width(), m_epsilon,
+                                  reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
+                                  reinterpret_cast<float*>(y.Buffer()), y.LDim(), m_statistics.Buffer(),
+                                  m_statistics.LDim(), sw, bw, stats_mode);
+    check_status(st, "layer_norm_layer::fp_compute");
+  }
+
+  /// layer_norm.cpp:292-348 / layer_norm.cu bp_compute.  The weight gradients are
+  /// overwritten (the reference zeroes them first, :300-309); handing them to the
+  /// optimizer (add_to_gradient, :330-347) stays with the caller.
+  void bp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    const Mat& dy = *io.prev_error_signals;
+    Mat& dx = *io.error_signals;
+    int64_t n, gn, G, stride;
+    get_normdims(n, gn, G, stride);
+    m_statistics_gradient.Resize(2 * G, x.Width());
+    const float* sw = m_scale ? m_scale_w : nullptr;
+    float* dsw = m_scale ? m_scale_grad : nullptr;
+    float* dbw = m_bias ? m_bias_grad : nullptr;
+    const size_t bytes = lbn_layer_norm_bwd_workspace_bytes(G, n, x.Width(), (dsw || dbw) ? 1 : 0,
+                                                            static_cast<int>(sizeof(T)));
+    void* ws = m_ws.reserve(bytes);
+    int st;
+    if (sizeof(T) == 2)
+      st = lbn_layer_norm_bwd_f16(io.stream, G, n, stride, x.Width(), m_epsilon, x.LockedBuffer(), x.LDim(),
+                                  dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+                                  m_statistics.LockedBuffer(), m_statistics.LDim(),
+                                  m_statistics_gradient.Buffer(), m_statistics_gradient.LDim(), sw, dsw, dbw,
+                                  ws, bytes);
+    else
+      st = lbn_layer_norm_bwd_f32(io.stream, G, n, stride, x.Width(), m_epsilon,
+                                  reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
+                                  reinterpret_cast<const float*>(dy.LockedBuffer()), dy.LDim(),
+                                  reinterpret_cast<float*>(dx.Buffer()), dx.LDim(),
+                                  m_statistics.LockedBuffer(), m_statistics.LDim(),
+                                  m_statistics_gradient.Buffer(), m_statistics_gradient.LDim(), sw, dsw, dbw,
+                                  ws, bytes);
+    check_status(st, "layer_norm_layer::bp_compute");
+  }
+
+private:
+  float m_epsilon;
+  bool m_scale, m_bias;
+  int m_start_dim, m_sd = 0;
+  std::vector<int64_t> m_dims;
+  const float* m_scale_w = nullptr;
+  const float* m_bias_w = nullptr;
+  float* m_scale_grad = nullptr;
+  float* m_bias_grad = nullptr;
+  workspace m_ws;
+};
+
+// ------------------------------------------------------------------ batch norm
+/// include/lbann/layers/regularizers/batch_normalization.hpp:130-199 with local
+/// statistics (statistics_group_size == 1).
+template <typename Mat = device_matrix<float>>
+class batch_normalization_layer {
+public:
+  batch_normalization_layer(double decay = 0.9, double epsilon = 1e-5, int statistics_group_size = 1,
+                            bool bessel_correction = true)
+    : m_decay(static_cast<float>(decay)), m_epsilon(static_cast<float>(epsilon)),
+      m_statistics_group_size(statistics_group_size), m_bessel_correction(bessel_correction)
+  {
+    if (statistics_group_size != 1)
+      throw exception("batch_normalization_layer: only local statistics (statistics_group_size == 1) "
+                      "run on one GPU; aggregate with the lbn_batch_norm_*_sums/_stats/_apply entry points");
+  }
+  void setup(const std::vector<int64_t>& dims)
+  {
+    m_dims = dims;
+    m_num_channels = dims.at(0);
+    m_channel_size = detail::product(dims, 1, dims.size());
+    m_mean_and_var.Resize(m_num_channels, 2);
+    m_mean_and_var_gradient.Resize(m_num_channels, 2);
+  }
+  /// weights 0..3: scale, bias, running mean, running variance (all device pointers).
+  void set_weights(const float* scale, const float* bias, float* running_mean, float* running_var)
+  {
+    m_w[0] = const_cast<float*>(scale); m_w[1] = const_cast<float*>(bias);
+    m_w[2] = running_mean; m_w[3] = running_var;
+  }
+  void set_weight_gradients(float* dscale, float* dbias) { m_scale_grad = dscale; m_bias_grad = dbias; }
+
+  layer_io<Mat> io;
+  bool is_training = true;                        // execution_mode::training
+  device_matrix<float> m_mean_and_var;            // C x 2: column 0 mean, column 1 variance
+  device_matrix<float> m_mean_and_var_gradient;   // C x 2
+  int stats_mode = LBN_STATS_TWO_PASS;
+
+  void fp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    Mat& y = *io.activations;
+    const size_t bytes = lbn_batch_norm_workspace_bytes(m_num_channels, m_channel_size, x.Width());
+    void* ws = m_ws.reserve(bytes);
+    float* mv = m_mean_and_var.Buffer();
+    check_status(lbn_batch_norm_fwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                        m_bessel_correction ? 1 : 0, m_epsilon, m_decay, is_training ? 1 : 0,
+                                        x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(), mv,
+                                        mv + m_mean_and_var.LDim(), m_w[0], m_w[1], m_w[2], m_w[3], ws, bytes,
+                                        stats_mode),
+                 "batch_normalization_layer::fp_compute");
+  }
+  void bp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    const Mat& dy = *io.prev_error_signals;
+    Mat& dx = *io.error_signals;
+    const size_t bytes = lbn_batch_norm_workspace_bytes(m_num_channels, m_channel_size, x.Width());
+    void* ws = m_ws.reserve(bytes);
+    const float* mv = m_mean_and_var.LockedBuffer();
+    float* mvg = m_mean_and_var_gradient.Buffer();
+    check_status(lbn_batch_norm_bwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                        m_bessel_correction ? 1 : 0, m_epsilon, is_training ? 1 : 0,
+                                        x.LockedBuffer(), x.LDim(), dy.LockedBuffer(), dy.LDim(), dx.Buffer(),
+                                        dx.LDim(), mv, mv + m_mean_and_var.LDim(), m_w[2], m_w[3], m_w[0],
+                                        m_scale_grad, m_bias_grad, mvg, mvg + m_mean_and_var_gradient.LDim(),
+                                        ws, bytes),
+                 "batch_normalization_layer::bp_compute");
+  }
+
+private:
+  float m_decay, m_epsilon;
+  int m_statistics_group_size;
+  bool m_bessel_correction;
+  std::vector<int64_t> m_dims;
+  int64_t m_num_channels = 0, m_channel_size = 0;
+  float* m_w[4] = {nullptr, nullptr, nullptr, nullptr};
+  float* m_scale_grad = nullptr;
+  float* m_bias_grad = nullptr;
+  workspace m_ws;
+};
+
+// --------------------------------------------------------- softmax / log-softmax
+enum class softmax_mode { INVALID, INSTANCE, CHANNEL };
+
+/// include/lbann/layers/activations/softmax.hpp:85-262, data-parallel layout.
+template <typename Mat = device_matrix<float>>
+class softmax_layer {
+public:
+  explicit softmax_layer(softmax_mode mode = softmax_mode::INSTANCE) : m_mode(mode)
+  {
+    // the CPU reference rejects everything else (dnn_lib/openmp/softmax.hpp:61-63)
+    if (mode != softmax_mode::INSTANCE) throw exception("Unsupported softmax mode");
+  }
+  layer_io<Mat> io;
+  void fp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    Mat& y = *io.activations;
+    const size_t bytes = lbn_softmax_workspace_bytes(x.Height(), x.Width());
+    check_status(lbn_softmax_fwd_f32(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(), y.Buffer(),
+                                     y.LDim(), m_ws.reserve(bytes), bytes),
+                 "softmax_layer::fp_compute");
+  }
+  void bp_compute()
+  {
+    const Mat& y = *io.activations;
+    const Mat& dy = *io.prev_error_signals;
+    Mat& dx = *io.error_signals;
+    const size_t bytes = lbn_softmax_workspace_bytes(y.Height(), y.Width());
+    check_status(lbn_softmax_bwd_f32(io.stream, y.Height(), y.Width(), y.LockedBuffer(), y.LDim(),
+                                     dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+                                     m_ws.reserve(bytes), bytes),
+                 "softmax_layer::bp_compute");
+  }
+private:
+  softmax_mode m_mode;
+  workspace m_ws;
+};
+
+/// include/lbann/layers/activations/log_softmax.hpp.
+template <typename Mat = device_matrix<float>>
+class log_softmax_layer {
+public:
+  layer_io<Mat> io;
+  void fp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    Mat& y = *io.activations;
+    const size_t bytes = lbn_softmax_workspace_bytes(x.Height(), x.Width());
+    check_status(lbn_log_softmax_fwd_f32(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(),
+                                         y.Buffer(), y.LDim(), m_ws.reserve(bytes), bytes),
+                 "log_softmax_layer::fp_compute");
+  }
+  void bp_compute()
+  {
+    const Mat& y = *io.activations;
+    const Mat& dy = *io.prev_error_signals;
+    Mat& dx = *io.error_signals;
+    const size_t bytes = lbn_softmax_workspace_bytes(y.Height(), y.Width());
+    check_status(lbn_log_softmax_bwd_f32(io.stream, y.Height(), y.Width(), y.LockedBuffer(), y.LDim(),
+                                         dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+                                         m_ws.reserve(bytes), bytes),
+                 "log_softmax_layer::bp_compute");
+  }
+private:
+  workspace m_ws;
+};
+
+// --------------------------------------------------------- channelwise softmax
+/// include/lbann/layers/misc/channelwise_softmax.hpp:50-107.
+template <typename Mat = device_matrix<float>>
+class channelwise_softmax_layer {
+public:
+  channelwise_softmax_layer(int64_t dim = 0, bool single_dim_mode = false)
+    : m_dim(dim), m_single_dim_mode(single_dim_mode) {}
+
+  /// setup_dims (channelwise_softmax_impl.hpp:33-56)
+  void setup(const std::vector<int64_t>& dims)
+  {
+    const int64_t nd = static_cast<int64_t>(dims.size());
+    if (m_dim < -nd || m_dim >= nd)
+      throw exception("Dimension " + std::to_string(m_dim) + " is out of bounds for Channelwise Softmax layer on tensor with " +
+                      std::to_string(nd) + " dimensions.");
+    if (!m_single_dim_mode && m_dim != 0 && m_dim != -nd && m_dim != nd - 1 && m_dim != -1)
+      throw exception("Channelwise softmax with all dimensions is only supported for the first or last tensor dimensions. Got dimension " +
+                      std::to_string(m_dim));
+    m_dims = dims;
+  }
+  /// channelwise_softmax_impl.hpp:58-104
+  void get_channel_size_and_stride(int64_t& channel_size, int64_t& channel_stride, int64_t& num_channels) const
+  {
+    const int64_t nd = static_cast<int64_t>(m_dims.size());
+    const int64_t dim = m_dim < 0 ? m_dim + nd : m_dim;
+    const int64_t total = detail::product(m_dims, 0, m_dims.size());
+    if (m_single_dim_mode) {
+      channel_size = m_dims[dim];
+      num_channels = total / channel_size;
+      channel_stride = detail::product(m_dims, dim, m_dims.size());
+    }
+    else {
+      channel_size = total / m_dims[dim];
+      num_channels = m_dims[dim];
+      channel_stride = dim == 0 ? channel_size : 1;
+    }
+  }
+  layer_io<Mat> io;
+  void fp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    Mat& y = *io.activations;
+    int64_t cs, stride, C;
+    get_channel_size_and_stride(cs, stride, C);
+    const size_t bytes = lbn_channelwise_softmax_workspace_bytes(C, cs, x.Width());
+    check_status(lbn_channelwise_softmax_fwd_f32(io.stream, C, cs, stride, x.Width(), x.LockedBuffer(), x.LDim(),
+                                                 y.Buffer(), y.LDim(), m_ws.reserve(bytes), bytes),
+                 "channelwise_softmax_layer::fp_compute");
+  }
+  void bp_compute()
+  {
+    const Mat& y = *io.activations;
+    const Mat& dy = *io.prev_error_signals;
+    Mat& dx = *io.error_signals;
+    int64_t cs, stride, C;
+    get_channel_size_and_stride(cs, stride, C);
+    const size_t bytes = lbn_channelwise_softmax_workspace_bytes(C, cs, y.Width());
+    check_status(lbn_channelwise_softmax_bwd_f32(io.stream, C, cs, stride, y.Width(), y.LockedBuffer(), y.LDim(),
+                                                 dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+                                                 m_ws.reserve(bytes), bytes),
+                 "channelwise_softmax_layer::bp_compute");
+  }
+private:
+  int64_t m_dim;
+  bool m_single_dim_mode;
+  std::vector<int64_t> m_dims;
+  workspace m_ws;
+};
+
+}  // namespace lbnorm

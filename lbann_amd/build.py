@@ -33,6 +33,19 @@ def build(jobs: int = 4) -> str:
     return LIB
 
 
+def build_adapter_driver() -> str:
+    """Compiles tests/cpp/adapter_driver.cpp (host code over the header-only C++ adapter)
+    into tests/cpp/libadapter_driver.so, linked against liblbnorm.so."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "cpp", "adapter_driver.cpp")
+    out = os.path.join(root, "tests", "cpp", "libadapter_driver.so")
+    subprocess.run([HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-shared",
+                    "-Wall", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", src, "-o", out,
+                    "-L" + HERE, "-llbnorm", "-Wl,-rpath,$ORIGIN/../../lbann_amd"], check=True)
+    return out
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_adapter_driver())
     sys.exit(0)

@@ -1,0 +1,122 @@
+"""The header-only C++ adapter (lbann_amd/adapter/lbnorm_layers.hpp) through its test
+driver: host-side behaviour on the CPU, numerical parity with the oracle on the GPU."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DRIVER = os.path.join(ROOT, "tests", "cpp", "libadapter_driver.so")
+
+i64, vp, cint, dbl = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_double
+
+
+def driver():
+    assert os.path.exists(DRIVER), "build it with `python -m lbann_amd.build`"
+    return ctypes.CDLL(DRIVER)
+
+
+def test_adapter_host_logic_and_errors():
+    """Dimension logic and the reference's error cases (bad softmax mode, bad start_dim,
+    bad channelwise dim, non-local batch-norm statistics) without touching a device."""
+    assert driver().drv_error_cases() == 0
+
+
+def _dims(d):
+    return (i64 * len(d))(*d), len(d)
+
+
+@pytest.mark.gpu
+def test_adapter_layers_match_oracle():
+    import torch
+    from oracle import cpu_oracle as orc
+    from tests.parity import TOL_F16, check
+    from lbann_amd.layers import DeviceMatrix
+    d = driver()
+    err = ctypes.create_string_buffer(512)
+    st = vp(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(3)
+    mk = lambda h, w, m=0.0, s=1.0: np.asfortranarray((rng.standard_normal((w, h)) * s + m).astype(np.float32).T)
+    dev = lambda a: torch.from_numpy(np.asarray(a, np.float32)).cuda()
+    p = lambda t: vp(t.data_ptr())
+
+    # ---- layer norm, start_dim = -1 on (6, 512) samples, affine, fp32 and fp16 storage
+    dims, w = (6, 512), 20
+    h = 6 * 512
+    g = (1 + 0.2 * rng.standard_normal(512)).astype(np.float32)
+    b = (0.2 * rng.standard_normal(512)).astype(np.float32)
+    for half in (0, 1):
+        x, dy = mk(h, w, 0.3, 1.5), mk(h, w)
+        if half:
+            x, dy = x.astype(np.float16).astype(np.float32), dy.astype(np.float16).astype(np.float32)
+        tdt = torch.float16 if half else torch.float32
+        mx, mdy = DeviceMatrix.from_numpy(x, dtype=tdt), DeviceMatrix.from_numpy(dy, dtype=tdt)
+        my, mdx = DeviceMatrix(h, w, dtype=tdt), DeviceMatrix(h, w, dtype=tdt)
+        gw, bw, dg, db = dev(g), dev(b), torch.empty(512).cuda(), torch.empty(512).cuda()
+        stats, sgrad = DeviceMatrix(12, w), DeviceMatrix(12, w)
+        da, nd = _dims(dims)
+        rc = d.drv_layer_norm(cint(half), da, cint(nd), cint(-1), cint(1), cint(1), dbl(1e-5), i64(h), i64(w), i64(h),
+                              mx.Buffer(), my.Buffer(), mdy.Buffer(), mdx.Buffer(), p(gw), p(bw), p(dg), p(db),
+                              stats.Buffer(), sgrad.Buffer(), st, err, cint(512))
+        assert rc == 0, err.value
+        y_ref, st_ref = orc.layer_norm_fwd(x, 6, 512, 512, 1e-5, g, b)
+        dx_ref, sg_ref, dg_ref, db_ref = orc.layer_norm_bwd(x, dy, st_ref, 6, 512, 512, 1e-5, g, True, True)
+        tol = TOL_F16 if half else 1e-5
+        check("adapter ln y", my.to_numpy(), y_ref, tol=tol)
+        check("adapter ln dx", mdx.to_numpy(), dx_ref, tol=tol)
+        check("adapter ln stats", stats.to_numpy(), st_ref, tol=tol)
+        check("adapter ln sgrad", sgrad.to_numpy(), sg_ref, tol=tol)
+        check("adapter ln dscale", dg.cpu().numpy(), dg_ref, tol=tol)
+        check("adapter ln dbias", db.cpu().numpy(), db_ref, tol=tol)
+
+    # ---- batch norm (8, 12, 12) x 10
+    dims, w = (8, 12, 12), 10
+    h = 8 * 144
+    x, dy = mk(h, w, 2.0, 3.0), mk(h, w)
+    g = rng.uniform(0.5, 1.5, 8).astype(np.float32)
+    b = (0.1 * rng.standard_normal(8)).astype(np.float32)
+    mx, mdy, my, mdx = DeviceMatrix.from_numpy(x), DeviceMatrix.from_numpy(dy), DeviceMatrix(h, w), DeviceMatrix(h, w)
+    gw, bw, rm, rv = dev(g), dev(b), torch.zeros(8).cuda(), torch.ones(8).cuda()
+    dg, db = torch.empty(8).cuda(), torch.empty(8).cuda()
+    mv, mvg = DeviceMatrix(8, 2), DeviceMatrix(8, 2)
+    da, nd = _dims(dims)
+    rc = d.drv_batch_norm(da, cint(nd), dbl(0.9), dbl(1e-5), cint(1), cint(1), i64(h), i64(w), i64(h), mx.Buffer(),
+                          my.Buffer(), mdy.Buffer(), mdx.Buffer(), p(gw), p(bw), p(rm), p(rv), p(dg), p(db),
+                          mv.Buffer(), mvg.Buffer(), st, err, cint(512))
+    assert rc == 0, err.value
+    rm0, rv0 = np.zeros(8, np.float32), np.ones(8, np.float32)
+    y_ref, m_ref, v_ref = orc.batch_norm_fwd(x, 8, 144, 1e-5, 0.9, g, b, rm0, rv0)
+    dx_ref, dg_ref, db_ref, dm_ref, dv_ref = orc.batch_norm_bwd(x, dy, 8, 144, 1e-5, m_ref, v_ref, g)
+    check("adapter bn y", my.to_numpy(), y_ref)
+    check("adapter bn dx", mdx.to_numpy(), dx_ref)
+    check("adapter bn mean/var", mv.to_numpy(), np.stack([m_ref, v_ref], axis=1))
+    check("adapter bn dmean/dvar", mvg.to_numpy(), np.stack([dm_ref, dv_ref], axis=1))
+    check("adapter bn dscale", dg.cpu().numpy(), dg_ref)
+    check("adapter bn dbias", db.cpu().numpy(), db_ref)
+    check("adapter bn running mean", rm.cpu().numpy(), rm0)
+    check("adapter bn running var", rv.cpu().numpy(), rv0)
+
+    # ---- softmax family, incl. a row long enough for the split kernels (workspace path)
+    for kind, h, w, dims, dim, single in ((0, 4096, 9, (4096,), 0, 0), (1, 1000, 7, (1000,), 0, 0),
+                                          (0, 70000, 2, (70000,), 0, 0), (2, 5 * 2 * 8, 11, (5, 2, 8), -1, 1),
+                                          (2, 16 * 256, 6, (16, 256), 0, 0)):
+        x, dy = mk(h, w, 0.0, 2.0), mk(h, w)
+        mx, mdy, my, mdx = DeviceMatrix.from_numpy(x), DeviceMatrix.from_numpy(dy), DeviceMatrix(h, w), DeviceMatrix(h, w)
+        da, nd = _dims(dims)
+        rc = d.drv_softmax_family(cint(kind), da, cint(nd), i64(dim), cint(single), i64(h), i64(w), i64(h),
+                                  mx.Buffer(), my.Buffer(), mdy.Buffer(), mdx.Buffer(), st, err, cint(512))
+        assert rc == 0, err.value
+        if kind == 0:
+            fwd, bwd = orc.softmax_fwd, orc.softmax_bwd
+        elif kind == 1:
+            fwd, bwd = orc.log_softmax_fwd, orc.log_softmax_bwd
+        else:
+            cs = dims[-1] if single else h // dims[0]
+            C = h // cs
+            fwd = lambda a: orc.channelwise_softmax_fwd(a, C, cs, cs)
+            bwd = lambda yy, gg: orc.channelwise_softmax_bwd(yy, gg, C, cs, cs)
+        f64 = lambda a: np.asfortranarray(np.asarray(a, np.float64))
+        y = my.to_numpy()
+        check(f"adapter softmax kind {kind} y", y, fwd(x), fwd(f64(x)))
+        check(f"adapter softmax kind {kind} dx", mdx.to_numpy(), bwd(y, dy), bwd(f64(y), f64(dy)))

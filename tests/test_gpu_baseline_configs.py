@@ -1,0 +1,162 @@
+"""Parity at the full benchmark shapes: the inputs bench.py uses, GPU through the C ABI
+against the CPU oracle (fp32 restatement, plus float64 where the fp32 reference is
+itself noisy), and size-independent invariants of each layer."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu_oracle as orc
+from tests.parity import TOL_F16, TOL_F32, check
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def L():
+    from lbann_amd import layers
+    layers.capi.lib()
+    assert torch.cuda.is_available()
+    return layers
+
+
+@pytest.fixture(scope="module")
+def W():
+    from lbann_amd import workloads
+    return workloads
+
+
+def f64(a):
+    return np.asfortranarray(np.asarray(a, dtype=np.float64))
+
+
+def f32(a):
+    return np.asfortranarray(np.asarray(a, dtype=np.float32))
+
+
+def test_cfg1_layer_norm_1024x128(L, W):
+    d = W.cfg1_layer_norm()
+    x, dy = f32(d["x"]), f32(d["dy"])
+    ln = L.layer_norm_layer(d["dims"], d["eps"], True, True, 0, d["scale"], d["bias"])
+    y = ln.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    dx = ln.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+    y_ref, st = orc.layer_norm_fwd(x, 1, 1024, 1024, 1e-5, d["scale"], d["bias"])
+    y_ex, st_ex = orc.layer_norm_fwd(f64(x), 1, 1024, 1024, 1e-5, f64(d["scale"]), f64(d["bias"]))
+    dx_ref, sg, dg, db = orc.layer_norm_bwd(x, dy, st, 1, 1024, 1024, 1e-5, d["scale"], True, True)
+    dx_ex, sg_ex, dg_ex, db_ex = orc.layer_norm_bwd(f64(x), f64(dy), st_ex, 1, 1024, 1024, 1e-5, f64(d["scale"]), True, True)
+    check("cfg1 y", y, y_ref, y_ex)
+    check("cfg1 stats", ln.m_statistics.to_numpy(), st, st_ex)
+    check("cfg1 dx", dx, dx_ref, dx_ex)
+    check("cfg1 stats grad", ln.m_statistics_gradient.to_numpy(), sg, sg_ex)
+    check("cfg1 dscale", ln.m_scale_gradient.to_numpy(), dg, dg_ex)
+    check("cfg1 dbias", ln.m_bias_gradient.to_numpy(), db, db_ex)
+    # scale 1, bias 0: every output column has zero mean and second moment var/(var+eps)
+    assert np.abs(y.astype(np.float64).mean(axis=0)).max() < 1e-6
+    assert np.abs(dx.astype(np.float64).sum(axis=0)).max() < 1e-3
+
+
+@pytest.mark.parametrize("kind", ["softmax", "log_softmax"])
+def test_cfg2_softmax_32768x512(L, W, kind):
+    d = W.cfg2_softmax()
+    x, dy = d["x"], f32(d["dy"])
+    layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
+    fwd, bwd = ((orc.softmax_fwd, orc.softmax_bwd) if kind == "softmax" else (orc.log_softmax_fwd, orc.log_softmax_bwd))
+    y = layer.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+    check(f"cfg2 {kind} y", y, fwd(x), fwd(f64(x)))
+    check(f"cfg2 {kind} dx", dx, bwd(y, dy), bwd(f64(y), f64(dy)))
+    y64 = y.astype(np.float64)
+    if kind == "softmax":
+        assert np.abs(y64.sum(axis=0) - 1).max() < 1e-5
+        assert np.abs(dx.astype(np.float64).sum(axis=0)).max() < 1e-4
+        assert (x == 30).sum() > 100000 and y[x == 30].min() > 1e-3   # the +30 entries carry the mass
+    else:
+        assert np.abs(np.exp(y64).sum(axis=0) - 1).max() < 1e-5
+
+
+@pytest.mark.parametrize("bessel", [True, False])
+def test_cfg3_batch_norm_64x256x56x56(L, W, bessel):
+    d = W.cfg3_batch_norm()
+    x, dy = f32(d["x"]), f32(d["dy"])
+    C, cs = 256, 56 * 56
+    bn = L.batch_normalization_layer(d["dims"], d["decay"], d["eps"], bessel, d["scale"], d["bias"])
+    y = bn.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    dx = bn.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+    mv, mvg = bn.m_mean_and_var.to_numpy(), bn.m_mean_and_var_gradient.to_numpy()
+    out = dict(y=y, dx=dx, mean=mv[:, 0], var=mv[:, 1], dmean=mvg[:, 0], dvar=mvg[:, 1],
+               dscale=bn.m_scale_gradient.to_numpy(), dbias=bn.m_bias_gradient.to_numpy(),
+               rmean=bn.weights[2].to_numpy(), rvar=bn.weights[3].to_numpy())
+    del bn
+    torch.cuda.empty_cache()
+    res = {}
+    for tag, conv in (("ref", f32), ("ex", f64)):
+        rm, rv = conv(np.zeros(C)), conv(np.ones(C))
+        r = {}
+        r["y"], r["mean"], r["var"] = orc.batch_norm_fwd(conv(x), C, cs, 1e-5, 0.9, conv(d["scale"]), conv(d["bias"]), rm, rv, bessel)
+        r["rmean"], r["rvar"] = rm, rv
+        r["dx"], r["dscale"], r["dbias"], r["dmean"], r["dvar"] = orc.batch_norm_bwd(
+            conv(x), conv(dy), C, cs, 1e-5, r["mean"], r["var"], conv(d["scale"]), bessel=bessel)
+        res[tag] = r
+    for k in out:
+        check(f"cfg3 {k}", out[k], res["ref"][k], res["ex"][k])
+    # every channel's input gradient sums to zero; y has the channel's bias as its mean
+    dxs = dx.astype(np.float64).reshape(cs, C, 64, order="F").sum(axis=(0, 2))
+    assert np.abs(dxs).max() < 0.05
+    ym = y.astype(np.float64).reshape(cs, C, 64, order="F").mean(axis=(0, 2))
+    assert np.abs(ym - d["bias"]).max() < 1e-5
+
+
+def test_cfg4_layer_norm_f16_4096x8192(L, W):
+    d = W.cfg4_layer_norm_f16()
+    x16, dy16 = d["x"], d["dy"]
+    x, dy = f32(x16), f32(dy16)      # the fp16-rounded values, which both sides see
+    n = 4096
+    ln = L.layer_norm_layer(d["dims"], d["eps"], True, True, 0, d["scale"], d["bias"])
+    y = ln.forward(L.DeviceMatrix.from_numpy(x16)).to_numpy()
+    dx = ln.backward(L.DeviceMatrix.from_numpy(dy16)).to_numpy()
+    stats, sgrad = ln.m_statistics.to_numpy(), ln.m_statistics_gradient.to_numpy()
+    dg, db = ln.m_scale_gradient.to_numpy(), ln.m_bias_gradient.to_numpy()
+    y_ref, st = orc.layer_norm_fwd(x, 1, n, n, 1e-5, d["scale"], d["bias"])
+    y_ex, st_ex = orc.layer_norm_fwd(f64(x), 1, n, n, 1e-5, f64(d["scale"]), f64(d["bias"]))
+    # mean to fp32 accuracy; variance, outputs and gradients are where the fp32 reference's
+    # E[x^2]-mean^2 cancels for |mean| >> stdev columns: judged against float64 there
+    check("cfg4 mean", stats[0], st[0], st_ex[0])
+    check("cfg4 var", stats[1], st[1], st_ex[1])
+    check("cfg4 y", y, y_ref, y_ex, tol=TOL_F16)
+    # backward against the oracle run on the GPU's own (more accurate) statistics, and on float64
+    dx_ref, sg_ref, dg_ref, db_ref = orc.layer_norm_bwd(x, dy, f32(stats), 1, n, n, 1e-5, d["scale"], True, True)
+    dx_ex, sg_ex, dg_ex, db_ex = orc.layer_norm_bwd(f64(x), f64(dy), st_ex, 1, n, n, 1e-5, f64(d["scale"]), True, True)
+    check("cfg4 dx", dx, dx_ref, dx_ex, tol=TOL_F16)
+    check("cfg4 stats grad", sgrad, sg_ref, sg_ex, tol=TOL_F16)
+    check("cfg4 dscale", dg, dg_ref, dg_ex, tol=TOL_F16)
+    check("cfg4 dbias", db, db_ref, db_ex, tol=TOL_F16)
+    assert np.isfinite(y).all() and np.isfinite(dx).all()
+
+
+def test_cfg5a_channelwise_softmax_256x64x4096(L, W):
+    d = W.cfg5a_channelwise_softmax()
+    x, dy = f32(d["x"]), f32(d["dy"])
+    C, S = d["dims"]
+    layer = L.channelwise_softmax_layer(d["dims"])
+    y = layer.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+    del layer
+    torch.cuda.empty_cache()
+    check("cfg5a y", y, orc.channelwise_softmax_fwd(x, C, S, S), orc.channelwise_softmax_fwd(f64(x), C, S, S))
+    check("cfg5a dx", dx, orc.channelwise_softmax_bwd(y, dy, C, S, S), orc.channelwise_softmax_bwd(f64(y), f64(dy), C, S, S))
+    sums = y.astype(np.float64).reshape(S, -1, order="F").sum(axis=0)
+    assert np.abs(sums - 1).max() < 1e-5
+
+
+def test_cfg5b_wide_softmax_262144x16(L, W):
+    d = W.cfg5b_wide_softmax()
+    x, dy = f32(d["x"]), f32(d["dy"])
+    layer = L.softmax_layer()
+    y = layer.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+    check("cfg5b y", y, orc.softmax_fwd(x), orc.softmax_fwd(f64(x)))
+    check("cfg5b dx", dx, orc.softmax_bwd(y, dy), orc.softmax_bwd(f64(y), f64(dy)))
+    assert np.abs(y.astype(np.float64).sum(axis=0) - 1).max() < 1e-5
+    # in place gives the same bits
+    xm = L.DeviceMatrix.from_numpy(x)
+    layer.forward(xm, in_place=True)
+    assert np.array_equal(xm.to_numpy(), y)
