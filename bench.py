@@ -55,8 +55,11 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
 
+    ld_pad = int(os.environ.get("LBN_BENCH_LDPAD", "0"))  # experiment knob: leading dimension = height + pad
+
     def upload(a, half=False):
-        return L.DeviceMatrix.from_numpy(a, dtype=torch.float16 if half else None)
+        return L.DeviceMatrix.from_numpy(a, dtype=torch.float16 if half else None,
+                                         ldim=a.shape[0] + ld_pad if ld_pad else None)
 
     # ---- workload table: name -> builder returning (fwd, bwd, elements, elem_size, samples, cpu_fn)
     def build_softmax(kind, data):

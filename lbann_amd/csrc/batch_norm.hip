@@ -54,8 +54,9 @@ bn_fwd_sums(const float* __restrict__ x, int64_t ldx, int64_t cs, int64_t w, int
   float s = 0.f, q = 0.f;
   const int64_t step = static_cast<int64_t>(P) * kBnThreads;
   for (int64_t j = static_cast<int64_t>(p) * kBnThreads + threadIdx.x; j < wk.total; j += step) {
-    const int64_t col = j / wk.seg;
-    const int64_t i = j - col * wk.seg;
+    const unsigned ucol = static_cast<unsigned>(j) / static_cast<unsigned>(wk.seg);  // j < 2^32 (host check)
+    const int64_t col = ucol;
+    const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(wk.seg);
     if (VEC) {
       float v[4];
       Vec16<float>::load(xc + col * ldx + 4 * i, v);
@@ -183,8 +184,9 @@ bn_fwd_apply(const float* __restrict__ x, float* __restrict__ y, int64_t ldx, in
   const float bias = beta[c];
   const int64_t step = static_cast<int64_t>(P) * kBnThreads;
   for (int64_t j = static_cast<int64_t>(p) * kBnThreads + threadIdx.x; j < wk.total; j += step) {
-    const int64_t col = j / wk.seg;
-    const int64_t i = j - col * wk.seg;
+    const unsigned ucol = static_cast<unsigned>(j) / static_cast<unsigned>(wk.seg);  // j < 2^32 (host check)
+    const int64_t col = ucol;
+    const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(wk.seg);
     if (VEC) {
       float v[4];
       Vec16<float>::load(xc + col * ldx + 4 * i, v);
@@ -216,8 +218,9 @@ bn_bwd_sums(const float* __restrict__ x, const float* __restrict__ dy, int64_t l
   float a = 0.f, b = 0.f;
   const int64_t step = static_cast<int64_t>(P) * kBnThreads;
   for (int64_t j = static_cast<int64_t>(p) * kBnThreads + threadIdx.x; j < wk.total; j += step) {
-    const int64_t col = j / wk.seg;
-    const int64_t i = j - col * wk.seg;
+    const unsigned ucol = static_cast<unsigned>(j) / static_cast<unsigned>(wk.seg);  // j < 2^32 (host check)
+    const int64_t col = ucol;
+    const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(wk.seg);
     if (VEC) {
       float v[4], g[4];
       Vec16<float>::load(xc + col * ldx + 4 * i, v);
@@ -314,8 +317,9 @@ bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ dy, float* _
   const float dvar_term = dvar * 2.f / static_cast<float>(num_per_sum - (bessel ? 1 : 0));
   const int64_t step = static_cast<int64_t>(P) * kBnThreads;
   for (int64_t j = static_cast<int64_t>(p) * kBnThreads + threadIdx.x; j < wk.total; j += step) {
-    const int64_t col = j / wk.seg;
-    const int64_t i = j - col * wk.seg;
+    const unsigned ucol = static_cast<unsigned>(j) / static_cast<unsigned>(wk.seg);  // j < 2^32 (host check)
+    const int64_t col = ucol;
+    const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(wk.seg);
     if (VEC) {
       float v[4], g[4];
       if (!zero) {
@@ -764,6 +768,7 @@ static int bn_check(int64_t C, int64_t cs, int64_t w, const int64_t* lds, int nl
   for (int i = 0; i < nld; ++i)
     if (w > 1 && lds[i] < C * cs) return LBN_ERR_INVALID_ARGUMENT;
   if (C > 65535) return LBN_ERR_UNSUPPORTED;  // channels ride on gridDim.y
+  if (cs * w >= (int64_t(1) << 32)) return LBN_ERR_UNSUPPORTED;  // per-channel index fits 32 bits
   return LBN_OK;
 }
 

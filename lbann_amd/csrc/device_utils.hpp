@@ -26,13 +26,34 @@ __device__ __forceinline__ int64_t imin64(int64_t a, int64_t b) { return a < b ?
 struct RowMap {
   int64_t groups;
   int64_t stride;
+  // Column and group of a row.  Row and group counts stay below 2^31 (checked on the
+  // host), so the division is a 32-bit one; whole-column rows skip it altogether.
+  __device__ __forceinline__ void split(int64_t row, int64_t& col, int64_t& g) const
+  {
+    if (groups == 1) {
+      col = row;
+      g = 0;
+    }
+    else {
+      const unsigned c = static_cast<unsigned>(row) / static_cast<unsigned>(groups);
+      col = c;
+      g = static_cast<unsigned>(row) - c * static_cast<unsigned>(groups);
+    }
+  }
   __device__ __forceinline__ int64_t offset(int64_t row, int64_t ld) const
   {
-    const int64_t col = row / groups;
-    const int64_t g = row - col * groups;
+    int64_t col, g;
+    split(row, col, g);
     return g * stride + col * ld;
   }
 };
+
+// Index of the calling wave inside its block, as a wave-uniform (scalar) value: row
+// indices and row base addresses derived from it stay in scalar registers.
+__device__ __forceinline__ int wave_index()
+{
+  return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWave);
+}
 
 // ---------------------------------------------------------------------------
 // 16-byte vector access for the two storage types.  Values are always widened to
@@ -56,11 +77,32 @@ struct Vec16<float> {
   }
   static __device__ __forceinline__ float load1(const float* p) { return *p; }
   static __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
+  // raw 16-byte register image of a vector (for software prefetch) and its widening
+  using raw_t = v4f;
+  static __device__ __forceinline__ raw_t load_raw(const float* p) { return *reinterpret_cast<const v4f*>(p); }
+  static __device__ __forceinline__ void unpack(const raw_t& r, float (&v)[4])
+  {
+    v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+  }
 };
 
 template <>
 struct Vec16<__half> {
   static constexpr int N = 8;
+  using raw_t = v4u;
+  static __device__ __forceinline__ raw_t load_raw(const __half* p) { return *reinterpret_cast<const v4u*>(p); }
+  static __device__ __forceinline__ void unpack(const raw_t& r, float (&v)[8])
+  {
+    const unsigned int w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __half2 h;
+      __builtin_memcpy(&h, &w[i], 4);
+      const float2 f = __half22float2(h);
+      v[2 * i] = f.x;
+      v[2 * i + 1] = f.y;
+    }
+  }
   static __device__ __forceinline__ void load(const __half* p, float (&v)[8])
   {
     const v4u r = *reinterpret_cast<const v4u*>(p);
@@ -118,19 +160,49 @@ __device__ __forceinline__ float exp_keep_denormals(float x)
   return tiny ? e * 5.42101086e-20f : e;                      // 2^-64
 }
 
+// 1/sqrt(v) for v > 0 from v_rsq_f32 and one Newton step (about 1 ulp), 5 operations
+// instead of the ~35 of a correctly rounded square root followed by a division.
+__device__ __forceinline__ float rsqrt_refined(float v)
+{
+  const float y = __builtin_amdgcn_rsqf(v);
+  const float h = 0.5f * v;
+  return __builtin_fmaf(y, __builtin_fmaf(-h * y, y, 0.5f), y);
+}
+
 // ---------------------------------------------------------------------------
-// Wave64 butterfly reductions: every lane ends with the result.
+// Wave64 reductions on the DPP data path (no LDS traffic): four cross-lane steps fold
+// every row of 16 lanes (quad swap, quad-pair swap, half-row mirror, row mirror), then
+// the four row results are read through scalar registers.  Every lane gets the result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v)
+{
+  return __builtin_bit_cast(
+    float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float read_lane(float v, int lane)
+{
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+constexpr int kDppQuadSwap1 = 0xB1;     // quad_perm:[1,0,3,2]
+constexpr int kDppQuadSwap2 = 0x4E;     // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;   // row_half_mirror
+constexpr int kDppRowMirror = 0x140;    // row_mirror
+
 __device__ __forceinline__ float wave_sum(float v)
 {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-  return v;
+  v += dpp_move<kDppQuadSwap1>(v);
+  v += dpp_move<kDppQuadSwap2>(v);
+  v += dpp_move<kDppHalfMirror>(v);
+  v += dpp_move<kDppRowMirror>(v);
+  return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
 }
 __device__ __forceinline__ float wave_max(float v)
 {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-  return v;
+  v = fmaxf(v, dpp_move<kDppQuadSwap1>(v));
+  v = fmaxf(v, dpp_move<kDppQuadSwap2>(v));
+  v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_move<kDppRowMirror>(v));
+  return fmaxf(fmaxf(read_lane(v, 0), read_lane(v, 16)), fmaxf(read_lane(v, 32), read_lane(v, 48)));
 }
 
 // Reductions over a team of NW waves (NW*64 consecutive threads of the block).

@@ -36,7 +36,7 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
   constexpr int NW = B::kWavesPerTeam;
   __shared__ float red[2][2 * NW];
   const int tid = threadIdx.x;
-  const int team = tid / TPR;
+  const int team = wave_index() / NW;  // wave-uniform: a team is a whole number of waves
   const int t = tid - team * TPR;
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
@@ -97,8 +97,8 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
   const float inv_stdev = 1.0f / sqrtf(var + eps);
 
   if (t == 0) {
-    const int64_t col = row / map.groups;
-    const int64_t g = row - col * map.groups;
+    int64_t col, g;
+    map.split(row, col, g);
     stats[g + col * ld_stats] = mean;
     stats[map.groups + g + col * ld_stats] = var;
   }
@@ -177,8 +177,8 @@ ln_fwd_generic(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t 
   }
   const float inv_stdev = 1.0f / sqrtf(var + eps);
   if (threadIdx.x == 0) {
-    const int64_t col = row / map.groups;
-    const int64_t g = row - col * map.groups;
+    int64_t col, g;
+    map.split(row, col, g);
     stats[g + col * ld_stats] = mean;
     stats[map.groups + g + col * ld_stats] = var;
   }
@@ -194,7 +194,16 @@ ln_fwd_generic(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t 
 // ================================================================== backward
 // Partial weight gradients: block b writes 2*n floats at part + b*2*n (dscale row
 // followed by dbias row).
-template <typename T, int TPR, int TEAMS, int V, bool WGRAD>
+//
+// Per element the kernel spends 9 VALU operations before the row reduction and 4
+// after it: with xh = (x - mean) / stdev,
+//   dbias += dy;  dscale += dy * xh;  gs = dy * scale;  A += gs;  B += gs * xh
+//   dx = gs / stdev + dmean / n + (dvar * 2 * stdev / n) * xh
+// where dmean = -A / stdev and dvar = -B / (2 stdev^2)  (layer_norm.cpp:198-257).
+//
+// DEPTH > 0: the still-packed 16-byte images of the next DEPTH rows of a team are in
+// flight while the current row is processed.
+template <typename T, int TPR, int TEAMS, int V, bool WGRAD, int DEPTH>
 __global__ void __launch_bounds__((RowBlock<TPR, TEAMS>::kThreads))
 ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ dx, int64_t ldx,
             int64_t lddy, int64_t lddx, RowMap map, int64_t rows, int nvec, int n, float eps,
@@ -203,13 +212,15 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
 {
   using B = RowBlock<TPR, TEAMS>;
   using IO = Vec16<T>;
+  using raw_t = typename IO::raw_t;
   constexpr int VE = IO::N;
   constexpr int NW = B::kWavesPerTeam;
   constexpr int kAccLds = (WGRAD && TEAMS > 1) ? 2 * TPR * V * VE : 1;
+  constexpr int NQ = DEPTH > 0 ? DEPTH : 1;
   __shared__ float red[2][TEAMS][2 * NW];
   __shared__ float acc_lds[kAccLds];
   const int tid = threadIdx.x;
-  const int team = tid / TPR;
+  const int team = wave_index() / NW;  // wave-uniform: a team is a whole number of waves
   const int t = tid - team * TPR;
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
@@ -238,72 +249,109 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
       for (int k = 0; k < VE; ++k) dg[i][k] = db[i][k] = 0.f;
   }
 
-  const float nf = static_cast<float>(n);
-  const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * TEAMS;
-  const int64_t iters = (rows + rows_per_iter - 1) / rows_per_iter;
-  for (int64_t it = 0; it < iters; ++it) {
-    const int64_t row = it * rows_per_iter + static_cast<int64_t>(blockIdx.x) * TEAMS + team;
-    const bool active = row < rows;
-    float xv[V][VE], gv[V][VE];
-    float mean = 0.f, inv_stdev = 0.f;
-    int64_t col = 0, g = 0;
-    if (active) {
-      col = row / map.groups;
-      g = row - col * map.groups;
+  raw_t qx[NQ][V], qg[NQ][V];  // rows in flight, packed
+  // All row arithmetic is wave-uniform (scalar registers).
+  auto issue = [&](raw_t (&rx)[V], raw_t (&rg)[V], int64_t row) {
+    if (row < rows) {
+      int64_t col, g;
+      map.split(row, col, g);
       const T* xr = x + g * map.stride + col * ldx;
       const T* gr = dy + g * map.stride + col * lddy;
 #pragma unroll
       for (int i = 0; i < V; ++i) {
         const int idx = t + i * TPR;
         if (idx < nvec) {
-          IO::load(xr + VE * idx, xv[i]);
-          IO::load(gr + VE * idx, gv[i]);
-        }
-        else {
-#pragma unroll
-          for (int k = 0; k < VE; ++k) xv[i][k] = gv[i][k] = 0.f;
+          rx[i] = IO::load_raw(xr + VE * idx);
+          rg[i] = IO::load_raw(gr + VE * idx);
         }
       }
-      mean = stats[g + col * ld_stats];
-      inv_stdev = 1.0f / sqrtf(stats[map.groups + g + col * ld_stats] + eps);
     }
+  };
+
+  const float inv_n = 1.0f / static_cast<float>(n);
+  const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * TEAMS;
+  const int64_t iters = (rows + rows_per_iter - 1) / rows_per_iter;
+  const int64_t first_row = static_cast<int64_t>(blockIdx.x) * TEAMS + team;
+  if (DEPTH > 0) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) issue(qx[d], qg[d], first_row + d * rows_per_iter);
+  }
+  for (int64_t it = 0; it < iters; ++it) {
+    const int64_t row = it * rows_per_iter + first_row;
+    const bool active = row < rows;
+    raw_t cx[V], cg[V];
+    if (DEPTH > 0) {
+      // take the oldest row in flight, shift the queue, refill its tail
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        cx[i] = qx[0][i];
+        cg[i] = qg[0][i];
+      }
+#pragma unroll
+      for (int d = 0; d + 1 < DEPTH; ++d)
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          qx[d][i] = qx[d + 1][i];
+          qg[d][i] = qg[d + 1][i];
+        }
+      issue(qx[DEPTH - 1], qg[DEPTH - 1], row + DEPTH * rows_per_iter);
+    }
+    else {
+      issue(cx, cg, row);
+    }
+    float inv_stdev = 0.f, mean = 0.f;
+    int64_t col = 0, g = 0;
+    if (active) {
+      map.split(row, col, g);
+      mean = stats[g + col * ld_stats];
+      inv_stdev = rsqrt_refined(stats[map.groups + g + col * ld_stats] + eps);
+    }
+    float xh[V][VE], gs[V][VE];
     float a = 0.f, b = 0.f;
     if (active) {
 #pragma unroll
       for (int i = 0; i < V; ++i) {
-        const bool ok = (t + i * TPR) < nvec;
+        if (t + i * TPR < nvec) {
+          float xv[VE], gv[VE];
+          IO::unpack(cx[i], xv);
+          IO::unpack(cg[i], gv);
 #pragma unroll
-        for (int k = 0; k < VE; ++k) {
-          const float xc = ok ? xv[i][k] - mean : 0.f;
-          xv[i][k] = xc;
-          if (WGRAD) {
-            db[i][k] += gv[i][k];
-            dg[i][k] += gv[i][k] * xc * inv_stdev;
+          for (int k = 0; k < VE; ++k) {
+            xh[i][k] = (xv[k] - mean) * inv_stdev;  // subtract first: x*inv - mean*inv would cancel
+            if (WGRAD) {
+              db[i][k] += gv[k];
+              dg[i][k] = __builtin_fmaf(gv[k], xh[i][k], dg[i][k]);
+            }
+            gs[i][k] = gv[k] * gam[i][k];
+            a += gs[i][k];
+            b = __builtin_fmaf(gs[i][k], xh[i][k], b);
           }
-          gv[i][k] *= gam[i][k];
-          a += gv[i][k];
-          b += gv[i][k] * xc;
+        }
+        else {
+#pragma unroll
+          for (int k = 0; k < VE; ++k) xh[i][k] = gs[i][k] = 0.f;
         }
       }
     }
     team_sum2<NW>(a, b, red[it & 1][team], wv, lane);
     if (active) {
       const float dmean = -a * inv_stdev;
-      const float dvar = -b * inv_stdev * inv_stdev * inv_stdev / 2;
+      const float dvar = -b * inv_stdev * inv_stdev * 0.5f;
       if (t == 0) {
         sgrad[g + col * ld_sgrad] = dmean;
         sgrad[map.groups + g + col * ld_sgrad] = dvar;
       }
-      const float c0 = dmean / nf;
-      const float c1 = dvar * 2.f / nf;
+      const float c0 = dmean * inv_n;
+      const float c1 = -b * inv_stdev * inv_n;  // dvar * 2 / n, per unit of xh = (x - mean) / stdev
       T* dr = dx + g * map.stride + col * lddx;
 #pragma unroll
       for (int i = 0; i < V; ++i) {
         const int idx = t + i * TPR;
         if (idx < nvec) {
 #pragma unroll
-          for (int k = 0; k < VE; ++k) gv[i][k] = gv[i][k] * inv_stdev + c0 + c1 * xv[i][k];
-          IO::store(dr + VE * idx, gv[i]);
+          for (int k = 0; k < VE; ++k)
+            gs[i][k] = __builtin_fmaf(gs[i][k], inv_stdev, __builtin_fmaf(c1, xh[i][k], c0));
+          IO::store(dr + VE * idx, gs[i]);
         }
       }
     }
@@ -409,8 +457,8 @@ ln_bwd_generic(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict_
   const int lane = threadIdx.x & (kWave - 1);
   const int wv = threadIdx.x / kWave;
   const int64_t row = blockIdx.x;
-  const int64_t col = row / map.groups;
-  const int64_t g = row - col * map.groups;
+  int64_t col, g;
+  map.split(row, col, g);
   const T* xr = x + g * map.stride + col * ldx;
   const T* gr = dy + g * map.stride + col * lddy;
   T* dr = dx + g * map.stride + col * lddx;
@@ -453,8 +501,8 @@ ln_wgrad_generic(const T* __restrict__ x, const T* __restrict__ dy, int64_t ldx,
   if (k >= n) return;
   float sg = 0.f, sb = 0.f;
   for (int64_t row = 0; row < rows; ++row) {
-    const int64_t col = row / map.groups;
-    const int64_t g = row - col * map.groups;
+    int64_t col, g;
+    map.split(row, col, g);
     const float mean = stats[g + col * ld_stats];
     const float inv_stdev = 1.0f / sqrtf(stats[map.groups + g + col * ld_stats] + eps);
     const float d = IO::load1(dy + g * map.stride + col * lddy + k);
@@ -482,6 +530,7 @@ fill_matrix(T* p, int64_t h, int64_t w, int64_t ld, float value)
 struct LnBwdPlan {
   int tpr, teams, v;
   int64_t blocks;  // == number of partial rows
+  int depth;       // rows in flight per team
 };
 
 // At most this many persistent blocks: each leaves 2*n floats of partial sums, so
@@ -490,30 +539,40 @@ constexpr int64_t kLnBwdMaxBlocks = 256;
 
 static LnBwdPlan plan_ln_bwd(int64_t nvec, int64_t rows, int ve)
 {
-  // per-thread registers hold x, dy, gamma and two accumulators: keep v <= 4 (fp32)
-  // or v <= 2 (fp16, 8 entries per vector)
+  static const int force_depth = std::getenv("LBN_LN_BWD_DEPTH") ? std::atoi(std::getenv("LBN_LN_BWD_DEPTH")) : -1;
+  static const int force_tpr = std::getenv("LBN_LN_BWD_TPR") ? std::atoi(std::getenv("LBN_LN_BWD_TPR")) : 0;
+  static const int force_teams = std::getenv("LBN_LN_BWD_TEAMS") ? std::atoi(std::getenv("LBN_LN_BWD_TEAMS")) : 0;
+  static const int64_t max_blocks = std::getenv("LBN_LN_BWD_BLOCKS") ? std::atoi(std::getenv("LBN_LN_BWD_BLOCKS")) : kLnBwdMaxBlocks;
+  // Registers per thread: two fp32 accumulators per owned entry plus the packed rows
+  // in flight.  Few vectors per thread leave room for a deeper prefetch, so the
+  // widest team that still keeps every thread busy is preferred.
+  LnBwdPlan p{0, 0, 0, 0, 0};
+  const int tprs[4] = {64, 256, 512, 1024};
+  const int teams[4] = {4, 4, 2, 1};
   const int max_v = ve == 8 ? 2 : 4;
-  LnBwdPlan p{0, 0, 0, 0};
-  if (ceil_div(nvec, 64) <= max_v) {
-    p.tpr = 64;
-    p.teams = 4;
+  int pick = -1;
+  for (int i = 0; i < 4; ++i) {
+    if (force_tpr && tprs[i] != force_tpr) continue;
+    const int64_t v = ceil_div(nvec, tprs[i]);
+    if (v > max_v) continue;
+    if (pick < 0) pick = i;
+    // prefer one vector per thread when the wider team is still fully used
+    if (v == 1 && nvec * 2 > tprs[i]) { pick = i; break; }
   }
-  else if (ceil_div(nvec, 256) <= max_v) {
-    p.tpr = 256;
-    p.teams = 4;
-  }
-  else if (ceil_div(nvec, 1024) <= max_v) {
-    p.tpr = 1024;
-    p.teams = 1;
-  }
-  else {
-    return p;
-  }
+  if (pick < 0) return p;
+  p.tpr = tprs[pick];
+  p.teams = teams[pick];
   p.v = round_up_pow2_le8(ceil_div(nvec, p.tpr));
+  if (p.tpr == 512 && p.v > 1) p.teams = 1;  // two such teams would not fit their LDS merge buffer
+  if (force_teams && force_teams <= p.teams) p.teams = force_teams;
   // spread small problems: fewer teams per block when rows are scarce
-  while (p.teams > 1 && p.tpr * p.teams > 256 && ceil_div(rows, p.teams) < kLnBwdMaxBlocks) p.teams /= 2;
+  while (p.teams > 1 && p.tpr * p.teams > 256 && ceil_div(rows, p.teams) < max_blocks) p.teams /= 2;
   p.blocks = ceil_div(rows, p.teams);
-  if (p.blocks > kLnBwdMaxBlocks) p.blocks = kLnBwdMaxBlocks;
+  if (p.blocks > max_blocks) p.blocks = max_blocks;
+  const int64_t rows_per_team = ceil_div(rows, p.blocks * p.teams);
+  p.depth = p.v == 1 ? 3 : (p.v == 2 ? 1 : 0);
+  if (rows_per_team <= 1) p.depth = 0;
+  if (force_depth >= 0 && force_depth <= 3) p.depth = p.v > 2 ? 0 : (p.v == 2 && force_depth > 1 ? 1 : force_depth);
   return p;
 }
 
@@ -566,7 +625,7 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
   return launch_status();
 }
 
-template <typename T, int TPR, int TEAMS, int V>
+template <typename T, int TPR, int TEAMS, int V, int DEPTH>
 static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const T* x, const T* dy,
                                T* dx, int64_t ldx, int64_t lddy, int64_t lddx, RowMap map,
                                int64_t rows, int nvec, int n, float eps, const float* stats,
@@ -576,10 +635,10 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
   using B = RowBlock<TPR, TEAMS>;
   const dim3 grid(static_cast<unsigned>(blocks)), block(B::kThreads);
   if (wgrad)
-    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, true>), grid, block, 0, st, x, dy, dx, ldx,
+    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, true, DEPTH>), grid, block, 0, st, x, dy, dx, ldx,
                        lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part);
   else
-    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, false>), grid, block, 0, st, x, dy, dx, ldx,
+    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, false, 0>), grid, block, 0, st, x, dy, dx, ldx,
                        lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part);
 }
 
@@ -632,16 +691,20 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
       }
       const int nvec = static_cast<int>(n / VE);
       bool launched = false;
-#define X(TPR, TEAMS, V)                                                                        \
-  if (!launched && p.tpr == TPR && p.teams == TEAMS && p.v == V) {                              \
-    launch_ln_bwd_rows<T, TPR, TEAMS, V>(st, wgrad, p.blocks, x, dy, dx, ldx, lddy, lddx, map,  \
-                                         rows, nvec, static_cast<int>(n), eps, stats, lds,      \
-                                         sgrad, ldsg, gamma, part);                             \
+#define X(TPR, TEAMS, V, D)                                                                     \
+  if (!launched && p.tpr == TPR && p.teams == TEAMS && p.v == V && p.depth == D) {              \
+    launch_ln_bwd_rows<T, TPR, TEAMS, V, D>(st, wgrad, p.blocks, x, dy, dx, ldx, lddy, lddx,    \
+                                            map, rows, nvec, static_cast<int>(n), eps, stats,   \
+                                            lds, sgrad, ldsg, gamma, part);                     \
     launched = true;                                                                            \
   }
-      X(64, 4, 1) X(64, 4, 2) X(256, 1, 1) X(256, 1, 2) X(256, 2, 1) X(256, 2, 2) X(256, 4, 1)
-      X(256, 4, 2) X(1024, 1, 1) X(1024, 1, 2)
-      if constexpr (VE == 4) { X(64, 4, 4) X(256, 1, 4) X(256, 2, 4) X(256, 4, 4) X(1024, 1, 4) }
+#define XD(TPR, TEAMS, V) X(TPR, TEAMS, V, 0) X(TPR, TEAMS, V, 1) X(TPR, TEAMS, V, 2) X(TPR, TEAMS, V, 3)
+#define XS(TPR, TEAMS, V) X(TPR, TEAMS, V, 0) X(TPR, TEAMS, V, 1)
+      XD(64, 4, 1) XS(64, 4, 2) XD(256, 1, 1) XS(256, 1, 2) XD(256, 2, 1) XS(256, 2, 2) XD(256, 4, 1)
+      XS(256, 4, 2) XD(512, 1, 1) XS(512, 1, 2) XD(512, 2, 1) XD(1024, 1, 1) XS(1024, 1, 2)
+      if constexpr (VE == 4) { X(64, 4, 4, 0) X(256, 1, 4, 0) X(256, 2, 4, 0) X(256, 4, 4, 0) X(512, 1, 4, 0) X(1024, 1, 4, 0) }
+#undef XS
+#undef XD
 #undef X
       if (launched) {
         if (wgrad) {

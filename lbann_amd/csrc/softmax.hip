@@ -5,7 +5,7 @@
 //
 //  * register-resident row kernels: TPR threads (one wave, 256 or 1024 threads)
 //    load a whole row with 128-bit coalesced loads, keep it in registers, reduce
-//    with wave64 shuffles (+ one LDS hop across waves), and store the result.
+//    on the wave64 DPP path (+ one LDS hop across waves), and store the result.
 //    Each tensor is read once and written once.  Used when rows are 16-byte
 //    aligned, a multiple of 4 long and at most 32768 entries.
 //  * split ("chunked") kernels for very long or unaligned rows: a row is cut into
@@ -37,7 +37,7 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
   constexpr int NW = B::kWavesPerTeam;
   __shared__ float red[2][NW];
   const int tid = threadIdx.x;
-  const int team = tid / TPR;
+  const int team = wave_index() / NW;  // wave-uniform: a team is a whole number of waves
   const int t = tid - team * TPR;
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
@@ -58,13 +58,15 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
     }
   }
 
-  // column maximum, starting from the lowest finite float like the reference
-  float m = -FLT_MAX;
+  // Thread-local pass first: every thread takes the maximum of its own entries and
+  // exponentiates against it as soon as its own loads have landed, without waiting
+  // for the rest of the row; the (max, sum) pairs are then merged wave -> team with
+  // a single barrier, and each thread rescales by exp(own max - row max) / row sum.
+  float m = -FLT_MAX;  // starts from the lowest finite float like the reference
 #pragma unroll
   for (int i = 0; i < V; ++i)
 #pragma unroll
     for (int k = 0; k < 4; ++k) m = fmaxf(m, v[i][k]);
-  m = team_max<NW>(m, red[0], wv, lane);
 
   float s = 0.f;
 #pragma unroll
@@ -78,11 +80,26 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
       v[i][k] = (KIND == kLogSoftmax) ? d : e;
     }
   }
-  s = team_sum<NW>(s, red[1], wv, lane);
+
+  // wave merge on the DPP path, then one LDS hop across the waves of the team
+  float gm = wave_max(m);
+  float gs = wave_sum(s * exp_fast(m - gm));
+  if (NW > 1) {
+    if (lane == 0) {
+      red[0][wv] = gm;
+      red[1][wv] = gs;
+    }
+    __syncthreads();
+    const float pm = lane < NW ? red[0][lane] : -FLT_MAX;
+    const float ps = lane < NW ? red[1][lane] : 0.f;
+    gm = wave_max(pm);
+    gs = wave_sum(ps * exp_fast(pm - gm));
+  }
 
   float* yr = y + map.offset(row, ldy);
-  const float scale = 1.0f / s;
-  const float lse = (KIND == kLogSoftmax) ? logf(s) : 0.f;
+  const float shift = m - gm;  // <= 0
+  const float f = exp_fast(shift) * (1.0f / gs);
+  const float lse = (KIND == kLogSoftmax) ? logf(gs) : 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const int idx = t + i * TPR;
@@ -90,14 +107,14 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         if (KIND == kSoftmax) {
-          const float r = scale * v[i][k];
+          const float r = f * v[i][k];
           v[i][k] = __builtin_isnormal(r) ? r : 0.f;
         }
         else if (KIND == kLogSoftmax) {
-          v[i][k] -= lse;
+          v[i][k] = (v[i][k] + shift) - lse;
         }
         else {
-          v[i][k] *= scale;
+          v[i][k] *= f;
         }
       }
       Vec16<float>::store(yr + 4 * idx, v[i]);
@@ -115,7 +132,7 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
   constexpr int NW = B::kWavesPerTeam;
   __shared__ float red[NW];
   const int tid = threadIdx.x;
-  const int team = tid / TPR;
+  const int team = wave_index() / NW;  // wave-uniform: a team is a whole number of waves
   const int t = tid - team * TPR;
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
@@ -316,6 +333,7 @@ sm_bwd_cluster(const float* y, const float* dy, float* dx, int64_t ldy, int64_t 
 // ================================================================ split rows
 // Block b handles chunk (b % S) of row (b / S); 256 threads per block.
 constexpr int kChunkThreads = 256;
+constexpr int kChunkUnroll = 4;
 
 // Merges the online-softmax pairs (m, acc) of the 256 threads; every thread gets the result.
 __device__ __forceinline__ void block_merge_max_sum(float& m, float& acc, float (*slot)[2])
@@ -352,11 +370,33 @@ sm_fwd_partial(const float* x, int64_t ldx, RowMap map, int64_t n, int64_t chunk
   const float* xr = x + map.offset(row, ldx);
   float m = -FLT_MAX, acc = 0.f;
   if (VEC) {
-    for (int64_t i = begin / 4 + threadIdx.x; i < end / 4; i += kChunkThreads) {
-      float v[4];
-      Vec16<float>::load(xr + 4 * i, v);
-      const float mn = fmaxf(fmaxf(fmaxf(m, v[0]), fmaxf(v[1], v[2])), v[3]);
-      acc = acc * exp_fast(m - mn) + ((exp_fast(v[0] - mn) + exp_fast(v[1] - mn)) + (exp_fast(v[2] - mn) + exp_fast(v[3] - mn)));
+    // four independent 16-byte loads per thread are in flight before any is used
+    for (int64_t i0 = begin / 4 + threadIdx.x; i0 < end / 4; i0 += kChunkUnroll * kChunkThreads) {
+      float v[kChunkUnroll][4];
+#pragma unroll
+      for (int u = 0; u < kChunkUnroll; ++u) {
+        const int64_t i = i0 + u * kChunkThreads;
+        if (i < end / 4) {
+          Vec16<float>::load(xr + 4 * i, v[u]);
+        }
+        else {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) v[u][k] = -FLT_MAX;
+        }
+      }
+      float mn = m;
+#pragma unroll
+      for (int u = 0; u < kChunkUnroll; ++u)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) mn = fmaxf(mn, v[u][k]);
+      float add = 0.f;
+#pragma unroll
+      for (int u = 0; u < kChunkUnroll; ++u) {
+        const bool ok = i0 + u * kChunkThreads < end / 4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) add += ok ? exp_fast(v[u][k] - mn) : 0.f;
+      }
+      acc = acc * exp_fast(m - mn) + add;
       m = mn;
     }
   }
@@ -403,12 +443,22 @@ sm_fwd_apply(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int
     return r;
   };
   if (VEC) {
-    for (int64_t i = begin / 4 + threadIdx.x; i < end / 4; i += kChunkThreads) {
-      float v[4];
-      Vec16<float>::load(xr + 4 * i, v);
+    for (int64_t i0 = begin / 4 + threadIdx.x; i0 < end / 4; i0 += kChunkUnroll * kChunkThreads) {
+      float v[kChunkUnroll][4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) v[k] = f(v[k]);
-      Vec16<float>::store(yr + 4 * i, v);
+      for (int u = 0; u < kChunkUnroll; ++u) {
+        const int64_t i = i0 + u * kChunkThreads;
+        if (i < end / 4) Vec16<float>::load(xr + 4 * i, v[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kChunkUnroll; ++u) {
+        const int64_t i = i0 + u * kChunkThreads;
+        if (i < end / 4) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) v[u][k] = f(v[u][k]);
+          Vec16<float>::store(yr + 4 * i, v[u]);
+        }
+      }
     }
   }
   else {
@@ -430,16 +480,22 @@ sm_bwd_partial(const float* y, const float* dy, int64_t ldy, int64_t lddy, RowMa
   const float* gr = dy + map.offset(row, lddy);
   float acc = 0.f;
   if (VEC) {
-    for (int64_t i = begin / 4 + threadIdx.x; i < end / 4; i += kChunkThreads) {
-      float g[4];
-      Vec16<float>::load(gr + 4 * i, g);
-      if (KIND == kLogSoftmax) {
-        acc += (g[0] + g[1]) + (g[2] + g[3]);
+    for (int64_t i0 = begin / 4 + threadIdx.x; i0 < end / 4; i0 += kChunkUnroll * kChunkThreads) {
+      float a[kChunkUnroll][4], g[kChunkUnroll][4];
+#pragma unroll
+      for (int u = 0; u < kChunkUnroll; ++u) {
+        const int64_t i = i0 + u * kChunkThreads;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) a[u][k] = g[u][k] = 0.f;
+        if (i < end / 4) {
+          Vec16<float>::load(gr + 4 * i, g[u]);
+          if (KIND != kLogSoftmax) Vec16<float>::load(yr + 4 * i, a[u]);
+        }
       }
-      else {
-        float a[4];
-        Vec16<float>::load(yr + 4 * i, a);
-        acc += (a[0] * g[0] + a[1] * g[1]) + (a[2] * g[2] + a[3] * g[3]);
+#pragma unroll
+      for (int u = 0; u < kChunkUnroll; ++u) {
+        if (KIND == kLogSoftmax) acc += (g[u][0] + g[u][1]) + (g[u][2] + g[u][3]);
+        else acc += (a[u][0] * g[u][0] + a[u][1] * g[u][1]) + (a[u][2] * g[u][2] + a[u][3] * g[u][3]);
       }
     }
   }
@@ -469,13 +525,25 @@ sm_bwd_apply(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ld
     return (KIND == kLogSoftmax) ? g - exp_fast(a) * sum : a * (g - sum);
   };
   if (VEC) {
-    for (int64_t i = begin / 4 + threadIdx.x; i < end / 4; i += kChunkThreads) {
-      float a[4], g[4];
-      Vec16<float>::load(yr + 4 * i, a);
-      Vec16<float>::load(gr + 4 * i, g);
+    for (int64_t i0 = begin / 4 + threadIdx.x; i0 < end / 4; i0 += kChunkUnroll * kChunkThreads) {
+      float a[kChunkUnroll][4], g[kChunkUnroll][4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) g[k] = f(a[k], g[k]);
-      Vec16<float>::store(dr + 4 * i, g);
+      for (int u = 0; u < kChunkUnroll; ++u) {
+        const int64_t i = i0 + u * kChunkThreads;
+        if (i < end / 4) {
+          Vec16<float>::load(yr + 4 * i, a[u]);
+          Vec16<float>::load(gr + 4 * i, g[u]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kChunkUnroll; ++u) {
+        const int64_t i = i0 + u * kChunkThreads;
+        if (i < end / 4) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) g[u][k] = f(a[u][k], g[u][k]);
+          Vec16<float>::store(dr + 4 * i, g[u]);
+        }
+      }
     }
   }
   else {
@@ -514,10 +582,17 @@ static size_t sm_workspace_bytes(int64_t n, int64_t rows)
   return chunked > cluster ? chunked : cluster;
 }
 
-static bool cluster_enabled()
+// The register-resident cluster kernels read every element once but pay a rendezvous
+// (a few microseconds) and a slot-reset launch; the two-kernel split path reads the
+// input twice.  While the tensor fits the last-level caches the second read costs no
+// HBM traffic, so the cluster path is used only for larger footprints.
+constexpr int64_t kClusterMinBytes = int64_t(48) << 20;
+
+static bool cluster_enabled(int64_t rows, int64_t n)
 {
   static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
-  return !disabled;
+  static const bool forced = std::getenv("LBN_FORCE_CLUSTER") != nullptr;
+  return !disabled && (forced || rows * n * 4 >= kClusterMinBytes);
 }
 
 #define LBN_ROW_CASES(X)                                                                     \
@@ -554,7 +629,7 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #undef X
     }
   }
-  if (vec && cluster_enabled() && n / 4 < (int64_t(1) << 30)) {
+  if (vec && cluster_enabled(rows, n) && n / 4 < (int64_t(1) << 30)) {
     const ClusterPlan cp = plan_cluster(n / 4, 8);
     if (cp.M) {
       if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
@@ -625,7 +700,7 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #undef X
     }
   }
-  if (vec && cluster_enabled() && n / 4 < (int64_t(1) << 30)) {
+  if (vec && cluster_enabled(rows, n) && n / 4 < (int64_t(1) << 30)) {
     const ClusterPlan cp = plan_cluster(n / 4, 4);
     if (cp.M) {
       if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;

@@ -137,14 +137,14 @@ class _Layer:
         if in_place:
             self.activations = x
         else:
-            self.activations = DeviceMatrix(x.height, x.width, dtype=x.dtype, device=self.device)
+            self.activations = DeviceMatrix(x.height, x.width, dtype=x.dtype, ldim=x.ldim, device=self.device)
 
     def bind_backward(self, dy, in_place=False):
         self.prev_error_signals = dy
         if in_place:
             self.error_signals = dy
         else:
-            self.error_signals = DeviceMatrix(dy.height, dy.width, dtype=dy.dtype, device=self.device)
+            self.error_signals = DeviceMatrix(dy.height, dy.width, dtype=dy.dtype, ldim=dy.ldim, device=self.device)
 
     # fp_call()/bp_call() return (entry point name, argument tuple) of the C-ABI call
     # that is the body of the reference's fp_compute()/bp_compute().

@@ -43,6 +43,7 @@ SM_SHAPES = [
     (512, 7, 64),          # ld > height (a view into a taller matrix), still 16-byte aligned
     (7, 19, 0), (31, 5, 0), (1001, 4, 0), (130, 3, 3),   # unaligned / odd heights: scalar split kernels
     (32772, 2, 0), (70000, 3, 0), (262144, 2, 0),        # longer than the register path: split kernels
+    (262148, 48, 0), (100000, 130, 0),                   # long rows, large footprint: register-resident clusters
     (1, 6, 0),
 ]
 
