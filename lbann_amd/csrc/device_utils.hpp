@@ -152,12 +152,27 @@ __device__ __forceinline__ float exp_fast(float x)
   return __builtin_fmaf(e, r * kLn2, e);
 }
 
+// exp(x) in two operations (one multiply, one v_exp_f32): relative error up to about
+// |x| * 3e-8.  Only for terms that are summed and never stored, such as the
+// denominator of log-softmax, where that error is far below the result's own rounding.
+__device__ __forceinline__ float exp_quick(float x)
+{
+  return __builtin_amdgcn_exp2f(x * 1.44269502162933349609375f);
+}
+
 __device__ __forceinline__ float exp_keep_denormals(float x)
 {
   // below exp(-87.3) the result is denormal: evaluate 2^64 times larger, scale back
   const bool tiny = x < -87.0f;
   const float e = exp_fast(tiny ? x + 44.3614196f : x);       // 64*ln2
   return tiny ? e * 5.42101086e-20f : e;                      // 2^-64
+}
+
+// log(s) for the sum of a max-shifted softmax row, which always lies in [1, n] (the row
+// maximum contributes exp(0) = 1): one v_log_f32 and a multiply, about 1 ulp there.
+__device__ __forceinline__ float log_of_sum(float s)
+{
+  return __builtin_amdgcn_logf(s) * 0.693147182464599609375f;
 }
 
 // 1/sqrt(v) for v > 0 from v_rsq_f32 and one Newton step (about 1 ulp), 5 operations

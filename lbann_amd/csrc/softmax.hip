@@ -28,17 +28,18 @@ enum SmKind : int { kSoftmax = 0, kLogSoftmax = 1, kChannelwise = 2 };
 constexpr int kMaxChunks = 64;  // S <= one wave, so a wave merges the partials of a row
 
 // ======================================================= register-resident rows
+// 1024-thread blocks are held to 64 registers so that two of them share a compute unit.
 template <int TPR, int V, int KIND>
-__global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
+__global__ void __launch_bounds__(RowBlock<TPR>::kThreads, (TPR == 1024 ? 8 : 1))
 sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
-            int nvec)
+            unsigned nvec)
 {
   using B = RowBlock<TPR>;
   constexpr int NW = B::kWavesPerTeam;
   __shared__ float red[2][NW];
-  const int tid = threadIdx.x;
+  const unsigned tid = threadIdx.x;
   const int team = wave_index() / NW;  // wave-uniform: a team is a whole number of waves
-  const int t = tid - team * TPR;
+  const unsigned t = tid - team * TPR;  // unsigned: addresses become scalar base + 32-bit offset
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
   const int64_t row = static_cast<int64_t>(blockIdx.x) * B::kTeams + team;
@@ -48,9 +49,9 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
   float v[V][4];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    const int idx = t + i * TPR;
+    const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      Vec16<float>::load(xr + 4 * idx, v[i]);
+      Vec16<float>::load(xr + 4u * idx, v[i]);
     }
     else {
 #pragma unroll
@@ -75,9 +76,13 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const float d = v[i][k] - m;
-      const float e = ok ? (KIND == kChannelwise ? exp_keep_denormals(d) : exp_fast(d)) : 0.f;
+      float e;
+      if (KIND == kLogSoftmax) e = exp_quick(d);  // only summed: x stays in the registers for the output
+      else if (KIND == kChannelwise) e = exp_keep_denormals(d);
+      else e = exp_fast(d);
+      e = ok ? e : 0.f;
       s += e;
-      v[i][k] = (KIND == kLogSoftmax) ? d : e;
+      if (KIND != kLogSoftmax) v[i][k] = e;
     }
   }
 
@@ -99,10 +104,10 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
   float* yr = y + map.offset(row, ldy);
   const float shift = m - gm;  // <= 0
   const float f = exp_fast(shift) * (1.0f / gs);
-  const float lse = (KIND == kLogSoftmax) ? logf(gs) : 0.f;
+  const float lse = (KIND == kLogSoftmax) ? log_of_sum(gs) : 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    const int idx = t + i * TPR;
+    const unsigned idx = t + i * TPR;
     if (idx < nvec) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
@@ -111,13 +116,13 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
           v[i][k] = __builtin_isnormal(r) ? r : 0.f;
         }
         else if (KIND == kLogSoftmax) {
-          v[i][k] = (v[i][k] + shift) - lse;
+          v[i][k] = (v[i][k] - gm) - lse;
         }
         else {
           v[i][k] *= f;
         }
       }
-      Vec16<float>::store(yr + 4 * idx, v[i]);
+      Vec16<float>::store(yr + 4u * idx, v[i]);
     }
   }
 }
@@ -126,14 +131,14 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
 template <int TPR, int V, int KIND>
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
 sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
-            RowMap map, int64_t rows, int nvec)
+            RowMap map, int64_t rows, unsigned nvec)
 {
   using B = RowBlock<TPR>;
   constexpr int NW = B::kWavesPerTeam;
   __shared__ float red[NW];
-  const int tid = threadIdx.x;
+  const unsigned tid = threadIdx.x;
   const int team = wave_index() / NW;  // wave-uniform: a team is a whole number of waves
-  const int t = tid - team * TPR;
+  const unsigned t = tid - team * TPR;  // unsigned: addresses become scalar base + 32-bit offset
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
   const int64_t row = static_cast<int64_t>(blockIdx.x) * B::kTeams + team;
@@ -144,10 +149,10 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
   float a[V][4], g[V][4];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    const int idx = t + i * TPR;
+    const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      Vec16<float>::load(yr + 4 * idx, a[i]);
-      Vec16<float>::load(gr + 4 * idx, g[i]);
+      Vec16<float>::load(yr + 4u * idx, a[i]);
+      Vec16<float>::load(gr + 4u * idx, g[i]);
     }
     else {
 #pragma unroll
@@ -164,14 +169,14 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
   float* dr = dx + map.offset(row, lddx);
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    const int idx = t + i * TPR;
+    const unsigned idx = t + i * TPR;
     if (idx < nvec) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         if (KIND == kLogSoftmax) g[i][k] = g[i][k] - exp_fast(a[i][k]) * s;
         else g[i][k] = a[i][k] * (g[i][k] - s);
       }
-      Vec16<float>::store(dr + 4 * idx, g[i]);
+      Vec16<float>::store(dr + 4u * idx, g[i]);
     }
   }
 }
@@ -247,7 +252,7 @@ sm_fwd_cluster(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, i
     float* yr = y + map.offset(row, ldy);
     const float shift = m - gm;                       // <= 0: this share's maximum against the row's
     const float f = exp_fast(shift) * (1.0f / gs);    // rescales exp(x - m) to exp(x - gm) / sum
-    const float lse = (KIND == kLogSoftmax) ? logf(gs) : 0.f;
+    const float lse = (KIND == kLogSoftmax) ? log_of_sum(gs) : 0.f;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       const unsigned idx = base + i * kClusterThreads;
@@ -432,7 +437,7 @@ sm_fwd_apply(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int
   const float m = wave_max(pm);
   const float sum = wave_sum(ps * exp_fast(pm - m));
   const float scale = 1.0f / sum;
-  const float lse = (KIND == kLogSoftmax) ? logf(sum) : 0.f;
+  const float lse = (KIND == kLogSoftmax) ? log_of_sum(sum) : 0.f;
   const float* xr = x + map.offset(row, ldx);
   float* yr = y + map.offset(row, ldy);
   auto f = [&](float v) -> float {
@@ -616,7 +621,7 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   if (vec) {
     const RowConfig c = pick_row_config(n / 4, rows);
     if (c.tpr) {
-      const int nvec = static_cast<int>(n / 4);
+      const unsigned nvec = static_cast<unsigned>(n / 4);
 #define X(TPR, V)                                                                            \
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
@@ -687,7 +692,7 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     // still fits, so 1024-thread blocks keep two blocks per compute unit
     const RowConfig c = pick_row_config(n / 4, rows);
     if (c.tpr) {
-      const int nvec = static_cast<int>(n / 4);
+      const unsigned nvec = static_cast<unsigned>(n / 4);
 #define X(TPR, V)                                                                            \
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
