@@ -20,17 +20,19 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-u
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
-def _compile(src):
-    obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    subprocess.run([HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj], check=True)
+def _compile(src, extra=(), tag=""):
+    obj = os.path.join(CSRC, src.replace(".hip", tag + ".o"))
+    subprocess.run([HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj], check=True)
     return obj
 
 
-def build(jobs: int = 4) -> str:
+def build(jobs: int = 4, extra=(), lib: str = LIB, tag: str = "") -> str:
+    """`extra` adds compiler flags (e.g. -DLBN_NT_STORE=0) and `lib`/`tag` name an alternative
+    output, for side-by-side experiments; lbann_amd.capi loads $LBN_LIB when it is set."""
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(_compile, SOURCES))
-    subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], check=True)
-    return LIB
+        objs = list(ex.map(lambda s: _compile(s, extra, tag), SOURCES))
+    subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *objs], check=True)
+    return lib
 
 
 def build_adapter_driver() -> str:

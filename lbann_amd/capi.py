@@ -6,7 +6,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "liblbnorm.so")
+LIB_PATH = os.environ.get("LBN_LIB") or os.path.join(_HERE, "liblbnorm.so")
 
 i64 = ctypes.c_int64
 f32 = ctypes.c_float

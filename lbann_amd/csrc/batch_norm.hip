@@ -403,6 +403,7 @@ struct BnFwdArgs {
   float eps, decay;
   int64_t n;
   ClusterWorkspace cw;
+  ClusterTag tag;
   float* mean_out;
   float* var_out;
   const float* gamma;
@@ -449,7 +450,7 @@ __device__ __forceinline__ void bn_fwd_reduce(const BnFwdArgs& a, const BnIndex<
     }
   }
   team_sum2<T / kWave>(s, q, red, tid / kWave, tid & (kWave - 1));
-  if (tid == 0) cluster_publish(s, q, a.cw.slots + static_cast<int64_t>(ch) * a.M, k);
+  if (tid == 0) cluster_publish(s, q, a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, k, a.tag);
 }
 
 // (3) of a step: statistics of channel `ch` from the cluster's partials, output from tile `t`.
@@ -460,7 +461,7 @@ __device__ __forceinline__ void bn_fwd_finish(const BnFwdArgs& a, const BnIndex<
   const unsigned tid = threadIdx.x;
   if (tid < kWave) {
     float ts, tq;
-    cluster_collect(a.cw.slots + static_cast<int64_t>(ch) * a.M, a.M, a.cw.error, 0.f, 0.f, ts, tq);
+    cluster_collect(a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, a.M, a.tag, a.cw.error, 0.f, 0.f, ts, tq);
     ts = wave_sum(ts);
     tq = wave_sum(tq);
     if (tid == 0) {
@@ -530,6 +531,7 @@ struct BnBwdArgs {
   float eps;
   int64_t n;
   ClusterWorkspace cw;
+  ClusterTag tag;
   const float* mean_in;
   const float* var_in;
   const float* gamma;
@@ -576,7 +578,7 @@ __device__ __forceinline__ void bn_bwd_reduce(const BnBwdArgs& a, const BnIndex<
     }
   }
   team_sum2<T / kWave>(sa, sb, red, tid / kWave, tid & (kWave - 1));
-  if (tid == 0) cluster_publish(sa, sb, a.cw.slots + static_cast<int64_t>(ch) * a.M, k);
+  if (tid == 0) cluster_publish(sa, sb, a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, k, a.tag);
 }
 
 template <int T, int V>
@@ -588,7 +590,7 @@ __device__ __forceinline__ void bn_bwd_finish(const BnBwdArgs& a, const BnIndex<
   const float scale = t.scale;
   if (tid < kWave) {
     float ta, tb;
-    cluster_collect(a.cw.slots + static_cast<int64_t>(ch) * a.M, a.M, a.cw.error, 0.f, 0.f, ta, tb);
+    cluster_collect(a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, a.M, a.tag, a.cw.error, 0.f, 0.f, ta, tb);
     ta = wave_sum(ta);
     tb = wave_sum(tb);
     if (tid == 0) {
@@ -694,7 +696,6 @@ static bool bn_launch_fwd_cluster(hipStream_t st, const BnFwdArgs& a, int64_t C,
   const int cap = cluster_capacity(bn_fwd_cluster<T, V>, T);
   const int64_t ncl = cap / a.M < C ? cap / a.M : C;
   if (ncl < 1) return false;
-  launch_cluster_reset(st, a.cw, C * a.M);
   hipLaunchKernelGGL((bn_fwd_cluster<T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
   return true;
 }
@@ -705,7 +706,6 @@ static bool bn_launch_bwd_cluster(hipStream_t st, const BnBwdArgs& a, int64_t C,
   const int cap = cluster_capacity(bn_bwd_cluster<T, V>, T);
   const int64_t ncl = cap / a.M < C ? cap / a.M : C;
   if (ncl < 1) return false;
-  launch_cluster_reset(st, a.cw, C * a.M);
   hipLaunchKernelGGL((bn_bwd_cluster<T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
   return true;
 }
@@ -727,7 +727,7 @@ static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   const BnClusterShape p = bn_cluster_shape(E, 4, 256);
   if (!p.T) return false;
   const BnFwdArgs a{x, y, ldx, ldy, cs, static_cast<int>(C), p.M, pivot, bessel, eps, decay, cs * w,
-                    cluster_workspace(ws), mean, var, scale, bias, rmean, rvar};
+                    cluster_workspace(ws), next_cluster_tag(), mean, var, scale, bias, rmean, rvar};
   const unsigned seg = static_cast<unsigned>(cs / 4), Eu = static_cast<unsigned>(E);
 #define X(TT, VV) \
   if (p.T == TT && p.V == VV) return bn_launch_fwd_cluster<TT, VV>(st, a, C, seg, Eu);
@@ -747,7 +747,7 @@ static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   const BnClusterShape p = bn_cluster_shape(E, 2, 256);
   if (!p.T) return false;
   const BnBwdArgs a{x, dy, dx, ldx, lddy, lddx, cs, static_cast<int>(C), p.M, bessel, eps, cs * w,
-                    cluster_workspace(ws), mean, var, scale, dscale, dbias, dmean, dvar};
+                    cluster_workspace(ws), next_cluster_tag(), mean, var, scale, dscale, dbias, dmean, dvar};
   const unsigned seg = static_cast<unsigned>(cs / 4), Eu = static_cast<unsigned>(E);
 #define X(TT, VV) \
   if (p.T == TT && p.V == VV) return bn_launch_bwd_cluster<TT, VV>(st, a, C, seg, Eu);

@@ -5,25 +5,28 @@
 // one partial pair, waits until all M partials of the cluster are there, and then
 // finishes from its registers: every tensor is read from memory exactly once.
 //
-// Protocol (no fences, no cache write-back or invalidation): every slot is one
-// 64-bit word holding two floats.  A small kernel fills the slots of the call with
-// an "empty" pattern; a workgroup publishes with ONE relaxed device-scope atomic
-// 64-bit store, and one wave of each workgroup polls the M slots of its item in
-// parallel (lane j reads slot j) with relaxed device-scope atomic loads until none
-// is empty.  The pair is the only data that crosses workgroups, so no ordering with
-// other memory traffic is needed.  Published NaNs are canonicalised so that a
-// payload can never look like the empty pattern.
+// Protocol (no fences, no cache write-back or invalidation, no clearing pass): a slot
+// is two 64-bit words, each holding one float of the pair and one half of a 64-bit
+// call tag.  The tag is drawn per call from a process-wide counter, so whatever an
+// earlier call (or anything else) left in the workspace can never look published: a
+// slot counts only when both of its words carry the two halves of this call's tag.
+// A workgroup publishes with two relaxed device-scope atomic 64-bit stores, and one
+// wave of each workgroup polls the M slots of its item in parallel (lane j reads slot
+// j) with relaxed device-scope atomic loads.  The pair is the only data that crosses
+// workgroups, so no ordering with other memory traffic is needed.
 //
 // Forward progress: the launch never exceeds the number of workgroups the device
 // can hold at once (cluster_capacity(), from the occupancy query), so all members
 // of a cluster are resident together and the wait always ends.  As a second line of
-// defence the wait gives up after kClusterMaxPolls polls and raises the error word
-// in the workspace instead of spinning forever; results are then undefined but
-// every wave still exits.
+// defence the wait gives up after kClusterMaxPolls polls and raises the (sticky)
+// error word in the workspace instead of spinning forever; results are then undefined
+// but every wave still exits.
 #pragma once
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <chrono>
 #include <cstdint>
 #include <map>
 #include <mutex>
@@ -34,63 +37,72 @@ namespace lbn {
 constexpr int kClusterThreads = 256;  // workgroup size of the row-cluster (softmax) kernels
 constexpr int kClusterMaxM = 64;  // one wave polls and merges the partials of an item
 constexpr int kClusterMaxPolls = 1 << 21;
-constexpr unsigned long long kSlotEmpty = ~0ull;
 
-__device__ __forceinline__ unsigned long long cluster_pack(float a, float b)
+struct ClusterTag {
+  unsigned lo, hi;
+};
+
+// A fresh tag per call.  The counter starts from the clock so that slots written by
+// an earlier process into recycled device memory do not match either.
+inline ClusterTag next_cluster_tag()
 {
-  if (a != a) a = __builtin_nanf("");
-  if (b != b) b = __builtin_nanf("");
-  return (static_cast<unsigned long long>(__float_as_uint(b)) << 32) | __float_as_uint(a);
+  static std::atomic<uint64_t> counter{
+    static_cast<uint64_t>(std::chrono::steady_clock::now().time_since_epoch().count()) * 0x9E3779B97F4A7C15ull};
+  const uint64_t v = counter.fetch_add(0x9E3779B97F4A7C15ull, std::memory_order_relaxed);
+  return {static_cast<unsigned>(v), static_cast<unsigned>(v >> 32)};
+}
+
+__device__ __forceinline__ unsigned long long cluster_word(float value, unsigned tag)
+{
+  return (static_cast<unsigned long long>(tag) << 32) | __float_as_uint(value);
 }
 
 // Publishes the pair (a, b) of workgroup k; called by one lane.
-__device__ __forceinline__ void cluster_publish(float a, float b, unsigned long long* slots, int k)
+__device__ __forceinline__ void cluster_publish(float a, float b, unsigned long long* slots, int k,
+                                                ClusterTag tag)
 {
-  __hip_atomic_store(slots + k, cluster_pack(a, b), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(slots + 2 * k, cluster_word(a, tag.lo), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(slots + 2 * k + 1, cluster_word(b, tag.hi), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Called by all 64 lanes of ONE wave per workgroup (convergent).  Waits until the M
 // slots of an item are published.  On return lane j < M holds the pair published by
 // workgroup j in (ra, rb); lanes >= M hold (na, nb).
-__device__ __forceinline__ void cluster_collect(unsigned long long* slots, int M, int* error_word,
-                                                float na, float nb, float& ra, float& rb)
+__device__ __forceinline__ void cluster_collect(unsigned long long* slots, int M, ClusterTag tag,
+                                                int* error_word, float na, float nb, float& ra,
+                                                float& rb)
 {
   const int lane = threadIdx.x & 63;
-  unsigned long long raw = 0;
+  unsigned long long wa = 0, wb = 0;
+  bool have = false;
   int polls = 0;
   for (;;) {
-    raw = lane < M ? __hip_atomic_load(slots + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
-    if (__all(raw != kSlotEmpty)) break;
+    if (lane < M) {
+      wa = __hip_atomic_load(slots + 2 * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      wb = __hip_atomic_load(slots + 2 * lane + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      have = static_cast<unsigned>(wa >> 32) == tag.lo && static_cast<unsigned>(wb >> 32) == tag.hi;
+    }
+    if (__all(have || lane >= M)) break;
     if (++polls > kClusterMaxPolls) {
       if (lane == 0) __hip_atomic_store(error_word, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       break;
     }
     __builtin_amdgcn_s_sleep(1);
   }
-  const bool have = lane < M && raw != kSlotEmpty;
-  ra = have ? __uint_as_float(static_cast<unsigned>(raw)) : na;
-  rb = have ? __uint_as_float(static_cast<unsigned>(raw >> 32)) : nb;
+  ra = have ? __uint_as_float(static_cast<unsigned>(wa)) : na;
+  rb = have ? __uint_as_float(static_cast<unsigned>(wb)) : nb;
 }
 
 // Publish and collect in one go.
 __device__ __forceinline__ void cluster_exchange(float a, float b, unsigned long long* slots, int k,
-                                                 int M, int* error_word, float na, float nb,
-                                                 float& ra, float& rb)
+                                                 int M, ClusterTag tag, int* error_word, float na,
+                                                 float nb, float& ra, float& rb)
 {
-  if ((threadIdx.x & 63) == 0) cluster_publish(a, b, slots, k);
-  cluster_collect(slots, M, error_word, na, nb, ra, rb);
+  if ((threadIdx.x & 63) == 0) cluster_publish(a, b, slots, k, tag);
+  cluster_collect(slots, M, tag, error_word, na, nb, ra, rb);
 }
 
-// Marks `n` slots empty and clears the error word.
-static __global__ void __launch_bounds__(256)
-cluster_reset(unsigned long long* slots, int64_t n, int* error_word)
-{
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (i < n) slots[i] = kSlotEmpty;
-  if (i == 0) *error_word = 0;
-}
-
-// Layout of the cluster part of a workspace: int error[16], then 64-bit slots.
+// Layout of the cluster part of a workspace: int error[16], then two 64-bit words per slot.
 struct ClusterWorkspace {
   int* error;
   unsigned long long* slots;
@@ -98,19 +110,13 @@ struct ClusterWorkspace {
 
 inline size_t cluster_workspace_bytes(int64_t items)
 {
-  return 64 + static_cast<size_t>(items) * kClusterMaxM * sizeof(unsigned long long);
+  return 64 + static_cast<size_t>(items) * kClusterMaxM * 2 * sizeof(unsigned long long);
 }
 
 inline ClusterWorkspace cluster_workspace(void* ws)
 {
   char* base = static_cast<char*>(ws);
   return {reinterpret_cast<int*>(base), reinterpret_cast<unsigned long long*>(base + 64)};
-}
-
-inline void launch_cluster_reset(hipStream_t st, const ClusterWorkspace& cw, int64_t nslots)
-{
-  hipLaunchKernelGGL(cluster_reset, dim3(static_cast<unsigned>((nslots + 255) / 256)), dim3(256), 0, st,
-                     cw.slots, nslots, cw.error);
 }
 
 // Cluster shape for an item of E 16-byte vectors: V vectors per thread (<= max_v), M

@@ -29,7 +29,7 @@ constexpr int kMaxChunks = 64;  // S <= one wave, so a wave merges the partials 
 
 // ======================================================= register-resident rows
 // 1024-thread blocks are held to 64 registers so that two of them share a compute unit.
-template <int TPR, int V, int KIND>
+template <int TPR, int V, int KIND, bool STREAM>
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads, (TPR == 1024 ? 8 : 1))
 sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
             unsigned nvec)
@@ -51,7 +51,8 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      Vec16<float>::load(xr + 4u * idx, v[i]);
+      if (STREAM) Vec16<float>::load_stream(xr + 4u * idx, v[i]);
+      else Vec16<float>::load(xr + 4u * idx, v[i]);
     }
     else {
 #pragma unroll
@@ -128,7 +129,7 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
 }
 
 // softmax / channelwise: dx = y * (dy - dot(y, dy));  log-softmax: dx = dy - exp(y) * sum(dy)
-template <int TPR, int V, int KIND>
+template <int TPR, int V, int KIND, bool STREAM>
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
 sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
             RowMap map, int64_t rows, unsigned nvec)
@@ -151,8 +152,14 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      Vec16<float>::load(yr + 4u * idx, a[i]);
-      Vec16<float>::load(gr + 4u * idx, g[i]);
+      if (STREAM) {
+        Vec16<float>::load_stream(yr + 4u * idx, a[i]);
+        Vec16<float>::load_stream(gr + 4u * idx, g[i]);
+      }
+      else {
+        Vec16<float>::load(yr + 4u * idx, a[i]);
+        Vec16<float>::load(gr + 4u * idx, g[i]);
+      }
     }
     else {
 #pragma unroll
@@ -191,7 +198,7 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
 template <int V, int KIND>
 __global__ void __launch_bounds__(kClusterThreads)
 sm_fwd_cluster(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
-               unsigned nvec, int M, ClusterWorkspace cw)
+               unsigned nvec, int M, ClusterWorkspace cw, ClusterTag tag)
 {
   constexpr int NW = kClusterThreads / kWave;
   __shared__ float red[2][NW];
@@ -238,7 +245,7 @@ sm_fwd_cluster(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, i
     s = team_sum<NW>(s, red[1], wv, lane);
     if (tid < kWave) {
       float pm, ps;
-      cluster_exchange(m, s, cw.slots + row * M, k, M, cw.error, -FLT_MAX, 0.f, pm, ps);
+      cluster_exchange(m, s, cw.slots + row * M * 2, k, M, tag, cw.error, -FLT_MAX, 0.f, pm, ps);
       const float gmax = wave_max(pm);
       const float gsum = wave_sum(ps * exp_fast(pm - gmax));
       if (tid == 0) {
@@ -279,7 +286,7 @@ sm_fwd_cluster(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, i
 template <int V, int KIND>
 __global__ void __launch_bounds__(kClusterThreads)
 sm_bwd_cluster(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
-               RowMap map, int64_t rows, unsigned nvec, int M, ClusterWorkspace cw)
+               RowMap map, int64_t rows, unsigned nvec, int M, ClusterWorkspace cw, ClusterTag tag)
 {
   constexpr int NW = kClusterThreads / kWave;
   __shared__ float red[NW];
@@ -313,7 +320,7 @@ sm_bwd_cluster(const float* y, const float* dy, float* dx, int64_t ldy, int64_t 
     s = team_sum<NW>(s, red, tid / kWave, tid & (kWave - 1));
     if (tid < kWave) {
       float pt, unused;
-      cluster_exchange(s, 0.f, cw.slots + row * M, k, M, cw.error, 0.f, 0.f, pt, unused);
+      cluster_exchange(s, 0.f, cw.slots + row * M * 2, k, M, tag, cw.error, 0.f, 0.f, pt, unused);
       pt = wave_sum(pt);
       if (tid == 0) bc[0] = pt;
     }
@@ -593,6 +600,18 @@ static size_t sm_workspace_bytes(int64_t n, int64_t rows)
 // HBM traffic, so the cluster path is used only for larger footprints.
 constexpr int64_t kClusterMinBytes = int64_t(48) << 20;
 
+// Inputs are loaded with the streaming (non-temporal) hint once the bytes a call moves
+// exceed what the 256 MB Infinity Cache could keep for a later reader; smaller working
+// sets are left to the cache, where the next kernel usually finds them.
+constexpr int64_t kStreamLoadMinBytes = int64_t(384) << 20;
+
+static int stream_loads(int64_t rows, int64_t n, int tensors)
+{
+  static const int forced = std::getenv("LBN_STREAM_LOADS") ? std::atoi(std::getenv("LBN_STREAM_LOADS")) : -1;
+  if (forced >= 0) return forced;
+  return rows * n * 4 * tensors >= kStreamLoadMinBytes ? 1 : 0;
+}
+
 static bool cluster_enabled(int64_t rows, int64_t n)
 {
   static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
@@ -626,8 +645,12 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
     const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
-    hipLaunchKernelGGL((sm_fwd_rows<TPR, V, KIND>), dim3(grid), dim3(B::kThreads), 0, st, x, \
-                       y, ldx, ldy, map, rows, nvec);                                        \
+    if (stream_loads(rows, n, 2))                                                            \
+      hipLaunchKernelGGL((sm_fwd_rows<TPR, V, KIND, true>), dim3(grid), dim3(B::kThreads), 0, st, \
+                         x, y, ldx, ldy, map, rows, nvec);                                   \
+    else                                                                                     \
+      hipLaunchKernelGGL((sm_fwd_rows<TPR, V, KIND, false>), dim3(grid), dim3(B::kThreads), 0, st, \
+                         x, y, ldx, ldy, map, rows, nvec);                                   \
     return launch_status();                                                                  \
   }
       LBN_ROW_CASES(X)
@@ -644,10 +667,9 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     const int cap = cluster_capacity(sm_fwd_cluster<VV, KIND>, kClusterThreads);                 \
     const int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                   \
     if (ncl >= 1) {                                                                              \
-      launch_cluster_reset(st, cw, rows * cp.M);                                                 \
       hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND>), dim3(static_cast<unsigned>(ncl * cp.M)),    \
                          dim3(kClusterThreads), 0, st, x, y, ldx, ldy, map, rows,                \
-                         static_cast<unsigned>(n / 4), cp.M, cw);                                \
+                         static_cast<unsigned>(n / 4), cp.M, cw, next_cluster_tag());            \
       return launch_status();                                                                    \
     }                                                                                            \
   }
@@ -697,8 +719,12 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
     const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
-    hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND>), dim3(grid), dim3(B::kThreads), 0, st, y, \
-                       dy, dx, ldy, lddy, lddx, map, rows, nvec);                            \
+    if (stream_loads(rows, n, 3))                                                            \
+      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, true>), dim3(grid), dim3(B::kThreads), 0, st, \
+                         y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
+    else                                                                                     \
+      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, false>), dim3(grid), dim3(B::kThreads), 0, st, \
+                         y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
     return launch_status();                                                                  \
   }
       LBN_ROW_CASES(X)
@@ -715,10 +741,9 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     const int cap = cluster_capacity(sm_bwd_cluster<VV, KIND>, kClusterThreads);                 \
     const int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                   \
     if (ncl >= 1) {                                                                              \
-      launch_cluster_reset(st, cw, rows * cp.M);                                                 \
       hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND>), dim3(static_cast<unsigned>(ncl * cp.M)),    \
                          dim3(kClusterThreads), 0, st, y, dy, dx, ldy, lddy, lddx, map, rows,    \
-                         static_cast<unsigned>(n / 4), cp.M, cw);                                \
+                         static_cast<unsigned>(n / 4), cp.M, cw, next_cluster_tag());            \
       return launch_status();                                                                    \
     }                                                                                            \
   }
