@@ -603,7 +603,7 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                    rows_aligned16(y, stride, ldy, G, w, sizeof(T)) &&
                    (!gamma || aligned16(gamma)) && (!beta || aligned16(beta));
   if (vec) {
-    const RowConfig c = pick_row_config(n / VE, rows, VE == 8 ? 4 : 8);
+    const RowConfig c = pick_row_config(n / VE, rows, 8);
     if (c.tpr) {
       const int nvec = static_cast<int>(n / VE);
 #define X(TPR, V)                                                                              \
@@ -616,7 +616,8 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     return launch_status();                                                                    \
   }
       X(64, 1) X(64, 2) X(64, 4) X(256, 1) X(256, 2) X(256, 4) X(1024, 1) X(1024, 2) X(1024, 4)
-      if constexpr (VE == 4) { X(64, 8) X(256, 8) X(1024, 8) }
+      X(64, 8) X(256, 8)
+      if constexpr (VE == 4) { X(1024, 8) }
 #undef X
     }
   }
