@@ -28,9 +28,8 @@
 #include <atomic>
 #include <chrono>
 #include <cstdint>
-#include <map>
-#include <mutex>
-#include <utility>
+
+#include "host_utils.hpp"
 
 namespace lbn {
 
@@ -134,25 +133,11 @@ inline ClusterPlan plan_cluster(int64_t E, int max_v, int threads = kClusterThre
   return {static_cast<int>(V), static_cast<int>(M)};
 }
 
-// Workgroups of `threads` threads running `kernel` that the current device holds at
-// once.  Queried once per (kernel, device); the cache is the only process-wide
-// state of the library and holds hardware facts only.
+// Workgroups of `threads` threads running `kernel` that the current device holds at once.
 template <typename K>
 inline int cluster_capacity(K kernel, int threads)
 {
-  static std::mutex mu;
-  static std::map<std::pair<const void*, int>, int> cache;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return 0;
-  const auto key = std::make_pair(reinterpret_cast<const void*>(kernel), dev);
-  std::lock_guard<std::mutex> lock(mu);
-  auto it = cache.find(key);
-  if (it != cache.end()) return it->second;
-  int cus = 0, per_cu = 0;
-  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess) return 0;
-  cache[key] = cus * per_cu;
-  return cus * per_cu;
+  return resident_blocks(kernel, threads);
 }
 
 }  // namespace lbn

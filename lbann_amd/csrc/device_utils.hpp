@@ -214,13 +214,15 @@ __device__ __forceinline__ float rsqrt_refined(float v)
 
 // ---------------------------------------------------------------------------
 // Wave64 reductions on the DPP data path (no LDS traffic): four cross-lane steps fold
-// every row of 16 lanes (quad swap, quad-pair swap, half-row mirror, row mirror), then
-// the four row results are read through scalar registers.  Every lane gets the result.
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v)
+// every row of 16 lanes (quad swap, quad-pair swap, half-row mirror, row mirror), two
+// row broadcasts (lane 15 of a row into the next row, lane 31 into the upper half) then
+// chain the four rows, which leaves the result of the whole wave in lane 63.
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp_move(float v, float old = 0.f)
 {
-  return __builtin_bit_cast(
-    float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old),
+                                                               __builtin_bit_cast(int, v), CTRL,
+                                                               ROW_MASK, 0xF, false));
 }
 __device__ __forceinline__ float read_lane(float v, int lane)
 {
@@ -230,23 +232,33 @@ constexpr int kDppQuadSwap1 = 0xB1;     // quad_perm:[1,0,3,2]
 constexpr int kDppQuadSwap2 = 0x4E;     // quad_perm:[2,3,0,1]
 constexpr int kDppHalfMirror = 0x141;   // row_half_mirror
 constexpr int kDppRowMirror = 0x140;    // row_mirror
+constexpr int kDppRowBcast15 = 0x142;   // lane 15 of each row to the next row
+constexpr int kDppRowBcast31 = 0x143;   // lane 31 to rows 2 and 3
 
-__device__ __forceinline__ float wave_sum(float v)
+// Sum over the wave, valid in lane 63 only.
+__device__ __forceinline__ float wave_sum_in_last(float v)
 {
   v += dpp_move<kDppQuadSwap1>(v);
   v += dpp_move<kDppQuadSwap2>(v);
   v += dpp_move<kDppHalfMirror>(v);
   v += dpp_move<kDppRowMirror>(v);
-  return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
+  v += dpp_move<kDppRowBcast15, 0xA>(v);  // rows 1 and 3 add rows 0 and 2; the others add 0
+  v += dpp_move<kDppRowBcast31, 0xC>(v);  // row 3 adds rows 0+1
+  return v;
 }
-__device__ __forceinline__ float wave_max(float v)
+__device__ __forceinline__ float wave_max_in_last(float v)
 {
   v = fmaxf(v, dpp_move<kDppQuadSwap1>(v));
   v = fmaxf(v, dpp_move<kDppQuadSwap2>(v));
   v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
   v = fmaxf(v, dpp_move<kDppRowMirror>(v));
-  return fmaxf(fmaxf(read_lane(v, 0), read_lane(v, 16)), fmaxf(read_lane(v, 32), read_lane(v, 48)));
+  v = fmaxf(v, dpp_move<kDppRowBcast15, 0xA>(v, v));  // disabled rows keep their own value
+  v = fmaxf(v, dpp_move<kDppRowBcast31, 0xC>(v, v));
+  return v;
 }
+// Every lane gets the result.
+__device__ __forceinline__ float wave_sum(float v) { return read_lane(wave_sum_in_last(v), kWave - 1); }
+__device__ __forceinline__ float wave_max(float v) { return read_lane(wave_max_in_last(v), kWave - 1); }
 
 // Reductions over a team of NW waves (NW*64 consecutive threads of the block).
 // `slot` must point to NW floats (2*NW for the pair version) of LDS that no other
@@ -256,9 +268,9 @@ __device__ __forceinline__ float wave_max(float v)
 template <int NW>
 __device__ __forceinline__ float team_sum(float v, float* slot, int wave_in_team, int lane)
 {
-  v = wave_sum(v);
-  if constexpr (NW == 1) return v;
-  if (lane == 0) slot[wave_in_team] = v;
+  if constexpr (NW == 1) return wave_sum(v);
+  v = wave_sum_in_last(v);
+  if (lane == kWave - 1) slot[wave_in_team] = v;
   __syncthreads();
   float r = slot[0];
 #pragma unroll
@@ -269,9 +281,9 @@ __device__ __forceinline__ float team_sum(float v, float* slot, int wave_in_team
 template <int NW>
 __device__ __forceinline__ float team_max(float v, float* slot, int wave_in_team, int lane)
 {
-  v = wave_max(v);
-  if constexpr (NW == 1) return v;
-  if (lane == 0) slot[wave_in_team] = v;
+  if constexpr (NW == 1) return wave_max(v);
+  v = wave_max_in_last(v);
+  if (lane == kWave - 1) slot[wave_in_team] = v;
   __syncthreads();
   float r = slot[0];
 #pragma unroll
@@ -283,10 +295,14 @@ template <int NW>
 __device__ __forceinline__ void team_sum2(float& a, float& b, float* slot, int wave_in_team,
                                           int lane)
 {
-  a = wave_sum(a);
-  b = wave_sum(b);
-  if constexpr (NW == 1) return;
-  if (lane == 0) {
+  if constexpr (NW == 1) {
+    a = wave_sum(a);
+    b = wave_sum(b);
+    return;
+  }
+  a = wave_sum_in_last(a);
+  b = wave_sum_in_last(b);
+  if (lane == kWave - 1) {
     slot[2 * wave_in_team] = a;
     slot[2 * wave_in_team + 1] = b;
   }

@@ -6,6 +6,9 @@
 
 #include <cstdint>
 #include <cstdlib>
+#include <map>
+#include <mutex>
+#include <utility>
 
 #include "../../include/lbnorm.h"
 
@@ -80,6 +83,27 @@ inline RowConfig pick_row_config(int64_t nvec, int64_t rows, int max_v = 8)
   while (pick < 2 && vs[pick] > 1 && rows * (tprs[pick] / 64) < want_waves && vs[pick + 1] != 0)
     ++pick;
   return {tprs[pick], vs[pick]};
+}
+
+// Workgroups of `threads` threads running `kernel` that the current device holds at
+// once.  Queried once per (kernel, device); the cache is the only process-wide
+// state of the library besides the call-tag counter and holds hardware facts only.
+template <typename K>
+inline int resident_blocks(K kernel, int threads)
+{
+  static std::mutex mu;
+  static std::map<std::pair<const void*, int>, int> cache;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  const auto key = std::make_pair(reinterpret_cast<const void*>(kernel), dev);
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = cache.find(key);
+  if (it != cache.end()) return it->second;
+  int cus = 0, per_cu = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess) return 0;
+  cache[key] = cus * per_cu;
+  return cus * per_cu;
 }
 
 }  // namespace lbn

@@ -17,119 +17,178 @@
 //    no atomics, bitwise reproducible.
 //  * generic kernels (one 256-thread block per row, scalar access) cover rows that
 //    are unaligned, not a multiple of the vector length, or too long for registers.
+#include <type_traits>
+
 #include "device_utils.hpp"
 #include "host_utils.hpp"
 
 namespace lbn {
 
 // ================================================================== forward
+// A team of TPR threads owns a row in registers (V 16-byte vectors per thread) and
+// walks the rows blockIdx.x*teams + team, + gridDim.x*teams, ...; the launch is one
+// resident wave of blocks.  The team's next row is in flight, still packed, while the
+// current one is processed, and threads that own at most 16 entries keep their scale
+// and bias in registers across rows.
+//
+// Per element: one conversion, the sum, the centred value and its square (or, in
+// sum-of-squares mode, the square of the raw value), then d * (1/stdev) and one
+// multiply-add with scale and bias.  Means use a multiplication by 1/n.
 template <typename T, int TPR, int V>
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
 ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy, RowMap map,
-            int64_t rows, int nvec, int n, float eps, float* __restrict__ stats,
+            int64_t rows, int nvec, float inv_n, float eps, float* __restrict__ stats,
             int64_t ld_stats, const float* __restrict__ gamma, const float* __restrict__ beta,
             int sumsq)
 {
   using B = RowBlock<TPR>;
   using IO = Vec16<T>;
+  using raw_t = typename IO::raw_t;
   constexpr int VE = IO::N;
   constexpr int NW = B::kWavesPerTeam;
-  __shared__ float red[2][2 * NW];
+  constexpr bool kWeightsInRegs = V * VE <= 16;
+  constexpr bool kPrefetch = V * VE < 32;  // wider rows: the registers only hold the current row
+  constexpr int WV = kWeightsInRegs ? V : 1;
+  __shared__ float red[4][B::kTeams][2 * NW];
   const int tid = threadIdx.x;
   const int team = wave_index() / NW;  // wave-uniform: a team is a whole number of waves
   const int t = tid - team * TPR;
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * B::kTeams + team;
-  if (B::kTeams > 1 && row >= rows) return;
 
-  const T* xr = x + map.offset(row, ldx);
-  float v[V][VE];
+  // A vector past the end of the row re-reads vector 0 and is masked out of the sums.
+  bool ok[V];
+  int voff[V];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    const int idx = t + i * TPR;
-    if (idx < nvec) {
-      IO::load(xr + VE * idx, v[i]);
-    }
-    else {
-#pragma unroll
-      for (int k = 0; k < VE; ++k) v[i][k] = 0.f;
-    }
+    ok[i] = t + i * TPR < nvec;
+    voff[i] = ok[i] ? VE * (t + i * TPR) : 0;
   }
-
-  const float inv_n = 1.0f / static_cast<float>(n);
-  float mean, var;
-  if (sumsq) {
-    float s = 0.f, q = 0.f;
+  auto load_weights = [&](const float* w, int i, float fill, float (&out)[VE]) {
 #pragma unroll
-    for (int i = 0; i < V; ++i)
+    for (int k = 0; k < VE; ++k) out[k] = fill;
+    if (w) {
 #pragma unroll
-      for (int k = 0; k < VE; ++k) {
-        s += v[i][k];
-        q += v[i][k] * v[i][k];
+      for (int k4 = 0; k4 < VE; k4 += 4) {
+        float q4[4];
+        Vec16<float>::load(w + voff[i] + k4, q4);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) out[k4 + k] = q4[k];
       }
-    team_sum2<NW>(s, q, red[0], wv, lane);
-    mean = s / static_cast<float>(n);
-    const float sqmean = q / static_cast<float>(n);
-    var = fmaxf(sqmean - mean * mean, 0.f);
-  }
-  else {
-    float s = 0.f;
-#pragma unroll
-    for (int i = 0; i < V; ++i)
-#pragma unroll
-      for (int k = 0; k < VE; ++k) s += v[i][k];
-    s = team_sum<NW>(s, red[0], wv, lane);
-    mean = s * inv_n;
-    float q = 0.f;
+    }
+  };
+  float gam[WV][VE], bet[WV][VE];
+  if constexpr (kWeightsInRegs) {
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      const bool ok = (t + i * TPR) < nvec;
-#pragma unroll
-      for (int k = 0; k < VE; ++k) {
-        const float d = v[i][k] - mean;
-        q += ok ? d * d : 0.f;
-      }
+      load_weights(gamma, i, 1.f, gam[i]);
+      load_weights(beta, i, 0.f, bet[i]);
     }
-    q = team_sum<NW>(q, red[1], wv, lane);
-    var = q * inv_n;
-  }
-  const float inv_stdev = 1.0f / sqrtf(var + eps);
-
-  if (t == 0) {
-    int64_t col, g;
-    map.split(row, col, g);
-    stats[g + col * ld_stats] = mean;
-    stats[map.groups + g + col * ld_stats] = var;
   }
 
-  T* yr = y + map.offset(row, ldy);
+  const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * B::kTeams;
+  const int64_t iters = (rows + rows_per_iter - 1) / rows_per_iter;
+  const int64_t first_row = static_cast<int64_t>(blockIdx.x) * B::kTeams + team;
+  raw_t q[V];  // the row in flight
+  auto issue = [&](int64_t row) {
+    const T* xr = x + map.offset(row < rows ? row : rows - 1, ldx);  // wave-uniform
 #pragma unroll
-  for (int i = 0; i < V; ++i) {
-    const int idx = t + i * TPR;
-    if (idx < nvec) {
+    for (int i = 0; i < V; ++i) q[i] = IO::load_raw(xr + voff[i]);
+  };
+
+  // full: every thread owns V whole vectors, nothing is masked.
+  auto process = [&](int64_t it, auto full) {
+    constexpr bool kFull = decltype(full)::value;
+    const int64_t row = it * rows_per_iter + first_row;
+    if constexpr (!kPrefetch) issue(row);
+    float v[V][VE];
 #pragma unroll
-      for (int k = 0; k < VE; ++k) v[i][k] = (v[i][k] - mean) * inv_stdev;
-      if (gamma) {
+    for (int i = 0; i < V; ++i) {
+      IO::unpack(q[i], v[i]);
+      if (!kFull && !ok[i]) {
 #pragma unroll
-        for (int k4 = 0; k4 < VE; k4 += 4) {
-          float w[4];
-          Vec16<float>::load(gamma + VE * idx + k4, w);
-#pragma unroll
-          for (int k = 0; k < 4; ++k) v[i][k4 + k] *= w[k];
-        }
+        for (int k = 0; k < VE; ++k) v[i][k] = 0.f;
       }
-      if (beta) {
-#pragma unroll
-        for (int k4 = 0; k4 < VE; k4 += 4) {
-          float w[4];
-          Vec16<float>::load(beta + VE * idx + k4, w);
-#pragma unroll
-          for (int k = 0; k < 4; ++k) v[i][k4 + k] += w[k];
-        }
-      }
-      IO::store(yr + VE * idx, v[i]);
     }
+    if constexpr (kPrefetch) {
+      if (it + 1 < iters) issue(row + rows_per_iter);
+    }
+    float* slots = red[2 * (it & 1)][team];
+    float mean, var;
+    if (sumsq) {
+      float s = 0.f, sq = 0.f;
+#pragma unroll
+      for (int i = 0; i < V; ++i)
+#pragma unroll
+        for (int k = 0; k < VE; ++k) {
+          s += v[i][k];
+          sq = __builtin_fmaf(v[i][k], v[i][k], sq);
+        }
+      team_sum2<NW>(s, sq, slots, wv, lane);
+      mean = s * inv_n;
+      var = fmaxf(__builtin_fmaf(-mean, mean, sq * inv_n), 0.f);
+#pragma unroll
+      for (int i = 0; i < V; ++i)
+#pragma unroll
+        for (int k = 0; k < VE; ++k) v[i][k] -= mean;
+    }
+    else {
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < V; ++i)
+#pragma unroll
+        for (int k = 0; k < VE; ++k) s += v[i][k];
+      s = team_sum<NW>(s, slots, wv, lane);
+      mean = s * inv_n;
+      float sq = 0.f;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+#pragma unroll
+        for (int k = 0; k < VE; ++k) {
+          v[i][k] -= mean;
+          const float d = (kFull || ok[i]) ? v[i][k] : 0.f;
+          sq = __builtin_fmaf(d, d, sq);
+        }
+      }
+      sq = team_sum<NW>(sq, red[2 * (it & 1) + 1][team], wv, lane);
+      var = sq * inv_n;
+    }
+    if (row < rows) {
+      const float inv_stdev = rsqrt_refined(var + eps);
+      int64_t col, g;
+      map.split(row, col, g);
+      if (t == 0) {
+        stats[g + col * ld_stats] = mean;
+        stats[map.groups + g + col * ld_stats] = var;
+      }
+      T* yr = y + g * map.stride + col * ldy;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        if (kFull || ok[i]) {
+          if constexpr (kWeightsInRegs) {
+#pragma unroll
+            for (int k = 0; k < VE; ++k)
+              v[i][k] = __builtin_fmaf(v[i][k] * inv_stdev, gam[i][k], bet[i][k]);
+          }
+          else {
+            float gw[VE], bw[VE];
+            load_weights(gamma, i, 1.f, gw);
+            load_weights(beta, i, 0.f, bw);
+#pragma unroll
+            for (int k = 0; k < VE; ++k) v[i][k] = __builtin_fmaf(v[i][k] * inv_stdev, gw[k], bw[k]);
+          }
+          IO::store(yr + voff[i], v[i]);
+        }
+      }
+    }
+  };
+
+  if constexpr (kPrefetch) issue(first_row);
+  if (nvec == TPR * V) {
+    for (int64_t it = 0; it < iters; ++it) process(it, std::true_type{});
+  }
+  else {
+    for (int64_t it = 0; it < iters; ++it) process(it, std::false_type{});
   }
 }
 
@@ -201,9 +260,9 @@ ln_fwd_generic(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t 
 //   dx = gs / stdev + dmean / n + (dvar * 2 * stdev / n) * xh
 // where dmean = -A / stdev and dvar = -B / (2 stdev^2)  (layer_norm.cpp:198-257).
 //
-// DEPTH > 0: the still-packed 16-byte images of the next DEPTH rows of a team are in
-// flight while the current row is processed.
-template <typename T, int TPR, int TEAMS, int V, bool WGRAD, int DEPTH>
+// A team's next row is in flight, still packed, while the current one is processed,
+// unless a thread owns 32 entries: then the registers only hold the current row.
+template <typename T, int TPR, int TEAMS, int V, bool WGRAD>
 __global__ void __launch_bounds__((RowBlock<TPR, TEAMS>::kThreads))
 ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ dx, int64_t ldx,
             int64_t lddy, int64_t lddx, RowMap map, int64_t rows, int nvec, int n, float eps,
@@ -216,7 +275,7 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   constexpr int VE = IO::N;
   constexpr int NW = B::kWavesPerTeam;
   constexpr int kAccLds = (WGRAD && TEAMS > 1) ? 2 * TPR * V * VE : 1;
-  constexpr int NQ = DEPTH > 0 ? DEPTH : 1;
+  constexpr bool kPrefetch = V * VE < 32;
   __shared__ float red[2][TEAMS][2 * NW];
   __shared__ float acc_lds[kAccLds];
   const int tid = threadIdx.x;
@@ -249,92 +308,80 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
       for (int k = 0; k < VE; ++k) dg[i][k] = db[i][k] = 0.f;
   }
 
-  raw_t qx[NQ][V], qg[NQ][V];  // rows in flight, packed
+  // A row in flight: its still-packed 16-byte vectors and its two statistics.
+  struct Slot {
+    raw_t x[V], g[V];
+    float mean, var;
+  };
+  // Loads are issued unconditionally: a row past the end re-reads the last row, a
+  // vector past the end of a row re-reads vector 0.
   // All row arithmetic is wave-uniform (scalar registers).
-  auto issue = [&](raw_t (&rx)[V], raw_t (&rg)[V], int64_t row) {
-    if (row < rows) {
-      int64_t col, g;
-      map.split(row, col, g);
-      const T* xr = x + g * map.stride + col * ldx;
-      const T* gr = dy + g * map.stride + col * lddy;
+  bool ok[V];
+  int voff[V];
 #pragma unroll
-      for (int i = 0; i < V; ++i) {
-        const int idx = t + i * TPR;
-        if (idx < nvec) {
-          rx[i] = IO::load_raw(xr + VE * idx);
-          rg[i] = IO::load_raw(gr + VE * idx);
-        }
-      }
+  for (int i = 0; i < V; ++i) {
+    ok[i] = t + i * TPR < nvec;
+    voff[i] = ok[i] ? VE * (t + i * TPR) : 0;
+  }
+  auto issue = [&](Slot& s, int64_t row) {
+    int64_t col, g;
+    map.split(row < rows ? row : rows - 1, col, g);
+    const T* xr = x + g * map.stride + col * ldx;
+    const T* gr = dy + g * map.stride + col * lddy;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      s.x[i] = IO::load_raw(xr + voff[i]);
+      s.g[i] = IO::load_raw(gr + voff[i]);
     }
+    s.mean = stats[g + col * ld_stats];
+    s.var = stats[map.groups + g + col * ld_stats];
   };
 
   const float inv_n = 1.0f / static_cast<float>(n);
   const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * TEAMS;
   const int64_t iters = (rows + rows_per_iter - 1) / rows_per_iter;
   const int64_t first_row = static_cast<int64_t>(blockIdx.x) * TEAMS + team;
-  if (DEPTH > 0) {
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) issue(qx[d], qg[d], first_row + d * rows_per_iter);
-  }
-  for (int64_t it = 0; it < iters; ++it) {
+
+  // One row: s holds it on entry and, after its registers are unpacked, is refilled
+  // (refill) with the team's next row, which stays in flight until its turn.
+  // full: the row exists and every thread owns V whole vectors of it, so nothing is
+  // masked.
+  auto process = [&](Slot& s, int64_t it, auto refill, auto full) {
+    constexpr bool kFull = decltype(full)::value;
     const int64_t row = it * rows_per_iter + first_row;
-    const bool active = row < rows;
-    raw_t cx[V], cg[V];
-    if (DEPTH > 0) {
-      // take the oldest row in flight, shift the queue, refill its tail
-#pragma unroll
-      for (int i = 0; i < V; ++i) {
-        cx[i] = qx[0][i];
-        cg[i] = qg[0][i];
-      }
-#pragma unroll
-      for (int d = 0; d + 1 < DEPTH; ++d)
-#pragma unroll
-        for (int i = 0; i < V; ++i) {
-          qx[d][i] = qx[d + 1][i];
-          qg[d][i] = qg[d + 1][i];
-        }
-      issue(qx[DEPTH - 1], qg[DEPTH - 1], row + DEPTH * rows_per_iter);
-    }
-    else {
-      issue(cx, cg, row);
-    }
-    float inv_stdev = 0.f, mean = 0.f;
-    int64_t col = 0, g = 0;
-    if (active) {
-      map.split(row, col, g);
-      mean = stats[g + col * ld_stats];
-      inv_stdev = rsqrt_refined(stats[map.groups + g + col * ld_stats] + eps);
-    }
+    const bool active = kFull || row < rows;
+    if constexpr (!kPrefetch) issue(s, row);
+    const float mean = s.mean;
+    const float inv_stdev = rsqrt_refined(s.var + eps);
     float xh[V][VE], gs[V][VE];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      IO::unpack(s.x[i], xh[i]);
+      IO::unpack(s.g[i], gs[i]);
+    }
+    if constexpr (kPrefetch && decltype(refill)::value) issue(s, row + rows_per_iter);
     float a = 0.f, b = 0.f;
-    if (active) {
 #pragma unroll
-      for (int i = 0; i < V; ++i) {
-        if (t + i * TPR < nvec) {
-          float xv[VE], gv[VE];
-          IO::unpack(cx[i], xv);
-          IO::unpack(cg[i], gv);
+    for (int i = 0; i < V; ++i) {
+      const bool use = kFull || (active && ok[i]);
 #pragma unroll
-          for (int k = 0; k < VE; ++k) {
-            xh[i][k] = (xv[k] - mean) * inv_stdev;  // subtract first: x*inv - mean*inv would cancel
-            if (WGRAD) {
-              db[i][k] += gv[k];
-              dg[i][k] = __builtin_fmaf(gv[k], xh[i][k], dg[i][k]);
-            }
-            gs[i][k] = gv[k] * gam[i][k];
-            a += gs[i][k];
-            b = __builtin_fmaf(gs[i][k], xh[i][k], b);
-          }
+      for (int k = 0; k < VE; ++k) {
+        // masked entries (re-read data of another vector or row) count as x = mean, dy = 0
+        const float gv = use ? gs[i][k] : 0.f;
+        xh[i][k] = use ? (xh[i][k] - mean) * inv_stdev : 0.f;  // subtract first: x*inv - mean*inv would cancel
+        if (WGRAD) {
+          db[i][k] += gv;
+          dg[i][k] = __builtin_fmaf(gv, xh[i][k], dg[i][k]);
         }
-        else {
-#pragma unroll
-          for (int k = 0; k < VE; ++k) xh[i][k] = gs[i][k] = 0.f;
-        }
+        gs[i][k] = gv * gam[i][k];
+        a += gs[i][k];
+        b = __builtin_fmaf(gs[i][k], xh[i][k], b);
       }
     }
     team_sum2<NW>(a, b, red[it & 1][team], wv, lane);
     if (active) {
+      int64_t col, g;
+      map.split(row, col, g);
       const float dmean = -a * inv_stdev;
       const float dvar = -b * inv_stdev * inv_stdev * 0.5f;
       if (t == 0) {
@@ -346,16 +393,29 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
       T* dr = dx + g * map.stride + col * lddx;
 #pragma unroll
       for (int i = 0; i < V; ++i) {
-        const int idx = t + i * TPR;
-        if (idx < nvec) {
+        if (kFull || ok[i]) {
 #pragma unroll
           for (int k = 0; k < VE; ++k)
             gs[i][k] = __builtin_fmaf(gs[i][k], inv_stdev, __builtin_fmaf(c1, xh[i][k], c0));
-          IO::store(dr + VE * idx, gs[i]);
+          IO::store(dr + voff[i], gs[i]);
         }
       }
     }
+  };
+
+  // The main loop covers the iterations in which every team has a row; the last,
+  // partly filled iteration is masked.
+  Slot q;
+  if constexpr (kPrefetch) issue(q, first_row);
+  const int64_t full_iters = rows / rows_per_iter;
+  int64_t it = 0;
+  if (nvec == TPR * V) {
+    for (; it < full_iters; ++it) process(q, it, std::true_type{}, std::true_type{});
   }
+  else {
+    for (; it < full_iters; ++it) process(q, it, std::true_type{}, std::false_type{});
+  }
+  if (it < iters) process(q, it, std::false_type{}, std::false_type{});
 
   if (WGRAD) {
     float* out = part + static_cast<int64_t>(blockIdx.x) * 2 * n;
@@ -408,38 +468,55 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   }
 }
 
-// Sums P partial rows: grid (ceil(n/32), 2): y == 0 dscale, y == 1 dbias.  A block
-// is 32 feature columns x 8 row groups; the order of additions is fixed.
+// Sums P partial rows: grid (ceil(n/32), 2): y == 0 dscale, y == 1 dbias.  A block is
+// 8 groups of four feature columns x 32 row groups; a thread has its (up to 8) 16-byte
+// loads in flight together, so the kernel costs about one trip to memory.  The order
+// of additions is fixed.  n is a multiple of 4 and part is 16-byte aligned.
 __global__ void __launch_bounds__(256)
 ln_wgrad_reduce(const float* __restrict__ part, int64_t P, int64_t n, float* __restrict__ dscale,
                 float* __restrict__ dbias)
 {
-  __shared__ float sm[8][33];
+  __shared__ float sm[32][33];
+  __shared__ float sm2[8][33];
   float* out = blockIdx.y == 0 ? dscale : dbias;
   if (!out) return;
-  const int kx = threadIdx.x & 31;
-  const int pg = threadIdx.x >> 5;
-  const int64_t k = static_cast<int64_t>(blockIdx.x) * 32 + kx;
-  const float* src = part + blockIdx.y * n + k;
-  float acc = 0.f;
+  const int kq = threadIdx.x & 7;   // column quad
+  const int pg = threadIdx.x >> 3;  // row group
+  const int64_t k = static_cast<int64_t>(blockIdx.x) * 32 + 4 * kq;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
   if (k < n) {
-    int64_t p = pg;
-    for (; p + 24 < P; p += 32) {
-      const float a0 = src[p * 2 * n];
-      const float a1 = src[(p + 8) * 2 * n];
-      const float a2 = src[(p + 16) * 2 * n];
-      const float a3 = src[(p + 24) * 2 * n];
-      acc += (a0 + a1) + (a2 + a3);
-    }
-    for (; p < P; p += 8) acc += src[p * 2 * n];
-  }
-  sm[pg][kx] = acc;
-  __syncthreads();
-  if (pg == 0 && k < n) {
-    float r = sm[0][kx];
+    const float* src = part + blockIdx.y * n + k;
+    for (int64_t p0 = pg; p0 < P; p0 += 256) {
+      float w[8][4];
 #pragma unroll
-    for (int i = 1; i < 8; ++i) r += sm[i][kx];
-    out[k] = r;
+      for (int j = 0; j < 8; ++j) {
+        const int64_t p = p0 + 32 * j;
+        if (p < P) {
+          Vec16<float>::load(src + p * 2 * n, w[j]);
+        }
+        else {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) w[j][c] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        acc[c] += ((w[0][c] + w[1][c]) + (w[2][c] + w[3][c])) + ((w[4][c] + w[5][c]) + (w[6][c] + w[7][c]));
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) sm[pg][4 * kq + c] = acc[c];
+  __syncthreads();
+  {
+    const int c = threadIdx.x & 31, o = threadIdx.x >> 5;
+    sm2[o][c] = (sm[4 * o][c] + sm[4 * o + 1][c]) + (sm[4 * o + 2][c] + sm[4 * o + 3][c]);
+  }
+  __syncthreads();
+  if (threadIdx.x < 32) {
+    const int c = threadIdx.x;
+    const int64_t kc = static_cast<int64_t>(blockIdx.x) * 32 + c;
+    if (kc < n)
+      out[kc] = ((sm2[0][c] + sm2[1][c]) + (sm2[2][c] + sm2[3][c])) + ((sm2[4][c] + sm2[5][c]) + (sm2[6][c] + sm2[7][c]));
   }
 }
 
@@ -530,49 +607,56 @@ fill_matrix(T* p, int64_t h, int64_t w, int64_t ld, float value)
 struct LnBwdPlan {
   int tpr, teams, v;
   int64_t blocks;  // == number of partial rows
-  int depth;       // rows in flight per team
 };
 
-// At most this many persistent blocks: each leaves 2*n floats of partial sums, so
-// fewer blocks mean less extra traffic; 256 = one per compute unit.
-constexpr int64_t kLnBwdMaxBlocks = 256;
+// Persistent blocks: each leaves 2*n floats of partial sums, which are written once
+// and read once, so fewer blocks mean less extra traffic, while more blocks hide more
+// latency.  One block per compute unit (256) is the floor; the count doubles (up to
+// 1024) as long as the partial sums stay below 1/20 of the tensor traffic.
+constexpr int64_t kLnBwdMinBlocks = 256;
+constexpr int64_t kLnBwdMaxBlocks = 1024;
 
+static int64_t ln_bwd_block_limit(int64_t rows, int elem_bytes)
+{
+  static const int64_t forced = std::getenv("LBN_LN_BWD_BLOCKS") ? std::atoi(std::getenv("LBN_LN_BWD_BLOCKS")) : 0;
+  if (forced > 0) return forced;
+  // partial traffic / tensor traffic = blocks * 2n * 4 * 2 / (3 * rows * n * elem_bytes)
+  int64_t blocks = kLnBwdMinBlocks;
+  while (blocks < kLnBwdMaxBlocks && 2 * blocks * 16 * 20 <= 3 * rows * elem_bytes) blocks *= 2;
+  return blocks;
+}
+
+// Blocks have at most 512 threads, which leaves every thread 256 registers: per owned
+// entry a thread keeps the scale, two fp32 accumulators and two fp32 working values.
+// Narrow teams with several vectors per thread spend the least on the row reduction,
+// so the narrowest team that owns at most 16 entries per thread is taken; rows too
+// long for that go to 512-thread teams with up to 32 entries per thread.
 static LnBwdPlan plan_ln_bwd(int64_t nvec, int64_t rows, int ve)
 {
-  static const int force_depth = std::getenv("LBN_LN_BWD_DEPTH") ? std::atoi(std::getenv("LBN_LN_BWD_DEPTH")) : -1;
   static const int force_tpr = std::getenv("LBN_LN_BWD_TPR") ? std::atoi(std::getenv("LBN_LN_BWD_TPR")) : 0;
   static const int force_teams = std::getenv("LBN_LN_BWD_TEAMS") ? std::atoi(std::getenv("LBN_LN_BWD_TEAMS")) : 0;
-  static const int64_t max_blocks = std::getenv("LBN_LN_BWD_BLOCKS") ? std::atoi(std::getenv("LBN_LN_BWD_BLOCKS")) : kLnBwdMaxBlocks;
-  // Registers per thread: two fp32 accumulators per owned entry plus the packed rows
-  // in flight.  Few vectors per thread leave room for a deeper prefetch, so the
-  // widest team that still keeps every thread busy is preferred.
-  LnBwdPlan p{0, 0, 0, 0, 0};
-  const int tprs[4] = {64, 256, 512, 1024};
-  const int teams[4] = {4, 4, 2, 1};
-  const int max_v = ve == 8 ? 2 : 4;
+  const int64_t max_blocks = ln_bwd_block_limit(rows, 16 / ve);
+  LnBwdPlan p{0, 0, 0, 0};
+  const int tprs[3] = {64, 256, 512};
+  const int teams[3] = {4, 2, 1};
+  const int v_pref = 16 / ve, v_max = 32 / ve;
   int pick = -1;
-  for (int i = 0; i < 4; ++i) {
-    if (force_tpr && tprs[i] != force_tpr) continue;
-    const int64_t v = ceil_div(nvec, tprs[i]);
-    if (v > max_v) continue;
-    if (pick < 0) pick = i;
-    // prefer one vector per thread when the wider team is still fully used
-    if (v == 1 && nvec * 2 > tprs[i]) { pick = i; break; }
-  }
+  for (int pass = 0; pass < 2 && pick < 0; ++pass)
+    for (int i = 0; i < 3 && pick < 0; ++i) {
+      if (force_tpr && tprs[i] != force_tpr) continue;
+      const int64_t v = ceil_div(nvec, tprs[i]);
+      // 32 entries per thread are instantiated for the widest team only
+      if (v <= (pass == 0 ? v_pref : (tprs[i] == 512 || force_tpr ? v_max : v_pref))) pick = i;
+    }
   if (pick < 0) return p;
   p.tpr = tprs[pick];
   p.teams = teams[pick];
   p.v = round_up_pow2_le8(ceil_div(nvec, p.tpr));
-  if (p.tpr == 512 && p.v > 1) p.teams = 1;  // two such teams would not fit their LDS merge buffer
   if (force_teams && force_teams <= p.teams) p.teams = force_teams;
   // spread small problems: fewer teams per block when rows are scarce
-  while (p.teams > 1 && p.tpr * p.teams > 256 && ceil_div(rows, p.teams) < max_blocks) p.teams /= 2;
+  while (p.teams > 1 && p.tpr * p.teams > 256 && ceil_div(rows, p.teams) < kLnBwdMinBlocks) p.teams /= 2;
   p.blocks = ceil_div(rows, p.teams);
   if (p.blocks > max_blocks) p.blocks = max_blocks;
-  const int64_t rows_per_team = ceil_div(rows, p.blocks * p.teams);
-  p.depth = p.v == 1 ? 3 : (p.v == 2 ? 1 : 0);
-  if (rows_per_team <= 1) p.depth = 0;
-  if (force_depth >= 0 && force_depth <= 3) p.depth = p.v > 2 ? 0 : (p.v == 2 && force_depth > 1 ? 1 : force_depth);
   return p;
 }
 
@@ -609,10 +693,14 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
 #define X(TPR, V)                                                                              \
   if (c.tpr == TPR && c.v == V) {                                                              \
     using B = RowBlock<TPR>;                                                                   \
-    const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                    \
-    hipLaunchKernelGGL((ln_fwd_rows<T, TPR, V>), dim3(grid), dim3(B::kThreads), 0, st, x, y,   \
-                       ldx, ldy, map, rows, nvec, static_cast<int>(n), eps, stats, lds, gamma, \
-                       beta, sumsq);                                                           \
+    const int64_t units = ceil_div(rows, B::kTeams);                                           \
+    const int64_t resident = resident_blocks(ln_fwd_rows<T, TPR, V>, B::kThreads);             \
+    if (resident <= 0) return LBN_ERR_UNSUPPORTED;                                             \
+    /* one wave of blocks, each walking the same number of rows */                             \
+    const int64_t grid = ceil_div(units, ceil_div(units, resident));                           \
+    hipLaunchKernelGGL((ln_fwd_rows<T, TPR, V>), dim3(static_cast<unsigned>(grid)),            \
+                       dim3(B::kThreads), 0, st, x, y, ldx, ldy, map, rows, nvec,              \
+                       1.0f / static_cast<float>(n), eps, stats, lds, gamma, beta, sumsq);     \
     return launch_status();                                                                    \
   }
       X(64, 1) X(64, 2) X(64, 4) X(256, 1) X(256, 2) X(256, 4) X(1024, 1) X(1024, 2) X(1024, 4)
@@ -626,7 +714,7 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
   return launch_status();
 }
 
-template <typename T, int TPR, int TEAMS, int V, int DEPTH>
+template <typename T, int TPR, int TEAMS, int V>
 static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const T* x, const T* dy,
                                T* dx, int64_t ldx, int64_t lddy, int64_t lddx, RowMap map,
                                int64_t rows, int nvec, int n, float eps, const float* stats,
@@ -636,10 +724,10 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
   using B = RowBlock<TPR, TEAMS>;
   const dim3 grid(static_cast<unsigned>(blocks)), block(B::kThreads);
   if (wgrad)
-    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, true, DEPTH>), grid, block, 0, st, x, dy, dx, ldx,
+    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, true>), grid, block, 0, st, x, dy, dx, ldx,
                        lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part);
   else
-    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, false, 0>), grid, block, 0, st, x, dy, dx, ldx,
+    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, false>), grid, block, 0, st, x, dy, dx, ldx,
                        lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part);
 }
 
@@ -692,20 +780,16 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
       }
       const int nvec = static_cast<int>(n / VE);
       bool launched = false;
-#define X(TPR, TEAMS, V, D)                                                                     \
-  if (!launched && p.tpr == TPR && p.teams == TEAMS && p.v == V && p.depth == D) {              \
-    launch_ln_bwd_rows<T, TPR, TEAMS, V, D>(st, wgrad, p.blocks, x, dy, dx, ldx, lddy, lddx,    \
-                                            map, rows, nvec, static_cast<int>(n), eps, stats,   \
-                                            lds, sgrad, ldsg, gamma, part);                     \
+#define X(TPR, TEAMS, V)                                                                        \
+  if (!launched && p.tpr == TPR && p.teams == TEAMS && p.v == V) {                              \
+    launch_ln_bwd_rows<T, TPR, TEAMS, V>(st, wgrad, p.blocks, x, dy, dx, ldx, lddy, lddx, map,  \
+                                         rows, nvec, static_cast<int>(n), eps, stats, lds,      \
+                                         sgrad, ldsg, gamma, part);                             \
     launched = true;                                                                            \
   }
-#define XD(TPR, TEAMS, V) X(TPR, TEAMS, V, 0) X(TPR, TEAMS, V, 1) X(TPR, TEAMS, V, 2) X(TPR, TEAMS, V, 3)
-#define XS(TPR, TEAMS, V) X(TPR, TEAMS, V, 0) X(TPR, TEAMS, V, 1)
-      XD(64, 4, 1) XS(64, 4, 2) XD(256, 1, 1) XS(256, 1, 2) XD(256, 2, 1) XS(256, 2, 2) XD(256, 4, 1)
-      XS(256, 4, 2) XD(512, 1, 1) XS(512, 1, 2) XD(512, 2, 1) XD(1024, 1, 1) XS(1024, 1, 2)
-      if constexpr (VE == 4) { X(64, 4, 4, 0) X(256, 1, 4, 0) X(256, 2, 4, 0) X(256, 4, 4, 0) X(512, 1, 4, 0) X(1024, 1, 4, 0) }
-#undef XS
-#undef XD
+      X(64, 4, 1) X(64, 4, 2) X(64, 4, 4) X(256, 2, 1) X(256, 2, 2) X(256, 1, 1) X(256, 1, 2)
+      X(512, 1, 1) X(512, 1, 2) X(512, 1, 4)
+      if constexpr (VE == 4) { X(256, 2, 4) X(256, 1, 4) X(512, 1, 8) }
 #undef X
       if (launched) {
         if (wgrad) {
