@@ -131,6 +131,10 @@ def main():
         "cfg4_layer_norm_f16": ("LayerNorm fwd+bwd fp16 storage 4096x8192", lambda: build_ln(W.cfg4_layer_norm_f16(), True)),
         "cfg5a_channelwise_softmax": ("ChannelwiseSoftmax fwd+bwd fp32 256x64x4096", lambda: build_cws(W.cfg5a_channelwise_softmax())),
         "cfg5b_wide_softmax": ("Softmax fwd+bwd fp32 262144x16 (split rows)", lambda: build_softmax("softmax", W.cfg5b_wide_softmax())),
+        # not a baseline configuration: cfg5b's rows at 16x the width, where the multi-workgroup
+        # split kernels run long enough to be measured against bandwidth rather than launch latency
+        "extra_wide_softmax_w256": ("Softmax fwd+bwd fp32 262144x256 (split rows, informational)",
+                                    lambda: build_softmax("softmax", W.cfg5b_wide_softmax(w=256))),
     }
     headline = "cfg2_softmax"
     if args.layers == "all":
@@ -186,6 +190,35 @@ def main():
         bwd_b2b = a.elapsed_time(b) / steps
         return wall, fwd, bwd, bwd_b2b
 
+    def measure_cold(builder, set_bytes, steps, warmup):
+        """Whole-step wall clock with the tensors rotated among enough independent copies
+        (>= 1 GiB in total) that no step finds its inputs in L2 or the Infinity Cache."""
+        copies = max(2, min(512, -(-(1 << 30) // set_bytes)))
+        lib = L.capi.lib()
+        calls = []
+        keep = []
+        for _ in range(copies):
+            layer = builder()[0]
+            keep.append(layer)
+            fname, fargs = layer.fp_call()
+            bname, bargs = layer.bp_call()
+            calls.append((getattr(lib, fname), fargs, getattr(lib, bname), bargs))
+
+        def run(n, first):
+            for i in range(first, first + n):
+                ffn, fargs, bfn, bargs = calls[i % copies]
+                if ffn(*fargs) or bfn(*bargs):
+                    raise RuntimeError("kernel launch failed")
+
+        run(warmup, 0)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run(steps, warmup)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        del keep
+        return wall, copies
+
     results = {}
     cpu_threads = None
     for name in names:
@@ -207,6 +240,12 @@ def main():
             "fwd_gbs": fwd_b / (f_ms * 1e-3) / 1e9, "bwd_gbs": bwd_b / (b_ms * 1e-3) / 1e9,
             "bwd_back_to_back_ms": bwd_b2b,
         }
+        if 4 * elems * esize <= (256 << 20):
+            # small working set: a second, cold figure next to the cache-resident one
+            cwall, copies = measure_cold(builder, 4 * elems * esize, args.steps, args.warmup)
+            cms = cwall / args.steps * 1e3
+            r["cold"] = {"copies": copies, "ms_per_step": cms, "gbs": (fwd_b + bwd_b) / (cms * 1e-3) / 1e9,
+                         "frac_of_hbm_peak": (fwd_b + bwd_b) / (cms * 1e-3) / 1e9 / HBM_PEAK_GBS}
         if not args.no_cpu:
             from oracle import cpu_oracle as orc
             cpu_threads = orc.max_threads()
@@ -218,6 +257,7 @@ def main():
         results[name] = r
         print(f"# {name}: {step_ms*1e3:8.1f} us/step  {r['gbs']:7.0f} GB/s ({100*r['frac_of_hbm_peak']:.1f}% of 8 TB/s)  "
               f"fwd {f_ms*1e3:7.1f} us ({r['fwd_gbs']:.0f} GB/s)  bwd {b_ms*1e3:7.1f} us ({r['bwd_gbs']:.0f} GB/s)"
+              + (f"  cold {r['cold']['ms_per_step']*1e3:.1f} us/step" if "cold" in r else "")
               + (f"  cpu {r['cpu']['gbs']:.1f} GB/s" if "cpu" in r else ""), file=sys.stderr, flush=True)
         del layer
         torch.cuda.empty_cache()

@@ -189,156 +189,249 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
 }
 
 
+// Merges the online-softmax pairs (m, acc) of the 256 threads of a workgroup (defined
+// with the split-row kernels below).
+__device__ __forceinline__ void block_merge_max_sum(float& m, float& acc, float (*slot)[2]);
+
 // ================================================ register-resident row clusters
 // Rows too long for one workgroup's registers: a cluster of M workgroups shares a
 // row, workgroup k keeps vectors [k*256*V, (k+1)*256*V) in registers, the cluster
 // exchanges one (max, sum) pair per workgroup and every workgroup finishes from its
 // registers.  One read and one write per element, and safe in place: a workgroup
 // has read its whole share before it writes any of it, and shares are disjoint.
-template <int V, int KIND>
-__global__ void __launch_bounds__(kClusterThreads)
-sm_fwd_cluster(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
-               unsigned nvec, int M, ClusterWorkspace cw, ClusterTag tag)
+//
+// The grid is persistent (cluster cl handles rows cl, cl + nclusters, ...) and rotates
+// three register tiles so that nothing waits on something issued in the same step: in
+// step s a workgroup (1) reduces tile s+1, whose loads were issued a step earlier, and
+// publishes its partial pair, (2) issues the loads of tile s+2, (3) collects the
+// cluster's partials of tile s, published a step earlier, and finishes tile s.
+struct SmClusterArgs {
+  const float* a;  // forward: x; backward: y
+  const float* g;  // backward: dy
+  float* out;
+  int64_t lda, ldg, ldo;
+  RowMap map;
+  int64_t rows;
+  unsigned nvec;
+  int M;
+  ClusterWorkspace cw;
+  ClusterTag tag;
+  __device__ __forceinline__ unsigned long long* slots(int64_t row) const { return cw.slots + row * M * 2; }
+};
+
+template <int V>
+struct SmFwdTile {
+  float v[V][4];
+  float m;  // the thread's own maximum: v holds exp(x - m) (or x - m for log-softmax)
+};
+
+template <int V>
+__device__ __forceinline__ void sm_cl_load(float (&t)[V][4], const float* rowp, unsigned base,
+                                           unsigned nvec, float fill)
 {
-  constexpr int NW = kClusterThreads / kWave;
-  __shared__ float red[2][NW];
-  __shared__ float bc[2];
-  const int nclusters = gridDim.x / M;
-  const int cl = blockIdx.x / M;
-  const int k = blockIdx.x - cl * M;
-  const unsigned tid = threadIdx.x;
-  const int lane = tid & (kWave - 1);
-  const int wv = tid / kWave;
-  const unsigned base = static_cast<unsigned>(k) * (kClusterThreads * V) + tid;
-  for (int64_t row = cl; row < rows; row += nclusters) {
-    const float* xr = x + map.offset(row, ldx);
-    float v[V][4];
 #pragma unroll
-    for (int i = 0; i < V; ++i) {
-      const unsigned idx = base + i * kClusterThreads;
-      if (idx < nvec) {
-        Vec16<float>::load(xr + 4 * static_cast<int64_t>(idx), v[i]);
-      }
-      else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[i][j] = -FLT_MAX;
-      }
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = base + i * kClusterThreads;
+    if (idx < nvec) {
+      Vec16<float>::load(rowp + 4 * static_cast<int64_t>(idx), t[i]);
     }
-    float m = -FLT_MAX;
+    else {
 #pragma unroll
-    for (int i = 0; i < V; ++i)
+      for (int j = 0; j < 4; ++j) t[i][j] = fill;
+    }
+  }
+}
+
+// (1) of a step: thread-local online softmax, one merge of the (max, sum) pairs of the
+// workgroup, published for the cluster.
+template <int V, int KIND>
+__device__ __forceinline__ void sm_cl_fwd_reduce(const SmClusterArgs& a, int64_t row, int k, unsigned base,
+                                                 SmFwdTile<V>& t, float (*red)[2])
+{
+  float m = -FLT_MAX;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) m = fmaxf(m, v[i][j]);
-    m = team_max<NW>(m, red[0], wv, lane);
-    float s = 0.f;
+  for (int i = 0; i < V; ++i)
 #pragma unroll
-    for (int i = 0; i < V; ++i) {
-      const bool ok = base + i * kClusterThreads < nvec;
+    for (int j = 0; j < 4; ++j) m = fmaxf(m, t.v[i][j]);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const bool ok = base + i * kClusterThreads < a.nvec;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float d = t.v[i][j] - m;
+      const float e = ok ? (KIND == kChannelwise ? exp_keep_denormals(d) : exp_fast(d)) : 0.f;
+      s += e;
+      t.v[i][j] = (KIND == kLogSoftmax) ? d : e;
+    }
+  }
+  t.m = m;
+  block_merge_max_sum(m, s, red);
+  if (threadIdx.x == 0) cluster_publish(m, s, a.slots(row), k, a.tag);
+}
+
+// (3) of a step.
+template <int V, int KIND>
+__device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t row, unsigned base,
+                                                 SmFwdTile<V>& t, float* bc)
+{
+  if (threadIdx.x < kWave) {
+    float pm, ps;
+    cluster_collect(a.slots(row), a.M, a.tag, a.cw.error, -FLT_MAX, 0.f, pm, ps);
+    const float gmax = wave_max(pm);
+    const float gsum = wave_sum(ps * exp_fast(pm - gmax));
+    if (threadIdx.x == 0) {
+      bc[0] = gmax;
+      bc[1] = gsum;
+    }
+  }
+  __syncthreads();
+  const float gm = bc[0];
+  const float gs = bc[1];
+  float* yr = a.out + a.map.offset(row, a.ldo);
+  const float shift = t.m - gm;                     // <= 0: this thread's maximum against the row's
+  const float f = exp_fast(shift) * (1.0f / gs);    // rescales exp(x - m) to exp(x - gm) / sum
+  const float lse = (KIND == kLogSoftmax) ? log_of_sum(gs) : 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = base + i * kClusterThreads;
+    if (idx < a.nvec) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float d = v[i][j] - m;
-        const float e = ok ? (KIND == kChannelwise ? exp_keep_denormals(d) : exp_fast(d)) : 0.f;
-        s += e;
-        v[i][j] = (KIND == kLogSoftmax) ? d : e;
-      }
-    }
-    s = team_sum<NW>(s, red[1], wv, lane);
-    if (tid < kWave) {
-      float pm, ps;
-      cluster_exchange(m, s, cw.slots + row * M * 2, k, M, tag, cw.error, -FLT_MAX, 0.f, pm, ps);
-      const float gmax = wave_max(pm);
-      const float gsum = wave_sum(ps * exp_fast(pm - gmax));
-      if (tid == 0) {
-        bc[0] = gmax;
-        bc[1] = gsum;
-      }
-    }
-    __syncthreads();
-    const float gm = bc[0];
-    const float gs = bc[1];
-    float* yr = y + map.offset(row, ldy);
-    const float shift = m - gm;                       // <= 0: this share's maximum against the row's
-    const float f = exp_fast(shift) * (1.0f / gs);    // rescales exp(x - m) to exp(x - gm) / sum
-    const float lse = (KIND == kLogSoftmax) ? log_of_sum(gs) : 0.f;
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-      const unsigned idx = base + i * kClusterThreads;
-      if (idx < nvec) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (KIND == kSoftmax) {
-            const float r = f * v[i][j];
-            v[i][j] = __builtin_isnormal(r) ? r : 0.f;
-          }
-          else if (KIND == kLogSoftmax) {
-            v[i][j] = (v[i][j] + shift) - lse;
-          }
-          else {
-            v[i][j] *= f;
-          }
+        if (KIND == kSoftmax) {
+          const float r = f * t.v[i][j];
+          t.v[i][j] = __builtin_isnormal(r) ? r : 0.f;
         }
-        Vec16<float>::store(yr + 4 * static_cast<int64_t>(idx), v[i]);
+        else if (KIND == kLogSoftmax) {
+          t.v[i][j] = (t.v[i][j] + shift) - lse;
+        }
+        else {
+          t.v[i][j] *= f;
+        }
       }
+      Vec16<float>::store(yr + 4 * static_cast<int64_t>(idx), t.v[i]);
     }
   }
 }
 
 template <int V, int KIND>
-__global__ void __launch_bounds__(kClusterThreads)
-sm_bwd_cluster(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
-               RowMap map, int64_t rows, unsigned nvec, int M, ClusterWorkspace cw, ClusterTag tag)
+__device__ __forceinline__ void sm_cl_fwd_step(const SmClusterArgs& a, int64_t row, int64_t nc, int k,
+                                               unsigned base, SmFwdTile<V>& F, SmFwdTile<V>& R,
+                                               SmFwdTile<V>& L, float (*red)[2], float* bc)
 {
-  constexpr int NW = kClusterThreads / kWave;
-  __shared__ float red[NW];
+  if (row + nc < a.rows) sm_cl_fwd_reduce<V, KIND>(a, row + nc, k, base, R, red);
+  if (row + 2 * nc < a.rows)
+    sm_cl_load<V>(L.v, a.a + a.map.offset(row + 2 * nc, a.lda), base, a.nvec, -FLT_MAX);
+  asm volatile("" ::: "memory");  // keep the loads above the wait below
+  sm_cl_fwd_finish<V, KIND>(a, row, base, F, bc);
+}
+
+template <int V, int KIND>
+__global__ void __launch_bounds__(kClusterThreads)
+sm_fwd_cluster(SmClusterArgs a)
+{
+  __shared__ float red[kClusterThreads / kWave][2];
+  __shared__ float bc[2];
+  const int64_t nc = gridDim.x / a.M;
+  const int64_t cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - static_cast<int>(cl) * a.M;
+  const unsigned base = static_cast<unsigned>(k) * (kClusterThreads * V) + threadIdx.x;
+  if (cl >= a.rows) return;
+  SmFwdTile<V> t0, t1, t2;
+  sm_cl_load<V>(t0.v, a.a + a.map.offset(cl, a.lda), base, a.nvec, -FLT_MAX);
+  if (cl + nc < a.rows) sm_cl_load<V>(t1.v, a.a + a.map.offset(cl + nc, a.lda), base, a.nvec, -FLT_MAX);
+  sm_cl_fwd_reduce<V, KIND>(a, cl, k, base, t0, red);
+  for (int64_t row = cl; row < a.rows; row += 3 * nc) {
+    sm_cl_fwd_step<V, KIND>(a, row, nc, k, base, t0, t1, t2, red, bc);
+    if (row + nc < a.rows) sm_cl_fwd_step<V, KIND>(a, row + nc, nc, k, base, t1, t2, t0, red, bc);
+    if (row + 2 * nc < a.rows) sm_cl_fwd_step<V, KIND>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc);
+  }
+}
+
+template <int V>
+struct SmBwdTile {
+  float a[V][4];
+  float g[V][4];
+};
+
+template <int V, int KIND>
+__device__ __forceinline__ void sm_cl_bwd_reduce(const SmClusterArgs& a, int64_t row, int k,
+                                                 const SmBwdTile<V>& t, float* red)
+{
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s += (KIND == kLogSoftmax) ? t.g[i][j] : t.a[i][j] * t.g[i][j];
+  s = team_sum<kClusterThreads / kWave>(s, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+  if (threadIdx.x == 0) cluster_publish(s, 0.f, a.slots(row), k, a.tag);
+}
+
+template <int V, int KIND>
+__device__ __forceinline__ void sm_cl_bwd_finish(const SmClusterArgs& a, int64_t row, unsigned base,
+                                                 SmBwdTile<V>& t, float* bc)
+{
+  if (threadIdx.x < kWave) {
+    float pt, unused;
+    cluster_collect(a.slots(row), a.M, a.tag, a.cw.error, 0.f, 0.f, pt, unused);
+    pt = wave_sum(pt);
+    if (threadIdx.x == 0) bc[0] = pt;
+  }
+  __syncthreads();
+  const float tot = bc[0];
+  float* dr = a.out + a.map.offset(row, a.ldo);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = base + i * kClusterThreads;
+    if (idx < a.nvec) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (KIND == kLogSoftmax) t.g[i][j] = t.g[i][j] - exp_fast(t.a[i][j]) * tot;
+        else t.g[i][j] = t.a[i][j] * (t.g[i][j] - tot);
+      }
+      Vec16<float>::store(dr + 4 * static_cast<int64_t>(idx), t.g[i]);
+    }
+  }
+}
+
+template <int V>
+__device__ __forceinline__ void sm_cl_bwd_load(const SmClusterArgs& a, int64_t row, unsigned base,
+                                               SmBwdTile<V>& t)
+{
+  sm_cl_load<V>(t.a, a.a + a.map.offset(row, a.lda), base, a.nvec, 0.f);
+  sm_cl_load<V>(t.g, a.g + a.map.offset(row, a.ldg), base, a.nvec, 0.f);
+}
+
+template <int V, int KIND>
+__device__ __forceinline__ void sm_cl_bwd_step(const SmClusterArgs& a, int64_t row, int64_t nc, int k,
+                                               unsigned base, SmBwdTile<V>& F, SmBwdTile<V>& R,
+                                               SmBwdTile<V>& L, float* red, float* bc)
+{
+  if (row + nc < a.rows) sm_cl_bwd_reduce<V, KIND>(a, row + nc, k, R, red);
+  if (row + 2 * nc < a.rows) sm_cl_bwd_load<V>(a, row + 2 * nc, base, L);
+  asm volatile("" ::: "memory");
+  sm_cl_bwd_finish<V, KIND>(a, row, base, F, bc);
+}
+
+template <int V, int KIND>
+__global__ void __launch_bounds__(kClusterThreads)
+sm_bwd_cluster(SmClusterArgs a)
+{
+  __shared__ float red[kClusterThreads / kWave];
   __shared__ float bc[1];
-  const int nclusters = gridDim.x / M;
-  const int cl = blockIdx.x / M;
-  const int k = blockIdx.x - cl * M;
-  const unsigned tid = threadIdx.x;
-  const unsigned base = static_cast<unsigned>(k) * (kClusterThreads * V) + tid;
-  for (int64_t row = cl; row < rows; row += nclusters) {
-    const float* yr = y + map.offset(row, ldy);
-    const float* gr = dy + map.offset(row, lddy);
-    float a[V][4], g[V][4];
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-      const unsigned idx = base + i * kClusterThreads;
-      if (idx < nvec) {
-        Vec16<float>::load(yr + 4 * static_cast<int64_t>(idx), a[i]);
-        Vec16<float>::load(gr + 4 * static_cast<int64_t>(idx), g[i]);
-      }
-      else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) a[i][j] = g[i][j] = 0.f;
-      }
-    }
-    float s = 0.f;
-#pragma unroll
-    for (int i = 0; i < V; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) s += (KIND == kLogSoftmax) ? g[i][j] : a[i][j] * g[i][j];
-    s = team_sum<NW>(s, red, tid / kWave, tid & (kWave - 1));
-    if (tid < kWave) {
-      float pt, unused;
-      cluster_exchange(s, 0.f, cw.slots + row * M * 2, k, M, tag, cw.error, 0.f, 0.f, pt, unused);
-      pt = wave_sum(pt);
-      if (tid == 0) bc[0] = pt;
-    }
-    __syncthreads();
-    const float tot = bc[0];
-    float* dr = dx + map.offset(row, lddx);
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-      const unsigned idx = base + i * kClusterThreads;
-      if (idx < nvec) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (KIND == kLogSoftmax) g[i][j] = g[i][j] - exp_fast(a[i][j]) * tot;
-          else g[i][j] = a[i][j] * (g[i][j] - tot);
-        }
-        Vec16<float>::store(dr + 4 * static_cast<int64_t>(idx), g[i]);
-      }
-    }
+  const int64_t nc = gridDim.x / a.M;
+  const int64_t cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - static_cast<int>(cl) * a.M;
+  const unsigned base = static_cast<unsigned>(k) * (kClusterThreads * V) + threadIdx.x;
+  if (cl >= a.rows) return;
+  SmBwdTile<V> t0, t1, t2;
+  sm_cl_bwd_load<V>(a, cl, base, t0);
+  if (cl + nc < a.rows) sm_cl_bwd_load<V>(a, cl + nc, base, t1);
+  sm_cl_bwd_reduce<V, KIND>(a, cl, k, t0, red);
+  for (int64_t row = cl; row < a.rows; row += 3 * nc) {
+    sm_cl_bwd_step<V, KIND>(a, row, nc, k, base, t0, t1, t2, red, bc);
+    if (row + nc < a.rows) sm_cl_bwd_step<V, KIND>(a, row + nc, nc, k, base, t1, t2, t0, red, bc);
+    if (row + 2 * nc < a.rows) sm_cl_bwd_step<V, KIND>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc);
   }
 }
 
@@ -658,18 +751,22 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     }
   }
   if (vec && cluster_enabled(rows, n) && n / 4 < (int64_t(1) << 30)) {
-    const ClusterPlan cp = plan_cluster(n / 4, 8);
+    // four vectors per thread keep five workgroups per CU resident; eight only for rows that need it
+    ClusterPlan cp = plan_cluster(n / 4, 4);
+    if (!cp.M) cp = plan_cluster(n / 4, 8);
     if (cp.M) {
       if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
       const ClusterWorkspace cw = cluster_workspace(ws);
 #define X(VV)                                                                                    \
   if (cp.V == VV) {                                                                              \
     const int cap = cluster_capacity(sm_fwd_cluster<VV, KIND>, kClusterThreads);                 \
-    const int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                   \
+    int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
     if (ncl >= 1) {                                                                              \
+      ncl = ceil_div(rows, ceil_div(rows, ncl)); /* every cluster walks the same number of rows */ \
+      const SmClusterArgs a{x, nullptr, y, ldx, 0, ldy, map, rows, static_cast<unsigned>(n / 4), \
+                            cp.M, cw, next_cluster_tag()};                                       \
       hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND>), dim3(static_cast<unsigned>(ncl * cp.M)),    \
-                         dim3(kClusterThreads), 0, st, x, y, ldx, ldy, map, rows,                \
-                         static_cast<unsigned>(n / 4), cp.M, cw, next_cluster_tag());            \
+                         dim3(kClusterThreads), 0, st, a);                                       \
       return launch_status();                                                                    \
     }                                                                                            \
   }
@@ -739,11 +836,13 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #define X(VV)                                                                                    \
   if (cp.V == VV) {                                                                              \
     const int cap = cluster_capacity(sm_bwd_cluster<VV, KIND>, kClusterThreads);                 \
-    const int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                   \
+    int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
     if (ncl >= 1) {                                                                              \
+      ncl = ceil_div(rows, ceil_div(rows, ncl));                                                 \
+      const SmClusterArgs a{y, dy, dx, ldy, lddy, lddx, map, rows, static_cast<unsigned>(n / 4), \
+                            cp.M, cw, next_cluster_tag()};                                       \
       hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND>), dim3(static_cast<unsigned>(ncl * cp.M)),    \
-                         dim3(kClusterThreads), 0, st, y, dy, dx, ldy, lddy, lddx, map, rows,    \
-                         static_cast<unsigned>(n / 4), cp.M, cw, next_cluster_tag());            \
+                         dim3(kClusterThreads), 0, st, a);                                       \
       return launch_status();                                                                    \
     }                                                                                            \
   }
