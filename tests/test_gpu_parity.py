@@ -148,6 +148,10 @@ LN_CASES = [
     ((8, 512), -1, 33, True, 0), ((8, 512), 0, 6, True, 0), ((16, 64), 1, 700, True, 0),
     ((512,), 0, 6, True, 32), ((100,), 0, 6, True, 3), ((2048,), 0, 2000, True, 0),
     ((5, 1), -1, 4, False, 0),
+    # backward plans: 512-thread teams with 32 entries per thread (masked and full), many
+    # short rows (more than 256 persistent blocks), teams that leave threads idle
+    ((12288,), 0, 5, True, 0), ((8192,), 0, 600, True, 0), ((768,), 0, 3000, True, 0),
+    ((256,), 0, 70000, True, 0), ((5000,), 0, 40, True, 0),
 ]
 
 
@@ -208,7 +212,8 @@ def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
 
 @pytest.mark.parametrize("dims,start_dim,w,pad", [((4096,), 0, 64, 0), ((512,), 0, 100, 0), ((64,), 0, 9, 0),
                                                    ((8, 1024), -1, 5, 0), ((100,), 0, 7, 0), ((2048,), 0, 600, 8),
-                                                   ((16384,), 0, 3, 0)])
+                                                   ((16384,), 0, 3, 0), ((16384,), 0, 40, 0), ((8192,), 0, 300, 0),
+                                                   ((768,), 0, 1000, 0), ((12288,), 0, 9, 0)])
 def test_layer_norm_f16(L, dims, start_dim, w, pad):
     rng = np.random.default_rng(int(np.prod(dims)) * 3 + w)
     h = int(np.prod(dims))
