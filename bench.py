@@ -123,6 +123,21 @@ def main():
             return t1 - t0, t2 - t1
         return layer, data["x"].size, 4, data["x"].shape[1], cpu
 
+    def build_in(data):
+        x, dy = upload(data["x"]), upload(data["dy"])
+        layer = L.instance_norm_layer(data["dims"], data["eps"])
+        layer.bind_forward(x)
+        layer.bind_backward(dy)
+        C = data["dims"][0]
+        cs = data["x"].shape[0] // C
+
+        def cpu():
+            from oracle import cpu_oracle as orc
+            t0 = time.perf_counter(); _, sums = orc.instance_norm_fwd(data["x"], C, cs, data["eps"]); t1 = time.perf_counter()
+            orc.instance_norm_bwd(data["x"], data["dy"], sums, C, cs, data["eps"]); t2 = time.perf_counter()
+            return t1 - t0, t2 - t1
+        return layer, data["x"].size, 4, data["x"].shape[1], cpu
+
     table = {
         "cfg2_softmax": ("Softmax fwd+bwd fp32 32768x512", lambda: build_softmax("softmax", W.cfg2_softmax())),
         "cfg2_log_softmax": ("LogSoftmax fwd+bwd fp32 32768x512", lambda: build_softmax("log_softmax", W.cfg2_softmax())),
@@ -131,6 +146,9 @@ def main():
         "cfg4_layer_norm_f16": ("LayerNorm fwd+bwd fp16 storage 4096x8192", lambda: build_ln(W.cfg4_layer_norm_f16(), True)),
         "cfg5a_channelwise_softmax": ("ChannelwiseSoftmax fwd+bwd fp32 256x64x4096", lambda: build_cws(W.cfg5a_channelwise_softmax())),
         "cfg5b_wide_softmax": ("Softmax fwd+bwd fp32 262144x16 (split rows)", lambda: build_softmax("softmax", W.cfg5b_wide_softmax())),
+        # not a baseline configuration: the first layer beyond the five (instance norm) on cfg3's tensor
+        "extra_instance_norm": ("InstanceNorm fwd+bwd fp32 NCHW 64x256x56x56 (informational)",
+                                lambda: build_in(W.cfg3_batch_norm())),
         # not a baseline configuration: cfg5b's rows at 16x the width, where the multi-workgroup
         # split kernels run long enough to be measured against bandwidth rather than launch latency
         "extra_wide_softmax_w256": ("Softmax fwd+bwd fp32 262144x256 (split rows, informational)",

@@ -88,6 +88,31 @@ int lbn_layer_norm_bwd_f16(lbn_stream_t stream, int64_t num_groups, int64_t norm
                            const float* scale, float* dscale, float* dbias,
                            void* workspace, size_t workspace_bytes);
 
+/* --------------------------------------------------------------- instance norm
+ * Replaces instance_norm_layer::fp_compute / bp_compute
+ * (src/layers/regularizers/instance_norm.cpp:47-127, :137-245; GPU code
+ * instance_norm.cu).  A sample is `channels` contiguous slabs of `channel_size`
+ * entries; every (sample, channel) slab is normalised on its own with the biased
+ * variance, no scale or bias.  stats is the layer's workspace matrix
+ * (2*channels x width): the reference keeps sum(x) and sum(x^2) there
+ * (instance_norm.cpp:72-89), this library keeps the mean in rows [0,C) and the
+ * variance in rows [C,2C); the matrix is private to the layer, which only hands it
+ * from forward to backward.  channel_size <= 1: y = 0 and dx = 0
+ * (instance_norm.cpp:65-68, :164-167).  The backward workspace takes the place of
+ * the reference's local statistics-gradient matrix (instance_norm.cpp:173-174). */
+int lbn_instance_norm_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                              int64_t width, float epsilon,
+                              const float* x, int64_t ldx, float* y, int64_t ldy,
+                              float* stats, int64_t ld_stats);
+size_t lbn_instance_norm_bwd_workspace_bytes(int64_t channels, int64_t channel_size,
+                                             int64_t width);
+int lbn_instance_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                              int64_t width, float epsilon,
+                              const float* x, int64_t ldx, const float* dy, int64_t lddy,
+                              float* dx, int64_t lddx,
+                              const float* stats, int64_t ld_stats,
+                              void* workspace, size_t workspace_bytes);
+
 /* ------------------------------------------------------------------ batch norm
  * Replaces batch_normalization_layer::fp_compute / bp_compute
  * (src/layers/regularizers/batch_normalization.cpp:37-175, :178-329).

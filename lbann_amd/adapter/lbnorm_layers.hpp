@@ -467,4 +467,52 @@ private:
   workspace m_ws;
 };
 
+// ------------------------------------------------------------------ instance norm
+/// include/lbann/layers/regularizers/instance_norm.hpp:52-100.
+template <typename Mat = device_matrix<float>>
+class instance_norm_layer {
+public:
+  explicit instance_norm_layer(double epsilon = 1e-5) : m_epsilon(static_cast<float>(epsilon)) {}
+
+  /// setup_dims (instance_norm.hpp:163-168): output dims = input dims, channels first
+  void setup(const std::vector<int64_t>& dims)
+  {
+    if (dims.empty()) throw exception("instance norm layer needs at least one tensor dimension");
+    m_dims = dims;
+  }
+  int64_t num_channels() const { return m_dims.front(); }
+  int64_t channel_size() const { return detail::product(m_dims, 0, m_dims.size()) / m_dims.front(); }
+
+  layer_io<Mat> io;
+  /// means in rows [0,C), variances in rows [C,2C) of every column
+  device_matrix<float> m_workspace;
+
+  void fp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    Mat& y = *io.activations;
+    m_workspace.Resize(2 * num_channels(), x.Width());
+    check_status(lbn_instance_norm_fwd_f32(io.stream, num_channels(), channel_size(), x.Width(), m_epsilon,
+                                           x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(),
+                                           m_workspace.Buffer(), m_workspace.LDim()),
+                 "instance_norm_layer::fp_compute");
+  }
+  void bp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    const Mat& dy = *io.prev_error_signals;
+    Mat& dx = *io.error_signals;
+    const size_t bytes = lbn_instance_norm_bwd_workspace_bytes(num_channels(), channel_size(), x.Width());
+    check_status(lbn_instance_norm_bwd_f32(io.stream, num_channels(), channel_size(), x.Width(), m_epsilon,
+                                           x.LockedBuffer(), x.LDim(), dy.LockedBuffer(), dy.LDim(),
+                                           dx.Buffer(), dx.LDim(), m_workspace.LockedBuffer(),
+                                           m_workspace.LDim(), m_ws.reserve(bytes), bytes),
+                 "instance_norm_layer::bp_compute");
+  }
+private:
+  float m_epsilon;
+  std::vector<int64_t> m_dims;
+  workspace m_ws;
+};
+
 }  // namespace lbnorm

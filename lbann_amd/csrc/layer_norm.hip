@@ -726,9 +726,16 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
   if (wgrad)
     hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, true>), grid, block, 0, st, x, dy, dx, ldx,
                        lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part);
-  else
-    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, false>), grid, block, 0, st, x, dy, dx, ldx,
+  else {
+    // nothing to accumulate across rows: one resident wave of blocks, each walking the
+    // same number of rows with the next row in flight
+    const int64_t units = ceil_div(rows, TEAMS);
+    int64_t resident = resident_blocks(ln_bwd_rows<T, TPR, TEAMS, V, false>, B::kThreads);
+    if (resident < 1) resident = 1;
+    const dim3 all(static_cast<unsigned>(ceil_div(units, ceil_div(units, resident))));
+    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, false>), all, block, 0, st, x, dy, dx, ldx,
                        lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part);
+  }
 }
 
 template <typename T>
@@ -774,9 +781,6 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
         const size_t need = static_cast<size_t>(p.blocks) * 2 * n * sizeof(float);
         if (!ws || ws_bytes < need || !aligned16(ws)) return LBN_ERR_WORKSPACE;
         part = static_cast<float*>(ws);
-      }
-      else {
-        p.blocks = ceil_div(rows, p.teams);  // nothing to accumulate: one pass, all rows at once
       }
       const int nvec = static_cast<int>(n / VE);
       bool launched = false;
@@ -863,6 +867,37 @@ int lbn_layer_norm_bwd_f16(lbn_stream_t stream, int64_t num_groups, int64_t norm
                         static_cast<const __half*>(x), ldx, static_cast<const __half*>(dy), lddy,
                         static_cast<__half*>(dx), lddx, stats, ld_stats, stats_grad, ld_stats_grad,
                         scale, dscale, dbias, workspace, workspace_bytes);
+}
+
+// Instance norm is layer norm over groups of channel_size entries without scale and
+// bias (instance_norm.cpp:47-231 against layer_norm.cpp:41-258: the same statistics,
+// the same 2/n factor in backward, the same constant output for single-entry groups).
+int lbn_instance_norm_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                              int64_t width, float epsilon, const float* x, int64_t ldx, float* y,
+                              int64_t ldy, float* stats, int64_t ld_stats)
+{
+  return ln_fwd<float>(as_stream(stream), channels, channel_size, channel_size, width, epsilon, x,
+                       ldx, y, ldy, stats, ld_stats, nullptr, nullptr, LBN_STATS_TWO_PASS);
+}
+
+size_t lbn_instance_norm_bwd_workspace_bytes(int64_t channels, int64_t channel_size, int64_t width)
+{
+  if (channels <= 0 || channel_size <= 0 || width <= 0) return 0;
+  return static_cast<size_t>(2 * channels) * static_cast<size_t>(width) * sizeof(float);
+}
+
+int lbn_instance_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                              int64_t width, float epsilon, const float* x, int64_t ldx,
+                              const float* dy, int64_t lddy, float* dx, int64_t lddx,
+                              const float* stats, int64_t ld_stats, void* workspace,
+                              size_t workspace_bytes)
+{
+  if (channels > 0 && channel_size > 0 && width > 0 &&
+      (!workspace || workspace_bytes < lbn_instance_norm_bwd_workspace_bytes(channels, channel_size, width)))
+    return LBN_ERR_WORKSPACE;
+  return ln_bwd<float>(as_stream(stream), channels, channel_size, channel_size, width, epsilon, x,
+                       ldx, dy, lddy, dx, lddx, stats, ld_stats, static_cast<float*>(workspace),
+                       2 * channels, nullptr, nullptr, nullptr, nullptr, 0);
 }
 
 }  // extern "C"

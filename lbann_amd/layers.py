@@ -227,6 +227,36 @@ class layer_norm_layer(_Layer):
                  self.m_statistics_gradient.ldim, scale, dscale, dbias, ws, nb))
 
 
+class instance_norm_layer(_Layer):
+    """lbann::instance_norm_layer (include/lbann/layers/regularizers/instance_norm.hpp):
+    channels = leading output dimension, every (sample, channel) slab normalised on its own."""
+
+    def __init__(self, dims, epsilon=1e-5, device="cuda"):
+        super().__init__(device)
+        self.dims = tuple(int(d) for d in dims)
+        self.m_epsilon = float(epsilon)
+        self.num_channels = self.dims[0]
+        self.channel_size = _prod(self.dims) // self.num_channels
+        self.m_workspace = None  # (2*channels x width): means, then variances
+
+    def fp_call(self):
+        x, y = self.prev_activations, self.activations
+        if self.m_workspace is None or self.m_workspace.width != x.width:
+            self.m_workspace = DeviceMatrix(2 * self.num_channels, x.width, device=self.device)
+        return ("lbn_instance_norm_fwd_f32",
+                (_stream(), self.num_channels, self.channel_size, x.width, self.m_epsilon, x.Buffer(),
+                 x.ldim, y.Buffer(), y.ldim, self.m_workspace.Buffer(), self.m_workspace.ldim))
+
+    def bp_call(self):
+        x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
+        ws, nb = self._ws.get(capi.lib().lbn_instance_norm_bwd_workspace_bytes(
+            self.num_channels, self.channel_size, x.width), self.device)
+        return ("lbn_instance_norm_bwd_f32",
+                (_stream(), self.num_channels, self.channel_size, x.width, self.m_epsilon, x.Buffer(),
+                 x.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim, self.m_workspace.Buffer(),
+                 self.m_workspace.ldim, ws, nb))
+
+
 class batch_normalization_layer(_Layer):
     """lbann::batch_normalization_layer (include/lbann/layers/regularizers/batch_normalization.hpp:130-199),
     local statistics (statistics_group_size == 1)."""

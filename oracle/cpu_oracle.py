@@ -177,3 +177,24 @@ def channelwise_softmax_bwd(y, dy, C, cs, stride):
     getattr(lib(), f"orc_channelwise_softmax_bwd_{suf}")(
         _i64(C), _i64(cs), _i64(stride), _i64(w), *_mat(y), *_mat(dy), *_mat(dx))
     return dx
+
+
+# --------------------------------------------------------------- instance norm
+def instance_norm_fwd(x, C, cs, eps):
+    """Returns (y, sums) with sums (2C x w): rows [0,C) sum(x), [C,2C) sum(x^2) per sample."""
+    suf, cf = _suffix(x)
+    h, w = x.shape
+    y = fmat(h, w, x.dtype)
+    sums = np.zeros((2 * C, w), dtype=x.dtype, order="F")
+    getattr(lib(), f"orc_instance_norm_fwd_{suf}")(
+        _i64(C), _i64(cs), _i64(w), cf(eps), *_mat(x), *_mat(y), *_mat(sums))
+    return y, sums
+
+
+def instance_norm_bwd(x, dy, sums, C, cs, eps):
+    suf, cf = _suffix(x)
+    h, w = x.shape
+    dx = fmat(h, w, x.dtype)
+    getattr(lib(), f"orc_instance_norm_bwd_{suf}")(
+        _i64(C), _i64(cs), _i64(w), cf(eps), *_mat(x), *_mat(dy), *_mat(dx), *_mat(sums))
+    return dx

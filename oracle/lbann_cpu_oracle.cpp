@@ -25,6 +25,7 @@
 //   softmax         include/lbann/utils/dnn_lib/openmp/softmax.hpp:39-117 (fwd), :119-181 (bwd)
 //   log-softmax     src/layers/activations/log_softmax.cpp:35-93 (fwd), :95-136 (bwd)
 //   channelwise sm  src/layers/misc/channelwise_softmax.cpp:41-99 (fwd), :121-169 (bwd)
+//   instance norm   src/layers/regularizers/instance_norm.cpp:47-113 (fwd), :137-231 (bwd)
 
 #include <algorithm>
 #include <cmath>
@@ -477,6 +478,91 @@ void cws_bwd(idx C, idx cs, idx stride, idx w, CMat<T> y, CMat<T> dy, Mat<T> dx)
   }
 }
 
+// ------------------------------------------------------------ instance norm
+// instance_norm.cpp:47-113.  sums is the layer's workspace, (2C x w): rows [0,C) hold
+// sum(x), rows [C,2C) sum(x^2) of each (channel, sample).
+template <typename T>
+void in_fwd(idx C, idx cs, idx w, T eps, CMat<T> x, Mat<T> y, Mat<T> sums)
+{
+  if (cs <= 1) {  // :65-68: the output is constant
+    for (idx k = 0; k < w; ++k)
+      for (idx i = 0; i < C * cs; ++i) y(i, k) = T(0);
+    return;
+  }
+  for (idx k = 0; k < w; ++k)
+    for (idx j = 0; j < 2 * C; ++j) sums(j, k) = T(0);
+#pragma omp parallel for collapse(2)
+  for (idx k = 0; k < w; ++k) {
+    for (idx j = 0; j < C; ++j) {
+      T& sum = sums(j, k);
+      T& sqsum = sums(C + j, k);
+      for (idx i = 0; i < cs; ++i) {
+        const T v = x(i + j * cs, k);
+        sum += v;
+        sqsum += v * v;
+      }
+    }
+  }
+  const T mean_scale = T(1.) / cs;
+#pragma omp parallel for collapse(2)
+  for (idx k = 0; k < w; ++k) {
+    for (idx j = 0; j < C; ++j) {
+      const T mean = sums(j, k) * mean_scale;
+      const T sqmean = sums(C + j, k) * mean_scale;
+      T var = sqmean - mean * mean;
+      var = std::max(var, T(0.));
+      const T inv_stdev = T(1.) / std::sqrt(var + eps);
+      for (idx i = 0; i < cs; ++i) y(i + j * cs, k) = (x(i + j * cs, k) - mean) * inv_stdev;
+    }
+  }
+}
+
+// instance_norm.cpp:137-231.  The variance is recomputed from the sums WITHOUT the
+// clamp at zero of the forward pass (:186, :211), and the last factor is 2/cs (:225-226).
+template <typename T>
+void in_bwd(idx C, idx cs, idx w, T eps, CMat<T> x, CMat<T> dy, Mat<T> dx, CMat<T> sums)
+{
+  if (cs <= 1) {  // :164-167
+    for (idx k = 0; k < w; ++k)
+      for (idx i = 0; i < C * cs; ++i) dx(i, k) = T(0);
+    return;
+  }
+  std::vector<T> sgrad(static_cast<size_t>(2 * C * w), T(0));
+  const T mean_scale = T(1.) / cs;
+#pragma omp parallel for collapse(2)
+  for (idx k = 0; k < w; ++k) {
+    for (idx j = 0; j < C; ++j) {
+      const T mean = sums(j, k) * mean_scale;
+      const T sqmean = sums(C + j, k) * mean_scale;
+      const T var = sqmean - mean * mean;
+      const T inv_stdev = T(1.) / std::sqrt(var + eps);
+      T& dmean = sgrad[j + k * 2 * C];
+      T& dvar = sgrad[C + j + k * 2 * C];
+      for (idx i = 0; i < cs; ++i) {
+        const T g = dy(i + j * cs, k);
+        dmean += g;
+        dvar += g * (x(i + j * cs, k) - mean);
+      }
+      dmean *= -inv_stdev;
+      dvar *= -inv_stdev * inv_stdev * inv_stdev / 2;
+    }
+  }
+#pragma omp parallel for collapse(2)
+  for (idx k = 0; k < w; ++k) {
+    for (idx j = 0; j < C; ++j) {
+      const T mean = sums(j, k) * mean_scale;
+      const T sqmean = sums(C + j, k) * mean_scale;
+      const T var = sqmean - mean * mean;
+      const T inv_stdev = T(1.) / std::sqrt(var + eps);
+      const T dmean = sgrad[j + k * 2 * C];
+      const T dvar = sgrad[C + j + k * 2 * C];
+      for (idx i = 0; i < cs; ++i)
+        dx(i + j * cs, k) = (dy(i + j * cs, k) * inv_stdev + dmean / cs +
+                             dvar * (x(i + j * cs, k) - mean) * 2 / cs);
+    }
+  }
+}
+
 }  // namespace
 
 // C interface (one _f32 and one _f64 entry per function), bound by oracle/cpu_oracle.py.
@@ -517,7 +603,13 @@ void cws_bwd(idx C, idx cs, idx stride, idx w, CMat<T> y, CMat<T> dy, Mat<T> dx)
   { cws_fwd<T>(C, cs, stride, w, {x, ldx}, {y, ldy}); }                                  \
   extern "C" void orc_channelwise_softmax_bwd_##SUF(idx C, idx cs, idx stride, idx w,    \
       const T* y, idx ldy, const T* dy, idx lddy, T* dx, idx lddx)                       \
-  { cws_bwd<T>(C, cs, stride, w, {y, ldy}, {dy, lddy}, {dx, lddx}); }
+  { cws_bwd<T>(C, cs, stride, w, {y, ldy}, {dy, lddy}, {dx, lddx}); }                    \
+  extern "C" void orc_instance_norm_fwd_##SUF(idx C, idx cs, idx w, T eps, const T* x,   \
+      idx ldx, T* y, idx ldy, T* sums, idx lds)                                          \
+  { in_fwd<T>(C, cs, w, eps, {x, ldx}, {y, ldy}, {sums, lds}); }                         \
+  extern "C" void orc_instance_norm_bwd_##SUF(idx C, idx cs, idx w, T eps, const T* x,   \
+      idx ldx, const T* dy, idx lddy, T* dx, idx lddx, const T* sums, idx lds)           \
+  { in_bwd<T>(C, cs, w, eps, {x, ldx}, {dy, lddy}, {dx, lddx}, {sums, lds}); }
 
 ORC_INSTANTIATE(f32, float)
 ORC_INSTANTIATE(f64, double)

@@ -17,6 +17,7 @@ Datasets and tolerances (reference file:line):
   softmax               ci_test/unit_tests/test_unit_layer_softmax.py:21-24, :38-48
   log_softmax           ci_test/unit_tests/test_unit_layer_log_softmax.py:21-24, :38-48
   channelwise_softmax   ci_test/unit_tests/test_unit_layer_channelwise_softmax.py:21-26, :47-54, :109-137
+  instance_norm         ci_test/unit_tests/test_unit_layer_instance_norm.py:21-24, :38-44
 
 Run:  python tests/golden/make_reference_fixtures.py
 """
@@ -130,6 +131,18 @@ def main():
         y = e / e.sum(axis=axes, keepdims=True)
         fx[f"cws_y_{tag}"] = y.reshape(15, -1)
         fx[f"cws_metric_{tag}"] = np.float64(l2norm2_metric(y))
+
+    # ---- instance norm on (5,3,7) samples: per (sample, channel) statistics over the
+    # trailing (3,7) slab, biased variance, eps 1e-5, no affine.
+    np.random.seed(20200107)
+    x = np.random.normal(loc=0.5, size=(15, 5 * 3 * 7)).astype(np.float32)
+    xd = x.astype(np.float64).reshape(15, 5, 3, 7)
+    mean = xd.mean(axis=(2, 3), keepdims=True)
+    var = xd.var(axis=(2, 3), ddof=0, keepdims=True)
+    y = (xd - mean) / np.sqrt(var + 1e-5)
+    fx["in_x"] = x
+    fx["in_y"] = y.reshape(15, -1)
+    fx["in_metric"] = np.float64(l2norm2_metric(y))
 
     np.savez_compressed(OUT, **fx)
     print(OUT, os.path.getsize(OUT), "bytes,", len(fx), "arrays")

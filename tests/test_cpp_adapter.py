@@ -120,3 +120,16 @@ def test_adapter_layers_match_oracle():
         y = my.to_numpy()
         check(f"adapter softmax kind {kind} y", y, fwd(x), fwd(f64(x)))
         check(f"adapter softmax kind {kind} dx", mdx.to_numpy(), bwd(y, dy), bwd(f64(y), f64(dy)))
+
+    # ---- instance norm on (6, 20, 20) samples
+    dims, w = (6, 20, 20), 9
+    h = 6 * 400
+    x, dy = mk(h, w, 0.5, 2.0), mk(h, w)
+    mx, mdy, my, mdx = DeviceMatrix.from_numpy(x), DeviceMatrix.from_numpy(dy), DeviceMatrix(h, w), DeviceMatrix(h, w)
+    da, nd = _dims(dims)
+    rc = d.drv_instance_norm(da, cint(nd), dbl(1e-5), i64(h), i64(w), i64(h), mx.Buffer(), my.Buffer(),
+                             mdy.Buffer(), mdx.Buffer(), st, err, cint(512))
+    assert rc == 0, err.value
+    y_ref, sums = orc.instance_norm_fwd(x, 6, 400, 1e-5)
+    check("adapter instance norm y", my.to_numpy(), y_ref)
+    check("adapter instance norm dx", mdx.to_numpy(), orc.instance_norm_bwd(x, dy, sums, 6, 400, 1e-5))

@@ -225,6 +225,25 @@ def test_layer_norm_f16(L, dims, start_dim, w, pad):
     _ln_run(L, x, dy, dims, start_dim, True, pad, scale, bias, tol=TOL_F16, half=True)
 
 
+# ===================================================================== instance norm
+@pytest.mark.parametrize("dims,w,pad", [((5, 3, 7), 15, 0), ((64, 56, 56), 6, 0), ((8, 1024), 33, 0),
+                                        ((3, 100000), 2, 0), ((7, 1), 5, 0), ((16, 31), 40, 4),
+                                        ((256, 16, 16), 64, 0)])
+def test_instance_norm(L, dims, w, pad):
+    rng = np.random.default_rng(int(np.prod(dims)) + 7 * w)
+    h = int(np.prod(dims))
+    C, cs = dims[0], h // dims[0]
+    x, dy = rand(rng, h, w, 0.5, 2.0), rand(rng, h, w)
+    layer = L.instance_norm_layer(dims, 1e-5)
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    y32, s32 = orc.instance_norm_fwd(f32(x), C, cs, 1e-5)
+    y64, s64 = orc.instance_norm_fwd(f64(x), C, cs, 1e-5)
+    check(f"instance_norm y dims={dims}", y, y32, y64)
+    check(f"instance_norm dx dims={dims}", dx, orc.instance_norm_bwd(f32(x), f32(dy), s32, C, cs, 1e-5),
+          orc.instance_norm_bwd(f64(x), f64(dy), s64, C, cs, 1e-5))
+
+
 # ===================================================================== batch norm
 BN_CASES = [
     # dims (C, ...), width, bessel, ld_pad
@@ -369,6 +388,9 @@ def test_reference_fixtures_on_gpu(L, golden):
         y = L.channelwise_softmax_layer((5, 2, 7), **kw).forward(L.DeviceMatrix.from_numpy(T(golden["cws_x"]))).to_numpy()
         assert abs(met(y) - float(golden[f"cws_metric_{tag}"])) <= 8 * float(golden[f"cws_metric_{tag}"]) * F32_EPS
         assert rel_err(y.T, golden[f"cws_y_{tag}"]) < TOL_F32
+    y = L.instance_norm_layer((5, 3, 7)).forward(L.DeviceMatrix.from_numpy(T(golden["in_x"]))).to_numpy()
+    assert abs(met(y) - float(golden["in_metric"])) <= 8 * float(golden["in_metric"]) * F32_EPS
+    assert rel_err(y.T, golden["in_y"]) < TOL_F32
 
 
 # ===================================================================== boundary behaviour

@@ -385,3 +385,54 @@ def test_leading_dimension_and_f32_f64_agreement():
     assert np.array_equal(a, c)
     y64 = orc.softmax_fwd(packed.astype(np.float64, order="F"))
     assert rel_err(orc.softmax_fwd(packed), y64) < 1e-6
+
+
+# ============================================================== instance norm
+@pytest.mark.parametrize("dt,tol", [(np.float32, 2e-6), (np.float64, 1e-12)])
+def test_instance_norm_golden(golden, dt, tol):
+    x = F(golden["in_x"], dt)
+    y, sums = orc.instance_norm_fwd(x, 5, 21, 1e-5)
+    assert rel_err(y.T, golden["in_y"]) < tol
+    val = float(golden["in_metric"])
+    assert abs(metric(y) - val) <= 8 * val * F32_EPS   # the reference test's acceptance band
+    xd = golden["in_x"].astype(np.float64).reshape(15, 5, 21)
+    assert rel_err(sums[:5].T, xd.sum(axis=2)) < 10 * tol
+    assert rel_err(sums[5:].T, (xd * xd).sum(axis=2)) < 10 * tol
+
+
+def test_instance_norm_matches_torch_and_layer_norm():
+    rng = np.random.default_rng(21)
+    C, cs, w = 4, 9, 6
+    x = np.asfortranarray(rng.normal(0.5, 2.0, size=(C * cs, w)))
+    dy = np.asfortranarray(rng.normal(size=(C * cs, w)))
+    y, sums = orc.instance_norm_fwd(x, C, cs, 1e-5)
+    dx = orc.instance_norm_bwd(x, dy, sums, C, cs, 1e-5)
+    xt = torch.tensor(x.T.reshape(w, C, cs), requires_grad=True)
+    yt = torch.nn.functional.instance_norm(xt, eps=1e-5)
+    yt.backward(torch.tensor(dy.T.reshape(w, C, cs)))
+    assert rel_err(y.T.reshape(w, C, cs), yt.detach().numpy()) < 1e-13
+    assert rel_err(dx.T.reshape(w, C, cs), xt.grad.numpy()) < 1e-12
+    # the same numbers as layer norm over groups of cs entries, without scale and bias
+    y2, stats = orc.layer_norm_fwd(x, C, cs, cs, 1e-5)
+    dx2, _, _, _ = orc.layer_norm_bwd(x, dy, stats, C, cs, cs, 1e-5)
+    assert rel_err(y, y2) < 1e-13 and rel_err(dx, dx2) < 1e-12
+
+
+def test_instance_norm_bwd_finite_difference_and_single_entry_channels():
+    rng = np.random.default_rng(22)
+    C, cs, w = 3, 5, 2
+    x = np.asfortranarray(rng.normal(0.3, 1.5, size=(C * cs, w)))
+    dy = np.asfortranarray(rng.normal(size=(C * cs, w)))
+    eps = 1e-3
+
+    def loss():
+        return float(np.sum(orc.instance_norm_fwd(x, C, cs, eps)[0] * dy))
+
+    _, sums = orc.instance_norm_fwd(x, C, cs, eps)
+    dx = orc.instance_norm_bwd(x, dy, sums, C, cs, eps)
+    assert rel_err(dx, _fd(loss, x)) < 1e-7
+    assert np.abs(dx.reshape(cs, -1, order="F").sum(axis=0)).max() < 1e-12
+    # channels of one entry: constant output, zero gradient (instance_norm.cpp:65-68, :164-167)
+    x1 = np.asfortranarray(rng.normal(size=(7, 3)).astype(np.float32))
+    y1, s1 = orc.instance_norm_fwd(x1, 7, 1, 1e-5)
+    assert not y1.any() and not orc.instance_norm_bwd(x1, x1, s1, 7, 1, 1e-5).any()
