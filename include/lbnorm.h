@@ -46,6 +46,15 @@ typedef void* lbn_stream_t; /* a hipStream_t; NULL is the default stream */
 int lbn_version(void);
 const char* lbn_status_string(int status);
 
+/* Diagnostic, not part of any layer: the batch-norm and wide-softmax kernels in which
+ * several workgroups share a channel or a row wait for each other with a bounded
+ * number of polls; a wait that runs out raises a sticky flag in the workspace and the
+ * results of that call are then undefined.  This call waits for `stream`, copies the
+ * flag of `workspace` (the pointer that was passed to the compute call) to the host
+ * and stores it in *timed_out (0 or 1).  It is the only entry point that synchronises.
+ * It has no counterpart in the reference, whose kernels do not wait across workgroups. */
+int lbn_workspace_timed_out(lbn_stream_t stream, const void* workspace, int* timed_out);
+
 /* ------------------------------------------------------------------ layer norm
  * Replaces layer_norm_layer::fp_compute / bp_compute
  * (src/layers/regularizers/layer_norm.cpp:263-290, :292-348; math :41-136, :139-258).

@@ -19,7 +19,8 @@
 // can hold at once (cluster_capacity(), from the occupancy query), so all members
 // of a cluster are resident together and the wait always ends.  As a second line of
 // defence the wait gives up after kClusterMaxPolls polls and raises the (sticky)
-// error word in the workspace instead of spinning forever; results are then undefined
+// error word in the workspace (lbn_workspace_timed_out() reads it) instead of spinning
+// forever; results are then undefined
 // but every wave still exits.
 #pragma once
 
@@ -36,6 +37,9 @@ namespace lbn {
 constexpr int kClusterThreads = 256;  // workgroup size of the row-cluster (softmax) kernels
 constexpr int kClusterMaxM = 64;  // one wave polls and merges the partials of an item
 constexpr int kClusterMaxPolls = 1 << 21;
+// Value of the workspace's first word after a wait ran out of polls (anything else,
+// including whatever the memory held before, means that none did).
+constexpr int kClusterTimedOut = 0x7E57FA11;
 
 struct ClusterTag {
   unsigned lo, hi;
@@ -83,7 +87,7 @@ __device__ __forceinline__ void cluster_collect(unsigned long long* slots, int M
     }
     if (__all(have || lane >= M)) break;
     if (++polls > kClusterMaxPolls) {
-      if (lane == 0) __hip_atomic_store(error_word, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) __hip_atomic_store(error_word, kClusterTimedOut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       break;
     }
     __builtin_amdgcn_s_sleep(1);

@@ -441,3 +441,25 @@ def test_results_are_bitwise_reproducible(L):
                      yb, db, bn.m_scale_gradient.to_numpy()])
     for a, b in zip(*outs):
         assert np.array_equal(a, b)
+
+
+def test_rendezvous_flag_stays_clear(L):
+    """The kernels in which workgroups wait for each other (batch norm channels, softmax rows
+    shared by a cluster) leave the time-out flag of their workspace clear."""
+    import ctypes
+    from lbann_amd import capi
+    rng = np.random.default_rng(77)
+    flag = ctypes.c_int(-1)
+    stream = capi.vp(torch.cuda.current_stream().cuda_stream)
+    bn = L.batch_normalization_layer((16, 28, 28))
+    bn.forward(L.DeviceMatrix.from_numpy(rand(rng, 16 * 784, 8)))
+    bn.backward(L.DeviceMatrix.from_numpy(rand(rng, 16 * 784, 8)))
+    capi.call("lbn_workspace_timed_out", stream, capi.vp(bn._ws.buf.data_ptr()), ctypes.byref(flag))
+    assert flag.value == 0
+    sm = L.softmax_layer()
+    sm.forward(L.DeviceMatrix.from_numpy(rand(rng, 262148, 48)))   # rows shared by clusters
+    flag.value = -1
+    capi.call("lbn_workspace_timed_out", stream, capi.vp(sm._ws.buf.data_ptr()), ctypes.byref(flag))
+    assert flag.value == 0
+    capi.call("lbn_workspace_timed_out", stream, capi.vp(None), ctypes.byref(flag))
+    assert flag.value == 0
