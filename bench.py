@@ -138,6 +138,21 @@ def main():
             return t1 - t0, t2 - t1
         return layer, data["x"].size, 4, data["x"].shape[1], cpu
 
+    def build_ebn(data):
+        x, dy = upload(data["x"]), upload(data["dy"])
+        layer = L.entrywise_batch_normalization_layer(data["dims"], data["decay"], data["eps"])
+        layer.bind_forward(x)
+        layer.bind_backward(dy)
+        h = data["x"].shape[0]
+
+        def cpu():
+            from oracle import cpu_oracle as orc
+            rm, rv = np.zeros(h, np.float32), np.ones(h, np.float32)
+            t0 = time.perf_counter(); _, st = orc.entrywise_batch_norm_fwd(data["x"], data["decay"], data["eps"], rm, rv); t1 = time.perf_counter()
+            orc.entrywise_batch_norm_bwd(data["x"], data["dy"], st, data["eps"]); t2 = time.perf_counter()
+            return t1 - t0, t2 - t1
+        return layer, data["x"].size, 4, data["x"].shape[1], cpu
+
     table = {
         "cfg2_softmax": ("Softmax fwd+bwd fp32 32768x512", lambda: build_softmax("softmax", W.cfg2_softmax())),
         "cfg2_log_softmax": ("LogSoftmax fwd+bwd fp32 32768x512", lambda: build_softmax("log_softmax", W.cfg2_softmax())),
@@ -149,6 +164,8 @@ def main():
         # not a baseline configuration: the first layer beyond the five (instance norm) on cfg3's tensor
         "extra_instance_norm": ("InstanceNorm fwd+bwd fp32 NCHW 64x256x56x56 (informational)",
                                 lambda: build_in(W.cfg3_batch_norm())),
+        "extra_entrywise_batch_norm": ("EntrywiseBatchNorm train fwd+bwd fp32 1048576x64 (informational)",
+                                       lambda: build_ebn(W.extra_entrywise_batch_norm())),
         # not a baseline configuration: cfg5b's rows at 16x the width, where the multi-workgroup
         # split kernels run long enough to be measured against bandwidth rather than launch latency
         "extra_wide_softmax_w256": ("Softmax fwd+bwd fp32 262144x256 (split rows, informational)",

@@ -122,6 +122,35 @@ int lbn_instance_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t cha
                               const float* stats, int64_t ld_stats,
                               void* workspace, size_t workspace_bytes);
 
+/* ------------------------------------------------------- entry-wise batch norm
+ * Replaces entrywise_batch_normalization_layer::fp_compute / bp_compute
+ * (src/layers/regularizers/entrywise_batch_normalization.cpp:52-202, :210-414; GPU
+ * code entrywise_batch_normalization.cu).  Every entry of the sample tensor (matrix
+ * row) has its own statistics over the mini-batch (matrix columns): the variance is
+ * Bessel corrected (times n/(n-1)), there is no scale or bias.  stats and stats_grad
+ * are (height x 2): column 0 mean resp. dL/dmean, column 1 variance resp. dL/dvar
+ * (m_batch_statistics, m_batch_statistics_gradient).  training != 0: statistics from
+ * the mini-batch, running_mean / running_var (the layer's two weights, length height)
+ * updated with `decay` when width > 1; a single sample gives variance 1, y = 0 and
+ * dx = 0.  training == 0: forward normalises with the running statistics and writes
+ * neither them nor stats; backward is dx = dy / sqrt(running_var + epsilon) and reads
+ * neither x nor stats (both may be NULL).  Statistics are over the local width: with
+ * several ranks the reference sums them across the mini-batch (:97-100, :301-303),
+ * which is outside this library.  Where the reference's E[x^2] - mean^2 can come out
+ * negative, the variance here is clamped at zero. */
+int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                     float decay, float epsilon, int training,
+                                     const float* x, int64_t ldx, float* y, int64_t ldy,
+                                     float* stats, int64_t ld_stats,
+                                     float* running_mean, float* running_var);
+int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                     float epsilon, int training,
+                                     const float* x, int64_t ldx, const float* dy, int64_t lddy,
+                                     float* dx, int64_t lddx,
+                                     const float* stats, int64_t ld_stats,
+                                     float* stats_grad, int64_t ld_stats_grad,
+                                     const float* running_var);
+
 /* ------------------------------------------------------------------ batch norm
  * Replaces batch_normalization_layer::fp_compute / bp_compute
  * (src/layers/regularizers/batch_normalization.cpp:37-175, :178-329).

@@ -515,4 +515,57 @@ private:
   workspace m_ws;
 };
 
+// ---------------------------------------------------------- entry-wise batch norm
+/// include/lbann/layers/regularizers/entrywise_batch_normalization.hpp: statistics of
+/// every tensor entry over the mini-batch; weights 0/1 are the running mean/variance.
+template <typename Mat = device_matrix<float>>
+class entrywise_batch_normalization_layer {
+public:
+  entrywise_batch_normalization_layer(double decay = 0.9, double epsilon = 1e-5)
+    : m_decay(static_cast<float>(decay)), m_epsilon(static_cast<float>(epsilon)) {}
+
+  void setup(const std::vector<int64_t>& dims)
+  {
+    m_size = detail::product(dims, 0, dims.size());
+    m_batch_statistics.Resize(m_size, 2);
+    m_batch_statistics_gradient.Resize(m_size, 2);
+  }
+  /// device pointers to `size` floats each
+  void set_weights(float* running_mean, float* running_var) { m_w[0] = running_mean; m_w[1] = running_var; }
+
+  layer_io<Mat> io;
+  bool is_training = true;                             // execution_mode::training
+  device_matrix<float> m_batch_statistics;             // size x 2: mean, variance
+  device_matrix<float> m_batch_statistics_gradient;    // size x 2
+
+  void fp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    Mat& y = *io.activations;
+    if (!m_w[0] || !m_w[1]) throw exception("entrywise_batch_normalization_layer: weights are not set");
+    check_status(lbn_entrywise_batch_norm_fwd_f32(io.stream, x.Height(), x.Width(), m_decay, m_epsilon,
+                                                  is_training ? 1 : 0, x.LockedBuffer(), x.LDim(), y.Buffer(),
+                                                  y.LDim(), m_batch_statistics.Buffer(),
+                                                  m_batch_statistics.LDim(), m_w[0], m_w[1]),
+                 "entrywise_batch_normalization_layer::fp_compute");
+  }
+  void bp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    const Mat& dy = *io.prev_error_signals;
+    Mat& dx = *io.error_signals;
+    check_status(lbn_entrywise_batch_norm_bwd_f32(io.stream, x.Height(), x.Width(), m_epsilon,
+                                                  is_training ? 1 : 0, x.LockedBuffer(), x.LDim(),
+                                                  dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+                                                  m_batch_statistics.LockedBuffer(), m_batch_statistics.LDim(),
+                                                  m_batch_statistics_gradient.Buffer(),
+                                                  m_batch_statistics_gradient.LDim(), m_w[1]),
+                 "entrywise_batch_normalization_layer::bp_compute");
+  }
+private:
+  float m_decay, m_epsilon;
+  int64_t m_size = 0;
+  float* m_w[2] = {nullptr, nullptr};
+};
+
 }  // namespace lbnorm

@@ -257,6 +257,39 @@ class instance_norm_layer(_Layer):
                  self.m_workspace.ldim, ws, nb))
 
 
+class entrywise_batch_normalization_layer(_Layer):
+    """lbann::entrywise_batch_normalization_layer
+    (include/lbann/layers/regularizers/entrywise_batch_normalization.hpp): per-entry statistics
+    over the mini-batch; weights[0] running mean, weights[1] running variance."""
+
+    def __init__(self, dims, decay=0.9, epsilon=1e-5, device="cuda"):
+        super().__init__(device)
+        self.dims = tuple(int(d) for d in dims)
+        self.m_decay, self.m_epsilon = float(decay), float(epsilon)
+        h = _prod(self.dims)
+        # default weights (entrywise_batch_normalization.hpp:159-176): mean 0, variance 1
+        self.weights = [_Vector(h, device, np.zeros(h)), _Vector(h, device, np.ones(h))]
+        self.m_batch_statistics = DeviceMatrix(h, 2, device=device)
+        self.m_batch_statistics_gradient = DeviceMatrix(h, 2, device=device)
+        self.training = True
+
+    def fp_call(self):
+        x, y = self.prev_activations, self.activations
+        st = self.m_batch_statistics
+        return ("lbn_entrywise_batch_norm_fwd_f32",
+                (_stream(), x.height, x.width, self.m_decay, self.m_epsilon, int(self.training), x.Buffer(),
+                 x.ldim, y.Buffer(), y.ldim, st.Buffer(), st.ldim, self.weights[0].Buffer(),
+                 self.weights[1].Buffer()))
+
+    def bp_call(self):
+        x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
+        st, sg = self.m_batch_statistics, self.m_batch_statistics_gradient
+        return ("lbn_entrywise_batch_norm_bwd_f32",
+                (_stream(), x.height, x.width, self.m_epsilon, int(self.training), x.Buffer(), x.ldim,
+                 dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim, st.Buffer(), st.ldim, sg.Buffer(), sg.ldim,
+                 self.weights[1].Buffer()))
+
+
 class batch_normalization_layer(_Layer):
     """lbann::batch_normalization_layer (include/lbann/layers/regularizers/batch_normalization.hpp:130-199),
     local statistics (statistics_group_size == 1)."""

@@ -75,6 +75,12 @@ def cfg5b_wide_softmax(h=262144, w=16):
     return dict(x=_normal(rng, h, w), dy=_normal(rng, h, w))
 
 
+def extra_entrywise_batch_norm(h=1048576, w=64):
+    """Entry-wise batch norm fp32 (not a baseline configuration): 2^20 entries x 64 samples."""
+    rng = _rng(7)
+    return dict(x=_normal(rng, h, w, 2.0, 3.0), dy=_normal(rng, h, w), eps=1e-5, decay=0.9, dims=(h,))
+
+
 # algorithmic (compulsory) bytes: forward reads x and writes y, backward reads two
 # tensors and writes one; per-column / per-channel vectors are not counted.
 def algorithmic_bytes(elements, elem_size):

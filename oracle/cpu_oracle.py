@@ -198,3 +198,31 @@ def instance_norm_bwd(x, dy, sums, C, cs, eps):
     getattr(lib(), f"orc_instance_norm_bwd_{suf}")(
         _i64(C), _i64(cs), _i64(w), cf(eps), *_mat(x), *_mat(dy), *_mat(dx), *_mat(sums))
     return dx
+
+
+# ------------------------------------------------------- entry-wise batch norm
+def entrywise_batch_norm_fwd(x, decay, eps, running_mean, running_var, training=True):
+    """Returns (y, stats) with stats (h x 2): column 0 mean, column 1 variance (Bessel
+    corrected) of every entry over the mini-batch; running_mean/var are updated in place
+    when training and the batch has more than one sample."""
+    suf, cf = _suffix(x)
+    h, w = x.shape
+    y = fmat(h, w, x.dtype)
+    stats = np.zeros((h, 2), dtype=x.dtype, order="F")
+    assert running_mean.dtype == x.dtype and running_var.dtype == x.dtype
+    getattr(lib(), f"orc_entrywise_batch_norm_fwd_{suf}")(
+        _i64(h), _i64(w), cf(decay), cf(eps), ctypes.c_int(int(training)), *_mat(x), *_mat(y),
+        *_mat(stats), _vec(running_mean), _vec(running_var))
+    return y, stats
+
+
+def entrywise_batch_norm_bwd(x, dy, stats, eps, running_var=None, training=True):
+    """Returns (dx, stats_grad) with stats_grad (h x 2): dL/dmean, dL/dvar."""
+    suf, cf = _suffix(x)
+    h, w = x.shape
+    dx = fmat(h, w, x.dtype)
+    sgrad = np.zeros((h, 2), dtype=x.dtype, order="F")
+    getattr(lib(), f"orc_entrywise_batch_norm_bwd_{suf}")(
+        _i64(h), _i64(w), cf(eps), ctypes.c_int(int(training)), *_mat(x), *_mat(dy), *_mat(dx),
+        *_mat(stats), *_mat(sgrad), _vec(running_var))
+    return dx, sgrad

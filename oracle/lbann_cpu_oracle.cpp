@@ -26,6 +26,8 @@
 //   log-softmax     src/layers/activations/log_softmax.cpp:35-93 (fwd), :95-136 (bwd)
 //   channelwise sm  src/layers/misc/channelwise_softmax.cpp:41-99 (fwd), :121-169 (bwd)
 //   instance norm   src/layers/regularizers/instance_norm.cpp:47-113 (fwd), :137-231 (bwd)
+//   entry-wise bn   src/layers/regularizers/entrywise_batch_normalization.cpp:52-202 (fwd),
+//                   :210-414 (bwd)
 
 #include <algorithm>
 #include <cmath>
@@ -563,6 +565,114 @@ void in_bwd(idx C, idx cs, idx w, T eps, CMat<T> x, CMat<T> dy, Mat<T> dx, CMat<
   }
 }
 
+// ------------------------------------------------- entry-wise batch norm
+// entrywise_batch_normalization.cpp:52-202.  Statistics per entry (matrix row) over
+// the mini-batch (matrix columns); stats is (h x 2): column 0 mean, column 1 variance
+// (Bessel corrected, not clamped).  The reference walks the rows in blocks of one
+// cache line (:44-45); within a block the column loop is outside the row loop, which
+// fixes the order in which each row's sums are accumulated: ascending columns.
+template <typename T>
+void ebn_fwd(idx h, idx w, T decay, T eps, int training, CMat<T> x, Mat<T> y, Mat<T> stats,
+             T* rmean, T* rvar)
+{
+  const idx bsize = std::max<idx>(64 / static_cast<idx>(sizeof(float)), 1);  // DataType is float
+  const T* mean = rmean;
+  const T* var = rvar;
+  if (training) {
+    for (idx r = 0; r < h; ++r) stats(r, 0) = stats(r, 1) = T(0);
+#pragma omp parallel for
+    for (idx r0 = 0; r0 < h; r0 += bsize) {
+      const idx r1 = std::min(r0 + bsize, h);
+      for (idx c = 0; c < w; ++c)
+        for (idx r = r0; r < r1; ++r) {
+          const T v = x(r, c);
+          stats(r, 0) += v;
+          stats(r, 1) += v * v;
+        }
+    }
+    if (w <= 1) {  // :103-106: the means already hold x
+      for (idx r = 0; r < h; ++r) stats(r, 1) = T(1);
+    }
+    else {
+#pragma omp parallel for
+      for (idx r = 0; r < h; ++r) {
+        const T sum = stats(r, 0);
+        const T sqsum = stats(r, 1);
+        const T m = sum / w;
+        const T sqmean = sqsum / w;
+        const T v = (sqmean - m * m) * w / (w - 1);
+        stats(r, 0) = m;
+        stats(r, 1) = v;
+        rmean[r] = decay * rmean[r] + (T(1) - decay) * m;
+        rvar[r] = decay * rvar[r] + (T(1) - decay) * v;
+      }
+    }
+    mean = &stats(0, 0);
+    var = &stats(0, 1);
+  }
+  // apply_batchnorm, :128-157
+#pragma omp parallel for
+  for (idx r0 = 0; r0 < h; r0 += bsize) {
+    const idx r1 = std::min(r0 + bsize, h);
+    T inv_stdev[64];
+    for (idx r = r0; r < r1; ++r) inv_stdev[r - r0] = 1 / std::sqrt(var[r] + eps);
+    for (idx c = 0; c < w; ++c)
+      for (idx r = r0; r < r1; ++r) y(r, c) = (x(r, c) - mean[r]) * inv_stdev[r - r0];
+  }
+}
+
+// entrywise_batch_normalization.cpp:210-414.  sgrad is (h x 2): dL/dmean, dL/dvar
+// (written in training mode only).
+template <typename T>
+void ebn_bwd(idx h, idx w, T eps, int training, CMat<T> x, CMat<T> dy, Mat<T> dx, CMat<T> stats,
+             Mat<T> sgrad, const T* rvar)
+{
+  const idx bsize = std::max<idx>(64 / static_cast<idx>(sizeof(float)), 1);
+  if (!training) {  // :352-392
+#pragma omp parallel for
+    for (idx r0 = 0; r0 < h; r0 += bsize) {
+      const idx r1 = std::min(r0 + bsize, h);
+      T inv_stdev[64];
+      for (idx r = r0; r < r1; ++r) inv_stdev[r - r0] = 1 / std::sqrt(rvar[r] + eps);
+      for (idx c = 0; c < w; ++c)
+        for (idx r = r0; r < r1; ++r) dx(r, c) = dy(r, c) * inv_stdev[r - r0];
+    }
+    return;
+  }
+  if (w <= 1) {  // :257-261
+    for (idx c = 0; c < w; ++c)
+      for (idx r = 0; r < h; ++r) dx(r, c) = T(0);
+    return;
+  }
+  for (idx r = 0; r < h; ++r) sgrad(r, 0) = sgrad(r, 1) = T(0);
+#pragma omp parallel for
+  for (idx r0 = 0; r0 < h; r0 += bsize) {
+    const idx r1 = std::min(r0 + bsize, h);
+    T inv_stdev[64];
+    for (idx r = r0; r < r1; ++r) inv_stdev[r - r0] = 1 / std::sqrt(stats(r, 1) + eps);
+    for (idx c = 0; c < w; ++c)
+      for (idx r = r0; r < r1; ++r) {
+        const T is = inv_stdev[r - r0];
+        const T g = dy(r, c);
+        sgrad(r, 0) += -g * is;
+        sgrad(r, 1) += -g * (x(r, c) - stats(r, 0)) * is * is * is / 2;
+      }
+  }
+  const T wt = static_cast<T>(w);
+  const T inv_w = T(1) / wt;
+  const T inv_wm1 = T(1) / (wt - T(1));
+#pragma omp parallel for
+  for (idx r0 = 0; r0 < h; r0 += bsize) {
+    const idx r1 = std::min(r0 + bsize, h);
+    T inv_stdev[64];
+    for (idx r = r0; r < r1; ++r) inv_stdev[r - r0] = 1 / std::sqrt(stats(r, 1) + eps);
+    for (idx c = 0; c < w; ++c)
+      for (idx r = r0; r < r1; ++r)
+        dx(r, c) = (dy(r, c) * inv_stdev[r - r0] + sgrad(r, 0) * inv_w +
+                    sgrad(r, 1) * (x(r, c) - stats(r, 0)) * 2 * inv_wm1);
+  }
+}
+
 }  // namespace
 
 // C interface (one _f32 and one _f64 entry per function), bound by oracle/cpu_oracle.py.
@@ -609,7 +719,17 @@ void in_bwd(idx C, idx cs, idx w, T eps, CMat<T> x, CMat<T> dy, Mat<T> dx, CMat<
   { in_fwd<T>(C, cs, w, eps, {x, ldx}, {y, ldy}, {sums, lds}); }                         \
   extern "C" void orc_instance_norm_bwd_##SUF(idx C, idx cs, idx w, T eps, const T* x,   \
       idx ldx, const T* dy, idx lddy, T* dx, idx lddx, const T* sums, idx lds)           \
-  { in_bwd<T>(C, cs, w, eps, {x, ldx}, {dy, lddy}, {dx, lddx}, {sums, lds}); }
+  { in_bwd<T>(C, cs, w, eps, {x, ldx}, {dy, lddy}, {dx, lddx}, {sums, lds}); }          \
+  extern "C" void orc_entrywise_batch_norm_fwd_##SUF(idx h, idx w, T decay, T eps,       \
+      int training, const T* x, idx ldx, T* y, idx ldy, T* stats, idx lds, T* rmean,     \
+      T* rvar)                                                                           \
+  { ebn_fwd<T>(h, w, decay, eps, training, {x, ldx}, {y, ldy}, {stats, lds}, rmean,      \
+               rvar); }                                                                  \
+  extern "C" void orc_entrywise_batch_norm_bwd_##SUF(idx h, idx w, T eps, int training,  \
+      const T* x, idx ldx, const T* dy, idx lddy, T* dx, idx lddx, const T* stats,       \
+      idx lds, T* sgrad, idx ldsg, const T* rvar)                                        \
+  { ebn_bwd<T>(h, w, eps, training, {x, ldx}, {dy, lddy}, {dx, lddx}, {stats, lds},      \
+               {sgrad, ldsg}, rvar); }
 
 ORC_INSTANTIATE(f32, float)
 ORC_INSTANTIATE(f64, double)

@@ -157,6 +157,33 @@ int drv_instance_norm(const int64_t* dims, int nd, double eps, int64_t h, int64_
   }
 }
 
+int drv_entrywise_batch_norm(const int64_t* dims, int nd, double decay, double eps, int training, int64_t h,
+                             int64_t w, int64_t ld, float* x, float* y, float* dy, float* dx, float* rmean,
+                             float* rvar, float* stats_out, float* sgrad_out, void* stream, char* err,
+                             int errlen)
+{
+  try {
+    entrywise_batch_normalization_layer<> layer(decay, eps);
+    layer.setup(std::vector<int64_t>(dims, dims + nd));
+    layer.is_training = training != 0;
+    layer.set_weights(rmean, rvar);
+    device_matrix<float> mx, my, mdy, mdx;
+    attach(mx, h, w, x, ld); attach(my, h, w, y, ld); attach(mdy, h, w, dy, ld); attach(mdx, h, w, dx, ld);
+    layer.io.prev_activations = &mx; layer.io.activations = &my;
+    layer.io.prev_error_signals = &mdy; layer.io.error_signals = &mdx;
+    layer.io.stream = static_cast<hipStream_t>(stream);
+    layer.fp_compute();
+    layer.bp_compute();
+    copy_out(stats_out, layer.m_batch_statistics, layer.io.stream);
+    copy_out(sgrad_out, layer.m_batch_statistics_gradient, layer.io.stream);
+    check_hip(hipStreamSynchronize(layer.io.stream), "sync");
+    return 0;
+  }
+  catch (const std::exception& e) {
+    return fail(e, err, errlen);
+  }
+}
+
 // Host-only checks of the error behaviour the reference has: returns the number of
 // cases that did NOT throw as they should.
 int drv_error_cases(void)

@@ -18,6 +18,8 @@ Datasets and tolerances (reference file:line):
   log_softmax           ci_test/unit_tests/test_unit_layer_log_softmax.py:21-24, :38-48
   channelwise_softmax   ci_test/unit_tests/test_unit_layer_channelwise_softmax.py:21-26, :47-54, :109-137
   instance_norm         ci_test/unit_tests/test_unit_layer_instance_norm.py:21-24, :38-44
+  entrywise_batch_norm  ci_test/unit_tests/test_unit_layer_entrywise_batch_normalization.py:21-25
+                        (no forward pin there: gradient check only)
 
 Run:  python tests/golden/make_reference_fixtures.py
 """
@@ -143,6 +145,21 @@ def main():
     fx["in_x"] = x
     fx["in_y"] = y.reshape(15, -1)
     fx["in_metric"] = np.float64(l2norm2_metric(y))
+
+    # ---- entry-wise batch norm dataset (the reference pins only gradients on it); the
+    # stored expectation is the training-mode definition in float64: per-entry mean and
+    # Bessel-corrected variance over the mini-batch (the first 14 samples, as the test's
+    # mini-batch size is num_samples // 2, and all 29), eps 1e-5, no scale or bias.
+    np.random.seed(20190815)
+    x = np.random.normal(size=(29, 7 * 5 * 3)).astype(np.float32)
+    fx["ebn_x"] = x
+    for tag, batch in (("mb14", x[:14]), ("all29", x)):
+        xd = batch.astype(np.float64)
+        mean = xd.mean(axis=0)
+        var = xd.var(axis=0, ddof=1)
+        fx[f"ebn_{tag}_mean"] = mean
+        fx[f"ebn_{tag}_var"] = var
+        fx[f"ebn_{tag}_y"] = (xd - mean) / np.sqrt(var + 1e-5)
 
     np.savez_compressed(OUT, **fx)
     print(OUT, os.path.getsize(OUT), "bytes,", len(fx), "arrays")

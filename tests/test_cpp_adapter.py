@@ -133,3 +133,25 @@ def test_adapter_layers_match_oracle():
     y_ref, sums = orc.instance_norm_fwd(x, 6, 400, 1e-5)
     check("adapter instance norm y", my.to_numpy(), y_ref)
     check("adapter instance norm dx", mdx.to_numpy(), orc.instance_norm_bwd(x, dy, sums, 6, 400, 1e-5))
+
+    # ---- entry-wise batch norm on (4, 40) samples, 12 per mini-batch
+    dims, w = (4, 40), 12
+    h = 160
+    x, dy = mk(h, w, 0.5, 2.0), mk(h, w)
+    mx, mdy, my, mdx = DeviceMatrix.from_numpy(x), DeviceMatrix.from_numpy(dy), DeviceMatrix(h, w), DeviceMatrix(h, w)
+    rm, rv = torch.zeros(h).cuda(), torch.ones(h).cuda()
+    stats, sgrad = DeviceMatrix(h, 2), DeviceMatrix(h, 2)
+    da, nd = _dims(dims)
+    rc = d.drv_entrywise_batch_norm(da, cint(nd), dbl(0.9), dbl(1e-5), cint(1), i64(h), i64(w), i64(h), mx.Buffer(),
+                                    my.Buffer(), mdy.Buffer(), mdx.Buffer(), p(rm), p(rv), stats.Buffer(),
+                                    sgrad.Buffer(), st, err, cint(512))
+    assert rc == 0, err.value
+    rm0, rv0 = np.zeros(h, np.float32), np.ones(h, np.float32)
+    y_ref, st_ref = orc.entrywise_batch_norm_fwd(x, 0.9, 1e-5, rm0, rv0)
+    dx_ref, sg_ref = orc.entrywise_batch_norm_bwd(x, dy, st_ref, 1e-5)
+    check("adapter entrywise bn y", my.to_numpy(), y_ref)
+    check("adapter entrywise bn dx", mdx.to_numpy(), dx_ref)
+    check("adapter entrywise bn stats", stats.to_numpy(), st_ref)
+    check("adapter entrywise bn stats grad", sgrad.to_numpy(), sg_ref)
+    check("adapter entrywise bn running mean", rm.cpu().numpy(), rm0)
+    check("adapter entrywise bn running var", rv.cpu().numpy(), rv0)

@@ -244,6 +244,38 @@ def test_instance_norm(L, dims, w, pad):
           orc.instance_norm_bwd(f64(x), f64(dy), s64, C, cs, 1e-5))
 
 
+# ===================================================================== entry-wise batch norm
+@pytest.mark.parametrize("h,w,pad", [(105, 14, 0), (105, 29, 0), (4096, 64, 0), (4096, 256, 0), (1024, 300, 0),
+                                     (200000, 16, 0), (64, 1, 0), (260, 7, 4), (258, 9, 0), (100000, 33, 0)])
+def test_entrywise_batch_norm(L, h, w, pad):
+    rng = np.random.default_rng(h + 3 * w)
+    x, dy = rand(rng, h, w, 0.5, 2.0), rand(rng, h, w)
+    rm0 = rng.normal(size=h).astype(np.float32)
+    rv0 = rng.uniform(0.5, 2.0, size=h).astype(np.float32)
+
+    def oracle(conv, training):
+        rm, rv = conv(rm0).copy(), conv(rv0).copy()
+        y, st = orc.entrywise_batch_norm_fwd(conv(x), 0.9, 1e-5, rm, rv, training)
+        dx, sg = orc.entrywise_batch_norm_bwd(conv(x), conv(dy), st, 1e-5, rv, training)
+        return dict(y=y, stats=st, dx=dx, sgrad=sg, rmean=rm, rvar=rv)
+
+    for training in (True, False):
+        layer = L.entrywise_batch_normalization_layer((h,), 0.9, 1e-5)
+        layer.weights[0].tensor.copy_(torch.from_numpy(rm0))
+        layer.weights[1].tensor.copy_(torch.from_numpy(rv0))
+        layer.training = training
+        y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+        dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+        got = dict(y=y, dx=dx, rmean=layer.weights[0].to_numpy(), rvar=layer.weights[1].to_numpy())
+        if training:
+            got["stats"] = layer.m_batch_statistics.to_numpy()
+            if w > 1:
+                got["sgrad"] = layer.m_batch_statistics_gradient.to_numpy()
+        r32, r64 = oracle(f32, training), oracle(f64, training)
+        for k in got:
+            check(f"entrywise_bn {k} h={h} w={w} training={training}", got[k], r32[k], r64[k])
+
+
 # ===================================================================== batch norm
 BN_CASES = [
     # dims (C, ...), width, bessel, ld_pad
@@ -388,6 +420,13 @@ def test_reference_fixtures_on_gpu(L, golden):
         y = L.channelwise_softmax_layer((5, 2, 7), **kw).forward(L.DeviceMatrix.from_numpy(T(golden["cws_x"]))).to_numpy()
         assert abs(met(y) - float(golden[f"cws_metric_{tag}"])) <= 8 * float(golden[f"cws_metric_{tag}"]) * F32_EPS
         assert rel_err(y.T, golden[f"cws_y_{tag}"]) < TOL_F32
+    for tag, rows in (("mb14", 14), ("all29", 29)):
+        eb = L.entrywise_batch_normalization_layer((7, 5, 3))
+        y = eb.forward(L.DeviceMatrix.from_numpy(T(golden["ebn_x"][:rows]))).to_numpy()
+        assert rel_err(y.T, golden[f"ebn_{tag}_y"]) < TOL_F32
+        st = eb.m_batch_statistics.to_numpy()
+        assert rel_err(st[:, 0], golden[f"ebn_{tag}_mean"]) < TOL_F32
+        assert rel_err(st[:, 1], golden[f"ebn_{tag}_var"]) < TOL_F32
     y = L.instance_norm_layer((5, 3, 7)).forward(L.DeviceMatrix.from_numpy(T(golden["in_x"]))).to_numpy()
     assert abs(met(y) - float(golden["in_metric"])) <= 8 * float(golden["in_metric"]) * F32_EPS
     assert rel_err(y.T, golden["in_y"]) < TOL_F32

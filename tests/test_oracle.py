@@ -436,3 +436,73 @@ def test_instance_norm_bwd_finite_difference_and_single_entry_channels():
     x1 = np.asfortranarray(rng.normal(size=(7, 3)).astype(np.float32))
     y1, s1 = orc.instance_norm_fwd(x1, 7, 1, 1e-5)
     assert not y1.any() and not orc.instance_norm_bwd(x1, x1, s1, 7, 1, 1e-5).any()
+
+
+# ====================================================== entry-wise batch norm
+@pytest.mark.parametrize("tag,rows", [("mb14", 14), ("all29", 29)])
+def test_entrywise_batch_norm_golden(golden, tag, rows):
+    for dt, tol in ((np.float32, 3e-6), (np.float64, 1e-12)):
+        x = F(golden["ebn_x"][:rows], dt)
+        rm, rv = np.zeros(105, dt), np.ones(105, dt)
+        y, stats = orc.entrywise_batch_norm_fwd(x, 0.9, 1e-5, rm, rv)
+        assert rel_err(y.T, golden[f"ebn_{tag}_y"]) < tol
+        assert rel_err(stats[:, 0], golden[f"ebn_{tag}_mean"]) < tol
+        assert rel_err(stats[:, 1], golden[f"ebn_{tag}_var"]) < 10 * tol
+        # running statistics: exponential moving average from (0, 1) with decay 0.9
+        assert rel_err(rm, 0.1 * golden[f"ebn_{tag}_mean"]) < 10 * tol
+        assert rel_err(rv, 0.9 + 0.1 * golden[f"ebn_{tag}_var"]) < 10 * tol
+
+
+def test_entrywise_batch_norm_matches_torch_autograd_and_inference():
+    rng = np.random.default_rng(31)
+    h, w = 23, 11
+    x = np.asfortranarray(rng.normal(0.5, 2.0, size=(h, w)))
+    dy = np.asfortranarray(rng.normal(size=(h, w)))
+    rm, rv = rng.normal(size=h), rng.uniform(0.5, 2.0, size=h)
+    rm0, rv0 = rm.copy(), rv.copy()
+    y, stats = orc.entrywise_batch_norm_fwd(x, 0.8, 1e-4, rm, rv)
+    xt = torch.tensor(x.T, requires_grad=True)
+    yt = (xt - xt.mean(0)) / torch.sqrt(xt.var(0, unbiased=True) + 1e-4)
+    yt.backward(torch.tensor(dy.T))
+    dx, _ = orc.entrywise_batch_norm_bwd(x, dy, stats, 1e-4)
+    assert rel_err(y.T, yt.detach().numpy()) < 1e-13 and rel_err(dx.T, xt.grad.numpy()) < 1e-12
+    assert rel_err(rm, 0.8 * rm0 + 0.2 * x.mean(1)) < 1e-13
+    assert rel_err(rv, 0.8 * rv0 + 0.2 * x.var(1, ddof=1)) < 1e-13
+    # inference: running statistics in, nothing updated, gradient is dy / stdev
+    rm1, rv1 = rm.copy(), rv.copy()
+    yi, _ = orc.entrywise_batch_norm_fwd(x, 0.8, 1e-4, rm1, rv1, training=False)
+    assert rel_err(yi, (x - rm[:, None]) / np.sqrt(rv[:, None] + 1e-4)) < 1e-13
+    assert np.array_equal(rm1, rm) and np.array_equal(rv1, rv)
+    dxi, _ = orc.entrywise_batch_norm_bwd(x, dy, stats, 1e-4, rv, training=False)
+    assert rel_err(dxi, dy / np.sqrt(rv[:, None] + 1e-4)) < 1e-13
+
+
+def test_entrywise_batch_norm_bwd_finite_difference_and_single_sample():
+    rng = np.random.default_rng(32)
+    h, w = 4, 5
+    x = np.asfortranarray(rng.normal(0.3, 1.5, size=(h, w)))
+    dy = np.asfortranarray(rng.normal(size=(h, w)))
+    eps = 1e-3
+
+    def loss():
+        return float(np.sum(orc.entrywise_batch_norm_fwd(x, 0.9, eps, np.zeros(h), np.ones(h))[0] * dy))
+
+    _, stats = orc.entrywise_batch_norm_fwd(x, 0.9, eps, np.zeros(h), np.ones(h))
+    dx, sgrad = orc.entrywise_batch_norm_bwd(x, dy, stats, eps)
+    assert rel_err(dx, _fd(loss, x)) < 1e-7
+    assert np.abs(dx.sum(axis=1)).max() < 1e-12          # every entry's gradient sums to zero over the batch
+    mean, var = stats[:, 0].copy(), stats[:, 1].copy()
+
+    def loss_mv():
+        return float(np.sum((x - mean[:, None]) / np.sqrt(var[:, None] + eps) * dy))
+
+    assert rel_err(sgrad[:, 0], _fd(loss_mv, mean)) < 1e-7
+    assert rel_err(sgrad[:, 1], _fd(loss_mv, var, h=1e-6)) < 1e-6
+    # one sample: variance 1, running statistics untouched, zero gradient
+    # (entrywise_batch_normalization.cpp:103-106, :257-261)
+    x1 = np.asfortranarray(rng.normal(size=(6, 1)).astype(np.float32))
+    rm, rv = np.full(6, 0.25, np.float32), np.full(6, 2.0, np.float32)
+    y1, s1 = orc.entrywise_batch_norm_fwd(x1, 0.9, 1e-5, rm, rv)
+    assert not y1.any() and np.array_equal(s1[:, 0], x1[:, 0]) and (s1[:, 1] == 1).all()
+    assert (rm == 0.25).all() and (rv == 2.0).all()
+    assert not orc.entrywise_batch_norm_bwd(x1, x1, s1, 1e-5)[0].any()
