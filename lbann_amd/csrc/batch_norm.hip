@@ -656,9 +656,18 @@ struct BnClusterShape {
   int T, V, M;
 };
 
+// Larger workgroups pay the per-step costs (two barriers, one rendezvous) over more
+// bytes: 512 threads are taken when that still splits a channel over at least 8
+// workgroups (1024 measured the same), otherwise the smallest size that fits.
 static BnClusterShape bn_cluster_shape(int64_t E, int max_v, int first_t)
 {
   static const int force_t = std::getenv("LBN_BN_CLUSTER_T") ? std::atoi(std::getenv("LBN_BN_CLUSTER_T")) : 0;
+  if (!force_t) {
+    for (int T = 512; T >= first_t; T /= 2) {
+      const ClusterPlan p = plan_cluster(E, max_v, T);
+      if (p.M >= 8) return {T, p.V, p.M};
+    }
+  }
   for (int T = force_t ? force_t : first_t; T <= 1024; T *= 2) {
     const ClusterPlan p = plan_cluster(E, max_v, T);
     if (p.M) return {T, p.V, p.M};
