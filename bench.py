@@ -31,6 +31,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", default="all", help="all | headline | comma list of cfg names")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cold", action="store_true", help="skip the cold-cache leg of the small working sets")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also time a plain elementwise copy of 256 MiB (torch kernel): the practical "
                          "streaming ceiling, and the known-size kernel that scales the rocprof byte counters")
@@ -275,7 +276,7 @@ def main():
             "fwd_gbs": fwd_b / (f_ms * 1e-3) / 1e9, "bwd_gbs": bwd_b / (b_ms * 1e-3) / 1e9,
             "bwd_back_to_back_ms": bwd_b2b,
         }
-        if 4 * elems * esize <= (256 << 20):
+        if not args.no_cold and 4 * elems * esize <= (256 << 20):
             # small working set: a second, cold figure next to the cache-resident one
             cwall, copies = measure_cold(builder, 4 * elems * esize, args.steps, args.warmup)
             cms = cwall / args.steps * 1e3
