@@ -52,3 +52,14 @@ def test_host_mirror_dimension_logic():
     assert cw.get_channel_size_and_stride() == (7, 7, 10)
     cw.dims, cw.m_dim, cw.m_single_dim_mode = (64, 4096), 0, False
     assert cw.get_channel_size_and_stride() == (4096, 4096, 64)
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/lbnorm.h compiles as C99 and as C++17 on its own (no HIP, no torch types)."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "lbnorm.h"\nint (*entry)(void) = lbn_version;\nint main(void) { return entry ? LBN_OK : LBN_ERR_UNSUPPORTED; }\n')
+    inc = os.path.join(root, "include")
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", f"-I{inc}", str(src)], check=True)
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", f"-I{inc}", str(src)], check=True)
