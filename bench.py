@@ -273,6 +273,7 @@ def main():
             "samples_per_s": samples / (step_ms * 1e-3),
             "fwd_ms": f_ms, "bwd_ms": b_ms,
             "fwd_ms_min": min(fwd), "bwd_ms_min": min(bwd),
+            "fwd_ms_median": statistics.median(fwd), "bwd_ms_median": statistics.median(bwd),
             "fwd_gbs": fwd_b / (f_ms * 1e-3) / 1e9, "bwd_gbs": bwd_b / (b_ms * 1e-3) / 1e9,
             "bwd_back_to_back_ms": bwd_b2b,
         }

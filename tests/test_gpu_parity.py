@@ -502,3 +502,37 @@ def test_rendezvous_flag_stays_clear(L):
     assert flag.value == 0
     capi.call("lbn_workspace_timed_out", stream, capi.vp(None), ctypes.byref(flag))
     assert flag.value == 0
+
+
+def test_concurrent_host_threads_on_separate_streams(L):
+    """Two host threads drive different layers on their own streams at the same time (the
+    entry points are re-entrant: per-call tags, a locked occupancy cache, caller-owned
+    scratch); each result equals the one the same call gives on its own."""
+    import threading
+    rng = np.random.default_rng(91)
+    xs, xb = rand(rng, 262148, 48), rand(rng, 16 * 784, 32, 2.0, 3.0)   # row clusters / channel clusters
+    xl = rand(rng, 4096, 300)
+
+    def run_softmax(out):
+        s = torch.cuda.Stream()
+        with torch.cuda.stream(s):
+            out.append([L.softmax_layer().forward(L.DeviceMatrix.from_numpy(xs)).to_numpy() for _ in range(4)])
+
+    def run_norms(out):
+        s = torch.cuda.Stream()
+        with torch.cuda.stream(s):
+            r = []
+            for _ in range(4):
+                r.append(L.batch_normalization_layer((16, 28, 28)).forward(L.DeviceMatrix.from_numpy(xb)).to_numpy())
+                r.append(L.layer_norm_layer((4096,)).forward(L.DeviceMatrix.from_numpy(xl)).to_numpy())
+            out.append(r)
+
+    alone_a, alone_b = [], []
+    run_softmax(alone_a)
+    run_norms(alone_b)
+    got_a, got_b = [], []
+    ta, tb = threading.Thread(target=run_softmax, args=(got_a,)), threading.Thread(target=run_norms, args=(got_b,))
+    ta.start(); tb.start(); ta.join(); tb.join()
+    torch.cuda.synchronize()
+    for a, b in zip(alone_a[0] + alone_b[0], got_a[0] + got_b[0]):
+        assert np.array_equal(a, b)
