@@ -160,3 +160,57 @@ def test_cfg5b_wide_softmax_262144x16(L, W):
     xm = L.DeviceMatrix.from_numpy(x)
     layer.forward(xm, in_place=True)
     assert np.array_equal(xm.to_numpy(), y)
+
+
+# ------------------------------------------------------------------ beyond the five configurations
+def test_extra_instance_norm_on_the_cfg3_tensor(L, W):
+    d = W.cfg3_batch_norm()
+    x, dy = f32(d["x"]), f32(d["dy"])
+    C, cs = 256, 3136
+    layer = L.instance_norm_layer(d["dims"], d["eps"])
+    y = layer.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+    y32, s32 = orc.instance_norm_fwd(x, C, cs, d["eps"])
+    check("instance norm y", y, y32)
+    # the fp32 reference sums 3136 entries of mean 2 sequentially: float64 decides ties
+    x64, dy64 = f64(x), f64(dy)
+    y64, s64 = orc.instance_norm_fwd(x64, C, cs, d["eps"])
+    check("instance norm dx", dx, orc.instance_norm_bwd(x, dy, s32, C, cs, d["eps"]),
+          orc.instance_norm_bwd(x64, dy64, s64, C, cs, d["eps"]))
+    # every (sample, channel) slab: zero mean output, zero-sum gradient
+    assert np.abs(y.reshape(cs, -1, order="F").astype(np.float64).mean(axis=0)).max() < 1e-5
+    assert np.abs(dx.reshape(cs, -1, order="F").astype(np.float64).sum(axis=0)).max() < 2e-2
+
+
+def test_extra_entrywise_batch_norm_262144x64(L, W):
+    d = W.extra_entrywise_batch_norm(h=262144)
+    x, dy = f32(d["x"]), f32(d["dy"])
+    h = x.shape[0]
+    layer = L.entrywise_batch_normalization_layer(d["dims"], d["decay"], d["eps"])
+    y = layer.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+    rm, rv = np.zeros(h, np.float32), np.ones(h, np.float32)
+    y32, st32 = orc.entrywise_batch_norm_fwd(x, d["decay"], d["eps"], rm, rv)
+    rm64, rv64 = np.zeros(h), np.ones(h)
+    y64, st64 = orc.entrywise_batch_norm_fwd(f64(x), d["decay"], d["eps"], rm64, rv64)
+    check("entrywise bn y", y, y32, y64)
+    check("entrywise bn stats", layer.m_batch_statistics.to_numpy(), st32, st64)
+    check("entrywise bn running mean", layer.weights[0].to_numpy(), rm, rm64)
+    check("entrywise bn running var", layer.weights[1].to_numpy(), rv, rv64)
+    dx32, sg32 = orc.entrywise_batch_norm_bwd(x, dy, st32, d["eps"])
+    dx64, sg64 = orc.entrywise_batch_norm_bwd(f64(x), f64(dy), st64, d["eps"])
+    check("entrywise bn dx", dx, dx32, dx64)
+    check("entrywise bn stats grad", layer.m_batch_statistics_gradient.to_numpy(), sg32, sg64)
+    assert np.abs(dx.astype(np.float64).sum(axis=1)).max() < 1e-3   # per entry, over the batch
+
+
+def test_extra_wide_softmax_row_clusters_262144x64(L, W):
+    d = W.cfg5b_wide_softmax(w=64)   # 64 MiB per tensor: rows shared by clusters of workgroups
+    x, dy = f32(d["x"]), f32(d["dy"])
+    sm = L.softmax_layer()
+    y = sm.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    dx = sm.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+    y64 = orc.softmax_fwd(f64(x))
+    check("wide softmax y", y, orc.softmax_fwd(x), y64)
+    check("wide softmax dx", dx, orc.softmax_bwd(y, dy), orc.softmax_bwd(f64(y), f64(dy)))
+    assert np.abs(y.astype(np.float64).sum(axis=0) - 1).max() < 1e-5
