@@ -1,0 +1,154 @@
+"""Seeded sweep over small random shapes, leading dimensions and layer options: every
+layer, GPU through the C ABI against the CPU oracle.  The shapes are drawn so that the
+vector kernels, their masked variants and the scalar fallbacks are all hit (lengths that
+are and are not multiples of 4 or 8, padded leading dimensions, single rows and columns)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu_oracle as orc
+from tests.parity import TOL_F16, TOL_F32, check
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def L():
+    from lbann_amd import layers
+    layers.capi.lib()
+    assert torch.cuda.is_available()
+    return layers
+
+
+def f64(a):
+    return np.asfortranarray(np.asarray(a, dtype=np.float64))
+
+
+def f32(a):
+    return np.asfortranarray(np.asarray(a, dtype=np.float32))
+
+
+def rand(rng, h, w, mean=0.0, std=1.0):
+    return np.asfortranarray((rng.standard_normal((w, h)) * std + mean).astype(np.float32).T)
+
+
+def draw_length(rng):
+    """Mostly vector-friendly lengths, some odd ones, a few long ones."""
+    kind = rng.integers(0, 10)
+    if kind < 5:
+        return int(rng.integers(1, 400)) * 8
+    if kind < 8:
+        return int(rng.integers(1, 3000))
+    return int(rng.integers(3000, 40000))
+
+
+CASES = list(range(24))
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_softmax_family_random(L, case):
+    rng = np.random.default_rng(1000 + case)
+    n, w = draw_length(rng), int(rng.integers(1, 40))
+    pad = int(rng.choice([0, 0, 4, 3]))
+    x, dy = rand(rng, n, w, 0.0, 2.5), rand(rng, n, w)
+    for kind, layer, fwd, bwd in (("softmax", L.softmax_layer(), orc.softmax_fwd, orc.softmax_bwd),
+                                  ("log_softmax", L.log_softmax_layer(), orc.log_softmax_fwd, orc.log_softmax_bwd)):
+        y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=n + pad)).to_numpy()
+        dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=n + pad)).to_numpy()
+        check(f"{kind} y n={n} w={w} pad={pad}", y, fwd(x), fwd(f64(x)))
+        check(f"{kind} dx n={n} w={w} pad={pad}", dx, bwd(y, dy), bwd(f64(y), f64(dy)))
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_channelwise_softmax_and_instance_norm_random(L, case):
+    rng = np.random.default_rng(2000 + case)
+    C, cs, w = int(rng.integers(1, 12)), min(draw_length(rng), 6000), int(rng.integers(1, 12))
+    h = C * cs
+    pad = int(rng.choice([0, 0, 4, 1]))
+    x, dy = rand(rng, h, w, 0.3, 1.5), rand(rng, h, w)
+    cw = L.channelwise_softmax_layer((C, cs))
+    y = cw.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    dx = cw.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    check(f"channelwise y C={C} cs={cs} w={w}", y, orc.channelwise_softmax_fwd(x, C, cs, cs),
+          orc.channelwise_softmax_fwd(f64(x), C, cs, cs))
+    check(f"channelwise dx C={C} cs={cs} w={w}", dx, orc.channelwise_softmax_bwd(y, dy, C, cs, cs),
+          orc.channelwise_softmax_bwd(f64(y), f64(dy), C, cs, cs))
+    inl = L.instance_norm_layer((C, cs), 1e-5)
+    y = inl.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    dx = inl.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    y32, s32 = orc.instance_norm_fwd(x, C, cs, 1e-5)
+    y64, s64 = orc.instance_norm_fwd(f64(x), C, cs, 1e-5)
+    check(f"instance norm y C={C} cs={cs} w={w}", y, y32, y64)
+    check(f"instance norm dx C={C} cs={cs} w={w}", dx, orc.instance_norm_bwd(x, dy, s32, C, cs, 1e-5),
+          orc.instance_norm_bwd(f64(x), f64(dy), s64, C, cs, 1e-5))
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_layer_norm_random(L, case):
+    rng = np.random.default_rng(3000 + case)
+    G, n, w = int(rng.choice([1, 1, 2, 5])), min(draw_length(rng), 20000), int(rng.integers(1, 30))
+    half = bool(case % 3 == 2)
+    affine = bool(case % 2)
+    h = G * n
+    pad = int(rng.choice([0, 0, 8, 2]))
+    x, dy = rand(rng, h, w, 0.3, 1.5), rand(rng, h, w)
+    if half:
+        x, dy = x.astype(np.float16).astype(np.float32), dy.astype(np.float16).astype(np.float32)
+    g = (1 + 0.2 * rng.standard_normal(n)).astype(np.float32) if affine else None
+    b = (0.2 * rng.standard_normal(n)).astype(np.float32) if affine else None
+    kw = dict(scale_values=g, bias_values=b) if affine else {}
+    dims, sd = ((G, n), 1) if G > 1 else ((n,), 0)
+    layer = L.layer_norm_layer(dims, 1e-5, affine, affine, sd, **kw)
+    tdt = torch.float16 if half else torch.float32
+    tol = TOL_F16 if half else TOL_F32
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, dtype=tdt, ldim=h + pad)).to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, dtype=tdt, ldim=h + pad)).to_numpy()
+    ref, ex = {}, {}
+    for dst, conv in ((ref, f32), (ex, f64)):
+        gg = None if g is None else conv(g)
+        bb = None if b is None else conv(b)
+        dst["y"], st = orc.layer_norm_fwd(conv(x), G, n, n, 1e-5, gg, bb)
+        dst["dx"], _, dst["dscale"], dst["dbias"] = orc.layer_norm_bwd(conv(x), conv(dy), st, G, n, n, 1e-5, gg,
+                                                                         affine, affine)
+    tag = f"G={G} n={n} w={w} half={half} affine={affine} pad={pad}"
+    check("layer norm y " + tag, y, ref["y"], ex["y"], tol=tol)
+    if n > 1:
+        check("layer norm dx " + tag, dx, ref["dx"], ex["dx"], tol=tol)
+    if affine:
+        check("layer norm dscale " + tag, layer.m_scale_gradient.to_numpy(), ref["dscale"], ex["dscale"], tol=tol)
+        check("layer norm dbias " + tag, layer.m_bias_gradient.to_numpy(), ref["dbias"], ex["dbias"], tol=tol)
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_batch_norms_random(L, case):
+    rng = np.random.default_rng(4000 + case)
+    C, cs, w = int(rng.integers(1, 20)), min(draw_length(rng), 5000), int(rng.integers(2, 24))
+    h = C * cs
+    pad = int(rng.choice([0, 0, 4, 1]))
+    bessel = bool(case % 2)
+    x, dy = rand(rng, h, w, 2.0, 3.0), rand(rng, h, w)
+    g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    b = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    bn = L.batch_normalization_layer((C, cs), 0.9, 1e-5, bessel, g, b)
+    y = bn.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    dx = bn.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    ref, ex = {}, {}
+    for dst, conv in ((ref, f32), (ex, f64)):
+        rm, rv = conv(np.zeros(C)), conv(np.ones(C))
+        dst["y"], m, v = orc.batch_norm_fwd(conv(x), C, cs, 1e-5, 0.9, conv(g), conv(b), rm, rv, bessel)
+        dst["dx"], dst["dscale"], dst["dbias"], _, _ = orc.batch_norm_bwd(conv(x), conv(dy), C, cs, 1e-5, m, v,
+                                                                         conv(g), bessel=bessel)
+    tag = f"C={C} cs={cs} w={w} bessel={bessel} pad={pad}"
+    check("batch norm y " + tag, y, ref["y"], ex["y"])
+    check("batch norm dx " + tag, dx, ref["dx"], ex["dx"])
+    check("batch norm dscale " + tag, bn.m_scale_gradient.to_numpy(), ref["dscale"], ex["dscale"])
+    check("batch norm dbias " + tag, bn.m_bias_gradient.to_numpy(), ref["dbias"], ex["dbias"])
+    # entry-wise batch norm on the same data
+    eb = L.entrywise_batch_normalization_layer((h,), 0.9, 1e-5)
+    y = eb.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    dx = eb.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    y32, st32 = orc.entrywise_batch_norm_fwd(x, 0.9, 1e-5, np.zeros(h, np.float32), np.ones(h, np.float32))
+    y64, st64 = orc.entrywise_batch_norm_fwd(f64(x), 0.9, 1e-5, np.zeros(h), np.ones(h))
+    check("entrywise bn y " + tag, y, y32, y64)
+    check("entrywise bn dx " + tag, dx, orc.entrywise_batch_norm_bwd(x, dy, st32, 1e-5)[0],
+          orc.entrywise_batch_norm_bwd(f64(x), f64(dy), st64, 1e-5)[0])
