@@ -162,7 +162,10 @@ int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_
  * the running statistics with `decay`; training == 0 normalises with the running
  * statistics and leaves mean/var untouched.  bessel != 0 scales the variance by
  * n/(n-1) (the reference default).  The variance is clamped below at epsilon and
- * epsilon is added again under the square root, as the reference does. */
+ * epsilon is added again under the square root, as the reference does.  The _f16
+ * variants store x, y, dy, dx as IEEE binary16 and compute in fp32, with statistics,
+ * weights and their gradients in fp32 (the accumulation type the reference's GPU code
+ * uses for half data, BNAcc, batch_normalization.hpp:60-71). */
 size_t lbn_batch_norm_workspace_bytes(int64_t channels, int64_t channel_size, int64_t width);
 int lbn_batch_norm_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
                            int64_t width, int bessel, float epsilon, float decay,
@@ -174,6 +177,20 @@ int lbn_batch_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t channe
                            int64_t width, int bessel, float epsilon, int training,
                            const float* x, int64_t ldx, const float* dy, int64_t lddy,
                            float* dx, int64_t lddx, const float* mean, const float* var,
+                           const float* running_mean, const float* running_var,
+                           const float* scale, float* dscale, float* dbias,
+                           float* dmean, float* dvar,
+                           void* workspace, size_t workspace_bytes);
+int lbn_batch_norm_fwd_f16(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                           int64_t width, int bessel, float epsilon, float decay,
+                           int training, const void* x, int64_t ldx, void* y, int64_t ldy,
+                           float* mean, float* var, const float* scale, const float* bias,
+                           float* running_mean, float* running_var,
+                           void* workspace, size_t workspace_bytes, int flags);
+int lbn_batch_norm_bwd_f16(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                           int64_t width, int bessel, float epsilon, int training,
+                           const void* x, int64_t ldx, const void* dy, int64_t lddy,
+                           void* dx, int64_t lddx, const float* mean, const float* var,
                            const float* running_mean, const float* running_var,
                            const float* scale, float* dscale, float* dbias,
                            float* dmean, float* dvar,

@@ -252,9 +252,12 @@ private:
 
 // ------------------------------------------------------------------ batch norm
 /// include/lbann/layers/regularizers/batch_normalization.hpp:130-199 with local
-/// statistics (statistics_group_size == 1).
-template <typename Mat = device_matrix<float>>
+/// statistics (statistics_group_size == 1).  T is the storage type of the activations
+/// and error signals: float, or a 2-byte type holding IEEE binary16; statistics and
+/// weights are float either way.
+template <typename T = float, typename Mat = device_matrix<T>>
 class batch_normalization_layer {
+  static_assert(sizeof(T) == 4 || sizeof(T) == 2, "fp32 or fp16 storage");
 public:
   batch_normalization_layer(double decay = 0.9, double epsilon = 1e-5, int statistics_group_size = 1,
                             bool bessel_correction = true)
@@ -294,12 +297,21 @@ public:
     const size_t bytes = lbn_batch_norm_workspace_bytes(m_num_channels, m_channel_size, x.Width());
     void* ws = m_ws.reserve(bytes);
     float* mv = m_mean_and_var.Buffer();
-    check_status(lbn_batch_norm_fwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
-                                        m_bessel_correction ? 1 : 0, m_epsilon, m_decay, is_training ? 1 : 0,
-                                        x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(), mv,
-                                        mv + m_mean_and_var.LDim(), m_w[0], m_w[1], m_w[2], m_w[3], ws, bytes,
-                                        stats_mode),
-                 "batch_normalization_layer::fp_compute");
+    int st;
+    if (sizeof(T) == 2)
+      st = lbn_batch_norm_fwd_f16(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                  m_bessel_correction ? 1 : 0, m_epsilon, m_decay, is_training ? 1 : 0,
+                                  x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(), mv,
+                                  mv + m_mean_and_var.LDim(), m_w[0], m_w[1], m_w[2], m_w[3], ws, bytes,
+                                  stats_mode);
+    else
+      st = lbn_batch_norm_fwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                  m_bessel_correction ? 1 : 0, m_epsilon, m_decay, is_training ? 1 : 0,
+                                  reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
+                                  reinterpret_cast<float*>(y.Buffer()), y.LDim(), mv,
+                                  mv + m_mean_and_var.LDim(), m_w[0], m_w[1], m_w[2], m_w[3], ws, bytes,
+                                  stats_mode);
+    check_status(st, "batch_normalization_layer::fp_compute");
   }
   void bp_compute()
   {
@@ -310,13 +322,23 @@ public:
     void* ws = m_ws.reserve(bytes);
     const float* mv = m_mean_and_var.LockedBuffer();
     float* mvg = m_mean_and_var_gradient.Buffer();
-    check_status(lbn_batch_norm_bwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
-                                        m_bessel_correction ? 1 : 0, m_epsilon, is_training ? 1 : 0,
-                                        x.LockedBuffer(), x.LDim(), dy.LockedBuffer(), dy.LDim(), dx.Buffer(),
-                                        dx.LDim(), mv, mv + m_mean_and_var.LDim(), m_w[2], m_w[3], m_w[0],
-                                        m_scale_grad, m_bias_grad, mvg, mvg + m_mean_and_var_gradient.LDim(),
-                                        ws, bytes),
-                 "batch_normalization_layer::bp_compute");
+    int st;
+    if (sizeof(T) == 2)
+      st = lbn_batch_norm_bwd_f16(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                  m_bessel_correction ? 1 : 0, m_epsilon, is_training ? 1 : 0,
+                                  x.LockedBuffer(), x.LDim(), dy.LockedBuffer(), dy.LDim(), dx.Buffer(),
+                                  dx.LDim(), mv, mv + m_mean_and_var.LDim(), m_w[2], m_w[3], m_w[0],
+                                  m_scale_grad, m_bias_grad, mvg, mvg + m_mean_and_var_gradient.LDim(), ws,
+                                  bytes);
+    else
+      st = lbn_batch_norm_bwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                  m_bessel_correction ? 1 : 0, m_epsilon, is_training ? 1 : 0,
+                                  reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
+                                  reinterpret_cast<const float*>(dy.LockedBuffer()), dy.LDim(),
+                                  reinterpret_cast<float*>(dx.Buffer()), dx.LDim(), mv,
+                                  mv + m_mean_and_var.LDim(), m_w[2], m_w[3], m_w[0], m_scale_grad,
+                                  m_bias_grad, mvg, mvg + m_mean_and_var_gradient.LDim(), ws, bytes);
+    check_status(st, "batch_normalization_layer::bp_compute");
   }
 
 private:

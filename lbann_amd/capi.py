@@ -44,6 +44,10 @@ PROTOTYPES = {
                                       vp, vp, vp, vp, vp, sz, cint]),
     "lbn_batch_norm_bwd_f32": (cint, [vp, i64, i64, i64, cint, f32, cint, vp, i64, vp, i64, vp, i64, vp,
                                       vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]),
+    "lbn_batch_norm_fwd_f16": (cint, [vp, i64, i64, i64, cint, f32, f32, cint, vp, i64, vp, i64, vp, vp,
+                                      vp, vp, vp, vp, vp, sz, cint]),
+    "lbn_batch_norm_bwd_f16": (cint, [vp, i64, i64, i64, cint, f32, cint, vp, i64, vp, i64, vp, i64, vp,
+                                      vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]),
     "lbn_batch_norm_fwd_sums_f32": (cint, [vp, i64, i64, i64, vp, i64, vp, vp, vp, sz]),
     "lbn_batch_norm_fwd_stats_f32": (cint, [vp, i64, i64, cint, f32, f32, vp, vp, vp, vp]),
     "lbn_batch_norm_fwd_apply_f32": (cint, [vp, i64, i64, i64, f32, vp, i64, vp, i64, vp, vp, vp, vp]),

@@ -1,4 +1,6 @@
-// Batch normalization forward and backward for gfx950 (fp32).
+// Batch normalization forward and backward for gfx950: fp32 storage, and IEEE binary16
+// storage of x, y, dy, dx with all arithmetic, statistics and weights in fp32 (S is the
+// storage type of every kernel below).
 //
 // Channel c of an NCHW mini-batch is the row range [c*cs, (c+1)*cs) of every matrix
 // column, so a per-channel reduction crosses all columns: `width` segments of `cs`
@@ -31,26 +33,28 @@ struct ChannelWalk {
   int64_t total; // accesses per channel = seg * width
 };
 
-template <bool VEC>
+template <typename S, bool VEC>
 __device__ __forceinline__ ChannelWalk make_walk(int64_t cs, int64_t w)
 {
-  const int64_t seg = VEC ? cs / 4 : cs;
+  const int64_t seg = VEC ? cs / Vec16<S>::N : cs;
   return {cs, seg, seg * w};
 }
 
 // ------------------------------------------------------------------ forward sums
-template <bool VEC>
+template <typename S, bool VEC>
 __global__ void __launch_bounds__(kBnThreads)
-bn_fwd_sums(const float* __restrict__ x, int64_t ldx, int64_t cs, int64_t w, int use_pivot,
+bn_fwd_sums(const S* __restrict__ x, int64_t ldx, int64_t cs, int64_t w, int use_pivot,
             float2* __restrict__ part)
 {
   __shared__ float red[2 * (kBnThreads / kWave)];
   const int P = gridDim.x;
   const int p = blockIdx.x;
   const int64_t c = blockIdx.y;
-  const ChannelWalk wk = make_walk<VEC>(cs, w);
-  const float* xc = x + c * cs;
-  const float K = use_pivot ? xc[0] : 0.f;
+  const ChannelWalk wk = make_walk<S, VEC>(cs, w);
+  using IO = Vec16<S>;
+  constexpr int VE = IO::N;
+  const S* xc = x + c * cs;
+  const float K = use_pivot ? IO::load1(xc) : 0.f;
   float s = 0.f, q = 0.f;
   const int64_t step = static_cast<int64_t>(P) * kBnThreads;
   for (int64_t j = static_cast<int64_t>(p) * kBnThreads + threadIdx.x; j < wk.total; j += step) {
@@ -58,17 +62,17 @@ bn_fwd_sums(const float* __restrict__ x, int64_t ldx, int64_t cs, int64_t w, int
     const int64_t col = ucol;
     const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(wk.seg);
     if (VEC) {
-      float v[4];
-      Vec16<float>::load(xc + col * ldx + 4 * i, v);
+      float v[VE];
+      IO::load(xc + col * ldx + VE * i, v);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
+      for (int k = 0; k < VE; ++k) {
         const float d = v[k] - K;
         s += d;
         q += d * d;
       }
     }
     else {
-      const float d = xc[col * ldx + i] - K;
+      const float d = IO::load1(xc + col * ldx + i) - K;
       s += d;
       q += d * d;
     }
@@ -138,9 +142,9 @@ bn_stats_from_sums(int64_t C, int64_t n, int bessel, float eps, float decay,
 // ----------------------------------------------------------------- forward apply
 // FROM_PART: statistics come from the partial sums in `part` (training, fused path)
 // and workgroup 0 of each channel publishes them; otherwise mean/var are inputs.
-template <bool VEC, bool FROM_PART>
+template <typename S, bool VEC, bool FROM_PART>
 __global__ void __launch_bounds__(kBnThreads)
-bn_fwd_apply(const float* __restrict__ x, float* __restrict__ y, int64_t ldx, int64_t ldy,
+bn_fwd_apply(const S* __restrict__ x, S* __restrict__ y, int64_t ldx, int64_t ldy,
              int64_t cs, int64_t w, int use_pivot, int bessel, float eps, float decay,
              const float2* __restrict__ part, float* __restrict__ mean_io,
              float* __restrict__ var_io, const float* __restrict__ gamma,
@@ -149,14 +153,16 @@ bn_fwd_apply(const float* __restrict__ x, float* __restrict__ y, int64_t ldx, in
   const int P = gridDim.x;
   const int p = blockIdx.x;
   const int64_t c = blockIdx.y;
-  const ChannelWalk wk = make_walk<VEC>(cs, w);
-  const float* xc = x + c * cs;
-  float* yc = y + c * cs;
+  const ChannelWalk wk = make_walk<S, VEC>(cs, w);
+  using IO = Vec16<S>;
+  constexpr int VE = IO::N;
+  const S* xc = x + c * cs;
+  S* yc = y + c * cs;
   float mean, var;
   if (FROM_PART) {
     const int64_t n = cs * w;
     if (n <= 1) {
-      mean = xc[0];
+      mean = IO::load1(xc);
       var = 1.f;
       if (p == 0 && threadIdx.x == 0) {
         mean_io[c] = mean;
@@ -164,7 +170,7 @@ bn_fwd_apply(const float* __restrict__ x, float* __restrict__ y, int64_t ldx, in
       }
     }
     else {
-      const float K = use_pivot ? xc[0] : 0.f;
+      const float K = use_pivot ? IO::load1(xc) : 0.f;
       const float2 r = merge_partials(part, c, P);
       stats_from_sums(r.x, r.y, K, n, bessel, eps, mean, var);
       if (p == 0 && threadIdx.x == 0) {
@@ -188,32 +194,34 @@ bn_fwd_apply(const float* __restrict__ x, float* __restrict__ y, int64_t ldx, in
     const int64_t col = ucol;
     const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(wk.seg);
     if (VEC) {
-      float v[4];
-      Vec16<float>::load(xc + col * ldx + 4 * i, v);
+      float v[VE];
+      IO::load(xc + col * ldx + VE * i, v);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) v[k] = scale * ((v[k] - mean) * inv_stdev) + bias;
-      Vec16<float>::store(yc + col * ldy + 4 * i, v);
+      for (int k = 0; k < VE; ++k) v[k] = scale * ((v[k] - mean) * inv_stdev) + bias;
+      IO::store(yc + col * ldy + VE * i, v);
     }
     else {
-      yc[col * ldy + i] = scale * ((xc[col * ldx + i] - mean) * inv_stdev) + bias;
+      IO::store1(yc + col * ldy + i, scale * ((IO::load1(xc + col * ldx + i) - mean) * inv_stdev) + bias);
     }
   }
 }
 
 // ----------------------------------------------------------------- backward sums
 // Two sums per channel carry all four gradients: A = sum(dy), B = sum(dy * (x - mean)).
-template <bool VEC>
+template <typename S, bool VEC>
 __global__ void __launch_bounds__(kBnThreads)
-bn_bwd_sums(const float* __restrict__ x, const float* __restrict__ dy, int64_t ldx, int64_t lddy,
+bn_bwd_sums(const S* __restrict__ x, const S* __restrict__ dy, int64_t ldx, int64_t lddy,
             int64_t cs, int64_t w, const float* __restrict__ mean_in, float2* __restrict__ part)
 {
   __shared__ float red[2 * (kBnThreads / kWave)];
   const int P = gridDim.x;
   const int p = blockIdx.x;
   const int64_t c = blockIdx.y;
-  const ChannelWalk wk = make_walk<VEC>(cs, w);
-  const float* xc = x + c * cs;
-  const float* gc = dy + c * cs;
+  const ChannelWalk wk = make_walk<S, VEC>(cs, w);
+  using IO = Vec16<S>;
+  constexpr int VE = IO::N;
+  const S* xc = x + c * cs;
+  const S* gc = dy + c * cs;
   const float mean = mean_in[c];
   float a = 0.f, b = 0.f;
   const int64_t step = static_cast<int64_t>(P) * kBnThreads;
@@ -222,19 +230,19 @@ bn_bwd_sums(const float* __restrict__ x, const float* __restrict__ dy, int64_t l
     const int64_t col = ucol;
     const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(wk.seg);
     if (VEC) {
-      float v[4], g[4];
-      Vec16<float>::load(xc + col * ldx + 4 * i, v);
-      Vec16<float>::load(gc + col * lddy + 4 * i, g);
+      float v[VE], g[VE];
+      IO::load(xc + col * ldx + VE * i, v);
+      IO::load(gc + col * lddy + VE * i, g);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
+      for (int k = 0; k < VE; ++k) {
         a += g[k];
         b += g[k] * (v[k] - mean);
       }
     }
     else {
-      const float g = gc[col * lddy + i];
+      const float g = IO::load1(gc + col * lddy + i);
       a += g;
-      b += g * (xc[col * ldx + i] - mean);
+      b += g * (IO::load1(xc + col * ldx + i) - mean);
     }
   }
   team_sum2<kBnThreads / kWave>(a, b, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
@@ -275,9 +283,9 @@ bn_store_grads(const float2* __restrict__ part, int P, float eps, const float* _
 // FROM_PART: gradients of the statistics come from the partial sums (fused path) and
 // workgroup 0 of each channel publishes dscale, dbias, dmean, dvar; otherwise dmean
 // and dvar are inputs (already reduced over ranks by the caller).
-template <bool VEC, bool FROM_PART>
+template <typename S, bool VEC, bool FROM_PART>
 __global__ void __launch_bounds__(kBnThreads)
-bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ dx,
+bn_bwd_apply(const S* __restrict__ x, const S* __restrict__ dy, S* __restrict__ dx,
              int64_t ldx, int64_t lddy, int64_t lddx, int64_t cs, int64_t w, int64_t num_per_sum,
              int bessel, float eps, int training, const float2* __restrict__ part,
              const float* __restrict__ mean_in, const float* __restrict__ var_in,
@@ -287,10 +295,12 @@ bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ dy, float* _
   const int P = gridDim.x;
   const int p = blockIdx.x;
   const int64_t c = blockIdx.y;
-  const ChannelWalk wk = make_walk<VEC>(cs, w);
-  const float* xc = x + c * cs;
-  const float* gc = dy + c * cs;
-  float* dc = dx + c * cs;
+  const ChannelWalk wk = make_walk<S, VEC>(cs, w);
+  using IO = Vec16<S>;
+  constexpr int VE = IO::N;
+  const S* xc = x + c * cs;
+  const S* gc = dy + c * cs;
+  S* dc = dx + c * cs;
   const float mean = mean_in[c];
   const float inv_stdev = 1.0f / sqrtf(var_in[c] + eps);
   const float scale = gamma[c];
@@ -321,25 +331,27 @@ bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ dy, float* _
     const int64_t col = ucol;
     const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(wk.seg);
     if (VEC) {
-      float v[4], g[4];
+      float v[VE], g[VE];
       if (!zero) {
-        Vec16<float>::load(xc + col * ldx + 4 * i, v);
-        Vec16<float>::load(gc + col * lddy + 4 * i, g);
+        IO::load(xc + col * ldx + VE * i, v);
+        IO::load(gc + col * lddy + VE * i, g);
       }
 #pragma unroll
-      for (int k = 0; k < 4; ++k) g[k] = zero ? 0.f : g[k] * k0 + dmean_term + dvar_term * (v[k] - mean);
-      Vec16<float>::store(dc + col * lddx + 4 * i, g);
+      for (int k = 0; k < VE; ++k) g[k] = zero ? 0.f : g[k] * k0 + dmean_term + dvar_term * (v[k] - mean);
+      IO::store(dc + col * lddx + VE * i, g);
     }
     else {
-      dc[col * lddx + i] =
-        zero ? 0.f : gc[col * lddy + i] * k0 + dmean_term + dvar_term * (xc[col * ldx + i] - mean);
+      IO::store1(dc + col * lddx + i,
+                 zero ? 0.f
+                      : IO::load1(gc + col * lddy + i) * k0 + dmean_term +
+                          dvar_term * (IO::load1(xc + col * ldx + i) - mean));
     }
   }
 }
 
 
 // ===================================================== register-resident clusters
-// A channel (E = cs/4 * w vectors) is shared by a cluster of M workgroups of T
+// A channel (E = cs/VE * w 16-byte vectors of VE entries) is shared by a cluster of M workgroups of T
 // threads; workgroup k keeps vectors [k*T*V, (k+1)*T*V) in registers.  The grid is
 // persistent: cluster cl handles channels cl, cl + nclusters, ...
 //
@@ -369,35 +381,38 @@ __device__ __forceinline__ BnIndex<V> bn_make_index(int k, unsigned seg, unsigne
   return ix;
 }
 
-template <int V>
-__device__ __forceinline__ void bn_tile_load(float (&t)[V][4], const float* base, int64_t ld,
+template <typename S, int V>
+__device__ __forceinline__ void bn_tile_load(float (&t)[V][Vec16<S>::N], const S* base, int64_t ld,
                                              const BnIndex<V>& ix)
 {
+  constexpr int VE = Vec16<S>::N;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     if (ix.ok[i]) {
-      Vec16<float>::load(base + static_cast<int64_t>(ix.col[i]) * ld + 4 * static_cast<int64_t>(ix.pos[i]), t[i]);
+      Vec16<S>::load(base + static_cast<int64_t>(ix.col[i]) * ld + VE * static_cast<int64_t>(ix.pos[i]), t[i]);
     }
     else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) t[i][j] = 0.f;
+      for (int j = 0; j < VE; ++j) t[i][j] = 0.f;
     }
   }
 }
 
-template <int V>
-__device__ __forceinline__ void bn_tile_store(const float (&t)[V][4], float* base, int64_t ld,
+template <typename S, int V>
+__device__ __forceinline__ void bn_tile_store(const float (&t)[V][Vec16<S>::N], S* base, int64_t ld,
                                               const BnIndex<V>& ix)
 {
+  constexpr int VE = Vec16<S>::N;
 #pragma unroll
   for (int i = 0; i < V; ++i)
     if (ix.ok[i])
-      Vec16<float>::store(base + static_cast<int64_t>(ix.col[i]) * ld + 4 * static_cast<int64_t>(ix.pos[i]), t[i]);
+      Vec16<S>::store(base + static_cast<int64_t>(ix.col[i]) * ld + VE * static_cast<int64_t>(ix.pos[i]), t[i]);
 }
 
+template <typename S>
 struct BnFwdArgs {
-  const float* x;
-  float* y;
+  const S* x;
+  S* y;
   int64_t ldx, ldy, cs;
   int C, M, use_pivot, bessel;
   float eps, decay;
@@ -415,27 +430,27 @@ struct BnFwdArgs {
 // A register tile: a workgroup's share of one channel plus the channel's scalars,
 // all loaded at the same point of the pipeline so that no step waits on a load it
 // issued itself.
-template <int V>
+template <typename S, int V>
 struct BnFwdTile {
-  float v[V][4];
+  float v[V][Vec16<S>::N];
   float K, scale, bias;
 };
 
-template <int V>
-__device__ __forceinline__ void bn_fwd_load(BnFwdTile<V>& t, const BnFwdArgs& a, int ch,
+template <typename S, int V>
+__device__ __forceinline__ void bn_fwd_load(BnFwdTile<S, V>& t, const BnFwdArgs<S>& a, int ch,
                                             const BnIndex<V>& ix)
 {
-  const float* xc = a.x + static_cast<int64_t>(ch) * a.cs;
-  bn_tile_load<V>(t.v, xc, a.ldx, ix);
-  t.K = a.use_pivot ? xc[0] : 0.f;
+  const S* xc = a.x + static_cast<int64_t>(ch) * a.cs;
+  bn_tile_load<S, V>(t.v, xc, a.ldx, ix);
+  t.K = a.use_pivot ? Vec16<S>::load1(xc) : 0.f;
   t.scale = a.gamma[ch];
   t.bias = a.beta[ch];
 }
 
 // (1) of a step: partial sums of channel `ch` from tile `t`, published for the cluster.
-template <int T, int V>
-__device__ __forceinline__ void bn_fwd_reduce(const BnFwdArgs& a, const BnIndex<V>& ix, int ch, int k,
-                                              const BnFwdTile<V>& t, float* red)
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_fwd_reduce(const BnFwdArgs<S>& a, const BnIndex<V>& ix, int ch, int k,
+                                              const BnFwdTile<S, V>& t, float* red)
 {
   const unsigned tid = threadIdx.x;
   const float K = t.K;
@@ -443,7 +458,7 @@ __device__ __forceinline__ void bn_fwd_reduce(const BnFwdArgs& a, const BnIndex<
 #pragma unroll
   for (int i = 0; i < V; ++i) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < Vec16<S>::N; ++j) {
       const float d = ix.ok[i] ? t.v[i][j] - K : 0.f;
       s += d;
       q += d * d;
@@ -454,9 +469,9 @@ __device__ __forceinline__ void bn_fwd_reduce(const BnFwdArgs& a, const BnIndex<
 }
 
 // (3) of a step: statistics of channel `ch` from the cluster's partials, output from tile `t`.
-template <int T, int V>
-__device__ __forceinline__ void bn_fwd_finish(const BnFwdArgs& a, const BnIndex<V>& ix, int ch, int k,
-                                              BnFwdTile<V>& t, float* bc)
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_fwd_finish(const BnFwdArgs<S>& a, const BnIndex<V>& ix, int ch, int k,
+                                              BnFwdTile<S, V>& t, float* bc)
 {
   const unsigned tid = threadIdx.x;
   if (tid < kWave) {
@@ -483,26 +498,26 @@ __device__ __forceinline__ void bn_fwd_finish(const BnFwdArgs& a, const BnIndex<
 #pragma unroll
   for (int i = 0; i < V; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) t.v[i][j] = t.scale * ((t.v[i][j] - mean) * inv_stdev) + t.bias;
-  bn_tile_store<V>(t.v, a.y + static_cast<int64_t>(ch) * a.cs, a.ldy, ix);
+    for (int j = 0; j < Vec16<S>::N; ++j) t.v[i][j] = t.scale * ((t.v[i][j] - mean) * inv_stdev) + t.bias;
+  bn_tile_store<S, V>(t.v, a.y + static_cast<int64_t>(ch) * a.cs, a.ldy, ix);
 }
 
 // One step of the rotation: F finishes channel ch, R holds channel ch + nc, L
 // receives channel ch + 2 nc.
-template <int T, int V>
-__device__ __forceinline__ void bn_fwd_step(const BnFwdArgs& a, const BnIndex<V>& ix, int ch, int nc, int k,
-                                            BnFwdTile<V>& F, BnFwdTile<V>& R, BnFwdTile<V>& L,
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_fwd_step(const BnFwdArgs<S>& a, const BnIndex<V>& ix, int ch, int nc, int k,
+                                            BnFwdTile<S, V>& F, BnFwdTile<S, V>& R, BnFwdTile<S, V>& L,
                                             float* red, float* bc)
 {
-  if (ch + nc < a.C) bn_fwd_reduce<T, V>(a, ix, ch + nc, k, R, red);
-  if (ch + 2 * nc < a.C) bn_fwd_load<V>(L, a, ch + 2 * nc, ix);
+  if (ch + nc < a.C) bn_fwd_reduce<S, T, V>(a, ix, ch + nc, k, R, red);
+  if (ch + 2 * nc < a.C) bn_fwd_load<S, V>(L, a, ch + 2 * nc, ix);
   asm volatile("" ::: "memory");  // keep the loads above the wait below
-  bn_fwd_finish<T, V>(a, ix, ch, k, F, bc);
+  bn_fwd_finish<S, T, V>(a, ix, ch, k, F, bc);
 }
 
-template <int T, int V>
+template <typename S, int T, int V>
 __global__ void __launch_bounds__(T)
-bn_fwd_cluster(BnFwdArgs a, unsigned seg, unsigned E)
+bn_fwd_cluster(BnFwdArgs<S> a, unsigned seg, unsigned E)
 {
   __shared__ float red[2 * (T / kWave)];
   __shared__ float bc[2];
@@ -510,22 +525,23 @@ bn_fwd_cluster(BnFwdArgs a, unsigned seg, unsigned E)
   const int cl = blockIdx.x / a.M;
   const int k = blockIdx.x - cl * a.M;
   const BnIndex<V> ix = bn_make_index<T, V>(k, seg, E);
-  BnFwdTile<V> t0, t1, t2;
+  BnFwdTile<S, V> t0, t1, t2;
   if (cl >= a.C) return;
-  bn_fwd_load<V>(t0, a, cl, ix);
-  if (cl + nc < a.C) bn_fwd_load<V>(t1, a, cl + nc, ix);
-  bn_fwd_reduce<T, V>(a, ix, cl, k, t0, red);
+  bn_fwd_load<S, V>(t0, a, cl, ix);
+  if (cl + nc < a.C) bn_fwd_load<S, V>(t1, a, cl + nc, ix);
+  bn_fwd_reduce<S, T, V>(a, ix, cl, k, t0, red);
   for (int ch = cl; ch < a.C; ch += 3 * nc) {
-    bn_fwd_step<T, V>(a, ix, ch, nc, k, t0, t1, t2, red, bc);
-    if (ch + nc < a.C) bn_fwd_step<T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, red, bc);
-    if (ch + 2 * nc < a.C) bn_fwd_step<T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, red, bc);
+    bn_fwd_step<S, T, V>(a, ix, ch, nc, k, t0, t1, t2, red, bc);
+    if (ch + nc < a.C) bn_fwd_step<S, T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, red, bc);
+    if (ch + 2 * nc < a.C) bn_fwd_step<S, T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, red, bc);
   }
 }
 
+template <typename S>
 struct BnBwdArgs {
-  const float* x;
-  const float* dy;
-  float* dx;
+  const S* x;
+  const S* dy;
+  S* dx;
   int64_t ldx, lddy, lddx, cs;
   int C, M, bessel;
   float eps;
@@ -541,19 +557,19 @@ struct BnBwdArgs {
   float* dvar_out;
 };
 
-template <int V>
+template <typename S, int V>
 struct BnBwdTile {
-  float x[V][4];
-  float g[V][4];
+  float x[V][Vec16<S>::N];
+  float g[V][Vec16<S>::N];
   float mean, var, scale;
 };
 
-template <int V>
-__device__ __forceinline__ void bn_bwd_load(BnBwdTile<V>& t, const BnBwdArgs& a, int ch,
+template <typename S, int V>
+__device__ __forceinline__ void bn_bwd_load(BnBwdTile<S, V>& t, const BnBwdArgs<S>& a, int ch,
                                             const BnIndex<V>& ix)
 {
-  bn_tile_load<V>(t.x, a.x + static_cast<int64_t>(ch) * a.cs, a.ldx, ix);
-  bn_tile_load<V>(t.g, a.dy + static_cast<int64_t>(ch) * a.cs, a.lddy, ix);
+  bn_tile_load<S, V>(t.x, a.x + static_cast<int64_t>(ch) * a.cs, a.ldx, ix);
+  bn_tile_load<S, V>(t.g, a.dy + static_cast<int64_t>(ch) * a.cs, a.lddy, ix);
   t.mean = a.mean_in[ch];
   t.var = a.var_in[ch];
   t.scale = a.gamma[ch];
@@ -561,9 +577,9 @@ __device__ __forceinline__ void bn_bwd_load(BnBwdTile<V>& t, const BnBwdArgs& a,
 
 // Centres x in place (the finish step needs x - mean) and publishes
 // A = sum(dy), B = sum(dy * (x - mean)).
-template <int T, int V>
-__device__ __forceinline__ void bn_bwd_reduce(const BnBwdArgs& a, const BnIndex<V>& ix, int ch, int k,
-                                              BnBwdTile<V>& t, float* red)
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_bwd_reduce(const BnBwdArgs<S>& a, const BnIndex<V>& ix, int ch, int k,
+                                              BnBwdTile<S, V>& t, float* red)
 {
   const unsigned tid = threadIdx.x;
   const float mean = t.mean;
@@ -571,7 +587,7 @@ __device__ __forceinline__ void bn_bwd_reduce(const BnBwdArgs& a, const BnIndex<
 #pragma unroll
   for (int i = 0; i < V; ++i) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < Vec16<S>::N; ++j) {
       t.x[i][j] = ix.ok[i] ? t.x[i][j] - mean : 0.f;
       sa += t.g[i][j];
       sb += t.g[i][j] * t.x[i][j];
@@ -581,9 +597,9 @@ __device__ __forceinline__ void bn_bwd_reduce(const BnBwdArgs& a, const BnIndex<
   if (tid == 0) cluster_publish(sa, sb, a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, k, a.tag);
 }
 
-template <int T, int V>
-__device__ __forceinline__ void bn_bwd_finish(const BnBwdArgs& a, const BnIndex<V>& ix, int ch, int k,
-                                              BnBwdTile<V>& t, float* bc)
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_bwd_finish(const BnBwdArgs<S>& a, const BnIndex<V>& ix, int ch, int k,
+                                              BnBwdTile<S, V>& t, float* bc)
 {
   const unsigned tid = threadIdx.x;
   const float inv_stdev = 1.0f / sqrtf(t.var + a.eps);
@@ -613,25 +629,25 @@ __device__ __forceinline__ void bn_bwd_finish(const BnBwdArgs& a, const BnIndex<
 #pragma unroll
   for (int i = 0; i < V; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) t.g[i][j] = t.g[i][j] * k0 + dmean_term + dvar_term * t.x[i][j];
-  bn_tile_store<V>(t.g, a.dx + static_cast<int64_t>(ch) * a.cs, a.lddx, ix);
+    for (int j = 0; j < Vec16<S>::N; ++j) t.g[i][j] = t.g[i][j] * k0 + dmean_term + dvar_term * t.x[i][j];
+  bn_tile_store<S, V>(t.g, a.dx + static_cast<int64_t>(ch) * a.cs, a.lddx, ix);
 }
 
-template <int T, int V>
-__device__ __forceinline__ void bn_bwd_step(const BnBwdArgs& a, const BnIndex<V>& ix, int ch, int nc, int k,
-                                            BnBwdTile<V>& F, BnBwdTile<V>& R, BnBwdTile<V>& L, float* red,
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_bwd_step(const BnBwdArgs<S>& a, const BnIndex<V>& ix, int ch, int nc, int k,
+                                            BnBwdTile<S, V>& F, BnBwdTile<S, V>& R, BnBwdTile<S, V>& L, float* red,
                                             float* bc)
 {
-  if (ch + nc < a.C) bn_bwd_reduce<T, V>(a, ix, ch + nc, k, R, red);
-  if (ch + 2 * nc < a.C) bn_bwd_load<V>(L, a, ch + 2 * nc, ix);
+  if (ch + nc < a.C) bn_bwd_reduce<S, T, V>(a, ix, ch + nc, k, R, red);
+  if (ch + 2 * nc < a.C) bn_bwd_load<S, V>(L, a, ch + 2 * nc, ix);
   asm volatile("" ::: "memory");
-  bn_bwd_finish<T, V>(a, ix, ch, k, F, bc);
+  bn_bwd_finish<S, T, V>(a, ix, ch, k, F, bc);
 }
 
 // Backward in training mode: x and dy are read once, dx written once.
-template <int T, int V>
+template <typename S, int T, int V>
 __global__ void __launch_bounds__(T)
-bn_bwd_cluster(BnBwdArgs a, unsigned seg, unsigned E)
+bn_bwd_cluster(BnBwdArgs<S> a, unsigned seg, unsigned E)
 {
   __shared__ float red[2 * (T / kWave)];
   __shared__ float bc[2];
@@ -639,15 +655,15 @@ bn_bwd_cluster(BnBwdArgs a, unsigned seg, unsigned E)
   const int cl = blockIdx.x / a.M;
   const int k = blockIdx.x - cl * a.M;
   const BnIndex<V> ix = bn_make_index<T, V>(k, seg, E);
-  BnBwdTile<V> t0, t1, t2;
+  BnBwdTile<S, V> t0, t1, t2;
   if (cl >= a.C) return;
-  bn_bwd_load<V>(t0, a, cl, ix);
-  if (cl + nc < a.C) bn_bwd_load<V>(t1, a, cl + nc, ix);
-  bn_bwd_reduce<T, V>(a, ix, cl, k, t0, red);
+  bn_bwd_load<S, V>(t0, a, cl, ix);
+  if (cl + nc < a.C) bn_bwd_load<S, V>(t1, a, cl + nc, ix);
+  bn_bwd_reduce<S, T, V>(a, ix, cl, k, t0, red);
   for (int ch = cl; ch < a.C; ch += 3 * nc) {
-    bn_bwd_step<T, V>(a, ix, ch, nc, k, t0, t1, t2, red, bc);
-    if (ch + nc < a.C) bn_bwd_step<T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, red, bc);
-    if (ch + 2 * nc < a.C) bn_bwd_step<T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, red, bc);
+    bn_bwd_step<S, T, V>(a, ix, ch, nc, k, t0, t1, t2, red, bc);
+    if (ch + nc < a.C) bn_bwd_step<S, T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, red, bc);
+    if (ch + 2 * nc < a.C) bn_bwd_step<S, T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, red, bc);
   }
 }
 
@@ -699,77 +715,79 @@ static size_t bn_workspace(int64_t C, int64_t cs, int64_t w)
 
 // Launches the register-resident forward when the shape allows it.  Returns false
 // when the caller must use the two-kernel path.
-template <int T, int V>
-static bool bn_launch_fwd_cluster(hipStream_t st, const BnFwdArgs& a, int64_t C, unsigned seg, unsigned E)
+template <typename S, int T, int V>
+static bool bn_launch_fwd_cluster(hipStream_t st, const BnFwdArgs<S>& a, int64_t C, unsigned seg, unsigned E)
 {
-  const int cap = cluster_capacity(bn_fwd_cluster<T, V>, T);
+  const int cap = cluster_capacity(bn_fwd_cluster<S, T, V>, T);
   const int64_t ncl = cap / a.M < C ? cap / a.M : C;
   if (ncl < 1) return false;
-  hipLaunchKernelGGL((bn_fwd_cluster<T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
+  hipLaunchKernelGGL((bn_fwd_cluster<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
   return true;
 }
 
-template <int T, int V>
-static bool bn_launch_bwd_cluster(hipStream_t st, const BnBwdArgs& a, int64_t C, unsigned seg, unsigned E)
+template <typename S, int T, int V>
+static bool bn_launch_bwd_cluster(hipStream_t st, const BnBwdArgs<S>& a, int64_t C, unsigned seg, unsigned E)
 {
-  const int cap = cluster_capacity(bn_bwd_cluster<T, V>, T);
+  const int cap = cluster_capacity(bn_bwd_cluster<S, T, V>, T);
   const int64_t ncl = cap / a.M < C ? cap / a.M : C;
   if (ncl < 1) return false;
-  hipLaunchKernelGGL((bn_bwd_cluster<T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
+  hipLaunchKernelGGL((bn_bwd_cluster<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
   return true;
 }
 
+template <typename S>
 static bool bn_cluster_usable(int64_t C, int64_t cs, int64_t w, const void* ws)
 {
   static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
-  const int64_t E = cs / 4 * w;
+  const int64_t E = cs / Vec16<S>::N * w;
   return !disabled && E < (int64_t(1) << 31) - 8192 && cs * w > 1 && C <= (1 << 24) && aligned16(ws);
 }
 
+// A thread keeps at most 16 entries of a forward tile and 8 + 8 of a backward tile in
+// fp32 registers, whatever the storage type.
+template <typename S>
 static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w, int pivot, int bessel,
-                               float eps, float decay, const float* x, int64_t ldx, float* y,
-                               int64_t ldy, float* mean, float* var, const float* scale,
-                               const float* bias, float* rmean, float* rvar, void* ws)
+                               float eps, float decay, const S* x, int64_t ldx, S* y, int64_t ldy,
+                               float* mean, float* var, const float* scale, const float* bias,
+                               float* rmean, float* rvar, void* ws)
 {
-  if (!bn_cluster_usable(C, cs, w, ws)) return false;
-  const int64_t E = cs / 4 * w;
-  const BnClusterShape p = bn_cluster_shape(E, 4, 256);
+  constexpr int VE = Vec16<S>::N;
+  if (!bn_cluster_usable<S>(C, cs, w, ws)) return false;
+  const int64_t E = cs / VE * w;
+  const BnClusterShape p = bn_cluster_shape(E, 16 / VE, 256);
   if (!p.T) return false;
-  const BnFwdArgs a{x, y, ldx, ldy, cs, static_cast<int>(C), p.M, pivot, bessel, eps, decay, cs * w,
-                    cluster_workspace(ws), next_cluster_tag(), mean, var, scale, bias, rmean, rvar};
-  const unsigned seg = static_cast<unsigned>(cs / 4), Eu = static_cast<unsigned>(E);
+  const BnFwdArgs<S> a{x, y, ldx, ldy, cs, static_cast<int>(C), p.M, pivot, bessel, eps, decay, cs * w,
+                       cluster_workspace(ws), next_cluster_tag(), mean, var, scale, bias, rmean, rvar};
+  const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(E);
 #define X(TT, VV) \
-  if (p.T == TT && p.V == VV) return bn_launch_fwd_cluster<TT, VV>(st, a, C, seg, Eu);
-  X(256, 1) X(256, 2) X(256, 3) X(256, 4) X(512, 1) X(512, 2) X(512, 3) X(512, 4) X(1024, 1) X(1024, 2)
-  X(1024, 3) X(1024, 4)
-#undef X
-  return false;
-}
-
-static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bessel, float eps,
-                               const float* x, int64_t ldx, const float* dy, int64_t lddy, float* dx,
-                               int64_t lddx, const float* mean, const float* var, const float* scale,
-                               float* dscale, float* dbias, float* dmean, float* dvar, void* ws)
-{
-  if (!bn_cluster_usable(C, cs, w, ws)) return false;
-  const int64_t E = cs / 4 * w;
-  const BnClusterShape p = bn_cluster_shape(E, 2, 256);
-  if (!p.T) return false;
-  const BnBwdArgs a{x, dy, dx, ldx, lddy, lddx, cs, static_cast<int>(C), p.M, bessel, eps, cs * w,
-                    cluster_workspace(ws), next_cluster_tag(), mean, var, scale, dscale, dbias, dmean, dvar};
-  const unsigned seg = static_cast<unsigned>(cs / 4), Eu = static_cast<unsigned>(E);
-#define X(TT, VV) \
-  if (p.T == TT && p.V == VV) return bn_launch_bwd_cluster<TT, VV>(st, a, C, seg, Eu);
+  if (p.T == TT && p.V == VV) return bn_launch_fwd_cluster<S, TT, VV>(st, a, C, seg, Eu);
   X(256, 1) X(256, 2) X(512, 1) X(512, 2) X(1024, 1) X(1024, 2)
+  if constexpr (VE == 4) { X(256, 3) X(256, 4) X(512, 3) X(512, 4) X(1024, 3) X(1024, 4) }
 #undef X
   return false;
 }
 
-struct BnShape {
-  int64_t C, cs, w;
-  int P;
-  bool ok;
-};
+template <typename S>
+static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bessel, float eps,
+                               const S* x, int64_t ldx, const S* dy, int64_t lddy, S* dx, int64_t lddx,
+                               const float* mean, const float* var, const float* scale, float* dscale,
+                               float* dbias, float* dmean, float* dvar, void* ws)
+{
+  constexpr int VE = Vec16<S>::N;
+  if (!bn_cluster_usable<S>(C, cs, w, ws)) return false;
+  const int64_t E = cs / VE * w;
+  const BnClusterShape p = bn_cluster_shape(E, 8 / VE, 256);
+  if (!p.T) return false;
+  const BnBwdArgs<S> a{x, dy, dx, ldx, lddy, lddx, cs, static_cast<int>(C), p.M, bessel, eps, cs * w,
+                       cluster_workspace(ws), next_cluster_tag(), mean, var, scale, dscale, dbias, dmean, dvar};
+  const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(E);
+#define X(TT, VV) \
+  if (p.T == TT && p.V == VV) return bn_launch_bwd_cluster<S, TT, VV>(st, a, C, seg, Eu);
+  X(256, 1) X(512, 1) X(1024, 1)
+  if constexpr (VE == 4) { X(256, 2) X(512, 2) X(1024, 2) }
+#undef X
+  return false;
+}
 
 static int bn_check(int64_t C, int64_t cs, int64_t w, const int64_t* lds, int nld)
 {
@@ -781,9 +799,113 @@ static int bn_check(int64_t C, int64_t cs, int64_t w, const int64_t* lds, int nl
   return LBN_OK;
 }
 
+template <typename S>
 static bool bn_vec_ok(int64_t cs, int64_t w, const void* a, int64_t lda)
 {
-  return cs % 4 == 0 && aligned16(a) && (w <= 1 || lda % 4 == 0);
+  constexpr int VE = Vec16<S>::N;
+  return cs % VE == 0 && aligned16(a) && (w <= 1 || lda % VE == 0);
+}
+
+// Forward with given statistics (inference mode, and the last step of a caller that
+// reduces the statistics over ranks itself).
+template <typename S>
+static int bn_fwd_apply_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, float epsilon, const S* x,
+                             int64_t ldx, S* y, int64_t ldy, const float* mean, const float* var,
+                             const float* scale, const float* bias)
+{
+  const int64_t lds[2] = {ldx, ldy};
+  if (int e = bn_check(C, cs, w, lds, 2)) return e;
+  if (C == 0 || cs == 0 || w == 0) return LBN_OK;
+  if (!x || !y || !mean || !var || !scale || !bias) return LBN_ERR_INVALID_ARGUMENT;
+  const int P = bn_split(C, cs, w);
+  const dim3 grid(P, static_cast<unsigned>(C));
+  float* m = const_cast<float*>(mean);
+  float* v = const_cast<float*>(var);
+  if (bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, y, ldy))
+    hipLaunchKernelGGL((bn_fwd_apply<S, true, false>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs,
+                       w, 0, 0, epsilon, 0.f, nullptr, m, v, scale, bias, nullptr, nullptr);
+  else
+    hipLaunchKernelGGL((bn_fwd_apply<S, false, false>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs,
+                       w, 0, 0, epsilon, 0.f, nullptr, m, v, scale, bias, nullptr, nullptr);
+  return launch_status();
+}
+
+template <typename S>
+static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bessel, float epsilon,
+                       float decay, int training, const S* x, int64_t ldx, S* y, int64_t ldy, float* mean,
+                       float* var, const float* scale, const float* bias, float* running_mean,
+                       float* running_var, void* workspace, size_t workspace_bytes, int flags)
+{
+  if (!training) {
+    if (!running_mean || !running_var) return LBN_ERR_INVALID_ARGUMENT;
+    return bn_fwd_apply_host<S>(st, C, cs, w, epsilon, x, ldx, y, ldy, running_mean, running_var, scale, bias);
+  }
+  const int64_t lds[2] = {ldx, ldy};
+  if (int e = bn_check(C, cs, w, lds, 2)) return e;
+  if (C == 0 || cs == 0 || w == 0) return LBN_OK;
+  if (!x || !y || !mean || !var || !scale || !bias || !running_mean || !running_var)
+    return LBN_ERR_INVALID_ARGUMENT;
+  if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
+  const int P = bn_split(C, cs, w);
+  float2* part = static_cast<float2*>(workspace);
+  const dim3 grid(P, static_cast<unsigned>(C));
+  const int pivot = (flags & LBN_STATS_SUMSQ) ? 0 : 1;
+  const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, y, ldy);
+  if (vec && bn_try_fwd_cluster<S>(st, C, cs, w, pivot, bessel, epsilon, decay, x, ldx, y, ldy, mean, var,
+                                   scale, bias, running_mean, running_var, workspace))
+    return launch_status();
+  if (vec) {
+    hipLaunchKernelGGL((bn_fwd_sums<S, true>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, pivot, part);
+    hipLaunchKernelGGL((bn_fwd_apply<S, true, true>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs, w,
+                       pivot, bessel, epsilon, decay, part, mean, var, scale, bias, running_mean,
+                       running_var);
+  }
+  else {
+    hipLaunchKernelGGL((bn_fwd_sums<S, false>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, pivot, part);
+    hipLaunchKernelGGL((bn_fwd_apply<S, false, true>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs, w,
+                       pivot, bessel, epsilon, decay, part, mean, var, scale, bias, running_mean,
+                       running_var);
+  }
+  return launch_status();
+}
+
+template <typename S>
+static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bessel, float epsilon,
+                       int training, const S* x, int64_t ldx, const S* dy, int64_t lddy, S* dx,
+                       int64_t lddx, const float* mean, const float* var, const float* running_mean,
+                       const float* running_var, const float* scale, float* dscale, float* dbias,
+                       float* dmean, float* dvar, void* workspace, size_t workspace_bytes)
+{
+  const int64_t lds[3] = {ldx, lddy, lddx};
+  if (int e = bn_check(C, cs, w, lds, 3)) return e;
+  if (C == 0 || cs == 0 || w == 0) return LBN_OK;
+  const float* use_mean = training ? mean : running_mean;
+  const float* use_var = training ? var : running_var;
+  if (!x || !dy || !dx || !use_mean || !use_var || !scale || !dscale || !dbias || !dmean || !dvar)
+    return LBN_ERR_INVALID_ARGUMENT;
+  if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
+  const int P = bn_split(C, cs, w);
+  float2* part = static_cast<float2*>(workspace);
+  const dim3 grid(P, static_cast<unsigned>(C));
+  const int64_t n = cs * w;
+  const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, dy, lddy) && bn_vec_ok<S>(cs, w, dx, lddx);
+  if (training && vec &&
+      bn_try_bwd_cluster<S>(st, C, cs, w, bessel, epsilon, x, ldx, dy, lddy, dx, lddx, use_mean, use_var,
+                            scale, dscale, dbias, dmean, dvar, workspace))
+    return launch_status();
+  if (vec) {
+    hipLaunchKernelGGL((bn_bwd_sums<S, true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean, part);
+    hipLaunchKernelGGL((bn_bwd_apply<S, true, true>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,
+                       lddx, cs, w, n, bessel, epsilon, training, part, use_mean, use_var, scale, dscale,
+                       dbias, dmean, dvar);
+  }
+  else {
+    hipLaunchKernelGGL((bn_bwd_sums<S, false>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean, part);
+    hipLaunchKernelGGL((bn_bwd_apply<S, false, true>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,
+                       lddx, cs, w, n, bessel, epsilon, training, part, use_mean, use_var, scale, dscale,
+                       dbias, dmean, dvar);
+  }
+  return launch_status();
 }
 
 }  // namespace lbn
@@ -810,10 +932,10 @@ int lbn_batch_norm_fwd_sums_f32(lbn_stream_t stream, int64_t C, int64_t cs, int6
   float2* part = static_cast<float2*>(workspace);
   const dim3 grid(P, static_cast<unsigned>(C));
   hipStream_t st = as_stream(stream);
-  if (bn_vec_ok(cs, w, x, ldx))
-    hipLaunchKernelGGL((bn_fwd_sums<true>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, 0, part);
+  if (bn_vec_ok<float>(cs, w, x, ldx))
+    hipLaunchKernelGGL((bn_fwd_sums<float, true>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, 0, part);
   else
-    hipLaunchKernelGGL((bn_fwd_sums<false>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, 0, part);
+    hipLaunchKernelGGL((bn_fwd_sums<float, false>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, 0, part);
   hipLaunchKernelGGL(bn_store_sums, dim3(static_cast<unsigned>(C)), dim3(kWave), 0, st, part, P, mean, var);
   return launch_status();
 }
@@ -836,22 +958,7 @@ int lbn_batch_norm_fwd_apply_f32(lbn_stream_t stream, int64_t C, int64_t cs, int
                                  const float* mean, const float* var, const float* scale,
                                  const float* bias)
 {
-  const int64_t lds[2] = {ldx, ldy};
-  if (int e = bn_check(C, cs, w, lds, 2)) return e;
-  if (C == 0 || cs == 0 || w == 0) return LBN_OK;
-  if (!x || !y || !mean || !var || !scale || !bias) return LBN_ERR_INVALID_ARGUMENT;
-  const int P = bn_split(C, cs, w);
-  const dim3 grid(P, static_cast<unsigned>(C));
-  hipStream_t st = as_stream(stream);
-  float* m = const_cast<float*>(mean);
-  float* v = const_cast<float*>(var);
-  if (bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, y, ldy))
-    hipLaunchKernelGGL((bn_fwd_apply<true, false>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs,
-                       w, 0, 0, epsilon, 0.f, nullptr, m, v, scale, bias, nullptr, nullptr);
-  else
-    hipLaunchKernelGGL((bn_fwd_apply<false, false>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs,
-                       w, 0, 0, epsilon, 0.f, nullptr, m, v, scale, bias, nullptr, nullptr);
-  return launch_status();
+  return bn_fwd_apply_host<float>(as_stream(stream), C, cs, w, epsilon, x, ldx, y, ldy, mean, var, scale, bias);
 }
 
 int lbn_batch_norm_fwd_f32(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w, int bessel,
@@ -860,39 +967,20 @@ int lbn_batch_norm_fwd_f32(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
                            const float* bias, float* running_mean, float* running_var,
                            void* workspace, size_t workspace_bytes, int flags)
 {
-  if (!training) {
-    if (!running_mean || !running_var) return LBN_ERR_INVALID_ARGUMENT;
-    return lbn_batch_norm_fwd_apply_f32(stream, C, cs, w, epsilon, x, ldx, y, ldy, running_mean,
-                                        running_var, scale, bias);
-  }
-  const int64_t lds[2] = {ldx, ldy};
-  if (int e = bn_check(C, cs, w, lds, 2)) return e;
-  if (C == 0 || cs == 0 || w == 0) return LBN_OK;
-  if (!x || !y || !mean || !var || !scale || !bias || !running_mean || !running_var)
-    return LBN_ERR_INVALID_ARGUMENT;
-  if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
-  const int P = bn_split(C, cs, w);
-  float2* part = static_cast<float2*>(workspace);
-  const dim3 grid(P, static_cast<unsigned>(C));
-  hipStream_t st = as_stream(stream);
-  const int pivot = (flags & LBN_STATS_SUMSQ) ? 0 : 1;
-  if (bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, y, ldy) &&
-      bn_try_fwd_cluster(st, C, cs, w, pivot, bessel, epsilon, decay, x, ldx, y, ldy, mean, var, scale,
-                         bias, running_mean, running_var, workspace))
-    return launch_status();
-  if (bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, y, ldy)) {
-    hipLaunchKernelGGL((bn_fwd_sums<true>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, pivot, part);
-    hipLaunchKernelGGL((bn_fwd_apply<true, true>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs, w,
-                       pivot, bessel, epsilon, decay, part, mean, var, scale, bias, running_mean,
-                       running_var);
-  }
-  else {
-    hipLaunchKernelGGL((bn_fwd_sums<false>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, pivot, part);
-    hipLaunchKernelGGL((bn_fwd_apply<false, true>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs, w,
-                       pivot, bessel, epsilon, decay, part, mean, var, scale, bias, running_mean,
-                       running_var);
-  }
-  return launch_status();
+  return bn_fwd_host<float>(as_stream(stream), C, cs, w, bessel, epsilon, decay, training, x, ldx, y, ldy,
+                            mean, var, scale, bias, running_mean, running_var, workspace, workspace_bytes,
+                            flags);
+}
+
+int lbn_batch_norm_fwd_f16(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w, int bessel,
+                           float epsilon, float decay, int training, const void* x, int64_t ldx,
+                           void* y, int64_t ldy, float* mean, float* var, const float* scale,
+                           const float* bias, float* running_mean, float* running_var,
+                           void* workspace, size_t workspace_bytes, int flags)
+{
+  return bn_fwd_host<__half>(as_stream(stream), C, cs, w, bessel, epsilon, decay, training,
+                             static_cast<const __half*>(x), ldx, static_cast<__half*>(y), ldy, mean, var,
+                             scale, bias, running_mean, running_var, workspace, workspace_bytes, flags);
 }
 
 int lbn_batch_norm_bwd_sums_f32(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w,
@@ -911,10 +999,10 @@ int lbn_batch_norm_bwd_sums_f32(lbn_stream_t stream, int64_t C, int64_t cs, int6
   float2* part = static_cast<float2*>(workspace);
   const dim3 grid(P, static_cast<unsigned>(C));
   hipStream_t st = as_stream(stream);
-  if (bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, dy, lddy))
-    hipLaunchKernelGGL((bn_bwd_sums<true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, mean, part);
+  if (bn_vec_ok<float>(cs, w, x, ldx) && bn_vec_ok<float>(cs, w, dy, lddy))
+    hipLaunchKernelGGL((bn_bwd_sums<float, true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, mean, part);
   else
-    hipLaunchKernelGGL((bn_bwd_sums<false>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, mean, part);
+    hipLaunchKernelGGL((bn_bwd_sums<float, false>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, mean, part);
   hipLaunchKernelGGL(bn_store_grads, dim3(static_cast<unsigned>(C)), dim3(kWave), 0, st, part, P, epsilon,
                      mean, var, scale, dscale, dbias, dmean, dvar);
   return launch_status();
@@ -935,12 +1023,12 @@ int lbn_batch_norm_bwd_apply_f32(lbn_stream_t stream, int64_t C, int64_t cs, int
   hipStream_t st = as_stream(stream);
   float* dm = const_cast<float*>(dmean);
   float* dv = const_cast<float*>(dvar);
-  if (bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, dy, lddy) && bn_vec_ok(cs, w, dx, lddx))
-    hipLaunchKernelGGL((bn_bwd_apply<true, false>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,
+  if (bn_vec_ok<float>(cs, w, x, ldx) && bn_vec_ok<float>(cs, w, dy, lddy) && bn_vec_ok<float>(cs, w, dx, lddx))
+    hipLaunchKernelGGL((bn_bwd_apply<float, true, false>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,
                        lddx, cs, w, num_per_sum, bessel, epsilon, 1, nullptr, mean, var, scale, nullptr,
                        nullptr, dm, dv);
   else
-    hipLaunchKernelGGL((bn_bwd_apply<false, false>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,
+    hipLaunchKernelGGL((bn_bwd_apply<float, false, false>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,
                        lddx, cs, w, num_per_sum, bessel, epsilon, 1, nullptr, mean, var, scale, nullptr,
                        nullptr, dm, dv);
   return launch_status();
@@ -954,36 +1042,22 @@ int lbn_batch_norm_bwd_f32(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
                            float* dbias, float* dmean, float* dvar, void* workspace,
                            size_t workspace_bytes)
 {
-  const int64_t lds[3] = {ldx, lddy, lddx};
-  if (int e = bn_check(C, cs, w, lds, 3)) return e;
-  if (C == 0 || cs == 0 || w == 0) return LBN_OK;
-  const float* use_mean = training ? mean : running_mean;
-  const float* use_var = training ? var : running_var;
-  if (!x || !dy || !dx || !use_mean || !use_var || !scale || !dscale || !dbias || !dmean || !dvar)
-    return LBN_ERR_INVALID_ARGUMENT;
-  if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
-  const int P = bn_split(C, cs, w);
-  float2* part = static_cast<float2*>(workspace);
-  const dim3 grid(P, static_cast<unsigned>(C));
-  hipStream_t st = as_stream(stream);
-  const int64_t n = cs * w;
-  if (training && bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, dy, lddy) && bn_vec_ok(cs, w, dx, lddx) &&
-      bn_try_bwd_cluster(st, C, cs, w, bessel, epsilon, x, ldx, dy, lddy, dx, lddx, use_mean, use_var,
-                         scale, dscale, dbias, dmean, dvar, workspace))
-    return launch_status();
-  if (bn_vec_ok(cs, w, x, ldx) && bn_vec_ok(cs, w, dy, lddy) && bn_vec_ok(cs, w, dx, lddx)) {
-    hipLaunchKernelGGL((bn_bwd_sums<true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean, part);
-    hipLaunchKernelGGL((bn_bwd_apply<true, true>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,
-                       lddx, cs, w, n, bessel, epsilon, training, part, use_mean, use_var, scale, dscale,
-                       dbias, dmean, dvar);
-  }
-  else {
-    hipLaunchKernelGGL((bn_bwd_sums<false>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean, part);
-    hipLaunchKernelGGL((bn_bwd_apply<false, true>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,
-                       lddx, cs, w, n, bessel, epsilon, training, part, use_mean, use_var, scale, dscale,
-                       dbias, dmean, dvar);
-  }
-  return launch_status();
+  return bn_bwd_host<float>(as_stream(stream), C, cs, w, bessel, epsilon, training, x, ldx, dy, lddy, dx, lddx,
+                            mean, var, running_mean, running_var, scale, dscale, dbias, dmean, dvar, workspace,
+                            workspace_bytes);
+}
+
+int lbn_batch_norm_bwd_f16(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w, int bessel,
+                           float epsilon, int training, const void* x, int64_t ldx, const void* dy,
+                           int64_t lddy, void* dx, int64_t lddx, const float* mean, const float* var,
+                           const float* running_mean, const float* running_var, const float* scale,
+                           float* dscale, float* dbias, float* dmean, float* dvar, void* workspace,
+                           size_t workspace_bytes)
+{
+  return bn_bwd_host<__half>(as_stream(stream), C, cs, w, bessel, epsilon, training,
+                             static_cast<const __half*>(x), ldx, static_cast<const __half*>(dy), lddy,
+                             static_cast<__half*>(dx), lddx, mean, var, running_mean, running_var, scale,
+                             dscale, dbias, dmean, dvar, workspace, workspace_bytes);
 }
 
 }  // extern "C"

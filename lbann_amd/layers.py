@@ -324,7 +324,7 @@ class batch_normalization_layer(_Layer):
         x, y = self.prev_activations, self.activations
         C, cs = self.num_channels, self.channel_size
         ws, nb = self._ws.get(capi.lib().lbn_batch_norm_workspace_bytes(C, cs, x.width), self.device)
-        return ("lbn_batch_norm_fwd_f32",
+        return (f"lbn_batch_norm_fwd_{'f16' if x.dtype == torch.float16 else 'f32'}",
                 (_stream(), C, cs, x.width, int(self.m_bessel_correction),
                  self.m_epsilon, self.m_decay, int(self.training), x.Buffer(), x.ldim, y.Buffer(), y.ldim,
                  self._col(self.m_mean_and_var, 0), self._col(self.m_mean_and_var, 1),
@@ -335,7 +335,7 @@ class batch_normalization_layer(_Layer):
         x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
         C, cs = self.num_channels, self.channel_size
         ws, nb = self._ws.get(capi.lib().lbn_batch_norm_workspace_bytes(C, cs, x.width), self.device)
-        return ("lbn_batch_norm_bwd_f32",
+        return (f"lbn_batch_norm_bwd_{'f16' if x.dtype == torch.float16 else 'f32'}",
                 (_stream(), C, cs, x.width, int(self.m_bessel_correction),
                  self.m_epsilon, int(self.training), x.Buffer(), x.ldim, dy.Buffer(), dy.ldim, dx.Buffer(),
                  dx.ldim, self._col(self.m_mean_and_var, 0), self._col(self.m_mean_and_var, 1),

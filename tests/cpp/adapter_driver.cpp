@@ -59,6 +59,31 @@ int run_layer_norm(const int64_t* dims, int nd, int start_dim, int scale, int bi
 
 }  // namespace
 
+template <typename T>
+static int run_batch_norm(const int64_t* dims, int nd, double decay, double eps, int bessel, int training,
+                          int64_t h, int64_t w, int64_t ld, void* x, void* y, void* dy, void* dx,
+                          const float* gw, const float* bw, float* rmean, float* rvar, float* dg, float* db,
+                          float* mean_var_out, float* mean_var_grad_out, void* stream)
+{
+  batch_normalization_layer<T> layer(decay, eps, 1, bessel != 0);
+  layer.setup(std::vector<int64_t>(dims, dims + nd));
+  layer.is_training = training != 0;
+  device_matrix<T> mx, my, mdy, mdx;
+  attach(mx, h, w, static_cast<T*>(x), ld); attach(my, h, w, static_cast<T*>(y), ld);
+  attach(mdy, h, w, static_cast<T*>(dy), ld); attach(mdx, h, w, static_cast<T*>(dx), ld);
+  layer.io.prev_activations = &mx; layer.io.activations = &my;
+  layer.io.prev_error_signals = &mdy; layer.io.error_signals = &mdx;
+  layer.io.stream = static_cast<hipStream_t>(stream);
+  layer.set_weights(gw, bw, rmean, rvar);
+  layer.set_weight_gradients(dg, db);
+  layer.fp_compute();
+  layer.bp_compute();
+  copy_out(mean_var_out, layer.m_mean_and_var, layer.io.stream);
+  copy_out(mean_var_grad_out, layer.m_mean_and_var_gradient, layer.io.stream);
+  check_hip(hipStreamSynchronize(layer.io.stream), "sync");
+  return 0;
+}
+
 extern "C" {
 
 int drv_layer_norm(int half, const int64_t* dims, int nd, int start_dim, int scale, int bias, double eps,
@@ -78,28 +103,17 @@ int drv_layer_norm(int half, const int64_t* dims, int nd, int start_dim, int sca
   }
 }
 
-int drv_batch_norm(const int64_t* dims, int nd, double decay, double eps, int bessel, int training, int64_t h,
-                   int64_t w, int64_t ld, float* x, float* y, float* dy, float* dx, const float* gw,
+int drv_batch_norm(int half, const int64_t* dims, int nd, double decay, double eps, int bessel, int training,
+                   int64_t h, int64_t w, int64_t ld, void* x, void* y, void* dy, void* dx, const float* gw,
                    const float* bw, float* rmean, float* rvar, float* dg, float* db, float* mean_var_out,
                    float* mean_var_grad_out, void* stream, char* err, int errlen)
 {
   try {
-    batch_normalization_layer<> layer(decay, eps, 1, bessel != 0);
-    layer.setup(std::vector<int64_t>(dims, dims + nd));
-    layer.is_training = training != 0;
-    device_matrix<float> mx, my, mdy, mdx;
-    attach(mx, h, w, x, ld); attach(my, h, w, y, ld); attach(mdy, h, w, dy, ld); attach(mdx, h, w, dx, ld);
-    layer.io.prev_activations = &mx; layer.io.activations = &my;
-    layer.io.prev_error_signals = &mdy; layer.io.error_signals = &mdx;
-    layer.io.stream = static_cast<hipStream_t>(stream);
-    layer.set_weights(gw, bw, rmean, rvar);
-    layer.set_weight_gradients(dg, db);
-    layer.fp_compute();
-    layer.bp_compute();
-    copy_out(mean_var_out, layer.m_mean_and_var, layer.io.stream);
-    copy_out(mean_var_grad_out, layer.m_mean_and_var_gradient, layer.io.stream);
-    check_hip(hipStreamSynchronize(layer.io.stream), "sync");
-    return 0;
+    if (half)
+      return run_batch_norm<uint16_t>(dims, nd, decay, eps, bessel, training, h, w, ld, x, y, dy, dx, gw, bw,
+                                      rmean, rvar, dg, db, mean_var_out, mean_var_grad_out, stream);
+    return run_batch_norm<float>(dims, nd, decay, eps, bessel, training, h, w, ld, x, y, dy, dx, gw, bw, rmean,
+                                 rvar, dg, db, mean_var_out, mean_var_grad_out, stream);
   }
   catch (const std::exception& e) {
     return fail(e, err, errlen);
@@ -195,6 +209,7 @@ int drv_error_cases(void)
   try { channelwise_softmax_layer<> l(3, false); l.setup({2, 3, 4}); ++missed; } catch (const exception&) {}
   try { channelwise_softmax_layer<> l(1, false); l.setup({2, 3, 4}); ++missed; } catch (const exception&) {}
   try { batch_normalization_layer<> l(0.9, 1e-5, 0, true); ++missed; } catch (const exception&) {}
+  { batch_normalization_layer<uint16_t> half_storage(0.9, 1e-5, 1, true); (void)half_storage; }
   {
     layer_norm_layer<float> l(1e-5, true, true, -1);
     l.setup({31, 2, 5});

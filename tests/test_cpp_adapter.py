@@ -70,32 +70,38 @@ def test_adapter_layers_match_oracle():
         check("adapter ln dscale", dg.cpu().numpy(), dg_ref, tol=tol)
         check("adapter ln dbias", db.cpu().numpy(), db_ref, tol=tol)
 
-    # ---- batch norm (8, 12, 12) x 10
+    # ---- batch norm (8, 12, 12) x 10, fp32 and fp16 storage
     dims, w = (8, 12, 12), 10
     h = 8 * 144
-    x, dy = mk(h, w, 2.0, 3.0), mk(h, w)
     g = rng.uniform(0.5, 1.5, 8).astype(np.float32)
     b = (0.1 * rng.standard_normal(8)).astype(np.float32)
-    mx, mdy, my, mdx = DeviceMatrix.from_numpy(x), DeviceMatrix.from_numpy(dy), DeviceMatrix(h, w), DeviceMatrix(h, w)
-    gw, bw, rm, rv = dev(g), dev(b), torch.zeros(8).cuda(), torch.ones(8).cuda()
-    dg, db = torch.empty(8).cuda(), torch.empty(8).cuda()
-    mv, mvg = DeviceMatrix(8, 2), DeviceMatrix(8, 2)
-    da, nd = _dims(dims)
-    rc = d.drv_batch_norm(da, cint(nd), dbl(0.9), dbl(1e-5), cint(1), cint(1), i64(h), i64(w), i64(h), mx.Buffer(),
-                          my.Buffer(), mdy.Buffer(), mdx.Buffer(), p(gw), p(bw), p(rm), p(rv), p(dg), p(db),
-                          mv.Buffer(), mvg.Buffer(), st, err, cint(512))
-    assert rc == 0, err.value
-    rm0, rv0 = np.zeros(8, np.float32), np.ones(8, np.float32)
-    y_ref, m_ref, v_ref = orc.batch_norm_fwd(x, 8, 144, 1e-5, 0.9, g, b, rm0, rv0)
-    dx_ref, dg_ref, db_ref, dm_ref, dv_ref = orc.batch_norm_bwd(x, dy, 8, 144, 1e-5, m_ref, v_ref, g)
-    check("adapter bn y", my.to_numpy(), y_ref)
-    check("adapter bn dx", mdx.to_numpy(), dx_ref)
-    check("adapter bn mean/var", mv.to_numpy(), np.stack([m_ref, v_ref], axis=1))
-    check("adapter bn dmean/dvar", mvg.to_numpy(), np.stack([dm_ref, dv_ref], axis=1))
-    check("adapter bn dscale", dg.cpu().numpy(), dg_ref)
-    check("adapter bn dbias", db.cpu().numpy(), db_ref)
-    check("adapter bn running mean", rm.cpu().numpy(), rm0)
-    check("adapter bn running var", rv.cpu().numpy(), rv0)
+    for half in (0, 1):
+        x, dy = mk(h, w, 2.0, 3.0), mk(h, w)
+        if half:
+            x, dy = x.astype(np.float16).astype(np.float32), dy.astype(np.float16).astype(np.float32)
+        tdt = torch.float16 if half else torch.float32
+        tol = TOL_F16 if half else 1e-5
+        mx, mdy = DeviceMatrix.from_numpy(x, dtype=tdt), DeviceMatrix.from_numpy(dy, dtype=tdt)
+        my, mdx = DeviceMatrix(h, w, dtype=tdt), DeviceMatrix(h, w, dtype=tdt)
+        gw, bw, rm, rv = dev(g), dev(b), torch.zeros(8).cuda(), torch.ones(8).cuda()
+        dg, db = torch.empty(8).cuda(), torch.empty(8).cuda()
+        mv, mvg = DeviceMatrix(8, 2), DeviceMatrix(8, 2)
+        da, nd = _dims(dims)
+        rc = d.drv_batch_norm(cint(half), da, cint(nd), dbl(0.9), dbl(1e-5), cint(1), cint(1), i64(h), i64(w),
+                              i64(h), mx.Buffer(), my.Buffer(), mdy.Buffer(), mdx.Buffer(), p(gw), p(bw), p(rm),
+                              p(rv), p(dg), p(db), mv.Buffer(), mvg.Buffer(), st, err, cint(512))
+        assert rc == 0, err.value
+        rm0, rv0 = np.zeros(8, np.float32), np.ones(8, np.float32)
+        y_ref, m_ref, v_ref = orc.batch_norm_fwd(x, 8, 144, 1e-5, 0.9, g, b, rm0, rv0)
+        dx_ref, dg_ref, db_ref, dm_ref, dv_ref = orc.batch_norm_bwd(x, dy, 8, 144, 1e-5, m_ref, v_ref, g)
+        check("adapter bn y", my.to_numpy(), y_ref, tol=tol)
+        check("adapter bn dx", mdx.to_numpy(), dx_ref, tol=tol)
+        check("adapter bn mean/var", mv.to_numpy(), np.stack([m_ref, v_ref], axis=1), tol=tol)
+        check("adapter bn dmean/dvar", mvg.to_numpy(), np.stack([dm_ref, dv_ref], axis=1), tol=tol)
+        check("adapter bn dscale", dg.cpu().numpy(), dg_ref, tol=tol)
+        check("adapter bn dbias", db.cpu().numpy(), db_ref, tol=tol)
+        check("adapter bn running mean", rm.cpu().numpy(), rm0, tol=tol)
+        check("adapter bn running var", rv.cpu().numpy(), rv0, tol=tol)
 
     # ---- softmax family, incl. a row long enough for the split kernels (workspace path)
     for kind, h, w, dims, dim, single in ((0, 4096, 9, (4096,), 0, 0), (1, 1000, 7, (1000,), 0, 0),

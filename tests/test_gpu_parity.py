@@ -286,7 +286,7 @@ BN_CASES = [
 ]
 
 
-def _bn_run(L, x, dy, dims, bessel, pad, scale, bias, mode=None, training=True):
+def _bn_run(L, x, dy, dims, bessel, pad, scale, bias, mode=None, training=True, half=False):
     h, w = x.shape
     C = dims[0]
     cs = h // C
@@ -297,9 +297,11 @@ def _bn_run(L, x, dy, dims, bessel, pad, scale, bias, mode=None, training=True):
     rv0 = (1.0 + 0.05 * np.arange(C)).astype(np.float32)
     layer.weights[2].tensor[:C] = torch.from_numpy(rm0).cuda()
     layer.weights[3].tensor[:C] = torch.from_numpy(rv0).cuda()
-    y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    tdt = torch.float16 if half else torch.float32
+    tol = TOL_F16 if half else TOL_F32
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, dtype=tdt, ldim=h + pad)).to_numpy()
     mv = layer.m_mean_and_var.to_numpy()
-    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, dtype=tdt, ldim=h + pad)).to_numpy()
     mvg = layer.m_mean_and_var_gradient.to_numpy()
     out = dict(y=y, dx=dx, dscale=layer.m_scale_gradient.to_numpy(), dbias=layer.m_bias_gradient.to_numpy(),
                dmean=mvg[:, 0], dvar=mvg[:, 1], rmean=layer.weights[2].to_numpy(), rvar=layer.weights[3].to_numpy())
@@ -313,7 +315,7 @@ def _bn_run(L, x, dy, dims, bessel, pad, scale, bias, mode=None, training=True):
         dst["rmean"], dst["rvar"] = rm, rv
         dst["dx"], dst["dscale"], dst["dbias"], dst["dmean"], dst["dvar"] = orc.batch_norm_bwd(
             xx, gg, C, cs, 1e-5, dst["mean"], dst["var"], sc, rm, rv, bessel, training)
-    return {k: check(f"batch_norm {k} dims={dims} w={w}", out[k], ref[k], ex[k]) for k in out}
+    return {k: check(f"batch_norm {k} dims={dims} w={w} half={half}", out[k], ref[k], ex[k], tol=tol) for k in out}
 
 
 @pytest.mark.parametrize("dims,w,bessel,pad", BN_CASES)
@@ -325,6 +327,22 @@ def test_batch_norm(L, dims, w, bessel, pad):
     scale = rng.uniform(0.5, 1.5, C).astype(np.float32)
     bias = (0.1 * rng.standard_normal(C)).astype(np.float32)
     _bn_run(L, x, dy, dims, bessel, pad, scale, bias)
+
+
+@pytest.mark.parametrize("dims,w,bessel,pad,training", [
+    ((8, 16, 16), 12, True, 0, True), ((16, 28, 28), 8, False, 0, True), ((7, 5, 3), 14, True, 0, True),
+    ((5, 24), 10, True, 8, True), ((256, 8, 8), 32, True, 0, True), ((3, 56, 56), 16, True, 0, False),
+    ((2, 100000), 3, True, 0, True), ((64, 56, 56), 16, True, 0, True)])
+def test_batch_norm_f16(L, dims, w, bessel, pad, training):
+    """fp16 storage, fp32 arithmetic: the oracle sees the fp16-rounded inputs."""
+    rng = np.random.default_rng(int(np.prod(dims)) * 5 + w)
+    h = int(np.prod(dims))
+    x = rand(rng, h, w, 2.0, 3.0).astype(np.float16).astype(np.float32)
+    dy = rand(rng, h, w).astype(np.float16).astype(np.float32)
+    C = dims[0]
+    scale = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    _bn_run(L, x, dy, dims, bessel, pad, scale, bias, training=training, half=True)
 
 
 def test_batch_norm_inference_and_reference_formula(L):
