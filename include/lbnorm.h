@@ -17,6 +17,12 @@
  * *_workspace_bytes() function returns the size needed for a given shape
  * (possibly 0, in which case NULL may be passed).  A workspace only carries data
  * between the kernels of one call.
+ *
+ * HIP graphs: the compute entry points may be called on a stream that is recording
+ * (hipStreamBeginCapture); they record kernel launches only.  While recording they
+ * avoid the kernels in which workgroups wait for each other (those take a per-call
+ * tag as an argument, which a replay would repeat) and use their multi-kernel
+ * paths instead, so a replayed call can be slower than an eager one.
  */
 #ifndef LBNORM_H_INCLUDED
 #define LBNORM_H_INCLUDED

@@ -736,11 +736,12 @@ static bool bn_launch_bwd_cluster(hipStream_t st, const BnBwdArgs<S>& a, int64_t
 }
 
 template <typename S>
-static bool bn_cluster_usable(int64_t C, int64_t cs, int64_t w, const void* ws)
+static bool bn_cluster_usable(int64_t C, int64_t cs, int64_t w, const void* ws, hipStream_t st)
 {
   static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
   const int64_t E = cs / Vec16<S>::N * w;
-  return !disabled && E < (int64_t(1) << 31) - 8192 && cs * w > 1 && C <= (1 << 24) && aligned16(ws);
+  return !disabled && E < (int64_t(1) << 31) - 8192 && cs * w > 1 && C <= (1 << 24) && aligned16(ws) &&
+         !stream_is_capturing(st);
 }
 
 // A thread keeps at most 16 entries of a forward tile and 8 + 8 of a backward tile in
@@ -752,7 +753,7 @@ static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
                                float* rmean, float* rvar, void* ws)
 {
   constexpr int VE = Vec16<S>::N;
-  if (!bn_cluster_usable<S>(C, cs, w, ws)) return false;
+  if (!bn_cluster_usable<S>(C, cs, w, ws, st)) return false;
   const int64_t E = cs / VE * w;
   const BnClusterShape p = bn_cluster_shape(E, 16 / VE, 256);
   if (!p.T) return false;
@@ -774,7 +775,7 @@ static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
                                float* dbias, float* dmean, float* dvar, void* ws)
 {
   constexpr int VE = Vec16<S>::N;
-  if (!bn_cluster_usable<S>(C, cs, w, ws)) return false;
+  if (!bn_cluster_usable<S>(C, cs, w, ws, st)) return false;
   const int64_t E = cs / VE * w;
   const BnClusterShape p = bn_cluster_shape(E, 8 / VE, 256);
   if (!p.T) return false;

@@ -23,6 +23,20 @@ inline int launch_status()
   return e == hipSuccess ? LBN_OK : static_cast<int>(e);
 }
 
+// True while `st` records into a HIP graph.  A recorded launch is replayed with the
+// arguments it was recorded with, so anything that must differ from call to call (the
+// rendezvous tag of the cluster kernels) cannot go into a graph: entry points fall
+// back to their multi-kernel paths while this holds.
+inline bool stream_is_capturing(hipStream_t st)
+{
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // True when every row start of a matrix walked with (stride, ld) keeps 16-byte

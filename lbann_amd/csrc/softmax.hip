@@ -705,11 +705,11 @@ static int stream_loads(int64_t rows, int64_t n, int tensors)
   return rows * n * 4 * tensors >= kStreamLoadMinBytes ? 1 : 0;
 }
 
-static bool cluster_enabled(int64_t rows, int64_t n)
+static bool cluster_enabled(int64_t rows, int64_t n, hipStream_t st)
 {
   static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
   static const bool forced = std::getenv("LBN_FORCE_CLUSTER") != nullptr;
-  return !disabled && (forced || rows * n * 4 >= kClusterMinBytes);
+  return !disabled && (forced || rows * n * 4 >= kClusterMinBytes) && !stream_is_capturing(st);
 }
 
 #define LBN_ROW_CASES(X)                                                                     \
@@ -750,7 +750,7 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #undef X
     }
   }
-  if (vec && cluster_enabled(rows, n) && n / 4 < (int64_t(1) << 30)) {
+  if (vec && cluster_enabled(rows, n, st) && n / 4 < (int64_t(1) << 30)) {
     // four vectors per thread keep five workgroups per CU resident; eight only for rows that need it
     ClusterPlan cp = plan_cluster(n / 4, 4);
     if (!cp.M) cp = plan_cluster(n / 4, 8);
@@ -828,7 +828,7 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #undef X
     }
   }
-  if (vec && cluster_enabled(rows, n) && n / 4 < (int64_t(1) << 30)) {
+  if (vec && cluster_enabled(rows, n, st) && n / 4 < (int64_t(1) << 30)) {
     const ClusterPlan cp = plan_cluster(n / 4, 4);
     if (cp.M) {
       if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
