@@ -154,6 +154,50 @@ def main():
             return t1 - t0, t2 - t1
         return layer, data["x"].size, 4, data["x"].shape[1], cpu
 
+    def build_ce(data):
+        h, w = data["x"].shape
+        rng = np.random.default_rng(7)
+        pred = np.asfortranarray(rng.uniform(0.05, 1.0, (w, h)).astype(np.float32).T)
+        truth = np.asfortranarray(rng.uniform(0.0, 1.0, (w, h)).astype(np.float32).T)
+        dloss = rng.standard_normal(w).astype(np.float32)
+        layer = L.cross_entropy_layer((h,))
+        layer.forward(upload(pred), upload(truth))
+        layer.backward(L.DeviceMatrix.from_numpy(dloss.reshape(1, -1)))
+
+        def cpu():
+            from oracle import cpu_oracle as orc
+            t0 = time.perf_counter(); orc.cross_entropy_fwd(pred, truth); t1 = time.perf_counter()
+            orc.cross_entropy_bwd(pred, truth, dloss); t2 = time.perf_counter()
+            return t1 - t0, t2 - t1
+        # forward reads prediction and ground truth; backward reads both and writes both gradients
+        return layer, pred.size, 4, w, cpu, (2 * pred.size * 4, 4 * pred.size * 4)
+
+    def build_sb(data, kind):
+        x, dy = upload(data["x"]), upload(data["dy"])
+        h = data["x"].shape[0]
+        rng = np.random.default_rng(11)
+        if kind == "entrywise":
+            layer, n = L.entrywise_scale_bias_layer((h,)), h
+        else:
+            layer, n = L.channelwise_scale_bias_layer(data["dims"]), data["dims"][0]
+        wts = np.asfortranarray(np.stack([rng.normal(1, 1, n), rng.normal(0, 1, n)], axis=1).astype(np.float32))
+        layer.set_weights(wts[:, 0], wts[:, 1])
+        layer.bind_forward(x)
+        layer.bind_backward(dy)
+
+        def cpu():
+            from oracle import cpu_oracle as orc
+            if kind == "entrywise":
+                t0 = time.perf_counter(); orc.entrywise_scale_bias_fwd(data["x"], wts); t1 = time.perf_counter()
+                orc.entrywise_scale_bias_bwd(data["x"], data["dy"], wts); t2 = time.perf_counter()
+            else:
+                C = n
+                cs = h // C
+                t0 = time.perf_counter(); orc.channelwise_scale_bias_fwd(data["x"], wts, C, cs); t1 = time.perf_counter()
+                orc.channelwise_scale_bias_bwd(data["x"], data["dy"], wts, C, cs); t2 = time.perf_counter()
+            return t1 - t0, t2 - t1
+        return layer, data["x"].size, 4, data["x"].shape[1], cpu
+
     table = {
         "cfg2_softmax": ("Softmax fwd+bwd fp32 32768x512", lambda: build_softmax("softmax", W.cfg2_softmax())),
         "cfg2_log_softmax": ("LogSoftmax fwd+bwd fp32 32768x512", lambda: build_softmax("log_softmax", W.cfg2_softmax())),
@@ -171,6 +215,13 @@ def main():
         # split kernels run long enough to be measured against bandwidth rather than launch latency
         "extra_wide_softmax_w256": ("Softmax fwd+bwd fp32 262144x256 (split rows, informational)",
                                     lambda: build_softmax("softmax", W.cfg5b_wide_softmax(w=256))),
+        # not baseline configurations: the layers either side of the path, on the tensors of cfg2 / cfg3
+        "extra_cross_entropy": ("CrossEntropy (dense ground truth) fwd+bwd fp32 32768x512 (informational)",
+                                lambda: build_ce(W.cfg2_softmax())),
+        "extra_entrywise_scale_bias": ("EntrywiseScaleBias fwd+bwd fp32 1048576x64 (informational)",
+                                       lambda: build_sb(W.extra_entrywise_batch_norm(), "entrywise")),
+        "extra_channelwise_scale_bias": ("ChannelwiseScaleBias fwd+bwd fp32 NCHW 64x256x56x56 (informational)",
+                                         lambda: build_sb(W.cfg3_batch_norm(), "channelwise")),
     }
     headline = "cfg2_softmax"
     if args.layers == "all":
@@ -259,8 +310,10 @@ def main():
     cpu_threads = None
     for name in names:
         desc, builder = table[name]
-        layer, elems, esize, samples, cpu = builder()
-        fwd_b, bwd_b = W.algorithmic_bytes(elems, esize)
+        built = builder()
+        layer, elems, esize, samples, cpu = built[:5]
+        # (forward, backward) bytes: 2 and 3 tensors unless the builder says otherwise
+        fwd_b, bwd_b = built[5] if len(built) > 5 else W.algorithmic_bytes(elems, esize)
         wall, fwd, bwd, bwd_b2b = measure(layer, args.steps, args.warmup)
         f_ms, b_ms = statistics.mean(fwd), statistics.mean(bwd)
         step_ms = wall / args.steps * 1e3

@@ -282,6 +282,71 @@ int lbn_channelwise_softmax_bwd_f32(lbn_stream_t stream, int64_t channels,
                                     const float* dy, int64_t lddy, float* dx, int64_t lddx,
                                     void* workspace, size_t workspace_bytes);
 
+/* --------------------------------------------------------------- cross entropy
+ * The layer that consumes the softmax output.  Replaces
+ * cross_entropy_layer::local_fp_compute / local_bp_compute
+ * (src/layers/loss/cross_entropy.cpp:35-73, :75-120; GPU code cross_entropy.cu).
+ * loss[c*ld_loss] = -sum over rows with xhat > 0 of xhat * log(prediction) for column c
+ * (the layer's 1 x width workspace matrix, before its sum across ranks,
+ * cross_entropy_impl.hpp:186-201).  Backward: dprediction = -dloss * xhat / prediction
+ * where xhat > 0 and 0 elsewhere; dground_truth = -dloss * log(prediction), with
+ * dloss[c*ld_dloss] the gradient w.r.t. column c's loss.
+ * use_labels == 0: ground_truth has the shape of prediction.  use_labels != 0: it
+ * holds one class index per spatial position, stored as a floating-point number in rows
+ * [0, spatial_size) of its column; row r of prediction is class r / spatial_size at
+ * position r % spatial_size and xhat(r) = 1 where the position's label, converted to
+ * int, equals the class, else 0; dground_truth is not written and may be NULL.
+ * spatial_size is ignored when use_labels == 0. */
+size_t lbn_cross_entropy_fwd_workspace_bytes(int64_t height, int64_t width);
+int lbn_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                              int64_t spatial_size,
+                              const float* prediction, int64_t ld_prediction,
+                              const float* ground_truth, int64_t ld_ground_truth,
+                              float* loss, int64_t ld_loss,
+                              void* workspace, size_t workspace_bytes);
+int lbn_cross_entropy_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                              int64_t spatial_size,
+                              const float* prediction, int64_t ld_prediction,
+                              const float* ground_truth, int64_t ld_ground_truth,
+                              const float* dloss, int64_t ld_dloss,
+                              float* dprediction, int64_t ld_dprediction,
+                              float* dground_truth, int64_t ld_dground_truth);
+
+/* ------------------------------------------------------- scale and bias layers
+ * The learned affine layers that follow a normalization layer without one.  Replace
+ * entrywise_scale_bias_layer::fp_compute / bp_compute
+ * (src/layers/learning/entrywise_scale_bias.cpp:35-60, :62-113) and
+ * channelwise_scale_bias_layer::fp_compute / bp_compute
+ * (src/layers/learning/channelwise_scale_bias.cpp:33-73, :75-135).
+ * y = a*x + b; dx = a*dy; da = sum(x*dy), db = sum(dy) over everything that shares the
+ * pair (a, b): one pair per matrix row over the mini-batch (entry-wise), or one per
+ * channel = rows [c*channel_size, (c+1)*channel_size) of every column (channel-wise).
+ * weights is the layer's single weights matrix, (height x 2) resp. (channels x 2):
+ * column 0 scale, column 1 bias; weights_grad has the same shape and is overwritten
+ * (the caller adds it to the optimizer's gradient, entrywise_scale_bias.cpp:139-145). */
+int lbn_entrywise_scale_bias_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                     const float* x, int64_t ldx, float* y, int64_t ldy,
+                                     const float* weights, int64_t ld_weights);
+size_t lbn_entrywise_scale_bias_bwd_workspace_bytes(int64_t height, int64_t width);
+int lbn_entrywise_scale_bias_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                     const float* x, int64_t ldx, const float* dy, int64_t lddy,
+                                     float* dx, int64_t lddx,
+                                     const float* weights, int64_t ld_weights,
+                                     float* weights_grad, int64_t ld_weights_grad,
+                                     void* workspace, size_t workspace_bytes);
+int lbn_channelwise_scale_bias_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                       int64_t width, const float* x, int64_t ldx,
+                                       float* y, int64_t ldy,
+                                       const float* weights, int64_t ld_weights);
+size_t lbn_channelwise_scale_bias_bwd_workspace_bytes(int64_t channels, int64_t channel_size,
+                                                      int64_t width);
+int lbn_channelwise_scale_bias_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                       int64_t width, const float* x, int64_t ldx,
+                                       const float* dy, int64_t lddy, float* dx, int64_t lddx,
+                                       const float* weights, int64_t ld_weights,
+                                       float* weights_grad, int64_t ld_weights_grad,
+                                       void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -9,6 +9,8 @@
 //   softmax_layer               src/layers/activations/softmax.cu      (data-parallel branch)
 //   log_softmax_layer           src/layers/activations/log_softmax.cu
 //   channelwise_softmax_layer   src/layers/misc/channelwise_softmax.cu
+// and, beyond those five, instance_norm_layer, entrywise_batch_normalization_layer,
+// cross_entropy_layer, entrywise_scale_bias_layer and channelwise_scale_bias_layer.
 //
 // `Mat` is any local-matrix type with the El::Matrix<T, El::Device::GPU> accessors
 //   Height(), Width(), LDim(), Buffer(), LockedBuffer()
@@ -18,6 +20,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdint>
 #include <functional>
 #include <numeric>
@@ -588,6 +591,165 @@ private:
   float m_decay, m_epsilon;
   int64_t m_size = 0;
   float* m_w[2] = {nullptr, nullptr};
+};
+
+// ------------------------------------------------------------------ cross entropy
+/// include/lbann/layers/loss/cross_entropy.hpp:75-190.  Two parents: the prediction
+/// (io.prev_activations) and the ground truth (prev_ground_truth); the output is the
+/// layer's 1 x width workspace matrix, which the reference sums across ranks and copies
+/// into its activations (cross_entropy_impl.hpp:186-201).  bp_compute() reads the
+/// gradient w.r.t. that row from io.prev_error_signals and writes io.error_signals
+/// (w.r.t. the prediction) and, without use_labels, ground_truth_error_signals.
+template <typename Mat = device_matrix<float>>
+class cross_entropy_layer {
+public:
+  explicit cross_entropy_layer(bool use_labels = false) : m_use_labels(use_labels) {}
+
+  /// setup_dims (cross_entropy_impl.hpp:39-155): the two inputs' dimensions
+  void setup(const std::vector<int64_t>& prediction_dims, const std::vector<int64_t>& ground_truth_dims)
+  {
+    if (m_use_labels) {
+      if (ground_truth_dims.empty() || ground_truth_dims[0] != 1)
+        throw exception("cross entropy layer expects the 0-th dimension of the tensor to be 1 when use labels is enabled.");
+      if (prediction_dims.size() != ground_truth_dims.size() || prediction_dims.size() < 2)
+        throw exception("cross entropy layer expects both input tensors to have the same number of dimensions and have >2 "
+                        "dimensions when use_labels is enabled.");
+      if (!std::equal(prediction_dims.begin() + 1, prediction_dims.end(), ground_truth_dims.begin() + 1))
+        throw exception("cross entropy layer expects both input tensors to have the same shape after the 0-th dimesion when "
+                        "use_labels is enabled.");
+    }
+    else if (prediction_dims != ground_truth_dims) {
+      throw exception("cross entropy layer has input tensors with different dimensions");
+    }
+    m_spatial_sample_size = detail::product(prediction_dims, 1, prediction_dims.size());
+  }
+
+  layer_io<Mat> io;
+  const Mat* prev_ground_truth = nullptr;       // get_local_prev_activations(1)
+  Mat* ground_truth_error_signals = nullptr;    // get_local_error_signals(1); unused with use_labels
+
+  void fp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    const Mat& t = *prev_ground_truth;
+    Mat& loss = *io.activations;
+    const size_t bytes = lbn_cross_entropy_fwd_workspace_bytes(x.Height(), x.Width());
+    check_status(lbn_cross_entropy_fwd_f32(io.stream, x.Height(), x.Width(), m_use_labels ? 1 : 0,
+                                           m_spatial_sample_size, x.LockedBuffer(), x.LDim(), t.LockedBuffer(),
+                                           t.LDim(), loss.Buffer(), loss.LDim(), m_ws.reserve(bytes), bytes),
+                 "cross_entropy_layer::fp_compute");
+  }
+  void bp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    const Mat& t = *prev_ground_truth;
+    const Mat& dy = *io.prev_error_signals;
+    Mat& dx = *io.error_signals;
+    Mat* dt = m_use_labels ? nullptr : ground_truth_error_signals;
+    check_status(lbn_cross_entropy_bwd_f32(io.stream, x.Height(), x.Width(), m_use_labels ? 1 : 0,
+                                           m_spatial_sample_size, x.LockedBuffer(), x.LDim(), t.LockedBuffer(),
+                                           t.LDim(), dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+                                           dt ? dt->Buffer() : nullptr, dt ? dt->LDim() : 0),
+                 "cross_entropy_layer::bp_compute");
+  }
+private:
+  bool m_use_labels;
+  int64_t m_spatial_sample_size = 1;
+  workspace m_ws;
+};
+
+// ---------------------------------------------------------- scale and bias layers
+/// include/lbann/layers/learning/entrywise_scale_bias.hpp:57-203.  One weights matrix
+/// (size x 2: scale, bias; the framework owns it) and m_weights_gradient of that shape.
+template <typename Mat = device_matrix<float>>
+class entrywise_scale_bias_layer {
+public:
+  void setup(const std::vector<int64_t>& dims)
+  {
+    m_size = detail::product(dims, 0, dims.size());
+    m_weights_gradient.Resize(m_size, 2);
+  }
+  /// device pointer to the (size x 2) column-major weights values and their leading dimension
+  void set_weights(const float* values, int64_t ldim) { m_weights = values; m_ld_weights = ldim; }
+
+  layer_io<Mat> io;
+  device_matrix<float> m_weights_gradient;
+
+  void fp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    Mat& y = *io.activations;
+    if (!m_weights) throw exception("entrywise_scale_bias_layer: weights are not set");
+    check_status(lbn_entrywise_scale_bias_fwd_f32(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(),
+                                                  y.Buffer(), y.LDim(), m_weights, m_ld_weights),
+                 "entrywise_scale_bias_layer::fp_compute");
+  }
+  void bp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    const Mat& dy = *io.prev_error_signals;
+    Mat& dx = *io.error_signals;
+    if (!m_weights) throw exception("entrywise_scale_bias_layer: weights are not set");
+    const size_t bytes = lbn_entrywise_scale_bias_bwd_workspace_bytes(x.Height(), x.Width());
+    check_status(lbn_entrywise_scale_bias_bwd_f32(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(),
+                                                  dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(), m_weights,
+                                                  m_ld_weights, m_weights_gradient.Buffer(),
+                                                  m_weights_gradient.LDim(), m_ws.reserve(bytes), bytes),
+                 "entrywise_scale_bias_layer::bp_compute");
+  }
+private:
+  int64_t m_size = 0;
+  const float* m_weights = nullptr;
+  int64_t m_ld_weights = 0;
+  workspace m_ws;
+};
+
+/// include/lbann/layers/learning/channelwise_scale_bias.hpp:60-206.  Weights are
+/// (num_channels x 2), num_channels = dims[0].
+template <typename Mat = device_matrix<float>>
+class channelwise_scale_bias_layer {
+public:
+  void setup(const std::vector<int64_t>& dims)
+  {
+    if (dims.empty()) throw exception("channelwise_scale_bias_layer: empty dimensions");
+    m_num_channels = dims[0];
+    m_channel_size = detail::product(dims, 1, dims.size());
+    m_weights_gradient.Resize(m_num_channels, 2);
+  }
+  void set_weights(const float* values, int64_t ldim) { m_weights = values; m_ld_weights = ldim; }
+
+  layer_io<Mat> io;
+  device_matrix<float> m_weights_gradient;
+
+  void fp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    Mat& y = *io.activations;
+    if (!m_weights) throw exception("channelwise_scale_bias_layer: weights are not set");
+    check_status(lbn_channelwise_scale_bias_fwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                                    x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(), m_weights,
+                                                    m_ld_weights),
+                 "channelwise_scale_bias_layer::fp_compute");
+  }
+  void bp_compute()
+  {
+    const Mat& x = *io.prev_activations;
+    const Mat& dy = *io.prev_error_signals;
+    Mat& dx = *io.error_signals;
+    if (!m_weights) throw exception("channelwise_scale_bias_layer: weights are not set");
+    const size_t bytes = lbn_channelwise_scale_bias_bwd_workspace_bytes(m_num_channels, m_channel_size, x.Width());
+    check_status(lbn_channelwise_scale_bias_bwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                                    x.LockedBuffer(), x.LDim(), dy.LockedBuffer(), dy.LDim(),
+                                                    dx.Buffer(), dx.LDim(), m_weights, m_ld_weights,
+                                                    m_weights_gradient.Buffer(), m_weights_gradient.LDim(),
+                                                    m_ws.reserve(bytes), bytes),
+                 "channelwise_scale_bias_layer::bp_compute");
+  }
+private:
+  int64_t m_num_channels = 0, m_channel_size = 0;
+  const float* m_weights = nullptr;
+  int64_t m_ld_weights = 0;
+  workspace m_ws;
 };
 
 }  // namespace lbnorm

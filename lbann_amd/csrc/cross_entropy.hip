@@ -1,0 +1,293 @@
+// Cross entropy between a predicted distribution x and a ground truth xhat, per sample
+// (matrix column): loss = -sum over entries with xhat > 0 of xhat * log(x); backward
+// gives dx = -dy * xhat / x where xhat > 0 (0 elsewhere) and dxhat = -dy * log(x).
+// Reference CPU code: src/layers/loss/cross_entropy.cpp:35-73 (local_fp_cpu), :75-120
+// (local_bp_cpu).
+//
+// Two ground-truth formats, as in the reference:
+//  * dense: xhat has the shape of x.
+//  * labels (use_labels): xhat holds one class index per spatial position, stored as a
+//    floating-point number in rows [0, spatial) of its column; row r of x belongs to
+//    class r / spatial at position r % spatial and xhat(r) is 1 where the position's
+//    label equals the class, else 0.  The forward pass therefore needs one entry of x
+//    per position: it gathers x(label*spatial + position) instead of streaming all of x.
+//
+// grid = (width, P): the P workgroups of a column stride over its 16-byte vectors
+// (scalars for unaligned shapes); the forward pass reduces each workgroup's partial sum
+// in a fixed order and, when P > 1, a one-wave kernel per column adds the P partials.
+// No atomics.
+#include <cmath>
+
+#include "device_utils.hpp"
+#include "host_utils.hpp"
+
+namespace lbn {
+
+constexpr int kCeThreads = 256;
+constexpr int kCeWaves = kCeThreads / kWave;
+constexpr int kCeMaxParts = 64;
+
+struct CeArgs {
+  int64_t h, w, spatial;
+  const float* x;
+  const float* truth;
+  int64_t ldx, ldt;
+  float* loss;  // forward: element c at loss[c*ld_loss]
+  int64_t ld_loss;
+  const float* dy;  // backward: element c at dy[c*lddy]
+  int64_t lddy;
+  float* dx;
+  float* dtruth;
+  int64_t lddx, lddt;
+  float* part;  // [w][P]
+};
+
+__device__ __forceinline__ float ce_term(float xhat, float x) { return xhat > 0.f ? -xhat * logf(x) : 0.f; }
+
+// The class index a label entry stands for: conversion to int as in the reference
+// (`const int truth_label = local_ground_truth(offset, col)`, cross_entropy.cpp:58).
+__device__ __forceinline__ int64_t ce_label(float v) { return static_cast<int64_t>(static_cast<int>(v)); }
+
+__device__ __forceinline__ void ce_store_partial(const CeArgs& a, float sum, float* red)
+{
+  sum = team_sum<kCeWaves>(sum, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+  if (threadIdx.x == 0) {
+    const int64_t c = blockIdx.x;
+    if (gridDim.y == 1) a.loss[c * a.ld_loss] = sum;
+    else a.part[c * gridDim.y + blockIdx.y] = sum;
+  }
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(kCeThreads)
+ce_fwd_dense(CeArgs a)
+{
+  __shared__ float red[kCeWaves];
+  const int64_t c = blockIdx.x;
+  const float* xc = a.x + c * a.ldx;
+  const float* tc = a.truth + c * a.ldt;
+  const int64_t n = VEC ? a.h / 4 : a.h;
+  const int64_t step = static_cast<int64_t>(gridDim.y) * kCeThreads;
+  float sum = 0.f;
+  for (int64_t j = static_cast<int64_t>(blockIdx.y) * kCeThreads + threadIdx.x; j < n; j += step) {
+    if (VEC) {
+      float v[4], t[4];
+      Vec16<float>::load(xc + 4 * j, v);
+      Vec16<float>::load(tc + 4 * j, t);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) sum += ce_term(t[k], v[k]);
+    }
+    else {
+      sum += ce_term(tc[j], xc[j]);
+    }
+  }
+  ce_store_partial(a, sum, red);
+}
+
+// One thread per spatial position: gather the entry of x its label points at.
+__global__ void __launch_bounds__(kCeThreads)
+ce_fwd_labels(CeArgs a)
+{
+  __shared__ float red[kCeWaves];
+  const int64_t c = blockIdx.x;
+  const float* xc = a.x + c * a.ldx;
+  const float* tc = a.truth + c * a.ldt;
+  const int64_t positions = a.spatial < a.h ? a.spatial : a.h;
+  const int64_t step = static_cast<int64_t>(gridDim.y) * kCeThreads;
+  float sum = 0.f;
+  for (int64_t o = static_cast<int64_t>(blockIdx.y) * kCeThreads + threadIdx.x; o < positions; o += step) {
+    const int64_t label = ce_label(tc[o]);
+    const int64_t r = label * a.spatial + o;
+    if (label >= 0 && r < a.h) sum += -logf(xc[r]);
+  }
+  ce_store_partial(a, sum, red);
+}
+
+__global__ void __launch_bounds__(kWave)
+ce_merge_parts(int P, const float* __restrict__ part, float* __restrict__ loss, int64_t ld_loss)
+{
+  const int64_t c = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float v = wave_sum(lane < P ? part[c * P + lane] : 0.f);
+  if (lane == 0) loss[c * ld_loss] = v;
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(kCeThreads)
+ce_bwd_dense(CeArgs a)
+{
+  const int64_t c = blockIdx.x;
+  const float g = a.dy[c * a.lddy];
+  const float* xc = a.x + c * a.ldx;
+  const float* tc = a.truth + c * a.ldt;
+  float* dxc = a.dx + c * a.lddx;
+  float* dtc = a.dtruth + c * a.lddt;
+  const int64_t n = VEC ? a.h / 4 : a.h;
+  const int64_t step = static_cast<int64_t>(gridDim.y) * kCeThreads;
+  for (int64_t j = static_cast<int64_t>(blockIdx.y) * kCeThreads + threadIdx.x; j < n; j += step) {
+    if (VEC) {
+      float v[4], t[4], d[4], dt[4];
+      Vec16<float>::load(xc + 4 * j, v);
+      Vec16<float>::load(tc + 4 * j, t);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        dt[k] = -g * logf(v[k]);
+        d[k] = t[k] > 0.f ? -g * t[k] / v[k] : 0.f;
+      }
+      Vec16<float>::store(dxc + 4 * j, d);
+      Vec16<float>::store(dtc + 4 * j, dt);
+    }
+    else {
+      const float v = xc[j], t = tc[j];
+      dtc[j] = -g * logf(v);
+      dxc[j] = t > 0.f ? -g * t / v : 0.f;
+    }
+  }
+}
+
+// VEC: spatial is a multiple of 4, so the 4 rows of a vector share a class.
+template <bool VEC>
+__global__ void __launch_bounds__(kCeThreads)
+ce_bwd_labels(CeArgs a)
+{
+  const int64_t c = blockIdx.x;
+  const float g = a.dy[c * a.lddy];
+  const float* xc = a.x + c * a.ldx;
+  const float* tc = a.truth + c * a.ldt;
+  float* dxc = a.dx + c * a.lddx;
+  const int64_t n = VEC ? a.h / 4 : a.h;
+  const unsigned per_class = static_cast<unsigned>(VEC ? a.spatial / 4 : a.spatial);  // < 2^32 (host check)
+  const int64_t step = static_cast<int64_t>(gridDim.y) * kCeThreads;
+  for (int64_t j = static_cast<int64_t>(blockIdx.y) * kCeThreads + threadIdx.x; j < n; j += step) {
+    const unsigned cls = static_cast<unsigned>(j) / per_class;  // j < 2^32 (host check)
+    const unsigned pos = static_cast<unsigned>(j) - cls * per_class;
+    if (VEC) {
+      float t[4], d[4] = {0.f, 0.f, 0.f, 0.f};
+      Vec16<float>::load(tc + 4 * static_cast<int64_t>(pos), t);
+      bool hit[4];
+      bool any = false;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        hit[k] = ce_label(t[k]) == static_cast<int64_t>(cls);
+        any |= hit[k];
+      }
+      if (any) {
+        float v[4];
+        Vec16<float>::load(xc + 4 * j, v);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) d[k] = hit[k] ? -g / v[k] : 0.f;
+      }
+      Vec16<float>::store(dxc + 4 * j, d);
+    }
+    else {
+      dxc[j] = ce_label(tc[pos]) == static_cast<int64_t>(cls) ? -g / xc[j] : 0.f;
+    }
+  }
+}
+
+// Workgroups per column: about 2048 in total, each with at least four units per thread.
+static int ce_parts(int64_t w, int64_t units_per_column)
+{
+  int64_t p = ceil_div(2048, w);
+  const int64_t most = ceil_div(units_per_column, 4 * kCeThreads);
+  if (p > most) p = most;
+  if (p > kCeMaxParts) p = kCeMaxParts;
+  return static_cast<int>(p < 1 ? 1 : p);
+}
+
+static int ce_check(int64_t h, int64_t w, int use_labels, int64_t spatial, int64_t ldx, int64_t ldt)
+{
+  if (h < 0 || w < 0) return LBN_ERR_INVALID_ARGUMENT;
+  if (use_labels && spatial < 1) return LBN_ERR_INVALID_ARGUMENT;
+  if (w > 1 && (ldx < h || ldt < (use_labels ? (spatial < h ? spatial : h) : h))) return LBN_ERR_INVALID_ARGUMENT;
+  if (h >= (int64_t(1) << 32) || w >= (int64_t(1) << 31) || (use_labels && spatial >= (int64_t(1) << 32)))
+    return LBN_ERR_UNSUPPORTED;
+  return LBN_OK;
+}
+
+static bool ce_vec_ok(int64_t h, int64_t w, const void* p, int64_t ld)
+{
+  return h % 4 == 0 && aligned16(p) && (w <= 1 || ld % 4 == 0);
+}
+
+}  // namespace lbn
+
+using namespace lbn;
+
+extern "C" {
+
+size_t lbn_cross_entropy_fwd_workspace_bytes(int64_t height, int64_t width)
+{
+  if (height <= 0 || width <= 0) return 0;
+  return static_cast<size_t>(width) * kCeMaxParts * sizeof(float);
+}
+
+int lbn_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                              int64_t spatial_size, const float* prediction, int64_t ld_prediction,
+                              const float* ground_truth, int64_t ld_ground_truth, float* loss,
+                              int64_t ld_loss, void* workspace, size_t workspace_bytes)
+{
+  if (int e = ce_check(height, width, use_labels, spatial_size, ld_prediction, ld_ground_truth)) return e;
+  if (width == 0) return LBN_OK;
+  if (!loss || ld_loss < 1) return LBN_ERR_INVALID_ARGUMENT;
+  if (height > 0 && (!prediction || !ground_truth)) return LBN_ERR_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  CeArgs a{};
+  a.h = height, a.w = width, a.spatial = use_labels ? spatial_size : 1;
+  a.x = prediction, a.truth = ground_truth, a.ldx = ld_prediction, a.ldt = ld_ground_truth;
+  a.loss = loss, a.ld_loss = ld_loss, a.part = static_cast<float*>(workspace);
+  const bool vec = !use_labels && ce_vec_ok(height, width, prediction, ld_prediction) &&
+                   ce_vec_ok(height, width, ground_truth, ld_ground_truth);
+  const int64_t units = use_labels ? (spatial_size < height ? spatial_size : height) : (vec ? height / 4 : height);
+  const int P = ce_parts(width, units);
+  if (P > 1 && (!workspace || workspace_bytes < static_cast<size_t>(width) * P * sizeof(float) ||
+                (reinterpret_cast<uintptr_t>(workspace) & 3u)))
+    return LBN_ERR_WORKSPACE;
+  const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
+  if (use_labels) hipLaunchKernelGGL(ce_fwd_labels, grid, dim3(kCeThreads), 0, st, a);
+  else if (vec) hipLaunchKernelGGL((ce_fwd_dense<true>), grid, dim3(kCeThreads), 0, st, a);
+  else hipLaunchKernelGGL((ce_fwd_dense<false>), grid, dim3(kCeThreads), 0, st, a);
+  if (P > 1)
+    hipLaunchKernelGGL(ce_merge_parts, dim3(static_cast<unsigned>(width)), dim3(kWave), 0, st, P, a.part, loss,
+                       ld_loss);
+  return launch_status();
+}
+
+int lbn_cross_entropy_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                              int64_t spatial_size, const float* prediction, int64_t ld_prediction,
+                              const float* ground_truth, int64_t ld_ground_truth, const float* dloss,
+                              int64_t ld_dloss, float* dprediction, int64_t ld_dprediction,
+                              float* dground_truth, int64_t ld_dground_truth)
+{
+  if (int e = ce_check(height, width, use_labels, spatial_size, ld_prediction, ld_ground_truth)) return e;
+  if (height == 0 || width == 0) return LBN_OK;
+  if (!prediction || !ground_truth || !dloss || !dprediction || ld_dloss < 1) return LBN_ERR_INVALID_ARGUMENT;
+  if (width > 1 && ld_dprediction < height) return LBN_ERR_INVALID_ARGUMENT;
+  if (!use_labels && (!dground_truth || (width > 1 && ld_dground_truth < height))) return LBN_ERR_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  CeArgs a{};
+  a.h = height, a.w = width, a.spatial = use_labels ? spatial_size : 1;
+  a.x = prediction, a.truth = ground_truth, a.ldx = ld_prediction, a.ldt = ld_ground_truth;
+  a.dy = dloss, a.lddy = ld_dloss, a.dx = dprediction, a.lddx = ld_dprediction;
+  a.dtruth = dground_truth, a.lddt = ld_dground_truth;
+  bool vec = ce_vec_ok(height, width, prediction, ld_prediction) &&
+             ce_vec_ok(height, width, dprediction, ld_dprediction);
+  if (use_labels)
+    vec = vec && spatial_size % 4 == 0 && aligned16(ground_truth) && (width <= 1 || ld_ground_truth % 4 == 0);
+  else
+    vec = vec && ce_vec_ok(height, width, ground_truth, ld_ground_truth) &&
+          ce_vec_ok(height, width, dground_truth, ld_dground_truth);
+  const int P = ce_parts(width, vec ? height / 4 : height);
+  const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
+  if (use_labels) {
+    if (vec) hipLaunchKernelGGL((ce_bwd_labels<true>), grid, dim3(kCeThreads), 0, st, a);
+    else hipLaunchKernelGGL((ce_bwd_labels<false>), grid, dim3(kCeThreads), 0, st, a);
+  }
+  else {
+    if (vec) hipLaunchKernelGGL((ce_bwd_dense<true>), grid, dim3(kCeThreads), 0, st, a);
+    else hipLaunchKernelGGL((ce_bwd_dense<false>), grid, dim3(kCeThreads), 0, st, a);
+  }
+  return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,542 @@
+// Entry-wise and channel-wise scale/bias layers: y = a*x + b with one (a, b) pair per
+// entry of the sample tensor (a matrix row) or per channel (a block of channel_size
+// rows); backward gives dx = a*dy and the weight gradients da = sum(x*dy), db = sum(dy)
+// over everything that shares the pair.
+// Reference CPU code: src/layers/learning/entrywise_scale_bias.cpp:35-60 (forward),
+// :62-113 (backward); src/layers/learning/channelwise_scale_bias.cpp:33-73, :75-135.
+//
+// Both are streaming kernels (forward moves 8 bytes per entry, backward 12); the only
+// structure is where the weight-gradient sums run:
+//  * entry-wise: along the strided direction of the column-major matrix.  A 256-thread
+//    block owns 256/GW rows; consecutive lanes take consecutive row quads (16 bytes),
+//    the 4*GW column groups of the block each walk every (4*GW)-th column of the block's
+//    column slab, and the groups merge their sums by lane exchange and through LDS in a
+//    fixed order.  Short matrices are cut into column slabs (grid.y) so that the launch
+//    still fills the device; the slabs' partial sums go through the workspace and a
+//    second small kernel adds them in slab order.
+//  * channel-wise: along a channel, which is `width` segments of channel_size contiguous
+//    entries.  grid = (channels, P): the P workgroups of a channel stride over its
+//    16-byte vectors, reduce their partial pair, and a one-wave kernel per channel merges
+//    the P pairs in order.
+// Unaligned shapes take scalar variants of the same kernels.  No atomics: results do
+// not depend on scheduling.
+#include "device_utils.hpp"
+#include "host_utils.hpp"
+
+namespace lbn {
+
+constexpr int kSbThreads = 256;
+constexpr int kSbWaves = kSbThreads / kWave;
+constexpr int kSbMaxParts = 64;  // one wave merges the partial pairs of a channel
+
+// ===================================================================== entry-wise
+struct EsbArgs {
+  int64_t h, w;
+  const float* x;
+  const float* dy;
+  float* out;  // y or dx
+  int64_t ldx, lddy, ldo;
+  const float* weights;  // (h x 2): scale, bias
+  int64_t ld_weights;
+  float* wgrad;  // (h x 2)
+  int64_t ld_wgrad;
+  float2* part;  // [slabs][h] partial (da, db) when the columns are cut into slabs
+  int64_t slab_width;
+};
+
+// Thread (row quad q, column group g) of a block; GW column groups share a wave.
+template <int GW>
+struct EsbPos {
+  static constexpr int kQuads = kWave / GW;
+  static constexpr int kRows = 4 * kQuads;
+  static constexpr int kGroups = kSbWaves * GW;
+  int q, g;
+  __device__ __forceinline__ EsbPos()
+  {
+    const int lane = threadIdx.x & (kWave - 1);
+    q = lane & (kQuads - 1);
+    g = lane / kQuads + GW * (threadIdx.x / kWave);
+  }
+};
+
+template <int GW>
+__global__ void __launch_bounds__(kSbThreads)
+esb_fwd_tile(EsbArgs a)
+{
+  using P = EsbPos<GW>;
+  const P p;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * P::kRows + 4 * p.q;
+  if (r0 >= a.h) return;  // h is a multiple of 4
+  const int64_t c0 = static_cast<int64_t>(blockIdx.y) * a.slab_width;
+  const int64_t c1 = imin64(c0 + a.slab_width, a.w);
+  float sc[4], bi[4];
+  Vec16<float>::load(a.weights + r0, sc);
+  Vec16<float>::load(a.weights + r0 + a.ld_weights, bi);
+  int64_t c = c0 + p.g;
+  for (; c + 3 * P::kGroups < c1; c += 4 * P::kGroups) {
+    float v[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) Vec16<float>::load(a.x + r0 + (c + j * P::kGroups) * a.ldx, v[j]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[j][r] = sc[r] * v[j][r] + bi[r];
+      Vec16<float>::store(a.out + r0 + (c + j * P::kGroups) * a.ldo, v[j]);
+    }
+  }
+  for (; c < c1; c += P::kGroups) {
+    float v[4];
+    Vec16<float>::load(a.x + r0 + c * a.ldx, v);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) v[r] = sc[r] * v[r] + bi[r];
+    Vec16<float>::store(a.out + r0 + c * a.ldo, v);
+  }
+}
+
+template <int GW>
+__global__ void __launch_bounds__(kSbThreads)
+esb_bwd_tile(EsbArgs a)
+{
+  using P = EsbPos<GW>;
+  __shared__ float lds[kSbWaves][P::kRows][2];
+  const P p;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * P::kRows + 4 * p.q;
+  const bool row_ok = r0 < a.h;
+  const int64_t c0 = static_cast<int64_t>(blockIdx.y) * a.slab_width;
+  const int64_t c1 = row_ok ? imin64(c0 + a.slab_width, a.w) : 0;
+  const int64_t rr = row_ok ? r0 : 0;
+  float sc[4];
+  Vec16<float>::load(a.weights + rr, sc);
+  float da[4] = {0.f, 0.f, 0.f, 0.f}, db[4] = {0.f, 0.f, 0.f, 0.f};
+  int64_t c = c0 + p.g;
+  for (; c + P::kGroups < c1; c += 2 * P::kGroups) {
+    float v[2][4], g[2][4];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      Vec16<float>::load(a.x + rr + (c + j * P::kGroups) * a.ldx, v[j]);
+      Vec16<float>::load(a.dy + rr + (c + j * P::kGroups) * a.lddy, g[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      float d[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        da[r] = __builtin_fmaf(v[j][r], g[j][r], da[r]);
+        db[r] += g[j][r];
+        d[r] = sc[r] * g[j][r];
+      }
+      Vec16<float>::store(a.out + rr + (c + j * P::kGroups) * a.ldo, d);
+    }
+  }
+  for (; c < c1; c += P::kGroups) {
+    float v[4], g[4], d[4];
+    Vec16<float>::load(a.x + rr + c * a.ldx, v);
+    Vec16<float>::load(a.dy + rr + c * a.lddy, g);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      da[r] = __builtin_fmaf(v[r], g[r], da[r]);
+      db[r] += g[r];
+      d[r] = sc[r] * g[r];
+    }
+    Vec16<float>::store(a.out + rr + c * a.ldo, d);
+  }
+  // merge the column groups: inside a wave by lane exchange, across waves through LDS
+  if (GW == 4) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      da[r] += __shfl_xor(da[r], 16);
+      db[r] += __shfl_xor(db[r], 16);
+      da[r] += __shfl_xor(da[r], 32);
+      db[r] += __shfl_xor(db[r], 32);
+    }
+  }
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  if (lane < P::kQuads) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      lds[wave][4 * p.q + r][0] = da[r];
+      lds[wave][4 * p.q + r][1] = db[r];
+    }
+  }
+  __syncthreads();
+  if (p.g != 0 || !row_ok) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float sa = 0.f, sb = 0.f;
+#pragma unroll
+    for (int k = 0; k < kSbWaves; ++k) {
+      sa += lds[k][4 * p.q + r][0];
+      sb += lds[k][4 * p.q + r][1];
+    }
+    da[r] = sa;
+    db[r] = sb;
+  }
+  if (gridDim.y == 1) {
+    Vec16<float>::store(a.wgrad + r0, da);
+    Vec16<float>::store(a.wgrad + r0 + a.ld_wgrad, db);
+  }
+  else {
+    float2* dst = a.part + static_cast<int64_t>(blockIdx.y) * a.h + r0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) dst[r] = make_float2(da[r], db[r]);
+  }
+}
+
+// Adds the slabs' partial pairs of every row in slab order.
+__global__ void __launch_bounds__(256)
+esb_merge_slabs(int64_t h, int slabs, const float2* __restrict__ part, float* __restrict__ wgrad,
+                int64_t ld_wgrad)
+{
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (r >= h) return;
+  float sa = 0.f, sb = 0.f;
+  for (int s = 0; s < slabs; ++s) {
+    const float2 v = part[static_cast<int64_t>(s) * h + r];
+    sa += v.x;
+    sb += v.y;
+  }
+  wgrad[r] = sa;
+  wgrad[r + ld_wgrad] = sb;
+}
+
+// One thread per row, scalar and coalesced: any shape and alignment.
+__global__ void __launch_bounds__(256)
+esb_fwd_generic(EsbArgs a)
+{
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (r >= a.h) return;
+  const float sc = a.weights[r], bi = a.weights[r + a.ld_weights];
+  const int64_t c0 = static_cast<int64_t>(blockIdx.y) * a.slab_width;
+  const int64_t c1 = imin64(c0 + a.slab_width, a.w);
+  for (int64_t c = c0; c < c1; ++c) a.out[r + c * a.ldo] = sc * a.x[r + c * a.ldx] + bi;
+}
+
+__global__ void __launch_bounds__(256)
+esb_bwd_generic(EsbArgs a)
+{
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (r >= a.h) return;
+  const float sc = a.weights[r];
+  float da = 0.f, db = 0.f;
+  for (int64_t c = 0; c < a.w; ++c) {
+    const float g = a.dy[r + c * a.lddy];
+    da = __builtin_fmaf(a.x[r + c * a.ldx], g, da);
+    db += g;
+    a.out[r + c * a.ldo] = sc * g;
+  }
+  a.wgrad[r] = da;
+  a.wgrad[r + a.ld_wgrad] = db;
+}
+
+// Column slabs for a launch of `row_tiles` workgroups per slab: enough slabs to give the
+// device about four workgroups per compute unit, each slab at least `min_width` wide.
+static int esb_slabs(int64_t row_tiles, int64_t w, int64_t min_width)
+{
+  const int64_t want = ceil_div(1024, row_tiles);
+  const int64_t most = w / min_width > 1 ? w / min_width : 1;
+  int64_t s = want < most ? want : most;
+  if (s > kSbMaxParts) s = kSbMaxParts;
+  return static_cast<int>(s < 1 ? 1 : s);
+}
+
+static bool sb_vec_ok(int64_t h, int64_t w, const void* p, int64_t ld)
+{
+  return h % 4 == 0 && aligned16(p) && (w <= 1 || ld % 4 == 0);
+}
+
+static int sb_check(int64_t h, int64_t w, const int64_t* lds, int nld)
+{
+  if (h < 0 || w < 0) return LBN_ERR_INVALID_ARGUMENT;
+  for (int i = 0; i < nld; ++i)
+    if (w > 1 && lds[i] < h) return LBN_ERR_INVALID_ARGUMENT;
+  if (h > (int64_t(1) << 40) || w > (int64_t(1) << 40)) return LBN_ERR_UNSUPPORTED;
+  return LBN_OK;
+}
+
+// Launch shape of the tile kernels.  Sixteen column groups over 64 rows (GW = 4) measured
+// 4-8 % faster than four groups over 256 rows on 1048576 x 64 and 802816 x 64 matrices;
+// mini-batches narrower than 16 columns would leave most of those groups idle and take
+// GW = 1.
+struct EsbPlan {
+  int gw;
+  int64_t tiles;
+  int slabs;
+  int64_t slab_width;
+};
+
+static EsbPlan esb_plan(int64_t h, int64_t w)
+{
+  EsbPlan p;
+  p.gw = w >= 16 ? 4 : 1;
+  p.tiles = ceil_div(h, p.gw == 1 ? EsbPos<1>::kRows : EsbPos<4>::kRows);
+  p.slab_width = ceil_div(w, esb_slabs(p.tiles, w, 4 * kSbWaves * p.gw));
+  p.slabs = static_cast<int>(ceil_div(w, p.slab_width));
+  return p;
+}
+
+// =================================================================== channel-wise
+struct CsbArgs {
+  int64_t cs, w;
+  const float* x;
+  const float* dy;
+  float* out;
+  int64_t ldx, lddy, ldo;
+  const float* weights;  // (C x 2)
+  int64_t ld_weights;
+  float* wgrad;
+  int64_t ld_wgrad;
+  float2* part;  // [C][P]
+};
+
+template <bool VEC>
+__global__ void __launch_bounds__(kSbThreads)
+csb_fwd(CsbArgs a)
+{
+  const int64_t ch = blockIdx.x;
+  const float sc = a.weights[ch], bi = a.weights[ch + a.ld_weights];
+  const float* xc = a.x + ch * a.cs;
+  float* yc = a.out + ch * a.cs;
+  const int64_t seg = VEC ? a.cs / 4 : a.cs;
+  const int64_t total = seg * a.w;
+  const int64_t step = static_cast<int64_t>(gridDim.y) * kSbThreads;
+  for (int64_t j = static_cast<int64_t>(blockIdx.y) * kSbThreads + threadIdx.x; j < total; j += step) {
+    const unsigned ucol = static_cast<unsigned>(j) / static_cast<unsigned>(seg);  // j < 2^32 (host check)
+    const int64_t col = ucol;
+    const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(seg);
+    if (VEC) {
+      float v[4];
+      Vec16<float>::load(xc + col * a.ldx + 4 * i, v);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = sc * v[k] + bi;
+      Vec16<float>::store(yc + col * a.ldo + 4 * i, v);
+    }
+    else {
+      yc[col * a.ldo + i] = sc * xc[col * a.ldx + i] + bi;
+    }
+  }
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(kSbThreads)
+csb_bwd(CsbArgs a)
+{
+  __shared__ float red[2 * kSbWaves];
+  const int64_t ch = blockIdx.x;
+  const float sc = a.weights[ch];
+  const float* xc = a.x + ch * a.cs;
+  const float* gc = a.dy + ch * a.cs;
+  float* dc = a.out + ch * a.cs;
+  const int64_t seg = VEC ? a.cs / 4 : a.cs;
+  const int64_t total = seg * a.w;
+  const int64_t step = static_cast<int64_t>(gridDim.y) * kSbThreads;
+  float da = 0.f, db = 0.f;
+  for (int64_t j = static_cast<int64_t>(blockIdx.y) * kSbThreads + threadIdx.x; j < total; j += step) {
+    const unsigned ucol = static_cast<unsigned>(j) / static_cast<unsigned>(seg);
+    const int64_t col = ucol;
+    const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(seg);
+    if (VEC) {
+      float v[4], g[4], d[4];
+      Vec16<float>::load(xc + col * a.ldx + 4 * i, v);
+      Vec16<float>::load(gc + col * a.lddy + 4 * i, g);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        da = __builtin_fmaf(v[k], g[k], da);
+        db += g[k];
+        d[k] = sc * g[k];
+      }
+      Vec16<float>::store(dc + col * a.ldo + 4 * i, d);
+    }
+    else {
+      const float g = gc[col * a.lddy + i];
+      da = __builtin_fmaf(xc[col * a.ldx + i], g, da);
+      db += g;
+      dc[col * a.ldo + i] = sc * g;
+    }
+  }
+  team_sum2<kSbWaves>(da, db, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+  if (threadIdx.x == 0) {
+    if (gridDim.y == 1) {
+      a.wgrad[ch] = da;
+      a.wgrad[ch + a.ld_wgrad] = db;
+    }
+    else {
+      a.part[ch * gridDim.y + blockIdx.y] = make_float2(da, db);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(kWave)
+csb_merge_parts(int P, const float2* __restrict__ part, float* __restrict__ wgrad, int64_t ld_wgrad)
+{
+  const int64_t ch = blockIdx.x;
+  const int lane = threadIdx.x;
+  float a = 0.f, b = 0.f;
+  if (lane < P) {
+    const float2 v = part[ch * P + lane];
+    a = v.x;
+    b = v.y;
+  }
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if (lane == 0) {
+    wgrad[ch] = a;
+    wgrad[ch + ld_wgrad] = b;
+  }
+}
+
+// Workgroups per channel: about 2048 in total, each with at least four vectors per thread.
+static int csb_parts(int64_t C, int64_t vectors_per_channel)
+{
+  int64_t p = ceil_div(2048, C);
+  const int64_t most = ceil_div(vectors_per_channel, 4 * kSbThreads);
+  if (p > most) p = most;
+  if (p > kSbMaxParts) p = kSbMaxParts;
+  return static_cast<int>(p < 1 ? 1 : p);
+}
+
+static int csb_check(int64_t C, int64_t cs, int64_t w, const int64_t* lds, int nld)
+{
+  if (C < 0 || cs < 0 || w < 0) return LBN_ERR_INVALID_ARGUMENT;
+  if (C > 0 && cs > (int64_t(1) << 40) / C) return LBN_ERR_UNSUPPORTED;
+  for (int i = 0; i < nld; ++i)
+    if (w > 1 && lds[i] < C * cs) return LBN_ERR_INVALID_ARGUMENT;
+  if (C >= (int64_t(1) << 31) || cs * w >= (int64_t(1) << 32)) return LBN_ERR_UNSUPPORTED;
+  return LBN_OK;
+}
+
+static bool csb_vec_ok(int64_t cs, int64_t w, const void* p, int64_t ld)
+{
+  return cs % 4 == 0 && aligned16(p) && (w <= 1 || ld % 4 == 0);
+}
+
+}  // namespace lbn
+
+using namespace lbn;
+
+extern "C" {
+
+int lbn_entrywise_scale_bias_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* x,
+                                     int64_t ldx, float* y, int64_t ldy, const float* weights,
+                                     int64_t ld_weights)
+{
+  const int64_t lds[2] = {ldx, ldy};
+  if (int e = sb_check(height, width, lds, 2)) return e;
+  if (height == 0 || width == 0) return LBN_OK;
+  if (!x || !y || !weights || ld_weights < height) return LBN_ERR_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  EsbArgs a{height, width, x, nullptr, y, ldx, 0, ldy, weights, ld_weights, nullptr, 0, nullptr, width};
+  if (sb_vec_ok(height, width, x, ldx) && sb_vec_ok(height, width, y, ldy) && aligned16(weights) &&
+      ld_weights % 4 == 0) {
+    const EsbPlan p = esb_plan(height, width);
+    a.slab_width = p.slab_width;
+    const dim3 grid(static_cast<unsigned>(p.tiles), static_cast<unsigned>(p.slabs));
+    if (p.gw == 1) hipLaunchKernelGGL((esb_fwd_tile<1>), grid, dim3(kSbThreads), 0, st, a);
+    else hipLaunchKernelGGL((esb_fwd_tile<4>), grid, dim3(kSbThreads), 0, st, a);
+    return launch_status();
+  }
+  const int64_t tiles = ceil_div(height, 256);
+  a.slab_width = ceil_div(width, esb_slabs(tiles, width, 8));
+  const dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(ceil_div(width, a.slab_width)));
+  hipLaunchKernelGGL(esb_fwd_generic, grid, dim3(256), 0, st, a);
+  return launch_status();
+}
+
+size_t lbn_entrywise_scale_bias_bwd_workspace_bytes(int64_t height, int64_t width)
+{
+  if (height <= 0 || width <= 0) return 0;
+  const EsbPlan p = esb_plan(height, width);
+  return p.slabs > 1 ? static_cast<size_t>(p.slabs) * static_cast<size_t>(height) * sizeof(float2) : 0;
+}
+
+int lbn_entrywise_scale_bias_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* x,
+                                     int64_t ldx, const float* dy, int64_t lddy, float* dx,
+                                     int64_t lddx, const float* weights, int64_t ld_weights,
+                                     float* weights_grad, int64_t ld_weights_grad, void* workspace,
+                                     size_t workspace_bytes)
+{
+  const int64_t lds[3] = {ldx, lddy, lddx};
+  if (int e = sb_check(height, width, lds, 3)) return e;
+  if (height == 0 || width == 0) return LBN_OK;
+  if (!x || !dy || !dx || !weights || !weights_grad || ld_weights < height || ld_weights_grad < height)
+    return LBN_ERR_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  EsbArgs a{height, width, x, dy, dx, ldx, lddy, lddx, weights, ld_weights, weights_grad, ld_weights_grad,
+            static_cast<float2*>(workspace), width};
+  if (sb_vec_ok(height, width, x, ldx) && sb_vec_ok(height, width, dy, lddy) &&
+      sb_vec_ok(height, width, dx, lddx) && aligned16(weights) && aligned16(weights_grad) &&
+      ld_weights_grad % 4 == 0) {
+    const EsbPlan p = esb_plan(height, width);
+    const int slabs = p.slabs;
+    a.slab_width = p.slab_width;
+    if (slabs > 1 && (!workspace || !aligned16(workspace) ||
+                      workspace_bytes < static_cast<size_t>(slabs) * height * sizeof(float2)))
+      return LBN_ERR_WORKSPACE;
+    const dim3 grid(static_cast<unsigned>(p.tiles), static_cast<unsigned>(slabs));
+    if (p.gw == 1) hipLaunchKernelGGL((esb_bwd_tile<1>), grid, dim3(kSbThreads), 0, st, a);
+    else hipLaunchKernelGGL((esb_bwd_tile<4>), grid, dim3(kSbThreads), 0, st, a);
+    if (slabs > 1)
+      hipLaunchKernelGGL(esb_merge_slabs, dim3(static_cast<unsigned>(ceil_div(height, 256))), dim3(256), 0,
+                         st, height, slabs, a.part, weights_grad, ld_weights_grad);
+    return launch_status();
+  }
+  hipLaunchKernelGGL(esb_bwd_generic, dim3(static_cast<unsigned>(ceil_div(height, 256))), dim3(256), 0, st, a);
+  return launch_status();
+}
+
+int lbn_channelwise_scale_bias_fwd_f32(lbn_stream_t stream, int64_t num_channels, int64_t channel_size,
+                                       int64_t width, const float* x, int64_t ldx, float* y,
+                                       int64_t ldy, const float* weights, int64_t ld_weights)
+{
+  const int64_t lds[2] = {ldx, ldy};
+  if (int e = csb_check(num_channels, channel_size, width, lds, 2)) return e;
+  if (num_channels == 0 || channel_size == 0 || width == 0) return LBN_OK;
+  if (!x || !y || !weights || ld_weights < num_channels) return LBN_ERR_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  const CsbArgs a{channel_size, width, x, nullptr, y, ldx, 0, ldy, weights, ld_weights, nullptr, 0, nullptr};
+  const bool vec = csb_vec_ok(channel_size, width, x, ldx) && csb_vec_ok(channel_size, width, y, ldy);
+  const int P = csb_parts(num_channels, (vec ? channel_size / 4 : channel_size) * width);
+  const dim3 grid(static_cast<unsigned>(num_channels), static_cast<unsigned>(P));
+  if (vec) hipLaunchKernelGGL((csb_fwd<true>), grid, dim3(kSbThreads), 0, st, a);
+  else hipLaunchKernelGGL((csb_fwd<false>), grid, dim3(kSbThreads), 0, st, a);
+  return launch_status();
+}
+
+size_t lbn_channelwise_scale_bias_bwd_workspace_bytes(int64_t num_channels, int64_t channel_size,
+                                                      int64_t width)
+{
+  if (num_channels <= 0 || channel_size <= 0 || width <= 0) return 0;
+  return static_cast<size_t>(num_channels) * kSbMaxParts * sizeof(float2);
+}
+
+int lbn_channelwise_scale_bias_bwd_f32(lbn_stream_t stream, int64_t num_channels, int64_t channel_size,
+                                       int64_t width, const float* x, int64_t ldx, const float* dy,
+                                       int64_t lddy, float* dx, int64_t lddx, const float* weights,
+                                       int64_t ld_weights, float* weights_grad, int64_t ld_weights_grad,
+                                       void* workspace, size_t workspace_bytes)
+{
+  const int64_t lds[3] = {ldx, lddy, lddx};
+  if (int e = csb_check(num_channels, channel_size, width, lds, 3)) return e;
+  if (num_channels == 0 || channel_size == 0 || width == 0) return LBN_OK;
+  if (!x || !dy || !dx || !weights || !weights_grad || ld_weights < num_channels ||
+      ld_weights_grad < num_channels)
+    return LBN_ERR_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  const bool vec = csb_vec_ok(channel_size, width, x, ldx) && csb_vec_ok(channel_size, width, dy, lddy) &&
+                   csb_vec_ok(channel_size, width, dx, lddx);
+  const int P = csb_parts(num_channels, (vec ? channel_size / 4 : channel_size) * width);
+  if (P > 1 && (!workspace || workspace_bytes < static_cast<size_t>(num_channels) * P * sizeof(float2) ||
+                (reinterpret_cast<uintptr_t>(workspace) & 7u)))
+    return LBN_ERR_WORKSPACE;
+  const CsbArgs a{channel_size, width, x, dy, dx, ldx, lddy, lddx, weights, ld_weights, weights_grad,
+                  ld_weights_grad, static_cast<float2*>(workspace)};
+  const dim3 grid(static_cast<unsigned>(num_channels), static_cast<unsigned>(P));
+  if (vec) hipLaunchKernelGGL((csb_bwd<true>), grid, dim3(kSbThreads), 0, st, a);
+  else hipLaunchKernelGGL((csb_bwd<false>), grid, dim3(kSbThreads), 0, st, a);
+  if (P > 1)
+    hipLaunchKernelGGL(csb_merge_parts, dim3(static_cast<unsigned>(num_channels)), dim3(kWave), 0, st, P,
+                       a.part, weights_grad, ld_weights_grad);
+  return launch_status();
+}
+
+}  // extern "C"

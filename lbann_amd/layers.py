@@ -416,3 +416,129 @@ class channelwise_softmax_layer(_Layer):
         return ("lbn_channelwise_softmax_bwd_f32",
                 (_stream(), C, cs, stride, y.width, y.Buffer(), y.ldim, dy.Buffer(), dy.ldim, dx.Buffer(),
                  dx.ldim, ws, nb))
+
+
+class _scale_bias_layer(_Layer):
+    """Shared state of the two scale/bias layers: one weights matrix (n x 2), column 0 scale
+    (default 1), column 1 bias (default 0), and m_weights_gradient of the same shape."""
+
+    def _setup_weights(self, n, device):
+        self.weights = DeviceMatrix(n, 2, device=device)
+        self.weights.tensor[0].fill_(1.0)
+        self.weights.tensor[1].fill_(0.0)
+        self.m_weights_gradient = DeviceMatrix(n, 2, device=device)
+
+    def set_weights(self, scale, bias):
+        n = self.weights.height
+        self.weights.tensor[0, :n] = torch.as_tensor(np.asarray(scale, np.float32).reshape(-1)).to(self.device)
+        self.weights.tensor[1, :n] = torch.as_tensor(np.asarray(bias, np.float32).reshape(-1)).to(self.device)
+
+
+class entrywise_scale_bias_layer(_scale_bias_layer):
+    """lbann::entrywise_scale_bias_layer (include/lbann/layers/learning/entrywise_scale_bias.hpp:57-203)."""
+
+    def __init__(self, dims, device="cuda"):
+        super().__init__(device)
+        self.dims = tuple(int(d) for d in dims)
+        self._setup_weights(_prod(self.dims), device)
+
+    def fp_call(self):
+        x, y, wt = self.prev_activations, self.activations, self.weights
+        return ("lbn_entrywise_scale_bias_fwd_f32",
+                (_stream(), x.height, x.width, x.Buffer(), x.ldim, y.Buffer(), y.ldim, wt.Buffer(), wt.ldim))
+
+    def bp_call(self):
+        x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
+        wt, wg = self.weights, self.m_weights_gradient
+        ws, nb = self._ws.get(capi.lib().lbn_entrywise_scale_bias_bwd_workspace_bytes(x.height, x.width),
+                              self.device)
+        return ("lbn_entrywise_scale_bias_bwd_f32",
+                (_stream(), x.height, x.width, x.Buffer(), x.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim,
+                 wt.Buffer(), wt.ldim, wg.Buffer(), wg.ldim, ws, nb))
+
+
+class channelwise_scale_bias_layer(_scale_bias_layer):
+    """lbann::channelwise_scale_bias_layer (include/lbann/layers/learning/channelwise_scale_bias.hpp:60-206)."""
+
+    def __init__(self, dims, device="cuda"):
+        super().__init__(device)
+        self.dims = tuple(int(d) for d in dims)
+        self.num_channels = self.dims[0]
+        self.channel_size = _prod(self.dims[1:])
+        self._setup_weights(self.num_channels, device)
+
+    def fp_call(self):
+        x, y, wt = self.prev_activations, self.activations, self.weights
+        return ("lbn_channelwise_scale_bias_fwd_f32",
+                (_stream(), self.num_channels, self.channel_size, x.width, x.Buffer(), x.ldim, y.Buffer(), y.ldim,
+                 wt.Buffer(), wt.ldim))
+
+    def bp_call(self):
+        x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
+        wt, wg = self.weights, self.m_weights_gradient
+        C, cs = self.num_channels, self.channel_size
+        ws, nb = self._ws.get(capi.lib().lbn_channelwise_scale_bias_bwd_workspace_bytes(C, cs, x.width), self.device)
+        return ("lbn_channelwise_scale_bias_bwd_f32",
+                (_stream(), C, cs, x.width, x.Buffer(), x.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim,
+                 wt.Buffer(), wt.ldim, wg.Buffer(), wg.ldim, ws, nb))
+
+
+class cross_entropy_layer:
+    """lbann::cross_entropy_layer (include/lbann/layers/loss/cross_entropy.hpp:75-190): two
+    parents (prediction, ground truth), output of dims {1}.  `dims` are the prediction's
+    dimensions; with use_labels the ground truth has dims (1, dims[1:]) and holds class
+    indices (cross_entropy_impl.hpp:59-133)."""
+
+    def __init__(self, dims, use_labels=False, device="cuda"):
+        self.device = device
+        self.dims = tuple(int(d) for d in dims)
+        self.m_use_labels = bool(use_labels)
+        if self.m_use_labels and len(self.dims) < 2:
+            raise ValueError("cross entropy layer expects both input tensors to have the same number of "
+                             "dimensions and have >2 dimensions when use_labels is enabled.")
+        self.spatial_sample_size = _prod(self.dims[1:])
+        self.prev_activations = [None, None]
+        self.activations = None
+        self.prev_error_signals = None
+        self.error_signals = [None, None]
+        self._ws = _Workspace()
+
+    def fp_call(self):
+        x, t, y = self.prev_activations[0], self.prev_activations[1], self.activations
+        ws, nb = self._ws.get(capi.lib().lbn_cross_entropy_fwd_workspace_bytes(x.height, x.width), self.device)
+        return ("lbn_cross_entropy_fwd_f32",
+                (_stream(), x.height, x.width, int(self.m_use_labels), self.spatial_sample_size, x.Buffer(), x.ldim,
+                 t.Buffer(), t.ldim, y.Buffer(), y.ldim, ws, nb))
+
+    def bp_call(self):
+        x, t, dy = self.prev_activations[0], self.prev_activations[1], self.prev_error_signals
+        dx, dt = self.error_signals
+        return ("lbn_cross_entropy_bwd_f32",
+                (_stream(), x.height, x.width, int(self.m_use_labels), self.spatial_sample_size, x.Buffer(), x.ldim,
+                 t.Buffer(), t.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim,
+                 dt.Buffer() if dt is not None else _null(), dt.ldim if dt is not None else 0))
+
+    def fp_compute(self):
+        name, args = self.fp_call()
+        call(name, *args)
+
+    def bp_compute(self):
+        name, args = self.bp_call()
+        call(name, *args)
+
+    def forward(self, prediction, ground_truth):
+        self.prev_activations = [prediction, ground_truth]
+        self.activations = DeviceMatrix(1, prediction.width, device=self.device)
+        self.fp_compute()
+        return self.activations
+
+    def backward(self, dy):
+        """dy: (1 x width) gradient w.r.t. the loss.  Returns [dL/dprediction, dL/dground_truth];
+        the second is None with use_labels (the reference leaves that error signal untouched)."""
+        x, t = self.prev_activations
+        self.prev_error_signals = dy
+        self.error_signals = [DeviceMatrix(x.height, x.width, ldim=x.ldim, device=self.device),
+                              None if self.m_use_labels else DeviceMatrix(t.height, t.width, ldim=t.ldim,
+                                                                          device=self.device)]
+        self.bp_compute()
+        return self.error_signals

@@ -226,3 +226,73 @@ def entrywise_batch_norm_bwd(x, dy, stats, eps, running_var=None, training=True)
         _i64(h), _i64(w), cf(eps), ctypes.c_int(int(training)), *_mat(x), *_mat(dy), *_mat(dx),
         *_mat(stats), *_mat(sgrad), _vec(running_var))
     return dx, sgrad
+
+
+# --------------------------------------------------------------- cross entropy
+def cross_entropy_fwd(x, truth, use_labels=False):
+    """Returns the (w,) loss.  With use_labels, truth is (spatial x w) class indices stored
+    as floating point and x is (classes*spatial x w)."""
+    suf, _ = _suffix(x)
+    h, w = x.shape
+    spatial = truth.shape[0] if use_labels else 1
+    loss = np.zeros(w, dtype=x.dtype)
+    getattr(lib(), f"orc_cross_entropy_fwd_{suf}")(
+        _i64(h), _i64(w), ctypes.c_int(int(use_labels)), _i64(spatial), *_mat(x), *_mat(truth), _vec(loss))
+    return loss
+
+
+def cross_entropy_bwd(x, truth, dy, use_labels=False):
+    """dy is the (w,) gradient w.r.t. the loss.  Returns (dx, dtruth); dtruth is None with
+    use_labels (the reference leaves it untouched)."""
+    suf, _ = _suffix(x)
+    h, w = x.shape
+    spatial = truth.shape[0] if use_labels else 1
+    dx = fmat(h, w, x.dtype)
+    dtruth = fmat(h, w, x.dtype)
+    dy = np.ascontiguousarray(dy, dtype=x.dtype)
+    getattr(lib(), f"orc_cross_entropy_bwd_{suf}")(
+        _i64(h), _i64(w), ctypes.c_int(int(use_labels)), _i64(spatial), *_mat(x), *_mat(truth), _vec(dy),
+        *_mat(dx), *_mat(dtruth))
+    return dx, (None if use_labels else dtruth)
+
+
+# ------------------------------------------------------------ scale/bias layers
+def entrywise_scale_bias_fwd(x, weights):
+    """weights is (h x 2): column 0 scale, column 1 bias."""
+    suf, _ = _suffix(x)
+    h, w = x.shape
+    y = fmat(h, w, x.dtype)
+    getattr(lib(), f"orc_entrywise_scale_bias_fwd_{suf}")(_i64(h), _i64(w), *_mat(x), *_mat(y), *_mat(weights))
+    return y
+
+
+def entrywise_scale_bias_bwd(x, dy, weights):
+    """Returns (dx, weights_grad) with weights_grad (h x 2)."""
+    suf, _ = _suffix(x)
+    h, w = x.shape
+    dx = fmat(h, w, x.dtype)
+    wgrad = np.zeros((h, 2), dtype=x.dtype, order="F")
+    getattr(lib(), f"orc_entrywise_scale_bias_bwd_{suf}")(
+        _i64(h), _i64(w), *_mat(x), *_mat(dy), *_mat(dx), *_mat(weights), *_mat(wgrad))
+    return dx, wgrad
+
+
+def channelwise_scale_bias_fwd(x, weights, C, cs):
+    """weights is (C x 2): column 0 scale, column 1 bias."""
+    suf, _ = _suffix(x)
+    h, w = x.shape
+    y = fmat(h, w, x.dtype)
+    getattr(lib(), f"orc_channelwise_scale_bias_fwd_{suf}")(
+        _i64(C), _i64(cs), _i64(w), *_mat(x), *_mat(y), *_mat(weights))
+    return y
+
+
+def channelwise_scale_bias_bwd(x, dy, weights, C, cs):
+    """Returns (dx, weights_grad) with weights_grad (C x 2)."""
+    suf, _ = _suffix(x)
+    h, w = x.shape
+    dx = fmat(h, w, x.dtype)
+    wgrad = np.zeros((C, 2), dtype=x.dtype, order="F")
+    getattr(lib(), f"orc_channelwise_scale_bias_bwd_{suf}")(
+        _i64(C), _i64(cs), _i64(w), *_mat(x), *_mat(dy), *_mat(dx), *_mat(weights), *_mat(wgrad))
+    return dx, wgrad

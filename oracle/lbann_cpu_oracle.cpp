@@ -1,5 +1,6 @@
 // CPU oracle: a restatement of LBANN's CPU (OpenMP) implementation of the
-// forward/backward compute of five layers.  TEST INFRASTRUCTURE ONLY: this file
+// forward/backward compute of the normalization, softmax and neighbouring layers
+// listed below.  TEST INFRASTRUCTURE ONLY: this file
 // is the checker that the HIP kernels are compared against and the timed CPU
 // baseline of the benchmark; nothing in the product path may call it.
 //
@@ -28,6 +29,9 @@
 //   instance norm   src/layers/regularizers/instance_norm.cpp:47-113 (fwd), :137-231 (bwd)
 //   entry-wise bn   src/layers/regularizers/entrywise_batch_normalization.cpp:52-202 (fwd),
 //                   :210-414 (bwd)
+//   cross entropy   src/layers/loss/cross_entropy.cpp:35-73 (fwd), :75-120 (bwd)
+//   entry-wise scale/bias    src/layers/learning/entrywise_scale_bias.cpp:35-60, :62-113
+//   channel-wise scale/bias  src/layers/learning/channelwise_scale_bias.cpp:33-73, :75-135
 
 #include <algorithm>
 #include <cmath>
@@ -673,6 +677,126 @@ void ebn_bwd(idx h, idx w, T eps, int training, CMat<T> x, CMat<T> dy, Mat<T> dx
   }
 }
 
+// ----------------------------------------------------------- cross entropy
+// cross_entropy.cpp:35-73 (local_fp_cpu).  loss(0,c) = sum over rows with xhat > 0 of
+// -xhat*log(x), accumulated in row order.  With use_labels the ground truth holds one
+// class index per spatial position (rows [0,spatial) of truth) and
+// xhat(row) = (truth(row % spatial) == row / spatial).
+template <typename T>
+void ce_fwd(idx h, idx w, int use_labels, idx spatial, CMat<T> x, CMat<T> truth, T* loss)
+{
+#pragma omp parallel for
+  for (idx c = 0; c < w; ++c) {
+    T sum = T(0);
+    for (idx r = 0; r < h; ++r) {
+      T xhat;
+      if (use_labels) {
+        const idx channel = r / spatial;
+        const idx offset = r % spatial;
+        const int label = static_cast<int>(truth(offset, c));
+        xhat = T(label == channel ? 1. : 0.);
+      }
+      else {
+        xhat = truth(r, c);
+      }
+      if (xhat > T(0)) sum += -xhat * std::log(x(r, c));
+    }
+    loss[c] = sum;
+  }
+}
+
+// cross_entropy.cpp:75-120 (local_bp_cpu).  dy is the (1 x w) gradient w.r.t. the loss.
+// dtruth is written only without use_labels.
+template <typename T>
+void ce_bwd(idx h, idx w, int use_labels, idx spatial, CMat<T> x, CMat<T> truth, const T* dy,
+            Mat<T> dx, Mat<T> dtruth)
+{
+#pragma omp parallel for collapse(2)
+  for (idx c = 0; c < w; ++c) {
+    for (idx r = 0; r < h; ++r) {
+      const T g = dy[c];
+      const T v = x(r, c);
+      T xhat;
+      if (use_labels) {
+        const idx channel = r / spatial;
+        const idx offset = r % spatial;
+        const int label = static_cast<int>(truth(offset, c));
+        xhat = T(label == channel ? 1. : 0.);
+      }
+      else {
+        xhat = truth(r, c);
+        dtruth(r, c) = -g * std::log(v);
+      }
+      dx(r, c) = (xhat > T(0)) ? -g * xhat / v : T(0);
+    }
+  }
+}
+
+// ----------------------------------------------------- entry-wise scale/bias
+// entrywise_scale_bias.cpp:35-60 (fp_impl), :62-113 (bp_impl).  weights is (h x 2):
+// column 0 scale, column 1 bias; wgrad likewise.  Row sums accumulate over ascending
+// columns (rows are walked in blocks of one cache line, the column loop outside).
+template <typename T>
+void esb_fwd(idx h, idx w, CMat<T> x, Mat<T> y, CMat<T> weights)
+{
+#pragma omp parallel for collapse(2)
+  for (idx c = 0; c < w; ++c)
+    for (idx r = 0; r < h; ++r) y(r, c) = weights(r, 0) * x(r, c) + weights(r, 1);
+}
+
+template <typename T>
+void esb_bwd(idx h, idx w, CMat<T> x, CMat<T> dy, Mat<T> dx, CMat<T> weights, Mat<T> wgrad)
+{
+  for (idx r = 0; r < h; ++r) wgrad(r, 0) = wgrad(r, 1) = T(0);
+  const idx bsize = std::max<idx>(64 / static_cast<idx>(sizeof(float)), 1);  // DataType is float
+#pragma omp parallel for
+  for (idx r0 = 0; r0 < h; r0 += bsize) {
+    const idx r1 = std::min(r0 + bsize, h);
+    for (idx c = 0; c < w; ++c)
+      for (idx r = r0; r < r1; ++r) {
+        const T g = dy(r, c);
+        dx(r, c) = weights(r, 0) * g;
+        wgrad(r, 0) += x(r, c) * g;
+        wgrad(r, 1) += g;
+      }
+  }
+}
+
+// --------------------------------------------------- channel-wise scale/bias
+// channelwise_scale_bias.cpp:33-73 (fp_compute), :75-135 (bp_compute).  Channel ch is
+// rows [ch*cs, (ch+1)*cs) of every column; weights is (C x 2): scale, bias.  Sums run
+// over columns, then rows, in order.
+template <typename T>
+void csb_fwd(idx C, idx cs, idx w, CMat<T> x, Mat<T> y, CMat<T> weights)
+{
+#pragma omp parallel for
+  for (idx ch = 0; ch < C; ++ch) {
+    const T a = weights(ch, 0);
+    const T b = weights(ch, 1);
+    for (idx c = 0; c < w; ++c)
+      for (idx r = ch * cs; r < (ch + 1) * cs; ++r) y(r, c) = a * x(r, c) + b;
+  }
+}
+
+template <typename T>
+void csb_bwd(idx C, idx cs, idx w, CMat<T> x, CMat<T> dy, Mat<T> dx, CMat<T> weights, Mat<T> wgrad)
+{
+#pragma omp parallel for
+  for (idx ch = 0; ch < C; ++ch) {
+    const T a = weights(ch, 0);
+    T da = T(0), db = T(0);
+    for (idx c = 0; c < w; ++c)
+      for (idx r = ch * cs; r < (ch + 1) * cs; ++r) {
+        const T g = dy(r, c);
+        da += x(r, c) * g;
+        db += g;
+        dx(r, c) = a * g;
+      }
+    wgrad(ch, 0) = da;
+    wgrad(ch, 1) = db;
+  }
+}
+
 }  // namespace
 
 // C interface (one _f32 and one _f64 entry per function), bound by oracle/cpu_oracle.py.
@@ -729,7 +853,30 @@ void ebn_bwd(idx h, idx w, T eps, int training, CMat<T> x, CMat<T> dy, Mat<T> dx
       const T* x, idx ldx, const T* dy, idx lddy, T* dx, idx lddx, const T* stats,       \
       idx lds, T* sgrad, idx ldsg, const T* rvar)                                        \
   { ebn_bwd<T>(h, w, eps, training, {x, ldx}, {dy, lddy}, {dx, lddx}, {stats, lds},      \
-               {sgrad, ldsg}, rvar); }
+               {sgrad, ldsg}, rvar); }                                                   \
+  extern "C" void orc_cross_entropy_fwd_##SUF(idx h, idx w, int use_labels, idx spatial, \
+      const T* x, idx ldx, const T* truth, idx ldt, T* loss)                             \
+  { ce_fwd<T>(h, w, use_labels, spatial, {x, ldx}, {truth, ldt}, loss); }                \
+  extern "C" void orc_cross_entropy_bwd_##SUF(idx h, idx w, int use_labels, idx spatial, \
+      const T* x, idx ldx, const T* truth, idx ldt, const T* dy, T* dx, idx lddx,        \
+      T* dtruth, idx lddt)                                                               \
+  { ce_bwd<T>(h, w, use_labels, spatial, {x, ldx}, {truth, ldt}, dy, {dx, lddx},         \
+              {dtruth, lddt}); }                                                         \
+  extern "C" void orc_entrywise_scale_bias_fwd_##SUF(idx h, idx w, const T* x, idx ldx,  \
+      T* y, idx ldy, const T* weights, idx ldw)                                          \
+  { esb_fwd<T>(h, w, {x, ldx}, {y, ldy}, {weights, ldw}); }                              \
+  extern "C" void orc_entrywise_scale_bias_bwd_##SUF(idx h, idx w, const T* x, idx ldx,  \
+      const T* dy, idx lddy, T* dx, idx lddx, const T* weights, idx ldw, T* wgrad,       \
+      idx ldwg)                                                                          \
+  { esb_bwd<T>(h, w, {x, ldx}, {dy, lddy}, {dx, lddx}, {weights, ldw}, {wgrad, ldwg}); } \
+  extern "C" void orc_channelwise_scale_bias_fwd_##SUF(idx C, idx cs, idx w, const T* x, \
+      idx ldx, T* y, idx ldy, const T* weights, idx ldw)                                 \
+  { csb_fwd<T>(C, cs, w, {x, ldx}, {y, ldy}, {weights, ldw}); }                          \
+  extern "C" void orc_channelwise_scale_bias_bwd_##SUF(idx C, idx cs, idx w, const T* x, \
+      idx ldx, const T* dy, idx lddy, T* dx, idx lddx, const T* weights, idx ldw,        \
+      T* wgrad, idx ldwg)                                                                \
+  { csb_bwd<T>(C, cs, w, {x, ldx}, {dy, lddy}, {dx, lddx}, {weights, ldw},               \
+               {wgrad, ldwg}); }
 
 ORC_INSTANTIATE(f32, float)
 ORC_INSTANTIATE(f64, double)

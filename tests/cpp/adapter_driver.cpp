@@ -198,6 +198,58 @@ int drv_entrywise_batch_norm(const int64_t* dims, int nd, double decay, double e
   }
 }
 
+int drv_cross_entropy(const int64_t* pred_dims, const int64_t* truth_dims, int nd, int use_labels, int64_t h,
+                      int64_t ht, int64_t w, float* x, float* truth, float* loss, float* dloss, float* dx,
+                      float* dtruth, void* stream, char* err, int errlen)
+{
+  try {
+    cross_entropy_layer<> layer(use_labels != 0);
+    layer.setup(std::vector<int64_t>(pred_dims, pred_dims + nd), std::vector<int64_t>(truth_dims, truth_dims + nd));
+    device_matrix<float> mx, mt, ml, mdl, mdx, mdt;
+    attach(mx, h, w, x, h); attach(mt, ht, w, truth, ht); attach(ml, 1, w, loss, 1); attach(mdl, 1, w, dloss, 1);
+    attach(mdx, h, w, dx, h); attach(mdt, ht, w, dtruth, ht);
+    layer.io.prev_activations = &mx; layer.prev_ground_truth = &mt; layer.io.activations = &ml;
+    layer.io.prev_error_signals = &mdl; layer.io.error_signals = &mdx; layer.ground_truth_error_signals = &mdt;
+    layer.io.stream = static_cast<hipStream_t>(stream);
+    layer.fp_compute();
+    layer.bp_compute();
+    check_hip(hipStreamSynchronize(layer.io.stream), "sync");
+    return 0;
+  }
+  catch (const std::exception& e) {
+    return fail(e, err, errlen);
+  }
+}
+
+// kind: 0 entry-wise, 1 channel-wise.  weights: (n x 2) column-major, n = h resp. dims[0].
+int drv_scale_bias(int kind, const int64_t* dims, int nd, int64_t h, int64_t w, int64_t ld, float* x, float* y,
+                   float* dy, float* dx, const float* weights, int64_t ld_weights, float* wgrad_out,
+                   void* stream, char* err, int errlen)
+{
+  try {
+    device_matrix<float> mx, my, mdy, mdx;
+    attach(mx, h, w, x, ld); attach(my, h, w, y, ld); attach(mdy, h, w, dy, ld); attach(mdx, h, w, dx, ld);
+    auto run = [&](auto& layer) {
+      layer.setup(std::vector<int64_t>(dims, dims + nd));
+      layer.set_weights(weights, ld_weights);
+      layer.io.prev_activations = &mx; layer.io.activations = &my;
+      layer.io.prev_error_signals = &mdy; layer.io.error_signals = &mdx;
+      layer.io.stream = static_cast<hipStream_t>(stream);
+      layer.fp_compute();
+      layer.bp_compute();
+      copy_out(wgrad_out, layer.m_weights_gradient, layer.io.stream);
+      check_hip(hipStreamSynchronize(layer.io.stream), "sync");
+    };
+    if (kind == 0) { entrywise_scale_bias_layer<> l; run(l); }
+    else { channelwise_scale_bias_layer<> l; run(l); }
+    return 0;
+  }
+  catch (const std::exception& e) {
+    return fail(e, err, errlen);
+  }
+}
+
+
 // Host-only checks of the error behaviour the reference has: returns the number of
 // cases that did NOT throw as they should.
 int drv_error_cases(void)
@@ -210,6 +262,12 @@ int drv_error_cases(void)
   try { channelwise_softmax_layer<> l(1, false); l.setup({2, 3, 4}); ++missed; } catch (const exception&) {}
   try { batch_normalization_layer<> l(0.9, 1e-5, 0, true); ++missed; } catch (const exception&) {}
   { batch_normalization_layer<uint16_t> half_storage(0.9, 1e-5, 1, true); (void)half_storage; }
+  // cross entropy with labels: ground truth must be (1, spatial...) matching the prediction's spatial dims
+  try { cross_entropy_layer<> l(true); l.setup({3, 8, 8}, {2, 8, 8}); ++missed; } catch (const exception&) {}
+  try { cross_entropy_layer<> l(true); l.setup({3}, {1}); ++missed; } catch (const exception&) {}
+  try { cross_entropy_layer<> l(true); l.setup({3, 8, 8}, {1, 8, 4}); ++missed; } catch (const exception&) {}
+  try { cross_entropy_layer<> l(false); l.setup({3, 8}, {3, 4}); ++missed; } catch (const exception&) {}
+  { cross_entropy_layer<> l(true); l.setup({3, 4, 4, 4}, {1, 4, 4, 4}); }
   {
     layer_norm_layer<float> l(1e-5, true, true, -1);
     l.setup({31, 2, 5});

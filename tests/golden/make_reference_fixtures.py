@@ -20,6 +20,10 @@ Datasets and tolerances (reference file:line):
   instance_norm         ci_test/unit_tests/test_unit_layer_instance_norm.py:21-24, :38-44
   entrywise_batch_norm  ci_test/unit_tests/test_unit_layer_entrywise_batch_normalization.py:21-25
                         (no forward pin there: gradient check only)
+  cross_entropy         ci_test/unit_tests/test_unit_layer_cross_entropy.py:29-36, :53-76, :147-164,
+                        :192-209
+  entrywise_scale_bias  ci_test/unit_tests/test_unit_layer_entrywise_scale_bias.py:21-27, :98-110
+  channelwise_scale_bias ci_test/unit_tests/test_unit_layer_channelwise_scale_bias.py:21-27, :90-103
 
 Run:  python tests/golden/make_reference_fixtures.py
 """
@@ -160,6 +164,43 @@ def main():
         fx[f"ebn_{tag}_mean"] = mean
         fx[f"ebn_{tag}_var"] = var
         fx[f"ebn_{tag}_y"] = (xd - mean) / np.sqrt(var + 1e-5)
+
+    # ---- cross entropy dataset: 23 samples of (2*3, 64) U(0.25, 1) plus 64 labels in {0,1,2}.
+    # The reference feeds channels 0..2 as the prediction, channels 3..5 as a dense ground
+    # truth, and the labels as the ground truth of the use_labels cases; its metric is the
+    # mean over samples of (1e-3 * loss)^2.
+    np.random.seed(202303102)
+    samples = np.random.uniform(low=0.25, high=1, size=(23, 6, 64)).astype(np.float32)
+    labels = np.random.randint(3, size=(23, 1, 64)).astype(np.float32)
+    pred, dense = samples[:, :3, :].reshape(23, 192), samples[:, 3:, :].reshape(23, 192)
+    fx["ce_prediction"], fx["ce_dense_truth"], fx["ce_labels"] = pred, dense, labels.reshape(23, 64)
+    pd = pred.astype(np.float64)
+    loss_dense = -np.sum(dense.astype(np.float64) * np.log(pd), axis=1)
+    lab = labels.reshape(23, 64).astype(np.int64)
+    picked = np.take_along_axis(pd.reshape(23, 3, 64), lab[:, None, :], axis=1)[:, 0, :]
+    loss_labels = -np.sum(np.log(picked), axis=1)
+    fx["ce_loss_dense"], fx["ce_loss_labels"] = loss_dense, loss_labels
+    fx["ce_metric_dense"] = np.float64(np.mean((1e-3 * loss_dense) ** 2))
+    fx["ce_metric_labels"] = np.float64(np.mean((1e-3 * loss_labels) ** 2))
+    fx["ce_metric_tol"] = np.float64(8 * np.finfo(np.float32).eps)  # relative, as in the reference
+
+    # ---- entry-wise scale/bias: 29 x (7,5,3) N(0,1); scale N(1,1), bias N(0,1) per entry
+    np.random.seed(20190723)
+    x = np.random.normal(size=(29, 105)).astype(np.float32)
+    scale = np.random.normal(loc=1, size=(7, 5, 3)).astype(np.float32)
+    bias = np.random.normal(loc=0, size=(7, 5, 3)).astype(np.float32)
+    y = scale.reshape(1, 105).astype(np.float64) * x.astype(np.float64) + bias.reshape(1, 105).astype(np.float64)
+    fx["esb_x"], fx["esb_scale"], fx["esb_bias"], fx["esb_y"] = x, scale.reshape(105), bias.reshape(105), y
+    fx["esb_metric"] = np.float64(l2norm2_metric(y))
+
+    # ---- channel-wise scale/bias: 23 x (7,5,3) N(0,1); scale N(1,1), bias N(0,1) per channel
+    np.random.seed(20190719)
+    x = np.random.normal(size=(23, 105)).astype(np.float32)
+    scale = np.random.normal(loc=1, size=(7, 1, 1)).astype(np.float32)
+    bias = np.random.normal(loc=0, size=(7, 1, 1)).astype(np.float32)
+    y = (scale.astype(np.float64) * x.reshape(23, 7, 5, 3).astype(np.float64) + bias.astype(np.float64)).reshape(23, 105)
+    fx["csb_x"], fx["csb_scale"], fx["csb_bias"], fx["csb_y"] = x, scale.reshape(7), bias.reshape(7), y
+    fx["csb_metric"] = np.float64(l2norm2_metric(y))
 
     np.savez_compressed(OUT, **fx)
     print(OUT, os.path.getsize(OUT), "bytes,", len(fx), "arrays")

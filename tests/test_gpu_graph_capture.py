@@ -49,6 +49,10 @@ CASES = [
      ("m_mean_and_var", "m_mean_and_var_gradient", "m_scale_gradient", "m_bias_gradient")),
     ("batch norm f16", lambda L: L.batch_normalization_layer((32, 28, 28)), 32 * 784, 16, torch.float16,
      ("m_mean_and_var", "m_scale_gradient", "m_bias_gradient")),
+    ("entry-wise scale/bias", lambda L: L.entrywise_scale_bias_layer((512,)), 512, 2048, torch.float32,
+     ("m_weights_gradient",)),
+    ("channel-wise scale/bias", lambda L: L.channelwise_scale_bias_layer((8, 64, 64)), 8 * 4096, 16, torch.float32,
+     ("m_weights_gradient",)),
     ("batch norm small", lambda L: L.batch_normalization_layer((7, 5, 3)), 105, 14, torch.float32,
      ("m_mean_and_var", "m_mean_and_var_gradient")),
 ]

@@ -1,0 +1,223 @@
+"""GPU parity of the layers either side of the normalization / softmax path: cross
+entropy (consumes the softmax output) and the entry-wise / channel-wise scale-bias
+layers (the learned affine after a normalization layer), through the C ABI against
+the CPU oracle.  Tolerance 1e-5 (tests/parity.py), with the float64 oracle as the
+tie-breaker where the fp32 reference is itself noisier than that.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu_oracle as orc
+from tests.parity import TOL_F32, check, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def L():
+    from lbann_amd import layers
+    layers.capi.lib()
+    assert torch.cuda.is_available()
+    return layers
+
+
+def f64(a):
+    return np.asfortranarray(np.asarray(a, dtype=np.float64))
+
+
+def f32(a):
+    return np.asfortranarray(np.asarray(a, dtype=np.float32))
+
+
+def rand(rng, h, w, mean=0.0, std=1.0):
+    return np.asfortranarray((rng.standard_normal((w, h)) * std + mean).astype(np.float32).T)
+
+
+def vec_to_row(L, v):
+    return L.DeviceMatrix.from_numpy(np.asarray(v, np.float32).reshape(1, -1))
+
+
+# ===================================================================== cross entropy
+CE_DENSE = [
+    # (h, w, ld_pad)
+    (10, 128, 0), (1000, 64, 0), (192, 23, 0), (4096, 33, 0), (7, 5, 0), (1001, 3, 0), (130, 4, 2),
+    (512, 9, 64), (300000, 3, 0), (1 << 20, 2, 0), (65536, 40, 0), (1, 6, 0),
+]
+
+
+@pytest.mark.parametrize("h,w,pad", CE_DENSE)
+def test_cross_entropy_dense(L, h, w, pad):
+    rng = np.random.default_rng(h * 7 + w)
+    x = np.asfortranarray(rng.uniform(0.05, 1.0, (w, h)).astype(np.float32).T)
+    truth = np.asfortranarray(rng.uniform(-0.3, 1.0, (w, h)).astype(np.float32).T)  # a quarter <= 0: skipped
+    truth[0, :] = 0.0
+    dy = rng.standard_normal(w).astype(np.float32)
+    layer = L.cross_entropy_layer((h,))
+    ld = h + pad
+    loss = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=ld), L.DeviceMatrix.from_numpy(truth, ldim=ld)).to_numpy()
+    check(f"cross entropy loss {h}x{w}", loss[0], orc.cross_entropy_fwd(x, truth), orc.cross_entropy_fwd(f64(x), f64(truth)))
+    dx, dt = layer.backward(vec_to_row(L, dy))
+    rx, rt = orc.cross_entropy_bwd(x, truth, dy)
+    ex, et = orc.cross_entropy_bwd(f64(x), f64(truth), dy.astype(np.float64))
+    got = dx.to_numpy()
+    check(f"cross entropy dx {h}x{w}", got, rx, ex)
+    assert np.all(got[truth <= 0] == 0.0)
+    check(f"cross entropy dtruth {h}x{w}", dt.to_numpy(), rt, et)
+
+
+CE_LABELS = [
+    # (classes, spatial dims, w, ld_pad)
+    (3, (8, 8), 23, 0), (3, (4, 4, 4), 11, 0), (10, (1,), 64, 0), (5, (7, 3), 9, 0), (4, (6,), 5, 3),
+    (21, (64, 64), 6, 0), (2, (300, 300), 3, 0), (1000, (1,), 128, 0), (19, (128, 130), 2, 0),
+]
+
+
+@pytest.mark.parametrize("classes,spatial,w,pad", CE_LABELS)
+def test_cross_entropy_labels(L, classes, spatial, w, pad):
+    rng = np.random.default_rng(classes * 100 + w)
+    sp = int(np.prod(spatial))
+    h = classes * sp
+    x = np.asfortranarray(rng.uniform(0.05, 1.0, (w, h)).astype(np.float32).T)
+    labels = np.asfortranarray(rng.integers(0, classes, (w, sp)).astype(np.float32).T)
+    if sp > 2:
+        labels[1, 0] = classes      # a label no class matches contributes nothing
+        labels[2, 0] = -3.0
+    dy = rng.standard_normal(w).astype(np.float32)
+    layer = L.cross_entropy_layer((classes,) + tuple(spatial), use_labels=True)
+    loss = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad),
+                         L.DeviceMatrix.from_numpy(labels, ldim=sp + pad)).to_numpy()
+    check(f"cross entropy (labels) loss {classes}x{sp}x{w}", loss[0], orc.cross_entropy_fwd(x, labels, True),
+          orc.cross_entropy_fwd(f64(x), f64(labels), True))
+    dx, none = layer.backward(vec_to_row(L, dy))
+    assert none is None
+    check(f"cross entropy (labels) dx {classes}x{sp}x{w}", dx.to_numpy(), orc.cross_entropy_bwd(x, labels, dy, True)[0],
+          orc.cross_entropy_bwd(f64(x), f64(labels), dy.astype(np.float64), True)[0])
+
+
+def test_cross_entropy_after_softmax(L):
+    """softmax -> cross entropy and back, as in a classifier's last two layers."""
+    rng = np.random.default_rng(3)
+    h, w = 1000, 96
+    logits = rand(rng, h, w, 0, 2)
+    onehot = np.zeros((h, w), np.float32, order="F")
+    onehot[rng.integers(0, h, w), np.arange(w)] = 1.0
+    sm, ce = L.softmax_layer(), L.cross_entropy_layer((h,))
+    p = sm.forward(L.DeviceMatrix.from_numpy(logits))
+    loss = ce.forward(p, L.DeviceMatrix.from_numpy(onehot)).to_numpy()[0]
+    dy = np.full(w, 1.0 / w, np.float32)
+    dp, _ = ce.backward(vec_to_row(L, dy))
+    dlogits = sm.backward(dp).to_numpy()
+    p64 = orc.softmax_fwd(f64(logits))
+    check("softmax+ce loss", loss, orc.cross_entropy_fwd(orc.softmax_fwd(logits), onehot), orc.cross_entropy_fwd(p64, f64(onehot)))
+    # closed form of the composition: (softmax - onehot) / w
+    assert rel_err(dlogits, (p64 - onehot) / w) < 5e-6
+
+
+# ===================================================================== scale/bias layers
+ESB_SHAPES = [
+    # (h, w, ld_pad)   tile kernels with 64 and 256 rows per workgroup, column slabs, scalar fallback
+    (105, 29, 0), (4096, 64, 0), (64, 1024, 0), (1024, 4096, 0), (256 * 512, 24, 0), (256 * 512 + 8, 5, 0),
+    (2048, 17, 4), (1001, 7, 0), (130, 3, 3), (4, 300, 0), (1, 9, 0), (8192, 1, 0), (300000, 16, 0),
+]
+
+
+@pytest.mark.parametrize("h,w,pad", ESB_SHAPES)
+def test_entrywise_scale_bias(L, h, w, pad):
+    rng = np.random.default_rng(h + 13 * w)
+    x, dy = rand(rng, h, w, 0.5, 2.0), rand(rng, h, w)
+    wts = np.asfortranarray(np.stack([rng.normal(1, 1, h), rng.normal(0, 1, h)], axis=1).astype(np.float32))
+    layer = L.entrywise_scale_bias_layer((h,))
+    layer.set_weights(wts[:, 0], wts[:, 1])
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    check(f"entrywise scale/bias y {h}x{w}", y, orc.entrywise_scale_bias_fwd(x, wts), orc.entrywise_scale_bias_fwd(f64(x), f64(wts)))
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    rdx, rwg = orc.entrywise_scale_bias_bwd(x, dy, wts)
+    edx, ewg = orc.entrywise_scale_bias_bwd(f64(x), f64(dy), f64(wts))
+    check(f"entrywise scale/bias dx {h}x{w}", dx, rdx, edx)
+    check(f"entrywise scale/bias dweights {h}x{w}", layer.m_weights_gradient.to_numpy(), rwg, ewg)
+
+
+CSB_CASES = [
+    # dims (C, ...), w, ld_pad
+    ((7, 5, 3), 23, 0), ((64, 56, 56), 8, 0), ((3, 224, 224), 4, 0), ((256, 4, 4), 32, 0), ((2048, 1, 1), 64, 0),
+    ((5, 12), 10, 4), ((5, 13), 10, 0), ((1, 100000), 3, 0), ((2, 1), 1, 0), ((70000, 1), 2, 0), ((16, 128, 128), 16, 0),
+]
+
+
+@pytest.mark.parametrize("dims,w,pad", CSB_CASES)
+def test_channelwise_scale_bias(L, dims, w, pad):
+    rng = np.random.default_rng(int(np.prod(dims)) + w)
+    C, cs = dims[0], int(np.prod(dims[1:]))
+    h = C * cs
+    x, dy = rand(rng, h, w, 0.5, 2.0), rand(rng, h, w)
+    wts = np.asfortranarray(np.stack([rng.normal(1, 1, C), rng.normal(0, 1, C)], axis=1).astype(np.float32))
+    layer = L.channelwise_scale_bias_layer(dims)
+    layer.set_weights(wts[:, 0], wts[:, 1])
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    check(f"channelwise scale/bias y {dims}x{w}", y, orc.channelwise_scale_bias_fwd(x, wts, C, cs),
+          orc.channelwise_scale_bias_fwd(f64(x), f64(wts), C, cs))
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    rdx, rwg = orc.channelwise_scale_bias_bwd(x, dy, wts, C, cs)
+    edx, ewg = orc.channelwise_scale_bias_bwd(f64(x), f64(dy), f64(wts), C, cs)
+    check(f"channelwise scale/bias dx {dims}x{w}", dx, rdx, edx)
+    check(f"channelwise scale/bias dweights {dims}x{w}", layer.m_weights_gradient.to_numpy(), rwg, ewg)
+
+
+# ===================================================================== golden fixtures, boundary behaviour
+def test_neighbour_layer_fixtures_on_gpu(L, golden):
+    F32_EPS = np.finfo(np.float32).eps
+    T = lambda a: np.asfortranarray(np.asarray(a).T)
+    met = lambda y: float(np.mean(np.sum(np.asarray(y, np.float64) ** 2, axis=0)))
+    pred = L.DeviceMatrix.from_numpy(T(golden["ce_prediction"]))
+    loss = L.cross_entropy_layer((192,)).forward(pred, L.DeviceMatrix.from_numpy(T(golden["ce_dense_truth"]))).to_numpy()[0]
+    assert rel_err(loss, golden["ce_loss_dense"]) < TOL_F32
+    val = float(golden["ce_metric_dense"])
+    assert abs(np.mean((1e-3 * loss.astype(np.float64)) ** 2) - val) <= val * float(golden["ce_metric_tol"])
+    for dims in ((3, 8, 8), (3, 4, 4, 4)):   # the reference's 2-D and 3-D label cases
+        loss = L.cross_entropy_layer(dims, use_labels=True).forward(
+            pred, L.DeviceMatrix.from_numpy(T(golden["ce_labels"]))).to_numpy()[0]
+        assert rel_err(loss, golden["ce_loss_labels"]) < TOL_F32
+        val = float(golden["ce_metric_labels"])
+        assert abs(np.mean((1e-3 * loss.astype(np.float64)) ** 2) - val) <= val * float(golden["ce_metric_tol"])
+    esb = L.entrywise_scale_bias_layer((7, 5, 3))
+    esb.set_weights(golden["esb_scale"], golden["esb_bias"])
+    y = esb.forward(L.DeviceMatrix.from_numpy(T(golden["esb_x"]))).to_numpy()
+    assert rel_err(y.T, golden["esb_y"]) < TOL_F32
+    assert abs(met(y) - float(golden["esb_metric"])) <= 8 * float(golden["esb_metric"]) * F32_EPS
+    csb = L.channelwise_scale_bias_layer((7, 5, 3))
+    csb.set_weights(golden["csb_scale"], golden["csb_bias"])
+    y = csb.forward(L.DeviceMatrix.from_numpy(T(golden["csb_x"]))).to_numpy()
+    assert rel_err(y.T, golden["csb_y"]) < TOL_F32
+    assert abs(met(y) - float(golden["csb_metric"])) <= 8 * float(golden["csb_metric"]) * F32_EPS
+
+
+def test_neighbour_layers_empty_and_rejected_arguments(L):
+    from lbann_amd import capi
+    st = capi.vp(torch.cuda.current_stream().cuda_stream)
+    null = capi.vp(None)
+    lib = capi.lib()
+    buf = torch.zeros(4096, device="cuda")
+    p = capi.vp(buf.data_ptr())
+    # empty inputs: nothing to do
+    assert lib.lbn_entrywise_scale_bias_fwd_f32(st, 0, 4, null, 1, null, 1, null, 1) == 0
+    assert lib.lbn_channelwise_scale_bias_fwd_f32(st, 4, 8, 0, null, 32, null, 32, null, 4) == 0
+    assert lib.lbn_cross_entropy_fwd_f32(st, 8, 0, 0, 1, null, 8, null, 8, null, 1, null, 0) == 0
+    assert lib.lbn_cross_entropy_bwd_f32(st, 0, 3, 0, 1, null, 1, null, 1, null, 1, null, 1, null, 1) == 0
+    # a sample without entries has loss 0
+    buf.fill_(7.0)
+    assert lib.lbn_cross_entropy_fwd_f32(st, 0, 3, 0, 1, null, 1, null, 1, p, 1, null, 0) == 0
+    torch.cuda.synchronize()
+    assert buf[:3].tolist() == [0.0, 0.0, 0.0] and buf[3].item() == 7.0
+    # rejected: leading dimension below the height, missing matrices, missing workspace
+    assert lib.lbn_entrywise_scale_bias_fwd_f32(st, 8, 4, p, 4, p, 8, p, 8) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_entrywise_scale_bias_fwd_f32(st, 8, 4, p, 8, p, 8, p, 4) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_channelwise_scale_bias_bwd_f32(st, 2, 4, 4, p, 8, p, 8, null, 8, p, 2, p, 2, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_cross_entropy_fwd_f32(st, 8, 4, 1, 0, p, 8, p, 8, p, 1, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_cross_entropy_bwd_f32(st, 8, 4, 0, 1, p, 8, p, 8, p, 1, p, 8, null, 8) == capi.LBN_ERR_INVALID_ARGUMENT
+    big = torch.zeros(64 * 8192, device="cuda")
+    pb = capi.vp(big.data_ptr())
+    assert lib.lbn_entrywise_scale_bias_bwd_workspace_bytes(64, 8192) > 0
+    assert lib.lbn_entrywise_scale_bias_bwd_f32(st, 64, 8192, pb, 64, pb, 64, pb, 64, p, 64, p, 64, null, 0) == capi.LBN_ERR_WORKSPACE
+    assert lib.lbn_cross_entropy_fwd_f32(st, 65536, 8, 0, 1, pb, 65536, pb, 65536, p, 1, null, 0) == capi.LBN_ERR_WORKSPACE
+    torch.cuda.synchronize()

@@ -152,3 +152,52 @@ def test_batch_norms_random(L, case):
     check("entrywise bn y " + tag, y, y32, y64)
     check("entrywise bn dx " + tag, dx, orc.entrywise_batch_norm_bwd(x, dy, st32, 1e-5)[0],
           orc.entrywise_batch_norm_bwd(f64(x), f64(dy), st64, 1e-5)[0])
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_cross_entropy_and_scale_bias_random(L, case):
+    rng = np.random.default_rng(5000 + case)
+    C = int(rng.integers(1, 12))
+    cs = draw_length(rng) // int(rng.choice([1, 4, 16])) + 1 if case % 3 else int(rng.integers(1, 60)) * 4
+    h, w = C * cs, int(rng.integers(1, 70))
+    pad = int(rng.choice([0, 0, 4, 3]))
+    tag = f"C={C} cs={cs} w={w} pad={pad}"
+    x, dy = rand(rng, h, w, 0.5, 2.0), rand(rng, h, w)
+    # scale/bias layers
+    for kind, n in (("entrywise", h), ("channelwise", C)):
+        wts = np.asfortranarray(np.stack([rng.normal(1, 1, n), rng.normal(0, 1, n)], axis=1).astype(np.float32))
+        if kind == "entrywise":
+            layer = L.entrywise_scale_bias_layer((h,))
+            fwd = lambda a, b: orc.entrywise_scale_bias_fwd(a, b)
+            bwd = lambda a, g, b: orc.entrywise_scale_bias_bwd(a, g, b)
+        else:
+            layer = L.channelwise_scale_bias_layer((C, cs))
+            fwd = lambda a, b: orc.channelwise_scale_bias_fwd(a, b, C, cs)
+            bwd = lambda a, g, b: orc.channelwise_scale_bias_bwd(a, g, b, C, cs)
+        layer.set_weights(wts[:, 0], wts[:, 1])
+        y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+        dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+        check(f"{kind} scale/bias y {tag}", y, fwd(x, wts), fwd(f64(x), f64(wts)))
+        rdx, rwg = bwd(x, dy, wts)
+        edx, ewg = bwd(f64(x), f64(dy), f64(wts))
+        check(f"{kind} scale/bias dx {tag}", dx, rdx, edx)
+        check(f"{kind} scale/bias dweights {tag}", layer.m_weights_gradient.to_numpy(), rwg, ewg)
+    # cross entropy, dense ground truth and labels (C classes, cs spatial positions)
+    pred = np.asfortranarray(rng.uniform(0.05, 1.0, (w, h)).astype(np.float32).T)
+    dense = np.asfortranarray(rng.uniform(-0.3, 1.0, (w, h)).astype(np.float32).T)
+    labels = np.asfortranarray(rng.integers(0, C, (w, cs)).astype(np.float32).T)
+    dloss = rng.standard_normal(w).astype(np.float32)
+    drow = L.DeviceMatrix.from_numpy(dloss.reshape(1, -1))
+    for use_labels, truth, dims in ((False, dense, (h,)), (True, labels, (C, cs))):
+        layer = L.cross_entropy_layer(dims, use_labels=use_labels)
+        tpad = pad if truth.shape[0] + pad >= truth.shape[0] else 0
+        loss = layer.forward(L.DeviceMatrix.from_numpy(pred, ldim=h + pad),
+                             L.DeviceMatrix.from_numpy(truth, ldim=truth.shape[0] + tpad)).to_numpy()[0]
+        check(f"cross entropy loss labels={use_labels} {tag}", loss, orc.cross_entropy_fwd(pred, truth, use_labels),
+              orc.cross_entropy_fwd(f64(pred), f64(truth), use_labels))
+        dx, dt = layer.backward(drow)
+        rdx, rdt = orc.cross_entropy_bwd(pred, truth, dloss, use_labels)
+        edx, edt = orc.cross_entropy_bwd(f64(pred), f64(truth), dloss.astype(np.float64), use_labels)
+        check(f"cross entropy dx labels={use_labels} {tag}", dx.to_numpy(), rdx, edx)
+        if not use_labels:
+            check(f"cross entropy dtruth {tag}", dt.to_numpy(), rdt, edt)

@@ -506,3 +506,94 @@ def test_entrywise_batch_norm_bwd_finite_difference_and_single_sample():
     assert not y1.any() and np.array_equal(s1[:, 0], x1[:, 0]) and (s1[:, 1] == 1).all()
     assert (rm == 0.25).all() and (rv == 2.0).all()
     assert not orc.entrywise_batch_norm_bwd(x1, x1, s1, 1e-5)[0].any()
+
+
+# ============================================================== cross entropy
+@pytest.mark.parametrize("dt,tol", [(np.float32, 2e-6), (np.float64, 1e-12)])
+def test_cross_entropy_golden(golden, dt, tol):
+    x = F(golden["ce_prediction"], dt)
+    dense, labels = F(golden["ce_dense_truth"], dt), F(golden["ce_labels"], dt)
+    loss = orc.cross_entropy_fwd(x, dense)
+    assert rel_err(loss, golden["ce_loss_dense"]) < tol
+    val = float(golden["ce_metric_dense"])
+    assert abs(np.mean((1e-3 * loss.astype(np.float64)) ** 2) - val) <= val * float(golden["ce_metric_tol"])
+    loss = orc.cross_entropy_fwd(x, labels, use_labels=True)
+    assert rel_err(loss, golden["ce_loss_labels"]) < tol
+    val = float(golden["ce_metric_labels"])
+    assert abs(np.mean((1e-3 * loss.astype(np.float64)) ** 2) - val) <= val * float(golden["ce_metric_tol"])
+
+
+def test_cross_entropy_backward_matches_autograd_and_skips_nonpositive_truth():
+    rng = np.random.default_rng(5)
+    h, w = 24, 7
+    x = np.asfortranarray(rng.uniform(0.25, 1.0, (h, w)))
+    truth = np.asfortranarray(rng.uniform(-0.5, 1.0, (h, w)))   # a third of the entries <= 0
+    truth[3, 2] = 0.0
+    dy = rng.standard_normal(w)
+    loss = orc.cross_entropy_fwd(x, truth)
+    pos = truth > 0
+    assert np.allclose(loss, -(np.where(pos, truth, 0.0) * np.log(x)).sum(axis=0), rtol=1e-13)
+    dx, dtruth = orc.cross_entropy_bwd(x, truth, dy)
+    tx = torch.tensor(x, requires_grad=True)
+    tt = torch.tensor(truth, requires_grad=True)
+    obj = (-(tt * torch.log(tx)) * torch.tensor(dy)).sum()
+    gx, gt = torch.autograd.grad(obj, (tx, tt))
+    assert np.allclose(dx[pos], gx.numpy()[pos], rtol=1e-12)
+    assert np.all(dx[~pos] == 0.0)                       # the reference zeroes them (xhat > 0 test)
+    assert np.allclose(dtruth, gt.numpy(), rtol=1e-12)   # dxhat = -dy log x everywhere
+    # labels: one class index per spatial position, prediction rows are class-major
+    classes, spatial = 4, 6
+    x = np.asfortranarray(rng.uniform(0.25, 1.0, (classes * spatial, w)))
+    lab = rng.integers(0, classes, (spatial, w))
+    onehot = np.zeros((classes, spatial, w))
+    for c in range(w):
+        onehot[lab[:, c], np.arange(spatial), c] = 1.0
+    onehot = np.asfortranarray(onehot.reshape(classes * spatial, w))
+    labf = np.asfortranarray(lab.astype(np.float64))
+    assert np.array_equal(orc.cross_entropy_fwd(x, labf, use_labels=True), orc.cross_entropy_fwd(x, onehot))
+    dxl, none = orc.cross_entropy_bwd(x, labf, dy, use_labels=True)
+    assert none is None
+    assert np.array_equal(dxl, orc.cross_entropy_bwd(x, onehot, dy)[0])
+
+
+# ============================================================ scale/bias layers
+@pytest.mark.parametrize("dt,tol", [(np.float32, 2e-6), (np.float64, 1e-12)])
+def test_scale_bias_golden(golden, dt, tol):
+    x = F(golden["esb_x"], dt)
+    wts = np.asfortranarray(np.stack([golden["esb_scale"], golden["esb_bias"]], axis=1).astype(dt))
+    y = orc.entrywise_scale_bias_fwd(x, wts)
+    assert rel_err(y.T, golden["esb_y"]) < tol
+    val = float(golden["esb_metric"])
+    assert abs(metric(y) - val) <= 8 * val * F32_EPS
+    x = F(golden["csb_x"], dt)
+    wts = np.asfortranarray(np.stack([golden["csb_scale"], golden["csb_bias"]], axis=1).astype(dt))
+    y = orc.channelwise_scale_bias_fwd(x, wts, 7, 15)
+    assert rel_err(y.T, golden["csb_y"]) < tol
+    val = float(golden["csb_metric"])
+    assert abs(metric(y) - val) <= 8 * val * F32_EPS
+
+
+def test_scale_bias_backward_matches_autograd():
+    rng = np.random.default_rng(11)
+    C, cs, w = 5, 6, 9
+    h = C * cs
+    x = np.asfortranarray(rng.standard_normal((h, w)))
+    dy = np.asfortranarray(rng.standard_normal((h, w)))
+    tx = torch.tensor(x, requires_grad=True)
+    tdy = torch.tensor(dy)
+    # entry-wise: one (scale, bias) per row
+    wts = np.asfortranarray(rng.standard_normal((h, 2)))
+    tw = torch.tensor(wts, requires_grad=True)
+    y = tw[:, 0:1] * tx + tw[:, 1:2]
+    assert np.allclose(orc.entrywise_scale_bias_fwd(x, wts), y.detach().numpy(), rtol=1e-13)
+    gx, gw = torch.autograd.grad((y * tdy).sum(), (tx, tw))
+    dx, wg = orc.entrywise_scale_bias_bwd(x, dy, wts)
+    assert np.allclose(dx, gx.numpy(), rtol=1e-12) and np.allclose(wg, gw.numpy(), rtol=1e-11, atol=1e-13)
+    # channel-wise: one (scale, bias) per block of cs rows
+    wts = np.asfortranarray(rng.standard_normal((C, 2)))
+    tw = torch.tensor(wts, requires_grad=True)
+    y = tw[:, 0].repeat_interleave(cs)[:, None] * tx + tw[:, 1].repeat_interleave(cs)[:, None]
+    assert np.allclose(orc.channelwise_scale_bias_fwd(x, wts, C, cs), y.detach().numpy(), rtol=1e-13)
+    gx, gw = torch.autograd.grad((y * tdy).sum(), (tx, tw))
+    dx, wg = orc.channelwise_scale_bias_bwd(x, dy, wts, C, cs)
+    assert np.allclose(dx, gx.numpy(), rtol=1e-12) and np.allclose(wg, gw.numpy(), rtol=1e-11, atol=1e-13)
