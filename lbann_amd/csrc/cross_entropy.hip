@@ -48,9 +48,10 @@ __device__ __forceinline__ float ce_term(float xhat, float x) { return xhat > 0.
 // (`const int truth_label = local_ground_truth(offset, col)`, cross_entropy.cpp:58).
 __device__ __forceinline__ int64_t ce_label(float v) { return static_cast<int64_t>(static_cast<int>(v)); }
 
+template <int T>
 __device__ __forceinline__ void ce_store_partial(const CeArgs& a, float sum, float* red)
 {
-  sum = team_sum<kCeWaves>(sum, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+  sum = team_sum<T / kWave>(sum, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
   if (threadIdx.x == 0) {
     const int64_t c = blockIdx.x;
     if (gridDim.y == 1) a.loss[c * a.ld_loss] = sum;
@@ -58,18 +59,18 @@ __device__ __forceinline__ void ce_store_partial(const CeArgs& a, float sum, flo
   }
 }
 
-template <bool VEC>
-__global__ void __launch_bounds__(kCeThreads)
+template <bool VEC, int T>
+__global__ void __launch_bounds__(T)
 ce_fwd_dense(CeArgs a)
 {
-  __shared__ float red[kCeWaves];
+  __shared__ float red[T / kWave];
   const int64_t c = blockIdx.x;
   const float* xc = a.x + c * a.ldx;
   const float* tc = a.truth + c * a.ldt;
   const int64_t n = VEC ? a.h / 4 : a.h;
-  const int64_t step = static_cast<int64_t>(gridDim.y) * kCeThreads;
+  const int64_t step = static_cast<int64_t>(gridDim.y) * T;
   float sum = 0.f;
-  for (int64_t j = static_cast<int64_t>(blockIdx.y) * kCeThreads + threadIdx.x; j < n; j += step) {
+  for (int64_t j = static_cast<int64_t>(blockIdx.y) * T + threadIdx.x; j < n; j += step) {
     if (VEC) {
       float v[4], t[4];
       Vec16<float>::load(xc + 4 * j, v);
@@ -81,7 +82,7 @@ ce_fwd_dense(CeArgs a)
       sum += ce_term(tc[j], xc[j]);
     }
   }
-  ce_store_partial(a, sum, red);
+  ce_store_partial<T>(a, sum, red);
 }
 
 // One thread per spatial position: gather the entry of x its label points at.
@@ -100,7 +101,7 @@ ce_fwd_labels(CeArgs a)
     const int64_t r = label * a.spatial + o;
     if (label >= 0 && r < a.h) sum += -logf(xc[r]);
   }
-  ce_store_partial(a, sum, red);
+  ce_store_partial<kCeThreads>(a, sum, red);
 }
 
 __global__ void __launch_bounds__(kWave)
@@ -185,11 +186,12 @@ ce_bwd_labels(CeArgs a)
   }
 }
 
-// Workgroups per column: about 2048 in total, each with at least four units per thread.
-static int ce_parts(int64_t w, int64_t units_per_column)
+// Workgroups of `threads` threads per column: about 2048 * 256 threads in total, each
+// thread with at least four units.
+static int ce_parts(int64_t w, int64_t units_per_column, int threads = kCeThreads)
 {
-  int64_t p = ceil_div(2048, w);
-  const int64_t most = ceil_div(units_per_column, 4 * kCeThreads);
+  int64_t p = ceil_div(2048 * kCeThreads, w * threads);
+  const int64_t most = ceil_div(units_per_column, 4 * threads);
   if (p > most) p = most;
   if (p > kCeMaxParts) p = kCeMaxParts;
   return static_cast<int>(p < 1 ? 1 : p);
@@ -239,14 +241,19 @@ int lbn_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width
   const bool vec = !use_labels && ce_vec_ok(height, width, prediction, ld_prediction) &&
                    ce_vec_ok(height, width, ground_truth, ld_ground_truth);
   const int64_t units = use_labels ? (spatial_size < height ? spatial_size : height) : (vec ? height / 4 : height);
-  const int P = ce_parts(width, units);
+  // 1024-thread workgroups when that fills the device with one workgroup per column: no
+  // partial sums to merge, so no second kernel
+  const bool big = !use_labels && units >= 4 * 1024 && width >= 256;
+  const int P = ce_parts(width, units, big ? 1024 : kCeThreads);
   if (P > 1 && (!workspace || workspace_bytes < static_cast<size_t>(width) * P * sizeof(float) ||
                 (reinterpret_cast<uintptr_t>(workspace) & 3u)))
     return LBN_ERR_WORKSPACE;
   const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
   if (use_labels) hipLaunchKernelGGL(ce_fwd_labels, grid, dim3(kCeThreads), 0, st, a);
-  else if (vec) hipLaunchKernelGGL((ce_fwd_dense<true>), grid, dim3(kCeThreads), 0, st, a);
-  else hipLaunchKernelGGL((ce_fwd_dense<false>), grid, dim3(kCeThreads), 0, st, a);
+  else if (vec && big) hipLaunchKernelGGL((ce_fwd_dense<true, 1024>), grid, dim3(1024), 0, st, a);
+  else if (vec) hipLaunchKernelGGL((ce_fwd_dense<true, kCeThreads>), grid, dim3(kCeThreads), 0, st, a);
+  else if (big) hipLaunchKernelGGL((ce_fwd_dense<false, 1024>), grid, dim3(1024), 0, st, a);
+  else hipLaunchKernelGGL((ce_fwd_dense<false, kCeThreads>), grid, dim3(kCeThreads), 0, st, a);
   if (P > 1)
     hipLaunchKernelGGL(ce_merge_parts, dim3(static_cast<unsigned>(width)), dim3(kWave), 0, st, P, a.part, loss,
                        ld_loss);

@@ -317,11 +317,11 @@ csb_fwd(CsbArgs a)
   }
 }
 
-template <bool VEC>
-__global__ void __launch_bounds__(kSbThreads)
+template <bool VEC, int T>
+__global__ void __launch_bounds__(T)
 csb_bwd(CsbArgs a)
 {
-  __shared__ float red[2 * kSbWaves];
+  __shared__ float red[2 * (T / kWave)];
   const int64_t ch = blockIdx.x;
   const float sc = a.weights[ch];
   const float* xc = a.x + ch * a.cs;
@@ -329,9 +329,9 @@ csb_bwd(CsbArgs a)
   float* dc = a.out + ch * a.cs;
   const int64_t seg = VEC ? a.cs / 4 : a.cs;
   const int64_t total = seg * a.w;
-  const int64_t step = static_cast<int64_t>(gridDim.y) * kSbThreads;
+  const int64_t step = static_cast<int64_t>(gridDim.y) * T;
   float da = 0.f, db = 0.f;
-  for (int64_t j = static_cast<int64_t>(blockIdx.y) * kSbThreads + threadIdx.x; j < total; j += step) {
+  for (int64_t j = static_cast<int64_t>(blockIdx.y) * T + threadIdx.x; j < total; j += step) {
     const unsigned ucol = static_cast<unsigned>(j) / static_cast<unsigned>(seg);
     const int64_t col = ucol;
     const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(seg);
@@ -354,7 +354,7 @@ csb_bwd(CsbArgs a)
       dc[col * a.ldo + i] = sc * g;
     }
   }
-  team_sum2<kSbWaves>(da, db, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+  team_sum2<T / kWave>(da, db, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
   if (threadIdx.x == 0) {
     if (gridDim.y == 1) {
       a.wgrad[ch] = da;
@@ -385,11 +385,12 @@ csb_merge_parts(int P, const float2* __restrict__ part, float* __restrict__ wgra
   }
 }
 
-// Workgroups per channel: about 2048 in total, each with at least four vectors per thread.
-static int csb_parts(int64_t C, int64_t vectors_per_channel)
+// Workgroups of `threads` threads per channel: about 2048 * 256 threads in total, each
+// thread with at least four vectors.
+static int csb_parts(int64_t C, int64_t vectors_per_channel, int threads = kSbThreads)
 {
-  int64_t p = ceil_div(2048, C);
-  const int64_t most = ceil_div(vectors_per_channel, 4 * kSbThreads);
+  int64_t p = ceil_div(2048 * kSbThreads, C * threads);
+  const int64_t most = ceil_div(vectors_per_channel, 4 * threads);
   if (p > most) p = most;
   if (p > kSbMaxParts) p = kSbMaxParts;
   return static_cast<int>(p < 1 ? 1 : p);
@@ -524,15 +525,21 @@ int lbn_channelwise_scale_bias_bwd_f32(lbn_stream_t stream, int64_t num_channels
   hipStream_t st = as_stream(stream);
   const bool vec = csb_vec_ok(channel_size, width, x, ldx) && csb_vec_ok(channel_size, width, dy, lddy) &&
                    csb_vec_ok(channel_size, width, dx, lddx);
-  const int P = csb_parts(num_channels, (vec ? channel_size / 4 : channel_size) * width);
+  const int64_t units = (vec ? channel_size / 4 : channel_size) * width;
+  // 1024-thread workgroups when that fills the device with one workgroup per channel: no
+  // partial sums to merge, so no second kernel
+  const bool big = units >= 4 * 1024 && num_channels >= 256;
+  const int P = big ? 1 : csb_parts(num_channels, units);
   if (P > 1 && (!workspace || workspace_bytes < static_cast<size_t>(num_channels) * P * sizeof(float2) ||
                 (reinterpret_cast<uintptr_t>(workspace) & 7u)))
     return LBN_ERR_WORKSPACE;
   const CsbArgs a{channel_size, width, x, dy, dx, ldx, lddy, lddx, weights, ld_weights, weights_grad,
                   ld_weights_grad, static_cast<float2*>(workspace)};
   const dim3 grid(static_cast<unsigned>(num_channels), static_cast<unsigned>(P));
-  if (vec) hipLaunchKernelGGL((csb_bwd<true>), grid, dim3(kSbThreads), 0, st, a);
-  else hipLaunchKernelGGL((csb_bwd<false>), grid, dim3(kSbThreads), 0, st, a);
+  if (vec && big) hipLaunchKernelGGL((csb_bwd<true, 1024>), grid, dim3(1024), 0, st, a);
+  else if (vec) hipLaunchKernelGGL((csb_bwd<true, kSbThreads>), grid, dim3(kSbThreads), 0, st, a);
+  else if (big) hipLaunchKernelGGL((csb_bwd<false, 1024>), grid, dim3(1024), 0, st, a);
+  else hipLaunchKernelGGL((csb_bwd<false, kSbThreads>), grid, dim3(kSbThreads), 0, st, a);
   if (P > 1)
     hipLaunchKernelGGL(csb_merge_parts, dim3(static_cast<unsigned>(num_channels)), dim3(kWave), 0, st, P,
                        a.part, weights_grad, ld_weights_grad);

@@ -43,6 +43,7 @@ CE_DENSE = [
     # (h, w, ld_pad)
     (10, 128, 0), (1000, 64, 0), (192, 23, 0), (4096, 33, 0), (7, 5, 0), (1001, 3, 0), (130, 4, 2),
     (512, 9, 64), (300000, 3, 0), (1 << 20, 2, 0), (65536, 40, 0), (1, 6, 0),
+    (16384, 256, 0), (4101, 257, 0),   # one 1024-thread workgroup per column, vector and scalar
 ]
 
 
@@ -142,6 +143,7 @@ CSB_CASES = [
     # dims (C, ...), w, ld_pad
     ((7, 5, 3), 23, 0), ((64, 56, 56), 8, 0), ((3, 224, 224), 4, 0), ((256, 4, 4), 32, 0), ((2048, 1, 1), 64, 0),
     ((5, 12), 10, 4), ((5, 13), 10, 0), ((1, 100000), 3, 0), ((2, 1), 1, 0), ((70000, 1), 2, 0), ((16, 128, 128), 16, 0),
+    ((256, 28, 28), 24, 0), ((256, 7, 3), 200, 0),   # one 1024-thread workgroup per channel, vector and scalar
 ]
 
 
