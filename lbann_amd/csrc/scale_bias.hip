@@ -289,8 +289,8 @@ struct CsbArgs {
   float2* part;  // [C][P]
 };
 
-template <bool VEC>
-__global__ void __launch_bounds__(kSbThreads)
+template <bool VEC, int T>
+__global__ void __launch_bounds__(T)
 csb_fwd(CsbArgs a)
 {
   const int64_t ch = blockIdx.x;
@@ -299,8 +299,8 @@ csb_fwd(CsbArgs a)
   float* yc = a.out + ch * a.cs;
   const int64_t seg = VEC ? a.cs / 4 : a.cs;
   const int64_t total = seg * a.w;
-  const int64_t step = static_cast<int64_t>(gridDim.y) * kSbThreads;
-  for (int64_t j = static_cast<int64_t>(blockIdx.y) * kSbThreads + threadIdx.x; j < total; j += step) {
+  const int64_t step = static_cast<int64_t>(gridDim.y) * T;
+  for (int64_t j = static_cast<int64_t>(blockIdx.y) * T + threadIdx.x; j < total; j += step) {
     const unsigned ucol = static_cast<unsigned>(j) / static_cast<unsigned>(seg);  // j < 2^32 (host check)
     const int64_t col = ucol;
     const int64_t i = static_cast<unsigned>(j) - ucol * static_cast<unsigned>(seg);
@@ -385,12 +385,12 @@ csb_merge_parts(int P, const float2* __restrict__ part, float* __restrict__ wgra
   }
 }
 
-// Workgroups of `threads` threads per channel: about 2048 * 256 threads in total, each
-// thread with at least four vectors.
-static int csb_parts(int64_t C, int64_t vectors_per_channel, int threads = kSbThreads)
+// 256-thread workgroups per channel: about 2048 in total, each thread with at least four
+// vectors.
+static int csb_parts(int64_t C, int64_t vectors_per_channel)
 {
-  int64_t p = ceil_div(2048 * kSbThreads, C * threads);
-  const int64_t most = ceil_div(vectors_per_channel, 4 * threads);
+  int64_t p = ceil_div(2048, C);
+  const int64_t most = ceil_div(vectors_per_channel, 4 * kSbThreads);
   if (p > most) p = most;
   if (p > kSbMaxParts) p = kSbMaxParts;
   return static_cast<int>(p < 1 ? 1 : p);
@@ -496,10 +496,16 @@ int lbn_channelwise_scale_bias_fwd_f32(lbn_stream_t stream, int64_t num_channels
   hipStream_t st = as_stream(stream);
   const CsbArgs a{channel_size, width, x, nullptr, y, ldx, 0, ldy, weights, ld_weights, nullptr, 0, nullptr};
   const bool vec = csb_vec_ok(channel_size, width, x, ldx) && csb_vec_ok(channel_size, width, y, ldy);
-  const int P = csb_parts(num_channels, (vec ? channel_size / 4 : channel_size) * width);
+  const int64_t units = (vec ? channel_size / 4 : channel_size) * width;
+  // one 1024-thread workgroup per channel once there are enough channels to fill the device:
+  // measured 64.8 us against 69.7 us for eight 256-thread workgroups per channel (256 x 3136 x 64)
+  const bool big = units >= 4 * 1024 && num_channels >= 256;
+  const int P = big ? 1 : csb_parts(num_channels, units);
   const dim3 grid(static_cast<unsigned>(num_channels), static_cast<unsigned>(P));
-  if (vec) hipLaunchKernelGGL((csb_fwd<true>), grid, dim3(kSbThreads), 0, st, a);
-  else hipLaunchKernelGGL((csb_fwd<false>), grid, dim3(kSbThreads), 0, st, a);
+  if (vec && big) hipLaunchKernelGGL((csb_fwd<true, 1024>), grid, dim3(1024), 0, st, a);
+  else if (vec) hipLaunchKernelGGL((csb_fwd<true, kSbThreads>), grid, dim3(kSbThreads), 0, st, a);
+  else if (big) hipLaunchKernelGGL((csb_fwd<false, 1024>), grid, dim3(1024), 0, st, a);
+  else hipLaunchKernelGGL((csb_fwd<false, kSbThreads>), grid, dim3(kSbThreads), 0, st, a);
   return launch_status();
 }
 
