@@ -5,7 +5,7 @@
 // Channel c of an NCHW mini-batch is the row range [c*cs, (c+1)*cs) of every matrix
 // column, so a per-channel reduction crosses all columns: `width` segments of `cs`
 // contiguous floats.  The reduction is split over P workgroups per channel
-// (grid P x C) that walk the channel's segments with 128-bit coalesced loads and
+// (grid C x P) that walk the channel's segments with 128-bit coalesced loads and
 // leave one partial pair per workgroup in the workspace; the apply kernel (same
 // grid) merges the P partials in a fixed order in its prologue, workgroup 0 of each
 // channel writes the statistics, and all P workgroups stream the channel once more
@@ -47,9 +47,9 @@ bn_fwd_sums(const S* __restrict__ x, int64_t ldx, int64_t cs, int64_t w, int use
             float2* __restrict__ part)
 {
   __shared__ float red[2 * (kBnThreads / kWave)];
-  const int P = gridDim.x;
-  const int p = blockIdx.x;
-  const int64_t c = blockIdx.y;
+  const int P = gridDim.y;
+  const int p = blockIdx.y;
+  const int64_t c = blockIdx.x;
   const ChannelWalk wk = make_walk<S, VEC>(cs, w);
   using IO = Vec16<S>;
   constexpr int VE = IO::N;
@@ -150,9 +150,9 @@ bn_fwd_apply(const S* __restrict__ x, S* __restrict__ y, int64_t ldx, int64_t ld
              float* __restrict__ var_io, const float* __restrict__ gamma,
              const float* __restrict__ beta, float* __restrict__ rmean, float* __restrict__ rvar)
 {
-  const int P = gridDim.x;
-  const int p = blockIdx.x;
-  const int64_t c = blockIdx.y;
+  const int P = gridDim.y;
+  const int p = blockIdx.y;
+  const int64_t c = blockIdx.x;
   const ChannelWalk wk = make_walk<S, VEC>(cs, w);
   using IO = Vec16<S>;
   constexpr int VE = IO::N;
@@ -214,9 +214,9 @@ bn_bwd_sums(const S* __restrict__ x, const S* __restrict__ dy, int64_t ldx, int6
             int64_t cs, int64_t w, const float* __restrict__ mean_in, float2* __restrict__ part)
 {
   __shared__ float red[2 * (kBnThreads / kWave)];
-  const int P = gridDim.x;
-  const int p = blockIdx.x;
-  const int64_t c = blockIdx.y;
+  const int P = gridDim.y;
+  const int p = blockIdx.y;
+  const int64_t c = blockIdx.x;
   const ChannelWalk wk = make_walk<S, VEC>(cs, w);
   using IO = Vec16<S>;
   constexpr int VE = IO::N;
@@ -292,9 +292,9 @@ bn_bwd_apply(const S* __restrict__ x, const S* __restrict__ dy, S* __restrict__ 
              const float* __restrict__ gamma, float* __restrict__ dscale,
              float* __restrict__ dbias, float* __restrict__ dmean_io, float* __restrict__ dvar_io)
 {
-  const int P = gridDim.x;
-  const int p = blockIdx.x;
-  const int64_t c = blockIdx.y;
+  const int P = gridDim.y;
+  const int p = blockIdx.y;
+  const int64_t c = blockIdx.x;
   const ChannelWalk wk = make_walk<S, VEC>(cs, w);
   using IO = Vec16<S>;
   constexpr int VE = IO::N;
@@ -795,7 +795,7 @@ static int bn_check(int64_t C, int64_t cs, int64_t w, const int64_t* lds, int nl
   if (C < 0 || cs < 0 || w < 0) return LBN_ERR_INVALID_ARGUMENT;
   for (int i = 0; i < nld; ++i)
     if (w > 1 && lds[i] < C * cs) return LBN_ERR_INVALID_ARGUMENT;
-  if (C > 65535) return LBN_ERR_UNSUPPORTED;  // channels ride on gridDim.y
+  if (C >= (int64_t(1) << 31)) return LBN_ERR_UNSUPPORTED;  // channels ride on gridDim.x
   if (cs * w >= (int64_t(1) << 32)) return LBN_ERR_UNSUPPORTED;  // per-channel index fits 32 bits
   return LBN_OK;
 }
@@ -819,7 +819,7 @@ static int bn_fwd_apply_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, f
   if (C == 0 || cs == 0 || w == 0) return LBN_OK;
   if (!x || !y || !mean || !var || !scale || !bias) return LBN_ERR_INVALID_ARGUMENT;
   const int P = bn_split(C, cs, w);
-  const dim3 grid(P, static_cast<unsigned>(C));
+  const dim3 grid(static_cast<unsigned>(C), P);
   float* m = const_cast<float*>(mean);
   float* v = const_cast<float*>(var);
   if (bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, y, ldy))
@@ -849,7 +849,7 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
   const int P = bn_split(C, cs, w);
   float2* part = static_cast<float2*>(workspace);
-  const dim3 grid(P, static_cast<unsigned>(C));
+  const dim3 grid(static_cast<unsigned>(C), P);
   const int pivot = (flags & LBN_STATS_SUMSQ) ? 0 : 1;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, y, ldy);
   if (vec && bn_try_fwd_cluster<S>(st, C, cs, w, pivot, bessel, epsilon, decay, x, ldx, y, ldy, mean, var,
@@ -887,7 +887,7 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
   const int P = bn_split(C, cs, w);
   float2* part = static_cast<float2*>(workspace);
-  const dim3 grid(P, static_cast<unsigned>(C));
+  const dim3 grid(static_cast<unsigned>(C), P);
   const int64_t n = cs * w;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, dy, lddy) && bn_vec_ok<S>(cs, w, dx, lddx);
   if (training && vec &&
@@ -931,7 +931,7 @@ int lbn_batch_norm_fwd_sums_f32(lbn_stream_t stream, int64_t C, int64_t cs, int6
   if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
   const int P = bn_split(C, cs, w);
   float2* part = static_cast<float2*>(workspace);
-  const dim3 grid(P, static_cast<unsigned>(C));
+  const dim3 grid(static_cast<unsigned>(C), P);
   hipStream_t st = as_stream(stream);
   if (bn_vec_ok<float>(cs, w, x, ldx))
     hipLaunchKernelGGL((bn_fwd_sums<float, true>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, 0, part);
@@ -998,7 +998,7 @@ int lbn_batch_norm_bwd_sums_f32(lbn_stream_t stream, int64_t C, int64_t cs, int6
   if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
   const int P = bn_split(C, cs, w);
   float2* part = static_cast<float2*>(workspace);
-  const dim3 grid(P, static_cast<unsigned>(C));
+  const dim3 grid(static_cast<unsigned>(C), P);
   hipStream_t st = as_stream(stream);
   if (bn_vec_ok<float>(cs, w, x, ldx) && bn_vec_ok<float>(cs, w, dy, lddy))
     hipLaunchKernelGGL((bn_bwd_sums<float, true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, mean, part);
@@ -1020,7 +1020,7 @@ int lbn_batch_norm_bwd_apply_f32(lbn_stream_t stream, int64_t C, int64_t cs, int
   if (C == 0 || cs == 0 || w == 0) return LBN_OK;
   if (!x || !dy || !dx || !mean || !var || !scale || !dmean || !dvar) return LBN_ERR_INVALID_ARGUMENT;
   const int P = bn_split(C, cs, w);
-  const dim3 grid(P, static_cast<unsigned>(C));
+  const dim3 grid(static_cast<unsigned>(C), P);
   hipStream_t st = as_stream(stream);
   float* dm = const_cast<float*>(dmean);
   float* dv = const_cast<float*>(dvar);

@@ -282,7 +282,7 @@ BN_CASES = [
     ((7, 5, 3), 14, True, 0), ((7, 5, 3), 29, False, 0), ((8, 16, 16), 12, True, 0),
     ((256, 4, 4), 32, True, 0), ((3, 56, 56), 16, True, 0), ((16, 28, 28), 8, False, 0),
     ((5, 12), 10, True, 4), ((5, 13), 10, True, 0), ((2, 1), 1, True, 0), ((1, 100000), 3, True, 0),
-    ((70, 1), 50, True, 0),
+    ((70, 1), 50, True, 0), ((70000, 1), 3, True, 0),   # more channels than gridDim.y could hold
 ]
 
 
