@@ -21,6 +21,7 @@
 
 #include "device_utils.hpp"
 #include "host_utils.hpp"
+#include "layer_norm_long.hpp"
 
 namespace lbn {
 
@@ -660,12 +661,24 @@ static LnBwdPlan plan_ln_bwd(int64_t nvec, int64_t rows, int ve)
   return p;
 }
 
+// Row slabs of ln_wgrad_columns: about 2048 workgroups in total, at most one slab per row.
+static int64_t ln_wgrad_slabs(int64_t units, int64_t rows)
+{
+  int64_t s = ceil_div(2048, ceil_div(units, 256));
+  if (s > rows) s = rows;
+  if (s > 256) s = 256;
+  return s < 1 ? 1 : s;
+}
+
 static size_t ln_bwd_workspace(int64_t n, int64_t rows, int ve)
 {
-  if (n <= 0 || rows <= 0 || n % ve != 0) return 0;
-  const LnBwdPlan p = plan_ln_bwd(n / ve, rows, ve);
-  if (!p.tpr) return 0;
-  return static_cast<size_t>(p.blocks) * 2 * n * sizeof(float);
+  if (n <= 0 || rows <= 0) return 0;
+  if (n % ve == 0) {
+    const LnBwdPlan p = plan_ln_bwd(n / ve, rows, ve);
+    if (p.tpr) return static_cast<size_t>(p.blocks) * 2 * n * sizeof(float);
+    return static_cast<size_t>(ln_wgrad_slabs(n / ve, rows)) * 2 * n * sizeof(float);
+  }
+  return static_cast<size_t>(ln_wgrad_slabs(n, rows)) * 2 * n * sizeof(float);
 }
 
 template <typename T>
@@ -708,6 +721,10 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
       if constexpr (VE == 4) { X(1024, 8) }
 #undef X
     }
+    // longer than the register kernels hold
+    hipLaunchKernelGGL((ln_fwd_long<T>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st, x, y,
+                       ldx, ldy, map, n / VE, 1.0f / static_cast<float>(n), eps, stats, lds, gamma, beta, sumsq);
+    return launch_status();
   }
   hipLaunchKernelGGL((ln_fwd_generic<T>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, st, x, y,
                      ldx, ldy, map, n, eps, stats, lds, gamma, beta, sumsq);
@@ -803,12 +820,41 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
         return launch_status();
       }
     }
+    // longer than the register kernels hold
+    hipLaunchKernelGGL((ln_bwd_long<T>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st, x, dy,
+                       dx, ldx, lddy, lddx, map, n / VE, 1.0f / static_cast<float>(n), eps, stats, lds, sgrad,
+                       ldsg, gamma);
   }
-  hipLaunchKernelGGL((ln_bwd_generic<T>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, st, x, dy,
-                     dx, ldx, lddy, lddx, map, n, eps, stats, lds, sgrad, ldsg, gamma);
-  if (wgrad)
-    hipLaunchKernelGGL((ln_wgrad_generic<T>), dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256),
-                       0, st, x, dy, ldx, lddy, map, rows, n, eps, stats, lds, dgamma, dbeta);
+  else {
+    hipLaunchKernelGGL((ln_bwd_generic<T>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, st, x, dy,
+                       dx, ldx, lddy, lddx, map, n, eps, stats, lds, sgrad, ldsg, gamma);
+  }
+  if (wgrad) {
+    // weight gradients of the two paths above: row slabs -> partial rows -> fixed-order sum
+    const int64_t units = vec ? n / VE : n;
+    const int64_t slabs = ln_wgrad_slabs(units, rows);
+    if (ws && aligned16(ws) && ws_bytes >= static_cast<size_t>(slabs) * 2 * n * sizeof(float)) {
+      float* wpart = static_cast<float*>(ws);
+      const dim3 grid(static_cast<unsigned>(ceil_div(units, 256)), static_cast<unsigned>(slabs));
+      if (vec)
+        hipLaunchKernelGGL((ln_wgrad_columns<T, true>), grid, dim3(256), 0, st, x, dy, ldx, lddy, map, rows,
+                           units, n, eps, stats, lds, wpart);
+      else
+        hipLaunchKernelGGL((ln_wgrad_columns<T, false>), grid, dim3(256), 0, st, x, dy, ldx, lddy, map, rows,
+                           units, n, eps, stats, lds, wpart);
+      if (n % 4 == 0)
+        hipLaunchKernelGGL(ln_wgrad_reduce, dim3(static_cast<unsigned>(ceil_div(n, 32)), 2), dim3(256), 0, st,
+                           wpart, slabs, n, dgamma, dbeta);
+      else
+        hipLaunchKernelGGL(ln_wgrad_reduce_scalar, dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0,
+                           st, wpart, slabs, n, dgamma, dbeta);
+    }
+    else {
+      // no scratch: one thread per feature walks every row
+      hipLaunchKernelGGL((ln_wgrad_generic<T>), dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256),
+                         0, st, x, dy, ldx, lddy, map, rows, n, eps, stats, lds, dgamma, dbeta);
+    }
+  }
   return launch_status();
 }
 

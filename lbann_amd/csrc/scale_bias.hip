@@ -250,7 +250,7 @@ static int sb_check(int64_t h, int64_t w, const int64_t* lds, int nld)
   if (h < 0 || w < 0) return LBN_ERR_INVALID_ARGUMENT;
   for (int i = 0; i < nld; ++i)
     if (w > 1 && lds[i] < h) return LBN_ERR_INVALID_ARGUMENT;
-  if (h > (int64_t(1) << 40) || w > (int64_t(1) << 40)) return LBN_ERR_UNSUPPORTED;
+  if (h > (int64_t(1) << 36) || w > (int64_t(1) << 40)) return LBN_ERR_UNSUPPORTED;  // 64 rows per workgroup, gridDim.x < 2^31
   return LBN_OK;
 }
 

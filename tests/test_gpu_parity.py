@@ -152,6 +152,10 @@ LN_CASES = [
     # short rows (more than 256 persistent blocks), teams that leave threads idle
     ((12288,), 0, 5, True, 0), ((8192,), 0, 600, True, 0), ((768,), 0, 3000, True, 0),
     ((256,), 0, 70000, True, 0), ((5000,), 0, 40, True, 0),
+    # rows longer than the register kernels hold: one 1024-thread workgroup per row, weight
+    # gradients by row slabs (vector and scalar), groups, padded leading dimension
+    ((150528,), 0, 6, True, 0), ((65536,), 0, 300, True, 0), ((4, 20000), -1, 9, True, 0),
+    ((20001,), 0, 7, True, 0), ((20004,), 0, 5, True, 4), ((3, 224, 224), 0, 3, False, 0),
 ]
 
 
@@ -200,7 +204,7 @@ def test_layer_norm_f32(L, dims, start_dim, w, affine, pad):
     _ln_run(L, x, dy, dims, start_dim, affine, pad, scale, bias)
 
 
-@pytest.mark.parametrize("dims,start_dim,w", [((1024,), 0, 64), ((31,), 0, 15), ((8, 512), -1, 9)])
+@pytest.mark.parametrize("dims,start_dim,w", [((1024,), 0, 64), ((31,), 0, 15), ((8, 512), -1, 9), ((40000,), 0, 4)])
 def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
     """E[x^2]-mean^2 mode reproduces the reference's variance, clamp included."""
     rng = np.random.default_rng(5)
@@ -213,7 +217,8 @@ def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
 @pytest.mark.parametrize("dims,start_dim,w,pad", [((4096,), 0, 64, 0), ((512,), 0, 100, 0), ((64,), 0, 9, 0),
                                                    ((8, 1024), -1, 5, 0), ((100,), 0, 7, 0), ((2048,), 0, 600, 8),
                                                    ((16384,), 0, 3, 0), ((16384,), 0, 40, 0), ((8192,), 0, 300, 0),
-                                                   ((768,), 0, 1000, 0), ((12288,), 0, 9, 0)])
+                                                   ((768,), 0, 1000, 0), ((12288,), 0, 9, 0),
+                                                   ((32768,), 0, 20, 0), ((150528,), 0, 3, 0), ((20000,), 0, 5, 8)])
 def test_layer_norm_f16(L, dims, start_dim, w, pad):
     rng = np.random.default_rng(int(np.prod(dims)) * 3 + w)
     h = int(np.prod(dims))
@@ -228,7 +233,7 @@ def test_layer_norm_f16(L, dims, start_dim, w, pad):
 # ===================================================================== instance norm
 @pytest.mark.parametrize("dims,w,pad", [((5, 3, 7), 15, 0), ((64, 56, 56), 6, 0), ((8, 1024), 33, 0),
                                         ((3, 100000), 2, 0), ((7, 1), 5, 0), ((16, 31), 40, 4),
-                                        ((256, 16, 16), 64, 0)])
+                                        ((256, 16, 16), 64, 0), ((3, 224, 224), 8, 0), ((2, 64, 64, 64), 2, 0)])
 def test_instance_norm(L, dims, w, pad):
     rng = np.random.default_rng(int(np.prod(dims)) + 7 * w)
     h = int(np.prod(dims))
