@@ -15,9 +15,13 @@
 // entry), sum(x-K) and sum((x-K)^2), which removes the cancellation of
 // E[x^2]-mean^2 when |mean| >> stdev at no extra cost; LBN_STATS_SUMSQ selects
 // K = 0, the reference's formula (batch_normalization.cpp:70-85, :124-128).
+#include <type_traits>
+
 #include "cluster_sync.hpp"
 #include "device_utils.hpp"
 #include "host_utils.hpp"
+#include "batch_norm_math.hpp"
+#include "batch_norm_rows.hpp"
 
 namespace lbn {
 
@@ -92,19 +96,6 @@ __device__ __forceinline__ float2 merge_partials(const float2* part, int64_t c, 
     b = v.y;
   }
   return make_float2(wave_sum(a), wave_sum(b));
-}
-
-// Mean / variance from sums about pivot K over n values, with the reference's Bessel
-// factor and epsilon floor (batch_normalization.cpp:118-131).
-__device__ __forceinline__ void stats_from_sums(float s, float q, float K, int64_t n, int bessel,
-                                                float eps, float& mean, float& var)
-{
-  const float nf = static_cast<float>(n);
-  const float dm = s / nf;
-  const float sqmean = q / nf;
-  mean = K + dm;
-  var = nf * (sqmean - dm * dm) / (nf - static_cast<float>(bessel ? 1 : 0));
-  var = fmaxf(var, eps);
 }
 
 // Raw per-channel sums for callers that all-reduce them: mean[c] = sum, var[c] = sqsum.
@@ -247,16 +238,6 @@ bn_bwd_sums(const S* __restrict__ x, const S* __restrict__ dy, int64_t ldx, int6
   }
   team_sum2<kBnThreads / kWave>(a, b, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
   if (threadIdx.x == 0) part[c * P + p] = make_float2(a, b);
-}
-
-__device__ __forceinline__ void grads_from_sums(float A, float B, float scale, float inv_stdev,
-                                                float& dscale, float& dbias, float& dmean,
-                                                float& dvar)
-{
-  dscale = B * inv_stdev;
-  dbias = A;
-  dmean = -(scale * inv_stdev) * A;
-  dvar = -scale * B * (inv_stdev * inv_stdev * inv_stdev / 2);
 }
 
 __global__ void __launch_bounds__(kWave)
@@ -710,7 +691,12 @@ static size_t bn_workspace(int64_t C, int64_t cs, int64_t w)
   if (C <= 0 || cs <= 0 || w <= 0) return 0;
   const size_t split = static_cast<size_t>(C) * bn_split(C, cs, w) * sizeof(float2);
   const size_t cluster = cluster_workspace_bytes(C);
-  return split > cluster ? split : cluster;
+  size_t need = split > cluster ? split : cluster;
+  if (cs % 4 != 0 && (C * cs) % 4 == 0) {  // the row-tile path of batch_norm_rows.hpp
+    const size_t rows = bn_rt_workspace_bytes(C * cs, w);
+    if (rows > need) need = rows;
+  }
+  return need;
 }
 
 // Launches the register-resident forward when the shape allows it.  Returns false
@@ -807,6 +793,29 @@ static bool bn_vec_ok(int64_t cs, int64_t w, const void* a, int64_t lda)
   return cs % VE == 0 && aligned16(a) && (w <= 1 || lda % VE == 0);
 }
 
+// ---- channels that are not whole 16-byte vectors, on a matrix whose row quads are aligned
+// (batch_norm_rows.hpp).  fp32 only.
+static bool bn_rt_usable(int64_t C, int64_t cs, int64_t w, const void* a, int64_t lda)
+{
+  return cs % 4 != 0 && row_quads_ok(C * cs, w, a, lda);
+}
+
+template <bool BWD>
+static void bn_rt_launch_sums(hipStream_t st, const RowTilePlan& p, const BnRtArgs& a)
+{
+  const dim3 grid(static_cast<unsigned>(p.tiles), static_cast<unsigned>(p.slabs));
+  if (p.gw == 1) hipLaunchKernelGGL((bn_rt_sums<1, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
+  else hipLaunchKernelGGL((bn_rt_sums<4, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
+}
+
+template <bool BWD>
+static void bn_rt_launch_apply(hipStream_t st, const RowTilePlan& p, const BnRtArgs& a)
+{
+  const dim3 grid(static_cast<unsigned>(p.tiles), static_cast<unsigned>(p.slabs));
+  if (p.gw == 1) hipLaunchKernelGGL((bn_rt_apply<1, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
+  else hipLaunchKernelGGL((bn_rt_apply<4, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
+}
+
 // Forward with given statistics (inference mode, and the last step of a caller that
 // reduces the statistics over ranks itself).
 template <typename S>
@@ -818,6 +827,16 @@ static int bn_fwd_apply_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, f
   if (int e = bn_check(C, cs, w, lds, 2)) return e;
   if (C == 0 || cs == 0 || w == 0) return LBN_OK;
   if (!x || !y || !mean || !var || !scale || !bias) return LBN_ERR_INVALID_ARGUMENT;
+  if constexpr (std::is_same<S, float>::value) {
+    if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, y, ldy)) {
+      const RowTilePlan p = row_tile_plan(C * cs, w);
+      BnRtArgs a{};
+      a.h = C * cs, a.w = w, a.cs = cs, a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy;
+      a.slab_width = p.slab_width, a.eps = epsilon, a.mean = mean, a.var = var, a.scale = scale, a.bias = bias;
+      bn_rt_launch_apply<false>(st, p, a);
+      return launch_status();
+    }
+  }
   const int P = bn_split(C, cs, w);
   const dim3 grid(static_cast<unsigned>(C), P);
   float* m = const_cast<float*>(mean);
@@ -855,6 +874,23 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   if (vec && bn_try_fwd_cluster<S>(st, C, cs, w, pivot, bessel, epsilon, decay, x, ldx, y, ldy, mean, var,
                                    scale, bias, running_mean, running_var, workspace))
     return launch_status();
+  if constexpr (std::is_same<S, float>::value) {
+    if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, y, ldy) &&
+        (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0) {
+      const int64_t h = C * cs;
+      const RowTilePlan p = row_tile_plan(h, w);
+      BnRtArgs a{};
+      a.h = h, a.w = w, a.cs = cs, a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy;
+      a.slab_width = p.slab_width, a.part = part, a.use_pivot = pivot, a.eps = epsilon;
+      a.mean = mean, a.var = var, a.scale = scale, a.bias = bias;
+      bn_rt_launch_sums<false>(st, p, a);
+      hipLaunchKernelGGL(bn_rt_fwd_stats, dim3(static_cast<unsigned>(ceil_div(C, kRowTileWaves))),
+                         dim3(kRowTileThreads), 0, st, C, cs, w, h, p.slabs, part, x, pivot, bessel, epsilon,
+                         decay, mean, var, running_mean, running_var);
+      bn_rt_launch_apply<false>(st, p, a);
+      return launch_status();
+    }
+  }
   if (vec) {
     hipLaunchKernelGGL((bn_fwd_sums<S, true>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, pivot, part);
     hipLaunchKernelGGL((bn_fwd_apply<S, true, true>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs, w,
@@ -894,6 +930,25 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
       bn_try_bwd_cluster<S>(st, C, cs, w, bessel, epsilon, x, ldx, dy, lddy, dx, lddx, use_mean, use_var,
                             scale, dscale, dbias, dmean, dvar, workspace))
     return launch_status();
+  if constexpr (std::is_same<S, float>::value) {
+    if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, dy, lddy) && bn_rt_usable(C, cs, w, dx, lddx) &&
+        (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0) {
+      const int64_t h = C * cs;
+      const RowTilePlan p = row_tile_plan(h, w);
+      BnRtArgs a{};
+      a.h = h, a.w = w, a.cs = cs, a.x = x, a.dy = dy, a.out = dx, a.ldx = ldx, a.lddy = lddy, a.ldo = lddx;
+      a.slab_width = p.slab_width, a.part = part, a.eps = epsilon;
+      a.mean = use_mean, a.var = use_var, a.scale = scale, a.dmean = dmean, a.dvar = dvar;
+      a.count = static_cast<float>(n), a.count_bessel = static_cast<float>(n - (bessel ? 1 : 0));
+      a.zero = n <= 1;
+      bn_rt_launch_sums<true>(st, p, a);
+      hipLaunchKernelGGL(bn_rt_bwd_stats, dim3(static_cast<unsigned>(ceil_div(C, kRowTileWaves))),
+                         dim3(kRowTileThreads), 0, st, C, cs, h, p.slabs, part, epsilon, training, use_var, scale,
+                         dscale, dbias, dmean, dvar);
+      bn_rt_launch_apply<true>(st, p, a);
+      return launch_status();
+    }
+  }
   if (vec) {
     hipLaunchKernelGGL((bn_bwd_sums<S, true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean, part);
     hipLaunchKernelGGL((bn_bwd_apply<S, true, true>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,

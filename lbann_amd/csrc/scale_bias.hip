@@ -22,6 +22,7 @@
 // not depend on scheduling.
 #include "device_utils.hpp"
 #include "host_utils.hpp"
+#include "row_tiles.hpp"
 
 namespace lbn {
 
@@ -44,20 +45,8 @@ struct EsbArgs {
   int64_t slab_width;
 };
 
-// Thread (row quad q, column group g) of a block; GW column groups share a wave.
 template <int GW>
-struct EsbPos {
-  static constexpr int kQuads = kWave / GW;
-  static constexpr int kRows = 4 * kQuads;
-  static constexpr int kGroups = kSbWaves * GW;
-  int q, g;
-  __device__ __forceinline__ EsbPos()
-  {
-    const int lane = threadIdx.x & (kWave - 1);
-    q = lane & (kQuads - 1);
-    g = lane / kQuads + GW * (threadIdx.x / kWave);
-  }
-};
+using EsbPos = RowTilePos<GW>;
 
 template <int GW>
 __global__ void __launch_bounds__(kSbThreads)
@@ -140,38 +129,8 @@ esb_bwd_tile(EsbArgs a)
     }
     Vec16<float>::store(a.out + rr + c * a.ldo, d);
   }
-  // merge the column groups: inside a wave by lane exchange, across waves through LDS
-  if (GW == 4) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      da[r] += __shfl_xor(da[r], 16);
-      db[r] += __shfl_xor(db[r], 16);
-      da[r] += __shfl_xor(da[r], 32);
-      db[r] += __shfl_xor(db[r], 32);
-    }
-  }
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
-  if (lane < P::kQuads) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      lds[wave][4 * p.q + r][0] = da[r];
-      lds[wave][4 * p.q + r][1] = db[r];
-    }
-  }
-  __syncthreads();
+  row_tile_merge<GW>(da, db, lds, p);
   if (p.g != 0 || !row_ok) return;
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    float sa = 0.f, sb = 0.f;
-#pragma unroll
-    for (int k = 0; k < kSbWaves; ++k) {
-      sa += lds[k][4 * p.q + r][0];
-      sb += lds[k][4 * p.q + r][1];
-    }
-    da[r] = sa;
-    db[r] = sb;
-  }
   if (gridDim.y == 1) {
     Vec16<float>::store(a.wgrad + r0, da);
     Vec16<float>::store(a.wgrad + r0 + a.ld_wgrad, db);
@@ -229,21 +188,7 @@ esb_bwd_generic(EsbArgs a)
   a.wgrad[r + a.ld_wgrad] = db;
 }
 
-// Column slabs for a launch of `row_tiles` workgroups per slab: enough slabs to give the
-// device about four workgroups per compute unit, each slab at least `min_width` wide.
-static int esb_slabs(int64_t row_tiles, int64_t w, int64_t min_width)
-{
-  const int64_t want = ceil_div(1024, row_tiles);
-  const int64_t most = w / min_width > 1 ? w / min_width : 1;
-  int64_t s = want < most ? want : most;
-  if (s > kSbMaxParts) s = kSbMaxParts;
-  return static_cast<int>(s < 1 ? 1 : s);
-}
-
-static bool sb_vec_ok(int64_t h, int64_t w, const void* p, int64_t ld)
-{
-  return h % 4 == 0 && aligned16(p) && (w <= 1 || ld % 4 == 0);
-}
+static bool sb_vec_ok(int64_t h, int64_t w, const void* p, int64_t ld) { return row_quads_ok(h, w, p, ld); }
 
 static int sb_check(int64_t h, int64_t w, const int64_t* lds, int nld)
 {
@@ -252,27 +197,6 @@ static int sb_check(int64_t h, int64_t w, const int64_t* lds, int nld)
     if (w > 1 && lds[i] < h) return LBN_ERR_INVALID_ARGUMENT;
   if (h > (int64_t(1) << 36) || w > (int64_t(1) << 40)) return LBN_ERR_UNSUPPORTED;  // 64 rows per workgroup, gridDim.x < 2^31
   return LBN_OK;
-}
-
-// Launch shape of the tile kernels.  Sixteen column groups over 64 rows (GW = 4) measured
-// 4-8 % faster than four groups over 256 rows on 1048576 x 64 and 802816 x 64 matrices;
-// mini-batches narrower than 16 columns would leave most of those groups idle and take
-// GW = 1.
-struct EsbPlan {
-  int gw;
-  int64_t tiles;
-  int slabs;
-  int64_t slab_width;
-};
-
-static EsbPlan esb_plan(int64_t h, int64_t w)
-{
-  EsbPlan p;
-  p.gw = w >= 16 ? 4 : 1;
-  p.tiles = ceil_div(h, p.gw == 1 ? EsbPos<1>::kRows : EsbPos<4>::kRows);
-  p.slab_width = ceil_div(w, esb_slabs(p.tiles, w, 4 * kSbWaves * p.gw));
-  p.slabs = static_cast<int>(ceil_div(w, p.slab_width));
-  return p;
 }
 
 // =================================================================== channel-wise
@@ -429,7 +353,7 @@ int lbn_entrywise_scale_bias_fwd_f32(lbn_stream_t stream, int64_t height, int64_
   EsbArgs a{height, width, x, nullptr, y, ldx, 0, ldy, weights, ld_weights, nullptr, 0, nullptr, width};
   if (sb_vec_ok(height, width, x, ldx) && sb_vec_ok(height, width, y, ldy) && aligned16(weights) &&
       ld_weights % 4 == 0) {
-    const EsbPlan p = esb_plan(height, width);
+    const RowTilePlan p = row_tile_plan(height, width);
     a.slab_width = p.slab_width;
     const dim3 grid(static_cast<unsigned>(p.tiles), static_cast<unsigned>(p.slabs));
     if (p.gw == 1) hipLaunchKernelGGL((esb_fwd_tile<1>), grid, dim3(kSbThreads), 0, st, a);
@@ -437,7 +361,10 @@ int lbn_entrywise_scale_bias_fwd_f32(lbn_stream_t stream, int64_t height, int64_
     return launch_status();
   }
   const int64_t tiles = ceil_div(height, 256);
-  a.slab_width = ceil_div(width, esb_slabs(tiles, width, 8));
+  int64_t slabs = ceil_div(1024, tiles);  // as in row_tile_plan, slabs of at least 8 columns
+  if (slabs > width / 8) slabs = width / 8;
+  if (slabs > kRowTileMaxSlabs) slabs = kRowTileMaxSlabs;
+  a.slab_width = ceil_div(width, slabs < 1 ? 1 : slabs);
   const dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(ceil_div(width, a.slab_width)));
   hipLaunchKernelGGL(esb_fwd_generic, grid, dim3(256), 0, st, a);
   return launch_status();
@@ -446,7 +373,7 @@ int lbn_entrywise_scale_bias_fwd_f32(lbn_stream_t stream, int64_t height, int64_
 size_t lbn_entrywise_scale_bias_bwd_workspace_bytes(int64_t height, int64_t width)
 {
   if (height <= 0 || width <= 0) return 0;
-  const EsbPlan p = esb_plan(height, width);
+  const RowTilePlan p = row_tile_plan(height, width);
   return p.slabs > 1 ? static_cast<size_t>(p.slabs) * static_cast<size_t>(height) * sizeof(float2) : 0;
 }
 
@@ -467,7 +394,7 @@ int lbn_entrywise_scale_bias_bwd_f32(lbn_stream_t stream, int64_t height, int64_
   if (sb_vec_ok(height, width, x, ldx) && sb_vec_ok(height, width, dy, lddy) &&
       sb_vec_ok(height, width, dx, lddx) && aligned16(weights) && aligned16(weights_grad) &&
       ld_weights_grad % 4 == 0) {
-    const EsbPlan p = esb_plan(height, width);
+    const RowTilePlan p = row_tile_plan(height, width);
     const int slabs = p.slabs;
     a.slab_width = p.slab_width;
     if (slabs > 1 && (!workspace || !aligned16(workspace) ||

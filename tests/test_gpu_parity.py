@@ -288,6 +288,9 @@ BN_CASES = [
     ((256, 4, 4), 32, True, 0), ((3, 56, 56), 16, True, 0), ((16, 28, 28), 8, False, 0),
     ((5, 12), 10, True, 4), ((5, 13), 10, True, 0), ((2, 1), 1, True, 0), ((1, 100000), 3, True, 0),
     ((70, 1), 50, True, 0), ((70000, 1), 3, True, 0),   # more channels than gridDim.y could hold
+    # channels that are not whole 16-byte vectors on a quad-aligned matrix: row-tile kernels
+    ((2048, 7, 7), 16, True, 0), ((4096,), 64, True, 0), ((64, 7, 7), 300, False, 0), ((12, 3, 3), 20, True, 0),
+    ((8, 5), 7, True, 4), ((4, 1), 1, True, 0), ((1024, 1), 2048, True, 0),
 ]
 
 
@@ -361,6 +364,16 @@ def test_batch_norm_inference_and_reference_formula(L):
     _bn_run(L, x, dy, dims, True, 0, scale, bias, training=False)
     _bn_run(L, x, dy, dims, True, 0, scale, bias, mode=L.LBN_STATS_SUMSQ)
     _bn_run(L, x, dy, dims, True, 0, scale, bias)
+    # the same three modes through the row-tile kernels (7 x 7 channels)
+    dims, w = (16, 7, 7), 12
+    h = int(np.prod(dims))
+    x, dy = rand(rng, h, w, 2.0, 3.0), rand(rng, h, w)
+    x[:49, :] = 4.0
+    scale = rng.uniform(0.5, 1.5, 16).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(16)).astype(np.float32)
+    _bn_run(L, x, dy, dims, True, 0, scale, bias, training=False)
+    _bn_run(L, x, dy, dims, True, 0, scale, bias, mode=L.LBN_STATS_SUMSQ)
+    _bn_run(L, x, dy, dims, False, 0, scale, bias)
 
 
 def test_batch_norm_split_entry_points(L):
