@@ -28,8 +28,34 @@ enum SmKind : int { kSoftmax = 0, kLogSoftmax = 1, kChannelwise = 2 };
 constexpr int kMaxChunks = 64;  // S <= one wave, so a wave merges the partials of a row
 
 // ======================================================= register-resident rows
+// Access unit of the row kernels: W = 4 is a 16-byte vector (rows start on 16-byte
+// boundaries and their length is a multiple of 4), W = 1 a single float for rows that are
+// only 4-byte aligned (odd lengths such as 197 or 1001): a wave instruction then still
+// reads 256 contiguous bytes.
+template <int W>
+struct RowIO;
+template <>
+struct RowIO<4> {
+  template <bool STREAM>
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4])
+  {
+    if (STREAM) Vec16<float>::load_stream(p, v);
+    else Vec16<float>::load(p, v);
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) { Vec16<float>::store(p, v); }
+};
+template <>
+struct RowIO<1> {
+  template <bool STREAM>
+  static __device__ __forceinline__ void load(const float* p, float (&v)[1])
+  {
+    v[0] = *p;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[1]) { *p = v[0]; }
+};
+
 // 1024-thread blocks are held to 64 registers so that two of them share a compute unit.
-template <int TPR, int V, int KIND, bool STREAM>
+template <int TPR, int V, int KIND, bool STREAM, int W = 4>
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads, (TPR == 1024 ? 8 : 1))
 sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
             unsigned nvec)
@@ -46,17 +72,16 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
   if (B::kTeams > 1 && row >= rows) return;  // whole waves leave; no barrier below in that case
 
   const float* xr = x + map.offset(row, ldx);
-  float v[V][4];
+  float v[V][W];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      if (STREAM) Vec16<float>::load_stream(xr + 4u * idx, v[i]);
-      else Vec16<float>::load(xr + 4u * idx, v[i]);
+      RowIO<W>::template load<STREAM>(xr + unsigned(W) * idx, v[i]);
     }
     else {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) v[i][k] = -FLT_MAX;
+      for (int k = 0; k < W; ++k) v[i][k] = -FLT_MAX;
     }
   }
 
@@ -68,14 +93,14 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
 #pragma unroll
   for (int i = 0; i < V; ++i)
 #pragma unroll
-    for (int k = 0; k < 4; ++k) m = fmaxf(m, v[i][k]);
+    for (int k = 0; k < W; ++k) m = fmaxf(m, v[i][k]);
 
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const bool ok = (t + i * TPR) < nvec;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < W; ++k) {
       const float d = v[i][k] - m;
       float e;
       if (KIND == kLogSoftmax) e = exp_quick(d);  // only summed: x stays in the registers for the output
@@ -111,7 +136,7 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
+      for (int k = 0; k < W; ++k) {
         if (KIND == kSoftmax) {
           const float r = f * v[i][k];
           v[i][k] = __builtin_isnormal(r) ? r : 0.f;
@@ -123,13 +148,13 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
           v[i][k] *= f;
         }
       }
-      Vec16<float>::store(yr + 4u * idx, v[i]);
+      RowIO<W>::store(yr + unsigned(W) * idx, v[i]);
     }
   }
 }
 
 // softmax / channelwise: dx = y * (dy - dot(y, dy));  log-softmax: dx = dy - exp(y) * sum(dy)
-template <int TPR, int V, int KIND, bool STREAM>
+template <int TPR, int V, int KIND, bool STREAM, int W = 4>
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
 sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
             RowMap map, int64_t rows, unsigned nvec)
@@ -147,30 +172,24 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
 
   const float* yr = y + map.offset(row, ldy);
   const float* gr = dy + map.offset(row, lddy);
-  float a[V][4], g[V][4];
+  float a[V][W], g[V][W];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      if (STREAM) {
-        Vec16<float>::load_stream(yr + 4u * idx, a[i]);
-        Vec16<float>::load_stream(gr + 4u * idx, g[i]);
-      }
-      else {
-        Vec16<float>::load(yr + 4u * idx, a[i]);
-        Vec16<float>::load(gr + 4u * idx, g[i]);
-      }
+      RowIO<W>::template load<STREAM>(yr + unsigned(W) * idx, a[i]);
+      RowIO<W>::template load<STREAM>(gr + unsigned(W) * idx, g[i]);
     }
     else {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) a[i][k] = g[i][k] = 0.f;
+      for (int k = 0; k < W; ++k) a[i][k] = g[i][k] = 0.f;
     }
   }
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i)
 #pragma unroll
-    for (int k = 0; k < 4; ++k) s += (KIND == kLogSoftmax) ? g[i][k] : a[i][k] * g[i][k];
+    for (int k = 0; k < W; ++k) s += (KIND == kLogSoftmax) ? g[i][k] : a[i][k] * g[i][k];
   s = team_sum<NW>(s, red, wv, lane);
 
   float* dr = dx + map.offset(row, lddx);
@@ -179,11 +198,11 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
+      for (int k = 0; k < W; ++k) {
         if (KIND == kLogSoftmax) g[i][k] = g[i][k] - exp_fast(a[i][k]) * s;
         else g[i][k] = a[i][k] * (g[i][k] - s);
       }
-      Vec16<float>::store(dr + 4u * idx, g[i]);
+      RowIO<W>::store(dr + unsigned(W) * idx, g[i]);
     }
   }
 }
@@ -462,6 +481,66 @@ __device__ __forceinline__ void block_merge_max_sum(float& m, float& acc, float 
   acc = bs;
 }
 
+// A run of `len` floats at p, cut at 16-byte boundaries: `head` leading scalars, `nvec`
+// aligned vectors, `tail` trailing scalars.  Rows whose starts are only 4-byte aligned
+// (odd lengths, e.g. a vocabulary of 50257 entries) still move almost all of their bytes
+// with 16-byte accesses this way.
+struct Peel {
+  int head, tail;
+  int64_t nvec;
+  // index (relative to p) of the edge scalar thread t handles, for t < head + tail
+  __device__ __forceinline__ int64_t edge(int t) const { return t < head ? t : head + 4 * nvec + (t - head); }
+};
+
+__device__ __forceinline__ Peel peel16(const float* p, int64_t len)
+{
+  Peel r;
+  r.head = static_cast<int>((4 - ((reinterpret_cast<uintptr_t>(p) >> 2) & 3)) & 3);
+  if (r.head > len) r.head = static_cast<int>(len);
+  r.nvec = (len - r.head) / 4;
+  r.tail = static_cast<int>(len - r.head - 4 * r.nvec);
+  return r;
+}
+
+__device__ __forceinline__ bool same_phase16(const void* a, const void* b)
+{
+  return ((reinterpret_cast<uintptr_t>(a) ^ reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
+}
+
+// Online (max, sum of exp) over nvec aligned vectors at base, strided over the workgroup;
+// four independent 16-byte loads per thread are in flight before any is used.
+__device__ __forceinline__ void sm_reduce_vectors(const float* base, int64_t nvec, float& m, float& acc)
+{
+  for (int64_t i0 = threadIdx.x; i0 < nvec; i0 += kChunkUnroll * kChunkThreads) {
+    float v[kChunkUnroll][4];
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+      if (i < nvec) {
+        Vec16<float>::load(base + 4 * i, v[u]);
+      }
+      else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[u][k] = -FLT_MAX;
+      }
+    }
+    float mn = m;
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) mn = fmaxf(mn, v[u][k]);
+    float add = 0.f;
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const bool ok = i0 + u * kChunkThreads < nvec;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) add += ok ? exp_fast(v[u][k] - mn) : 0.f;
+    }
+    acc = acc * exp_fast(m - mn) + add;
+    m = mn;
+  }
+}
+
 template <bool VEC>
 __global__ void __launch_bounds__(kChunkThreads)
 sm_fwd_partial(const float* x, int64_t ldx, RowMap map, int64_t n, int64_t chunk, int S,
@@ -472,49 +551,44 @@ sm_fwd_partial(const float* x, int64_t ldx, RowMap map, int64_t n, int64_t chunk
   const int s = blockIdx.x - row * S;
   const int64_t begin = s * chunk;
   const int64_t end = imin64(n, begin + chunk);
-  const float* xr = x + map.offset(row, ldx);
+  const float* p = x + map.offset(row, ldx) + begin;
   float m = -FLT_MAX, acc = 0.f;
   if (VEC) {
-    // four independent 16-byte loads per thread are in flight before any is used
-    for (int64_t i0 = begin / 4 + threadIdx.x; i0 < end / 4; i0 += kChunkUnroll * kChunkThreads) {
-      float v[kChunkUnroll][4];
-#pragma unroll
-      for (int u = 0; u < kChunkUnroll; ++u) {
-        const int64_t i = i0 + u * kChunkThreads;
-        if (i < end / 4) {
-          Vec16<float>::load(xr + 4 * i, v[u]);
-        }
-        else {
-#pragma unroll
-          for (int k = 0; k < 4; ++k) v[u][k] = -FLT_MAX;
-        }
-      }
-      float mn = m;
-#pragma unroll
-      for (int u = 0; u < kChunkUnroll; ++u)
-#pragma unroll
-        for (int k = 0; k < 4; ++k) mn = fmaxf(mn, v[u][k]);
-      float add = 0.f;
-#pragma unroll
-      for (int u = 0; u < kChunkUnroll; ++u) {
-        const bool ok = i0 + u * kChunkThreads < end / 4;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) add += ok ? exp_fast(v[u][k] - mn) : 0.f;
-      }
-      acc = acc * exp_fast(m - mn) + add;
-      m = mn;
-    }
+    sm_reduce_vectors(p, (end - begin) / 4, m, acc);
   }
   else {
-    for (int64_t i = begin + threadIdx.x; i < end; i += kChunkThreads) {
-      const float v = xr[i];
-      const float mn = fmaxf(m, v);
-      acc = acc * exp_fast(m - mn) + exp_fast(v - mn);
-      m = mn;
+    const Peel pl = peel16(p, end - begin);
+    if (static_cast<int>(threadIdx.x) < pl.head + pl.tail) {
+      m = p[pl.edge(threadIdx.x)];
+      acc = 1.f;
     }
+    sm_reduce_vectors(p + pl.head, pl.nvec, m, acc);
   }
   block_merge_max_sum(m, acc, slot);
   if (threadIdx.x == 0) part[blockIdx.x] = make_float2(m, acc);
+}
+
+// out[i] = f(in[i]) over nvec aligned vectors, strided over the workgroup.
+template <typename F>
+__device__ __forceinline__ void sm_map_vectors(const float* in, float* out, int64_t nvec, F f)
+{
+  for (int64_t i0 = threadIdx.x; i0 < nvec; i0 += kChunkUnroll * kChunkThreads) {
+    float v[kChunkUnroll][4];
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+      if (i < nvec) Vec16<float>::load(in + 4 * i, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+      if (i < nvec) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[u][k] = f(v[u][k]);
+        Vec16<float>::store(out + 4 * i, v[u]);
+      }
+    }
+  }
 }
 
 template <bool VEC, int KIND>
@@ -538,8 +612,9 @@ sm_fwd_apply(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int
   const float sum = wave_sum(ps * exp_fast(pm - m));
   const float scale = 1.0f / sum;
   const float lse = (KIND == kLogSoftmax) ? log_of_sum(sum) : 0.f;
-  const float* xr = x + map.offset(row, ldx);
-  float* yr = y + map.offset(row, ldy);
+  const float* xp = x + map.offset(row, ldx) + begin;
+  float* yp = y + map.offset(row, ldy) + begin;
+  const int64_t len = end - begin;
   auto f = [&](float v) -> float {
     const float d = v - m;
     if (KIND == kLogSoftmax) return d - lse;
@@ -548,27 +623,45 @@ sm_fwd_apply(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int
     return r;
   };
   if (VEC) {
-    for (int64_t i0 = begin / 4 + threadIdx.x; i0 < end / 4; i0 += kChunkUnroll * kChunkThreads) {
-      float v[kChunkUnroll][4];
-#pragma unroll
-      for (int u = 0; u < kChunkUnroll; ++u) {
-        const int64_t i = i0 + u * kChunkThreads;
-        if (i < end / 4) Vec16<float>::load(xr + 4 * i, v[u]);
-      }
-#pragma unroll
-      for (int u = 0; u < kChunkUnroll; ++u) {
-        const int64_t i = i0 + u * kChunkThreads;
-        if (i < end / 4) {
-#pragma unroll
-          for (int k = 0; k < 4; ++k) v[u][k] = f(v[u][k]);
-          Vec16<float>::store(yr + 4 * i, v[u]);
-        }
-      }
+    sm_map_vectors(xp, yp, len / 4, f);
+  }
+  else if (same_phase16(xp, yp)) {
+    const Peel pl = peel16(xp, len);
+    if (static_cast<int>(threadIdx.x) < pl.head + pl.tail) {
+      const int64_t e = pl.edge(threadIdx.x);
+      yp[e] = f(xp[e]);
     }
+    sm_map_vectors(xp + pl.head, yp + pl.head, pl.nvec, f);
   }
   else {
-    for (int64_t i = begin + threadIdx.x; i < end; i += kChunkThreads) yr[i] = f(xr[i]);
+    for (int64_t i = threadIdx.x; i < len; i += kChunkThreads) yp[i] = f(xp[i]);
   }
+}
+
+// sum of dy (log-softmax) or of y * dy over nvec aligned vectors, strided over the workgroup.
+template <int KIND>
+__device__ __forceinline__ float sm_dot_vectors(const float* yb, const float* gb, int64_t nvec)
+{
+  float acc = 0.f;
+  for (int64_t i0 = threadIdx.x; i0 < nvec; i0 += kChunkUnroll * kChunkThreads) {
+    float a[kChunkUnroll][4], g[kChunkUnroll][4];
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) a[u][k] = g[u][k] = 0.f;
+      if (i < nvec) {
+        Vec16<float>::load(gb + 4 * i, g[u]);
+        if (KIND != kLogSoftmax) Vec16<float>::load(yb + 4 * i, a[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      if (KIND == kLogSoftmax) acc += (g[u][0] + g[u][1]) + (g[u][2] + g[u][3]);
+      else acc += (a[u][0] * g[u][0] + a[u][1] * g[u][1]) + (a[u][2] * g[u][2] + a[u][3] * g[u][3]);
+    }
+  }
+  return acc;
 }
 
 template <bool VEC, int KIND>
@@ -581,35 +674,53 @@ sm_bwd_partial(const float* y, const float* dy, int64_t ldy, int64_t lddy, RowMa
   const int s = blockIdx.x - row * S;
   const int64_t begin = s * chunk;
   const int64_t end = imin64(n, begin + chunk);
-  const float* yr = y + map.offset(row, ldy);
-  const float* gr = dy + map.offset(row, lddy);
+  const float* yp = y + map.offset(row, ldy) + begin;
+  const float* gp = dy + map.offset(row, lddy) + begin;
+  const int64_t len = end - begin;
   float acc = 0.f;
   if (VEC) {
-    for (int64_t i0 = begin / 4 + threadIdx.x; i0 < end / 4; i0 += kChunkUnroll * kChunkThreads) {
-      float a[kChunkUnroll][4], g[kChunkUnroll][4];
-#pragma unroll
-      for (int u = 0; u < kChunkUnroll; ++u) {
-        const int64_t i = i0 + u * kChunkThreads;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) a[u][k] = g[u][k] = 0.f;
-        if (i < end / 4) {
-          Vec16<float>::load(gr + 4 * i, g[u]);
-          if (KIND != kLogSoftmax) Vec16<float>::load(yr + 4 * i, a[u]);
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < kChunkUnroll; ++u) {
-        if (KIND == kLogSoftmax) acc += (g[u][0] + g[u][1]) + (g[u][2] + g[u][3]);
-        else acc += (a[u][0] * g[u][0] + a[u][1] * g[u][1]) + (a[u][2] * g[u][2] + a[u][3] * g[u][3]);
-      }
+    acc = sm_dot_vectors<KIND>(yp, gp, len / 4);
+  }
+  else if (same_phase16(yp, gp)) {
+    const Peel pl = peel16(gp, len);
+    acc = sm_dot_vectors<KIND>(yp + pl.head, gp + pl.head, pl.nvec);
+    if (static_cast<int>(threadIdx.x) < pl.head + pl.tail) {
+      const int64_t e = pl.edge(threadIdx.x);
+      acc += (KIND == kLogSoftmax) ? gp[e] : yp[e] * gp[e];
     }
   }
   else {
-    for (int64_t i = begin + threadIdx.x; i < end; i += kChunkThreads)
-      acc += (KIND == kLogSoftmax) ? gr[i] : yr[i] * gr[i];
+    for (int64_t i = threadIdx.x; i < len; i += kChunkThreads)
+      acc += (KIND == kLogSoftmax) ? gp[i] : yp[i] * gp[i];
   }
   acc = team_sum<kChunkThreads / kWave>(acc, slot, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
   if (threadIdx.x == 0) part[blockIdx.x] = acc;
+}
+
+// out[i] = f(a[i], g[i]) over nvec aligned vectors, strided over the workgroup.
+template <typename F>
+__device__ __forceinline__ void sm_map2_vectors(const float* ab, const float* gb, float* out, int64_t nvec, F f)
+{
+  for (int64_t i0 = threadIdx.x; i0 < nvec; i0 += kChunkUnroll * kChunkThreads) {
+    float a[kChunkUnroll][4], g[kChunkUnroll][4];
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+      if (i < nvec) {
+        Vec16<float>::load(ab + 4 * i, a[u]);
+        Vec16<float>::load(gb + 4 * i, g[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+      if (i < nvec) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) g[u][k] = f(a[u][k], g[u][k]);
+        Vec16<float>::store(out + 4 * i, g[u]);
+      }
+    }
+  }
 }
 
 template <bool VEC, int KIND>
@@ -623,36 +734,26 @@ sm_bwd_apply(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ld
   const int64_t end = imin64(n, begin + chunk);
   const int lane = threadIdx.x & (kWave - 1);
   const float sum = wave_sum(lane < S ? part[row * S + lane] : 0.f);
-  const float* yr = y + map.offset(row, ldy);
-  const float* gr = dy + map.offset(row, lddy);
-  float* dr = dx + map.offset(row, lddx);
+  const float* yp = y + map.offset(row, ldy) + begin;
+  const float* gp = dy + map.offset(row, lddy) + begin;
+  float* dp = dx + map.offset(row, lddx) + begin;
+  const int64_t len = end - begin;
   auto f = [&](float a, float g) -> float {
     return (KIND == kLogSoftmax) ? g - exp_fast(a) * sum : a * (g - sum);
   };
   if (VEC) {
-    for (int64_t i0 = begin / 4 + threadIdx.x; i0 < end / 4; i0 += kChunkUnroll * kChunkThreads) {
-      float a[kChunkUnroll][4], g[kChunkUnroll][4];
-#pragma unroll
-      for (int u = 0; u < kChunkUnroll; ++u) {
-        const int64_t i = i0 + u * kChunkThreads;
-        if (i < end / 4) {
-          Vec16<float>::load(yr + 4 * i, a[u]);
-          Vec16<float>::load(gr + 4 * i, g[u]);
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < kChunkUnroll; ++u) {
-        const int64_t i = i0 + u * kChunkThreads;
-        if (i < end / 4) {
-#pragma unroll
-          for (int k = 0; k < 4; ++k) g[u][k] = f(a[u][k], g[u][k]);
-          Vec16<float>::store(dr + 4 * i, g[u]);
-        }
-      }
+    sm_map2_vectors(yp, gp, dp, len / 4, f);
+  }
+  else if (same_phase16(yp, gp) && same_phase16(yp, dp)) {
+    const Peel pl = peel16(yp, len);
+    if (static_cast<int>(threadIdx.x) < pl.head + pl.tail) {
+      const int64_t e = pl.edge(threadIdx.x);
+      dp[e] = f(yp[e], gp[e]);
     }
+    sm_map2_vectors(yp + pl.head, gp + pl.head, dp + pl.head, pl.nvec, f);
   }
   else {
-    for (int64_t i = begin + threadIdx.x; i < end; i += kChunkThreads) dr[i] = f(yr[i], gr[i]);
+    for (int64_t i = threadIdx.x; i < len; i += kChunkThreads) dp[i] = f(yp[i], gp[i]);
   }
 }
 
@@ -678,6 +779,7 @@ static ChunkPlan plan_chunks(int64_t n, int64_t rows)
 }
 
 constexpr int64_t kMaxRowVectors = 8192;  // longest row the one-workgroup register kernels hold
+constexpr int64_t kMaxScalarRow = 8192;   // the same in floats for rows accessed one float at a time
 
 static size_t sm_workspace_bytes(int64_t n, int64_t rows)
 {
@@ -744,6 +846,23 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     else                                                                                     \
       hipLaunchKernelGGL((sm_fwd_rows<TPR, V, KIND, false>), dim3(grid), dim3(B::kThreads), 0, st, \
                          x, y, ldx, ldy, map, rows, nvec);                                   \
+    return launch_status();                                                                  \
+  }
+      LBN_ROW_CASES(X)
+#undef X
+    }
+  }
+  else if (n <= kMaxScalarRow) {
+    // rows that are only 4-byte aligned and short enough for registers: one float per access
+    const RowConfig c = pick_row_config(n, rows);
+    if (c.tpr) {
+      const unsigned nvec = static_cast<unsigned>(n);
+#define X(TPR, V)                                                                            \
+  if (c.tpr == TPR && c.v == V) {                                                            \
+    using B = RowBlock<TPR>;                                                                 \
+    const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
+    hipLaunchKernelGGL((sm_fwd_rows<TPR, V, KIND, false, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
+                       x, y, ldx, ldy, map, rows, nvec);                                     \
     return launch_status();                                                                  \
   }
       LBN_ROW_CASES(X)
@@ -822,6 +941,22 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     else                                                                                     \
       hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, false>), dim3(grid), dim3(B::kThreads), 0, st, \
                          y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
+    return launch_status();                                                                  \
+  }
+      LBN_ROW_CASES(X)
+#undef X
+    }
+  }
+  else if (n <= kMaxScalarRow) {
+    const RowConfig c = pick_row_config(n, rows);
+    if (c.tpr) {
+      const unsigned nvec = static_cast<unsigned>(n);
+#define X(TPR, V)                                                                            \
+  if (c.tpr == TPR && c.v == V) {                                                            \
+    using B = RowBlock<TPR>;                                                                 \
+    const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
+    hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, false, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
+                       y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                         \
     return launch_status();                                                                  \
   }
       LBN_ROW_CASES(X)

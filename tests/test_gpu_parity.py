@@ -45,6 +45,9 @@ SM_SHAPES = [
     (32772, 2, 0), (70000, 3, 0), (262144, 2, 0),        # longer than the register path: split kernels
     (262148, 48, 0), (100000, 130, 0),                   # long rows, large footprint: register-resident clusters
     (1, 6, 0),
+    # rows that are only 4-byte aligned: one float per access in registers up to 8192 entries,
+    # 16-byte accesses with scalar edges in the split kernels beyond
+    (197, 70, 0), (8191, 9, 0), (8193, 3, 0), (30522, 5, 0), (50257, 6, 0), (10, 300, 0), (4099, 7, 1),
 ]
 
 
@@ -120,7 +123,7 @@ CWS_CASES = [
     # dims, dim, single_dim_mode, width
     ((5, 2, 7), 0, False, 15), ((5, 2, 7), -1, True, 15), ((64, 256), 0, False, 9),
     ((4, 8, 128), -1, True, 3), ((16, 4096), 0, False, 3), ((3, 40000), 0, False, 2),
-    ((6, 10), 0, False, 4),
+    ((6, 10), 0, False, 4), ((12, 197, 197), -1, True, 3), ((5, 1001), 0, False, 6), ((3, 9001), 0, False, 2),
 ]
 
 
