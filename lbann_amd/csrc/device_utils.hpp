@@ -109,6 +109,63 @@ struct Vec16<float> {
   }
 };
 
+// fp32 storage accessed one element at a time: for matrices whose rows start on 4-byte
+// but not 16-byte boundaries (odd row lengths).  Consecutive lanes then take consecutive
+// floats, so a wave instruction still reads 256 contiguous bytes.
+struct f32x1 {
+  float v;
+};
+
+template <>
+struct Vec16<f32x1> {
+  static constexpr int N = 1;
+  using raw_t = float;
+  static __device__ __forceinline__ raw_t load_raw(const f32x1* p) { return p->v; }
+  static __device__ __forceinline__ void unpack(const raw_t& r, float (&v)[1]) { v[0] = r; }
+  static __device__ __forceinline__ void load(const f32x1* p, float (&v)[1]) { v[0] = p->v; }
+  static __device__ __forceinline__ void store(f32x1* p, const float (&v)[1]) { p->v = v[0]; }
+  static __device__ __forceinline__ float load1(const f32x1* p) { return p->v; }
+  static __device__ __forceinline__ void store1(f32x1* p, float v) { p->v = v; }
+};
+
+// VE consecutive fp32 weights (scale, bias, their partial gradients) at p: 16-byte accesses
+// when a thread owns at least four of them, single floats otherwise.
+template <int VE>
+__device__ __forceinline__ void load_f32_run(const float* p, float (&out)[VE])
+{
+  if constexpr (VE >= 4) {
+#pragma unroll
+    for (int k4 = 0; k4 < VE; k4 += 4) {
+      float q4[4];
+      Vec16<float>::load(p + k4, q4);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) out[k4 + k] = q4[k];
+    }
+  }
+  else {
+#pragma unroll
+    for (int k = 0; k < VE; ++k) out[k] = p[k];
+  }
+}
+
+template <int VE>
+__device__ __forceinline__ void store_f32_run(float* p, const float (&in)[VE])
+{
+  if constexpr (VE >= 4) {
+#pragma unroll
+    for (int k4 = 0; k4 < VE; k4 += 4) {
+      float q4[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) q4[k] = in[k4 + k];
+      Vec16<float>::store(p + k4, q4);
+    }
+  }
+  else {
+#pragma unroll
+    for (int k = 0; k < VE; ++k) p[k] = in[k];
+  }
+}
+
 template <>
 struct Vec16<__half> {
   static constexpr int N = 8;

@@ -68,15 +68,7 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
   auto load_weights = [&](const float* w, int i, float fill, float (&out)[VE]) {
 #pragma unroll
     for (int k = 0; k < VE; ++k) out[k] = fill;
-    if (w) {
-#pragma unroll
-      for (int k4 = 0; k4 < VE; k4 += 4) {
-        float q4[4];
-        Vec16<float>::load(w + voff[i] + k4, q4);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) out[k4 + k] = q4[k];
-      }
-    }
+    if (w) load_f32_run<VE>(w + voff[i], out);
   };
   float gam[WV][VE], bet[WV][VE];
   if constexpr (kWeightsInRegs) {
@@ -126,8 +118,11 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
           sq = __builtin_fmaf(v[i][k], v[i][k], sq);
         }
       team_sum2<NW>(s, sq, slots, wv, lane);
-      mean = s * inv_n;
-      var = fmaxf(__builtin_fmaf(-mean, mean, sq * inv_n), 0.f);
+      // the reference's own expression (layer_norm.cpp:99-112): true divisions, no fused
+      // multiply-add, so that its cancellation and clamp come out the same
+      const float nf = static_cast<float>(nvec * VE);
+      mean = s / nf;
+      var = fmaxf(__fsub_rn(sq / nf, __fmul_rn(mean, mean)), 0.f);
 #pragma unroll
       for (int i = 0; i < V; ++i)
 #pragma unroll
@@ -291,15 +286,7 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
     const int idx = t + i * TPR;
 #pragma unroll
     for (int k = 0; k < VE; ++k) gam[i][k] = 1.f;
-    if (gamma && idx < nvec) {
-#pragma unroll
-      for (int k4 = 0; k4 < VE; k4 += 4) {
-        float w[4];
-        Vec16<float>::load(gamma + VE * idx + k4, w);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) gam[i][k4 + k] = w[k];
-      }
-    }
+    if (gamma && idx < nvec) load_f32_run<VE>(gamma + VE * idx, gam[i]);
   }
   float dg[WGRAD ? V : 1][VE], db[WGRAD ? V : 1][VE];
   if (WGRAD) {
@@ -453,16 +440,8 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
       for (int i = 0; i < V; ++i) {
         const int idx = t + i * TPR;
         if (idx < nvec) {
-#pragma unroll
-          for (int k4 = 0; k4 < VE; k4 += 4) {
-            float w[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) w[k] = dg[i][k4 + k];
-            Vec16<float>::store(out + VE * idx + k4, w);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) w[k] = db[i][k4 + k];
-            Vec16<float>::store(out + n + VE * idx + k4, w);
-          }
+          store_f32_run<VE>(out + VE * idx, dg[i]);
+          store_f32_run<VE>(out + n + VE * idx, db[i]);
         }
       }
     }
@@ -632,15 +611,16 @@ static int64_t ln_bwd_block_limit(int64_t rows, int elem_bytes)
 // Narrow teams with several vectors per thread spend the least on the row reduction,
 // so the narrowest team that owns at most 16 entries per thread is taken; rows too
 // long for that go to 512-thread teams with up to 32 entries per thread.
-static LnBwdPlan plan_ln_bwd(int64_t nvec, int64_t rows, int ve)
+static LnBwdPlan plan_ln_bwd(int64_t nvec, int64_t rows, int ve, int elem_bytes)
 {
   static const int force_tpr = std::getenv("LBN_LN_BWD_TPR") ? std::atoi(std::getenv("LBN_LN_BWD_TPR")) : 0;
   static const int force_teams = std::getenv("LBN_LN_BWD_TEAMS") ? std::atoi(std::getenv("LBN_LN_BWD_TEAMS")) : 0;
-  const int64_t max_blocks = ln_bwd_block_limit(rows, 16 / ve);
+  const int64_t max_blocks = ln_bwd_block_limit(rows, elem_bytes);
   LnBwdPlan p{0, 0, 0, 0};
   const int tprs[3] = {64, 256, 512};
   const int teams[3] = {4, 2, 1};
-  const int v_pref = 16 / ve, v_max = 32 / ve;
+  // at most 8 access units per thread are instantiated
+  const int v_pref = 16 / ve < 8 ? 16 / ve : 8, v_max = 32 / ve < 8 ? 32 / ve : 8;
   int pick = -1;
   for (int pass = 0; pass < 2 && pick < 0; ++pass)
     for (int i = 0; i < 3 && pick < 0; ++i) {
@@ -670,15 +650,60 @@ static int64_t ln_wgrad_slabs(int64_t units, int64_t rows)
   return s < 1 ? 1 : s;
 }
 
+constexpr int64_t kLnMaxScalarRowFwd = 8192;  // rows accessed one float at a time: 1024 threads x 8
+constexpr int64_t kLnMaxScalarRowBwd = 4096;  // 512 threads x 8
+
+// ve: entries per 16-byte vector of the storage type (4: fp32, 8: fp16).  The size does not
+// depend on pointers or leading dimensions, which the query does not see, so it covers
+// every path the shape can take: 16-byte vectors, single floats, row slabs.
 static size_t ln_bwd_workspace(int64_t n, int64_t rows, int ve)
 {
   if (n <= 0 || rows <= 0) return 0;
+  const int elem_bytes = 16 / ve;
+  size_t need = static_cast<size_t>(ln_wgrad_slabs(n, rows)) * 2 * n * sizeof(float);
+  auto cover = [&](size_t bytes) { if (bytes > need) need = bytes; };
   if (n % ve == 0) {
-    const LnBwdPlan p = plan_ln_bwd(n / ve, rows, ve);
-    if (p.tpr) return static_cast<size_t>(p.blocks) * 2 * n * sizeof(float);
-    return static_cast<size_t>(ln_wgrad_slabs(n / ve, rows)) * 2 * n * sizeof(float);
+    const LnBwdPlan p = plan_ln_bwd(n / ve, rows, ve, elem_bytes);
+    if (p.tpr) cover(static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
+    else cover(static_cast<size_t>(ln_wgrad_slabs(n / ve, rows)) * 2 * n * sizeof(float));
   }
-  return static_cast<size_t>(ln_wgrad_slabs(n, rows)) * 2 * n * sizeof(float);
+  if (ve == 4 && n <= kLnMaxScalarRowBwd) {  // fp32 rows off the 16-byte grid: one float per access
+    const LnBwdPlan p = plan_ln_bwd(n, rows, 1, 4);
+    if (p.tpr) cover(static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
+  }
+  return need;
+}
+
+// Register-resident forward over rows of `units` access units (16-byte vectors, or single
+// floats for ST = f32x1).  Returns 1 when launched, 0 when no configuration holds the row,
+// -1 when the occupancy query fails.
+template <typename ST>
+static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, int64_t ldy, RowMap map,
+                              int64_t rows, int64_t units, float inv_n, float eps, float* stats, int64_t lds,
+                              const float* gamma, const float* beta, int sumsq)
+{
+  constexpr int VE = Vec16<ST>::N;
+  const RowConfig c = pick_row_config(units, rows, 8);
+  if (!c.tpr) return 0;
+  const int nvec = static_cast<int>(units);
+#define X(TPR, V)                                                                              \
+  if (c.tpr == TPR && c.v == V) {                                                              \
+    using B = RowBlock<TPR>;                                                                   \
+    const int64_t work = ceil_div(rows, B::kTeams);                                            \
+    const int64_t resident = resident_blocks(ln_fwd_rows<ST, TPR, V>, B::kThreads);            \
+    if (resident <= 0) return -1;                                                              \
+    /* one wave of blocks, each walking the same number of rows */                             \
+    const int64_t grid = ceil_div(work, ceil_div(work, resident));                             \
+    hipLaunchKernelGGL((ln_fwd_rows<ST, TPR, V>), dim3(static_cast<unsigned>(grid)),           \
+                       dim3(B::kThreads), 0, st, x, y, ldx, ldy, map, rows, nvec, inv_n, eps,  \
+                       stats, lds, gamma, beta, sumsq);                                        \
+    return 1;                                                                                  \
+  }
+  X(64, 1) X(64, 2) X(64, 4) X(256, 1) X(256, 2) X(256, 4) X(1024, 1) X(1024, 2) X(1024, 4)
+  X(64, 8) X(256, 8)
+  if constexpr (VE <= 4) { X(1024, 8) }
+#undef X
+  return 0;
 }
 
 template <typename T>
@@ -699,32 +724,22 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
   const bool vec = (n % VE == 0) && rows_aligned16(x, stride, ldx, G, w, sizeof(T)) &&
                    rows_aligned16(y, stride, ldy, G, w, sizeof(T)) &&
                    (!gamma || aligned16(gamma)) && (!beta || aligned16(beta));
+  const float inv_n = 1.0f / static_cast<float>(n);
   if (vec) {
-    const RowConfig c = pick_row_config(n / VE, rows, 8);
-    if (c.tpr) {
-      const int nvec = static_cast<int>(n / VE);
-#define X(TPR, V)                                                                              \
-  if (c.tpr == TPR && c.v == V) {                                                              \
-    using B = RowBlock<TPR>;                                                                   \
-    const int64_t units = ceil_div(rows, B::kTeams);                                           \
-    const int64_t resident = resident_blocks(ln_fwd_rows<T, TPR, V>, B::kThreads);             \
-    if (resident <= 0) return LBN_ERR_UNSUPPORTED;                                             \
-    /* one wave of blocks, each walking the same number of rows */                             \
-    const int64_t grid = ceil_div(units, ceil_div(units, resident));                           \
-    hipLaunchKernelGGL((ln_fwd_rows<T, TPR, V>), dim3(static_cast<unsigned>(grid)),            \
-                       dim3(B::kThreads), 0, st, x, y, ldx, ldy, map, rows, nvec,              \
-                       1.0f / static_cast<float>(n), eps, stats, lds, gamma, beta, sumsq);     \
-    return launch_status();                                                                    \
-  }
-      X(64, 1) X(64, 2) X(64, 4) X(256, 1) X(256, 2) X(256, 4) X(1024, 1) X(1024, 2) X(1024, 4)
-      X(64, 8) X(256, 8)
-      if constexpr (VE == 4) { X(1024, 8) }
-#undef X
-    }
+    if (int r = ln_fwd_rows_launch<T>(st, x, y, ldx, ldy, map, rows, n / VE, inv_n, eps, stats, lds, gamma,
+                                      beta, sumsq))
+      return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
     // longer than the register kernels hold
     hipLaunchKernelGGL((ln_fwd_long<T>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st, x, y,
-                       ldx, ldy, map, n / VE, 1.0f / static_cast<float>(n), eps, stats, lds, gamma, beta, sumsq);
+                       ldx, ldy, map, n / VE, inv_n, eps, stats, lds, gamma, beta, sumsq);
     return launch_status();
+  }
+  if constexpr (std::is_same<T, float>::value) {
+    if (n > 1 && n <= kLnMaxScalarRowFwd) {  // rows off the 16-byte grid: the same kernels, one float per access
+      if (int r = ln_fwd_rows_launch<f32x1>(st, reinterpret_cast<const f32x1*>(x), reinterpret_cast<f32x1*>(y),
+                                            ldx, ldy, map, rows, n, inv_n, eps, stats, lds, gamma, beta, sumsq))
+        return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
+    }
   }
   hipLaunchKernelGGL((ln_fwd_generic<T>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, st, x, y,
                      ldx, ldy, map, n, eps, stats, lds, gamma, beta, sumsq);
@@ -753,6 +768,51 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
     hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, false>), all, block, 0, st, x, dy, dx, ldx,
                        lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part);
   }
+}
+
+// Register-resident backward over rows of `units` access units, weight gradients included
+// (partial rows in the workspace, then the fixed-order reduction).  Returns 1 when launched,
+// 0 when no configuration holds the row, -1 when the workspace is missing or too small.
+template <typename ST>
+static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST* dy, ST* dx, int64_t ldx,
+                              int64_t lddy, int64_t lddx, RowMap map, int64_t rows, int64_t units, int64_t n,
+                              int elem_bytes, float eps, const float* stats, int64_t lds, float* sgrad,
+                              int64_t ldsg, const float* gamma, float* dgamma, float* dbeta, void* ws,
+                              size_t ws_bytes)
+{
+  constexpr int VE = Vec16<ST>::N;
+  const LnBwdPlan p = plan_ln_bwd(units, rows, VE, elem_bytes);
+  if (!p.tpr) return 0;
+  float* part = nullptr;
+  if (wgrad) {
+    const size_t need = static_cast<size_t>(p.blocks) * 2 * n * sizeof(float);
+    if (!ws || ws_bytes < need || !aligned16(ws)) return -1;
+    part = static_cast<float*>(ws);
+  }
+  const int nvec = static_cast<int>(units);
+  bool launched = false;
+#define X(TPR, TEAMS, V)                                                                        \
+  if (!launched && p.tpr == TPR && p.teams == TEAMS && p.v == V) {                              \
+    launch_ln_bwd_rows<ST, TPR, TEAMS, V>(st, wgrad, p.blocks, x, dy, dx, ldx, lddy, lddx, map, \
+                                          rows, nvec, static_cast<int>(n), eps, stats, lds,     \
+                                          sgrad, ldsg, gamma, part);                            \
+    launched = true;                                                                            \
+  }
+  X(64, 4, 1) X(64, 4, 2) X(64, 4, 4) X(256, 2, 1) X(256, 2, 2) X(256, 1, 1) X(256, 1, 2)
+  X(512, 1, 1) X(512, 1, 2) X(512, 1, 4)
+  if constexpr (VE <= 4) { X(256, 2, 4) X(256, 1, 4) X(512, 1, 8) }
+  if constexpr (VE == 1) { X(64, 4, 8) X(256, 2, 8) X(256, 1, 8) }
+#undef X
+  if (!launched) return 0;
+  if (wgrad) {
+    if (n % 4 == 0)
+      hipLaunchKernelGGL(ln_wgrad_reduce, dim3(static_cast<unsigned>(ceil_div(n, 32)), 2), dim3(256), 0, st,
+                         part, p.blocks, n, dgamma, dbeta);
+    else
+      hipLaunchKernelGGL(ln_wgrad_reduce_scalar, dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, st,
+                         part, p.blocks, n, dgamma, dbeta);
+  }
+  return 1;
 }
 
 template <typename T>
@@ -791,41 +851,24 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                    rows_aligned16(dx, stride, lddx, G, w, sizeof(T)) &&
                    (!gamma || aligned16(gamma));
   if (vec) {
-    LnBwdPlan p = plan_ln_bwd(n / VE, rows, VE);
-    if (p.tpr) {
-      float* part = nullptr;
-      if (wgrad) {
-        const size_t need = static_cast<size_t>(p.blocks) * 2 * n * sizeof(float);
-        if (!ws || ws_bytes < need || !aligned16(ws)) return LBN_ERR_WORKSPACE;
-        part = static_cast<float*>(ws);
-      }
-      const int nvec = static_cast<int>(n / VE);
-      bool launched = false;
-#define X(TPR, TEAMS, V)                                                                        \
-  if (!launched && p.tpr == TPR && p.teams == TEAMS && p.v == V) {                              \
-    launch_ln_bwd_rows<T, TPR, TEAMS, V>(st, wgrad, p.blocks, x, dy, dx, ldx, lddy, lddx, map,  \
-                                         rows, nvec, static_cast<int>(n), eps, stats, lds,      \
-                                         sgrad, ldsg, gamma, part);                             \
-    launched = true;                                                                            \
-  }
-      X(64, 4, 1) X(64, 4, 2) X(64, 4, 4) X(256, 2, 1) X(256, 2, 2) X(256, 1, 1) X(256, 1, 2)
-      X(512, 1, 1) X(512, 1, 2) X(512, 1, 4)
-      if constexpr (VE == 4) { X(256, 2, 4) X(256, 1, 4) X(512, 1, 8) }
-#undef X
-      if (launched) {
-        if (wgrad) {
-          const dim3 grid(static_cast<unsigned>(ceil_div(n, 32)), 2);
-          hipLaunchKernelGGL(ln_wgrad_reduce, grid, dim3(256), 0, st, part, p.blocks, n, dgamma, dbeta);
-        }
-        return launch_status();
-      }
-    }
+    if (int r = ln_bwd_rows_launch<T>(st, wgrad, x, dy, dx, ldx, lddy, lddx, map, rows, n / VE, n, sizeof(T), eps,
+                                      stats, lds, sgrad, ldsg, gamma, dgamma, dbeta, ws, ws_bytes))
+      return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
     // longer than the register kernels hold
     hipLaunchKernelGGL((ln_bwd_long<T>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st, x, dy,
                        dx, ldx, lddy, lddx, map, n / VE, 1.0f / static_cast<float>(n), eps, stats, lds, sgrad,
                        ldsg, gamma);
   }
   else {
+    if constexpr (std::is_same<T, float>::value) {
+      if (n <= kLnMaxScalarRowBwd) {  // rows off the 16-byte grid: the same kernels, one float per access
+        if (int r = ln_bwd_rows_launch<f32x1>(st, wgrad, reinterpret_cast<const f32x1*>(x),
+                                              reinterpret_cast<const f32x1*>(dy), reinterpret_cast<f32x1*>(dx), ldx,
+                                              lddy, lddx, map, rows, n, n, 4, eps, stats, lds, sgrad, ldsg, gamma,
+                                              dgamma, dbeta, ws, ws_bytes))
+          return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
+      }
+    }
     hipLaunchKernelGGL((ln_bwd_generic<T>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, st, x, dy,
                        dx, ldx, lddy, lddx, map, n, eps, stats, lds, sgrad, ldsg, gamma);
   }

@@ -67,9 +67,14 @@ ln_fwd_long(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
     }
   }
   team_sum2<kLongWaves>(s, q, red, wv, lane);
-  const float dm = s * inv_n;
+  float dm = s * inv_n;
+  float var = fmaxf(__builtin_fmaf(-dm, dm, q * inv_n), 0.f);
+  if (sumsq) {  // the reference's own expression: true divisions, no fused multiply-add
+    const float nf = static_cast<float>(nvec * VE);
+    dm = s / nf;
+    var = fmaxf(__fsub_rn(q / nf, __fmul_rn(dm, dm)), 0.f);
+  }
   const float mean = K + dm;
-  const float var = fmaxf(__builtin_fmaf(-dm, dm, q * inv_n), 0.f);
   const float inv_stdev = 1.0f / sqrtf(var + eps);
   if (threadIdx.x == 0) {
     stats[g + col * ld_stats] = mean;

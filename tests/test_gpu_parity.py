@@ -159,6 +159,9 @@ LN_CASES = [
     # gradients by row slabs (vector and scalar), groups, padded leading dimension
     ((150528,), 0, 6, True, 0), ((65536,), 0, 300, True, 0), ((4, 20000), -1, 9, True, 0),
     ((20001,), 0, 7, True, 0), ((20004,), 0, 5, True, 4), ((3, 224, 224), 0, 3, False, 0),
+    # rows off the 16-byte grid: the register kernels with one float per access
+    ((1001,), 0, 40, True, 0), ((197, 769), -1, 3, True, 0), ((4095,), 0, 9, True, 0), ((4097,), 0, 9, True, 0),
+    ((8191,), 0, 5, False, 0), ((49,), 0, 3000, True, 0), ((1000,), 0, 17, True, 3), ((7,), 0, 100000, True, 0),
 ]
 
 
@@ -236,7 +239,8 @@ def test_layer_norm_f16(L, dims, start_dim, w, pad):
 # ===================================================================== instance norm
 @pytest.mark.parametrize("dims,w,pad", [((5, 3, 7), 15, 0), ((64, 56, 56), 6, 0), ((8, 1024), 33, 0),
                                         ((3, 100000), 2, 0), ((7, 1), 5, 0), ((16, 31), 40, 4),
-                                        ((256, 16, 16), 64, 0), ((3, 224, 224), 8, 0), ((2, 64, 64, 64), 2, 0)])
+                                        ((256, 16, 16), 64, 0), ((3, 224, 224), 8, 0), ((2, 64, 64, 64), 2, 0),
+                                        ((256, 7, 7), 32, 0), ((64, 3, 3), 9, 0), ((5, 4097), 6, 0)])
 def test_instance_norm(L, dims, w, pad):
     rng = np.random.default_rng(int(np.prod(dims)) + 7 * w)
     h = int(np.prod(dims))
