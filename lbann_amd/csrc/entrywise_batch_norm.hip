@@ -255,6 +255,131 @@ ebn_bwd_tile(EbnArgs a)
   }
 }
 
+// Mini-batches wider than the tile kernels hold in registers: the same tiling, two passes
+// over the workgroup's rows x all columns (sums, then the output); the second pass re-reads
+// what the first streamed.
+template <int GW>
+__global__ void __launch_bounds__(kEbnThreads)
+ebn_fwd_wide(EbnArgs a)
+{
+  using P = EbnPos<GW>;
+  __shared__ float lds[kEbnWaves][P::kRows][2];
+  const P p;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * P::kRows + 4 * p.q;
+  const bool row_ok = r0 < a.h;
+  const int64_t rr = row_ok ? r0 : 0;
+  const int64_t w = row_ok ? a.w : 0;
+  float K[4];
+  Vec16<float>::load(a.x + rr, K);
+  float s[4] = {0.f, 0.f, 0.f, 0.f}, sq[4] = {0.f, 0.f, 0.f, 0.f};
+  int64_t c = p.g;
+  for (; c + P::kGroups < w; c += 2 * P::kGroups) {
+    float v[2][4];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) Vec16<float>::load(a.x + rr + (c + j * P::kGroups) * a.ldx, v[j]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float d = v[j][r] - K[r];
+        s[r] += d;
+        sq[r] = __builtin_fmaf(d, d, sq[r]);
+      }
+  }
+  for (; c < w; c += P::kGroups) {
+    float v[4];
+    Vec16<float>::load(a.x + rr + c * a.ldx, v);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float d = v[r] - K[r];
+      s[r] += d;
+      sq[r] = __builtin_fmaf(d, d, sq[r]);
+    }
+  }
+  ebn_merge<GW>(s, sq, lds, p);
+  if (!row_ok) return;
+  float mean[4], var[4], inv[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    ebn_stats_from_sums(s[r], sq[r], K[r], a.w, mean[r], var[r]);
+    inv[r] = 1.0f / sqrtf(var[r] + a.eps);
+  }
+  if (p.g == 0) {
+    Vec16<float>::store(a.stats + r0, mean);
+    Vec16<float>::store(a.stats + r0 + a.ld_stats, var);
+    float rm[4], rv[4];  // w > 1 here: entrywise_batch_normalization.cpp:121-122
+    Vec16<float>::load(a.rmean + r0, rm);
+    Vec16<float>::load(a.rvar + r0, rv);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      rm[r] = a.decay * rm[r] + (1.f - a.decay) * mean[r];
+      rv[r] = a.decay * rv[r] + (1.f - a.decay) * var[r];
+    }
+    Vec16<float>::store(a.rmean + r0, rm);
+    Vec16<float>::store(a.rvar + r0, rv);
+  }
+  for (c = p.g; c < w; c += P::kGroups) {
+    float v[4];
+    Vec16<float>::load(a.x + r0 + c * a.ldx, v);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) v[r] = (v[r] - mean[r]) * inv[r];
+    Vec16<float>::store(a.out + r0 + c * a.ldo, v);
+  }
+}
+
+template <int GW>
+__global__ void __launch_bounds__(kEbnThreads)
+ebn_bwd_wide(EbnArgs a)
+{
+  using P = EbnPos<GW>;
+  __shared__ float lds[kEbnWaves][P::kRows][2];
+  const P p;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * P::kRows + 4 * p.q;
+  const bool row_ok = r0 < a.h;
+  const int64_t rr = row_ok ? r0 : 0;
+  const int64_t w = row_ok ? a.w : 0;
+  float mean[4], var[4], inv[4];
+  Vec16<float>::load(a.stats + rr, mean);
+  Vec16<float>::load(a.stats + rr + a.ld_stats, var);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) inv[r] = 1.0f / sqrtf(var[r] + a.eps);
+  float sa[4] = {0.f, 0.f, 0.f, 0.f}, sb[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int64_t c = p.g; c < w; c += P::kGroups) {
+    float v[4], g[4];
+    Vec16<float>::load(a.x + rr + c * a.ldx, v);
+    Vec16<float>::load(a.dy + rr + c * a.lddy, g);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      sa[r] += g[r];
+      sb[r] = __builtin_fmaf(g[r], v[r] - mean[r], sb[r]);
+    }
+  }
+  ebn_merge<GW>(sa, sb, lds, p);
+  if (!row_ok) return;
+  const float wf = static_cast<float>(a.w);
+  float dmean[4], dvar[4], c0[4], c1[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    dmean[r] = -sa[r] * inv[r];
+    dvar[r] = -sb[r] * inv[r] * inv[r] * inv[r] * 0.5f;
+    c0[r] = dmean[r] / wf;
+    c1[r] = dvar[r] * 2.f / (wf - 1.f);
+  }
+  if (p.g == 0) {
+    Vec16<float>::store(a.sgrad + r0, dmean);
+    Vec16<float>::store(a.sgrad + r0 + a.ld_sgrad, dvar);
+  }
+  for (int64_t c = p.g; c < w; c += P::kGroups) {
+    float v[4], g[4];
+    Vec16<float>::load(a.x + r0 + c * a.ldx, v);
+    Vec16<float>::load(a.dy + r0 + c * a.lddy, g);
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      g[r] = __builtin_fmaf(g[r], inv[r], __builtin_fmaf(c1[r], v[r] - mean[r], c0[r]));
+    Vec16<float>::store(a.out + r0 + c * a.ldo, g);
+  }
+}
+
 // One thread per row.  TRAINING: statistics from the mini-batch (written to stats, running
 // statistics updated); otherwise the running statistics are used as they are.
 template <bool TRAINING>
@@ -386,6 +511,11 @@ int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_
     LBN_EBN_TILE_CASES(X)
 #undef X
   }
+  if (training && vec) {  // wider than the register tiles
+    hipLaunchKernelGGL((ebn_fwd_wide<4>), dim3(static_cast<unsigned>(ceil_div(height, EbnPos<4>::kRows))),
+                       dim3(kEbnThreads), 0, st, a);
+    return launch_status();
+  }
   const dim3 grid(static_cast<unsigned>(ceil_div(height, 256))), block(256);
   if (training) hipLaunchKernelGGL((ebn_fwd_generic<true>), grid, block, 0, st, a);
   else hipLaunchKernelGGL((ebn_fwd_generic<false>), grid, block, 0, st, a);
@@ -430,6 +560,11 @@ int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_
   }
     LBN_EBN_TILE_CASES(X)
 #undef X
+  }
+  if (vec) {  // wider than the register tiles
+    hipLaunchKernelGGL((ebn_bwd_wide<4>), dim3(static_cast<unsigned>(ceil_div(height, EbnPos<4>::kRows))),
+                       dim3(kEbnThreads), 0, st, a);
+    return launch_status();
   }
   hipLaunchKernelGGL((ebn_bwd_generic<true>), dim3(static_cast<unsigned>(ceil_div(height, 256))),
                      dim3(256), 0, st, a);
