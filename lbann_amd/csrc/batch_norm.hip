@@ -10,6 +10,9 @@
 // grid) merges the P partials in a fixed order in its prologue, workgroup 0 of each
 // channel writes the statistics, and all P workgroups stream the channel once more
 // to write the output.  No atomics: results are bitwise reproducible.
+// Training-mode calls on aligned shapes take the single-pass register-resident
+// cluster kernels further down; fp32 channels that are not a whole number of 16-byte
+// vectors take the row-tile kernels of batch_norm_rows.hpp.
 //
 // Forward statistics are accumulated about a per-channel pivot (the channel's first
 // entry), sum(x-K) and sum((x-K)^2), which removes the cancellation of

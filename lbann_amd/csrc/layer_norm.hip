@@ -15,8 +15,11 @@
 //    teams of a block merge through LDS, every block leaves one partial row in the
 //    workspace, and a second small kernel sums the partial rows in a fixed order:
 //    no atomics, bitwise reproducible.
-//  * generic kernels (one 256-thread block per row, scalar access) cover rows that
-//    are unaligned, not a multiple of the vector length, or too long for registers.
+//  * fp32 rows off the 16-byte grid (odd lengths or leading dimensions) run the same
+//    register kernels on a storage type that is accessed one float at a time (f32x1).
+//  * rows longer than the register kernels hold: layer_norm_long.hpp.
+//  * generic kernels (one 256-thread block per row, scalar access) cover what is left
+//    (fp16 rows that are not a multiple of 8 long, very long unaligned rows).
 #include <type_traits>
 
 #include "device_utils.hpp"

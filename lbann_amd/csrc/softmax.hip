@@ -1,15 +1,21 @@
 // Softmax, log-softmax and channelwise softmax, forward and backward, for gfx950.
 //
 // All three layers reduce over independent contiguous rows (a matrix column, or a
-// channel window of a column).  Two kernel families cover every shape:
+// channel window of a column).  Three kernel families cover every shape:
 //
 //  * register-resident row kernels: TPR threads (one wave, 256 or 1024 threads)
 //    load a whole row with 128-bit coalesced loads, keep it in registers, reduce
 //    on the wave64 DPP path (+ one LDS hop across waves), and store the result.
 //    Each tensor is read once and written once.  Used when rows are 16-byte
-//    aligned, a multiple of 4 long and at most 32768 entries.
-//  * split ("chunked") kernels for very long or unaligned rows: a row is cut into
-//    S chunks, one workgroup each.  Kernel 1 leaves one partial reduction per chunk
+//    aligned, a multiple of 4 long and at most 32768 entries; rows that are only
+//    4-byte aligned (odd lengths) run the same kernels with one float per access up
+//    to 8192 entries.
+//  * register-resident clusters: rows too long for one workgroup whose tensors
+//    exceed the caches are shared by a cluster of workgroups that exchange one
+//    (max, sum) pair through memory.
+//  * split ("chunked") kernels for the remaining long or unaligned rows: a row is cut
+//    into S chunks, one workgroup each; chunks that start off a 16-byte boundary are
+//    walked as leading scalars, aligned vectors and trailing scalars.  Kernel 1 leaves one partial reduction per chunk
 //    in the workspace (for softmax an online (max, sum) pair), kernel 2 merges the
 //    S partials and writes its chunk.  Kernel 1 reads everything before kernel 2
 //    writes anything, so in-place operation stays safe with many workgroups per row.
