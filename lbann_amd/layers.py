@@ -1,4 +1,6 @@
-"""Host-side mirror of the five LBANN layer classes, over the C ABI.
+"""Host-side mirror of the LBANN layer classes (layer norm, batch norm, softmax, log-softmax,
+channelwise softmax; instance norm, entry-wise batch norm, cross entropy and the two scale/bias
+layers), over the C ABI.
 
 Each class keeps the reference layer's constructor parameters, its member
 matrices and its two compute hooks, `fp_compute()` and `bp_compute()`
