@@ -313,6 +313,25 @@ __device__ __forceinline__ float wave_max_in_last(float v)
   v = fmaxf(v, dpp_move<kDppRowBcast31, 0xC>(v, v));
   return v;
 }
+// Sum / maximum over each group of 16 consecutive lanes (a DPP row); every lane of the
+// group gets the result.  Lanes of other groups are never read, so whole groups may be
+// inactive.
+__device__ __forceinline__ float row16_sum(float v)
+{
+  v += dpp_move<kDppQuadSwap1>(v);
+  v += dpp_move<kDppQuadSwap2>(v);
+  v += dpp_move<kDppHalfMirror>(v);
+  v += dpp_move<kDppRowMirror>(v);
+  return v;
+}
+__device__ __forceinline__ float row16_max(float v)
+{
+  v = fmaxf(v, dpp_move<kDppQuadSwap1>(v, v));
+  v = fmaxf(v, dpp_move<kDppQuadSwap2>(v, v));
+  v = fmaxf(v, dpp_move<kDppHalfMirror>(v, v));
+  v = fmaxf(v, dpp_move<kDppRowMirror>(v, v));
+  return v;
+}
 // Every lane gets the result.
 __device__ __forceinline__ float wave_sum(float v) { return read_lane(wave_sum_in_last(v), kWave - 1); }
 __device__ __forceinline__ float wave_max(float v) { return read_lane(wave_max_in_last(v), kWave - 1); }

@@ -48,6 +48,9 @@ SM_SHAPES = [
     # rows that are only 4-byte aligned: one float per access in registers up to 8192 entries,
     # 16-byte accesses with scalar edges in the split kernels beyond
     (197, 70, 0), (8191, 9, 0), (8193, 3, 0), (30522, 5, 0), (50257, 6, 0), (10, 300, 0), (4099, 7, 1),
+    # many short rows: teams of 16 lanes, four rows per wave (vector and single-float access)
+    (16, 5000, 0), (64, 4100, 0), (128, 4096, 0), (200, 4500, 0), (256, 4097, 0), (10, 5000, 0), (49, 6000, 0),
+    (63, 4096, 1), (12, 4095, 0),
 ]
 
 
@@ -124,6 +127,7 @@ CWS_CASES = [
     ((5, 2, 7), 0, False, 15), ((5, 2, 7), -1, True, 15), ((64, 256), 0, False, 9),
     ((4, 8, 128), -1, True, 3), ((16, 4096), 0, False, 3), ((3, 40000), 0, False, 2),
     ((6, 10), 0, False, 4), ((12, 197, 197), -1, True, 3), ((5, 1001), 0, False, 6), ((3, 9001), 0, False, 2),
+    ((16, 64, 64), -1, True, 8), ((512, 49), -1, True, 16), ((4096, 8), 0, False, 3),
 ]
 
 
