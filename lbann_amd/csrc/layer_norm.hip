@@ -49,13 +49,16 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
   using IO = Vec16<T>;
   using raw_t = typename IO::raw_t;
   constexpr int VE = IO::N;
-  constexpr int NW = B::kWavesPerTeam;
+  constexpr bool kSub = TPR < kWave;  // short rows: a team is one DPP row of 16 lanes, four rows per wave
+  static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
+  constexpr int NW = kSub ? 1 : B::kWavesPerTeam;
   constexpr bool kWeightsInRegs = V * VE <= 16;
   constexpr bool kPrefetch = V * VE < 32;  // wider rows: the registers only hold the current row
   constexpr int WV = kWeightsInRegs ? V : 1;
   __shared__ float red[4][B::kTeams][2 * NW];
   const int tid = threadIdx.x;
-  const int team = wave_index() / NW;  // wave-uniform: a team is a whole number of waves
+  // a team is a whole number of waves (then its index is wave-uniform) or a DPP row
+  const int team = kSub ? tid / TPR : wave_index() / NW;
   const int t = tid - team * TPR;
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
@@ -120,7 +123,13 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
           s += v[i][k];
           sq = __builtin_fmaf(v[i][k], v[i][k], sq);
         }
-      team_sum2<NW>(s, sq, slots, wv, lane);
+      if constexpr (kSub) {
+        s = row16_sum(s);
+        sq = row16_sum(sq);
+      }
+      else {
+        team_sum2<NW>(s, sq, slots, wv, lane);
+      }
       // the reference's own expression (layer_norm.cpp:99-112): true divisions, no fused
       // multiply-add, so that its cancellation and clamp come out the same
       const float nf = static_cast<float>(nvec * VE);
@@ -137,7 +146,7 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
       for (int i = 0; i < V; ++i)
 #pragma unroll
         for (int k = 0; k < VE; ++k) s += v[i][k];
-      s = team_sum<NW>(s, slots, wv, lane);
+      s = kSub ? row16_sum(s) : team_sum<NW>(s, slots, wv, lane);
       mean = s * inv_n;
       float sq = 0.f;
 #pragma unroll
@@ -149,7 +158,7 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
           sq = __builtin_fmaf(d, d, sq);
         }
       }
-      sq = team_sum<NW>(sq, red[2 * (it & 1) + 1][team], wv, lane);
+      sq = kSub ? row16_sum(sq) : team_sum<NW>(sq, red[2 * (it & 1) + 1][team], wv, lane);
       var = sq * inv_n;
     }
     if (row < rows) {
@@ -272,13 +281,15 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   using IO = Vec16<T>;
   using raw_t = typename IO::raw_t;
   constexpr int VE = IO::N;
-  constexpr int NW = B::kWavesPerTeam;
+  constexpr bool kSub = TPR < kWave;
+  static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
+  constexpr int NW = kSub ? 1 : B::kWavesPerTeam;
   constexpr int kAccLds = (WGRAD && TEAMS > 1) ? 2 * TPR * V * VE : 1;
   constexpr bool kPrefetch = V * VE < 32;
   __shared__ float red[2][TEAMS][2 * NW];
   __shared__ float acc_lds[kAccLds];
   const int tid = threadIdx.x;
-  const int team = wave_index() / NW;  // wave-uniform: a team is a whole number of waves
+  const int team = kSub ? tid / TPR : wave_index() / NW;
   const int t = tid - team * TPR;
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
@@ -369,7 +380,13 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
         b = __builtin_fmaf(gs[i][k], xh[i][k], b);
       }
     }
-    team_sum2<NW>(a, b, red[it & 1][team], wv, lane);
+    if constexpr (kSub) {
+      a = row16_sum(a);
+      b = row16_sum(b);
+    }
+    else {
+      team_sum2<NW>(a, b, red[it & 1][team], wv, lane);
+    }
     if (active) {
       int64_t col, g;
       map.split(row, col, g);
@@ -636,6 +653,12 @@ static LnBwdPlan plan_ln_bwd(int64_t nvec, int64_t rows, int ve, int elem_bytes)
   p.tpr = tprs[pick];
   p.teams = teams[pick];
   p.v = round_up_pow2_le8(ceil_div(nvec, p.tpr));
+  if (!force_tpr && nvec <= 32 && rows >= 4096) {
+    // many short rows: teams of 16 lanes, four rows per wave
+    p.tpr = 16;
+    p.teams = 16;
+    p.v = nvec <= 16 ? 1 : 2;
+  }
   if (force_teams && force_teams <= p.teams) p.teams = force_teams;
   // spread small problems: fewer teams per block when rows are scarce
   while (p.teams > 1 && p.tpr * p.teams > 256 && ceil_div(rows, p.teams) < kLnBwdMinBlocks) p.teams /= 2;
@@ -686,7 +709,11 @@ static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, i
                               const float* gamma, const float* beta, int sumsq)
 {
   constexpr int VE = Vec16<ST>::N;
-  const RowConfig c = pick_row_config(units, rows, 8);
+  RowConfig c = pick_row_config(units, rows, 8);
+  // many short rows: teams of 16 lanes, four rows per wave, instead of mostly idle waves
+  // (layer norm rows of 64 entries x 65536: 60 us per step against 150 us with one wave per row;
+  // at 64 units per row the two shapes measure the same and the wave-wide team is kept)
+  if (units <= 32 && rows >= 4096) c = {16, units <= 16 ? 1 : 2};
   if (!c.tpr) return 0;
   const int nvec = static_cast<int>(units);
 #define X(TPR, V)                                                                              \
@@ -702,6 +729,7 @@ static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, i
                        stats, lds, gamma, beta, sumsq);                                        \
     return 1;                                                                                  \
   }
+  X(16, 1) X(16, 2)
   X(64, 1) X(64, 2) X(64, 4) X(256, 1) X(256, 2) X(256, 4) X(1024, 1) X(1024, 2) X(1024, 4)
   X(64, 8) X(256, 8)
   if constexpr (VE <= 4) { X(1024, 8) }
@@ -801,6 +829,7 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
                                           sgrad, ldsg, gamma, part);                            \
     launched = true;                                                                            \
   }
+  X(16, 16, 1) X(16, 16, 2)
   X(64, 4, 1) X(64, 4, 2) X(64, 4, 4) X(256, 2, 1) X(256, 2, 2) X(256, 1, 1) X(256, 1, 2)
   X(512, 1, 1) X(512, 1, 2) X(512, 1, 4)
   if constexpr (VE <= 4) { X(256, 2, 4) X(256, 1, 4) X(512, 1, 8) }
