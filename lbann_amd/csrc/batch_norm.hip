@@ -689,13 +689,18 @@ static int bn_split(int64_t C, int64_t cs, int64_t w)
   return static_cast<int>(P);
 }
 
+// Channels that are not whole vectors, and channels of one or two vectors, whose segments
+// the channel walk would fetch one 16- or 32-byte piece per column (16384 x 4, w = 256:
+// 450 us per step that way).
+static bool bn_rt_shape(int64_t cs) { return cs % 4 != 0 || cs <= 8; }
+
 static size_t bn_workspace(int64_t C, int64_t cs, int64_t w)
 {
   if (C <= 0 || cs <= 0 || w <= 0) return 0;
   const size_t split = static_cast<size_t>(C) * bn_split(C, cs, w) * sizeof(float2);
   const size_t cluster = cluster_workspace_bytes(C);
   size_t need = split > cluster ? split : cluster;
-  if (cs % 4 != 0 && (C * cs) % 4 == 0) {  // the row-tile path of batch_norm_rows.hpp
+  if (bn_rt_shape(cs) && (C * cs) % 4 == 0) {  // the row-tile path of batch_norm_rows.hpp
     const size_t rows = bn_rt_workspace_bytes(C * cs, w);
     if (rows > need) need = rows;
   }
@@ -800,7 +805,7 @@ static bool bn_vec_ok(int64_t cs, int64_t w, const void* a, int64_t lda)
 // (batch_norm_rows.hpp).  fp32 only.
 static bool bn_rt_usable(int64_t C, int64_t cs, int64_t w, const void* a, int64_t lda)
 {
-  return cs % 4 != 0 && row_quads_ok(C * cs, w, a, lda);
+  return bn_rt_shape(cs) && row_quads_ok(C * cs, w, a, lda);
 }
 
 template <bool BWD>
@@ -874,9 +879,6 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   const dim3 grid(static_cast<unsigned>(C), P);
   const int pivot = (flags & LBN_STATS_SUMSQ) ? 0 : 1;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, y, ldy);
-  if (vec && bn_try_fwd_cluster<S>(st, C, cs, w, pivot, bessel, epsilon, decay, x, ldx, y, ldy, mean, var,
-                                   scale, bias, running_mean, running_var, workspace))
-    return launch_status();
   if constexpr (std::is_same<S, float>::value) {
     if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, y, ldy) &&
         (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0) {
@@ -894,6 +896,9 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
       return launch_status();
     }
   }
+  if (vec && bn_try_fwd_cluster<S>(st, C, cs, w, pivot, bessel, epsilon, decay, x, ldx, y, ldy, mean, var,
+                                   scale, bias, running_mean, running_var, workspace))
+    return launch_status();
   if (vec) {
     hipLaunchKernelGGL((bn_fwd_sums<S, true>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, pivot, part);
     hipLaunchKernelGGL((bn_fwd_apply<S, true, true>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs, w,
@@ -929,10 +934,6 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   const dim3 grid(static_cast<unsigned>(C), P);
   const int64_t n = cs * w;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, dy, lddy) && bn_vec_ok<S>(cs, w, dx, lddx);
-  if (training && vec &&
-      bn_try_bwd_cluster<S>(st, C, cs, w, bessel, epsilon, x, ldx, dy, lddy, dx, lddx, use_mean, use_var,
-                            scale, dscale, dbias, dmean, dvar, workspace))
-    return launch_status();
   if constexpr (std::is_same<S, float>::value) {
     if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, dy, lddy) && bn_rt_usable(C, cs, w, dx, lddx) &&
         (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0) {
@@ -952,6 +953,10 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
       return launch_status();
     }
   }
+  if (training && vec &&
+      bn_try_bwd_cluster<S>(st, C, cs, w, bessel, epsilon, x, ldx, dy, lddy, dx, lddx, use_mean, use_var,
+                            scale, dscale, dbias, dmean, dvar, workspace))
+    return launch_status();
   if (vec) {
     hipLaunchKernelGGL((bn_bwd_sums<S, true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean, part);
     hipLaunchKernelGGL((bn_bwd_apply<S, true, true>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,

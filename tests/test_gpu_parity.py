@@ -308,6 +308,7 @@ BN_CASES = [
     # channels that are not whole 16-byte vectors on a quad-aligned matrix: row-tile kernels
     ((2048, 7, 7), 16, True, 0), ((4096,), 64, True, 0), ((64, 7, 7), 300, False, 0), ((12, 3, 3), 20, True, 0),
     ((8, 5), 7, True, 4), ((4, 1), 1, True, 0), ((1024, 1), 2048, True, 0),
+    ((512, 2, 2), 40, True, 0), ((300, 8), 33, False, 0), ((64, 4), 700, True, 4),   # one or two vectors per channel
 ]
 
 
