@@ -824,6 +824,36 @@ static void bn_rt_launch_apply(hipStream_t st, const RowTilePlan& p, const BnRtA
   else hipLaunchKernelGGL((bn_rt_apply<4, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
 }
 
+// Register-resident row tiles (one kernel, one read) for mini-batches of at most 256 columns
+// whose channels fit a workgroup's rows; false: use the three-kernel row-tile path.
+template <bool BWD>
+static bool bn_rt_try_tile(hipStream_t st, BnRtTileArgs a)
+{
+  int gw = 0, cpt = 0;
+  if (a.w <= 256 && (a.rows_eff = bn_rt_tile_rows(a.cs, RowTilePos<4>::kRows)) > 0) {
+    gw = 4;
+    cpt = static_cast<int>(ceil_div(a.w, RowTilePos<4>::kGroups));
+  }
+  else if (a.w <= 64 && (a.rows_eff = bn_rt_tile_rows(a.cs, RowTilePos<1>::kRows)) > 0) {
+    gw = 1;
+    cpt = static_cast<int>(ceil_div(a.w, RowTilePos<1>::kGroups));
+  }
+  else {
+    return false;
+  }
+  cpt = cpt <= 1 ? 1 : cpt <= 2 ? 2 : cpt <= 4 ? 4 : cpt <= 8 ? 8 : 16;
+  const dim3 grid(static_cast<unsigned>(ceil_div(a.h, a.rows_eff)));
+#define X(C, G)                                                                                         \
+  if (cpt == C && gw == G) {                                                                            \
+    if (BWD) hipLaunchKernelGGL((bn_rt_bwd_tile<C, G>), grid, dim3(kRowTileThreads), 0, st, a);         \
+    else hipLaunchKernelGGL((bn_rt_fwd_tile<C, G>), grid, dim3(kRowTileThreads), 0, st, a);             \
+    return true;                                                                                        \
+  }
+  X(1, 4) X(2, 4) X(4, 4) X(8, 4) X(16, 4) X(1, 1) X(2, 1) X(4, 1) X(8, 1) X(16, 1)
+#undef X
+  return false;
+}
+
 // Forward with given statistics (inference mode, and the last step of a caller that
 // reduces the statistics over ranks itself).
 template <typename S>
@@ -883,6 +913,13 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
     if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, y, ldy) &&
         (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0) {
       const int64_t h = C * cs;
+      {
+        BnRtTileArgs t{};
+        t.h = h, t.w = w, t.cs = cs, t.n = cs * w, t.x = x, t.out = y, t.ldx = ldx, t.ldo = ldy;
+        t.use_pivot = pivot, t.bessel = bessel, t.eps = epsilon, t.decay = decay, t.mean = mean, t.var = var;
+        t.scale = scale, t.bias = bias, t.rmean = running_mean, t.rvar = running_var;
+        if (bn_rt_try_tile<false>(st, t)) return launch_status();
+      }
       const RowTilePlan p = row_tile_plan(h, w);
       BnRtArgs a{};
       a.h = h, a.w = w, a.cs = cs, a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy;
@@ -938,6 +975,14 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
     if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, dy, lddy) && bn_rt_usable(C, cs, w, dx, lddx) &&
         (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0) {
       const int64_t h = C * cs;
+      {
+        BnRtTileArgs t{};
+        t.h = h, t.w = w, t.cs = cs, t.n = n, t.x = x, t.dy = dy, t.out = dx, t.ldx = ldx, t.lddy = lddy, t.ldo = lddx;
+        t.bessel = bessel, t.training = training, t.eps = epsilon;
+        t.mean = const_cast<float*>(use_mean), t.var = const_cast<float*>(use_var), t.scale = scale;
+        t.dscale = dscale, t.dbias = dbias, t.dmean = dmean, t.dvar = dvar;
+        if (bn_rt_try_tile<true>(st, t)) return launch_status();
+      }
       const RowTilePlan p = row_tile_plan(h, w);
       BnRtArgs a{};
       a.h = h, a.w = w, a.cs = cs, a.x = x, a.dy = dy, a.out = dx, a.ldx = ldx, a.lddy = lddy, a.ldo = lddx;

@@ -224,6 +224,252 @@ bn_rt_apply(BnRtArgs a)
   }
 }
 
+
+// ---- register-resident variant for mini-batches of at most 256 columns ------------------
+// A workgroup keeps (rows x all columns) in registers (the entry-wise batch norm tiling:
+// 256 rows x <= 64 columns with GW = 1, 64 rows x <= 256 columns with GW = 4) and owns
+// whole channels: it takes `rows_eff` rows, the largest multiple of lcm(cs, 4) that fits.
+// Per-row pairs are merged over the column groups in LDS, one thread per channel adds its
+// cs rows and finishes the channel, and the output is written from registers: one kernel,
+// x (and dy) read once.
+struct BnRtTileArgs {
+  int64_t h, w, cs, n;  // n = cs * w
+  int rows_eff;         // rows per workgroup: a multiple of cs and of 4
+  const float* x;
+  const float* dy;
+  float* out;
+  int64_t ldx, lddy, ldo;
+  int use_pivot, bessel, training;
+  float eps, decay;
+  float* mean;    // forward: written; backward: read
+  float* var;
+  const float* scale;
+  const float* bias;
+  float* rmean;
+  float* rvar;
+  float* dscale;
+  float* dbias;
+  float* dmean;
+  float* dvar;
+};
+
+// Shared front end: merges the per-row pairs (a, b) of the column groups and returns, in
+// chan[c][0..1], the totals of local channel c (c < nch) of this workgroup.
+template <int GW>
+__device__ __forceinline__ void bn_rt_tile_channel_totals(float (&a)[4], float (&b)[4],
+                                                          float (*lds)[RowTilePos<GW>::kRows][2],
+                                                          float (*chan)[4], const RowTilePos<GW>& p, int cs,
+                                                          int nch)
+{
+  using P = RowTilePos<GW>;
+  if (GW == 4) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      a[r] += __shfl_xor(a[r], 16);
+      b[r] += __shfl_xor(b[r], 16);
+      a[r] += __shfl_xor(a[r], 32);
+      b[r] += __shfl_xor(b[r], 32);
+    }
+  }
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  if (lane < P::kQuads) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      lds[wave][4 * p.q + r][0] = a[r];
+      lds[wave][4 * p.q + r][1] = b[r];
+    }
+  }
+  __syncthreads();
+  const int c = threadIdx.x;
+  if (c < nch) {
+    float sa = 0.f, sb = 0.f;
+    for (int i = c * cs; i < (c + 1) * cs; ++i) {
+#pragma unroll
+      for (int k = 0; k < kRowTileWaves; ++k) {
+        sa += lds[k][i][0];
+        sb += lds[k][i][1];
+      }
+    }
+    chan[c][0] = sa;
+    chan[c][1] = sb;
+  }
+  __syncthreads();
+}
+
+template <int CPT, int GW>
+__global__ void __launch_bounds__(kRowTileThreads)
+bn_rt_fwd_tile(BnRtTileArgs a)
+{
+  using P = RowTilePos<GW>;
+  __shared__ float lds[kRowTileWaves][P::kRows][2];
+  __shared__ float chan[P::kRows][4];
+  const P p;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * a.rows_eff;
+  const int local = 4 * p.q;
+  const int64_t rows_here = imin64(a.rows_eff, a.h - base);  // a multiple of cs and of 4
+  const bool row_ok = local < rows_here;
+  const int64_t r0 = base + (row_ok ? local : 0);
+  const int cs = static_cast<int>(a.cs);
+  const int nch = static_cast<int>(rows_here / cs);
+
+  float K[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) K[r] = a.use_pivot ? a.x[((r0 + r) / cs) * cs] : 0.f;
+  float v[CPT][4];
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) {
+    const int64_t c = p.g + P::kGroups * j;
+    if (row_ok && c < a.w) {
+      Vec16<float>::load(a.x + r0 + c * a.ldx, v[j]);
+    }
+    else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[j][r] = K[r];
+    }
+  }
+  float s[4] = {0.f, 0.f, 0.f, 0.f}, sq[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < CPT; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float d = v[j][r] - K[r];
+      s[r] += d;
+      sq[r] = __builtin_fmaf(d, d, sq[r]);
+    }
+  bn_rt_tile_channel_totals<GW>(s, sq, lds, chan, p, cs, nch);
+  // one thread per channel finishes it and leaves (mean, 1/stdev) for the rows
+  if (static_cast<int>(threadIdx.x) < nch) {
+    const int64_t ch = base / cs + threadIdx.x;
+    float m, var;
+    if (a.n <= 1) {  // batch_normalization.cpp:118-120
+      m = a.x[ch * cs];
+      var = 1.f;
+    }
+    else {
+      const float Kc = a.use_pivot ? a.x[ch * cs] : 0.f;
+      stats_from_sums(chan[threadIdx.x][0], chan[threadIdx.x][1], Kc, a.n, a.bessel, a.eps, m, var);
+      a.rmean[ch] = a.decay * a.rmean[ch] + (1.f - a.decay) * m;
+      a.rvar[ch] = a.decay * a.rvar[ch] + (1.f - a.decay) * var;
+    }
+    a.mean[ch] = m;
+    a.var[ch] = var;
+    chan[threadIdx.x][2] = m;
+    chan[threadIdx.x][3] = 1.0f / sqrtf(var + a.eps);
+  }
+  __syncthreads();
+  if (!row_ok) return;
+  float mean[4], inv[4], sc[4], bi[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int lc = (local + r) / cs;
+    mean[r] = chan[lc][2];
+    inv[r] = chan[lc][3];
+    sc[r] = a.scale[base / cs + lc];
+    bi[r] = a.bias[base / cs + lc];
+  }
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) {
+    const int64_t c = p.g + P::kGroups * j;
+    if (c < a.w) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[j][r] = sc[r] * ((v[j][r] - mean[r]) * inv[r]) + bi[r];
+      Vec16<float>::store(a.out + r0 + c * a.ldo, v[j]);
+    }
+  }
+}
+
+template <int CPT, int GW>
+__global__ void __launch_bounds__(kRowTileThreads)
+bn_rt_bwd_tile(BnRtTileArgs a)
+{
+  using P = RowTilePos<GW>;
+  __shared__ float lds[kRowTileWaves][P::kRows][2];
+  __shared__ float chan[P::kRows][4];
+  const P p;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * a.rows_eff;
+  const int local = 4 * p.q;
+  const int64_t rows_here = imin64(a.rows_eff, a.h - base);
+  const bool row_ok = local < rows_here;
+  const int64_t r0 = base + (row_ok ? local : 0);
+  const int cs = static_cast<int>(a.cs);
+  const int nch = static_cast<int>(rows_here / cs);
+
+  float mean[4], k0[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int64_t ch = (r0 + r) / cs;
+    mean[r] = a.mean[ch];
+    k0[r] = a.scale[ch] * (1.0f / sqrtf(a.var[ch] + a.eps));
+  }
+  float xc[CPT][4], g[CPT][4];
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) {
+    const int64_t c = p.g + P::kGroups * j;
+    if (row_ok && c < a.w) {
+      Vec16<float>::load(a.x + r0 + c * a.ldx, xc[j]);
+      Vec16<float>::load(a.dy + r0 + c * a.lddy, g[j]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) xc[j][r] -= mean[r];
+    }
+    else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) xc[j][r] = g[j][r] = 0.f;
+    }
+  }
+  float sa[4] = {0.f, 0.f, 0.f, 0.f}, sb[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < CPT; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      sa[r] += g[j][r];
+      sb[r] = __builtin_fmaf(g[j][r], xc[j][r], sb[r]);
+    }
+  bn_rt_tile_channel_totals<GW>(sa, sb, lds, chan, p, cs, nch);
+  if (static_cast<int>(threadIdx.x) < nch) {
+    const int64_t ch = base / cs + threadIdx.x;
+    const float inv_stdev = 1.0f / sqrtf(a.var[ch] + a.eps);
+    float ds, db, dm, dv;
+    grads_from_sums(chan[threadIdx.x][0], chan[threadIdx.x][1], a.scale[ch], inv_stdev, ds, db, dm, dv);
+    if (!a.training) dm = dv = 0.f;  // statistics are constants outside training
+    a.dscale[ch] = ds;
+    a.dbias[ch] = db;
+    a.dmean[ch] = dm;
+    a.dvar[ch] = dv;
+    chan[threadIdx.x][2] = dm / static_cast<float>(a.n);
+    chan[threadIdx.x][3] = dv * 2.f / static_cast<float>(a.n - (a.bessel ? 1 : 0));
+  }
+  __syncthreads();
+  if (!row_ok) return;
+  float k1[4], k2[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int lc = (local + r) / cs;
+    k1[r] = chan[lc][2];
+    k2[r] = chan[lc][3];
+  }
+  const bool zero = a.n <= 1;
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) {
+    const int64_t c = p.g + P::kGroups * j;
+    if (c < a.w) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) g[j][r] = zero ? 0.f : g[j][r] * k0[r] + k1[r] + k2[r] * xc[j][r];
+      Vec16<float>::store(a.out + r0 + c * a.ldo, g[j]);
+    }
+  }
+}
+
+// Rows a workgroup of the register-resident variant takes: the largest multiple of
+// lcm(cs, 4) within `rows` (0: channels too long for a workgroup).
+inline int bn_rt_tile_rows(int64_t cs, int rows)
+{
+  int64_t l = cs;
+  while (l % 4 != 0) l += cs;  // lcm(cs, 4)
+  if (l > rows) return 0;
+  return static_cast<int>((rows / l) * l);
+}
+
 inline size_t bn_rt_workspace_bytes(int64_t h, int64_t w)
 {
   const RowTilePlan p = row_tile_plan(h, w);

@@ -309,6 +309,10 @@ BN_CASES = [
     ((2048, 7, 7), 16, True, 0), ((4096,), 64, True, 0), ((64, 7, 7), 300, False, 0), ((12, 3, 3), 20, True, 0),
     ((8, 5), 7, True, 4), ((4, 1), 1, True, 0), ((1024, 1), 2048, True, 0),
     ((512, 2, 2), 40, True, 0), ((300, 8), 33, False, 0), ((64, 4), 700, True, 4),   # one or two vectors per channel
+    # register-resident row tiles (w <= 256): 64-row and 256-row layouts, every columns-per-thread count
+    ((4096,), 5, True, 0), ((4096,), 30, True, 0), ((1024, 1), 100, True, 0), ((2000, 2), 200, False, 0),
+    ((333, 4), 256, True, 0), ((128, 7, 7), 3, True, 0), ((128, 7, 7), 10, True, 0), ((64, 7, 7), 24, True, 0),
+    ((64, 7, 7), 40, False, 0), ((32, 7, 7), 64, True, 4), ((40, 5, 5), 50, True, 0), ((16, 3, 3), 250, True, 0),
 ]
 
 
