@@ -693,6 +693,7 @@ static int bn_split(int64_t C, int64_t cs, int64_t w)
 // the channel walk would fetch one 16- or 32-byte piece per column (16384 x 4, w = 256:
 // 450 us per step that way).
 static bool bn_rt_shape(int64_t cs) { return cs % 4 != 0 || cs <= 8; }
+constexpr int64_t kBnTileMaxCs = 16;  // aligned channels up to here still try the register-resident row tile
 
 static size_t bn_workspace(int64_t C, int64_t cs, int64_t w)
 {
@@ -910,6 +911,15 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   const int pivot = (flags & LBN_STATS_SUMSQ) ? 0 : 1;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, y, ldy);
   if constexpr (std::is_same<S, float>::value) {
+    // channels of three or four vectors: the register tile when the mini-batch fits it
+    // (1024 x 16, w = 256: 19 us per step against 25 us for clusters), else clusters
+    if (!bn_rt_shape(cs) && cs <= kBnTileMaxCs && row_quads_ok(C * cs, w, x, ldx) && row_quads_ok(C * cs, w, y, ldy)) {
+      BnRtTileArgs t{};
+      t.h = C * cs, t.w = w, t.cs = cs, t.n = cs * w, t.x = x, t.out = y, t.ldx = ldx, t.ldo = ldy;
+      t.use_pivot = pivot, t.bessel = bessel, t.eps = epsilon, t.decay = decay, t.mean = mean, t.var = var;
+      t.scale = scale, t.bias = bias, t.rmean = running_mean, t.rvar = running_var;
+      if (bn_rt_try_tile<false>(st, t)) return launch_status();
+    }
     if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, y, ldy) &&
         (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0) {
       const int64_t h = C * cs;
@@ -972,6 +982,15 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   const int64_t n = cs * w;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, dy, lddy) && bn_vec_ok<S>(cs, w, dx, lddx);
   if constexpr (std::is_same<S, float>::value) {
+    if (!bn_rt_shape(cs) && cs <= kBnTileMaxCs && row_quads_ok(C * cs, w, x, ldx) && row_quads_ok(C * cs, w, dy, lddy) &&
+        row_quads_ok(C * cs, w, dx, lddx)) {
+      BnRtTileArgs t{};
+      t.h = C * cs, t.w = w, t.cs = cs, t.n = n, t.x = x, t.dy = dy, t.out = dx, t.ldx = ldx, t.lddy = lddy, t.ldo = lddx;
+      t.bessel = bessel, t.training = training, t.eps = epsilon;
+      t.mean = const_cast<float*>(use_mean), t.var = const_cast<float*>(use_var), t.scale = scale;
+      t.dscale = dscale, t.dbias = dbias, t.dmean = dmean, t.dvar = dvar;
+      if (bn_rt_try_tile<true>(st, t)) return launch_status();
+    }
     if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, dy, lddy) && bn_rt_usable(C, cs, w, dx, lddx) &&
         (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0) {
       const int64_t h = C * cs;

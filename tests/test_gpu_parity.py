@@ -313,6 +313,7 @@ BN_CASES = [
     ((4096,), 5, True, 0), ((4096,), 30, True, 0), ((1024, 1), 100, True, 0), ((2000, 2), 200, False, 0),
     ((333, 4), 256, True, 0), ((128, 7, 7), 3, True, 0), ((128, 7, 7), 10, True, 0), ((64, 7, 7), 24, True, 0),
     ((64, 7, 7), 40, False, 0), ((32, 7, 7), 64, True, 4), ((40, 5, 5), 50, True, 0), ((16, 3, 3), 250, True, 0),
+    ((256, 4, 4), 200, True, 0), ((100, 12), 64, True, 0),
 ]
 
 
