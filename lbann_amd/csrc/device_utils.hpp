@@ -128,6 +128,39 @@ struct Vec16<f32x1> {
   static __device__ __forceinline__ void store1(f32x1* p, float v) { p->v = v; }
 };
 
+// fp16 storage accessed one pair (4 bytes) at a time: for rows whose length is even but
+// not a multiple of 8, or that start on 4-byte but not 16-byte boundaries.  The type has
+// the size of one half, so pointer offsets count halves like those of __half.
+struct f16x2 {
+  unsigned short bits;
+};
+
+template <>
+struct Vec16<f16x2> {
+  static constexpr int N = 2;
+  using raw_t = unsigned int;
+  static __device__ __forceinline__ raw_t load_raw(const f16x2* p)
+  {
+    return *reinterpret_cast<const unsigned int*>(p);
+  }
+  static __device__ __forceinline__ void unpack(const raw_t& r, float (&v)[2])
+  {
+    __half2 h;
+    __builtin_memcpy(&h, &r, 4);
+    const float2 f = __half22float2(h);
+    v[0] = f.x;
+    v[1] = f.y;
+  }
+  static __device__ __forceinline__ void load(const f16x2* p, float (&v)[2]) { unpack(load_raw(p), v); }
+  static __device__ __forceinline__ void store(f16x2* p, const float (&v)[2])
+  {
+    const __half2 h = __floats2half2_rn(v[0], v[1]);
+    unsigned int w;
+    __builtin_memcpy(&w, &h, 4);
+    *reinterpret_cast<unsigned int*>(p) = w;
+  }
+};
+
 // VE consecutive fp32 weights (scale, bias, their partial gradients) at p: 16-byte accesses
 // when a thread owns at least four of them, single floats otherwise.
 template <int VE>

@@ -676,6 +676,13 @@ static int64_t ln_wgrad_slabs(int64_t units, int64_t rows)
   return s < 1 ? 1 : s;
 }
 
+// fp16 rows that can be walked in 4-byte pairs: even offsets everywhere.
+static bool rows_aligned4(const void* base, int64_t stride, int64_t ld, int64_t groups, int64_t width)
+{
+  return (reinterpret_cast<uintptr_t>(base) & 3u) == 0 && (groups <= 1 || stride % 2 == 0) &&
+         (width <= 1 || ld % 2 == 0);
+}
+
 constexpr int64_t kLnMaxScalarRowFwd = 8192;  // rows accessed one float at a time: 1024 threads x 8
 constexpr int64_t kLnMaxScalarRowBwd = 4096;  // 512 threads x 8
 
@@ -695,6 +702,10 @@ static size_t ln_bwd_workspace(int64_t n, int64_t rows, int ve)
   }
   if (ve == 4 && n <= kLnMaxScalarRowBwd) {  // fp32 rows off the 16-byte grid: one float per access
     const LnBwdPlan p = plan_ln_bwd(n, rows, 1, 4);
+    if (p.tpr) cover(static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
+  }
+  if (ve == 8 && n % 2 == 0 && n / 2 <= kLnMaxScalarRowBwd) {  // fp16 rows: one pair per access
+    const LnBwdPlan p = plan_ln_bwd(n / 2, rows, 2, 2);
     if (p.tpr) cover(static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
   }
   return need;
@@ -765,6 +776,16 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                        ldx, ldy, map, n / VE, inv_n, eps, stats, lds, gamma, beta, sumsq);
     return launch_status();
   }
+  if constexpr (std::is_same<T, __half>::value) {
+    // fp16 rows off the 16-byte grid with an even length: the same kernels, one pair per access
+    if (n % 2 == 0 && n / 2 <= kLnMaxScalarRowFwd && rows_aligned4(x, stride, ldx, G, w) &&
+        rows_aligned4(y, stride, ldy, G, w)) {
+      if (int r = ln_fwd_rows_launch<f16x2>(st, reinterpret_cast<const f16x2*>(x), reinterpret_cast<f16x2*>(y),
+                                            ldx, ldy, map, rows, n / 2, inv_n, eps, stats,
+                                            lds, gamma, beta, sumsq))
+        return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
+    }
+  }
   if constexpr (std::is_same<T, float>::value) {
     if (n > 1 && n <= kLnMaxScalarRowFwd) {  // rows off the 16-byte grid: the same kernels, one float per access
       if (int r = ln_fwd_rows_launch<f32x1>(st, reinterpret_cast<const f32x1*>(x), reinterpret_cast<f32x1*>(y),
@@ -833,7 +854,7 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
   X(64, 4, 1) X(64, 4, 2) X(64, 4, 4) X(256, 2, 1) X(256, 2, 2) X(256, 1, 1) X(256, 1, 2)
   X(512, 1, 1) X(512, 1, 2) X(512, 1, 4)
   if constexpr (VE <= 4) { X(256, 2, 4) X(256, 1, 4) X(512, 1, 8) }
-  if constexpr (VE == 1) { X(64, 4, 8) X(256, 2, 8) X(256, 1, 8) }
+  if constexpr (VE <= 2) { X(64, 4, 8) X(256, 2, 8) X(256, 1, 8) }
 #undef X
   if (!launched) return 0;
   if (wgrad) {
@@ -892,6 +913,16 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                        ldsg, gamma);
   }
   else {
+    if constexpr (std::is_same<T, __half>::value) {
+      if (n % 2 == 0 && n / 2 <= kLnMaxScalarRowBwd && rows_aligned4(x, stride, ldx, G, w) &&
+          rows_aligned4(dy, stride, lddy, G, w) && rows_aligned4(dx, stride, lddx, G, w)) {
+        if (int r = ln_bwd_rows_launch<f16x2>(st, wgrad, reinterpret_cast<const f16x2*>(x),
+                                              reinterpret_cast<const f16x2*>(dy), reinterpret_cast<f16x2*>(dx),
+                                              ldx, lddy, lddx, map, rows, n / 2, n, 2,
+                                              eps, stats, lds, sgrad, ldsg, gamma, dgamma, dbeta, ws, ws_bytes))
+          return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
+      }
+    }
     if constexpr (std::is_same<T, float>::value) {
       if (n <= kLnMaxScalarRowBwd) {  // rows off the 16-byte grid: the same kernels, one float per access
         if (int r = ln_bwd_rows_launch<f32x1>(st, wgrad, reinterpret_cast<const f32x1*>(x),

@@ -232,7 +232,11 @@ def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
                                                    ((16384,), 0, 3, 0), ((16384,), 0, 40, 0), ((8192,), 0, 300, 0),
                                                    ((768,), 0, 1000, 0), ((12288,), 0, 9, 0),
                                                    ((32768,), 0, 20, 0), ((150528,), 0, 3, 0), ((20000,), 0, 5, 8),
-                                                   ((1024, 256), -1, 8, 0), ((512, 64), -1, 16, 0), ((128, 512), -1, 40, 0)])
+                                                   ((1024, 256), -1, 8, 0), ((512, 64), -1, 16, 0), ((128, 512), -1, 40, 0),
+                                                   # even lengths that are not a multiple of 8: one pair per access
+                                                   ((4100,), 0, 40, 0), ((1002,), 0, 33, 0), ((6, 770), -1, 9, 0),
+                                                   ((8190,), 0, 5, 2), ((16382,), 0, 3, 0), ((4100, 12), -1, 2, 0),
+                                                   ((1001,), 0, 7, 0)])   # odd: scalar fallback
 def test_layer_norm_f16(L, dims, start_dim, w, pad):
     rng = np.random.default_rng(int(np.prod(dims)) * 3 + w)
     h = int(np.prod(dims))
