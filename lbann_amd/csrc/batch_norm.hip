@@ -504,7 +504,7 @@ __global__ void __launch_bounds__(T)
 bn_fwd_cluster(BnFwdArgs<S> a, unsigned seg, unsigned E)
 {
   __shared__ float red[2 * (T / kWave)];
-  __shared__ float bc[2];
+  __shared__ float bc[3][2];
   const int nc = gridDim.x / a.M;
   const int cl = blockIdx.x / a.M;
   const int k = blockIdx.x - cl * a.M;
@@ -514,10 +514,13 @@ bn_fwd_cluster(BnFwdArgs<S> a, unsigned seg, unsigned E)
   bn_fwd_load<S, V>(t0, a, cl, ix);
   if (cl + nc < a.C) bn_fwd_load<S, V>(t1, a, cl + nc, ix);
   bn_fwd_reduce<S, T, V>(a, ix, cl, k, t0, red);
+  __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
+  // Each position of the rotation has its own broadcast pair: a step without a reduction has
+  // no barrier between the reads of one finish and the write of the next.
   for (int ch = cl; ch < a.C; ch += 3 * nc) {
-    bn_fwd_step<S, T, V>(a, ix, ch, nc, k, t0, t1, t2, red, bc);
-    if (ch + nc < a.C) bn_fwd_step<S, T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, red, bc);
-    if (ch + 2 * nc < a.C) bn_fwd_step<S, T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, red, bc);
+    bn_fwd_step<S, T, V>(a, ix, ch, nc, k, t0, t1, t2, red, bc[0]);
+    if (ch + nc < a.C) bn_fwd_step<S, T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, red, bc[1]);
+    if (ch + 2 * nc < a.C) bn_fwd_step<S, T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, red, bc[2]);
   }
 }
 
@@ -634,7 +637,7 @@ __global__ void __launch_bounds__(T)
 bn_bwd_cluster(BnBwdArgs<S> a, unsigned seg, unsigned E)
 {
   __shared__ float red[2 * (T / kWave)];
-  __shared__ float bc[2];
+  __shared__ float bc[3][2];
   const int nc = gridDim.x / a.M;
   const int cl = blockIdx.x / a.M;
   const int k = blockIdx.x - cl * a.M;
@@ -644,10 +647,13 @@ bn_bwd_cluster(BnBwdArgs<S> a, unsigned seg, unsigned E)
   bn_bwd_load<S, V>(t0, a, cl, ix);
   if (cl + nc < a.C) bn_bwd_load<S, V>(t1, a, cl + nc, ix);
   bn_bwd_reduce<S, T, V>(a, ix, cl, k, t0, red);
+  __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
+  // Each position of the rotation has its own broadcast pair: a step without a reduction has
+  // no barrier between the reads of one finish and the write of the next.
   for (int ch = cl; ch < a.C; ch += 3 * nc) {
-    bn_bwd_step<S, T, V>(a, ix, ch, nc, k, t0, t1, t2, red, bc);
-    if (ch + nc < a.C) bn_bwd_step<S, T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, red, bc);
-    if (ch + 2 * nc < a.C) bn_bwd_step<S, T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, red, bc);
+    bn_bwd_step<S, T, V>(a, ix, ch, nc, k, t0, t1, t2, red, bc[0]);
+    if (ch + nc < a.C) bn_bwd_step<S, T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, red, bc[1]);
+    if (ch + 2 * nc < a.C) bn_bwd_step<S, T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, red, bc[2]);
   }
 }
 

@@ -108,16 +108,16 @@ __device__ __forceinline__ float2 bn_rt_channel_total(const float2* part, int64_
                                                       int64_t c)
 {
   const int lane = threadIdx.x & (kWave - 1);
-  float a = 0.f, b = 0.f;
+  double a = 0., b = 0.;  // a lane adds up to slabs x cs / 64 partials in sequence
   for (int s = 0; s < slabs; ++s) {
     const float2* row = part + static_cast<int64_t>(s) * h + c * cs;
     for (int64_t i = lane; i < cs; i += kWave) {
       const float2 v = row[i];
-      a += v.x;
-      b += v.y;
+      a += static_cast<double>(v.x);
+      b += static_cast<double>(v.y);
     }
   }
-  return make_float2(wave_sum(a), wave_sum(b));
+  return make_float2(wave_sum(static_cast<float>(a)), wave_sum(static_cast<float>(b)));
 }
 
 // One wave per channel (4 channels per workgroup).
@@ -283,16 +283,18 @@ __device__ __forceinline__ void bn_rt_tile_channel_totals(float (&a)[4], float (
   __syncthreads();
   const int c = threadIdx.x;
   if (c < nch) {
-    float sa = 0.f, sb = 0.f;
+    // one thread adds cs x waves partials in sequence: in double, so that sums about a pivot
+    // far from the mean (large partials, small total) lose nothing here
+    double sa = 0., sb = 0.;
     for (int i = c * cs; i < (c + 1) * cs; ++i) {
 #pragma unroll
       for (int k = 0; k < kRowTileWaves; ++k) {
-        sa += lds[k][i][0];
-        sb += lds[k][i][1];
+        sa += static_cast<double>(lds[k][i][0]);
+        sb += static_cast<double>(lds[k][i][1]);
       }
     }
-    chan[c][0] = sa;
-    chan[c][1] = sb;
+    chan[c][0] = static_cast<float>(sa);
+    chan[c][1] = static_cast<float>(sb);
   }
   __syncthreads();
 }

@@ -361,7 +361,7 @@ __global__ void __launch_bounds__(kClusterThreads)
 sm_fwd_cluster(SmClusterArgs a)
 {
   __shared__ float red[kClusterThreads / kWave][2];
-  __shared__ float bc[2];
+  __shared__ float bc[3][2];
   const int64_t nc = gridDim.x / a.M;
   const int64_t cl = blockIdx.x / a.M;
   const int k = blockIdx.x - static_cast<int>(cl) * a.M;
@@ -371,10 +371,13 @@ sm_fwd_cluster(SmClusterArgs a)
   sm_cl_load<V>(t0.v, a.a + a.map.offset(cl, a.lda), base, a.nvec, -FLT_MAX);
   if (cl + nc < a.rows) sm_cl_load<V>(t1.v, a.a + a.map.offset(cl + nc, a.lda), base, a.nvec, -FLT_MAX);
   sm_cl_fwd_reduce<V, KIND>(a, cl, k, base, t0, red);
+  __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
+  // Each position of the rotation has its own broadcast slot: a step without a reduction has
+  // no barrier between the reads of one finish and the write of the next.
   for (int64_t row = cl; row < a.rows; row += 3 * nc) {
-    sm_cl_fwd_step<V, KIND>(a, row, nc, k, base, t0, t1, t2, red, bc);
-    if (row + nc < a.rows) sm_cl_fwd_step<V, KIND>(a, row + nc, nc, k, base, t1, t2, t0, red, bc);
-    if (row + 2 * nc < a.rows) sm_cl_fwd_step<V, KIND>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc);
+    sm_cl_fwd_step<V, KIND>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
+    if (row + nc < a.rows) sm_cl_fwd_step<V, KIND>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
+    if (row + 2 * nc < a.rows) sm_cl_fwd_step<V, KIND>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
   }
 }
 
@@ -448,7 +451,7 @@ __global__ void __launch_bounds__(kClusterThreads)
 sm_bwd_cluster(SmClusterArgs a)
 {
   __shared__ float red[kClusterThreads / kWave];
-  __shared__ float bc[1];
+  __shared__ float bc[3][1];
   const int64_t nc = gridDim.x / a.M;
   const int64_t cl = blockIdx.x / a.M;
   const int k = blockIdx.x - static_cast<int>(cl) * a.M;
@@ -458,10 +461,13 @@ sm_bwd_cluster(SmClusterArgs a)
   sm_cl_bwd_load<V>(a, cl, base, t0);
   if (cl + nc < a.rows) sm_cl_bwd_load<V>(a, cl + nc, base, t1);
   sm_cl_bwd_reduce<V, KIND>(a, cl, k, t0, red);
+  __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
+  // Each position of the rotation has its own broadcast slot: a step without a reduction has
+  // no barrier between the reads of one finish and the write of the next.
   for (int64_t row = cl; row < a.rows; row += 3 * nc) {
-    sm_cl_bwd_step<V, KIND>(a, row, nc, k, base, t0, t1, t2, red, bc);
-    if (row + nc < a.rows) sm_cl_bwd_step<V, KIND>(a, row + nc, nc, k, base, t1, t2, t0, red, bc);
-    if (row + 2 * nc < a.rows) sm_cl_bwd_step<V, KIND>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc);
+    sm_cl_bwd_step<V, KIND>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
+    if (row + nc < a.rows) sm_cl_bwd_step<V, KIND>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
+    if (row + 2 * nc < a.rows) sm_cl_bwd_step<V, KIND>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
   }
 }
 

@@ -318,6 +318,8 @@ BN_CASES = [
     ((333, 4), 256, True, 0), ((128, 7, 7), 3, True, 0), ((128, 7, 7), 10, True, 0), ((64, 7, 7), 24, True, 0),
     ((64, 7, 7), 40, False, 0), ((32, 7, 7), 64, True, 4), ((40, 5, 5), 50, True, 0), ((16, 3, 3), 250, True, 0),
     ((256, 4, 4), 200, True, 0), ((100, 12), 64, True, 0),
+    # more channels than resident clusters: some clusters take two or three channels in turn, others one
+    ((478, 16), 577, True, 0), ((1500, 4, 4), 600, False, 0), ((900, 64), 300, True, 0),
 ]
 
 

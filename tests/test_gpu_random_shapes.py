@@ -2,6 +2,8 @@
 layer, GPU through the C ABI against the CPU oracle.  The shapes are drawn so that the
 vector kernels, their masked variants and the scalar fallbacks are all hit (lengths that
 are and are not multiples of 4 or 8, padded leading dimensions, single rows and columns)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -42,7 +44,8 @@ def draw_length(rng):
     return int(rng.integers(3000, 40000))
 
 
-CASES = list(range(24))
+# LBN_RANDOM_CASES widens the sweep for a one-off soak; the default keeps the suite short
+CASES = list(range(int(os.environ.get("LBN_RANDOM_CASES", "24"))))
 
 
 @pytest.mark.parametrize("case", CASES)
@@ -201,3 +204,98 @@ def test_cross_entropy_and_scale_bias_random(L, case):
         check(f"cross entropy dx labels={use_labels} {tag}", dx.to_numpy(), rdx, edx)
         if not use_labels:
             check(f"cross entropy dtruth {tag}", dt.to_numpy(), rdt, edt)
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_many_short_rows_random(L, case):
+    """Thousands of rows of a few to a few hundred entries: the 16-lane teams and the
+    single-float / pair-access variants of the row kernels."""
+    rng = np.random.default_rng(6000 + case)
+    n = int(rng.choice([rng.integers(1, 40), rng.integers(1, 12) * 4, rng.integers(1, 40) * 8, rng.integers(40, 300)]))
+    G = int(rng.choice([1, 1, 3, 16]))
+    w = int(rng.integers(4096 // G + 1, 9000 // G + 2))
+    h = G * n
+    pad = int(rng.choice([0, 0, 0, 4, 1]))
+    tag = f"G={G} n={n} w={w} pad={pad}"
+    x, dy = rand(rng, h, w, 0.3, 1.5), rand(rng, h, w)
+    # channelwise softmax over G windows of n entries
+    cw = L.channelwise_softmax_layer((G, n))
+    y = cw.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    dx = cw.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    check("channelwise y " + tag, y, orc.channelwise_softmax_fwd(x, G, n, n), orc.channelwise_softmax_fwd(f64(x), G, n, n))
+    check("channelwise dx " + tag, dx, orc.channelwise_softmax_bwd(y, dy, G, n, n),
+          orc.channelwise_softmax_bwd(f64(y), f64(dy), G, n, n))
+    # layer norm over the same rows, fp32 and fp16 storage, with and without weights
+    for half in (False, True):
+        affine = bool((case + half) % 2)
+        xs, gs = (x.astype(np.float16).astype(np.float32), dy.astype(np.float16).astype(np.float32)) if half else (x, dy)
+        g = (1 + 0.2 * rng.standard_normal(n)).astype(np.float32) if affine else None
+        b = (0.2 * rng.standard_normal(n)).astype(np.float32) if affine else None
+        kw = dict(scale_values=g, bias_values=b) if affine else {}
+        dims, sd = ((G, n), 1) if G > 1 else ((n,), 0)
+        layer = L.layer_norm_layer(dims, 1e-5, affine, affine, sd, **kw)
+        tdt, tol = (torch.float16, TOL_F16) if half else (torch.float32, TOL_F32)
+        yy = layer.forward(L.DeviceMatrix.from_numpy(xs, dtype=tdt, ldim=h + pad)).to_numpy()
+        dd = layer.backward(L.DeviceMatrix.from_numpy(gs, dtype=tdt, ldim=h + pad)).to_numpy()
+        ref, ex = {}, {}
+        for dst, conv in ((ref, f32), (ex, f64)):
+            gg = None if g is None else conv(g)
+            bb = None if b is None else conv(b)
+            dst["y"], st = orc.layer_norm_fwd(conv(xs), G, n, n, 1e-5, gg, bb)
+            dst["dx"], _, dst["dscale"], dst["dbias"] = orc.layer_norm_bwd(conv(xs), conv(gs), st, G, n, n, 1e-5, gg,
+                                                                             affine, affine)
+        t2 = tag + f" half={half} affine={affine}"
+        check("layer norm y " + t2, yy, ref["y"], ex["y"], tol=tol)
+        if n > 1:
+            check("layer norm dx " + t2, dd, ref["dx"], ex["dx"], tol=tol)
+        if affine:
+            check("layer norm dscale " + t2, layer.m_scale_gradient.to_numpy(), ref["dscale"], ex["dscale"], tol=tol)
+            check("layer norm dbias " + t2, layer.m_bias_gradient.to_numpy(), ref["dbias"], ex["dbias"], tol=tol)
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_small_channels_random(L, case):
+    """Batch norm and channel-wise scale/bias on channels of 1 to 70 entries: the row-tile
+    kernels (register-resident and three-kernel) next to the channel walk."""
+    rng = np.random.default_rng(7000 + case)
+    cs = int(rng.choice([1, 1, 2, 4, 8, 9, 16, 25, 49, rng.integers(1, 70)]))
+    C = int(rng.integers(1, 600))
+    w = int(rng.choice([rng.integers(1, 70), rng.integers(70, 300), rng.integers(300, 700)]))
+    h = C * cs
+    pad = int(rng.choice([0, 0, 0, 4, 2]))
+    bessel = bool(case % 2)
+    tag = f"C={C} cs={cs} w={w} pad={pad}"
+    x, dy = rand(rng, h, w, 2.0, 3.0), rand(rng, h, w)
+    g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    b = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    bn = L.batch_normalization_layer((C, cs), 0.9, 1e-5, bessel, g, b)
+    y = bn.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    dx = bn.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    mv = bn.m_mean_and_var.to_numpy()
+    ref, ex = {}, {}
+    for dst, conv in ((ref, f32), (ex, f64)):
+        rm, rv = conv(np.zeros(C)), conv(np.ones(C))
+        dst["y"], m, v = orc.batch_norm_fwd(conv(x), C, cs, 1e-5, 0.9, conv(g), conv(b), rm, rv, bessel)
+        dst["mean"], dst["var"], dst["rmean"], dst["rvar"] = m, v, rm, rv
+        dst["dx"], dst["dscale"], dst["dbias"], dst["dmean"], dst["dvar"] = orc.batch_norm_bwd(
+            conv(x), conv(dy), C, cs, 1e-5, m, v, conv(g), bessel=bessel)
+    mvg = bn.m_mean_and_var_gradient.to_numpy()
+    got = dict(y=y, dx=dx, mean=mv[:, 0], var=mv[:, 1], dscale=bn.m_scale_gradient.to_numpy(),
+               dbias=bn.m_bias_gradient.to_numpy(), dmean=mvg[:, 0], dvar=mvg[:, 1],
+               rmean=bn.weights[2].to_numpy(), rvar=bn.weights[3].to_numpy())
+    if cs * w <= 1:
+        for k in ("dmean", "dvar", "dscale", "dbias"):
+            got.pop(k)
+    for k in got:
+        check(f"batch norm {k} {tag}", got[k], ref[k], ex[k])
+    wts = np.asfortranarray(np.stack([g, b], axis=1))
+    sb = L.channelwise_scale_bias_layer((C, cs))
+    sb.set_weights(g, b)
+    y = sb.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    dx = sb.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    check("channelwise scale/bias y " + tag, y, orc.channelwise_scale_bias_fwd(x, wts, C, cs),
+          orc.channelwise_scale_bias_fwd(f64(x), f64(wts), C, cs))
+    rdx, rwg = orc.channelwise_scale_bias_bwd(x, dy, wts, C, cs)
+    edx, ewg = orc.channelwise_scale_bias_bwd(f64(x), f64(dy), f64(wts), C, cs)
+    check("channelwise scale/bias dx " + tag, dx, rdx, edx)
+    check("channelwise scale/bias dweights " + tag, sb.m_weights_gradient.to_numpy(), rwg, ewg)
