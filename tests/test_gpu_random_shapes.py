@@ -299,3 +299,76 @@ def test_small_channels_random(L, case):
     edx, ewg = orc.channelwise_scale_bias_bwd(f64(x), f64(dy), f64(wts), C, cs)
     check("channelwise scale/bias dx " + tag, dx, rdx, edx)
     check("channelwise scale/bias dweights " + tag, sb.m_weights_gradient.to_numpy(), rwg, ewg)
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_many_long_rows_random(L, case):
+    """More long rows than the device holds clusters at once: the persistent cluster kernels
+    rotate through several rows per workgroup, and the long-row layer norm streams them."""
+    rng = np.random.default_rng(8000 + case)
+    n = int(rng.choice([rng.integers(4200, 9000) * 4, rng.integers(9000, 40000) * 4, rng.integers(17000, 150000)]))
+    w = int(rng.integers(2, max(3, 12_000_000 // n)))
+    pad = int(rng.choice([0, 0, 4, 1]))
+    tag = f"n={n} w={w} pad={pad}"
+    x, dy = rand(rng, n, w, 0.0, 2.5), rand(rng, n, w)
+    kind, layer, fwd, bwd = (("softmax", L.softmax_layer(), orc.softmax_fwd, orc.softmax_bwd),
+                             ("log_softmax", L.log_softmax_layer(), orc.log_softmax_fwd, orc.log_softmax_bwd))[case % 2]
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=n + pad)).to_numpy()
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=n + pad)).to_numpy()
+    check(f"{kind} y {tag}", y, fwd(x), fwd(f64(x)))
+    check(f"{kind} dx {tag}", dx, bwd(y, dy), bwd(f64(y), f64(dy)))
+    half = bool(case % 3 == 1)
+    if half:
+        x, dy = x.astype(np.float16).astype(np.float32), dy.astype(np.float16).astype(np.float32)
+    g = (1 + 0.2 * rng.standard_normal(n)).astype(np.float32)
+    b = (0.2 * rng.standard_normal(n)).astype(np.float32)
+    ln = L.layer_norm_layer((n,), 1e-5, True, True, 0, scale_values=g, bias_values=b)
+    tdt, tol = (torch.float16, TOL_F16) if half else (torch.float32, TOL_F32)
+    y = ln.forward(L.DeviceMatrix.from_numpy(x, dtype=tdt, ldim=n + pad)).to_numpy()
+    dx = ln.backward(L.DeviceMatrix.from_numpy(dy, dtype=tdt, ldim=n + pad)).to_numpy()
+    ref, ex = {}, {}
+    for dst, conv in ((ref, f32), (ex, f64)):
+        dst["y"], st = orc.layer_norm_fwd(conv(x), 1, n, n, 1e-5, conv(g), conv(b))
+        dst["dx"], _, dst["dscale"], dst["dbias"] = orc.layer_norm_bwd(conv(x), conv(dy), st, 1, n, n, 1e-5, conv(g),
+                                                                         True, True)
+    check(f"layer norm y {tag} half={half}", y, ref["y"], ex["y"], tol=tol)
+    check(f"layer norm dx {tag} half={half}", dx, ref["dx"], ex["dx"], tol=tol)
+    check(f"layer norm dscale {tag} half={half}", ln.m_scale_gradient.to_numpy(), ref["dscale"], ex["dscale"], tol=tol)
+    check(f"layer norm dbias {tag} half={half}", ln.m_bias_gradient.to_numpy(), ref["dbias"], ex["dbias"], tol=tol)
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_many_large_channels_random(L, case):
+    """Batch norm with more channels than resident clusters (fp32 and fp16 storage) and channel
+    sizes from a few vectors to a few thousand."""
+    rng = np.random.default_rng(9000 + case)
+    cs = int(rng.choice([8, 12, 16, 24, 32, 64, 196, 784, rng.integers(3, 200) * 8]))
+    w = int(rng.choice([rng.integers(2, 40), rng.integers(40, 400), rng.integers(400, 1200)]))
+    C = int(max(2, min(3000, rng.integers(4_000_000, 16_000_000) // (cs * w))))
+    h = C * cs
+    pad = int(rng.choice([0, 0, 8, 4]))
+    half = bool(case % 3 == 2)
+    bessel = bool(case % 2)
+    tag = f"C={C} cs={cs} w={w} pad={pad} half={half}"
+    x, dy = rand(rng, h, w, 2.0, 3.0), rand(rng, h, w)
+    if half:
+        x, dy = x.astype(np.float16).astype(np.float32), dy.astype(np.float16).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    b = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    bn = L.batch_normalization_layer((C, cs), 0.9, 1e-5, bessel, g, b)
+    tdt, tol = (torch.float16, TOL_F16) if half else (torch.float32, TOL_F32)
+    y = bn.forward(L.DeviceMatrix.from_numpy(x, dtype=tdt, ldim=h + pad)).to_numpy()
+    dx = bn.backward(L.DeviceMatrix.from_numpy(dy, dtype=tdt, ldim=h + pad)).to_numpy()
+    mv, mvg = bn.m_mean_and_var.to_numpy(), bn.m_mean_and_var_gradient.to_numpy()
+    ref, ex = {}, {}
+    for dst, conv in ((ref, f32), (ex, f64)):
+        rm, rv = conv(np.zeros(C)), conv(np.ones(C))
+        dst["y"], m, v = orc.batch_norm_fwd(conv(x), C, cs, 1e-5, 0.9, conv(g), conv(b), rm, rv, bessel)
+        dst["mean"], dst["var"] = m, v
+        dst["dx"], dst["dscale"], dst["dbias"], dst["dmean"], dst["dvar"] = orc.batch_norm_bwd(
+            conv(x), conv(dy), C, cs, 1e-5, m, v, conv(g), bessel=bessel)
+    got = dict(y=y, dx=dx, mean=mv[:, 0], var=mv[:, 1], dscale=bn.m_scale_gradient.to_numpy(),
+               dbias=bn.m_bias_gradient.to_numpy(), dmean=mvg[:, 0], dvar=mvg[:, 1])
+    for k in got:
+        # statistics and their gradients are fp32 whatever the storage type
+        check(f"batch norm {k} {tag}", got[k], ref[k], ex[k], tol=tol if k in ("y", "dx") else TOL_F32)
