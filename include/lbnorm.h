@@ -19,10 +19,13 @@
  * between the kernels of one call.
  *
  * HIP graphs: the compute entry points may be called on a stream that is recording
- * (hipStreamBeginCapture); they record kernel launches only.  While recording they
- * avoid the kernels in which workgroups wait for each other (those take a per-call
- * tag as an argument, which a replay would repeat) and use their multi-kernel
- * paths instead, so a replayed call can be slower than an eager one.
+ * (hipStreamBeginCapture); they record kernel launches only.  The kernels in which
+ * workgroups wait for each other tell one call's partial results from another's by
+ * a tag; a recorded call repeats its arguments, so while recording such a kernel is
+ * preceded by a one-thread kernel that advances a counter in the workspace, which
+ * the tag takes in.  The workspace passed while recording is therefore part of the
+ * graph's state: keep it allocated, and do not run two replays that share it at the
+ * same time.
  */
 #ifndef LBNORM_H_INCLUDED
 #define LBNORM_H_INCLUDED

@@ -511,6 +511,7 @@ bn_fwd_cluster(BnFwdArgs<S> a, unsigned seg, unsigned E)
   const BnIndex<V> ix = bn_make_index<T, V>(k, seg, E);
   BnFwdTile<S, V> t0, t1, t2;
   if (cl >= a.C) return;
+  cluster_resolve_tag(a.tag);
   bn_fwd_load<S, V>(t0, a, cl, ix);
   if (cl + nc < a.C) bn_fwd_load<S, V>(t1, a, cl + nc, ix);
   bn_fwd_reduce<S, T, V>(a, ix, cl, k, t0, red);
@@ -644,6 +645,7 @@ bn_bwd_cluster(BnBwdArgs<S> a, unsigned seg, unsigned E)
   const BnIndex<V> ix = bn_make_index<T, V>(k, seg, E);
   BnBwdTile<S, V> t0, t1, t2;
   if (cl >= a.C) return;
+  cluster_resolve_tag(a.tag);
   bn_bwd_load<S, V>(t0, a, cl, ix);
   if (cl + nc < a.C) bn_bwd_load<S, V>(t1, a, cl + nc, ix);
   bn_bwd_reduce<S, T, V>(a, ix, cl, k, t0, red);
@@ -737,12 +739,11 @@ static bool bn_launch_bwd_cluster(hipStream_t st, const BnBwdArgs<S>& a, int64_t
 }
 
 template <typename S>
-static bool bn_cluster_usable(int64_t C, int64_t cs, int64_t w, const void* ws, hipStream_t st)
+static bool bn_cluster_usable(int64_t C, int64_t cs, int64_t w, const void* ws)
 {
   static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
   const int64_t E = cs / Vec16<S>::N * w;
-  return !disabled && E < (int64_t(1) << 31) - 8192 && cs * w > 1 && C <= (1 << 24) && aligned16(ws) &&
-         !stream_is_capturing(st);
+  return !disabled && E < (int64_t(1) << 31) - 8192 && cs * w > 1 && C <= (1 << 24) && aligned16(ws);
 }
 
 // A thread keeps at most 16 entries of a forward tile and 8 + 8 of a backward tile in
@@ -754,12 +755,12 @@ static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
                                float* rmean, float* rvar, void* ws)
 {
   constexpr int VE = Vec16<S>::N;
-  if (!bn_cluster_usable<S>(C, cs, w, ws, st)) return false;
+  if (!bn_cluster_usable<S>(C, cs, w, ws)) return false;
   const int64_t E = cs / VE * w;
   const BnClusterShape p = bn_cluster_shape(E, 16 / VE, 256);
   if (!p.T) return false;
   const BnFwdArgs<S> a{x, y, ldx, ldy, cs, static_cast<int>(C), p.M, pivot, bessel, eps, decay, cs * w,
-                       cluster_workspace(ws), next_cluster_tag(), mean, var, scale, bias, rmean, rvar};
+                       cluster_workspace(ws), cluster_call_tag(st, cluster_workspace(ws)), mean, var, scale, bias, rmean, rvar};
   const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(E);
 #define X(TT, VV) \
   if (p.T == TT && p.V == VV) return bn_launch_fwd_cluster<S, TT, VV>(st, a, C, seg, Eu);
@@ -776,12 +777,12 @@ static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
                                float* dbias, float* dmean, float* dvar, void* ws)
 {
   constexpr int VE = Vec16<S>::N;
-  if (!bn_cluster_usable<S>(C, cs, w, ws, st)) return false;
+  if (!bn_cluster_usable<S>(C, cs, w, ws)) return false;
   const int64_t E = cs / VE * w;
   const BnClusterShape p = bn_cluster_shape(E, 8 / VE, 256);
   if (!p.T) return false;
   const BnBwdArgs<S> a{x, dy, dx, ldx, lddy, lddx, cs, static_cast<int>(C), p.M, bessel, eps, cs * w,
-                       cluster_workspace(ws), next_cluster_tag(), mean, var, scale, dscale, dbias, dmean, dvar};
+                       cluster_workspace(ws), cluster_call_tag(st, cluster_workspace(ws)), mean, var, scale, dscale, dbias, dmean, dvar};
   const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(E);
 #define X(TT, VV) \
   if (p.T == TT && p.V == VV) return bn_launch_bwd_cluster<S, TT, VV>(st, a, C, seg, Eu);

@@ -7,9 +7,11 @@
 //
 // Protocol (no fences, no cache write-back or invalidation, no clearing pass): a slot
 // is two 64-bit words, each holding one float of the pair and one half of a 64-bit
-// call tag.  The tag is drawn per call from a process-wide counter, so whatever an
-// earlier call (or anything else) left in the workspace can never look published: a
-// slot counts only when both of its words carry the two halves of this call's tag.
+// call tag.  The tag is drawn per call from a process-wide counter (and, for a call that a
+// HIP graph replays, advanced per replay through a counter word in the workspace), so
+// whatever an earlier call (or anything else) left in the workspace can never look
+// published: a slot counts only when both of its words carry the two halves of this
+// call's tag.
 // A workgroup publishes with two relaxed device-scope atomic 64-bit stores, and one
 // wave of each workgroup polls the M slots of its item in parallel (lane j reads slot
 // j) with relaxed device-scope atomic loads.  The pair is the only data that crosses
@@ -43,6 +45,10 @@ constexpr int kClusterTimedOut = 0x7E57FA11;
 
 struct ClusterTag {
   unsigned lo, hi;
+  // Null for an ordinary call.  A call recorded into a HIP graph repeats its arguments on
+  // every replay, so there the tag also takes in a counter word in the workspace that a
+  // one-thread kernel node in front of the cluster kernel advances (cluster_call_tag()).
+  const unsigned long long* replay_word;
 };
 
 // A fresh tag per call.  The counter starts from the clock so that slots written by
@@ -52,7 +58,27 @@ inline ClusterTag next_cluster_tag()
   static std::atomic<uint64_t> counter{
     static_cast<uint64_t>(std::chrono::steady_clock::now().time_since_epoch().count()) * 0x9E3779B97F4A7C15ull};
   const uint64_t v = counter.fetch_add(0x9E3779B97F4A7C15ull, std::memory_order_relaxed);
-  return {static_cast<unsigned>(v), static_cast<unsigned>(v >> 32)};
+  return {static_cast<unsigned>(v), static_cast<unsigned>(v >> 32), nullptr};
+}
+
+// First thing a cluster kernel does with its tag: fold in the replay counter, if any.  All
+// workgroups read the same value: the node that advances the word precedes the kernel.
+__device__ __forceinline__ void cluster_resolve_tag(ClusterTag& tag)
+{
+  if (tag.replay_word) {
+    const unsigned long long v = __hip_atomic_load(tag.replay_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    tag.lo ^= static_cast<unsigned>(v);
+    tag.hi ^= static_cast<unsigned>(v >> 32);
+  }
+}
+
+// Whatever the word held before (the workspace is never cleared), successive replays see
+// successive values; xor-ed with the recorded call's own tag they stay distinct from the
+// tags of every other call that used this memory.
+static __global__ void __launch_bounds__(64)
+cluster_advance_replay_word(unsigned long long* word)
+{
+  if (threadIdx.x == 0) *word += 0x9E3779B97F4A7C15ull;
 }
 
 __device__ __forceinline__ unsigned long long cluster_word(float value, unsigned tag)
@@ -105,9 +131,11 @@ __device__ __forceinline__ void cluster_exchange(float a, float b, unsigned long
   cluster_collect(slots, M, tag, error_word, na, nb, ra, rb);
 }
 
-// Layout of the cluster part of a workspace: int error[16], then two 64-bit words per slot.
+// Layout of the cluster part of a workspace: 64 bytes of header (error word at byte 0, replay
+// counter at byte 8), then two 64-bit words per slot.
 struct ClusterWorkspace {
   int* error;
+  unsigned long long* replay_word;
   unsigned long long* slots;
 };
 
@@ -119,7 +147,20 @@ inline size_t cluster_workspace_bytes(int64_t items)
 inline ClusterWorkspace cluster_workspace(void* ws)
 {
   char* base = static_cast<char*>(ws);
-  return {reinterpret_cast<int*>(base), reinterpret_cast<unsigned long long*>(base + 64)};
+  return {reinterpret_cast<int*>(base), reinterpret_cast<unsigned long long*>(base + 8),
+          reinterpret_cast<unsigned long long*>(base + 64)};
+}
+
+// The tag of one cluster call on stream `st`.  On a stream that is being recorded into a graph
+// this also records the node that advances the workspace's replay counter.
+inline ClusterTag cluster_call_tag(hipStream_t st, const ClusterWorkspace& cw)
+{
+  ClusterTag tag = next_cluster_tag();
+  if (stream_is_capturing(st)) {
+    hipLaunchKernelGGL(cluster_advance_replay_word, dim3(1), dim3(64), 0, st, cw.replay_word);
+    tag.replay_word = cw.replay_word;
+  }
+  return tag;
 }
 
 // Cluster shape for an item of E 16-byte vectors: V vectors per thread (<= max_v), M

@@ -25,8 +25,7 @@ inline int launch_status()
 
 // True while `st` records into a HIP graph.  A recorded launch is replayed with the
 // arguments it was recorded with, so anything that must differ from call to call (the
-// rendezvous tag of the cluster kernels) cannot go into a graph: entry points fall
-// back to their multi-kernel paths while this holds.
+// rendezvous tag of the cluster kernels) has to come from device memory there.
 inline bool stream_is_capturing(hipStream_t st)
 {
   hipStreamCaptureStatus status = hipStreamCaptureStatusNone;

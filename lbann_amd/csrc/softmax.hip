@@ -367,6 +367,7 @@ sm_fwd_cluster(SmClusterArgs a)
   const int k = blockIdx.x - static_cast<int>(cl) * a.M;
   const unsigned base = static_cast<unsigned>(k) * (kClusterThreads * V) + threadIdx.x;
   if (cl >= a.rows) return;
+  cluster_resolve_tag(a.tag);
   SmFwdTile<V> t0, t1, t2;
   sm_cl_load<V>(t0.v, a.a + a.map.offset(cl, a.lda), base, a.nvec, -FLT_MAX);
   if (cl + nc < a.rows) sm_cl_load<V>(t1.v, a.a + a.map.offset(cl + nc, a.lda), base, a.nvec, -FLT_MAX);
@@ -457,6 +458,7 @@ sm_bwd_cluster(SmClusterArgs a)
   const int k = blockIdx.x - static_cast<int>(cl) * a.M;
   const unsigned base = static_cast<unsigned>(k) * (kClusterThreads * V) + threadIdx.x;
   if (cl >= a.rows) return;
+  cluster_resolve_tag(a.tag);
   SmBwdTile<V> t0, t1, t2;
   sm_cl_bwd_load<V>(a, cl, base, t0);
   if (cl + nc < a.rows) sm_cl_bwd_load<V>(a, cl + nc, base, t1);
@@ -833,11 +835,11 @@ static int stream_loads(int64_t rows, int64_t n, int tensors)
   return rows * n * 4 * tensors >= kStreamLoadMinBytes ? 1 : 0;
 }
 
-static bool cluster_enabled(int64_t rows, int64_t n, hipStream_t st)
+static bool cluster_enabled(int64_t rows, int64_t n)
 {
   static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
   static const bool forced = std::getenv("LBN_FORCE_CLUSTER") != nullptr;
-  return !disabled && (forced || rows * n * 4 >= kClusterMinBytes) && !stream_is_capturing(st);
+  return !disabled && (forced || rows * n * 4 >= kClusterMinBytes);
 }
 
 #define LBN_ROW_CASES(X)                                                                     \
@@ -895,7 +897,7 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #undef X
     }
   }
-  if (vec && cluster_enabled(rows, n, st) && n / 4 < (int64_t(1) << 30)) {
+  if (vec && cluster_enabled(rows, n) && n / 4 < (int64_t(1) << 30)) {
     // four vectors per thread keep five workgroups per CU resident; eight only for rows that need it
     ClusterPlan cp = plan_cluster(n / 4, 4);
     if (!cp.M) cp = plan_cluster(n / 4, 8);
@@ -909,7 +911,7 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     if (ncl >= 1) {                                                                              \
       ncl = ceil_div(rows, ceil_div(rows, ncl)); /* every cluster walks the same number of rows */ \
       const SmClusterArgs a{x, nullptr, y, ldx, 0, ldy, map, rows, static_cast<unsigned>(n / 4), \
-                            cp.M, cw, next_cluster_tag()};                                       \
+                            cp.M, cw, cluster_call_tag(st, cw)};                                 \
       hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND>), dim3(static_cast<unsigned>(ncl * cp.M)),    \
                          dim3(kClusterThreads), 0, st, a);                                       \
       return launch_status();                                                                    \
@@ -989,7 +991,7 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #undef X
     }
   }
-  if (vec && cluster_enabled(rows, n, st) && n / 4 < (int64_t(1) << 30)) {
+  if (vec && cluster_enabled(rows, n) && n / 4 < (int64_t(1) << 30)) {
     const ClusterPlan cp = plan_cluster(n / 4, 4);
     if (cp.M) {
       if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
@@ -1001,7 +1003,7 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     if (ncl >= 1) {                                                                              \
       ncl = ceil_div(rows, ceil_div(rows, ncl));                                                 \
       const SmClusterArgs a{y, dy, dx, ldy, lddy, lddx, map, rows, static_cast<unsigned>(n / 4), \
-                            cp.M, cw, next_cluster_tag()};                                       \
+                            cp.M, cw, cluster_call_tag(st, cw)};                                 \
       hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND>), dim3(static_cast<unsigned>(ncl * cp.M)),    \
                          dim3(kClusterThreads), 0, st, a);                                       \
       return launch_status();                                                                    \
