@@ -18,7 +18,9 @@
 // entry), sum(x-K) and sum((x-K)^2), which removes the cancellation of
 // E[x^2]-mean^2 when |mean| >> stdev at no extra cost; LBN_STATS_SUMSQ selects
 // K = 0, the reference's formula (batch_normalization.cpp:70-85, :124-128).
+#include <initializer_list>
 #include <type_traits>
+#include <utility>
 
 #include "cluster_sync.hpp"
 #include "device_utils.hpp"
@@ -365,32 +367,26 @@ __device__ __forceinline__ BnIndex<V> bn_make_index(int k, unsigned seg, unsigne
   return ix;
 }
 
+// Tiles stay in registers as the raw vectors that were loaded (fp16 data stays packed: half
+// the registers of its fp32 image, so twice the bytes in flight per thread) and are widened
+// to fp32 vector by vector where they are used.
 template <typename S, int V>
-__device__ __forceinline__ void bn_tile_load(float (&t)[V][Vec16<S>::N], const S* base, int64_t ld,
+__device__ __forceinline__ void bn_tile_load(typename Vec16<S>::raw_t (&t)[V], const S* base, int64_t ld,
                                              const BnIndex<V>& ix)
 {
   constexpr int VE = Vec16<S>::N;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    if (ix.ok[i]) {
-      Vec16<S>::load(base + static_cast<int64_t>(ix.col[i]) * ld + VE * static_cast<int64_t>(ix.pos[i]), t[i]);
-    }
-    else {
-#pragma unroll
-      for (int j = 0; j < VE; ++j) t[i][j] = 0.f;
-    }
+    t[i] = typename Vec16<S>::raw_t{};
+    if (ix.ok[i])
+      t[i] = Vec16<S>::load_raw(base + static_cast<int64_t>(ix.col[i]) * ld + VE * static_cast<int64_t>(ix.pos[i]));
   }
 }
 
 template <typename S, int V>
-__device__ __forceinline__ void bn_tile_store(const float (&t)[V][Vec16<S>::N], S* base, int64_t ld,
-                                              const BnIndex<V>& ix)
+__device__ __forceinline__ S* bn_tile_address(S* base, int64_t ld, const BnIndex<V>& ix, int i)
 {
-  constexpr int VE = Vec16<S>::N;
-#pragma unroll
-  for (int i = 0; i < V; ++i)
-    if (ix.ok[i])
-      Vec16<S>::store(base + static_cast<int64_t>(ix.col[i]) * ld + VE * static_cast<int64_t>(ix.pos[i]), t[i]);
+  return base + static_cast<int64_t>(ix.col[i]) * ld + Vec16<S>::N * static_cast<int64_t>(ix.pos[i]);
 }
 
 template <typename S>
@@ -416,7 +412,7 @@ struct BnFwdArgs {
 // issued itself.
 template <typename S, int V>
 struct BnFwdTile {
-  float v[V][Vec16<S>::N];
+  typename Vec16<S>::raw_t v[V];
   float K, scale, bias;
 };
 
@@ -441,9 +437,11 @@ __device__ __forceinline__ void bn_fwd_reduce(const BnFwdArgs<S>& a, const BnInd
   float s = 0.f, q = 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
+    float v[Vec16<S>::N];
+    Vec16<S>::unpack(t.v[i], v);
 #pragma unroll
     for (int j = 0; j < Vec16<S>::N; ++j) {
-      const float d = ix.ok[i] ? t.v[i][j] - K : 0.f;
+      const float d = ix.ok[i] ? v[j] - K : 0.f;
       s += d;
       q += d * d;
     }
@@ -479,11 +477,16 @@ __device__ __forceinline__ void bn_fwd_finish(const BnFwdArgs<S>& a, const BnInd
   __syncthreads();
   const float mean = bc[0];
   const float inv_stdev = bc[1];
+  S* yc = a.y + static_cast<int64_t>(ch) * a.cs;
 #pragma unroll
-  for (int i = 0; i < V; ++i)
+  for (int i = 0; i < V; ++i) {
+    if (!ix.ok[i]) continue;
+    float v[Vec16<S>::N];
+    Vec16<S>::unpack(t.v[i], v);
 #pragma unroll
-    for (int j = 0; j < Vec16<S>::N; ++j) t.v[i][j] = t.scale * ((t.v[i][j] - mean) * inv_stdev) + t.bias;
-  bn_tile_store<S, V>(t.v, a.y + static_cast<int64_t>(ch) * a.cs, a.ldy, ix);
+    for (int j = 0; j < Vec16<S>::N; ++j) v[j] = t.scale * ((v[j] - mean) * inv_stdev) + t.bias;
+    Vec16<S>::store(bn_tile_address<S, V>(yc, a.ldy, ix, i), v);
+  }
 }
 
 // One step of the rotation: F finishes channel ch, R holds channel ch + nc, L
@@ -547,8 +550,8 @@ struct BnBwdArgs {
 
 template <typename S, int V>
 struct BnBwdTile {
-  float x[V][Vec16<S>::N];
-  float g[V][Vec16<S>::N];
+  typename Vec16<S>::raw_t x[V];
+  typename Vec16<S>::raw_t g[V];
   float mean, var, scale;
 };
 
@@ -563,22 +566,23 @@ __device__ __forceinline__ void bn_bwd_load(BnBwdTile<S, V>& t, const BnBwdArgs<
   t.scale = a.gamma[ch];
 }
 
-// Centres x in place (the finish step needs x - mean) and publishes
-// A = sum(dy), B = sum(dy * (x - mean)).
+// Publishes A = sum(dy), B = sum(dy * (x - mean)); vectors past the end hold zeros in dy.
 template <typename S, int T, int V>
 __device__ __forceinline__ void bn_bwd_reduce(const BnBwdArgs<S>& a, const BnIndex<V>& ix, int ch, int k,
-                                              BnBwdTile<S, V>& t, float* red)
+                                              const BnBwdTile<S, V>& t, float* red)
 {
   const unsigned tid = threadIdx.x;
   const float mean = t.mean;
   float sa = 0.f, sb = 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
+    float x[Vec16<S>::N], g[Vec16<S>::N];
+    Vec16<S>::unpack(t.x[i], x);
+    Vec16<S>::unpack(t.g[i], g);
 #pragma unroll
     for (int j = 0; j < Vec16<S>::N; ++j) {
-      t.x[i][j] = ix.ok[i] ? t.x[i][j] - mean : 0.f;
-      sa += t.g[i][j];
-      sb += t.g[i][j] * t.x[i][j];
+      sa += g[j];
+      sb += g[j] * (x[j] - mean);
     }
   }
   team_sum2<T / kWave>(sa, sb, red, tid / kWave, tid & (kWave - 1));
@@ -614,11 +618,18 @@ __device__ __forceinline__ void bn_bwd_finish(const BnBwdArgs<S>& a, const BnInd
   const float dmean_term = bc[0];
   const float dvar_term = bc[1];
   const float k0 = scale * inv_stdev;
+  const float mean = t.mean;
+  S* dxc = a.dx + static_cast<int64_t>(ch) * a.cs;
 #pragma unroll
-  for (int i = 0; i < V; ++i)
+  for (int i = 0; i < V; ++i) {
+    if (!ix.ok[i]) continue;
+    float x[Vec16<S>::N], g[Vec16<S>::N];
+    Vec16<S>::unpack(t.x[i], x);
+    Vec16<S>::unpack(t.g[i], g);
 #pragma unroll
-    for (int j = 0; j < Vec16<S>::N; ++j) t.g[i][j] = t.g[i][j] * k0 + dmean_term + dvar_term * t.x[i][j];
-  bn_tile_store<S, V>(t.g, a.dx + static_cast<int64_t>(ch) * a.cs, a.lddx, ix);
+    for (int j = 0; j < Vec16<S>::N; ++j) g[j] = g[j] * k0 + dmean_term + dvar_term * (x[j] - mean);
+    Vec16<S>::store(bn_tile_address<S, V>(dxc, a.lddx, ix, i), g);
+  }
 }
 
 template <typename S, int T, int V>
@@ -746,8 +757,8 @@ static bool bn_cluster_usable(int64_t C, int64_t cs, int64_t w, const void* ws)
   return !disabled && E < (int64_t(1) << 31) - 8192 && cs * w > 1 && C <= (1 << 24) && aligned16(ws);
 }
 
-// A thread keeps at most 16 entries of a forward tile and 8 + 8 of a backward tile in
-// fp32 registers, whatever the storage type.
+// A thread keeps at most four raw vectors of a forward tile and two (four when a vector is 8
+// bytes) of each tensor of a backward tile.
 template <typename S>
 static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w, int pivot, int bessel,
                                float eps, float decay, const S* x, int64_t ldx, S* y, int64_t ldy,
@@ -757,7 +768,7 @@ static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   constexpr int VE = Vec16<S>::N;
   if (!bn_cluster_usable<S>(C, cs, w, ws)) return false;
   const int64_t E = cs / VE * w;
-  const BnClusterShape p = bn_cluster_shape(E, 16 / VE, 256);
+  const BnClusterShape p = bn_cluster_shape(E, 4, 256);
   if (!p.T) return false;
   const BnFwdArgs<S> a{x, y, ldx, ldy, cs, static_cast<int>(C), p.M, pivot, bessel, eps, decay, cs * w,
                        cluster_workspace(ws), cluster_call_tag(st, cluster_workspace(ws)), mean, var, scale, bias, rmean, rvar};
@@ -765,7 +776,7 @@ static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
 #define X(TT, VV) \
   if (p.T == TT && p.V == VV) return bn_launch_fwd_cluster<S, TT, VV>(st, a, C, seg, Eu);
   X(256, 1) X(256, 2) X(512, 1) X(512, 2) X(1024, 1) X(1024, 2)
-  if constexpr (VE == 4) { X(256, 3) X(256, 4) X(512, 3) X(512, 4) X(1024, 3) X(1024, 4) }
+  X(256, 3) X(256, 4) X(512, 3) X(512, 4) X(1024, 3) X(1024, 4)
 #undef X
   return false;
 }
@@ -779,15 +790,16 @@ static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   constexpr int VE = Vec16<S>::N;
   if (!bn_cluster_usable<S>(C, cs, w, ws)) return false;
   const int64_t E = cs / VE * w;
-  const BnClusterShape p = bn_cluster_shape(E, 8 / VE, 256);
+  constexpr bool kShortVectors = sizeof(typename Vec16<S>::raw_t) == 8;
+  const BnClusterShape p = bn_cluster_shape(E, kShortVectors ? 4 : 2, 256);
   if (!p.T) return false;
   const BnBwdArgs<S> a{x, dy, dx, ldx, lddy, lddx, cs, static_cast<int>(C), p.M, bessel, eps, cs * w,
                        cluster_workspace(ws), cluster_call_tag(st, cluster_workspace(ws)), mean, var, scale, dscale, dbias, dmean, dvar};
   const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(E);
 #define X(TT, VV) \
   if (p.T == TT && p.V == VV) return bn_launch_bwd_cluster<S, TT, VV>(st, a, C, seg, Eu);
-  X(256, 1) X(512, 1) X(1024, 1)
-  if constexpr (VE == 4) { X(256, 2) X(512, 2) X(1024, 2) }
+  X(256, 1) X(512, 1) X(1024, 1) X(256, 2) X(512, 2) X(1024, 2)
+  if constexpr (kShortVectors) { X(256, 3) X(512, 3) X(1024, 3) X(256, 4) X(512, 4) X(1024, 4) }
 #undef X
   return false;
 }
@@ -806,7 +818,20 @@ template <typename S>
 static bool bn_vec_ok(int64_t cs, int64_t w, const void* a, int64_t lda)
 {
   constexpr int VE = Vec16<S>::N;
-  return cs % VE == 0 && aligned16(a) && (w <= 1 || lda % VE == 0);
+  constexpr uintptr_t bytes = VE * sizeof(S);  // 16, or 8 for fp16 in fours
+  return cs % VE == 0 && reinterpret_cast<uintptr_t>(a) % bytes == 0 && (w <= 1 || lda % VE == 0);
+}
+
+// fp16 channels that are whole fours but not whole eights (196 = 14 x 14), or matrices aligned
+// to 8 but not 16 bytes: the same kernels with 8-byte accesses instead of the scalar walk.
+static bool bn_f16_in_fours(int64_t cs, int64_t w, std::initializer_list<std::pair<const void*, int64_t>> mats)
+{
+  bool eights = true, fours = true;
+  for (const auto& m : mats) {
+    eights = eights && bn_vec_ok<__half>(cs, w, m.first, m.second);
+    fours = fours && bn_vec_ok<f16x4>(cs, w, m.first, m.second);
+  }
+  return fours && !eights;
 }
 
 // ---- channels that are not whole 16-byte vectors, on a matrix whose row quads are aligned
@@ -1113,6 +1138,10 @@ int lbn_batch_norm_fwd_f16(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
                            const float* bias, float* running_mean, float* running_var,
                            void* workspace, size_t workspace_bytes, int flags)
 {
+  if (C > 0 && cs > 0 && w > 0 && bn_f16_in_fours(cs, w, {{x, ldx}, {y, ldy}}))
+    return bn_fwd_host<f16x4>(as_stream(stream), C, cs, w, bessel, epsilon, decay, training,
+                              static_cast<const f16x4*>(x), ldx, static_cast<f16x4*>(y), ldy, mean, var,
+                              scale, bias, running_mean, running_var, workspace, workspace_bytes, flags);
   return bn_fwd_host<__half>(as_stream(stream), C, cs, w, bessel, epsilon, decay, training,
                              static_cast<const __half*>(x), ldx, static_cast<__half*>(y), ldy, mean, var,
                              scale, bias, running_mean, running_var, workspace, workspace_bytes, flags);
@@ -1189,6 +1218,11 @@ int lbn_batch_norm_bwd_f16(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
                            float* dscale, float* dbias, float* dmean, float* dvar, void* workspace,
                            size_t workspace_bytes)
 {
+  if (C > 0 && cs > 0 && w > 0 && bn_f16_in_fours(cs, w, {{x, ldx}, {dy, lddy}, {dx, lddx}}))
+    return bn_bwd_host<f16x4>(as_stream(stream), C, cs, w, bessel, epsilon, training,
+                              static_cast<const f16x4*>(x), ldx, static_cast<const f16x4*>(dy), lddy,
+                              static_cast<f16x4*>(dx), lddx, mean, var, running_mean, running_var, scale,
+                              dscale, dbias, dmean, dvar, workspace, workspace_bytes);
   return bn_bwd_host<__half>(as_stream(stream), C, cs, w, bessel, epsilon, training,
                              static_cast<const __half*>(x), ldx, static_cast<const __half*>(dy), lddy,
                              static_cast<__half*>(dx), lddx, mean, var, running_mean, running_var, scale,

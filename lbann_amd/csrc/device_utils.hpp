@@ -161,6 +161,45 @@ struct Vec16<f16x2> {
   }
 };
 
+// fp16 storage accessed four values (8 bytes) at a time: for channels and rows whose length
+// is a multiple of 4 but not of 8 (14 x 14 feature maps: 196 entries).  Sized like one half,
+// so pointer offsets count halves.
+struct f16x4 {
+  unsigned short bits;
+};
+
+template <>
+struct Vec16<f16x4> {
+  static constexpr int N = 4;
+  using raw_t = uint2;
+  static __device__ __forceinline__ raw_t load_raw(const f16x4* p) { return *reinterpret_cast<const uint2*>(p); }
+  static __device__ __forceinline__ void unpack(const raw_t& r, float (&v)[4])
+  {
+    __half2 lo, hi;
+    __builtin_memcpy(&lo, &r.x, 4);
+    __builtin_memcpy(&hi, &r.y, 4);
+    const float2 a = __half22float2(lo), b = __half22float2(hi);
+    v[0] = a.x; v[1] = a.y; v[2] = b.x; v[3] = b.y;
+  }
+  static __device__ __forceinline__ void load(const f16x4* p, float (&v)[4]) { unpack(load_raw(p), v); }
+  static __device__ __forceinline__ void store(f16x4* p, const float (&v)[4])
+  {
+    const __half2 lo = __floats2half2_rn(v[0], v[1]), hi = __floats2half2_rn(v[2], v[3]);
+    uint2 r;
+    __builtin_memcpy(&r.x, &lo, 4);
+    __builtin_memcpy(&r.y, &hi, 4);
+    *reinterpret_cast<uint2*>(p) = r;
+  }
+  static __device__ __forceinline__ float load1(const f16x4* p)
+  {
+    return __half2float(*reinterpret_cast<const __half*>(p));
+  }
+  static __device__ __forceinline__ void store1(f16x4* p, float v)
+  {
+    *reinterpret_cast<__half*>(p) = __float2half_rn(v);
+  }
+};
+
 // VE consecutive fp32 weights (scale, bias, their partial gradients) at p: 16-byte accesses
 // when a thread owns at least four of them, single floats otherwise.
 template <int VE>

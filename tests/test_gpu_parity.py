@@ -369,7 +369,10 @@ def test_batch_norm(L, dims, w, bessel, pad):
 @pytest.mark.parametrize("dims,w,bessel,pad,training", [
     ((8, 16, 16), 12, True, 0, True), ((16, 28, 28), 8, False, 0, True), ((7, 5, 3), 14, True, 0, True),
     ((5, 24), 10, True, 8, True), ((256, 8, 8), 32, True, 0, True), ((3, 56, 56), 16, True, 0, False),
-    ((2, 100000), 3, True, 0, True), ((64, 56, 56), 16, True, 0, True)])
+    ((2, 100000), 3, True, 0, True), ((64, 56, 56), 16, True, 0, True),
+    # channels of whole fours but not eights, or a leading dimension padded by four: 8-byte accesses
+    ((1024, 14, 14), 32, True, 0, True), ((256, 14, 14), 600, False, 0, True), ((6, 10, 10), 9, True, 0, False),
+    ((16, 28, 28), 8, True, 4, True), ((40, 12), 64, True, 0, True), ((3, 4), 5, True, 4, True)])
 def test_batch_norm_f16(L, dims, w, bessel, pad, training):
     """fp16 storage, fp32 arithmetic: the oracle sees the fp16-rounded inputs."""
     rng = np.random.default_rng(int(np.prod(dims)) * 5 + w)
