@@ -26,6 +26,12 @@
  * the tag takes in.  The workspace passed while recording is therefore part of the
  * graph's state: keep it allocated, and do not run two replays that share it at the
  * same time.
+ *
+ * Those kernels size their grid to the workgroups the idle device holds at once.  Next
+ * to other streams' kernels they still complete (members of a cluster are consecutive
+ * blocks, dispatched in order), only later; every wait is bounded and a wait that ran
+ * out is reported by lbn_workspace_timed_out().  Setting LBN_NO_CLUSTER=1 in the
+ * environment selects the multi-kernel paths instead.
  */
 #ifndef LBNORM_H_INCLUDED
 #define LBNORM_H_INCLUDED
