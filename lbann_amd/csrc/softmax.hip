@@ -60,9 +60,10 @@ struct RowIO<1> {
   static __device__ __forceinline__ void store(float* p, const float (&v)[1]) { *p = v[0]; }
 };
 
-// 1024-thread blocks are held to 64 registers so that two of them share a compute unit.
+// 1024-thread blocks are held to 64 registers so that two of them share a compute unit
+// (not those with 32 accesses per thread, which would spill).
 template <int TPR, int V, int KIND, bool STREAM, int W = 4>
-__global__ void __launch_bounds__(RowBlock<TPR>::kThreads, (TPR == 1024 ? 8 : 1))
+__global__ void __launch_bounds__(RowBlock<TPR>::kThreads, (TPR == 1024 && V <= 16 ? 8 : 1))
 sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
             unsigned nvec)
 {
@@ -249,46 +250,46 @@ struct SmClusterArgs {
   __device__ __forceinline__ unsigned long long* slots(int64_t row) const { return cw.slots + row * M * 2; }
 };
 
-template <int V>
+template <int V, int W = 4>
 struct SmFwdTile {
-  float v[V][4];
+  float v[V][W];
   float m;  // the thread's own maximum: v holds exp(x - m) (or x - m for log-softmax)
 };
 
-template <int V>
-__device__ __forceinline__ void sm_cl_load(float (&t)[V][4], const float* rowp, unsigned base,
+template <int V, int W>
+__device__ __forceinline__ void sm_cl_load(float (&t)[V][W], const float* rowp, unsigned base,
                                            unsigned nvec, float fill)
 {
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = base + i * kClusterThreads;
     if (idx < nvec) {
-      Vec16<float>::load(rowp + 4 * static_cast<int64_t>(idx), t[i]);
+      RowIO<W>::template load<false>(rowp + W * static_cast<int64_t>(idx), t[i]);
     }
     else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) t[i][j] = fill;
+      for (int j = 0; j < W; ++j) t[i][j] = fill;
     }
   }
 }
 
 // (1) of a step: thread-local online softmax, one merge of the (max, sum) pairs of the
 // workgroup, published for the cluster.
-template <int V, int KIND>
+template <int V, int KIND, int W = 4>
 __device__ __forceinline__ void sm_cl_fwd_reduce(const SmClusterArgs& a, int64_t row, int k, unsigned base,
-                                                 SmFwdTile<V>& t, float (*red)[2])
+                                                 SmFwdTile<V, W>& t, float (*red)[2])
 {
   float m = -FLT_MAX;
 #pragma unroll
   for (int i = 0; i < V; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) m = fmaxf(m, t.v[i][j]);
+    for (int j = 0; j < W; ++j) m = fmaxf(m, t.v[i][j]);
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const bool ok = base + i * kClusterThreads < a.nvec;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < W; ++j) {
       const float d = t.v[i][j] - m;
       const float e = ok ? (KIND == kChannelwise ? exp_keep_denormals(d) : exp_fast(d)) : 0.f;
       s += e;
@@ -301,9 +302,9 @@ __device__ __forceinline__ void sm_cl_fwd_reduce(const SmClusterArgs& a, int64_t
 }
 
 // (3) of a step.
-template <int V, int KIND>
+template <int V, int KIND, int W = 4>
 __device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t row, unsigned base,
-                                                 SmFwdTile<V>& t, float* bc)
+                                                 SmFwdTile<V, W>& t, float* bc)
 {
   if (threadIdx.x < kWave) {
     float pm, ps;
@@ -327,7 +328,7 @@ __device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t
     const unsigned idx = base + i * kClusterThreads;
     if (idx < a.nvec) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < W; ++j) {
         if (KIND == kSoftmax) {
           const float r = f * t.v[i][j];
           t.v[i][j] = __builtin_isnormal(r) ? r : 0.f;
@@ -339,24 +340,24 @@ __device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t
           t.v[i][j] *= f;
         }
       }
-      Vec16<float>::store(yr + 4 * static_cast<int64_t>(idx), t.v[i]);
+      RowIO<W>::store(yr + W * static_cast<int64_t>(idx), t.v[i]);
     }
   }
 }
 
-template <int V, int KIND>
+template <int V, int KIND, int W = 4>
 __device__ __forceinline__ void sm_cl_fwd_step(const SmClusterArgs& a, int64_t row, int64_t nc, int k,
-                                               unsigned base, SmFwdTile<V>& F, SmFwdTile<V>& R,
-                                               SmFwdTile<V>& L, float (*red)[2], float* bc)
+                                               unsigned base, SmFwdTile<V, W>& F, SmFwdTile<V, W>& R,
+                                               SmFwdTile<V, W>& L, float (*red)[2], float* bc)
 {
-  if (row + nc < a.rows) sm_cl_fwd_reduce<V, KIND>(a, row + nc, k, base, R, red);
+  if (row + nc < a.rows) sm_cl_fwd_reduce<V, KIND, W>(a, row + nc, k, base, R, red);
   if (row + 2 * nc < a.rows)
-    sm_cl_load<V>(L.v, a.a + a.map.offset(row + 2 * nc, a.lda), base, a.nvec, -FLT_MAX);
+    sm_cl_load<V, W>(L.v, a.a + a.map.offset(row + 2 * nc, a.lda), base, a.nvec, -FLT_MAX);
   asm volatile("" ::: "memory");  // keep the loads above the wait below
-  sm_cl_fwd_finish<V, KIND>(a, row, base, F, bc);
+  sm_cl_fwd_finish<V, KIND, W>(a, row, base, F, bc);
 }
 
-template <int V, int KIND>
+template <int V, int KIND, int W = 4>
 __global__ void __launch_bounds__(kClusterThreads)
 sm_fwd_cluster(SmClusterArgs a)
 {
@@ -368,42 +369,42 @@ sm_fwd_cluster(SmClusterArgs a)
   const unsigned base = static_cast<unsigned>(k) * (kClusterThreads * V) + threadIdx.x;
   if (cl >= a.rows) return;
   cluster_resolve_tag(a.tag);
-  SmFwdTile<V> t0, t1, t2;
-  sm_cl_load<V>(t0.v, a.a + a.map.offset(cl, a.lda), base, a.nvec, -FLT_MAX);
-  if (cl + nc < a.rows) sm_cl_load<V>(t1.v, a.a + a.map.offset(cl + nc, a.lda), base, a.nvec, -FLT_MAX);
-  sm_cl_fwd_reduce<V, KIND>(a, cl, k, base, t0, red);
+  SmFwdTile<V, W> t0, t1, t2;
+  sm_cl_load<V, W>(t0.v, a.a + a.map.offset(cl, a.lda), base, a.nvec, -FLT_MAX);
+  if (cl + nc < a.rows) sm_cl_load<V, W>(t1.v, a.a + a.map.offset(cl + nc, a.lda), base, a.nvec, -FLT_MAX);
+  sm_cl_fwd_reduce<V, KIND, W>(a, cl, k, base, t0, red);
   __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
   // Each position of the rotation has its own broadcast slot: a step without a reduction has
   // no barrier between the reads of one finish and the write of the next.
   for (int64_t row = cl; row < a.rows; row += 3 * nc) {
-    sm_cl_fwd_step<V, KIND>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
-    if (row + nc < a.rows) sm_cl_fwd_step<V, KIND>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
-    if (row + 2 * nc < a.rows) sm_cl_fwd_step<V, KIND>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
+    sm_cl_fwd_step<V, KIND, W>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
+    if (row + nc < a.rows) sm_cl_fwd_step<V, KIND, W>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
+    if (row + 2 * nc < a.rows) sm_cl_fwd_step<V, KIND, W>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
   }
 }
 
-template <int V>
+template <int V, int W = 4>
 struct SmBwdTile {
-  float a[V][4];
-  float g[V][4];
+  float a[V][W];
+  float g[V][W];
 };
 
-template <int V, int KIND>
+template <int V, int KIND, int W = 4>
 __device__ __forceinline__ void sm_cl_bwd_reduce(const SmClusterArgs& a, int64_t row, int k,
-                                                 const SmBwdTile<V>& t, float* red)
+                                                 const SmBwdTile<V, W>& t, float* red)
 {
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) s += (KIND == kLogSoftmax) ? t.g[i][j] : t.a[i][j] * t.g[i][j];
+    for (int j = 0; j < W; ++j) s += (KIND == kLogSoftmax) ? t.g[i][j] : t.a[i][j] * t.g[i][j];
   s = team_sum<kClusterThreads / kWave>(s, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
   if (threadIdx.x == 0) cluster_publish(s, 0.f, a.slots(row), k, a.tag);
 }
 
-template <int V, int KIND>
+template <int V, int KIND, int W = 4>
 __device__ __forceinline__ void sm_cl_bwd_finish(const SmClusterArgs& a, int64_t row, unsigned base,
-                                                 SmBwdTile<V>& t, float* bc)
+                                                 SmBwdTile<V, W>& t, float* bc)
 {
   if (threadIdx.x < kWave) {
     float pt, unused;
@@ -419,35 +420,35 @@ __device__ __forceinline__ void sm_cl_bwd_finish(const SmClusterArgs& a, int64_t
     const unsigned idx = base + i * kClusterThreads;
     if (idx < a.nvec) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < W; ++j) {
         if (KIND == kLogSoftmax) t.g[i][j] = t.g[i][j] - exp_fast(t.a[i][j]) * tot;
         else t.g[i][j] = t.a[i][j] * (t.g[i][j] - tot);
       }
-      Vec16<float>::store(dr + 4 * static_cast<int64_t>(idx), t.g[i]);
+      RowIO<W>::store(dr + W * static_cast<int64_t>(idx), t.g[i]);
     }
   }
 }
 
-template <int V>
+template <int V, int W>
 __device__ __forceinline__ void sm_cl_bwd_load(const SmClusterArgs& a, int64_t row, unsigned base,
-                                               SmBwdTile<V>& t)
+                                               SmBwdTile<V, W>& t)
 {
-  sm_cl_load<V>(t.a, a.a + a.map.offset(row, a.lda), base, a.nvec, 0.f);
-  sm_cl_load<V>(t.g, a.g + a.map.offset(row, a.ldg), base, a.nvec, 0.f);
+  sm_cl_load<V, W>(t.a, a.a + a.map.offset(row, a.lda), base, a.nvec, 0.f);
+  sm_cl_load<V, W>(t.g, a.g + a.map.offset(row, a.ldg), base, a.nvec, 0.f);
 }
 
-template <int V, int KIND>
+template <int V, int KIND, int W = 4>
 __device__ __forceinline__ void sm_cl_bwd_step(const SmClusterArgs& a, int64_t row, int64_t nc, int k,
-                                               unsigned base, SmBwdTile<V>& F, SmBwdTile<V>& R,
-                                               SmBwdTile<V>& L, float* red, float* bc)
+                                               unsigned base, SmBwdTile<V, W>& F, SmBwdTile<V, W>& R,
+                                               SmBwdTile<V, W>& L, float* red, float* bc)
 {
-  if (row + nc < a.rows) sm_cl_bwd_reduce<V, KIND>(a, row + nc, k, R, red);
-  if (row + 2 * nc < a.rows) sm_cl_bwd_load<V>(a, row + 2 * nc, base, L);
+  if (row + nc < a.rows) sm_cl_bwd_reduce<V, KIND, W>(a, row + nc, k, R, red);
+  if (row + 2 * nc < a.rows) sm_cl_bwd_load<V, W>(a, row + 2 * nc, base, L);
   asm volatile("" ::: "memory");
-  sm_cl_bwd_finish<V, KIND>(a, row, base, F, bc);
+  sm_cl_bwd_finish<V, KIND, W>(a, row, base, F, bc);
 }
 
-template <int V, int KIND>
+template <int V, int KIND, int W = 4>
 __global__ void __launch_bounds__(kClusterThreads)
 sm_bwd_cluster(SmClusterArgs a)
 {
@@ -459,17 +460,17 @@ sm_bwd_cluster(SmClusterArgs a)
   const unsigned base = static_cast<unsigned>(k) * (kClusterThreads * V) + threadIdx.x;
   if (cl >= a.rows) return;
   cluster_resolve_tag(a.tag);
-  SmBwdTile<V> t0, t1, t2;
-  sm_cl_bwd_load<V>(a, cl, base, t0);
-  if (cl + nc < a.rows) sm_cl_bwd_load<V>(a, cl + nc, base, t1);
-  sm_cl_bwd_reduce<V, KIND>(a, cl, k, t0, red);
+  SmBwdTile<V, W> t0, t1, t2;
+  sm_cl_bwd_load<V, W>(a, cl, base, t0);
+  if (cl + nc < a.rows) sm_cl_bwd_load<V, W>(a, cl + nc, base, t1);
+  sm_cl_bwd_reduce<V, KIND, W>(a, cl, k, t0, red);
   __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
   // Each position of the rotation has its own broadcast slot: a step without a reduction has
   // no barrier between the reads of one finish and the write of the next.
   for (int64_t row = cl; row < a.rows; row += 3 * nc) {
-    sm_cl_bwd_step<V, KIND>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
-    if (row + nc < a.rows) sm_cl_bwd_step<V, KIND>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
-    if (row + 2 * nc < a.rows) sm_cl_bwd_step<V, KIND>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
+    sm_cl_bwd_step<V, KIND, W>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
+    if (row + nc < a.rows) sm_cl_bwd_step<V, KIND, W>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
+    if (row + 2 * nc < a.rows) sm_cl_bwd_step<V, KIND, W>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
   }
 }
 
@@ -797,8 +798,8 @@ static ChunkPlan plan_chunks(int64_t n, int64_t rows)
   return {static_cast<int>(S), chunk};
 }
 
-constexpr int64_t kMaxRowVectors = 8192;  // longest row the one-workgroup register kernels hold
 constexpr int64_t kMaxScalarRow = 8192;   // the same in floats for rows accessed one float at a time
+constexpr int64_t kMaxScalarLongRow = 32768;  // with 16 or 32 floats per thread: still one kernel, one read
 
 // Rows of at most 64 access units, when there are many of them, go to teams of 16 lanes
 // (four rows per wave) instead of leaving most of a wave idle: attention rows of 64
@@ -813,7 +814,7 @@ static size_t sm_workspace_bytes(int64_t n, int64_t rows)
 {
   if (n <= 0 || rows <= 0) return 0;
   const size_t chunked = static_cast<size_t>(rows) * plan_chunks(n, rows).S * sizeof(float2);
-  const size_t cluster = (n / 4 > kMaxRowVectors) ? cluster_workspace_bytes(rows) : 0;
+  const size_t cluster = (n > kMaxScalarLongRow) ? cluster_workspace_bytes(rows) : 0;
   return chunked > cluster ? chunked : cluster;
 }
 
@@ -840,6 +841,59 @@ static bool cluster_enabled(int64_t rows, int64_t n)
   static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
   static const bool forced = std::getenv("LBN_FORCE_CLUSTER") != nullptr;
   return !disabled && (forced || rows * n * 4 >= kClusterMinBytes);
+}
+
+// Launch of the cluster kernels for rows of `units` accesses of W floats each.  Returns -1 when
+// the plan or the device's capacity does not allow it (the caller goes on to the split
+// kernels), otherwise the call's status.
+template <int KIND, int W>
+static int sm_fwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, int64_t rows, const float* x,
+                                 int64_t ldx, float* y, int64_t ldy, RowMap map, void* ws, size_t ws_bytes)
+{
+  if (!cp.M) return -1;
+  if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
+  const ClusterWorkspace cw = cluster_workspace(ws);
+#define X(VV)                                                                                    \
+  if (cp.V == VV) {                                                                              \
+    const int cap = cluster_capacity(sm_fwd_cluster<VV, KIND, W>, kClusterThreads);              \
+    int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
+    if (ncl < 1) return -1;                                                                      \
+    ncl = ceil_div(rows, ceil_div(rows, ncl)); /* every cluster walks the same number of rows */ \
+    const SmClusterArgs a{x, nullptr, y, ldx, 0, ldy, map, rows, static_cast<unsigned>(units),   \
+                          cp.M, cw, cluster_call_tag(st, cw)};                                   \
+    hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND, W>), dim3(static_cast<unsigned>(ncl * cp.M)),   \
+                       dim3(kClusterThreads), 0, st, a);                                         \
+    return launch_status();                                                                      \
+  }
+  X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8)
+#undef X
+  return -1;
+}
+
+template <int KIND, int W>
+static int sm_bwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, int64_t rows, const float* y,
+                                 int64_t ldy, const float* dy, int64_t lddy, float* dx, int64_t lddx, RowMap map,
+                                 void* ws, size_t ws_bytes)
+{
+  if (!cp.M) return -1;
+  if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
+  const ClusterWorkspace cw = cluster_workspace(ws);
+#define X(VV)                                                                                    \
+  if (cp.V == VV) {                                                                              \
+    const int cap = cluster_capacity(sm_bwd_cluster<VV, KIND, W>, kClusterThreads);              \
+    int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
+    if (ncl < 1) return -1;                                                                      \
+    ncl = ceil_div(rows, ceil_div(rows, ncl));                                                   \
+    const SmClusterArgs a{y, dy, dx, ldy, lddy, lddx, map, rows, static_cast<unsigned>(units),   \
+                          cp.M, cw, cluster_call_tag(st, cw)};                                   \
+    hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND, W>), dim3(static_cast<unsigned>(ncl * cp.M)),   \
+                       dim3(kClusterThreads), 0, st, a);                                         \
+    return launch_status();                                                                      \
+  }
+  X(1) X(2) X(3) X(4)
+  if constexpr (W == 1) { X(5) X(6) X(7) X(8) }
+#undef X
+  return -1;
 }
 
 #define LBN_ROW_CASES(X)                                                                     \
@@ -897,29 +951,31 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #undef X
     }
   }
-  if (vec && cluster_enabled(rows, n) && n / 4 < (int64_t(1) << 30)) {
-    // four vectors per thread keep five workgroups per CU resident; eight only for rows that need it
-    ClusterPlan cp = plan_cluster(n / 4, 4);
-    if (!cp.M) cp = plan_cluster(n / 4, 8);
-    if (cp.M) {
-      if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
-      const ClusterWorkspace cw = cluster_workspace(ws);
-#define X(VV)                                                                                    \
-  if (cp.V == VV) {                                                                              \
-    const int cap = cluster_capacity(sm_fwd_cluster<VV, KIND>, kClusterThreads);                 \
-    int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
-    if (ncl >= 1) {                                                                              \
-      ncl = ceil_div(rows, ceil_div(rows, ncl)); /* every cluster walks the same number of rows */ \
-      const SmClusterArgs a{x, nullptr, y, ldx, 0, ldy, map, rows, static_cast<unsigned>(n / 4), \
-                            cp.M, cw, cluster_call_tag(st, cw)};                                 \
-      hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND>), dim3(static_cast<unsigned>(ncl * cp.M)),    \
-                         dim3(kClusterThreads), 0, st, a);                                       \
-      return launch_status();                                                                    \
-    }                                                                                            \
+  else if (n <= kMaxScalarLongRow) {
+    // the same up to 32768 entries (16385 x 4096: one kernel instead of partials + apply)
+    const unsigned nvec = static_cast<unsigned>(n);
+    const unsigned grid = static_cast<unsigned>(rows);
+    if (n <= 16 * 1024)
+      hipLaunchKernelGGL((sm_fwd_rows<1024, 16, KIND, false, 1>), dim3(grid), dim3(1024), 0, st, x, y, ldx, ldy,
+                         map, rows, nvec);
+    else
+      hipLaunchKernelGGL((sm_fwd_rows<1024, 32, KIND, false, 1>), dim3(grid), dim3(1024), 0, st, x, y, ldx, ldy,
+                         map, rows, nvec);
+    return launch_status();
   }
-      X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8)
-#undef X
+  if (cluster_enabled(rows, n)) {
+    int r = -1;
+    if (vec && n / 4 < (int64_t(1) << 30)) {
+      // four vectors per thread keep five workgroups per CU resident; eight only for rows that need it
+      ClusterPlan cp = plan_cluster(n / 4, 4);
+      if (!cp.M) cp = plan_cluster(n / 4, 8);
+      r = sm_fwd_cluster_launch<KIND, 4>(st, cp, n / 4, rows, x, ldx, y, ldy, map, ws, ws_bytes);
     }
+    else if (!vec) {
+      // rows off the 16-byte grid (a vocabulary of 50257 entries): the same kernel, one float per access
+      r = sm_fwd_cluster_launch<KIND, 1>(st, plan_cluster(n, 8), n, rows, x, ldx, y, ldy, map, ws, ws_bytes);
+    }
+    if (r >= 0) return r;
   }
   const ChunkPlan p = plan_chunks(n, rows);
   if (rows * p.S > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
@@ -991,27 +1047,26 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #undef X
     }
   }
-  if (vec && cluster_enabled(rows, n) && n / 4 < (int64_t(1) << 30)) {
-    const ClusterPlan cp = plan_cluster(n / 4, 4);
-    if (cp.M) {
-      if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
-      const ClusterWorkspace cw = cluster_workspace(ws);
-#define X(VV)                                                                                    \
-  if (cp.V == VV) {                                                                              \
-    const int cap = cluster_capacity(sm_bwd_cluster<VV, KIND>, kClusterThreads);                 \
-    int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
-    if (ncl >= 1) {                                                                              \
-      ncl = ceil_div(rows, ceil_div(rows, ncl));                                                 \
-      const SmClusterArgs a{y, dy, dx, ldy, lddy, lddx, map, rows, static_cast<unsigned>(n / 4), \
-                            cp.M, cw, cluster_call_tag(st, cw)};                                 \
-      hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND>), dim3(static_cast<unsigned>(ncl * cp.M)),    \
-                         dim3(kClusterThreads), 0, st, a);                                       \
-      return launch_status();                                                                    \
-    }                                                                                            \
+  else if (n <= kMaxScalarLongRow) {
+    const unsigned nvec = static_cast<unsigned>(n);
+    const unsigned grid = static_cast<unsigned>(rows);
+    if (n <= 16 * 1024)
+      hipLaunchKernelGGL((sm_bwd_rows<1024, 16, KIND, false, 1>), dim3(grid), dim3(1024), 0, st, y, dy, dx, ldy,
+                         lddy, lddx, map, rows, nvec);
+    else
+      hipLaunchKernelGGL((sm_bwd_rows<1024, 32, KIND, false, 1>), dim3(grid), dim3(1024), 0, st, y, dy, dx, ldy,
+                         lddy, lddx, map, rows, nvec);
+    return launch_status();
   }
-      X(1) X(2) X(3) X(4)
-#undef X
-    }
+  if (cluster_enabled(rows, n)) {
+    int r = -1;
+    if (vec && n / 4 < (int64_t(1) << 30))
+      r = sm_bwd_cluster_launch<KIND, 4>(st, plan_cluster(n / 4, 4), n / 4, rows, y, ldy, dy, lddy, dx, lddx, map, ws,
+                                         ws_bytes);
+    else if (!vec)
+      r = sm_bwd_cluster_launch<KIND, 1>(st, plan_cluster(n, 8), n, rows, y, ldy, dy, lddy, dx, lddx, map, ws,
+                                         ws_bytes);
+    if (r >= 0) return r;
   }
   const ChunkPlan p = plan_chunks(n, rows);
   if (rows * p.S > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;

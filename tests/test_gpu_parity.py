@@ -45,9 +45,12 @@ SM_SHAPES = [
     (32772, 2, 0), (70000, 3, 0), (262144, 2, 0),        # longer than the register path: split kernels
     (262148, 48, 0), (100000, 130, 0),                   # long rows, large footprint: register-resident clusters
     (1, 6, 0),
-    # rows that are only 4-byte aligned: one float per access in registers up to 8192 entries,
-    # 16-byte accesses with scalar edges in the split kernels beyond
+    # rows that are only 4-byte aligned: one float per access in registers up to 32768 entries;
+    # beyond, the cluster kernels with one float per access when the tensor is large, else
+    # 16-byte accesses with scalar edges in the split kernels
     (197, 70, 0), (8191, 9, 0), (8193, 3, 0), (30522, 5, 0), (50257, 6, 0), (10, 300, 0), (4099, 7, 1),
+    (16383, 5, 0), (16385, 4, 0), (32767, 3, 0), (32769, 3, 0), (50257, 270, 0), (131071, 101, 0), (131075, 101, 0),
+    (40001, 700, 1),       # more rows than resident clusters
     # many short rows: teams of 16 lanes, four rows per wave (vector and single-float access)
     (16, 5000, 0), (64, 4100, 0), (128, 4096, 0), (200, 4500, 0), (256, 4097, 0), (10, 5000, 0), (49, 6000, 0),
     (63, 4096, 1), (12, 4095, 0),
