@@ -31,6 +31,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", default="all", help="all | headline | comma list of cfg names")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay leg")
     ap.add_argument("--no-cold", action="store_true", help="skip the cold-cache leg of the small working sets")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also time a plain elementwise copy of 256 MiB (torch kernel): the practical "
@@ -277,6 +278,28 @@ def main():
         bwd_b2b = a.elapsed_time(b) / steps
         return wall, fwd, bwd, bwd_b2b
 
+    def measure_graph(layer, steps, warmup):
+        """Wall seconds for `steps` steps replayed from ONE HIP graph that holds `steps` recorded
+        steps (forward + backward each): what a caller that records its training step pays, with
+        the host's launch cost out of the picture."""
+        lib = L.capi.lib()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            # the calls bind the recording stream, which is the current one in here
+            fname, fargs = layer.fp_call()
+            bname, bargs = layer.bp_call()
+            ffn, bfn = getattr(lib, fname), getattr(lib, bname)
+            for _ in range(steps):
+                if ffn(*fargs) or bfn(*bargs):
+                    raise RuntimeError("kernel launch failed while recording")
+        for _ in range(max(1, warmup // 5)):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
     def measure_cold(builder, set_bytes, steps, warmup):
         """Whole-step wall clock with the tensors rotated among enough independent copies
         (>= 1 GiB in total) that no step finds its inputs in L2 or the Infinity Cache."""
@@ -330,6 +353,10 @@ def main():
             "fwd_gbs": fwd_b / (f_ms * 1e-3) / 1e9, "bwd_gbs": bwd_b / (b_ms * 1e-3) / 1e9,
             "bwd_back_to_back_ms": bwd_b2b,
         }
+        if not args.no_graph:
+            gms = measure_graph(layer, args.steps, args.warmup) / args.steps * 1e3
+            r["graph_replay"] = {"ms_per_step": gms, "gbs": (fwd_b + bwd_b) / (gms * 1e-3) / 1e9,
+                                 "frac_of_hbm_peak": (fwd_b + bwd_b) / (gms * 1e-3) / 1e9 / HBM_PEAK_GBS}
         if not args.no_cold and 4 * elems * esize <= (256 << 20):
             # small working set: a second, cold figure next to the cache-resident one
             cwall, copies = measure_cold(builder, 4 * elems * esize, args.steps, args.warmup)
@@ -347,6 +374,7 @@ def main():
         results[name] = r
         print(f"# {name}: {step_ms*1e3:8.1f} us/step  {r['gbs']:7.0f} GB/s ({100*r['frac_of_hbm_peak']:.1f}% of 8 TB/s)  "
               f"fwd {f_ms*1e3:7.1f} us ({r['fwd_gbs']:.0f} GB/s)  bwd {b_ms*1e3:7.1f} us ({r['bwd_gbs']:.0f} GB/s)"
+              + (f"  graph {r['graph_replay']['ms_per_step']*1e3:.1f} us/step" if "graph_replay" in r else "")
               + (f"  cold {r['cold']['ms_per_step']*1e3:.1f} us/step" if "cold" in r else "")
               + (f"  cpu {r['cpu']['gbs']:.1f} GB/s" if "cpu" in r else ""), file=sys.stderr, flush=True)
         del layer
