@@ -109,8 +109,11 @@ def main():
             return t1 - t0, t2 - t1
         return layer, data["x"].size, 2 if half else 4, data["x"].shape[1], cpu
 
-    def build_bn(data):
-        x, dy = upload(data["x"]), upload(data["dy"])
+    def build_bn(data, half=False):
+        if half:  # fp16 storage: both sides see the rounded values
+            data = dict(data, x=np.asfortranarray(data["x"].astype(np.float16).astype(np.float32)),
+                        dy=np.asfortranarray(data["dy"].astype(np.float16).astype(np.float32)))
+        x, dy = upload(data["x"], half), upload(data["dy"], half)
         layer = L.batch_normalization_layer(data["dims"], data["decay"], data["eps"], True, data["scale"], data["bias"])
         layer.bind_forward(x)
         layer.bind_backward(dy)
@@ -123,7 +126,7 @@ def main():
             t0 = time.perf_counter(); _, m, v = orc.batch_norm_fwd(data["x"], C, cs, data["eps"], data["decay"], data["scale"], data["bias"], rm, rv); t1 = time.perf_counter()
             orc.batch_norm_bwd(data["x"], data["dy"], C, cs, data["eps"], m, v, data["scale"]); t2 = time.perf_counter()
             return t1 - t0, t2 - t1
-        return layer, data["x"].size, 4, data["x"].shape[1], cpu
+        return layer, data["x"].size, 2 if half else 4, data["x"].shape[1], cpu
 
     def build_in(data):
         x, dy = upload(data["x"]), upload(data["dy"])
@@ -223,6 +226,11 @@ def main():
                                        lambda: build_sb(W.extra_entrywise_batch_norm(), "entrywise")),
         "extra_channelwise_scale_bias": ("ChannelwiseScaleBias fwd+bwd fp32 NCHW 64x256x56x56 (informational)",
                                          lambda: build_sb(W.cfg3_batch_norm(), "channelwise")),
+        # not baseline configurations: fp16 storage for batch norm, and softmax rows off the 16-byte grid
+        "extra_batch_norm_f16": ("BatchNorm train fwd+bwd fp16 storage NCHW 64x256x56x56 (informational)",
+                                 lambda: build_bn(W.cfg3_batch_norm(), True)),
+        "extra_softmax_vocab_50257": ("Softmax fwd+bwd fp32 50257x1024, rows 4-byte aligned (informational)",
+                                      lambda: build_softmax("softmax", W.cfg5b_wide_softmax(h=50257, w=1024))),
     }
     headline = "cfg2_softmax"
     if args.layers == "all":
