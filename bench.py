@@ -109,6 +109,14 @@ def main():
             return t1 - t0, t2 - t1
         return layer, data["x"].size, 2 if half else 4, data["x"].shape[1], cpu
 
+    def whole_sample_ln():
+        d = W.cfg3_batch_norm()
+        n = d["x"].shape[0]
+        rng = np.random.default_rng(0x4C420009)
+        return dict(x=d["x"], dy=d["dy"], eps=1e-5, dims=(n,),
+                    scale=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32),
+                    bias=(0.1 * rng.standard_normal(n)).astype(np.float32))
+
     def build_bn(data, half=False):
         if half:  # fp16 storage: both sides see the rounded values
             data = dict(data, x=np.asfortranarray(data["x"].astype(np.float16).astype(np.float32)),
@@ -226,6 +234,10 @@ def main():
                                        lambda: build_sb(W.extra_entrywise_batch_norm(), "entrywise")),
         "extra_channelwise_scale_bias": ("ChannelwiseScaleBias fwd+bwd fp32 NCHW 64x256x56x56 (informational)",
                                          lambda: build_sb(W.cfg3_batch_norm(), "channelwise")),
+        # not a baseline configuration: the layer's default (start_dim = 0) on an image tensor normalises
+        # whole samples: 64 rows of 802816 entries, with per-entry scale and bias
+        "extra_layer_norm_whole_sample": ("LayerNorm fwd+bwd fp32 802816x64, whole samples (informational)",
+                                          lambda: build_ln(whole_sample_ln(), False)),
         # not baseline configurations: fp16 storage for batch norm, and softmax rows off the 16-byte grid
         "extra_batch_norm_f16": ("BatchNorm train fwd+bwd fp16 storage NCHW 64x256x56x56 (informational)",
                                  lambda: build_bn(W.cfg3_batch_norm(), True)),

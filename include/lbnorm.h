@@ -81,17 +81,26 @@ int lbn_workspace_timed_out(lbn_stream_t stream, const void* workspace, int* tim
  * Backward overwrites dscale/dbias (length norm_size) when they are non-NULL;
  * dscale != NULL requires scale != NULL.  The _f16 variants store x, y, dy, dx as
  * IEEE binary16 and compute in fp32; statistics, scale, bias and their gradients
- * stay fp32. */
+ * stay fp32.
+ * Forward scratch is optional: it is only used for groups too long for one workgroup's
+ * registers (tens of thousands of entries: the layer's default, start_dim = 0,
+ * normalises over a whole sample), which are then shared by several workgroups and
+ * read once; with workspace == NULL such groups are read twice by one workgroup
+ * each.  lbn_layer_norm_fwd_workspace_bytes() is 0 for every other shape. */
+size_t lbn_layer_norm_fwd_workspace_bytes(int64_t num_groups, int64_t norm_size,
+                                          int64_t width, int elem_bytes);
 int lbn_layer_norm_fwd_f32(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
                            int64_t norm_stride, int64_t width, float epsilon,
                            const float* x, int64_t ldx, float* y, int64_t ldy,
                            float* stats, int64_t ld_stats,
-                           const float* scale, const float* bias, int flags);
+                           const float* scale, const float* bias,
+                           void* workspace, size_t workspace_bytes, int flags);
 int lbn_layer_norm_fwd_f16(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
                            int64_t norm_stride, int64_t width, float epsilon,
                            const void* x, int64_t ldx, void* y, int64_t ldy,
                            float* stats, int64_t ld_stats,
-                           const float* scale, const float* bias, int flags);
+                           const float* scale, const float* bias,
+                           void* workspace, size_t workspace_bytes, int flags);
 size_t lbn_layer_norm_bwd_workspace_bytes(int64_t num_groups, int64_t norm_size,
                                           int64_t width, int has_weight_grads,
                                           int elem_bytes);

@@ -193,16 +193,19 @@ public:
     m_statistics.Resize(2 * G, x.Width());
     const float* sw = m_scale ? m_scale_w : nullptr;
     const float* bw = m_bias ? m_bias_w : nullptr;
+    // scratch is only needed (and only non-zero) for groups of tens of thousands of entries
+    const size_t bytes = lbn_layer_norm_fwd_workspace_bytes(G, n, x.Width(), static_cast<int>(sizeof(T)));
+    void* ws = m_ws.reserve(bytes);
     int st;
     if (sizeof(T) == 2)
       st = lbn_layer_norm_fwd_f16(io.stream, G, n, stride, x.Width(), m_epsilon, x.LockedBuffer(), x.LDim(),
                                   y.Buffer(), y.LDim(), m_statistics.Buffer(), m_statistics.LDim(), sw, bw,
-                                  stats_mode);
+                                  ws, bytes, stats_mode);
     else
       st = lbn_layer_norm_fwd_f32(io.stream, G, n, stride, x.Width(), m_epsilon,
                                   reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
                                   reinterpret_cast<float*>(y.Buffer()), y.LDim(), m_statistics.Buffer(),
-                                  m_statistics.LDim(), sw, bw, stats_mode);
+                                  m_statistics.LDim(), sw, bw, ws, bytes, stats_mode);
     check_status(st, "layer_norm_layer::fp_compute");
   }
 

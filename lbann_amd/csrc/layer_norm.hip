@@ -24,6 +24,7 @@
 
 #include "device_utils.hpp"
 #include "host_utils.hpp"
+#include "layer_norm_cluster.hpp"
 #include "layer_norm_long.hpp"
 
 namespace lbn {
@@ -686,6 +687,33 @@ static bool rows_aligned4(const void* base, int64_t stride, int64_t ld, int64_t 
 constexpr int64_t kLnMaxScalarRowFwd = 8192;  // rows accessed one float at a time: 1024 threads x 8
 constexpr int64_t kLnMaxScalarRowBwd = 4096;  // 512 threads x 8
 
+// ---- rows longer than the register kernels hold: clusters of workgroups (layer_norm_cluster.hpp)
+
+static size_t ln_cluster_slot_bytes(int64_t rows, int M)
+{
+  return 64 + static_cast<size_t>(rows) * M * 2 * sizeof(unsigned long long);
+}
+
+// Partial rows of the weight gradients start on a 256-byte boundary behind the slots.
+static size_t ln_cluster_part_offset(int64_t rows, int M) { return (ln_cluster_slot_bytes(rows, M) + 255) & ~size_t(255); }
+
+// Workspace of the cluster path for rows of n entries (0: the shape does not take it).
+static size_t ln_cluster_fwd_workspace(int64_t n, int64_t rows, int ve)
+{
+  if (n % ve != 0) return 0;
+  const ClusterPlan cp = plan_ln_cluster(n / ve, kLnClFwdUnits / (kLnClThreads * ve));
+  return cp.M ? ln_cluster_slot_bytes(rows, cp.M) : 0;
+}
+
+static size_t ln_cluster_bwd_workspace(int64_t n, int64_t rows, int ve)
+{
+  if (n % ve != 0) return 0;
+  const ClusterPlan cp = plan_ln_cluster(n / ve, kLnClBwdUnits / (kLnClThreads * ve));
+  if (!cp.M) return 0;
+  return ln_cluster_part_offset(rows, cp.M) +
+         static_cast<size_t>(ln_cluster_count_bound(rows, cp.M)) * 2 * n * sizeof(float);
+}
+
 // ve: entries per 16-byte vector of the storage type (4: fp32, 8: fp16).  The size does not
 // depend on pointers or leading dimensions, which the query does not see, so it covers
 // every path the shape can take: 16-byte vectors, single floats, row slabs.
@@ -699,6 +727,7 @@ static size_t ln_bwd_workspace(int64_t n, int64_t rows, int ve)
     const LnBwdPlan p = plan_ln_bwd(n / ve, rows, ve, elem_bytes);
     if (p.tpr) cover(static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
     else cover(static_cast<size_t>(ln_wgrad_slabs(n / ve, rows)) * 2 * n * sizeof(float));
+    if (!p.tpr) cover(ln_cluster_bwd_workspace(n, rows, ve));  // long rows: slots, then one partial row per cluster
   }
   if (ve == 4 && n <= kLnMaxScalarRowBwd) {  // fp32 rows off the 16-byte grid: one float per access
     const LnBwdPlan p = plan_ln_bwd(n, rows, 1, 4);
@@ -748,10 +777,92 @@ static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, i
   return 0;
 }
 
+// Both return 1 when launched, 0 when the shape, the workspace or the device's capacity does
+// not allow the cluster path (the caller goes on to the two-pass kernels).
+template <typename T>
+static int ln_fwd_cluster_launch(hipStream_t st, const T* x, T* y, int64_t ldx, int64_t ldy, RowMap map,
+                                 int64_t rows, int64_t n, float eps, float* stats, int64_t lds,
+                                 const float* gamma, const float* beta, int sumsq, void* ws, size_t ws_bytes)
+{
+  constexpr int VE = Vec16<T>::N;
+  constexpr int kMaxV = kLnClFwdUnits / (kLnClThreads * VE);
+  const ClusterPlan cp = plan_ln_cluster(n / VE, kMaxV);
+  if (!cp.M || !ws || !aligned16(ws) || ws_bytes < ln_cluster_slot_bytes(rows, cp.M)) return 0;
+  const ClusterWorkspace cw = cluster_workspace(ws);
+  const bool affine = gamma || beta;
+#define X(VV)                                                                                        \
+  if (cp.V == VV) {                                                                                  \
+    const int cap = affine ? cluster_capacity(ln_fwd_cluster<T, VV, true>, kLnClThreads)             \
+                           : cluster_capacity(ln_fwd_cluster<T, VV, false>, kLnClThreads);           \
+    int64_t nc = cap / cp.M < rows ? cap / cp.M : rows;                                              \
+    if (nc < 1) return 0;                                                                            \
+    nc = ceil_div(rows, ceil_div(rows, nc)); /* every cluster walks the same number of rows */       \
+    LnClArgs<T> a{};                                                                                 \
+    a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy, a.map = map, a.rows = rows, a.n = n;               \
+    a.nvec = static_cast<unsigned>(n / VE), a.M = cp.M, a.sumsq = sumsq;                             \
+    a.inv_n = 1.0f / static_cast<float>(n), a.eps = eps, a.stats = stats, a.ld_stats = lds;          \
+    a.gamma = gamma, a.beta = beta, a.cw = cw, a.tag = cluster_call_tag(st, cw);                     \
+    const dim3 grid(static_cast<unsigned>(nc * cp.M));                                               \
+    if (affine) hipLaunchKernelGGL((ln_fwd_cluster<T, VV, true>), grid, dim3(kLnClThreads), 0, st, a); \
+    else hipLaunchKernelGGL((ln_fwd_cluster<T, VV, false>), grid, dim3(kLnClThreads), 0, st, a);     \
+    return 1;                                                                                        \
+  }
+  X(1) X(2)
+  if constexpr (kMaxV >= 4) { X(3) X(4) }
+#undef X
+  return 0;
+}
+
+template <typename T>
+static int ln_bwd_cluster_launch(hipStream_t st, bool wgrad, const T* x, const T* dy, T* dx, int64_t ldx,
+                                 int64_t lddy, int64_t lddx, RowMap map, int64_t rows, int64_t n, float eps,
+                                 const float* stats, int64_t lds, float* sgrad, int64_t ldsg,
+                                 const float* gamma, float* dgamma, float* dbeta, void* ws, size_t ws_bytes)
+{
+  constexpr int VE = Vec16<T>::N;
+  constexpr int kMaxV = kLnClBwdUnits / (kLnClThreads * VE);
+  const ClusterPlan cp = plan_ln_cluster(n / VE, kMaxV);
+  if (!cp.M || !ws || !aligned16(ws)) return 0;
+  const size_t need = wgrad ? ln_cluster_bwd_workspace(n, rows, VE) : ln_cluster_slot_bytes(rows, cp.M);
+  if (ws_bytes < need) return 0;
+  const ClusterWorkspace cw = cluster_workspace(ws);
+  float* wpart = reinterpret_cast<float*>(static_cast<char*>(ws) + ln_cluster_part_offset(rows, cp.M));
+#define X(VV)                                                                                        \
+  if (cp.V == VV) {                                                                                  \
+    const int cap = wgrad ? cluster_capacity(ln_bwd_cluster<T, VV, true>, kLnClThreads)              \
+                          : cluster_capacity(ln_bwd_cluster<T, VV, false>, kLnClThreads);            \
+    int64_t nc = cap / cp.M;                                                                         \
+    const int64_t bound = ln_cluster_count_bound(rows, cp.M);                                        \
+    if (nc > bound) nc = bound;                                                                      \
+    if (nc < 1) return 0;                                                                            \
+    nc = ceil_div(rows, ceil_div(rows, nc));                                                         \
+    LnClArgs<T> a{};                                                                                 \
+    a.x = x, a.dy = dy, a.out = dx, a.ldx = ldx, a.lddy = lddy, a.ldo = lddx, a.map = map;           \
+    a.rows = rows, a.n = n, a.nvec = static_cast<unsigned>(n / VE), a.M = cp.M;                      \
+    a.inv_n = 1.0f / static_cast<float>(n), a.eps = eps, a.stats = const_cast<float*>(stats);        \
+    a.ld_stats = lds, a.sgrad = sgrad, a.ld_sgrad = ldsg, a.gamma = gamma, a.wpart = wpart;          \
+    a.cw = cw, a.tag = cluster_call_tag(st, cw);                                                     \
+    const dim3 grid(static_cast<unsigned>(nc * cp.M));                                               \
+    if (wgrad) {                                                                                     \
+      hipLaunchKernelGGL((ln_bwd_cluster<T, VV, true>), grid, dim3(kLnClThreads), 0, st, a);         \
+      hipLaunchKernelGGL(ln_wgrad_reduce_wide, dim3(static_cast<unsigned>(ceil_div(n / 2, 256))), dim3(256), 0, \
+                         st, wpart, nc, n, dgamma, dbeta);                                           \
+    }                                                                                                \
+    else {                                                                                           \
+      hipLaunchKernelGGL((ln_bwd_cluster<T, VV, false>), grid, dim3(kLnClThreads), 0, st, a);        \
+    }                                                                                                \
+    return 1;                                                                                        \
+  }
+  X(1)
+  if constexpr (kMaxV >= 2) { X(2) }
+#undef X
+  return 0;
+}
+
 template <typename T>
 static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t w, float eps,
                   const T* x, int64_t ldx, T* y, int64_t ldy, float* stats, int64_t lds,
-                  const float* gamma, const float* beta, int flags)
+                  const float* gamma, const float* beta, void* ws, size_t ws_bytes, int flags)
 {
   constexpr int VE = Vec16<T>::N;
   if (G < 0 || n < 0 || w < 0 || stride < 0) return LBN_ERR_INVALID_ARGUMENT;
@@ -771,7 +882,9 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     if (int r = ln_fwd_rows_launch<T>(st, x, y, ldx, ldy, map, rows, n / VE, inv_n, eps, stats, lds, gamma,
                                       beta, sumsq))
       return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
-    // longer than the register kernels hold
+    // longer than the register kernels hold: clusters when the caller gave scratch, else two passes
+    if (ln_fwd_cluster_launch<T>(st, x, y, ldx, ldy, map, rows, n, eps, stats, lds, gamma, beta, sumsq, ws, ws_bytes))
+      return launch_status();
     hipLaunchKernelGGL((ln_fwd_long<T>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st, x, y,
                        ldx, ldy, map, n / VE, inv_n, eps, stats, lds, gamma, beta, sumsq);
     return launch_status();
@@ -907,7 +1020,10 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     if (int r = ln_bwd_rows_launch<T>(st, wgrad, x, dy, dx, ldx, lddy, lddx, map, rows, n / VE, n, sizeof(T), eps,
                                       stats, lds, sgrad, ldsg, gamma, dgamma, dbeta, ws, ws_bytes))
       return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
-    // longer than the register kernels hold
+    // longer than the register kernels hold: clusters (weight gradients included), else two passes
+    if (ln_bwd_cluster_launch<T>(st, wgrad, x, dy, dx, ldx, lddy, lddx, map, rows, n, eps, stats, lds, sgrad, ldsg,
+                                 gamma, dgamma, dbeta, ws, ws_bytes))
+      return launch_status();
     hipLaunchKernelGGL((ln_bwd_long<T>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st, x, dy,
                        dx, ldx, lddy, lddx, map, n / VE, 1.0f / static_cast<float>(n), eps, stats, lds, sgrad,
                        ldsg, gamma);
@@ -970,30 +1086,47 @@ using namespace lbn;
 
 extern "C" {
 
+size_t lbn_layer_norm_fwd_workspace_bytes(int64_t num_groups, int64_t norm_size, int64_t width, int elem_bytes)
+{
+  if (num_groups <= 0 || norm_size <= 0 || width <= 0) return 0;
+  const int ve = elem_bytes == 2 ? 8 : 4;
+  // only rows beyond the one-workgroup kernels use scratch
+  if (norm_size % ve != 0 || pick_row_config(norm_size / ve, num_groups * width, 8).tpr) return 0;
+  return ln_cluster_fwd_workspace(norm_size, num_groups * width, ve);
+}
+
 int lbn_layer_norm_fwd_f32(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
                            int64_t norm_stride, int64_t width, float epsilon, const float* x,
                            int64_t ldx, float* y, int64_t ldy, float* stats, int64_t ld_stats,
-                           const float* scale, const float* bias, int flags)
+                           const float* scale, const float* bias, void* workspace,
+                           size_t workspace_bytes, int flags)
 {
   return ln_fwd<float>(as_stream(stream), num_groups, norm_size, norm_stride, width, epsilon, x, ldx,
-                       y, ldy, stats, ld_stats, scale, bias, flags);
+                       y, ldy, stats, ld_stats, scale, bias, workspace, workspace_bytes, flags);
 }
 
 int lbn_layer_norm_fwd_f16(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
                            int64_t norm_stride, int64_t width, float epsilon, const void* x,
                            int64_t ldx, void* y, int64_t ldy, float* stats, int64_t ld_stats,
-                           const float* scale, const float* bias, int flags)
+                           const float* scale, const float* bias, void* workspace,
+                           size_t workspace_bytes, int flags)
 {
   return ln_fwd<__half>(as_stream(stream), num_groups, norm_size, norm_stride, width, epsilon,
                         static_cast<const __half*>(x), ldx, static_cast<__half*>(y), ldy, stats,
-                        ld_stats, scale, bias, flags);
+                        ld_stats, scale, bias, workspace, workspace_bytes, flags);
 }
 
 size_t lbn_layer_norm_bwd_workspace_bytes(int64_t num_groups, int64_t norm_size, int64_t width,
                                           int has_weight_grads, int elem_bytes)
 {
-  if (!has_weight_grads || num_groups <= 0 || width <= 0) return 0;
-  return ln_bwd_workspace(norm_size, num_groups * width, elem_bytes == 2 ? 8 : 4);
+  if (num_groups <= 0 || norm_size <= 0 || width <= 0) return 0;
+  const int ve = elem_bytes == 2 ? 8 : 4;
+  const int64_t rows = num_groups * width;
+  if (has_weight_grads) return ln_bwd_workspace(norm_size, rows, ve);
+  // without weight gradients only the cluster kernels of long rows use scratch (their slots)
+  if (norm_size % ve != 0 || plan_ln_bwd(norm_size / ve, rows, ve, elem_bytes == 2 ? 2 : 4).tpr) return 0;
+  const ClusterPlan cp = plan_ln_cluster(norm_size / ve, kLnClBwdUnits / (kLnClThreads * ve));
+  return cp.M ? ln_cluster_slot_bytes(rows, cp.M) : 0;
 }
 
 int lbn_layer_norm_bwd_f32(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
@@ -1029,7 +1162,7 @@ int lbn_instance_norm_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t cha
                               int64_t ldy, float* stats, int64_t ld_stats)
 {
   return ln_fwd<float>(as_stream(stream), channels, channel_size, channel_size, width, epsilon, x,
-                       ldx, y, ldy, stats, ld_stats, nullptr, nullptr, LBN_STATS_TWO_PASS);
+                       ldx, y, ldy, stats, ld_stats, nullptr, nullptr, nullptr, 0, LBN_STATS_TWO_PASS);
 }
 
 size_t lbn_instance_norm_bwd_workspace_bytes(int64_t channels, int64_t channel_size, int64_t width)

@@ -1,0 +1,478 @@
+// Layer norm over rows too long for one workgroup's registers (a whole image sample:
+// the layer's default is to normalise over every entry of a sample), when there are
+// too few rows to fill the device with one workgroup per row.  Math as in
+// layer_norm.hip (layer_norm.cpp:41-136, :139-258).
+//
+// A cluster of M workgroups of 1024 threads shares a row (cluster_sync.hpp): workgroup k
+// keeps vectors [k*1024*V, (k+1)*1024*V) in registers, the cluster exchanges one pair of
+// partial sums per row and every workgroup finishes its share from registers, so x (and
+// dy) cross HBM once.  The grid is persistent (cluster cl takes rows cl, cl + nclusters,
+// ...) and rotates three register tiles like the batch-norm and softmax cluster kernels:
+// in a step a workgroup reduces the tile loaded a step earlier and publishes its sums,
+// issues the loads of the tile after that, then collects the sums of the oldest tile and
+// writes its output.
+//
+// A workgroup always owns the same feature positions, so it copies its slice of scale and
+// bias into LDS once (thread-private cells) instead of fetching 8 bytes of weights per
+// entry and row from the caches.
+//
+// Backward with weight gradients: for the same reason
+// it accumulates its slice of dscale / dbias over all its rows in LDS (thread-private
+// cells again, no synchronisation) and writes one partial row per cluster at the end;
+// ln_wgrad_reduce adds the clusters' rows in a fixed order.
+#pragma once
+
+#include "cluster_sync.hpp"
+#include "device_utils.hpp"
+
+namespace lbn {
+
+constexpr int kLnClThreads = 1024;
+constexpr int kLnClWaves = kLnClThreads / kWave;
+constexpr int kLnClMaxM = 128;       // a wave polls two slots per lane
+constexpr int kLnClFwdUnits = 16384;  // entries per workgroup in forward: 2 x 64 KiB of LDS for scale and bias
+constexpr int kLnClBwdUnits = 8192;   // in backward: 2 x 32 KiB of LDS accumulators and 32 KiB for the scale
+
+template <typename T>
+struct LnClArgs {
+  const T* x;
+  const T* dy;  // backward only
+  T* out;       // forward: y; backward: dx
+  int64_t ldx, lddy, ldo;
+  RowMap map;
+  int64_t rows;
+  int64_t n;
+  unsigned nvec;
+  int M, sumsq;
+  float inv_n, eps;
+  float* stats;  // forward: written; backward: read
+  int64_t ld_stats;
+  float* sgrad;  // backward: written
+  int64_t ld_sgrad;
+  const float* gamma;
+  const float* beta;
+  float* wpart;  // backward with weight gradients: one row of 2n floats per cluster
+  ClusterWorkspace cw;
+  ClusterTag tag;
+  __device__ __forceinline__ unsigned long long* slots(int64_t row) const { return cw.slots + row * M * 2; }
+};
+
+// cluster_collect() for up to 128 members: lane j polls slots j and j + 64.  Returns the
+// wave's totals in every lane.
+__device__ __forceinline__ void ln_cl_collect(unsigned long long* slots, int M, ClusterTag tag, int* error_word,
+                                              float& ta, float& tb)
+{
+  const int lane = threadIdx.x & 63;
+  unsigned long long w[2][2] = {{0, 0}, {0, 0}};
+  bool have[2] = {false, false};
+  int polls = 0;
+  for (;;) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int j = lane + 64 * h;
+      if (j < M && !have[h]) {
+        w[h][0] = __hip_atomic_load(slots + 2 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        w[h][1] = __hip_atomic_load(slots + 2 * j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        have[h] = static_cast<unsigned>(w[h][0] >> 32) == tag.lo && static_cast<unsigned>(w[h][1] >> 32) == tag.hi;
+      }
+    }
+    if (__all((have[0] || lane >= M) && (have[1] || lane + 64 >= M))) break;
+    if (++polls > kClusterMaxPolls) {
+      if (lane == 0) __hip_atomic_store(error_word, kClusterTimedOut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+  float a = 0.f, b = 0.f;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    if (have[h]) {
+      a += __uint_as_float(static_cast<unsigned>(w[h][0]));
+      b += __uint_as_float(static_cast<unsigned>(w[h][1]));
+    }
+  }
+  ta = wave_sum(a);
+  tb = wave_sum(b);
+}
+
+// Copies this thread's V vectors of a weight array (or `fill` when there is none) into its
+// LDS cells: cell i of thread t is cells[(i * 1024 + t) * VE ...].
+template <typename T, int V>
+__device__ __forceinline__ void ln_cl_stage_weights(const float* w, float fill, unsigned base, unsigned nvec,
+                                                    float* cells)
+{
+  constexpr int VE = Vec16<T>::N;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = base + i * kLnClThreads;
+    float v[VE];
+#pragma unroll
+    for (int e = 0; e < VE; ++e) v[e] = fill;
+    if (w && idx < nvec) load_f32_run<VE>(w + VE * static_cast<int64_t>(idx), v);
+    float* cell = cells + (i * kLnClThreads + threadIdx.x) * VE;
+#pragma unroll
+    for (int e = 0; e < VE; ++e) cell[e] = v[e];
+  }
+}
+
+// ------------------------------------------------------------------------ forward
+template <typename T, int V>
+struct LnClFwdTile {
+  typename Vec16<T>::raw_t v[V];
+  float K;  // pivot of the sums: the row's first entry, or 0 for the reference's formula
+};
+
+template <typename T, int V>
+__device__ __forceinline__ void ln_cl_fwd_load(LnClFwdTile<T, V>& t, const LnClArgs<T>& a, int64_t row, unsigned base)
+{
+  using IO = Vec16<T>;
+  const T* xr = a.x + a.map.offset(row, a.ldx);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = base + i * kLnClThreads;
+    t.v[i] = typename IO::raw_t{};
+    if (idx < a.nvec) t.v[i] = IO::load_raw(xr + IO::N * static_cast<int64_t>(idx));
+  }
+  t.K = a.sumsq ? 0.f : IO::load1(xr);
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void ln_cl_fwd_reduce(const LnClArgs<T>& a, int64_t row, int k, unsigned base,
+                                                 const LnClFwdTile<T, V>& t, float* red)
+{
+  using IO = Vec16<T>;
+  float s = 0.f, q = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    if (base + i * kLnClThreads < a.nvec) {
+      float v[IO::N];
+      IO::unpack(t.v[i], v);
+#pragma unroll
+      for (int e = 0; e < IO::N; ++e) {
+        const float d = v[e] - t.K;
+        s += d;
+        q = __builtin_fmaf(d, d, q);
+      }
+    }
+  }
+  team_sum2<kLnClWaves>(s, q, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+  if (threadIdx.x == 0) cluster_publish(s, q, a.slots(row), k, a.tag);
+}
+
+template <typename T, int V, bool AFFINE>
+__device__ __forceinline__ void ln_cl_fwd_finish(const LnClArgs<T>& a, int64_t row, int k, unsigned base,
+                                                 const LnClFwdTile<T, V>& t, float* bc, const float* wts)
+{
+  using IO = Vec16<T>;
+  if (threadIdx.x < kWave) {
+    float ts, tq;
+    ln_cl_collect(a.slots(row), a.M, a.tag, a.cw.error, ts, tq);
+    if (threadIdx.x == 0) {
+      float dm = ts * a.inv_n;
+      float var = fmaxf(__builtin_fmaf(-dm, dm, tq * a.inv_n), 0.f);
+      if (a.sumsq) {  // the reference's own expression (layer_norm.cpp:99-112): true divisions, no fused multiply-add
+        const float nf = static_cast<float>(a.n);
+        dm = ts / nf;
+        var = fmaxf(__fsub_rn(tq / nf, __fmul_rn(dm, dm)), 0.f);
+      }
+      const float mean = t.K + dm;
+      bc[0] = mean;
+      bc[1] = 1.0f / sqrtf(var + a.eps);
+      if (k == 0) {
+        int64_t col, g;
+        a.map.split(row, col, g);
+        a.stats[g + col * a.ld_stats] = mean;
+        a.stats[a.map.groups + g + col * a.ld_stats] = var;
+      }
+    }
+  }
+  __syncthreads();
+  const float mean = bc[0];
+  const float inv_stdev = bc[1];
+  T* yr = a.out + a.map.offset(row, a.ldo);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = base + i * kLnClThreads;
+    if (idx < a.nvec) {
+      float v[IO::N];
+      IO::unpack(t.v[i], v);
+      if (AFFINE) {
+        const float* ga = wts + (i * kLnClThreads + threadIdx.x) * IO::N;
+        const float* be = ga + kLnClThreads * V * IO::N;
+#pragma unroll
+        for (int e = 0; e < IO::N; ++e) v[e] = __builtin_fmaf((v[e] - mean) * inv_stdev, ga[e], be[e]);
+      }
+      else {
+#pragma unroll
+        for (int e = 0; e < IO::N; ++e) v[e] = (v[e] - mean) * inv_stdev;
+      }
+      IO::store(yr + IO::N * static_cast<int64_t>(idx), v);
+    }
+  }
+}
+
+template <typename T, int V, bool AFFINE>
+__device__ __forceinline__ void ln_cl_fwd_step(const LnClArgs<T>& a, int64_t row, int64_t nc, int k, unsigned base,
+                                               LnClFwdTile<T, V>& F, LnClFwdTile<T, V>& R, LnClFwdTile<T, V>& L,
+                                               float* red, float* bc, const float* wts)
+{
+  if (row + nc < a.rows) ln_cl_fwd_reduce<T, V>(a, row + nc, k, base, R, red);
+  if (row + 2 * nc < a.rows) ln_cl_fwd_load<T, V>(L, a, row + 2 * nc, base);
+  asm volatile("" ::: "memory");  // keep the loads above the wait below
+  ln_cl_fwd_finish<T, V, AFFINE>(a, row, k, base, F, bc, wts);
+}
+
+template <typename T, int V, bool AFFINE>
+__global__ void __launch_bounds__(kLnClThreads)
+ln_fwd_cluster(LnClArgs<T> a)
+{
+  static_assert(kLnClThreads * V * Vec16<T>::N <= kLnClFwdUnits, "a workgroup's share of scale and bias must fit LDS");
+  __shared__ float red[2 * kLnClWaves];
+  __shared__ float bc[3][2];
+  __shared__ float wts[AFFINE ? 2 * kLnClThreads * V * Vec16<T>::N : 1];  // scale cells, then bias cells
+  const int64_t nc = gridDim.x / a.M;
+  const int64_t cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - static_cast<int>(cl) * a.M;
+  const unsigned base = static_cast<unsigned>(k) * (kLnClThreads * V) + threadIdx.x;
+  if (cl >= a.rows) return;
+  cluster_resolve_tag(a.tag);
+  if (AFFINE) {  // read back by the same thread only: no barrier needed
+    ln_cl_stage_weights<T, V>(a.gamma, 1.f, base, a.nvec, wts);
+    ln_cl_stage_weights<T, V>(a.beta, 0.f, base, a.nvec, wts + kLnClThreads * V * Vec16<T>::N);
+  }
+  LnClFwdTile<T, V> t0, t1, t2;
+  ln_cl_fwd_load<T, V>(t0, a, cl, base);
+  if (cl + nc < a.rows) ln_cl_fwd_load<T, V>(t1, a, cl + nc, base);
+  ln_cl_fwd_reduce<T, V>(a, cl, k, base, t0, red);
+  __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
+  // one broadcast pair per position of the rotation: a step without a reduction has no
+  // barrier between the reads of one finish and the write of the next
+  for (int64_t row = cl; row < a.rows; row += 3 * nc) {
+    ln_cl_fwd_step<T, V, AFFINE>(a, row, nc, k, base, t0, t1, t2, red, bc[0], wts);
+    if (row + nc < a.rows) ln_cl_fwd_step<T, V, AFFINE>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1], wts);
+    if (row + 2 * nc < a.rows) ln_cl_fwd_step<T, V, AFFINE>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2], wts);
+  }
+}
+
+// ----------------------------------------------------------------------- backward
+template <typename T, int V>
+struct LnClBwdTile {
+  typename Vec16<T>::raw_t x[V];
+  typename Vec16<T>::raw_t g[V];
+  float mean, inv_stdev;
+};
+
+template <typename T, int V>
+__device__ __forceinline__ void ln_cl_bwd_load(LnClBwdTile<T, V>& t, const LnClArgs<T>& a, int64_t row, unsigned base)
+{
+  using IO = Vec16<T>;
+  int64_t col, g;
+  a.map.split(row, col, g);
+  const T* xr = a.x + g * a.map.stride + col * a.ldx;
+  const T* gr = a.dy + g * a.map.stride + col * a.lddy;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = base + i * kLnClThreads;
+    t.x[i] = typename IO::raw_t{};
+    t.g[i] = typename IO::raw_t{};
+    if (idx < a.nvec) {
+      t.x[i] = IO::load_raw(xr + IO::N * static_cast<int64_t>(idx));
+      t.g[i] = IO::load_raw(gr + IO::N * static_cast<int64_t>(idx));
+    }
+  }
+  t.mean = a.stats[g + col * a.ld_stats];
+  t.inv_stdev = 1.0f / sqrtf(a.stats[a.map.groups + g + col * a.ld_stats] + a.eps);
+}
+
+// A = sum(dy * scale), B = sum(dy * scale * xh) with xh = (x - mean) / stdev.
+template <typename T, int V>
+__device__ __forceinline__ void ln_cl_bwd_reduce(const LnClArgs<T>& a, int64_t row, int k, unsigned base,
+                                                 const LnClBwdTile<T, V>& t, float* red, const float* scale_cells)
+{
+  using IO = Vec16<T>;
+  constexpr int VE = IO::N;
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = base + i * kLnClThreads;
+    if (idx < a.nvec) {
+      float x[VE], g[VE];
+      IO::unpack(t.x[i], x);
+      IO::unpack(t.g[i], g);
+      const float* ga = scale_cells + (i * kLnClThreads + threadIdx.x) * VE;
+#pragma unroll
+      for (int e = 0; e < VE; ++e) {
+        const float xh = (x[e] - t.mean) * t.inv_stdev;
+        const float gs = g[e] * ga[e];
+        sa += gs;
+        sb = __builtin_fmaf(gs, xh, sb);
+      }
+    }
+  }
+  team_sum2<kLnClWaves>(sa, sb, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+  if (threadIdx.x == 0) cluster_publish(sa, sb, a.slots(row), k, a.tag);
+}
+
+// dx from the cluster's sums; the weight gradients dscale += dy * xh, dbias += dy go to this
+// thread's cells of `acc` here, after the rendezvous, where nobody waits for them.
+template <typename T, int V, bool WGRAD>
+__device__ __forceinline__ void ln_cl_bwd_finish(const LnClArgs<T>& a, int64_t row, int k, unsigned base,
+                                                 const LnClBwdTile<T, V>& t, float* bc, const float* scale_cells,
+                                                 float* acc)
+{
+  using IO = Vec16<T>;
+  constexpr int VE = IO::N;
+  const float inv_stdev = t.inv_stdev;
+  int64_t col, g;
+  a.map.split(row, col, g);
+  if (threadIdx.x < kWave) {
+    float ta, tb;
+    ln_cl_collect(a.slots(row), a.M, a.tag, a.cw.error, ta, tb);
+    if (threadIdx.x == 0) {
+      const float dmean = -ta * inv_stdev;
+      const float dvar = -tb * inv_stdev * inv_stdev * 0.5f;
+      bc[0] = dmean * a.inv_n;
+      bc[1] = -tb * inv_stdev * a.inv_n;  // dvar * 2 / n per unit of xh
+      if (k == 0) {
+        a.sgrad[g + col * a.ld_sgrad] = dmean;
+        a.sgrad[a.map.groups + g + col * a.ld_sgrad] = dvar;
+      }
+    }
+  }
+  __syncthreads();
+  const float c0 = bc[0];
+  const float c1 = bc[1];
+  T* dr = a.out + g * a.map.stride + col * a.ldo;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = base + i * kLnClThreads;
+    if (idx < a.nvec) {
+      float x[VE], d[VE];
+      IO::unpack(t.x[i], x);
+      IO::unpack(t.g[i], d);
+      const float* ga = scale_cells + (i * kLnClThreads + threadIdx.x) * VE;
+      float* cell = acc + (i * kLnClThreads + threadIdx.x) * VE;
+#pragma unroll
+      for (int e = 0; e < VE; ++e) {
+        const float xh = (x[e] - t.mean) * inv_stdev;
+        if (WGRAD) {
+          cell[e] = __builtin_fmaf(d[e], xh, cell[e]);
+          cell[kLnClBwdUnits + e] += d[e];
+        }
+        d[e] = __builtin_fmaf(d[e] * ga[e], inv_stdev, __builtin_fmaf(c1, xh, c0));
+      }
+      IO::store(dr + VE * static_cast<int64_t>(idx), d);
+    }
+  }
+}
+
+template <typename T, int V, bool WGRAD>
+__device__ __forceinline__ void ln_cl_bwd_step(const LnClArgs<T>& a, int64_t row, int64_t nc, int k, unsigned base,
+                                               LnClBwdTile<T, V>& F, LnClBwdTile<T, V>& R, LnClBwdTile<T, V>& L,
+                                               float* red, float* bc, float* acc, const float* scale_cells)
+{
+  if (row + nc < a.rows) ln_cl_bwd_reduce<T, V>(a, row + nc, k, base, R, red, scale_cells);
+  if (row + 2 * nc < a.rows) ln_cl_bwd_load<T, V>(L, a, row + 2 * nc, base);
+  asm volatile("" ::: "memory");
+  ln_cl_bwd_finish<T, V, WGRAD>(a, row, k, base, F, bc, scale_cells, acc);
+}
+
+template <typename T, int V, bool WGRAD>
+__global__ void __launch_bounds__(kLnClThreads)
+ln_bwd_cluster(LnClArgs<T> a)
+{
+  constexpr int VE = Vec16<T>::N;
+  static_assert(kLnClThreads * V * VE <= kLnClBwdUnits, "a workgroup's share must fit the LDS accumulators");
+  __shared__ float red[2 * kLnClWaves];
+  __shared__ float bc[3][2];
+  __shared__ float acc[WGRAD ? 2 * kLnClBwdUnits : 1];
+  __shared__ float scale_cells[kLnClThreads * V * VE];
+  const int64_t nc = gridDim.x / a.M;
+  const int64_t cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - static_cast<int>(cl) * a.M;
+  const unsigned base = static_cast<unsigned>(k) * (kLnClThreads * V) + threadIdx.x;
+  if (cl >= a.rows) return;
+  cluster_resolve_tag(a.tag);
+  if (WGRAD) {
+    for (int p = threadIdx.x; p < 2 * kLnClBwdUnits; p += kLnClThreads) acc[p] = 0.f;  // each thread clears its own cells
+  }
+  ln_cl_stage_weights<T, V>(a.gamma, 1.f, base, a.nvec, scale_cells);  // read back by the same thread only
+  LnClBwdTile<T, V> t0, t1, t2;
+  ln_cl_bwd_load<T, V>(t0, a, cl, base);
+  if (cl + nc < a.rows) ln_cl_bwd_load<T, V>(t1, a, cl + nc, base);
+  if (WGRAD) __syncthreads();  // the clearing loop above is strided differently from the cells' owners
+  ln_cl_bwd_reduce<T, V>(a, cl, k, base, t0, red, scale_cells);
+  __syncthreads();
+  for (int64_t row = cl; row < a.rows; row += 3 * nc) {
+    ln_cl_bwd_step<T, V, WGRAD>(a, row, nc, k, base, t0, t1, t2, red, bc[0], acc, scale_cells);
+    if (row + nc < a.rows)
+      ln_cl_bwd_step<T, V, WGRAD>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1], acc, scale_cells);
+    if (row + 2 * nc < a.rows)
+      ln_cl_bwd_step<T, V, WGRAD>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2], acc, scale_cells);
+  }
+  if (WGRAD) {
+    // this cluster's partial row: 2n floats, dscale then dbias
+    float* out = a.wpart + cl * 2 * a.n;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = base + i * kLnClThreads;
+      if (idx < a.nvec) {
+        const float* cell = acc + (i * kLnClThreads + threadIdx.x) * VE;
+        float dg[VE], db[VE];
+#pragma unroll
+        for (int e = 0; e < VE; ++e) {
+          dg[e] = cell[e];
+          db[e] = cell[kLnClBwdUnits + e];
+        }
+        store_f32_run<VE>(out + VE * static_cast<int64_t>(idx), dg);
+        store_f32_run<VE>(out + a.n + VE * static_cast<int64_t>(idx), db);
+      }
+    }
+  }
+}
+
+// Adds the P partial rows (2n floats each: dscale then dbias) that the clusters wrote, in
+// order.  Long rows and few partials: a thread owns four consecutive positions and walks
+// the rows, so every access is a coalesced 16-byte one.  n is a multiple of 4.
+__global__ void __launch_bounds__(256)
+ln_wgrad_reduce_wide(const float* __restrict__ part, int64_t P, int64_t n, float* __restrict__ dscale,
+                     float* __restrict__ dbias)
+{
+  const int64_t q = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (q >= n / 2) return;  // 2n / 4 quads
+  const int64_t j = 4 * q;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int64_t p = 0; p < P; ++p) {
+    float w[4];
+    Vec16<float>::load(part + p * 2 * n + j, w);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] += w[c];
+  }
+  float* out = j < n ? dscale : dbias;
+  if (!out) return;
+  const int64_t k = j < n ? j : j - n;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) out[k + c] = acc[c];
+}
+
+// ------------------------------------------------------------------------ host side
+// Cluster shape for rows of nvec vectors with at most max_v vectors per thread.
+inline ClusterPlan plan_ln_cluster(int64_t nvec, int max_v)
+{
+  const int64_t per = kLnClThreads;
+  const int64_t M = (nvec + per * max_v - 1) / (per * max_v);
+  if (M < 1 || M > kLnClMaxM) return {0, 0};
+  return {static_cast<int>((nvec + per * M - 1) / (per * M)), static_cast<int>(M)};
+}
+
+// Clusters a launch may use: bounded by what the workspace query assumes (it cannot ask the
+// device), by the rows and by the workgroups the device holds at once.
+inline int64_t ln_cluster_count_bound(int64_t rows, int M)
+{
+  int64_t nc = 512 / M;
+  if (nc > rows) nc = rows;
+  return nc < 1 ? 1 : nc;
+}
+
+}  // namespace lbn

@@ -199,6 +199,17 @@ class layer_norm_layer(_Layer):
     def _suffix(self):
         return "f16" if self.prev_activations.dtype == torch.float16 else "f32"
 
+    def _scratch(self):
+        """One scratch buffer for both directions, sized for the larger need, so that neither
+        call's bound pointer is invalidated by the other growing it."""
+        x = self.prev_activations
+        G, n = self.num_normalized, self.normalization_size
+        esize = 2 if x.dtype == torch.float16 else 4
+        lib = capi.lib()
+        need = max(lib.lbn_layer_norm_fwd_workspace_bytes(G, n, x.width, esize),
+                   lib.lbn_layer_norm_bwd_workspace_bytes(G, n, x.width, int(self.m_scale or self.m_bias), esize))
+        return self._ws.get(need, self.device)
+
     def fp_call(self):
         x, y = self.prev_activations, self.activations
         G, n = self.num_normalized, self.normalization_size
@@ -206,10 +217,11 @@ class layer_norm_layer(_Layer):
             self.m_statistics = DeviceMatrix(2 * G, x.width, device=self.device)
         scale = self.weights[0].Buffer() if self.m_scale else _null()
         bias = self.weights[-1].Buffer() if self.m_bias else _null()
+        ws, nb = self._scratch()
         return (f"lbn_layer_norm_fwd_{self._suffix()}",
                 (_stream(), G, n, self.normalization_stride, x.width,
                  self.m_epsilon, x.Buffer(), x.ldim, y.Buffer(), y.ldim, self.m_statistics.Buffer(),
-                 self.m_statistics.ldim, scale, bias, self.stats_mode))
+                 self.m_statistics.ldim, scale, bias, ws, nb, self.stats_mode))
 
     def bp_call(self):
         x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
@@ -219,9 +231,7 @@ class layer_norm_layer(_Layer):
         scale = self.weights[0].Buffer() if self.m_scale else _null()
         dscale = self.m_scale_gradient.Buffer() if self.m_scale else _null()
         dbias = self.m_bias_gradient.Buffer() if self.m_bias else _null()
-        wgrad = int(self.m_scale or self.m_bias)
-        esize = 2 if x.dtype == torch.float16 else 4
-        ws, nb = self._ws.get(capi.lib().lbn_layer_norm_bwd_workspace_bytes(G, n, x.width, wgrad, esize), self.device)
+        ws, nb = self._scratch()
         return (f"lbn_layer_norm_bwd_{self._suffix()}",
                 (_stream(), G, n, self.normalization_stride, x.width,
                  self.m_epsilon, x.Buffer(), x.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim,

@@ -39,6 +39,10 @@ def test_binding_matches_header():
     assert lib.lbn_softmax_workspace_bytes(0, 16) == 0
     assert lib.lbn_batch_norm_workspace_bytes(256, 3136, 64) > 0
     assert lib.lbn_layer_norm_bwd_workspace_bytes(1, 4096, 8192, 0, 2) == 0
+    assert lib.lbn_layer_norm_fwd_workspace_bytes(1, 4096, 8192, 2) == 0
+    assert lib.lbn_layer_norm_fwd_workspace_bytes(1, 802816, 64, 4) >= 64 * 49 * 16     # slots of 64 rows x 49 workgroups
+    assert lib.lbn_layer_norm_bwd_workspace_bytes(1, 802816, 64, 0, 4) >= 64 * 98 * 16
+    assert lib.lbn_layer_norm_bwd_workspace_bytes(1, 802816, 64, 1, 4) >= 2 * 2 * 802816 * 4
     assert lib.lbn_layer_norm_bwd_workspace_bytes(1, 4096, 8192, 1, 2) >= 2 * 4096 * 4
 
 

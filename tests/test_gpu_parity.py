@@ -166,6 +166,10 @@ LN_CASES = [
     # gradients by row slabs (vector and scalar), groups, padded leading dimension
     ((150528,), 0, 6, True, 0), ((65536,), 0, 300, True, 0), ((4, 20000), -1, 9, True, 0),
     ((20001,), 0, 7, True, 0), ((20004,), 0, 5, True, 4), ((3, 224, 224), 0, 3, False, 0),
+    # the same lengths on the 16-byte grid share a row among a cluster of workgroups: up to 128 members
+    # (1048576 entries backward), beyond that the two-pass kernels again; more rows than clusters
+    ((802816,), 0, 5, True, 0), ((1048576,), 0, 3, True, 0), ((1048580,), 0, 2, True, 0), ((32772,), 0, 700, True, 0),
+    ((2, 100000), -1, 40, True, 8), ((50000,), 0, 33, False, 0),
     # rows off the 16-byte grid: the register kernels with one float per access
     ((1001,), 0, 40, True, 0), ((197, 769), -1, 3, True, 0), ((4095,), 0, 9, True, 0), ((4097,), 0, 9, True, 0),
     ((8191,), 0, 5, False, 0), ((49,), 0, 3000, True, 0), ((1000,), 0, 17, True, 3), ((7,), 0, 100000, True, 0),
@@ -239,7 +243,10 @@ def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
                                                    # even lengths that are not a multiple of 8: one pair per access
                                                    ((4100,), 0, 40, 0), ((1002,), 0, 33, 0), ((6, 770), -1, 9, 0),
                                                    ((8190,), 0, 5, 2), ((16382,), 0, 3, 0), ((4100, 12), -1, 2, 0),
-                                                   ((1001,), 0, 7, 0)])   # odd: scalar fallback
+                                                   ((1001,), 0, 7, 0),   # odd: scalar fallback
+                                                   # long rows shared by clusters of workgroups
+                                                   ((802816,), 0, 4, 0), ((65536,), 0, 150, 0), ((2, 100000), -1, 20, 8),
+                                                   ((1048576,), 0, 2, 0)])
 def test_layer_norm_f16(L, dims, start_dim, w, pad):
     rng = np.random.default_rng(int(np.prod(dims)) * 3 + w)
     h = int(np.prod(dims))
@@ -514,14 +521,14 @@ def test_empty_and_rejected_arguments(L):
     # empty inputs: success, nothing launched, no pointer touched
     assert lib.lbn_softmax_fwd_f32(st, 0, 5, null, 0, null, 0, null, 0) == 0
     assert lib.lbn_softmax_fwd_f32(st, 8, 0, null, 8, null, 8, null, 0) == 0
-    assert lib.lbn_layer_norm_fwd_f32(st, 1, 8, 8, 0, 1e-5, null, 8, null, 8, null, 2, null, null, 0) == 0
+    assert lib.lbn_layer_norm_fwd_f32(st, 1, 8, 8, 0, 1e-5, null, 8, null, 8, null, 2, null, null, null, 0, 0) == 0
     assert lib.lbn_batch_norm_fwd_f32(st, 0, 4, 4, 1, 1e-5, 0.9, 1, null, 0, null, 0, null, null, null, null, null, null, null, 0, 0) == 0
     assert lib.lbn_channelwise_softmax_bwd_f32(st, 4, 0, 0, 3, null, 0, null, 0, null, 0, null, 0) == 0
     # rejected arguments come back as negative status codes, never as a fault
     assert lib.lbn_softmax_fwd_f32(st, -1, 5, p, 8, p, 8, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT
     assert lib.lbn_softmax_fwd_f32(st, 8, 2, p, 4, p, 8, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT   # ld < height
     assert lib.lbn_softmax_fwd_f32(st, 8, 2, null, 8, p, 8, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT
-    assert lib.lbn_softmax_fwd_f32(st, 9001, 2, p, 9001, p, 9001, null, 0) == capi.LBN_ERR_WORKSPACE  # split path needs scratch
+    assert lib.lbn_softmax_fwd_f32(st, 40001, 2, p, 40001, p, 40001, null, 0) == capi.LBN_ERR_WORKSPACE  # split path needs scratch
     assert lib.lbn_batch_norm_fwd_f32(st, 2, 4, 2, 1, 1e-5, 0.9, 1, p, 8, p, 8, p, p, p, p, p, p, null, 0, 0) == capi.LBN_ERR_WORKSPACE
     assert lib.lbn_layer_norm_bwd_f32(st, 1, 8, 8, 2, 1e-5, p, 8, p, 8, p, 8, p, 2, p, 2, null, p, null, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT
     assert b"workspace" in lib.lbn_status_string(capi.LBN_ERR_WORKSPACE)
