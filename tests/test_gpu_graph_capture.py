@@ -44,6 +44,8 @@ CASES = [
      ("m_statistics", "m_statistics_gradient", "m_scale_gradient", "m_bias_gradient")),
     ("layer norm f16", lambda L: L.layer_norm_layer((4096,), 1e-5, True, True), 4096, 256, torch.float16,
      ("m_statistics", "m_scale_gradient", "m_bias_gradient")),
+    ("layer norm clusters", lambda L: L.layer_norm_layer((150528,), 1e-5, True, True), 150528, 40, torch.float32,
+     ("m_statistics", "m_statistics_gradient", "m_scale_gradient", "m_bias_gradient")),
     ("instance norm", lambda L: L.instance_norm_layer((8, 32, 32)), 8192, 24, torch.float32, ()),
     ("entry-wise batch norm", lambda L: L.entrywise_batch_normalization_layer((4096,)), 4096, 48, torch.float32,
      ("m_batch_statistics", "m_batch_statistics_gradient")),
