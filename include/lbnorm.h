@@ -132,11 +132,16 @@ int lbn_layer_norm_bwd_f16(lbn_stream_t stream, int64_t num_groups, int64_t norm
  * variance in rows [C,2C); the matrix is private to the layer, which only hands it
  * from forward to backward.  channel_size <= 1: y = 0 and dx = 0
  * (instance_norm.cpp:65-68, :164-167).  The backward workspace takes the place of
- * the reference's local statistics-gradient matrix (instance_norm.cpp:173-174). */
+ * the reference's local statistics-gradient matrix (instance_norm.cpp:173-174).
+ * Forward scratch is optional and only non-zero for channels of tens of thousands
+ * of entries (volumes), as for layer norm. */
+size_t lbn_instance_norm_fwd_workspace_bytes(int64_t channels, int64_t channel_size,
+                                             int64_t width);
 int lbn_instance_norm_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
                               int64_t width, float epsilon,
                               const float* x, int64_t ldx, float* y, int64_t ldy,
-                              float* stats, int64_t ld_stats);
+                              float* stats, int64_t ld_stats,
+                              void* workspace, size_t workspace_bytes);
 size_t lbn_instance_norm_bwd_workspace_bytes(int64_t channels, int64_t channel_size,
                                              int64_t width);
 int lbn_instance_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,

@@ -520,9 +520,10 @@ public:
     const Mat& x = *io.prev_activations;
     Mat& y = *io.activations;
     m_workspace.Resize(2 * num_channels(), x.Width());
+    const size_t bytes = lbn_instance_norm_fwd_workspace_bytes(num_channels(), channel_size(), x.Width());
     check_status(lbn_instance_norm_fwd_f32(io.stream, num_channels(), channel_size(), x.Width(), m_epsilon,
                                            x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(),
-                                           m_workspace.Buffer(), m_workspace.LDim()),
+                                           m_workspace.Buffer(), m_workspace.LDim(), m_ws_fwd.reserve(bytes), bytes),
                  "instance_norm_layer::fp_compute");
   }
   void bp_compute()
@@ -540,7 +541,8 @@ public:
 private:
   float m_epsilon;
   std::vector<int64_t> m_dims;
-  workspace m_ws;
+  workspace m_ws;      // backward: statistics gradients, then the cluster kernels' slots
+  workspace m_ws_fwd;  // forward scratch (long channels only)
 };
 
 // ---------------------------------------------------------- entry-wise batch norm

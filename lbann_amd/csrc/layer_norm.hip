@@ -1157,18 +1157,32 @@ int lbn_layer_norm_bwd_f16(lbn_stream_t stream, int64_t num_groups, int64_t norm
 // Instance norm is layer norm over groups of channel_size entries without scale and
 // bias (instance_norm.cpp:47-231 against layer_norm.cpp:41-258: the same statistics,
 // the same 2/n factor in backward, the same constant output for single-entry groups).
+size_t lbn_instance_norm_fwd_workspace_bytes(int64_t channels, int64_t channel_size, int64_t width)
+{
+  return lbn_layer_norm_fwd_workspace_bytes(channels, channel_size, width, 4);
+}
+
 int lbn_instance_norm_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
                               int64_t width, float epsilon, const float* x, int64_t ldx, float* y,
-                              int64_t ldy, float* stats, int64_t ld_stats)
+                              int64_t ldy, float* stats, int64_t ld_stats, void* workspace,
+                              size_t workspace_bytes)
 {
   return ln_fwd<float>(as_stream(stream), channels, channel_size, channel_size, width, epsilon, x,
-                       ldx, y, ldy, stats, ld_stats, nullptr, nullptr, nullptr, 0, LBN_STATS_TWO_PASS);
+                       ldx, y, ldy, stats, ld_stats, nullptr, nullptr, workspace, workspace_bytes,
+                       LBN_STATS_TWO_PASS);
+}
+
+// The statistics gradients (2 * channels x width floats) come first; channels too long for
+// one workgroup add the cluster kernels' slots behind them, on a 256-byte boundary.
+static size_t in_sgrad_bytes(int64_t channels, int64_t width)
+{
+  return (static_cast<size_t>(2 * channels) * static_cast<size_t>(width) * sizeof(float) + 255) & ~size_t(255);
 }
 
 size_t lbn_instance_norm_bwd_workspace_bytes(int64_t channels, int64_t channel_size, int64_t width)
 {
   if (channels <= 0 || channel_size <= 0 || width <= 0) return 0;
-  return static_cast<size_t>(2 * channels) * static_cast<size_t>(width) * sizeof(float);
+  return in_sgrad_bytes(channels, width) + lbn_layer_norm_bwd_workspace_bytes(channels, channel_size, width, 0, 4);
 }
 
 int lbn_instance_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
@@ -1178,11 +1192,17 @@ int lbn_instance_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t cha
                               size_t workspace_bytes)
 {
   if (channels > 0 && channel_size > 0 && width > 0 &&
-      (!workspace || workspace_bytes < lbn_instance_norm_bwd_workspace_bytes(channels, channel_size, width)))
+      (!workspace || workspace_bytes < static_cast<size_t>(2 * channels) * static_cast<size_t>(width) * sizeof(float)))
     return LBN_ERR_WORKSPACE;
+  void* slots = nullptr;
+  size_t slot_bytes = 0;
+  if (channels > 0 && width > 0 && workspace_bytes > in_sgrad_bytes(channels, width)) {
+    slots = static_cast<char*>(workspace) + in_sgrad_bytes(channels, width);
+    slot_bytes = workspace_bytes - in_sgrad_bytes(channels, width);
+  }
   return ln_bwd<float>(as_stream(stream), channels, channel_size, channel_size, width, epsilon, x,
                        ldx, dy, lddy, dx, lddx, stats, ld_stats, static_cast<float*>(workspace),
-                       2 * channels, nullptr, nullptr, nullptr, nullptr, 0);
+                       2 * channels, nullptr, nullptr, nullptr, slots, slot_bytes);
 }
 
 }  // extern "C"

@@ -250,14 +250,17 @@ class instance_norm_layer(_Layer):
         self.num_channels = self.dims[0]
         self.channel_size = _prod(self.dims) // self.num_channels
         self.m_workspace = None  # (2*channels x width): means, then variances
+        self._ws_fwd = _Workspace()  # forward scratch of its own: backward's holds the statistics gradients
 
     def fp_call(self):
         x, y = self.prev_activations, self.activations
         if self.m_workspace is None or self.m_workspace.width != x.width:
             self.m_workspace = DeviceMatrix(2 * self.num_channels, x.width, device=self.device)
+        ws, nb = self._ws_fwd.get(capi.lib().lbn_instance_norm_fwd_workspace_bytes(
+            self.num_channels, self.channel_size, x.width), self.device)
         return ("lbn_instance_norm_fwd_f32",
                 (_stream(), self.num_channels, self.channel_size, x.width, self.m_epsilon, x.Buffer(),
-                 x.ldim, y.Buffer(), y.ldim, self.m_workspace.Buffer(), self.m_workspace.ldim))
+                 x.ldim, y.Buffer(), y.ldim, self.m_workspace.Buffer(), self.m_workspace.ldim, ws, nb))
 
     def bp_call(self):
         x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals

@@ -260,6 +260,8 @@ def test_layer_norm_f16(L, dims, start_dim, w, pad):
 
 # ===================================================================== instance norm
 @pytest.mark.parametrize("dims,w,pad", [((5, 3, 7), 15, 0), ((64, 56, 56), 6, 0), ((8, 1024), 33, 0),
+                                        ((2, 1048576), 2, 0), ((4, 96, 96, 96), 3, 0),   # volumes: clusters of workgroups per channel
+                                        ((3, 50000), 40, 4),
                                         ((3, 100000), 2, 0), ((7, 1), 5, 0), ((16, 31), 40, 4),
                                         ((256, 16, 16), 64, 0), ((3, 224, 224), 8, 0), ((2, 64, 64, 64), 2, 0),
                                         ((256, 7, 7), 32, 0), ((64, 3, 3), 9, 0), ((5, 4097), 6, 0),
