@@ -824,43 +824,48 @@ static bool bn_vec_ok(int64_t cs, int64_t w, const void* a, int64_t lda)
 
 // fp16 channels that are whole fours but not whole eights (196 = 14 x 14), or matrices aligned
 // to 8 but not 16 bytes: the same kernels with 8-byte accesses instead of the scalar walk.
-static bool bn_f16_in_fours(int64_t cs, int64_t w, std::initializer_list<std::pair<const void*, int64_t>> mats)
+// The same storage tag also carries the row-tile kernels (channels of any odd size on a matrix
+// whose rows come in aligned fours: 7 x 7 maps, single-entry channels).
+static bool bn_f16_in_fours(int64_t C, int64_t cs, int64_t w,
+                            std::initializer_list<std::pair<const void*, int64_t>> mats)
 {
-  bool eights = true, fours = true;
+  bool eights = true, fours = true, tiles = cs % 4 != 0 || cs <= 8;
   for (const auto& m : mats) {
     eights = eights && bn_vec_ok<__half>(cs, w, m.first, m.second);
     fours = fours && bn_vec_ok<f16x4>(cs, w, m.first, m.second);
+    tiles = tiles && row_quads_ok(C * cs, w, m.first, m.second, 2);
   }
-  return fours && !eights;
+  return !eights && (fours || tiles);
 }
 
 // ---- channels that are not whole 16-byte vectors, on a matrix whose row quads are aligned
-// (batch_norm_rows.hpp).  fp32 only.
+// (batch_norm_rows.hpp).  Storage types with four entries per access: float and f16x4.
+template <typename S>
 static bool bn_rt_usable(int64_t C, int64_t cs, int64_t w, const void* a, int64_t lda)
 {
-  return bn_rt_shape(cs) && row_quads_ok(C * cs, w, a, lda);
+  return bn_rt_shape(cs) && row_quads_ok(C * cs, w, a, lda, sizeof(S));
 }
 
-template <bool BWD>
-static void bn_rt_launch_sums(hipStream_t st, const RowTilePlan& p, const BnRtArgs& a)
+template <typename S, bool BWD>
+static void bn_rt_launch_sums(hipStream_t st, const RowTilePlan& p, const BnRtArgs<S>& a)
 {
   const dim3 grid(static_cast<unsigned>(p.tiles), static_cast<unsigned>(p.slabs));
-  if (p.gw == 1) hipLaunchKernelGGL((bn_rt_sums<1, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
-  else hipLaunchKernelGGL((bn_rt_sums<4, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
+  if (p.gw == 1) hipLaunchKernelGGL((bn_rt_sums<S, 1, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
+  else hipLaunchKernelGGL((bn_rt_sums<S, 4, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
 }
 
-template <bool BWD>
-static void bn_rt_launch_apply(hipStream_t st, const RowTilePlan& p, const BnRtArgs& a)
+template <typename S, bool BWD>
+static void bn_rt_launch_apply(hipStream_t st, const RowTilePlan& p, const BnRtArgs<S>& a)
 {
   const dim3 grid(static_cast<unsigned>(p.tiles), static_cast<unsigned>(p.slabs));
-  if (p.gw == 1) hipLaunchKernelGGL((bn_rt_apply<1, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
-  else hipLaunchKernelGGL((bn_rt_apply<4, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
+  if (p.gw == 1) hipLaunchKernelGGL((bn_rt_apply<S, 1, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
+  else hipLaunchKernelGGL((bn_rt_apply<S, 4, BWD>), grid, dim3(kRowTileThreads), 0, st, a);
 }
 
 // Register-resident row tiles (one kernel, one read) for mini-batches of at most 256 columns
 // whose channels fit a workgroup's rows; false: use the three-kernel row-tile path.
-template <bool BWD>
-static bool bn_rt_try_tile(hipStream_t st, BnRtTileArgs a)
+template <typename S, bool BWD>
+static bool bn_rt_try_tile(hipStream_t st, BnRtTileArgs<S> a)
 {
   int gw = 0, cpt = 0;
   if (a.w <= 256 && (a.rows_eff = bn_rt_tile_rows(a.cs, RowTilePos<4>::kRows)) > 0) {
@@ -878,8 +883,8 @@ static bool bn_rt_try_tile(hipStream_t st, BnRtTileArgs a)
   const dim3 grid(static_cast<unsigned>(ceil_div(a.h, a.rows_eff)));
 #define X(C, G)                                                                                         \
   if (cpt == C && gw == G) {                                                                            \
-    if (BWD) hipLaunchKernelGGL((bn_rt_bwd_tile<C, G>), grid, dim3(kRowTileThreads), 0, st, a);         \
-    else hipLaunchKernelGGL((bn_rt_fwd_tile<C, G>), grid, dim3(kRowTileThreads), 0, st, a);             \
+    if (BWD) hipLaunchKernelGGL((bn_rt_bwd_tile<S, C, G>), grid, dim3(kRowTileThreads), 0, st, a);         \
+    else hipLaunchKernelGGL((bn_rt_fwd_tile<S, C, G>), grid, dim3(kRowTileThreads), 0, st, a);             \
     return true;                                                                                        \
   }
   X(1, 4) X(2, 4) X(4, 4) X(8, 4) X(16, 4) X(1, 1) X(2, 1) X(4, 1) X(8, 1) X(16, 1)
@@ -898,13 +903,13 @@ static int bn_fwd_apply_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, f
   if (int e = bn_check(C, cs, w, lds, 2)) return e;
   if (C == 0 || cs == 0 || w == 0) return LBN_OK;
   if (!x || !y || !mean || !var || !scale || !bias) return LBN_ERR_INVALID_ARGUMENT;
-  if constexpr (std::is_same<S, float>::value) {
-    if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, y, ldy)) {
+  if constexpr (Vec16<S>::N == 4) {  // float or fp16 in fours: the row-tile kernels
+    if (bn_rt_usable<S>(C, cs, w, x, ldx) && bn_rt_usable<S>(C, cs, w, y, ldy)) {
       const RowTilePlan p = row_tile_plan(C * cs, w);
-      BnRtArgs a{};
+      BnRtArgs<S> a{};
       a.h = C * cs, a.w = w, a.cs = cs, a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy;
       a.slab_width = p.slab_width, a.eps = epsilon, a.mean = mean, a.var = var, a.scale = scale, a.bias = bias;
-      bn_rt_launch_apply<false>(st, p, a);
+      bn_rt_launch_apply<S, false>(st, p, a);
       return launch_status();
     }
   }
@@ -942,36 +947,36 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   const dim3 grid(static_cast<unsigned>(C), P);
   const int pivot = (flags & LBN_STATS_SUMSQ) ? 0 : 1;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, y, ldy);
-  if constexpr (std::is_same<S, float>::value) {
+  if constexpr (Vec16<S>::N == 4) {  // float or fp16 in fours: the row-tile kernels
     // channels of three or four vectors: the register tile when the mini-batch fits it
     // (1024 x 16, w = 256: 19 us per step against 25 us for clusters), else clusters
-    if (!bn_rt_shape(cs) && cs <= kBnTileMaxCs && row_quads_ok(C * cs, w, x, ldx) && row_quads_ok(C * cs, w, y, ldy)) {
-      BnRtTileArgs t{};
+    if (!bn_rt_shape(cs) && cs <= kBnTileMaxCs && row_quads_ok(C * cs, w, x, ldx, sizeof(S)) && row_quads_ok(C * cs, w, y, ldy, sizeof(S))) {
+      BnRtTileArgs<S> t{};
       t.h = C * cs, t.w = w, t.cs = cs, t.n = cs * w, t.x = x, t.out = y, t.ldx = ldx, t.ldo = ldy;
       t.use_pivot = pivot, t.bessel = bessel, t.eps = epsilon, t.decay = decay, t.mean = mean, t.var = var;
       t.scale = scale, t.bias = bias, t.rmean = running_mean, t.rvar = running_var;
-      if (bn_rt_try_tile<false>(st, t)) return launch_status();
+      if (bn_rt_try_tile<S, false>(st, t)) return launch_status();
     }
-    if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, y, ldy) &&
+    if (bn_rt_usable<S>(C, cs, w, x, ldx) && bn_rt_usable<S>(C, cs, w, y, ldy) &&
         (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0) {
       const int64_t h = C * cs;
       {
-        BnRtTileArgs t{};
+        BnRtTileArgs<S> t{};
         t.h = h, t.w = w, t.cs = cs, t.n = cs * w, t.x = x, t.out = y, t.ldx = ldx, t.ldo = ldy;
         t.use_pivot = pivot, t.bessel = bessel, t.eps = epsilon, t.decay = decay, t.mean = mean, t.var = var;
         t.scale = scale, t.bias = bias, t.rmean = running_mean, t.rvar = running_var;
-        if (bn_rt_try_tile<false>(st, t)) return launch_status();
+        if (bn_rt_try_tile<S, false>(st, t)) return launch_status();
       }
       const RowTilePlan p = row_tile_plan(h, w);
-      BnRtArgs a{};
+      BnRtArgs<S> a{};
       a.h = h, a.w = w, a.cs = cs, a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy;
       a.slab_width = p.slab_width, a.part = part, a.use_pivot = pivot, a.eps = epsilon;
       a.mean = mean, a.var = var, a.scale = scale, a.bias = bias;
-      bn_rt_launch_sums<false>(st, p, a);
-      hipLaunchKernelGGL(bn_rt_fwd_stats, dim3(static_cast<unsigned>(ceil_div(C, kRowTileWaves))),
+      bn_rt_launch_sums<S, false>(st, p, a);
+      hipLaunchKernelGGL(bn_rt_fwd_stats<S>, dim3(static_cast<unsigned>(ceil_div(C, kRowTileWaves))),
                          dim3(kRowTileThreads), 0, st, C, cs, w, h, p.slabs, part, x, pivot, bessel, epsilon,
                          decay, mean, var, running_mean, running_var);
-      bn_rt_launch_apply<false>(st, p, a);
+      bn_rt_launch_apply<S, false>(st, p, a);
       return launch_status();
     }
   }
@@ -1013,39 +1018,39 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   const dim3 grid(static_cast<unsigned>(C), P);
   const int64_t n = cs * w;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, dy, lddy) && bn_vec_ok<S>(cs, w, dx, lddx);
-  if constexpr (std::is_same<S, float>::value) {
-    if (!bn_rt_shape(cs) && cs <= kBnTileMaxCs && row_quads_ok(C * cs, w, x, ldx) && row_quads_ok(C * cs, w, dy, lddy) &&
-        row_quads_ok(C * cs, w, dx, lddx)) {
-      BnRtTileArgs t{};
+  if constexpr (Vec16<S>::N == 4) {  // float or fp16 in fours: the row-tile kernels
+    if (!bn_rt_shape(cs) && cs <= kBnTileMaxCs && row_quads_ok(C * cs, w, x, ldx, sizeof(S)) && row_quads_ok(C * cs, w, dy, lddy, sizeof(S)) &&
+        row_quads_ok(C * cs, w, dx, lddx, sizeof(S))) {
+      BnRtTileArgs<S> t{};
       t.h = C * cs, t.w = w, t.cs = cs, t.n = n, t.x = x, t.dy = dy, t.out = dx, t.ldx = ldx, t.lddy = lddy, t.ldo = lddx;
       t.bessel = bessel, t.training = training, t.eps = epsilon;
       t.mean = const_cast<float*>(use_mean), t.var = const_cast<float*>(use_var), t.scale = scale;
       t.dscale = dscale, t.dbias = dbias, t.dmean = dmean, t.dvar = dvar;
-      if (bn_rt_try_tile<true>(st, t)) return launch_status();
+      if (bn_rt_try_tile<S, true>(st, t)) return launch_status();
     }
-    if (bn_rt_usable(C, cs, w, x, ldx) && bn_rt_usable(C, cs, w, dy, lddy) && bn_rt_usable(C, cs, w, dx, lddx) &&
+    if (bn_rt_usable<S>(C, cs, w, x, ldx) && bn_rt_usable<S>(C, cs, w, dy, lddy) && bn_rt_usable<S>(C, cs, w, dx, lddx) &&
         (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0) {
       const int64_t h = C * cs;
       {
-        BnRtTileArgs t{};
+        BnRtTileArgs<S> t{};
         t.h = h, t.w = w, t.cs = cs, t.n = n, t.x = x, t.dy = dy, t.out = dx, t.ldx = ldx, t.lddy = lddy, t.ldo = lddx;
         t.bessel = bessel, t.training = training, t.eps = epsilon;
         t.mean = const_cast<float*>(use_mean), t.var = const_cast<float*>(use_var), t.scale = scale;
         t.dscale = dscale, t.dbias = dbias, t.dmean = dmean, t.dvar = dvar;
-        if (bn_rt_try_tile<true>(st, t)) return launch_status();
+        if (bn_rt_try_tile<S, true>(st, t)) return launch_status();
       }
       const RowTilePlan p = row_tile_plan(h, w);
-      BnRtArgs a{};
+      BnRtArgs<S> a{};
       a.h = h, a.w = w, a.cs = cs, a.x = x, a.dy = dy, a.out = dx, a.ldx = ldx, a.lddy = lddy, a.ldo = lddx;
       a.slab_width = p.slab_width, a.part = part, a.eps = epsilon;
       a.mean = use_mean, a.var = use_var, a.scale = scale, a.dmean = dmean, a.dvar = dvar;
       a.count = static_cast<float>(n), a.count_bessel = static_cast<float>(n - (bessel ? 1 : 0));
       a.zero = n <= 1;
-      bn_rt_launch_sums<true>(st, p, a);
+      bn_rt_launch_sums<S, true>(st, p, a);
       hipLaunchKernelGGL(bn_rt_bwd_stats, dim3(static_cast<unsigned>(ceil_div(C, kRowTileWaves))),
                          dim3(kRowTileThreads), 0, st, C, cs, h, p.slabs, part, epsilon, training, use_var, scale,
                          dscale, dbias, dmean, dvar);
-      bn_rt_launch_apply<true>(st, p, a);
+      bn_rt_launch_apply<S, true>(st, p, a);
       return launch_status();
     }
   }
@@ -1138,7 +1143,7 @@ int lbn_batch_norm_fwd_f16(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
                            const float* bias, float* running_mean, float* running_var,
                            void* workspace, size_t workspace_bytes, int flags)
 {
-  if (C > 0 && cs > 0 && w > 0 && bn_f16_in_fours(cs, w, {{x, ldx}, {y, ldy}}))
+  if (C > 0 && cs > 0 && w > 0 && bn_f16_in_fours(C, cs, w, {{x, ldx}, {y, ldy}}))
     return bn_fwd_host<f16x4>(as_stream(stream), C, cs, w, bessel, epsilon, decay, training,
                               static_cast<const f16x4*>(x), ldx, static_cast<f16x4*>(y), ldy, mean, var,
                               scale, bias, running_mean, running_var, workspace, workspace_bytes, flags);
@@ -1218,7 +1223,7 @@ int lbn_batch_norm_bwd_f16(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
                            float* dscale, float* dbias, float* dmean, float* dvar, void* workspace,
                            size_t workspace_bytes)
 {
-  if (C > 0 && cs > 0 && w > 0 && bn_f16_in_fours(cs, w, {{x, ldx}, {dy, lddy}, {dx, lddx}}))
+  if (C > 0 && cs > 0 && w > 0 && bn_f16_in_fours(C, cs, w, {{x, ldx}, {dy, lddy}, {dx, lddx}}))
     return bn_bwd_host<f16x4>(as_stream(stream), C, cs, w, bessel, epsilon, training,
                               static_cast<const f16x4*>(x), ldx, static_cast<const f16x4*>(dy), lddy,
                               static_cast<f16x4*>(dx), lddx, mean, var, running_mean, running_var, scale,

@@ -1,5 +1,5 @@
 // Batch norm for channels that are not a whole number of 16-byte vectors (channel_size
-// 1 after a fully-connected layer, 49 for 7 x 7 feature maps, ...), fp32.  The kernels of
+// 1 after a fully-connected layer, 49 for 7 x 7 feature maps, ...), fp32 or fp16 storage.  The kernels of
 // batch_norm.hip walk a channel's segments, which then start at odd offsets and, for tiny
 // channels, are a few bytes per column; here lanes run along consecutive matrix ROWS
 // instead (row_tiles.hpp), whatever channel a row belongs to:
@@ -21,11 +21,13 @@
 
 namespace lbn {
 
+// S: storage type with four entries per access (float: 16 bytes; f16x4: 8 bytes of fp16).
+template <typename S>
 struct BnRtArgs {
   int64_t h, w, cs;
-  const float* x;
-  const float* dy;
-  float* out;  // y or dx
+  const S* x;
+  const S* dy;
+  S* out;  // y or dx
   int64_t ldx, lddy, ldo;
   int64_t slab_width;
   float2* part;  // [slabs][h]
@@ -45,9 +47,9 @@ struct BnRtArgs {
 // Forward: (s, q) = sums of (x - K) and (x - K)^2 with K the first entry of the row's
 // channel (0 for the reference's E[x^2] - mean^2 formula).  Backward: (A, B) = sums of dy
 // and dy * (x - mean).
-template <int GW, bool BWD>
+template <typename S, int GW, bool BWD>
 __global__ void __launch_bounds__(kRowTileThreads)
-bn_rt_sums(BnRtArgs a)
+bn_rt_sums(BnRtArgs<S> a)
 {
   using P = RowTilePos<GW>;
   __shared__ float lds[kRowTileWaves][P::kRows][2];
@@ -61,7 +63,7 @@ bn_rt_sums(BnRtArgs a)
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int64_t ch = (rr + r) / a.cs;
-    K[r] = BWD ? a.mean[ch] : (a.use_pivot ? a.x[ch * a.cs] : 0.f);
+    K[r] = BWD ? a.mean[ch] : (a.use_pivot ? Vec16<S>::load1(a.x + ch * a.cs) : 0.f);
   }
   float sa[4] = {0.f, 0.f, 0.f, 0.f}, sb[4] = {0.f, 0.f, 0.f, 0.f};
   auto add = [&](const float (&v)[4], const float (&g)[4]) {
@@ -83,16 +85,16 @@ bn_rt_sums(BnRtArgs a)
     float v[2][4], g[2][4];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      Vec16<float>::load(a.x + rr + (c + j * P::kGroups) * a.ldx, v[j]);
-      if (BWD) Vec16<float>::load(a.dy + rr + (c + j * P::kGroups) * a.lddy, g[j]);
+      Vec16<S>::load(a.x + rr + (c + j * P::kGroups) * a.ldx, v[j]);
+      if (BWD) Vec16<S>::load(a.dy + rr + (c + j * P::kGroups) * a.lddy, g[j]);
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) add(v[j], g[j]);
   }
   for (; c < c1; c += P::kGroups) {
     float v[4], g[4];
-    Vec16<float>::load(a.x + rr + c * a.ldx, v);
-    if (BWD) Vec16<float>::load(a.dy + rr + c * a.lddy, g);
+    Vec16<S>::load(a.x + rr + c * a.ldx, v);
+    if (BWD) Vec16<S>::load(a.dy + rr + c * a.lddy, g);
     add(v, g);
   }
   row_tile_merge<GW>(sa, sb, lds, p);
@@ -121,9 +123,10 @@ __device__ __forceinline__ float2 bn_rt_channel_total(const float2* part, int64_
 }
 
 // One wave per channel (4 channels per workgroup).
+template <typename S>
 __global__ void __launch_bounds__(kRowTileThreads)
 bn_rt_fwd_stats(int64_t C, int64_t cs, int64_t w, int64_t h, int slabs, const float2* __restrict__ part,
-                const float* __restrict__ x, int use_pivot, int bessel, float eps, float decay,
+                const S* __restrict__ x, int use_pivot, int bessel, float eps, float decay,
                 float* __restrict__ mean, float* __restrict__ var, float* __restrict__ rmean,
                 float* __restrict__ rvar)
 {
@@ -133,11 +136,11 @@ bn_rt_fwd_stats(int64_t C, int64_t cs, int64_t w, int64_t h, int slabs, const fl
   if ((threadIdx.x & (kWave - 1)) != 0) return;
   const int64_t n = cs * w;
   if (n <= 1) {  // batch_normalization.cpp:118-120: the mean holds x, the variance is 1
-    mean[c] = x[c * cs];
+    mean[c] = Vec16<S>::load1(x + c * cs);
     var[c] = 1.f;
     return;
   }
-  const float K = use_pivot ? x[c * cs] : 0.f;
+  const float K = use_pivot ? Vec16<S>::load1(x + c * cs) : 0.f;
   float m, v;
   stats_from_sums(t.x, t.y, K, n, bessel, eps, m, v);
   mean[c] = m;
@@ -167,9 +170,9 @@ bn_rt_bwd_stats(int64_t C, int64_t cs, int64_t h, int slabs, const float2* __res
 
 // Forward: y = scale * ((x - mean) * inv_stdev) + bias.
 // Backward: dx = dy * scale * inv_stdev + dmean / n + dvar * 2 / (n - bessel) * (x - mean).
-template <int GW, bool BWD>
+template <typename S, int GW, bool BWD>
 __global__ void __launch_bounds__(kRowTileThreads)
-bn_rt_apply(BnRtArgs a)
+bn_rt_apply(BnRtArgs<S> a)
 {
   using P = RowTilePos<GW>;
   const P p;
@@ -206,21 +209,21 @@ bn_rt_apply(BnRtArgs a)
     float v[2][4], g[2][4];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      Vec16<float>::load(a.x + r0 + (c + j * P::kGroups) * a.ldx, v[j]);
-      if (BWD) Vec16<float>::load(a.dy + r0 + (c + j * P::kGroups) * a.lddy, g[j]);
+      Vec16<S>::load(a.x + r0 + (c + j * P::kGroups) * a.ldx, v[j]);
+      if (BWD) Vec16<S>::load(a.dy + r0 + (c + j * P::kGroups) * a.lddy, g[j]);
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       finish(v[j], g[j]);
-      Vec16<float>::store(a.out + r0 + (c + j * P::kGroups) * a.ldo, v[j]);
+      Vec16<S>::store(a.out + r0 + (c + j * P::kGroups) * a.ldo, v[j]);
     }
   }
   for (; c < c1; c += P::kGroups) {
     float v[4], g[4];
-    Vec16<float>::load(a.x + r0 + c * a.ldx, v);
-    if (BWD) Vec16<float>::load(a.dy + r0 + c * a.lddy, g);
+    Vec16<S>::load(a.x + r0 + c * a.ldx, v);
+    if (BWD) Vec16<S>::load(a.dy + r0 + c * a.lddy, g);
     finish(v, g);
-    Vec16<float>::store(a.out + r0 + c * a.ldo, v);
+    Vec16<S>::store(a.out + r0 + c * a.ldo, v);
   }
 }
 
@@ -232,12 +235,13 @@ bn_rt_apply(BnRtArgs a)
 // Per-row pairs are merged over the column groups in LDS, one thread per channel adds its
 // cs rows and finishes the channel, and the output is written from registers: one kernel,
 // x (and dy) read once.
+template <typename S>
 struct BnRtTileArgs {
   int64_t h, w, cs, n;  // n = cs * w
   int rows_eff;         // rows per workgroup: a multiple of cs and of 4
-  const float* x;
-  const float* dy;
-  float* out;
+  const S* x;
+  const S* dy;
+  S* out;
   int64_t ldx, lddy, ldo;
   int use_pivot, bessel, training;
   float eps, decay;
@@ -299,9 +303,9 @@ __device__ __forceinline__ void bn_rt_tile_channel_totals(float (&a)[4], float (
   __syncthreads();
 }
 
-template <int CPT, int GW>
+template <typename S, int CPT, int GW>
 __global__ void __launch_bounds__(kRowTileThreads)
-bn_rt_fwd_tile(BnRtTileArgs a)
+bn_rt_fwd_tile(BnRtTileArgs<S> a)
 {
   using P = RowTilePos<GW>;
   __shared__ float lds[kRowTileWaves][P::kRows][2];
@@ -317,13 +321,13 @@ bn_rt_fwd_tile(BnRtTileArgs a)
 
   float K[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) K[r] = a.use_pivot ? a.x[((r0 + r) / cs) * cs] : 0.f;
+  for (int r = 0; r < 4; ++r) K[r] = a.use_pivot ? Vec16<S>::load1(a.x + ((r0 + r) / cs) * cs) : 0.f;
   float v[CPT][4];
 #pragma unroll
   for (int j = 0; j < CPT; ++j) {
     const int64_t c = p.g + P::kGroups * j;
     if (row_ok && c < a.w) {
-      Vec16<float>::load(a.x + r0 + c * a.ldx, v[j]);
+      Vec16<S>::load(a.x + r0 + c * a.ldx, v[j]);
     }
     else {
 #pragma unroll
@@ -345,11 +349,11 @@ bn_rt_fwd_tile(BnRtTileArgs a)
     const int64_t ch = base / cs + threadIdx.x;
     float m, var;
     if (a.n <= 1) {  // batch_normalization.cpp:118-120
-      m = a.x[ch * cs];
+      m = Vec16<S>::load1(a.x + ch * cs);
       var = 1.f;
     }
     else {
-      const float Kc = a.use_pivot ? a.x[ch * cs] : 0.f;
+      const float Kc = a.use_pivot ? Vec16<S>::load1(a.x + ch * cs) : 0.f;
       stats_from_sums(chan[threadIdx.x][0], chan[threadIdx.x][1], Kc, a.n, a.bessel, a.eps, m, var);
       a.rmean[ch] = a.decay * a.rmean[ch] + (1.f - a.decay) * m;
       a.rvar[ch] = a.decay * a.rvar[ch] + (1.f - a.decay) * var;
@@ -376,14 +380,14 @@ bn_rt_fwd_tile(BnRtTileArgs a)
     if (c < a.w) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) v[j][r] = sc[r] * ((v[j][r] - mean[r]) * inv[r]) + bi[r];
-      Vec16<float>::store(a.out + r0 + c * a.ldo, v[j]);
+      Vec16<S>::store(a.out + r0 + c * a.ldo, v[j]);
     }
   }
 }
 
-template <int CPT, int GW>
+template <typename S, int CPT, int GW>
 __global__ void __launch_bounds__(kRowTileThreads)
-bn_rt_bwd_tile(BnRtTileArgs a)
+bn_rt_bwd_tile(BnRtTileArgs<S> a)
 {
   using P = RowTilePos<GW>;
   __shared__ float lds[kRowTileWaves][P::kRows][2];
@@ -409,8 +413,8 @@ bn_rt_bwd_tile(BnRtTileArgs a)
   for (int j = 0; j < CPT; ++j) {
     const int64_t c = p.g + P::kGroups * j;
     if (row_ok && c < a.w) {
-      Vec16<float>::load(a.x + r0 + c * a.ldx, xc[j]);
-      Vec16<float>::load(a.dy + r0 + c * a.lddy, g[j]);
+      Vec16<S>::load(a.x + r0 + c * a.ldx, xc[j]);
+      Vec16<S>::load(a.dy + r0 + c * a.lddy, g[j]);
 #pragma unroll
       for (int r = 0; r < 4; ++r) xc[j][r] -= mean[r];
     }
@@ -457,7 +461,7 @@ bn_rt_bwd_tile(BnRtTileArgs a)
     if (c < a.w) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) g[j][r] = zero ? 0.f : g[j][r] * k0[r] + k1[r] + k2[r] * xc[j][r];
-      Vec16<float>::store(a.out + r0 + c * a.ldo, g[j]);
+      Vec16<S>::store(a.out + r0 + c * a.ldo, g[j]);
     }
   }
 }

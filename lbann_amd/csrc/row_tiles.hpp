@@ -101,10 +101,10 @@ inline RowTilePlan row_tile_plan(int64_t h, int64_t w)
   return p;
 }
 
-// 16-byte row quads need h % 4 == 0 and every column start aligned.
-inline bool row_quads_ok(int64_t h, int64_t w, const void* p, int64_t ld)
+// Row quads (16 bytes of fp32, 8 bytes of fp16) need h % 4 == 0 and every column start aligned.
+inline bool row_quads_ok(int64_t h, int64_t w, const void* p, int64_t ld, int elem_bytes = 4)
 {
-  return h % 4 == 0 && aligned16(p) && (w <= 1 || ld % 4 == 0);
+  return h % 4 == 0 && reinterpret_cast<uintptr_t>(p) % (4 * elem_bytes) == 0 && (w <= 1 || ld % 4 == 0);
 }
 
 }  // namespace lbn

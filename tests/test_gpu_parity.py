@@ -384,7 +384,11 @@ def test_batch_norm(L, dims, w, bessel, pad):
     ((2, 100000), 3, True, 0, True), ((64, 56, 56), 16, True, 0, True),
     # channels of whole fours but not eights, or a leading dimension padded by four: 8-byte accesses
     ((1024, 14, 14), 32, True, 0, True), ((256, 14, 14), 600, False, 0, True), ((6, 10, 10), 9, True, 0, False),
-    ((16, 28, 28), 8, True, 4, True), ((40, 12), 64, True, 0, True), ((3, 4), 5, True, 4, True)])
+    ((16, 28, 28), 8, True, 4, True), ((40, 12), 64, True, 0, True), ((3, 4), 5, True, 4, True),
+    # channels of odd sizes on matrices whose rows come in aligned fours: the row-tile kernels on fp16
+    ((2048, 7, 7), 16, True, 0, True), ((4096,), 64, True, 0, True), ((64, 7, 7), 300, False, 0, True),
+    ((12, 3, 3), 20, True, 0, True), ((1024, 1), 2048, True, 0, True), ((128, 7, 7), 10, True, 0, False),
+    ((32, 7, 7), 64, True, 4, True), ((2000, 2), 200, False, 0, True), ((100, 12), 64, True, 0, True)])
 def test_batch_norm_f16(L, dims, w, bessel, pad, training):
     """fp16 storage, fp32 arithmetic: the oracle sees the fp16-rounded inputs."""
     rng = np.random.default_rng(int(np.prod(dims)) * 5 + w)

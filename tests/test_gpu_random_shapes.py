@@ -264,13 +264,17 @@ def test_small_channels_random(L, case):
     h = C * cs
     pad = int(rng.choice([0, 0, 0, 4, 2]))
     bessel = bool(case % 2)
-    tag = f"C={C} cs={cs} w={w} pad={pad}"
+    half = bool(case % 3 == 2)   # fp16 storage: the same kernels with 8-byte row quads
+    tag = f"C={C} cs={cs} w={w} pad={pad} half={half}"
     x, dy = rand(rng, h, w, 2.0, 3.0), rand(rng, h, w)
+    if half:
+        x, dy = x.astype(np.float16).astype(np.float32), dy.astype(np.float16).astype(np.float32)
     g = rng.uniform(0.5, 1.5, C).astype(np.float32)
     b = (0.1 * rng.standard_normal(C)).astype(np.float32)
     bn = L.batch_normalization_layer((C, cs), 0.9, 1e-5, bessel, g, b)
-    y = bn.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
-    dx = bn.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    tdt = torch.float16 if half else torch.float32
+    y = bn.forward(L.DeviceMatrix.from_numpy(x, dtype=tdt, ldim=h + pad)).to_numpy()
+    dx = bn.backward(L.DeviceMatrix.from_numpy(dy, dtype=tdt, ldim=h + pad)).to_numpy()
     mv = bn.m_mean_and_var.to_numpy()
     ref, ex = {}, {}
     for dst, conv in ((ref, f32), (ex, f64)):
@@ -287,7 +291,7 @@ def test_small_channels_random(L, case):
         for k in ("dmean", "dvar", "dscale", "dbias"):
             got.pop(k)
     for k in got:
-        check(f"batch norm {k} {tag}", got[k], ref[k], ex[k])
+        check(f"batch norm {k} {tag}", got[k], ref[k], ex[k], tol=TOL_F16 if half and k in ("y", "dx") else TOL_F32)
     wts = np.asfortranarray(np.stack([g, b], axis=1))
     sb = L.channelwise_scale_bias_layer((C, cs))
     sb.set_weights(g, b)
