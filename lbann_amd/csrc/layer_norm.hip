@@ -702,7 +702,7 @@ static size_t ln_cluster_fwd_workspace(int64_t n, int64_t rows, int ve)
 {
   if (n % ve != 0) return 0;
   const ClusterPlan cp = plan_ln_cluster(n / ve, kLnClFwdUnits / (kLnClThreads * ve));
-  return cp.M ? ln_cluster_slot_bytes(rows, cp.M) : 0;
+  return cp.M ? ln_cluster_slot_bytes(rows, kLnClMaxM) : 0;  // a launch may widen its clusters up to the maximum
 }
 
 static size_t ln_cluster_bwd_workspace(int64_t n, int64_t rows, int ve)
@@ -710,7 +710,7 @@ static size_t ln_cluster_bwd_workspace(int64_t n, int64_t rows, int ve)
   if (n % ve != 0) return 0;
   const ClusterPlan cp = plan_ln_cluster(n / ve, kLnClBwdUnits / (kLnClThreads * ve));
   if (!cp.M) return 0;
-  return ln_cluster_part_offset(rows, cp.M) +
+  return ln_cluster_part_offset(rows, kLnClMaxM) +
          static_cast<size_t>(ln_cluster_count_bound(rows, cp.M)) * 2 * n * sizeof(float);
 }
 
@@ -787,22 +787,21 @@ static int ln_fwd_cluster_launch(hipStream_t st, const T* x, T* y, int64_t ldx, 
   constexpr int VE = Vec16<T>::N;
   constexpr int kMaxV = kLnClFwdUnits / (kLnClThreads * VE);
   const ClusterPlan cp = plan_ln_cluster(n / VE, kMaxV);
-  if (!cp.M || !ws || !aligned16(ws) || ws_bytes < ln_cluster_slot_bytes(rows, cp.M)) return 0;
+  if (!cp.M || !ws || !aligned16(ws)) return 0;
   const ClusterWorkspace cw = cluster_workspace(ws);
   const bool affine = gamma || beta;
 #define X(VV)                                                                                        \
   if (cp.V == VV) {                                                                                  \
     const int cap = affine ? cluster_capacity(ln_fwd_cluster<T, VV, true>, kLnClThreads)             \
                            : cluster_capacity(ln_fwd_cluster<T, VV, false>, kLnClThreads);           \
-    int64_t nc = cap / cp.M < rows ? cap / cp.M : rows;                                              \
-    if (nc < 1) return 0;                                                                            \
-    nc = ceil_div(rows, ceil_div(rows, nc)); /* every cluster walks the same number of rows */       \
+    const LnClusterLaunch l = plan_ln_cluster_launch(n / VE, rows, cp, cap, rows);                   \
+    if (!l.M || l.V > VV || ws_bytes < ln_cluster_slot_bytes(rows, l.M)) return 0;                   \
     LnClArgs<T> a{};                                                                                 \
     a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy, a.map = map, a.rows = rows, a.n = n;               \
-    a.nvec = static_cast<unsigned>(n / VE), a.M = cp.M, a.sumsq = sumsq;                             \
+    a.nvec = static_cast<unsigned>(n / VE), a.per_wg = l.per_wg, a.M = l.M, a.sumsq = sumsq;         \
     a.inv_n = 1.0f / static_cast<float>(n), a.eps = eps, a.stats = stats, a.ld_stats = lds;          \
     a.gamma = gamma, a.beta = beta, a.cw = cw, a.tag = cluster_call_tag(st, cw);                     \
-    const dim3 grid(static_cast<unsigned>(nc * cp.M));                                               \
+    const dim3 grid(static_cast<unsigned>(l.clusters * l.M));                                        \
     if (affine) hipLaunchKernelGGL((ln_fwd_cluster<T, VV, true>), grid, dim3(kLnClThreads), 0, st, a); \
     else hipLaunchKernelGGL((ln_fwd_cluster<T, VV, false>), grid, dim3(kLnClThreads), 0, st, a);     \
     return 1;                                                                                        \
@@ -823,26 +822,24 @@ static int ln_bwd_cluster_launch(hipStream_t st, bool wgrad, const T* x, const T
   constexpr int kMaxV = kLnClBwdUnits / (kLnClThreads * VE);
   const ClusterPlan cp = plan_ln_cluster(n / VE, kMaxV);
   if (!cp.M || !ws || !aligned16(ws)) return 0;
-  const size_t need = wgrad ? ln_cluster_bwd_workspace(n, rows, VE) : ln_cluster_slot_bytes(rows, cp.M);
+  const size_t need = wgrad ? ln_cluster_bwd_workspace(n, rows, VE) : ln_cluster_slot_bytes(rows, kLnClMaxM);
   if (ws_bytes < need) return 0;
   const ClusterWorkspace cw = cluster_workspace(ws);
-  float* wpart = reinterpret_cast<float*>(static_cast<char*>(ws) + ln_cluster_part_offset(rows, cp.M));
+  float* wpart = reinterpret_cast<float*>(static_cast<char*>(ws) + ln_cluster_part_offset(rows, kLnClMaxM));
 #define X(VV)                                                                                        \
   if (cp.V == VV) {                                                                                  \
     const int cap = wgrad ? cluster_capacity(ln_bwd_cluster<T, VV, true>, kLnClThreads)              \
                           : cluster_capacity(ln_bwd_cluster<T, VV, false>, kLnClThreads);            \
-    int64_t nc = cap / cp.M;                                                                         \
-    const int64_t bound = ln_cluster_count_bound(rows, cp.M);                                        \
-    if (nc > bound) nc = bound;                                                                      \
-    if (nc < 1) return 0;                                                                            \
-    nc = ceil_div(rows, ceil_div(rows, nc));                                                         \
+    const LnClusterLaunch l = plan_ln_cluster_launch(n / VE, rows, cp, cap, ln_cluster_count_bound(rows, cp.M)); \
+    if (!l.M || l.V > VV) return 0;                                                                  \
+    const int64_t nc = l.clusters;                                                                   \
     LnClArgs<T> a{};                                                                                 \
     a.x = x, a.dy = dy, a.out = dx, a.ldx = ldx, a.lddy = lddy, a.ldo = lddx, a.map = map;           \
-    a.rows = rows, a.n = n, a.nvec = static_cast<unsigned>(n / VE), a.M = cp.M;                      \
+    a.rows = rows, a.n = n, a.nvec = static_cast<unsigned>(n / VE), a.per_wg = l.per_wg, a.M = l.M;  \
     a.inv_n = 1.0f / static_cast<float>(n), a.eps = eps, a.stats = const_cast<float*>(stats);        \
     a.ld_stats = lds, a.sgrad = sgrad, a.ld_sgrad = ldsg, a.gamma = gamma, a.wpart = wpart;          \
     a.cw = cw, a.tag = cluster_call_tag(st, cw);                                                     \
-    const dim3 grid(static_cast<unsigned>(nc * cp.M));                                               \
+    const dim3 grid(static_cast<unsigned>(nc * l.M));                                                \
     if (wgrad) {                                                                                     \
       hipLaunchKernelGGL((ln_bwd_cluster<T, VV, true>), grid, dim3(kLnClThreads), 0, st, a);         \
       hipLaunchKernelGGL(ln_wgrad_reduce_wide, dim3(static_cast<unsigned>(ceil_div(n / 2, 256))), dim3(256), 0, \
@@ -1126,7 +1123,7 @@ size_t lbn_layer_norm_bwd_workspace_bytes(int64_t num_groups, int64_t norm_size,
   // without weight gradients only the cluster kernels of long rows use scratch (their slots)
   if (norm_size % ve != 0 || plan_ln_bwd(norm_size / ve, rows, ve, elem_bytes == 2 ? 2 : 4).tpr) return 0;
   const ClusterPlan cp = plan_ln_cluster(norm_size / ve, kLnClBwdUnits / (kLnClThreads * ve));
-  return cp.M ? ln_cluster_slot_bytes(rows, cp.M) : 0;
+  return cp.M ? ln_cluster_slot_bytes(rows, kLnClMaxM) : 0;
 }
 
 int lbn_layer_norm_bwd_f32(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,

@@ -43,6 +43,7 @@ struct LnClArgs {
   int64_t rows;
   int64_t n;
   unsigned nvec;
+  unsigned per_wg;  // vectors per workgroup: workgroup k owns [k * per_wg, (k + 1) * per_wg) of a row
   int M, sumsq;
   float inv_n, eps;
   float* stats;  // forward: written; backward: read
@@ -233,9 +234,13 @@ ln_fwd_cluster(LnClArgs<T> a)
   const int64_t nc = gridDim.x / a.M;
   const int64_t cl = blockIdx.x / a.M;
   const int k = blockIdx.x - static_cast<int>(cl) * a.M;
-  const unsigned base = static_cast<unsigned>(k) * (kLnClThreads * V) + threadIdx.x;
+  const unsigned base = static_cast<unsigned>(k) * a.per_wg + threadIdx.x;
   if (cl >= a.rows) return;
   cluster_resolve_tag(a.tag);
+  {  // from here on `nvec` is the end of this workgroup's share
+    const unsigned end = (static_cast<unsigned>(k) + 1) * a.per_wg;
+    if (end < a.nvec) a.nvec = end;
+  }
   if (AFFINE) {  // read back by the same thread only: no barrier needed
     ln_cl_stage_weights<T, V>(a.gamma, 1.f, base, a.nvec, wts);
     ln_cl_stage_weights<T, V>(a.beta, 0.f, base, a.nvec, wts + kLnClThreads * V * Vec16<T>::N);
@@ -390,9 +395,13 @@ ln_bwd_cluster(LnClArgs<T> a)
   const int64_t nc = gridDim.x / a.M;
   const int64_t cl = blockIdx.x / a.M;
   const int k = blockIdx.x - static_cast<int>(cl) * a.M;
-  const unsigned base = static_cast<unsigned>(k) * (kLnClThreads * V) + threadIdx.x;
+  const unsigned base = static_cast<unsigned>(k) * a.per_wg + threadIdx.x;
   if (cl >= a.rows) return;
   cluster_resolve_tag(a.tag);
+  {  // from here on `nvec` is the end of this workgroup's share
+    const unsigned end = (static_cast<unsigned>(k) + 1) * a.per_wg;
+    if (end < a.nvec) a.nvec = end;
+  }
   if (WGRAD) {
     for (int p = threadIdx.x; p < 2 * kLnClBwdUnits; p += kLnClThreads) acc[p] = 0.f;  // each thread clears its own cells
   }
@@ -457,13 +466,45 @@ ln_wgrad_reduce_wide(const float* __restrict__ part, int64_t P, int64_t n, float
 }
 
 // ------------------------------------------------------------------------ host side
-// Cluster shape for rows of nvec vectors with at most max_v vectors per thread.
+// Cluster shape for rows of nvec vectors with at most max_v vectors per thread: the fewest
+// workgroups per row that hold it (what the workspace query plans with).
 inline ClusterPlan plan_ln_cluster(int64_t nvec, int max_v)
 {
   const int64_t per = kLnClThreads;
   const int64_t M = (nvec + per * max_v - 1) / (per * max_v);
   if (M < 1 || M > kLnClMaxM) return {0, 0};
   return {static_cast<int>((nvec + per * M - 1) / (per * M)), static_cast<int>(M)};
+}
+
+// What a launch uses on a device that holds `cap` workgroups: as many clusters as the
+// minimal shape allows, then the workgroups that would stay idle are given to the clusters
+// (a row of 98 shares on 256 compute units runs as 2 clusters of 128 instead of 2 of 98).
+struct LnClusterLaunch {
+  int M, V;
+  int64_t clusters;
+  unsigned per_wg;
+};
+
+inline LnClusterLaunch plan_ln_cluster_launch(int64_t nvec, int64_t rows, ClusterPlan min_plan, int64_t cap,
+                                              int64_t max_clusters)
+{
+  LnClusterLaunch l{0, 0, 0, 0};
+  if (!min_plan.M) return l;
+  int64_t nc = cap / min_plan.M;
+  if (nc > rows) nc = rows;
+  if (nc > max_clusters) nc = max_clusters;
+  if (nc < 1) return l;
+  nc = (rows + (rows + nc - 1) / nc - 1) / ((rows + nc - 1) / nc);  // every cluster walks the same number of rows
+  int64_t M = cap / nc;
+  if (M > kLnClMaxM) M = kLnClMaxM;
+  if (M < min_plan.M) M = min_plan.M;
+  const int64_t per_wg = (nvec + M - 1) / M;
+  M = (nvec + per_wg - 1) / per_wg;  // drop workgroups that would own nothing
+  l.M = static_cast<int>(M);
+  l.V = static_cast<int>((per_wg + kLnClThreads - 1) / kLnClThreads);
+  l.clusters = nc;
+  l.per_wg = static_cast<unsigned>(per_wg);
+  return l;
 }
 
 // Clusters a launch may use: bounded by what the workspace query assumes (it cannot ask the
