@@ -458,9 +458,7 @@ __device__ __forceinline__ void bn_fwd_finish(const BnFwdArgs<S>& a, const BnInd
   const unsigned tid = threadIdx.x;
   if (tid < kWave) {
     float ts, tq;
-    cluster_collect(a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, a.M, a.tag, a.cw.error, 0.f, 0.f, ts, tq);
-    ts = wave_sum(ts);
-    tq = wave_sum(tq);
+    cluster_collect_sums(a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, a.M, a.tag, a.cw.error, ts, tq);
     if (tid == 0) {
       float mean, var;
       stats_from_sums(ts, tq, t.K, a.n, a.bessel, a.eps, mean, var);
@@ -598,9 +596,7 @@ __device__ __forceinline__ void bn_bwd_finish(const BnBwdArgs<S>& a, const BnInd
   const float scale = t.scale;
   if (tid < kWave) {
     float ta, tb;
-    cluster_collect(a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, a.M, a.tag, a.cw.error, 0.f, 0.f, ta, tb);
-    ta = wave_sum(ta);
-    tb = wave_sum(tb);
+    cluster_collect_sums(a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, a.M, a.tag, a.cw.error, ta, tb);
     if (tid == 0) {
       float ds, db, dmean, dvar;
       grads_from_sums(ta, tb, scale, inv_stdev, ds, db, dmean, dvar);
@@ -683,12 +679,12 @@ static BnClusterShape bn_cluster_shape(int64_t E, int max_v, int first_t)
   static const int force_t = std::getenv("LBN_BN_CLUSTER_T") ? std::atoi(std::getenv("LBN_BN_CLUSTER_T")) : 0;
   if (!force_t) {
     for (int T = 512; T >= first_t; T /= 2) {
-      const ClusterPlan p = plan_cluster(E, max_v, T);
+      const ClusterPlan p = plan_cluster(E, max_v, T, kClusterMaxSumM);
       if (p.M >= 8) return {T, p.V, p.M};
     }
   }
   for (int T = force_t ? force_t : first_t; T <= 1024; T *= 2) {
-    const ClusterPlan p = plan_cluster(E, max_v, T);
+    const ClusterPlan p = plan_cluster(E, max_v, T, kClusterMaxSumM);
     if (p.M) return {T, p.V, p.M};
     if (force_t) break;
   }
@@ -718,7 +714,7 @@ static size_t bn_workspace(int64_t C, int64_t cs, int64_t w)
 {
   if (C <= 0 || cs <= 0 || w <= 0) return 0;
   const size_t split = static_cast<size_t>(C) * bn_split(C, cs, w) * sizeof(float2);
-  const size_t cluster = cluster_workspace_bytes(C);
+  const size_t cluster = cluster_workspace_bytes(C, kClusterMaxSumM);
   size_t need = split > cluster ? split : cluster;
   if (bn_rt_shape(cs) && (C * cs) % 4 == 0) {  // the row-tile path of batch_norm_rows.hpp
     const size_t rows = bn_rt_workspace_bytes(C * cs, w);

@@ -122,6 +122,64 @@ __device__ __forceinline__ void cluster_collect(unsigned long long* slots, int M
   rb = have ? __uint_as_float(static_cast<unsigned>(wb)) : nb;
 }
 
+// The same for clusters of up to 2 x 64 members whose pairs are simply added: lane j polls
+// slots j and j + 64; every lane returns the cluster's totals.  (Four slots per lane were
+// measured: the extra registers of the polling wave cost the cluster kernels, which sit at
+// the 128-register boundary, a factor of 1.3 to 3.)
+constexpr int kClusterSumSlotsPerLane = 2;
+constexpr int kClusterMaxSumM = 64 * kClusterSumSlotsPerLane;
+
+__device__ __forceinline__ float cluster_wave_total(float v)
+{
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+__device__ __forceinline__ void cluster_collect_sums(unsigned long long* slots, int M, ClusterTag tag,
+                                                     int* error_word, float& ta, float& tb)
+{
+  const int lane = threadIdx.x & 63;
+  constexpr int H = kClusterSumSlotsPerLane;
+  unsigned long long w[H][2];
+  bool have[H];
+#pragma unroll
+  for (int h = 0; h < H; ++h) {
+    w[h][0] = w[h][1] = 0;
+    have[h] = false;
+  }
+  int polls = 0;
+  for (;;) {
+    bool all = true;
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const int j = lane + 64 * h;
+      if (j < M && !have[h]) {
+        w[h][0] = __hip_atomic_load(slots + 2 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        w[h][1] = __hip_atomic_load(slots + 2 * j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        have[h] = static_cast<unsigned>(w[h][0] >> 32) == tag.lo && static_cast<unsigned>(w[h][1] >> 32) == tag.hi;
+      }
+      all = all && (have[h] || j >= M);
+    }
+    if (__all(all)) break;
+    if (++polls > kClusterMaxPolls) {
+      if (lane == 0) __hip_atomic_store(error_word, kClusterTimedOut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+  float a = 0.f, b = 0.f;
+#pragma unroll
+  for (int h = 0; h < H; ++h) {
+    if (have[h]) {
+      a += __uint_as_float(static_cast<unsigned>(w[h][0]));
+      b += __uint_as_float(static_cast<unsigned>(w[h][1]));
+    }
+  }
+  ta = cluster_wave_total(a);
+  tb = cluster_wave_total(b);
+}
+
 // Publish and collect in one go.
 __device__ __forceinline__ void cluster_exchange(float a, float b, unsigned long long* slots, int k,
                                                  int M, ClusterTag tag, int* error_word, float na,
@@ -139,9 +197,9 @@ struct ClusterWorkspace {
   unsigned long long* slots;
 };
 
-inline size_t cluster_workspace_bytes(int64_t items)
+inline size_t cluster_workspace_bytes(int64_t items, int max_m = kClusterMaxM)
 {
-  return 64 + static_cast<size_t>(items) * kClusterMaxM * 2 * sizeof(unsigned long long);
+  return 64 + static_cast<size_t>(items) * max_m * 2 * sizeof(unsigned long long);
 }
 
 inline ClusterWorkspace cluster_workspace(void* ws)
@@ -169,11 +227,11 @@ struct ClusterPlan {
   int V, M;
 };
 
-inline ClusterPlan plan_cluster(int64_t E, int max_v, int threads = kClusterThreads)
+inline ClusterPlan plan_cluster(int64_t E, int max_v, int threads = kClusterThreads, int max_m = kClusterMaxM)
 {
   const int64_t per_v = threads;
   const int64_t M = (E + per_v * max_v - 1) / (per_v * max_v);
-  if (M > kClusterMaxM || M < 1) return {0, 0};
+  if (M > max_m || M < 1) return {0, 0};
   const int64_t V = (E + per_v * M - 1) / (per_v * M);
   return {static_cast<int>(V), static_cast<int>(M)};
 }

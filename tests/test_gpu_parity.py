@@ -332,6 +332,8 @@ BN_CASES = [
     ((256, 4, 4), 200, True, 0), ((100, 12), 64, True, 0),
     # more channels than resident clusters: some clusters take two or three channels in turn, others one
     ((478, 16), 577, True, 0), ((1500, 4, 4), 600, False, 0), ((900, 64), 300, True, 0),
+    # channels of up to a million entries: clusters of more than 64 workgroups (two slots per polling lane)
+    ((3, 56, 56), 256, True, 0), ((2, 802816), 1, True, 0), ((2, 1000000), 1, False, 0), ((1, 1100000), 1, True, 0),
 ]
 
 
@@ -388,7 +390,8 @@ def test_batch_norm(L, dims, w, bessel, pad):
     # channels of odd sizes on matrices whose rows come in aligned fours: the row-tile kernels on fp16
     ((2048, 7, 7), 16, True, 0, True), ((4096,), 64, True, 0, True), ((64, 7, 7), 300, False, 0, True),
     ((12, 3, 3), 20, True, 0, True), ((1024, 1), 2048, True, 0, True), ((128, 7, 7), 10, True, 0, False),
-    ((32, 7, 7), 64, True, 4, True), ((2000, 2), 200, False, 0, True), ((100, 12), 64, True, 0, True)])
+    ((32, 7, 7), 64, True, 4, True), ((2000, 2), 200, False, 0, True), ((100, 12), 64, True, 0, True),
+    ((3, 56, 56), 512, True, 0, True), ((2, 2000000), 1, True, 0, True)])   # clusters of more than 64 workgroups
 def test_batch_norm_f16(L, dims, w, bessel, pad, training):
     """fp16 storage, fp32 arithmetic: the oracle sees the fp16-rounded inputs."""
     rng = np.random.default_rng(int(np.prod(dims)) * 5 + w)
