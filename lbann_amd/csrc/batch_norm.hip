@@ -27,6 +27,7 @@
 #include "host_utils.hpp"
 #include "batch_norm_math.hpp"
 #include "batch_norm_rows.hpp"
+#include "batch_norm_stream.hpp"
 
 namespace lbn {
 
@@ -800,6 +801,36 @@ static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   return false;
 }
 
+// Channels too large for the register-resident clusters: clusters that stream their share
+// twice (batch_norm_stream.hpp).  False: the caller uses the sums -> apply kernels.
+template <typename S, bool BWD>
+static bool bn_try_stream(hipStream_t st, BnStreamArgs<S> a, int64_t C, int64_t cs, int64_t w, void* ws)
+{
+  static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
+  constexpr int VE = Vec16<S>::N;
+  const int64_t E = cs / VE * w;
+  if (disabled || !aligned16(ws) || E >= (int64_t(1) << 31) || C > (1 << 24)) return false;
+  const int cap = BWD ? cluster_capacity(bn_bwd_stream<S>, kBnStreamThreads)
+                      : cluster_capacity(bn_fwd_stream<S>, kBnStreamThreads);
+  int64_t M = cap < kClusterMaxSumM ? cap : kClusterMaxSumM;
+  if (M < 1) return false;
+  const int64_t share = ceil_div(E, M);
+  M = ceil_div(E, share);
+  static const int max_nc = std::getenv("LBN_BN_STREAM_CLUSTERS") ? std::atoi(std::getenv("LBN_BN_STREAM_CLUSTERS")) : 0;
+  int64_t nc = cap / M;
+  if (max_nc > 0 && nc > max_nc) nc = max_nc;
+  if (nc > C) nc = C;
+  if (nc < 1) return false;
+  a.cs = cs, a.C = static_cast<int>(C), a.M = static_cast<int>(M), a.n = cs * w;
+  a.seg = static_cast<unsigned>(cs / VE), a.E = static_cast<unsigned>(E), a.share = static_cast<unsigned>(share);
+  a.cw = cluster_workspace(ws);
+  a.tag = cluster_call_tag(st, a.cw);
+  const dim3 grid(static_cast<unsigned>(nc * M));
+  if (BWD) hipLaunchKernelGGL(bn_bwd_stream<S>, grid, dim3(kBnStreamThreads), 0, st, a);
+  else hipLaunchKernelGGL(bn_fwd_stream<S>, grid, dim3(kBnStreamThreads), 0, st, a);
+  return true;
+}
+
 static int bn_check(int64_t C, int64_t cs, int64_t w, const int64_t* lds, int nld)
 {
   if (C < 0 || cs < 0 || w < 0) return LBN_ERR_INVALID_ARGUMENT;
@@ -979,6 +1010,13 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   if (vec && bn_try_fwd_cluster<S>(st, C, cs, w, pivot, bessel, epsilon, decay, x, ldx, y, ldy, mean, var,
                                    scale, bias, running_mean, running_var, workspace))
     return launch_status();
+  if (vec && cs * w > 1) {
+    BnStreamArgs<S> sa{};
+    sa.x = x, sa.out = y, sa.ldx = ldx, sa.ldo = ldy, sa.use_pivot = pivot, sa.bessel = bessel, sa.eps = epsilon;
+    sa.decay = decay, sa.mean = mean, sa.var = var, sa.scale = scale, sa.bias = bias;
+    sa.rmean = running_mean, sa.rvar = running_var;
+    if (bn_try_stream<S, false>(st, sa, C, cs, w, workspace)) return launch_status();
+  }
   if (vec) {
     hipLaunchKernelGGL((bn_fwd_sums<S, true>), grid, dim3(kBnThreads), 0, st, x, ldx, cs, w, pivot, part);
     hipLaunchKernelGGL((bn_fwd_apply<S, true, true>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs, w,
@@ -1054,6 +1092,13 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
       bn_try_bwd_cluster<S>(st, C, cs, w, bessel, epsilon, x, ldx, dy, lddy, dx, lddx, use_mean, use_var,
                             scale, dscale, dbias, dmean, dvar, workspace))
     return launch_status();
+  if (training && vec && n > 1) {
+    BnStreamArgs<S> sa{};
+    sa.x = x, sa.dy = dy, sa.out = dx, sa.ldx = ldx, sa.lddy = lddy, sa.ldo = lddx, sa.bessel = bessel;
+    sa.eps = epsilon, sa.mean = const_cast<float*>(use_mean), sa.var = const_cast<float*>(use_var), sa.scale = scale;
+    sa.dscale = dscale, sa.dbias = dbias, sa.dmean = dmean, sa.dvar = dvar;
+    if (bn_try_stream<S, true>(st, sa, C, cs, w, workspace)) return launch_status();
+  }
   if (vec) {
     hipLaunchKernelGGL((bn_bwd_sums<S, true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean, part);
     hipLaunchKernelGGL((bn_bwd_apply<S, true, true>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy,

@@ -1,0 +1,229 @@
+// Batch norm for channels too large for the register-resident clusters of batch_norm.hip
+// (more than about a million entries per channel: 112 x 112 maps at a mini-batch of 256,
+// volumes).  Math as in batch_norm.hip (batch_normalization.cpp:37-175, :178-329).
+//
+// A cluster of M workgroups shares a channel as before, but a workgroup's share no longer
+// fits its registers: it streams the share once for the sums, publishes them, collects the
+// cluster's sums (cluster_sync.hpp) and streams the same share again for the output.  The
+// second pass re-reads what the same workgroup read a moment ago: a cluster's channel is
+// a few tens of MiB at most and only a few clusters are active, so it comes from the
+// caches and x (and dy) cross HBM once, against twice for the sums -> apply kernels.
+// Persistent grid: cluster cl takes channels cl, cl + nclusters, ...
+#pragma once
+
+#include <type_traits>
+
+#include "batch_norm_math.hpp"
+#include "cluster_sync.hpp"
+#include "device_utils.hpp"
+
+namespace lbn {
+
+constexpr int kBnStreamThreads = 512;
+constexpr int kBnStreamWaves = kBnStreamThreads / kWave;
+constexpr int kBnStreamUnroll = 4;
+
+template <typename S>
+struct BnStreamArgs {
+  const S* x;
+  const S* dy;  // backward only
+  S* out;       // y or dx
+  int64_t ldx, lddy, ldo, cs;
+  int C, M, use_pivot, bessel, training;
+  float eps, decay;
+  int64_t n;       // entries per channel
+  unsigned seg;    // vectors per column segment of a channel
+  unsigned E;      // vectors per channel
+  unsigned share;  // vectors per workgroup
+  ClusterWorkspace cw;
+  ClusterTag tag;
+  float* mean;  // forward: written; backward: read
+  float* var;
+  const float* scale;
+  const float* bias;
+  float* rmean;
+  float* rvar;
+  float* dscale;
+  float* dbias;
+  float* dmean;
+  float* dvar;
+};
+
+// Offset of vector e of a channel inside a matrix with leading dimension ld.
+template <typename S>
+__device__ __forceinline__ int64_t bn_stream_offset(unsigned e, unsigned seg, int64_t ld)
+{
+  const unsigned col = e / seg;
+  return static_cast<int64_t>(col) * ld + Vec16<S>::N * static_cast<int64_t>(e - col * seg);
+}
+
+// Calls f(e, count) for this thread's vectors of the workgroup's share [begin, end): U
+// vectors a workgroup-stride apart per call (the caller issues their loads together), then
+// the leftovers one at a time.  `count` is a compile-time constant.
+template <int U, typename F>
+__device__ __forceinline__ void bn_stream_walk(unsigned begin, unsigned end, F&& f)
+{
+  unsigned e = begin + threadIdx.x;
+  for (; e + (U - 1) * kBnStreamThreads < end; e += U * kBnStreamThreads) f(e, std::integral_constant<int, U>{});
+  for (; e < end; e += kBnStreamThreads) f(e, std::integral_constant<int, 1>{});
+}
+
+template <typename S>
+__global__ void __launch_bounds__(kBnStreamThreads)
+bn_fwd_stream(BnStreamArgs<S> a)
+{
+  using IO = Vec16<S>;
+  constexpr int VE = IO::N;
+  __shared__ float red[2 * kBnStreamWaves];
+  __shared__ float bc[2];
+  const int nc = gridDim.x / a.M;
+  const int cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - cl * a.M;
+  if (cl >= a.C) return;
+  cluster_resolve_tag(a.tag);
+  const unsigned begin = static_cast<unsigned>(k) * a.share;
+  const unsigned end = begin + a.share < a.E ? begin + a.share : a.E;
+  for (int ch = cl; ch < a.C; ch += nc) {
+    const S* xc = a.x + static_cast<int64_t>(ch) * a.cs;
+    S* yc = a.out + static_cast<int64_t>(ch) * a.cs;
+    const float K = a.use_pivot ? IO::load1(xc) : 0.f;
+    float s = 0.f, q = 0.f;
+    bn_stream_walk<kBnStreamUnroll>(begin, end, [&](unsigned e, auto count) {
+      constexpr int N = decltype(count)::value;
+      float v[N][VE];
+#pragma unroll
+      for (int u = 0; u < N; ++u) IO::load(xc + bn_stream_offset<S>(e + u * kBnStreamThreads, a.seg, a.ldx), v[u]);
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          const float d = v[u][j] - K;
+          s += d;
+          q = __builtin_fmaf(d, d, q);
+        }
+      }
+    });
+    team_sum2<kBnStreamWaves>(s, q, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+    unsigned long long* slots = a.cw.slots + static_cast<int64_t>(ch) * a.M * 2;
+    if (threadIdx.x == 0) cluster_publish(s, q, slots, k, a.tag);
+    if (threadIdx.x < kWave) {
+      float ts, tq;
+      cluster_collect_sums(slots, a.M, a.tag, a.cw.error, ts, tq);
+      if (threadIdx.x == 0) {
+        float mean, var;
+        stats_from_sums(ts, tq, K, a.n, a.bessel, a.eps, mean, var);
+        bc[0] = mean;
+        bc[1] = 1.0f / sqrtf(var + a.eps);
+        if (k == 0) {
+          a.mean[ch] = mean;
+          a.var[ch] = var;
+          a.rmean[ch] = a.decay * a.rmean[ch] + (1.f - a.decay) * mean;
+          a.rvar[ch] = a.decay * a.rvar[ch] + (1.f - a.decay) * var;
+        }
+      }
+    }
+    __syncthreads();
+    const float mean = bc[0];
+    const float inv_stdev = bc[1];
+    const float scale = a.scale[ch], bias = a.bias[ch];
+    bn_stream_walk<kBnStreamUnroll>(begin, end, [&](unsigned e, auto count) {
+      constexpr int N = decltype(count)::value;
+      float v[N][VE];
+#pragma unroll
+      for (int u = 0; u < N; ++u) IO::load(xc + bn_stream_offset<S>(e + u * kBnStreamThreads, a.seg, a.ldx), v[u]);
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+#pragma unroll
+        for (int j = 0; j < VE; ++j) v[u][j] = scale * ((v[u][j] - mean) * inv_stdev) + bias;
+        IO::store(yc + bn_stream_offset<S>(e + u * kBnStreamThreads, a.seg, a.ldo), v[u]);
+      }
+    });
+    __syncthreads();  // bc and red are written again for the next channel
+  }
+}
+
+// Training-mode backward (statistics are variables of the loss).
+template <typename S>
+__global__ void __launch_bounds__(kBnStreamThreads)
+bn_bwd_stream(BnStreamArgs<S> a)
+{
+  using IO = Vec16<S>;
+  constexpr int VE = IO::N;
+  constexpr int U = kBnStreamUnroll / 2;  // two tensors per step
+  __shared__ float red[2 * kBnStreamWaves];
+  __shared__ float bc[2];
+  const int nc = gridDim.x / a.M;
+  const int cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - cl * a.M;
+  if (cl >= a.C) return;
+  cluster_resolve_tag(a.tag);
+  const unsigned begin = static_cast<unsigned>(k) * a.share;
+  const unsigned end = begin + a.share < a.E ? begin + a.share : a.E;
+  for (int ch = cl; ch < a.C; ch += nc) {
+    const S* xc = a.x + static_cast<int64_t>(ch) * a.cs;
+    const S* gc = a.dy + static_cast<int64_t>(ch) * a.cs;
+    S* dc = a.out + static_cast<int64_t>(ch) * a.cs;
+    const float mean = a.mean[ch];
+    const float inv_stdev = 1.0f / sqrtf(a.var[ch] + a.eps);
+    const float scale = a.scale[ch];
+    float sa = 0.f, sb = 0.f;
+    bn_stream_walk<U>(begin, end, [&](unsigned e, auto count) {
+      constexpr int N = decltype(count)::value;
+      float x[N][VE], g[N][VE];
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+        IO::load(xc + bn_stream_offset<S>(e + u * kBnStreamThreads, a.seg, a.ldx), x[u]);
+        IO::load(gc + bn_stream_offset<S>(e + u * kBnStreamThreads, a.seg, a.lddy), g[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          sa += g[u][j];
+          sb = __builtin_fmaf(g[u][j], x[u][j] - mean, sb);
+        }
+      }
+    });
+    team_sum2<kBnStreamWaves>(sa, sb, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+    unsigned long long* slots = a.cw.slots + static_cast<int64_t>(ch) * a.M * 2;
+    if (threadIdx.x == 0) cluster_publish(sa, sb, slots, k, a.tag);
+    if (threadIdx.x < kWave) {
+      float ta, tb;
+      cluster_collect_sums(slots, a.M, a.tag, a.cw.error, ta, tb);
+      if (threadIdx.x == 0) {
+        float ds, db, dmean, dvar;
+        grads_from_sums(ta, tb, scale, inv_stdev, ds, db, dmean, dvar);
+        bc[0] = dmean / static_cast<float>(a.n);
+        bc[1] = dvar * 2.f / static_cast<float>(a.n - (a.bessel ? 1 : 0));
+        if (k == 0) {
+          a.dscale[ch] = ds;
+          a.dbias[ch] = db;
+          a.dmean[ch] = dmean;
+          a.dvar[ch] = dvar;
+        }
+      }
+    }
+    __syncthreads();
+    const float dmean_term = bc[0];
+    const float dvar_term = bc[1];
+    const float k0 = scale * inv_stdev;
+    bn_stream_walk<U>(begin, end, [&](unsigned e, auto count) {
+      constexpr int N = decltype(count)::value;
+      float x[N][VE], g[N][VE];
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+        IO::load(xc + bn_stream_offset<S>(e + u * kBnStreamThreads, a.seg, a.ldx), x[u]);
+        IO::load(gc + bn_stream_offset<S>(e + u * kBnStreamThreads, a.seg, a.lddy), g[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+#pragma unroll
+        for (int j = 0; j < VE; ++j) g[u][j] = g[u][j] * k0 + dmean_term + dvar_term * (x[u][j] - mean);
+        IO::store(dc + bn_stream_offset<S>(e + u * kBnStreamThreads, a.seg, a.ldo), g[u]);
+      }
+    });
+    __syncthreads();
+  }
+}
+
+}  // namespace lbn

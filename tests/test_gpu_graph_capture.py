@@ -59,6 +59,8 @@ CASES = [
      ("m_weights_gradient",)),
     ("batch norm clusters in turn", lambda L: L.batch_normalization_layer((1500, 4, 4)), 1500 * 16, 600, torch.float32,
      ("m_mean_and_var", "m_mean_and_var_gradient", "m_scale_gradient", "m_bias_gradient")),
+    ("batch norm streaming clusters", lambda L: L.batch_normalization_layer((3, 1200000)), 3600000, 2, torch.float32,
+     ("m_mean_and_var", "m_mean_and_var_gradient", "m_scale_gradient", "m_bias_gradient")),
     ("batch norm small", lambda L: L.batch_normalization_layer((7, 5, 3)), 105, 14, torch.float32,
      ("m_mean_and_var", "m_mean_and_var_gradient")),
 ]

@@ -334,6 +334,8 @@ BN_CASES = [
     ((478, 16), 577, True, 0), ((1500, 4, 4), 600, False, 0), ((900, 64), 300, True, 0),
     # channels of up to a million entries: clusters of more than 64 workgroups (two slots per polling lane)
     ((3, 56, 56), 256, True, 0), ((2, 802816), 1, True, 0), ((2, 1000000), 1, False, 0), ((1, 1100000), 1, True, 0),
+    # beyond that: clusters that stream their share twice (backward from 1 M entries, forward from 2 M)
+    ((3, 112, 112), 256, True, 0), ((2, 2400000), 1, False, 0), ((5, 1300000), 2, True, 4), ((1, 6000000), 1, True, 0),
 ]
 
 
@@ -391,7 +393,8 @@ def test_batch_norm(L, dims, w, bessel, pad):
     ((2048, 7, 7), 16, True, 0, True), ((4096,), 64, True, 0, True), ((64, 7, 7), 300, False, 0, True),
     ((12, 3, 3), 20, True, 0, True), ((1024, 1), 2048, True, 0, True), ((128, 7, 7), 10, True, 0, False),
     ((32, 7, 7), 64, True, 4, True), ((2000, 2), 200, False, 0, True), ((100, 12), 64, True, 0, True),
-    ((3, 56, 56), 512, True, 0, True), ((2, 2000000), 1, True, 0, True)])   # clusters of more than 64 workgroups
+    ((3, 56, 56), 512, True, 0, True), ((2, 2000000), 1, True, 0, True),   # clusters of more than 64 workgroups
+    ((3, 112, 112), 512, True, 0, True), ((2, 2500000), 2, False, 0, True)])   # streaming clusters
 def test_batch_norm_f16(L, dims, w, bessel, pad, training):
     """fp16 storage, fp32 arithmetic: the oracle sees the fp16-rounded inputs."""
     rng = np.random.default_rng(int(np.prod(dims)) * 5 + w)
