@@ -700,16 +700,16 @@ static size_t ln_cluster_part_offset(int64_t rows, int M) { return (ln_cluster_s
 // Workspace of the cluster path for rows of n entries (0: the shape does not take it).
 static size_t ln_cluster_fwd_workspace(int64_t n, int64_t rows, int ve)
 {
-  if (n % ve != 0) return 0;
-  const ClusterPlan cp = plan_ln_cluster(n / ve, kLnClFwdUnits / (kLnClThreads * ve));
-  return cp.M ? ln_cluster_slot_bytes(rows, kLnClMaxM) : 0;  // a launch may widen its clusters up to the maximum
+  if (n % ve != 0 || n / ve >= (int64_t(1) << 31)) return 0;
+  // register clusters (a launch may widen them up to the maximum) or, beyond their reach, streaming clusters
+  return ln_cluster_slot_bytes(rows, kLnClMaxM);
 }
 
 static size_t ln_cluster_bwd_workspace(int64_t n, int64_t rows, int ve)
 {
   if (n % ve != 0) return 0;
   const ClusterPlan cp = plan_ln_cluster(n / ve, kLnClBwdUnits / (kLnClThreads * ve));
-  if (!cp.M) return 0;
+  if (!cp.M) return 0;  // rows beyond the register clusters keep the two-pass kernels when weights have gradients
   return ln_cluster_part_offset(rows, kLnClMaxM) +
          static_cast<size_t>(ln_cluster_count_bound(rows, cp.M)) * 2 * n * sizeof(float);
 }
@@ -856,6 +856,34 @@ static int ln_bwd_cluster_launch(hipStream_t st, bool wgrad, const T* x, const T
   return 0;
 }
 
+// Rows beyond the register clusters: clusters that stream their share twice.  1: launched.
+template <typename T, bool BWD>
+static int ln_stream_launch(hipStream_t st, LnClArgs<T> a, int64_t rows, int64_t n, void* ws, size_t ws_bytes)
+{
+  static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
+  constexpr int VE = Vec16<T>::N;
+  const int64_t nvec = n / VE;
+  if (disabled || !ws || !aligned16(ws) || nvec >= (int64_t(1) << 31)) return 0;
+  const int cap = BWD ? cluster_capacity(ln_bwd_stream<T>, kLnStreamThreads)
+                      : cluster_capacity(ln_fwd_stream<T>, kLnStreamThreads);
+  int64_t M = cap < kLnClMaxM ? cap : kLnClMaxM;
+  if (M < 1) return 0;
+  int64_t nc = cap / M;
+  if (nc > rows) nc = rows;
+  M = cap / nc < kLnClMaxM ? cap / nc : kLnClMaxM;  // few rows: wider clusters instead of idle workgroups
+  const int64_t share = ceil_div(nvec, M);
+  M = ceil_div(nvec, share);
+  if (ws_bytes < ln_cluster_slot_bytes(rows, static_cast<int>(M))) return 0;
+  a.rows = rows, a.n = n, a.nvec = static_cast<unsigned>(nvec), a.per_wg = static_cast<unsigned>(share);
+  a.M = static_cast<int>(M), a.inv_n = 1.0f / static_cast<float>(n);
+  a.cw = cluster_workspace(ws);
+  a.tag = cluster_call_tag(st, a.cw);
+  const dim3 grid(static_cast<unsigned>(nc * M));
+  if (BWD) hipLaunchKernelGGL(ln_bwd_stream<T>, grid, dim3(kLnStreamThreads), 0, st, a);
+  else hipLaunchKernelGGL(ln_fwd_stream<T>, grid, dim3(kLnStreamThreads), 0, st, a);
+  return 1;
+}
+
 template <typename T>
 static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t w, float eps,
                   const T* x, int64_t ldx, T* y, int64_t ldy, float* stats, int64_t lds,
@@ -882,6 +910,12 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     // longer than the register kernels hold: clusters when the caller gave scratch, else two passes
     if (ln_fwd_cluster_launch<T>(st, x, y, ldx, ldy, map, rows, n, eps, stats, lds, gamma, beta, sumsq, ws, ws_bytes))
       return launch_status();
+    if (rows < 512) {  // few giant rows: one workgroup per row would leave most of the device idle
+      LnClArgs<T> a{};
+      a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy, a.map = map, a.sumsq = sumsq, a.eps = eps;
+      a.stats = stats, a.ld_stats = lds, a.gamma = gamma, a.beta = beta;
+      if (ln_stream_launch<T, false>(st, a, rows, n, ws, ws_bytes)) return launch_status();
+    }
     hipLaunchKernelGGL((ln_fwd_long<T>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st, x, y,
                        ldx, ldy, map, n / VE, inv_n, eps, stats, lds, gamma, beta, sumsq);
     return launch_status();
@@ -1021,6 +1055,12 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     if (ln_bwd_cluster_launch<T>(st, wgrad, x, dy, dx, ldx, lddy, lddx, map, rows, n, eps, stats, lds, sgrad, ldsg,
                                  gamma, dgamma, dbeta, ws, ws_bytes))
       return launch_status();
+    if (!wgrad && rows < 512) {
+      LnClArgs<T> a{};
+      a.x = x, a.dy = dy, a.out = dx, a.ldx = ldx, a.lddy = lddy, a.ldo = lddx, a.map = map, a.eps = eps;
+      a.stats = const_cast<float*>(stats), a.ld_stats = lds, a.sgrad = sgrad, a.ld_sgrad = ldsg, a.gamma = gamma;
+      if (ln_stream_launch<T, true>(st, a, rows, n, ws, ws_bytes)) return launch_status();
+    }
     hipLaunchKernelGGL((ln_bwd_long<T>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st, x, dy,
                        dx, ldx, lddy, lddx, map, n / VE, 1.0f / static_cast<float>(n), eps, stats, lds, sgrad,
                        ldsg, gamma);
@@ -1122,8 +1162,7 @@ size_t lbn_layer_norm_bwd_workspace_bytes(int64_t num_groups, int64_t norm_size,
   if (has_weight_grads) return ln_bwd_workspace(norm_size, rows, ve);
   // without weight gradients only the cluster kernels of long rows use scratch (their slots)
   if (norm_size % ve != 0 || plan_ln_bwd(norm_size / ve, rows, ve, elem_bytes == 2 ? 2 : 4).tpr) return 0;
-  const ClusterPlan cp = plan_ln_cluster(norm_size / ve, kLnClBwdUnits / (kLnClThreads * ve));
-  return cp.M ? ln_cluster_slot_bytes(rows, kLnClMaxM) : 0;
+  return norm_size / ve < (int64_t(1) << 31) ? ln_cluster_slot_bytes(rows, kLnClMaxM) : 0;
 }
 
 int lbn_layer_norm_bwd_f32(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,

@@ -22,6 +22,8 @@
 // ln_wgrad_reduce adds the clusters' rows in a fixed order.
 #pragma once
 
+#include <type_traits>
+
 #include "cluster_sync.hpp"
 #include "device_utils.hpp"
 
@@ -476,6 +478,207 @@ inline int64_t ln_cluster_count_bound(int64_t rows, int M)
   int64_t nc = 512 / M;
   if (nc > rows) nc = rows;
   return nc < 1 ? 1 : nc;
+}
+
+}  // namespace lbn
+
+// ------------------------------------------------- rows beyond the register clusters
+// Rows of millions of entries (instance norm over volumes: 256^3 is 16.8 M entries per
+// channel): a workgroup's share no longer fits its registers, and there are so few rows that
+// one workgroup per row would leave most of the device idle.  As in batch_norm_stream.hpp a
+// cluster shares a row and every workgroup streams its share twice, the second time from
+// the caches; persistent over rows.  Weight gradients are not produced here (a slice of
+// dscale / dbias of this size fits neither registers nor LDS): layer norm with weights on
+// such rows keeps the two-pass kernels.
+namespace lbn {
+
+constexpr int kLnStreamThreads = 512;
+constexpr int kLnStreamWaves = kLnStreamThreads / kWave;
+constexpr int kLnStreamUnroll = 4;
+
+template <int U, typename F>
+__device__ __forceinline__ void ln_stream_walk(unsigned begin, unsigned end, F&& f)
+{
+  unsigned e = begin + threadIdx.x;
+  for (; e + (U - 1) * kLnStreamThreads < end; e += U * kLnStreamThreads) f(e, std::integral_constant<int, U>{});
+  for (; e < end; e += kLnStreamThreads) f(e, std::integral_constant<int, 1>{});
+}
+
+template <typename T>
+__device__ __forceinline__ void ln_stream_weights(const float* w, unsigned e, float fill, float (&out)[Vec16<T>::N])
+{
+  constexpr int VE = Vec16<T>::N;
+#pragma unroll
+  for (int k = 0; k < VE; ++k) out[k] = fill;
+  if (w) load_f32_run<VE>(w + VE * static_cast<int64_t>(e), out);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kLnStreamThreads)
+ln_fwd_stream(LnClArgs<T> a)
+{
+  using IO = Vec16<T>;
+  constexpr int VE = IO::N;
+  __shared__ float red[2 * kLnStreamWaves];
+  __shared__ float bc[2];
+  const int64_t nc = gridDim.x / a.M;
+  const int64_t cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - static_cast<int>(cl) * a.M;
+  if (cl >= a.rows) return;
+  cluster_resolve_tag(a.tag);
+  const unsigned begin = static_cast<unsigned>(k) * a.per_wg;
+  const unsigned end = begin + a.per_wg < a.nvec ? begin + a.per_wg : a.nvec;
+  for (int64_t row = cl; row < a.rows; row += nc) {
+    const T* xr = a.x + a.map.offset(row, a.ldx);
+    T* yr = a.out + a.map.offset(row, a.ldo);
+    const float K = a.sumsq ? 0.f : IO::load1(xr);
+    float s = 0.f, q = 0.f;
+    ln_stream_walk<kLnStreamUnroll>(begin, end, [&](unsigned e, auto count) {
+      constexpr int N = decltype(count)::value;
+      float v[N][VE];
+#pragma unroll
+      for (int u = 0; u < N; ++u) IO::load(xr + VE * static_cast<int64_t>(e + u * kLnStreamThreads), v[u]);
+#pragma unroll
+      for (int u = 0; u < N; ++u)
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          const float d = v[u][j] - K;
+          s += d;
+          q = __builtin_fmaf(d, d, q);
+        }
+    });
+    team_sum2<kLnStreamWaves>(s, q, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+    if (threadIdx.x == 0) cluster_publish(s, q, a.slots(row), k, a.tag);
+    if (threadIdx.x < kWave) {
+      float ts, tq;
+      cluster_collect_sums(a.slots(row), a.M, a.tag, a.cw.error, ts, tq);
+      if (threadIdx.x == 0) {
+        float dm = ts * a.inv_n;
+        float var = fmaxf(__builtin_fmaf(-dm, dm, tq * a.inv_n), 0.f);
+        if (a.sumsq) {  // the reference's own expression (layer_norm.cpp:99-112)
+          const float nf = static_cast<float>(a.n);
+          dm = ts / nf;
+          var = fmaxf(__fsub_rn(tq / nf, __fmul_rn(dm, dm)), 0.f);
+        }
+        bc[0] = K + dm;
+        bc[1] = 1.0f / sqrtf(var + a.eps);
+        if (k == 0) {
+          int64_t col, g;
+          a.map.split(row, col, g);
+          a.stats[g + col * a.ld_stats] = K + dm;
+          a.stats[a.map.groups + g + col * a.ld_stats] = var;
+        }
+      }
+    }
+    __syncthreads();
+    const float mean = bc[0];
+    const float inv_stdev = bc[1];
+    ln_stream_walk<kLnStreamUnroll>(begin, end, [&](unsigned e, auto count) {
+      constexpr int N = decltype(count)::value;
+      float v[N][VE];
+#pragma unroll
+      for (int u = 0; u < N; ++u) IO::load(xr + VE * static_cast<int64_t>(e + u * kLnStreamThreads), v[u]);
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+        float ga[VE], be[VE];
+        ln_stream_weights<T>(a.gamma, e + u * kLnStreamThreads, 1.f, ga);
+        ln_stream_weights<T>(a.beta, e + u * kLnStreamThreads, 0.f, be);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) v[u][j] = __builtin_fmaf((v[u][j] - mean) * inv_stdev, ga[j], be[j]);
+        IO::store(yr + VE * static_cast<int64_t>(e + u * kLnStreamThreads), v[u]);
+      }
+    });
+    __syncthreads();  // bc and red are written again for the next row
+  }
+}
+
+// Backward without weight gradients.
+template <typename T>
+__global__ void __launch_bounds__(kLnStreamThreads)
+ln_bwd_stream(LnClArgs<T> a)
+{
+  using IO = Vec16<T>;
+  constexpr int VE = IO::N;
+  constexpr int U = kLnStreamUnroll / 2;  // two tensors per step
+  __shared__ float red[2 * kLnStreamWaves];
+  __shared__ float bc[2];
+  const int64_t nc = gridDim.x / a.M;
+  const int64_t cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - static_cast<int>(cl) * a.M;
+  if (cl >= a.rows) return;
+  cluster_resolve_tag(a.tag);
+  const unsigned begin = static_cast<unsigned>(k) * a.per_wg;
+  const unsigned end = begin + a.per_wg < a.nvec ? begin + a.per_wg : a.nvec;
+  for (int64_t row = cl; row < a.rows; row += nc) {
+    int64_t col, g;
+    a.map.split(row, col, g);
+    const T* xr = a.x + g * a.map.stride + col * a.ldx;
+    const T* gr = a.dy + g * a.map.stride + col * a.lddy;
+    T* dr = a.out + g * a.map.stride + col * a.ldo;
+    const float mean = a.stats[g + col * a.ld_stats];
+    const float inv_stdev = 1.0f / sqrtf(a.stats[a.map.groups + g + col * a.ld_stats] + a.eps);
+    float sa = 0.f, sb = 0.f;
+    ln_stream_walk<U>(begin, end, [&](unsigned e, auto count) {
+      constexpr int N = decltype(count)::value;
+      float x[N][VE], d[N][VE];
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+        IO::load(xr + VE * static_cast<int64_t>(e + u * kLnStreamThreads), x[u]);
+        IO::load(gr + VE * static_cast<int64_t>(e + u * kLnStreamThreads), d[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+        float ga[VE];
+        ln_stream_weights<T>(a.gamma, e + u * kLnStreamThreads, 1.f, ga);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          const float gs = d[u][j] * ga[j];
+          sa += gs;
+          sb = __builtin_fmaf(gs, (x[u][j] - mean) * inv_stdev, sb);
+        }
+      }
+    });
+    team_sum2<kLnStreamWaves>(sa, sb, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+    if (threadIdx.x == 0) cluster_publish(sa, sb, a.slots(row), k, a.tag);
+    if (threadIdx.x < kWave) {
+      float ta, tb;
+      cluster_collect_sums(a.slots(row), a.M, a.tag, a.cw.error, ta, tb);
+      if (threadIdx.x == 0) {
+        const float dmean = -ta * inv_stdev;
+        const float dvar = -tb * inv_stdev * inv_stdev * 0.5f;
+        bc[0] = dmean * a.inv_n;
+        bc[1] = -tb * inv_stdev * a.inv_n;  // dvar * 2 / n per unit of xh
+        if (k == 0) {
+          a.sgrad[g + col * a.ld_sgrad] = dmean;
+          a.sgrad[a.map.groups + g + col * a.ld_sgrad] = dvar;
+        }
+      }
+    }
+    __syncthreads();
+    const float c0 = bc[0];
+    const float c1 = bc[1];
+    ln_stream_walk<U>(begin, end, [&](unsigned e, auto count) {
+      constexpr int N = decltype(count)::value;
+      float x[N][VE], d[N][VE];
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+        IO::load(xr + VE * static_cast<int64_t>(e + u * kLnStreamThreads), x[u]);
+        IO::load(gr + VE * static_cast<int64_t>(e + u * kLnStreamThreads), d[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+        float ga[VE];
+        ln_stream_weights<T>(a.gamma, e + u * kLnStreamThreads, 1.f, ga);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          const float xh = (x[u][j] - mean) * inv_stdev;
+          d[u][j] = __builtin_fmaf(d[u][j] * ga[j], inv_stdev, __builtin_fmaf(c1, xh, c0));
+        }
+        IO::store(dr + VE * static_cast<int64_t>(e + u * kLnStreamThreads), d[u]);
+      }
+    });
+    __syncthreads();
+  }
 }
 
 }  // namespace lbn

@@ -47,6 +47,7 @@ CASES = [
     ("layer norm clusters", lambda L: L.layer_norm_layer((150528,), 1e-5, True, True), 150528, 40, torch.float32,
      ("m_statistics", "m_statistics_gradient", "m_scale_gradient", "m_bias_gradient")),
     ("instance norm", lambda L: L.instance_norm_layer((8, 32, 32)), 8192, 24, torch.float32, ()),
+    ("instance norm streaming clusters", lambda L: L.instance_norm_layer((2, 2400000)), 4800000, 2, torch.float32, ()),
     ("entry-wise batch norm", lambda L: L.entrywise_batch_normalization_layer((4096,)), 4096, 48, torch.float32,
      ("m_batch_statistics", "m_batch_statistics_gradient")),
     ("batch norm clusters", lambda L: L.batch_normalization_layer((64, 56, 56)), 64 * 3136, 16, torch.float32,

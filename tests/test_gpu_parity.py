@@ -170,6 +170,8 @@ LN_CASES = [
     # (1048576 entries backward), beyond that the two-pass kernels again; more rows than clusters
     ((802816,), 0, 5, True, 0), ((1048576,), 0, 3, True, 0), ((1048580,), 0, 2, True, 0), ((32772,), 0, 700, True, 0),
     ((2, 100000), -1, 40, True, 8), ((50000,), 0, 33, False, 0),
+    # rows of millions of entries: clusters that stream their share twice (forward; backward without weights)
+    ((3000000,), 0, 3, False, 0), ((2500000,), 0, 2, True, 0), ((2, 2200000), -1, 2, False, 4), ((9000000,), 0, 1, False, 0),
     # rows off the 16-byte grid: the register kernels with one float per access
     ((1001,), 0, 40, True, 0), ((197, 769), -1, 3, True, 0), ((4095,), 0, 9, True, 0), ((4097,), 0, 9, True, 0),
     ((8191,), 0, 5, False, 0), ((49,), 0, 3000, True, 0), ((1000,), 0, 17, True, 3), ((7,), 0, 100000, True, 0),
@@ -246,7 +248,7 @@ def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
                                                    ((1001,), 0, 7, 0),   # odd: scalar fallback
                                                    # long rows shared by clusters of workgroups
                                                    ((802816,), 0, 4, 0), ((65536,), 0, 150, 0), ((2, 100000), -1, 20, 8),
-                                                   ((1048576,), 0, 2, 0)])
+                                                   ((1048576,), 0, 2, 0), ((5000000,), 0, 2, 0)])
 def test_layer_norm_f16(L, dims, start_dim, w, pad):
     rng = np.random.default_rng(int(np.prod(dims)) * 3 + w)
     h = int(np.prod(dims))
@@ -261,6 +263,7 @@ def test_layer_norm_f16(L, dims, start_dim, w, pad):
 # ===================================================================== instance norm
 @pytest.mark.parametrize("dims,w,pad", [((5, 3, 7), 15, 0), ((64, 56, 56), 6, 0), ((8, 1024), 33, 0),
                                         ((2, 1048576), 2, 0), ((4, 96, 96, 96), 3, 0),   # volumes: clusters of workgroups per channel
+                                        ((2, 160, 160, 160), 1, 0), ((3, 2500000), 2, 4),   # streaming clusters
                                         ((3, 50000), 40, 4),
                                         ((3, 100000), 2, 0), ((7, 1), 5, 0), ((16, 31), 40, 4),
                                         ((256, 16, 16), 64, 0), ((3, 224, 224), 8, 0), ((2, 64, 64, 64), 2, 0),
