@@ -358,7 +358,8 @@ def main():
         # (forward, backward) bytes: 2 and 3 tensors unless the builder says otherwise
         fwd_b, bwd_b = built[5] if len(built) > 5 else W.algorithmic_bytes(elems, esize)
         wall, fwd, bwd, bwd_b2b = measure(layer, args.steps, args.warmup)
-        f_ms, b_ms = statistics.mean(fwd), statistics.mean(bwd)
+        # medians: one slow launch among the timed ones (a clock ramp, a page fault) must not set the figure
+        f_ms, b_ms = statistics.median(fwd), statistics.median(bwd)
         step_ms = wall / args.steps * 1e3
         r = {
             "workload": desc,
@@ -369,7 +370,7 @@ def main():
             "samples_per_s": samples / (step_ms * 1e-3),
             "fwd_ms": f_ms, "bwd_ms": b_ms,
             "fwd_ms_min": min(fwd), "bwd_ms_min": min(bwd),
-            "fwd_ms_median": statistics.median(fwd), "bwd_ms_median": statistics.median(bwd),
+            "fwd_ms_mean": statistics.mean(fwd), "bwd_ms_mean": statistics.mean(bwd),
             "fwd_gbs": fwd_b / (f_ms * 1e-3) / 1e9, "bwd_gbs": bwd_b / (b_ms * 1e-3) / 1e9,
             "bwd_back_to_back_ms": bwd_b2b,
         }

@@ -139,6 +139,13 @@ __device__ __forceinline__ float cluster_wave_total(float v)
 __device__ __forceinline__ void cluster_collect_sums(unsigned long long* slots, int M, ClusterTag tag,
                                                      int* error_word, float& ta, float& tb)
 {
+  if (M <= 64) {  // the common case keeps the one-slot loop
+    float ra, rb;
+    cluster_collect(slots, M, tag, error_word, 0.f, 0.f, ra, rb);
+    ta = cluster_wave_total(ra);
+    tb = cluster_wave_total(rb);
+    return;
+  }
   const int lane = threadIdx.x & 63;
   constexpr int H = kClusterSumSlotsPerLane;
   unsigned long long w[H][2];
