@@ -32,6 +32,7 @@
 #include <chrono>
 #include <cstdint>
 
+#include "device_utils.hpp"
 #include "host_utils.hpp"
 
 namespace lbn {
@@ -129,17 +130,17 @@ __device__ __forceinline__ void cluster_collect(unsigned long long* slots, int M
 constexpr int kClusterSumSlotsPerLane = 2;
 constexpr int kClusterMaxSumM = 64 * kClusterSumSlotsPerLane;
 
-__device__ __forceinline__ float cluster_wave_total(float v)
-{
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-  return v;
-}
+// On the DPP path (device_utils.hpp): a butterfly of shuffles here cost layer norm over
+// 64 huge rows 8 % of its time, the collecting wave being what every other wave waits for.
+__device__ __forceinline__ float cluster_wave_total(float v) { return wave_sum(v); }
 
+// ONE_SLOT_PATH: clusters of up to 64 take the one-slot loop (2.5 % on batch norm's usual
+// shapes); kernels whose clusters are mostly larger leave it out and save its registers.
+template <bool ONE_SLOT_PATH = true>
 __device__ __forceinline__ void cluster_collect_sums(unsigned long long* slots, int M, ClusterTag tag,
                                                      int* error_word, float& ta, float& tb)
 {
-  if (M <= 64) {  // the common case keeps the one-slot loop
+  if (ONE_SLOT_PATH && M <= 64) {
     float ra, rb;
     cluster_collect(slots, M, tag, error_word, 0.f, 0.f, ra, rb);
     ta = cluster_wave_total(ra);
