@@ -109,6 +109,13 @@ def main():
             return t1 - t0, t2 - t1
         return layer, data["x"].size, 2 if half else 4, data["x"].shape[1], cpu
 
+    def volume_in():
+        # 16 channels of 160^3 voxels, 2 samples: 32 rows of 4.1 M entries (501 MiB per tensor)
+        rng = np.random.default_rng(0x4C42000A)
+        h, w = 16 * 160 ** 3, 2
+        mk = lambda m, sd: np.asfortranarray((rng.standard_normal((w, h), dtype=np.float32) * sd + m).T)
+        return dict(x=mk(0.5, 2.0), dy=mk(0.0, 1.0), eps=1e-5, dims=(16, 160, 160, 160))
+
     def whole_sample_ln():
         d = W.cfg3_batch_norm()
         n = d["x"].shape[0]
@@ -238,6 +245,9 @@ def main():
         # whole samples: 64 rows of 802816 entries, with per-entry scale and bias
         "extra_layer_norm_whole_sample": ("LayerNorm fwd+bwd fp32 802816x64, whole samples (informational)",
                                           lambda: build_ln(whole_sample_ln(), False)),
+        # not a baseline configuration: instance norm on volumes, where a channel is millions of voxels
+        "extra_instance_norm_volume": ("InstanceNorm fwd+bwd fp32 16x160^3 x 2 (informational)",
+                                       lambda: build_in(volume_in())),
         # not baseline configurations: fp16 storage for batch norm, and softmax rows off the 16-byte grid
         "extra_batch_norm_f16": ("BatchNorm train fwd+bwd fp16 storage NCHW 64x256x56x56 (informational)",
                                  lambda: build_bn(W.cfg3_batch_norm(), True)),
