@@ -22,6 +22,12 @@ namespace lbn {
 constexpr int kBnStreamThreads = 512;
 constexpr int kBnStreamWaves = kBnStreamThreads / kWave;
 constexpr int kBnStreamUnroll = 4;
+// Vectors per thread at the head of a workgroup's share that stay in registers between the
+// two passes (a 112 x 112 map at a mini-batch of 256 over 128 workgroups is 13 vectors per
+// thread: read once).
+// Half as many for the eight-entry vectors, whose unpacked form takes the registers.
+template <typename S> constexpr int kBnStreamKeepFwd = Vec16<S>::N > 4 ? 8 : 16;
+template <typename S> constexpr int kBnStreamKeepBwd = Vec16<S>::N > 4 ? 4 : 8;
 
 template <typename S>
 struct BnStreamArgs {
@@ -83,12 +89,33 @@ bn_fwd_stream(BnStreamArgs<S> a)
   cluster_resolve_tag(a.tag);
   const unsigned begin = static_cast<unsigned>(k) * a.share;
   const unsigned end = begin + a.share < a.E ? begin + a.share : a.E;
+  const unsigned rest = begin + kBnStreamKeepFwd<S> * kBnStreamThreads;  // where streaming takes over
   for (int ch = cl; ch < a.C; ch += nc) {
     const S* xc = a.x + static_cast<int64_t>(ch) * a.cs;
     S* yc = a.out + static_cast<int64_t>(ch) * a.cs;
     const float K = a.use_pivot ? IO::load1(xc) : 0.f;
     float s = 0.f, q = 0.f;
-    bn_stream_walk<kBnStreamUnroll>(begin, end, [&](unsigned e, auto count) {
+    typename IO::raw_t kept[kBnStreamKeepFwd<S>];
+#pragma unroll
+    for (int i = 0; i < kBnStreamKeepFwd<S>; ++i) {
+      const unsigned e = begin + threadIdx.x + i * kBnStreamThreads;
+      kept[i] = typename IO::raw_t{};
+      if (e < end) kept[i] = IO::load_raw(xc + bn_stream_offset<S>(e, a.seg, a.ldx));
+    }
+#pragma unroll
+    for (int i = 0; i < kBnStreamKeepFwd<S>; ++i) {
+      if (begin + threadIdx.x + i * kBnStreamThreads < end) {
+        float v[VE];
+        IO::unpack(kept[i], v);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          const float d = v[j] - K;
+          s += d;
+          q = __builtin_fmaf(d, d, q);
+        }
+      }
+    }
+    bn_stream_walk<kBnStreamUnroll>(rest, end, [&](unsigned e, auto count) {
       constexpr int N = decltype(count)::value;
       float v[N][VE];
 #pragma unroll
@@ -126,7 +153,18 @@ bn_fwd_stream(BnStreamArgs<S> a)
     const float mean = bc[0];
     const float inv_stdev = bc[1];
     const float scale = a.scale[ch], bias = a.bias[ch];
-    bn_stream_walk<kBnStreamUnroll>(begin, end, [&](unsigned e, auto count) {
+#pragma unroll
+    for (int i = 0; i < kBnStreamKeepFwd<S>; ++i) {
+      const unsigned e = begin + threadIdx.x + i * kBnStreamThreads;
+      if (e < end) {
+        float v[VE];
+        IO::unpack(kept[i], v);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) v[j] = scale * ((v[j] - mean) * inv_stdev) + bias;
+        IO::store(yc + bn_stream_offset<S>(e, a.seg, a.ldo), v);
+      }
+    }
+    bn_stream_walk<kBnStreamUnroll>(rest, end, [&](unsigned e, auto count) {
       constexpr int N = decltype(count)::value;
       float v[N][VE];
 #pragma unroll
@@ -159,6 +197,7 @@ bn_bwd_stream(BnStreamArgs<S> a)
   cluster_resolve_tag(a.tag);
   const unsigned begin = static_cast<unsigned>(k) * a.share;
   const unsigned end = begin + a.share < a.E ? begin + a.share : a.E;
+  const unsigned rest = begin + kBnStreamKeepBwd<S> * kBnStreamThreads;
   for (int ch = cl; ch < a.C; ch += nc) {
     const S* xc = a.x + static_cast<int64_t>(ch) * a.cs;
     const S* gc = a.dy + static_cast<int64_t>(ch) * a.cs;
@@ -167,7 +206,31 @@ bn_bwd_stream(BnStreamArgs<S> a)
     const float inv_stdev = 1.0f / sqrtf(a.var[ch] + a.eps);
     const float scale = a.scale[ch];
     float sa = 0.f, sb = 0.f;
-    bn_stream_walk<U>(begin, end, [&](unsigned e, auto count) {
+    typename IO::raw_t kept_x[kBnStreamKeepBwd<S>], kept_g[kBnStreamKeepBwd<S>];
+#pragma unroll
+    for (int i = 0; i < kBnStreamKeepBwd<S>; ++i) {
+      const unsigned e = begin + threadIdx.x + i * kBnStreamThreads;
+      kept_x[i] = typename IO::raw_t{};
+      kept_g[i] = typename IO::raw_t{};
+      if (e < end) {
+        kept_x[i] = IO::load_raw(xc + bn_stream_offset<S>(e, a.seg, a.ldx));
+        kept_g[i] = IO::load_raw(gc + bn_stream_offset<S>(e, a.seg, a.lddy));
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kBnStreamKeepBwd<S>; ++i) {
+      if (begin + threadIdx.x + i * kBnStreamThreads < end) {
+        float x[VE], g[VE];
+        IO::unpack(kept_x[i], x);
+        IO::unpack(kept_g[i], g);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          sa += g[j];
+          sb = __builtin_fmaf(g[j], x[j] - mean, sb);
+        }
+      }
+    }
+    bn_stream_walk<U>(rest, end, [&](unsigned e, auto count) {
       constexpr int N = decltype(count)::value;
       float x[N][VE], g[N][VE];
 #pragma unroll
@@ -207,7 +270,19 @@ bn_bwd_stream(BnStreamArgs<S> a)
     const float dmean_term = bc[0];
     const float dvar_term = bc[1];
     const float k0 = scale * inv_stdev;
-    bn_stream_walk<U>(begin, end, [&](unsigned e, auto count) {
+#pragma unroll
+    for (int i = 0; i < kBnStreamKeepBwd<S>; ++i) {
+      const unsigned e = begin + threadIdx.x + i * kBnStreamThreads;
+      if (e < end) {
+        float x[VE], g[VE];
+        IO::unpack(kept_x[i], x);
+        IO::unpack(kept_g[i], g);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) g[j] = g[j] * k0 + dmean_term + dvar_term * (x[j] - mean);
+        IO::store(dc + bn_stream_offset<S>(e, a.seg, a.ldo), g);
+      }
+    }
+    bn_stream_walk<U>(rest, end, [&](unsigned e, auto count) {
       constexpr int N = decltype(count)::value;
       float x[N][VE], g[N][VE];
 #pragma unroll

@@ -864,8 +864,11 @@ static int ln_stream_launch(hipStream_t st, LnClArgs<T> a, int64_t rows, int64_t
   constexpr int VE = Vec16<T>::N;
   const int64_t nvec = n / VE;
   if (disabled || !ws || !aligned16(ws) || nvec >= (int64_t(1) << 31)) return 0;
-  const int cap = BWD ? cluster_capacity(ln_bwd_stream<T>, kLnStreamThreads)
-                      : cluster_capacity(ln_fwd_stream<T>, kLnStreamThreads);
+  const bool affine = a.gamma || a.beta;
+  const int cap = BWD ? (affine ? cluster_capacity(ln_bwd_stream<T, true>, kLnStreamThreads)
+                                : cluster_capacity(ln_bwd_stream<T, false>, kLnStreamThreads))
+                      : (affine ? cluster_capacity(ln_fwd_stream<T, true>, kLnStreamThreads)
+                                : cluster_capacity(ln_fwd_stream<T, false>, kLnStreamThreads));
   int64_t M = cap < kLnClMaxM ? cap : kLnClMaxM;
   if (M < 1) return 0;
   int64_t nc = cap / M;
@@ -879,8 +882,10 @@ static int ln_stream_launch(hipStream_t st, LnClArgs<T> a, int64_t rows, int64_t
   a.cw = cluster_workspace(ws);
   a.tag = cluster_call_tag(st, a.cw);
   const dim3 grid(static_cast<unsigned>(nc * M));
-  if (BWD) hipLaunchKernelGGL(ln_bwd_stream<T>, grid, dim3(kLnStreamThreads), 0, st, a);
-  else hipLaunchKernelGGL(ln_fwd_stream<T>, grid, dim3(kLnStreamThreads), 0, st, a);
+  if (BWD && affine) hipLaunchKernelGGL((ln_bwd_stream<T, true>), grid, dim3(kLnStreamThreads), 0, st, a);
+  else if (BWD) hipLaunchKernelGGL((ln_bwd_stream<T, false>), grid, dim3(kLnStreamThreads), 0, st, a);
+  else if (affine) hipLaunchKernelGGL((ln_fwd_stream<T, true>), grid, dim3(kLnStreamThreads), 0, st, a);
+  else hipLaunchKernelGGL((ln_fwd_stream<T, false>), grid, dim3(kLnStreamThreads), 0, st, a);
   return 1;
 }
 

@@ -535,6 +535,11 @@ namespace lbn {
 constexpr int kLnStreamThreads = 512;
 constexpr int kLnStreamWaves = kLnStreamThreads / kWave;
 constexpr int kLnStreamUnroll = 4;
+// Vectors per thread at the head of a workgroup's share that stay in registers between the
+// two passes (16.8 M-entry rows over 128 workgroups are 64 vectors per thread, 4.1 M-entry rows
+// 16: the latter are then read once).
+constexpr int kLnStreamKeepFwd = 16;
+constexpr int kLnStreamKeepBwd = 8;
 
 template <int U, typename F>
 __device__ __forceinline__ void ln_stream_walk(unsigned begin, unsigned end, F&& f)
@@ -544,21 +549,24 @@ __device__ __forceinline__ void ln_stream_walk(unsigned begin, unsigned end, F&&
   for (; e < end; e += kLnStreamThreads) f(e, std::integral_constant<int, 1>{});
 }
 
-template <typename T>
+// AFFINE = false (instance norm, layer norm without weights): no loads, the fill value only.
+template <typename T, bool AFFINE>
 __device__ __forceinline__ void ln_stream_weights(const float* w, unsigned e, float fill, float (&out)[Vec16<T>::N])
 {
   constexpr int VE = Vec16<T>::N;
 #pragma unroll
   for (int k = 0; k < VE; ++k) out[k] = fill;
-  if (w) load_f32_run<VE>(w + VE * static_cast<int64_t>(e), out);
+  if (AFFINE && w) load_f32_run<VE>(w + VE * static_cast<int64_t>(e), out);
 }
 
-template <typename T>
+template <typename T, bool AFFINE>
 __global__ void __launch_bounds__(kLnStreamThreads)
 ln_fwd_stream(LnClArgs<T> a)
 {
   using IO = Vec16<T>;
   constexpr int VE = IO::N;
+  // with weights the second pass also holds their loads: half the cache keeps it off the stack
+  constexpr int KEEP = AFFINE ? kLnStreamKeepFwd / 2 : kLnStreamKeepFwd;
   __shared__ float red[2 * kLnStreamWaves];
   __shared__ float bc[2];
   const int64_t nc = gridDim.x / a.M;
@@ -568,12 +576,34 @@ ln_fwd_stream(LnClArgs<T> a)
   cluster_resolve_tag(a.tag);
   const unsigned begin = static_cast<unsigned>(k) * a.per_wg;
   const unsigned end = begin + a.per_wg < a.nvec ? begin + a.per_wg : a.nvec;
+  const unsigned rest_fwd = begin + KEEP * kLnStreamThreads;  // where streaming takes over
   for (int64_t row = cl; row < a.rows; row += nc) {
     const T* xr = a.x + a.map.offset(row, a.ldx);
     T* yr = a.out + a.map.offset(row, a.ldo);
     const float K = a.sumsq ? 0.f : IO::load1(xr);
     float s = 0.f, q = 0.f;
-    ln_stream_walk<kLnStreamUnroll>(begin, end, [&](unsigned e, auto count) {
+    // the head of the share stays in registers for the second pass
+    typename IO::raw_t kept[KEEP];
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+      const unsigned e = begin + threadIdx.x + i * kLnStreamThreads;
+      kept[i] = typename IO::raw_t{};
+      if (e < end) kept[i] = IO::load_raw(xr + VE * static_cast<int64_t>(e));
+    }
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+      if (begin + threadIdx.x + i * kLnStreamThreads < end) {
+        float v[VE];
+        IO::unpack(kept[i], v);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          const float d = v[j] - K;
+          s += d;
+          q = __builtin_fmaf(d, d, q);
+        }
+      }
+    }
+    ln_stream_walk<kLnStreamUnroll>(rest_fwd, end, [&](unsigned e, auto count) {
       constexpr int N = decltype(count)::value;
       float v[N][VE];
 #pragma unroll
@@ -613,7 +643,20 @@ ln_fwd_stream(LnClArgs<T> a)
     __syncthreads();
     const float mean = bc[0];
     const float inv_stdev = bc[1];
-    ln_stream_walk<kLnStreamUnroll>(begin, end, [&](unsigned e, auto count) {
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+      const unsigned e = begin + threadIdx.x + i * kLnStreamThreads;
+      if (e < end) {
+        float v[VE], ga[VE], be[VE];
+        IO::unpack(kept[i], v);
+        ln_stream_weights<T, AFFINE>(a.gamma, e, 1.f, ga);
+        ln_stream_weights<T, AFFINE>(a.beta, e, 0.f, be);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) v[j] = __builtin_fmaf((v[j] - mean) * inv_stdev, ga[j], be[j]);
+        IO::store(yr + VE * static_cast<int64_t>(e), v);
+      }
+    }
+    ln_stream_walk<kLnStreamUnroll>(rest_fwd, end, [&](unsigned e, auto count) {
       constexpr int N = decltype(count)::value;
       float v[N][VE];
 #pragma unroll
@@ -621,8 +664,8 @@ ln_fwd_stream(LnClArgs<T> a)
 #pragma unroll
       for (int u = 0; u < N; ++u) {
         float ga[VE], be[VE];
-        ln_stream_weights<T>(a.gamma, e + u * kLnStreamThreads, 1.f, ga);
-        ln_stream_weights<T>(a.beta, e + u * kLnStreamThreads, 0.f, be);
+        ln_stream_weights<T, AFFINE>(a.gamma, e + u * kLnStreamThreads, 1.f, ga);
+        ln_stream_weights<T, AFFINE>(a.beta, e + u * kLnStreamThreads, 0.f, be);
 #pragma unroll
         for (int j = 0; j < VE; ++j) v[u][j] = __builtin_fmaf((v[u][j] - mean) * inv_stdev, ga[j], be[j]);
         IO::store(yr + VE * static_cast<int64_t>(e + u * kLnStreamThreads), v[u]);
@@ -633,7 +676,7 @@ ln_fwd_stream(LnClArgs<T> a)
 }
 
 // Backward without weight gradients.
-template <typename T>
+template <typename T, bool AFFINE>
 __global__ void __launch_bounds__(kLnStreamThreads)
 ln_bwd_stream(LnClArgs<T> a)
 {
@@ -649,6 +692,7 @@ ln_bwd_stream(LnClArgs<T> a)
   cluster_resolve_tag(a.tag);
   const unsigned begin = static_cast<unsigned>(k) * a.per_wg;
   const unsigned end = begin + a.per_wg < a.nvec ? begin + a.per_wg : a.nvec;
+  const unsigned rest_bwd = begin + kLnStreamKeepBwd * kLnStreamThreads;
   for (int64_t row = cl; row < a.rows; row += nc) {
     int64_t col, g;
     a.map.split(row, col, g);
@@ -658,7 +702,34 @@ ln_bwd_stream(LnClArgs<T> a)
     const float mean = a.stats[g + col * a.ld_stats];
     const float inv_stdev = 1.0f / sqrtf(a.stats[a.map.groups + g + col * a.ld_stats] + a.eps);
     float sa = 0.f, sb = 0.f;
-    ln_stream_walk<U>(begin, end, [&](unsigned e, auto count) {
+    typename IO::raw_t kept_x[kLnStreamKeepBwd], kept_g[kLnStreamKeepBwd];
+#pragma unroll
+    for (int i = 0; i < kLnStreamKeepBwd; ++i) {
+      const unsigned e = begin + threadIdx.x + i * kLnStreamThreads;
+      kept_x[i] = typename IO::raw_t{};
+      kept_g[i] = typename IO::raw_t{};
+      if (e < end) {
+        kept_x[i] = IO::load_raw(xr + VE * static_cast<int64_t>(e));
+        kept_g[i] = IO::load_raw(gr + VE * static_cast<int64_t>(e));
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kLnStreamKeepBwd; ++i) {
+      const unsigned e = begin + threadIdx.x + i * kLnStreamThreads;
+      if (e < end) {
+        float x[VE], d[VE], ga[VE];
+        IO::unpack(kept_x[i], x);
+        IO::unpack(kept_g[i], d);
+        ln_stream_weights<T, AFFINE>(a.gamma, e, 1.f, ga);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          const float gs = d[j] * ga[j];
+          sa += gs;
+          sb = __builtin_fmaf(gs, (x[j] - mean) * inv_stdev, sb);
+        }
+      }
+    }
+    ln_stream_walk<U>(rest_bwd, end, [&](unsigned e, auto count) {
       constexpr int N = decltype(count)::value;
       float x[N][VE], d[N][VE];
 #pragma unroll
@@ -669,7 +740,7 @@ ln_bwd_stream(LnClArgs<T> a)
 #pragma unroll
       for (int u = 0; u < N; ++u) {
         float ga[VE];
-        ln_stream_weights<T>(a.gamma, e + u * kLnStreamThreads, 1.f, ga);
+        ln_stream_weights<T, AFFINE>(a.gamma, e + u * kLnStreamThreads, 1.f, ga);
 #pragma unroll
         for (int j = 0; j < VE; ++j) {
           const float gs = d[u][j] * ga[j];
@@ -697,7 +768,23 @@ ln_bwd_stream(LnClArgs<T> a)
     __syncthreads();
     const float c0 = bc[0];
     const float c1 = bc[1];
-    ln_stream_walk<U>(begin, end, [&](unsigned e, auto count) {
+#pragma unroll
+    for (int i = 0; i < kLnStreamKeepBwd; ++i) {
+      const unsigned e = begin + threadIdx.x + i * kLnStreamThreads;
+      if (e < end) {
+        float x[VE], d[VE], ga[VE];
+        IO::unpack(kept_x[i], x);
+        IO::unpack(kept_g[i], d);
+        ln_stream_weights<T, AFFINE>(a.gamma, e, 1.f, ga);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          const float xh = (x[j] - mean) * inv_stdev;
+          d[j] = __builtin_fmaf(d[j] * ga[j], inv_stdev, __builtin_fmaf(c1, xh, c0));
+        }
+        IO::store(dr + VE * static_cast<int64_t>(e), d);
+      }
+    }
+    ln_stream_walk<U>(rest_bwd, end, [&](unsigned e, auto count) {
       constexpr int N = decltype(count)::value;
       float x[N][VE], d[N][VE];
 #pragma unroll
@@ -708,7 +795,7 @@ ln_bwd_stream(LnClArgs<T> a)
 #pragma unroll
       for (int u = 0; u < N; ++u) {
         float ga[VE];
-        ln_stream_weights<T>(a.gamma, e + u * kLnStreamThreads, 1.f, ga);
+        ln_stream_weights<T, AFFINE>(a.gamma, e + u * kLnStreamThreads, 1.f, ga);
 #pragma unroll
         for (int j = 0; j < VE; ++j) {
           const float xh = (x[u][j] - mean) * inv_stdev;
