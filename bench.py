@@ -217,6 +217,31 @@ def main():
             return t1 - t0, t2 - t1
         return layer, data["x"].size, 4, data["x"].shape[1], cpu
 
+    def build_sink(h, w):
+        """The optimizer's gradient buffer taking a (h x w) contribution: "forward" is the first
+        contribution of a step (cleared buffer: overwrite, 2 tensors of traffic), "backward" a later
+        one (ready buffer: accumulate, 3 tensors)."""
+        rng = np.random.default_rng(13)
+        c = np.asfortranarray(rng.standard_normal((w, h)).astype(np.float32).T)
+        g0 = np.asfortranarray(rng.standard_normal((w, h)).astype(np.float32).T)
+        contrib, grad = upload(c), upload(g0)
+
+        class sink:
+            def fp_call(self):
+                return "lbn_gradient_sink_f32", (L._stream(), h, w, 0.0, 1.0, contrib.Buffer(), contrib.ldim,
+                                                 grad.Buffer(), grad.ldim)
+
+            def bp_call(self):
+                return "lbn_gradient_sink_f32", (L._stream(), h, w, 1.0, 1.0, contrib.Buffer(), contrib.ldim,
+                                                 grad.Buffer(), grad.ldim)
+
+        def cpu():
+            from oracle import cpu_oracle as orc
+            t0 = time.perf_counter(); orc.gradient_sink(g0, c, 0.0, 1.0); t1 = time.perf_counter()
+            orc.gradient_sink(g0, c, 1.0, 1.0); t2 = time.perf_counter()
+            return t1 - t0, t2 - t1
+        return sink(), h * w, 4, w, cpu
+
     table = {
         "cfg2_softmax": ("Softmax fwd+bwd fp32 32768x512", lambda: build_softmax("softmax", W.cfg2_softmax())),
         "cfg2_log_softmax": ("LogSoftmax fwd+bwd fp32 32768x512", lambda: build_softmax("log_softmax", W.cfg2_softmax())),
@@ -253,6 +278,9 @@ def main():
                                  lambda: build_bn(W.cfg3_batch_norm(), True)),
         "extra_softmax_vocab_50257": ("Softmax fwd+bwd fp32 50257x1024, rows 4-byte aligned (informational)",
                                       lambda: build_softmax("softmax", W.cfg5b_wide_softmax(h=50257, w=1024))),
+        # not a baseline configuration: where weight gradients go next (a 4096 x 4096 weight matrix)
+        "extra_gradient_sink": ("Gradient buffer overwrite+accumulate fp32 4096x4096 (informational)",
+                                lambda: build_sink(4096, 4096)),
     }
     headline = "cfg2_softmax"
     if args.layers == "all":

@@ -370,6 +370,20 @@ int lbn_channelwise_scale_bias_bwd_f32(lbn_stream_t stream, int64_t channels, in
                                        float* weights_grad, int64_t ld_weights_grad,
                                        void* workspace, size_t workspace_bytes);
 
+/* ------------------------------------------------ the optimizer's gradient buffer
+ * Where dscale / dbias / weights_grad go next.  Replaces the Scale + Axpy pair of
+ * optimizer::add_to_gradient (include/lbann/optimizers/optimizer_impl.hpp:207-217) on
+ * the local (height x width, column-major) matrices:
+ *   gradient = buf_scale * gradient + in_scale * contribution
+ * with buf_scale and in_scale as get_gradient_buffer (:219-288) picks them from the
+ * buffer's status (cleared: 0 and 1; ready: 1 and 1), in_scale already multiplied by
+ * add_to_gradient's scale argument.  buf_scale == 0 overwrites: the buffer's previous
+ * contents are not read (they may never have been initialised).  Each product and the
+ * sum are rounded separately, like the two library calls. */
+int lbn_gradient_sink_f32(lbn_stream_t stream, int64_t height, int64_t width, float buf_scale,
+                          float in_scale, const float* contribution, int64_t ld_contribution,
+                          float* gradient, int64_t ld_gradient);
+
 #ifdef __cplusplus
 }
 #endif

@@ -10,7 +10,8 @@
 //   log_softmax_layer           src/layers/activations/log_softmax.cu
 //   channelwise_softmax_layer   src/layers/misc/channelwise_softmax.cu
 // and, beyond those five, instance_norm_layer, entrywise_batch_normalization_layer,
-// cross_entropy_layer, entrywise_scale_bias_layer and channelwise_scale_bias_layer.
+// cross_entropy_layer, entrywise_scale_bias_layer and channelwise_scale_bias_layer,
+// and gradient_buffer, where their weight gradients go (optimizer::add_to_gradient).
 //
 // `Mat` is any local-matrix type with the El::Matrix<T, El::Device::GPU> accessors
 //   Height(), Width(), LDim(), Buffer(), LockedBuffer()
@@ -755,6 +756,75 @@ private:
   const float* m_weights = nullptr;
   int64_t m_ld_weights = 0;
   workspace m_ws;
+};
+
+/// Where the layers' weight gradients go: optimizer::add_to_gradient and
+/// get_gradient_buffer (include/lbann/optimizers/optimizer_impl.hpp:207-288) with the
+/// status values of include/lbann/optimizers/optimizer.hpp:54-70, for one process: the
+/// buffer's RedundantSize is 1, so needing a synchronisation changes the status only.
+/// The buffer starts cleared; the first contribution overwrites it without reading it.
+enum class optimizer_gradient_status { ready, cleared, sync_needed, sync_started };
+
+class gradient_buffer {
+public:
+  gradient_buffer() = default;
+  gradient_buffer(int64_t height, int64_t width) { setup(height, width); }
+  void setup(int64_t height, int64_t width)
+  {
+    m_gradient.Resize(height, width);
+    m_status = optimizer_gradient_status::cleared;
+  }
+  /// View of a gradient matrix owned by someone else.
+  void attach(int64_t height, int64_t width, float* buffer, int64_t ldim)
+  {
+    m_gradient.Attach(height, width, buffer, ldim);
+    m_status = optimizer_gradient_status::cleared;
+  }
+  void clear() { m_status = optimizer_gradient_status::cleared; }
+  optimizer_gradient_status get_status() const { return m_status; }
+  void set_status(optimizer_gradient_status s) { m_status = s; }
+  device_matrix<float>& local_gradient() { return m_gradient; }
+
+  /// The factors for the buffer and for the contribution, and the status transition.
+  void get_gradient_scales(float& buf_scale, float& in_scale, bool sync_needed)
+  {
+    switch (m_status) {
+    case optimizer_gradient_status::ready:
+      buf_scale = 1.f; in_scale = 1.f;
+      if (sync_needed) m_status = optimizer_gradient_status::sync_needed;
+      break;
+    case optimizer_gradient_status::cleared:
+      buf_scale = 0.f; in_scale = 1.f;
+      m_status = sync_needed ? optimizer_gradient_status::sync_needed : optimizer_gradient_status::ready;
+      break;
+    case optimizer_gradient_status::sync_needed:
+      buf_scale = 1.f; in_scale = 1.f;
+      break;
+    default:
+      throw exception("unexpected gradient status (sync_started)");
+    }
+  }
+
+  /// contrib: height x width values with leading dimension ldim, in device memory.
+  void add_to_gradient(lbn_stream_t stream, const float* contrib, int64_t ldim, float scale = 1.f,
+                       bool sync_needed = false)
+  {
+    float buf_scale, in_scale;
+    get_gradient_scales(buf_scale, in_scale, sync_needed);
+    check_status(lbn_gradient_sink_f32(stream, m_gradient.Height(), m_gradient.Width(), buf_scale,
+                                       in_scale * scale, contrib, ldim, m_gradient.Buffer(), m_gradient.LDim()),
+                 "gradient_buffer::add_to_gradient");
+  }
+  template <typename Mat>
+  void add_to_gradient(lbn_stream_t stream, const Mat& contrib, float scale = 1.f, bool sync_needed = false)
+  {
+    if (contrib.Height() != m_gradient.Height() || contrib.Width() != m_gradient.Width())
+      throw exception("gradient_buffer::add_to_gradient: contribution has the wrong shape");
+    add_to_gradient(stream, contrib.LockedBuffer(), contrib.LDim(), scale, sync_needed);
+  }
+private:
+  device_matrix<float> m_gradient;
+  optimizer_gradient_status m_status = optimizer_gradient_status::cleared;
 };
 
 }  // namespace lbnorm

@@ -75,6 +75,7 @@ PROTOTYPES = {
     "lbn_channelwise_scale_bias_bwd_workspace_bytes": (sz, [i64, i64, i64]),
     "lbn_channelwise_scale_bias_bwd_f32": (cint, [vp, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, i64,
                                                   vp, sz]),
+    "lbn_gradient_sink_f32": (cint, [vp, i64, i64, f32, f32, vp, i64, vp, i64]),
 }
 
 _lib = None

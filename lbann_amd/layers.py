@@ -557,3 +557,58 @@ class cross_entropy_layer:
                                                                           device=self.device)]
         self.bp_compute()
         return self.error_signals
+
+
+class gradient_buffer:
+    """The optimizer's gradient buffer as the layers see it: optimizer::add_to_gradient and
+    get_gradient_buffer (include/lbann/optimizers/optimizer_impl.hpp:207-288) with their status
+    machine (include/lbann/optimizers/optimizer.hpp:54-70), for one process (RedundantSize = 1,
+    so a needed synchronisation changes the status and nothing else).
+
+    `gradient` is a (height x width) DeviceMatrix.  It starts `cleared`: the first contribution
+    overwrites it without reading it, later ones accumulate."""
+
+    READY, CLEARED, SYNC_NEEDED = "ready", "cleared", "sync_needed"
+
+    def __init__(self, height, width=1, device="cuda"):
+        self.gradient = DeviceMatrix(height, width, device=device)
+        self.status = self.CLEARED
+
+    def clear(self):
+        self.status = self.CLEARED
+
+    def _scales(self, sync_needed):
+        # (buf_scale, in_scale) and the status transition of get_gradient_buffer
+        if self.status == self.READY:
+            if sync_needed:
+                self.status = self.SYNC_NEEDED
+            return 1.0, 1.0
+        if self.status == self.CLEARED:
+            self.status = self.SYNC_NEEDED if sync_needed else self.READY
+            return 0.0, 1.0
+        if self.status == self.SYNC_NEEDED:
+            return 1.0, 1.0
+        raise ValueError(f"unexpected gradient status ({self.status})")
+
+    def add_to_gradient(self, contrib, scale=1.0, sync_needed=False, ldim=None):
+        """contrib: a DeviceMatrix of the buffer's shape, or a _Vector / torch tensor holding one column
+        (then `ldim` is its leading dimension when the buffer has several columns)."""
+        g = self.gradient
+        buf_scale, in_scale = self._scales(sync_needed)
+        if isinstance(contrib, DeviceMatrix):
+            if (contrib.height, contrib.width) != (g.height, g.width):
+                raise ValueError("gradient contribution has the wrong shape")
+            ptr, ld = contrib.Buffer(), contrib.ldim
+        else:
+            t = contrib.tensor if hasattr(contrib, "tensor") else contrib
+            ld = int(ldim) if ldim is not None else g.height
+            if t.numel() < (g.width - 1) * ld + g.height:
+                raise ValueError("gradient contribution is too small")
+            ptr = capi.vp(t.data_ptr())
+        call("lbn_gradient_sink_f32", _stream(), g.height, g.width, buf_scale, in_scale * float(scale), ptr, ld,
+             g.Buffer(), g.ldim)
+
+    def finish_sync(self):
+        """What the all-reduce completes on several processes; here the values are already final."""
+        if self.status == self.SYNC_NEEDED:
+            self.status = self.READY

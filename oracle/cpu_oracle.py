@@ -296,3 +296,14 @@ def channelwise_scale_bias_bwd(x, dy, weights, C, cs):
     getattr(lib(), f"orc_channelwise_scale_bias_bwd_{suf}")(
         _i64(C), _i64(cs), _i64(w), *_mat(x), *_mat(dy), *_mat(dx), *_mat(weights), *_mat(wgrad))
     return dx, wgrad
+
+
+def gradient_sink(gradient, contribution, buf_scale, alpha):
+    """gradient = buf_scale * gradient + alpha * contribution as Scale + Axpy; returns the new gradient."""
+    suf, cf = _suffix(contribution)
+    h, w = contribution.shape
+    g = np.array(gradient, dtype=contribution.dtype, order="F", copy=True)
+    assert g.shape == (h, w)
+    getattr(lib(), f"orc_gradient_sink_{suf}")(
+        _i64(h), _i64(w), cf(buf_scale), cf(alpha), *_mat(contribution), *_mat(g))
+    return g

@@ -32,6 +32,7 @@
 //   cross entropy   src/layers/loss/cross_entropy.cpp:35-73 (fwd), :75-120 (bwd)
 //   entry-wise scale/bias    src/layers/learning/entrywise_scale_bias.cpp:35-60, :62-113
 //   channel-wise scale/bias  src/layers/learning/channelwise_scale_bias.cpp:33-73, :75-135
+//   gradient buffer update   include/lbann/optimizers/optimizer_impl.hpp:207-217
 
 #include <algorithm>
 #include <cmath>
@@ -797,6 +798,27 @@ void csb_bwd(idx C, idx cs, idx w, CMat<T> x, CMat<T> dy, Mat<T> dx, CMat<T> wei
   }
 }
 
+// ------------------------------------------------------- gradient buffer update
+// optimizer::add_to_gradient (optimizer_impl.hpp:207-217): El::Scale(buf_scale, grad) then
+// El::Axpy(alpha, contrib, grad), on local matrices.  Hydrogen (>= 1.5.0, not part of the
+// reference tree) documents Scale by zero as zeroing the matrix whatever it held, and by
+// one as a no-op; Axpy is y += alpha * x element by element.  Two statements, so that the
+// scaled buffer is rounded before the sum as with the two calls.
+template <typename T>
+void grad_sink(idx h, idx w, T buf_scale, T alpha, CMat<T> contrib, Mat<T> grad)
+{
+  for (idx c = 0; c < w; ++c)
+    for (idx r = 0; r < h; ++r) {
+      if (buf_scale == T(0)) grad(r, c) = T(0);
+      else if (buf_scale != T(1)) grad(r, c) = buf_scale * grad(r, c);
+    }
+  for (idx c = 0; c < w; ++c)
+    for (idx r = 0; r < h; ++r) {
+      const T t = alpha * contrib(r, c);
+      grad(r, c) = grad(r, c) + t;
+    }
+}
+
 }  // namespace
 
 // C interface (one _f32 and one _f64 entry per function), bound by oracle/cpu_oracle.py.
@@ -876,7 +898,10 @@ void csb_bwd(idx C, idx cs, idx w, CMat<T> x, CMat<T> dy, Mat<T> dx, CMat<T> wei
       idx ldx, const T* dy, idx lddy, T* dx, idx lddx, const T* weights, idx ldw,        \
       T* wgrad, idx ldwg)                                                                \
   { csb_bwd<T>(C, cs, w, {x, ldx}, {dy, lddy}, {dx, lddx}, {weights, ldw},               \
-               {wgrad, ldwg}); }
+               {wgrad, ldwg}); }                                                         \
+  extern "C" void orc_gradient_sink_##SUF(idx h, idx w, T buf_scale, T alpha,             \
+      const T* contrib, idx ldc, T* grad, idx ldg)                                       \
+  { grad_sink<T>(h, w, buf_scale, alpha, {contrib, ldc}, {grad, ldg}); }
 
 ORC_INSTANTIATE(f32, float)
 ORC_INSTANTIATE(f64, double)

@@ -252,9 +252,65 @@ int drv_scale_bias(int kind, const int64_t* dims, int nd, int64_t h, int64_t w, 
 
 // Host-only checks of the error behaviour the reference has: returns the number of
 // cases that did NOT throw as they should.
+// Channel-wise scale/bias backward twice on the same inputs, the weight gradient handed to an
+// attached gradient buffer each time with factors `scale0`, `scale1`: gradient_out (C x 2)
+// ends as scale0 * dW + scale1 * dW, statuses[k] the buffer's status after step k.
+int drv_gradient_buffer(const int64_t* dims, int nd, int64_t h, int64_t w, const float* x, const float* dy,
+                        float* dx, const float* weights, float* gradient_out, int64_t ld_gradient, float scale0,
+                        float scale1, int* statuses, void* stream, char* err, int errlen)
+{
+  try {
+    channelwise_scale_bias_layer<> layer;
+    layer.setup(std::vector<int64_t>(dims, dims + nd));
+    layer.set_weights(weights, dims[0]);
+    device_matrix<float> mx, mdy, mdx;
+    mx.Attach(h, w, const_cast<float*>(x), h);
+    mdy.Attach(h, w, const_cast<float*>(dy), h);
+    mdx.Attach(h, w, dx, h);
+    layer.io.stream = static_cast<hipStream_t>(stream);
+    layer.io.prev_activations = &mx;
+    layer.io.prev_error_signals = &mdy;
+    layer.io.error_signals = &mdx;
+    gradient_buffer sink;
+    sink.attach(dims[0], 2, gradient_out, ld_gradient);
+    const float scales[2] = {scale0, scale1};
+    for (int k = 0; k < 2; ++k) {
+      layer.bp_compute();
+      sink.add_to_gradient(stream, layer.m_weights_gradient, scales[k], k == 1);
+      statuses[k] = static_cast<int>(sink.get_status());
+    }
+    return 0;
+  } catch (const std::exception& e) {
+    return fail(e, err, errlen);
+  }
+}
+
 int drv_error_cases(void)
 {
   int missed = 0;
+  {
+    // the gradient buffer's status machine (optimizer_impl.hpp:262-287), no device touched
+    gradient_buffer b;
+    float bs = -1.f, is = -1.f;
+    using S = optimizer_gradient_status;
+    if (b.get_status() != S::cleared) ++missed;
+    b.get_gradient_scales(bs, is, false);
+    if (bs != 0.f || is != 1.f || b.get_status() != S::ready) ++missed;
+    b.get_gradient_scales(bs, is, true);
+    if (bs != 1.f || is != 1.f || b.get_status() != S::sync_needed) ++missed;
+    b.get_gradient_scales(bs, is, false);
+    if (bs != 1.f || is != 1.f || b.get_status() != S::sync_needed) ++missed;
+    b.clear();
+    b.get_gradient_scales(bs, is, true);
+    if (bs != 0.f || b.get_status() != S::sync_needed) ++missed;
+    b.set_status(S::sync_started);
+    try { b.get_gradient_scales(bs, is, false); ++missed; } catch (const exception&) {}
+    device_matrix<float> wrong;
+    wrong.Attach(3, 1, nullptr, 3);
+    gradient_buffer c;
+    c.attach(4, 1, nullptr, 4);
+    try { c.add_to_gradient(nullptr, wrong); ++missed; } catch (const exception&) {}
+  }
   try { softmax_layer<> l(softmax_mode::CHANNEL); ++missed; } catch (const exception&) {}
   try { layer_norm_layer<float> l(1e-5, false, false, 2); l.setup({4, 4}); ++missed; } catch (const exception&) {}
   try { layer_norm_layer<float> l(1e-5, false, false, -3); l.setup({4, 4}); ++missed; } catch (const exception&) {}

@@ -14,6 +14,9 @@ i64, vp, cint, dbl = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_dou
 
 def driver():
     assert os.path.exists(DRIVER), "build it with `python -m lbann_amd.build`"
+    # torch first: it brings its own HIP runtime, and the driver must bind to that one
+    # rather than pull a second runtime into the process
+    import torch  # noqa: F401
     return ctypes.CDLL(DRIVER)
 
 
@@ -206,3 +209,27 @@ def test_adapter_layers_match_oracle():
         check(f"adapter scale/bias {kind} y", my.to_numpy(), y_ref)
         check(f"adapter scale/bias {kind} dx", mdx.to_numpy(), dx_ref)
         check(f"adapter scale/bias {kind} dweights", mwg.to_numpy(), wg_ref)
+
+    # ---- channel-wise scale/bias weight gradients into a gradient buffer, twice
+    wts = np.asfortranarray(np.stack([rng.normal(1, 1, 8), rng.normal(0, 1, 8)], axis=1).astype(np.float32))
+    mx, mdy, mdx = DeviceMatrix.from_numpy(x), DeviceMatrix.from_numpy(dy), DeviceMatrix(h, w)
+    mw, grad = DeviceMatrix.from_numpy(wts), DeviceMatrix(8, 2, ldim=12, fill=float("nan"))
+    statuses = (ctypes.c_int * 2)()
+    da, nd = _dims(dims)
+    rc = d.drv_gradient_buffer(da, cint(nd), i64(h), i64(w), mx.Buffer(), mdy.Buffer(), mdx.Buffer(), mw.Buffer(),
+                               grad.Buffer(), i64(12), ctypes.c_float(0.5), ctypes.c_float(-2.0), statuses, st, err,
+                               cint(512))
+    assert rc == 0, err.value
+    assert list(statuses) == [0, 2]          # ready after the first contribution, sync_needed after the second
+    _, wg_ref = orc.channelwise_scale_bias_bwd(x, dy, wts, 8, 144)
+    wg_dev = None
+    # the buffer holds Scale + Axpy of the device's own weight gradient, to the bit
+    mwg = DeviceMatrix(8, 2)
+    rc = d.drv_scale_bias(cint(1), da, cint(nd), i64(h), i64(w), i64(h), mx.Buffer(), DeviceMatrix(h, w).Buffer(),
+                          mdy.Buffer(), mdx.Buffer(), mw.Buffer(), i64(8), mwg.Buffer(), st, err, cint(512))
+    assert rc == 0, err.value
+    wg_dev = mwg.to_numpy()
+    exp = orc.gradient_sink(orc.gradient_sink(np.zeros((8, 2), np.float32), wg_dev, 0.0, 0.5), wg_dev, 1.0, -2.0)
+    assert grad.to_numpy().tobytes() == exp.tobytes()
+    check("adapter gradient buffer", grad.to_numpy(), -1.5 * wg_ref)
+    assert torch.isnan(grad.tensor[:, 8:]).all()

@@ -223,3 +223,85 @@ def test_neighbour_layers_empty_and_rejected_arguments(L):
     assert lib.lbn_entrywise_scale_bias_bwd_f32(st, 64, 8192, pb, 64, pb, 64, pb, 64, p, 64, p, 64, null, 0) == capi.LBN_ERR_WORKSPACE
     assert lib.lbn_cross_entropy_fwd_f32(st, 65536, 8, 0, 1, pb, 65536, pb, 65536, p, 1, null, 0) == capi.LBN_ERR_WORKSPACE
     torch.cuda.synchronize()
+
+
+# ===================================================================== gradient buffer
+SINK_SHAPES = [
+    # (h, w, contribution pad, gradient pad)
+    (4096, 1, 0, 0), (8192, 2, 0, 0), (37, 5, 0, 0), (37, 5, 3, 1), (1, 1, 0, 0), (256, 2, 4, 8),
+    (1026, 3, 2, 2), (3, 1000, 0, 1), (1 << 22, 1, 0, 0), ((1 << 21) + 1, 2, 0, 0), (2048, 2048, 0, 0),
+]
+
+
+@pytest.mark.parametrize("h,w,cpad,gpad", SINK_SHAPES)
+def test_gradient_sink_bit_exact(L, h, w, cpad, gpad):
+    """lbn_gradient_sink_f32 against the oracle's Scale + Axpy: same bits, padding untouched."""
+    from lbann_amd import capi
+    rng = np.random.default_rng(h + 31 * w)
+    c = rand(rng, h, w)
+    c[0, 0] = -0.0
+    g0 = rand(rng, h, w)
+    st = capi.vp(torch.cuda.current_stream().cuda_stream)
+    dc = L.DeviceMatrix.from_numpy(c, ldim=h + cpad)
+    for buf_scale, alpha in ((1.0, 1.0), (0.0, 1.0), (1.0, 0.37), (0.0, -2.5), (-1.25, 0.37)):
+        dg = L.DeviceMatrix(h, w, ldim=h + gpad, fill=float("nan") if buf_scale == 0.0 else 123.0)
+        if buf_scale != 0.0:
+            dg.tensor[:, :h] = torch.from_numpy(np.ascontiguousarray(g0.T)).cuda()
+        assert capi.lib().lbn_gradient_sink_f32(st, h, w, buf_scale, alpha, dc.Buffer(), dc.ldim, dg.Buffer(), dg.ldim) == 0
+        got = dg.to_numpy()
+        exp = orc.gradient_sink(g0, c, buf_scale, alpha)
+        assert got.tobytes() == np.asfortranarray(exp).tobytes(), (buf_scale, alpha, rel_err(got, exp))
+        if gpad:
+            pad = dg.tensor[:, h:].cpu().numpy()
+            assert (np.isnan(pad).all() if buf_scale == 0.0 else (pad == 123.0).all())
+
+
+def test_gradient_buffer_takes_layer_norm_weight_gradients(L):
+    """Two mini-batches through layer norm's backward, dscale / dbias handed to gradient
+    buffers as the reference's bp_compute does (layer_norm.cpp:342-343): the first
+    contribution overwrites an uninitialised buffer, the second accumulates."""
+    rng = np.random.default_rng(342)
+    n, w = 1024, 48
+    gamma = rng.standard_normal(n).astype(np.float32)
+    beta = rng.standard_normal(n).astype(np.float32)
+    layer = L.layer_norm_layer((n,), scale=True, bias=True, scale_values=gamma, bias_values=beta)
+    sink_s, sink_b = L.gradient_buffer(n), L.gradient_buffer(n)
+    sink_s.gradient.tensor.fill_(float("nan"))
+    sink_b.gradient.tensor.fill_(float("nan"))
+    exp_s = exp_b = None
+    for step in range(2):
+        x, dy = rand(rng, n, w, 0.5, 2.0), rand(rng, n, w)
+        layer.forward(L.DeviceMatrix.from_numpy(x))
+        layer.backward(L.DeviceMatrix.from_numpy(dy))
+        ds, db = layer.m_scale_gradient.to_numpy().reshape(n, 1), layer.m_bias_gradient.to_numpy().reshape(n, 1)
+        sink_s.add_to_gradient(layer.m_scale_gradient, scale=1.0, sync_needed=True)
+        sink_b.add_to_gradient(layer.m_bias_gradient, scale=1.0, sync_needed=True)
+        exp_s = orc.gradient_sink(np.zeros((n, 1), np.float32) if step == 0 else exp_s, f32(ds), float(step), 1.0)
+        exp_b = orc.gradient_sink(np.zeros((n, 1), np.float32) if step == 0 else exp_b, f32(db), float(step), 1.0)
+        assert sink_s.status == sink_s.SYNC_NEEDED
+    assert sink_s.gradient.to_numpy().tobytes() == exp_s.tobytes()
+    assert sink_b.gradient.to_numpy().tobytes() == exp_b.tobytes()
+    sink_s.finish_sync()
+    sink_s.clear()
+    assert sink_s.status == sink_s.CLEARED
+    wrong = L.DeviceMatrix(n + 1, 1, fill=0.0)
+    with pytest.raises(ValueError):
+        sink_s.add_to_gradient(wrong)
+
+
+def test_gradient_sink_empty_and_rejected_arguments(L):
+    from lbann_amd import capi
+    st = capi.vp(torch.cuda.current_stream().cuda_stream)
+    null = capi.vp(None)
+    lib = capi.lib()
+    buf = torch.zeros(4096, device="cuda")
+    p = capi.vp(buf.data_ptr())
+    assert lib.lbn_gradient_sink_f32(st, 0, 4, 1.0, 1.0, null, 1, null, 1) == 0
+    assert lib.lbn_gradient_sink_f32(st, 4, 0, 1.0, 1.0, null, 4, null, 4) == 0
+    assert lib.lbn_gradient_sink_f32(st, -1, 4, 1.0, 1.0, p, 4, p, 4) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_gradient_sink_f32(st, 8, 4, 1.0, 1.0, p, 4, p, 8) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_gradient_sink_f32(st, 8, 4, 1.0, 1.0, p, 8, p, 4) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_gradient_sink_f32(st, 8, 4, 1.0, 1.0, null, 8, p, 8) == capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_gradient_sink_f32(st, 8, 4, 1.0, 1.0, p, 8, null, 8) == capi.LBN_ERR_INVALID_ARGUMENT
+    torch.cuda.synchronize()
+    assert float(buf.abs().sum()) == 0.0

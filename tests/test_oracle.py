@@ -597,3 +597,58 @@ def test_scale_bias_backward_matches_autograd():
     gx, gw = torch.autograd.grad((y * tdy).sum(), (tx, tw))
     dx, wg = orc.channelwise_scale_bias_bwd(x, dy, wts, C, cs)
     assert np.allclose(dx, gx.numpy(), rtol=1e-12) and np.allclose(wg, gw.numpy(), rtol=1e-11, atol=1e-13)
+
+
+# ------------------------------------------------------------- gradient buffer update
+def test_gradient_sink_against_elementwise_arithmetic():
+    """Scale + Axpy of optimizer::add_to_gradient, checked against numpy's own float32
+    arithmetic (each product and the sum rounded once) and against what the two library
+    calls fix: a scale of zero discards NaN/Inf already in the buffer, a scale of one
+    leaves the buffer's bits alone, a product of -0 lands as +0 on a zeroed buffer."""
+    rng = np.random.default_rng(207)
+    h, w = 37, 5
+    g = np.asfortranarray(rng.standard_normal((h, w)).astype(np.float32))
+    c = np.asfortranarray(rng.standard_normal((h, w)).astype(np.float32))
+    a = np.float32(0.37)
+    # ready buffer: g + a * c
+    out = orc.gradient_sink(g, c, 1.0, a)
+    assert out.tobytes() == (g + a * c).astype(np.float32).tobytes()
+    # general factor: two roundings on the buffer side
+    b = np.float32(-1.25)
+    out = orc.gradient_sink(g, c, b, a)
+    assert out.tobytes() == ((b * g).astype(np.float32) + (a * c).astype(np.float32)).tobytes()
+    # cleared buffer: contents are not read
+    dirty = g.copy(order="F")
+    dirty[3, 1], dirty[0, 0], dirty[5, 4] = np.nan, np.inf, -np.inf
+    out = orc.gradient_sink(dirty, c, 0.0, a)
+    assert out.tobytes() == (np.float32(0) + (a * c).astype(np.float32)).tobytes()
+    assert np.isfinite(out).all()
+    zc = np.zeros((h, w), dtype=np.float32, order="F")
+    zc[2, 2] = -0.0
+    out = orc.gradient_sink(dirty, zc, 0.0, 1.0)
+    assert not np.signbit(out).any()
+    # the input gradient is not modified, the contribution's padding is skipped
+    wide = np.asfortranarray(rng.standard_normal((h + 3, w)).astype(np.float32))
+    out = orc.gradient_sink(g, wide[:h], 1.0, 2.0)
+    assert np.array_equal(out, g + np.float32(2) * wide[:h])
+    # float64 instance
+    out = orc.gradient_sink(g.astype(np.float64), c.astype(np.float64), 1.0, 0.5)
+    assert np.array_equal(out, g.astype(np.float64) + 0.5 * c.astype(np.float64))
+
+
+def test_gradient_buffer_status_machine():
+    """get_gradient_buffer's choice of factors (optimizer_impl.hpp:219-288) on the host."""
+    from lbann_amd.layers import gradient_buffer as GB
+    b = GB.__new__(GB)
+    b.status = GB.CLEARED
+    assert b._scales(False) == (0.0, 1.0) and b.status == GB.READY
+    assert b._scales(False) == (1.0, 1.0) and b.status == GB.READY
+    assert b._scales(True) == (1.0, 1.0) and b.status == GB.SYNC_NEEDED
+    assert b._scales(False) == (1.0, 1.0) and b.status == GB.SYNC_NEEDED
+    b.finish_sync()
+    assert b.status == GB.READY
+    b.clear()
+    assert b._scales(True) == (0.0, 1.0) and b.status == GB.SYNC_NEEDED
+    b.status = "bogus"
+    with pytest.raises(ValueError):
+        b._scales(False)
