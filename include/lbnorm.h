@@ -164,8 +164,8 @@ int lbn_instance_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t cha
  * dx = 0.  training == 0: forward normalises with the running statistics and writes
  * neither them nor stats; backward is dx = dy / sqrt(running_var + epsilon) and reads
  * neither x nor stats (both may be NULL).  Statistics are over the local width: with
- * several ranks the reference sums them across the mini-batch (:97-100, :301-303),
- * which is outside this library.  Where the reference's E[x^2] - mean^2 can come out
+ * several ranks the reference sums them across the mini-batch (:97-100, :301-303):
+ * use the split entry points below.  Where the reference's E[x^2] - mean^2 can come out
  * negative, the variance here is clamped at zero. */
 int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
                                      float decay, float epsilon, int training,
@@ -179,6 +179,42 @@ int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_
                                      const float* stats, int64_t ld_stats,
                                      float* stats_grad, int64_t ld_stats_grad,
                                      const float* running_var);
+
+/* The same computation cut where the reference places its all-reduces, for callers whose
+ * mini-batch is spread over several ranks (entrywise_batch_normalization.cpp:97-100 and
+ * :301-303): local sums -> [caller's all-reduce of the (height x 2) matrix] -> statistics
+ * -> apply.  `width` is the local number of columns, `statistics_count` the global one
+ * (input.Width() in the reference, :101 and :267).
+ * fwd_sums writes per-row sum(x) into column 0 of stats and sum(x^2) into column 1
+ * (:78-95; zeros for width == 0); fwd_stats turns the reduced sums into mean and variance
+ * in place and updates the running statistics (:101-125; statistics_count <= 1: variance 1,
+ * running statistics untouched); fwd_apply normalises with any (mean, var) pair of
+ * vectors: the two stats columns in training, the running statistics in inference
+ * (:131-160).  bwd_sums writes the local parts of dL/dmean, dL/dvar into stats_grad
+ * (:275-299); bwd_apply forms dx from the reduced stats_grad (:305-335;
+ * statistics_count <= 1: dx = 0). */
+int lbn_entrywise_batch_norm_fwd_sums_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                          const float* x, int64_t ldx,
+                                          float* stats, int64_t ld_stats);
+int lbn_entrywise_batch_norm_fwd_stats_f32(lbn_stream_t stream, int64_t height,
+                                           int64_t statistics_count, float decay,
+                                           float* stats, int64_t ld_stats,
+                                           float* running_mean, float* running_var);
+int lbn_entrywise_batch_norm_fwd_apply_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                           float epsilon, const float* x, int64_t ldx,
+                                           float* y, int64_t ldy,
+                                           const float* mean, const float* var);
+int lbn_entrywise_batch_norm_bwd_sums_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                          float epsilon, const float* x, int64_t ldx,
+                                          const float* dy, int64_t lddy,
+                                          const float* stats, int64_t ld_stats,
+                                          float* stats_grad, int64_t ld_stats_grad);
+int lbn_entrywise_batch_norm_bwd_apply_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                           int64_t statistics_count, float epsilon,
+                                           const float* x, int64_t ldx,
+                                           const float* dy, int64_t lddy, float* dx, int64_t lddx,
+                                           const float* stats, int64_t ld_stats,
+                                           const float* stats_grad, int64_t ld_stats_grad);
 
 /* ------------------------------------------------------------------ batch norm
  * Replaces batch_normalization_layer::fp_compute / bp_compute

@@ -75,6 +75,12 @@ PROTOTYPES = {
     "lbn_channelwise_scale_bias_bwd_workspace_bytes": (sz, [i64, i64, i64]),
     "lbn_channelwise_scale_bias_bwd_f32": (cint, [vp, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, i64,
                                                   vp, sz]),
+    "lbn_entrywise_batch_norm_fwd_sums_f32": (cint, [vp, i64, i64, vp, i64, vp, i64]),
+    "lbn_entrywise_batch_norm_fwd_stats_f32": (cint, [vp, i64, i64, f32, vp, i64, vp, vp]),
+    "lbn_entrywise_batch_norm_fwd_apply_f32": (cint, [vp, i64, i64, f32, vp, i64, vp, i64, vp, vp]),
+    "lbn_entrywise_batch_norm_bwd_sums_f32": (cint, [vp, i64, i64, f32, vp, i64, vp, i64, vp, i64, vp, i64]),
+    "lbn_entrywise_batch_norm_bwd_apply_f32": (cint, [vp, i64, i64, i64, f32, vp, i64, vp, i64, vp, i64, vp, i64,
+                                                      vp, i64]),
     "lbn_gradient_sink_f32": (cint, [vp, i64, i64, f32, f32, vp, i64, vp, i64]),
 }
 

@@ -275,12 +275,19 @@ class instance_norm_layer(_Layer):
 class entrywise_batch_normalization_layer(_Layer):
     """lbann::entrywise_batch_normalization_layer
     (include/lbann/layers/regularizers/entrywise_batch_normalization.hpp): per-entry statistics
-    over the mini-batch; weights[0] running mean, weights[1] running variance."""
+    over the mini-batch; weights[0] running mean, weights[1] running variance.
 
-    def __init__(self, dims, decay=0.9, epsilon=1e-5, device="cuda"):
+    `comm_allreduce(matrix)` stands for the reference's comm.allreduce over the mini-batch's
+    ranks (entrywise_batch_normalization.cpp:97-100, :301-303): when given, it is called on the
+    (height x 2) matrix of local sums, which it must replace by their sum over the ranks, and
+    `statistics_count` is the global mini-batch size (input.Width() there); the layer then
+    runs the split entry points around it."""
+
+    def __init__(self, dims, decay=0.9, epsilon=1e-5, device="cuda", comm_allreduce=None, statistics_count=None):
         super().__init__(device)
         self.dims = tuple(int(d) for d in dims)
         self.m_decay, self.m_epsilon = float(decay), float(epsilon)
+        self.comm_allreduce, self.statistics_count = comm_allreduce, statistics_count
         h = _prod(self.dims)
         # default weights (entrywise_batch_normalization.hpp:159-176): mean 0, variance 1
         self.weights = [_Vector(h, device, np.zeros(h)), _Vector(h, device, np.ones(h))]
@@ -303,6 +310,39 @@ class entrywise_batch_normalization_layer(_Layer):
                 (_stream(), x.height, x.width, self.m_epsilon, int(self.training), x.Buffer(), x.ldim,
                  dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim, st.Buffer(), st.ldim, sg.Buffer(), sg.ldim,
                  self.weights[1].Buffer()))
+
+    def _col(self, m, j):
+        return capi.vp(m.tensor.data_ptr() + 4 * j * m.ldim)
+
+    def fp_compute(self):
+        if self.comm_allreduce is None:
+            return super().fp_compute()
+        x, y, st = self.prev_activations, self.activations, self.m_batch_statistics
+        if self.training:
+            count = int(self.statistics_count if self.statistics_count is not None else x.width)
+            call("lbn_entrywise_batch_norm_fwd_sums_f32", _stream(), x.height, x.width, x.Buffer(), x.ldim,
+                 st.Buffer(), st.ldim)
+            self.comm_allreduce(st)
+            call("lbn_entrywise_batch_norm_fwd_stats_f32", _stream(), x.height, count, self.m_decay, st.Buffer(),
+                 st.ldim, self.weights[0].Buffer(), self.weights[1].Buffer())
+            mean, var = self._col(st, 0), self._col(st, 1)
+        else:
+            mean, var = self.weights[0].Buffer(), self.weights[1].Buffer()
+        call("lbn_entrywise_batch_norm_fwd_apply_f32", _stream(), x.height, x.width, self.m_epsilon, x.Buffer(), x.ldim,
+             y.Buffer(), y.ldim, mean, var)
+
+    def bp_compute(self):
+        if self.comm_allreduce is None or not self.training:
+            return super().bp_compute()
+        x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
+        st, sg = self.m_batch_statistics, self.m_batch_statistics_gradient
+        count = int(self.statistics_count if self.statistics_count is not None else x.width)
+        if count > 1:
+            call("lbn_entrywise_batch_norm_bwd_sums_f32", _stream(), x.height, x.width, self.m_epsilon, x.Buffer(),
+                 x.ldim, dy.Buffer(), dy.ldim, st.Buffer(), st.ldim, sg.Buffer(), sg.ldim)
+            self.comm_allreduce(sg)
+        call("lbn_entrywise_batch_norm_bwd_apply_f32", _stream(), x.height, x.width, count, self.m_epsilon, x.Buffer(),
+             x.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim, st.Buffer(), st.ldim, sg.Buffer(), sg.ldim)
 
 
 class batch_normalization_layer(_Layer):

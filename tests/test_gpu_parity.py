@@ -317,6 +317,167 @@ def test_entrywise_batch_norm(L, h, w, pad):
             check(f"entrywise_bn {k} h={h} w={w} training={training}", got[k], r32[k], r64[k])
 
 
+@pytest.mark.parametrize("h,w,w0,pad", [(105, 29, 14, 0), (4096, 64, 32, 0), (1024, 300, 7, 0), (260, 7, 3, 4),
+                                        (258, 9, 9, 0), (100000, 33, 16, 0), (8196, 257, 200, 4), (60, 513, 512, 0),
+                                        (64, 1, 1, 0), (64, 2, 1, 0)])
+def test_entrywise_batch_norm_split_over_two_ranks(L, h, w, w0, pad):
+    """The mini-batch's columns [0, w0) on one rank and [w0, w) on another: local sums, their
+    sum in place of the all-reduce, statistics with the global count, apply per rank; the
+    same for backward.  Together the two ranks must give what the reference gives on the
+    whole mini-batch (entrywise_batch_normalization.cpp:97-100, :301-303)."""
+    from lbann_amd import capi
+    rng = np.random.default_rng(h + 5 * w)
+    x, dy = rand(rng, h, w, 0.5, 2.0), rand(rng, h, w)
+    rm0 = rng.normal(size=h).astype(np.float32)
+    rv0 = rng.uniform(0.5, 2.0, size=h).astype(np.float32)
+    st = capi.vp(torch.cuda.current_stream().cuda_stream)
+    p = lambda t: capi.vp(t.data_ptr())
+    parts = [(0, w0), (w0, w)]
+    xs = [L.DeviceMatrix.from_numpy(x[:, a:b], ldim=h + pad) for a, b in parts]
+    gs = [L.DeviceMatrix.from_numpy(dy[:, a:b], ldim=h + pad) for a, b in parts]
+    ys = [L.DeviceMatrix(h, b - a, ldim=h + pad, fill=float("nan")) for a, b in parts]
+    ds = [L.DeviceMatrix(h, b - a, ldim=h + pad, fill=float("nan")) for a, b in parts]
+    ldst = h + pad
+
+    def oracle(conv):
+        rm, rv = conv(rm0).copy(), conv(rv0).copy()
+        y, stt = orc.entrywise_batch_norm_fwd(conv(x), 0.9, 1e-5, rm, rv, True)
+        dx, sg = orc.entrywise_batch_norm_bwd(conv(x), conv(dy), stt, 1e-5, rv, True)
+        return dict(y=y, stats=stt, dx=dx, sgrad=sg, rmean=rm, rvar=rv)
+
+    # forward: sums per rank -> "all-reduce" -> statistics (the same on both ranks) -> apply
+    local = [L.DeviceMatrix(h, 2, ldim=ldst, fill=float("nan")) for _ in parts]
+    for m, xm in zip(local, xs):
+        capi.call("lbn_entrywise_batch_norm_fwd_sums_f32", st, h, xm.width, xm.Buffer(), xm.ldim, m.Buffer(), m.ldim)
+    sums = local[0].to_numpy().astype(np.float64)
+    assert rel_err(sums[:, 0], x[:, :w0].astype(np.float64).sum(axis=1)) < 1e-5
+    assert rel_err(sums[:, 1], (x[:, :w0].astype(np.float64) ** 2).sum(axis=1)) < 1e-5
+    stats = L.DeviceMatrix(h, 2, ldim=ldst)
+    stats.tensor[:, :h] = local[0].tensor[:, :h] + local[1].tensor[:, :h]
+    rm, rv = torch.from_numpy(rm0).cuda(), torch.from_numpy(rv0).cuda()
+    capi.call("lbn_entrywise_batch_norm_fwd_stats_f32", st, h, w, 0.9, stats.Buffer(), stats.ldim, p(rm), p(rv))
+    mean_ptr = stats.Buffer()
+    var_ptr = capi.vp(stats.tensor.data_ptr() + 4 * stats.ldim)
+    for xm, ym in zip(xs, ys):
+        capi.call("lbn_entrywise_batch_norm_fwd_apply_f32", st, h, xm.width, 1e-5, xm.Buffer(), xm.ldim, ym.Buffer(),
+                  ym.ldim, mean_ptr, var_ptr)
+    # backward
+    glocal = [L.DeviceMatrix(h, 2, ldim=ldst, fill=float("nan")) for _ in parts]
+    for m, xm, gm in zip(glocal, xs, gs):
+        capi.call("lbn_entrywise_batch_norm_bwd_sums_f32", st, h, xm.width, 1e-5, xm.Buffer(), xm.ldim, gm.Buffer(),
+                  gm.ldim, stats.Buffer(), stats.ldim, m.Buffer(), m.ldim)
+    sgrad = L.DeviceMatrix(h, 2, ldim=ldst)
+    sgrad.tensor[:, :h] = glocal[0].tensor[:, :h] + glocal[1].tensor[:, :h]
+    for xm, gm, dm in zip(xs, gs, ds):
+        capi.call("lbn_entrywise_batch_norm_bwd_apply_f32", st, h, xm.width, w, 1e-5, xm.Buffer(), xm.ldim, gm.Buffer(),
+                  gm.ldim, dm.Buffer(), dm.ldim, stats.Buffer(), stats.ldim, sgrad.Buffer(), sgrad.ldim)
+    got = dict(y=np.concatenate([m.to_numpy() for m in ys], axis=1), stats=stats.to_numpy(),
+               dx=np.concatenate([m.to_numpy() for m in ds], axis=1), rmean=rm.cpu().numpy(), rvar=rv.cpu().numpy())
+    if w > 1:
+        got["sgrad"] = sgrad.to_numpy()
+    r32, r64 = oracle(f32), oracle(f64)
+    for k in got:
+        check(f"entrywise_bn split {k} h={h} w={w} w0={w0}", got[k], r32[k], r64[k])
+    if pad:
+        assert torch.isnan(ys[0].tensor[:, h:]).all() and torch.isnan(ds[0].tensor[:, h:]).all()
+    # inference: apply with the running statistics equals the unsplit call's inference mode
+    ym = L.DeviceMatrix(h, xs[0].width, ldim=h + pad)
+    rm_i, rv_i = torch.from_numpy(rm0).cuda(), torch.from_numpy(rv0).cuda()
+    capi.call("lbn_entrywise_batch_norm_fwd_apply_f32", st, h, xs[0].width, 1e-5, xs[0].Buffer(), xs[0].ldim, ym.Buffer(),
+              ym.ldim, p(rm_i), p(rv_i))
+    y_inf, _ = orc.entrywise_batch_norm_fwd(f32(x[:, :w0]), 0.9, 1e-5, rm0.copy(), rv0.copy(), False)
+    check("entrywise_bn split inference y", ym.to_numpy(), y_inf)
+
+
+def test_entrywise_batch_norm_layer_with_allreduce_hook(L):
+    """The layer mirror with a collective: two layer objects (ranks) hold 20 and 13 columns of
+    one mini-batch; the hook adds what the other rank computed, as comm.allreduce would."""
+    rng = np.random.default_rng(97)
+    h, w, w0 = 1000, 33, 20
+    x, dy = rand(rng, h, w, -0.3, 1.5), rand(rng, h, w)
+    halves = [(0, w0), (w0, w)]
+    # lock-step emulation: rank 1's local sums are computed first through the C ABI
+    # and handed to rank 0's hook, then the other way round
+    from lbann_amd import capi
+    st = capi.vp(torch.cuda.current_stream().cuda_stream)
+    mats = [L.DeviceMatrix.from_numpy(x[:, a:b]) for a, b in halves]
+    gmats = [L.DeviceMatrix.from_numpy(dy[:, a:b]) for a, b in halves]
+    results = []
+    for me, other in ((0, 1), (1, 0)):
+        phase = {"n": 0}
+
+        def hook(m, me=me, other=other, phase=phase):
+            peer = L.DeviceMatrix(h, 2)
+            if phase["n"] == 0:
+                capi.call("lbn_entrywise_batch_norm_fwd_sums_f32", st, h, mats[other].width, mats[other].Buffer(),
+                          mats[other].ldim, peer.Buffer(), peer.ldim)
+            else:
+                capi.call("lbn_entrywise_batch_norm_bwd_sums_f32", st, h, mats[other].width, 1e-5, mats[other].Buffer(),
+                          mats[other].ldim, gmats[other].Buffer(), gmats[other].ldim, layer.m_batch_statistics.Buffer(),
+                          layer.m_batch_statistics.ldim, peer.Buffer(), peer.ldim)
+            m.tensor[:, :h] += peer.tensor[:, :h]
+            phase["n"] += 1
+
+        layer = L.entrywise_batch_normalization_layer((h,), 0.9, 1e-5, comm_allreduce=hook, statistics_count=w)
+        y = layer.forward(mats[me]).to_numpy()
+        dx = layer.backward(gmats[me]).to_numpy()
+        assert phase["n"] == 2
+        results.append((y, dx, layer.m_batch_statistics.to_numpy(), layer.weights[0].to_numpy(), layer.weights[1].to_numpy()))
+    rm, rv = np.zeros(h, np.float32), np.ones(h, np.float32)
+    y_ref, st_ref = orc.entrywise_batch_norm_fwd(x, 0.9, 1e-5, rm, rv, True)
+    dx_ref, _ = orc.entrywise_batch_norm_bwd(x, dy, st_ref, 1e-5, rv, True)
+    x64, dy64 = f64(x), f64(dy)
+    y64, st64 = orc.entrywise_batch_norm_fwd(x64, 0.9, 1e-5, np.zeros(h), np.ones(h), True)
+    dx64, _ = orc.entrywise_batch_norm_bwd(x64, dy64, st64, 1e-5, np.ones(h), True)
+    check("hooked entrywise_bn y", np.concatenate([r[0] for r in results], axis=1), y_ref, y64)
+    check("hooked entrywise_bn dx", np.concatenate([r[1] for r in results], axis=1), dx_ref, dx64)
+    for r in results:
+        check("hooked entrywise_bn stats", r[2], st_ref, st64)
+        check("hooked entrywise_bn running mean", r[3], rm)
+        check("hooked entrywise_bn running var", r[4], rv)
+    # inference through the hooked layer: running statistics, no collective
+    layer.training = False
+    y_inf = layer.forward(mats[1]).to_numpy()
+    y_inf_ref, _ = orc.entrywise_batch_norm_fwd(f32(x[:, w0:]), 0.9, 1e-5, rm.copy(), rv.copy(), False)
+    check("hooked entrywise_bn inference", y_inf, y_inf_ref)
+
+
+def test_entrywise_batch_norm_split_empty_and_rejected_arguments(L):
+    from lbann_amd import capi
+    st = capi.vp(torch.cuda.current_stream().cuda_stream)
+    null = capi.vp(None)
+    lib = capi.lib()
+    buf = torch.full((4096,), 3.0, device="cuda")
+    p = capi.vp(buf.data_ptr())
+    # a rank without local columns contributes zero sums
+    assert lib.lbn_entrywise_batch_norm_fwd_sums_f32(st, 16, 0, null, 16, p, 16) == 0
+    assert lib.lbn_entrywise_batch_norm_bwd_sums_f32(st, 10, 0, 1e-5, null, 10, null, 10, p, 2048, capi.vp(buf.data_ptr() + 4 * 64), 10) == 0
+    torch.cuda.synchronize()
+    assert buf[:32].abs().sum().item() == 0.0 and buf[32].item() == 3.0
+    assert buf[64:84].abs().sum().item() == 0.0 and buf[84].item() == 3.0
+    assert lib.lbn_entrywise_batch_norm_fwd_sums_f32(st, 0, 4, null, 1, null, 1) == 0
+    assert lib.lbn_entrywise_batch_norm_fwd_apply_f32(st, 8, 0, 1e-5, null, 8, null, 8, null, null) == 0
+    # a single sample in the whole mini-batch: variance 1, running statistics untouched, dx = 0
+    buf.fill_(3.0)
+    run = torch.full((16,), 5.0, device="cuda")
+    assert lib.lbn_entrywise_batch_norm_fwd_stats_f32(st, 8, 1, 0.9, p, 8, capi.vp(run.data_ptr()), capi.vp(run.data_ptr() + 32)) == 0
+    assert lib.lbn_entrywise_batch_norm_bwd_apply_f32(st, 8, 1, 1, 1e-5, null, 8, null, 8, capi.vp(buf.data_ptr() + 4 * 100), 8, null, 8, null, 8) == 0
+    torch.cuda.synchronize()
+    assert buf[:8].tolist() == [3.0] * 8 and buf[8:16].tolist() == [1.0] * 8 and (run == 5.0).all()
+    assert buf[100:108].abs().sum().item() == 0.0 and buf[108].item() == 3.0
+    # rejected
+    E = capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_entrywise_batch_norm_fwd_sums_f32(st, 8, 4, p, 4, p, 8) == E
+    assert lib.lbn_entrywise_batch_norm_fwd_sums_f32(st, 8, 4, p, 8, p, 4) == E
+    assert lib.lbn_entrywise_batch_norm_fwd_sums_f32(st, 8, 4, null, 8, p, 8) == E
+    assert lib.lbn_entrywise_batch_norm_fwd_stats_f32(st, 8, 4, 0.9, p, 8, null, p) == E
+    assert lib.lbn_entrywise_batch_norm_fwd_apply_f32(st, 8, 4, 1e-5, p, 8, p, 8, null, p) == E
+    assert lib.lbn_entrywise_batch_norm_bwd_sums_f32(st, 8, 4, 1e-5, p, 8, p, 8, p, 8, null, 8) == E
+    assert lib.lbn_entrywise_batch_norm_bwd_apply_f32(st, 8, 4, 4, 1e-5, p, 8, p, 8, null, 8, p, 8, p, 8) == E
+    assert lib.lbn_entrywise_batch_norm_bwd_apply_f32(st, 8, 4, 4, 1e-5, p, 8, p, 8, p, 8, p, 4, p, 8) == E
+    torch.cuda.synchronize()
+
+
 # ===================================================================== batch norm
 BN_CASES = [
     # dims (C, ...), width, bessel, ld_pad
