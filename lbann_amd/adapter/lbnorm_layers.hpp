@@ -564,6 +564,16 @@ public:
   /// device pointers to `size` floats each
   void set_weights(float* running_mean, float* running_var) { m_w[0] = running_mean; m_w[1] = running_var; }
 
+  /// The mini-batch spread over several ranks: `allreduce` stands for comm.allreduce(...,
+  /// El::mpi::SUM) of the reference (entrywise_batch_normalization.cpp:97-100, :301-303) and
+  /// must replace the (size x 2) matrix of local sums by its sum over the ranks, ordered on
+  /// io.stream; `statistics_count` is the global mini-batch size (input.Width() there).
+  void set_statistics_allreduce(std::function<void(device_matrix<float>&)> allreduce, int64_t statistics_count)
+  {
+    m_allreduce = std::move(allreduce);
+    m_statistics_count = statistics_count;
+  }
+
   layer_io<Mat> io;
   bool is_training = true;                             // execution_mode::training
   device_matrix<float> m_batch_statistics;             // size x 2: mean, variance
@@ -574,6 +584,25 @@ public:
     const Mat& x = *io.prev_activations;
     Mat& y = *io.activations;
     if (!m_w[0] || !m_w[1]) throw exception("entrywise_batch_normalization_layer: weights are not set");
+    if (m_allreduce) {
+      const char* where = "entrywise_batch_normalization_layer::fp_compute";
+      device_matrix<float>& st = m_batch_statistics;
+      const float* mean = m_w[0];
+      const float* var = m_w[1];
+      if (is_training) {
+        check_status(lbn_entrywise_batch_norm_fwd_sums_f32(io.stream, x.Height(), x.Width(), x.LockedBuffer(),
+                                                           x.LDim(), st.Buffer(), st.LDim()), where);
+        m_allreduce(st);
+        check_status(lbn_entrywise_batch_norm_fwd_stats_f32(io.stream, x.Height(), m_statistics_count, m_decay,
+                                                            st.Buffer(), st.LDim(), m_w[0], m_w[1]), where);
+        mean = st.LockedBuffer();
+        var = st.LockedBuffer() + st.LDim();
+      }
+      check_status(lbn_entrywise_batch_norm_fwd_apply_f32(io.stream, x.Height(), x.Width(), m_epsilon,
+                                                          x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(), mean, var),
+                   where);
+      return;
+    }
     check_status(lbn_entrywise_batch_norm_fwd_f32(io.stream, x.Height(), x.Width(), m_decay, m_epsilon,
                                                   is_training ? 1 : 0, x.LockedBuffer(), x.LDim(), y.Buffer(),
                                                   y.LDim(), m_batch_statistics.Buffer(),
@@ -585,6 +614,24 @@ public:
     const Mat& x = *io.prev_activations;
     const Mat& dy = *io.prev_error_signals;
     Mat& dx = *io.error_signals;
+    if (m_allreduce && is_training) {
+      const char* where = "entrywise_batch_normalization_layer::bp_compute";
+      device_matrix<float>& st = m_batch_statistics;
+      device_matrix<float>& sg = m_batch_statistics_gradient;
+      if (m_statistics_count > 1) {
+        check_status(lbn_entrywise_batch_norm_bwd_sums_f32(io.stream, x.Height(), x.Width(), m_epsilon,
+                                                           x.LockedBuffer(), x.LDim(), dy.LockedBuffer(), dy.LDim(),
+                                                           st.LockedBuffer(), st.LDim(), sg.Buffer(), sg.LDim()),
+                     where);
+        m_allreduce(sg);
+      }
+      check_status(lbn_entrywise_batch_norm_bwd_apply_f32(io.stream, x.Height(), x.Width(), m_statistics_count,
+                                                          m_epsilon, x.LockedBuffer(), x.LDim(), dy.LockedBuffer(),
+                                                          dy.LDim(), dx.Buffer(), dx.LDim(), st.LockedBuffer(),
+                                                          st.LDim(), sg.LockedBuffer(), sg.LDim()),
+                   where);
+      return;
+    }
     check_status(lbn_entrywise_batch_norm_bwd_f32(io.stream, x.Height(), x.Width(), m_epsilon,
                                                   is_training ? 1 : 0, x.LockedBuffer(), x.LDim(),
                                                   dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
@@ -597,6 +644,8 @@ private:
   float m_decay, m_epsilon;
   int64_t m_size = 0;
   float* m_w[2] = {nullptr, nullptr};
+  std::function<void(device_matrix<float>&)> m_allreduce;
+  int64_t m_statistics_count = 0;
 };
 
 // ------------------------------------------------------------------ cross entropy

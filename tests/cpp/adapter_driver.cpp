@@ -198,6 +198,61 @@ int drv_entrywise_batch_norm(const int64_t* dims, int nd, double decay, double e
   }
 }
 
+// One mini-batch of w columns held by two ranks (columns [0, w0) and [w0, w)), each with its
+// own layer object and running statistics (rmean2 / rvar2: two vectors of h floats each).  The
+// all-reduce hook of a rank computes the other rank's local sums through the C ABI and adds
+// them with the gradient-buffer kernel, which is what the collective would leave behind.
+int drv_entrywise_batch_norm_two_ranks(const int64_t* dims, int nd, double decay, double eps, int64_t h,
+                                       int64_t w, int64_t w0, int64_t ld, float* x, float* y, float* dy,
+                                       float* dx, float* rmean2, float* rvar2, float* stats_out, void* stream,
+                                       char* err, int errlen)
+{
+  try {
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t first[2] = {0, w0}, count[2] = {w0, w - w0};
+    for (int me = 0; me < 2; ++me) {
+      const int other = 1 - me;
+      entrywise_batch_normalization_layer<> layer(decay, eps);
+      layer.setup(std::vector<int64_t>(dims, dims + nd));
+      layer.set_weights(rmean2 + me * h, rvar2 + me * h);
+      device_matrix<float> mx, my, mdy, mdx, peer(h, 2);
+      attach(mx, h, count[me], x + first[me] * ld, ld); attach(my, h, count[me], y + first[me] * ld, ld);
+      attach(mdy, h, count[me], dy + first[me] * ld, ld); attach(mdx, h, count[me], dx + first[me] * ld, ld);
+      layer.io.prev_activations = &mx; layer.io.activations = &my;
+      layer.io.prev_error_signals = &mdy; layer.io.error_signals = &mdx;
+      layer.io.stream = st;
+      int phase = 0;
+      layer.set_statistics_allreduce(
+        [&](device_matrix<float>& m) {
+          const float* px = x + first[other] * ld;
+          const float* pdy = dy + first[other] * ld;
+          if (phase == 0)
+            check_status(lbn_entrywise_batch_norm_fwd_sums_f32(st, h, count[other], px, ld, peer.Buffer(), peer.LDim()),
+                         "peer sums");
+          else
+            check_status(lbn_entrywise_batch_norm_bwd_sums_f32(st, h, count[other], static_cast<float>(eps), px, ld, pdy,
+                                                               ld, layer.m_batch_statistics.LockedBuffer(),
+                                                               layer.m_batch_statistics.LDim(), peer.Buffer(),
+                                                               peer.LDim()),
+                         "peer gradient sums");
+          check_status(lbn_gradient_sink_f32(st, h, 2, 1.f, 1.f, peer.LockedBuffer(), peer.LDim(), m.Buffer(), m.LDim()),
+                       "sum over ranks");
+          ++phase;
+        },
+        w);
+      layer.fp_compute();
+      layer.bp_compute();
+      if (phase != (w > 1 ? 2 : 1)) throw exception("all-reduce hook called an unexpected number of times");
+      if (me == 0) copy_out(stats_out, layer.m_batch_statistics, st);
+      check_hip(hipStreamSynchronize(st), "sync");
+    }
+    return 0;
+  }
+  catch (const std::exception& e) {
+    return fail(e, err, errlen);
+  }
+}
+
 int drv_cross_entropy(const int64_t* pred_dims, const int64_t* truth_dims, int nd, int use_labels, int64_t h,
                       int64_t ht, int64_t w, float* x, float* truth, float* loss, float* dloss, float* dx,
                       float* dtruth, void* stream, char* err, int errlen)

@@ -233,3 +233,29 @@ def test_adapter_layers_match_oracle():
     assert grad.to_numpy().tobytes() == exp.tobytes()
     check("adapter gradient buffer", grad.to_numpy(), -1.5 * wg_ref)
     assert torch.isnan(grad.tensor[:, 8:]).all()
+
+    # ---- entry-wise batch norm with the mini-batch on two ranks (all-reduce hook of the adapter)
+    dims, w, w0 = (5, 8, 6), 27, 11
+    h = 240
+    x, dy = mk(h, w, -0.4, 1.7), mk(h, w)
+    mx, mdy, my, mdx = DeviceMatrix.from_numpy(x), DeviceMatrix.from_numpy(dy), DeviceMatrix(h, w), DeviceMatrix(h, w)
+    rm2 = torch.zeros(2 * h, device="cuda")
+    rv2 = torch.ones(2 * h, device="cuda")
+    stats = DeviceMatrix(h, 2)
+    da, nd = _dims(dims)
+    rc = d.drv_entrywise_batch_norm_two_ranks(da, cint(nd), dbl(0.9), dbl(1e-5), i64(h), i64(w), i64(w0), i64(h), mx.Buffer(),
+                                              my.Buffer(), mdy.Buffer(), mdx.Buffer(), p(rm2), p(rv2), stats.Buffer(), st, err,
+                                              cint(512))
+    assert rc == 0, err.value
+    rm0, rv0 = np.zeros(h, np.float32), np.ones(h, np.float32)
+    y_ref, st_ref = orc.entrywise_batch_norm_fwd(x, 0.9, 1e-5, rm0, rv0)
+    dx_ref, _ = orc.entrywise_batch_norm_bwd(x, dy, st_ref, 1e-5)
+    x64, dy64 = x.astype(np.float64, order="F"), dy.astype(np.float64, order="F")
+    y64, st64 = orc.entrywise_batch_norm_fwd(x64, 0.9, 1e-5, np.zeros(h), np.ones(h))
+    dx64, _ = orc.entrywise_batch_norm_bwd(x64, dy64, st64, 1e-5)
+    check("adapter two-rank entrywise bn y", my.to_numpy(), y_ref, y64)
+    check("adapter two-rank entrywise bn dx", mdx.to_numpy(), dx_ref, dx64)
+    check("adapter two-rank entrywise bn stats", stats.to_numpy(), st_ref, st64)
+    for k in range(2):
+        check("adapter two-rank running mean", rm2[k * h:(k + 1) * h].cpu().numpy(), rm0)
+        check("adapter two-rank running var", rv2[k * h:(k + 1) * h].cpu().numpy(), rv0)
