@@ -309,6 +309,21 @@ int lbn_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
                         const float* y, int64_t ldy, const float* dy, int64_t lddy,
                         float* dx, int64_t lddx, void* workspace, size_t workspace_bytes);
 
+/* Softmax forward for callers that cannot allocate device memory or hand over a
+ * workspace: code running under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, results
+ * and kernels as lbn_softmax_fwd_f32, but the scratch is an array that is part of the
+ * library's code object (lbn_softmax_fwd_static_scratch_max_bytes() bytes, 1 MiB, held
+ * by every GPU the library runs on until the process ends); the call itself allocates
+ * and frees nothing.  Shapes with lbn_softmax_workspace_bytes(height, width) above that
+ * size are rejected with LBN_ERR_UNSUPPORTED before anything is launched.  All calls on
+ * one GPU share the array: two such calls that overlap in time on one GPU (different
+ * streams, or concurrent graph replays) race on it and are not supported; calls on one
+ * stream are ordered and safe.  Nothing in the array has to start at zero. */
+size_t lbn_softmax_fwd_static_scratch_max_bytes(void);
+int lbn_softmax_fwd_static_scratch_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                       const float* x, int64_t ldx, float* y, int64_t ldy);
+
 /* ----------------------------------------------------------------- log-softmax
  * Replaces log_softmax_layer::fp_compute / bp_compute
  * (src/layers/activations/log_softmax.cpp:35-93, :95-136, :140-156).

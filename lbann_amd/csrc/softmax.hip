@@ -27,6 +27,8 @@
 #include "device_utils.hpp"
 #include "host_utils.hpp"
 
+#include <mutex>
+
 namespace lbn {
 
 enum SmKind : int { kSoftmax = 0, kLogSoftmax = 1, kChannelwise = 2 };
@@ -1084,6 +1086,38 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   return launch_status();
 }
 
+// ------------------------------------------------------------ library-owned scratch
+// Scratch of the entry point that allocates nothing: one array per GPU, part of the code
+// object, so it exists from the moment the library is loaded until the process ends.  The
+// array's name is only a host-side handle: host code uses the address that
+// hipGetSymbolAddress() reports for the current device, looked up once per device.
+constexpr size_t kStaticScratchBytes = size_t(1) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+
+// Device address of `scratch` on the current device; *out stays null on failure.
+static int static_scratch_address(void** out)
+{
+  static std::mutex mu;
+  static void* address[kMaxDevices] = {};
+  *out = nullptr;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (dev < 0 || dev >= kMaxDevices) return LBN_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!address[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (!p) return static_cast<int>(hipErrorInvalidSymbol);
+    address[dev] = p;
+  }
+  *out = address[dev];
+  return LBN_OK;
+}
+
 }  // namespace lbn
 
 using namespace lbn;
@@ -1112,6 +1146,20 @@ int lbn_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, cons
                         void* workspace, size_t workspace_bytes)
 {
   return sm_bwd<kSoftmax>(as_stream(stream), 1, height, height, width, y, ldy, dy, lddy, dx, lddx, workspace, workspace_bytes);
+}
+
+size_t lbn_softmax_fwd_static_scratch_max_bytes(void) { return kStaticScratchBytes; }
+
+int lbn_softmax_fwd_static_scratch_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* x,
+                                       int64_t ldx, float* y, int64_t ldy)
+{
+  if (height < 0 || width < 0) return LBN_ERR_INVALID_ARGUMENT;
+  if (height == 0 || width == 0) return LBN_OK;
+  if (sm_workspace_bytes(height, width) > kStaticScratchBytes) return LBN_ERR_UNSUPPORTED;
+  void* ptr = nullptr;
+  const int status = static_scratch_address(&ptr);
+  if (status != LBN_OK) return status;
+  return sm_fwd<kSoftmax>(as_stream(stream), 1, height, height, width, x, ldx, y, ldy, ptr, kStaticScratchBytes);
 }
 
 int lbn_log_softmax_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* x,
