@@ -27,11 +27,29 @@
  * graph's state: keep it allocated, and do not run two replays that share it at the
  * same time.
  *
- * Those kernels size their grid to the workgroups the idle device holds at once.  Next
- * to other streams' kernels they still complete (members of a cluster are consecutive
- * blocks, dispatched in order), only later; every wait is bounded and a wait that ran
- * out is reported by lbn_workspace_timed_out().  Setting LBN_NO_CLUSTER=1 in the
- * environment selects the multi-kernel paths instead.
+ * Waits across workgroups.  Those kernels ("cluster kernels": batch norm, softmax and
+ * layer norm over rows too long for one workgroup) size their grid to the workgroups the
+ * idle device holds at once, so that all members of a cluster are resident together and
+ * every wait ends.  Two things this rests on are assumptions about the hardware, not
+ * guarantees of the HIP API: the occupancy query describes a device that runs nothing
+ * else, and workgroups are dispatched in block order (members of a cluster are
+ * consecutive blocks, so a launch that shares the device still has at most one partly
+ * resident cluster, whose missing members are the next to start).  Supported use: one
+ * cluster kernel on the device at a time, i.e. calls on one stream (or on several, when
+ * their cluster calls do not overlap); cluster calls running concurrently on several
+ * streams can each hold part of the device and wait on each other until the poll bound.
+ * Callers that cannot promise this set LBN_NO_CLUSTER=1 in the environment, which selects
+ * the multi-kernel paths everywhere.  Every wait is bounded: a wait that runs out raises
+ * a sticky error word in the workspace's first 64 bytes (written by nothing else), the
+ * kernel ends normally with undefined results, and the entry point has long returned 0.
+ * lbn_workspace_timed_out() reads that word; a caller who wants to rely on it clears the
+ * first 64 bytes of a workspace once after allocating it (recycled memory may hold
+ * anything) and checks where results are consumed.  The two host-side mirrors of the
+ * layer classes do both.
+ *
+ * Process-wide state of the library: the counter the per-call tags are drawn from (an
+ * atomic), the cached occupancy figures per kernel and device, and the environment
+ * switches, each read once.  Nothing else outlives a call.
  */
 #ifndef LBNORM_H_INCLUDED
 #define LBNORM_H_INCLUDED
@@ -69,6 +87,16 @@ const char* lbn_status_string(int status);
  * and stores it in *timed_out (0 or 1).  It is the only entry point that synchronises.
  * It has no counterpart in the reference, whose kernels do not wait across workgroups. */
 int lbn_workspace_timed_out(lbn_stream_t stream, const void* workspace, int* timed_out);
+
+/* Diagnostic: exercises the designed exit of a wait that cannot end.  Launches ONE
+ * workgroup that acts as member 0 of a cluster of two, publishes its pair (1, 2) and polls
+ * for a member 1 that does not exist; after max_polls (1..65536) rounds the wait gives up,
+ * raises the error word of `workspace` (at least 128 bytes, 16-byte aligned) and the
+ * kernel ends like any other.  out4 (4 floats, device) receives member 0's pair and the
+ * stand-in (-1, -1) of the absent member.  Afterwards lbn_workspace_timed_out() reports 1
+ * for this workspace until its header is cleared.  No counterpart in the reference. */
+int lbn_selftest_cluster_wait_gives_up(lbn_stream_t stream, void* workspace, size_t workspace_bytes,
+                                       int max_polls, float* out4);
 
 /* ------------------------------------------------------------------ layer norm
  * Replaces layer_norm_layer::fp_compute / bp_compute

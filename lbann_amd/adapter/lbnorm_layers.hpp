@@ -23,6 +23,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <cstdlib>
 #include <functional>
 #include <numeric>
 #include <stdexcept>
@@ -102,24 +103,83 @@ private:
   bool m_owned = false;
 };
 
+namespace detail {
+/// LBN_CHECK_CLUSTER_WAITS=1 in the environment: every compute hook checks its workspace's
+/// error word right after the call (this waits for the stream: a debugging mode).
+inline bool check_every_call()
+{
+  static const bool on = [] {
+    const char* v = std::getenv("LBN_CHECK_CLUSTER_WAITS");
+    return v && *v && *v != '0';
+  }();
+  return on;
+}
+inline bool stream_is_capturing(hipStream_t st)
+{
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+}  // namespace detail
+
 /// Scratch buffer a layer owns (the role of the reference's m_workspace members).
+///
+/// The compute hooks only enqueue kernels as long as the buffer is large enough; it grows
+/// (hipFree + hipMalloc, which wait for the device) when a larger mini-batch arrives.  A
+/// caller that must not hit that inside a step, or that records its step into a HIP graph,
+/// sizes it up front: `layer.scratch().reserve(bytes, stream)` with the *_workspace_bytes()
+/// of its largest mini-batch.  Growing while the stream records is refused.
+///
+/// The first 64 bytes hold the error word of the kernels that wait across workgroups; they
+/// are cleared when the buffer is allocated, and check() turns a raised word into an
+/// exception: call it (through the layer's check_cluster_waits()) where a step's results are
+/// consumed; it waits for the stream.
 class workspace {
 public:
   workspace() = default;
   workspace(const workspace&) = delete;
   workspace& operator=(const workspace&) = delete;
   ~workspace() { if (m_buf) (void)hipFree(m_buf); }
-  void* reserve(size_t bytes)
+  void* reserve(size_t bytes, hipStream_t stream = nullptr)
   {
     if (bytes > m_bytes) {
+      if (detail::stream_is_capturing(stream))
+        throw exception("workspace::reserve: the scratch buffer would have to grow (" + std::to_string(m_bytes) +
+                        " -> " + std::to_string(bytes) + " bytes) while the stream records a graph; "
+                        "reserve it before recording");
       if (m_buf) (void)hipFree(m_buf);
       m_buf = nullptr;
-      check_hip(hipMalloc(&m_buf, bytes), "workspace::reserve");
-      m_bytes = bytes;
+      m_bytes = 0;
+      const size_t alloc = bytes < 64 ? 64 : bytes;
+      check_hip(hipMalloc(&m_buf, alloc), "workspace::reserve");
+      check_hip(hipMemsetAsync(m_buf, 0, 64, stream), "workspace::reserve (clearing the header)");
+      m_bytes = alloc;
     }
     return m_buf;
   }
   size_t bytes() const { return m_bytes; }
+  /// Throws if a wait between workgroups ran out in a call that used this buffer; clears the
+  /// word so that the next call starts clean.  Waits for `stream`.
+  void check(hipStream_t stream, const char* where)
+  {
+    if (!m_buf) return;
+    int timed_out = 0;
+    check_status(lbn_workspace_timed_out(stream, m_buf, &timed_out), where);
+    if (timed_out) {
+      check_hip(hipMemsetAsync(m_buf, 0, 64, stream), where);
+      throw exception(std::string(where) + ": a bounded wait between workgroups ran out; the results of that "
+                      "call are undefined");
+    }
+  }
+  /// The debugging mode's check after every call.
+  void after_call(hipStream_t stream, const char* where)
+  {
+    if (detail::check_every_call()) check(stream, where);
+  }
+
 private:
   void* m_buf = nullptr;
   size_t m_bytes = 0;
@@ -196,7 +256,7 @@ public:
     const float* bw = m_bias ? m_bias_w : nullptr;
     // scratch is only needed (and only non-zero) for groups of tens of thousands of entries
     const size_t bytes = lbn_layer_norm_fwd_workspace_bytes(G, n, x.Width(), static_cast<int>(sizeof(T)));
-    void* ws = m_ws.reserve(bytes);
+    void* ws = m_ws.reserve(bytes, io.stream);
     int st;
     if (sizeof(T) == 2)
       st = lbn_layer_norm_fwd_f16(io.stream, G, n, stride, x.Width(), m_epsilon, x.LockedBuffer(), x.LDim(),
@@ -208,6 +268,7 @@ public:
                                   reinterpret_cast<float*>(y.Buffer()), y.LDim(), m_statistics.Buffer(),
                                   m_statistics.LDim(), sw, bw, ws, bytes, stats_mode);
     check_status(st, "layer_norm_layer::fp_compute");
+    m_ws.after_call(io.stream, "layer_norm_layer::fp_compute");
   }
 
   /// layer_norm.cpp:292-348 / layer_norm.cu bp_compute.  The weight gradients are
@@ -226,7 +287,7 @@ public:
     float* dbw = m_bias ? m_bias_grad : nullptr;
     const size_t bytes = lbn_layer_norm_bwd_workspace_bytes(G, n, x.Width(), (dsw || dbw) ? 1 : 0,
                                                             static_cast<int>(sizeof(T)));
-    void* ws = m_ws.reserve(bytes);
+    void* ws = m_ws.reserve(bytes, io.stream);
     int st;
     if (sizeof(T) == 2)
       st = lbn_layer_norm_bwd_f16(io.stream, G, n, stride, x.Width(), m_epsilon, x.LockedBuffer(), x.LDim(),
@@ -243,6 +304,16 @@ public:
                                   m_statistics_gradient.Buffer(), m_statistics_gradient.LDim(), sw, dsw, dbw,
                                   ws, bytes);
     check_status(st, "layer_norm_layer::bp_compute");
+    m_ws.after_call(io.stream, "layer_norm_layer::bp_compute");
+  }
+
+  /// The layer's scratch buffer (reserve it up front to keep the hooks free of allocation).
+  workspace& scratch() { return m_ws; }
+  /// Throws if a wait between workgroups ran out in a call of this layer since the last
+  /// check; waits for the stream.  Call where a step's results are consumed.
+  void check_cluster_waits()
+  {
+    m_ws.check(io.stream, "check_cluster_waits");
   }
 
 private:
@@ -302,7 +373,7 @@ public:
     const Mat& x = *io.prev_activations;
     Mat& y = *io.activations;
     const size_t bytes = lbn_batch_norm_workspace_bytes(m_num_channels, m_channel_size, x.Width());
-    void* ws = m_ws.reserve(bytes);
+    void* ws = m_ws.reserve(bytes, io.stream);
     float* mv = m_mean_and_var.Buffer();
     int st;
     if (sizeof(T) == 2)
@@ -319,6 +390,7 @@ public:
                                   mv + m_mean_and_var.LDim(), m_w[0], m_w[1], m_w[2], m_w[3], ws, bytes,
                                   stats_mode);
     check_status(st, "batch_normalization_layer::fp_compute");
+    m_ws.after_call(io.stream, "batch_normalization_layer::fp_compute");
   }
   void bp_compute()
   {
@@ -326,7 +398,7 @@ public:
     const Mat& dy = *io.prev_error_signals;
     Mat& dx = *io.error_signals;
     const size_t bytes = lbn_batch_norm_workspace_bytes(m_num_channels, m_channel_size, x.Width());
-    void* ws = m_ws.reserve(bytes);
+    void* ws = m_ws.reserve(bytes, io.stream);
     const float* mv = m_mean_and_var.LockedBuffer();
     float* mvg = m_mean_and_var_gradient.Buffer();
     int st;
@@ -346,6 +418,16 @@ public:
                                   mv + m_mean_and_var.LDim(), m_w[2], m_w[3], m_w[0], m_scale_grad,
                                   m_bias_grad, mvg, mvg + m_mean_and_var_gradient.LDim(), ws, bytes);
     check_status(st, "batch_normalization_layer::bp_compute");
+    m_ws.after_call(io.stream, "batch_normalization_layer::bp_compute");
+  }
+
+  /// The layer's scratch buffer (reserve it up front to keep the hooks free of allocation).
+  workspace& scratch() { return m_ws; }
+  /// Throws if a wait between workgroups ran out in a call of this layer since the last
+  /// check; waits for the stream.  Call where a step's results are consumed.
+  void check_cluster_waits()
+  {
+    m_ws.check(io.stream, "check_cluster_waits");
   }
 
 private:
@@ -379,8 +461,9 @@ public:
     Mat& y = *io.activations;
     const size_t bytes = lbn_softmax_workspace_bytes(x.Height(), x.Width());
     check_status(lbn_softmax_fwd_f32(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(), y.Buffer(),
-                                     y.LDim(), m_ws.reserve(bytes), bytes),
+                                     y.LDim(), m_ws.reserve(bytes, io.stream), bytes),
                  "softmax_layer::fp_compute");
+    m_ws.after_call(io.stream, "softmax_layer::fp_compute");
   }
   void bp_compute()
   {
@@ -390,9 +473,19 @@ public:
     const size_t bytes = lbn_softmax_workspace_bytes(y.Height(), y.Width());
     check_status(lbn_softmax_bwd_f32(io.stream, y.Height(), y.Width(), y.LockedBuffer(), y.LDim(),
                                      dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
-                                     m_ws.reserve(bytes), bytes),
+                                     m_ws.reserve(bytes, io.stream), bytes),
                  "softmax_layer::bp_compute");
+    m_ws.after_call(io.stream, "softmax_layer::bp_compute");
   }
+  /// The layer's scratch buffer (reserve it up front to keep the hooks free of allocation).
+  workspace& scratch() { return m_ws; }
+  /// Throws if a wait between workgroups ran out in a call of this layer since the last
+  /// check; waits for the stream.  Call where a step's results are consumed.
+  void check_cluster_waits()
+  {
+    m_ws.check(io.stream, "check_cluster_waits");
+  }
+
 private:
   softmax_mode m_mode;
   workspace m_ws;
@@ -409,8 +502,9 @@ public:
     Mat& y = *io.activations;
     const size_t bytes = lbn_softmax_workspace_bytes(x.Height(), x.Width());
     check_status(lbn_log_softmax_fwd_f32(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(),
-                                         y.Buffer(), y.LDim(), m_ws.reserve(bytes), bytes),
+                                         y.Buffer(), y.LDim(), m_ws.reserve(bytes, io.stream), bytes),
                  "log_softmax_layer::fp_compute");
+    m_ws.after_call(io.stream, "log_softmax_layer::fp_compute");
   }
   void bp_compute()
   {
@@ -420,9 +514,19 @@ public:
     const size_t bytes = lbn_softmax_workspace_bytes(y.Height(), y.Width());
     check_status(lbn_log_softmax_bwd_f32(io.stream, y.Height(), y.Width(), y.LockedBuffer(), y.LDim(),
                                          dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
-                                         m_ws.reserve(bytes), bytes),
+                                         m_ws.reserve(bytes, io.stream), bytes),
                  "log_softmax_layer::bp_compute");
+    m_ws.after_call(io.stream, "log_softmax_layer::bp_compute");
   }
+  /// The layer's scratch buffer (reserve it up front to keep the hooks free of allocation).
+  workspace& scratch() { return m_ws; }
+  /// Throws if a wait between workgroups ran out in a call of this layer since the last
+  /// check; waits for the stream.  Call where a step's results are consumed.
+  void check_cluster_waits()
+  {
+    m_ws.check(io.stream, "check_cluster_waits");
+  }
+
 private:
   workspace m_ws;
 };
@@ -473,8 +577,9 @@ public:
     get_channel_size_and_stride(cs, stride, C);
     const size_t bytes = lbn_channelwise_softmax_workspace_bytes(C, cs, x.Width());
     check_status(lbn_channelwise_softmax_fwd_f32(io.stream, C, cs, stride, x.Width(), x.LockedBuffer(), x.LDim(),
-                                                 y.Buffer(), y.LDim(), m_ws.reserve(bytes), bytes),
+                                                 y.Buffer(), y.LDim(), m_ws.reserve(bytes, io.stream), bytes),
                  "channelwise_softmax_layer::fp_compute");
+    m_ws.after_call(io.stream, "channelwise_softmax_layer::fp_compute");
   }
   void bp_compute()
   {
@@ -486,9 +591,19 @@ public:
     const size_t bytes = lbn_channelwise_softmax_workspace_bytes(C, cs, y.Width());
     check_status(lbn_channelwise_softmax_bwd_f32(io.stream, C, cs, stride, y.Width(), y.LockedBuffer(), y.LDim(),
                                                  dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
-                                                 m_ws.reserve(bytes), bytes),
+                                                 m_ws.reserve(bytes, io.stream), bytes),
                  "channelwise_softmax_layer::bp_compute");
+    m_ws.after_call(io.stream, "channelwise_softmax_layer::bp_compute");
   }
+  /// The layer's scratch buffer (reserve it up front to keep the hooks free of allocation).
+  workspace& scratch() { return m_ws; }
+  /// Throws if a wait between workgroups ran out in a call of this layer since the last
+  /// check; waits for the stream.  Call where a step's results are consumed.
+  void check_cluster_waits()
+  {
+    m_ws.check(io.stream, "check_cluster_waits");
+  }
+
 private:
   int64_t m_dim;
   bool m_single_dim_mode;
@@ -524,8 +639,9 @@ public:
     const size_t bytes = lbn_instance_norm_fwd_workspace_bytes(num_channels(), channel_size(), x.Width());
     check_status(lbn_instance_norm_fwd_f32(io.stream, num_channels(), channel_size(), x.Width(), m_epsilon,
                                            x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(),
-                                           m_workspace.Buffer(), m_workspace.LDim(), m_ws_fwd.reserve(bytes), bytes),
+                                           m_workspace.Buffer(), m_workspace.LDim(), m_ws_fwd.reserve(bytes, io.stream), bytes),
                  "instance_norm_layer::fp_compute");
+    m_ws_fwd.after_call(io.stream, "instance_norm_layer::fp_compute");
   }
   void bp_compute()
   {
@@ -536,9 +652,20 @@ public:
     check_status(lbn_instance_norm_bwd_f32(io.stream, num_channels(), channel_size(), x.Width(), m_epsilon,
                                            x.LockedBuffer(), x.LDim(), dy.LockedBuffer(), dy.LDim(),
                                            dx.Buffer(), dx.LDim(), m_workspace.LockedBuffer(),
-                                           m_workspace.LDim(), m_ws.reserve(bytes), bytes),
+                                           m_workspace.LDim(), m_ws.reserve(bytes, io.stream), bytes),
                  "instance_norm_layer::bp_compute");
+    m_ws.after_call(io.stream, "instance_norm_layer::bp_compute");
   }
+  /// The layer's scratch buffer (reserve it up front to keep the hooks free of allocation).
+  workspace& scratch() { return m_ws; }
+  /// Throws if a wait between workgroups ran out in a call of this layer since the last
+  /// check; waits for the stream.  Call where a step's results are consumed.
+  void check_cluster_waits()
+  {
+    m_ws_fwd.check(io.stream, "instance_norm_layer (forward scratch)");
+    m_ws.check(io.stream, "check_cluster_waits");
+  }
+
 private:
   float m_epsilon;
   std::vector<int64_t> m_dims;
@@ -691,7 +818,7 @@ public:
     const size_t bytes = lbn_cross_entropy_fwd_workspace_bytes(x.Height(), x.Width());
     check_status(lbn_cross_entropy_fwd_f32(io.stream, x.Height(), x.Width(), m_use_labels ? 1 : 0,
                                            m_spatial_sample_size, x.LockedBuffer(), x.LDim(), t.LockedBuffer(),
-                                           t.LDim(), loss.Buffer(), loss.LDim(), m_ws.reserve(bytes), bytes),
+                                           t.LDim(), loss.Buffer(), loss.LDim(), m_ws.reserve(bytes, io.stream), bytes),
                  "cross_entropy_layer::fp_compute");
   }
   void bp_compute()
@@ -749,7 +876,7 @@ public:
     check_status(lbn_entrywise_scale_bias_bwd_f32(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(),
                                                   dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(), m_weights,
                                                   m_ld_weights, m_weights_gradient.Buffer(),
-                                                  m_weights_gradient.LDim(), m_ws.reserve(bytes), bytes),
+                                                  m_weights_gradient.LDim(), m_ws.reserve(bytes, io.stream), bytes),
                  "entrywise_scale_bias_layer::bp_compute");
   }
 private:
@@ -797,7 +924,7 @@ public:
                                                     x.LockedBuffer(), x.LDim(), dy.LockedBuffer(), dy.LDim(),
                                                     dx.Buffer(), dx.LDim(), m_weights, m_ld_weights,
                                                     m_weights_gradient.Buffer(), m_weights_gradient.LDim(),
-                                                    m_ws.reserve(bytes), bytes),
+                                                    m_ws.reserve(bytes, io.stream), bytes),
                  "channelwise_scale_bias_layer::bp_compute");
   }
 private:

@@ -667,6 +667,237 @@ bn_bwd_cluster(BnBwdArgs<S> a, unsigned seg, unsigned E)
   }
 }
 
+// ------------------------------------------------ the same rotation without barriers
+// Variant of the cluster kernels above in which the waves of a workgroup never meet at a
+// barrier after the start-up (WaveMerge in cluster_sync.hpp): a wave adds its share, leaves
+// the pair in LDS and counts itself in; the last wave to do so publishes the workgroup's
+// sums; the first wave that needs the cluster's totals polls for them and hands them to the
+// others through LDS.  Measured on 64 x 256 x 56 x 56: fp16 storage, whose steps are half as
+// long, gains 6 % (91.7 against 97.7 us per step); fp32 loses 2.5 % (186 against 181 us), so
+// the host side picks this variant for 16-bit storage only.  Letting every wave poll the
+// cluster for itself was 30 % slower: a wave's polling loads return only after its earlier
+// stores are acknowledged, and then all waves wait for that instead of one.
+// (1) of a step: partial sums of channel `ch` from tile `t`; the wave that completes the
+// workgroup's sums publishes them for the cluster.  No barrier: see WaveMerge.
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_fwd_reduce_ws(const BnFwdArgs<S>& a, const BnIndex<V>& ix, int ch, int k,
+                                              const BnFwdTile<S, V>& t, WaveMerge<T / kWave>& stage)
+{
+  const float K = t.K;
+  float s = 0.f, q = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    float v[Vec16<S>::N];
+    Vec16<S>::unpack(t.v[i], v);
+#pragma unroll
+    for (int j = 0; j < Vec16<S>::N; ++j) {
+      const float d = ix.ok[i] ? v[j] - K : 0.f;
+      s += d;
+      q += d * d;
+    }
+  }
+  s = wave_sum_in_last(s);
+  q = wave_sum_in_last(q);
+  if (wave_merge_arrive(stage, s, q)) {
+    wave_merge_read(stage, 0.f, 0.f, s, q);
+    s = wave_sum_in_last(s);  // waves in index order: the same sum whichever wave came last
+    q = wave_sum_in_last(q);
+    if ((threadIdx.x & (kWave - 1)) == kWave - 1)
+      cluster_publish(s, q, a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, k, a.tag);
+  }
+}
+
+// (3) of a step, per wave: statistics of channel `ch` from the cluster's partials (the
+// first round of polling loads is already under way in `poll`), output from tile `t`.
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_fwd_finish_ws(const BnFwdArgs<S>& a, const BnIndex<V>& ix, int ch, int k,
+                                              BnFwdTile<S, V>& t, ClusterPollWide& poll,
+                                              WaveMerge<T / kWave>& stage_f, bool poller, unsigned use)
+{
+  float ts, tq;
+  if (poller) {
+    cluster_poll_sums(poll, a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, a.M, a.tag, a.cw.error, ts, tq);
+    wave_merge_broadcast(stage_f, use, ts, tq);
+  }
+  else {
+    wave_merge_wait(stage_f, use, ts, tq);
+  }
+  float mean, var;
+  stats_from_sums(ts, tq, t.K, a.n, a.bessel, a.eps, mean, var);
+  const float inv_stdev = 1.0f / sqrtf(var + a.eps);
+  if (k == 0 && threadIdx.x == 0) {
+    a.mean_out[ch] = mean;
+    a.var_out[ch] = var;
+    a.rmean[ch] = a.decay * a.rmean[ch] + (1.f - a.decay) * mean;
+    a.rvar[ch] = a.decay * a.rvar[ch] + (1.f - a.decay) * var;
+  }
+  S* yc = a.y + static_cast<int64_t>(ch) * a.cs;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    if (!ix.ok[i]) continue;
+    float v[Vec16<S>::N];
+    Vec16<S>::unpack(t.v[i], v);
+#pragma unroll
+    for (int j = 0; j < Vec16<S>::N; ++j) v[j] = t.scale * ((v[j] - mean) * inv_stdev) + t.bias;
+    Vec16<S>::store(bn_tile_address<S, V>(yc, a.ldy, ix, i), v);
+  }
+}
+
+// One step of the rotation: F finishes channel ch, R holds channel ch + nc, L
+// receives channel ch + 2 nc.  The polling loads for F go out before the loads of L, so
+// their words are back first and L's loads stay in flight while F is written.
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_fwd_step_ws(const BnFwdArgs<S>& a, const BnIndex<V>& ix, int ch, int nc, int k,
+                                            BnFwdTile<S, V>& F, BnFwdTile<S, V>& R, BnFwdTile<S, V>& L,
+                                            WaveMerge<T / kWave>& stage_r, WaveMerge<T / kWave>& stage_f,
+                                            unsigned use)
+{
+  if (ch + nc < a.C) bn_fwd_reduce_ws<S, T, V>(a, ix, ch + nc, k, R, stage_r);
+  ClusterPollWide poll;
+  const bool poller = wave_merge_claim(stage_f);
+  if (poller) cluster_poll_issue(poll, a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, a.M);
+  asm volatile("" ::: "memory");  // polling loads first, then the tile
+  if (ch + 2 * nc < a.C) bn_fwd_load<S, V>(L, a, ch + 2 * nc, ix);
+  asm volatile("" ::: "memory");  // keep the loads above the wait below
+  bn_fwd_finish_ws<S, T, V>(a, ix, ch, k, F, poll, stage_f, poller, use);
+}
+
+template <typename S, int T, int V>
+__global__ void __launch_bounds__(T)
+bn_fwd_cluster_ws(BnFwdArgs<S> a, unsigned seg, unsigned E)
+{
+  __shared__ WaveMerge<T / kWave> stage[3];  // one per position of the rotation
+  const int nc = gridDim.x / a.M;
+  const int cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - cl * a.M;
+  const BnIndex<V> ix = bn_make_index<T, V>(k, seg, E);
+  BnFwdTile<S, V> t0, t1, t2;
+  if (cl >= a.C) return;
+  cluster_resolve_tag(a.tag);
+  bn_fwd_load<S, V>(t0, a, cl, ix);
+  if (cl + nc < a.C) bn_fwd_load<S, V>(t1, a, cl + nc, ix);
+  wave_merge_init(stage, 3);
+  __syncthreads();  // the kernel's only barrier
+  bn_fwd_reduce_ws<S, T, V>(a, ix, cl, k, t0, stage[0]);
+  unsigned use = 0;
+  for (int ch = cl; ch < a.C; ch += 3 * nc, ++use) {
+    bn_fwd_step_ws<S, T, V>(a, ix, ch, nc, k, t0, t1, t2, stage[1], stage[0], use);
+    if (ch + nc < a.C) bn_fwd_step_ws<S, T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, stage[2], stage[1], use);
+    if (ch + 2 * nc < a.C) bn_fwd_step_ws<S, T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, stage[0], stage[2], use);
+  }
+}
+
+// Publishes A = sum(dy), B = sum(dy * (x - mean)); vectors past the end hold zeros in dy.
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_bwd_reduce_ws(const BnBwdArgs<S>& a, const BnIndex<V>& ix, int ch, int k,
+                                              const BnBwdTile<S, V>& t, WaveMerge<T / kWave>& stage)
+{
+  const float mean = t.mean;
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    float x[Vec16<S>::N], g[Vec16<S>::N];
+    Vec16<S>::unpack(t.x[i], x);
+    Vec16<S>::unpack(t.g[i], g);
+#pragma unroll
+    for (int j = 0; j < Vec16<S>::N; ++j) {
+      sa += g[j];
+      sb += g[j] * (x[j] - mean);
+    }
+  }
+  sa = wave_sum_in_last(sa);
+  sb = wave_sum_in_last(sb);
+  if (wave_merge_arrive(stage, sa, sb)) {
+    wave_merge_read(stage, 0.f, 0.f, sa, sb);
+    sa = wave_sum_in_last(sa);
+    sb = wave_sum_in_last(sb);
+    if ((threadIdx.x & (kWave - 1)) == kWave - 1)
+      cluster_publish(sa, sb, a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, k, a.tag);
+  }
+}
+
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_bwd_finish_ws(const BnBwdArgs<S>& a, const BnIndex<V>& ix, int ch, int k,
+                                              BnBwdTile<S, V>& t, ClusterPollWide& poll,
+                                              WaveMerge<T / kWave>& stage_f, bool poller, unsigned use)
+{
+  const float inv_stdev = 1.0f / sqrtf(t.var + a.eps);
+  const float scale = t.scale;
+  float ta, tb;
+  if (poller) {
+    cluster_poll_sums(poll, a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, a.M, a.tag, a.cw.error, ta, tb);
+    wave_merge_broadcast(stage_f, use, ta, tb);
+  }
+  else {
+    wave_merge_wait(stage_f, use, ta, tb);
+  }
+  float ds, db, dmean, dvar;
+  grads_from_sums(ta, tb, scale, inv_stdev, ds, db, dmean, dvar);
+  const float dmean_term = dmean / static_cast<float>(a.n);
+  const float dvar_term = dvar * 2.f / static_cast<float>(a.n - (a.bessel ? 1 : 0));
+  if (k == 0 && threadIdx.x == 0) {
+    a.dscale[ch] = ds;
+    a.dbias[ch] = db;
+    a.dmean_out[ch] = dmean;
+    a.dvar_out[ch] = dvar;
+  }
+  const float k0 = scale * inv_stdev;
+  const float mean = t.mean;
+  S* dxc = a.dx + static_cast<int64_t>(ch) * a.cs;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    if (!ix.ok[i]) continue;
+    float x[Vec16<S>::N], g[Vec16<S>::N];
+    Vec16<S>::unpack(t.x[i], x);
+    Vec16<S>::unpack(t.g[i], g);
+#pragma unroll
+    for (int j = 0; j < Vec16<S>::N; ++j) g[j] = g[j] * k0 + dmean_term + dvar_term * (x[j] - mean);
+    Vec16<S>::store(bn_tile_address<S, V>(dxc, a.lddx, ix, i), g);
+  }
+}
+
+template <typename S, int T, int V>
+__device__ __forceinline__ void bn_bwd_step_ws(const BnBwdArgs<S>& a, const BnIndex<V>& ix, int ch, int nc, int k,
+                                            BnBwdTile<S, V>& F, BnBwdTile<S, V>& R, BnBwdTile<S, V>& L,
+                                            WaveMerge<T / kWave>& stage_r, WaveMerge<T / kWave>& stage_f,
+                                            unsigned use)
+{
+  if (ch + nc < a.C) bn_bwd_reduce_ws<S, T, V>(a, ix, ch + nc, k, R, stage_r);
+  ClusterPollWide poll;
+  const bool poller = wave_merge_claim(stage_f);
+  if (poller) cluster_poll_issue(poll, a.cw.slots + static_cast<int64_t>(ch) * a.M * 2, a.M);
+  asm volatile("" ::: "memory");
+  if (ch + 2 * nc < a.C) bn_bwd_load<S, V>(L, a, ch + 2 * nc, ix);
+  asm volatile("" ::: "memory");
+  bn_bwd_finish_ws<S, T, V>(a, ix, ch, k, F, poll, stage_f, poller, use);
+}
+
+// Backward in training mode: x and dy are read once, dx written once.
+template <typename S, int T, int V>
+__global__ void __launch_bounds__(T)
+bn_bwd_cluster_ws(BnBwdArgs<S> a, unsigned seg, unsigned E)
+{
+  __shared__ WaveMerge<T / kWave> stage[3];
+  const int nc = gridDim.x / a.M;
+  const int cl = blockIdx.x / a.M;
+  const int k = blockIdx.x - cl * a.M;
+  const BnIndex<V> ix = bn_make_index<T, V>(k, seg, E);
+  BnBwdTile<S, V> t0, t1, t2;
+  if (cl >= a.C) return;
+  cluster_resolve_tag(a.tag);
+  bn_bwd_load<S, V>(t0, a, cl, ix);
+  if (cl + nc < a.C) bn_bwd_load<S, V>(t1, a, cl + nc, ix);
+  wave_merge_init(stage, 3);
+  __syncthreads();  // the kernel's only barrier
+  bn_bwd_reduce_ws<S, T, V>(a, ix, cl, k, t0, stage[0]);
+  unsigned use = 0;
+  for (int ch = cl; ch < a.C; ch += 3 * nc, ++use) {
+    bn_bwd_step_ws<S, T, V>(a, ix, ch, nc, k, t0, t1, t2, stage[1], stage[0], use);
+    if (ch + nc < a.C) bn_bwd_step_ws<S, T, V>(a, ix, ch + nc, nc, k, t1, t2, t0, stage[2], stage[1], use);
+    if (ch + 2 * nc < a.C) bn_bwd_step_ws<S, T, V>(a, ix, ch + 2 * nc, nc, k, t2, t0, t1, stage[0], stage[2], use);
+  }
+}
+
 // Workgroup size and vectors per thread of a cluster launch for channels of E vectors.
 struct BnClusterShape {
   int T, V, M;
@@ -692,6 +923,10 @@ static BnClusterShape bn_cluster_shape(int64_t E, int max_v, int first_t)
   return {0, 0, 0};
 }
 
+// 16-bit storage runs the barrier-free variant of the cluster kernels.
+template <typename S>
+constexpr bool kBnWaveSync = sizeof(S) == 2;
+
 // ==================================================================== host side
 // Workgroups per channel: about 4096 workgroups in total, each with at least four
 // accesses per thread, at most one wave's worth so a wave can merge the partials.
@@ -714,11 +949,11 @@ constexpr int64_t kBnTileMaxCs = 16;  // aligned channels up to here still try t
 static size_t bn_workspace(int64_t C, int64_t cs, int64_t w)
 {
   if (C <= 0 || cs <= 0 || w <= 0) return 0;
-  const size_t split = static_cast<size_t>(C) * bn_split(C, cs, w) * sizeof(float2);
+  const size_t split = kWorkspaceHeaderBytes + static_cast<size_t>(C) * bn_split(C, cs, w) * sizeof(float2);
   const size_t cluster = cluster_workspace_bytes(C, kClusterMaxSumM);
   size_t need = split > cluster ? split : cluster;
   if (bn_rt_shape(cs) && (C * cs) % 4 == 0) {  // the row-tile path of batch_norm_rows.hpp
-    const size_t rows = bn_rt_workspace_bytes(C * cs, w);
+    const size_t rows = kWorkspaceHeaderBytes + bn_rt_workspace_bytes(C * cs, w);
     if (rows > need) need = rows;
   }
   return need;
@@ -729,20 +964,30 @@ static size_t bn_workspace(int64_t C, int64_t cs, int64_t w)
 template <typename S, int T, int V>
 static bool bn_launch_fwd_cluster(hipStream_t st, const BnFwdArgs<S>& a, int64_t C, unsigned seg, unsigned E)
 {
-  const int cap = cluster_capacity(bn_fwd_cluster<S, T, V>, T);
+  int cap;
+  if constexpr (kBnWaveSync<S>) cap = cluster_capacity(bn_fwd_cluster_ws<S, T, V>, T);
+  else cap = cluster_capacity(bn_fwd_cluster<S, T, V>, T);
   const int64_t ncl = cap / a.M < C ? cap / a.M : C;
   if (ncl < 1) return false;
-  hipLaunchKernelGGL((bn_fwd_cluster<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
+  if constexpr (kBnWaveSync<S>)
+    hipLaunchKernelGGL((bn_fwd_cluster_ws<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
+  else
+    hipLaunchKernelGGL((bn_fwd_cluster<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
   return true;
 }
 
 template <typename S, int T, int V>
 static bool bn_launch_bwd_cluster(hipStream_t st, const BnBwdArgs<S>& a, int64_t C, unsigned seg, unsigned E)
 {
-  const int cap = cluster_capacity(bn_bwd_cluster<S, T, V>, T);
+  int cap;
+  if constexpr (kBnWaveSync<S>) cap = cluster_capacity(bn_bwd_cluster_ws<S, T, V>, T);
+  else cap = cluster_capacity(bn_bwd_cluster<S, T, V>, T);
   const int64_t ncl = cap / a.M < C ? cap / a.M : C;
   if (ncl < 1) return false;
-  hipLaunchKernelGGL((bn_bwd_cluster<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
+  if constexpr (kBnWaveSync<S>)
+    hipLaunchKernelGGL((bn_bwd_cluster_ws<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
+  else
+    hipLaunchKernelGGL((bn_bwd_cluster<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
   return true;
 }
 
@@ -970,7 +1215,7 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
     return LBN_ERR_INVALID_ARGUMENT;
   if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
   const int P = bn_split(C, cs, w);
-  float2* part = static_cast<float2*>(workspace);
+  float2* part = static_cast<float2*>(workspace_payload(workspace));
   const dim3 grid(static_cast<unsigned>(C), P);
   const int pivot = (flags & LBN_STATS_SUMSQ) ? 0 : 1;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, y, ldy);
@@ -1048,7 +1293,7 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
     return LBN_ERR_INVALID_ARGUMENT;
   if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
   const int P = bn_split(C, cs, w);
-  float2* part = static_cast<float2*>(workspace);
+  float2* part = static_cast<float2*>(workspace_payload(workspace));
   const dim3 grid(static_cast<unsigned>(C), P);
   const int64_t n = cs * w;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, dy, lddy) && bn_vec_ok<S>(cs, w, dx, lddx);
@@ -1135,7 +1380,7 @@ int lbn_batch_norm_fwd_sums_f32(lbn_stream_t stream, int64_t C, int64_t cs, int6
   if (!x || !mean || !var) return LBN_ERR_INVALID_ARGUMENT;
   if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
   const int P = bn_split(C, cs, w);
-  float2* part = static_cast<float2*>(workspace);
+  float2* part = static_cast<float2*>(workspace_payload(workspace));
   const dim3 grid(static_cast<unsigned>(C), P);
   hipStream_t st = as_stream(stream);
   if (bn_vec_ok<float>(cs, w, x, ldx))
@@ -1206,7 +1451,7 @@ int lbn_batch_norm_bwd_sums_f32(lbn_stream_t stream, int64_t C, int64_t cs, int6
     return LBN_ERR_INVALID_ARGUMENT;
   if (!workspace || workspace_bytes < bn_workspace(C, cs, w)) return LBN_ERR_WORKSPACE;
   const int P = bn_split(C, cs, w);
-  float2* part = static_cast<float2*>(workspace);
+  float2* part = static_cast<float2*>(workspace_payload(workspace));
   const dim3 grid(static_cast<unsigned>(C), P);
   hipStream_t st = as_stream(stream);
   if (bn_vec_ok<float>(cs, w, x, ldx) && bn_vec_ok<float>(cs, w, dy, lddy))

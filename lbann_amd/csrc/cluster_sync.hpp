@@ -100,7 +100,7 @@ __device__ __forceinline__ void cluster_publish(float a, float b, unsigned long 
 // workgroup j in (ra, rb); lanes >= M hold (na, nb).
 __device__ __forceinline__ void cluster_collect(unsigned long long* slots, int M, ClusterTag tag,
                                                 int* error_word, float na, float nb, float& ra,
-                                                float& rb)
+                                                float& rb, int max_polls = kClusterMaxPolls)
 {
   const int lane = threadIdx.x & 63;
   unsigned long long wa = 0, wb = 0;
@@ -113,7 +113,7 @@ __device__ __forceinline__ void cluster_collect(unsigned long long* slots, int M
       have = static_cast<unsigned>(wa >> 32) == tag.lo && static_cast<unsigned>(wb >> 32) == tag.hi;
     }
     if (__all(have || lane >= M)) break;
-    if (++polls > kClusterMaxPolls) {
+    if (++polls > max_polls) {
       if (lane == 0) __hip_atomic_store(error_word, kClusterTimedOut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       break;
     }
@@ -188,6 +188,198 @@ __device__ __forceinline__ void cluster_collect_sums(unsigned long long* slots, 
   tb = cluster_wave_total(b);
 }
 
+// ------------------------------------------------- waves that never meet at a barrier
+// A variant of the cluster kernels keeps its waves free of workgroup barriers: a wave
+// leaves its partial pair in LDS and counts itself in; the wave that arrives last adds the
+// workgroup's pairs in wave order (so the result does not depend on which wave that was)
+// and publishes them for the cluster; the first wave that needs the cluster's totals takes
+// the polling duty and hands them to the others through LDS.  A fast wave is then never
+// held back by the slowest wave of its workgroup, only by the data it needs.
+//
+// `count` and `claim` are never reset: a use of the stage is complete when they reach the
+// next multiple of NW; `ready` counts completed hand-overs.  A stage may be reused for
+// item i + 2 or later: a wave gets to item i + 2 only after it has seen item i published,
+// which the last wave of item i does after it has read the stage.
+template <int NW>
+struct WaveMerge {
+  float part[NW][2];
+  unsigned count;
+  unsigned claim, ready;
+  float total[2];
+};
+
+// Zeroes the counters of `n` stages; the caller follows with the kernel's one barrier.
+template <int NW>
+__device__ __forceinline__ void wave_merge_init(WaveMerge<NW>* stages, int n)
+{
+  if (static_cast<int>(threadIdx.x) < n) stages[threadIdx.x].count = stages[threadIdx.x].claim = stages[threadIdx.x].ready = 0;
+}
+
+// Called by every wave of the workgroup once per item, with its pair valid in lane 63.
+// True (in all lanes) in the wave that arrived last.
+template <int NW>
+__device__ __forceinline__ bool wave_merge_arrive(WaveMerge<NW>& st, float a, float b)
+{
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = wave_index();
+  unsigned prev = 0;
+  if (lane == kWave - 1) {
+    st.part[wave][0] = a;
+    st.part[wave][1] = b;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");  // LDS only: no wait for global memory
+    prev = __hip_atomic_fetch_add(&st.count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  prev = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(prev), kWave - 1));
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+  return prev % NW == NW - 1;
+}
+
+// Finish side with one polling wave per workgroup: the first wave to ask takes the duty
+// (true), polls the cluster, and hands the totals to the others through LDS; `use` counts
+// the earlier uses of the stage.
+template <int NW>
+__device__ __forceinline__ bool wave_merge_claim(WaveMerge<NW>& st)
+{
+  unsigned prev = 0;
+  if ((threadIdx.x & (kWave - 1)) == kWave - 1)
+    prev = __hip_atomic_fetch_add(&st.claim, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  prev = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(prev), kWave - 1));
+  return prev % NW == 0;
+}
+
+template <int NW>
+__device__ __forceinline__ void wave_merge_broadcast(WaveMerge<NW>& st, unsigned use, float a, float b)
+{
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    st.total[0] = a;
+    st.total[1] = b;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __hip_atomic_store(&st.ready, use + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+}
+
+template <int NW>
+__device__ __forceinline__ void wave_merge_wait(WaveMerge<NW>& st, unsigned use, float& a, float& b)
+{
+  // bounded like the cluster polls: the polling wave gives up after kClusterMaxPolls rounds
+  // and still broadcasts, so this loop ends as well
+  while (__hip_atomic_load(&st.ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != use + 1)
+    __builtin_amdgcn_s_sleep(1);
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+  a = st.total[0];
+  b = st.total[1];
+}
+
+// In the last wave: lane j < NW gets the pair of wave j, the other lanes (na, nb).
+template <int NW>
+__device__ __forceinline__ void wave_merge_read(const WaveMerge<NW>& st, float na, float nb, float& a, float& b)
+{
+  static_assert(NW <= kWave, "one lane per wave of the workgroup");
+  const int lane = threadIdx.x & (kWave - 1);
+  a = lane < NW ? st.part[lane][0] : na;
+  b = lane < NW ? st.part[lane][1] : nb;
+}
+
+// One round of polling loads of a cluster's M slots, H slots per lane (lane j takes slots
+// j, j + 64, ...), without waiting for them: issued ahead of other loads, the words are
+// back first (a wave's loads return in order).
+template <int H>
+struct ClusterPoll {
+  unsigned long long w[H][2];
+};
+
+template <int H>
+__device__ __forceinline__ void cluster_poll_issue(ClusterPoll<H>& p, const unsigned long long* slots, int M)
+{
+  const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int h = 0; h < H; ++h) {
+    const int j = lane + kWave * h;
+    p.w[h][0] = p.w[h][1] = 0;
+    if (j < M) {
+      p.w[h][0] = __hip_atomic_load(slots + 2 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      p.w[h][1] = __hip_atomic_load(slots + 2 * j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// Completes a poll begun with cluster_poll_issue(): polls again until all M slots carry the
+// call's tag (bounded as in cluster_collect()).  On return have[h] tells whether lane j's
+// slot j + 64 h holds a published pair, in the low halves of p.w[h].
+template <int H>
+__device__ __forceinline__ void cluster_poll_complete(ClusterPoll<H>& p, const unsigned long long* slots, int M,
+                                                      ClusterTag tag, int* error_word, bool (&have)[H])
+{
+  const int lane = threadIdx.x & (kWave - 1);
+  int polls = 0;
+  for (;;) {
+    bool all = true;
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      have[h] = static_cast<unsigned>(p.w[h][0] >> 32) == tag.lo && static_cast<unsigned>(p.w[h][1] >> 32) == tag.hi;
+      all = all && (have[h] || lane + kWave * h >= M);
+    }
+    if (__all(all)) break;
+    if (++polls > kClusterMaxPolls) {
+      if (lane == 0) __hip_atomic_store(error_word, kClusterTimedOut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const int j = lane + kWave * h;
+      if (j < M && !have[h]) {
+        p.w[h][0] = __hip_atomic_load(slots + 2 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        p.w[h][1] = __hip_atomic_load(slots + 2 * j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+}
+
+// The cluster's totals of pairs that are simply added; every lane returns them.
+template <int H>
+__device__ __forceinline__ void cluster_poll_sums(ClusterPoll<H>& p, const unsigned long long* slots, int M,
+                                                  ClusterTag tag, int* error_word, float& ta, float& tb)
+{
+  bool have[H];
+  cluster_poll_complete<H>(p, slots, M, tag, error_word, have);
+  float a = 0.f, b = 0.f;
+#pragma unroll
+  for (int h = 0; h < H; ++h) {
+    if (have[h]) {
+      a += __uint_as_float(static_cast<unsigned>(p.w[h][0]));
+      b += __uint_as_float(static_cast<unsigned>(p.w[h][1]));
+    }
+  }
+  ta = cluster_wave_total(a);
+  tb = cluster_wave_total(b);
+}
+
+// Clusters of up to 2 x 64 members: two one-slot-per-lane polls, the second only when
+// M > 64.  (One loop over two slots per lane costs the compiler's register coalescer
+// several seconds per kernel; two plain loops cost nothing.)
+struct ClusterPollWide {
+  ClusterPoll<1> lo, hi;
+};
+
+__device__ __forceinline__ void cluster_poll_issue(ClusterPollWide& p, const unsigned long long* slots, int M)
+{
+  cluster_poll_issue(p.lo, slots, M < kWave ? M : kWave);
+  if (M > kWave) cluster_poll_issue(p.hi, slots + 2 * kWave, M - kWave);
+}
+
+__device__ __forceinline__ void cluster_poll_sums(ClusterPollWide& p, const unsigned long long* slots, int M,
+                                                  ClusterTag tag, int* error_word, float& ta, float& tb)
+{
+  cluster_poll_sums(p.lo, slots, M < kWave ? M : kWave, tag, error_word, ta, tb);
+  if (M > kWave) {
+    float ha, hb;
+    cluster_poll_sums(p.hi, slots + 2 * kWave, M - kWave, tag, error_word, ha, hb);
+    ta += ha;
+    tb += hb;
+  }
+}
+
 // Publish and collect in one go.
 __device__ __forceinline__ void cluster_exchange(float a, float b, unsigned long long* slots, int k,
                                                  int M, ClusterTag tag, int* error_word, float na,
@@ -197,8 +389,14 @@ __device__ __forceinline__ void cluster_exchange(float a, float b, unsigned long
   cluster_collect(slots, M, tag, error_word, na, nb, ra, rb);
 }
 
-// Layout of the cluster part of a workspace: 64 bytes of header (error word at byte 0, replay
-// counter at byte 8), then two 64-bit words per slot.
+// Layout of a workspace: 64 bytes of header (error word at byte 0, replay counter at byte 8)
+// that only the cluster kernels write, then the call's scratch: two 64-bit words per slot for
+// a cluster kernel, partial sums for the multi-kernel paths (workspace_payload()).  Keeping
+// the partial sums out of the header means that a call which takes a multi-kernel path can
+// neither clear a raised error word nor raise one by accident.
+constexpr size_t kWorkspaceHeaderBytes = 64;
+
+inline void* workspace_payload(void* ws) { return static_cast<char*>(ws) + kWorkspaceHeaderBytes; }
 struct ClusterWorkspace {
   int* error;
   unsigned long long* replay_word;

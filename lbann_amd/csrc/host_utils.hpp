@@ -14,9 +14,16 @@
 
 namespace lbn {
 
-inline hipStream_t as_stream(lbn_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+// Every entry point converts its stream argument first: that is also where an error left
+// behind by an earlier, unrelated HIP call of this thread is dropped, so that
+// launch_status() below reports this call's launches only.
+inline hipStream_t as_stream(lbn_stream_t s)
+{
+  (void)hipGetLastError();
+  return reinterpret_cast<hipStream_t>(s);
+}
 
-// Status of the launches issued so far by this thread: 0 or the hipError_t.
+// Status of the launches issued by this thread since the entry point began: 0 or the hipError_t.
 inline int launch_status()
 {
   const hipError_t e = hipGetLastError();

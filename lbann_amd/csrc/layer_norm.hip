@@ -260,6 +260,97 @@ ln_fwd_generic(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t 
 }
 
 // ================================================================== backward
+// Weight gradients of small problems without any exchange between workgroups: dscale and
+// dbias of a feature depend on x, dy and the FORWARD statistics only (xh = (x - mean) /
+// stdev needs nothing from this pass), so a workgroup can form them for a slice of eight
+// access units of features over all rows by reading that column slice itself.  The tensors
+// are read a second time, from the caches: worth it while they fit them, where it saves
+// the partial rows, the reduction kernel and its launch (1024 x 128: three dependent
+// kernels per step become two).  Threads = 8 access units x (threads / 8) row groups; the
+// sums over rows and row groups run in a fixed order.
+template <typename T>
+struct LnColLoads {
+  typename Vec16<T>::raw_t x[4], g[4];
+  float mean[4], var[4];
+};
+
+template <typename T, int THREADS>
+__device__ __forceinline__ void ln_cols_issue(LnColLoads<T>& c, const T* x, const T* dy, int64_t ldx, int64_t lddy,
+                                              const RowMap& map, int64_t rows, int n, const float* stats,
+                                              int64_t ld_stats, int64_t slice, int64_t row0)
+{
+  constexpr int VE = Vec16<T>::N;
+  constexpr int RG = THREADS / 8;
+  const int kq = threadIdx.x & 7, pg = threadIdx.x >> 3;
+  int64_t k = (slice * 8 + kq) * VE;
+  if (k >= n) k = 0;  // loads past the end re-read valid memory and are masked when used
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int64_t r = row0 + pg + RG * j;
+    if (r >= rows) r = rows - 1;
+    int64_t col, g;
+    map.split(r, col, g);
+    c.x[j] = Vec16<T>::load_raw(x + g * map.stride + col * ldx + k);
+    c.g[j] = Vec16<T>::load_raw(dy + g * map.stride + col * lddy + k);
+    c.mean[j] = stats[g + col * ld_stats];
+    c.var[j] = stats[map.groups + g + col * ld_stats];
+  }
+}
+
+template <typename T, int THREADS>
+__device__ __forceinline__ void ln_cols_accumulate(const LnColLoads<T>& c, int64_t rows, int n, float eps,
+                                                   int64_t slice, int64_t row0, float (&dg)[Vec16<T>::N],
+                                                   float (&db)[Vec16<T>::N])
+{
+  constexpr int VE = Vec16<T>::N;
+  constexpr int RG = THREADS / 8;
+  const int kq = threadIdx.x & 7, pg = threadIdx.x >> 3;
+  const bool col_ok = (slice * 8 + kq) * VE < n;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const bool use = col_ok && row0 + pg + RG * j < rows;
+    const float inv_stdev = rsqrt_refined(c.var[j] + eps);
+    float xv[VE], gv[VE];
+    Vec16<T>::unpack(c.x[j], xv);
+    Vec16<T>::unpack(c.g[j], gv);
+#pragma unroll
+    for (int e = 0; e < VE; ++e) {
+      const float g = use ? gv[e] : 0.f;
+      db[e] += g;
+      dg[e] = __builtin_fmaf(g, (xv[e] - c.mean[j]) * inv_stdev, dg[e]);
+    }
+  }
+}
+
+// Adds the row groups' sums of a slice through LDS (sm: 2 x RG x (8 VE + 1) floats) and writes
+// the slice's entries of dscale and dbias.
+template <typename T, int THREADS>
+__device__ __forceinline__ void ln_cols_finish(float* sm, int n, int64_t slice, const float (&dg)[Vec16<T>::N],
+                                               const float (&db)[Vec16<T>::N], float* dscale, float* dbias)
+{
+  constexpr int VE = Vec16<T>::N;
+  constexpr int RG = THREADS / 8;
+  constexpr int W = 8 * VE + 1;
+  const int kq = threadIdx.x & 7, pg = threadIdx.x >> 3;
+#pragma unroll
+  for (int e = 0; e < VE; ++e) {
+    sm[pg * W + kq * VE + e] = dg[e];
+    sm[(RG + pg) * W + kq * VE + e] = db[e];
+  }
+  __syncthreads();
+  if (threadIdx.x < 2 * 8 * VE) {
+    const int which = threadIdx.x / (8 * VE), c = threadIdx.x - which * (8 * VE);
+    const float* col = sm + which * RG * W + c;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int r = 0; r < RG; r += 4) acc += (col[r * W] + col[(r + 1) * W]) + (col[(r + 2) * W] + col[(r + 3) * W]);
+    const int64_t k = slice * 8 * VE + c;
+    float* out = which == 0 ? dscale : dbias;
+    if (out && k < n) out[k] = acc;
+  }
+  __syncthreads();  // the next slice writes sm again
+}
+
 // Partial weight gradients: block b writes 2*n floats at part + b*2*n (dscale row
 // followed by dbias row).
 //
@@ -271,13 +362,19 @@ ln_fwd_generic(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t 
 //
 // A team's next row is in flight, still packed, while the current one is processed,
 // unless a thread owns 32 entries: then the registers only hold the current row.
-template <typename T, int TPR, int TEAMS, int V, bool WGRAD>
+//
+// COLS (small problems, instead of WGRAD): the workgroup also forms dscale and dbias of its
+// feature slices from the column slices of x and dy (ln_cols_*); `part` is unused and
+// (dscale, dbias) are written directly.  The first column loads go out before the row work.
+template <typename T, int TPR, int TEAMS, int V, bool WGRAD, bool COLS = false>
 __global__ void __launch_bounds__((RowBlock<TPR, TEAMS>::kThreads))
 ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ dx, int64_t ldx,
             int64_t lddy, int64_t lddx, RowMap map, int64_t rows, int nvec, int n, float eps,
             const float* __restrict__ stats, int64_t ld_stats, float* __restrict__ sgrad,
-            int64_t ld_sgrad, const float* __restrict__ gamma, float* __restrict__ part)
+            int64_t ld_sgrad, const float* __restrict__ gamma, float* __restrict__ part,
+            float* __restrict__ dscale, float* __restrict__ dbias)
 {
+  static_assert(!(WGRAD && COLS), "one way of forming the weight gradients");
   using B = RowBlock<TPR, TEAMS>;
   using IO = Vec16<T>;
   using raw_t = typename IO::raw_t;
@@ -289,11 +386,18 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   constexpr bool kPrefetch = V * VE < 32;
   __shared__ float red[2][TEAMS][2 * NW];
   __shared__ float acc_lds[kAccLds];
+  constexpr int kColLds = COLS ? 2 * (B::kThreads / 8) * (8 * VE + 1) : 1;
+  __shared__ float col_lds[kColLds];
   const int tid = threadIdx.x;
   const int team = kSub ? tid / TPR : wave_index() / NW;
   const int t = tid - team * TPR;
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
+
+  LnColLoads<T> cols;
+  const int64_t col_slices = (n + 8 * VE - 1) / (8 * VE);
+  if constexpr (COLS)
+    ln_cols_issue<T, B::kThreads>(cols, x, dy, ldx, lddy, map, rows, n, stats, ld_stats, blockIdx.x, 0);
 
   float gam[V][VE];
 #pragma unroll
@@ -425,6 +529,21 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
     for (; it < full_iters; ++it) process(q, it, std::true_type{}, std::false_type{});
   }
   if (it < iters) process(q, it, std::false_type{}, std::false_type{});
+
+  if constexpr (COLS) {
+    constexpr int64_t kRowsPerPass = 4 * (B::kThreads / 8);
+    for (int64_t slice = blockIdx.x; slice < col_slices; slice += gridDim.x) {
+      float cg[VE], cb[VE];
+#pragma unroll
+      for (int e = 0; e < VE; ++e) cg[e] = cb[e] = 0.f;
+      for (int64_t row0 = 0; row0 < rows; row0 += kRowsPerPass) {
+        if (slice != blockIdx.x || row0 != 0)
+          ln_cols_issue<T, B::kThreads>(cols, x, dy, ldx, lddy, map, rows, n, stats, ld_stats, slice, row0);
+        ln_cols_accumulate<T, B::kThreads>(cols, rows, n, eps, slice, row0, cg, cb);
+      }
+      ln_cols_finish<T, B::kThreads>(col_lds, n, slice, cg, cb, dscale, dbias);
+    }
+  }
 
   if (WGRAD) {
     float* out = part + static_cast<int64_t>(blockIdx.x) * 2 * n;
@@ -668,6 +787,14 @@ static LnBwdPlan plan_ln_bwd(int64_t nvec, int64_t rows, int ve, int elem_bytes)
   return p;
 }
 
+// Problems whose weight gradients the backward kernel forms itself from column slices (a
+// second read of x and dy, served by the caches): few rows, and tensors that fit an L2.
+static bool ln_bwd_small(int64_t rows, int64_t n, int elem_bytes)
+{
+  static const bool off = std::getenv("LBN_LN_NO_FUSED_WGRAD") != nullptr;
+  return !off && rows <= 512 && rows * n * elem_bytes <= (int64_t(2) << 20);
+}
+
 // Row slabs of ln_wgrad_columns: about 2048 workgroups in total, at most one slab per row.
 static int64_t ln_wgrad_slabs(int64_t units, int64_t rows)
 {
@@ -721,21 +848,23 @@ static size_t ln_bwd_workspace(int64_t n, int64_t rows, int ve)
 {
   if (n <= 0 || rows <= 0) return 0;
   const int elem_bytes = 16 / ve;
-  size_t need = static_cast<size_t>(ln_wgrad_slabs(n, rows)) * 2 * n * sizeof(float);
+  // partial rows of the multi-kernel paths sit behind the header that the cluster kernels own
+  const size_t H = kWorkspaceHeaderBytes;
+  size_t need = H + static_cast<size_t>(ln_wgrad_slabs(n, rows)) * 2 * n * sizeof(float);
   auto cover = [&](size_t bytes) { if (bytes > need) need = bytes; };
   if (n % ve == 0) {
     const LnBwdPlan p = plan_ln_bwd(n / ve, rows, ve, elem_bytes);
-    if (p.tpr) cover(static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
-    else cover(static_cast<size_t>(ln_wgrad_slabs(n / ve, rows)) * 2 * n * sizeof(float));
+    if (p.tpr) cover(H + static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
+    else cover(H + static_cast<size_t>(ln_wgrad_slabs(n / ve, rows)) * 2 * n * sizeof(float));
     if (!p.tpr) cover(ln_cluster_bwd_workspace(n, rows, ve));  // long rows: slots, then one partial row per cluster
   }
   if (ve == 4 && n <= kLnMaxScalarRowBwd) {  // fp32 rows off the 16-byte grid: one float per access
     const LnBwdPlan p = plan_ln_bwd(n, rows, 1, 4);
-    if (p.tpr) cover(static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
+    if (p.tpr) cover(H + static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
   }
   if (ve == 8 && n % 2 == 0 && n / 2 <= kLnMaxScalarRowBwd) {  // fp16 rows: one pair per access
     const LnBwdPlan p = plan_ln_bwd(n / 2, rows, 2, 2);
-    if (p.tpr) cover(static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
+    if (p.tpr) cover(H + static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
   }
   return need;
 }
@@ -958,7 +1087,7 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
   const dim3 grid(static_cast<unsigned>(blocks)), block(B::kThreads);
   if (wgrad)
     hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, true>), grid, block, 0, st, x, dy, dx, ldx,
-                       lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part);
+                       lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part, nullptr, nullptr);
   else {
     // nothing to accumulate across rows: one resident wave of blocks, each walking the
     // same number of rows with the next row in flight
@@ -967,7 +1096,7 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
     if (resident < 1) resident = 1;
     const dim3 all(static_cast<unsigned>(ceil_div(units, ceil_div(units, resident))));
     hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, false>), all, block, 0, st, x, dy, dx, ldx,
-                       lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part);
+                       lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part, nullptr, nullptr);
   }
 }
 
@@ -984,11 +1113,28 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
   constexpr int VE = Vec16<ST>::N;
   const LnBwdPlan p = plan_ln_bwd(units, rows, VE, elem_bytes);
   if (!p.tpr) return 0;
+  if constexpr (VE >= 4) {
+    if (wgrad && ln_bwd_small(rows, n, elem_bytes)) {
+      // tensors that fit the caches: weight gradients from column slices, in the same kernel
+      const int nvec_s = static_cast<int>(units);
+#define X(TPR, TEAMS, V)                                                                              \
+  if (p.tpr == TPR && p.teams == TEAMS && p.v == V) {                                                 \
+    using B = RowBlock<TPR, TEAMS>;                                                                   \
+    hipLaunchKernelGGL((ln_bwd_rows<ST, TPR, TEAMS, V, false, true>), dim3(static_cast<unsigned>(p.blocks)), \
+                       dim3(B::kThreads), 0, st, x, dy, dx, ldx, lddy, lddx, map, rows, nvec_s,       \
+                       static_cast<int>(n), eps, stats, lds, sgrad, ldsg, gamma, nullptr, dgamma, dbeta); \
+    return 1;                                                                                         \
+  }
+      X(64, 4, 1) X(64, 4, 2) X(64, 4, 4) X(256, 2, 1) X(256, 2, 2) X(256, 1, 1) X(256, 1, 2)
+      if constexpr (VE == 4) { X(256, 2, 4) X(256, 1, 4) }
+#undef X
+    }
+  }
   float* part = nullptr;
   if (wgrad) {
-    const size_t need = static_cast<size_t>(p.blocks) * 2 * n * sizeof(float);
+    const size_t need = kWorkspaceHeaderBytes + static_cast<size_t>(p.blocks) * 2 * n * sizeof(float);
     if (!ws || ws_bytes < need || !aligned16(ws)) return -1;
-    part = static_cast<float*>(ws);
+    part = static_cast<float*>(workspace_payload(ws));
   }
   const int nvec = static_cast<int>(units);
   bool launched = false;
@@ -1097,8 +1243,8 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     // weight gradients of the two paths above: row slabs -> partial rows -> fixed-order sum
     const int64_t units = vec ? n / VE : n;
     const int64_t slabs = ln_wgrad_slabs(units, rows);
-    if (ws && aligned16(ws) && ws_bytes >= static_cast<size_t>(slabs) * 2 * n * sizeof(float)) {
-      float* wpart = static_cast<float*>(ws);
+    if (ws && aligned16(ws) && ws_bytes >= kWorkspaceHeaderBytes + static_cast<size_t>(slabs) * 2 * n * sizeof(float)) {
+      float* wpart = static_cast<float*>(workspace_payload(ws));
       const dim3 grid(static_cast<unsigned>(ceil_div(units, 256)), static_cast<unsigned>(slabs));
       if (vec)
         hipLaunchKernelGGL((ln_wgrad_columns<T, true>), grid, dim3(256), 0, st, x, dy, ldx, lddy, map, rows,
@@ -1213,17 +1359,21 @@ int lbn_instance_norm_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t cha
                        LBN_STATS_TWO_PASS);
 }
 
-// The statistics gradients (2 * channels x width floats) come first; channels too long for
-// one workgroup add the cluster kernels' slots behind them, on a 256-byte boundary.
-static size_t in_sgrad_bytes(int64_t channels, int64_t width)
+// The scratch of the layer-norm kernels comes first (at least the 64-byte header, so that
+// lbn_workspace_timed_out() finds the error word where it does for every other layer), the
+// statistics gradients (2 * channels x width floats) behind it on a 256-byte boundary.
+static size_t in_scratch_bytes(int64_t channels, int64_t channel_size, int64_t width)
 {
-  return (static_cast<size_t>(2 * channels) * static_cast<size_t>(width) * sizeof(float) + 255) & ~size_t(255);
+  size_t b = lbn_layer_norm_bwd_workspace_bytes(channels, channel_size, width, 0, 4);
+  if (b < kWorkspaceHeaderBytes) b = kWorkspaceHeaderBytes;
+  return (b + 255) & ~size_t(255);
 }
 
 size_t lbn_instance_norm_bwd_workspace_bytes(int64_t channels, int64_t channel_size, int64_t width)
 {
   if (channels <= 0 || channel_size <= 0 || width <= 0) return 0;
-  return in_sgrad_bytes(channels, width) + lbn_layer_norm_bwd_workspace_bytes(channels, channel_size, width, 0, 4);
+  return in_scratch_bytes(channels, channel_size, width) +
+         static_cast<size_t>(2 * channels) * static_cast<size_t>(width) * sizeof(float);
 }
 
 int lbn_instance_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
@@ -1232,18 +1382,15 @@ int lbn_instance_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t cha
                               const float* stats, int64_t ld_stats, void* workspace,
                               size_t workspace_bytes)
 {
-  if (channels > 0 && channel_size > 0 && width > 0 &&
-      (!workspace || workspace_bytes < static_cast<size_t>(2 * channels) * static_cast<size_t>(width) * sizeof(float)))
+  if (channels < 0 || channel_size < 0 || width < 0) return LBN_ERR_INVALID_ARGUMENT;
+  if (channels == 0 || channel_size == 0 || width == 0) return LBN_OK;
+  if (!workspace || workspace_bytes < lbn_instance_norm_bwd_workspace_bytes(channels, channel_size, width))
     return LBN_ERR_WORKSPACE;
-  void* slots = nullptr;
-  size_t slot_bytes = 0;
-  if (channels > 0 && width > 0 && workspace_bytes > in_sgrad_bytes(channels, width)) {
-    slots = static_cast<char*>(workspace) + in_sgrad_bytes(channels, width);
-    slot_bytes = workspace_bytes - in_sgrad_bytes(channels, width);
-  }
+  const size_t scratch = in_scratch_bytes(channels, channel_size, width);
+  float* sgrad = reinterpret_cast<float*>(static_cast<char*>(workspace) + scratch);
   return ln_bwd<float>(as_stream(stream), channels, channel_size, channel_size, width, epsilon, x,
-                       ldx, dy, lddy, dx, lddx, stats, ld_stats, static_cast<float*>(workspace),
-                       2 * channels, nullptr, nullptr, nullptr, slots, slot_bytes);
+                       ldx, dy, lddy, dx, lddx, stats, ld_stats, sgrad, 2 * channels, nullptr, nullptr, nullptr,
+                       workspace, scratch);
 }
 
 }  // extern "C"

@@ -815,7 +815,7 @@ static RowConfig pick_sm_row_config(int64_t units, int64_t rows)
 static size_t sm_workspace_bytes(int64_t n, int64_t rows)
 {
   if (n <= 0 || rows <= 0) return 0;
-  const size_t chunked = static_cast<size_t>(rows) * plan_chunks(n, rows).S * sizeof(float2);
+  const size_t chunked = kWorkspaceHeaderBytes + static_cast<size_t>(rows) * plan_chunks(n, rows).S * sizeof(float2);
   const size_t cluster = (n > kMaxScalarLongRow) ? cluster_workspace_bytes(rows) : 0;
   return chunked > cluster ? chunked : cluster;
 }
@@ -826,10 +826,14 @@ static size_t sm_workspace_bytes(int64_t n, int64_t rows)
 // HBM traffic, so the cluster path is used only for larger footprints.
 constexpr int64_t kClusterMinBytes = int64_t(48) << 20;
 
-// Inputs are loaded with the streaming (non-temporal) hint once the bytes a call moves
-// exceed what the 256 MB Infinity Cache could keep for a later reader; smaller working
-// sets are left to the cache, where the next kernel usually finds them.
-constexpr int64_t kStreamLoadMinBytes = int64_t(384) << 20;
+// Inputs are loaded with the streaming (non-temporal) hint once a call moves more than a
+// fraction of the 256 MB Infinity Cache: the hint does not slow a read that hits the cache
+// (an input its producer has just written), and it keeps a tensor that is read exactly once
+// from pushing out lines that someone will read again.  Measured on 32768 x 512 (128 / 192 MiB
+// moved per call): with every step's tensors cold 58.1 against 62.4 us per step; a benchmark
+// loop that re-reads the same buffers every step loses the reuse it was getting for free (56.0
+// against 53.7 us).  Smaller working sets are left to the caches.
+constexpr int64_t kStreamLoadMinBytes = int64_t(96) << 20;
 
 static int stream_loads(int64_t rows, int64_t n, int tensors)
 {
@@ -838,11 +842,30 @@ static int stream_loads(int64_t rows, int64_t n, int tensors)
   return rows * n * 4 * tensors >= kStreamLoadMinBytes ? 1 : 0;
 }
 
-static bool cluster_enabled(int64_t rows, int64_t n)
+// A few very long rows whose tensors fit the caches (262144 x 16): one cluster kernel
+// (20.6 us per step) against two split kernels per direction (22.7 us), except while a graph
+// is recorded, where the cluster kernel needs a second node (24.1 us).
+constexpr int64_t kFewRows = 64;
+
+static bool cluster_enabled(hipStream_t st, int64_t rows, int64_t n)
 {
   static const bool disabled = std::getenv("LBN_NO_CLUSTER") != nullptr;
   static const bool forced = std::getenv("LBN_FORCE_CLUSTER") != nullptr;
-  return !disabled && (forced || rows * n * 4 >= kClusterMinBytes);
+  if (disabled) return false;
+  if (forced || rows * n * 4 >= kClusterMinBytes) return true;
+  return rows <= kFewRows && !stream_is_capturing(st);
+}
+
+// Clusters of a launch that could hold `fit` of them at once.  Every cluster walks the same
+// number of rows.  When all rows would fit at once (a few very long rows), a cluster still
+// takes two rows as long as every compute unit keeps a workgroup: the second row's loads are
+// in flight while the first row's partials cross the cluster, and the first row is written
+// while the second one's do (262144 x 16: 13.1 against 14.7 us backward).
+static int64_t cluster_count(int64_t rows, int64_t fit, int M)
+{
+  int64_t per = ceil_div(rows, fit);
+  if (per == 1 && rows >= 2 && ceil_div(rows, 2) * M >= 256) per = 2;
+  return ceil_div(rows, per);
 }
 
 // Launch of the cluster kernels for rows of `units` accesses of W floats each.  Returns -1 when
@@ -860,7 +883,7 @@ static int sm_fwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, 
     const int cap = cluster_capacity(sm_fwd_cluster<VV, KIND, W>, kClusterThreads);              \
     int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
     if (ncl < 1) return -1;                                                                      \
-    ncl = ceil_div(rows, ceil_div(rows, ncl)); /* every cluster walks the same number of rows */ \
+    ncl = cluster_count(rows, ncl, cp.M);                                                        \
     const SmClusterArgs a{x, nullptr, y, ldx, 0, ldy, map, rows, static_cast<unsigned>(units),   \
                           cp.M, cw, cluster_call_tag(st, cw)};                                   \
     hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND, W>), dim3(static_cast<unsigned>(ncl * cp.M)),   \
@@ -885,7 +908,7 @@ static int sm_bwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, 
     const int cap = cluster_capacity(sm_bwd_cluster<VV, KIND, W>, kClusterThreads);              \
     int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
     if (ncl < 1) return -1;                                                                      \
-    ncl = ceil_div(rows, ceil_div(rows, ncl));                                                   \
+    ncl = cluster_count(rows, ncl, cp.M);                                                        \
     const SmClusterArgs a{y, dy, dx, ldy, lddy, lddx, map, rows, static_cast<unsigned>(units),   \
                           cp.M, cw, cluster_call_tag(st, cw)};                                   \
     hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND, W>), dim3(static_cast<unsigned>(ncl * cp.M)),   \
@@ -965,7 +988,7 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
                          map, rows, nvec);
     return launch_status();
   }
-  if (cluster_enabled(rows, n)) {
+  if (cluster_enabled(st, rows, n)) {
     int r = -1;
     if (vec && n / 4 < (int64_t(1) << 30)) {
       // four vectors per thread keep five workgroups per CU resident; eight only for rows that need it
@@ -981,8 +1004,8 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   }
   const ChunkPlan p = plan_chunks(n, rows);
   if (rows * p.S > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
-  if (!ws || ws_bytes < static_cast<size_t>(rows) * p.S * sizeof(float2)) return LBN_ERR_WORKSPACE;
-  float2* part = static_cast<float2*>(ws);
+  if (!ws || ws_bytes < kWorkspaceHeaderBytes + static_cast<size_t>(rows) * p.S * sizeof(float2)) return LBN_ERR_WORKSPACE;
+  float2* part = static_cast<float2*>(workspace_payload(ws));
   const dim3 grid(static_cast<unsigned>(rows * p.S)), block(kChunkThreads);
   if (vec) {
     hipLaunchKernelGGL((sm_fwd_partial<true>), grid, block, 0, st, x, ldx, map, n, p.chunk, p.S, part);
@@ -1060,7 +1083,7 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
                          lddy, lddx, map, rows, nvec);
     return launch_status();
   }
-  if (cluster_enabled(rows, n)) {
+  if (cluster_enabled(st, rows, n)) {
     int r = -1;
     if (vec && n / 4 < (int64_t(1) << 30))
       r = sm_bwd_cluster_launch<KIND, 4>(st, plan_cluster(n / 4, 4), n / 4, rows, y, ldy, dy, lddy, dx, lddx, map, ws,
@@ -1072,8 +1095,8 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   }
   const ChunkPlan p = plan_chunks(n, rows);
   if (rows * p.S > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
-  if (!ws || ws_bytes < static_cast<size_t>(rows) * p.S * sizeof(float2)) return LBN_ERR_WORKSPACE;
-  float* part = static_cast<float*>(ws);
+  if (!ws || ws_bytes < kWorkspaceHeaderBytes + static_cast<size_t>(rows) * p.S * sizeof(float2)) return LBN_ERR_WORKSPACE;
+  float* part = static_cast<float*>(workspace_payload(ws));
   const dim3 grid(static_cast<unsigned>(rows * p.S)), block(kChunkThreads);
   if (vec) {
     hipLaunchKernelGGL((sm_bwd_partial<true, KIND>), grid, block, 0, st, y, dy, ldy, lddy, map, n, p.chunk, p.S, part);

@@ -75,7 +75,9 @@ class DeviceMatrix:
         return m
 
     def to_numpy(self):
-        """Returns an (height, width) array."""
+        """Returns an (height, width) array.  Results are consumed here: a wait between
+        workgroups that ran out in any call since the last check raises ClusterWaitTimedOut."""
+        check_cluster_waits()
         t = self.tensor[: self.width, : self.height]
         if t.dtype == torch.float16:
             t = t.float()
@@ -96,6 +98,7 @@ class _Vector:
         return capi.vp(self.tensor.data_ptr())
 
     def to_numpy(self):
+        check_cluster_waits()
         return self.tensor[: self.n].cpu().numpy()
 
 
@@ -107,18 +110,59 @@ def _null():
     return capi.vp(None)
 
 
-class _Workspace:
-    """Scratch memory owned by a layer, grown on demand (never shrunk)."""
+class ClusterWaitTimedOut(LbnError):
+    """A kernel in which workgroups wait for each other gave up on a wait (the sticky error
+    word of a workspace is raised): the results of that call are undefined."""
 
-    def __init__(self):
+    def __init__(self, where):
+        RuntimeError.__init__(self, f"a bounded wait between workgroups ran out ({where}); "
+                                    "results of that call are undefined")
+        self.status = None
+
+
+# Workspaces handed to a compute call since the last check: their error words are read where
+# results are consumed (DeviceMatrix.to_numpy, which waits for the device anyway), so that a
+# wait that ran out surfaces as an exception instead of as silently wrong numbers.  With
+# LBN_CHECK_CLUSTER_WAITS=1 in the environment every fp_compute()/bp_compute() checks its own
+# workspace right after the call (this synchronises: a debugging mode).
+_PENDING = {}
+_CHECK_EVERY_CALL = bool(int(__import__("os").environ.get("LBN_CHECK_CLUSTER_WAITS", "0") or 0))
+
+
+def check_cluster_waits():
+    """Raises ClusterWaitTimedOut if any workspace used since the last check has its error
+    word raised; clears the word, so that the next use of the workspace starts clean."""
+    pending = list(_PENDING.values())
+    _PENDING.clear()
+    for ws in pending:
+        if ws.buf is None:
+            continue
+        flag = capi.cint(0)
+        call("lbn_workspace_timed_out", _stream(), capi.vp(ws.buf.data_ptr()), flag)
+        if flag.value:
+            ws.buf[:64].zero_()
+            raise ClusterWaitTimedOut(f"workspace of {ws.owner}")
+
+
+class _Workspace:
+    """Scratch memory owned by a layer, grown on demand (never shrunk).  The first 64 bytes
+    (the error word of the kernels that wait across workgroups) are cleared when the memory
+    is allocated: recycled device memory may hold anything."""
+
+    def __init__(self, owner="a layer", header=True):
         self.buf = None
+        self.owner = owner
+        self.header = header  # False: scratch of a layer none of whose kernels wait across workgroups
 
     def get(self, nbytes, device):
         nbytes = int(nbytes)
         if nbytes == 0:
             return _null(), 0
         if self.buf is None or self.buf.numel() < nbytes:
-            self.buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            self.buf = torch.empty(max(nbytes, 64), dtype=torch.uint8, device=device)
+            self.buf[:64].zero_()
+        if self.header:
+            _PENDING[id(self)] = self
         return capi.vp(self.buf.data_ptr()), nbytes
 
 
@@ -131,7 +175,7 @@ class _Layer:
         self.activations = None         # output y
         self.prev_error_signals = None  # dL/dy
         self.error_signals = None       # dL/dx
-        self._ws = _Workspace()
+        self._ws = _Workspace(type(self).__name__)
 
     # what fp_setup_inputs/outputs and bp_setup_gradient_wrt_inputs do
     def bind_forward(self, x, in_place=False):
@@ -153,10 +197,14 @@ class _Layer:
     def fp_compute(self):
         name, args = self.fp_call()
         call(name, *args)
+        if _CHECK_EVERY_CALL:
+            check_cluster_waits()
 
     def bp_compute(self):
         name, args = self.bp_call()
         call(name, *args)
+        if _CHECK_EVERY_CALL:
+            check_cluster_waits()
 
     def forward(self, x, in_place=False):
         self.bind_forward(x, in_place)
@@ -250,7 +298,7 @@ class instance_norm_layer(_Layer):
         self.num_channels = self.dims[0]
         self.channel_size = _prod(self.dims) // self.num_channels
         self.m_workspace = None  # (2*channels x width): means, then variances
-        self._ws_fwd = _Workspace()  # forward scratch of its own: backward's holds the statistics gradients
+        self._ws_fwd = _Workspace("instance_norm_layer (forward)")  # forward scratch of its own: backward's holds the statistics gradients
 
     def fp_call(self):
         x, y = self.prev_activations, self.activations
@@ -505,6 +553,7 @@ class entrywise_scale_bias_layer(_scale_bias_layer):
     def bp_call(self):
         x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
         wt, wg = self.weights, self.m_weights_gradient
+        self._ws.header = False
         ws, nb = self._ws.get(capi.lib().lbn_entrywise_scale_bias_bwd_workspace_bytes(x.height, x.width),
                               self.device)
         return ("lbn_entrywise_scale_bias_bwd_f32",
@@ -532,6 +581,7 @@ class channelwise_scale_bias_layer(_scale_bias_layer):
         x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
         wt, wg = self.weights, self.m_weights_gradient
         C, cs = self.num_channels, self.channel_size
+        self._ws.header = False
         ws, nb = self._ws.get(capi.lib().lbn_channelwise_scale_bias_bwd_workspace_bytes(C, cs, x.width), self.device)
         return ("lbn_channelwise_scale_bias_bwd_f32",
                 (_stream(), C, cs, x.width, x.Buffer(), x.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim,
@@ -556,7 +606,7 @@ class cross_entropy_layer:
         self.activations = None
         self.prev_error_signals = None
         self.error_signals = [None, None]
-        self._ws = _Workspace()
+        self._ws = _Workspace("cross_entropy_layer", header=False)
 
     def fp_call(self):
         x, t, y = self.prev_activations[0], self.prev_activations[1], self.activations
@@ -576,10 +626,14 @@ class cross_entropy_layer:
     def fp_compute(self):
         name, args = self.fp_call()
         call(name, *args)
+        if _CHECK_EVERY_CALL:
+            check_cluster_waits()
 
     def bp_compute(self):
         name, args = self.bp_call()
         call(name, *args)
+        if _CHECK_EVERY_CALL:
+            check_cluster_waits()
 
     def forward(self, prediction, ground_truth):
         self.prev_activations = [prediction, ground_truth]

@@ -2,6 +2,7 @@
 // part of data_type_layer::forward_prop / back_prop_impl_ -- attaches the framework's
 // matrices, calls fp_compute() / bp_compute() -- on device buffers handed in by the
 // Python tests.  Exceptions are turned into a non-zero return and a message.
+#include <cstdio>
 #include <cstring>
 #include <string>
 
@@ -336,6 +337,43 @@ int drv_gradient_buffer(const int64_t* dims, int nd, int64_t h, int64_t w, const
     }
     return 0;
   } catch (const std::exception& e) {
+    return fail(e, err, errlen);
+  }
+}
+
+// A softmax layer on a (h x w) problem that uses scratch: forward, then the wait check, which
+// must pass; then the designed give-up exit is run on the layer's own scratch buffer and
+// the next check must throw (returns 0 only if it did, with the message in err), after which
+// the word is clear again and a further forward + check pass.
+int drv_cluster_wait_check(int64_t h, int64_t w, float* x, float* y, float* out4, void* stream, char* err,
+                           int errlen)
+{
+  try {
+    device_matrix<float> mx, my;
+    attach(mx, h, w, x, h); attach(my, h, w, y, h);
+    softmax_layer<> layer;
+    layer.io.prev_activations = &mx; layer.io.activations = &my;
+    layer.io.stream = static_cast<hipStream_t>(stream);
+    layer.fp_compute();
+    layer.check_cluster_waits();
+    if (layer.scratch().bytes() < 128) throw exception("the test shape was expected to use scratch");
+    check_status(lbn_selftest_cluster_wait_gives_up(stream, layer.scratch().reserve(0), layer.scratch().bytes(), 32,
+                                                    out4), "selftest");
+    bool thrown = false;
+    try {
+      layer.check_cluster_waits();
+    }
+    catch (const exception& e) {
+      thrown = true;
+      std::snprintf(err, errlen, "%s", e.what());
+    }
+    if (!thrown) throw exception("check_cluster_waits() did not report the wait that gave up");
+    layer.fp_compute();
+    layer.check_cluster_waits();
+    check_hip(hipStreamSynchronize(layer.io.stream), "sync");
+    return 0;
+  }
+  catch (const std::exception& e) {
     return fail(e, err, errlen);
   }
 }

@@ -317,6 +317,27 @@ def test_entrywise_batch_norm(L, h, w, pad):
             check(f"entrywise_bn {k} h={h} w={w} training={training}", got[k], r32[k], r64[k])
 
 
+def test_entrywise_batch_norm_clamps_negative_variance(L):
+    """Where the reference's fp32 E[x^2] - mean^2 is negative (tests/test_oracle.py pins that
+    it keeps -2 and returns NaN), both GPU paths clamp the variance at zero: y is finite."""
+    from lbann_amd import capi
+    x = f32(np.array([[3198.374755859375, 3198.375], [1.0, 3.0], [0.5, -0.5], [2.0, 2.0]], dtype=np.float32))
+    layer = L.entrywise_batch_normalization_layer((4,), 0.9, 1e-5)
+    y = layer.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    stats = layer.m_batch_statistics.to_numpy()
+    assert np.isfinite(y).all() and stats[0, 1] >= 0.0
+    assert stats[1, 1] == np.float32(2.0)
+    # the split statistics step on the reference's own sums: same clamp
+    xd = L.DeviceMatrix.from_numpy(x)
+    st = L.DeviceMatrix(4, 2)
+    rm, rv = L._Vector(4, "cuda", np.zeros(4)), L._Vector(4, "cuda", np.ones(4))
+    s = capi.vp(torch.cuda.current_stream().cuda_stream)
+    L.call("lbn_entrywise_batch_norm_fwd_sums_f32", s, 4, 2, xd.Buffer(), xd.ldim, st.Buffer(), st.ldim)
+    L.call("lbn_entrywise_batch_norm_fwd_stats_f32", s, 4, 2, 0.9, st.Buffer(), st.ldim, rm.Buffer(), rv.Buffer())
+    split = st.to_numpy()
+    assert split[0, 1] == 0.0 and split[1, 1] == np.float32(2.0)
+
+
 @pytest.mark.parametrize("h,w,w0,pad", [(105, 29, 14, 0), (4096, 64, 32, 0), (1024, 300, 7, 0), (260, 7, 3, 4),
                                         (258, 9, 9, 0), (100000, 33, 16, 0), (8196, 257, 200, 4), (60, 513, 512, 0),
                                         (64, 1, 1, 0), (64, 2, 1, 0)])

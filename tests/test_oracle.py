@@ -477,6 +477,21 @@ def test_entrywise_batch_norm_matches_torch_autograd_and_inference():
     assert rel_err(dxi, dy / np.sqrt(rv[:, None] + 1e-4)) < 1e-13
 
 
+def test_entrywise_batch_norm_reference_variance_is_not_clamped():
+    """E[x^2] - mean^2 in fp32 can come out negative for a pair of nearly equal large values;
+    the reference keeps that value (entrywise_batch_normalization.cpp:118, no clamp), times the
+    Bessel factor, and its output for that entry is then NaN once var + epsilon < 0.  The GPU
+    kernels clamp the difference at zero instead (a documented deviation, checked by
+    tests/test_gpu_parity.py::test_entrywise_batch_norm_clamps_negative_variance)."""
+    x = np.asfortranarray(np.array([[3198.374755859375, 3198.375], [1.0, 3.0]], dtype=np.float32))
+    rm, rv = np.zeros(2, np.float32), np.ones(2, np.float32)
+    y, stats = orc.entrywise_batch_norm_fwd(x, 0.9, 1e-5, rm, rv)
+    assert stats[0, 1] == np.float32(-2.0)            # (-1) * w / (w - 1) with w = 2
+    assert np.isnan(y[0]).all()                       # 1 / sqrt(-2 + 1e-5)
+    assert stats[1, 1] == np.float32(2.0) and np.isfinite(y[1]).all()   # the ordinary row is untouched
+    assert rv[0] == np.float32(0.9) * np.float32(1.0) + (np.float32(1.0) - np.float32(0.9)) * np.float32(-2.0)
+
+
 def test_entrywise_batch_norm_bwd_finite_difference_and_single_sample():
     rng = np.random.default_rng(32)
     h, w = 4, 5
