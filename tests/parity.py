@@ -37,17 +37,41 @@ def rel_err(a, b):
     return float(np.max(np.abs(a - b) / denom))
 
 
+# Every check() of the process, in call order: what the parity report is written from
+# (tests/conftest.py writes it when the GPU tests end; tests/parity_report.py formats it).
+REPORT = []
+
+
 def check(name, got, ref32, exact64=None, tol=TOL_F32, slack=1.0):
-    """Returns the dict of measured errors; raises AssertionError when the gate fails."""
+    """Returns the dict of measured errors; raises AssertionError when the gate fails.
+
+    The dict names the leg that passed: "fp32 reference" (within `tol` of the restated
+    reference) or "float64" (at least as close to the float64 evaluation as the fp32
+    reference is).  With `exact64` given, all three distances are measured and recorded
+    whichever leg passes."""
     e_ref = rel_err(got, ref32)
-    out = {"name": name, "vs_ref": e_ref}
+    out = {"name": name, "tol": tol, "vs_ref": e_ref, "leg": "fp32 reference" if e_ref <= tol else None}
+    if exact64 is not None:
+        out["vs_exact"] = rel_err(got, exact64)
+        out["ref_vs_exact"] = rel_err(ref32, exact64)
+    REPORT.append(out)
     if e_ref <= tol:
         return out
     assert exact64 is not None, f"{name}: err vs fp32 reference {e_ref:.3e} > {tol:.1e}"
-    e_exact = rel_err(got, exact64)
-    e_ref_exact = rel_err(ref32, exact64)
-    out.update(vs_exact=e_exact, ref_vs_exact=e_ref_exact)
+    e_exact, e_ref_exact = out["vs_exact"], out["ref_vs_exact"]
     assert e_exact <= max(tol, slack * e_ref_exact), (
         f"{name}: err vs fp32 reference {e_ref:.3e} > {tol:.1e} and err vs float64 "
         f"{e_exact:.3e} > reference's own {e_ref_exact:.3e}")
+    out["leg"] = "float64"
+    return out
+
+
+def record(name, got, ref32, exact64=None, tol=TOL_F32):
+    """Measures and records like check() but never fails: for comparisons that are reported
+    for information (a different summation formula, say) and gated elsewhere."""
+    out = {"name": name, "tol": tol, "vs_ref": rel_err(got, ref32), "leg": "informational"}
+    if exact64 is not None:
+        out["vs_exact"] = rel_err(got, exact64)
+        out["ref_vs_exact"] = rel_err(ref32, exact64)
+    REPORT.append(out)
     return out
