@@ -923,9 +923,14 @@ static BnClusterShape bn_cluster_shape(int64_t E, int max_v, int first_t)
   return {0, 0, 0};
 }
 
-// 16-bit storage runs the barrier-free variant of the cluster kernels.
+// 16-bit storage runs the barrier-free variant of the cluster kernels, fp32 the one with
+// barriers; LBN_BN_WAVE_SYNC=0|1 in the environment forces one of them for every type.
 template <typename S>
-constexpr bool kBnWaveSync = sizeof(S) == 2;
+static bool bn_wave_sync()
+{
+  static const int forced = std::getenv("LBN_BN_WAVE_SYNC") ? std::atoi(std::getenv("LBN_BN_WAVE_SYNC")) : -1;
+  return forced >= 0 ? forced != 0 : sizeof(S) == 2;
+}
 
 // ==================================================================== host side
 // Workgroups per channel: about 4096 workgroups in total, each with at least four
@@ -964,12 +969,11 @@ static size_t bn_workspace(int64_t C, int64_t cs, int64_t w)
 template <typename S, int T, int V>
 static bool bn_launch_fwd_cluster(hipStream_t st, const BnFwdArgs<S>& a, int64_t C, unsigned seg, unsigned E)
 {
-  int cap;
-  if constexpr (kBnWaveSync<S>) cap = cluster_capacity(bn_fwd_cluster_ws<S, T, V>, T);
-  else cap = cluster_capacity(bn_fwd_cluster<S, T, V>, T);
+  const bool ws = bn_wave_sync<S>();
+  const int cap = ws ? cluster_capacity(bn_fwd_cluster_ws<S, T, V>, T) : cluster_capacity(bn_fwd_cluster<S, T, V>, T);
   const int64_t ncl = cap / a.M < C ? cap / a.M : C;
   if (ncl < 1) return false;
-  if constexpr (kBnWaveSync<S>)
+  if (ws)
     hipLaunchKernelGGL((bn_fwd_cluster_ws<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
   else
     hipLaunchKernelGGL((bn_fwd_cluster<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
@@ -979,12 +983,11 @@ static bool bn_launch_fwd_cluster(hipStream_t st, const BnFwdArgs<S>& a, int64_t
 template <typename S, int T, int V>
 static bool bn_launch_bwd_cluster(hipStream_t st, const BnBwdArgs<S>& a, int64_t C, unsigned seg, unsigned E)
 {
-  int cap;
-  if constexpr (kBnWaveSync<S>) cap = cluster_capacity(bn_bwd_cluster_ws<S, T, V>, T);
-  else cap = cluster_capacity(bn_bwd_cluster<S, T, V>, T);
+  const bool ws = bn_wave_sync<S>();
+  const int cap = ws ? cluster_capacity(bn_bwd_cluster_ws<S, T, V>, T) : cluster_capacity(bn_bwd_cluster<S, T, V>, T);
   const int64_t ncl = cap / a.M < C ? cap / a.M : C;
   if (ncl < 1) return false;
-  if constexpr (kBnWaveSync<S>)
+  if (ws)
     hipLaunchKernelGGL((bn_bwd_cluster_ws<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);
   else
     hipLaunchKernelGGL((bn_bwd_cluster<S, T, V>), dim3(static_cast<unsigned>(ncl * a.M)), dim3(T), 0, st, a, seg, E);

@@ -166,7 +166,7 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
 }
 
 // softmax / channelwise: dx = y * (dy - dot(y, dy));  log-softmax: dx = dy - exp(y) * sum(dy)
-template <int TPR, int V, int KIND, bool STREAM, int W = 4>
+template <int TPR, int V, int KIND, int STREAM, int W = 4>  // STREAM: bit 0 streams y, bit 1 dy
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
 sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
             RowMap map, int64_t rows, unsigned nvec)
@@ -191,8 +191,8 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      RowIO<W>::template load<STREAM>(yr + unsigned(W) * idx, a[i]);
-      RowIO<W>::template load<STREAM>(gr + unsigned(W) * idx, g[i]);
+      RowIO<W>::template load<(STREAM & 1) != 0>(yr + unsigned(W) * idx, a[i]);
+      RowIO<W>::template load<(STREAM & 2) != 0>(gr + unsigned(W) * idx, g[i]);
     }
     else {
 #pragma unroll
@@ -275,6 +275,11 @@ __device__ __forceinline__ void sm_cl_load(float (&t)[V][W], const float* rowp, 
   }
 }
 
+// The entries are exponentiated here, in front of the publication, and only rescaled after the
+// exchange.  Summing a two-operation exponential here and exponentiating against the row's
+// maximum afterwards (less work before the partials can leave) was measured: no gain on
+// 262144 x 16 or 262144 x 256, and rows read one float at a time lose a third (50257 x 1024
+// forward 137 against 87 us).
 // (1) of a step: thread-local online softmax, one merge of the (max, sum) pairs of the
 // workgroup, published for the cluster.
 template <int V, int KIND, int W = 4>
@@ -826,14 +831,19 @@ static size_t sm_workspace_bytes(int64_t n, int64_t rows)
 // HBM traffic, so the cluster path is used only for larger footprints.
 constexpr int64_t kClusterMinBytes = int64_t(48) << 20;
 
-// Inputs are loaded with the streaming (non-temporal) hint once a call moves more than a
-// fraction of the 256 MB Infinity Cache: the hint does not slow a read that hits the cache
-// (an input its producer has just written), and it keeps a tensor that is read exactly once
-// from pushing out lines that someone will read again.  Measured on 32768 x 512 (128 / 192 MiB
-// moved per call): with every step's tensors cold 58.1 against 62.4 us per step; a benchmark
-// loop that re-reads the same buffers every step loses the reuse it was getting for free (56.0
-// against 53.7 us).  Smaller working sets are left to the caches.
-constexpr int64_t kStreamLoadMinBytes = int64_t(96) << 20;
+// Streaming (non-temporal) loads keep a tensor that is read exactly once from pushing out
+// lines that someone will read again.  Whether that pays depends on where the tensor is:
+// measured on 32768 x 512 (64 MiB per tensor), us per step with the same buffers every step
+// ("resident") / with every step's tensors rotated out of the caches ("cold"):
+//   nothing streamed 52.8 / 62.7    backward streams y 52.3 / 60.9    y and dy 55.3 / 56.4
+//   forward streams x 55.2 / 61.6   x and y 55.9 / 56.7               all three 54.5 / 58.4
+// In a training step the forward input and the upstream gradient have just been written by
+// the neighbouring layers and sit in the 256 MB Infinity Cache, while y was written a whole
+// forward and backward sweep ago: y is streamed once a call moves more than a third of
+// that cache, which costs nothing when the others are resident and helps when they are not.
+// Calls that move more than the cache holds stream everything.
+constexpr int64_t kStreamLoadMinBytes = int64_t(384) << 20;
+constexpr int64_t kStreamOldInputMinBytes = int64_t(96) << 20;
 
 static int stream_loads(int64_t rows, int64_t n, int tensors)
 {
@@ -846,6 +856,15 @@ static int stream_loads(int64_t rows, int64_t n, int tensors)
 // (20.6 us per step) against two split kernels per direction (22.7 us), except while a graph
 // is recorded, where the cluster kernel needs a second node (24.1 us).
 constexpr int64_t kFewRows = 64;
+
+// Backward: bit 0 streams y, bit 1 streams dy (LBN_STREAM_LOADS_BWD overrides, for experiments).
+static int stream_loads_bwd(int64_t rows, int64_t n)
+{
+  static const int forced = std::getenv("LBN_STREAM_LOADS_BWD") ? std::atoi(std::getenv("LBN_STREAM_LOADS_BWD")) : -1;
+  if (forced >= 0) return forced & 3;
+  if (stream_loads(rows, n, 3)) return 3;
+  return rows * n * 4 * 3 >= kStreamOldInputMinBytes ? 1 : 0;
+}
 
 static bool cluster_enabled(hipStream_t st, int64_t rows, int64_t n)
 {
@@ -860,7 +879,10 @@ static bool cluster_enabled(hipStream_t st, int64_t rows, int64_t n)
 // number of rows.  When all rows would fit at once (a few very long rows), a cluster still
 // takes two rows as long as every compute unit keeps a workgroup: the second row's loads are
 // in flight while the first row's partials cross the cluster, and the first row is written
-// while the second one's do (262144 x 16: 13.1 against 14.7 us backward).
+// while the second one's do (262144 x 16: 13.1 against 14.7 us backward).  Four rows per
+// cluster, all loaded up front by one workgroup per compute unit, were measured and are
+// slower (forward 14.1 against 10.0 us per launch, backward the same 10.6): one wave per
+// SIMD cannot overlap the exponentials of one row with the loads of the next.
 static int64_t cluster_count(int64_t rows, int64_t fit, int M)
 {
   int64_t per = ceil_div(rows, fit);
@@ -1044,11 +1066,18 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
     const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
-    if (stream_loads(rows, n, 3))                                                            \
-      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, true>), dim3(grid), dim3(B::kThreads), 0, st, \
+    const int hint = stream_loads_bwd(rows, n);                                              \
+    if (hint == 3)                                                                           \
+      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, 3>), dim3(grid), dim3(B::kThreads), 0, st, \
+                         y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
+    else if (hint == 1)                                                                      \
+      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
+                         y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
+    else if (hint == 2)                                                                      \
+      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, 2>), dim3(grid), dim3(B::kThreads), 0, st, \
                          y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
     else                                                                                     \
-      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, false>), dim3(grid), dim3(B::kThreads), 0, st, \
+      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, 0>), dim3(grid), dim3(B::kThreads), 0, st, \
                          y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
     return launch_status();                                                                  \
   }
@@ -1064,7 +1093,7 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
     const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
-    hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, false, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
+    hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, 0, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
                        y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                         \
     return launch_status();                                                                  \
   }
@@ -1076,10 +1105,10 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     const unsigned nvec = static_cast<unsigned>(n);
     const unsigned grid = static_cast<unsigned>(rows);
     if (n <= 16 * 1024)
-      hipLaunchKernelGGL((sm_bwd_rows<1024, 16, KIND, false, 1>), dim3(grid), dim3(1024), 0, st, y, dy, dx, ldy,
+      hipLaunchKernelGGL((sm_bwd_rows<1024, 16, KIND, 0, 1>), dim3(grid), dim3(1024), 0, st, y, dy, dx, ldy,
                          lddy, lddx, map, rows, nvec);
     else
-      hipLaunchKernelGGL((sm_bwd_rows<1024, 32, KIND, false, 1>), dim3(grid), dim3(1024), 0, st, y, dy, dx, ldy,
+      hipLaunchKernelGGL((sm_bwd_rows<1024, 32, KIND, 0, 1>), dim3(grid), dim3(1024), 0, st, y, dy, dx, ldy,
                          lddy, lddx, map, rows, nvec);
     return launch_status();
   }

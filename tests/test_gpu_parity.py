@@ -81,6 +81,30 @@ def test_softmax_family(L, kind, h, w, pad):
 
 
 @pytest.mark.parametrize("kind", ["softmax", "log_softmax", "channelwise"])
+@pytest.mark.parametrize("h,w,in_place", [(262144, 17, False), (65536, 40, False), (262144, 16, True), (131072, 31, True)])
+def test_few_long_rows_all_in_flight(L, kind, h, w, in_place):
+    """A handful of rows far longer than a workgroup holds, all resident at once: the cluster
+    kernels with two rows per cluster (odd row counts leave the last cluster with one)."""
+    rng = np.random.default_rng(h + 7 * w)
+    x, dy = rand(rng, h, w, 0, 2), rand(rng, h, w)
+    if kind == "channelwise":
+        layer = L.channelwise_softmax_layer((2, h // 2))       # two windows per sample: 2 w rows of h / 2
+        fwd = lambda a: orc.channelwise_softmax_fwd(a, 2, h // 2, h // 2)
+        bwd = lambda y, g: orc.channelwise_softmax_bwd(y, g, 2, h // 2, h // 2)
+    else:
+        layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
+        fwd, bwd = _sm_oracle(kind)
+    xm = L.DeviceMatrix.from_numpy(x)
+    y = layer.forward(xm, in_place=in_place).to_numpy()
+    check(f"{kind} few long rows y {h}x{w}", y, fwd(x), fwd(f64(x)))
+    gm = L.DeviceMatrix.from_numpy(dy)
+    dx = layer.backward(gm, in_place=in_place).to_numpy()
+    check(f"{kind} few long rows dx {h}x{w}", dx, bwd(f32(y), dy), bwd(f64(y), f64(dy)))
+    if kind != "log_softmax":
+        assert np.abs(y.astype(np.float64).reshape(-1, (2 if kind == "channelwise" else 1) * w, order="F").sum(axis=0) - 1).max() < 1e-5
+
+
+@pytest.mark.parametrize("kind", ["softmax", "log_softmax", "channelwise"])
 @pytest.mark.parametrize("h,w", [(4096, 6), (777, 5), (70000, 2)])
 def test_softmax_family_in_place(L, kind, h, w):
     rng = np.random.default_rng(h + w)
