@@ -64,8 +64,11 @@ def main():
                                          ldim=a.shape[0] + ld_pad if ld_pad else None)
 
     # ---- workload table: name -> builder returning (fwd, bwd, elements, elem_size, samples, cpu_fn)
-    def build_softmax(kind, data):
-        x, dy = upload(data["x"]), upload(data["dy"])
+    def build_softmax(kind, data, half=False):
+        if half:  # fp16 storage: both sides see the rounded values
+            data = dict(data, x=np.asfortranarray(data["x"].astype(np.float16).astype(np.float32)),
+                        dy=np.asfortranarray(data["dy"].astype(np.float16).astype(np.float32)))
+        x, dy = upload(data["x"], half), upload(data["dy"], half)
         layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
         layer.bind_forward(x)
         layer.bind_backward(dy)
@@ -77,7 +80,7 @@ def main():
             t0 = time.perf_counter(); y = f(data["x"]); t1 = time.perf_counter()
             b(y, data["dy"]); t2 = time.perf_counter()
             return t1 - t0, t2 - t1
-        return layer, data["x"].size, 4, data["x"].shape[1], cpu
+        return layer, data["x"].size, 2 if half else 4, data["x"].shape[1], cpu
 
     def build_cws(data):
         x, dy = upload(data["x"]), upload(data["dy"])
@@ -276,6 +279,8 @@ def main():
         # not baseline configurations: fp16 storage for batch norm, and softmax rows off the 16-byte grid
         "extra_batch_norm_f16": ("BatchNorm train fwd+bwd fp16 storage NCHW 64x256x56x56 (informational)",
                                  lambda: build_bn(W.cfg3_batch_norm(), True)),
+        "extra_softmax_f16": ("Softmax fwd+bwd fp16 storage 32768x512 (informational)",
+                              lambda: build_softmax("softmax", W.cfg2_softmax(), True)),
         "extra_softmax_vocab_50257": ("Softmax fwd+bwd fp32 50257x1024, rows 4-byte aligned (informational)",
                                       lambda: build_softmax("softmax", W.cfg5b_wide_softmax(h=50257, w=1024))),
         # not a baseline configuration: where weight gradients go next (a 4096 x 4096 weight matrix)

@@ -364,6 +364,27 @@ int lbn_log_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
                             const float* y, int64_t ldy, const float* dy, int64_t lddy,
                             float* dx, int64_t lddx, void* workspace, size_t workspace_bytes);
 
+/* fp16 storage for the two layers above: the reference instantiates softmax_layer and
+ * log_softmax_layer for half precision too (src/layers/activations/softmax.cpp:236-243,
+ * log_softmax.cpp:160-167, LBANN_INSTANTIATE_CPU_HALF / GPU_HALF).  x, y, dy, dx are IEEE
+ * binary16 in memory; all arithmetic (maximum, exponentials, sums) is fp32, where the
+ * reference's half instantiation also accumulates in half; results are rounded to nearest
+ * even on store, and softmax's flush of non-normal results applies to the fp32 value before
+ * rounding (binary16 denormals are kept).  Same arguments as the _f32 entry points (leading
+ * dimensions in elements); the workspace is not used and may be NULL.  In place allowed. */
+int lbn_softmax_fwd_f16(lbn_stream_t stream, int64_t height, int64_t width,
+                        const void* x, int64_t ldx, void* y, int64_t ldy,
+                        void* workspace, size_t workspace_bytes);
+int lbn_softmax_bwd_f16(lbn_stream_t stream, int64_t height, int64_t width,
+                        const void* y, int64_t ldy, const void* dy, int64_t lddy,
+                        void* dx, int64_t lddx, void* workspace, size_t workspace_bytes);
+int lbn_log_softmax_fwd_f16(lbn_stream_t stream, int64_t height, int64_t width,
+                            const void* x, int64_t ldx, void* y, int64_t ldy,
+                            void* workspace, size_t workspace_bytes);
+int lbn_log_softmax_bwd_f16(lbn_stream_t stream, int64_t height, int64_t width,
+                            const void* y, int64_t ldy, const void* dy, int64_t lddy,
+                            void* dx, int64_t lddx, void* workspace, size_t workspace_bytes);
+
 /* --------------------------------------------------------- channelwise softmax
  * Replaces channelwise_softmax_layer::fp_compute / bp_compute
  * (src/layers/misc/channelwise_softmax.cpp:41-113, :121-184).  Each sample holds

@@ -29,6 +29,7 @@
 #include <stdexcept>
 #include <string>
 #include <type_traits>
+#include <utility>
 #include <vector>
 
 #include "../../include/lbnorm.h"
@@ -204,6 +205,10 @@ inline int64_t product(const std::vector<int64_t>& d, size_t from, size_t to)
   return p;
 }
 template <typename T> struct is_half : std::false_type {};
+/// Element type of a matrix class (what Buffer() points to): 2-byte elements select the
+/// fp16-storage entry points.
+template <typename Mat>
+using element_t = std::remove_cv_t<std::remove_pointer_t<decltype(std::declval<Mat&>().Buffer())>>;
 }  // namespace detail
 
 // ------------------------------------------------------------------ layer norm
@@ -460,8 +465,9 @@ public:
     const Mat& x = *io.prev_activations;
     Mat& y = *io.activations;
     const size_t bytes = lbn_softmax_workspace_bytes(x.Height(), x.Width());
-    check_status(lbn_softmax_fwd_f32(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(), y.Buffer(),
-                                     y.LDim(), m_ws.reserve(bytes, io.stream), bytes),
+    const auto fwd = sizeof(detail::element_t<Mat>) == 2 ? &lbn_softmax_fwd_f16 : &call_f32_fwd;
+    check_status(fwd(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(),
+                     m_ws.reserve(bytes, io.stream), bytes),
                  "softmax_layer::fp_compute");
     m_ws.after_call(io.stream, "softmax_layer::fp_compute");
   }
@@ -471,9 +477,9 @@ public:
     const Mat& dy = *io.prev_error_signals;
     Mat& dx = *io.error_signals;
     const size_t bytes = lbn_softmax_workspace_bytes(y.Height(), y.Width());
-    check_status(lbn_softmax_bwd_f32(io.stream, y.Height(), y.Width(), y.LockedBuffer(), y.LDim(),
-                                     dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
-                                     m_ws.reserve(bytes, io.stream), bytes),
+    const auto bwd = sizeof(detail::element_t<Mat>) == 2 ? &lbn_softmax_bwd_f16 : &call_f32_bwd;
+    check_status(bwd(io.stream, y.Height(), y.Width(), y.LockedBuffer(), y.LDim(), dy.LockedBuffer(), dy.LDim(),
+                     dx.Buffer(), dx.LDim(), m_ws.reserve(bytes, io.stream), bytes),
                  "softmax_layer::bp_compute");
     m_ws.after_call(io.stream, "softmax_layer::bp_compute");
   }
@@ -487,6 +493,18 @@ public:
   }
 
 private:
+  // the fp32 entry points behind the pointer types of the fp16 ones
+  static int call_f32_fwd(lbn_stream_t st, int64_t h, int64_t w, const void* x, int64_t ldx, void* y, int64_t ldy,
+                          void* ws, size_t bytes)
+  {
+    return lbn_softmax_fwd_f32(st, h, w, static_cast<const float*>(x), ldx, static_cast<float*>(y), ldy, ws, bytes);
+  }
+  static int call_f32_bwd(lbn_stream_t st, int64_t h, int64_t w, const void* y, int64_t ldy, const void* dy,
+                          int64_t lddy, void* dx, int64_t lddx, void* ws, size_t bytes)
+  {
+    return lbn_softmax_bwd_f32(st, h, w, static_cast<const float*>(y), ldy, static_cast<const float*>(dy), lddy,
+                               static_cast<float*>(dx), lddx, ws, bytes);
+  }
   softmax_mode m_mode;
   workspace m_ws;
 };
@@ -501,8 +519,9 @@ public:
     const Mat& x = *io.prev_activations;
     Mat& y = *io.activations;
     const size_t bytes = lbn_softmax_workspace_bytes(x.Height(), x.Width());
-    check_status(lbn_log_softmax_fwd_f32(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(),
-                                         y.Buffer(), y.LDim(), m_ws.reserve(bytes, io.stream), bytes),
+    const auto fwd = sizeof(detail::element_t<Mat>) == 2 ? &lbn_log_softmax_fwd_f16 : &call_f32_fwd;
+    check_status(fwd(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(),
+                     m_ws.reserve(bytes, io.stream), bytes),
                  "log_softmax_layer::fp_compute");
     m_ws.after_call(io.stream, "log_softmax_layer::fp_compute");
   }
@@ -512,9 +531,9 @@ public:
     const Mat& dy = *io.prev_error_signals;
     Mat& dx = *io.error_signals;
     const size_t bytes = lbn_softmax_workspace_bytes(y.Height(), y.Width());
-    check_status(lbn_log_softmax_bwd_f32(io.stream, y.Height(), y.Width(), y.LockedBuffer(), y.LDim(),
-                                         dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
-                                         m_ws.reserve(bytes, io.stream), bytes),
+    const auto bwd = sizeof(detail::element_t<Mat>) == 2 ? &lbn_log_softmax_bwd_f16 : &call_f32_bwd;
+    check_status(bwd(io.stream, y.Height(), y.Width(), y.LockedBuffer(), y.LDim(), dy.LockedBuffer(), dy.LDim(),
+                     dx.Buffer(), dx.LDim(), m_ws.reserve(bytes, io.stream), bytes),
                  "log_softmax_layer::bp_compute");
     m_ws.after_call(io.stream, "log_softmax_layer::bp_compute");
   }
@@ -528,6 +547,17 @@ public:
   }
 
 private:
+  static int call_f32_fwd(lbn_stream_t st, int64_t h, int64_t w, const void* x, int64_t ldx, void* y, int64_t ldy,
+                          void* ws, size_t bytes)
+  {
+    return lbn_log_softmax_fwd_f32(st, h, w, static_cast<const float*>(x), ldx, static_cast<float*>(y), ldy, ws, bytes);
+  }
+  static int call_f32_bwd(lbn_stream_t st, int64_t h, int64_t w, const void* y, int64_t ldy, const void* dy,
+                          int64_t lddy, void* dx, int64_t lddx, void* ws, size_t bytes)
+  {
+    return lbn_log_softmax_bwd_f32(st, h, w, static_cast<const float*>(y), ldy, static_cast<const float*>(dy), lddy,
+                                   static_cast<float*>(dx), lddx, ws, bytes);
+  }
   workspace m_ws;
 };
 

@@ -65,6 +65,10 @@ PROTOTYPES = {
     "lbn_softmax_fwd_static_scratch_f32": (cint, [vp, i64, i64, vp, i64, vp, i64]),
     "lbn_log_softmax_fwd_f32": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_log_softmax_bwd_f32": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
+    "lbn_softmax_fwd_f16": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, sz]),
+    "lbn_softmax_bwd_f16": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
+    "lbn_log_softmax_fwd_f16": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, sz]),
+    "lbn_log_softmax_bwd_f16": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_channelwise_softmax_workspace_bytes": (sz, [i64, i64, i64]),
     "lbn_channelwise_softmax_fwd_f32": (cint, [vp, i64, i64, i64, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_channelwise_softmax_bwd_f32": (cint, [vp, i64, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, sz]),

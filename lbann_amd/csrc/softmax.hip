@@ -28,6 +28,7 @@
 #include "host_utils.hpp"
 
 #include <mutex>
+#include <type_traits>
 
 namespace lbn {
 
@@ -40,10 +41,10 @@ constexpr int kMaxChunks = 64;  // S <= one wave, so a wave merges the partials 
 // boundaries and their length is a multiple of 4), W = 1 a single float for rows that are
 // only 4-byte aligned (odd lengths such as 197 or 1001): a wave instruction then still
 // reads 256 contiguous bytes.
-template <int W>
+template <typename S, int W>
 struct RowIO;
 template <>
-struct RowIO<4> {
+struct RowIO<float, 4> {
   template <bool STREAM>
   static __device__ __forceinline__ void load(const float* p, float (&v)[4])
   {
@@ -53,7 +54,7 @@ struct RowIO<4> {
   static __device__ __forceinline__ void store(float* p, const float (&v)[4]) { Vec16<float>::store(p, v); }
 };
 template <>
-struct RowIO<1> {
+struct RowIO<float, 1> {
   template <bool STREAM>
   static __device__ __forceinline__ void load(const float* p, float (&v)[1])
   {
@@ -61,12 +62,38 @@ struct RowIO<1> {
   }
   static __device__ __forceinline__ void store(float* p, const float (&v)[1]) { *p = v[0]; }
 };
+// fp16 storage: 16-byte vectors of eight halves, or single halves for rows off the 16-byte
+// grid; values are widened to fp32 on load and rounded to nearest even on store.
+template <>
+struct RowIO<__half, 8> {
+  template <bool STREAM>
+  static __device__ __forceinline__ void load(const __half* p, float (&v)[8])
+  {
+    Vec16<__half>::load(p, v);
+  }
+  static __device__ __forceinline__ void store(__half* p, const float (&v)[8]) { Vec16<__half>::store(p, v); }
+};
+template <>
+struct RowIO<__half, 1> {
+  template <bool STREAM>
+  static __device__ __forceinline__ void load(const __half* p, float (&v)[1])
+  {
+    v[0] = __half2float(*p);
+  }
+  static __device__ __forceinline__ void store(__half* p, const float (&v)[1]) { *p = __float2half_rn(v[0]); }
+};
+
+template <typename S>
+struct RowLoad {
+  static __device__ __forceinline__ float get(const S* p) { float v[1]; RowIO<S, 1>::template load<false>(p, v); return v[0]; }
+  static __device__ __forceinline__ void put(S* p, float r) { const float v[1] = {r}; RowIO<S, 1>::store(p, v); }
+};
 
 // 1024-thread blocks are held to 64 registers so that two of them share a compute unit
-// (not those with 32 accesses per thread, which would spill).
-template <int TPR, int V, int KIND, bool STREAM, int W = 4>
-__global__ void __launch_bounds__(RowBlock<TPR>::kThreads, (TPR == 1024 && V <= 16 ? 8 : 1))
-sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
+// (not those with 32 accesses or more than 32 values per thread, which would spill).
+template <typename S, int TPR, int V, int KIND, bool STREAM, int W = 16 / sizeof(S)>
+__global__ void __launch_bounds__(RowBlock<TPR>::kThreads, (TPR == 1024 && V <= 16 && V * W <= 32 ? 8 : 1))
+sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
             unsigned nvec)
 {
   using B = RowBlock<TPR>;
@@ -83,13 +110,13 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
   const int64_t row = static_cast<int64_t>(blockIdx.x) * B::kTeams + team;
   if (B::kTeams > 1 && row >= rows) return;  // whole waves leave; no barrier below in that case
 
-  const float* xr = x + map.offset(row, ldx);
+  const S* xr = x + map.offset(row, ldx);
   float v[V][W];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      RowIO<W>::template load<STREAM>(xr + unsigned(W) * idx, v[i]);
+      RowIO<S, W>::template load<STREAM>(xr + unsigned(W) * idx, v[i]);
     }
     else {
 #pragma unroll
@@ -139,7 +166,7 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
     gs = wave_sum(ps * exp_fast(pm - gm));
   }
 
-  float* yr = y + map.offset(row, ldy);
+  S* yr = y + map.offset(row, ldy);
   const float shift = m - gm;  // <= 0
   const float f = exp_fast(shift) * (1.0f / gs);
   const float lse = (KIND == kLogSoftmax) ? log_of_sum(gs) : 0.f;
@@ -160,15 +187,15 @@ sm_fwd_rows(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int6
           v[i][k] *= f;
         }
       }
-      RowIO<W>::store(yr + unsigned(W) * idx, v[i]);
+      RowIO<S, W>::store(yr + unsigned(W) * idx, v[i]);
     }
   }
 }
 
 // softmax / channelwise: dx = y * (dy - dot(y, dy));  log-softmax: dx = dy - exp(y) * sum(dy)
-template <int TPR, int V, int KIND, int STREAM, int W = 4>  // STREAM: bit 0 streams y, bit 1 dy
+template <typename S, int TPR, int V, int KIND, int STREAM, int W = 16 / sizeof(S)>  // STREAM: bit 0 streams y, bit 1 dy
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
-sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
+sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx,
             RowMap map, int64_t rows, unsigned nvec)
 {
   using B = RowBlock<TPR>;
@@ -184,15 +211,15 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
   const int64_t row = static_cast<int64_t>(blockIdx.x) * B::kTeams + team;
   if (B::kTeams > 1 && row >= rows) return;
 
-  const float* yr = y + map.offset(row, ldy);
-  const float* gr = dy + map.offset(row, lddy);
+  const S* yr = y + map.offset(row, ldy);
+  const S* gr = dy + map.offset(row, lddy);
   float a[V][W], g[V][W];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      RowIO<W>::template load<(STREAM & 1) != 0>(yr + unsigned(W) * idx, a[i]);
-      RowIO<W>::template load<(STREAM & 2) != 0>(gr + unsigned(W) * idx, g[i]);
+      RowIO<S, W>::template load<(STREAM & 1) != 0>(yr + unsigned(W) * idx, a[i]);
+      RowIO<S, W>::template load<(STREAM & 2) != 0>(gr + unsigned(W) * idx, g[i]);
     }
     else {
 #pragma unroll
@@ -206,7 +233,7 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
     for (int k = 0; k < W; ++k) s += (KIND == kLogSoftmax) ? g[i][k] : a[i][k] * g[i][k];
   s = kSub ? row16_sum(s) : team_sum<NW>(s, red, wv, lane);
 
-  float* dr = dx + map.offset(row, lddx);
+  S* dr = dx + map.offset(row, lddx);
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
@@ -216,7 +243,7 @@ sm_bwd_rows(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ldd
         if (KIND == kLogSoftmax) g[i][k] = g[i][k] - exp_fast(a[i][k]) * s;
         else g[i][k] = a[i][k] * (g[i][k] - s);
       }
-      RowIO<W>::store(dr + unsigned(W) * idx, g[i]);
+      RowIO<S, W>::store(dr + unsigned(W) * idx, g[i]);
     }
   }
 }
@@ -266,7 +293,7 @@ __device__ __forceinline__ void sm_cl_load(float (&t)[V][W], const float* rowp, 
   for (int i = 0; i < V; ++i) {
     const unsigned idx = base + i * kClusterThreads;
     if (idx < nvec) {
-      RowIO<W>::template load<false>(rowp + W * static_cast<int64_t>(idx), t[i]);
+      RowIO<float, W>::template load<false>(rowp + W * static_cast<int64_t>(idx), t[i]);
     }
     else {
 #pragma unroll
@@ -347,7 +374,7 @@ __device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t
           t.v[i][j] *= f;
         }
       }
-      RowIO<W>::store(yr + W * static_cast<int64_t>(idx), t.v[i]);
+      RowIO<float, W>::store(yr + W * static_cast<int64_t>(idx), t.v[i]);
     }
   }
 }
@@ -431,7 +458,7 @@ __device__ __forceinline__ void sm_cl_bwd_finish(const SmClusterArgs& a, int64_t
         if (KIND == kLogSoftmax) t.g[i][j] = t.g[i][j] - exp_fast(t.a[i][j]) * tot;
         else t.g[i][j] = t.a[i][j] * (t.g[i][j] - tot);
       }
-      RowIO<W>::store(dr + W * static_cast<int64_t>(idx), t.g[i]);
+      RowIO<float, W>::store(dr + W * static_cast<int64_t>(idx), t.g[i]);
     }
   }
 }
@@ -784,6 +811,63 @@ sm_bwd_apply(const float* y, const float* dy, float* dx, int64_t ldy, int64_t ld
   }
 }
 
+// ============================================= fp16 rows beyond the register kernels
+// One 256-thread workgroup per row, element-wise access, fp32 arithmetic: maximum, sum of
+// exponentials, output (the input is read three times; rows this long in fp16 storage are
+// rare, so this is the complete-coverage path, not a tuned one).
+template <typename S, int KIND>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_fwd_generic(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t n)
+{
+  __shared__ float red[kChunkThreads / kWave];
+  const int64_t row = blockIdx.x;
+  const S* xr = x + map.offset(row, ldx);
+  S* yr = y + map.offset(row, ldy);
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  float m = -FLT_MAX;
+  for (int64_t i = threadIdx.x; i < n; i += kChunkThreads) m = fmaxf(m, RowLoad<S>::get(xr + i));
+  m = team_max<kChunkThreads / kWave>(m, red, wv, lane);
+  __syncthreads();
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += kChunkThreads) s += exp_fast(RowLoad<S>::get(xr + i) - m);
+  s = team_sum<kChunkThreads / kWave>(s, red, wv, lane);
+  const float f = 1.0f / s;
+  const float lse = (KIND == kLogSoftmax) ? log_of_sum(s) : 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += kChunkThreads) {
+    const float d = RowLoad<S>::get(xr + i) - m;
+    float r;
+    if (KIND == kLogSoftmax) {
+      r = d - lse;
+    }
+    else {
+      r = f * exp_fast(d);
+      r = __builtin_isnormal(r) ? r : 0.f;
+    }
+    RowLoad<S>::put(yr + i, r);
+  }
+}
+
+template <typename S, int KIND>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_bwd_generic(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx, RowMap map, int64_t n)
+{
+  __shared__ float red[kChunkThreads / kWave];
+  const int64_t row = blockIdx.x;
+  const S* yr = y + map.offset(row, ldy);
+  const S* gr = dy + map.offset(row, lddy);
+  S* dr = dx + map.offset(row, lddx);
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += kChunkThreads)
+    s += (KIND == kLogSoftmax) ? RowLoad<S>::get(gr + i) : RowLoad<S>::get(yr + i) * RowLoad<S>::get(gr + i);
+  s = team_sum<kChunkThreads / kWave>(s, red, wv, lane);
+  // in place (dx aliasing dy): element i is read and written by the same thread, after the sum
+  for (int64_t i = threadIdx.x; i < n; i += kChunkThreads) {
+    const float a = RowLoad<S>::get(yr + i), g = RowLoad<S>::get(gr + i);
+    RowLoad<S>::put(dr + i, (KIND == kLogSoftmax) ? g - exp_fast(a) * s : a * (g - s));
+  }
+}
+
 // ==================================================================== host side
 struct ChunkPlan {
   int S;
@@ -947,10 +1031,11 @@ static int sm_bwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, 
   X(16, 1) X(16, 2) X(16, 4) X(64, 1) X(64, 2) X(64, 4) X(64, 8) X(256, 1) X(256, 2) X(256, 4) X(256, 8) X(1024, 1)      \
   X(1024, 2) X(1024, 4) X(1024, 8)
 
-template <int KIND>
+template <int KIND, typename S = float>
 static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int64_t w,
-                  const float* x, int64_t ldx, float* y, int64_t ldy, void* ws, size_t ws_bytes)
+                  const S* x, int64_t ldx, S* y, int64_t ldy, void* ws, size_t ws_bytes)
 {
+  constexpr int VE = 16 / sizeof(S);  // entries per 16-byte vector
   if (groups < 0 || n < 0 || w < 0 || stride < 0) return LBN_ERR_INVALID_ARGUMENT;
   if (groups == 0 || n == 0 || w == 0) return LBN_OK;
   if (!x || !y) return LBN_ERR_INVALID_ARGUMENT;
@@ -959,21 +1044,21 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   const int64_t rows = groups * w;
   if (rows > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
   const RowMap map{groups, stride};
-  const bool vec = (n % 4 == 0) && rows_aligned16(x, stride, ldx, groups, w, 4) &&
-                   rows_aligned16(y, stride, ldy, groups, w, 4);
+  const bool vec = (n % VE == 0) && rows_aligned16(x, stride, ldx, groups, w, sizeof(S)) &&
+                   rows_aligned16(y, stride, ldy, groups, w, sizeof(S));
   if (vec) {
-    const RowConfig c = pick_sm_row_config(n / 4, rows);
+    const RowConfig c = pick_sm_row_config(n / VE, rows);
     if (c.tpr) {
-      const unsigned nvec = static_cast<unsigned>(n / 4);
+      const unsigned nvec = static_cast<unsigned>(n / VE);
 #define X(TPR, V)                                                                            \
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
     const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
-    if (stream_loads(rows, n, 2))                                                            \
-      hipLaunchKernelGGL((sm_fwd_rows<TPR, V, KIND, true>), dim3(grid), dim3(B::kThreads), 0, st, \
+    if (stream_loads(rows, n * sizeof(S) / 4, 2))                                            \
+      hipLaunchKernelGGL((sm_fwd_rows<S, TPR, V, KIND, true>), dim3(grid), dim3(B::kThreads), 0, st, \
                          x, y, ldx, ldy, map, rows, nvec);                                   \
     else                                                                                     \
-      hipLaunchKernelGGL((sm_fwd_rows<TPR, V, KIND, false>), dim3(grid), dim3(B::kThreads), 0, st, \
+      hipLaunchKernelGGL((sm_fwd_rows<S, TPR, V, KIND, false>), dim3(grid), dim3(B::kThreads), 0, st, \
                          x, y, ldx, ldy, map, rows, nvec);                                   \
     return launch_status();                                                                  \
   }
@@ -990,7 +1075,7 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
     const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
-    hipLaunchKernelGGL((sm_fwd_rows<TPR, V, KIND, false, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
+    hipLaunchKernelGGL((sm_fwd_rows<S, TPR, V, KIND, false, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
                        x, y, ldx, ldy, map, rows, nvec);                                     \
     return launch_status();                                                                  \
   }
@@ -1003,48 +1088,57 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     const unsigned nvec = static_cast<unsigned>(n);
     const unsigned grid = static_cast<unsigned>(rows);
     if (n <= 16 * 1024)
-      hipLaunchKernelGGL((sm_fwd_rows<1024, 16, KIND, false, 1>), dim3(grid), dim3(1024), 0, st, x, y, ldx, ldy,
+      hipLaunchKernelGGL((sm_fwd_rows<S, 1024, 16, KIND, false, 1>), dim3(grid), dim3(1024), 0, st, x, y, ldx, ldy,
                          map, rows, nvec);
     else
-      hipLaunchKernelGGL((sm_fwd_rows<1024, 32, KIND, false, 1>), dim3(grid), dim3(1024), 0, st, x, y, ldx, ldy,
+      hipLaunchKernelGGL((sm_fwd_rows<S, 1024, 32, KIND, false, 1>), dim3(grid), dim3(1024), 0, st, x, y, ldx, ldy,
                          map, rows, nvec);
     return launch_status();
   }
-  if (cluster_enabled(st, rows, n)) {
-    int r = -1;
-    if (vec && n / 4 < (int64_t(1) << 30)) {
-      // four vectors per thread keep five workgroups per CU resident; eight only for rows that need it
-      ClusterPlan cp = plan_cluster(n / 4, 4);
-      if (!cp.M) cp = plan_cluster(n / 4, 8);
-      r = sm_fwd_cluster_launch<KIND, 4>(st, cp, n / 4, rows, x, ldx, y, ldy, map, ws, ws_bytes);
-    }
-    else if (!vec) {
-      // rows off the 16-byte grid (a vocabulary of 50257 entries): the same kernel, one float per access
-      r = sm_fwd_cluster_launch<KIND, 1>(st, plan_cluster(n, 8), n, rows, x, ldx, y, ldy, map, ws, ws_bytes);
-    }
-    if (r >= 0) return r;
-  }
-  const ChunkPlan p = plan_chunks(n, rows);
-  if (rows * p.S > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
-  if (!ws || ws_bytes < kWorkspaceHeaderBytes + static_cast<size_t>(rows) * p.S * sizeof(float2)) return LBN_ERR_WORKSPACE;
-  float2* part = static_cast<float2*>(workspace_payload(ws));
-  const dim3 grid(static_cast<unsigned>(rows * p.S)), block(kChunkThreads);
-  if (vec) {
-    hipLaunchKernelGGL((sm_fwd_partial<true>), grid, block, 0, st, x, ldx, map, n, p.chunk, p.S, part);
-    hipLaunchKernelGGL((sm_fwd_apply<true, KIND>), grid, block, 0, st, x, y, ldx, ldy, map, n, p.chunk, p.S, part);
+  if constexpr (!std::is_same<S, float>::value) {
+    // fp16 rows beyond the register kernels: one workgroup per row, three passes
+    hipLaunchKernelGGL((sm_fwd_generic<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kChunkThreads), 0, st, x, y,
+                       ldx, ldy, map, n);
+    return launch_status();
   }
   else {
-    hipLaunchKernelGGL((sm_fwd_partial<false>), grid, block, 0, st, x, ldx, map, n, p.chunk, p.S, part);
-    hipLaunchKernelGGL((sm_fwd_apply<false, KIND>), grid, block, 0, st, x, y, ldx, ldy, map, n, p.chunk, p.S, part);
+    if (cluster_enabled(st, rows, n)) {
+      int r = -1;
+      if (vec && n / 4 < (int64_t(1) << 30)) {
+        // four vectors per thread keep five workgroups per CU resident; eight only for rows that need it
+        ClusterPlan cp = plan_cluster(n / 4, 4);
+        if (!cp.M) cp = plan_cluster(n / 4, 8);
+        r = sm_fwd_cluster_launch<KIND, 4>(st, cp, n / 4, rows, x, ldx, y, ldy, map, ws, ws_bytes);
+      }
+      else if (!vec) {
+        // rows off the 16-byte grid (a vocabulary of 50257 entries): the same kernel, one float per access
+        r = sm_fwd_cluster_launch<KIND, 1>(st, plan_cluster(n, 8), n, rows, x, ldx, y, ldy, map, ws, ws_bytes);
+      }
+      if (r >= 0) return r;
+    }
+    const ChunkPlan p = plan_chunks(n, rows);
+    if (rows * p.S > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+    if (!ws || ws_bytes < kWorkspaceHeaderBytes + static_cast<size_t>(rows) * p.S * sizeof(float2)) return LBN_ERR_WORKSPACE;
+    float2* part = static_cast<float2*>(workspace_payload(ws));
+    const dim3 grid(static_cast<unsigned>(rows * p.S)), block(kChunkThreads);
+    if (vec) {
+      hipLaunchKernelGGL((sm_fwd_partial<true>), grid, block, 0, st, x, ldx, map, n, p.chunk, p.S, part);
+      hipLaunchKernelGGL((sm_fwd_apply<true, KIND>), grid, block, 0, st, x, y, ldx, ldy, map, n, p.chunk, p.S, part);
+    }
+    else {
+      hipLaunchKernelGGL((sm_fwd_partial<false>), grid, block, 0, st, x, ldx, map, n, p.chunk, p.S, part);
+      hipLaunchKernelGGL((sm_fwd_apply<false, KIND>), grid, block, 0, st, x, y, ldx, ldy, map, n, p.chunk, p.S, part);
+    }
+    return launch_status();
   }
-  return launch_status();
 }
 
-template <int KIND>
+template <int KIND, typename S = float>
 static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int64_t w,
-                  const float* y, int64_t ldy, const float* dy, int64_t lddy, float* dx,
+                  const S* y, int64_t ldy, const S* dy, int64_t lddy, S* dx,
                   int64_t lddx, void* ws, size_t ws_bytes)
 {
+  constexpr int VE = 16 / sizeof(S);
   if (groups < 0 || n < 0 || w < 0 || stride < 0) return LBN_ERR_INVALID_ARGUMENT;
   if (groups == 0 || n == 0 || w == 0) return LBN_OK;
   if (!y || !dy || !dx) return LBN_ERR_INVALID_ARGUMENT;
@@ -1053,31 +1147,32 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   const int64_t rows = groups * w;
   if (rows > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
   const RowMap map{groups, stride};
-  const bool vec = (n % 4 == 0) && rows_aligned16(y, stride, ldy, groups, w, 4) &&
-                   rows_aligned16(dy, stride, lddy, groups, w, 4) &&
-                   rows_aligned16(dx, stride, lddx, groups, w, 4);
+  const bool vec = (n % VE == 0) && rows_aligned16(y, stride, ldy, groups, w, sizeof(S)) &&
+                   rows_aligned16(dy, stride, lddy, groups, w, sizeof(S)) &&
+                   rows_aligned16(dx, stride, lddx, groups, w, sizeof(S));
   if (vec) {
     // two tensors live in registers: cap each at 4 vectors per thread when a row
     // still fits, so 1024-thread blocks keep two blocks per compute unit
-    const RowConfig c = pick_sm_row_config(n / 4, rows);
+    const RowConfig c = pick_sm_row_config(n / VE, rows);
     if (c.tpr) {
-      const unsigned nvec = static_cast<unsigned>(n / 4);
+      const unsigned nvec = static_cast<unsigned>(n / VE);
 #define X(TPR, V)                                                                            \
+  if constexpr (!(TPR == 1024 && V * VE > 32)) /* two tensors of more would not fit 128 registers */ \
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
     const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
-    const int hint = stream_loads_bwd(rows, n);                                              \
+    const int hint = stream_loads_bwd(rows, n * sizeof(S) / 4);                              \
     if (hint == 3)                                                                           \
-      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, 3>), dim3(grid), dim3(B::kThreads), 0, st, \
+      hipLaunchKernelGGL((sm_bwd_rows<S, TPR, V, KIND, 3>), dim3(grid), dim3(B::kThreads), 0, st, \
                          y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
     else if (hint == 1)                                                                      \
-      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
+      hipLaunchKernelGGL((sm_bwd_rows<S, TPR, V, KIND, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
                          y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
     else if (hint == 2)                                                                      \
-      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, 2>), dim3(grid), dim3(B::kThreads), 0, st, \
+      hipLaunchKernelGGL((sm_bwd_rows<S, TPR, V, KIND, 2>), dim3(grid), dim3(B::kThreads), 0, st, \
                          y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
     else                                                                                     \
-      hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, 0>), dim3(grid), dim3(B::kThreads), 0, st, \
+      hipLaunchKernelGGL((sm_bwd_rows<S, TPR, V, KIND, 0>), dim3(grid), dim3(B::kThreads), 0, st, \
                          y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \
     return launch_status();                                                                  \
   }
@@ -1093,7 +1188,7 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
     const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
-    hipLaunchKernelGGL((sm_bwd_rows<TPR, V, KIND, 0, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
+    hipLaunchKernelGGL((sm_bwd_rows<S, TPR, V, KIND, 0, 1>), dim3(grid), dim3(B::kThreads), 0, st, \
                        y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                         \
     return launch_status();                                                                  \
   }
@@ -1101,41 +1196,50 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #undef X
     }
   }
-  else if (n <= kMaxScalarLongRow) {
+  else if (n <= (std::is_same<S, float>::value ? kMaxScalarLongRow : 16 * 1024)) {
     const unsigned nvec = static_cast<unsigned>(n);
     const unsigned grid = static_cast<unsigned>(rows);
-    if (n <= 16 * 1024)
-      hipLaunchKernelGGL((sm_bwd_rows<1024, 16, KIND, 0, 1>), dim3(grid), dim3(1024), 0, st, y, dy, dx, ldy,
+    if (n <= 16 * 1024) {
+      hipLaunchKernelGGL((sm_bwd_rows<S, 1024, 16, KIND, 0, 1>), dim3(grid), dim3(1024), 0, st, y, dy, dx, ldy,
                          lddy, lddx, map, rows, nvec);
-    else
-      hipLaunchKernelGGL((sm_bwd_rows<1024, 32, KIND, 0, 1>), dim3(grid), dim3(1024), 0, st, y, dy, dx, ldy,
+    }
+    else if constexpr (std::is_same<S, float>::value) {
+      hipLaunchKernelGGL((sm_bwd_rows<S, 1024, 32, KIND, 0, 1>), dim3(grid), dim3(1024), 0, st, y, dy, dx, ldy,
                          lddy, lddx, map, rows, nvec);
+    }
     return launch_status();
   }
-  if (cluster_enabled(st, rows, n)) {
-    int r = -1;
-    if (vec && n / 4 < (int64_t(1) << 30))
-      r = sm_bwd_cluster_launch<KIND, 4>(st, plan_cluster(n / 4, 4), n / 4, rows, y, ldy, dy, lddy, dx, lddx, map, ws,
-                                         ws_bytes);
-    else if (!vec)
-      r = sm_bwd_cluster_launch<KIND, 1>(st, plan_cluster(n, 8), n, rows, y, ldy, dy, lddy, dx, lddx, map, ws,
-                                         ws_bytes);
-    if (r >= 0) return r;
-  }
-  const ChunkPlan p = plan_chunks(n, rows);
-  if (rows * p.S > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
-  if (!ws || ws_bytes < kWorkspaceHeaderBytes + static_cast<size_t>(rows) * p.S * sizeof(float2)) return LBN_ERR_WORKSPACE;
-  float* part = static_cast<float*>(workspace_payload(ws));
-  const dim3 grid(static_cast<unsigned>(rows * p.S)), block(kChunkThreads);
-  if (vec) {
-    hipLaunchKernelGGL((sm_bwd_partial<true, KIND>), grid, block, 0, st, y, dy, ldy, lddy, map, n, p.chunk, p.S, part);
-    hipLaunchKernelGGL((sm_bwd_apply<true, KIND>), grid, block, 0, st, y, dy, dx, ldy, lddy, lddx, map, n, p.chunk, p.S, part);
+  if constexpr (!std::is_same<S, float>::value) {
+    hipLaunchKernelGGL((sm_bwd_generic<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kChunkThreads), 0, st, y, dy,
+                       dx, ldy, lddy, lddx, map, n);
+    return launch_status();
   }
   else {
-    hipLaunchKernelGGL((sm_bwd_partial<false, KIND>), grid, block, 0, st, y, dy, ldy, lddy, map, n, p.chunk, p.S, part);
-    hipLaunchKernelGGL((sm_bwd_apply<false, KIND>), grid, block, 0, st, y, dy, dx, ldy, lddy, lddx, map, n, p.chunk, p.S, part);
+    if (cluster_enabled(st, rows, n)) {
+      int r = -1;
+      if (vec && n / 4 < (int64_t(1) << 30))
+        r = sm_bwd_cluster_launch<KIND, 4>(st, plan_cluster(n / 4, 4), n / 4, rows, y, ldy, dy, lddy, dx, lddx, map, ws,
+                                           ws_bytes);
+      else if (!vec)
+        r = sm_bwd_cluster_launch<KIND, 1>(st, plan_cluster(n, 8), n, rows, y, ldy, dy, lddy, dx, lddx, map, ws,
+                                           ws_bytes);
+      if (r >= 0) return r;
+    }
+    const ChunkPlan p = plan_chunks(n, rows);
+    if (rows * p.S > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+    if (!ws || ws_bytes < kWorkspaceHeaderBytes + static_cast<size_t>(rows) * p.S * sizeof(float2)) return LBN_ERR_WORKSPACE;
+    float* part = static_cast<float*>(workspace_payload(ws));
+    const dim3 grid(static_cast<unsigned>(rows * p.S)), block(kChunkThreads);
+    if (vec) {
+      hipLaunchKernelGGL((sm_bwd_partial<true, KIND>), grid, block, 0, st, y, dy, ldy, lddy, map, n, p.chunk, p.S, part);
+      hipLaunchKernelGGL((sm_bwd_apply<true, KIND>), grid, block, 0, st, y, dy, dx, ldy, lddy, lddx, map, n, p.chunk, p.S, part);
+    }
+    else {
+      hipLaunchKernelGGL((sm_bwd_partial<false, KIND>), grid, block, 0, st, y, dy, ldy, lddy, map, n, p.chunk, p.S, part);
+      hipLaunchKernelGGL((sm_bwd_apply<false, KIND>), grid, block, 0, st, y, dy, dx, ldy, lddy, lddx, map, n, p.chunk, p.S, part);
+    }
+    return launch_status();
   }
-  return launch_status();
 }
 
 // ------------------------------------------------------------ library-owned scratch
@@ -1225,6 +1329,40 @@ int lbn_log_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, 
                             void* workspace, size_t workspace_bytes)
 {
   return sm_bwd<kLogSoftmax>(as_stream(stream), 1, height, height, width, y, ldy, dy, lddy, dx, lddx, workspace, workspace_bytes);
+}
+
+// fp16 storage (IEEE binary16 in memory, fp32 arithmetic); the workspace arguments are there for
+// symmetry with the fp32 entry points and are not used.
+int lbn_softmax_fwd_f16(lbn_stream_t stream, int64_t height, int64_t width, const void* x, int64_t ldx, void* y,
+                        int64_t ldy, void* workspace, size_t workspace_bytes)
+{
+  return sm_fwd<kSoftmax, __half>(as_stream(stream), 1, height, height, width, static_cast<const __half*>(x), ldx,
+                                  static_cast<__half*>(y), ldy, workspace, workspace_bytes);
+}
+
+int lbn_softmax_bwd_f16(lbn_stream_t stream, int64_t height, int64_t width, const void* y, int64_t ldy,
+                        const void* dy, int64_t lddy, void* dx, int64_t lddx, void* workspace,
+                        size_t workspace_bytes)
+{
+  return sm_bwd<kSoftmax, __half>(as_stream(stream), 1, height, height, width, static_cast<const __half*>(y), ldy,
+                                  static_cast<const __half*>(dy), lddy, static_cast<__half*>(dx), lddx, workspace,
+                                  workspace_bytes);
+}
+
+int lbn_log_softmax_fwd_f16(lbn_stream_t stream, int64_t height, int64_t width, const void* x, int64_t ldx,
+                            void* y, int64_t ldy, void* workspace, size_t workspace_bytes)
+{
+  return sm_fwd<kLogSoftmax, __half>(as_stream(stream), 1, height, height, width, static_cast<const __half*>(x), ldx,
+                                     static_cast<__half*>(y), ldy, workspace, workspace_bytes);
+}
+
+int lbn_log_softmax_bwd_f16(lbn_stream_t stream, int64_t height, int64_t width, const void* y, int64_t ldy,
+                            const void* dy, int64_t lddy, void* dx, int64_t lddx, void* workspace,
+                            size_t workspace_bytes)
+{
+  return sm_bwd<kLogSoftmax, __half>(as_stream(stream), 1, height, height, width, static_cast<const __half*>(y), ldy,
+                                     static_cast<const __half*>(dy), lddy, static_cast<__half*>(dx), lddx, workspace,
+                                     workspace_bytes);
 }
 
 int lbn_channelwise_softmax_fwd_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,

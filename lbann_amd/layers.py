@@ -450,16 +450,20 @@ class batch_normalization_layer(_Layer):
 class _softmax_like(_Layer):
     _name = None
 
+    @staticmethod
+    def _suffix(m):
+        return "f16" if m.dtype == torch.float16 else "f32"
+
     def fp_call(self):
         x, y = self.prev_activations, self.activations
         ws, nb = self._ws.get(capi.lib().lbn_softmax_workspace_bytes(x.height, x.width), self.device)
-        return (f"lbn_{self._name}_fwd_f32",
+        return (f"lbn_{self._name}_fwd_{self._suffix(x)}",
                 (_stream(), x.height, x.width, x.Buffer(), x.ldim, y.Buffer(), y.ldim, ws, nb))
 
     def bp_call(self):
         y, dy, dx = self.activations, self.prev_error_signals, self.error_signals
         ws, nb = self._ws.get(capi.lib().lbn_softmax_workspace_bytes(y.height, y.width), self.device)
-        return (f"lbn_{self._name}_bwd_f32",
+        return (f"lbn_{self._name}_bwd_{self._suffix(y)}",
                 (_stream(), y.height, y.width, y.Buffer(), y.ldim, dy.Buffer(), dy.ldim, dx.Buffer(),
                  dx.ldim, ws, nb))
 

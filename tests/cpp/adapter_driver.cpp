@@ -341,6 +341,32 @@ int drv_gradient_buffer(const int64_t* dims, int nd, int64_t h, int64_t w, const
   }
 }
 
+// fp16 storage through the adapter: a matrix type with 2-byte elements selects the _f16 entry
+// points.  kind: 0 softmax, 1 log-softmax.
+int drv_softmax_family_f16(int kind, int64_t h, int64_t w, int64_t ld, void* x, void* y, void* dy, void* dx,
+                           void* stream, char* err, int errlen)
+{
+  try {
+    using half_bits = unsigned short;
+    device_matrix<half_bits> mx, my, mdy, mdx;
+    attach(mx, h, w, x, ld); attach(my, h, w, y, ld); attach(mdy, h, w, dy, ld); attach(mdx, h, w, dx, ld);
+    auto bind = [&](auto& layer) {
+      layer.io.prev_activations = &mx; layer.io.activations = &my;
+      layer.io.prev_error_signals = &mdy; layer.io.error_signals = &mdx;
+      layer.io.stream = static_cast<hipStream_t>(stream);
+      layer.fp_compute();
+      layer.bp_compute();
+      check_hip(hipStreamSynchronize(layer.io.stream), "sync");
+    };
+    if (kind == 0) { softmax_layer<device_matrix<half_bits>> l; bind(l); }
+    else { log_softmax_layer<device_matrix<half_bits>> l; bind(l); }
+    return 0;
+  }
+  catch (const std::exception& e) {
+    return fail(e, err, errlen);
+  }
+}
+
 // A softmax layer on a (h x w) problem that uses scratch: forward, then the wait check, which
 // must pass; then the designed give-up exit is run on the layer's own scratch buffer and
 // the next check must throw (returns 0 only if it did, with the message in err), after which

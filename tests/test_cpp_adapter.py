@@ -130,6 +130,24 @@ def test_adapter_layers_match_oracle():
         check(f"adapter softmax kind {kind} y", y, fwd(x), fwd(f64(x)))
         check(f"adapter softmax kind {kind} dx", mdx.to_numpy(), bwd(y, dy), bwd(f64(y), f64(dy)))
 
+    # ---- softmax and log-softmax on fp16 storage: a matrix type with 2-byte elements
+    import torch as _torch
+    h, w = 4096, 12
+    x16 = mk(h, w, 0.0, 2.0).astype(np.float16)
+    dy16 = mk(h, w).astype(np.float16)
+    xf, dyf = np.asfortranarray(x16.astype(np.float32)), np.asfortranarray(dy16.astype(np.float32))
+    for kind in (0, 1):
+        mx = DeviceMatrix.from_numpy(x16, dtype=_torch.float16)
+        mdy = DeviceMatrix.from_numpy(dy16, dtype=_torch.float16)
+        my, mdx = DeviceMatrix(h, w, dtype=_torch.float16), DeviceMatrix(h, w, dtype=_torch.float16)
+        rc = d.drv_softmax_family_f16(cint(kind), i64(h), i64(w), i64(h), mx.Buffer(), my.Buffer(), mdy.Buffer(),
+                                      mdx.Buffer(), st, err, cint(512))
+        assert rc == 0, err.value
+        fwd, bwd = (orc.softmax_fwd, orc.softmax_bwd) if kind == 0 else (orc.log_softmax_fwd, orc.log_softmax_bwd)
+        y = my.to_numpy()
+        check(f"adapter f16 softmax kind {kind} y", y, fwd(xf), tol=TOL_F16)
+        check(f"adapter f16 softmax kind {kind} dx", mdx.to_numpy(), bwd(np.asfortranarray(y), dyf), tol=TOL_F16)
+
     # ---- instance norm on (6, 20, 20) samples
     dims, w = (6, 20, 20), 9
     h = 6 * 400

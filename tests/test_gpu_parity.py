@@ -80,6 +80,55 @@ def test_softmax_family(L, kind, h, w, pad):
     check(f"{kind} dx {h}x{w}", dx, bwd(f32(y), dy), bwd(f64(y), f64(dy)))
 
 
+@pytest.mark.parametrize("kind", ["softmax", "log_softmax"])
+@pytest.mark.parametrize("h,w,pad,in_place", [
+    (1000, 37, 0, False), (4096, 64, 0, False), (32768, 48, 0, True), (65536, 9, 0, False),   # 16-byte vectors
+    (197, 50, 0, False), (1001, 33, 3, False), (16385, 6, 0, True),                          # single halves
+    (64, 5000, 0, False), (24, 4099, 0, False),                                             # short rows, 16-lane teams
+    (70000, 3, 0, False), (40001, 2, 0, True), (131072, 2, 0, False),                        # beyond the register kernels
+])
+def test_softmax_family_f16_storage(L, kind, h, w, pad, in_place):
+    """fp16 storage, fp32 arithmetic (softmax.cpp:236-243 instantiates the layers for half):
+    both sides see the fp16-rounded inputs; the oracle is the fp32 restatement on them."""
+    rng = np.random.default_rng(3 * h + w)
+    x16 = rand(rng, h, w, 0, 2).astype(np.float16)
+    dy16 = rand(rng, h, w).astype(np.float16)
+    x, dy = f32(x16), f32(dy16)
+    layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
+    fwd, bwd = _sm_oracle(kind)
+    ld = h + pad
+    xm = L.DeviceMatrix.from_numpy(x16, dtype=torch.float16, ldim=ld)
+    ym = layer.forward(xm, in_place=in_place)
+    assert ym.dtype == torch.float16 and (ym is xm) == in_place
+    y = ym.to_numpy()
+    check(f"{kind} f16 y {h}x{w}", y, fwd(x), fwd(f64(x)), tol=TOL_F16)
+    gm = L.DeviceMatrix.from_numpy(dy16, dtype=torch.float16, ldim=ld)
+    dx = layer.backward(gm, in_place=in_place).to_numpy()
+    # backward consumes the layer's own (fp16) output, as in the framework
+    check(f"{kind} f16 dx {h}x{w}", dx, bwd(f32(y), dy), bwd(f64(y), f64(dy)), tol=TOL_F16)
+    if kind == "softmax":
+        assert np.abs(y.astype(np.float64).sum(axis=0) - 1).max() < 2e-3 * np.sqrt(h)
+
+
+def test_softmax_f16_special_values(L):
+    """A column of equal values, one with a dominant entry, one with -inf entries, one NaN."""
+    h = 256
+    x = np.zeros((h, 4), dtype=np.float16)
+    x[:, 0] = 3.0
+    x[7, 1] = 60000.0
+    x[:, 2] = -np.inf
+    x[5, 2] = 1.0
+    x[9, 3] = np.nan
+    layer = L.softmax_layer()
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, dtype=torch.float16)).to_numpy()
+    ref = orc.softmax_fwd(f32(x))
+    assert np.allclose(y[:, 0], 1.0 / h, rtol=2e-3)
+    assert y[7, 1] == 1.0 and y[:, 1].sum() == 1.0
+    assert y[5, 2] == 1.0 and y[:, 2].sum() == 1.0
+    # a NaN in the column: the reference's output for that column is all zeros (non-normal results are flushed)
+    assert (ref[:, 3] == 0).all() and (y[:, 3] == 0).all()
+
+
 @pytest.mark.parametrize("kind", ["softmax", "log_softmax", "channelwise"])
 @pytest.mark.parametrize("h,w,in_place", [(262144, 17, False), (65536, 40, False), (262144, 16, True), (131072, 31, True)])
 def test_few_long_rows_all_in_flight(L, kind, h, w, in_place):
