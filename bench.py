@@ -194,6 +194,37 @@ def main():
         # forward reads prediction and ground truth; backward reads both and writes both gradients
         return layer, pred.size, 4, w, cpu, (2 * pred.size * 4, 4 * pred.size * 4)
 
+    def build_sm_ce(data):
+        """The classification tail: "forward" is softmax and cross entropy in one call (reads x and
+        the ground truth, writes y: 3 tensors), "backward" the cross-entropy backward that follows
+        (reads y and the ground truth, writes both gradients: 4 tensors)."""
+        h, w = data["x"].shape
+        rng = np.random.default_rng(17)
+        truth = np.asfortranarray(rng.uniform(0.0, 1.0, (w, h)).astype(np.float32).T)
+        dloss = rng.standard_normal(w).astype(np.float32)
+        sm, ce = L.softmax_layer(), L.cross_entropy_layer((h,))
+        x, t = upload(data["x"]), upload(truth)
+        y, loss = L.softmax_cross_entropy_forward(sm, ce, x, t)
+        ce.backward(L.DeviceMatrix.from_numpy(dloss.reshape(1, -1)))
+        ws, nb = sm._ws.get(L.capi.lib().lbn_softmax_cross_entropy_fwd_workspace_bytes(h, w), dev)
+
+        class tail:
+            def fp_call(self):
+                return "lbn_softmax_cross_entropy_fwd_f32", (L._stream(), h, w, 0, 1, x.Buffer(), x.ldim, t.Buffer(),
+                                                             t.ldim, y.Buffer(), y.ldim, loss.Buffer(), loss.ldim, ws, nb)
+
+            def bp_call(self):
+                return ce.bp_call()
+
+        def cpu():
+            from oracle import cpu_oracle as orc
+            t0 = time.perf_counter(); yy = orc.softmax_fwd(data["x"]); orc.cross_entropy_fwd(yy, truth)
+            t1 = time.perf_counter()
+            orc.cross_entropy_bwd(yy, truth, dloss); t2 = time.perf_counter()
+            return t1 - t0, t2 - t1
+        keep = (sm, ce, x, t, y, loss)  # noqa: F841  (owned by the closure for the life of the row)
+        return tail(), h * w, 4, w, cpu, (3 * h * w * 4, 4 * h * w * 4)
+
     def build_sb(data, kind):
         x, dy = upload(data["x"]), upload(data["dy"])
         h = data["x"].shape[0]
@@ -265,6 +296,8 @@ def main():
         # not baseline configurations: the layers either side of the path, on the tensors of cfg2 / cfg3
         "extra_cross_entropy": ("CrossEntropy (dense ground truth) fwd+bwd fp32 32768x512 (informational)",
                                 lambda: build_ce(W.cfg2_softmax())),
+        "extra_softmax_cross_entropy": ("Softmax+CrossEntropy fused fwd, CrossEntropy bwd fp32 32768x512 (informational)",
+                                        lambda: build_sm_ce(W.cfg2_softmax())),
         "extra_entrywise_scale_bias": ("EntrywiseScaleBias fwd+bwd fp32 1048576x64 (informational)",
                                        lambda: build_sb(W.extra_entrywise_batch_norm(), "entrywise")),
         "extra_channelwise_scale_bias": ("ChannelwiseScaleBias fwd+bwd fp32 NCHW 64x256x56x56 (informational)",
@@ -533,7 +566,7 @@ def main():
         "config": {"workload": h["workload"], "samples": 512, "classes": 32768,
                    "samples_per_s": h["samples_per_s"], "frac_of_hbm_peak": h["frac_of_hbm_peak"],
                    "cold_frac": frac_of(h.get("cold")), "per_config": per_config},
-        "roofline": {"bound": "hbm", "kernel": "sm_bwd_rows<1024,8,softmax>", "achieved": dom_gbs,
+        "roofline": {"bound": "hbm", "kernel": "sm_bwd_rows<float,1024,8,softmax>", "achieved": dom_gbs,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom_gbs / HBM_PEAK_GBS,
                      "bytes_per_launch": dom_bytes, "avg_launch_ms": dom_ms,
                      "avg_launch_source": ("rocprofv3 per-dispatch average (profiles/bench_all_layers_kernel_trace.md), "

@@ -435,6 +435,24 @@ int lbn_cross_entropy_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width
                               float* dprediction, int64_t ld_dprediction,
                               float* dground_truth, int64_t ld_dground_truth);
 
+/* Softmax forward and the cross-entropy forward of its output in one pass: y as
+ * lbn_softmax_fwd_f32 writes it (softmax.cpp:43-109, flush included) and loss as
+ * lbn_cross_entropy_fwd_f32(prediction = y) gives it (cross_entropy.cpp:35-73), for the
+ * softmax -> cross_entropy pair that ends the reference's classification models.  The
+ * results are those of the two calls made one after the other; the cross entropy reads y
+ * from registers instead of from memory.  Rows that fit a workgroup's registers
+ * (height a multiple of 4, 16-byte aligned columns, at most 32768 entries) with a dense
+ * ground truth, or labels with spatial_size == 1, take the fused kernel; every other shape
+ * runs the two layers' kernels back to back inside this call.  The workspace serves both. */
+size_t lbn_softmax_cross_entropy_fwd_workspace_bytes(int64_t height, int64_t width);
+int lbn_softmax_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                                      int64_t spatial_size,
+                                      const float* x, int64_t ldx,
+                                      const float* ground_truth, int64_t ld_ground_truth,
+                                      float* y, int64_t ldy,
+                                      float* loss, int64_t ld_loss,
+                                      void* workspace, size_t workspace_bytes);
+
 /* ------------------------------------------------------- scale and bias layers
  * The learned affine layers that follow a normalization layer without one.  Replace
  * entrywise_scale_bias_layer::fp_compute / bp_compute

@@ -851,6 +851,26 @@ public:
                                            t.LDim(), loss.Buffer(), loss.LDim(), m_ws.reserve(bytes, io.stream), bytes),
                  "cross_entropy_layer::fp_compute");
   }
+  /// fp_compute() of `sm`, a softmax layer whose output is this layer's prediction
+  /// (sm.io.activations == io.prev_activations), and this layer's own, as one call: the
+  /// results of sm.fp_compute() followed by fp_compute().  fp32 storage.
+  void fp_compute_with(softmax_layer<Mat>& sm)
+  {
+    static_assert(sizeof(detail::element_t<Mat>) == 4, "the fused forward takes fp32 matrices");
+    if (sm.io.activations != io.prev_activations)
+      throw exception("cross_entropy_layer::fp_compute_with: the softmax layer's output is not this layer's prediction");
+    const Mat& x = *sm.io.prev_activations;
+    Mat& y = *sm.io.activations;
+    const Mat& t = *prev_ground_truth;
+    Mat& loss = *io.activations;
+    const size_t bytes = lbn_softmax_cross_entropy_fwd_workspace_bytes(x.Height(), x.Width());
+    check_status(lbn_softmax_cross_entropy_fwd_f32(sm.io.stream, x.Height(), x.Width(), m_use_labels ? 1 : 0,
+                                                   m_spatial_sample_size, x.LockedBuffer(), x.LDim(),
+                                                   t.LockedBuffer(), t.LDim(), y.Buffer(), y.LDim(), loss.Buffer(),
+                                                   loss.LDim(), sm.scratch().reserve(bytes, sm.io.stream), bytes),
+                 "cross_entropy_layer::fp_compute_with");
+    sm.scratch().after_call(sm.io.stream, "cross_entropy_layer::fp_compute_with");
+  }
   void bp_compute()
   {
     const Mat& x = *io.prev_activations;

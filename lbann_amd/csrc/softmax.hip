@@ -192,6 +192,108 @@ sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows
   }
 }
 
+// Softmax forward with the cross entropy against a ground truth taken in the same pass
+// (the consumer of the softmax output, src/layers/loss/cross_entropy.cpp:35-73): the row's
+// outputs are written as sm_fwd_rows writes them, and loss = -sum over entries with
+// xhat > 0 of xhat * log(y) is formed from the values that were just stored (flush included:
+// an entry flushed to 0 under a positive xhat gives an infinite loss, as it does when the two
+// layers run one after the other).  Saves the second layer's read of y.
+// LABELS: the ground truth is one class index per column, stored as a float in row 0
+// (use_labels with a spatial size of 1): xhat is 1 at that row and 0 elsewhere.
+template <int TPR, int V, bool LABELS>
+__global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
+sm_ce_fwd_rows(const float* x, const float* truth, float* y, float* loss, int64_t ldx, int64_t ldt, int64_t ldy,
+               int64_t ld_loss, int64_t rows, unsigned nvec)
+{
+  using B = RowBlock<TPR>;
+  constexpr int W = 4;
+  constexpr bool kSub = TPR < kWave;
+  static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
+  constexpr int NW = kSub ? 1 : B::kWavesPerTeam;
+  __shared__ float red[2][NW];
+  __shared__ float red_loss[NW];
+  const unsigned tid = threadIdx.x;
+  const int team = kSub ? static_cast<int>(tid) / TPR : wave_index() / NW;
+  const unsigned t = tid - team * TPR;
+  const int lane = tid & (kWave - 1);
+  const int wv = t / kWave;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * B::kTeams + team;
+  if (B::kTeams > 1 && row >= rows) return;
+
+  const float* xr = x + row * ldx;
+  const float* tr = truth + row * ldt;
+  float v[V][W], xh[LABELS ? 1 : V][W];
+  int label = -1;
+  if (LABELS) label = static_cast<int>(tr[0]);  // conversion to int as in the reference (cross_entropy.cpp:58)
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = t + i * TPR;
+    if (idx < nvec) {
+      RowIO<float, W>::template load<false>(xr + unsigned(W) * idx, v[i]);
+      if (!LABELS) RowIO<float, W>::template load<false>(tr + unsigned(W) * idx, xh[i]);
+    }
+    else {
+#pragma unroll
+      for (int k = 0; k < W; ++k) {
+        v[i][k] = -FLT_MAX;
+        if (!LABELS) xh[i][k] = 0.f;
+      }
+    }
+  }
+  float m = -FLT_MAX;
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+#pragma unroll
+    for (int k = 0; k < W; ++k) m = fmaxf(m, v[i][k]);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const bool ok = (t + i * TPR) < nvec;
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      const float e = ok ? exp_fast(v[i][k] - m) : 0.f;
+      s += e;
+      v[i][k] = e;
+    }
+  }
+  float gm = kSub ? row16_max(m) : wave_max(m);
+  float gs = kSub ? row16_sum(s * exp_fast(m - gm)) : wave_sum(s * exp_fast(m - gm));
+  if (NW > 1) {
+    if (lane == 0) {
+      red[0][wv] = gm;
+      red[1][wv] = gs;
+    }
+    __syncthreads();
+    const float pm = lane < NW ? red[0][lane] : -FLT_MAX;
+    const float ps = lane < NW ? red[1][lane] : 0.f;
+    gm = wave_max(pm);
+    gs = wave_sum(ps * exp_fast(pm - gm));
+  }
+  float* yr = y + row * ldy;
+  const float f = exp_fast(m - gm) * (1.0f / gs);
+  float part = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = t + i * TPR;
+    if (idx < nvec) {
+#pragma unroll
+      for (int k = 0; k < W; ++k) {
+        const float r = f * v[i][k];
+        v[i][k] = __builtin_isnormal(r) ? r : 0.f;
+        if (LABELS) {
+          if (static_cast<int>(W * idx + k) == label) part += -logf(v[i][k]);
+        }
+        else if (xh[i][k] > 0.f) {
+          part += -xh[i][k] * logf(v[i][k]);
+        }
+      }
+      RowIO<float, W>::store(yr + unsigned(W) * idx, v[i]);
+    }
+  }
+  part = kSub ? row16_sum(part) : team_sum<NW>(part, red_loss, wv, lane);
+  if (t == 0) loss[row * ld_loss] = part;
+}
+
 // softmax / channelwise: dx = y * (dy - dot(y, dy));  log-softmax: dx = dy - exp(y) * sum(dy)
 template <typename S, int TPR, int V, int KIND, int STREAM, int W = 16 / sizeof(S)>  // STREAM: bit 0 streams y, bit 1 dy
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
@@ -1242,6 +1344,34 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   }
 }
 
+// Softmax forward fused with the cross-entropy forward.  Returns -1 when the shape is not one
+// the fused kernel takes (the caller then runs the two layers' kernels one after the other).
+static int sm_ce_fwd_fused(hipStream_t st, int64_t n, int64_t w, int labels, const float* x, int64_t ldx,
+                           const float* truth, int64_t ldt, float* y, int64_t ldy, float* loss, int64_t ld_loss)
+{
+  const bool vec = (n % 4 == 0) && rows_aligned16(x, n, ldx, 1, w, 4) && rows_aligned16(y, n, ldy, 1, w, 4) &&
+                   (labels || rows_aligned16(truth, n, ldt, 1, w, 4));
+  if (!vec) return -1;
+  const RowConfig c = pick_sm_row_config(n / 4, w);
+  if (!c.tpr) return -1;
+  const unsigned nvec = static_cast<unsigned>(n / 4);
+#define X(TPR, V)                                                                                      \
+  if (c.tpr == TPR && c.v == V) {                                                                      \
+    using B = RowBlock<TPR>;                                                                           \
+    const unsigned grid = static_cast<unsigned>(ceil_div(w, B::kTeams));                               \
+    if (labels)                                                                                        \
+      hipLaunchKernelGGL((sm_ce_fwd_rows<TPR, V, true>), dim3(grid), dim3(B::kThreads), 0, st, x, truth, y, loss, \
+                         ldx, ldt, ldy, ld_loss, w, nvec);                                             \
+    else                                                                                               \
+      hipLaunchKernelGGL((sm_ce_fwd_rows<TPR, V, false>), dim3(grid), dim3(B::kThreads), 0, st, x, truth, y, loss, \
+                         ldx, ldt, ldy, ld_loss, w, nvec);                                             \
+    return launch_status();                                                                            \
+  }
+  LBN_ROW_CASES(X)
+#undef X
+  return -1;
+}
+
 // ------------------------------------------------------------ library-owned scratch
 // Scratch of the entry point that allocates nothing: one array per GPU, part of the code
 // object, so it exists from the moment the library is loaded until the process ends.  The
@@ -1329,6 +1459,43 @@ int lbn_log_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, 
                             void* workspace, size_t workspace_bytes)
 {
   return sm_bwd<kLogSoftmax>(as_stream(stream), 1, height, height, width, y, ldy, dy, lddy, dx, lddx, workspace, workspace_bytes);
+}
+
+size_t lbn_softmax_cross_entropy_fwd_workspace_bytes(int64_t height, int64_t width)
+{
+  // the cross-entropy partial sums sit past the header that the softmax kernels keep their wait status in
+  const size_t a = lbn_softmax_workspace_bytes(height, width);
+  const size_t b = lbn_cross_entropy_fwd_workspace_bytes(height, width);
+  return a > b + kWorkspaceHeaderBytes ? a : (b ? b + kWorkspaceHeaderBytes : a);
+}
+
+int lbn_softmax_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                                      int64_t spatial_size, const float* x, int64_t ldx, const float* ground_truth,
+                                      int64_t ld_truth, float* y, int64_t ldy, float* loss, int64_t ld_loss,
+                                      void* workspace, size_t workspace_bytes)
+{
+  hipStream_t st = as_stream(stream);
+  if (height < 0 || width < 0 || ld_loss < 0) return LBN_ERR_INVALID_ARGUMENT;
+  if (width == 0) return LBN_OK;
+  if (height == 0)  // no softmax output; the loss of an empty column is 0
+    return lbn_cross_entropy_fwd_f32(stream, height, width, use_labels, spatial_size, y, ldy, ground_truth, ld_truth,
+                                     loss, ld_loss, nullptr, 0);
+  if (!x || !ground_truth || !y || !loss || ld_loss < 1) return LBN_ERR_INVALID_ARGUMENT;
+  if (use_labels && spatial_size < 1) return LBN_ERR_INVALID_ARGUMENT;
+  if (width > 1 && (ldx < height || ldy < height || ld_truth < (use_labels ? 1 : height)))
+    return LBN_ERR_INVALID_ARGUMENT;
+  if (!use_labels || spatial_size == 1) {
+    const int r = sm_ce_fwd_fused(st, height, width, use_labels ? 1 : 0, x, ldx, ground_truth, ld_truth, y, ldy,
+                                  loss, ld_loss);
+    if (r >= 0) return r;
+  }
+  // shapes the fused kernel does not take: the two layers' kernels one after the other
+  const int status = sm_fwd<kSoftmax>(st, 1, height, height, width, x, ldx, y, ldy, workspace, workspace_bytes);
+  if (status != LBN_OK) return status;
+  const bool room = workspace && workspace_bytes > kWorkspaceHeaderBytes;
+  return lbn_cross_entropy_fwd_f32(stream, height, width, use_labels, spatial_size, y, ldy, ground_truth, ld_truth,
+                                   loss, ld_loss, room ? workspace_payload(workspace) : nullptr,
+                                   room ? workspace_bytes - kWorkspaceHeaderBytes : 0);
 }
 
 // fp16 storage (IEEE binary16 in memory, fp32 arithmetic); the workspace arguments are there for

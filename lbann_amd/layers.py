@@ -657,6 +657,28 @@ class cross_entropy_layer:
         return self.error_signals
 
 
+def softmax_cross_entropy_forward(softmax, cross_entropy, x, ground_truth):
+    """Forward of a softmax_layer whose only child is a cross_entropy_layer, in one call
+    (lbn_softmax_cross_entropy_fwd_f32): what softmax.forward(x) followed by
+    cross_entropy.forward(y, ground_truth) computes, with both layers' members bound as
+    those two calls bind them, so each layer's backward runs unchanged afterwards.
+    Returns (y, loss).  fp32 storage only."""
+    if x.dtype != torch.float32:
+        raise TypeError("softmax_cross_entropy_forward takes fp32 matrices")
+    softmax.bind_forward(x)
+    y = softmax.activations
+    cross_entropy.prev_activations = [y, ground_truth]
+    cross_entropy.activations = DeviceMatrix(1, x.width, device=cross_entropy.device)
+    loss = cross_entropy.activations
+    ws, nb = softmax._ws.get(capi.lib().lbn_softmax_cross_entropy_fwd_workspace_bytes(x.height, x.width), softmax.device)
+    call("lbn_softmax_cross_entropy_fwd_f32", _stream(), x.height, x.width, int(cross_entropy.m_use_labels),
+         cross_entropy.spatial_sample_size, x.Buffer(), x.ldim, ground_truth.Buffer(), ground_truth.ldim,
+         y.Buffer(), y.ldim, loss.Buffer(), loss.ldim, ws, nb)
+    if _CHECK_EVERY_CALL:
+        check_cluster_waits()
+    return y, loss
+
+
 class gradient_buffer:
     """The optimizer's gradient buffer as the layers see it: optimizer::add_to_gradient and
     get_gradient_buffer (include/lbann/optimizers/optimizer_impl.hpp:207-288) with their status

@@ -27,10 +27,10 @@ COPY_KIB = 262144.0  # the calibration copy reads and writes 256 MiB
 # (workload, algorithmic bytes per launch): forward 2 tensors, backward 3, of E elements
 _E2, _E3, _E4, _E5A, _E5B = 16777216, 51380224, 33554432, 67108864, 4194304
 WORKLOADS = [
-    ("sm_fwd_rows<1024, 8, 0", None, "cfg2 softmax fwd 32768x512", 2 * _E2 * 4),
-    ("sm_bwd_rows<1024, 8, 0", None, "cfg2 softmax bwd", 3 * _E2 * 4),
-    ("sm_fwd_rows<1024, 8, 1", None, "cfg2 log-softmax fwd", 2 * _E2 * 4),
-    ("sm_bwd_rows<1024, 8, 1", None, "cfg2 log-softmax bwd", 3 * _E2 * 4),
+    ("sm_fwd_rows<float, 1024, 8, 0", None, "cfg2 softmax fwd 32768x512", 2 * _E2 * 4),
+    ("sm_bwd_rows<float, 1024, 8, 0", None, "cfg2 softmax bwd", 3 * _E2 * 4),
+    ("sm_fwd_rows<float, 1024, 8, 1", None, "cfg2 log-softmax fwd", 2 * _E2 * 4),
+    ("sm_bwd_rows<float, 1024, 8, 1", None, "cfg2 log-softmax bwd", 3 * _E2 * 4),
     ("bn_fwd_cluster<float", None, "cfg3 batch norm fwd 64x256x56x56", 2 * _E3 * 4),
     ("bn_bwd_cluster<float", None, "cfg3 batch norm bwd", 3 * _E3 * 4),
     ("bn_fwd_cluster_ws<__half", None, "extra: batch norm fp16 storage fwd 64x256x56x56", 2 * _E3 * 2),
@@ -42,8 +42,8 @@ WORKLOADS = [
     ("bn_bwd_cluster<__half", None, "extra: batch norm fp16 storage bwd, barrier variant (forced)", 3 * _E3 * 2),
     ("ln_fwd_rows<__half", None, "cfg4 layer norm f16 fwd 4096x8192", 2 * _E4 * 2),
     ("ln_bwd_rows<__half", None, "cfg4 layer norm f16 bwd (followed by ln_wgrad_reduce)", 3 * _E4 * 2),
-    ("sm_fwd_rows<256, 4, 2", None, "cfg5a channelwise softmax fwd 256x64x4096", 2 * _E5A * 4),
-    ("sm_bwd_rows<256, 4, 2", None, "cfg5a channelwise softmax bwd", 3 * _E5A * 4),
+    ("sm_fwd_rows<float, 256, 4, 2", None, "cfg5a channelwise softmax fwd 256x64x4096", 2 * _E5A * 4),
+    ("sm_bwd_rows<float, 256, 4, 2", None, "cfg5a channelwise softmax bwd", 3 * _E5A * 4),
     ("sm_fwd_cluster<4, 0, 4>", 512, "cfg5b softmax 262144x16 fwd (8 clusters of 64, two rows each)", 2 * _E5B * 4),
     ("sm_bwd_cluster<4, 0, 4>", 512, "cfg5b softmax 262144x16 bwd", 3 * _E5B * 4),
     ("sm_fwd_partial", None, "cfg5b softmax 262144x16 fwd, split path, kernel 1 of 2", _E5B * 4),
@@ -65,6 +65,9 @@ WORKLOADS = [
     ("ln_bwd_cluster", None, "extra: layer norm over whole samples bwd (followed by ln_wgrad_reduce_wide)", 3 * _E3 * 4),
     ("ebn_fwd_tile", None, "extra: entry-wise batch norm fwd 1048576x64", 2 * 67108864 * 4),
     ("ebn_bwd_tile", None, "extra: entry-wise batch norm bwd", 3 * 67108864 * 4),
+    ("sm_fwd_rows<__half, 1024, 4, 0", None, "extra: softmax fp16 storage fwd 32768x512", 2 * _E2 * 2),
+    ("sm_bwd_rows<__half, 1024, 4, 0", None, "extra: softmax fp16 storage bwd", 3 * _E2 * 2),
+    ("sm_ce_fwd_rows<1024, 8, false>", None, "extra: softmax + cross entropy fwd 32768x512 (x, truth, y)", 3 * _E2 * 4),
     ("ce_fwd_dense", None, "extra: cross entropy fwd 32768x512 (x, truth)", 2 * _E2 * 4),
     ("ce_bwd_dense", None, "extra: cross entropy bwd (x, truth, dx, dtruth)", 4 * _E2 * 4),
     ("esb_fwd_tile", None, "extra: entry-wise scale/bias fwd 1048576x64", 2 * 67108864 * 4),
@@ -74,7 +77,7 @@ WORKLOADS = [
     ("grad_sink_quads<true>", None, "extra: gradient buffer, cleared: overwrite 4096x4096", 2 * _E2 * 4),
     ("grad_sink_quads<false>", None, "extra: gradient buffer, ready: accumulate 4096x4096", 3 * _E2 * 4),
 ]
-HEADLINE = "sm_bwd_rows<1024, 8, 0"
+HEADLINE = "sm_bwd_rows<float, 1024, 8, 0"
 
 
 def _short(name):
@@ -164,11 +167,11 @@ def trace(args):
             w = _lookup(write, name, wgs) * wfac / 1024
             row += f" {f:.1f} | {w:.1f} | " + (f"{(f + w) * 1048576 / nbytes:.2f} |" if nbytes else "|")
             if nbytes and HEADLINE in name:
-                headline = {"kernel": "sm_bwd_rows<1024,8,softmax> at 32768x512",
+                headline = {"kernel": "sm_bwd_rows<float,1024,8,softmax> at 32768x512",
                             "traffic_bytes_per_launch": (f + w) * 1048576, "fetch_factor": ffac, "write_factor": wfac,
                             "rocprof_avg_us": avg / 1e3}
         elif nbytes and HEADLINE in name:
-            headline = {"kernel": "sm_bwd_rows<1024,8,softmax> at 32768x512", "rocprof_avg_us": avg / 1e3}
+            headline = {"kernel": "sm_bwd_rows<float,1024,8,softmax> at 32768x512", "rocprof_avg_us": avg / 1e3}
         print(row)
     if args.headline_json and headline:
         with open(args.headline_json, "w") as f:

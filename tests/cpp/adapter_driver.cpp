@@ -277,6 +277,34 @@ int drv_cross_entropy(const int64_t* pred_dims, const int64_t* truth_dims, int n
   }
 }
 
+// softmax followed by cross entropy through the fused forward, then both layers' backward
+int drv_softmax_cross_entropy(const int64_t* pred_dims, const int64_t* truth_dims, int nd, int use_labels, int64_t h,
+                              int64_t ht, int64_t w, float* x, float* y, float* truth, float* loss, float* dloss,
+                              float* dy, float* dx, float* dtruth, void* stream, char* err, int errlen)
+{
+  try {
+    softmax_layer<> sm;
+    cross_entropy_layer<> ce(use_labels != 0);
+    ce.setup(std::vector<int64_t>(pred_dims, pred_dims + nd), std::vector<int64_t>(truth_dims, truth_dims + nd));
+    device_matrix<float> mx, my, mt, ml, mdl, mdy, mdx, mdt;
+    attach(mx, h, w, x, h); attach(my, h, w, y, h); attach(mt, ht, w, truth, ht); attach(ml, 1, w, loss, 1);
+    attach(mdl, 1, w, dloss, 1); attach(mdy, h, w, dy, h); attach(mdx, h, w, dx, h); attach(mdt, ht, w, dtruth, ht);
+    sm.io.prev_activations = &mx; sm.io.activations = &my; sm.io.prev_error_signals = &mdy; sm.io.error_signals = &mdx;
+    ce.io.prev_activations = &my; ce.prev_ground_truth = &mt; ce.io.activations = &ml;
+    ce.io.prev_error_signals = &mdl; ce.io.error_signals = &mdy; ce.ground_truth_error_signals = &mdt;
+    sm.io.stream = ce.io.stream = static_cast<hipStream_t>(stream);
+    ce.fp_compute_with(sm);
+    ce.bp_compute();
+    sm.bp_compute();
+    sm.check_cluster_waits();
+    check_hip(hipStreamSynchronize(sm.io.stream), "sync");
+    return 0;
+  }
+  catch (const std::exception& e) {
+    return fail(e, err, errlen);
+  }
+}
+
 // kind: 0 entry-wise, 1 channel-wise.  weights: (n x 2) column-major, n = h resp. dims[0].
 int drv_scale_bias(int kind, const int64_t* dims, int nd, int64_t h, int64_t w, int64_t ld, float* x, float* y,
                    float* dy, float* dx, const float* weights, int64_t ld_weights, float* wgrad_out,

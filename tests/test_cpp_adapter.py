@@ -206,6 +206,31 @@ def test_adapter_layers_match_oracle():
         else:
             check("adapter cross entropy dtruth", mdt.to_numpy(), dt_ref)
 
+    # ---- softmax -> cross entropy through the fused forward: (1000,) dense (one kernel), (3, 8, 8) labels (two)
+    for use_labels, pdims, tdims in ((0, (1000,), (1000,)), (1, (3, 8, 8), (1, 8, 8))):
+        h, w = int(np.prod(pdims)), 20
+        x = mk(h, w, 0.0, 2.0)
+        if use_labels:
+            truth = np.asfortranarray(rng.integers(0, 3, (w, 64)).astype(np.float32).T)
+        else:
+            truth = np.asfortranarray(rng.uniform(-0.2, 1.0, (w, h)).astype(np.float32).T)
+        dloss = rng.standard_normal(w).astype(np.float32)
+        mx, my, mt = DeviceMatrix.from_numpy(x), DeviceMatrix(h, w), DeviceMatrix.from_numpy(truth)
+        ml, mdl = DeviceMatrix(1, w), DeviceMatrix.from_numpy(dloss.reshape(1, -1))
+        mdy, mdx, mdt = DeviceMatrix(h, w), DeviceMatrix(h, w), DeviceMatrix(truth.shape[0], w)
+        pa, nd = _dims(pdims)
+        ta, _ = _dims(tdims)
+        rc = d.drv_softmax_cross_entropy(pa, ta, cint(nd), cint(use_labels), i64(h), i64(truth.shape[0]), i64(w),
+                                         mx.Buffer(), my.Buffer(), mt.Buffer(), ml.Buffer(), mdl.Buffer(), mdy.Buffer(),
+                                         mdx.Buffer(), mdt.Buffer(), st, err, cint(512))
+        assert rc == 0, err.value
+        y_ref = orc.softmax_fwd(x)
+        check("adapter softmax+ce y", my.to_numpy(), y_ref)
+        check("adapter softmax+ce loss", ml.to_numpy()[0], orc.cross_entropy_fwd(y_ref, truth, bool(use_labels)))
+        dp_ref, _ = orc.cross_entropy_bwd(y_ref, truth, dloss, bool(use_labels))
+        check("adapter softmax+ce dprediction", mdy.to_numpy(), dp_ref)
+        check("adapter softmax+ce dx", mdx.to_numpy(), orc.softmax_bwd(y_ref, dp_ref))
+
     # ---- scale/bias layers on (8, 12, 12) x 10
     dims, w = (8, 12, 12), 10
     h = 8 * 144
