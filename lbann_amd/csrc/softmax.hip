@@ -89,13 +89,58 @@ struct RowLoad {
   static __device__ __forceinline__ void put(S* p, float r) { const float v[1] = {r}; RowIO<S, 1>::store(p, v); }
 };
 
+// Framed access: a row that starts off the 16-byte grid, addressed on it.  The frame begins at
+// the 16-byte boundary at or below the row's first entry, `shift` (0..3) entries earlier;
+// vector idx of the frame holds the row's entries 4 idx - shift ... 4 idx + 3 - shift.  Vectors
+// that lie inside the row move as 16 bytes; the first and the last move entry by entry, and
+// what lies outside the row is neither read nor written.  Every tensor of a call must have the
+// same shift in every row (same_frames() on the host).
+struct RowFrame {
+  unsigned shift;
+  unsigned nvec;  // vectors of the frame that hold entries of the row
+};
+
+__device__ __forceinline__ RowFrame row_frame(const float* rowp, unsigned n)
+{
+  const unsigned shift = (static_cast<unsigned>(reinterpret_cast<uintptr_t>(rowp)) >> 2) & 3u;
+  return {shift, (shift + n + 3u) >> 2};
+}
+
+__device__ __forceinline__ void frame_load(const float* framep, unsigned idx, RowFrame fr, unsigned n, float fill,
+                                           float (&v)[4])
+{
+  const unsigned e0 = 4u * idx;
+  if (e0 >= fr.shift && e0 + 4u <= fr.shift + n) {
+    Vec16<float>::load(framep + e0, v);
+  }
+  else {
+#pragma unroll
+    for (unsigned j = 0; j < 4; ++j) v[j] = (e0 + j >= fr.shift && e0 + j < fr.shift + n) ? framep[e0 + j] : fill;
+  }
+}
+
+__device__ __forceinline__ void frame_store(float* framep, unsigned idx, RowFrame fr, unsigned n, const float (&v)[4])
+{
+  const unsigned e0 = 4u * idx;
+  if (e0 >= fr.shift && e0 + 4u <= fr.shift + n) {
+    Vec16<float>::store(framep + e0, v);
+  }
+  else {
+#pragma unroll
+    for (unsigned j = 0; j < 4; ++j)
+      if (e0 + j >= fr.shift && e0 + j < fr.shift + n) framep[e0 + j] = v[j];
+  }
+}
+
 // 1024-thread blocks are held to 64 registers so that two of them share a compute unit
 // (not those with 32 accesses or more than 32 values per thread, which would spill).
-template <typename S, int TPR, int V, int KIND, bool STREAM, int W = 16 / sizeof(S)>
+// FR (fp32): framed access for rows off the 16-byte grid; `nvec` is then the row length in entries.
+template <typename S, int TPR, int V, int KIND, bool STREAM, int W = 16 / sizeof(S), bool FR = false>
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads, (TPR == 1024 && V <= 16 && V * W <= 32 ? 8 : 1))
 sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
             unsigned nvec)
 {
+  static_assert(!FR || (std::is_same<S, float>::value && W == 4), "frames are made of 16-byte fp32 vectors");
   using B = RowBlock<TPR>;
   constexpr bool kSub = TPR < kWave;  // short rows: 16 lanes own a row, four rows per wave
   static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
@@ -111,12 +156,20 @@ sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows
   if (B::kTeams > 1 && row >= rows) return;  // whole waves leave; no barrier below in that case
 
   const S* xr = x + map.offset(row, ldx);
+  const unsigned n = nvec;
+  RowFrame fr{0, nvec};
+  if constexpr (FR) {
+    fr = row_frame(xr, n);
+    xr -= fr.shift;
+    nvec = fr.nvec;
+  }
   float v[V][W];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      RowIO<S, W>::template load<STREAM>(xr + unsigned(W) * idx, v[i]);
+      if constexpr (FR) frame_load(xr, idx, fr, n, -FLT_MAX, v[i]);
+      else RowIO<S, W>::template load<STREAM>(xr + unsigned(W) * idx, v[i]);
     }
     else {
 #pragma unroll
@@ -167,6 +220,7 @@ sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows
   }
 
   S* yr = y + map.offset(row, ldy);
+  if constexpr (FR) yr -= fr.shift;  // the same frames as x (same_frames() on the host)
   const float shift = m - gm;  // <= 0
   const float f = exp_fast(shift) * (1.0f / gs);
   const float lse = (KIND == kLogSoftmax) ? log_of_sum(gs) : 0.f;
@@ -187,7 +241,8 @@ sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows
           v[i][k] *= f;
         }
       }
-      RowIO<S, W>::store(yr + unsigned(W) * idx, v[i]);
+      if constexpr (FR) frame_store(yr, idx, fr, n, v[i]);
+      else RowIO<S, W>::store(yr + unsigned(W) * idx, v[i]);
     }
   }
 }
@@ -295,11 +350,13 @@ sm_ce_fwd_rows(const float* x, const float* truth, float* y, float* loss, int64_
 }
 
 // softmax / channelwise: dx = y * (dy - dot(y, dy));  log-softmax: dx = dy - exp(y) * sum(dy)
-template <typename S, int TPR, int V, int KIND, int STREAM, int W = 16 / sizeof(S)>  // STREAM: bit 0 streams y, bit 1 dy
+// STREAM: bit 0 streams y, bit 1 dy.  FR as in sm_fwd_rows.
+template <typename S, int TPR, int V, int KIND, int STREAM, int W = 16 / sizeof(S), bool FR = false>
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
 sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx,
             RowMap map, int64_t rows, unsigned nvec)
 {
+  static_assert(!FR || (std::is_same<S, float>::value && W == 4), "frames are made of 16-byte fp32 vectors");
   using B = RowBlock<TPR>;
   constexpr bool kSub = TPR < kWave;
   static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
@@ -315,13 +372,27 @@ sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t l
 
   const S* yr = y + map.offset(row, ldy);
   const S* gr = dy + map.offset(row, lddy);
+  const unsigned n = nvec;
+  RowFrame fr{0, nvec};
+  if constexpr (FR) {
+    fr = row_frame(yr, n);
+    yr -= fr.shift;
+    gr -= fr.shift;
+    nvec = fr.nvec;
+  }
   float a[V][W], g[V][W];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
-      RowIO<S, W>::template load<(STREAM & 1) != 0>(yr + unsigned(W) * idx, a[i]);
-      RowIO<S, W>::template load<(STREAM & 2) != 0>(gr + unsigned(W) * idx, g[i]);
+      if constexpr (FR) {
+        frame_load(yr, idx, fr, n, 0.f, a[i]);
+        frame_load(gr, idx, fr, n, 0.f, g[i]);
+      }
+      else {
+        RowIO<S, W>::template load<(STREAM & 1) != 0>(yr + unsigned(W) * idx, a[i]);
+        RowIO<S, W>::template load<(STREAM & 2) != 0>(gr + unsigned(W) * idx, g[i]);
+      }
     }
     else {
 #pragma unroll
@@ -336,6 +407,7 @@ sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t l
   s = kSub ? row16_sum(s) : team_sum<NW>(s, red, wv, lane);
 
   S* dr = dx + map.offset(row, lddx);
+  if constexpr (FR) dr -= fr.shift;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
@@ -345,7 +417,8 @@ sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t l
         if (KIND == kLogSoftmax) g[i][k] = g[i][k] - exp_fast(a[i][k]) * s;
         else g[i][k] = a[i][k] * (g[i][k] - s);
       }
-      RowIO<S, W>::store(dr + unsigned(W) * idx, g[i]);
+      if constexpr (FR) frame_store(dr, idx, fr, n, g[i]);
+      else RowIO<S, W>::store(dr + unsigned(W) * idx, g[i]);
     }
   }
 }
@@ -375,10 +448,17 @@ struct SmClusterArgs {
   RowMap map;
   int64_t rows;
   unsigned nvec;
+  unsigned n;  // framed access: entries per row (nvec is then the largest frame)
   int M;
   ClusterWorkspace cw;
   ClusterTag tag;
   __device__ __forceinline__ unsigned long long* slots(int64_t row) const { return cw.slots + row * M * 2; }
+  // vectors of row `row` (every tensor has the same frames)
+  template <bool FR>
+  __device__ __forceinline__ unsigned row_nvec(int64_t row) const
+  {
+    return FR ? row_frame(a + map.offset(row, lda), n).nvec : nvec;
+  }
 };
 
 template <int V, int W = 4>
@@ -387,15 +467,23 @@ struct SmFwdTile {
   float m;  // the thread's own maximum: v holds exp(x - m) (or x - m for log-softmax)
 };
 
-template <int V, int W>
+template <int V, int W, bool FR = false>
 __device__ __forceinline__ void sm_cl_load(float (&t)[V][W], const float* rowp, unsigned base,
-                                           unsigned nvec, float fill)
+                                           unsigned nvec, float fill, unsigned n = 0)
 {
+  static_assert(!FR || W == 4, "frames are made of 16-byte vectors");
+  RowFrame fr{0, 0};
+  if constexpr (FR) {
+    fr = row_frame(rowp, n);
+    rowp -= fr.shift;
+    nvec = fr.nvec;
+  }
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = base + i * kClusterThreads;
     if (idx < nvec) {
-      RowIO<float, W>::template load<false>(rowp + W * static_cast<int64_t>(idx), t[i]);
+      if constexpr (FR) frame_load(rowp, idx, fr, n, fill, t[i]);
+      else RowIO<float, W>::template load<false>(rowp + W * static_cast<int64_t>(idx), t[i]);
     }
     else {
 #pragma unroll
@@ -411,10 +499,11 @@ __device__ __forceinline__ void sm_cl_load(float (&t)[V][W], const float* rowp, 
 // forward 137 against 87 us).
 // (1) of a step: thread-local online softmax, one merge of the (max, sum) pairs of the
 // workgroup, published for the cluster.
-template <int V, int KIND, int W = 4>
+template <int V, int KIND, int W = 4, bool FR = false>
 __device__ __forceinline__ void sm_cl_fwd_reduce(const SmClusterArgs& a, int64_t row, int k, unsigned base,
                                                  SmFwdTile<V, W>& t, float (*red)[2])
 {
+  const unsigned nvec = a.row_nvec<FR>(row);
   float m = -FLT_MAX;
 #pragma unroll
   for (int i = 0; i < V; ++i)
@@ -423,10 +512,11 @@ __device__ __forceinline__ void sm_cl_fwd_reduce(const SmClusterArgs& a, int64_t
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    const bool ok = base + i * kClusterThreads < a.nvec;
+    const bool ok = base + i * kClusterThreads < nvec;
 #pragma unroll
     for (int j = 0; j < W; ++j) {
       const float d = t.v[i][j] - m;
+      // (the entries of a frame's end vectors that lie outside the row hold -FLT_MAX: exp gives 0)
       const float e = ok ? (KIND == kChannelwise ? exp_keep_denormals(d) : exp_fast(d)) : 0.f;
       s += e;
       t.v[i][j] = (KIND == kLogSoftmax) ? d : e;
@@ -438,7 +528,7 @@ __device__ __forceinline__ void sm_cl_fwd_reduce(const SmClusterArgs& a, int64_t
 }
 
 // (3) of a step.
-template <int V, int KIND, int W = 4>
+template <int V, int KIND, int W = 4, bool FR = false>
 __device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t row, unsigned base,
                                                  SmFwdTile<V, W>& t, float* bc)
 {
@@ -456,13 +546,18 @@ __device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t
   const float gm = bc[0];
   const float gs = bc[1];
   float* yr = a.out + a.map.offset(row, a.ldo);
+  RowFrame fr{0, a.nvec};
+  if constexpr (FR) {
+    fr = row_frame(yr, a.n);
+    yr -= fr.shift;
+  }
   const float shift = t.m - gm;                     // <= 0: this thread's maximum against the row's
   const float f = exp_fast(shift) * (1.0f / gs);    // rescales exp(x - m) to exp(x - gm) / sum
   const float lse = (KIND == kLogSoftmax) ? log_of_sum(gs) : 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = base + i * kClusterThreads;
-    if (idx < a.nvec) {
+    if (idx < fr.nvec) {
 #pragma unroll
       for (int j = 0; j < W; ++j) {
         if (KIND == kSoftmax) {
@@ -476,24 +571,25 @@ __device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t
           t.v[i][j] *= f;
         }
       }
-      RowIO<float, W>::store(yr + W * static_cast<int64_t>(idx), t.v[i]);
+      if constexpr (FR) frame_store(yr, idx, fr, a.n, t.v[i]);
+      else RowIO<float, W>::store(yr + W * static_cast<int64_t>(idx), t.v[i]);
     }
   }
 }
 
-template <int V, int KIND, int W = 4>
+template <int V, int KIND, int W = 4, bool FR = false>
 __device__ __forceinline__ void sm_cl_fwd_step(const SmClusterArgs& a, int64_t row, int64_t nc, int k,
                                                unsigned base, SmFwdTile<V, W>& F, SmFwdTile<V, W>& R,
                                                SmFwdTile<V, W>& L, float (*red)[2], float* bc)
 {
-  if (row + nc < a.rows) sm_cl_fwd_reduce<V, KIND, W>(a, row + nc, k, base, R, red);
+  if (row + nc < a.rows) sm_cl_fwd_reduce<V, KIND, W, FR>(a, row + nc, k, base, R, red);
   if (row + 2 * nc < a.rows)
-    sm_cl_load<V, W>(L.v, a.a + a.map.offset(row + 2 * nc, a.lda), base, a.nvec, -FLT_MAX);
+    sm_cl_load<V, W, FR>(L.v, a.a + a.map.offset(row + 2 * nc, a.lda), base, a.nvec, -FLT_MAX, a.n);
   asm volatile("" ::: "memory");  // keep the loads above the wait below
-  sm_cl_fwd_finish<V, KIND, W>(a, row, base, F, bc);
+  sm_cl_fwd_finish<V, KIND, W, FR>(a, row, base, F, bc);
 }
 
-template <int V, int KIND, int W = 4>
+template <int V, int KIND, int W = 4, bool FR = false>
 __global__ void __launch_bounds__(kClusterThreads)
 sm_fwd_cluster(SmClusterArgs a)
 {
@@ -506,16 +602,16 @@ sm_fwd_cluster(SmClusterArgs a)
   if (cl >= a.rows) return;
   cluster_resolve_tag(a.tag);
   SmFwdTile<V, W> t0, t1, t2;
-  sm_cl_load<V, W>(t0.v, a.a + a.map.offset(cl, a.lda), base, a.nvec, -FLT_MAX);
-  if (cl + nc < a.rows) sm_cl_load<V, W>(t1.v, a.a + a.map.offset(cl + nc, a.lda), base, a.nvec, -FLT_MAX);
-  sm_cl_fwd_reduce<V, KIND, W>(a, cl, k, base, t0, red);
+  sm_cl_load<V, W, FR>(t0.v, a.a + a.map.offset(cl, a.lda), base, a.nvec, -FLT_MAX, a.n);
+  if (cl + nc < a.rows) sm_cl_load<V, W, FR>(t1.v, a.a + a.map.offset(cl + nc, a.lda), base, a.nvec, -FLT_MAX, a.n);
+  sm_cl_fwd_reduce<V, KIND, W, FR>(a, cl, k, base, t0, red);
   __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
   // Each position of the rotation has its own broadcast slot: a step without a reduction has
   // no barrier between the reads of one finish and the write of the next.
   for (int64_t row = cl; row < a.rows; row += 3 * nc) {
-    sm_cl_fwd_step<V, KIND, W>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
-    if (row + nc < a.rows) sm_cl_fwd_step<V, KIND, W>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
-    if (row + 2 * nc < a.rows) sm_cl_fwd_step<V, KIND, W>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
+    sm_cl_fwd_step<V, KIND, W, FR>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
+    if (row + nc < a.rows) sm_cl_fwd_step<V, KIND, W, FR>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
+    if (row + 2 * nc < a.rows) sm_cl_fwd_step<V, KIND, W, FR>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
   }
 }
 
@@ -538,7 +634,7 @@ __device__ __forceinline__ void sm_cl_bwd_reduce(const SmClusterArgs& a, int64_t
   if (threadIdx.x == 0) cluster_publish(s, 0.f, a.slots(row), k, a.tag);
 }
 
-template <int V, int KIND, int W = 4>
+template <int V, int KIND, int W = 4, bool FR = false>
 __device__ __forceinline__ void sm_cl_bwd_finish(const SmClusterArgs& a, int64_t row, unsigned base,
                                                  SmBwdTile<V, W>& t, float* bc)
 {
@@ -551,40 +647,46 @@ __device__ __forceinline__ void sm_cl_bwd_finish(const SmClusterArgs& a, int64_t
   __syncthreads();
   const float tot = bc[0];
   float* dr = a.out + a.map.offset(row, a.ldo);
+  RowFrame fr{0, a.nvec};
+  if constexpr (FR) {
+    fr = row_frame(dr, a.n);
+    dr -= fr.shift;
+  }
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = base + i * kClusterThreads;
-    if (idx < a.nvec) {
+    if (idx < fr.nvec) {
 #pragma unroll
       for (int j = 0; j < W; ++j) {
         if (KIND == kLogSoftmax) t.g[i][j] = t.g[i][j] - exp_fast(t.a[i][j]) * tot;
         else t.g[i][j] = t.a[i][j] * (t.g[i][j] - tot);
       }
-      RowIO<float, W>::store(dr + W * static_cast<int64_t>(idx), t.g[i]);
+      if constexpr (FR) frame_store(dr, idx, fr, a.n, t.g[i]);
+      else RowIO<float, W>::store(dr + W * static_cast<int64_t>(idx), t.g[i]);
     }
   }
 }
 
-template <int V, int W>
+template <int V, int W, bool FR = false>
 __device__ __forceinline__ void sm_cl_bwd_load(const SmClusterArgs& a, int64_t row, unsigned base,
                                                SmBwdTile<V, W>& t)
 {
-  sm_cl_load<V, W>(t.a, a.a + a.map.offset(row, a.lda), base, a.nvec, 0.f);
-  sm_cl_load<V, W>(t.g, a.g + a.map.offset(row, a.ldg), base, a.nvec, 0.f);
+  sm_cl_load<V, W, FR>(t.a, a.a + a.map.offset(row, a.lda), base, a.nvec, 0.f, a.n);
+  sm_cl_load<V, W, FR>(t.g, a.g + a.map.offset(row, a.ldg), base, a.nvec, 0.f, a.n);
 }
 
-template <int V, int KIND, int W = 4>
+template <int V, int KIND, int W = 4, bool FR = false>
 __device__ __forceinline__ void sm_cl_bwd_step(const SmClusterArgs& a, int64_t row, int64_t nc, int k,
                                                unsigned base, SmBwdTile<V, W>& F, SmBwdTile<V, W>& R,
                                                SmBwdTile<V, W>& L, float* red, float* bc)
 {
   if (row + nc < a.rows) sm_cl_bwd_reduce<V, KIND, W>(a, row + nc, k, R, red);
-  if (row + 2 * nc < a.rows) sm_cl_bwd_load<V, W>(a, row + 2 * nc, base, L);
+  if (row + 2 * nc < a.rows) sm_cl_bwd_load<V, W, FR>(a, row + 2 * nc, base, L);
   asm volatile("" ::: "memory");
-  sm_cl_bwd_finish<V, KIND, W>(a, row, base, F, bc);
+  sm_cl_bwd_finish<V, KIND, W, FR>(a, row, base, F, bc);
 }
 
-template <int V, int KIND, int W = 4>
+template <int V, int KIND, int W = 4, bool FR = false>
 __global__ void __launch_bounds__(kClusterThreads)
 sm_bwd_cluster(SmClusterArgs a)
 {
@@ -597,16 +699,16 @@ sm_bwd_cluster(SmClusterArgs a)
   if (cl >= a.rows) return;
   cluster_resolve_tag(a.tag);
   SmBwdTile<V, W> t0, t1, t2;
-  sm_cl_bwd_load<V, W>(a, cl, base, t0);
-  if (cl + nc < a.rows) sm_cl_bwd_load<V, W>(a, cl + nc, base, t1);
+  sm_cl_bwd_load<V, W, FR>(a, cl, base, t0);
+  if (cl + nc < a.rows) sm_cl_bwd_load<V, W, FR>(a, cl + nc, base, t1);
   sm_cl_bwd_reduce<V, KIND, W>(a, cl, k, t0, red);
   __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
   // Each position of the rotation has its own broadcast slot: a step without a reduction has
   // no barrier between the reads of one finish and the write of the next.
   for (int64_t row = cl; row < a.rows; row += 3 * nc) {
-    sm_cl_bwd_step<V, KIND, W>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
-    if (row + nc < a.rows) sm_cl_bwd_step<V, KIND, W>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
-    if (row + 2 * nc < a.rows) sm_cl_bwd_step<V, KIND, W>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
+    sm_cl_bwd_step<V, KIND, W, FR>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
+    if (row + nc < a.rows) sm_cl_bwd_step<V, KIND, W, FR>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
+    if (row + 2 * nc < a.rows) sm_cl_bwd_step<V, KIND, W, FR>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
   }
 }
 
@@ -1079,47 +1181,66 @@ static int64_t cluster_count(int64_t rows, int64_t fit, int M)
 // Launch of the cluster kernels for rows of `units` accesses of W floats each.  Returns -1 when
 // the plan or the device's capacity does not allow it (the caller goes on to the split
 // kernels), otherwise the call's status.
-template <int KIND, int W>
+// Framed access needs every tensor of the call to start each row at the same distance from a
+// 16-byte boundary: the base pointers agree modulo 16 bytes and, with more than one column,
+// so do the leading dimensions modulo 4 entries (the row stride inside a column is shared).
+static bool same_frames(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t w)
+{
+  const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+  return (pa & 3u) == 0 && ((pa ^ pb) & 15u) == 0 && (w <= 1 || ((lda - ldb) & 3) == 0);
+}
+
+static bool framed_access()
+{
+  static const bool off = std::getenv("LBN_NO_FRAMED_ACCESS") != nullptr;
+  return !off;
+}
+
+// FR: framed access (rows off the 16-byte grid moved as 16-byte vectors); `units` is then the
+// largest frame, (n + 3 + 3) / 4 vectors, and `n` the row length.
+template <int KIND, int W, bool FR = false>
 static int sm_fwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, int64_t rows, const float* x,
-                                 int64_t ldx, float* y, int64_t ldy, RowMap map, void* ws, size_t ws_bytes)
+                                 int64_t ldx, float* y, int64_t ldy, RowMap map, void* ws, size_t ws_bytes,
+                                 unsigned n = 0)
 {
   if (!cp.M) return -1;
   if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
   const ClusterWorkspace cw = cluster_workspace(ws);
 #define X(VV)                                                                                    \
   if (cp.V == VV) {                                                                              \
-    const int cap = cluster_capacity(sm_fwd_cluster<VV, KIND, W>, kClusterThreads);              \
+    const int cap = cluster_capacity(sm_fwd_cluster<VV, KIND, W, FR>, kClusterThreads);          \
     int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
     if (ncl < 1) return -1;                                                                      \
     ncl = cluster_count(rows, ncl, cp.M);                                                        \
     const SmClusterArgs a{x, nullptr, y, ldx, 0, ldy, map, rows, static_cast<unsigned>(units),   \
-                          cp.M, cw, cluster_call_tag(st, cw)};                                   \
-    hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND, W>), dim3(static_cast<unsigned>(ncl * cp.M)),   \
+                          n, cp.M, cw, cluster_call_tag(st, cw)};                                \
+    hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND, W, FR>), dim3(static_cast<unsigned>(ncl * cp.M)), \
                        dim3(kClusterThreads), 0, st, a);                                         \
     return launch_status();                                                                      \
   }
-  X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8)
+  X(1) X(2) X(3) X(4)
+  if constexpr (!FR) { X(5) X(6) X(7) X(8) }
 #undef X
   return -1;
 }
 
-template <int KIND, int W>
+template <int KIND, int W, bool FR = false>
 static int sm_bwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, int64_t rows, const float* y,
                                  int64_t ldy, const float* dy, int64_t lddy, float* dx, int64_t lddx, RowMap map,
-                                 void* ws, size_t ws_bytes)
+                                 void* ws, size_t ws_bytes, unsigned n = 0)
 {
   if (!cp.M) return -1;
   if (!ws || ws_bytes < cluster_workspace_bytes(rows) || !aligned16(ws)) return LBN_ERR_WORKSPACE;
   const ClusterWorkspace cw = cluster_workspace(ws);
 #define X(VV)                                                                                    \
   if (cp.V == VV) {                                                                              \
-    const int cap = cluster_capacity(sm_bwd_cluster<VV, KIND, W>, kClusterThreads);              \
+    const int cap = cluster_capacity(sm_bwd_cluster<VV, KIND, W, FR>, kClusterThreads);          \
     int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
     if (ncl < 1) return -1;                                                                      \
     ncl = cluster_count(rows, ncl, cp.M);                                                        \
     const SmClusterArgs a{y, dy, dx, ldy, lddy, lddx, map, rows, static_cast<unsigned>(units),   \
-                          cp.M, cw, cluster_call_tag(st, cw)};                                   \
-    hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND, W>), dim3(static_cast<unsigned>(ncl * cp.M)),   \
+                          n, cp.M, cw, cluster_call_tag(st, cw)};                                \
+    hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND, W, FR>), dim3(static_cast<unsigned>(ncl * cp.M)), \
                        dim3(kClusterThreads), 0, st, a);                                         \
     return launch_status();                                                                      \
   }
@@ -1132,6 +1253,67 @@ static int sm_bwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, 
 #define LBN_ROW_CASES(X)                                                                     \
   X(16, 1) X(16, 2) X(16, 4) X(64, 1) X(64, 2) X(64, 4) X(64, 8) X(256, 1) X(256, 2) X(256, 4) X(256, 8) X(1024, 1)      \
   X(1024, 2) X(1024, 4) X(1024, 8)
+
+// Rows off the 16-byte grid that fit a workgroup's registers as a frame of 16-byte vectors
+// (fp32 only).  False: not launched, the caller goes on to the one-float-per-access kernels.
+// Measured, us per step framed / one float per access: 197 x 151296: 126 / 105; 1001 x 16384:
+// 55 / 56; 4099 x 8192: 134 / 132; 8191 x 4096: 121 / 125; 16385 x 4096: 253 / 267;
+// 30522 x 2048: 233 / 248.  The two end vectors of a row cost more than the wider accesses
+// save until a row has a few thousand entries.
+constexpr int64_t kFramedMinRow = 8000;
+
+template <int KIND, typename S>
+static bool sm_fwd_framed_rows(hipStream_t st, int64_t n, int64_t w, int64_t rows, const S* x, int64_t ldx, S* y,
+                               int64_t ldy, RowMap map)
+{
+  if constexpr (!std::is_same<S, float>::value) {
+    return false;
+  }
+  else {
+    if (!framed_access() || n < kFramedMinRow || !same_frames(x, ldx, y, ldy, w)) return false;
+    const RowConfig c = pick_sm_row_config((n + 6) / 4, rows);
+    if (!c.tpr) return false;
+#define X(TPR, V)                                                                                      \
+  if (c.tpr == TPR && c.v == V) {                                                                      \
+    using B = RowBlock<TPR>;                                                                           \
+    const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                            \
+    hipLaunchKernelGGL((sm_fwd_rows<float, TPR, V, KIND, false, 4, true>), dim3(grid), dim3(B::kThreads), 0, st, \
+                       x, y, ldx, ldy, map, rows, static_cast<unsigned>(n));                           \
+    return true;                                                                                       \
+  }
+    LBN_ROW_CASES(X)
+#undef X
+    return false;
+  }
+}
+
+template <int KIND, typename S>
+static bool sm_bwd_framed_rows(hipStream_t st, int64_t n, int64_t w, int64_t rows, const S* y, int64_t ldy,
+                               const S* dy, int64_t lddy, S* dx, int64_t lddx, RowMap map)
+{
+  if constexpr (!std::is_same<S, float>::value) {
+    return false;
+  }
+  else {
+    if (!framed_access() || n < kFramedMinRow || !same_frames(y, ldy, dy, lddy, w) ||
+        !same_frames(y, ldy, dx, lddx, w))
+      return false;
+    const RowConfig c = pick_sm_row_config((n + 6) / 4, rows);
+    if (!c.tpr) return false;
+#define X(TPR, V)                                                                                      \
+  if constexpr (!(TPR == 1024 && V > 8)) /* two tensors of more would not fit 128 registers */         \
+  if (c.tpr == TPR && c.v == V) {                                                                      \
+    using B = RowBlock<TPR>;                                                                           \
+    const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                            \
+    hipLaunchKernelGGL((sm_bwd_rows<float, TPR, V, KIND, 0, 4, true>), dim3(grid), dim3(B::kThreads), 0, st, \
+                       y, dy, dx, ldy, lddy, lddx, map, rows, static_cast<unsigned>(n));               \
+    return true;                                                                                       \
+  }
+    LBN_ROW_CASES(X)
+#undef X
+    return false;
+  }
+}
 
 template <int KIND, typename S = float>
 static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int64_t w,
@@ -1167,6 +1349,9 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
       LBN_ROW_CASES(X)
 #undef X
     }
+  }
+  else if (sm_fwd_framed_rows<KIND>(st, n, w, rows, x, ldx, y, ldy, map)) {
+    return launch_status();
   }
   else if (n <= kMaxScalarRow) {
     // rows that are only 4-byte aligned and short enough for registers: one float per access
@@ -1213,8 +1398,15 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
         r = sm_fwd_cluster_launch<KIND, 4>(st, cp, n / 4, rows, x, ldx, y, ldy, map, ws, ws_bytes);
       }
       else if (!vec) {
-        // rows off the 16-byte grid (a vocabulary of 50257 entries): the same kernel, one float per access
-        r = sm_fwd_cluster_launch<KIND, 1>(st, plan_cluster(n, 8), n, rows, x, ldx, y, ldy, map, ws, ws_bytes);
+        // rows off the 16-byte grid (a vocabulary of 50257 entries): framed 16-byte access when both
+        // tensors sit on the grid alike, else the same kernel with one float per access.  50257 x 1024,
+        // us per step framed / one float per access: softmax 210 / 220, log-softmax 209 / 254
+        const int64_t frame = (n + 6) / 4;
+        if (framed_access() && same_frames(x, ldx, y, ldy, w) && n < (int64_t(1) << 31))
+          r = sm_fwd_cluster_launch<KIND, 4, true>(st, plan_cluster(frame, 4), frame, rows, x, ldx, y, ldy, map, ws,
+                                                   ws_bytes, static_cast<unsigned>(n));
+        if (r < 0)
+          r = sm_fwd_cluster_launch<KIND, 1>(st, plan_cluster(n, 8), n, rows, x, ldx, y, ldy, map, ws, ws_bytes);
       }
       if (r >= 0) return r;
     }
@@ -1282,6 +1474,9 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
 #undef X
     }
   }
+  else if (sm_bwd_framed_rows<KIND>(st, n, w, rows, y, ldy, dy, lddy, dx, lddx, map)) {
+    return launch_status();
+  }
   else if (n <= kMaxScalarRow) {
     const RowConfig c = pick_sm_row_config(n, rows);
     if (c.tpr) {
@@ -1322,9 +1517,16 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
       if (vec && n / 4 < (int64_t(1) << 30))
         r = sm_bwd_cluster_launch<KIND, 4>(st, plan_cluster(n / 4, 4), n / 4, rows, y, ldy, dy, lddy, dx, lddx, map, ws,
                                            ws_bytes);
-      else if (!vec)
-        r = sm_bwd_cluster_launch<KIND, 1>(st, plan_cluster(n, 8), n, rows, y, ldy, dy, lddy, dx, lddx, map, ws,
-                                           ws_bytes);
+      else if (!vec) {
+        const int64_t frame = (n + 6) / 4;
+        if (framed_access() && same_frames(y, ldy, dy, lddy, w) && same_frames(y, ldy, dx, lddx, w) &&
+            n < (int64_t(1) << 31))
+          r = sm_bwd_cluster_launch<KIND, 4, true>(st, plan_cluster(frame, 3), frame, rows, y, ldy, dy, lddy, dx, lddx,
+                                                   map, ws, ws_bytes, static_cast<unsigned>(n));
+        if (r < 0)
+          r = sm_bwd_cluster_launch<KIND, 1>(st, plan_cluster(n, 8), n, rows, y, ldy, dy, lddy, dx, lddx, map, ws,
+                                             ws_bytes);
+      }
       if (r >= 0) return r;
     }
     const ChunkPlan p = plan_chunks(n, rows);

@@ -44,8 +44,8 @@ WORKLOADS = [
     ("ln_bwd_rows<__half", None, "cfg4 layer norm f16 bwd (followed by ln_wgrad_reduce)", 3 * _E4 * 2),
     ("sm_fwd_rows<float, 256, 4, 2", None, "cfg5a channelwise softmax fwd 256x64x4096", 2 * _E5A * 4),
     ("sm_bwd_rows<float, 256, 4, 2", None, "cfg5a channelwise softmax bwd", 3 * _E5A * 4),
-    ("sm_fwd_cluster<4, 0, 4>", 512, "cfg5b softmax 262144x16 fwd (8 clusters of 64, two rows each)", 2 * _E5B * 4),
-    ("sm_bwd_cluster<4, 0, 4>", 512, "cfg5b softmax 262144x16 bwd", 3 * _E5B * 4),
+    ("sm_fwd_cluster<4, 0, 4, false>", 512, "cfg5b softmax 262144x16 fwd (8 clusters of 64, two rows each)", 2 * _E5B * 4),
+    ("sm_bwd_cluster<4, 0, 4, false>", 512, "cfg5b softmax 262144x16 bwd", 3 * _E5B * 4),
     ("sm_fwd_partial", None, "cfg5b softmax 262144x16 fwd, split path, kernel 1 of 2", _E5B * 4),
     ("sm_fwd_apply", None, "cfg5b fwd, split path, kernel 2 of 2", 2 * _E5B * 4),
     ("sm_bwd_partial", None, "cfg5b bwd, split path, kernel 1 of 2", 2 * _E5B * 4),
@@ -55,10 +55,10 @@ WORKLOADS = [
     ("ln_bwd_rows<float, 64, 4, 4, true", None, "cfg1 layer norm bwd (followed by ln_wgrad_reduce)", 3 * 131072 * 4),
     ("ln_fwd_rows<float, 256, 4>", None, "extra: instance norm fwd 64x256x56x56", 2 * _E3 * 4),
     ("ln_bwd_rows<float, 256, 2, 4, false", None, "extra: instance norm bwd", 3 * _E3 * 4),
-    ("sm_fwd_cluster<4, 0, 4>", None, "extra: softmax 262144x256 fwd (row clusters)", 2 * 67108864 * 4),
-    ("sm_bwd_cluster<4, 0, 4>", None, "extra: softmax 262144x256 bwd (row clusters)", 3 * 67108864 * 4),
-    ("sm_fwd_cluster<8, 0, 1>", None, "extra: softmax 50257x1024 fwd (row clusters, one float per access)", 2 * 50257 * 1024 * 4),
-    ("sm_bwd_cluster<8, 0, 1>", None, "extra: softmax 50257x1024 bwd", 3 * 50257 * 1024 * 4),
+    ("sm_fwd_cluster<4, 0, 4, false>", None, "extra: softmax 262144x256 fwd (row clusters)", 2 * 67108864 * 4),
+    ("sm_bwd_cluster<4, 0, 4, false>", None, "extra: softmax 262144x256 bwd (row clusters)", 3 * 67108864 * 4),
+    ("sm_fwd_cluster<4, 0, 4, true>", None, "extra: softmax 50257x1024 fwd (row clusters, framed 16-byte access)", 2 * 50257 * 1024 * 4),
+    ("sm_bwd_cluster<3, 0, 4, true>", None, "extra: softmax 50257x1024 bwd", 3 * 50257 * 1024 * 4),
     ("ln_fwd_stream", None, "extra: instance norm 16x160^3 x 2 fwd (streaming clusters)", 2 * 131072000 * 4),
     ("ln_bwd_stream", None, "extra: instance norm 16x160^3 x 2 bwd", 3 * 131072000 * 4),
     ("ln_fwd_cluster", None, "extra: layer norm over whole samples fwd 802816x64", 2 * _E3 * 4),

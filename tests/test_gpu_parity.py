@@ -153,6 +153,44 @@ def test_few_long_rows_all_in_flight(L, kind, h, w, in_place):
         assert np.abs(y.astype(np.float64).reshape(-1, (2 if kind == "channelwise" else 1) * w, order="F").sum(axis=0) - 1).max() < 1e-5
 
 
+@pytest.mark.parametrize("kind", ["softmax", "log_softmax"])
+@pytest.mark.parametrize("h,w,lds", [
+    (50257, 6, (0, 0, 0, 0)),     # every tensor on the same frames: 16-byte access inside the rows
+    (50257, 6, (0, 1, 2, 1)),     # leading dimensions that differ modulo 4: one float per access
+    (50257, 6, (3, 7, 11, 3)),    # differ, but agree modulo 4: framed again
+    (40002, 5, (1, 1, 1, 1)),     # even length, odd leading dimension
+    (131071, 3, (0, 4, 0, 8)),
+    # rows that fit one workgroup's registers: the same choice in the row kernels
+    (16385, 5, (0, 1, 2, 1)), (16385, 5, (0, 4, 8, 0)), (30522, 4, (2, 2, 2, 2)), (8191, 70, (0, 0, 0, 0)),
+    (32762, 3, (1, 1, 1, 1)), (32763, 3, (0, 0, 0, 0)),   # the longest frame of 8192 vectors, and one entry more
+])
+def test_long_rows_off_the_16_byte_grid(L, kind, h, w, lds):
+    """Long rows that do not start on 16-byte boundaries: the kernels move them as 16-byte vectors
+    between the rows' own first and last entries when x, y (and y, dy, dx) start every row at the
+    same distance from a boundary, else float by float.  Padding rows hold NaN on the way in and
+    must come back untouched."""
+    rng = np.random.default_rng(h + sum(lds))
+    x, dy = rand(rng, h, w, 0, 2), rand(rng, h, w)
+    x[rng.integers(0, h, size=50), :] = 25.0
+    fwd, bwd = _sm_oracle(kind)
+    layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
+    pad_x, pad_y, pad_dy, pad_dx = lds
+    layer.prev_activations = L.DeviceMatrix.from_numpy(x, ldim=h + pad_x)
+    layer.activations = L.DeviceMatrix(h, w, ldim=h + pad_y, fill=-7.0)
+    layer.fp_compute()
+    y = layer.activations.to_numpy()
+    check(f"{kind} off-grid y {h}x{w} {lds}", y, fwd(x), fwd(f64(x)))
+    if pad_y:
+        assert torch.all(layer.activations.tensor[:w, h:] == -7.0).item(), "wrote outside the rows"
+    layer.prev_error_signals = L.DeviceMatrix.from_numpy(dy, ldim=h + pad_dy)
+    layer.error_signals = L.DeviceMatrix(h, w, ldim=h + pad_dx, fill=-7.0)
+    layer.bp_compute()
+    dx = layer.error_signals.to_numpy()
+    check(f"{kind} off-grid dx {h}x{w} {lds}", dx, bwd(f32(y), dy), bwd(f64(y), f64(dy)))
+    if pad_dx:
+        assert torch.all(layer.error_signals.tensor[:w, h:] == -7.0).item(), "wrote outside the rows"
+
+
 @pytest.mark.parametrize("kind", ["softmax", "log_softmax", "channelwise"])
 @pytest.mark.parametrize("h,w", [(4096, 6), (777, 5), (70000, 2)])
 def test_softmax_family_in_place(L, kind, h, w):
