@@ -504,6 +504,38 @@ def main():
         copy_cal = {"bytes_read": 4 * n, "bytes_written": 4 * n, "ms": ms, "gbs": 8 * n / (ms * 1e-3) / 1e9}
         print(f"# copy 256 MiB -> 256 MiB: {ms*1e3:.1f} us, {copy_cal['gbs']:.0f} GB/s", file=sys.stderr)
 
+    # Yardstick for the cold figures: plain streaming kernels (torch's copy and add, nothing of this
+    # library) on tensors of the headline size rotated among >= 1 GiB of copies, i.e. what the part
+    # gives a kernel with no reuse, no dependence between workgroups and nothing to compute.
+    cold_yardstick = None
+    if not args.no_cold:
+        n = 32768 * 512
+        sets = 8
+        xs = [torch.randn(n, device=dev) for _ in range(sets)]
+        ds = [torch.randn(n, device=dev) for _ in range(sets)]
+        os_ = [torch.empty(n, device=dev) for _ in range(sets)]
+
+        def wall(fn, reps):
+            for i in range(sets):
+                fn(i)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(reps):
+                fn(i % sets)
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / reps
+
+        tc = wall(lambda i: os_[i].copy_(xs[i]), 10 * sets)
+        ta = wall(lambda i: torch.add(xs[i], ds[i], out=os_[i]), 10 * sets)
+        cold_yardstick = {"tensor_bytes": 4 * n,
+                          "copy_gbs": 8 * n / tc / 1e9, "copy_frac": round(8 * n / tc / 1e9 / HBM_PEAK_GBS, 4),
+                          "add_gbs": 12 * n / ta / 1e9, "add_frac": round(12 * n / ta / 1e9 / HBM_PEAK_GBS, 4)}
+        print(f"# cold yardstick (torch, 64 MiB tensors rotated): copy {cold_yardstick['copy_gbs']:.0f} GB/s "
+              f"({100*cold_yardstick['copy_frac']:.1f}%), add {cold_yardstick['add_gbs']:.0f} GB/s "
+              f"({100*cold_yardstick['add_frac']:.1f}%)", file=sys.stderr)
+        del xs, ds, os_
+        torch.cuda.empty_cache()
+
     h = results[headline]
     # Dominant kernel of the headline step: the backward row kernel (3 tensors against 2).  Its
     # launch duration is measured here with HIP events on the launch stream, one pair of events
@@ -565,8 +597,9 @@ def main():
                 "config.cold_frac is the same step with its tensors rotated among 1 GiB of copies",
         "config": {"workload": h["workload"], "samples": 512, "classes": 32768,
                    "samples_per_s": h["samples_per_s"], "frac_of_hbm_peak": h["frac_of_hbm_peak"],
-                   "cold_frac": frac_of(h.get("cold")), "per_config": per_config},
-        "roofline": {"bound": "hbm", "kernel": "sm_bwd_rows<float,1024,8,softmax>", "achieved": dom_gbs,
+                   "cold_frac": frac_of(h.get("cold")), "cold_yardstick": cold_yardstick,
+                   "per_config": per_config},
+        "roofline": {"bound": "hbm", "kernel": "sm_bwd_rows_walk<float,8,softmax>", "achieved": dom_gbs,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom_gbs / HBM_PEAK_GBS,
                      "bytes_per_launch": dom_bytes, "avg_launch_ms": dom_ms,
                      "avg_launch_source": ("rocprofv3 per-dispatch average (profiles/bench_all_layers_kernel_trace.md), "

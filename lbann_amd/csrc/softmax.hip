@@ -424,6 +424,86 @@ sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t l
 }
 
 
+// Backward for rows that fill a 1024-thread workgroup's registers (two tensors of V vectors per
+// thread: one workgroup per compute unit).  The grid is one resident wave of workgroups and a
+// workgroup walks rows b, b + grid, ...: once dx of a row is formed in the registers that held dy,
+// the registers that held y take the next row's y while dx is stored, and the next row's dy
+// follows the stores, so a compute unit's loads overlap its stores instead of alternating with them.
+// 32768 x 512: 50.9 us per step against 52.9 with one row per workgroup (log-softmax 51.5 against
+// 54.8).  The same walk in the forward kernel, whose rows need half the registers so that two
+// workgroups share a compute unit anyway, loses (53.0 against 51.2 us per step), and so does the
+// walk over fp16 rows of this length (backward 19.9 against 18.8 us): fp32 rows of 8 vectors only.
+template <typename S, int V, int KIND, int STREAM>
+__global__ void __launch_bounds__(1024)
+sm_bwd_rows_walk(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx,
+                 RowMap map, int64_t rows, unsigned nvec)
+{
+  constexpr int TPR = 1024, W = 16 / sizeof(S), NW = TPR / kWave;
+  __shared__ float red[2][NW];
+  const unsigned t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wv = wave_index();
+  float a[V][W], g[V][W];
+  auto load_y = [&](int64_t row) {
+    const S* yr = y + map.offset(row, ldy);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = t + i * TPR;
+      if (idx < nvec) {
+        RowIO<S, W>::template load<(STREAM & 1) != 0>(yr + unsigned(W) * idx, a[i]);
+      }
+      else {
+#pragma unroll
+        for (int k = 0; k < W; ++k) a[i][k] = 0.f;
+      }
+    }
+  };
+  auto load_dy = [&](int64_t row) {
+    const S* gr = dy + map.offset(row, lddy);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = t + i * TPR;
+      if (idx < nvec) {
+        RowIO<S, W>::template load<(STREAM & 2) != 0>(gr + unsigned(W) * idx, g[i]);
+      }
+      else {
+#pragma unroll
+        for (int k = 0; k < W; ++k) g[i][k] = 0.f;
+      }
+    }
+  };
+  int64_t row = blockIdx.x;
+  if (row >= rows) return;
+  load_y(row);
+  load_dy(row);
+  for (int it = 0; row < rows; row += gridDim.x, ++it) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+#pragma unroll
+      for (int k = 0; k < W; ++k) s += (KIND == kLogSoftmax) ? g[i][k] : a[i][k] * g[i][k];
+    s = team_sum<NW>(s, red[it & 1], wv, lane);
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+#pragma unroll
+      for (int k = 0; k < W; ++k) {
+        if (KIND == kLogSoftmax) g[i][k] = g[i][k] - exp_fast(a[i][k]) * s;
+        else g[i][k] = a[i][k] * (g[i][k] - s);
+      }
+    const int64_t next = row + gridDim.x;
+    if (next < rows) load_y(next);
+    asm volatile("" ::: "memory");  // y of the next row goes out ahead of this row's stores
+    S* dr = dx + map.offset(row, lddx);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = t + i * TPR;
+      if (idx < nvec) RowIO<S, W>::store(dr + unsigned(W) * idx, g[i]);
+    }
+    asm volatile("" ::: "memory");
+    if (next < rows) load_dy(next);
+  }
+}
+
 // Merges the online-softmax pairs (m, acc) of the 256 threads of a workgroup (defined
 // with the split-row kernels below).
 __device__ __forceinline__ void block_merge_max_sum(float& m, float& acc, float (*slot)[2]);
@@ -1427,6 +1507,27 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   }
 }
 
+// The walking backward kernel when the rows need more than one resident wave of workgroups.
+template <int KIND, typename S>
+static bool sm_bwd_walk(hipStream_t st, int hint, int64_t rows, unsigned nvec, const S* y, const S* dy,
+                        S* dx, int64_t ldy, int64_t lddy, int64_t lddx, RowMap map)
+{
+  constexpr int V = 32 / (16 / sizeof(S));  // 32 values of each tensor per thread
+  static const bool off = std::getenv("LBN_NO_BWD_WALK") != nullptr;
+  if (off) return false;
+#define W_(H)                                                                                          \
+  if (hint == H) {                                                                                     \
+    const int cap = resident_blocks(sm_bwd_rows_walk<S, V, KIND, H>, 1024);                            \
+    if (cap < 1 || rows <= cap) return false;                                                          \
+    hipLaunchKernelGGL((sm_bwd_rows_walk<S, V, KIND, H>), dim3(static_cast<unsigned>(cap)), dim3(1024), 0, st, y, dy, \
+                       dx, ldy, lddy, lddx, map, rows, nvec);                                          \
+    return true;                                                                                       \
+  }
+  W_(0) W_(1) W_(2) W_(3)
+#undef W_
+  return false;
+}
+
 template <int KIND, typename S = float>
 static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int64_t w,
                   const S* y, int64_t ldy, const S* dy, int64_t lddy, S* dx,
@@ -1456,6 +1557,9 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     using B = RowBlock<TPR>;                                                                 \
     const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
     const int hint = stream_loads_bwd(rows, n * sizeof(S) / 4);                              \
+    if constexpr (std::is_same<S, float>::value && TPR == 1024 && V == 8) {                  \
+      if (sm_bwd_walk<KIND>(st, hint, rows, nvec, y, dy, dx, ldy, lddy, lddx, map)) return launch_status(); \
+    }                                                                                        \
     if (hint == 3)                                                                           \
       hipLaunchKernelGGL((sm_bwd_rows<S, TPR, V, KIND, 3>), dim3(grid), dim3(B::kThreads), 0, st, \
                          y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                       \

@@ -28,9 +28,10 @@ COPY_KIB = 262144.0  # the calibration copy reads and writes 256 MiB
 _E2, _E3, _E4, _E5A, _E5B = 16777216, 51380224, 33554432, 67108864, 4194304
 WORKLOADS = [
     ("sm_fwd_rows<float, 1024, 8, 0", None, "cfg2 softmax fwd 32768x512", 2 * _E2 * 4),
-    ("sm_bwd_rows<float, 1024, 8, 0", None, "cfg2 softmax bwd", 3 * _E2 * 4),
+    ("sm_bwd_rows_walk<float, 8, 0", None, "cfg2 softmax bwd (a workgroup walks two rows)", 3 * _E2 * 4),
+    ("sm_bwd_rows<float, 1024, 8, 0", None, "cfg2 softmax bwd, one row per workgroup (LBN_NO_BWD_WALK)", 3 * _E2 * 4),
     ("sm_fwd_rows<float, 1024, 8, 1", None, "cfg2 log-softmax fwd", 2 * _E2 * 4),
-    ("sm_bwd_rows<float, 1024, 8, 1", None, "cfg2 log-softmax bwd", 3 * _E2 * 4),
+    ("sm_bwd_rows_walk<float, 8, 1", None, "cfg2 log-softmax bwd", 3 * _E2 * 4),
     ("bn_fwd_cluster<float", None, "cfg3 batch norm fwd 64x256x56x56", 2 * _E3 * 4),
     ("bn_bwd_cluster<float", None, "cfg3 batch norm bwd", 3 * _E3 * 4),
     ("bn_fwd_cluster_ws<__half", None, "extra: batch norm fp16 storage fwd 64x256x56x56", 2 * _E3 * 2),
@@ -77,7 +78,7 @@ WORKLOADS = [
     ("grad_sink_quads<true>", None, "extra: gradient buffer, cleared: overwrite 4096x4096", 2 * _E2 * 4),
     ("grad_sink_quads<false>", None, "extra: gradient buffer, ready: accumulate 4096x4096", 3 * _E2 * 4),
 ]
-HEADLINE = "sm_bwd_rows<float, 1024, 8, 0"
+HEADLINE = "sm_bwd_rows_walk<float, 8, 0"
 
 
 def _short(name):
@@ -167,11 +168,11 @@ def trace(args):
             w = _lookup(write, name, wgs) * wfac / 1024
             row += f" {f:.1f} | {w:.1f} | " + (f"{(f + w) * 1048576 / nbytes:.2f} |" if nbytes else "|")
             if nbytes and HEADLINE in name:
-                headline = {"kernel": "sm_bwd_rows<float,1024,8,softmax> at 32768x512",
+                headline = {"kernel": "sm_bwd_rows_walk<float,8,softmax> at 32768x512",
                             "traffic_bytes_per_launch": (f + w) * 1048576, "fetch_factor": ffac, "write_factor": wfac,
                             "rocprof_avg_us": avg / 1e3}
         elif nbytes and HEADLINE in name:
-            headline = {"kernel": "sm_bwd_rows<float,1024,8,softmax> at 32768x512", "rocprof_avg_us": avg / 1e3}
+            headline = {"kernel": "sm_bwd_rows_walk<float,8,softmax> at 32768x512", "rocprof_avg_us": avg / 1e3}
         print(row)
     if args.headline_json and headline:
         with open(args.headline_json, "w") as f:
