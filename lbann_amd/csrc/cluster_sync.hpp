@@ -339,6 +339,18 @@ __device__ __forceinline__ void cluster_poll_complete(ClusterPoll<H>& p, const u
   }
 }
 
+// Completes a one-slot-per-lane poll: lane j < M returns the pair workgroup j published, the
+// other lanes (na, nb), like cluster_collect().
+__device__ __forceinline__ void cluster_poll_pairs(ClusterPoll<1>& p, const unsigned long long* slots, int M,
+                                                   ClusterTag tag, int* error_word, float na, float nb, float& ra,
+                                                   float& rb)
+{
+  bool have[1];
+  cluster_poll_complete<1>(p, slots, M, tag, error_word, have);
+  ra = have[0] ? __uint_as_float(static_cast<unsigned>(p.w[0][0])) : na;
+  rb = have[0] ? __uint_as_float(static_cast<unsigned>(p.w[0][1])) : nb;
+}
+
 // The cluster's totals of pairs that are simply added; every lane returns them.
 template <int H>
 __device__ __forceinline__ void cluster_poll_sums(ClusterPoll<H>& p, const unsigned long long* slots, int M,

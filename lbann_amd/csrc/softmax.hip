@@ -608,13 +608,16 @@ __device__ __forceinline__ void sm_cl_fwd_reduce(const SmClusterArgs& a, int64_t
 }
 
 // (3) of a step.
+// `poll` holds the polling loads for `row`, issued before the previous finish's stores (a wave's
+// memory operations complete in order: a poll issued after stores waits for their acknowledgement);
+// the loads for `next_row` (< 0: none) go out here, ahead of this row's stores.
 template <int V, int KIND, int W = 4, bool FR = false>
 __device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t row, unsigned base,
-                                                 SmFwdTile<V, W>& t, float* bc)
+                                                 SmFwdTile<V, W>& t, float* bc, ClusterPoll<1>& poll, int64_t next_row)
 {
   if (threadIdx.x < kWave) {
     float pm, ps;
-    cluster_collect(a.slots(row), a.M, a.tag, a.cw.error, -FLT_MAX, 0.f, pm, ps);
+    cluster_poll_pairs(poll, a.slots(row), a.M, a.tag, a.cw.error, -FLT_MAX, 0.f, pm, ps);
     const float gmax = wave_max(pm);
     const float gsum = wave_sum(ps * exp_fast(pm - gmax));
     if (threadIdx.x == 0) {
@@ -625,6 +628,8 @@ __device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t
   __syncthreads();
   const float gm = bc[0];
   const float gs = bc[1];
+  if (next_row >= 0 && threadIdx.x < kWave) cluster_poll_issue(poll, a.slots(next_row), a.M);
+  asm volatile("" ::: "memory");
   float* yr = a.out + a.map.offset(row, a.ldo);
   RowFrame fr{0, a.nvec};
   if constexpr (FR) {
@@ -660,13 +665,14 @@ __device__ __forceinline__ void sm_cl_fwd_finish(const SmClusterArgs& a, int64_t
 template <int V, int KIND, int W = 4, bool FR = false>
 __device__ __forceinline__ void sm_cl_fwd_step(const SmClusterArgs& a, int64_t row, int64_t nc, int k,
                                                unsigned base, SmFwdTile<V, W>& F, SmFwdTile<V, W>& R,
-                                               SmFwdTile<V, W>& L, float (*red)[2], float* bc)
+                                               SmFwdTile<V, W>& L, float (*red)[2], float* bc,
+                                               ClusterPoll<1>& poll)
 {
   if (row + nc < a.rows) sm_cl_fwd_reduce<V, KIND, W, FR>(a, row + nc, k, base, R, red);
   if (row + 2 * nc < a.rows)
     sm_cl_load<V, W, FR>(L.v, a.a + a.map.offset(row + 2 * nc, a.lda), base, a.nvec, -FLT_MAX, a.n);
   asm volatile("" ::: "memory");  // keep the loads above the wait below
-  sm_cl_fwd_finish<V, KIND, W, FR>(a, row, base, F, bc);
+  sm_cl_fwd_finish<V, KIND, W, FR>(a, row, base, F, bc, poll, row + nc < a.rows ? row + nc : -1);
 }
 
 template <int V, int KIND, int W = 4, bool FR = false>
@@ -686,12 +692,15 @@ sm_fwd_cluster(SmClusterArgs a)
   if (cl + nc < a.rows) sm_cl_load<V, W, FR>(t1.v, a.a + a.map.offset(cl + nc, a.lda), base, a.nvec, -FLT_MAX, a.n);
   sm_cl_fwd_reduce<V, KIND, W, FR>(a, cl, k, base, t0, red);
   __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
+  ClusterPoll<1> poll;
+  if (threadIdx.x < kWave) cluster_poll_issue(poll, a.slots(cl), a.M);
   // Each position of the rotation has its own broadcast slot: a step without a reduction has
   // no barrier between the reads of one finish and the write of the next.
   for (int64_t row = cl; row < a.rows; row += 3 * nc) {
-    sm_cl_fwd_step<V, KIND, W, FR>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
-    if (row + nc < a.rows) sm_cl_fwd_step<V, KIND, W, FR>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
-    if (row + 2 * nc < a.rows) sm_cl_fwd_step<V, KIND, W, FR>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
+    sm_cl_fwd_step<V, KIND, W, FR>(a, row, nc, k, base, t0, t1, t2, red, bc[0], poll);
+    if (row + nc < a.rows) sm_cl_fwd_step<V, KIND, W, FR>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1], poll);
+    if (row + 2 * nc < a.rows)
+      sm_cl_fwd_step<V, KIND, W, FR>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2], poll);
   }
 }
 
@@ -716,16 +725,18 @@ __device__ __forceinline__ void sm_cl_bwd_reduce(const SmClusterArgs& a, int64_t
 
 template <int V, int KIND, int W = 4, bool FR = false>
 __device__ __forceinline__ void sm_cl_bwd_finish(const SmClusterArgs& a, int64_t row, unsigned base,
-                                                 SmBwdTile<V, W>& t, float* bc)
+                                                 SmBwdTile<V, W>& t, float* bc, ClusterPoll<1>& poll, int64_t next_row)
 {
   if (threadIdx.x < kWave) {
     float pt, unused;
-    cluster_collect(a.slots(row), a.M, a.tag, a.cw.error, 0.f, 0.f, pt, unused);
+    cluster_poll_pairs(poll, a.slots(row), a.M, a.tag, a.cw.error, 0.f, 0.f, pt, unused);
     pt = wave_sum(pt);
     if (threadIdx.x == 0) bc[0] = pt;
   }
   __syncthreads();
   const float tot = bc[0];
+  if (next_row >= 0 && threadIdx.x < kWave) cluster_poll_issue(poll, a.slots(next_row), a.M);
+  asm volatile("" ::: "memory");
   float* dr = a.out + a.map.offset(row, a.ldo);
   RowFrame fr{0, a.nvec};
   if constexpr (FR) {
@@ -758,12 +769,12 @@ __device__ __forceinline__ void sm_cl_bwd_load(const SmClusterArgs& a, int64_t r
 template <int V, int KIND, int W = 4, bool FR = false>
 __device__ __forceinline__ void sm_cl_bwd_step(const SmClusterArgs& a, int64_t row, int64_t nc, int k,
                                                unsigned base, SmBwdTile<V, W>& F, SmBwdTile<V, W>& R,
-                                               SmBwdTile<V, W>& L, float* red, float* bc)
+                                               SmBwdTile<V, W>& L, float* red, float* bc, ClusterPoll<1>& poll)
 {
   if (row + nc < a.rows) sm_cl_bwd_reduce<V, KIND, W>(a, row + nc, k, R, red);
   if (row + 2 * nc < a.rows) sm_cl_bwd_load<V, W, FR>(a, row + 2 * nc, base, L);
   asm volatile("" ::: "memory");
-  sm_cl_bwd_finish<V, KIND, W, FR>(a, row, base, F, bc);
+  sm_cl_bwd_finish<V, KIND, W, FR>(a, row, base, F, bc, poll, row + nc < a.rows ? row + nc : -1);
 }
 
 template <int V, int KIND, int W = 4, bool FR = false>
@@ -783,12 +794,15 @@ sm_bwd_cluster(SmClusterArgs a)
   if (cl + nc < a.rows) sm_cl_bwd_load<V, W, FR>(a, cl + nc, base, t1);
   sm_cl_bwd_reduce<V, KIND, W>(a, cl, k, t0, red);
   __syncthreads();  // the first step reduces again at once: every wave must have read `red` by then
+  ClusterPoll<1> poll;
+  if (threadIdx.x < kWave) cluster_poll_issue(poll, a.slots(cl), a.M);
   // Each position of the rotation has its own broadcast slot: a step without a reduction has
   // no barrier between the reads of one finish and the write of the next.
   for (int64_t row = cl; row < a.rows; row += 3 * nc) {
-    sm_cl_bwd_step<V, KIND, W, FR>(a, row, nc, k, base, t0, t1, t2, red, bc[0]);
-    if (row + nc < a.rows) sm_cl_bwd_step<V, KIND, W, FR>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1]);
-    if (row + 2 * nc < a.rows) sm_cl_bwd_step<V, KIND, W, FR>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2]);
+    sm_cl_bwd_step<V, KIND, W, FR>(a, row, nc, k, base, t0, t1, t2, red, bc[0], poll);
+    if (row + nc < a.rows) sm_cl_bwd_step<V, KIND, W, FR>(a, row + nc, nc, k, base, t1, t2, t0, red, bc[1], poll);
+    if (row + 2 * nc < a.rows)
+      sm_cl_bwd_step<V, KIND, W, FR>(a, row + 2 * nc, nc, k, base, t2, t0, t1, red, bc[2], poll);
   }
 }
 
