@@ -175,10 +175,11 @@ public:
                       "call are undefined");
     }
   }
-  /// The debugging mode's check after every call.
+  /// The debugging mode's check after every call (not while the stream is being captured into
+  /// a HIP graph: the check waits for the device).
   void after_call(hipStream_t stream, const char* where)
   {
-    if (detail::check_every_call()) check(stream, where);
+    if (detail::check_every_call() && !detail::stream_is_capturing(stream)) check(stream, where);
   }
 
 private:

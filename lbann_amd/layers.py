@@ -144,6 +144,14 @@ def check_cluster_waits():
             raise ClusterWaitTimedOut(f"workspace of {ws.owner}")
 
 
+def _after_call():
+    """The debugging mode's check after a compute call.  It waits for the device, which a stream
+    that is being captured into a HIP graph does not allow: calls recorded into a graph are
+    checked where their results are consumed, like every call outside the debugging mode."""
+    if _CHECK_EVERY_CALL and not torch.cuda.is_current_stream_capturing():
+        check_cluster_waits()
+
+
 class _Workspace:
     """Scratch memory owned by a layer, grown on demand (never shrunk).  The first 64 bytes
     (the error word of the kernels that wait across workgroups) are cleared when the memory
@@ -197,14 +205,12 @@ class _Layer:
     def fp_compute(self):
         name, args = self.fp_call()
         call(name, *args)
-        if _CHECK_EVERY_CALL:
-            check_cluster_waits()
+        _after_call()
 
     def bp_compute(self):
         name, args = self.bp_call()
         call(name, *args)
-        if _CHECK_EVERY_CALL:
-            check_cluster_waits()
+        _after_call()
 
     def forward(self, x, in_place=False):
         self.bind_forward(x, in_place)
@@ -630,14 +636,12 @@ class cross_entropy_layer:
     def fp_compute(self):
         name, args = self.fp_call()
         call(name, *args)
-        if _CHECK_EVERY_CALL:
-            check_cluster_waits()
+        _after_call()
 
     def bp_compute(self):
         name, args = self.bp_call()
         call(name, *args)
-        if _CHECK_EVERY_CALL:
-            check_cluster_waits()
+        _after_call()
 
     def forward(self, prediction, ground_truth):
         self.prev_activations = [prediction, ground_truth]
@@ -674,8 +678,7 @@ def softmax_cross_entropy_forward(softmax, cross_entropy, x, ground_truth):
     call("lbn_softmax_cross_entropy_fwd_f32", _stream(), x.height, x.width, int(cross_entropy.m_use_labels),
          cross_entropy.spatial_sample_size, x.Buffer(), x.ldim, ground_truth.Buffer(), ground_truth.ldim,
          y.Buffer(), y.ldim, loss.Buffer(), loss.ldim, ws, nb)
-    if _CHECK_EVERY_CALL:
-        check_cluster_waits()
+    _after_call()
     return y, loss
 
 

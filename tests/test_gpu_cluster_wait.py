@@ -58,9 +58,10 @@ def test_python_mirror_reports_a_wait_that_gave_up(L):
     out = torch.empty(4, device="cuda")
     L.call("lbn_selftest_cluster_wait_gives_up", L._stream(), L.capi.vp(ws.data_ptr()), ws.numel(), 16,
            L.capi.vp(out.data_ptr()))
-    y = layer.forward(L.DeviceMatrix.from_numpy(x))      # the next call registers the workspace for checking
     with pytest.raises(L.ClusterWaitTimedOut):
+        y = layer.forward(L.DeviceMatrix.from_numpy(x))  # the next call registers the workspace for checking
         y.to_numpy()                                     # results are consumed here: the raised word surfaces
+        # (with LBN_CHECK_CLUSTER_WAITS=1 in the environment the call itself raises)
     assert _flag(L, ws) == 0                             # reported once, then cleared
     y = layer.forward(L.DeviceMatrix.from_numpy(x))
     check("softmax after", y.to_numpy(), orc.softmax_fwd(x), orc.softmax_fwd(np.asfortranarray(x.astype(np.float64))))
