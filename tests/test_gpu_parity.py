@@ -191,6 +191,48 @@ def test_long_rows_off_the_16_byte_grid(L, kind, h, w, lds):
         assert torch.all(layer.error_signals.tensor[:w, h:] == -7.0).item(), "wrote outside the rows"
 
 
+@pytest.mark.parametrize("h", [16385, 50257])
+@pytest.mark.parametrize("offsets", [(1, 1, 1, 1), (1, 2, 1, 1), (3, 3, 3, 3), (2, 0, 2, 0), (0, 0, 1, 0)])
+def test_matrices_that_start_off_the_16_byte_grid(L, h, offsets):
+    """Views into larger allocations: base pointers 4, 8 or 12 bytes past a 16-byte boundary.
+    Tensors whose offsets agree take the 16-byte accesses, the others one float at a time; the
+    floats in front of and behind every matrix must come back untouched."""
+    w = 5
+    ox, oy, ody, odx = offsets
+    rng = np.random.default_rng(h + 7 * sum(offsets))
+    x, dy = rand(rng, h, w, 0, 2), rand(rng, h, w)
+    x[rng.integers(0, h, size=40), :] = 20.0
+    capi = L.capi
+    st = L._stream()
+
+    def device(a, off):
+        buf = torch.full((off + h * w + 8,), -7.0, device="cuda")
+        if a is not None:
+            buf[off:off + h * w] = torch.from_numpy(np.ascontiguousarray(a.T).reshape(-1)).cuda()
+        return buf
+
+    def host(buf, off):
+        assert torch.all(buf[:off] == -7.0).item() and torch.all(buf[off + h * w:] == -7.0).item(), "wrote outside the matrix"
+        return np.asfortranarray(buf[off:off + h * w].cpu().numpy().reshape(w, h).T)
+
+    ptr = lambda buf, off: capi.vp(buf.data_ptr() + 4 * off)
+    nb = capi.lib().lbn_softmax_workspace_bytes(h, w)
+    ws = torch.zeros(max(nb, 64), dtype=torch.uint8, device="cuda")
+    bx, by = device(x, ox), device(None, oy)
+    capi.call("lbn_softmax_fwd_f32", st, h, w, ptr(bx, ox), h, ptr(by, oy), h, capi.vp(ws.data_ptr()), nb)
+    y = host(by, oy)
+    check(f"softmax off-grid base y {h} {offsets}", y, orc.softmax_fwd(x), orc.softmax_fwd(f64(x)))
+    # backward reads the y it is given (offset oy), dy at ody, writes dx at odx
+    bdy, bdx = device(dy, ody), device(None, odx)
+    capi.call("lbn_softmax_bwd_f32", st, h, w, ptr(by, oy), h, ptr(bdy, ody), h, ptr(bdx, odx), h,
+              capi.vp(ws.data_ptr()), nb)
+    dx = host(bdx, odx)
+    check(f"softmax off-grid base dx {h} {offsets}", dx, orc.softmax_bwd(f32(y), dy), orc.softmax_bwd(f64(y), f64(dy)))
+    flag = capi.cint(0)
+    capi.call("lbn_workspace_timed_out", st, capi.vp(ws.data_ptr()), flag)
+    assert flag.value == 0
+
+
 @pytest.mark.parametrize("kind", ["softmax", "log_softmax", "channelwise"])
 @pytest.mark.parametrize("h,w", [(4096, 6), (777, 5), (70000, 2)])
 def test_softmax_family_in_place(L, kind, h, w):
