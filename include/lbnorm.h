@@ -34,12 +34,17 @@
  * guarantees of the HIP API: the occupancy query describes a device that runs nothing
  * else, and workgroups are dispatched in block order (members of a cluster are
  * consecutive blocks, so a launch that shares the device still has at most one partly
- * resident cluster, whose missing members are the next to start).  Supported use: one
- * cluster kernel on the device at a time, i.e. calls on one stream (or on several, when
- * their cluster calls do not overlap); cluster calls running concurrently on several
- * streams can each hold part of the device and wait on each other until the poll bound.
- * Callers that cannot promise this set LBN_NO_CLUSTER=1 in the environment, which selects
- * the multi-kernel paths everywhere.  Every wait is bounded: a wait that runs out raises
+ * resident cluster, whose missing members are the next to start).  Two cluster kernels must
+ * not share the device: each could hold part of it and wait for workgroups that cannot
+ * start.  The library sees to that for eager calls itself: a cluster kernel whose
+ * predecessor went to another stream is made to wait for it with an event (processes that
+ * use one stream for these calls pay nothing; the first call from a second stream waits
+ * for the device once), and launches from several host threads queue up behind a mutex.
+ * What it cannot order are replays of HIP graphs that contain cluster kernels: do not
+ * replay two such graphs, or one next to eager cluster calls of another stream, at the same
+ * time (or set LBN_NO_CLUSTER=1 in the environment, which selects the multi-kernel paths
+ * everywhere), and other work that occupies the device while a cluster kernel starts
+ * shrinks what the occupancy query promised.  Every wait is bounded: a wait that runs out raises
  * a sticky error word in the workspace's first 64 bytes (written by nothing else), the
  * kernel ends normally with undefined results, and the entry point has long returned 0.
  * lbn_workspace_timed_out() reads that word; a caller who wants to rely on it clears the
@@ -48,8 +53,9 @@
  * layer classes do both.
  *
  * Process-wide state of the library: the counter the per-call tags are drawn from (an
- * atomic), the cached occupancy figures per kernel and device, and the environment
- * switches, each read once.  Nothing else outlives a call.
+ * atomic), the cached occupancy figures per kernel and device, per device the stream of the
+ * last cluster kernel with its mutex and (once a second stream has been seen) one event,
+ * and the environment switches, each read once.  Nothing else outlives a call.
  */
 #ifndef LBNORM_H_INCLUDED
 #define LBNORM_H_INCLUDED

@@ -1015,6 +1015,7 @@ static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   const int64_t E = cs / VE * w;
   const BnClusterShape p = bn_cluster_shape(E, 4, 256);
   if (!p.T) return false;
+  ClusterLaunchGuard guard(st);
   const BnFwdArgs<S> a{x, y, ldx, ldy, cs, static_cast<int>(C), p.M, pivot, bessel, eps, decay, cs * w,
                        cluster_workspace(ws), cluster_call_tag(st, cluster_workspace(ws)), mean, var, scale, bias, rmean, rvar};
   const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(E);
@@ -1038,6 +1039,7 @@ static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   constexpr bool kShortVectors = sizeof(typename Vec16<S>::raw_t) == 8;
   const BnClusterShape p = bn_cluster_shape(E, kShortVectors ? 4 : 2, 256);
   if (!p.T) return false;
+  ClusterLaunchGuard guard(st);
   const BnBwdArgs<S> a{x, dy, dx, ldx, lddy, lddx, cs, static_cast<int>(C), p.M, bessel, eps, cs * w,
                        cluster_workspace(ws), cluster_call_tag(st, cluster_workspace(ws)), mean, var, scale, dscale, dbias, dmean, dvar};
   const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(E);
@@ -1072,6 +1074,7 @@ static bool bn_try_stream(hipStream_t st, BnStreamArgs<S> a, int64_t C, int64_t 
   a.cs = cs, a.C = static_cast<int>(C), a.M = static_cast<int>(M), a.n = cs * w;
   a.seg = static_cast<unsigned>(cs / VE), a.E = static_cast<unsigned>(E), a.share = static_cast<unsigned>(share);
   a.cw = cluster_workspace(ws);
+  ClusterLaunchGuard guard(st);
   a.tag = cluster_call_tag(st, a.cw);
   const dim3 grid(static_cast<unsigned>(nc * M));
   if (BWD) hipLaunchKernelGGL(bn_bwd_stream<S>, grid, dim3(kBnStreamThreads), 0, st, a);

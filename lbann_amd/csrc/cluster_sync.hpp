@@ -31,6 +31,7 @@
 #include <atomic>
 #include <chrono>
 #include <cstdint>
+#include <mutex>
 
 #include "device_utils.hpp"
 #include "host_utils.hpp"
@@ -441,6 +442,86 @@ inline ClusterTag cluster_call_tag(hipStream_t st, const ClusterWorkspace& cw)
   }
   return tag;
 }
+
+// Keeps the cluster kernels of a device from running side by side.  A cluster kernel sizes its
+// grid to what the device holds at once and its workgroups wait for each other: two of them
+// started from different streams could each get part of the device and wait for workgroups that
+// cannot be scheduled (the bounded waits would then give up and raise the error word).  One
+// guard lives around every cluster launch: when the previous cluster launch of the device went
+// to another stream, the new one is made to wait for it with an event; the guard also holds a
+// mutex, so that launches from several host threads queue up one at a time.
+//
+// A process that only ever uses one stream for these calls pays nothing: events are recorded
+// only from the moment a second stream shows up (that launch waits for the device once, the
+// earlier launch having left no event).  Streams that are being recorded into a HIP graph are
+// left alone: keeping graphs that contain cluster kernels from replaying side by side is up to
+// the caller.
+class ClusterLaunchGuard {
+ public:
+  explicit ClusterLaunchGuard(hipStream_t st) : st_(st), capturing_(stream_is_capturing(st))
+  {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+    state_ = &states()[dev];
+    state_->mu.lock();
+    if (capturing_ || !state_->have_last || state_->last == st) return;
+    if (!state_->several) {
+      state_->several = true;
+      make_event(*state_);
+      (void)hipDeviceSynchronize();
+    }
+    else if (state_->done) {
+      (void)hipStreamWaitEvent(st, state_->done, 0);
+    }
+  }
+  ~ClusterLaunchGuard()
+  {
+    if (!capturing_) {
+      if (state_->several && state_->done) (void)hipEventRecord(state_->done, st_);
+      state_->last = st_;
+      state_->have_last = true;
+    }
+    state_->mu.unlock();
+  }
+  ClusterLaunchGuard(const ClusterLaunchGuard&) = delete;
+  ClusterLaunchGuard& operator=(const ClusterLaunchGuard&) = delete;
+
+  // Creates the current device's event ahead of time, for callers that must not create
+  // anything later (the entry point that allocates nothing does this in its set-up).
+  static void prepare()
+  {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+    State& s = states()[dev];
+    std::lock_guard<std::mutex> lock(s.mu);
+    make_event(s);
+  }
+
+ private:
+  static constexpr int kMaxDevices = 64;
+  struct State {
+    std::mutex mu;
+    hipStream_t last = nullptr;
+    bool have_last = false;
+    bool several = false;      // cluster launches have come from more than one stream
+    hipEvent_t done = nullptr;  // recorded after every cluster launch once `several` is set
+  };
+  static State* states()
+  {
+    static State s[kMaxDevices];
+    return s;
+  }
+  static void make_event(State& s)
+  {
+    if (!s.done && hipEventCreateWithFlags(&s.done, hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      s.done = nullptr;
+    }
+  }
+  hipStream_t st_;
+  bool capturing_;
+  State* state_;
+};
 
 // Cluster shape for an item of E 16-byte vectors: V vectors per thread (<= max_v), M
 // workgroups of kClusterThreads per item (<= kClusterMaxM); M == 0: does not fit.

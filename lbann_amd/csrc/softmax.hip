@@ -1306,6 +1306,7 @@ static int sm_fwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, 
     int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
     if (ncl < 1) return -1;                                                                      \
     ncl = cluster_count(rows, ncl, cp.M);                                                        \
+    ClusterLaunchGuard guard(st);                                                                \
     const SmClusterArgs a{x, nullptr, y, ldx, 0, ldy, map, rows, static_cast<unsigned>(units),   \
                           n, cp.M, cw, cluster_call_tag(st, cw)};                                \
     hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND, W, FR>), dim3(static_cast<unsigned>(ncl * cp.M)), \
@@ -1332,6 +1333,7 @@ static int sm_bwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, 
     int64_t ncl = cap / cp.M < rows ? cap / cp.M : rows;                                         \
     if (ncl < 1) return -1;                                                                      \
     ncl = cluster_count(rows, ncl, cp.M);                                                        \
+    ClusterLaunchGuard guard(st);                                                                \
     const SmClusterArgs a{y, dy, dx, ldy, lddy, lddx, map, rows, static_cast<unsigned>(units),   \
                           n, cp.M, cw, cluster_call_tag(st, cw)};                                \
     hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND, W, FR>), dim3(static_cast<unsigned>(ncl * cp.M)), \
@@ -1719,6 +1721,9 @@ static int static_scratch_address(void** out)
     if (e != hipSuccess) return static_cast<int>(e);
     if (!p) return static_cast<int>(hipErrorInvalidSymbol);
     address[dev] = p;
+    // set-up, once per device: the event that orders cluster kernels across streams, so that
+    // no later call of the entry point that allocates nothing has to create it
+    ClusterLaunchGuard::prepare();
   }
   *out = address[dev];
   return LBN_OK;

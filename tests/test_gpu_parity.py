@@ -964,3 +964,33 @@ def test_concurrent_host_threads_on_separate_streams(L):
     torch.cuda.synchronize()
     for a, b in zip(alone_a[0] + alone_b[0], got_a[0] + got_b[0]):
         assert np.array_equal(a, b)
+
+
+def test_cluster_kernels_enqueued_on_two_streams_without_waiting(L):
+    """Kernels whose workgroups wait for each other must not share the device.  One host thread
+    enqueues many of them on two streams, alternately and without waiting in between: the library
+    orders them across the streams itself, every result equals the one computed on one stream, and
+    no wait runs out (to_numpy() checks the workspaces' error words)."""
+    rng = np.random.default_rng(17)
+    xs = rand(rng, 262144, 8)                     # a few long rows: row clusters
+    xb = rand(rng, 64 * 784, 64, 2.0, 3.0)        # channel clusters
+    sm_ref = L.softmax_layer().forward(L.DeviceMatrix.from_numpy(xs)).to_numpy()
+    bn_ref = L.batch_normalization_layer((64, 28, 28)).forward(L.DeviceMatrix.from_numpy(xb)).to_numpy()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    reps = 12
+    sms = [L.softmax_layer() for _ in range(reps)]
+    bns = [L.batch_normalization_layer((64, 28, 28)) for _ in range(reps)]
+    dxs, dxb = L.DeviceMatrix.from_numpy(xs), L.DeviceMatrix.from_numpy(xb)
+    torch.cuda.synchronize()
+    ys, yb = [], []
+    for i in range(reps):
+        with torch.cuda.stream(s1):
+            ys.append(sms[i].forward(dxs))
+        with torch.cuda.stream(s2):
+            yb.append(bns[i].forward(dxb))
+    torch.cuda.synchronize()
+    for y in ys:
+        assert np.array_equal(y.to_numpy(), sm_ref)
+    for y in yb:
+        assert np.array_equal(y.to_numpy(), bn_ref)
+
