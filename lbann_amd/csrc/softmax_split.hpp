@@ -1,0 +1,369 @@
+// Softmax family: the split ("chunked") kernels for rows that no register kernel takes, and the
+// one-workgroup-per-row kernels for fp16 rows beyond the register kernels.  Included by softmax.hip.
+#pragma once
+
+#include "softmax_rows.hpp"
+
+namespace lbn {
+
+// ================================================================ split rows
+// Block b handles chunk (b % S) of row (b / S); 256 threads per block.
+constexpr int kChunkThreads = 256;
+constexpr int kChunkUnroll = 4;
+
+// Merges the online-softmax pairs (m, acc) of the 256 threads; every thread gets the result.
+__device__ __forceinline__ void block_merge_max_sum(float& m, float& acc, float (*slot)[2])
+{
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wv = threadIdx.x / kWave;
+  const float wm = wave_max(m);
+  acc = wave_sum(acc * exp_fast(m - wm));
+  if (lane == 0) {
+    slot[wv][0] = wm;
+    slot[wv][1] = acc;
+  }
+  __syncthreads();
+  float bm = slot[0][0];
+#pragma unroll
+  for (int i = 1; i < kChunkThreads / kWave; ++i) bm = fmaxf(bm, slot[i][0]);
+  float bs = 0.f;
+#pragma unroll
+  for (int i = 0; i < kChunkThreads / kWave; ++i) bs += slot[i][1] * exp_fast(slot[i][0] - bm);
+  m = bm;
+  acc = bs;
+}
+
+// A run of `len` floats at p, cut at 16-byte boundaries: `head` leading scalars, `nvec`
+// aligned vectors, `tail` trailing scalars.  Rows whose starts are only 4-byte aligned
+// (odd lengths, e.g. a vocabulary of 50257 entries) still move almost all of their bytes
+// with 16-byte accesses this way.
+struct Peel {
+  int head, tail;
+  int64_t nvec;
+  // index (relative to p) of the edge scalar thread t handles, for t < head + tail
+  __device__ __forceinline__ int64_t edge(int t) const { return t < head ? t : head + 4 * nvec + (t - head); }
+};
+
+__device__ __forceinline__ Peel peel16(const float* p, int64_t len)
+{
+  Peel r;
+  r.head = static_cast<int>((4 - ((reinterpret_cast<uintptr_t>(p) >> 2) & 3)) & 3);
+  if (r.head > len) r.head = static_cast<int>(len);
+  r.nvec = (len - r.head) / 4;
+  r.tail = static_cast<int>(len - r.head - 4 * r.nvec);
+  return r;
+}
+
+__device__ __forceinline__ bool same_phase16(const void* a, const void* b)
+{
+  return ((reinterpret_cast<uintptr_t>(a) ^ reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
+}
+
+// Online (max, sum of exp) over nvec aligned vectors at base, strided over the workgroup;
+// four independent 16-byte loads per thread are in flight before any is used.
+__device__ __forceinline__ void sm_reduce_vectors(const float* base, int64_t nvec, float& m, float& acc)
+{
+  for (int64_t i0 = threadIdx.x; i0 < nvec; i0 += kChunkUnroll * kChunkThreads) {
+    float v[kChunkUnroll][4];
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+      if (i < nvec) {
+        Vec16<float>::load(base + 4 * i, v[u]);
+      }
+      else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[u][k] = -FLT_MAX;
+      }
+    }
+    float mn = m;
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) mn = fmaxf(mn, v[u][k]);
+    float add = 0.f;
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const bool ok = i0 + u * kChunkThreads < nvec;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) add += ok ? exp_fast(v[u][k] - mn) : 0.f;
+    }
+    acc = acc * exp_fast(m - mn) + add;
+    m = mn;
+  }
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_fwd_partial(const float* x, int64_t ldx, RowMap map, int64_t n, int64_t chunk, int S,
+               float2* part)
+{
+  __shared__ float slot[kChunkThreads / kWave][2];
+  const int64_t row = blockIdx.x / S;
+  const int s = blockIdx.x - row * S;
+  const int64_t begin = s * chunk;
+  const int64_t end = imin64(n, begin + chunk);
+  const float* p = x + map.offset(row, ldx) + begin;
+  float m = -FLT_MAX, acc = 0.f;
+  if (VEC) {
+    sm_reduce_vectors(p, (end - begin) / 4, m, acc);
+  }
+  else {
+    const Peel pl = peel16(p, end - begin);
+    if (static_cast<int>(threadIdx.x) < pl.head + pl.tail) {
+      m = p[pl.edge(threadIdx.x)];
+      acc = 1.f;
+    }
+    sm_reduce_vectors(p + pl.head, pl.nvec, m, acc);
+  }
+  block_merge_max_sum(m, acc, slot);
+  if (threadIdx.x == 0) part[blockIdx.x] = make_float2(m, acc);
+}
+
+// out[i] = f(in[i]) over nvec aligned vectors, strided over the workgroup.
+template <typename F>
+__device__ __forceinline__ void sm_map_vectors(const float* in, float* out, int64_t nvec, F f)
+{
+  for (int64_t i0 = threadIdx.x; i0 < nvec; i0 += kChunkUnroll * kChunkThreads) {
+    float v[kChunkUnroll][4];
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+      if (i < nvec) Vec16<float>::load(in + 4 * i, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+      if (i < nvec) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[u][k] = f(v[u][k]);
+        Vec16<float>::store(out + 4 * i, v[u]);
+      }
+    }
+  }
+}
+
+template <bool VEC, int KIND>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_fwd_apply(const float* x, float* y, int64_t ldx, int64_t ldy, RowMap map, int64_t n,
+             int64_t chunk, int S, const float2* part)
+{
+  const int64_t row = blockIdx.x / S;
+  const int s = blockIdx.x - row * S;
+  const int64_t begin = s * chunk;
+  const int64_t end = imin64(n, begin + chunk);
+  const int lane = threadIdx.x & (kWave - 1);
+  // every wave merges the S <= 64 partials of the row on its own
+  float pm = -FLT_MAX, ps = 0.f;
+  if (lane < S) {
+    const float2 p = part[row * S + lane];
+    pm = p.x;
+    ps = p.y;
+  }
+  const float m = wave_max(pm);
+  const float sum = wave_sum(ps * exp_fast(pm - m));
+  const float scale = 1.0f / sum;
+  const float lse = (KIND == kLogSoftmax) ? log_of_sum(sum) : 0.f;
+  const float* xp = x + map.offset(row, ldx) + begin;
+  float* yp = y + map.offset(row, ldy) + begin;
+  const int64_t len = end - begin;
+  auto f = [&](float v) -> float {
+    const float d = v - m;
+    if (KIND == kLogSoftmax) return d - lse;
+    const float r = scale * (KIND == kChannelwise ? exp_keep_denormals(d) : exp_fast(d));
+    if (KIND == kSoftmax) return __builtin_isnormal(r) ? r : 0.f;
+    return r;
+  };
+  if (VEC) {
+    sm_map_vectors(xp, yp, len / 4, f);
+  }
+  else if (same_phase16(xp, yp)) {
+    const Peel pl = peel16(xp, len);
+    if (static_cast<int>(threadIdx.x) < pl.head + pl.tail) {
+      const int64_t e = pl.edge(threadIdx.x);
+      yp[e] = f(xp[e]);
+    }
+    sm_map_vectors(xp + pl.head, yp + pl.head, pl.nvec, f);
+  }
+  else {
+    for (int64_t i = threadIdx.x; i < len; i += kChunkThreads) yp[i] = f(xp[i]);
+  }
+}
+
+// sum of dy (log-softmax) or of y * dy over nvec aligned vectors, strided over the workgroup.
+template <int KIND>
+__device__ __forceinline__ float sm_dot_vectors(const float* yb, const float* gb, int64_t nvec)
+{
+  float acc = 0.f;
+  for (int64_t i0 = threadIdx.x; i0 < nvec; i0 += kChunkUnroll * kChunkThreads) {
+    float a[kChunkUnroll][4], g[kChunkUnroll][4];
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) a[u][k] = g[u][k] = 0.f;
+      if (i < nvec) {
+        Vec16<float>::load(gb + 4 * i, g[u]);
+        if (KIND != kLogSoftmax) Vec16<float>::load(yb + 4 * i, a[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      if (KIND == kLogSoftmax) acc += (g[u][0] + g[u][1]) + (g[u][2] + g[u][3]);
+      else acc += (a[u][0] * g[u][0] + a[u][1] * g[u][1]) + (a[u][2] * g[u][2] + a[u][3] * g[u][3]);
+    }
+  }
+  return acc;
+}
+
+template <bool VEC, int KIND>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_bwd_partial(const float* y, const float* dy, int64_t ldy, int64_t lddy, RowMap map, int64_t n,
+               int64_t chunk, int S, float* part)
+{
+  __shared__ float slot[kChunkThreads / kWave];
+  const int64_t row = blockIdx.x / S;
+  const int s = blockIdx.x - row * S;
+  const int64_t begin = s * chunk;
+  const int64_t end = imin64(n, begin + chunk);
+  const float* yp = y + map.offset(row, ldy) + begin;
+  const float* gp = dy + map.offset(row, lddy) + begin;
+  const int64_t len = end - begin;
+  float acc = 0.f;
+  if (VEC) {
+    acc = sm_dot_vectors<KIND>(yp, gp, len / 4);
+  }
+  else if (same_phase16(yp, gp)) {
+    const Peel pl = peel16(gp, len);
+    acc = sm_dot_vectors<KIND>(yp + pl.head, gp + pl.head, pl.nvec);
+    if (static_cast<int>(threadIdx.x) < pl.head + pl.tail) {
+      const int64_t e = pl.edge(threadIdx.x);
+      acc += (KIND == kLogSoftmax) ? gp[e] : yp[e] * gp[e];
+    }
+  }
+  else {
+    for (int64_t i = threadIdx.x; i < len; i += kChunkThreads)
+      acc += (KIND == kLogSoftmax) ? gp[i] : yp[i] * gp[i];
+  }
+  acc = team_sum<kChunkThreads / kWave>(acc, slot, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+  if (threadIdx.x == 0) part[blockIdx.x] = acc;
+}
+
+// out[i] = f(a[i], g[i]) over nvec aligned vectors, strided over the workgroup.
+template <typename F>
+__device__ __forceinline__ void sm_map2_vectors(const float* ab, const float* gb, float* out, int64_t nvec, F f)
+{
+  for (int64_t i0 = threadIdx.x; i0 < nvec; i0 += kChunkUnroll * kChunkThreads) {
+    float a[kChunkUnroll][4], g[kChunkUnroll][4];
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+      if (i < nvec) {
+        Vec16<float>::load(ab + 4 * i, a[u]);
+        Vec16<float>::load(gb + 4 * i, g[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kChunkUnroll; ++u) {
+      const int64_t i = i0 + u * kChunkThreads;
+      if (i < nvec) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) g[u][k] = f(a[u][k], g[u][k]);
+        Vec16<float>::store(out + 4 * i, g[u]);
+      }
+    }
+  }
+}
+
+template <bool VEC, int KIND>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_bwd_apply(const float* y, const float* dy, float* dx, int64_t ldy, int64_t lddy, int64_t lddx,
+             RowMap map, int64_t n, int64_t chunk, int S, const float* part)
+{
+  const int64_t row = blockIdx.x / S;
+  const int s = blockIdx.x - row * S;
+  const int64_t begin = s * chunk;
+  const int64_t end = imin64(n, begin + chunk);
+  const int lane = threadIdx.x & (kWave - 1);
+  const float sum = wave_sum(lane < S ? part[row * S + lane] : 0.f);
+  const float* yp = y + map.offset(row, ldy) + begin;
+  const float* gp = dy + map.offset(row, lddy) + begin;
+  float* dp = dx + map.offset(row, lddx) + begin;
+  const int64_t len = end - begin;
+  auto f = [&](float a, float g) -> float {
+    return (KIND == kLogSoftmax) ? g - exp_fast(a) * sum : a * (g - sum);
+  };
+  if (VEC) {
+    sm_map2_vectors(yp, gp, dp, len / 4, f);
+  }
+  else if (same_phase16(yp, gp) && same_phase16(yp, dp)) {
+    const Peel pl = peel16(yp, len);
+    if (static_cast<int>(threadIdx.x) < pl.head + pl.tail) {
+      const int64_t e = pl.edge(threadIdx.x);
+      dp[e] = f(yp[e], gp[e]);
+    }
+    sm_map2_vectors(yp + pl.head, gp + pl.head, dp + pl.head, pl.nvec, f);
+  }
+  else {
+    for (int64_t i = threadIdx.x; i < len; i += kChunkThreads) dp[i] = f(yp[i], gp[i]);
+  }
+}
+
+// ============================================= fp16 rows beyond the register kernels
+// One 256-thread workgroup per row, element-wise access, fp32 arithmetic: maximum, sum of
+// exponentials, output (the input is read three times; rows this long in fp16 storage are
+// rare, so this is the complete-coverage path, not a tuned one).
+template <typename S, int KIND>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_fwd_generic(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t n)
+{
+  __shared__ float red[kChunkThreads / kWave];
+  const int64_t row = blockIdx.x;
+  const S* xr = x + map.offset(row, ldx);
+  S* yr = y + map.offset(row, ldy);
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  float m = -FLT_MAX;
+  for (int64_t i = threadIdx.x; i < n; i += kChunkThreads) m = fmaxf(m, RowLoad<S>::get(xr + i));
+  m = team_max<kChunkThreads / kWave>(m, red, wv, lane);
+  __syncthreads();
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += kChunkThreads) s += exp_fast(RowLoad<S>::get(xr + i) - m);
+  s = team_sum<kChunkThreads / kWave>(s, red, wv, lane);
+  const float f = 1.0f / s;
+  const float lse = (KIND == kLogSoftmax) ? log_of_sum(s) : 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += kChunkThreads) {
+    const float d = RowLoad<S>::get(xr + i) - m;
+    float r;
+    if (KIND == kLogSoftmax) {
+      r = d - lse;
+    }
+    else {
+      r = f * exp_fast(d);
+      r = __builtin_isnormal(r) ? r : 0.f;
+    }
+    RowLoad<S>::put(yr + i, r);
+  }
+}
+
+template <typename S, int KIND>
+__global__ void __launch_bounds__(kChunkThreads)
+sm_bwd_generic(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx, RowMap map, int64_t n)
+{
+  __shared__ float red[kChunkThreads / kWave];
+  const int64_t row = blockIdx.x;
+  const S* yr = y + map.offset(row, ldy);
+  const S* gr = dy + map.offset(row, lddy);
+  S* dr = dx + map.offset(row, lddx);
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += kChunkThreads)
+    s += (KIND == kLogSoftmax) ? RowLoad<S>::get(gr + i) : RowLoad<S>::get(yr + i) * RowLoad<S>::get(gr + i);
+  s = team_sum<kChunkThreads / kWave>(s, red, wv, lane);
+  // in place (dx aliasing dy): element i is read and written by the same thread, after the sum
+  for (int64_t i = threadIdx.x; i < n; i += kChunkThreads) {
+    const float a = RowLoad<S>::get(yr + i), g = RowLoad<S>::get(gr + i);
+    RowLoad<S>::put(dr + i, (KIND == kLogSoftmax) ? g - exp_fast(a) * s : a * (g - s));
+  }
+}
+
+}  // namespace lbn
