@@ -63,6 +63,43 @@ def test_softmax_family_random(L, case):
 
 
 @pytest.mark.parametrize("case", CASES)
+def test_softmax_f16_and_fused_cross_entropy_random(L, case):
+    """fp16-storage softmax / log-softmax (2e-3 against the fp32 oracle on the rounded values) and
+    the fused softmax + cross-entropy forward (oracle: the composition of the two restatements),
+    dense ground truth and class labels, on the same random shapes."""
+    rng = np.random.default_rng(7000 + case)
+    n, w = draw_length(rng), int(rng.integers(1, 40))
+    pad = int(rng.choice([0, 0, 8, 3]))
+    x, dy = rand(rng, n, w, 0.0, 2.5), rand(rng, n, w)
+    xh = f32(x.astype(np.float16))
+    dyh = f32(dy.astype(np.float16))
+    for kind, layer, fwd, bwd in (("softmax", L.softmax_layer(), orc.softmax_fwd, orc.softmax_bwd),
+                                  ("log_softmax", L.log_softmax_layer(), orc.log_softmax_fwd, orc.log_softmax_bwd)):
+        y = layer.forward(L.DeviceMatrix.from_numpy(xh, dtype=torch.float16, ldim=n + pad)).to_numpy()
+        check(f"random f16 {kind} y {n}x{w}", y, fwd(xh), fwd(f64(xh)), tol=TOL_F16)
+        dx = layer.backward(L.DeviceMatrix.from_numpy(dyh, dtype=torch.float16, ldim=n + pad)).to_numpy()
+        yh = f32(y)
+        check(f"random f16 {kind} dx {n}x{w}", dx, bwd(yh, dyh), bwd(f64(yh), f64(dyh)), tol=TOL_F16)
+    # fused forward: dense ground truth
+    truth = np.asfortranarray(rng.random((n, w)).astype(np.float32))
+    truth[rng.random((n, w)) < 0.5] = 0.0
+    sm, ce = L.softmax_layer(), L.cross_entropy_layer((n,))
+    y, loss = L.softmax_cross_entropy_forward(sm, ce, L.DeviceMatrix.from_numpy(x, ldim=n + pad),
+                                              L.DeviceMatrix.from_numpy(truth, ldim=n + pad))
+    y_ref, y64 = orc.softmax_fwd(x), orc.softmax_fwd(f64(x))
+    check(f"random fused y {n}x{w}", y.to_numpy(), y_ref, y64)
+    check(f"random fused loss {n}x{w}", loss.to_numpy()[0], orc.cross_entropy_fwd(y_ref, truth),
+          orc.cross_entropy_fwd(y64, f64(truth)))
+    # class labels, one per column
+    labels = np.asfortranarray(rng.integers(0, n, (1, w)).astype(np.float32))
+    sm, ce = L.softmax_layer(), L.cross_entropy_layer((n, 1), use_labels=True)
+    y, loss = L.softmax_cross_entropy_forward(sm, ce, L.DeviceMatrix.from_numpy(x, ldim=n + pad),
+                                              L.DeviceMatrix.from_numpy(labels))
+    check(f"random fused labels loss {n}x{w}", loss.to_numpy()[0], orc.cross_entropy_fwd(y_ref, labels, True),
+          orc.cross_entropy_fwd(y64, f64(labels), True))
+
+
+@pytest.mark.parametrize("case", CASES)
 def test_channelwise_softmax_and_instance_norm_random(L, case):
     rng = np.random.default_rng(2000 + case)
     C, cs, w = int(rng.integers(1, 12)), min(draw_length(rng), 6000), int(rng.integers(1, 12))
