@@ -334,7 +334,12 @@ int lbn_batch_norm_bwd_apply_f32(lbn_stream_t stream, int64_t channels, int64_t 
  * (include/lbann/utils/dnn_lib/openmp/softmax.hpp:39-117, :119-181), mode INSTANCE:
  * softmax over each column.  Results that are not normal floats (zero, denormal, NaN)
  * are written as 0, as that code does.  y may alias x and dx may alias dy (the layer
- * can run in place, softmax.hpp:134). */
+ * can run in place, softmax.hpp:134).  Any height, leading dimension and 4-byte aligned
+ * pointer is accepted.  Fastest: columns that start on 16-byte boundaries and a height
+ * that is a multiple of 4.  Columns off that grid move one float at a time, except that
+ * columns of 8000 entries or more still move as 16-byte vectors when the tensors of the
+ * call (x and y; y, dy and dx) have pointers that agree modulo 16 bytes and leading
+ * dimensions that agree modulo 4 entries. */
 size_t lbn_softmax_workspace_bytes(int64_t height, int64_t width);
 int lbn_softmax_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
                         const float* x, int64_t ldx, float* y, int64_t ldy,
