@@ -195,9 +195,10 @@ def main():
         return layer, pred.size, 4, w, cpu, (2 * pred.size * 4, 4 * pred.size * 4)
 
     def build_sm_ce(data):
-        """The classification tail: "forward" is softmax and cross entropy in one call (reads x and
-        the ground truth, writes y: 3 tensors), "backward" the cross-entropy backward that follows
-        (reads y and the ground truth, writes both gradients: 4 tensors)."""
+        """The classification tail, both layers as one call each way: "forward" is softmax and cross
+        entropy (reads x and the ground truth, writes y: 3 tensors), "backward" the gradient with
+        respect to the softmax input straight from y, the ground truth and the loss gradients (reads
+        y and the ground truth, writes dx: 3 tensors; the unfused pair moves 4 + 3 + 4 + 3)."""
         h, w = data["x"].shape
         rng = np.random.default_rng(17)
         truth = np.asfortranarray(rng.uniform(0.0, 1.0, (w, h)).astype(np.float32).T)
@@ -205,7 +206,8 @@ def main():
         sm, ce = L.softmax_layer(), L.cross_entropy_layer((h,))
         x, t = upload(data["x"]), upload(truth)
         y, loss = L.softmax_cross_entropy_forward(sm, ce, x, t)
-        ce.backward(L.DeviceMatrix.from_numpy(dloss.reshape(1, -1)))
+        dl = L.DeviceMatrix.from_numpy(dloss.reshape(1, -1))
+        dx = L.softmax_cross_entropy_backward(sm, ce, dl)
         ws, nb = sm._ws.get(L.capi.lib().lbn_softmax_cross_entropy_fwd_workspace_bytes(h, w), dev)
 
         class tail:
@@ -214,16 +216,18 @@ def main():
                                                              t.ldim, y.Buffer(), y.ldim, loss.Buffer(), loss.ldim, ws, nb)
 
             def bp_call(self):
-                return ce.bp_call()
+                return "lbn_softmax_cross_entropy_bwd_f32", (L._stream(), h, w, 0, 1, y.Buffer(), y.ldim, t.Buffer(),
+                                                             t.ldim, dl.Buffer(), dl.ldim, dx.Buffer(), dx.ldim,
+                                                             L._null(), 0, ws, nb)
 
         def cpu():
             from oracle import cpu_oracle as orc
             t0 = time.perf_counter(); yy = orc.softmax_fwd(data["x"]); orc.cross_entropy_fwd(yy, truth)
             t1 = time.perf_counter()
-            orc.cross_entropy_bwd(yy, truth, dloss); t2 = time.perf_counter()
+            dp, _ = orc.cross_entropy_bwd(yy, truth, dloss); orc.softmax_bwd(yy, dp); t2 = time.perf_counter()
             return t1 - t0, t2 - t1
-        keep = (sm, ce, x, t, y, loss)  # noqa: F841  (owned by the closure for the life of the row)
-        return tail(), h * w, 4, w, cpu, (3 * h * w * 4, 4 * h * w * 4)
+        keep = (sm, ce, x, t, y, loss, dl, dx)  # noqa: F841  (owned by the closure for the life of the row)
+        return tail(), h * w, 4, w, cpu, (3 * h * w * 4, 3 * h * w * 4)
 
     def build_sb(data, kind):
         x, dy = upload(data["x"]), upload(data["dy"])
@@ -296,7 +300,7 @@ def main():
         # not baseline configurations: the layers either side of the path, on the tensors of cfg2 / cfg3
         "extra_cross_entropy": ("CrossEntropy (dense ground truth) fwd+bwd fp32 32768x512 (informational)",
                                 lambda: build_ce(W.cfg2_softmax())),
-        "extra_softmax_cross_entropy": ("Softmax+CrossEntropy fused fwd, CrossEntropy bwd fp32 32768x512 (informational)",
+        "extra_softmax_cross_entropy": ("Softmax+CrossEntropy, each direction one call, fp32 32768x512 (informational)",
                                         lambda: build_sm_ce(W.cfg2_softmax())),
         "extra_entrywise_scale_bias": ("EntrywiseScaleBias fwd+bwd fp32 1048576x64 (informational)",
                                        lambda: build_sb(W.extra_entrywise_batch_norm(), "entrywise")),

@@ -429,7 +429,8 @@ int lbn_channelwise_softmax_bwd_f32(lbn_stream_t stream, int64_t channels,
  * holds one class index per spatial position, stored as a floating-point number in rows
  * [0, spatial_size) of its column; row r of prediction is class r / spatial_size at
  * position r % spatial_size and xhat(r) = 1 where the position's label, converted to
- * int, equals the class, else 0; dground_truth is not written and may be NULL.
+ * int, equals the class, else 0; dground_truth is not written and may be NULL (with a dense
+ * ground truth it is written unless it is NULL).
  * spatial_size is ignored when use_labels == 0. */
 size_t lbn_cross_entropy_fwd_workspace_bytes(int64_t height, int64_t width);
 int lbn_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
@@ -454,7 +455,17 @@ int lbn_cross_entropy_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width
  * from registers instead of from memory.  Rows that fit a workgroup's registers
  * (height a multiple of 4, 16-byte aligned columns, at most 32768 entries) with a dense
  * ground truth, or labels with spatial_size == 1, take the fused kernel; every other shape
- * runs the two layers' kernels back to back inside this call.  The workspace serves both. */
+ * runs the two layers' kernels back to back inside this call.  The workspace serves both.
+ *
+ * Backward of the same pair: dx, the gradient with respect to the softmax input, from y, the
+ * ground truth and dloss (the gradient of column c's loss at dloss[c*ld_dloss]), i.e. what
+ * lbn_cross_entropy_bwd_f32 (cross_entropy.cpp:75-120) followed by lbn_softmax_bwd_f32
+ * (openmp/softmax.hpp:119-181) computes, with the same operations, without writing the
+ * gradient with respect to the prediction in between (three tensors of traffic instead of
+ * seven).  dground_truth (dense ground truth only) is written when it is not NULL.  Shapes
+ * outside the fused kernel run the two kernels inside the call, the first leaving its result
+ * in dx and the second working in place on it; workspace as for lbn_softmax_bwd_f32
+ * (lbn_softmax_workspace_bytes). */
 size_t lbn_softmax_cross_entropy_fwd_workspace_bytes(int64_t height, int64_t width);
 int lbn_softmax_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
                                       int64_t spatial_size,
@@ -462,6 +473,14 @@ int lbn_softmax_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64
                                       const float* ground_truth, int64_t ld_ground_truth,
                                       float* y, int64_t ldy,
                                       float* loss, int64_t ld_loss,
+                                      void* workspace, size_t workspace_bytes);
+int lbn_softmax_cross_entropy_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                                      int64_t spatial_size,
+                                      const float* y, int64_t ldy,
+                                      const float* ground_truth, int64_t ld_ground_truth,
+                                      const float* dloss, int64_t ld_dloss,
+                                      float* dx, int64_t lddx,
+                                      float* dground_truth, int64_t ld_dground_truth,
                                       void* workspace, size_t workspace_bytes);
 
 /* ------------------------------------------------------- scale and bias layers

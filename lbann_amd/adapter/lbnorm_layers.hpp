@@ -872,6 +872,29 @@ public:
                  "cross_entropy_layer::fp_compute_with");
     sm.scratch().after_call(sm.io.stream, "cross_entropy_layer::fp_compute_with");
   }
+  /// bp_compute() of this layer and of `sm` as one call: sm.io.error_signals receives what
+  /// sm.bp_compute() would write after this layer's bp_compute(), and the gradient with respect
+  /// to the prediction (io.error_signals) is never written.  ground_truth_error_signals is
+  /// written when it is set (dense ground truth).  fp32 storage.
+  void bp_compute_with(softmax_layer<Mat>& sm)
+  {
+    static_assert(sizeof(detail::element_t<Mat>) == 4, "the fused backward takes fp32 matrices");
+    if (sm.io.activations != io.prev_activations)
+      throw exception("cross_entropy_layer::bp_compute_with: the softmax layer's output is not this layer's prediction");
+    const Mat& y = *io.prev_activations;
+    const Mat& t = *prev_ground_truth;
+    const Mat& dloss = *io.prev_error_signals;
+    Mat& dx = *sm.io.error_signals;
+    Mat* dt = m_use_labels ? nullptr : ground_truth_error_signals;
+    const size_t bytes = lbn_softmax_workspace_bytes(y.Height(), y.Width());
+    check_status(lbn_softmax_cross_entropy_bwd_f32(sm.io.stream, y.Height(), y.Width(), m_use_labels ? 1 : 0,
+                                                   m_spatial_sample_size, y.LockedBuffer(), y.LDim(),
+                                                   t.LockedBuffer(), t.LDim(), dloss.LockedBuffer(), dloss.LDim(),
+                                                   dx.Buffer(), dx.LDim(), dt ? dt->Buffer() : nullptr,
+                                                   dt ? dt->LDim() : 0, sm.scratch().reserve(bytes, sm.io.stream), bytes),
+                 "cross_entropy_layer::bp_compute_with");
+    sm.scratch().after_call(sm.io.stream, "cross_entropy_layer::bp_compute_with");
+  }
   void bp_compute()
   {
     const Mat& x = *io.prev_activations;

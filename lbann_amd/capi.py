@@ -74,6 +74,7 @@ PROTOTYPES = {
     "lbn_channelwise_softmax_bwd_f32": (cint, [vp, i64, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_softmax_cross_entropy_fwd_workspace_bytes": (sz, [i64, i64]),
     "lbn_softmax_cross_entropy_fwd_f32": (cint, [vp, i64, i64, cint, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
+    "lbn_softmax_cross_entropy_bwd_f32": (cint, [vp, i64, i64, cint, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_cross_entropy_fwd_workspace_bytes": (sz, [i64, i64]),
     "lbn_cross_entropy_fwd_f32": (cint, [vp, i64, i64, cint, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_cross_entropy_bwd_f32": (cint, [vp, i64, i64, cint, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, i64]),

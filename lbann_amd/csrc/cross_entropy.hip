@@ -136,11 +136,11 @@ ce_bwd_dense(CeArgs a)
         d[k] = t[k] > 0.f ? -g * t[k] / v[k] : 0.f;
       }
       Vec16<float>::store(dxc + 4 * j, d);
-      Vec16<float>::store(dtc + 4 * j, dt);
+      if (a.dtruth) Vec16<float>::store(dtc + 4 * j, dt);
     }
     else {
       const float v = xc[j], t = tc[j];
-      dtc[j] = -g * logf(v);
+      if (a.dtruth) dtc[j] = -g * logf(v);
       dxc[j] = t > 0.f ? -g * t / v : 0.f;
     }
   }
@@ -270,7 +270,7 @@ int lbn_cross_entropy_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width
   if (height == 0 || width == 0) return LBN_OK;
   if (!prediction || !ground_truth || !dloss || !dprediction || ld_dloss < 1) return LBN_ERR_INVALID_ARGUMENT;
   if (width > 1 && ld_dprediction < height) return LBN_ERR_INVALID_ARGUMENT;
-  if (!use_labels && (!dground_truth || (width > 1 && ld_dground_truth < height))) return LBN_ERR_INVALID_ARGUMENT;
+  if (!use_labels && dground_truth && width > 1 && ld_dground_truth < height) return LBN_ERR_INVALID_ARGUMENT;
   hipStream_t st = as_stream(stream);
   CeArgs a{};
   a.h = height, a.w = width, a.spatial = use_labels ? spatial_size : 1;

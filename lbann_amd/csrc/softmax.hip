@@ -566,6 +566,35 @@ static int sm_ce_fwd_fused(hipStream_t st, int64_t n, int64_t w, int labels, con
   return -1;
 }
 
+// Backward of the pair in one kernel; -1 when the shape is not one the fused kernel takes.
+static int sm_ce_bwd_fused(hipStream_t st, int64_t n, int64_t w, int labels, const float* y, int64_t ldy,
+                           const float* truth, int64_t ldt, const float* dloss, int64_t ld_dloss, float* dx,
+                           int64_t lddx, float* dtruth, int64_t lddt)
+{
+  const bool vec = (n % 4 == 0) && rows_aligned16(y, n, ldy, 1, w, 4) && rows_aligned16(dx, n, lddx, 1, w, 4) &&
+                   (labels || rows_aligned16(truth, n, ldt, 1, w, 4)) &&
+                   (labels || !dtruth || rows_aligned16(dtruth, n, lddt, 1, w, 4));
+  if (!vec) return -1;
+  const RowConfig c = pick_sm_row_config(n / 4, w);
+  if (!c.tpr) return -1;
+  const unsigned nvec = static_cast<unsigned>(n / 4);
+#define X(TPR, V)                                                                                      \
+  if (c.tpr == TPR && c.v == V) {                                                                      \
+    using B = RowBlock<TPR>;                                                                           \
+    const unsigned grid = static_cast<unsigned>(ceil_div(w, B::kTeams));                               \
+    if (labels)                                                                                        \
+      hipLaunchKernelGGL((sm_ce_bwd_rows<TPR, V, true>), dim3(grid), dim3(B::kThreads), 0, st, y, truth, dloss, dx, \
+                         nullptr, ldy, ldt, ld_dloss, lddx, 0, w, nvec);                               \
+    else                                                                                               \
+      hipLaunchKernelGGL((sm_ce_bwd_rows<TPR, V, false>), dim3(grid), dim3(B::kThreads), 0, st, y, truth, dloss, dx, \
+                         dtruth, ldy, ldt, ld_dloss, lddx, lddt, w, nvec);                             \
+    return launch_status();                                                                            \
+  }
+  LBN_ROW_CASES(X)
+#undef X
+  return -1;
+}
+
 // ------------------------------------------------------------ library-owned scratch
 // Scratch of the entry point that allocates nothing: one array per GPU, part of the code
 // object, so it exists from the moment the library is loaded until the process ends.  The
@@ -693,6 +722,33 @@ int lbn_softmax_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64
   return lbn_cross_entropy_fwd_f32(stream, height, width, use_labels, spatial_size, y, ldy, ground_truth, ld_truth,
                                    loss, ld_loss, room ? workspace_payload(workspace) : nullptr,
                                    room ? workspace_bytes - kWorkspaceHeaderBytes : 0);
+}
+
+int lbn_softmax_cross_entropy_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                                      int64_t spatial_size, const float* y, int64_t ldy, const float* ground_truth,
+                                      int64_t ld_truth, const float* dloss, int64_t ld_dloss, float* dx, int64_t lddx,
+                                      float* dground_truth, int64_t ld_dground_truth, void* workspace,
+                                      size_t workspace_bytes)
+{
+  hipStream_t st = as_stream(stream);
+  if (height < 0 || width < 0) return LBN_ERR_INVALID_ARGUMENT;
+  if (height == 0 || width == 0) return LBN_OK;
+  if (!y || !ground_truth || !dloss || !dx || ld_dloss < 1) return LBN_ERR_INVALID_ARGUMENT;
+  if (use_labels && spatial_size < 1) return LBN_ERR_INVALID_ARGUMENT;
+  if (width > 1 && (ldy < height || lddx < height || ld_truth < (use_labels ? 1 : height))) return LBN_ERR_INVALID_ARGUMENT;
+  if (!use_labels && dground_truth && width > 1 && ld_dground_truth < height) return LBN_ERR_INVALID_ARGUMENT;
+  if (!use_labels || spatial_size == 1) {
+    const int r = sm_ce_bwd_fused(st, height, width, use_labels ? 1 : 0, y, ldy, ground_truth, ld_truth, dloss,
+                                  ld_dloss, dx, lddx, use_labels ? nullptr : dground_truth, ld_dground_truth);
+    if (r >= 0) return r;
+  }
+  // shapes the fused kernel does not take: the cross-entropy backward leaves its gradient in dx,
+  // the softmax backward then runs in place on it (dx may alias dy there)
+  const int status = lbn_cross_entropy_bwd_f32(stream, height, width, use_labels, spatial_size, y, ldy, ground_truth,
+                                               ld_truth, dloss, ld_dloss, dx, lddx,
+                                               use_labels ? nullptr : dground_truth, ld_dground_truth);
+  if (status != LBN_OK) return status;
+  return sm_bwd<kSoftmax>(st, 1, height, height, width, y, ldy, dx, lddx, dx, lddx, workspace, workspace_bytes);
 }
 
 // fp16 storage (IEEE binary16 in memory, fp32 arithmetic); the workspace arguments are there for

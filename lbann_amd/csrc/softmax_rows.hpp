@@ -326,6 +326,92 @@ sm_ce_fwd_rows(const float* x, const float* truth, float* y, float* loss, int64_
   if (t == 0) loss[row * ld_loss] = part;
 }
 
+// Backward of the softmax -> cross-entropy pair in one pass: the gradient with respect to the
+// prediction, dp = -dloss * xhat / y where xhat > 0 and 0 elsewhere (cross_entropy.cpp:75-120), is
+// formed in registers from the ground truth and goes straight into the softmax backward,
+// dx = y * (dp - sum(y * dp)) (openmp/softmax.hpp:119-181), with the operations of the two kernels
+// it replaces (a division, then the products), so a flushed y under a positive xhat gives the
+// same NaN.  dp is never written; dtruth = -dloss * log(y) only when asked for (dense ground truth).
+// LABELS as in sm_ce_fwd_rows.
+template <int TPR, int V, bool LABELS>
+__global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
+sm_ce_bwd_rows(const float* y, const float* truth, const float* dloss, float* dx, float* dtruth, int64_t ldy,
+               int64_t ldt, int64_t ld_dloss, int64_t lddx, int64_t lddt, int64_t rows, unsigned nvec)
+{
+  using B = RowBlock<TPR>;
+  constexpr int W = 4;
+  constexpr bool kSub = TPR < kWave;
+  static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
+  constexpr int NW = kSub ? 1 : B::kWavesPerTeam;
+  __shared__ float red[NW];
+  const unsigned tid = threadIdx.x;
+  const int team = kSub ? static_cast<int>(tid) / TPR : wave_index() / NW;
+  const unsigned t = tid - team * TPR;
+  const int lane = tid & (kWave - 1);
+  const int wv = t / kWave;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * B::kTeams + team;
+  if (B::kTeams > 1 && row >= rows) return;
+
+  const float* yr = y + row * ldy;
+  const float* tr = truth + row * ldt;
+  const float gl = dloss[row * ld_dloss];
+  float a[V][W], g[V][W];
+  int label = -1;
+  if (LABELS) label = static_cast<int>(tr[0]);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = t + i * TPR;
+    if (idx < nvec) {
+      RowIO<float, W>::template load<false>(yr + unsigned(W) * idx, a[i]);
+      if (!LABELS) RowIO<float, W>::template load<false>(tr + unsigned(W) * idx, g[i]);
+    }
+    else {
+#pragma unroll
+      for (int k = 0; k < W; ++k) {
+        a[i][k] = 1.f;  // never divided into: the matching xhat is 0
+        g[i][k] = 0.f;
+      }
+    }
+  }
+  if (!LABELS && dtruth) {
+    float* dtr = dtruth + row * lddt;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = t + i * TPR;
+      if (idx < nvec) {
+        float dt[W];
+#pragma unroll
+        for (int k = 0; k < W; ++k) dt[k] = -gl * logf(a[i][k]);
+        RowIO<float, W>::store(dtr + unsigned(W) * idx, dt);
+      }
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = t + i * TPR;
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      float dp;
+      if (LABELS) dp = (idx < nvec && static_cast<int>(W * idx + k) == label) ? -gl / a[i][k] : 0.f;
+      else dp = g[i][k] > 0.f ? -gl * g[i][k] / a[i][k] : 0.f;
+      g[i][k] = dp;
+      if (idx < nvec) s += a[i][k] * dp;
+    }
+  }
+  s = kSub ? row16_sum(s) : team_sum<NW>(s, red, wv, lane);
+  float* dr = dx + row * lddx;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const unsigned idx = t + i * TPR;
+    if (idx < nvec) {
+#pragma unroll
+      for (int k = 0; k < W; ++k) g[i][k] = a[i][k] * (g[i][k] - s);
+      RowIO<float, W>::store(dr + unsigned(W) * idx, g[i]);
+    }
+  }
+}
+
 // softmax / channelwise: dx = y * (dy - dot(y, dy));  log-softmax: dx = dy - exp(y) * sum(dy)
 // STREAM: bit 0 streams y, bit 1 dy.  FR as in sm_fwd_rows.
 template <typename S, int TPR, int V, int KIND, int STREAM, int W = 16 / sizeof(S), bool FR = false>

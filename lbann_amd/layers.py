@@ -682,6 +682,32 @@ def softmax_cross_entropy_forward(softmax, cross_entropy, x, ground_truth):
     return y, loss
 
 
+def softmax_cross_entropy_backward(softmax, cross_entropy, dloss, want_dtruth=False):
+    """Backward of the pair in one call (lbn_softmax_cross_entropy_bwd_f32): what
+    cross_entropy.backward(dloss) followed by softmax.backward(dprediction) computes, without
+    the gradient with respect to the prediction ever being written.  The layers must have run
+    their forward (together or one after the other).  Returns dx; cross_entropy.error_signals
+    becomes [None, dtruth or None]."""
+    y, truth = cross_entropy.prev_activations
+    if y is not softmax.activations:
+        raise ValueError("the softmax layer's output is not the cross-entropy layer's prediction")
+    cross_entropy.prev_error_signals = dloss
+    dtruth = None
+    if want_dtruth and not cross_entropy.m_use_labels:
+        dtruth = DeviceMatrix(truth.height, truth.width, ldim=truth.ldim, device=cross_entropy.device)
+    cross_entropy.error_signals = [None, dtruth]
+    softmax.prev_error_signals = None
+    softmax.error_signals = DeviceMatrix(y.height, y.width, ldim=y.ldim, device=softmax.device)
+    dx = softmax.error_signals
+    ws, nb = softmax._ws.get(capi.lib().lbn_softmax_workspace_bytes(y.height, y.width), softmax.device)
+    call("lbn_softmax_cross_entropy_bwd_f32", _stream(), y.height, y.width, int(cross_entropy.m_use_labels),
+         cross_entropy.spatial_sample_size, y.Buffer(), y.ldim, truth.Buffer(), truth.ldim, dloss.Buffer(), dloss.ldim,
+         dx.Buffer(), dx.ldim, dtruth.Buffer() if dtruth is not None else _null(),
+         dtruth.ldim if dtruth is not None else 0, ws, nb)
+    _after_call()
+    return dx
+
+
 class gradient_buffer:
     """The optimizer's gradient buffer as the layers see it: optimizer::add_to_gradient and
     get_gradient_buffer (include/lbann/optimizers/optimizer_impl.hpp:207-288) with their status

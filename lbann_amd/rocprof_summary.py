@@ -69,6 +69,7 @@ WORKLOADS = [
     ("sm_fwd_rows<__half, 1024, 4, 0", None, "extra: softmax fp16 storage fwd 32768x512", 2 * _E2 * 2),
     ("sm_bwd_rows<__half, 1024, 4, 0", None, "extra: softmax fp16 storage bwd", 3 * _E2 * 2),
     ("sm_ce_fwd_rows<1024, 8, false>", None, "extra: softmax + cross entropy fwd 32768x512 (x, truth, y)", 3 * _E2 * 4),
+    ("sm_ce_bwd_rows<1024, 8, false>", None, "extra: softmax + cross entropy bwd (y, truth, dx)", 3 * _E2 * 4),
     ("ce_fwd_dense", None, "extra: cross entropy fwd 32768x512 (x, truth)", 2 * _E2 * 4),
     ("ce_bwd_dense", None, "extra: cross entropy bwd (x, truth, dx, dtruth)", 4 * _E2 * 4),
     ("esb_fwd_tile", None, "extra: entry-wise scale/bias fwd 1048576x64", 2 * 67108864 * 4),

@@ -278,9 +278,10 @@ int drv_cross_entropy(const int64_t* pred_dims, const int64_t* truth_dims, int n
 }
 
 // softmax followed by cross entropy through the fused forward, then both layers' backward
+// (fused_bwd: as one call, which leaves dy untouched)
 int drv_softmax_cross_entropy(const int64_t* pred_dims, const int64_t* truth_dims, int nd, int use_labels, int64_t h,
                               int64_t ht, int64_t w, float* x, float* y, float* truth, float* loss, float* dloss,
-                              float* dy, float* dx, float* dtruth, void* stream, char* err, int errlen)
+                              float* dy, float* dx, float* dtruth, int fused_bwd, void* stream, char* err, int errlen)
 {
   try {
     softmax_layer<> sm;
@@ -294,8 +295,13 @@ int drv_softmax_cross_entropy(const int64_t* pred_dims, const int64_t* truth_dim
     ce.io.prev_error_signals = &mdl; ce.io.error_signals = &mdy; ce.ground_truth_error_signals = &mdt;
     sm.io.stream = ce.io.stream = static_cast<hipStream_t>(stream);
     ce.fp_compute_with(sm);
-    ce.bp_compute();
-    sm.bp_compute();
+    if (fused_bwd) {
+      ce.bp_compute_with(sm);
+    }
+    else {
+      ce.bp_compute();
+      sm.bp_compute();
+    }
     sm.check_cluster_waits();
     check_hip(hipStreamSynchronize(sm.io.stream), "sync");
     return 0;

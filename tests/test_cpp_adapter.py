@@ -220,16 +220,23 @@ def test_adapter_layers_match_oracle():
         mdy, mdx, mdt = DeviceMatrix(h, w), DeviceMatrix(h, w), DeviceMatrix(truth.shape[0], w)
         pa, nd = _dims(pdims)
         ta, _ = _dims(tdims)
-        rc = d.drv_softmax_cross_entropy(pa, ta, cint(nd), cint(use_labels), i64(h), i64(truth.shape[0]), i64(w),
-                                         mx.Buffer(), my.Buffer(), mt.Buffer(), ml.Buffer(), mdl.Buffer(), mdy.Buffer(),
-                                         mdx.Buffer(), mdt.Buffer(), st, err, cint(512))
-        assert rc == 0, err.value
-        y_ref = orc.softmax_fwd(x)
-        check("adapter softmax+ce y", my.to_numpy(), y_ref)
-        check("adapter softmax+ce loss", ml.to_numpy()[0], orc.cross_entropy_fwd(y_ref, truth, bool(use_labels)))
-        dp_ref, _ = orc.cross_entropy_bwd(y_ref, truth, dloss, bool(use_labels))
-        check("adapter softmax+ce dprediction", mdy.to_numpy(), dp_ref)
-        check("adapter softmax+ce dx", mdx.to_numpy(), orc.softmax_bwd(y_ref, dp_ref))
+        for fused_bwd in (0, 1):
+            mdy.tensor.fill_(-3.0)
+            rc = d.drv_softmax_cross_entropy(pa, ta, cint(nd), cint(use_labels), i64(h), i64(truth.shape[0]), i64(w),
+                                             mx.Buffer(), my.Buffer(), mt.Buffer(), ml.Buffer(), mdl.Buffer(),
+                                             mdy.Buffer(), mdx.Buffer(), mdt.Buffer(), cint(fused_bwd), st, err, cint(512))
+            assert rc == 0, err.value
+            y_ref = orc.softmax_fwd(x)
+            check("adapter softmax+ce y", my.to_numpy(), y_ref)
+            check("adapter softmax+ce loss", ml.to_numpy()[0], orc.cross_entropy_fwd(y_ref, truth, bool(use_labels)))
+            dp_ref, dt_ref = orc.cross_entropy_bwd(y_ref, truth, dloss, bool(use_labels))
+            if fused_bwd:
+                assert torch.all(mdy.tensor == -3.0).item()   # the gradient w.r.t. the prediction is never written
+            else:
+                check("adapter softmax+ce dprediction", mdy.to_numpy(), dp_ref)
+            check("adapter softmax+ce dx", mdx.to_numpy(), orc.softmax_bwd(y_ref, dp_ref))
+            if not use_labels:
+                check("adapter softmax+ce dtruth", mdt.to_numpy(), dt_ref)
 
     # ---- scale/bias layers on (8, 12, 12) x 10
     dims, w = (8, 12, 12), 10

@@ -216,7 +216,9 @@ def test_neighbour_layers_empty_and_rejected_arguments(L):
     assert lib.lbn_entrywise_scale_bias_fwd_f32(st, 8, 4, p, 8, p, 8, p, 4) == capi.LBN_ERR_INVALID_ARGUMENT
     assert lib.lbn_channelwise_scale_bias_bwd_f32(st, 2, 4, 4, p, 8, p, 8, null, 8, p, 2, p, 2, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT
     assert lib.lbn_cross_entropy_fwd_f32(st, 8, 4, 1, 0, p, 8, p, 8, p, 1, null, 0) == capi.LBN_ERR_INVALID_ARGUMENT
-    assert lib.lbn_cross_entropy_bwd_f32(st, 8, 4, 0, 1, p, 8, p, 8, p, 1, p, 8, null, 8) == capi.LBN_ERR_INVALID_ARGUMENT
+    # dground_truth is optional (not written when NULL); given, its leading dimension must hold a column
+    assert lib.lbn_cross_entropy_bwd_f32(st, 8, 4, 0, 1, p, 8, p, 8, p, 1, p, 8, null, 8) == 0
+    assert lib.lbn_cross_entropy_bwd_f32(st, 8, 4, 0, 1, p, 8, p, 8, p, 1, p, 8, p, 4) == capi.LBN_ERR_INVALID_ARGUMENT
     big = torch.zeros(64 * 8192, device="cuda")
     pb = capi.vp(big.data_ptr())
     assert lib.lbn_entrywise_scale_bias_bwd_workspace_bytes(64, 8192) > 0

@@ -1,4 +1,5 @@
-"""GPU parity of the fused softmax -> cross-entropy forward (lbn_softmax_cross_entropy_fwd_f32).
+"""GPU parity of the fused softmax -> cross-entropy forward and backward
+(lbn_softmax_cross_entropy_fwd_f32, lbn_softmax_cross_entropy_bwd_f32).
 
 The oracle is the composition of the two restatements: cross_entropy_fwd(softmax_fwd(x), truth)
 (src/layers/activations/softmax.cpp:43-109 followed by src/layers/loss/cross_entropy.cpp:35-73).
@@ -136,6 +137,80 @@ def test_backward_after_fused_forward(L):
     check("softmax_ce bwd dprediction", dpred.to_numpy(), dp_ref)
     check("softmax_ce bwd dtruth", dtruth.to_numpy(), dt_ref)
     check("softmax_ce bwd dx", dx, orc.softmax_bwd(y, dp_ref))
+
+
+@pytest.mark.parametrize("h,w,pad", DENSE_SHAPES)
+@pytest.mark.parametrize("want_dtruth", [False, True])
+def test_backward_dense(L, h, w, pad, want_dtruth):
+    """Oracle: softmax_bwd(y, cross_entropy_bwd(y, truth, dloss).dprediction), the composition of
+    the two restatements (cross_entropy.cpp:75-120, openmp/softmax.hpp:119-181); also against the
+    library's own two calls."""
+    rng = np.random.default_rng(h * 17 + w)
+    x, t = rand(rng, h, w, 0, 2), dense_truth(rng, h, w, "soft")
+    g = rng.standard_normal(w).astype(np.float32)
+    ld = h + pad if pad else None
+    sm, ce = L.softmax_layer(), L.cross_entropy_layer((h,))
+    y, _ = L.softmax_cross_entropy_forward(sm, ce, L.DeviceMatrix.from_numpy(x, ldim=ld),
+                                           L.DeviceMatrix.from_numpy(t, ldim=ld))
+    yh = y.to_numpy()
+    dx = L.softmax_cross_entropy_backward(sm, ce, L.DeviceMatrix.from_numpy(g.reshape(1, w)), want_dtruth)
+    dp_ref, dt_ref = orc.cross_entropy_bwd(yh, t, g)
+    y64 = yh.astype(np.float64)
+    dp64, dt64 = orc.cross_entropy_bwd(np.asfortranarray(y64), np.asfortranarray(t.astype(np.float64)), g.astype(np.float64))
+    check(f"softmax_ce bwd dense {h}x{w} dx", dx.to_numpy(), orc.softmax_bwd(yh, dp_ref),
+          orc.softmax_bwd(np.asfortranarray(y64), dp64))
+    if want_dtruth:
+        check(f"softmax_ce bwd dense {h}x{w} dtruth", ce.error_signals[1].to_numpy(), dt_ref, dt64)
+    else:
+        assert ce.error_signals[1] is None
+    # the two calls one after the other, on the same y
+    sm2, ce2 = L.softmax_layer(), L.cross_entropy_layer((h,))
+    L.softmax_cross_entropy_forward(sm2, ce2, L.DeviceMatrix.from_numpy(x, ldim=ld), L.DeviceMatrix.from_numpy(t, ldim=ld))
+    dpred, _ = ce2.backward(L.DeviceMatrix.from_numpy(g.reshape(1, w)))
+    dx2 = sm2.backward(dpred).to_numpy()
+    check(f"softmax_ce bwd dense {h}x{w} dx vs two calls", dx.to_numpy(), dx2, orc.softmax_bwd(np.asfortranarray(y64), dp64))
+
+
+@pytest.mark.parametrize("classes,spatial,w", [(10, 1, 300), (1000, 1, 64), (1024, 1, 33), (50257, 1, 6), (32768, 1, 3),
+                                               (4, 64, 9), (21, 100, 7)])
+def test_backward_labels(L, classes, spatial, w):
+    rng = np.random.default_rng(classes * 3 + spatial)
+    h = classes * spatial
+    x = rand(rng, h, w, 0, 2)
+    t = np.asfortranarray(rng.integers(0, classes, (spatial, w)).astype(np.float32))
+    t[0, 0] = -1.0
+    g = rng.standard_normal(w).astype(np.float32)
+    sm, ce = L.softmax_layer(), L.cross_entropy_layer((classes, spatial), True)
+    y, _ = L.softmax_cross_entropy_forward(sm, ce, L.DeviceMatrix.from_numpy(x), L.DeviceMatrix.from_numpy(t))
+    yh = y.to_numpy()
+    dx = L.softmax_cross_entropy_backward(sm, ce, L.DeviceMatrix.from_numpy(g.reshape(1, w)))
+    dp_ref, _ = orc.cross_entropy_bwd(yh, t, g, True)
+    y64 = np.asfortranarray(yh.astype(np.float64))
+    dp64, _ = orc.cross_entropy_bwd(y64, np.asfortranarray(t.astype(np.float64)), g.astype(np.float64), True)
+    check(f"softmax_ce bwd labels {classes}x{spatial}x{w} dx", dx.to_numpy(), orc.softmax_bwd(yh, dp_ref),
+          orc.softmax_bwd(y64, dp64))
+
+
+def test_backward_flushed_entry_gives_the_same_nan(L):
+    """y flushed to zero under xhat > 0: the gradient with respect to the prediction is -inf there
+    and the softmax backward turns the column into NaN, fused or not."""
+    h, w = 1024, 3
+    x = np.zeros((h, w), np.float32, order="F")
+    x[0, :] = 200.0
+    t = np.zeros((h, w), np.float32, order="F")
+    t[0, 0] = 1.0
+    t[5, 1] = 1.0       # flushed entry under a positive xhat
+    g = np.ones(w, np.float32)
+    sm, ce = L.softmax_layer(), L.cross_entropy_layer((h,))
+    y, _ = L.softmax_cross_entropy_forward(sm, ce, L.DeviceMatrix.from_numpy(x), L.DeviceMatrix.from_numpy(t))
+    yh = y.to_numpy()
+    dx = L.softmax_cross_entropy_backward(sm, ce, L.DeviceMatrix.from_numpy(g.reshape(1, w))).to_numpy()
+    with np.errstate(all="ignore"):
+        ref = orc.softmax_bwd(yh, orc.cross_entropy_bwd(yh, t, g)[0])
+    assert np.array_equal(np.isnan(dx), np.isnan(ref))
+    assert np.isnan(dx[:, 1]).all() and np.isfinite(dx[:, 0]).all() and np.all(dx[:, 2] == 0)
+    ok = ~np.isnan(ref)
+    check("softmax_ce bwd flushed finite part", np.where(ok, dx, 0), np.where(ok, ref, 0))
 
 
 def test_empty_and_bad_arguments(L):
