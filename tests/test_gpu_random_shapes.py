@@ -90,6 +90,15 @@ def test_softmax_f16_and_fused_cross_entropy_random(L, case):
     check(f"random fused y {n}x{w}", y.to_numpy(), y_ref, y64)
     check(f"random fused loss {n}x{w}", loss.to_numpy()[0], orc.cross_entropy_fwd(y_ref, truth),
           orc.cross_entropy_fwd(y64, f64(truth)))
+    # fused backward: the composition of the two restated backward passes on the y the GPU wrote
+    g = rng.standard_normal(w).astype(np.float32)
+    yg = y.to_numpy()
+    dx = L.softmax_cross_entropy_backward(sm, ce, L.DeviceMatrix.from_numpy(g.reshape(1, w)), want_dtruth=bool(case % 2))
+    dp_ref, dt_ref = orc.cross_entropy_bwd(yg, truth, g)
+    dp64, dt64 = orc.cross_entropy_bwd(f64(yg), f64(truth), g.astype(np.float64))
+    check(f"random fused dx {n}x{w}", dx.to_numpy(), orc.softmax_bwd(yg, dp_ref), orc.softmax_bwd(f64(yg), dp64))
+    if case % 2:
+        check(f"random fused dtruth {n}x{w}", ce.error_signals[1].to_numpy(), dt_ref, dt64)
     # class labels, one per column
     labels = np.asfortranarray(rng.integers(0, n, (1, w)).astype(np.float32))
     sm, ce = L.softmax_layer(), L.cross_entropy_layer((n, 1), use_labels=True)
@@ -97,6 +106,11 @@ def test_softmax_f16_and_fused_cross_entropy_random(L, case):
                                               L.DeviceMatrix.from_numpy(labels))
     check(f"random fused labels loss {n}x{w}", loss.to_numpy()[0], orc.cross_entropy_fwd(y_ref, labels, True),
           orc.cross_entropy_fwd(y64, f64(labels), True))
+    yg = y.to_numpy()
+    dx = L.softmax_cross_entropy_backward(sm, ce, L.DeviceMatrix.from_numpy(g.reshape(1, w)))
+    dp_ref, _ = orc.cross_entropy_bwd(yg, labels, g, True)
+    dp64, _ = orc.cross_entropy_bwd(f64(yg), f64(labels), g.astype(np.float64), True)
+    check(f"random fused labels dx {n}x{w}", dx.to_numpy(), orc.softmax_bwd(yg, dp_ref), orc.softmax_bwd(f64(yg), dp64))
 
 
 @pytest.mark.parametrize("case", CASES)
