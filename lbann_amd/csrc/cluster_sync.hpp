@@ -32,6 +32,7 @@
 #include <chrono>
 #include <cstdint>
 #include <mutex>
+#include <thread>
 
 #include "device_utils.hpp"
 #include "host_utils.hpp"
@@ -465,7 +466,7 @@ class ClusterLaunchGuard {
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
     state_ = &states()[dev];
     state_->mu.lock();
-    if (capturing_ || !state_->have_last || state_->last == st) return;
+    if (capturing_ || !state_->have_last || same_stream_as_last()) return;
     if (!state_->several) {
       state_->several = true;
       make_event(*state_);
@@ -474,6 +475,9 @@ class ClusterLaunchGuard {
     else if (state_->done) {
       (void)hipStreamWaitEvent(st, state_->done, 0);
     }
+    else {
+      (void)hipDeviceSynchronize();  // no event could be created: order the launches the slow way
+    }
   }
   ~ClusterLaunchGuard()
   {
@@ -481,6 +485,7 @@ class ClusterLaunchGuard {
       if (state_->several && state_->done) (void)hipEventRecord(state_->done, st_);
       state_->last = st_;
       state_->have_last = true;
+      if (st_ == hipStreamPerThread) state_->last_thread = std::this_thread::get_id();
     }
     state_->mu.unlock();
   }
@@ -503,10 +508,17 @@ class ClusterLaunchGuard {
   struct State {
     std::mutex mu;
     hipStream_t last = nullptr;
+    std::thread::id last_thread;  // whose hipStreamPerThread `last` is, when it is that handle
     bool have_last = false;
     bool several = false;      // cluster launches have come from more than one stream
     hipEvent_t done = nullptr;  // recorded after every cluster launch once `several` is set
   };
+  // hipStreamPerThread is one handle for a different stream in every host thread.
+  bool same_stream_as_last() const
+  {
+    if (state_->last != st_) return false;
+    return st_ != hipStreamPerThread || state_->last_thread == std::this_thread::get_id();
+  }
   static State* states()
   {
     static State s[kMaxDevices];

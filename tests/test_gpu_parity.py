@@ -994,3 +994,48 @@ def test_cluster_kernels_enqueued_on_two_streams_without_waiting(L):
     for y in yb:
         assert np.array_equal(y.to_numpy(), bn_ref)
 
+
+
+def test_cluster_kernels_from_two_host_threads_on_the_per_thread_stream(L, monkeypatch):
+    """hipStreamPerThread is one handle that names a different stream in every host thread, so two
+    threads that pass it enqueue on two streams: the library must still keep their cluster kernels
+    apart.  Every result equals the one computed alone and no wait runs out."""
+    import threading
+
+    from lbann_amd import capi
+
+    rng = np.random.default_rng(23)
+    xs = rand(rng, 262144, 8)                     # a few long rows: row clusters
+    xb = rand(rng, 64 * 784, 64, 2.0, 3.0)        # channel clusters
+    sm_ref = L.softmax_layer().forward(L.DeviceMatrix.from_numpy(xs)).to_numpy()
+    bn_ref = L.batch_normalization_layer((64, 28, 28)).forward(L.DeviceMatrix.from_numpy(xb)).to_numpy()
+    dxs, dxb = L.DeviceMatrix.from_numpy(xs), L.DeviceMatrix.from_numpy(xb)
+    reps = 12
+    sms = [L.softmax_layer() for _ in range(reps)]
+    bns = [L.batch_normalization_layer((64, 28, 28)) for _ in range(reps)]
+    # first calls on the ordinary stream: the workspaces are allocated outside the threads
+    ys = [m.forward(dxs) for m in sms]
+    yb = [m.forward(dxb) for m in bns]
+    torch.cuda.synchronize()
+    ys, yb = [None] * reps, [None] * reps
+    monkeypatch.setattr(L, "_stream", lambda: capi.vp(2))  # hipStreamPerThread
+    errors = []
+
+    def run(layers, x, out):
+        try:
+            torch.cuda.set_device(0)
+            for i, m in enumerate(layers):
+                out[i] = m.forward(x)
+        except Exception as e:  # surfaced below: an exception in a thread would otherwise be lost
+            errors.append(e)
+
+    ta = threading.Thread(target=run, args=(sms, dxs, ys))
+    tb = threading.Thread(target=run, args=(bns, dxb, yb))
+    ta.start(); tb.start(); ta.join(); tb.join()
+    torch.cuda.synchronize()
+    monkeypatch.undo()
+    assert not errors, errors
+    for y in ys:
+        assert np.array_equal(y.to_numpy(), sm_ref)
+    for y in yb:
+        assert np.array_equal(y.to_numpy(), bn_ref)
