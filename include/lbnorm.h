@@ -447,6 +447,28 @@ int lbn_cross_entropy_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width
                               float* dprediction, int64_t ld_dprediction,
                               float* dground_truth, int64_t ld_dground_truth);
 
+/* fp16 storage: the reference instantiates cross_entropy_layer for half precision too
+ * (src/layers/loss/cross_entropy.cpp:157-166, LBANN_INSTANTIATE_CPU_HALF).  Every matrix
+ * (prediction, ground truth, loss, dloss and the two gradients) is IEEE binary16 in memory;
+ * logarithms, products and the sum over a column are fp32, where the reference's half
+ * instantiation also accumulates in half; results are rounded to nearest even on store (a
+ * loss or gradient beyond 65504 becomes infinite).  Labels are class indices stored as
+ * binary16, exact up to 2048.  Same arguments as the _f32 entry points, leading dimensions
+ * in elements; the workspace (fp32 partial sums) has the same size. */
+int lbn_cross_entropy_fwd_f16(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                              int64_t spatial_size,
+                              const void* prediction, int64_t ld_prediction,
+                              const void* ground_truth, int64_t ld_ground_truth,
+                              void* loss, int64_t ld_loss,
+                              void* workspace, size_t workspace_bytes);
+int lbn_cross_entropy_bwd_f16(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                              int64_t spatial_size,
+                              const void* prediction, int64_t ld_prediction,
+                              const void* ground_truth, int64_t ld_ground_truth,
+                              const void* dloss, int64_t ld_dloss,
+                              void* dprediction, int64_t ld_dprediction,
+                              void* dground_truth, int64_t ld_dground_truth);
+
 /* Softmax forward and the cross-entropy forward of its output in one pass: y as
  * lbn_softmax_fwd_f32 writes it (softmax.cpp:43-109, flush included) and loss as
  * lbn_cross_entropy_fwd_f32(prediction = y) gives it (cross_entropy.cpp:35-73), for the

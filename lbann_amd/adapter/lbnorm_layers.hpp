@@ -847,10 +847,17 @@ public:
     const Mat& t = *prev_ground_truth;
     Mat& loss = *io.activations;
     const size_t bytes = lbn_cross_entropy_fwd_workspace_bytes(x.Height(), x.Width());
-    check_status(lbn_cross_entropy_fwd_f32(io.stream, x.Height(), x.Width(), m_use_labels ? 1 : 0,
-                                           m_spatial_sample_size, x.LockedBuffer(), x.LDim(), t.LockedBuffer(),
-                                           t.LDim(), loss.Buffer(), loss.LDim(), m_ws.reserve(bytes, io.stream), bytes),
-                 "cross_entropy_layer::fp_compute");
+    // the reference instantiates the layer for half precision too (cross_entropy.cpp:157-166)
+    int status;
+    if constexpr (sizeof(detail::element_t<Mat>) == 2)
+      status = lbn_cross_entropy_fwd_f16(io.stream, x.Height(), x.Width(), m_use_labels ? 1 : 0,
+                                         m_spatial_sample_size, x.LockedBuffer(), x.LDim(), t.LockedBuffer(),
+                                         t.LDim(), loss.Buffer(), loss.LDim(), m_ws.reserve(bytes, io.stream), bytes);
+    else
+      status = lbn_cross_entropy_fwd_f32(io.stream, x.Height(), x.Width(), m_use_labels ? 1 : 0,
+                                         m_spatial_sample_size, x.LockedBuffer(), x.LDim(), t.LockedBuffer(),
+                                         t.LDim(), loss.Buffer(), loss.LDim(), m_ws.reserve(bytes, io.stream), bytes);
+    check_status(status, "cross_entropy_layer::fp_compute");
   }
   /// fp_compute() of `sm`, a softmax layer whose output is this layer's prediction
   /// (sm.io.activations == io.prev_activations), and this layer's own, as one call: the
@@ -902,11 +909,18 @@ public:
     const Mat& dy = *io.prev_error_signals;
     Mat& dx = *io.error_signals;
     Mat* dt = m_use_labels ? nullptr : ground_truth_error_signals;
-    check_status(lbn_cross_entropy_bwd_f32(io.stream, x.Height(), x.Width(), m_use_labels ? 1 : 0,
-                                           m_spatial_sample_size, x.LockedBuffer(), x.LDim(), t.LockedBuffer(),
-                                           t.LDim(), dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
-                                           dt ? dt->Buffer() : nullptr, dt ? dt->LDim() : 0),
-                 "cross_entropy_layer::bp_compute");
+    int status;
+    if constexpr (sizeof(detail::element_t<Mat>) == 2)
+      status = lbn_cross_entropy_bwd_f16(io.stream, x.Height(), x.Width(), m_use_labels ? 1 : 0,
+                                         m_spatial_sample_size, x.LockedBuffer(), x.LDim(), t.LockedBuffer(),
+                                         t.LDim(), dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+                                         dt ? dt->Buffer() : nullptr, dt ? dt->LDim() : 0);
+    else
+      status = lbn_cross_entropy_bwd_f32(io.stream, x.Height(), x.Width(), m_use_labels ? 1 : 0,
+                                         m_spatial_sample_size, x.LockedBuffer(), x.LDim(), t.LockedBuffer(),
+                                         t.LDim(), dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+                                         dt ? dt->Buffer() : nullptr, dt ? dt->LDim() : 0);
+    check_status(status, "cross_entropy_layer::bp_compute");
   }
 private:
   bool m_use_labels;

@@ -78,6 +78,8 @@ PROTOTYPES = {
     "lbn_cross_entropy_fwd_workspace_bytes": (sz, [i64, i64]),
     "lbn_cross_entropy_fwd_f32": (cint, [vp, i64, i64, cint, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_cross_entropy_bwd_f32": (cint, [vp, i64, i64, cint, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, i64]),
+    "lbn_cross_entropy_fwd_f16": (cint, [vp, i64, i64, cint, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
+    "lbn_cross_entropy_bwd_f16": (cint, [vp, i64, i64, cint, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, i64]),
     "lbn_entrywise_scale_bias_fwd_f32": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64]),
     "lbn_entrywise_scale_bias_bwd_workspace_bytes": (sz, [i64, i64]),
     "lbn_entrywise_scale_bias_bwd_f32": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, sz]),

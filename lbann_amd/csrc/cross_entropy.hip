@@ -27,17 +27,19 @@ constexpr int kCeThreads = 256;
 constexpr int kCeWaves = kCeThreads / kWave;
 constexpr int kCeMaxParts = 64;
 
+// S: the storage type of every matrix of the layer (float, or __half with fp32 arithmetic).
+template <typename S>
 struct CeArgs {
   int64_t h, w, spatial;
-  const float* x;
-  const float* truth;
+  const S* x;
+  const S* truth;
   int64_t ldx, ldt;
-  float* loss;  // forward: element c at loss[c*ld_loss]
+  S* loss;  // forward: element c at loss[c*ld_loss]
   int64_t ld_loss;
-  const float* dy;  // backward: element c at dy[c*lddy]
+  const S* dy;  // backward: element c at dy[c*lddy]
   int64_t lddy;
-  float* dx;
-  float* dtruth;
+  S* dx;
+  S* dtruth;
   int64_t lddx, lddt;
   float* part;  // [w][P]
 };
@@ -48,140 +50,148 @@ __device__ __forceinline__ float ce_term(float xhat, float x) { return xhat > 0.
 // (`const int truth_label = local_ground_truth(offset, col)`, cross_entropy.cpp:58).
 __device__ __forceinline__ int64_t ce_label(float v) { return static_cast<int64_t>(static_cast<int>(v)); }
 
-template <int T>
-__device__ __forceinline__ void ce_store_partial(const CeArgs& a, float sum, float* red)
+template <int T, typename S>
+__device__ __forceinline__ void ce_store_partial(const CeArgs<S>& a, float sum, float* red)
 {
   sum = team_sum<T / kWave>(sum, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
   if (threadIdx.x == 0) {
     const int64_t c = blockIdx.x;
-    if (gridDim.y == 1) a.loss[c * a.ld_loss] = sum;
+    if (gridDim.y == 1) Vec16<S>::store1(a.loss + c * a.ld_loss, sum);
     else a.part[c * gridDim.y + blockIdx.y] = sum;
   }
 }
 
-template <bool VEC, int T>
+template <bool VEC, int T, typename S>
 __global__ void __launch_bounds__(T)
-ce_fwd_dense(CeArgs a)
+ce_fwd_dense(CeArgs<S> a)
 {
+  constexpr int VE = Vec16<S>::N;
   __shared__ float red[T / kWave];
   const int64_t c = blockIdx.x;
-  const float* xc = a.x + c * a.ldx;
-  const float* tc = a.truth + c * a.ldt;
-  const int64_t n = VEC ? a.h / 4 : a.h;
+  const S* xc = a.x + c * a.ldx;
+  const S* tc = a.truth + c * a.ldt;
+  const int64_t n = VEC ? a.h / VE : a.h;
   const int64_t step = static_cast<int64_t>(gridDim.y) * T;
   float sum = 0.f;
   for (int64_t j = static_cast<int64_t>(blockIdx.y) * T + threadIdx.x; j < n; j += step) {
     if (VEC) {
-      float v[4], t[4];
-      Vec16<float>::load(xc + 4 * j, v);
-      Vec16<float>::load(tc + 4 * j, t);
+      float v[VE], t[VE];
+      Vec16<S>::load(xc + VE * j, v);
+      Vec16<S>::load(tc + VE * j, t);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) sum += ce_term(t[k], v[k]);
+      for (int k = 0; k < VE; ++k) sum += ce_term(t[k], v[k]);
     }
     else {
-      sum += ce_term(tc[j], xc[j]);
+      sum += ce_term(Vec16<S>::load1(tc + j), Vec16<S>::load1(xc + j));
     }
   }
   ce_store_partial<T>(a, sum, red);
 }
 
 // One thread per spatial position: gather the entry of x its label points at.
+template <typename S>
 __global__ void __launch_bounds__(kCeThreads)
-ce_fwd_labels(CeArgs a)
+ce_fwd_labels(CeArgs<S> a)
 {
   __shared__ float red[kCeWaves];
   const int64_t c = blockIdx.x;
-  const float* xc = a.x + c * a.ldx;
-  const float* tc = a.truth + c * a.ldt;
+  const S* xc = a.x + c * a.ldx;
+  const S* tc = a.truth + c * a.ldt;
   const int64_t positions = a.spatial < a.h ? a.spatial : a.h;
   const int64_t step = static_cast<int64_t>(gridDim.y) * kCeThreads;
   float sum = 0.f;
   for (int64_t o = static_cast<int64_t>(blockIdx.y) * kCeThreads + threadIdx.x; o < positions; o += step) {
-    const int64_t label = ce_label(tc[o]);
+    const int64_t label = ce_label(Vec16<S>::load1(tc + o));
     const int64_t r = label * a.spatial + o;
-    if (label >= 0 && r < a.h) sum += -logf(xc[r]);
+    if (label >= 0 && r < a.h) sum += -logf(Vec16<S>::load1(xc + r));
   }
   ce_store_partial<kCeThreads>(a, sum, red);
 }
 
+template <typename S>
 __global__ void __launch_bounds__(kWave)
-ce_merge_parts(int P, const float* __restrict__ part, float* __restrict__ loss, int64_t ld_loss)
+ce_merge_parts(int P, const float* __restrict__ part, S* __restrict__ loss, int64_t ld_loss)
 {
   const int64_t c = blockIdx.x;
   const int lane = threadIdx.x;
   const float v = wave_sum(lane < P ? part[c * P + lane] : 0.f);
-  if (lane == 0) loss[c * ld_loss] = v;
+  if (lane == 0) Vec16<S>::store1(loss + c * ld_loss, v);
 }
 
-template <bool VEC>
+template <bool VEC, typename S>
 __global__ void __launch_bounds__(kCeThreads)
-ce_bwd_dense(CeArgs a)
+ce_bwd_dense(CeArgs<S> a)
 {
+  constexpr int VE = Vec16<S>::N;
   const int64_t c = blockIdx.x;
-  const float g = a.dy[c * a.lddy];
-  const float* xc = a.x + c * a.ldx;
-  const float* tc = a.truth + c * a.ldt;
-  float* dxc = a.dx + c * a.lddx;
-  float* dtc = a.dtruth + c * a.lddt;
-  const int64_t n = VEC ? a.h / 4 : a.h;
+  const float g = Vec16<S>::load1(a.dy + c * a.lddy);
+  const S* xc = a.x + c * a.ldx;
+  const S* tc = a.truth + c * a.ldt;
+  S* dxc = a.dx + c * a.lddx;
+  S* dtc = a.dtruth + c * a.lddt;
+  const int64_t n = VEC ? a.h / VE : a.h;
   const int64_t step = static_cast<int64_t>(gridDim.y) * kCeThreads;
   for (int64_t j = static_cast<int64_t>(blockIdx.y) * kCeThreads + threadIdx.x; j < n; j += step) {
     if (VEC) {
-      float v[4], t[4], d[4], dt[4];
-      Vec16<float>::load(xc + 4 * j, v);
-      Vec16<float>::load(tc + 4 * j, t);
+      float v[VE], t[VE], d[VE], dt[VE];
+      Vec16<S>::load(xc + VE * j, v);
+      Vec16<S>::load(tc + VE * j, t);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
+      for (int k = 0; k < VE; ++k) {
         dt[k] = -g * logf(v[k]);
         d[k] = t[k] > 0.f ? -g * t[k] / v[k] : 0.f;
       }
-      Vec16<float>::store(dxc + 4 * j, d);
-      if (a.dtruth) Vec16<float>::store(dtc + 4 * j, dt);
+      Vec16<S>::store(dxc + VE * j, d);
+      if (a.dtruth) Vec16<S>::store(dtc + VE * j, dt);
     }
     else {
-      const float v = xc[j], t = tc[j];
-      if (a.dtruth) dtc[j] = -g * logf(v);
-      dxc[j] = t > 0.f ? -g * t / v : 0.f;
+      const float v = Vec16<S>::load1(xc + j), t = Vec16<S>::load1(tc + j);
+      if (a.dtruth) Vec16<S>::store1(dtc + j, -g * logf(v));
+      Vec16<S>::store1(dxc + j, t > 0.f ? -g * t / v : 0.f);
     }
   }
 }
 
-// VEC: spatial is a multiple of 4, so the 4 rows of a vector share a class.
-template <bool VEC>
+// VEC: spatial is a multiple of the vector's entries, so the rows of a vector share a class.
+template <bool VEC, typename S>
 __global__ void __launch_bounds__(kCeThreads)
-ce_bwd_labels(CeArgs a)
+ce_bwd_labels(CeArgs<S> a)
 {
+  constexpr int VE = Vec16<S>::N;
   const int64_t c = blockIdx.x;
-  const float g = a.dy[c * a.lddy];
-  const float* xc = a.x + c * a.ldx;
-  const float* tc = a.truth + c * a.ldt;
-  float* dxc = a.dx + c * a.lddx;
-  const int64_t n = VEC ? a.h / 4 : a.h;
-  const unsigned per_class = static_cast<unsigned>(VEC ? a.spatial / 4 : a.spatial);  // < 2^32 (host check)
+  const float g = Vec16<S>::load1(a.dy + c * a.lddy);
+  const S* xc = a.x + c * a.ldx;
+  const S* tc = a.truth + c * a.ldt;
+  S* dxc = a.dx + c * a.lddx;
+  const int64_t n = VEC ? a.h / VE : a.h;
+  const unsigned per_class = static_cast<unsigned>(VEC ? a.spatial / VE : a.spatial);  // < 2^32 (host check)
   const int64_t step = static_cast<int64_t>(gridDim.y) * kCeThreads;
   for (int64_t j = static_cast<int64_t>(blockIdx.y) * kCeThreads + threadIdx.x; j < n; j += step) {
     const unsigned cls = static_cast<unsigned>(j) / per_class;  // j < 2^32 (host check)
     const unsigned pos = static_cast<unsigned>(j) - cls * per_class;
     if (VEC) {
-      float t[4], d[4] = {0.f, 0.f, 0.f, 0.f};
-      Vec16<float>::load(tc + 4 * static_cast<int64_t>(pos), t);
-      bool hit[4];
+      float t[VE], d[VE];
+      Vec16<S>::load(tc + VE * static_cast<int64_t>(pos), t);
+      bool hit[VE];
       bool any = false;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
+      for (int k = 0; k < VE; ++k) {
+        d[k] = 0.f;
         hit[k] = ce_label(t[k]) == static_cast<int64_t>(cls);
         any |= hit[k];
       }
       if (any) {
-        float v[4];
-        Vec16<float>::load(xc + 4 * j, v);
+        float v[VE];
+        Vec16<S>::load(xc + VE * j, v);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) d[k] = hit[k] ? -g / v[k] : 0.f;
+        for (int k = 0; k < VE; ++k) d[k] = hit[k] ? -g / v[k] : 0.f;
       }
-      Vec16<float>::store(dxc + 4 * j, d);
+      Vec16<S>::store(dxc + VE * j, d);
     }
     else {
-      dxc[j] = ce_label(tc[pos]) == static_cast<int64_t>(cls) ? -g / xc[j] : 0.f;
+      Vec16<S>::store1(dxc + j, ce_label(Vec16<S>::load1(tc + pos)) == static_cast<int64_t>(cls)
+                                    ? -g / Vec16<S>::load1(xc + j)
+                                    : 0.f);
     }
   }
 }
@@ -207,9 +217,86 @@ static int ce_check(int64_t h, int64_t w, int use_labels, int64_t spatial, int64
   return LBN_OK;
 }
 
-static bool ce_vec_ok(int64_t h, int64_t w, const void* p, int64_t ld)
+// ve: entries per 16-byte vector.  A matrix that is not there (NULL) constrains nothing.
+static bool ce_vec_ok(int64_t h, int64_t w, const void* p, int64_t ld, int ve)
 {
-  return h % 4 == 0 && aligned16(p) && (w <= 1 || ld % 4 == 0);
+  return h % ve == 0 && aligned16(p) && (!p || w <= 1 || ld % ve == 0);
+}
+
+
+template <typename S>
+static int ce_fwd_impl(lbn_stream_t stream, int64_t height, int64_t width, int use_labels, int64_t spatial_size,
+                       const S* prediction, int64_t ld_prediction, const S* ground_truth, int64_t ld_ground_truth,
+                       S* loss, int64_t ld_loss, void* workspace, size_t workspace_bytes)
+{
+  constexpr int VE = Vec16<S>::N;
+  if (int e = ce_check(height, width, use_labels, spatial_size, ld_prediction, ld_ground_truth)) return e;
+  if (width == 0) return LBN_OK;
+  if (!loss || ld_loss < 1) return LBN_ERR_INVALID_ARGUMENT;
+  if (height > 0 && (!prediction || !ground_truth)) return LBN_ERR_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  CeArgs<S> a{};
+  a.h = height, a.w = width, a.spatial = use_labels ? spatial_size : 1;
+  a.x = prediction, a.truth = ground_truth, a.ldx = ld_prediction, a.ldt = ld_ground_truth;
+  a.loss = loss, a.ld_loss = ld_loss, a.part = static_cast<float*>(workspace);
+  const bool vec = !use_labels && ce_vec_ok(height, width, prediction, ld_prediction, VE) &&
+                   ce_vec_ok(height, width, ground_truth, ld_ground_truth, VE);
+  const int64_t units = use_labels ? (spatial_size < height ? spatial_size : height) : (vec ? height / VE : height);
+  // 1024-thread workgroups when that fills the device with one workgroup per column: no
+  // partial sums to merge, so no second kernel
+  const bool big = !use_labels && units >= 4 * 1024 && width >= 256;
+  const int P = ce_parts(width, units, big ? 1024 : kCeThreads);
+  if (P > 1 && (!workspace || workspace_bytes < static_cast<size_t>(width) * P * sizeof(float) ||
+                (reinterpret_cast<uintptr_t>(workspace) & 3u)))
+    return LBN_ERR_WORKSPACE;
+  const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
+  if (use_labels) hipLaunchKernelGGL((ce_fwd_labels<S>), grid, dim3(kCeThreads), 0, st, a);
+  else if (vec && big) hipLaunchKernelGGL((ce_fwd_dense<true, 1024, S>), grid, dim3(1024), 0, st, a);
+  else if (vec) hipLaunchKernelGGL((ce_fwd_dense<true, kCeThreads, S>), grid, dim3(kCeThreads), 0, st, a);
+  else if (big) hipLaunchKernelGGL((ce_fwd_dense<false, 1024, S>), grid, dim3(1024), 0, st, a);
+  else hipLaunchKernelGGL((ce_fwd_dense<false, kCeThreads, S>), grid, dim3(kCeThreads), 0, st, a);
+  if (P > 1)
+    hipLaunchKernelGGL((ce_merge_parts<S>), dim3(static_cast<unsigned>(width)), dim3(kWave), 0, st, P, a.part, loss,
+                       ld_loss);
+  return launch_status();
+}
+
+template <typename S>
+static int ce_bwd_impl(lbn_stream_t stream, int64_t height, int64_t width, int use_labels, int64_t spatial_size,
+                       const S* prediction, int64_t ld_prediction, const S* ground_truth, int64_t ld_ground_truth,
+                       const S* dloss, int64_t ld_dloss, S* dprediction, int64_t ld_dprediction, S* dground_truth,
+                       int64_t ld_dground_truth)
+{
+  constexpr int VE = Vec16<S>::N;
+  if (int e = ce_check(height, width, use_labels, spatial_size, ld_prediction, ld_ground_truth)) return e;
+  if (height == 0 || width == 0) return LBN_OK;
+  if (!prediction || !ground_truth || !dloss || !dprediction || ld_dloss < 1) return LBN_ERR_INVALID_ARGUMENT;
+  if (width > 1 && ld_dprediction < height) return LBN_ERR_INVALID_ARGUMENT;
+  if (!use_labels && dground_truth && width > 1 && ld_dground_truth < height) return LBN_ERR_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  CeArgs<S> a{};
+  a.h = height, a.w = width, a.spatial = use_labels ? spatial_size : 1;
+  a.x = prediction, a.truth = ground_truth, a.ldx = ld_prediction, a.ldt = ld_ground_truth;
+  a.dy = dloss, a.lddy = ld_dloss, a.dx = dprediction, a.lddx = ld_dprediction;
+  a.dtruth = dground_truth, a.lddt = ld_dground_truth;
+  bool vec = ce_vec_ok(height, width, prediction, ld_prediction, VE) &&
+             ce_vec_ok(height, width, dprediction, ld_dprediction, VE);
+  if (use_labels)
+    vec = vec && spatial_size % VE == 0 && aligned16(ground_truth) && (width <= 1 || ld_ground_truth % VE == 0);
+  else
+    vec = vec && ce_vec_ok(height, width, ground_truth, ld_ground_truth, VE) &&
+          ce_vec_ok(height, width, dground_truth, ld_dground_truth, VE);
+  const int P = ce_parts(width, vec ? height / VE : height);
+  const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
+  if (use_labels) {
+    if (vec) hipLaunchKernelGGL((ce_bwd_labels<true, S>), grid, dim3(kCeThreads), 0, st, a);
+    else hipLaunchKernelGGL((ce_bwd_labels<false, S>), grid, dim3(kCeThreads), 0, st, a);
+  }
+  else {
+    if (vec) hipLaunchKernelGGL((ce_bwd_dense<true, S>), grid, dim3(kCeThreads), 0, st, a);
+    else hipLaunchKernelGGL((ce_bwd_dense<false, S>), grid, dim3(kCeThreads), 0, st, a);
+  }
+  return launch_status();
 }
 
 }  // namespace lbn
@@ -229,35 +316,8 @@ int lbn_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width
                               const float* ground_truth, int64_t ld_ground_truth, float* loss,
                               int64_t ld_loss, void* workspace, size_t workspace_bytes)
 {
-  if (int e = ce_check(height, width, use_labels, spatial_size, ld_prediction, ld_ground_truth)) return e;
-  if (width == 0) return LBN_OK;
-  if (!loss || ld_loss < 1) return LBN_ERR_INVALID_ARGUMENT;
-  if (height > 0 && (!prediction || !ground_truth)) return LBN_ERR_INVALID_ARGUMENT;
-  hipStream_t st = as_stream(stream);
-  CeArgs a{};
-  a.h = height, a.w = width, a.spatial = use_labels ? spatial_size : 1;
-  a.x = prediction, a.truth = ground_truth, a.ldx = ld_prediction, a.ldt = ld_ground_truth;
-  a.loss = loss, a.ld_loss = ld_loss, a.part = static_cast<float*>(workspace);
-  const bool vec = !use_labels && ce_vec_ok(height, width, prediction, ld_prediction) &&
-                   ce_vec_ok(height, width, ground_truth, ld_ground_truth);
-  const int64_t units = use_labels ? (spatial_size < height ? spatial_size : height) : (vec ? height / 4 : height);
-  // 1024-thread workgroups when that fills the device with one workgroup per column: no
-  // partial sums to merge, so no second kernel
-  const bool big = !use_labels && units >= 4 * 1024 && width >= 256;
-  const int P = ce_parts(width, units, big ? 1024 : kCeThreads);
-  if (P > 1 && (!workspace || workspace_bytes < static_cast<size_t>(width) * P * sizeof(float) ||
-                (reinterpret_cast<uintptr_t>(workspace) & 3u)))
-    return LBN_ERR_WORKSPACE;
-  const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
-  if (use_labels) hipLaunchKernelGGL(ce_fwd_labels, grid, dim3(kCeThreads), 0, st, a);
-  else if (vec && big) hipLaunchKernelGGL((ce_fwd_dense<true, 1024>), grid, dim3(1024), 0, st, a);
-  else if (vec) hipLaunchKernelGGL((ce_fwd_dense<true, kCeThreads>), grid, dim3(kCeThreads), 0, st, a);
-  else if (big) hipLaunchKernelGGL((ce_fwd_dense<false, 1024>), grid, dim3(1024), 0, st, a);
-  else hipLaunchKernelGGL((ce_fwd_dense<false, kCeThreads>), grid, dim3(kCeThreads), 0, st, a);
-  if (P > 1)
-    hipLaunchKernelGGL(ce_merge_parts, dim3(static_cast<unsigned>(width)), dim3(kWave), 0, st, P, a.part, loss,
-                       ld_loss);
-  return launch_status();
+  return ce_fwd_impl<float>(stream, height, width, use_labels, spatial_size, prediction, ld_prediction, ground_truth,
+                            ld_ground_truth, loss, ld_loss, workspace, workspace_bytes);
 }
 
 int lbn_cross_entropy_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
@@ -266,35 +326,38 @@ int lbn_cross_entropy_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width
                               int64_t ld_dloss, float* dprediction, int64_t ld_dprediction,
                               float* dground_truth, int64_t ld_dground_truth)
 {
-  if (int e = ce_check(height, width, use_labels, spatial_size, ld_prediction, ld_ground_truth)) return e;
-  if (height == 0 || width == 0) return LBN_OK;
-  if (!prediction || !ground_truth || !dloss || !dprediction || ld_dloss < 1) return LBN_ERR_INVALID_ARGUMENT;
-  if (width > 1 && ld_dprediction < height) return LBN_ERR_INVALID_ARGUMENT;
-  if (!use_labels && dground_truth && width > 1 && ld_dground_truth < height) return LBN_ERR_INVALID_ARGUMENT;
-  hipStream_t st = as_stream(stream);
-  CeArgs a{};
-  a.h = height, a.w = width, a.spatial = use_labels ? spatial_size : 1;
-  a.x = prediction, a.truth = ground_truth, a.ldx = ld_prediction, a.ldt = ld_ground_truth;
-  a.dy = dloss, a.lddy = ld_dloss, a.dx = dprediction, a.lddx = ld_dprediction;
-  a.dtruth = dground_truth, a.lddt = ld_dground_truth;
-  bool vec = ce_vec_ok(height, width, prediction, ld_prediction) &&
-             ce_vec_ok(height, width, dprediction, ld_dprediction);
-  if (use_labels)
-    vec = vec && spatial_size % 4 == 0 && aligned16(ground_truth) && (width <= 1 || ld_ground_truth % 4 == 0);
-  else
-    vec = vec && ce_vec_ok(height, width, ground_truth, ld_ground_truth) &&
-          ce_vec_ok(height, width, dground_truth, ld_dground_truth);
-  const int P = ce_parts(width, vec ? height / 4 : height);
-  const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
-  if (use_labels) {
-    if (vec) hipLaunchKernelGGL((ce_bwd_labels<true>), grid, dim3(kCeThreads), 0, st, a);
-    else hipLaunchKernelGGL((ce_bwd_labels<false>), grid, dim3(kCeThreads), 0, st, a);
-  }
-  else {
-    if (vec) hipLaunchKernelGGL((ce_bwd_dense<true>), grid, dim3(kCeThreads), 0, st, a);
-    else hipLaunchKernelGGL((ce_bwd_dense<false>), grid, dim3(kCeThreads), 0, st, a);
-  }
-  return launch_status();
+  return ce_bwd_impl<float>(stream, height, width, use_labels, spatial_size, prediction, ld_prediction, ground_truth,
+                            ld_ground_truth, dloss, ld_dloss, dprediction, ld_dprediction, dground_truth,
+                            ld_dground_truth);
+}
+
+int lbn_cross_entropy_fwd_f16(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                              int64_t spatial_size, const void* prediction, int64_t ld_prediction,
+                              const void* ground_truth, int64_t ld_ground_truth, void* loss, int64_t ld_loss,
+                              void* workspace, size_t workspace_bytes)
+{
+  if ((reinterpret_cast<uintptr_t>(prediction) | reinterpret_cast<uintptr_t>(ground_truth) |
+       reinterpret_cast<uintptr_t>(loss)) & 1u)
+    return LBN_ERR_INVALID_ARGUMENT;
+  return ce_fwd_impl<__half>(stream, height, width, use_labels, spatial_size, static_cast<const __half*>(prediction),
+                             ld_prediction, static_cast<const __half*>(ground_truth), ld_ground_truth,
+                             static_cast<__half*>(loss), ld_loss, workspace, workspace_bytes);
+}
+
+int lbn_cross_entropy_bwd_f16(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,
+                              int64_t spatial_size, const void* prediction, int64_t ld_prediction,
+                              const void* ground_truth, int64_t ld_ground_truth, const void* dloss,
+                              int64_t ld_dloss, void* dprediction, int64_t ld_dprediction, void* dground_truth,
+                              int64_t ld_dground_truth)
+{
+  if ((reinterpret_cast<uintptr_t>(prediction) | reinterpret_cast<uintptr_t>(ground_truth) |
+       reinterpret_cast<uintptr_t>(dloss) | reinterpret_cast<uintptr_t>(dprediction) |
+       reinterpret_cast<uintptr_t>(dground_truth)) & 1u)
+    return LBN_ERR_INVALID_ARGUMENT;
+  return ce_bwd_impl<__half>(stream, height, width, use_labels, spatial_size, static_cast<const __half*>(prediction),
+                             ld_prediction, static_cast<const __half*>(ground_truth), ld_ground_truth,
+                             static_cast<const __half*>(dloss), ld_dloss, static_cast<__half*>(dprediction),
+                             ld_dprediction, static_cast<__half*>(dground_truth), ld_dground_truth);
 }
 
 }  // extern "C"

@@ -618,17 +618,26 @@ class cross_entropy_layer:
         self.error_signals = [None, None]
         self._ws = _Workspace("cross_entropy_layer", header=False)
 
+    @staticmethod
+    def _suffix(*matrices):
+        """fp32 or fp16 storage (the reference instantiates the layer for both,
+        cross_entropy.cpp:157-166); every matrix of a call has the layer's one data type."""
+        kinds = {m.dtype for m in matrices if m is not None}
+        if len(kinds) != 1:
+            raise TypeError(f"cross entropy: matrices of different types {sorted(map(str, kinds))}")
+        return "f16" if kinds.pop() == torch.float16 else "f32"
+
     def fp_call(self):
         x, t, y = self.prev_activations[0], self.prev_activations[1], self.activations
         ws, nb = self._ws.get(capi.lib().lbn_cross_entropy_fwd_workspace_bytes(x.height, x.width), self.device)
-        return ("lbn_cross_entropy_fwd_f32",
+        return (f"lbn_cross_entropy_fwd_{self._suffix(x, t, y)}",
                 (_stream(), x.height, x.width, int(self.m_use_labels), self.spatial_sample_size, x.Buffer(), x.ldim,
                  t.Buffer(), t.ldim, y.Buffer(), y.ldim, ws, nb))
 
     def bp_call(self):
         x, t, dy = self.prev_activations[0], self.prev_activations[1], self.prev_error_signals
         dx, dt = self.error_signals
-        return ("lbn_cross_entropy_bwd_f32",
+        return (f"lbn_cross_entropy_bwd_{self._suffix(x, t, dy, dx, dt)}",
                 (_stream(), x.height, x.width, int(self.m_use_labels), self.spatial_sample_size, x.Buffer(), x.ldim,
                  t.Buffer(), t.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim,
                  dt.Buffer() if dt is not None else _null(), dt.ldim if dt is not None else 0))
@@ -645,7 +654,7 @@ class cross_entropy_layer:
 
     def forward(self, prediction, ground_truth):
         self.prev_activations = [prediction, ground_truth]
-        self.activations = DeviceMatrix(1, prediction.width, device=self.device)
+        self.activations = DeviceMatrix(1, prediction.width, dtype=prediction.dtype, device=self.device)
         self.fp_compute()
         return self.activations
 
@@ -654,9 +663,9 @@ class cross_entropy_layer:
         the second is None with use_labels (the reference leaves that error signal untouched)."""
         x, t = self.prev_activations
         self.prev_error_signals = dy
-        self.error_signals = [DeviceMatrix(x.height, x.width, ldim=x.ldim, device=self.device),
-                              None if self.m_use_labels else DeviceMatrix(t.height, t.width, ldim=t.ldim,
-                                                                          device=self.device)]
+        self.error_signals = [DeviceMatrix(x.height, x.width, dtype=x.dtype, ldim=x.ldim, device=self.device),
+                              None if self.m_use_labels else DeviceMatrix(t.height, t.width, dtype=t.dtype,
+                                                                          ldim=t.ldim, device=self.device)]
         self.bp_compute()
         return self.error_signals
 

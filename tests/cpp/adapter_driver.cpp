@@ -401,6 +401,31 @@ int drv_softmax_family_f16(int kind, int64_t h, int64_t w, int64_t ld, void* x, 
   }
 }
 
+// Cross entropy with fp16 storage (dense ground truth): 2-byte elements select the _f16 entry points.
+int drv_cross_entropy_f16(const int64_t* dims, int nd, int64_t h, int64_t w, void* x, void* truth, void* loss,
+                          void* dloss, void* dx, void* dtruth, void* stream, char* err, int errlen)
+{
+  try {
+    using half_bits = unsigned short;
+    using M = device_matrix<half_bits>;
+    cross_entropy_layer<M> layer(false);
+    layer.setup(std::vector<int64_t>(dims, dims + nd), std::vector<int64_t>(dims, dims + nd));
+    M mx, mt, ml, mdl, mdx, mdt;
+    attach(mx, h, w, x, h); attach(mt, h, w, truth, h); attach(ml, 1, w, loss, 1); attach(mdl, 1, w, dloss, 1);
+    attach(mdx, h, w, dx, h); attach(mdt, h, w, dtruth, h);
+    layer.io.prev_activations = &mx; layer.prev_ground_truth = &mt; layer.io.activations = &ml;
+    layer.io.prev_error_signals = &mdl; layer.io.error_signals = &mdx; layer.ground_truth_error_signals = &mdt;
+    layer.io.stream = static_cast<hipStream_t>(stream);
+    layer.fp_compute();
+    layer.bp_compute();
+    check_hip(hipStreamSynchronize(layer.io.stream), "sync");
+    return 0;
+  }
+  catch (const std::exception& e) {
+    return fail(e, err, errlen);
+  }
+}
+
 // A softmax layer on a (h x w) problem that uses scratch: forward, then the wait check, which
 // must pass; then the designed give-up exit is run on the layer's own scratch buffer and
 // the next check must throw (returns 0 only if it did, with the message in err), after which

@@ -148,6 +148,25 @@ def test_adapter_layers_match_oracle():
         check(f"adapter f16 softmax kind {kind} y", y, fwd(xf), tol=TOL_F16)
         check(f"adapter f16 softmax kind {kind} dx", mdx.to_numpy(), bwd(np.asfortranarray(y), dyf), tol=TOL_F16)
 
+    # ---- cross entropy with fp16 storage
+    h, w = 520, 9
+    x16 = np.asfortranarray(rng.uniform(0.05, 1.0, (w, h)).astype(np.float16).T)
+    t16 = np.asfortranarray(rng.uniform(-0.3, 1.0, (w, h)).astype(np.float16).T)
+    g16 = rng.standard_normal(w).astype(np.float16)
+    half = _torch.float16
+    mx, mt = DeviceMatrix.from_numpy(x16, dtype=half), DeviceMatrix.from_numpy(t16, dtype=half)
+    mdl = DeviceMatrix.from_numpy(np.asfortranarray(g16.reshape(1, w)), dtype=half)
+    ml, mdx, mdt = DeviceMatrix(1, w, dtype=half), DeviceMatrix(h, w, dtype=half), DeviceMatrix(h, w, dtype=half)
+    da, nd = _dims((h,))
+    rc = d.drv_cross_entropy_f16(da, cint(nd), i64(h), i64(w), mx.Buffer(), mt.Buffer(), ml.Buffer(), mdl.Buffer(),
+                                 mdx.Buffer(), mdt.Buffer(), st, err, cint(512))
+    assert rc == 0, err.value
+    xf, tf, gf = (np.asfortranarray(a.astype(np.float32)) for a in (x16, t16, g16))
+    check("adapter f16 cross entropy loss", ml.to_numpy()[0].astype(np.float32), orc.cross_entropy_fwd(xf, tf), tol=TOL_F16)
+    dx_ref, dt_ref = orc.cross_entropy_bwd(xf, tf, gf)
+    check("adapter f16 cross entropy dx", mdx.to_numpy().astype(np.float32), dx_ref, tol=TOL_F16)
+    check("adapter f16 cross entropy dtruth", mdt.to_numpy().astype(np.float32), dt_ref, tol=TOL_F16)
+
     # ---- instance norm on (6, 20, 20) samples
     dims, w = (6, 20, 20), 9
     h = 6 * 400

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from oracle import cpu_oracle as orc
-from tests.parity import TOL_F32, check, rel_err
+from tests.parity import TOL_F16, TOL_F32, check, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -94,6 +94,90 @@ def test_cross_entropy_labels(L, classes, spatial, w, pad):
     assert none is None
     check(f"cross entropy (labels) dx {classes}x{sp}x{w}", dx.to_numpy(), orc.cross_entropy_bwd(x, labels, dy, True)[0],
           orc.cross_entropy_bwd(f64(x), f64(labels), dy.astype(np.float64), True)[0])
+
+
+CE_F16 = [
+    # (h, w, ld_pad): whole 16-byte vectors of 8, ragged heights, a padded leading dimension, 1024-thread columns
+    (16, 128, 0), (1000, 64, 0), (192, 23, 0), (4096, 33, 0), (7, 5, 0), (1001, 3, 0), (136, 4, 8), (130, 4, 2),
+    (16384, 256, 0), (4101, 257, 0), (65536, 40, 0), (300000, 3, 0), (1, 6, 0),
+]
+
+
+@pytest.mark.parametrize("h,w,pad", CE_F16)
+def test_cross_entropy_dense_f16(L, h, w, pad):
+    """fp16 storage (the reference instantiates the layer for half, cross_entropy.cpp:157-166):
+    the fp32 oracle on the same binary16 inputs, 2e-3."""
+    rng = np.random.default_rng(h * 11 + w)
+    x = np.asfortranarray(rng.uniform(0.05, 1.0, (w, h)).astype(np.float16).T)
+    truth = np.asfortranarray((rng.uniform(-0.3, 1.0, (w, h)) * min(1.0, 4096.0 / h)).astype(np.float16).T)
+    truth[0, :] = 0.0
+    dy = rng.standard_normal(w).astype(np.float16)
+    layer = L.cross_entropy_layer((h,))
+    ld = h + pad
+    half = torch.float16
+    loss = layer.forward(L.DeviceMatrix.from_numpy(x, dtype=half, ldim=ld),
+                         L.DeviceMatrix.from_numpy(truth, dtype=half, ldim=ld))
+    assert loss.dtype == half
+    check(f"cross entropy f16 loss {h}x{w}", f32(loss.to_numpy()[0]), orc.cross_entropy_fwd(f32(x), f32(truth)), tol=TOL_F16)
+    dym = L.DeviceMatrix.from_numpy(np.asfortranarray(dy.reshape(1, w)), dtype=half)
+    dx, dt = layer.backward(dym)
+    assert dx.dtype == half and dt.dtype == half
+    rx, rt = orc.cross_entropy_bwd(f32(x), f32(truth), f32(dy))
+    got = f32(dx.to_numpy())
+    check(f"cross entropy f16 dx {h}x{w}", got, rx, tol=TOL_F16)
+    assert np.all(got[f32(truth) <= 0] == 0.0)
+    check(f"cross entropy f16 dtruth {h}x{w}", f32(dt.to_numpy()), rt, tol=TOL_F16)
+
+
+@pytest.mark.parametrize("classes,spatial,w,pad", [(3, (8, 8), 23, 0), (10, (1,), 64, 0), (5, (7, 3), 9, 0),
+                                                  (4, (6,), 5, 3), (21, (64, 64), 6, 0), (1000, (1,), 128, 0),
+                                                  (2048, (1,), 16, 0)])
+def test_cross_entropy_labels_f16(L, classes, spatial, w, pad):
+    """Class indices stored as binary16 (exact up to 2048)."""
+    rng = np.random.default_rng(classes * 101 + w)
+    sp = int(np.prod(spatial))
+    h = classes * sp
+    x = np.asfortranarray(rng.uniform(0.05, 1.0, (w, h)).astype(np.float16).T)
+    labels = np.asfortranarray(rng.integers(0, classes, (w, sp)).astype(np.float16).T)
+    if sp > 2:
+        labels[1, 0] = classes      # a label no class matches contributes nothing
+        labels[2, 0] = -3.0
+    dy = rng.standard_normal(w).astype(np.float16)
+    half = torch.float16
+    layer = L.cross_entropy_layer((classes,) + tuple(spatial), use_labels=True)
+    loss = layer.forward(L.DeviceMatrix.from_numpy(x, dtype=half, ldim=h + pad),
+                         L.DeviceMatrix.from_numpy(labels, dtype=half, ldim=sp + pad)).to_numpy()
+    check(f"cross entropy f16 (labels) loss {classes}x{sp}x{w}", f32(loss[0]),
+          orc.cross_entropy_fwd(f32(x), f32(labels), True), tol=TOL_F16)
+    dx, dt = layer.backward(L.DeviceMatrix.from_numpy(np.asfortranarray(dy.reshape(1, w)), dtype=half))
+    assert dt is None
+    rx, _ = orc.cross_entropy_bwd(f32(x), f32(labels), f32(dy), True)
+    got = f32(dx.to_numpy())
+    check(f"cross entropy f16 (labels) dx {classes}x{sp}x{w}", got, rx, tol=TOL_F16)
+    assert np.array_equal(got == 0.0, rx == 0.0)
+
+
+def test_cross_entropy_f16_rejects_mixed_types_and_odd_pointers(L):
+    from lbann_amd import capi
+    layer = L.cross_entropy_layer((8,))
+    x = L.DeviceMatrix(8, 4, dtype=torch.float16, fill=0.5)
+    t32 = L.DeviceMatrix(8, 4, fill=0.5)
+    with pytest.raises(TypeError):
+        layer.forward(x, t32)
+    t = L.DeviceMatrix(8, 4, dtype=torch.float16, fill=0.5)
+    loss = L.DeviceMatrix(1, 4, dtype=torch.float16)
+    odd = capi.vp(x.tensor.data_ptr() + 1)
+    rc = capi.lib().lbn_cross_entropy_fwd_f16(capi.vp(None), 4, 4, 0, 1, odd, 8, t.Buffer(), 8, loss.Buffer(), 1,
+                                               capi.vp(None), 0)
+    assert rc == -1
+    # an empty mini-batch and an empty sample
+    assert capi.lib().lbn_cross_entropy_fwd_f16(capi.vp(None), 8, 0, 0, 1, x.Buffer(), 8, t.Buffer(), 8,
+                                                loss.Buffer(), 1, capi.vp(None), 0) == 0
+    loss.tensor.fill_(7.0)
+    assert capi.lib().lbn_cross_entropy_fwd_f16(capi.vp(None), 0, 4, 0, 1, capi.vp(None), 1, capi.vp(None), 1,
+                                                loss.Buffer(), 1, capi.vp(None), 0) == 0
+    torch.cuda.synchronize()
+    assert (loss.to_numpy() == 0).all()
 
 
 def test_cross_entropy_after_softmax(L):
