@@ -379,7 +379,8 @@ int lbn_log_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
  * log_softmax_layer for half precision too (src/layers/activations/softmax.cpp:236-243,
  * log_softmax.cpp:160-167, LBANN_INSTANTIATE_CPU_HALF / GPU_HALF).  x, y, dy, dx are IEEE
  * binary16 in memory; all arithmetic (maximum, exponentials, sums) is fp32, where the
- * reference's half instantiation also accumulates in half; results are rounded to nearest
+ * reference's half instantiation also accumulates in half (the exponential is evaluated to a
+ * relative error of about |x - max| * 3e-8, far inside binary16's rounding); results are rounded to nearest
  * even on store, and softmax's flush of non-normal results applies to the fp32 value before
  * rounding (binary16 denormals are kept).  Same arguments as the _f32 entry points (leading
  * dimensions in elements); the workspace is not used and may be NULL.  In place allowed. */

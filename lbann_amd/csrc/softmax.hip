@@ -283,6 +283,24 @@ static bool sm_bwd_framed_rows(hipStream_t st, int64_t n, int64_t w, int64_t row
   }
 }
 
+// The walking forward kernel for 16-bit rows of four vectors per thread, when the rows need
+// more than one workgroup per compute unit.
+template <int KIND, typename S>
+static bool sm_fwd_walk(hipStream_t st, int64_t rows, unsigned nvec, const S* x, S* y, int64_t ldx, int64_t ldy,
+                        RowMap map)
+{
+  static const bool off = std::getenv("LBN_NO_FWD_WALK") != nullptr;
+  if (off || KIND == kChannelwise) return false;
+  int cus = 0, dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+    return false;
+  if (rows <= cus) return false;
+  hipLaunchKernelGGL((sm_fwd_rows_walk<S, 4, KIND>), dim3(static_cast<unsigned>(cus)), dim3(1024), 0, st, x, y, ldx,
+                     ldy, map, rows, nvec);
+  return true;
+}
+
 template <int KIND, typename S = float>
 static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int64_t w,
                   const S* x, int64_t ldx, S* y, int64_t ldy, void* ws, size_t ws_bytes)
@@ -306,6 +324,9 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   if (c.tpr == TPR && c.v == V) {                                                            \
     using B = RowBlock<TPR>;                                                                 \
     const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                  \
+    if constexpr (sizeof(S) == 2 && TPR == 1024 && V == 4 && KIND != kChannelwise) {         \
+      if (sm_fwd_walk<KIND>(st, rows, nvec, x, y, ldx, ldy, map)) return launch_status();    \
+    }                                                                                        \
     if (stream_loads(rows, n * sizeof(S) / 4, 2))                                            \
       hipLaunchKernelGGL((sm_fwd_rows<S, TPR, V, KIND, true>), dim3(grid), dim3(B::kThreads), 0, st, \
                          x, y, ldx, ldy, map, rows, nvec);                                   \

@@ -174,6 +174,10 @@ sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows
       float e;
       if (KIND == kLogSoftmax) e = exp_quick(d);  // only summed: x stays in the registers for the output
       else if (KIND == kChannelwise) e = exp_keep_denormals(d);
+      // 16-bit storage rounds the result to 11 bits: the two-operation exponential (relative
+      // error |d| * 3e-8) is exact enough there, and the kernel is bound by these operations,
+      // not by memory, once an entry is two bytes
+      else if (sizeof(S) == 2) e = exp_quick(d);
       else e = exp_fast(d);
       e = ok ? e : 0.f;
       s += e;
@@ -220,6 +224,103 @@ sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows
       }
       if constexpr (FR) frame_store(yr, idx, fr, n, v[i]);
       else RowIO<S, W>::store(yr + unsigned(W) * idx, v[i]);
+    }
+  }
+}
+
+// Forward over 16-bit rows of 1024 threads: with two bytes per entry the exponentials, not the
+// memory, are what a compute unit spends its time on, and two workgroups that load, compute and
+// store in step leave the memory idle while they compute.  Here one workgroup per compute unit
+// walks rows b, b + grid, ...: the next row's packed vectors (16 bytes for 8 entries, so a
+// second row costs few registers) are requested before the current row is unpacked, arrive while
+// it is exponentiated, and its stores overlap the next row's arithmetic.
+template <typename S, int V, int KIND>
+__global__ void __launch_bounds__(1024)
+sm_fwd_rows_walk(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows, unsigned nvec)
+{
+  static_assert(sizeof(S) == 2, "packed 16-bit rows");
+  constexpr int TPR = 1024, W = Vec16<S>::N, NW = TPR / kWave;
+  using raw_t = typename Vec16<S>::raw_t;
+  __shared__ float red[2][2][NW];
+  const unsigned t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wv = wave_index();
+  raw_t nx[V];
+  auto request = [&](int64_t row) {
+    const S* xr = x + map.offset(row, ldx);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = t + i * TPR;
+      nx[i] = raw_t{};
+      if (idx < nvec) nx[i] = Vec16<S>::load_raw(xr + unsigned(W) * idx);
+    }
+  };
+  int64_t row = blockIdx.x;
+  if (row >= rows) return;
+  request(row);
+  for (int it = 0; row < rows; row += gridDim.x, ++it) {
+    float v[V][W];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      Vec16<S>::unpack(nx[i], v[i]);
+      if (t + i * TPR >= nvec) {
+#pragma unroll
+        for (int k = 0; k < W; ++k) v[i][k] = -FLT_MAX;
+      }
+    }
+    const int64_t next = row + gridDim.x;
+    if (next < rows) request(next);
+    asm volatile("" ::: "memory");  // the next row's loads go out ahead of this row's arithmetic
+
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+#pragma unroll
+      for (int k = 0; k < W; ++k) m = fmaxf(m, v[i][k]);
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const bool ok = (t + i * TPR) < nvec;
+#pragma unroll
+      for (int k = 0; k < W; ++k) {
+        float e = exp_quick(v[i][k] - m);
+        e = ok ? e : 0.f;
+        s += e;
+        if (KIND != kLogSoftmax) v[i][k] = e;
+      }
+    }
+    float gm = wave_max(m);
+    float gs = wave_sum(s * exp_fast(m - gm));
+    float (&rd)[2][NW] = red[it & 1];  // the next row writes the other pair: one barrier per row
+    if (lane == 0) {
+      rd[0][wv] = gm;
+      rd[1][wv] = gs;
+    }
+    __syncthreads();
+    const float pm = lane < NW ? rd[0][lane] : -FLT_MAX;
+    const float ps = lane < NW ? rd[1][lane] : 0.f;
+    gm = wave_max(pm);
+    gs = wave_sum(ps * exp_fast(pm - gm));
+
+    S* yr = y + map.offset(row, ldy);
+    const float f = exp_fast(m - gm) * (1.0f / gs);
+    const float lse = (KIND == kLogSoftmax) ? log_of_sum(gs) : 0.f;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = t + i * TPR;
+      if (idx < nvec) {
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+          if (KIND == kSoftmax) {
+            const float r = f * v[i][k];
+            v[i][k] = __builtin_isnormal(r) ? r : 0.f;
+          }
+          else {
+            v[i][k] = (v[i][k] - gm) - lse;
+          }
+        }
+        Vec16<S>::store(yr + unsigned(W) * idx, v[i]);
+      }
     }
   }
 }
@@ -477,7 +578,8 @@ sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t l
     if (idx < nvec) {
 #pragma unroll
       for (int k = 0; k < W; ++k) {
-        if (KIND == kLogSoftmax) g[i][k] = g[i][k] - exp_fast(a[i][k]) * s;
+        // (16-bit storage: the two-operation exponential, as in the forward kernel)
+        if (KIND == kLogSoftmax) g[i][k] = g[i][k] - (sizeof(S) == 2 ? exp_quick(a[i][k]) : exp_fast(a[i][k])) * s;
         else g[i][k] = a[i][k] * (g[i][k] - s);
       }
       if constexpr (FR) frame_store(dr, idx, fr, n, g[i]);

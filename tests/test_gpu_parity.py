@@ -86,6 +86,7 @@ def test_softmax_family(L, kind, h, w, pad):
     (197, 50, 0, False), (1001, 33, 3, False), (16385, 6, 0, True),                          # single halves
     (64, 5000, 0, False), (24, 4099, 0, False),                                             # short rows, 16-lane teams
     (70000, 3, 0, False), (40001, 2, 0, True), (131072, 2, 0, False),                        # beyond the register kernels
+    (32768, 300, 0, True), (20480, 513, 0, False), (24584, 260, 8, False),    # more rows than compute units: walked
 ])
 def test_softmax_family_f16_storage(L, kind, h, w, pad, in_place):
     """fp16 storage, fp32 arithmetic (softmax.cpp:236-243 instantiates the layers for half):
@@ -127,6 +128,32 @@ def test_softmax_f16_special_values(L):
     assert y[5, 2] == 1.0 and y[:, 2].sum() == 1.0
     # a NaN in the column: the reference's output for that column is all zeros (non-normal results are flushed)
     assert (ref[:, 3] == 0).all() and (y[:, 3] == 0).all()
+
+
+def test_softmax_f16_special_values_on_walked_rows(L):
+    """The same columns among more rows than the device has compute units (a workgroup walks
+    several rows there), each special column landing in a different position of the walk."""
+    h, w = 32768, 600
+    rng = np.random.default_rng(5)
+    x = rand(rng, h, w, 0, 2).astype(np.float16)
+    cols = {"equal": 3, "dominant": 258, "minus_inf": 301, "nan": 599}
+    x[:, cols["equal"]] = 3.0
+    x[7, cols["dominant"]] = 60000.0
+    x[:, cols["minus_inf"]] = -np.inf
+    x[5, cols["minus_inf"]] = 1.0
+    x[9, cols["nan"]] = np.nan
+    y = L.softmax_layer().forward(L.DeviceMatrix.from_numpy(x, dtype=torch.float16)).to_numpy()
+    ref = orc.softmax_fwd(f32(x))
+    assert np.allclose(f32(y[:, cols["equal"]]), 1.0 / h, rtol=2e-3)
+    assert y[7, cols["dominant"]] == 1.0 and y[:, cols["dominant"]].sum() == 1.0
+    assert y[5, cols["minus_inf"]] == 1.0 and y[:, cols["minus_inf"]].sum() == 1.0
+    assert (ref[:, cols["nan"]] == 0).all() and (y[:, cols["nan"]] == 0).all()
+    rest = [c for c in range(w) if c not in cols.values()]
+    check("softmax f16 walked rows y", f32(y[:, rest]), f32(ref[:, rest]), tol=TOL_F16)
+    ly = L.log_softmax_layer().forward(L.DeviceMatrix.from_numpy(x, dtype=torch.float16)).to_numpy()
+    lref = orc.log_softmax_fwd(f32(x))
+    check("log-softmax f16 walked rows y", f32(ly[:, rest]), f32(lref[:, rest]), tol=TOL_F16)
+    assert np.all(np.isneginf(ly[:, cols["minus_inf"]][np.arange(h) != 5])) and abs(float(ly[5, cols["minus_inf"]])) == 0.0
 
 
 @pytest.mark.parametrize("kind", ["softmax", "log_softmax", "channelwise"])
