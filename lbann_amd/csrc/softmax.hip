@@ -437,6 +437,20 @@ static bool sm_bwd_walk(hipStream_t st, int hint, int64_t rows, unsigned nvec, c
   return false;
 }
 
+// The same for 16-bit rows of four vectors per thread.
+template <int KIND, typename S>
+static bool sm_bwd_walk_packed(hipStream_t st, int64_t rows, unsigned nvec, const S* y, const S* dy, S* dx,
+                               int64_t ldy, int64_t lddy, int64_t lddx, RowMap map)
+{
+  static const bool off = std::getenv("LBN_NO_BWD_WALK") != nullptr;
+  if (off) return false;
+  const int cap = resident_blocks(sm_bwd_rows_walk_packed<S, 4, KIND>, 1024);
+  if (cap < 1 || rows <= cap) return false;
+  hipLaunchKernelGGL((sm_bwd_rows_walk_packed<S, 4, KIND>), dim3(static_cast<unsigned>(cap)), dim3(1024), 0, st, y,
+                     dy, dx, ldy, lddy, lddx, map, rows, nvec);
+  return true;
+}
+
 template <int KIND, typename S = float>
 static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int64_t w,
                   const S* y, int64_t ldy, const S* dy, int64_t lddy, S* dx,
@@ -468,6 +482,9 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     const int hint = stream_loads_bwd(rows, n * sizeof(S) / 4);                              \
     if constexpr (std::is_same<S, float>::value && TPR == 1024 && V == 8) {                  \
       if (sm_bwd_walk<KIND>(st, hint, rows, nvec, y, dy, dx, ldy, lddy, lddx, map)) return launch_status(); \
+    }                                                                                        \
+    if constexpr (sizeof(S) == 2 && TPR == 1024 && V == 4) {                                 \
+      if (sm_bwd_walk_packed<KIND>(st, rows, nvec, y, dy, dx, ldy, lddy, lddx, map)) return launch_status(); \
     }                                                                                        \
     if (hint == 3)                                                                           \
       hipLaunchKernelGGL((sm_bwd_rows<S, TPR, V, KIND, 3>), dim3(grid), dim3(B::kThreads), 0, st, \

@@ -669,4 +669,71 @@ sm_bwd_rows_walk(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int6
   }
 }
 
+// The walk over 16-bit rows: both tensors of the next row wait as packed vectors (16 bytes for 8
+// entries: 8 registers per thread and tensor at four vectors), so all of its loads go out before
+// the current row is touched, arrive during its arithmetic and stores, and no wait for them
+// stands behind a store.  (The fp32 walk above has no room for that and splits the next row's
+// loads around the stores; 16-bit rows walked that way lose against one row per workgroup.)
+template <typename S, int V, int KIND>
+__global__ void __launch_bounds__(1024)
+sm_bwd_rows_walk_packed(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx, RowMap map,
+                        int64_t rows, unsigned nvec)
+{
+  static_assert(sizeof(S) == 2, "packed 16-bit rows");
+  constexpr int TPR = 1024, W = Vec16<S>::N, NW = TPR / kWave;
+  using raw_t = typename Vec16<S>::raw_t;
+  __shared__ float red[2][NW];
+  const unsigned t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wv = wave_index();
+  raw_t ny[V], ng[V];
+  auto request = [&](int64_t row) {
+    const S* yr = y + map.offset(row, ldy);
+    const S* gr = dy + map.offset(row, lddy);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = t + i * TPR;
+      ny[i] = raw_t{};
+      ng[i] = raw_t{};
+      if (idx < nvec) {
+        ny[i] = Vec16<S>::load_raw(yr + unsigned(W) * idx);
+        ng[i] = Vec16<S>::load_raw(gr + unsigned(W) * idx);
+      }
+    }
+  };
+  int64_t row = blockIdx.x;
+  if (row >= rows) return;
+  request(row);
+  for (int it = 0; row < rows; row += gridDim.x, ++it) {
+    float a[V][W], g[V][W];  // vectors past the end of the row hold zeros
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      Vec16<S>::unpack(ny[i], a[i]);
+      Vec16<S>::unpack(ng[i], g[i]);
+    }
+    const int64_t next = row + gridDim.x;
+    if (next < rows) request(next);
+    asm volatile("" ::: "memory");  // the next row's loads go out ahead of this row's stores
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+#pragma unroll
+      for (int k = 0; k < W; ++k) s += (KIND == kLogSoftmax) ? g[i][k] : a[i][k] * g[i][k];
+    s = team_sum<NW>(s, red[it & 1], wv, lane);
+    S* dr = dx + map.offset(row, lddx);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const unsigned idx = t + i * TPR;
+      if (idx < nvec) {
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+          if (KIND == kLogSoftmax) g[i][k] = g[i][k] - exp_quick(a[i][k]) * s;
+          else g[i][k] = a[i][k] * (g[i][k] - s);
+        }
+        Vec16<S>::store(dr + unsigned(W) * idx, g[i]);
+      }
+    }
+  }
+}
+
 }  // namespace lbn
