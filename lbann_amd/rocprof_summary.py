@@ -66,8 +66,10 @@ WORKLOADS = [
     ("ln_bwd_cluster", None, "extra: layer norm over whole samples bwd (followed by ln_wgrad_reduce_wide)", 3 * _E3 * 4),
     ("ebn_fwd_tile", None, "extra: entry-wise batch norm fwd 1048576x64", 2 * 67108864 * 4),
     ("ebn_bwd_tile", None, "extra: entry-wise batch norm bwd", 3 * 67108864 * 4),
-    ("sm_fwd_rows<__half, 1024, 4, 0", None, "extra: softmax fp16 storage fwd 32768x512", 2 * _E2 * 2),
-    ("sm_bwd_rows<__half, 1024, 4, 0", None, "extra: softmax fp16 storage bwd", 3 * _E2 * 2),
+    ("sm_fwd_rows_walk<__half, 4, 0", None, "extra: softmax fp16 storage fwd 32768x512 (a workgroup walks two rows)", 2 * _E2 * 2),
+    ("sm_bwd_rows_walk_packed<__half, 4, 0", None, "extra: softmax fp16 storage bwd (a workgroup walks two rows)", 3 * _E2 * 2),
+    ("sm_fwd_rows<__half, 1024, 4, 0", None, "extra: softmax fp16 storage fwd 32768x512, one row per workgroup (forced)", 2 * _E2 * 2),
+    ("sm_bwd_rows<__half, 1024, 4, 0", None, "extra: softmax fp16 storage bwd, one row per workgroup (forced)", 3 * _E2 * 2),
     ("sm_ce_fwd_rows<1024, 8, false>", None, "extra: softmax + cross entropy fwd 32768x512 (x, truth, y)", 3 * _E2 * 4),
     ("sm_ce_bwd_rows<1024, 8, false>", None, "extra: softmax + cross entropy bwd (y, truth, dx)", 3 * _E2 * 4),
     ("ce_fwd_dense", None, "extra: cross entropy fwd 32768x512 (x, truth)", 2 * _E2 * 4),

@@ -1,4 +1,4 @@
-"""Formats the parity report that a GPU test run leaves in gpurun_out/parity_report.json:
+"""Formats the parity report (parity_report.json) that a GPU test run leaves in its output folder:
 
     python -m tests.parity_report [path] [prefix ...]
 
