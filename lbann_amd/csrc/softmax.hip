@@ -372,9 +372,14 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     return launch_status();
   }
   if constexpr (!std::is_same<S, float>::value) {
-    // fp16 rows beyond the register kernels: one workgroup per row, three passes
-    hipLaunchKernelGGL((sm_fwd_generic<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kChunkThreads), 0, st, x, y,
-                       ldx, ldy, map, n);
+    // fp16 rows beyond the register kernels: one workgroup per row, two passes of 16-byte
+    // accesses when the rows are made of whole aligned vectors, else three passes entry by entry
+    if (vec && n / VE < (int64_t(1) << 31))
+      hipLaunchKernelGGL((sm_fwd_long_packed<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
+                         x, y, ldx, ldy, map, static_cast<unsigned>(n / VE));
+    else
+      hipLaunchKernelGGL((sm_fwd_generic<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kChunkThreads), 0, st, x,
+                         y, ldx, ldy, map, n);
     return launch_status();
   }
   else {
@@ -537,8 +542,12 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     return launch_status();
   }
   if constexpr (!std::is_same<S, float>::value) {
-    hipLaunchKernelGGL((sm_bwd_generic<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kChunkThreads), 0, st, y, dy,
-                       dx, ldy, lddy, lddx, map, n);
+    if (vec && n / VE < (int64_t(1) << 31))
+      hipLaunchKernelGGL((sm_bwd_long_packed<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
+                         y, dy, dx, ldy, lddy, lddx, map, static_cast<unsigned>(n / VE));
+    else
+      hipLaunchKernelGGL((sm_bwd_generic<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kChunkThreads), 0, st, y,
+                         dy, dx, ldy, lddy, lddx, map, n);
     return launch_status();
   }
   else {

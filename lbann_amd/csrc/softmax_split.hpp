@@ -366,4 +366,160 @@ sm_bwd_generic(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_
   }
 }
 
+// The same rows when they are made of whole, aligned 16-byte vectors (a vocabulary of 128256
+// entries, say): one 1024-thread workgroup per row, packed 16-byte accesses, two passes.  The first
+// takes the maximum and the sum of exponentials together (a thread rescales its sum when its
+// maximum rises), the second writes the output; it finds the row in the last-level caches, so
+// the input crosses HBM once.  16-bit storage: the two-operation exponential (sm_fwd_rows).
+constexpr int kLongThreads = 1024;
+constexpr int kLongUnroll = 4;
+
+template <typename S, int KIND>
+__global__ void __launch_bounds__(kLongThreads)
+sm_fwd_long_packed(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, unsigned nvec)
+{
+  static_assert(sizeof(S) == 2, "packed 16-bit rows");
+  constexpr int W = Vec16<S>::N, NW = kLongThreads / kWave, U = kLongUnroll;
+  using raw_t = typename Vec16<S>::raw_t;
+  __shared__ float red[2][NW];
+  const int64_t row = blockIdx.x;
+  const S* xr = x + map.offset(row, ldx);
+  S* yr = y + map.offset(row, ldy);
+  const unsigned t = threadIdx.x;
+  const int lane = t & (kWave - 1), wv = t / kWave;
+  float m = -FLT_MAX, s = 0.f;
+  for (unsigned i0 = t; i0 < nvec; i0 += U * kLongThreads) {
+    raw_t r[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const unsigned idx = i0 + u * kLongThreads;
+      r[u] = raw_t{};
+      if (idx < nvec) r[u] = Vec16<S>::load_raw(xr + static_cast<int64_t>(W) * idx);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (i0 + u * kLongThreads >= nvec) continue;
+      float v[W];
+      Vec16<S>::unpack(r[u], v);
+      float vm = v[0];
+#pragma unroll
+      for (int k = 1; k < W; ++k) vm = fmaxf(vm, v[k]);
+      if (vm > m) {
+        s *= exp_quick(m - vm);
+        m = vm;
+      }
+#pragma unroll
+      for (int k = 0; k < W; ++k) s += exp_quick(v[k] - m);
+    }
+  }
+  float gm = wave_max(m);
+  float gs = wave_sum(s * exp_fast(m - gm));
+  if (lane == 0) {
+    red[0][wv] = gm;
+    red[1][wv] = gs;
+  }
+  __syncthreads();
+  const float pm = lane < NW ? red[0][lane] : -FLT_MAX;
+  const float ps = lane < NW ? red[1][lane] : 0.f;
+  gm = wave_max(pm);
+  gs = wave_sum(ps * exp_fast(pm - gm));
+  const float f = 1.0f / gs;
+  const float lse = (KIND == kLogSoftmax) ? log_of_sum(gs) : 0.f;
+  // in place: a thread writes the vectors it has just read, and every read of the first pass
+  // lies before the barrier above
+  for (unsigned i0 = t; i0 < nvec; i0 += U * kLongThreads) {
+    raw_t r[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const unsigned idx = i0 + u * kLongThreads;
+      r[u] = raw_t{};
+      if (idx < nvec) r[u] = Vec16<S>::load_raw(xr + static_cast<int64_t>(W) * idx);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const unsigned idx = i0 + u * kLongThreads;
+      if (idx >= nvec) continue;
+      float v[W];
+      Vec16<S>::unpack(r[u], v);
+#pragma unroll
+      for (int k = 0; k < W; ++k) {
+        const float d = v[k] - gm;
+        if (KIND == kLogSoftmax) {
+          v[k] = d - lse;
+        }
+        else {
+          const float e = f * exp_quick(d);
+          v[k] = __builtin_isnormal(e) ? e : 0.f;
+        }
+      }
+      Vec16<S>::store(yr + static_cast<int64_t>(W) * idx, v);
+    }
+  }
+}
+
+template <typename S, int KIND>
+__global__ void __launch_bounds__(kLongThreads)
+sm_bwd_long_packed(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx, RowMap map,
+                   unsigned nvec)
+{
+  static_assert(sizeof(S) == 2, "packed 16-bit rows");
+  constexpr int W = Vec16<S>::N, NW = kLongThreads / kWave, U = kLongUnroll / 2;
+  using raw_t = typename Vec16<S>::raw_t;
+  __shared__ float red[NW];
+  const int64_t row = blockIdx.x;
+  const S* yr = y + map.offset(row, ldy);
+  const S* gr = dy + map.offset(row, lddy);
+  S* dr = dx + map.offset(row, lddx);
+  const unsigned t = threadIdx.x;
+  const int lane = t & (kWave - 1), wv = t / kWave;
+  float s = 0.f;
+  for (unsigned i0 = t; i0 < nvec; i0 += U * kLongThreads) {
+    raw_t ra[U], rg[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const unsigned idx = i0 + u * kLongThreads;
+      ra[u] = raw_t{};
+      rg[u] = raw_t{};
+      if (idx < nvec) {
+        if (KIND != kLogSoftmax) ra[u] = Vec16<S>::load_raw(yr + static_cast<int64_t>(W) * idx);
+        rg[u] = Vec16<S>::load_raw(gr + static_cast<int64_t>(W) * idx);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float a[W], g[W];  // vectors past the end hold zeros
+      Vec16<S>::unpack(ra[u], a);
+      Vec16<S>::unpack(rg[u], g);
+#pragma unroll
+      for (int k = 0; k < W; ++k) s += (KIND == kLogSoftmax) ? g[k] : a[k] * g[k];
+    }
+  }
+  s = team_sum<NW>(s, red, wv, lane);
+  // in place (dx aliasing dy or y): a thread writes the vectors it has just read, after the sum
+  for (unsigned i0 = t; i0 < nvec; i0 += U * kLongThreads) {
+    raw_t ra[U], rg[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const unsigned idx = i0 + u * kLongThreads;
+      ra[u] = raw_t{};
+      rg[u] = raw_t{};
+      if (idx < nvec) {
+        ra[u] = Vec16<S>::load_raw(yr + static_cast<int64_t>(W) * idx);
+        rg[u] = Vec16<S>::load_raw(gr + static_cast<int64_t>(W) * idx);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const unsigned idx = i0 + u * kLongThreads;
+      if (idx >= nvec) continue;
+      float a[W], g[W];
+      Vec16<S>::unpack(ra[u], a);
+      Vec16<S>::unpack(rg[u], g);
+#pragma unroll
+      for (int k = 0; k < W; ++k) g[k] = (KIND == kLogSoftmax) ? g[k] - exp_quick(a[k]) * s : a[k] * (g[k] - s);
+      Vec16<S>::store(dr + static_cast<int64_t>(W) * idx, g);
+    }
+  }
+}
+
 }  // namespace lbn
