@@ -156,6 +156,21 @@ static bool same_frames(const void* a, int64_t lda, const void* b, int64_t ldb, 
   return (pa & 3u) == 0 && ((pa ^ pb) & 15u) == 0 && (w <= 1 || ((lda - ldb) & 3) == 0);
 }
 
+// The same for 16-bit entries (eight to a vector).
+static bool same_frames16(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t w)
+{
+  const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+  return (pa & 1u) == 0 && ((pa ^ pb) & 15u) == 0 && (w <= 1 || ((lda - ldb) & 7) == 0);
+}
+
+// Shortest 16-bit row off the 16-byte grid that takes the packed two-pass kernel rather than the
+// register kernels with one entry per access (LBN_F16_LONG_MIN overrides, for experiments).
+static int64_t packed_long_min16()
+{
+  static const int64_t v = std::getenv("LBN_F16_LONG_MIN") ? std::atoll(std::getenv("LBN_F16_LONG_MIN")) : 2048;
+  return v;
+}
+
 static bool framed_access()
 {
   static const bool off = std::getenv("LBN_NO_FRAMED_ACCESS") != nullptr;
@@ -342,6 +357,11 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   else if (sm_fwd_framed_rows<KIND>(st, n, w, rows, x, ldx, y, ldy, map)) {
     return launch_status();
   }
+  else if (sizeof(S) == 2 && n >= packed_long_min16() && groups == 1 && same_frames16(x, ldx, y, ldy, w) &&
+           framed_access()) {
+    // 16-bit rows off the 16-byte grid, long enough for a workgroup each: the packed two-pass
+    // kernel below instead of registers filled two bytes at a time
+  }
   else if (n <= kMaxScalarRow) {
     // rows that are only 4-byte aligned and short enough for registers: one float per access
     const RowConfig c = pick_sm_row_config(n, rows);
@@ -374,9 +394,12 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   if constexpr (!std::is_same<S, float>::value) {
     // fp16 rows beyond the register kernels: one workgroup per row, two passes of 16-byte
     // accesses when the rows are made of whole aligned vectors, else three passes entry by entry
-    if (vec && n / VE < (int64_t(1) << 31))
-      hipLaunchKernelGGL((sm_fwd_long_packed<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
-                         x, y, ldx, ldy, map, static_cast<unsigned>(n / VE));
+    if (vec && n < (int64_t(1) << 34))
+      hipLaunchKernelGGL((sm_fwd_long_packed<S, KIND, false>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads),
+                         0, st, x, y, ldx, ldy, map, n);
+    else if (groups == 1 && same_frames16(x, ldx, y, ldy, w) && n < (int64_t(1) << 34) && framed_access())
+      hipLaunchKernelGGL((sm_fwd_long_packed<S, KIND, true>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads),
+                         0, st, x, y, ldx, ldy, map, n);
     else
       hipLaunchKernelGGL((sm_fwd_generic<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kChunkThreads), 0, st, x,
                          y, ldx, ldy, map, n);
@@ -512,6 +535,10 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   else if (sm_bwd_framed_rows<KIND>(st, n, w, rows, y, ldy, dy, lddy, dx, lddx, map)) {
     return launch_status();
   }
+  else if (sizeof(S) == 2 && n >= packed_long_min16() && groups == 1 && same_frames16(y, ldy, dy, lddy, w) &&
+           same_frames16(y, ldy, dx, lddx, w) && framed_access()) {
+    // (as in the forward pass: the packed two-pass kernel below)
+  }
   else if (n <= kMaxScalarRow) {
     const RowConfig c = pick_sm_row_config(n, rows);
     if (c.tpr) {
@@ -542,9 +569,13 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     return launch_status();
   }
   if constexpr (!std::is_same<S, float>::value) {
-    if (vec && n / VE < (int64_t(1) << 31))
-      hipLaunchKernelGGL((sm_bwd_long_packed<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
-                         y, dy, dx, ldy, lddy, lddx, map, static_cast<unsigned>(n / VE));
+    if (vec && n < (int64_t(1) << 34))
+      hipLaunchKernelGGL((sm_bwd_long_packed<S, KIND, false>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads),
+                         0, st, y, dy, dx, ldy, lddy, lddx, map, n);
+    else if (groups == 1 && same_frames16(y, ldy, dy, lddy, w) && same_frames16(y, ldy, dx, lddx, w) &&
+             n < (int64_t(1) << 34) && framed_access())
+      hipLaunchKernelGGL((sm_bwd_long_packed<S, KIND, true>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads),
+                         0, st, y, dy, dx, ldy, lddy, lddx, map, n);
     else
       hipLaunchKernelGGL((sm_bwd_generic<S, KIND>), dim3(static_cast<unsigned>(rows)), dim3(kChunkThreads), 0, st, y,
                          dy, dx, ldy, lddy, lddx, map, n);

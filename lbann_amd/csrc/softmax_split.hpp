@@ -366,35 +366,70 @@ sm_bwd_generic(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_
   }
 }
 
-// The same rows when they are made of whole, aligned 16-byte vectors (a vocabulary of 128256
-// entries, say): one 1024-thread workgroup per row, packed 16-byte accesses, two passes.  The first
-// takes the maximum and the sum of exponentials together (a thread rescales its sum when its
-// maximum rises), the second writes the output; it finds the row in the last-level caches, so
-// the input crosses HBM once.  16-bit storage: the two-operation exponential (sm_fwd_rows).
+// The same rows in packed 16-byte accesses: one 1024-thread workgroup per row, two passes.  The
+// first takes the maximum and the sum of exponentials together (a thread rescales its sum when
+// its maximum rises), the second writes the output; it finds the row in the last-level caches,
+// so the input crosses HBM once.  16-bit storage: the two-operation exponential (sm_fwd_rows).
+// FR: rows that start off the 16-byte grid (a vocabulary of 50257 entries) are cut per row into
+// up to 7 leading entries, aligned vectors and up to 7 trailing entries; every tensor of the call
+// starts each row at the same distance from a 16-byte boundary (checked on the host).
 constexpr int kLongThreads = 1024;
 constexpr int kLongUnroll = 4;
 
-template <typename S, int KIND>
+// The cut of one row of n 16-bit entries at p.
+struct PackedRowCut {
+  unsigned head, nvec, tail;
+  // Entry handled by thread t < head + tail as a single value.
+  __device__ __forceinline__ int64_t edge(unsigned t) const
+  {
+    return t < head ? t : static_cast<int64_t>(head) + 8 * static_cast<int64_t>(nvec) + (t - head);
+  }
+};
+
+template <bool FR>
+__device__ __forceinline__ PackedRowCut packed_row_cut(const void* p, int64_t n)
+{
+  if (!FR) return {0u, static_cast<unsigned>(n / 8), 0u};
+  const unsigned shift = static_cast<unsigned>(reinterpret_cast<uintptr_t>(p) & 15u) / 2;
+  unsigned head = (8 - shift) & 7;
+  if (head > n) head = static_cast<unsigned>(n);
+  const unsigned nvec = static_cast<unsigned>((n - head) / 8);
+  return {head, nvec, static_cast<unsigned>(n - head - 8 * static_cast<int64_t>(nvec))};
+}
+
+template <typename S, int KIND, bool FR>
 __global__ void __launch_bounds__(kLongThreads)
-sm_fwd_long_packed(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, unsigned nvec)
+sm_fwd_long_packed(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t n)
 {
   static_assert(sizeof(S) == 2, "packed 16-bit rows");
   constexpr int W = Vec16<S>::N, NW = kLongThreads / kWave, U = kLongUnroll;
+  static_assert(W == 8, "eight entries per vector");
   using raw_t = typename Vec16<S>::raw_t;
   __shared__ float red[2][NW];
   const int64_t row = blockIdx.x;
   const S* xr = x + map.offset(row, ldx);
   S* yr = y + map.offset(row, ldy);
+  const PackedRowCut cut = packed_row_cut<FR>(xr, n);
+  const S* xv = xr + cut.head;
+  S* yv = yr + cut.head;
+  const unsigned nvec = cut.nvec;
   const unsigned t = threadIdx.x;
   const int lane = t & (kWave - 1), wv = t / kWave;
   float m = -FLT_MAX, s = 0.f;
+  const bool edge = FR && t < cut.head + cut.tail;
+  float ev = 0.f;
+  if (edge) {
+    ev = Vec16<S>::load1(xr + cut.edge(t));
+    m = fmaxf(m, ev);
+    s = exp_quick(ev - m);
+  }
   for (unsigned i0 = t; i0 < nvec; i0 += U * kLongThreads) {
     raw_t r[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const unsigned idx = i0 + u * kLongThreads;
       r[u] = raw_t{};
-      if (idx < nvec) r[u] = Vec16<S>::load_raw(xr + static_cast<int64_t>(W) * idx);
+      if (idx < nvec) r[u] = Vec16<S>::load_raw(xv + static_cast<int64_t>(W) * idx);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -425,15 +460,22 @@ sm_fwd_long_packed(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, unsig
   gs = wave_sum(ps * exp_fast(pm - gm));
   const float f = 1.0f / gs;
   const float lse = (KIND == kLogSoftmax) ? log_of_sum(gs) : 0.f;
-  // in place: a thread writes the vectors it has just read, and every read of the first pass
-  // lies before the barrier above
+  auto result = [&](float v) {
+    const float d = v - gm;
+    if (KIND == kLogSoftmax) return d - lse;
+    const float e = f * exp_quick(d);
+    return __builtin_isnormal(e) ? e : 0.f;
+  };
+  // in place: a thread writes what it has read itself, and every read of the first pass lies
+  // before the barrier above
+  if (edge) Vec16<S>::store1(yr + cut.edge(t), result(ev));
   for (unsigned i0 = t; i0 < nvec; i0 += U * kLongThreads) {
     raw_t r[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const unsigned idx = i0 + u * kLongThreads;
       r[u] = raw_t{};
-      if (idx < nvec) r[u] = Vec16<S>::load_raw(xr + static_cast<int64_t>(W) * idx);
+      if (idx < nvec) r[u] = Vec16<S>::load_raw(xv + static_cast<int64_t>(W) * idx);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -442,37 +484,39 @@ sm_fwd_long_packed(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, unsig
       float v[W];
       Vec16<S>::unpack(r[u], v);
 #pragma unroll
-      for (int k = 0; k < W; ++k) {
-        const float d = v[k] - gm;
-        if (KIND == kLogSoftmax) {
-          v[k] = d - lse;
-        }
-        else {
-          const float e = f * exp_quick(d);
-          v[k] = __builtin_isnormal(e) ? e : 0.f;
-        }
-      }
-      Vec16<S>::store(yr + static_cast<int64_t>(W) * idx, v);
+      for (int k = 0; k < W; ++k) v[k] = result(v[k]);
+      Vec16<S>::store(yv + static_cast<int64_t>(W) * idx, v);
     }
   }
 }
 
-template <typename S, int KIND>
+template <typename S, int KIND, bool FR>
 __global__ void __launch_bounds__(kLongThreads)
-sm_bwd_long_packed(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx, RowMap map,
-                   unsigned nvec)
+sm_bwd_long_packed(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx, RowMap map, int64_t n)
 {
   static_assert(sizeof(S) == 2, "packed 16-bit rows");
   constexpr int W = Vec16<S>::N, NW = kLongThreads / kWave, U = kLongUnroll / 2;
+  static_assert(W == 8, "eight entries per vector");
   using raw_t = typename Vec16<S>::raw_t;
   __shared__ float red[NW];
   const int64_t row = blockIdx.x;
   const S* yr = y + map.offset(row, ldy);
   const S* gr = dy + map.offset(row, lddy);
   S* dr = dx + map.offset(row, lddx);
+  const PackedRowCut cut = packed_row_cut<FR>(yr, n);
+  const S* yv = yr + cut.head;
+  const S* gv = gr + cut.head;
+  S* dv = dr + cut.head;
+  const unsigned nvec = cut.nvec;
   const unsigned t = threadIdx.x;
   const int lane = t & (kWave - 1), wv = t / kWave;
-  float s = 0.f;
+  const bool edge = FR && t < cut.head + cut.tail;
+  float ea = 0.f, eg = 0.f, s = 0.f;
+  if (edge) {
+    ea = Vec16<S>::load1(yr + cut.edge(t));
+    eg = Vec16<S>::load1(gr + cut.edge(t));
+    s = (KIND == kLogSoftmax) ? eg : ea * eg;
+  }
   for (unsigned i0 = t; i0 < nvec; i0 += U * kLongThreads) {
     raw_t ra[U], rg[U];
 #pragma unroll
@@ -481,8 +525,8 @@ sm_bwd_long_packed(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, in
       ra[u] = raw_t{};
       rg[u] = raw_t{};
       if (idx < nvec) {
-        if (KIND != kLogSoftmax) ra[u] = Vec16<S>::load_raw(yr + static_cast<int64_t>(W) * idx);
-        rg[u] = Vec16<S>::load_raw(gr + static_cast<int64_t>(W) * idx);
+        if (KIND != kLogSoftmax) ra[u] = Vec16<S>::load_raw(yv + static_cast<int64_t>(W) * idx);
+        rg[u] = Vec16<S>::load_raw(gv + static_cast<int64_t>(W) * idx);
       }
     }
 #pragma unroll
@@ -495,7 +539,9 @@ sm_bwd_long_packed(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, in
     }
   }
   s = team_sum<NW>(s, red, wv, lane);
-  // in place (dx aliasing dy or y): a thread writes the vectors it has just read, after the sum
+  auto result = [&](float a, float g) { return (KIND == kLogSoftmax) ? g - exp_quick(a) * s : a * (g - s); };
+  // in place (dx aliasing dy or y): a thread writes what it has read itself, after the sum
+  if (edge) Vec16<S>::store1(dr + cut.edge(t), result(ea, eg));
   for (unsigned i0 = t; i0 < nvec; i0 += U * kLongThreads) {
     raw_t ra[U], rg[U];
 #pragma unroll
@@ -504,8 +550,8 @@ sm_bwd_long_packed(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, in
       ra[u] = raw_t{};
       rg[u] = raw_t{};
       if (idx < nvec) {
-        ra[u] = Vec16<S>::load_raw(yr + static_cast<int64_t>(W) * idx);
-        rg[u] = Vec16<S>::load_raw(gr + static_cast<int64_t>(W) * idx);
+        ra[u] = Vec16<S>::load_raw(yv + static_cast<int64_t>(W) * idx);
+        rg[u] = Vec16<S>::load_raw(gv + static_cast<int64_t>(W) * idx);
       }
     }
 #pragma unroll
@@ -516,8 +562,8 @@ sm_bwd_long_packed(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, in
       Vec16<S>::unpack(ra[u], a);
       Vec16<S>::unpack(rg[u], g);
 #pragma unroll
-      for (int k = 0; k < W; ++k) g[k] = (KIND == kLogSoftmax) ? g[k] - exp_quick(a[k]) * s : a[k] * (g[k] - s);
-      Vec16<S>::store(dr + static_cast<int64_t>(W) * idx, g);
+      for (int k = 0; k < W; ++k) g[k] = result(a[k], g[k]);
+      Vec16<S>::store(dv + static_cast<int64_t>(W) * idx, g);
     }
   }
 }

@@ -87,7 +87,8 @@ def test_softmax_family(L, kind, h, w, pad):
     (64, 5000, 0, False), (24, 4099, 0, False),                                             # short rows, 16-lane teams
     (70000, 3, 0, False), (40001, 2, 0, True), (131072, 2, 0, False),                        # beyond the register kernels
     (32768, 300, 0, True), (20480, 513, 0, False), (24584, 260, 8, False),    # more rows than compute units: walked
-    (128256, 40, 0, True), (65544, 5, 8, False), (65540, 3, 0, False),        # long rows: two packed passes / entry by entry
+    (128256, 40, 0, True), (65544, 5, 8, False), (65540, 3, 0, False),        # long rows: two packed passes,
+    (50257, 9, 0, True), (40001, 5, 16, False), (33001, 7, 0, False), (32770, 4, 3, False),  # cut at 16-byte boundaries per row
 ])
 def test_softmax_family_f16_storage(L, kind, h, w, pad, in_place):
     """fp16 storage, fp32 arithmetic (softmax.cpp:236-243 instantiates the layers for half):
