@@ -53,7 +53,8 @@
  * layer classes do both.
  *
  * Process-wide state of the library: the counter the per-call tags are drawn from (an
- * atomic), the cached occupancy figures per kernel and device, per device the stream of the
+ * atomic), the cached occupancy figures per kernel and device and compute-unit counts per
+ * device, per device the stream of the
  * last cluster kernel with its mutex and (once a second stream has been seen) one event,
  * and the environment switches, each read once.  Nothing else outlives a call.
  */

@@ -6,6 +6,7 @@
 
 #include <cstdint>
 #include <cstdlib>
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -103,6 +104,20 @@ inline RowConfig pick_row_config(int64_t nvec, int64_t rows, int max_v = 8)
   while (pick < 2 && vs[pick] > 1 && rows * (tprs[pick] / 64) < want_waves && vs[pick + 1] != 0)
     ++pick;
   return {tprs[pick], vs[pick]};
+}
+
+// Compute units of the current device (0 if the query fails); asked once per device.
+inline int compute_units()
+{
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  int cus = cached[dev].load(std::memory_order_relaxed);
+  if (cus > 0) return cus;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) return 0;
+  cached[dev].store(cus, std::memory_order_relaxed);
+  return cus;
 }
 
 // Workgroups of `threads` threads running `kernel` that the current device holds at

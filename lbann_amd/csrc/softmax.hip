@@ -306,11 +306,8 @@ static bool sm_fwd_walk(hipStream_t st, int64_t rows, unsigned nvec, const S* x,
 {
   static const bool off = std::getenv("LBN_NO_FWD_WALK") != nullptr;
   if (off || KIND == kChannelwise) return false;
-  int cus = 0, dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess ||
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
-    return false;
-  if (rows <= cus) return false;
+  const int cus = compute_units();
+  if (cus < 1 || rows <= cus) return false;
   hipLaunchKernelGGL((sm_fwd_rows_walk<S, 4, KIND>), dim3(static_cast<unsigned>(cus)), dim3(1024), 0, st, x, y, ldx,
                      ldy, map, rows, nvec);
   return true;
