@@ -1160,7 +1160,7 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
       hipLaunchKernelGGL(ln_wgrad_reduce, dim3(static_cast<unsigned>(ceil_div(n, 32)), 2), dim3(256), 0, st,
                          part, p.blocks, n, dgamma, dbeta);
     else
-      hipLaunchKernelGGL(ln_wgrad_reduce_scalar, dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, st,
+      hipLaunchKernelGGL(ln_wgrad_reduce_scalar, dim3(static_cast<unsigned>(ceil_div(n, kWgradScalarCols)), 2), dim3(256), 0, st,
                          part, p.blocks, n, dgamma, dbeta);
   }
   return 1;
@@ -1259,7 +1259,7 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
         hipLaunchKernelGGL(ln_wgrad_reduce, dim3(static_cast<unsigned>(ceil_div(n, 32)), 2), dim3(256), 0, st,
                            wpart, slabs, n, dgamma, dbeta);
       else
-        hipLaunchKernelGGL(ln_wgrad_reduce_scalar, dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0,
+        hipLaunchKernelGGL(ln_wgrad_reduce_scalar, dim3(static_cast<unsigned>(ceil_div(n, kWgradScalarCols)), 2), dim3(256), 0,
                            st, wpart, slabs, n, dgamma, dbeta);
     }
     else {

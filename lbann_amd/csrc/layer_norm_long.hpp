@@ -265,21 +265,44 @@ ln_wgrad_columns(const T* __restrict__ x, const T* __restrict__ dy, int64_t ldx,
   }
 }
 
-// Scalar companion of ln_wgrad_reduce for n that is not a multiple of 4: one thread per
-// feature adds the P partial rows in order.
+// Scalar companion of ln_wgrad_reduce for n that is not a multiple of 4.  A workgroup takes
+// 32 features of one of the two rows (blockIdx.y: dscale, dbias): thread (c, g) adds the partial
+// rows g, g + 8, ... of feature c with eight loads in flight, and the eight groups are added
+// through LDS in a fixed order.  (One thread per feature walking all P rows by itself left a
+// 1001-feature problem with four workgroups: 107 us for 256 partial rows.)
+constexpr int kWgradScalarCols = 32;
 __global__ void __launch_bounds__(256)
 ln_wgrad_reduce_scalar(const float* __restrict__ part, int64_t P, int64_t n, float* __restrict__ dscale,
                        float* __restrict__ dbias)
 {
-  const int64_t k = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (k >= n) return;
-  float sg = 0.f, sb = 0.f;
-  for (int64_t p = 0; p < P; ++p) {
-    sg += part[p * 2 * n + k];
-    sb += part[p * 2 * n + n + k];
+  constexpr int C = kWgradScalarCols, G = 256 / C, U = 8;
+  __shared__ float sm[G][C + 1];
+  float* out = blockIdx.y == 0 ? dscale : dbias;
+  if (!out) return;
+  const int c = threadIdx.x % C, g = threadIdx.x / C;
+  const int64_t k = static_cast<int64_t>(blockIdx.x) * C + c;
+  float acc = 0.f;
+  if (k < n) {
+    const float* src = part + blockIdx.y * n + k;
+    for (int64_t p0 = g; p0 < P; p0 += static_cast<int64_t>(G) * U) {
+      float w[U];
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const int64_t q = p0 + static_cast<int64_t>(G) * j;
+        w[j] = q < P ? src[q * 2 * n] : 0.f;
+      }
+      acc += ((w[0] + w[1]) + (w[2] + w[3])) + ((w[4] + w[5]) + (w[6] + w[7]));
+    }
   }
-  if (dscale) dscale[k] = sg;
-  if (dbias) dbias[k] = sb;
+  sm[g][c] = acc;
+  __syncthreads();
+  if (threadIdx.x < C) {
+    const int64_t kc = static_cast<int64_t>(blockIdx.x) * C + threadIdx.x;
+    if (kc < n) {
+      const int t = threadIdx.x;
+      out[kc] = ((sm[0][t] + sm[1][t]) + (sm[2][t] + sm[3][t])) + ((sm[4][t] + sm[5][t]) + (sm[6][t] + sm[7][t]));
+    }
+  }
 }
 
 }  // namespace lbn
