@@ -122,18 +122,59 @@ __device__ __forceinline__ float2 bn_rt_channel_total(const float2* part, int64_
   return make_float2(wave_sum(static_cast<float>(a)), wave_sum(static_cast<float>(b)));
 }
 
-// One wave per channel (4 channels per workgroup).
-template <typename S>
+// The same by a whole workgroup, for channels of many rows (a 111 x 111 map: 12321 rows, which
+// one wave walked for 58 us): thread-strided with four independent loads in flight, waves added
+// through LDS in order.  Thread 0 gets the totals.
+constexpr int64_t kBnRtWideChannel = 256;  // rows x slabs from which a channel takes a workgroup
+
+__device__ __forceinline__ float2 bn_rt_channel_total_wide(const float2* part, int64_t h, int slabs, int64_t cs,
+                                                           int64_t c)
+{
+  __shared__ float2 red[kRowTileWaves];
+  constexpr int U = 4;
+  double a[U] = {0., 0., 0., 0.}, b[U] = {0., 0., 0., 0.};
+  for (int s = 0; s < slabs; ++s) {
+    const float2* row = part + static_cast<int64_t>(s) * h + c * cs;
+    for (int64_t i0 = threadIdx.x; i0 < cs; i0 += U * kRowTileThreads) {
+      float2 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t i = i0 + u * kRowTileThreads;
+        v[u] = i < cs ? row[i] : make_float2(0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        a[u] += static_cast<double>(v[u].x);
+        b[u] += static_cast<double>(v[u].y);
+      }
+    }
+  }
+  const float ta = wave_sum(static_cast<float>((a[0] + a[1]) + (a[2] + a[3])));
+  const float tb = wave_sum(static_cast<float>((b[0] + b[1]) + (b[2] + b[3])));
+  if ((threadIdx.x & (kWave - 1)) == 0) red[wave_index()] = make_float2(ta, tb);
+  __syncthreads();
+  float2 t = red[0];
+#pragma unroll
+  for (int k = 1; k < kRowTileWaves; ++k) {
+    t.x += red[k].x;
+    t.y += red[k].y;
+  }
+  return t;
+}
+
+// One wave per channel (4 channels per workgroup); WIDE: one workgroup per channel.
+template <typename S, bool WIDE>
 __global__ void __launch_bounds__(kRowTileThreads)
 bn_rt_fwd_stats(int64_t C, int64_t cs, int64_t w, int64_t h, int slabs, const float2* __restrict__ part,
                 const S* __restrict__ x, int use_pivot, int bessel, float eps, float decay,
                 float* __restrict__ mean, float* __restrict__ var, float* __restrict__ rmean,
                 float* __restrict__ rvar)
 {
-  const int64_t c = static_cast<int64_t>(blockIdx.x) * kRowTileWaves + wave_index();
+  const int64_t c = WIDE ? static_cast<int64_t>(blockIdx.x)
+                         : static_cast<int64_t>(blockIdx.x) * kRowTileWaves + wave_index();
   if (c >= C) return;
-  const float2 t = bn_rt_channel_total(part, h, slabs, cs, c);
-  if ((threadIdx.x & (kWave - 1)) != 0) return;
+  const float2 t = WIDE ? bn_rt_channel_total_wide(part, h, slabs, cs, c) : bn_rt_channel_total(part, h, slabs, cs, c);
+  if (WIDE ? threadIdx.x != 0 : (threadIdx.x & (kWave - 1)) != 0) return;
   const int64_t n = cs * w;
   if (n <= 1) {  // batch_normalization.cpp:118-120: the mean holds x, the variance is 1
     mean[c] = Vec16<S>::load1(x + c * cs);
@@ -149,16 +190,18 @@ bn_rt_fwd_stats(int64_t C, int64_t cs, int64_t w, int64_t h, int slabs, const fl
   rvar[c] = decay * rvar[c] + (1.f - decay) * v;
 }
 
+template <bool WIDE>
 __global__ void __launch_bounds__(kRowTileThreads)
 bn_rt_bwd_stats(int64_t C, int64_t cs, int64_t h, int slabs, const float2* __restrict__ part, float eps,
                 int training, const float* __restrict__ var, const float* __restrict__ scale,
                 float* __restrict__ dscale, float* __restrict__ dbias, float* __restrict__ dmean,
                 float* __restrict__ dvar)
 {
-  const int64_t c = static_cast<int64_t>(blockIdx.x) * kRowTileWaves + wave_index();
+  const int64_t c = WIDE ? static_cast<int64_t>(blockIdx.x)
+                         : static_cast<int64_t>(blockIdx.x) * kRowTileWaves + wave_index();
   if (c >= C) return;
-  const float2 t = bn_rt_channel_total(part, h, slabs, cs, c);
-  if ((threadIdx.x & (kWave - 1)) != 0) return;
+  const float2 t = WIDE ? bn_rt_channel_total_wide(part, h, slabs, cs, c) : bn_rt_channel_total(part, h, slabs, cs, c);
+  if (WIDE ? threadIdx.x != 0 : (threadIdx.x & (kWave - 1)) != 0) return;
   const float inv_stdev = 1.0f / sqrtf(var[c] + eps);
   float ds, db, dm, dv;
   grads_from_sums(t.x, t.y, scale[c], inv_stdev, ds, db, dm, dv);

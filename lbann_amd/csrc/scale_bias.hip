@@ -179,29 +179,66 @@ esb_merge_slabs(int64_t h, int slabs, const float2* __restrict__ part, float* __
 }
 
 // Channel-wise weight gradients from per-row pairs: one wave per channel adds the pairs of
-// its cs rows in every slab (lane-strided, then a wave sum: a fixed order).
+// its cs rows in every slab (lane-strided, then a wave sum: a fixed order).  WIDE: a whole
+// workgroup per channel with four loads per thread in flight, for channels of many rows (one
+// wave took 16 us over 3025 rows).
+constexpr int64_t kCsbWideChannel = 256;  // rows x slabs from which a channel takes a workgroup
+
+template <bool WIDE>
 __global__ void __launch_bounds__(kSbThreads)
 csb_merge_rows(int64_t C, int64_t cs, int64_t h, int slabs, const float2* __restrict__ part,
                float* __restrict__ wgrad, int64_t ld_wgrad)
 {
-  const int64_t ch = static_cast<int64_t>(blockIdx.x) * kSbWaves + wave_index();
+  __shared__ float2 red[kSbWaves];
+  const int64_t ch = WIDE ? static_cast<int64_t>(blockIdx.x)
+                          : static_cast<int64_t>(blockIdx.x) * kSbWaves + wave_index();
   if (ch >= C) return;
   const int lane = threadIdx.x & (kWave - 1);
-  float a = 0.f, b = 0.f;
+  constexpr int U = WIDE ? 4 : 1;
+  const int64_t first = WIDE ? threadIdx.x : lane;
+  const int64_t step = WIDE ? kSbThreads : kWave;
+  float a[U], b[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) a[u] = b[u] = 0.f;
   for (int s = 0; s < slabs; ++s) {
     const float2* row = part + static_cast<int64_t>(s) * h + ch * cs;
-    for (int64_t i = lane; i < cs; i += kWave) {
-      const float2 v = row[i];
-      a += v.x;
-      b += v.y;
+    for (int64_t i0 = first; i0 < cs; i0 += U * step) {
+      float2 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t i = i0 + u * step;
+        v[u] = i < cs ? row[i] : make_float2(0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        a[u] += v[u].x;
+        b[u] += v[u].y;
+      }
     }
   }
-  a = wave_sum(a);
-  b = wave_sum(b);
-  if (lane == 0) {
-    wgrad[ch] = a;
-    wgrad[ch + ld_wgrad] = b;
+  float ta = a[0], tb = b[0];
+  if (WIDE) {
+    ta = (a[0] + a[U > 1 ? 1 : 0]) + (a[U > 2 ? 2 : 0] + a[U > 3 ? 3 : 0]);
+    tb = (b[0] + b[U > 1 ? 1 : 0]) + (b[U > 2 ? 2 : 0] + b[U > 3 ? 3 : 0]);
   }
+  ta = wave_sum(ta);
+  tb = wave_sum(tb);
+  if (WIDE) {
+    if (lane == 0) red[wave_index()] = make_float2(ta, tb);
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    ta = red[0].x, tb = red[0].y;
+#pragma unroll
+    for (int k = 1; k < kSbWaves; ++k) {
+      ta += red[k].x;
+      tb += red[k].y;
+    }
+  }
+  else if (lane != 0) {
+    return;
+  }
+  wgrad[ch] = ta;
+  wgrad[ch + ld_wgrad] = tb;
 }
 
 // One thread per row, scalar and coalesced: any shape and alignment.
@@ -534,9 +571,13 @@ int lbn_channelwise_scale_bias_bwd_f32(lbn_stream_t stream, int64_t num_channels
     const dim3 grid(static_cast<unsigned>(p.tiles), static_cast<unsigned>(p.slabs));
     if (p.gw == 1) hipLaunchKernelGGL((esb_bwd_tile<1, true>), grid, dim3(kSbThreads), 0, st, e);
     else hipLaunchKernelGGL((esb_bwd_tile<4, true>), grid, dim3(kSbThreads), 0, st, e);
-    hipLaunchKernelGGL(csb_merge_rows, dim3(static_cast<unsigned>(ceil_div(num_channels, kSbWaves))),
-                       dim3(kSbThreads), 0, st, num_channels, channel_size, height, p.slabs, e.part, weights_grad,
-                       ld_weights_grad);
+    if (channel_size * p.slabs >= kCsbWideChannel)
+      hipLaunchKernelGGL(csb_merge_rows<true>, dim3(static_cast<unsigned>(num_channels)), dim3(kSbThreads), 0, st,
+                         num_channels, channel_size, height, p.slabs, e.part, weights_grad, ld_weights_grad);
+    else
+      hipLaunchKernelGGL(csb_merge_rows<false>, dim3(static_cast<unsigned>(ceil_div(num_channels, kSbWaves))),
+                         dim3(kSbThreads), 0, st, num_channels, channel_size, height, p.slabs, e.part, weights_grad,
+                         ld_weights_grad);
     return launch_status();
   }
   const bool vec = csb_vec_ok(channel_size, width, x, ldx) && csb_vec_ok(channel_size, width, dy, lddy) &&

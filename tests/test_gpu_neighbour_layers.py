@@ -228,6 +228,7 @@ CSB_CASES = [
     ((7, 5, 3), 23, 0), ((64, 56, 56), 8, 0), ((3, 224, 224), 4, 0), ((256, 4, 4), 32, 0), ((2048, 1, 1), 64, 0),
     ((5, 12), 10, 4), ((5, 13), 10, 0), ((1, 100000), 3, 0), ((2, 1), 1, 0), ((70000, 1), 2, 0), ((16, 128, 128), 16, 0),
     ((256, 28, 28), 24, 0), ((256, 7, 3), 200, 0),   # one 1024-thread workgroup per channel, vector and scalar
+    ((8, 55, 55), 40, 0), ((4, 111, 111), 12, 0), ((2048, 7, 7), 16, 0),   # odd maps: row tiling with channel lookup
 ]
 
 

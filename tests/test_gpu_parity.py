@@ -692,6 +692,7 @@ BN_CASES = [
     ((2048, 7, 7), 16, True, 0), ((4096,), 64, True, 0), ((64, 7, 7), 300, False, 0), ((12, 3, 3), 20, True, 0),
     ((8, 5), 7, True, 4), ((4, 1), 1, True, 0), ((1024, 1), 2048, True, 0),
     ((512, 2, 2), 40, True, 0), ((300, 8), 33, False, 0), ((64, 4), 700, True, 4),   # one or two vectors per channel
+    ((8, 55, 55), 300, True, 0), ((4, 111, 111), 20, False, 0), ((12, 27, 27), 400, True, 4),   # odd maps of many rows: a workgroup merges a channel
     # register-resident row tiles (w <= 256): 64-row and 256-row layouts, every columns-per-thread count
     ((4096,), 5, True, 0), ((4096,), 30, True, 0), ((1024, 1), 100, True, 0), ((2000, 2), 200, False, 0),
     ((333, 4), 256, True, 0), ((128, 7, 7), 3, True, 0), ((128, 7, 7), 10, True, 0), ((64, 7, 7), 24, True, 0),
@@ -760,6 +761,7 @@ def test_batch_norm(L, dims, w, bessel, pad):
     ((2048, 7, 7), 16, True, 0, True), ((4096,), 64, True, 0, True), ((64, 7, 7), 300, False, 0, True),
     ((12, 3, 3), 20, True, 0, True), ((1024, 1), 2048, True, 0, True), ((128, 7, 7), 10, True, 0, False),
     ((32, 7, 7), 64, True, 4, True), ((2000, 2), 200, False, 0, True), ((100, 12), 64, True, 0, True),
+    ((8, 55, 55), 300, True, 0, True), ((4, 111, 111), 20, False, 0, True),
     ((3, 56, 56), 512, True, 0, True), ((2, 2000000), 1, True, 0, True),   # clusters of more than 64 workgroups
     ((3, 112, 112), 512, True, 0, True), ((2, 2500000), 2, False, 0, True)])   # streaming clusters
 def test_batch_norm_f16(L, dims, w, bessel, pad, training):
