@@ -380,6 +380,26 @@ ebn_bwd_wide(EbnArgs a)
   }
 }
 
+// Walks the w columns of a row eight at a time: f(c, u) first loads column c + u for all u in
+// flight, g(c, u) then consumes them in order.  A thread of the kernels below owns one row and
+// would otherwise wait for one 4-byte load per iteration.
+template <typename Load, typename Use>
+__device__ __forceinline__ void ebn_walk_columns(int64_t w, Load&& load, Use&& use)
+{
+  constexpr int U = 8;
+  int64_t c = 0;
+  for (; c + U <= w; c += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) load(c + u, u);
+#pragma unroll
+    for (int u = 0; u < U; ++u) use(c + u, u);
+  }
+  for (; c < w; ++c) {
+    load(c, 0);
+    use(c, 0);
+  }
+}
+
 // One thread per row.  TRAINING: statistics from the mini-batch (written to stats, running
 // statistics updated); otherwise the running statistics are used as they are.
 template <bool TRAINING>
@@ -393,11 +413,14 @@ ebn_fwd_generic(EbnArgs a)
   if (TRAINING) {
     const float K = xr[0];
     float s = 0.f, q = 0.f;
-    for (int64_t c = 0; c < a.w; ++c) {
-      const float d = xr[c * a.ldx] - K;
-      s += d;
-      q = __builtin_fmaf(d, d, q);
-    }
+    float v[8];
+    ebn_walk_columns(
+      a.w, [&](int64_t c, int u) { v[u] = xr[c * a.ldx]; },
+      [&](int64_t, int u) {
+        const float d = v[u] - K;
+        s += d;
+        q = __builtin_fmaf(d, d, q);
+      });
     ebn_stats_from_sums(s, q, K, a.w, mean, var);
     a.stats[r] = mean;
     a.stats[r + a.ld_stats] = var;
@@ -412,7 +435,10 @@ ebn_fwd_generic(EbnArgs a)
   }
   const float inv = 1.0f / sqrtf(var + a.eps);
   float* yr = a.out + r;
-  for (int64_t c = 0; c < a.w; ++c) yr[c * a.ldo] = (xr[c * a.ldx] - mean) * inv;
+  float v[8];
+  ebn_walk_columns(
+    a.w, [&](int64_t c, int u) { v[u] = xr[c * a.ldx]; },
+    [&](int64_t c, int u) { yr[c * a.ldo] = (v[u] - mean) * inv; });
 }
 
 template <bool TRAINING>
@@ -425,18 +451,27 @@ ebn_bwd_generic(EbnArgs a)
   float* dr = a.out + r;
   if (!TRAINING) {  // entrywise_batch_normalization.cpp:352-392
     const float inv = 1.0f / sqrtf(a.rvar[r] + a.eps);
-    for (int64_t c = 0; c < a.w; ++c) dr[c * a.ldo] = gr[c * a.lddy] * inv;
+    float g[8];
+    ebn_walk_columns(
+      a.w, [&](int64_t c, int u) { g[u] = gr[c * a.lddy]; },
+      [&](int64_t c, int u) { dr[c * a.ldo] = g[u] * inv; });
     return;
   }
   const float* xr = a.x + r;
   const float mean = a.stats[r];
   const float inv = 1.0f / sqrtf(a.stats[r + a.ld_stats] + a.eps);
   float sa = 0.f, sb = 0.f;
-  for (int64_t c = 0; c < a.w; ++c) {
-    const float g = gr[c * a.lddy];
-    sa += g;
-    sb = __builtin_fmaf(g, xr[c * a.ldx] - mean, sb);
-  }
+  float g[8], v[8];
+  ebn_walk_columns(
+    a.w,
+    [&](int64_t c, int u) {
+      g[u] = gr[c * a.lddy];
+      v[u] = xr[c * a.ldx];
+    },
+    [&](int64_t, int u) {
+      sa += g[u];
+      sb = __builtin_fmaf(g[u], v[u] - mean, sb);
+    });
   const float wf = static_cast<float>(a.w);
   const float dmean = -sa * inv;
   const float dvar = -sb * inv * inv * inv * 0.5f;
@@ -444,8 +479,14 @@ ebn_bwd_generic(EbnArgs a)
   a.sgrad[r + a.ld_sgrad] = dvar;
   const float c0 = dmean / wf;
   const float c1 = dvar * 2.f / (wf - 1.f);
-  for (int64_t c = 0; c < a.w; ++c)
-    dr[c * a.ldo] = __builtin_fmaf(gr[c * a.lddy], inv, __builtin_fmaf(c1, xr[c * a.ldx] - mean, c0));
+  // in place (dx aliasing dy or x): a thread writes a column's entry after reading it
+  ebn_walk_columns(
+    a.w,
+    [&](int64_t c, int u) {
+      g[u] = gr[c * a.lddy];
+      v[u] = xr[c * a.ldx];
+    },
+    [&](int64_t c, int u) { dr[c * a.ldo] = __builtin_fmaf(g[u], inv, __builtin_fmaf(c1, v[u] - mean, c0)); });
 }
 
 __global__ void __launch_bounds__(256)
