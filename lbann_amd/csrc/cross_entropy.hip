@@ -25,7 +25,8 @@ namespace lbn {
 
 constexpr int kCeThreads = 256;
 constexpr int kCeWaves = kCeThreads / kWave;
-constexpr int kCeMaxParts = 64;
+constexpr int kCeMaxParts = 1024;      // workgroups per column (forward: their partial sums are merged by one wave)
+constexpr int kCeMaxPartsBwd = 16384;  // backward: nothing to merge
 
 // S: the storage type of every matrix of the layer (float, or __half with fp32 arithmetic).
 template <typename S>
@@ -88,6 +89,56 @@ ce_fwd_dense(CeArgs<S> a)
   ce_store_partial<T>(a, sum, red);
 }
 
+// Columns of at most 64 entries (ten classes, say) when there are many of them: a team of 16
+// lanes per column, four columns per wave, one entry per access (a wave still reads a
+// contiguous run when the columns are packed).  One workgroup per column would leave 246 of
+// its 256 threads idle: 21 classes x 1 M columns took 354 us forward that way.
+constexpr int kCeShortMax = 64;
+constexpr int kCeShortTeam = 16;
+constexpr int kCeShortColumns = kCeThreads / kCeShortTeam;  // per workgroup
+
+template <typename S>
+__global__ void __launch_bounds__(kCeThreads)
+ce_fwd_dense_short(CeArgs<S> a)
+{
+  const int team = threadIdx.x / kCeShortTeam, l = threadIdx.x % kCeShortTeam;
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * kCeShortColumns + team;
+  if (c >= a.w) return;  // whole teams leave: the DPP sum below never reads another team's lanes
+  const S* xc = a.x + c * a.ldx;
+  const S* tc = a.truth + c * a.ldt;
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < kCeShortMax / kCeShortTeam; ++k) {
+    const int64_t j = l + k * kCeShortTeam;
+    if (j < a.h) sum += ce_term(Vec16<S>::load1(tc + j), Vec16<S>::load1(xc + j));
+  }
+  sum = row16_sum(sum);
+  if (l == 0) Vec16<S>::store1(a.loss + c * a.ld_loss, sum);
+}
+
+template <typename S>
+__global__ void __launch_bounds__(kCeThreads)
+ce_bwd_dense_short(CeArgs<S> a)
+{
+  const int team = threadIdx.x / kCeShortTeam, l = threadIdx.x % kCeShortTeam;
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * kCeShortColumns + team;
+  if (c >= a.w) return;
+  const float g = Vec16<S>::load1(a.dy + c * a.lddy);
+  const S* xc = a.x + c * a.ldx;
+  const S* tc = a.truth + c * a.ldt;
+  S* dxc = a.dx + c * a.lddx;
+  S* dtc = a.dtruth + c * a.lddt;
+#pragma unroll
+  for (int k = 0; k < kCeShortMax / kCeShortTeam; ++k) {
+    const int64_t j = l + k * kCeShortTeam;
+    if (j < a.h) {
+      const float v = Vec16<S>::load1(xc + j), t = Vec16<S>::load1(tc + j);
+      if (a.dtruth) Vec16<S>::store1(dtc + j, -g * logf(v));
+      Vec16<S>::store1(dxc + j, t > 0.f ? -g * t / v : 0.f);
+    }
+  }
+}
+
 // One thread per spatial position: gather the entry of x its label points at.
 template <typename S>
 __global__ void __launch_bounds__(kCeThreads)
@@ -114,7 +165,9 @@ ce_merge_parts(int P, const float* __restrict__ part, S* __restrict__ loss, int6
 {
   const int64_t c = blockIdx.x;
   const int lane = threadIdx.x;
-  const float v = wave_sum(lane < P ? part[c * P + lane] : 0.f);
+  float acc = 0.f;
+  for (int p = lane; p < P; p += kWave) acc += part[c * P + p];  // lane-strided, then the wave: a fixed order
+  const float v = wave_sum(acc);
   if (lane == 0) Vec16<S>::store1(loss + c * ld_loss, v);
 }
 
@@ -197,14 +250,22 @@ ce_bwd_labels(CeArgs<S> a)
 }
 
 // Workgroups of `threads` threads per column: about 2048 * 256 threads in total, each
-// thread with at least four units.
-static int ce_parts(int64_t w, int64_t units_per_column, int threads = kCeThreads)
+// thread with at least four units.  (A single column of a segmentation map, 19 classes x
+// 1024 x 2048 positions, had been held to 64 workgroups: 426 us backward.)
+static int ce_parts(int64_t w, int64_t units_per_column, int threads = kCeThreads, int max_parts = kCeMaxParts)
 {
   int64_t p = ceil_div(2048 * kCeThreads, w * threads);
   const int64_t most = ceil_div(units_per_column, 4 * threads);
   if (p > most) p = most;
-  if (p > kCeMaxParts) p = kCeMaxParts;
+  if (p > max_parts) p = max_parts;
   return static_cast<int>(p < 1 ? 1 : p);
+}
+
+// The most partial sums per column a forward call can ask for (what the workspace holds).
+static int64_t ce_parts_bound(int64_t w)
+{
+  const int64_t p = ceil_div(2048, w);
+  return p > kCeMaxParts ? kCeMaxParts : p;
 }
 
 static int ce_check(int64_t h, int64_t w, int use_labels, int64_t spatial, int64_t ldx, int64_t ldt)
@@ -239,6 +300,11 @@ static int ce_fwd_impl(lbn_stream_t stream, int64_t height, int64_t width, int u
   a.h = height, a.w = width, a.spatial = use_labels ? spatial_size : 1;
   a.x = prediction, a.truth = ground_truth, a.ldx = ld_prediction, a.ldt = ld_ground_truth;
   a.loss = loss, a.ld_loss = ld_loss, a.part = static_cast<float*>(workspace);
+  if (!use_labels && height <= kCeShortMax && width >= 4096) {
+    hipLaunchKernelGGL((ce_fwd_dense_short<S>), dim3(static_cast<unsigned>(ceil_div(width, kCeShortColumns))),
+                       dim3(kCeThreads), 0, st, a);
+    return launch_status();
+  }
   const bool vec = !use_labels && ce_vec_ok(height, width, prediction, ld_prediction, VE) &&
                    ce_vec_ok(height, width, ground_truth, ld_ground_truth, VE);
   const int64_t units = use_labels ? (spatial_size < height ? spatial_size : height) : (vec ? height / VE : height);
@@ -279,6 +345,11 @@ static int ce_bwd_impl(lbn_stream_t stream, int64_t height, int64_t width, int u
   a.x = prediction, a.truth = ground_truth, a.ldx = ld_prediction, a.ldt = ld_ground_truth;
   a.dy = dloss, a.lddy = ld_dloss, a.dx = dprediction, a.lddx = ld_dprediction;
   a.dtruth = dground_truth, a.lddt = ld_dground_truth;
+  if (!use_labels && height <= kCeShortMax && width >= 4096) {
+    hipLaunchKernelGGL((ce_bwd_dense_short<S>), dim3(static_cast<unsigned>(ceil_div(width, kCeShortColumns))),
+                       dim3(kCeThreads), 0, st, a);
+    return launch_status();
+  }
   bool vec = ce_vec_ok(height, width, prediction, ld_prediction, VE) &&
              ce_vec_ok(height, width, dprediction, ld_dprediction, VE);
   if (use_labels)
@@ -286,7 +357,7 @@ static int ce_bwd_impl(lbn_stream_t stream, int64_t height, int64_t width, int u
   else
     vec = vec && ce_vec_ok(height, width, ground_truth, ld_ground_truth, VE) &&
           ce_vec_ok(height, width, dground_truth, ld_dground_truth, VE);
-  const int P = ce_parts(width, vec ? height / VE : height);
+  const int P = ce_parts(width, vec ? height / VE : height, kCeThreads, kCeMaxPartsBwd);
   const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
   if (use_labels) {
     if (vec) hipLaunchKernelGGL((ce_bwd_labels<true, S>), grid, dim3(kCeThreads), 0, st, a);
@@ -308,7 +379,7 @@ extern "C" {
 size_t lbn_cross_entropy_fwd_workspace_bytes(int64_t height, int64_t width)
 {
   if (height <= 0 || width <= 0) return 0;
-  return static_cast<size_t>(width) * kCeMaxParts * sizeof(float);
+  return static_cast<size_t>(width) * ce_parts_bound(width) * sizeof(float);
 }
 
 int lbn_cross_entropy_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, int use_labels,

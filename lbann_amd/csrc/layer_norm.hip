@@ -259,6 +259,30 @@ ln_fwd_generic(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t 
   }
 }
 
+// Rows of a single entry (instance norm on 1 x 1 maps): the mean is the entry, the variance 1
+// (layer_norm.cpp:70-77), one thread per row instead of a workgroup.
+template <typename T>
+__global__ void __launch_bounds__(256)
+ln_fwd_single(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
+              float eps, float* __restrict__ stats, int64_t ld_stats, const float* __restrict__ gamma,
+              const float* __restrict__ beta)
+{
+  using IO = Vec16<T>;
+  const float inv_stdev = 1.0f / sqrtf(1.f + eps);
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; row < rows;
+       row += static_cast<int64_t>(gridDim.x) * 256) {
+    int64_t col, g;
+    map.split(row, col, g);
+    const float v = IO::load1(x + g * map.stride + col * ldx);
+    stats[g + col * ld_stats] = v;
+    stats[map.groups + g + col * ld_stats] = 1.f;
+    float r = (v - v) * inv_stdev;  // 0, or NaN for an entry that is not finite, as in the general kernel
+    if (gamma) r *= gamma[0];
+    if (beta) r += beta[0];
+    IO::store1(y + g * map.stride + col * ldy, r);
+  }
+}
+
 // ================================================================== backward
 // Weight gradients of small problems without any exchange between workgroups: dscale and
 // dbias of a feature depend on x, dy and the FORWARD statistics only (xh = (x - mean) /
@@ -1040,6 +1064,12 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                    rows_aligned16(y, stride, ldy, G, w, sizeof(T)) &&
                    (!gamma || aligned16(gamma)) && (!beta || aligned16(beta));
   const float inv_n = 1.0f / static_cast<float>(n);
+  if (n == 1) {
+    const int64_t want = ceil_div(rows, 256);
+    hipLaunchKernelGGL((ln_fwd_single<T>), dim3(static_cast<unsigned>(want > 8192 ? 8192 : want)), dim3(256), 0, st, x,
+                       y, ldx, ldy, map, rows, eps, stats, lds, gamma, beta);
+    return launch_status();
+  }
   if (vec) {
     if (int r = ln_fwd_rows_launch<T>(st, x, y, ldx, ldy, map, rows, n / VE, inv_n, eps, stats, lds, gamma,
                                       beta, sumsq))

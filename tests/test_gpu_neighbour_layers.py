@@ -44,6 +44,8 @@ CE_DENSE = [
     (10, 128, 0), (1000, 64, 0), (192, 23, 0), (4096, 33, 0), (7, 5, 0), (1001, 3, 0), (130, 4, 2),
     (512, 9, 64), (300000, 3, 0), (1 << 20, 2, 0), (65536, 40, 0), (1, 6, 0),
     (16384, 256, 0), (4101, 257, 0),   # one 1024-thread workgroup per column, vector and scalar
+    (10, 5000, 0), (21, 70000, 0), (64, 4099, 3), (1, 6000, 0), (3, 100000, 0), (17, 4096, 0),   # 16-lane teams
+    (2000000, 1, 0), (600000, 2, 0),   # a column or two: many workgroups per column
 ]
 
 
@@ -71,6 +73,7 @@ CE_LABELS = [
     # (classes, spatial dims, w, ld_pad)
     (3, (8, 8), 23, 0), (3, (4, 4, 4), 11, 0), (10, (1,), 64, 0), (5, (7, 3), 9, 0), (4, (6,), 5, 3),
     (21, (64, 64), 6, 0), (2, (300, 300), 3, 0), (1000, (1,), 128, 0), (19, (128, 130), 2, 0),
+    (19, (512, 1024), 1, 0),   # one column of a large map: many workgroups per column
 ]
 
 
@@ -100,6 +103,7 @@ CE_F16 = [
     # (h, w, ld_pad): whole 16-byte vectors of 8, ragged heights, a padded leading dimension, 1024-thread columns
     (16, 128, 0), (1000, 64, 0), (192, 23, 0), (4096, 33, 0), (7, 5, 0), (1001, 3, 0), (136, 4, 8), (130, 4, 2),
     (16384, 256, 0), (4101, 257, 0), (65536, 40, 0), (300000, 3, 0), (1, 6, 0),
+    (10, 5000, 0), (33, 4500, 8), (64, 4100, 0),   # 16-lane teams
 ]
 
 
