@@ -1084,7 +1084,7 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
       if (ln_stream_launch<T, false>(st, a, rows, n, ws, ws_bytes)) return launch_status();
     }
     hipLaunchKernelGGL((ln_fwd_long<T>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st, x, y,
-                       ldx, ldy, map, n / VE, inv_n, eps, stats, lds, gamma, beta, sumsq);
+                       ldx, ldy, map, n / VE, 0, inv_n, eps, stats, lds, gamma, beta, sumsq);
     return launch_status();
   }
   if constexpr (std::is_same<T, __half>::value) {
@@ -1103,6 +1103,14 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                                             ldx, ldy, map, rows, n, inv_n, eps, stats, lds, gamma, beta, sumsq))
         return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
     }
+  }
+  if constexpr (std::is_same<T, float>::value) {
+    // fp32 rows off the 16-byte grid beyond the register kernels: two passes of 16-byte accesses
+    // at 4-byte alignment, the last n % 4 entries apart
+    hipLaunchKernelGGL((ln_fwd_long<f32u>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
+                       reinterpret_cast<const f32u*>(x), reinterpret_cast<f32u*>(y), ldx, ldy, map, n / 4,
+                       static_cast<int>(n % 4), inv_n, eps, stats, lds, gamma, beta, sumsq);
+    return launch_status();
   }
   hipLaunchKernelGGL((ln_fwd_generic<T>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, st, x, y,
                      ldx, ldy, map, n, eps, stats, lds, gamma, beta, sumsq);
@@ -1246,7 +1254,7 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
       if (ln_stream_launch<T, true>(st, a, rows, n, ws, ws_bytes)) return launch_status();
     }
     hipLaunchKernelGGL((ln_bwd_long<T>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st, x, dy,
-                       dx, ldx, lddy, lddx, map, n / VE, 1.0f / static_cast<float>(n), eps, stats, lds, sgrad,
+                       dx, ldx, lddy, lddx, map, n / VE, 0, 1.0f / static_cast<float>(n), eps, stats, lds, sgrad,
                        ldsg, gamma);
   }
   else {
@@ -1269,8 +1277,14 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
           return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
       }
     }
-    hipLaunchKernelGGL((ln_bwd_generic<T>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, st, x, dy,
-                       dx, ldx, lddy, lddx, map, n, eps, stats, lds, sgrad, ldsg, gamma);
+    if constexpr (std::is_same<T, float>::value)
+      hipLaunchKernelGGL((ln_bwd_long<f32u>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
+                         reinterpret_cast<const f32u*>(x), reinterpret_cast<const f32u*>(dy),
+                         reinterpret_cast<f32u*>(dx), ldx, lddy, lddx, map, n / 4, static_cast<int>(n % 4),
+                         1.0f / static_cast<float>(n), eps, stats, lds, sgrad, ldsg, gamma);
+    else
+      hipLaunchKernelGGL((ln_bwd_generic<T>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, st, x, dy,
+                         dx, ldx, lddy, lddx, map, n, eps, stats, lds, sgrad, ldsg, gamma);
   }
   if (wgrad) {
     // weight gradients of the two paths above: row slabs -> partial rows -> fixed-order sum

@@ -26,9 +26,11 @@ constexpr int kLongUnroll = 4;
 template <typename T>
 __global__ void __launch_bounds__(kLongThreads)
 ln_fwd_long(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy, RowMap map,
-            int64_t nvec, float inv_n, float eps, float* __restrict__ stats, int64_t ld_stats,
+            int64_t nvec, int tail, float inv_n, float eps, float* __restrict__ stats, int64_t ld_stats,
             const float* __restrict__ gamma, const float* __restrict__ beta, int sumsq)
 {
+  // tail: entries after the nvec whole vectors (rows of f32u data whose length is not a multiple
+  // of 4), one per thread of the first `tail` threads; 0 for every other storage type.
   using IO = Vec16<T>;
   constexpr int VE = IO::N;
   __shared__ float red[2 * kLongWaves];
@@ -42,6 +44,15 @@ ln_fwd_long(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
   const float K = sumsq ? 0.f : IO::load1(xr);
 
   float s = 0.f, q = 0.f;
+  const bool has_tail = static_cast<int>(threadIdx.x) < tail;
+  const int64_t tail_at = VE * nvec + threadIdx.x;
+  float tv = 0.f;
+  if (has_tail) {
+    tv = IO::load1(xr + tail_at);
+    const float d = tv - K;
+    s = d;
+    q = d * d;
+  }
   int64_t j = threadIdx.x;
   for (; j + (kLongUnroll - 1) * kLongThreads < nvec; j += kLongUnroll * kLongThreads) {
     float v[kLongUnroll][VE];
@@ -70,7 +81,7 @@ ln_fwd_long(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
   float dm = s * inv_n;
   float var = fmaxf(__builtin_fmaf(-dm, dm, q * inv_n), 0.f);
   if (sumsq) {  // the reference's own expression: true divisions, no fused multiply-add
-    const float nf = static_cast<float>(nvec * VE);
+    const float nf = static_cast<float>(nvec * VE + tail);
     dm = s / nf;
     var = fmaxf(__fsub_rn(q / nf, __fmul_rn(dm, dm)), 0.f);
   }
@@ -86,8 +97,8 @@ ln_fwd_long(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
 #pragma unroll
     for (int k4 = 0; k4 < VE; k4 += 4) {
       float w[4] = {1.f, 1.f, 1.f, 1.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
-      if (gamma) Vec16<float>::load(gamma + VE * jj + k4, w);
-      if (beta) Vec16<float>::load(beta + VE * jj + k4, b);
+      if (gamma) load_weights4<T>(gamma + VE * jj + k4, w);
+      if (beta) load_weights4<T>(beta + VE * jj + k4, b);
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         ga[k4 + k] = w[k];
@@ -98,6 +109,9 @@ ln_fwd_long(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
     for (int k = 0; k < VE; ++k) v[k] = __builtin_fmaf((v[k] - mean) * inv_stdev, ga[k], be[k]);
     IO::store(yr + VE * jj, v);
   };
+  if (has_tail)
+    IO::store1(yr + tail_at, __builtin_fmaf((tv - mean) * inv_stdev, gamma ? gamma[tail_at] : 1.f,
+                                            beta ? beta[tail_at] : 0.f));
   j = threadIdx.x;
   for (; j + (kLongUnroll - 1) * kLongThreads < nvec; j += kLongUnroll * kLongThreads) {
     float v[kLongUnroll][VE];
@@ -116,7 +130,7 @@ ln_fwd_long(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
 template <typename T>
 __global__ void __launch_bounds__(kLongThreads)
 ln_bwd_long(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ dx, int64_t ldx,
-            int64_t lddy, int64_t lddx, RowMap map, int64_t nvec, float inv_n, float eps,
+            int64_t lddy, int64_t lddx, RowMap map, int64_t nvec, int tail, float inv_n, float eps,
             const float* __restrict__ stats, int64_t ld_stats, float* __restrict__ sgrad,
             int64_t ld_sgrad, const float* __restrict__ gamma)
 {
@@ -140,7 +154,7 @@ ln_bwd_long(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
 #pragma unroll
     for (int k4 = 0; k4 < VE; k4 += 4) {
       float w[4] = {1.f, 1.f, 1.f, 1.f};
-      if (gamma) Vec16<float>::load(gamma + VE * jj + k4, w);
+      if (gamma) load_weights4<T>(gamma + VE * jj + k4, w);
 #pragma unroll
       for (int k = 0; k < 4; ++k) d[k4 + k] *= w[k];
     }
@@ -149,6 +163,16 @@ ln_bwd_long(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   };
 
   float a = 0.f, b = 0.f;
+  // (tail: as in ln_fwd_long) the thread's entry as xh and dy * scale
+  const bool has_tail = static_cast<int>(threadIdx.x) < tail;
+  const int64_t tail_at = VE * nvec + threadIdx.x;
+  float tx = 0.f, td = 0.f;
+  if (has_tail) {
+    tx = (IO::load1(xr + tail_at) - mean) * inv_stdev;
+    td = IO::load1(gr + tail_at) * (gamma ? gamma[tail_at] : 1.f);
+    a = td;
+    b = td * tx;
+  }
   int64_t j = threadIdx.x;
   for (; j + (U - 1) * kLongThreads < nvec; j += U * kLongThreads) {
     float v[U][VE], d[U][VE];
@@ -188,6 +212,7 @@ ln_bwd_long(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   const float c0 = dmean * inv_n;
   const float c1 = -b * inv_stdev * inv_n;  // dvar * 2 / n per unit of xh
 
+  if (has_tail) IO::store1(dr + tail_at, __builtin_fmaf(td, inv_stdev, __builtin_fmaf(c1, tx, c0)));
   j = threadIdx.x;
   for (; j + (U - 1) * kLongThreads < nvec; j += U * kLongThreads) {
     float v[U][VE], d[U][VE];

@@ -357,6 +357,9 @@ LN_CASES = [
     # rows off the 16-byte grid: the register kernels with one float per access
     ((1001,), 0, 40, True, 0), ((197, 769), -1, 3, True, 0), ((4095,), 0, 9, True, 0), ((4097,), 0, 9, True, 0),
     ((8191,), 0, 5, False, 0), ((49,), 0, 3000, True, 0), ((1000,), 0, 17, True, 3), ((7,), 0, 100000, True, 0),
+    # longer rows off the 16-byte grid: two passes of 16-byte accesses at 4-byte alignment, every n % 4
+    ((10001,), 0, 7, True, 0), ((50001,), 0, 5, False, 0), ((50002,), 0, 3, True, 1), ((30003,), 0, 4, True, 0),
+    ((3, 89401), -1, 3, False, 0), ((20000,), 0, 6, True, 1), ((1,), 0, 70000, True, 0),
     # many short rows: teams of 16 lanes, four rows per wave
     ((1024, 64), -1, 8, True, 0), ((512, 128), -1, 16, True, 0), ((64, 256), -1, 70, True, 0), ((4099, 16), -1, 3, False, 0),
     ((49,), 0, 5000, True, 0), ((600, 20), -1, 9, True, 0), ((4096, 8), -1, 1, True, 0), ((2048, 12), -1, 2, True, 4),
@@ -450,7 +453,8 @@ def test_layer_norm_f16(L, dims, start_dim, w, pad):
                                         ((3, 100000), 2, 0), ((7, 1), 5, 0), ((16, 31), 40, 4),
                                         ((256, 16, 16), 64, 0), ((3, 224, 224), 8, 0), ((2, 64, 64, 64), 2, 0),
                                         ((256, 7, 7), 32, 0), ((64, 3, 3), 9, 0), ((5, 4097), 6, 0),
-                                        ((256, 8, 8), 32, 0), ((512, 4, 4), 16, 0), ((64, 16, 16), 70, 0)])
+                                        ((256, 8, 8), 32, 0), ((512, 4, 4), 16, 0), ((64, 16, 16), 70, 0),
+                                        ((3, 299, 299), 5, 0), ((2, 111, 111), 9, 1), ((1024, 1), 300, 0)])
 def test_instance_norm(L, dims, w, pad):
     rng = np.random.default_rng(int(np.prod(dims)) + 7 * w)
     h = int(np.prod(dims))
