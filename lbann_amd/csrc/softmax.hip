@@ -65,9 +65,17 @@ constexpr int64_t kMaxScalarLongRow = 32768;  // with 16 or 32 floats per thread
 // Rows of at most 64 access units, when there are many of them, go to teams of 16 lanes
 // (four rows per wave) instead of leaving most of a wave idle: attention rows of 64
 // entries (16 x 64 x 64 x 256) went from 124 to 54 us per step, 10-class rows from 78 to 21.
-static RowConfig pick_sm_row_config(int64_t units, int64_t rows)
+// scalar: the units are single entries (rows off the 16-byte grid).  Eight of those per lane
+// cost eight registers, so rows of 257 to 512 entries stay with one wave (no barrier, four
+// rows per workgroup) instead of four waves with two entries each: 257 x 65536 forward 69 us
+// with four waves.
+static RowConfig pick_sm_row_config(int64_t units, int64_t rows, bool scalar = false)
 {
+  // (the same up to 1024 entries with sixteen per lane: 513 x 32768 forward 46 us with four waves)
   if (units <= 64 && rows >= 4096) return {16, units <= 16 ? 1 : units <= 32 ? 2 : 4};
+  if (scalar && units > 256 && units <= 512 && rows >= 2048) return {64, 8};
+  if (scalar && units > 512 && units <= 1024 && rows >= 2048) return {64, 16};
+  if (scalar && units > 1024 && units <= 2048 && rows >= 1024) return {256, 8};  // not sixteen waves of two entries
   return pick_row_config(units, rows);
 }
 
@@ -361,7 +369,7 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
   }
   else if (n <= kMaxScalarRow) {
     // rows that are only 4-byte aligned and short enough for registers: one float per access
-    const RowConfig c = pick_sm_row_config(n, rows);
+    const RowConfig c = pick_sm_row_config(n, rows, true);
     if (c.tpr) {
       const unsigned nvec = static_cast<unsigned>(n);
 #define X(TPR, V)                                                                            \
@@ -372,7 +380,7 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
                        x, y, ldx, ldy, map, rows, nvec);                                     \
     return launch_status();                                                                  \
   }
-      LBN_ROW_CASES(X)
+      LBN_ROW_CASES(X) X(64, 16)
 #undef X
     }
   }
@@ -537,7 +545,7 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     // (as in the forward pass: the packed two-pass kernel below)
   }
   else if (n <= kMaxScalarRow) {
-    const RowConfig c = pick_sm_row_config(n, rows);
+    const RowConfig c = pick_sm_row_config(n, rows, true);
     if (c.tpr) {
       const unsigned nvec = static_cast<unsigned>(n);
 #define X(TPR, V)                                                                            \
@@ -548,7 +556,7 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
                        y, dy, dx, ldy, lddy, lddx, map, rows, nvec);                         \
     return launch_status();                                                                  \
   }
-      LBN_ROW_CASES(X)
+      LBN_ROW_CASES(X) X(64, 16)
 #undef X
     }
   }
