@@ -907,6 +907,14 @@ static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, i
   // (layer norm rows of 64 entries x 65536: 60 us per step against 150 us with one wave per row;
   // at 64 units per row the two shapes measure the same and the wave-wide team is kept)
   if (units <= 32 && rows >= 4096) c = {16, units <= 16 ? 1 : 2};
+  // single floats cost one register each: rows just past 256, 512 or 1024 entries stay with one
+  // wave (or four) holding 8 or 16 of them instead of four (or sixteen) waves holding two
+  // (257 x 65536: 59 us forward, 1025 x 16384: 81 us that way)
+  if (VE == 1 && rows >= 2048) {
+    if (units > 256 && units <= 512) c = {64, 8};
+    else if (units > 512 && units <= 1024) c = {64, 16};
+    else if (units > 1024 && units <= 2048) c = {256, 8};
+  }
   if (!c.tpr) return 0;
   const int nvec = static_cast<int>(units);
 #define X(TPR, V)                                                                              \
@@ -926,6 +934,7 @@ static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, i
   X(64, 1) X(64, 2) X(64, 4) X(256, 1) X(256, 2) X(256, 4) X(1024, 1) X(1024, 2) X(1024, 4)
   X(64, 8) X(256, 8)
   if constexpr (VE <= 4) { X(1024, 8) }
+  if constexpr (VE == 1) { X(64, 16) }
 #undef X
   return 0;
 }
