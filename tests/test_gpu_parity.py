@@ -158,6 +158,25 @@ def test_softmax_f16_special_values_on_walked_rows(L):
     assert np.all(np.isneginf(ly[:, cols["minus_inf"]][np.arange(h) != 5])) and abs(float(ly[5, cols["minus_inf"]])) == 0.0
 
 
+@pytest.mark.parametrize("h", [70000, 50257])
+def test_softmax_f16_special_values_on_long_rows(L, h):
+    """Rows beyond the register kernels (two packed passes; 50257: cut at 16-byte boundaries)."""
+    x = np.zeros((h, 5), dtype=np.float16)
+    x[:, 0] = 3.0
+    x[h - 2, 1] = 60000.0
+    x[:, 2] = -np.inf
+    x[5, 2] = 1.0
+    x[9, 3] = np.nan
+    x[:, 4] = -np.inf
+    y = L.softmax_layer().forward(L.DeviceMatrix.from_numpy(x, dtype=torch.float16)).to_numpy()
+    ref = orc.softmax_fwd(f32(x))
+    assert np.allclose(f32(y[:, 0]), 1.0 / h, rtol=2e-3)
+    assert y[h - 2, 1] == 1.0 and y[:, 1].sum() == 1.0
+    assert y[5, 2] == 1.0 and y[:, 2].sum() == 1.0
+    assert (ref[:, 3] == 0).all() and (y[:, 3] == 0).all()
+    assert (ref[:, 4] == 0).all() and (y[:, 4] == 0).all()      # a column of -inf: 0 / 0, flushed
+
+
 @pytest.mark.parametrize("kind", ["softmax", "log_softmax", "channelwise"])
 @pytest.mark.parametrize("h,w,in_place", [(262144, 17, False), (65536, 40, False), (262144, 16, True), (131072, 31, True)])
 def test_few_long_rows_all_in_flight(L, kind, h, w, in_place):
