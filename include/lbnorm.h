@@ -201,19 +201,25 @@ int lbn_instance_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t cha
  * neither x nor stats (both may be NULL).  Statistics are over the local width: with
  * several ranks the reference sums them across the mini-batch (:97-100, :301-303):
  * use the split entry points below.  Where the reference's E[x^2] - mean^2 can come out
- * negative, the variance here is clamped at zero. */
+ * negative, the variance here is clamped at zero.
+ * The workspace is optional (NULL: none): with it, a mini-batch of more than 256 samples
+ * whose samples have few entries (4096 x 2048, say) is cut into column slabs that are
+ * summed side by side instead of by one workgroup per 64 rows. */
+size_t lbn_entrywise_batch_norm_workspace_bytes(int64_t height, int64_t width);
 int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
                                      float decay, float epsilon, int training,
                                      const float* x, int64_t ldx, float* y, int64_t ldy,
                                      float* stats, int64_t ld_stats,
-                                     float* running_mean, float* running_var);
+                                     float* running_mean, float* running_var,
+                                     void* workspace, size_t workspace_bytes);
 int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
                                      float epsilon, int training,
                                      const float* x, int64_t ldx, const float* dy, int64_t lddy,
                                      float* dx, int64_t lddx,
                                      const float* stats, int64_t ld_stats,
                                      float* stats_grad, int64_t ld_stats_grad,
-                                     const float* running_var);
+                                     const float* running_var,
+                                     void* workspace, size_t workspace_bytes);
 
 /* The same computation cut where the reference places its all-reduces, for callers whose
  * mini-batch is spread over several ranks (entrywise_batch_normalization.cpp:97-100 and

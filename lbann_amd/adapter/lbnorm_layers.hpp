@@ -761,10 +761,12 @@ public:
                    where);
       return;
     }
+    const size_t bytes = lbn_entrywise_batch_norm_workspace_bytes(x.Height(), x.Width());
     check_status(lbn_entrywise_batch_norm_fwd_f32(io.stream, x.Height(), x.Width(), m_decay, m_epsilon,
                                                   is_training ? 1 : 0, x.LockedBuffer(), x.LDim(), y.Buffer(),
                                                   y.LDim(), m_batch_statistics.Buffer(),
-                                                  m_batch_statistics.LDim(), m_w[0], m_w[1]),
+                                                  m_batch_statistics.LDim(), m_w[0], m_w[1],
+                                                  bytes ? m_ws.reserve(bytes, io.stream) : nullptr, bytes),
                  "entrywise_batch_normalization_layer::fp_compute");
   }
   void bp_compute()
@@ -790,15 +792,21 @@ public:
                    where);
       return;
     }
+    const size_t bytes = lbn_entrywise_batch_norm_workspace_bytes(x.Height(), x.Width());
     check_status(lbn_entrywise_batch_norm_bwd_f32(io.stream, x.Height(), x.Width(), m_epsilon,
                                                   is_training ? 1 : 0, x.LockedBuffer(), x.LDim(),
                                                   dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
                                                   m_batch_statistics.LockedBuffer(), m_batch_statistics.LDim(),
                                                   m_batch_statistics_gradient.Buffer(),
-                                                  m_batch_statistics_gradient.LDim(), m_w[1]),
+                                                  m_batch_statistics_gradient.LDim(), m_w[1],
+                                                  bytes ? m_ws.reserve(bytes, io.stream) : nullptr, bytes),
                  "entrywise_batch_normalization_layer::bp_compute");
   }
+  /// The layer's scratch buffer (partial sums of wide mini-batches; reserve it up front to
+  /// keep the hooks free of allocation).
+  workspace& scratch() { return m_ws; }
 private:
+  workspace m_ws;
   float m_decay, m_epsilon;
   int64_t m_size = 0;
   float* m_w[2] = {nullptr, nullptr};

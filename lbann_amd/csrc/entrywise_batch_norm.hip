@@ -24,6 +24,7 @@
 #include <cfloat>
 
 #include "device_utils.hpp"
+#include "entrywise_batch_norm_slabs.hpp"
 #include "host_utils.hpp"
 
 namespace lbn {
@@ -526,10 +527,17 @@ using namespace lbn;
 
 extern "C" {
 
+size_t lbn_entrywise_batch_norm_workspace_bytes(int64_t height, int64_t width)
+{
+  if (height <= 0 || width <= 0) return 0;
+  return ebn_slab_workspace_bytes(height, width);
+}
+
 int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, float decay,
                                      float epsilon, int training, const float* x, int64_t ldx,
                                      float* y, int64_t ldy, float* stats, int64_t ld_stats,
-                                     float* running_mean, float* running_var)
+                                     float* running_mean, float* running_var, void* workspace,
+                                     size_t workspace_bytes)
 {
   const int64_t lds[2] = {ldx, ldy};
   if (int e = ebn_check(height, width, lds, 2)) return e;
@@ -553,6 +561,10 @@ int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_
 #undef X
   }
   if (training && vec) {  // wider than the register tiles
+    // few rows: column slabs side by side when the caller gave scratch
+    if (ebn_slab_fwd(st, height, width, epsilon, decay, x, ldx, y, ldy, stats, ld_stats, running_mean, running_var,
+                     workspace, workspace_bytes))
+      return launch_status();
     hipLaunchKernelGGL((ebn_fwd_wide<4>), dim3(static_cast<unsigned>(ceil_div(height, EbnPos<4>::kRows))),
                        dim3(kEbnThreads), 0, st, a);
     return launch_status();
@@ -567,7 +579,7 @@ int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_
                                      int training, const float* x, int64_t ldx, const float* dy,
                                      int64_t lddy, float* dx, int64_t lddx, const float* stats,
                                      int64_t ld_stats, float* stats_grad, int64_t ld_stats_grad,
-                                     const float* running_var)
+                                     const float* running_var, void* workspace, size_t workspace_bytes)
 {
   const int64_t lds[3] = {ldx, lddy, lddx};
   if (int e = ebn_check(height, width, lds, 3)) return e;
@@ -603,6 +615,9 @@ int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_
 #undef X
   }
   if (vec) {  // wider than the register tiles
+    if (ebn_slab_bwd(st, height, width, epsilon, x, ldx, dy, lddy, dx, lddx, stats, ld_stats, stats_grad,
+                     ld_stats_grad, workspace, workspace_bytes))
+      return launch_status();
     hipLaunchKernelGGL((ebn_bwd_wide<4>), dim3(static_cast<unsigned>(ceil_div(height, EbnPos<4>::kRows))),
                        dim3(kEbnThreads), 0, st, a);
     return launch_status();

@@ -11,6 +11,7 @@
 // take every fourth column, so a wave instruction reads 1 KiB (256 B) of one column.  The
 // summing kernels merge the four waves' partial sums through LDS in a fixed order.
 #include "device_utils.hpp"
+#include "entrywise_batch_norm_slabs.hpp"
 #include "host_utils.hpp"
 
 namespace lbn {
@@ -44,7 +45,23 @@ struct SplitArgs {
   const float* var;
   float* sum0;      // column 0 of the (h x 2) result of a summing kernel
   float* sum1;      // column 1
+  // Column slabs (gridDim.y of the summing kernels): slab s sums columns [s * slab_cols,
+  // (s + 1) * slab_cols) into sum0 / sum1 + s * slab_stride.  One slab: all columns, no offset.
+  int64_t slab_cols;
+  int64_t slab_stride;
 };
+
+// Column range and output offset of a summing workgroup.
+struct SplitSlab {
+  int64_t c0, c1, out;
+};
+__device__ __forceinline__ SplitSlab split_slab(const SplitArgs& a, bool ok)
+{
+  if (gridDim.y == 1) return {0, ok ? a.w : 0, 0};
+  const int64_t c0 = static_cast<int64_t>(blockIdx.y) * a.slab_cols;
+  const int64_t c1 = c0 + a.slab_cols < a.w ? c0 + a.slab_cols : a.w;
+  return {c0, ok ? c1 : c0, static_cast<int64_t>(blockIdx.y) * a.slab_stride};
+}
 
 __device__ __forceinline__ float square_rounded(float v)
 {
@@ -93,11 +110,12 @@ ebn_split_fwd_sums(SplitArgs a)
   const int64_t r0 = (static_cast<int64_t>(blockIdx.x) * kWave + lane) * VE;
   const bool ok = r0 < a.h;
   const int64_t rr = ok ? r0 : 0;
-  const int64_t w = ok ? a.w : 0;
+  const SplitSlab sl = split_slab(a, ok);
+  const int64_t w = sl.c1;
   float s[VE], q[VE];
 #pragma unroll
   for (int r = 0; r < VE; ++r) s[r] = q[r] = 0.f;
-  int64_t c = wave;
+  int64_t c = sl.c0 + wave;
   for (; c + kSplitWaves < w; c += 2 * kSplitWaves) {
     float v[2][VE];
     RowItem<VE>::load(a.x + rr + c * a.ldx, v[0]);
@@ -120,8 +138,8 @@ ebn_split_fwd_sums(SplitArgs a)
     }
   }
   if (split_merge<VE>(s, q, lds) && ok) {
-    RowItem<VE>::store(a.sum0 + r0, s);
-    RowItem<VE>::store(a.sum1 + r0, q);
+    RowItem<VE>::store(a.sum0 + sl.out + r0, s);
+    RowItem<VE>::store(a.sum1 + sl.out + r0, q);
   }
 }
 
@@ -130,21 +148,20 @@ ebn_split_fwd_sums(SplitArgs a)
 // the mean already, the variance is 1 and the running statistics stay.  The variance is
 // clamped at zero where E[x^2] - mean^2 comes out negative.  Every operation is rounded on
 // its own, in the reference's order.
-__global__ void __launch_bounds__(256)
-ebn_split_fwd_stats(int64_t h, int64_t count, float decay, float* mean, float* var, float* rmean,
-                    float* rvar)
+// Row r: (sum, sum of squares) -> mean[r], var[r], running statistics updated.
+__device__ __forceinline__ void ebn_stats_of_row(int64_t r, float sum, float sumsq, int64_t count, float decay,
+                                                 float* mean, float* var, float* rmean, float* rvar)
 {
-  const int64_t r = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (r >= h) return;
   if (count <= 1) {
+    mean[r] = sum;
     var[r] = 1.f;
     return;
   }
   {
 #pragma clang fp contract(off)
     const float n = static_cast<float>(count);
-    const float m = mean[r] / n;
-    const float sqmean = var[r] / n;
+    const float m = sum / n;
+    const float sqmean = sumsq / n;
     const float mm = m * m;
     const float v = fmaxf(sqmean - mm, 0.f) * n / (n - 1.f);
     const float keep_m = decay * rmean[r];
@@ -155,6 +172,67 @@ ebn_split_fwd_stats(int64_t h, int64_t count, float decay, float* mean, float* v
     var[r] = v;
     rmean[r] = keep_m + new_m;
     rvar[r] = keep_v + new_v;
+  }
+}
+
+__global__ void __launch_bounds__(256)
+ebn_split_fwd_stats(int64_t h, int64_t count, float decay, float* mean, float* var, float* rmean,
+                    float* rvar)
+{
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (r >= h) return;
+  ebn_stats_of_row(r, mean[r], var[r], count, decay, mean, var, rmean, rvar);
+}
+
+// Adds the S slabs' partial pairs of every row: a workgroup takes 64 rows, its four waves every
+// fourth slab with eight loads in flight, and wave 0 adds the four waves' sums in order.  (One
+// thread per row walking 64 slabs by itself took 31 us for 4096 rows.)  STATS: the totals are
+// sums of x and x^2 and go on to mean, variance and the running statistics (out0 = mean,
+// out1 = variance); otherwise they are stored as they are.
+template <bool STATS>
+__global__ void __launch_bounds__(kSplitThreads)
+ebn_merge_slab_sums(int64_t h, int S, const float* __restrict__ part, int64_t slab_stride, float* out0, float* out1,
+                    int64_t count, float decay, float* rmean, float* rvar)
+{
+  __shared__ float lds[kSplitWaves][kWave][2];
+  constexpr int U = 8;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * kWave + lane;
+  const bool ok = r < h;
+  float a = 0.f, b = 0.f;
+  if (ok) {
+    for (int s0 = wave; s0 < S; s0 += U * kSplitWaves) {
+      float va[U], vb[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int sl = s0 + u * kSplitWaves;
+        va[u] = sl < S ? part[sl * slab_stride + r] : 0.f;
+        vb[u] = sl < S ? part[sl * slab_stride + h + r] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        a += va[u];
+        b += vb[u];
+      }
+    }
+  }
+  lds[wave][lane][0] = a;
+  lds[wave][lane][1] = b;
+  __syncthreads();
+  if (wave != 0 || !ok) return;
+  a = lds[0][lane][0], b = lds[0][lane][1];
+#pragma unroll
+  for (int k = 1; k < kSplitWaves; ++k) {
+    a += lds[k][lane][0];
+    b += lds[k][lane][1];
+  }
+  if (STATS) {
+    ebn_stats_of_row(r, a, b, count, decay, out0, out1, rmean, rvar);
+  }
+  else {
+    out0[r] = a;
+    out1[r] = b;
   }
 }
 
@@ -196,7 +274,6 @@ ebn_split_bwd_sums(SplitArgs a)
   const int64_t r0 = (static_cast<int64_t>(blockIdx.x) * kWave + lane) * VE;
   const bool ok = r0 < a.h;
   const int64_t rr = ok ? r0 : 0;
-  const int64_t w = ok ? a.w : 0;
   float mean[VE], inv[VE];
   RowItem<VE>::load(a.mean + rr, mean);
   RowItem<VE>::load(a.var + rr, inv);
@@ -205,7 +282,24 @@ ebn_split_bwd_sums(SplitArgs a)
   float sa[VE], sb[VE];
 #pragma unroll
   for (int r = 0; r < VE; ++r) sa[r] = sb[r] = 0.f;
-  for (int64_t c = wave; c < w; c += kSplitWaves) {
+  const SplitSlab sl = split_slab(a, ok);
+  int64_t c = sl.c0 + wave;
+  for (; c + kSplitWaves < sl.c1; c += 2 * kSplitWaves) {  // two columns of each tensor in flight
+    float v[2][VE], g[2][VE];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      RowItem<VE>::load(a.x + rr + (c + j * kSplitWaves) * a.ldx, v[j]);
+      RowItem<VE>::load(a.dy + rr + (c + j * kSplitWaves) * a.lddy, g[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < VE; ++r) {
+        sa[r] += g[j][r];
+        sb[r] = __builtin_fmaf(g[j][r], v[j][r] - mean[r], sb[r]);
+      }
+  }
+  for (; c < sl.c1; c += kSplitWaves) {
     float v[VE], g[VE];
     RowItem<VE>::load(a.x + rr + c * a.ldx, v);
     RowItem<VE>::load(a.dy + rr + c * a.lddy, g);
@@ -221,8 +315,8 @@ ebn_split_bwd_sums(SplitArgs a)
       sa[r] = -sa[r] * inv[r];
       sb[r] = -sb[r] * inv[r] * inv[r] * inv[r] * 0.5f;
     }
-    RowItem<VE>::store(a.sum0 + r0, sa);
-    RowItem<VE>::store(a.sum1 + r0, sb);
+    RowItem<VE>::store(a.sum0 + sl.out + r0, sa);
+    RowItem<VE>::store(a.sum1 + sl.out + r0, sb);
   }
 }
 
@@ -289,6 +383,83 @@ static int split_check(int64_t h, int64_t w, const int64_t* lds, int nld)
 static dim3 split_grid(int64_t h, int ve, int64_t col_chunks)
 {
   return dim3(static_cast<unsigned>(ceil_div(h, int64_t(kWave) * ve)), static_cast<unsigned>(col_chunks));
+}
+
+// ------------------------------------------------------------ one rank, column slabs
+// Slabs for an (h x w) problem: about four workgroups per compute unit in the summing kernel,
+// at least 16 columns (four per wave) a slab.  1: the path does not pay.
+constexpr int kSlabMinWidth = 1024;       // narrower mini-batches: one workgroup per 64 rows walks them in less time than four launches take
+constexpr int64_t kSlabMaxHeight = 4096;  // taller matrices fill the device well enough without slabs (measured)
+constexpr int kSlabMaxSlabs = 64;
+
+static int ebn_slab_count(int64_t h, int64_t w)
+{
+  if (h % 4 != 0 || h > kSlabMaxHeight || w < kSlabMinWidth) return 1;
+  const int64_t row_blocks = ceil_div(h, int64_t(kWave) * 4);
+  int64_t S = ceil_div(1024, row_blocks);
+  if (S > w / 16) S = w / 16;
+  if (S > kSlabMaxSlabs) S = kSlabMaxSlabs;
+  return static_cast<int>(S < 1 ? 1 : S);
+}
+
+size_t ebn_slab_workspace_bytes(int64_t h, int64_t w)
+{
+  const int S = ebn_slab_count(h, w);
+  return S > 1 ? static_cast<size_t>(S) * 2 * h * sizeof(float) : 0;
+}
+
+static bool ebn_slab_ready(int64_t h, int64_t w, void* ws, size_t ws_bytes)
+{
+  const size_t need = ebn_slab_workspace_bytes(h, w);
+  return need > 0 && ws && aligned16(ws) && ws_bytes >= need;
+}
+
+bool ebn_slab_fwd(hipStream_t st, int64_t h, int64_t w, float eps, float decay, const float* x, int64_t ldx, float* y,
+                  int64_t ldy, float* stats, int64_t ld_stats, float* running_mean, float* running_var, void* ws,
+                  size_t ws_bytes)
+{
+  if (!ebn_slab_ready(h, w, ws, ws_bytes)) return false;
+  if (!split_mat_vec_ok(h, w, x, ldx) || !split_mat_vec_ok(h, w, y, ldy) || !aligned16(stats) || ld_stats % 4 != 0)
+    return false;
+  if (w > int64_t(65535) * kSplitApplyCols) return false;
+  const int S = ebn_slab_count(h, w);
+  float* part = static_cast<float*>(ws);
+  SplitArgs a{};
+  a.h = h; a.w = w; a.eps = eps; a.x = x; a.ldx = ldx; a.out = y; a.ldo = ldy;
+  a.sum0 = part; a.sum1 = part + h; a.slab_cols = ceil_div(w, S); a.slab_stride = 2 * h;
+  hipLaunchKernelGGL((ebn_split_fwd_sums<4>), split_grid(h, 4, S), dim3(kSplitThreads), 0, st, a);
+  hipLaunchKernelGGL(ebn_merge_slab_sums<true>, dim3(static_cast<unsigned>(ceil_div(h, kWave))), dim3(kSplitThreads), 0,
+                     st, h, S, part, a.slab_stride, stats, stats + ld_stats, w, decay, running_mean, running_var);
+  a.mean = stats; a.var = stats + ld_stats;
+  hipLaunchKernelGGL((ebn_split_fwd_apply<4>), split_grid(h, 4, ceil_div(w, kSplitApplyCols)), dim3(kSplitThreads), 0,
+                     st, a);
+  return true;
+}
+
+bool ebn_slab_bwd(hipStream_t st, int64_t h, int64_t w, float eps, const float* x, int64_t ldx, const float* dy,
+                  int64_t lddy, float* dx, int64_t lddx, const float* stats, int64_t ld_stats, float* stats_grad,
+                  int64_t ld_stats_grad, void* ws, size_t ws_bytes)
+{
+  if (!ebn_slab_ready(h, w, ws, ws_bytes)) return false;
+  if (!split_mat_vec_ok(h, w, x, ldx) || !split_mat_vec_ok(h, w, dy, lddy) || !split_mat_vec_ok(h, w, dx, lddx) ||
+      !aligned16(stats) || ld_stats % 4 != 0 || !aligned16(stats_grad) || ld_stats_grad % 4 != 0)
+    return false;
+  if (w > int64_t(65535) * kSplitApplyCols) return false;
+  const int S = ebn_slab_count(h, w);
+  float* part = static_cast<float*>(ws);
+  SplitArgs a{};
+  a.h = h; a.w = w; a.eps = eps; a.count = static_cast<float>(w);
+  a.x = x; a.ldx = ldx; a.dy = dy; a.lddy = lddy; a.out = dx; a.ldo = lddx;
+  a.mean = stats; a.var = stats + ld_stats;
+  a.sum0 = part; a.sum1 = part + h; a.slab_cols = ceil_div(w, S); a.slab_stride = 2 * h;
+  hipLaunchKernelGGL((ebn_split_bwd_sums<4>), split_grid(h, 4, S), dim3(kSplitThreads), 0, st, a);
+  hipLaunchKernelGGL(ebn_merge_slab_sums<false>, dim3(static_cast<unsigned>(ceil_div(h, kWave))), dim3(kSplitThreads),
+                     0, st, h, S, part, a.slab_stride, stats_grad, stats_grad + ld_stats_grad, int64_t(0), 0.f,
+                     static_cast<float*>(nullptr), static_cast<float*>(nullptr));
+  a.sum0 = stats_grad; a.sum1 = stats_grad + ld_stats_grad;
+  hipLaunchKernelGGL((ebn_split_bwd_apply<4>), split_grid(h, 4, ceil_div(w, kSplitApplyCols)), dim3(kSplitThreads), 0,
+                     st, a);
+  return true;
 }
 
 }  // namespace lbn

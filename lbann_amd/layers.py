@@ -348,22 +348,29 @@ class entrywise_batch_normalization_layer(_Layer):
         self.m_batch_statistics = DeviceMatrix(h, 2, device=device)
         self.m_batch_statistics_gradient = DeviceMatrix(h, 2, device=device)
         self.training = True
+        self._ws = _Workspace(type(self).__name__, header=False)  # partial sums only: no kernel of this layer waits
+
+    def _scratch(self):
+        x = self.prev_activations
+        return self._ws.get(capi.lib().lbn_entrywise_batch_norm_workspace_bytes(x.height, x.width), self.device)
 
     def fp_call(self):
         x, y = self.prev_activations, self.activations
         st = self.m_batch_statistics
+        ws, nb = self._scratch()
         return ("lbn_entrywise_batch_norm_fwd_f32",
                 (_stream(), x.height, x.width, self.m_decay, self.m_epsilon, int(self.training), x.Buffer(),
                  x.ldim, y.Buffer(), y.ldim, st.Buffer(), st.ldim, self.weights[0].Buffer(),
-                 self.weights[1].Buffer()))
+                 self.weights[1].Buffer(), ws, nb))
 
     def bp_call(self):
         x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
         st, sg = self.m_batch_statistics, self.m_batch_statistics_gradient
+        ws, nb = self._scratch()
         return ("lbn_entrywise_batch_norm_bwd_f32",
                 (_stream(), x.height, x.width, self.m_epsilon, int(self.training), x.Buffer(), x.ldim,
                  dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim, st.Buffer(), st.ldim, sg.Buffer(), sg.ldim,
-                 self.weights[1].Buffer()))
+                 self.weights[1].Buffer(), ws, nb))
 
     def _col(self, m, j):
         return capi.vp(m.tensor.data_ptr() + 4 * j * m.ldim)

@@ -492,7 +492,8 @@ def test_instance_norm(L, dims, w, pad):
 # ===================================================================== entry-wise batch norm
 @pytest.mark.parametrize("h,w,pad", [(105, 14, 0), (105, 29, 0), (4096, 64, 0), (4096, 256, 0), (1024, 300, 0),
                                      (200000, 16, 0), (64, 1, 0), (260, 7, 4), (258, 9, 0), (100000, 33, 0),
-                                     (2048, 1000, 0), (8196, 257, 4), (60, 513, 0)])   # wider than the register tiles
+                                     (2048, 1000, 0), (8196, 257, 4), (60, 513, 0),   # wider than the register tiles
+                                     (4096, 1024, 0), (512, 4100, 0), (64, 5000, 4), (1000, 1777, 0), (4, 2000, 0), (4096, 1023, 0)])   # column slabs from 1024 columns
 def test_entrywise_batch_norm(L, h, w, pad):
     rng = np.random.default_rng(h + 3 * w)
     x, dy = rand(rng, h, w, 0.5, 2.0), rand(rng, h, w)
