@@ -28,7 +28,7 @@ namespace lbn {
 
 constexpr int kSbThreads = 256;
 constexpr int kSbWaves = kSbThreads / kWave;
-constexpr int kSbMaxParts = 64;  // one wave merges the partial pairs of a channel
+constexpr int kSbMaxParts = 1024;  // workgroups per channel; one wave merges their partial pairs
 
 // ===================================================================== entry-wise
 struct EsbArgs {
@@ -402,10 +402,10 @@ csb_merge_parts(int P, const float2* __restrict__ part, float* __restrict__ wgra
   const int64_t ch = blockIdx.x;
   const int lane = threadIdx.x;
   float a = 0.f, b = 0.f;
-  if (lane < P) {
-    const float2 v = part[ch * P + lane];
-    a = v.x;
-    b = v.y;
+  for (int p = lane; p < P; p += kWave) {  // lane-strided, then the wave: a fixed order
+    const float2 v = part[ch * P + p];
+    a += v.x;
+    b += v.y;
   }
   a = wave_sum(a);
   b = wave_sum(b);
@@ -417,6 +417,7 @@ csb_merge_parts(int P, const float2* __restrict__ part, float* __restrict__ wgra
 
 // 256-thread workgroups per channel: about 2048 in total, each thread with at least four
 // vectors.
+// (three channels of a 299 x 299 image had been held to 64 workgroups each)
 static int csb_parts(int64_t C, int64_t vectors_per_channel)
 {
   int64_t p = ceil_div(2048, C);
@@ -561,7 +562,9 @@ size_t lbn_channelwise_scale_bias_bwd_workspace_bytes(int64_t num_channels, int6
                                                       int64_t width)
 {
   if (num_channels <= 0 || channel_size <= 0 || width <= 0) return 0;
-  size_t need = static_cast<size_t>(num_channels) * kSbMaxParts * sizeof(float2);
+  // at most ceil(2048 / channels) workgroups per channel (csb_parts)
+  const int64_t parts = ceil_div(2048, num_channels) < kSbMaxParts ? ceil_div(2048, num_channels) : kSbMaxParts;
+  size_t need = static_cast<size_t>(num_channels) * parts * sizeof(float2);
   const int64_t height = num_channels * channel_size;
   if (csb_rows_shape(channel_size) && height % 4 == 0) {  // per-row pairs of the row tiling
     const size_t rows = static_cast<size_t>(row_tile_plan(height, width).slabs) * height * sizeof(float2);
