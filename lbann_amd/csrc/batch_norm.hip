@@ -32,7 +32,8 @@
 namespace lbn {
 
 constexpr int kBnThreads = 256;
-constexpr int kBnMaxSplit = 64;  // P <= one wave, so a wave merges a channel's partials
+constexpr int kBnMaxSplit = 1024;  // workgroups per channel; a wave merges a channel's partials (three channels of a
+                                   // 299 x 299 image had been held to 64 workgroups each)
 
 // Walks the elements of channel c owned by workgroup p: calls f(offset_in_x, offset_in_y...)
 // through index arithmetic shared by all kernels.  `unit` = floats per access (4 or 1),
@@ -96,10 +97,10 @@ __device__ __forceinline__ float2 merge_partials(const float2* part, int64_t c, 
 {
   const int lane = threadIdx.x & (kWave - 1);
   float a = 0.f, b = 0.f;
-  if (lane < P) {
-    const float2 v = part[c * P + lane];
-    a = v.x;
-    b = v.y;
+  for (int p = lane; p < P; p += kWave) {  // lane-strided, then the wave: a fixed order
+    const float2 v = part[c * P + p];
+    a += v.x;
+    b += v.y;
   }
   return make_float2(wave_sum(a), wave_sum(b));
 }
