@@ -206,10 +206,14 @@ bn_fwd_apply(const S* __restrict__ x, S* __restrict__ y, int64_t ldx, int64_t ld
 
 // ----------------------------------------------------------------- backward sums
 // Two sums per channel carry all four gradients: A = sum(dy), B = sum(dy * (x - mean)).
-template <typename S, bool VEC>
+// DX: outside training the statistics are constants, so dx = dy * scale / stdev needs none of
+// the sums and is written in the same pass (three tensors of traffic instead of five).
+template <typename S, bool VEC, bool DX = false>
 __global__ void __launch_bounds__(kBnThreads)
 bn_bwd_sums(const S* __restrict__ x, const S* __restrict__ dy, int64_t ldx, int64_t lddy,
-            int64_t cs, int64_t w, const float* __restrict__ mean_in, float2* __restrict__ part)
+            int64_t cs, int64_t w, const float* __restrict__ mean_in, float2* __restrict__ part,
+            const float* __restrict__ var_in = nullptr, const float* __restrict__ gamma = nullptr, float eps = 0.f,
+            S* dx = nullptr, int64_t lddx = 0)
 {
   __shared__ float red[2 * (kBnThreads / kWave)];
   const int P = gridDim.y;
@@ -221,6 +225,8 @@ bn_bwd_sums(const S* __restrict__ x, const S* __restrict__ dy, int64_t ldx, int6
   const S* xc = x + c * cs;
   const S* gc = dy + c * cs;
   const float mean = mean_in[c];
+  const float k0 = DX ? gamma[c] * (1.0f / sqrtf(var_in[c] + eps)) : 0.f;
+  S* dc = DX ? dx + c * cs : nullptr;
   float a = 0.f, b = 0.f;
   const int64_t step = static_cast<int64_t>(P) * kBnThreads;
   for (int64_t j = static_cast<int64_t>(p) * kBnThreads + threadIdx.x; j < wk.total; j += step) {
@@ -236,11 +242,17 @@ bn_bwd_sums(const S* __restrict__ x, const S* __restrict__ dy, int64_t ldx, int6
         a += g[k];
         b += g[k] * (v[k] - mean);
       }
+      if (DX) {  // in place (dx aliasing dy): the thread has read what it overwrites
+#pragma unroll
+        for (int k = 0; k < VE; ++k) g[k] *= k0;
+        IO::store(dc + col * lddx + VE * i, g);
+      }
     }
     else {
       const float g = IO::load1(gc + col * lddy + i);
       a += g;
       b += g * (IO::load1(xc + col * ldx + i) - mean);
+      if (DX) IO::store1(dc + col * lddx + i, g * k0);
     }
   }
   team_sum2<kBnThreads / kWave>(a, b, red, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
@@ -251,7 +263,7 @@ __global__ void __launch_bounds__(kWave)
 bn_store_grads(const float2* __restrict__ part, int P, float eps, const float* __restrict__ mean,
                const float* __restrict__ var, const float* __restrict__ gamma,
                float* __restrict__ dscale, float* __restrict__ dbias, float* __restrict__ dmean,
-               float* __restrict__ dvar)
+               float* __restrict__ dvar, int training = 1)
 {
   const int64_t c = blockIdx.x;
   const float2 r = merge_partials(part, c, P);
@@ -261,8 +273,8 @@ bn_store_grads(const float2* __restrict__ part, int P, float eps, const float* _
     grads_from_sums(r.x, r.y, gamma[c], inv_stdev, ds, db, dm, dv);
     dscale[c] = ds;
     dbias[c] = db;
-    dmean[c] = dm;
-    dvar[c] = dv;
+    dmean[c] = training ? dm : 0.f;  // statistics are constants outside training
+    dvar[c] = training ? dv : 0.f;
   }
   (void)mean;
 }
@@ -1359,6 +1371,18 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
     sa.eps = epsilon, sa.mean = const_cast<float*>(use_mean), sa.var = const_cast<float*>(use_var), sa.scale = scale;
     sa.dscale = dscale, sa.dbias = dbias, sa.dmean = dmean, sa.dvar = dvar;
     if (bn_try_stream<S, true>(st, sa, C, cs, w, workspace)) return launch_status();
+  }
+  if (!training && n > 1) {
+    // statistics are constants: dx in the same pass as the sums, then the four gradients
+    if (vec)
+      hipLaunchKernelGGL((bn_bwd_sums<S, true, true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean,
+                         part, use_var, scale, epsilon, dx, lddx);
+    else
+      hipLaunchKernelGGL((bn_bwd_sums<S, false, true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean,
+                         part, use_var, scale, epsilon, dx, lddx);
+    hipLaunchKernelGGL(bn_store_grads, dim3(static_cast<unsigned>(C)), dim3(kWave), 0, st, part,
+                       static_cast<int>(grid.y), epsilon, use_mean, use_var, scale, dscale, dbias, dmean, dvar, 0);
+    return launch_status();
   }
   if (vec) {
     hipLaunchKernelGGL((bn_bwd_sums<S, true>), grid, dim3(kBnThreads), 0, st, x, dy, ldx, lddy, cs, w, use_mean, part);
