@@ -571,7 +571,7 @@ int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_
   }
   const dim3 grid(static_cast<unsigned>(ceil_div(height, 256))), block(256);
   if (training) hipLaunchKernelGGL((ebn_fwd_generic<true>), grid, block, 0, st, a);
-  else hipLaunchKernelGGL((ebn_fwd_generic<false>), grid, block, 0, st, a);
+  else ebn_inference_fwd(st, height, width, epsilon, x, ldx, y, ldy, running_mean, running_var);
   return launch_status();
 }
 
@@ -590,8 +590,7 @@ int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_
                   ld_stats, stats_grad, ld_stats_grad, nullptr, const_cast<float*>(running_var)};
   if (!training) {
     if (!running_var) return LBN_ERR_INVALID_ARGUMENT;
-    hipLaunchKernelGGL((ebn_bwd_generic<false>), dim3(static_cast<unsigned>(ceil_div(height, 256))),
-                       dim3(256), 0, st, a);
+    ebn_inference_bwd(st, height, width, epsilon, dy, lddy, dx, lddx, running_var);
     return launch_status();
   }
   if (!x || !stats || !stats_grad || ld_stats < height || ld_stats_grad < height)

@@ -262,6 +262,30 @@ ebn_split_fwd_apply(SplitArgs a)
   }
 }
 
+// dx = dy / sqrt(var + eps): the backward pass outside training (:352-392).  Grid as above.
+template <int VE>
+__global__ void __launch_bounds__(kSplitThreads)
+ebn_split_scale_rows(SplitArgs a)
+{
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t r0 = (static_cast<int64_t>(blockIdx.x) * kWave + lane) * VE;
+  if (r0 >= a.h) return;
+  float inv[VE];
+  RowItem<VE>::load(a.var + r0, inv);
+#pragma unroll
+  for (int r = 0; r < VE; ++r) inv[r] = 1.0f / sqrtf(inv[r] + a.eps);
+  const int64_t c_begin = static_cast<int64_t>(blockIdx.y) * kSplitApplyCols;
+  const int64_t c_end = c_begin + kSplitApplyCols < a.w ? c_begin + kSplitApplyCols : a.w;
+  for (int64_t c = c_begin + wave; c < c_end; c += kSplitWaves) {
+    float g[VE];
+    RowItem<VE>::load(a.dy + r0 + c * a.lddy, g);
+#pragma unroll
+    for (int r = 0; r < VE; ++r) g[r] *= inv[r];
+    RowItem<VE>::store(a.out + r0 + c * a.ldo, g);
+  }
+}
+
 // sum0 = local part of dL/dmean = -sum(dy) / stdev, sum1 = of dL/dvar =
 // -sum(dy (x - mean)) / (2 stdev^3) (entrywise_batch_normalization.cpp:275-299).
 template <int VE>
@@ -460,6 +484,45 @@ bool ebn_slab_bwd(hipStream_t st, int64_t h, int64_t w, float eps, const float* 
   hipLaunchKernelGGL((ebn_split_bwd_apply<4>), split_grid(h, 4, ceil_div(w, kSplitApplyCols)), dim3(kSplitThreads), 0,
                      st, a);
   return true;
+}
+
+void ebn_inference_fwd(hipStream_t st, int64_t h, int64_t w, float eps, const float* x, int64_t ldx, float* y,
+                       int64_t ldy, const float* running_mean, const float* running_var)
+{
+  SplitArgs a{};
+  a.h = h; a.w = w; a.eps = eps; a.x = x; a.ldx = ldx; a.out = y; a.ldo = ldy;
+  a.mean = running_mean; a.var = running_var;
+  const bool vec = split_mat_vec_ok(h, w, x, ldx) && split_mat_vec_ok(h, w, y, ldy) && aligned16(running_mean) &&
+                   aligned16(running_var);
+  // columns beyond gridDim.y's reach: the call is repeated over column blocks
+  const int64_t per_call = int64_t(65535) * kSplitApplyCols;
+  for (int64_t c0 = 0; c0 < w; c0 += per_call) {
+    SplitArgs b = a;
+    b.w = w - c0 < per_call ? w - c0 : per_call;
+    b.x = x + c0 * ldx;
+    b.out = y + c0 * ldy;
+    const int64_t chunks = ceil_div(b.w, kSplitApplyCols);
+    if (vec) hipLaunchKernelGGL((ebn_split_fwd_apply<4>), split_grid(h, 4, chunks), dim3(kSplitThreads), 0, st, b);
+    else hipLaunchKernelGGL((ebn_split_fwd_apply<1>), split_grid(h, 1, chunks), dim3(kSplitThreads), 0, st, b);
+  }
+}
+
+void ebn_inference_bwd(hipStream_t st, int64_t h, int64_t w, float eps, const float* dy, int64_t lddy, float* dx,
+                       int64_t lddx, const float* running_var)
+{
+  SplitArgs a{};
+  a.h = h; a.w = w; a.eps = eps; a.dy = dy; a.lddy = lddy; a.out = dx; a.ldo = lddx; a.var = running_var;
+  const bool vec = split_mat_vec_ok(h, w, dy, lddy) && split_mat_vec_ok(h, w, dx, lddx) && aligned16(running_var);
+  const int64_t per_call = int64_t(65535) * kSplitApplyCols;
+  for (int64_t c0 = 0; c0 < w; c0 += per_call) {
+    SplitArgs b = a;
+    b.w = w - c0 < per_call ? w - c0 : per_call;
+    b.dy = dy + c0 * lddy;
+    b.out = dx + c0 * lddx;
+    const int64_t chunks = ceil_div(b.w, kSplitApplyCols);
+    if (vec) hipLaunchKernelGGL((ebn_split_scale_rows<4>), split_grid(h, 4, chunks), dim3(kSplitThreads), 0, st, b);
+    else hipLaunchKernelGGL((ebn_split_scale_rows<1>), split_grid(h, 1, chunks), dim3(kSplitThreads), 0, st, b);
+  }
 }
 
 }  // namespace lbn
