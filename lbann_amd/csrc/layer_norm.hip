@@ -1305,6 +1305,13 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
       if (vec)
         hipLaunchKernelGGL((ln_wgrad_columns<T, true>), grid, dim3(256), 0, st, x, dy, ldx, lddy, map, rows,
                            units, n, eps, stats, lds, wpart);
+      else if (std::is_same<T, float>::value && n >= 64) {
+        // fp32 rows off the 16-byte grid: 16-byte accesses at 4-byte alignment, the last n % 4 features apart
+        const dim3 ugrid(static_cast<unsigned>(ceil_div(n / 4 + 1, 256)), static_cast<unsigned>(slabs));
+        hipLaunchKernelGGL((ln_wgrad_columns<f32u, true>), ugrid, dim3(256), 0, st, reinterpret_cast<const f32u*>(x),
+                           reinterpret_cast<const f32u*>(dy), ldx, lddy, map, rows, n / 4, n, eps, stats, lds, wpart,
+                           static_cast<int>(n % 4));
+      }
       else
         hipLaunchKernelGGL((ln_wgrad_columns<T, false>), grid, dim3(256), 0, st, x, dy, ldx, lddy, map, rows,
                            units, n, eps, stats, lds, wpart);

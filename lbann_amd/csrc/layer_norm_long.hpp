@@ -247,16 +247,20 @@ template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
 ln_wgrad_columns(const T* __restrict__ x, const T* __restrict__ dy, int64_t ldx, int64_t lddy,
                  RowMap map, int64_t rows, int64_t units, int64_t n, float eps,
-                 const float* __restrict__ stats, int64_t ld_stats, float* __restrict__ wpart)
+                 const float* __restrict__ stats, int64_t ld_stats, float* __restrict__ wpart, int tail = 0)
 {
+  // tail (VEC only, f32u data): features after the `units` whole vectors; the thread after the
+  // last vector takes them entry by entry.
   using IO = Vec16<T>;
   constexpr int VE = VEC ? IO::N : 1;
   const int64_t k = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   const int64_t per = (rows + gridDim.y - 1) / gridDim.y;
   const int64_t r0 = static_cast<int64_t>(blockIdx.y) * per;
   const int64_t r1 = imin64(r0 + per, rows);
-  const bool ok = k < units;
+  const bool partial = VEC && tail > 0 && k == units;
+  const bool ok = k < units || partial;
   const int64_t off = ok ? VE * k : 0;
+  const int mine = partial ? tail : VE;  // entries of this thread's access unit
   float dg[VE], db[VE];
 #pragma unroll
   for (int e = 0; e < VE; ++e) dg[e] = db[e] = 0.f;
@@ -268,8 +272,17 @@ ln_wgrad_columns(const T* __restrict__ x, const T* __restrict__ dy, int64_t ldx,
     const float inv_stdev = 1.0f / sqrtf(stats[map.groups + g + col * ld_stats] + eps);
     float v[VE], d[VE];
     if constexpr (VEC) {
-      IO::load(x + g * map.stride + col * ldx + off, v);
-      IO::load(dy + g * map.stride + col * lddy + off, d);
+      if (!partial) {
+        IO::load(x + g * map.stride + col * ldx + off, v);
+        IO::load(dy + g * map.stride + col * lddy + off, d);
+      }
+      else {
+#pragma unroll
+        for (int e = 0; e < VE; ++e) {
+          v[e] = e < tail ? IO::load1(x + g * map.stride + col * ldx + off + e) : 0.f;
+          d[e] = e < tail ? IO::load1(dy + g * map.stride + col * lddy + off + e) : 0.f;
+        }
+      }
     }
     else {
       v[0] = IO::load1(x + g * map.stride + col * ldx + off);
@@ -285,8 +298,10 @@ ln_wgrad_columns(const T* __restrict__ x, const T* __restrict__ dy, int64_t ldx,
   float* out = wpart + static_cast<int64_t>(blockIdx.y) * 2 * n;
 #pragma unroll
   for (int e = 0; e < VE; ++e) {
-    out[off + e] = dg[e];
-    out[n + off + e] = db[e];
+    if (e < mine) {
+      out[off + e] = dg[e];
+      out[n + off + e] = db[e];
+    }
   }
 }
 
