@@ -835,6 +835,7 @@ static bool rows_aligned4(const void* base, int64_t stride, int64_t ld, int64_t 
          (width <= 1 || ld % 2 == 0);
 }
 
+constexpr int64_t kLnLongMin16 = 4096;  // shortest fp16 row of odd length that takes a 1024-thread workgroup of its own (1001 entries: 75 against 40 us)
 constexpr int64_t kLnMaxScalarRowFwd = 8192;  // rows accessed one float at a time: 1024 threads x 8
 constexpr int64_t kLnMaxScalarRowBwd = 4096;  // 512 threads x 8
 
@@ -1121,6 +1122,15 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                        static_cast<int>(n % 4), inv_n, eps, stats, lds, gamma, beta, sumsq);
     return launch_status();
   }
+  if constexpr (std::is_same<T, __half>::value) {
+    // fp16 rows of odd length (or off the 4-byte grid): the same, eight entries per access at 2-byte alignment
+    if (n >= kLnLongMin16) {
+      hipLaunchKernelGGL((ln_fwd_long<f16u>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
+                         reinterpret_cast<const f16u*>(x), reinterpret_cast<f16u*>(y), ldx, ldy, map, n / 8,
+                         static_cast<int>(n % 8), inv_n, eps, stats, lds, gamma, beta, sumsq);
+      return launch_status();
+    }
+  }
   hipLaunchKernelGGL((ln_fwd_generic<T>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, st, x, y,
                      ldx, ldy, map, n, eps, stats, lds, gamma, beta, sumsq);
   return launch_status();
@@ -1290,6 +1300,11 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
       hipLaunchKernelGGL((ln_bwd_long<f32u>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
                          reinterpret_cast<const f32u*>(x), reinterpret_cast<const f32u*>(dy),
                          reinterpret_cast<f32u*>(dx), ldx, lddy, lddx, map, n / 4, static_cast<int>(n % 4),
+                         1.0f / static_cast<float>(n), eps, stats, lds, sgrad, ldsg, gamma);
+    else if (std::is_same<T, __half>::value && n >= kLnLongMin16)
+      hipLaunchKernelGGL((ln_bwd_long<f16u>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
+                         reinterpret_cast<const f16u*>(x), reinterpret_cast<const f16u*>(dy),
+                         reinterpret_cast<f16u*>(dx), ldx, lddy, lddx, map, n / 8, static_cast<int>(n % 8),
                          1.0f / static_cast<float>(n), eps, stats, lds, sgrad, ldsg, gamma);
     else
       hipLaunchKernelGGL((ln_bwd_generic<T>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, st, x, dy,

@@ -449,7 +449,8 @@ def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
                                                    # even lengths that are not a multiple of 8: one pair per access
                                                    ((4100,), 0, 40, 0), ((1002,), 0, 33, 0), ((6, 770), -1, 9, 0),
                                                    ((8190,), 0, 5, 2), ((16382,), 0, 3, 0), ((4100, 12), -1, 2, 0),
-                                                   ((1001,), 0, 7, 0),   # odd: scalar fallback
+                                                   ((1001,), 0, 7, 0), ((4099,), 0, 9, 0), ((10001,), 0, 5, 1), ((513,), 0, 40, 0),   # odd: eight entries per access at 2-byte alignment
+                                                   ((50003,), 0, 3, 0), ((20002,), 0, 4, 1), ((301,), 0, 20, 0),   # (below 4096 entries: scalar fallback)
                                                    # long rows shared by clusters of workgroups
                                                    ((802816,), 0, 4, 0), ((65536,), 0, 150, 0), ((2, 100000), -1, 20, 8),
                                                    ((1048576,), 0, 2, 0), ((5000000,), 0, 2, 0)])
