@@ -401,9 +401,9 @@ __device__ __forceinline__ void ebn_walk_columns(int64_t w, Load&& load, Use&& u
   }
 }
 
-// One thread per row.  TRAINING: statistics from the mini-batch (written to stats, running
-// statistics updated); otherwise the running statistics are used as they are.
-template <bool TRAINING>
+// One thread per row, training mode: statistics from the mini-batch (written to stats, running
+// statistics updated).  (Outside training both directions are element-wise with per-row
+// coefficients and run on a two-dimensional grid, entrywise_batch_norm_slabs.hpp.)
 __global__ void __launch_bounds__(256)
 ebn_fwd_generic(EbnArgs a)
 {
@@ -411,7 +411,7 @@ ebn_fwd_generic(EbnArgs a)
   if (r >= a.h) return;
   const float* xr = a.x + r;
   float mean, var;
-  if (TRAINING) {
+  {
     const float K = xr[0];
     float s = 0.f, q = 0.f;
     float v[8];
@@ -430,10 +430,6 @@ ebn_fwd_generic(EbnArgs a)
       a.rvar[r] = a.decay * a.rvar[r] + (1.f - a.decay) * var;
     }
   }
-  else {
-    mean = a.rmean[r];
-    var = a.rvar[r];
-  }
   const float inv = 1.0f / sqrtf(var + a.eps);
   float* yr = a.out + r;
   float v[8];
@@ -442,7 +438,6 @@ ebn_fwd_generic(EbnArgs a)
     [&](int64_t c, int u) { yr[c * a.ldo] = (v[u] - mean) * inv; });
 }
 
-template <bool TRAINING>
 __global__ void __launch_bounds__(256)
 ebn_bwd_generic(EbnArgs a)
 {
@@ -450,14 +445,6 @@ ebn_bwd_generic(EbnArgs a)
   if (r >= a.h) return;
   const float* gr = a.dy + r;
   float* dr = a.out + r;
-  if (!TRAINING) {  // entrywise_batch_normalization.cpp:352-392
-    const float inv = 1.0f / sqrtf(a.rvar[r] + a.eps);
-    float g[8];
-    ebn_walk_columns(
-      a.w, [&](int64_t c, int u) { g[u] = gr[c * a.lddy]; },
-      [&](int64_t c, int u) { dr[c * a.ldo] = g[u] * inv; });
-    return;
-  }
   const float* xr = a.x + r;
   const float mean = a.stats[r];
   const float inv = 1.0f / sqrtf(a.stats[r + a.ld_stats] + a.eps);
@@ -570,7 +557,7 @@ int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_
     return launch_status();
   }
   const dim3 grid(static_cast<unsigned>(ceil_div(height, 256))), block(256);
-  if (training) hipLaunchKernelGGL((ebn_fwd_generic<true>), grid, block, 0, st, a);
+  if (training) hipLaunchKernelGGL(ebn_fwd_generic, grid, block, 0, st, a);
   else ebn_inference_fwd(st, height, width, epsilon, x, ldx, y, ldy, running_mean, running_var);
   return launch_status();
 }
@@ -621,7 +608,7 @@ int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_
                        dim3(kEbnThreads), 0, st, a);
     return launch_status();
   }
-  hipLaunchKernelGGL((ebn_bwd_generic<true>), dim3(static_cast<unsigned>(ceil_div(height, 256))),
+  hipLaunchKernelGGL(ebn_bwd_generic, dim3(static_cast<unsigned>(ceil_div(height, 256))),
                      dim3(256), 0, st, a);
   return launch_status();
 }
