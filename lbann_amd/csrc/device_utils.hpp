@@ -327,12 +327,14 @@ template <>
 struct Vec16<f16u> {
   static constexpr int N = 8;
   using raw_t = v4u;
-  static __device__ __forceinline__ void load(const f16u* p, float (&v)[8])
+  static __device__ __forceinline__ raw_t load_raw(const f16u* p)
   {
     v4u r;
     __builtin_memcpy(&r, p, 16);
-    Vec16<__half>::unpack(r, v);
+    return r;
   }
+  static __device__ __forceinline__ void unpack(const raw_t& r, float (&v)[8]) { Vec16<__half>::unpack(r, v); }
+  static __device__ __forceinline__ void load(const f16u* p, float (&v)[8]) { unpack(load_raw(p), v); }
   static __device__ __forceinline__ void store(f16u* p, const float (&v)[8])
   {
     unsigned int w[4];
@@ -346,6 +348,10 @@ struct Vec16<f16u> {
   static __device__ __forceinline__ float load1(const f16u* p) { return __half2float(p->v); }
   static __device__ __forceinline__ void store1(f16u* p, float v) { p->v = __float2half_rn(v); }
 };
+
+// Storage types whose 16-byte accesses need no alignment beyond that of one entry.
+template <typename T>
+struct UnalignedVec : std::integral_constant<bool, std::is_same<T, f16u>::value || std::is_same<T, f32u>::value> {};
 
 // ---------------------------------------------------------------------------
 // exp(x) for x <= ~0 (softmax arguments after max-subtraction) in 6 VALU operations

@@ -44,12 +44,16 @@ __global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
 ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy, RowMap map,
             int64_t rows, int nvec, float inv_n, float eps, float* __restrict__ stats,
             int64_t ld_stats, const float* __restrict__ gamma, const float* __restrict__ beta,
-            int sumsq)
+            int sumsq, int tail = 0)
 {
   using B = RowBlock<TPR>;
   using IO = Vec16<T>;
   using raw_t = typename IO::raw_t;
   constexpr int VE = IO::N;
+  // Storage types whose 16-byte accesses need no alignment take rows of any length: nvec counts
+  // a last vector of `tail` entries (0: none), which is read as the row's last VE entries,
+  // overlapping its neighbour; the entries it shares count and are stored once, by the neighbour.
+  constexpr bool kTail = UnalignedVec<T>::value;
   constexpr bool kSub = TPR < kWave;  // short rows: a team is one DPP row of 16 lanes, four rows per wave
   static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
   constexpr int NW = kSub ? 1 : B::kWavesPerTeam;
@@ -67,15 +71,25 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
   // A vector past the end of the row re-reads vector 0 and is masked out of the sums.
   bool ok[V];
   int voff[V];
+  int skip[V];  // leading entries of the vector that belong to its neighbour
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     ok[i] = t + i * TPR < nvec;
     voff[i] = ok[i] ? VE * (t + i * TPR) : 0;
+    skip[i] = 0;
+    if (kTail && tail && t + i * TPR == nvec - 1) {
+      skip[i] = VE - tail;
+      voff[i] -= skip[i];
+    }
   }
+  const int n_entries = (kTail && tail) ? (nvec - 1) * VE + tail : nvec * VE;
   auto load_weights = [&](const float* w, int i, float fill, float (&out)[VE]) {
 #pragma unroll
     for (int k = 0; k < VE; ++k) out[k] = fill;
-    if (w) load_f32_run<VE>(w + voff[i], out);
+    if (w) {
+      if constexpr (kTail) __builtin_memcpy(out, w + voff[i], sizeof(float) * VE);
+      else load_f32_run<VE>(w + voff[i], out);
+    }
   };
   float gam[WV][VE], bet[WV][VE];
   if constexpr (kWeightsInRegs) {
@@ -109,6 +123,11 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
 #pragma unroll
         for (int k = 0; k < VE; ++k) v[i][k] = 0.f;
       }
+      if constexpr (kTail) {
+#pragma unroll
+        for (int k = 0; k < VE; ++k)
+          if (k < skip[i]) v[i][k] = 0.f;
+      }
     }
     if constexpr (kPrefetch) {
       if (it + 1 < iters) issue(row + rows_per_iter);
@@ -133,7 +152,7 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
       }
       // the reference's own expression (layer_norm.cpp:99-112): true divisions, no fused
       // multiply-add, so that its cancellation and clamp come out the same
-      const float nf = static_cast<float>(nvec * VE);
+      const float nf = static_cast<float>(n_entries);
       mean = s / nf;
       var = fmaxf(__fsub_rn(sq / nf, __fmul_rn(mean, mean)), 0.f);
 #pragma unroll
@@ -155,7 +174,7 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
 #pragma unroll
         for (int k = 0; k < VE; ++k) {
           v[i][k] -= mean;
-          const float d = (kFull || ok[i]) ? v[i][k] : 0.f;
+          const float d = ((kFull || ok[i]) && !(kTail && k < skip[i])) ? v[i][k] : 0.f;
           sq = __builtin_fmaf(d, d, sq);
         }
       }
@@ -186,14 +205,23 @@ ln_fwd_rows(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_t ldy
 #pragma unroll
             for (int k = 0; k < VE; ++k) v[i][k] = __builtin_fmaf(v[i][k] * inv_stdev, gw[k], bw[k]);
           }
-          IO::store(yr + voff[i], v[i]);
+          bool whole = true;
+          if constexpr (kTail) {
+            if (skip[i]) {
+              whole = false;
+#pragma unroll
+              for (int k = 0; k < VE; ++k)
+                if (k >= skip[i]) IO::store1(yr + voff[i] + k, v[i][k]);
+            }
+          }
+          if (whole) IO::store(yr + voff[i], v[i]);
         }
       }
     }
   };
 
   if constexpr (kPrefetch) issue(first_row);
-  if (nvec == TPR * V) {
+  if (nvec == TPR * V && !(kTail && tail)) {
     for (int64_t it = 0; it < iters; ++it) process(it, std::true_type{});
   }
   else {
@@ -396,13 +424,16 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
             int64_t lddy, int64_t lddx, RowMap map, int64_t rows, int nvec, int n, float eps,
             const float* __restrict__ stats, int64_t ld_stats, float* __restrict__ sgrad,
             int64_t ld_sgrad, const float* __restrict__ gamma, float* __restrict__ part,
-            float* __restrict__ dscale, float* __restrict__ dbias)
+            float* __restrict__ dscale, float* __restrict__ dbias, int tail = 0)
 {
   static_assert(!(WGRAD && COLS), "one way of forming the weight gradients");
   using B = RowBlock<TPR, TEAMS>;
   using IO = Vec16<T>;
   using raw_t = typename IO::raw_t;
   constexpr int VE = IO::N;
+  // a last vector of `tail` entries, read as the row's last VE entries: see ln_fwd_rows
+  constexpr bool kTail = UnalignedVec<T>::value;
+  static_assert(!kTail || !(WGRAD || COLS), "rows with a partial vector leave the weight gradients to another kernel");
   constexpr bool kSub = TPR < kWave;
   static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
   constexpr int NW = kSub ? 1 : B::kWavesPerTeam;
@@ -423,13 +454,30 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   if constexpr (COLS)
     ln_cols_issue<T, B::kThreads>(cols, x, dy, ldx, lddy, map, rows, n, stats, ld_stats, blockIdx.x, 0);
 
+  // Loads are issued unconditionally: a row past the end re-reads the last row, a
+  // vector past the end of a row re-reads vector 0.
+  bool ok[V];
+  int voff[V];
+  int skip[V];  // leading entries of the vector that belong to its neighbour
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    ok[i] = t + i * TPR < nvec;
+    voff[i] = ok[i] ? VE * (t + i * TPR) : 0;
+    skip[i] = 0;
+    if (kTail && tail && t + i * TPR == nvec - 1) {
+      skip[i] = VE - tail;
+      voff[i] -= skip[i];
+    }
+  }
   float gam[V][VE];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    const int idx = t + i * TPR;
 #pragma unroll
     for (int k = 0; k < VE; ++k) gam[i][k] = 1.f;
-    if (gamma && idx < nvec) load_f32_run<VE>(gamma + VE * idx, gam[i]);
+    if (gamma && ok[i]) {
+      if constexpr (kTail) __builtin_memcpy(gam[i], gamma + voff[i], sizeof(float) * VE);
+      else load_f32_run<VE>(gamma + voff[i], gam[i]);
+    }
   }
   float dg[WGRAD ? V : 1][VE], db[WGRAD ? V : 1][VE];
   if (WGRAD) {
@@ -444,16 +492,7 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
     raw_t x[V], g[V];
     float mean, var;
   };
-  // Loads are issued unconditionally: a row past the end re-reads the last row, a
-  // vector past the end of a row re-reads vector 0.
   // All row arithmetic is wave-uniform (scalar registers).
-  bool ok[V];
-  int voff[V];
-#pragma unroll
-  for (int i = 0; i < V; ++i) {
-    ok[i] = t + i * TPR < nvec;
-    voff[i] = ok[i] ? VE * (t + i * TPR) : 0;
-  }
   auto issue = [&](Slot& s, int64_t row) {
     int64_t col, g;
     map.split(row < rows ? row : rows - 1, col, g);
@@ -494,10 +533,11 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
     float a = 0.f, b = 0.f;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      const bool use = kFull || (active && ok[i]);
+      const bool use_vec = kFull || (active && ok[i]);
 #pragma unroll
       for (int k = 0; k < VE; ++k) {
         // masked entries (re-read data of another vector or row) count as x = mean, dy = 0
+        const bool use = use_vec && !(kTail && k < skip[i]);
         const float gv = use ? gs[i][k] : 0.f;
         xh[i][k] = use ? (xh[i][k] - mean) * inv_stdev : 0.f;  // subtract first: x*inv - mean*inv would cancel
         if (WGRAD) {
@@ -534,7 +574,16 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
 #pragma unroll
           for (int k = 0; k < VE; ++k)
             gs[i][k] = __builtin_fmaf(gs[i][k], inv_stdev, __builtin_fmaf(c1, xh[i][k], c0));
-          IO::store(dr + voff[i], gs[i]);
+          bool whole = true;
+          if constexpr (kTail) {
+            if (skip[i]) {
+              whole = false;
+#pragma unroll
+              for (int k = 0; k < VE; ++k)
+                if (k >= skip[i]) IO::store1(dr + voff[i] + k, gs[i][k]);
+            }
+          }
+          if (whole) IO::store(dr + voff[i], gs[i]);
         }
       }
     }
@@ -546,7 +595,7 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   if constexpr (kPrefetch) issue(q, first_row);
   const int64_t full_iters = rows / rows_per_iter;
   int64_t it = 0;
-  if (nvec == TPR * V) {
+  if (nvec == TPR * V && !(kTail && tail)) {
     for (; it < full_iters; ++it) process(q, it, std::true_type{}, std::true_type{});
   }
   else {
@@ -900,8 +949,9 @@ static size_t ln_bwd_workspace(int64_t n, int64_t rows, int ve)
 template <typename ST>
 static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, int64_t ldy, RowMap map,
                               int64_t rows, int64_t units, float inv_n, float eps, float* stats, int64_t lds,
-                              const float* gamma, const float* beta, int sumsq)
+                              const float* gamma, const float* beta, int sumsq, int tail = 0)
 {
+  // tail: entries of a last, partial unit that `units` counts (storage types with unaligned access only)
   constexpr int VE = Vec16<ST>::N;
   RowConfig c = pick_row_config(units, rows, 8);
   // many short rows: teams of 16 lanes, four rows per wave, instead of mostly idle waves
@@ -928,7 +978,7 @@ static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, i
     const int64_t grid = ceil_div(work, ceil_div(work, resident));                             \
     hipLaunchKernelGGL((ln_fwd_rows<ST, TPR, V>), dim3(static_cast<unsigned>(grid)),           \
                        dim3(B::kThreads), 0, st, x, y, ldx, ldy, map, rows, nvec, inv_n, eps,  \
-                       stats, lds, gamma, beta, sumsq);                                        \
+                       stats, lds, gamma, beta, sumsq, tail);                                  \
     return 1;                                                                                  \
   }
   X(16, 1) X(16, 2)
@@ -1123,7 +1173,14 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     return launch_status();
   }
   if constexpr (std::is_same<T, __half>::value) {
-    // fp16 rows of odd length (or off the 4-byte grid): the same, eight entries per access at 2-byte alignment
+    // fp16 rows of odd length (or off the 4-byte grid): 16-byte accesses at 2-byte alignment, the last
+    // n % 8 entries in a vector that overlaps its neighbour; first the register kernels
+    if (n >= 8) {
+      if (int r = ln_fwd_rows_launch<f16u>(st, reinterpret_cast<const f16u*>(x), reinterpret_cast<f16u*>(y), ldx, ldy,
+                                           map, rows, ceil_div(n, 8), inv_n, eps, stats, lds, gamma, beta, sumsq,
+                                           static_cast<int>(n % 8)))
+        return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
+    }
     if (n >= kLnLongMin16) {
       hipLaunchKernelGGL((ln_fwd_long<f16u>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
                          reinterpret_cast<const f16u*>(x), reinterpret_cast<f16u*>(y), ldx, ldy, map, n / 8,
@@ -1141,14 +1198,18 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
                                T* dx, int64_t ldx, int64_t lddy, int64_t lddx, RowMap map,
                                int64_t rows, int nvec, int n, float eps, const float* stats,
                                int64_t lds, float* sgrad, int64_t ldsg, const float* gamma,
-                               float* part)
+                               float* part, int tail)
 {
   using B = RowBlock<TPR, TEAMS>;
   const dim3 grid(static_cast<unsigned>(blocks)), block(B::kThreads);
-  if (wgrad)
-    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, true>), grid, block, 0, st, x, dy, dx, ldx,
-                       lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part, nullptr, nullptr);
-  else {
+  if constexpr (!UnalignedVec<T>::value) {
+    if (wgrad) {
+      hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, true>), grid, block, 0, st, x, dy, dx, ldx,
+                         lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part, nullptr, nullptr);
+      return;
+    }
+  }
+  {
     // nothing to accumulate across rows: one resident wave of blocks, each walking the
     // same number of rows with the next row in flight
     const int64_t units = ceil_div(rows, TEAMS);
@@ -1156,24 +1217,28 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
     if (resident < 1) resident = 1;
     const dim3 all(static_cast<unsigned>(ceil_div(units, ceil_div(units, resident))));
     hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, false>), all, block, 0, st, x, dy, dx, ldx,
-                       lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part, nullptr, nullptr);
+                       lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part, nullptr, nullptr,
+                       tail);
   }
 }
 
 // Register-resident backward over rows of `units` access units, weight gradients included
 // (partial rows in the workspace, then the fixed-order reduction).  Returns 1 when launched,
 // 0 when no configuration holds the row, -1 when the workspace is missing or too small.
+// Storage types with unaligned access (tail: entries of a last, partial unit that `units`
+// counts) leave the weight gradients to the caller: wgrad is false for them.
 template <typename ST>
 static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST* dy, ST* dx, int64_t ldx,
                               int64_t lddy, int64_t lddx, RowMap map, int64_t rows, int64_t units, int64_t n,
                               int elem_bytes, float eps, const float* stats, int64_t lds, float* sgrad,
                               int64_t ldsg, const float* gamma, float* dgamma, float* dbeta, void* ws,
-                              size_t ws_bytes)
+                              size_t ws_bytes, int tail = 0)
 {
   constexpr int VE = Vec16<ST>::N;
+  if (UnalignedVec<ST>::value && wgrad) return 0;
   const LnBwdPlan p = plan_ln_bwd(units, rows, VE, elem_bytes);
   if (!p.tpr) return 0;
-  if constexpr (VE >= 4) {
+  if constexpr (VE >= 4 && !UnalignedVec<ST>::value) {
     if (wgrad && ln_bwd_small(rows, n, elem_bytes)) {
       // tensors that fit the caches: weight gradients from column slices, in the same kernel
       const int nvec_s = static_cast<int>(units);
@@ -1202,7 +1267,7 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
   if (!launched && p.tpr == TPR && p.teams == TEAMS && p.v == V) {                              \
     launch_ln_bwd_rows<ST, TPR, TEAMS, V>(st, wgrad, p.blocks, x, dy, dx, ldx, lddy, lddx, map, \
                                           rows, nvec, static_cast<int>(n), eps, stats, lds,     \
-                                          sgrad, ldsg, gamma, part);                            \
+                                          sgrad, ldsg, gamma, part, tail);                      \
     launched = true;                                                                            \
   }
   X(16, 16, 1) X(16, 16, 2)
@@ -1301,6 +1366,14 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                          reinterpret_cast<const f32u*>(x), reinterpret_cast<const f32u*>(dy),
                          reinterpret_cast<f32u*>(dx), ldx, lddy, lddx, map, n / 4, static_cast<int>(n % 4),
                          1.0f / static_cast<float>(n), eps, stats, lds, sgrad, ldsg, gamma);
+    else if (std::is_same<T, __half>::value && n >= 8 &&
+             ln_bwd_rows_launch<f16u>(st, false, reinterpret_cast<const f16u*>(x), reinterpret_cast<const f16u*>(dy),
+                                      reinterpret_cast<f16u*>(dx), ldx, lddy, lddx, map, rows, ceil_div(n, 8), n, 2, eps,
+                                      stats, lds, sgrad, ldsg, gamma, nullptr, nullptr, nullptr, 0,
+                                      static_cast<int>(n % 8)) == 1) {
+      // fp16 rows of odd length (or off the 4-byte grid) in registers: 16-byte accesses at 2-byte
+      // alignment; the weight gradients follow below
+    }
     else if (std::is_same<T, __half>::value && n >= kLnLongMin16)
       hipLaunchKernelGGL((ln_bwd_long<f16u>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
                          reinterpret_cast<const f16u*>(x), reinterpret_cast<const f16u*>(dy),
@@ -1326,6 +1399,13 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
         hipLaunchKernelGGL((ln_wgrad_columns<f32u, true>), ugrid, dim3(256), 0, st, reinterpret_cast<const f32u*>(x),
                            reinterpret_cast<const f32u*>(dy), ldx, lddy, map, rows, n / 4, n, eps, stats, lds, wpart,
                            static_cast<int>(n % 4));
+      }
+      else if (std::is_same<T, __half>::value && n >= 64) {
+        // fp16 rows off the 16-byte grid: 16-byte accesses at 2-byte alignment, the last n % 8 features apart
+        const dim3 ugrid(static_cast<unsigned>(ceil_div(n / 8 + 1, 256)), static_cast<unsigned>(slabs));
+        hipLaunchKernelGGL((ln_wgrad_columns<f16u, true>), ugrid, dim3(256), 0, st, reinterpret_cast<const f16u*>(x),
+                           reinterpret_cast<const f16u*>(dy), ldx, lddy, map, rows, n / 8, n, eps, stats, lds, wpart,
+                           static_cast<int>(n % 8));
       }
       else
         hipLaunchKernelGGL((ln_wgrad_columns<T, false>), grid, dim3(256), 0, st, x, dy, ldx, lddy, map, rows,

@@ -465,6 +465,29 @@ def test_layer_norm_f16(L, dims, start_dim, w, pad):
     _ln_run(L, x, dy, dims, start_dim, True, pad, scale, bias, tol=TOL_F16, half=True)
 
 
+@pytest.mark.parametrize("affine,mode", [(False, None), (True, None), (True, "sumsq")])
+@pytest.mark.parametrize("dims,start_dim,w,pad", [
+    ((9,), 0, 11, 0), ((15,), 0, 300, 0), ((17,), 0, 5000, 0), ((63,), 0, 40, 0), ((65,), 0, 4100, 0),
+    ((129,), 0, 33, 0), ((255,), 0, 4200, 0), ((257,), 0, 700, 0), ((511,), 0, 64, 0), ((1023,), 0, 9, 0),
+    ((1025,), 0, 70, 0), ((2047,), 0, 12, 0), ((2049,), 0, 300, 0), ((3001,), 0, 17, 0), ((4095,), 0, 5, 0),
+    ((4097,), 0, 40, 0), ((8191,), 0, 6, 0), ((16385,), 0, 7, 0), ((24001,), 0, 3, 0), ((32767,), 0, 4, 0),
+    ((6, 771), -1, 9, 0), ((3, 35), -1, 2000, 0),
+    # whole eights of entries behind odd leading dimensions: no partial vector, still unaligned
+    ((1024,), 0, 9, 1), ((64,), 0, 5000, 3), ((2048,), 0, 33, 5)])
+def test_layer_norm_f16_unaligned_rows(L, dims, start_dim, w, pad, affine, mode):
+    """fp16 rows that are not whole aligned vectors, in 16-byte accesses at 2-byte alignment: the row's
+    last n % 8 entries come from a vector that overlaps its neighbour."""
+    rng = np.random.default_rng(int(np.prod(dims)) * 11 + w + pad)
+    h = int(np.prod(dims))
+    x = rand(rng, h, w, 0.3, 1.5).astype(np.float16).astype(np.float32)
+    dy = rand(rng, h, w).astype(np.float16).astype(np.float32)
+    n = int(np.prod(dims[(start_dim if start_dim >= 0 else len(dims) + start_dim):]))
+    scale = (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(n)).astype(np.float32)
+    _ln_run(L, x, dy, dims, start_dim, affine, pad, scale, bias, tol=TOL_F16, half=True,
+            mode=L.LBN_STATS_SUMSQ if mode else None)
+
+
 # ===================================================================== instance norm
 @pytest.mark.parametrize("dims,w,pad", [((5, 3, 7), 15, 0), ((64, 56, 56), 6, 0), ((8, 1024), 33, 0),
                                         ((2, 1048576), 2, 0), ((4, 96, 96, 96), 3, 0),   # volumes: clusters of workgroups per channel
