@@ -141,6 +141,13 @@ template <>
 struct Vec16<f32u> {
   static constexpr int N = 4;
   using raw_t = v4f;
+  static __device__ __forceinline__ raw_t load_raw(const f32u* p)
+  {
+    v4f r;
+    __builtin_memcpy(&r, p, 16);
+    return r;
+  }
+  static __device__ __forceinline__ void unpack(const raw_t& r, float (&v)[4]) { Vec16<float>::unpack(r, v); }
   static __device__ __forceinline__ void load(const f32u* p, float (&v)[4]) { __builtin_memcpy(v, p, 16); }
   static __device__ __forceinline__ void store(f32u* p, const float (&v)[4]) { __builtin_memcpy(p, v, 16); }
   static __device__ __forceinline__ float load1(const f32u* p) { return p->v; }

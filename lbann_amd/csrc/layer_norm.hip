@@ -15,11 +15,15 @@
 //    teams of a block merge through LDS, every block leaves one partial row in the
 //    workspace, and a second small kernel sums the partial rows in a fixed order:
 //    no atomics, bitwise reproducible.
-//  * fp32 rows off the 16-byte grid (odd lengths or leading dimensions) run the same
-//    register kernels on a storage type that is accessed one float at a time (f32x1).
+//  * rows off the 16-byte grid (odd lengths or leading dimensions) run the same register
+//    kernels on other storage types: one float (f32x1) or one pair of halves (f16x2) per
+//    access, or 16-byte accesses at the alignment of one entry (f32u, f16u), where the row's
+//    last, partial vector is read as its last whole 16 bytes and the entries it shares with
+//    its neighbour are masked out.  Which one serves a shape is measured, not derived:
+//    ln_pairs_first, ln_vectors_first.
 //  * rows longer than the register kernels hold: layer_norm_long.hpp.
 //  * generic kernels (one 256-thread block per row, scalar access) cover what is left
-//    (fp16 rows that are not a multiple of 8 long, very long unaligned rows).
+//    (rows of fewer than 4 floats or 8 halves off the grid).
 #include <type_traits>
 
 #include "device_utils.hpp"
@@ -433,7 +437,7 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   constexpr int VE = IO::N;
   // a last vector of `tail` entries, read as the row's last VE entries: see ln_fwd_rows
   constexpr bool kTail = UnalignedVec<T>::value;
-  static_assert(!kTail || !(WGRAD || COLS), "rows with a partial vector leave the weight gradients to another kernel");
+  static_assert(!kTail || !COLS, "rows with a partial vector do not form weight gradients from column slices");
   constexpr bool kSub = TPR < kWave;
   static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
   constexpr int NW = kSub ? 1 : B::kWavesPerTeam;
@@ -630,7 +634,9 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
           for (int i = 0; i < V; ++i)
 #pragma unroll
             for (int k = 0; k < VE; ++k) {
-              const int p = (t + i * TPR) * VE + k;
+              // (a vector past the end of the row keeps a slot of its own behind the row's entries)
+              const int p = (kTail && ok[i]) ? voff[i] + k : (t + i * TPR) * VE + k;
+              if (kTail && k < skip[i]) continue;  // the neighbour's entry
               if (tm == 0) {
                 lg[p] = dg[i][k];
                 lb[p] = db[i][k];
@@ -651,10 +657,24 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
     else {
 #pragma unroll
       for (int i = 0; i < V; ++i) {
-        const int idx = t + i * TPR;
-        if (idx < nvec) {
-          store_f32_run<VE>(out + VE * idx, dg[i]);
-          store_f32_run<VE>(out + n + VE * idx, db[i]);
+        if (!ok[i]) continue;
+        if constexpr (kTail) {
+          if (skip[i]) {
+#pragma unroll
+            for (int k = 0; k < VE; ++k)
+              if (k >= skip[i]) {
+                out[voff[i] + k] = dg[i][k];
+                out[n + voff[i] + k] = db[i][k];
+              }
+          }
+          else {
+            __builtin_memcpy(out + voff[i], dg[i], sizeof(float) * VE);
+            __builtin_memcpy(out + n + voff[i], db[i], sizeof(float) * VE);
+          }
+        }
+        else {
+          store_f32_run<VE>(out + voff[i], dg[i]);
+          store_f32_run<VE>(out + n + voff[i], db[i]);
         }
       }
     }
@@ -884,6 +904,49 @@ static bool rows_aligned4(const void* base, int64_t stride, int64_t ld, int64_t 
          (width <= 1 || ld % 2 == 0);
 }
 
+// LBN_LN_NO_UNALIGNED_ROWS=1 keeps rows off the 16-byte grid away from the register kernels
+// with unaligned 16-byte accesses: single floats, pairs of halves, the two-pass kernels and
+// the generic kernels serve them instead (for tests of those paths).
+static bool ln_no_unaligned_rows()
+{
+  static const bool on = std::getenv("LBN_LN_NO_UNALIGNED_ROWS") != nullptr;
+  return on;
+}
+
+// fp16 rows of even length on the 4-byte grid can be walked in pairs or in 16-byte vectors at
+// 2-byte alignment.  Pairs give a short row more loads in flight per lane (258 x 65536 forward:
+// 22 against 28 us) and are kept up to 512 entries and wherever weights have gradients (1002 x
+// 16384 backward: 28 against 33 us); longer rows take the vectors (2050 x 8192 forward: 22
+// against 45 us), and so do rows of 65 to 256 entries when there are many: 32 vectors hold them,
+// a team of 16 lanes each (130 x 131072: 22 / 23 us against 32 / 37).
+constexpr int64_t kLnPairsMaxFwd16 = 512;
+
+static bool ln_pairs_first(int64_t n, int64_t rows)
+{
+  if (ln_no_unaligned_rows()) return true;
+  return n <= kLnPairsMaxFwd16 && !(n > 64 && n <= 256 && rows >= 4096);
+}
+
+// With weight gradients the pairs stay, except where 16 vectors hold one of many rows
+// (66 x 262144 backward: 46 against 78 us; 130 x 131072: 62 against 52 us).
+static bool ln_pairs_first_wgrad(int64_t n, int64_t rows)
+{
+  if (ln_no_unaligned_rows()) return true;
+  return !(n > 64 && n <= 128 && rows >= 4096);
+}
+
+// fp32 rows off the 16-byte grid can be walked one float at a time or in 16-byte vectors at
+// 4-byte alignment (the last n % 4 entries in a vector that overlaps its neighbour).  Vectors
+// win where 32 of them hold a row (teams of 16 lanes; 35 x 262144: 20 / 22 us against 49 / 62)
+// and beyond `longer_than` entries (2049 x 8192 forward: 26 against 47 us; 1025 x 16384
+// backward with weight gradients: 43 against 53 us); between, single floats are as fast or
+// a little faster (1001 x 16384 backward: 32 against 34 us).
+static bool ln_vectors_first(int64_t n, int64_t longer_than, int64_t rows)
+{
+  if (n < 4 || ln_no_unaligned_rows()) return false;
+  return (ceil_div(n, 4) <= 32 && rows >= 4096) || n > longer_than;
+}
+
 constexpr int64_t kLnLongMin16 = 4096;  // shortest fp16 row of odd length that takes a 1024-thread workgroup of its own (1001 entries: 75 against 40 us)
 constexpr int64_t kLnMaxScalarRowFwd = 8192;  // rows accessed one float at a time: 1024 threads x 8
 constexpr int64_t kLnMaxScalarRowBwd = 4096;  // 512 threads x 8
@@ -934,6 +997,10 @@ static size_t ln_bwd_workspace(int64_t n, int64_t rows, int ve)
   }
   if (ve == 4 && n <= kLnMaxScalarRowBwd) {  // fp32 rows off the 16-byte grid: one float per access
     const LnBwdPlan p = plan_ln_bwd(n, rows, 1, 4);
+    if (p.tpr) cover(H + static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
+  }
+  if (n >= ve) {  // rows off the 16-byte grid: a last, partial vector counts as a unit
+    const LnBwdPlan p = plan_ln_bwd(ceil_div(n, ve), rows, ve, elem_bytes);
     if (p.tpr) cover(H + static_cast<size_t>(p.blocks) * 2 * n * sizeof(float));
   }
   if (ve == 8 && n % 2 == 0 && n / 2 <= kLnMaxScalarRowBwd) {  // fp16 rows: one pair per access
@@ -1149,7 +1216,7 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
   }
   if constexpr (std::is_same<T, __half>::value) {
     // fp16 rows off the 16-byte grid with an even length: the same kernels, one pair per access
-    if (n % 2 == 0 && n / 2 <= kLnMaxScalarRowFwd && rows_aligned4(x, stride, ldx, G, w) &&
+    if (n % 2 == 0 && ln_pairs_first(n, rows) && rows_aligned4(x, stride, ldx, G, w) &&
         rows_aligned4(y, stride, ldy, G, w)) {
       if (int r = ln_fwd_rows_launch<f16x2>(st, reinterpret_cast<const f16x2*>(x), reinterpret_cast<f16x2*>(y),
                                             ldx, ldy, map, rows, n / 2, inv_n, eps, stats,
@@ -1158,15 +1225,21 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     }
   }
   if constexpr (std::is_same<T, float>::value) {
-    if (n > 1 && n <= kLnMaxScalarRowFwd) {  // rows off the 16-byte grid: the same kernels, one float per access
+    if (n > 1 && n <= kLnMaxScalarRowFwd && !ln_vectors_first(n, 2048, rows)) {  // rows off the 16-byte grid: the same kernels, one float per access
       if (int r = ln_fwd_rows_launch<f32x1>(st, reinterpret_cast<const f32x1*>(x), reinterpret_cast<f32x1*>(y),
                                             ldx, ldy, map, rows, n, inv_n, eps, stats, lds, gamma, beta, sumsq))
         return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
     }
   }
   if constexpr (std::is_same<T, float>::value) {
-    // fp32 rows off the 16-byte grid beyond the register kernels: two passes of 16-byte accesses
-    // at 4-byte alignment, the last n % 4 entries apart
+    // longer fp32 rows off the 16-byte grid: 16-byte accesses at 4-byte alignment, the last n % 4
+    // entries in a vector that overlaps its neighbour; first the register kernels, then two passes
+    if (!ln_no_unaligned_rows()) {
+      if (int r = ln_fwd_rows_launch<f32u>(st, reinterpret_cast<const f32u*>(x), reinterpret_cast<f32u*>(y), ldx, ldy,
+                                           map, rows, ceil_div(n, 4), inv_n, eps, stats, lds, gamma, beta, sumsq,
+                                           static_cast<int>(n % 4)))
+        return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
+    }
     hipLaunchKernelGGL((ln_fwd_long<f32u>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
                        reinterpret_cast<const f32u*>(x), reinterpret_cast<f32u*>(y), ldx, ldy, map, n / 4,
                        static_cast<int>(n % 4), inv_n, eps, stats, lds, gamma, beta, sumsq);
@@ -1175,7 +1248,7 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
   if constexpr (std::is_same<T, __half>::value) {
     // fp16 rows of odd length (or off the 4-byte grid): 16-byte accesses at 2-byte alignment, the last
     // n % 8 entries in a vector that overlaps its neighbour; first the register kernels
-    if (n >= 8) {
+    if (n >= 8 && !ln_no_unaligned_rows()) {
       if (int r = ln_fwd_rows_launch<f16u>(st, reinterpret_cast<const f16u*>(x), reinterpret_cast<f16u*>(y), ldx, ldy,
                                            map, rows, ceil_div(n, 8), inv_n, eps, stats, lds, gamma, beta, sumsq,
                                            static_cast<int>(n % 8)))
@@ -1202,14 +1275,11 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
 {
   using B = RowBlock<TPR, TEAMS>;
   const dim3 grid(static_cast<unsigned>(blocks)), block(B::kThreads);
-  if constexpr (!UnalignedVec<T>::value) {
-    if (wgrad) {
-      hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, true>), grid, block, 0, st, x, dy, dx, ldx,
-                         lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part, nullptr, nullptr);
-      return;
-    }
-  }
-  {
+  if (wgrad)
+    hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, true>), grid, block, 0, st, x, dy, dx, ldx,
+                       lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part, nullptr, nullptr,
+                       tail);
+  else {
     // nothing to accumulate across rows: one resident wave of blocks, each walking the
     // same number of rows with the next row in flight
     const int64_t units = ceil_div(rows, TEAMS);
@@ -1225,8 +1295,7 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
 // Register-resident backward over rows of `units` access units, weight gradients included
 // (partial rows in the workspace, then the fixed-order reduction).  Returns 1 when launched,
 // 0 when no configuration holds the row, -1 when the workspace is missing or too small.
-// Storage types with unaligned access (tail: entries of a last, partial unit that `units`
-// counts) leave the weight gradients to the caller: wgrad is false for them.
+// tail: entries of a last, partial unit that `units` counts (storage types with unaligned access only).
 template <typename ST>
 static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST* dy, ST* dx, int64_t ldx,
                               int64_t lddy, int64_t lddx, RowMap map, int64_t rows, int64_t units, int64_t n,
@@ -1235,7 +1304,6 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
                               size_t ws_bytes, int tail = 0)
 {
   constexpr int VE = Vec16<ST>::N;
-  if (UnalignedVec<ST>::value && wgrad) return 0;
   const LnBwdPlan p = plan_ln_bwd(units, rows, VE, elem_bytes);
   if (!p.tpr) return 0;
   if constexpr (VE >= 4 && !UnalignedVec<ST>::value) {
@@ -1343,7 +1411,7 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
   }
   else {
     if constexpr (std::is_same<T, __half>::value) {
-      if (n % 2 == 0 && n / 2 <= kLnMaxScalarRowBwd && rows_aligned4(x, stride, ldx, G, w) &&
+      if (n % 2 == 0 && n / 2 <= kLnMaxScalarRowBwd && (wgrad ? ln_pairs_first_wgrad(n, rows) : ln_pairs_first(n, rows)) && rows_aligned4(x, stride, ldx, G, w) &&
           rows_aligned4(dy, stride, lddy, G, w) && rows_aligned4(dx, stride, lddx, G, w)) {
         if (int r = ln_bwd_rows_launch<f16x2>(st, wgrad, reinterpret_cast<const f16x2*>(x),
                                               reinterpret_cast<const f16x2*>(dy), reinterpret_cast<f16x2*>(dx),
@@ -1352,12 +1420,32 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
           return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
       }
     }
+    if constexpr (std::is_same<T, __half>::value) {
+      // fp16 rows of odd length (or off the 4-byte grid) in registers: 16-byte accesses at 2-byte
+      // alignment, the last n % 8 entries in a vector that overlaps its neighbour
+      if (n >= 8 && !ln_no_unaligned_rows()) {
+        if (int r = ln_bwd_rows_launch<f16u>(st, wgrad, reinterpret_cast<const f16u*>(x),
+                                             reinterpret_cast<const f16u*>(dy), reinterpret_cast<f16u*>(dx), ldx,
+                                             lddy, lddx, map, rows, ceil_div(n, 8), n, 2, eps, stats, lds, sgrad, ldsg,
+                                             gamma, dgamma, dbeta, ws, ws_bytes, static_cast<int>(n % 8)))
+          return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
+      }
+    }
     if constexpr (std::is_same<T, float>::value) {
-      if (n <= kLnMaxScalarRowBwd) {  // rows off the 16-byte grid: the same kernels, one float per access
+      if (n <= kLnMaxScalarRowBwd && !ln_vectors_first(n, 1024, rows)) {  // rows off the 16-byte grid: the same kernels, one float per access
         if (int r = ln_bwd_rows_launch<f32x1>(st, wgrad, reinterpret_cast<const f32x1*>(x),
                                               reinterpret_cast<const f32x1*>(dy), reinterpret_cast<f32x1*>(dx), ldx,
                                               lddy, lddx, map, rows, n, n, 4, eps, stats, lds, sgrad, ldsg, gamma,
                                               dgamma, dbeta, ws, ws_bytes))
+          return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
+      }
+    }
+    if constexpr (std::is_same<T, float>::value) {
+      if (!ln_no_unaligned_rows()) {
+        if (int r = ln_bwd_rows_launch<f32u>(st, wgrad, reinterpret_cast<const f32u*>(x),
+                                             reinterpret_cast<const f32u*>(dy), reinterpret_cast<f32u*>(dx), ldx,
+                                             lddy, lddx, map, rows, ceil_div(n, 4), n, 4, eps, stats, lds, sgrad, ldsg,
+                                             gamma, dgamma, dbeta, ws, ws_bytes, static_cast<int>(n % 4)))
           return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
       }
     }
@@ -1366,14 +1454,6 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                          reinterpret_cast<const f32u*>(x), reinterpret_cast<const f32u*>(dy),
                          reinterpret_cast<f32u*>(dx), ldx, lddy, lddx, map, n / 4, static_cast<int>(n % 4),
                          1.0f / static_cast<float>(n), eps, stats, lds, sgrad, ldsg, gamma);
-    else if (std::is_same<T, __half>::value && n >= 8 &&
-             ln_bwd_rows_launch<f16u>(st, false, reinterpret_cast<const f16u*>(x), reinterpret_cast<const f16u*>(dy),
-                                      reinterpret_cast<f16u*>(dx), ldx, lddy, lddx, map, rows, ceil_div(n, 8), n, 2, eps,
-                                      stats, lds, sgrad, ldsg, gamma, nullptr, nullptr, nullptr, 0,
-                                      static_cast<int>(n % 8)) == 1) {
-      // fp16 rows of odd length (or off the 4-byte grid) in registers: 16-byte accesses at 2-byte
-      // alignment; the weight gradients follow below
-    }
     else if (std::is_same<T, __half>::value && n >= kLnLongMin16)
       hipLaunchKernelGGL((ln_bwd_long<f16u>), dim3(static_cast<unsigned>(rows)), dim3(kLongThreads), 0, st,
                          reinterpret_cast<const f16u*>(x), reinterpret_cast<const f16u*>(dy),

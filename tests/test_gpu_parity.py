@@ -450,7 +450,7 @@ def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
                                                    ((4100,), 0, 40, 0), ((1002,), 0, 33, 0), ((6, 770), -1, 9, 0),
                                                    ((8190,), 0, 5, 2), ((16382,), 0, 3, 0), ((4100, 12), -1, 2, 0),
                                                    ((1001,), 0, 7, 0), ((4099,), 0, 9, 0), ((10001,), 0, 5, 1), ((513,), 0, 40, 0),   # odd: eight entries per access at 2-byte alignment
-                                                   ((50003,), 0, 3, 0), ((20002,), 0, 4, 1), ((301,), 0, 20, 0),   # (below 4096 entries: scalar fallback)
+                                                   ((50003,), 0, 3, 0), ((20002,), 0, 4, 1), ((301,), 0, 20, 0),
                                                    # long rows shared by clusters of workgroups
                                                    ((802816,), 0, 4, 0), ((65536,), 0, 150, 0), ((2, 100000), -1, 20, 8),
                                                    ((1048576,), 0, 2, 0), ((5000000,), 0, 2, 0)])
@@ -486,6 +486,26 @@ def test_layer_norm_f16_unaligned_rows(L, dims, start_dim, w, pad, affine, mode)
     bias = (0.1 * rng.standard_normal(n)).astype(np.float32)
     _ln_run(L, x, dy, dims, start_dim, affine, pad, scale, bias, tol=TOL_F16, half=True,
             mode=L.LBN_STATS_SUMSQ if mode else None)
+
+
+@pytest.mark.parametrize("affine,mode", [(False, None), (True, None), (True, "sumsq")])
+@pytest.mark.parametrize("dims,start_dim,w,pad", [
+    ((5,), 0, 4100, 0), ((7,), 0, 9000, 1), ((35,), 0, 5000, 0), ((127,), 0, 4200, 0), ((126,), 0, 4100, 1),
+    ((2049,), 0, 70, 0), ((3001,), 0, 9, 0), ((4099,), 0, 33, 0), ((8191,), 0, 6, 0), ((10001,), 0, 12, 0),
+    ((12290,), 0, 5, 0), ((16383,), 0, 3, 0), ((16385,), 0, 3, 0), ((30001,), 0, 4, 0), ((32769,), 0, 2, 0),
+    ((3, 2731), -1, 9, 0), ((4, 33), -1, 1500, 0),
+    # whole fours of entries behind leading dimensions that are not: no partial vector, still unaligned
+    ((4096,), 0, 9, 1), ((64,), 0, 5000, 3), ((12288,), 0, 7, 2)])
+def test_layer_norm_f32_unaligned_rows(L, dims, start_dim, w, pad, affine, mode):
+    """fp32 rows that are not whole aligned vectors, in 16-byte accesses at 4-byte alignment: the row's
+    last n % 4 entries come from a vector that overlaps its neighbour."""
+    rng = np.random.default_rng(int(np.prod(dims)) * 13 + w + pad)
+    h = int(np.prod(dims))
+    x, dy = rand(rng, h, w, 0.3, 1.5), rand(rng, h, w)
+    n = int(np.prod(dims[(start_dim if start_dim >= 0 else len(dims) + start_dim):]))
+    scale = (1 + 0.3 * rng.standard_normal(n)).astype(np.float32)
+    bias = (0.3 * rng.standard_normal(n)).astype(np.float32)
+    _ln_run(L, x, dy, dims, start_dim, affine, pad, scale, bias, mode=L.LBN_STATS_SUMSQ if mode else None)
 
 
 # ===================================================================== instance norm
