@@ -306,6 +306,76 @@ static bool sm_bwd_framed_rows(hipStream_t st, int64_t n, int64_t w, int64_t row
   }
 }
 
+// 16-bit rows off the 16-byte grid (odd lengths or leading dimensions, any row stride) that fit a
+// workgroup's registers: the row kernels on 16-byte accesses at 2-byte alignment.  False: not
+// launched (LBN_NO_UNALIGNED_ROWS=1 keeps the paths that served these rows before, for tests).
+// Measured against what served them before (one half per access up to 2047 entries, the packed
+// two-pass kernel from there), us forward / backward: 257 x 65536: 32 / 26 -> 20 / 20; 1025 x
+// 16384: 34 / 26 -> 19 / 19; 2049 x 8192: 39 / 33 -> 21 / 19; 4097 x 4096: 25 / 21 -> 19 / 19;
+// 30522 x 2048 forward: 51 -> 46.  Not taken: rows of up to 64 entries, which single halves
+// spread over all 16 lanes of a team (21 x 1048576: 45 / 41 against 76 / 56), and rows that
+// leave a thread more than four vectors per tensor (50257 x 1024 backward: 133 against 74).
+constexpr int64_t kUnalignedRowMin = 65;
+constexpr int64_t kUnalignedRowMaxFwd = 32768;
+constexpr int64_t kUnalignedRowMaxBwd = 16384;
+static bool unaligned_rows()
+{
+  static const bool off = std::getenv("LBN_NO_UNALIGNED_ROWS") != nullptr;
+  return !off;
+}
+
+template <int KIND, typename S>
+static bool sm_fwd_unaligned_rows(hipStream_t st, int64_t n, int64_t rows, const S* x, int64_t ldx, S* y, int64_t ldy,
+                                  RowMap map)
+{
+  if constexpr (sizeof(S) != 2) {
+    return false;
+  }
+  else {
+    constexpr int W = 8;
+    if (!unaligned_rows() || n < kUnalignedRowMin || n > kUnalignedRowMaxFwd) return false;
+    const RowConfig c = pick_sm_row_config(ceil_div(n, W), rows);
+    if (!c.tpr) return false;
+#define X(TPR, V)                                                                                       \
+  if (c.tpr == TPR && c.v == V) {                                                                       \
+    using B = RowBlock<TPR>;                                                                            \
+    const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                             \
+    hipLaunchKernelGGL((sm_fwd_rows<S, TPR, V, KIND, false, W, false, true>), dim3(grid), dim3(B::kThreads), 0, st, \
+                       x, y, ldx, ldy, map, rows, static_cast<unsigned>(n));                            \
+    return true;                                                                                        \
+  }
+    LBN_ROW_CASES(X)
+#undef X
+    return false;
+  }
+}
+
+template <int KIND, typename S>
+static bool sm_bwd_unaligned_rows(hipStream_t st, int64_t n, int64_t rows, const S* y, int64_t ldy, const S* dy,
+                                  int64_t lddy, S* dx, int64_t lddx, RowMap map)
+{
+  if constexpr (sizeof(S) != 2) {
+    return false;
+  }
+  else {
+    constexpr int W = 8;
+    if (!unaligned_rows() || n < kUnalignedRowMin || n > kUnalignedRowMaxBwd) return false;
+    const RowConfig c = pick_sm_row_config(ceil_div(n, W), rows);
+    if (!c.tpr) return false;
+#define X(TPR, V)                                                                                       \
+  if (c.tpr == TPR && c.v == V) {                                                                       \
+    using B = RowBlock<TPR>;                                                                            \
+    const unsigned grid = static_cast<unsigned>(ceil_div(rows, B::kTeams));                             \
+    hipLaunchKernelGGL((sm_bwd_rows<S, TPR, V, KIND, 0, W, false, true>), dim3(grid), dim3(B::kThreads), 0, st, \
+                       y, dy, dx, ldy, lddy, lddx, map, rows, static_cast<unsigned>(n));                \
+    return true;                                                                                        \
+  }
+    LBN_ROW_CASES(X)
+#undef X
+    return false;
+  }
+}
+
 // The walking forward kernel for 16-bit rows of four vectors per thread, when the rows need
 // more than one workgroup per compute unit.
 template <int KIND, typename S>
@@ -360,6 +430,9 @@ static int sm_fwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     }
   }
   else if (sm_fwd_framed_rows<KIND>(st, n, w, rows, x, ldx, y, ldy, map)) {
+    return launch_status();
+  }
+  else if (sm_fwd_unaligned_rows<KIND>(st, n, rows, x, ldx, y, ldy, map)) {
     return launch_status();
   }
   else if (sizeof(S) == 2 && n >= packed_long_min16() && groups == 1 && same_frames16(x, ldx, y, ldy, w) &&
@@ -538,6 +611,9 @@ static int sm_bwd(hipStream_t st, int64_t groups, int64_t n, int64_t stride, int
     }
   }
   else if (sm_bwd_framed_rows<KIND>(st, n, w, rows, y, ldy, dy, lddy, dx, lddx, map)) {
+    return launch_status();
+  }
+  else if (sm_bwd_unaligned_rows<KIND>(st, n, rows, y, ldy, dy, lddy, dx, lddx, map)) {
     return launch_status();
   }
   else if (sizeof(S) == 2 && n >= packed_long_min16() && groups == 1 && same_frames16(y, ldy, dy, lddy, w) &&

@@ -60,6 +60,22 @@ struct RowIO<__half, 1> {
   static __device__ __forceinline__ void store(__half* p, const float (&v)[1]) { *p = __float2half_rn(v[0]); }
 };
 
+// 16-byte accesses at the alignment of one entry (rows off the 16-byte grid); the hardware
+// takes them at 93-95 % of the aligned rate.
+template <typename S, int W>
+struct RowIOUnaligned;
+template <>
+struct RowIOUnaligned<__half, 8> {
+  static __device__ __forceinline__ void load(const __half* p, float (&v)[8])
+  {
+    Vec16<f16u>::load(reinterpret_cast<const f16u*>(p), v);
+  }
+  static __device__ __forceinline__ void store(__half* p, const float (&v)[8])
+  {
+    Vec16<f16u>::store(reinterpret_cast<f16u*>(p), v);
+  }
+};
+
 template <typename S>
 struct RowLoad {
   static __device__ __forceinline__ float get(const S* p) { float v[1]; RowIO<S, 1>::template load<false>(p, v); return v[0]; }
@@ -112,12 +128,17 @@ __device__ __forceinline__ void frame_store(float* framep, unsigned idx, RowFram
 // 1024-thread blocks are held to 64 registers so that two of them share a compute unit
 // (not those with 32 accesses or more than 32 values per thread, which would spill).
 // FR (fp32): framed access for rows off the 16-byte grid; `nvec` is then the row length in entries.
-template <typename S, int TPR, int V, int KIND, bool STREAM, int W = 16 / sizeof(S), bool FR = false>
+// UA (16-bit storage): rows off the 16-byte grid in 16-byte accesses at 2-byte alignment; `nvec` is
+// the row length in entries (at least W).  A last, partial vector is read as the row's last W
+// entries, so it overlaps its neighbour: the entries the two share count as absent in the partial
+// vector and are stored by the neighbour only.
+template <typename S, int TPR, int V, int KIND, bool STREAM, int W = 16 / sizeof(S), bool FR = false, bool UA = false>
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads, (TPR == 1024 && V <= 16 && V * W <= 32 ? 8 : 1))
 sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows,
             unsigned nvec)
 {
   static_assert(!FR || (std::is_same<S, float>::value && W == 4), "frames are made of 16-byte fp32 vectors");
+  static_assert(!UA || (!FR && W == 16 / sizeof(S)), "unaligned access moves whole 16-byte vectors");
   using B = RowBlock<TPR>;
   constexpr bool kSub = TPR < kWave;  // short rows: 16 lanes own a row, four rows per wave
   static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
@@ -140,12 +161,27 @@ sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows
     xr -= fr.shift;
     nvec = fr.nvec;
   }
+  unsigned ua_skip = 0;  // UA: leading entries of the last vector that belong to its neighbour
+  if constexpr (UA) {
+    nvec = (n + W - 1) / W;
+    ua_skip = nvec * W - n;
+  }
+  // entry offset of vector idx, and how many of its leading entries are not its own
+  auto ua_off = [&](unsigned idx) { return (UA && idx == nvec - 1) ? n - W : unsigned(W) * idx; };
+  auto ua_foreign = [&](unsigned idx) { return (UA && idx == nvec - 1) ? ua_skip : 0u; };
   float v[V][W];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const unsigned idx = t + i * TPR;
     if (idx < nvec) {
       if constexpr (FR) frame_load(xr, idx, fr, n, -FLT_MAX, v[i]);
+      else if constexpr (UA) {
+        RowIOUnaligned<S, W>::load(xr + ua_off(idx), v[i]);
+        const unsigned foreign = ua_foreign(idx);
+#pragma unroll
+        for (int k = 0; k < W; ++k)
+          if (unsigned(k) < foreign) v[i][k] = -FLT_MAX;
+      }
       else RowIO<S, W>::template load<STREAM>(xr + unsigned(W) * idx, v[i]);
     }
     else {
@@ -167,9 +203,11 @@ sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    const bool ok = (t + i * TPR) < nvec;
+    const bool in_row = (t + i * TPR) < nvec;
+    const unsigned foreign = ua_foreign(t + i * TPR);
 #pragma unroll
     for (int k = 0; k < W; ++k) {
+      const bool ok = in_row && !(UA && unsigned(k) < foreign);
       const float d = v[i][k] - m;
       float e;
       if (KIND == kLogSoftmax) e = exp_quick(d);  // only summed: x stays in the registers for the output
@@ -223,6 +261,17 @@ sm_fwd_rows(const S* x, S* y, int64_t ldx, int64_t ldy, RowMap map, int64_t rows
         }
       }
       if constexpr (FR) frame_store(yr, idx, fr, n, v[i]);
+      else if constexpr (UA) {
+        const unsigned foreign = ua_foreign(idx);
+        if (foreign) {
+#pragma unroll
+          for (int k = 0; k < W; ++k)
+            if (unsigned(k) >= foreign) RowLoad<S>::put(yr + ua_off(idx) + k, v[i][k]);
+        }
+        else {
+          RowIOUnaligned<S, W>::store(yr + ua_off(idx), v[i]);
+        }
+      }
       else RowIO<S, W>::store(yr + unsigned(W) * idx, v[i]);
     }
   }
@@ -514,13 +563,14 @@ sm_ce_bwd_rows(const float* y, const float* truth, const float* dloss, float* dx
 }
 
 // softmax / channelwise: dx = y * (dy - dot(y, dy));  log-softmax: dx = dy - exp(y) * sum(dy)
-// STREAM: bit 0 streams y, bit 1 dy.  FR as in sm_fwd_rows.
-template <typename S, int TPR, int V, int KIND, int STREAM, int W = 16 / sizeof(S), bool FR = false>
+// STREAM: bit 0 streams y, bit 1 dy.  FR and UA as in sm_fwd_rows.
+template <typename S, int TPR, int V, int KIND, int STREAM, int W = 16 / sizeof(S), bool FR = false, bool UA = false>
 __global__ void __launch_bounds__(RowBlock<TPR>::kThreads)
 sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx,
             RowMap map, int64_t rows, unsigned nvec)
 {
   static_assert(!FR || (std::is_same<S, float>::value && W == 4), "frames are made of 16-byte fp32 vectors");
+  static_assert(!UA || (!FR && W == 16 / sizeof(S)), "unaligned access moves whole 16-byte vectors");
   using B = RowBlock<TPR>;
   constexpr bool kSub = TPR < kWave;
   static_assert(!kSub || TPR == 16, "sub-wave teams are one DPP row wide");
@@ -544,6 +594,13 @@ sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t l
     gr -= fr.shift;
     nvec = fr.nvec;
   }
+  unsigned ua_skip = 0;
+  if constexpr (UA) {
+    nvec = (n + W - 1) / W;
+    ua_skip = nvec * W - n;
+  }
+  auto ua_off = [&](unsigned idx) { return (UA && idx == nvec - 1) ? n - W : unsigned(W) * idx; };
+  auto ua_foreign = [&](unsigned idx) { return (UA && idx == nvec - 1) ? ua_skip : 0u; };
   float a[V][W], g[V][W];
 #pragma unroll
   for (int i = 0; i < V; ++i) {
@@ -552,6 +609,14 @@ sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t l
       if constexpr (FR) {
         frame_load(yr, idx, fr, n, 0.f, a[i]);
         frame_load(gr, idx, fr, n, 0.f, g[i]);
+      }
+      else if constexpr (UA) {
+        RowIOUnaligned<S, W>::load(yr + ua_off(idx), a[i]);
+        RowIOUnaligned<S, W>::load(gr + ua_off(idx), g[i]);
+        const unsigned foreign = ua_foreign(idx);
+#pragma unroll
+        for (int k = 0; k < W; ++k)
+          if (unsigned(k) < foreign) g[i][k] = 0.f;  // no share in the row sum (y is finite)
       }
       else {
         RowIO<S, W>::template load<(STREAM & 1) != 0>(yr + unsigned(W) * idx, a[i]);
@@ -583,6 +648,17 @@ sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t l
         else g[i][k] = a[i][k] * (g[i][k] - s);
       }
       if constexpr (FR) frame_store(dr, idx, fr, n, g[i]);
+      else if constexpr (UA) {
+        const unsigned foreign = ua_foreign(idx);
+        if (foreign) {
+#pragma unroll
+          for (int k = 0; k < W; ++k)
+            if (unsigned(k) >= foreign) RowLoad<S>::put(dr + ua_off(idx) + k, g[i][k]);
+        }
+        else {
+          RowIOUnaligned<S, W>::store(dr + ua_off(idx), g[i]);
+        }
+      }
       else RowIO<S, W>::store(dr + unsigned(W) * idx, g[i]);
     }
   }

@@ -113,6 +113,57 @@ def test_softmax_family_f16_storage(L, kind, h, w, pad, in_place):
         assert np.abs(y.astype(np.float64).sum(axis=0) - 1).max() < 2e-3 * np.sqrt(h)
 
 
+@pytest.mark.parametrize("kind", ["softmax", "log_softmax"])
+@pytest.mark.parametrize("h,w,pad", [
+    (9, 50, 0), (15, 5000, 0), (17, 4100, 1), (63, 40, 0), (65, 4200, 0), (129, 33, 0), (255, 5000, 0), (257, 700, 0),
+    (511, 64, 3), (513, 4100, 0), (1023, 9, 0), (1025, 70, 0), (2047, 12, 0), (2049, 300, 0), (3001, 17, 0),
+    (4095, 5, 0), (4097, 40, 0), (8191, 6, 0), (16385, 7, 0), (24001, 3, 0), (32767, 4, 0), (50001, 3, 0),
+    # whole eights of entries behind odd leading dimensions: no partial vector, still unaligned
+    (1024, 9, 1), (64, 5000, 3), (2048, 33, 5), (16, 4100, 1)])
+def test_softmax_family_f16_unaligned_rows(L, kind, h, w, pad):
+    """fp16 rows that are not whole aligned vectors, in 16-byte accesses at 2-byte alignment: the row's
+    last h % 8 entries come from a vector that overlaps its neighbour."""
+    rng = np.random.default_rng(7 * h + w + pad)
+    x16 = rand(rng, h, w, 0, 2).astype(np.float16)
+    x16[h - 1, ::3] = 9.0   # the maximum in the partial vector, or in its neighbour
+    x16[max(h - 9, 0), 1::3] = 9.0
+    dy16 = rand(rng, h, w).astype(np.float16)
+    x, dy = f32(x16), f32(dy16)
+    layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
+    fwd, bwd = _sm_oracle(kind)
+    y = layer.forward(L.DeviceMatrix.from_numpy(x16, dtype=torch.float16, ldim=h + pad)).to_numpy()
+    check(f"{kind} f16 y {h}x{w}", y, fwd(x), fwd(f64(x)), tol=TOL_F16)
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy16, dtype=torch.float16, ldim=h + pad)).to_numpy()
+    check(f"{kind} f16 dx {h}x{w}", dx, bwd(f32(y), dy), bwd(f64(y), f64(dy)), tol=TOL_F16)
+    if kind == "softmax":
+        assert np.abs(y.astype(np.float64).sum(axis=0) - 1).max() < 2e-3 * np.sqrt(h)
+
+
+@pytest.mark.parametrize("h", [13, 259, 1027])
+def test_softmax_f16_special_values_on_unaligned_rows(L, h):
+    """-inf, a dominant entry and NaN in the partial vector at the end of an odd row and in its neighbour."""
+    x = np.zeros((h, 5), dtype=np.float16)
+    x[:, 0] = 3.0
+    x[h - 1, 1] = 60000.0
+    x[:, 2] = -np.inf
+    x[h - 2, 2] = 1.0
+    x[h - 1, 3] = np.nan
+    x[h - 9, 4] = np.nan
+    layer = L.softmax_layer()
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, dtype=torch.float16)).to_numpy()
+    ref = orc.softmax_fwd(f32(x))
+    assert np.allclose(y[:, 0], 1.0 / h, rtol=2e-3)
+    assert y[h - 1, 1] == 1.0 and y[:, 1].sum() == 1.0
+    assert y[h - 2, 2] == 1.0 and y[:, 2].sum() == 1.0
+    assert (ref[:, 3:] == 0).all() and (y[:, 3:] == 0).all()
+    ls = L.log_softmax_layer()
+    yl = ls.forward(L.DeviceMatrix.from_numpy(x[:, :3], dtype=torch.float16)).to_numpy()
+    refl = orc.log_softmax_fwd(f32(x[:, :3]))
+    assert np.array_equal(np.isneginf(yl), np.isneginf(refl))
+    fin = np.isfinite(refl)
+    assert np.allclose(yl[fin], refl[fin], rtol=2e-3, atol=2e-3)
+
+
 def test_softmax_f16_special_values(L):
     """A column of equal values, one with a dominant entry, one with -inf entries, one NaN."""
     h = 256
