@@ -306,8 +306,8 @@ static bool sm_bwd_framed_rows(hipStream_t st, int64_t n, int64_t w, int64_t row
   }
 }
 
-// 16-bit rows off the 16-byte grid (odd lengths or leading dimensions, any row stride) that fit a
-// workgroup's registers: the row kernels on 16-byte accesses at 2-byte alignment.  False: not
+// Rows off the 16-byte grid (odd lengths or leading dimensions, any row stride) that fit a
+// workgroup's registers: the row kernels on 16-byte accesses at the alignment of one entry.  False: not
 // launched (LBN_NO_UNALIGNED_ROWS=1 keeps the paths that served these rows before, for tests).
 // Measured against what served them before (one half per access up to 2047 entries, the packed
 // two-pass kernel from there), us forward / backward: 257 x 65536: 32 / 26 -> 20 / 20; 1025 x
@@ -324,16 +324,26 @@ static bool unaligned_rows()
   return !off;
 }
 
+// fp32 rows: single floats are as fast or faster everywhere (257 to 1025 and 4097 entries: 23-32 us
+// forward against 27-32) except from 2049 to 4096 entries, where they fill 1024 threads with
+// two to four registers each (2049 x 8192: 44 / 38 us against 27 / 35 with unaligned vectors).
+template <typename S>
+static bool unaligned_rows_serve(int64_t n, int64_t longest)
+{
+  if (!unaligned_rows() || n > longest) return false;
+  return sizeof(S) == 2 ? n >= kUnalignedRowMin : (n > 2048 && n <= 4096);
+}
+
 template <int KIND, typename S>
 static bool sm_fwd_unaligned_rows(hipStream_t st, int64_t n, int64_t rows, const S* x, int64_t ldx, S* y, int64_t ldy,
                                   RowMap map)
 {
-  if constexpr (sizeof(S) != 2) {
+  if constexpr (KIND == kChannelwise) {
     return false;
   }
   else {
-    constexpr int W = 8;
-    if (!unaligned_rows() || n < kUnalignedRowMin || n > kUnalignedRowMaxFwd) return false;
+    constexpr int W = 16 / sizeof(S);
+    if (!unaligned_rows_serve<S>(n, kUnalignedRowMaxFwd)) return false;
     const RowConfig c = pick_sm_row_config(ceil_div(n, W), rows);
     if (!c.tpr) return false;
 #define X(TPR, V)                                                                                       \
@@ -354,12 +364,12 @@ template <int KIND, typename S>
 static bool sm_bwd_unaligned_rows(hipStream_t st, int64_t n, int64_t rows, const S* y, int64_t ldy, const S* dy,
                                   int64_t lddy, S* dx, int64_t lddx, RowMap map)
 {
-  if constexpr (sizeof(S) != 2) {
+  if constexpr (KIND == kChannelwise) {
     return false;
   }
   else {
-    constexpr int W = 8;
-    if (!unaligned_rows() || n < kUnalignedRowMin || n > kUnalignedRowMaxBwd) return false;
+    constexpr int W = 16 / sizeof(S);
+    if (!unaligned_rows_serve<S>(n, kUnalignedRowMaxBwd)) return false;
     const RowConfig c = pick_sm_row_config(ceil_div(n, W), rows);
     if (!c.tpr) return false;
 #define X(TPR, V)                                                                                       \

@@ -76,6 +76,12 @@ struct RowIOUnaligned<__half, 8> {
   }
 };
 
+template <>
+struct RowIOUnaligned<float, 4> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) { __builtin_memcpy(v, p, 16); }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) { __builtin_memcpy(p, v, 16); }
+};
+
 template <typename S>
 struct RowLoad {
   static __device__ __forceinline__ float get(const S* p) { float v[1]; RowIO<S, 1>::template load<false>(p, v); return v[0]; }
@@ -128,7 +134,7 @@ __device__ __forceinline__ void frame_store(float* framep, unsigned idx, RowFram
 // 1024-thread blocks are held to 64 registers so that two of them share a compute unit
 // (not those with 32 accesses or more than 32 values per thread, which would spill).
 // FR (fp32): framed access for rows off the 16-byte grid; `nvec` is then the row length in entries.
-// UA (16-bit storage): rows off the 16-byte grid in 16-byte accesses at 2-byte alignment; `nvec` is
+// UA: rows off the 16-byte grid in 16-byte accesses at the alignment of one entry; `nvec` is
 // the row length in entries (at least W).  A last, partial vector is read as the row's last W
 // entries, so it overlaps its neighbour: the entries the two share count as absent in the partial
 // vector and are stored by the neighbour only.

@@ -164,6 +164,23 @@ def test_softmax_f16_special_values_on_unaligned_rows(L, h):
     assert np.allclose(yl[fin], refl[fin], rtol=2e-3, atol=2e-3)
 
 
+@pytest.mark.parametrize("kind", ["softmax", "log_softmax"])
+@pytest.mark.parametrize("h,w,pad", [(2049, 70, 0), (2050, 9, 0), (3001, 17, 0), (3071, 300, 0), (4095, 5, 0),
+                                     (4096, 9, 1), (3072, 12, 3), (2052, 7, 2)])
+def test_softmax_family_f32_unaligned_rows(L, kind, h, w, pad):
+    """fp32 rows of 2049 to 4096 entries off the 16-byte grid, in 16-byte accesses at 4-byte alignment."""
+    rng = np.random.default_rng(5 * h + w + pad)
+    x, dy = rand(rng, h, w, 0, 2), rand(rng, h, w)
+    x[h - 1, ::3] = 30.0
+    x[h - 5, 1::3] = 30.0
+    fwd, bwd = _sm_oracle(kind)
+    layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad)).to_numpy()
+    check(f"{kind} y {h}x{w}", y, fwd(x), fwd(f64(x)))
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    check(f"{kind} dx {h}x{w}", dx, bwd(f32(y), dy), bwd(f64(y), f64(dy)))
+
+
 def test_softmax_f16_special_values(L):
     """A column of equal values, one with a dominant entry, one with -inf entries, one NaN."""
     h = 256
