@@ -844,7 +844,7 @@ static int64_t ln_bwd_block_limit(int64_t rows, int elem_bytes)
 // Narrow teams with several vectors per thread spend the least on the row reduction,
 // so the narrowest team that owns at most 16 entries per thread is taken; rows too
 // long for that go to 512-thread teams with up to 32 entries per thread.
-static LnBwdPlan plan_ln_bwd(int64_t nvec, int64_t rows, int ve, int elem_bytes)
+static LnBwdPlan plan_ln_bwd(int64_t nvec, int64_t rows, int ve, int elem_bytes, bool wgrad = true)
 {
   static const int force_tpr = std::getenv("LBN_LN_BWD_TPR") ? std::atoi(std::getenv("LBN_LN_BWD_TPR")) : 0;
   static const int force_teams = std::getenv("LBN_LN_BWD_TEAMS") ? std::atoi(std::getenv("LBN_LN_BWD_TEAMS")) : 0;
@@ -866,11 +866,13 @@ static LnBwdPlan plan_ln_bwd(int64_t nvec, int64_t rows, int ve, int elem_bytes)
   p.tpr = tprs[pick];
   p.teams = teams[pick];
   p.v = round_up_pow2_le8(ceil_div(nvec, p.tpr));
-  if (!force_tpr && nvec <= 32 && rows >= 4096) {
-    // many short rows: teams of 16 lanes, four rows per wave
+  if (!force_tpr && nvec <= (wgrad ? 32 : 64) && rows >= 4096) {
+    // many short rows: teams of 16 lanes, four rows per wave (four vectors per lane only without
+    // weight gradients, whose accumulators would double the registers: fp32 rows of 132 entries x
+    // 131072 backward 41 -> 35 us without, 45 -> 48 us with them)
     p.tpr = 16;
     p.teams = 16;
-    p.v = nvec <= 16 ? 1 : 2;
+    p.v = nvec <= 16 ? 1 : nvec <= 32 ? 2 : 4;
   }
   if (force_teams && force_teams <= p.teams) p.teams = force_teams;
   // spread small problems: fewer teams per block when rows are scarce
@@ -941,10 +943,11 @@ static bool ln_pairs_first_wgrad(int64_t n, int64_t rows)
 // and beyond `longer_than` entries (2049 x 8192 forward: 26 against 47 us; 1025 x 16384
 // backward with weight gradients: 43 against 53 us); between, single floats are as fast or
 // a little faster (1001 x 16384 backward: 32 against 34 us).
-static bool ln_vectors_first(int64_t n, int64_t longer_than, int64_t rows)
+// team_units: the most vectors that a team of 16 lanes takes (64 forward, 32 with weight gradients).
+static bool ln_vectors_first(int64_t n, int64_t longer_than, int64_t rows, int64_t team_units)
 {
   if (n < 4 || ln_no_unaligned_rows()) return false;
-  return (ceil_div(n, 4) <= 32 && rows >= 4096) || n > longer_than;
+  return (ceil_div(n, 4) <= team_units && rows >= 4096) || n > longer_than;
 }
 
 constexpr int64_t kLnLongMin16 = 4096;  // shortest fp16 row of odd length that takes a 1024-thread workgroup of its own (1001 entries: 75 against 40 us)
@@ -1024,7 +1027,9 @@ static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, i
   // many short rows: teams of 16 lanes, four rows per wave, instead of mostly idle waves
   // (layer norm rows of 64 entries x 65536: 60 us per step against 150 us with one wave per row;
   // at 64 units per row the two shapes measure the same and the wave-wide team is kept)
-  if (units <= 32 && rows >= 4096) c = {16, units <= 16 ? 1 : 2};
+  // (up to 64 units with four per lane: fp16 rows of 512 entries x 65536 26 -> 24 us, fp32 rows of
+  // 132 x 131072 32 -> 27 us)
+  if (units <= 64 && rows >= 4096) c = {16, units <= 16 ? 1 : units <= 32 ? 2 : 4};
   // single floats cost one register each: rows just past 256, 512 or 1024 entries stay with one
   // wave (or four) holding 8 or 16 of them instead of four (or sixteen) waves holding two
   // (257 x 65536: 59 us forward, 1025 x 16384: 81 us that way)
@@ -1048,7 +1053,7 @@ static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, i
                        stats, lds, gamma, beta, sumsq, tail);                                  \
     return 1;                                                                                  \
   }
-  X(16, 1) X(16, 2)
+  X(16, 1) X(16, 2) X(16, 4)
   X(64, 1) X(64, 2) X(64, 4) X(256, 1) X(256, 2) X(256, 4) X(1024, 1) X(1024, 2) X(1024, 4)
   X(64, 8) X(256, 8)
   if constexpr (VE <= 4) { X(1024, 8) }
@@ -1225,7 +1230,7 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     }
   }
   if constexpr (std::is_same<T, float>::value) {
-    if (n > 1 && n <= kLnMaxScalarRowFwd && !ln_vectors_first(n, 2048, rows)) {  // rows off the 16-byte grid: the same kernels, one float per access
+    if (n > 1 && n <= kLnMaxScalarRowFwd && !ln_vectors_first(n, 2048, rows, 64)) {  // rows off the 16-byte grid: the same kernels, one float per access
       if (int r = ln_fwd_rows_launch<f32x1>(st, reinterpret_cast<const f32x1*>(x), reinterpret_cast<f32x1*>(y),
                                             ldx, ldy, map, rows, n, inv_n, eps, stats, lds, gamma, beta, sumsq))
         return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
@@ -1304,7 +1309,7 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
                               size_t ws_bytes, int tail = 0)
 {
   constexpr int VE = Vec16<ST>::N;
-  const LnBwdPlan p = plan_ln_bwd(units, rows, VE, elem_bytes);
+  const LnBwdPlan p = plan_ln_bwd(units, rows, VE, elem_bytes, wgrad);
   if (!p.tpr) return 0;
   if constexpr (VE >= 4 && !UnalignedVec<ST>::value) {
     if (wgrad && ln_bwd_small(rows, n, elem_bytes)) {
@@ -1338,7 +1343,7 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
                                           sgrad, ldsg, gamma, part, tail);                      \
     launched = true;                                                                            \
   }
-  X(16, 16, 1) X(16, 16, 2)
+  X(16, 16, 1) X(16, 16, 2) X(16, 16, 4)
   X(64, 4, 1) X(64, 4, 2) X(64, 4, 4) X(256, 2, 1) X(256, 2, 2) X(256, 1, 1) X(256, 1, 2)
   X(512, 1, 1) X(512, 1, 2) X(512, 1, 4)
   if constexpr (VE <= 4) { X(256, 2, 4) X(256, 1, 4) X(512, 1, 8) }
@@ -1432,7 +1437,7 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
       }
     }
     if constexpr (std::is_same<T, float>::value) {
-      if (n <= kLnMaxScalarRowBwd && !ln_vectors_first(n, 1024, rows)) {  // rows off the 16-byte grid: the same kernels, one float per access
+      if (n <= kLnMaxScalarRowBwd && !ln_vectors_first(n, 1024, rows, wgrad ? 32 : 64)) {  // rows off the 16-byte grid: the same kernels, one float per access
         if (int r = ln_bwd_rows_launch<f32x1>(st, wgrad, reinterpret_cast<const f32x1*>(x),
                                               reinterpret_cast<const f32x1*>(dy), reinterpret_cast<f32x1*>(dx), ldx,
                                               lddy, lddx, map, rows, n, n, 4, eps, stats, lds, sgrad, ldsg, gamma,
