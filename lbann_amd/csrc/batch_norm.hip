@@ -1264,14 +1264,14 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
       a.slab_width = p.slab_width, a.part = part, a.use_pivot = pivot, a.eps = epsilon;
       a.mean = mean, a.var = var, a.scale = scale, a.bias = bias;
       bn_rt_launch_sums<S, false>(st, p, a);
-      if (cs * p.slabs >= kBnRtWideChannel)
-        hipLaunchKernelGGL((bn_rt_fwd_stats<S, true>), dim3(static_cast<unsigned>(C)), dim3(kRowTileThreads), 0, st,
-                           C, cs, w, h, p.slabs, part, x, pivot, bessel, epsilon, decay, mean, var, running_mean,
-                           running_var);
-      else
-        hipLaunchKernelGGL((bn_rt_fwd_stats<S, false>), dim3(static_cast<unsigned>(ceil_div(C, kRowTileWaves))),
-                           dim3(kRowTileThreads), 0, st, C, cs, w, h, p.slabs, part, x, pivot, bessel, epsilon,
-                           decay, mean, var, running_mean, running_var);
+      const int mode = bn_rt_stats_mode(cs, p.slabs);
+      const dim3 sgrid(bn_rt_stats_grid(mode, C));
+#define X(MODE)                                                                                              \
+  if (mode == MODE)                                                                                          \
+    hipLaunchKernelGGL((bn_rt_fwd_stats<S, MODE>), sgrid, dim3(kRowTileThreads), 0, st, C, cs, w, h, p.slabs, \
+                       part, x, pivot, bessel, epsilon, decay, mean, var, running_mean, running_var);
+      X(kBnRtWave) X(kBnRtWide) X(kBnRtThin)
+#undef X
       bn_rt_launch_apply<S, false>(st, p, a);
       return launch_status();
     }
@@ -1350,13 +1350,14 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
       a.count = static_cast<float>(n), a.count_bessel = static_cast<float>(n - (bessel ? 1 : 0));
       a.zero = n <= 1;
       bn_rt_launch_sums<S, true>(st, p, a);
-      if (cs * p.slabs >= kBnRtWideChannel)
-        hipLaunchKernelGGL(bn_rt_bwd_stats<true>, dim3(static_cast<unsigned>(C)), dim3(kRowTileThreads), 0, st, C,
-                           cs, h, p.slabs, part, epsilon, training, use_var, scale, dscale, dbias, dmean, dvar);
-      else
-        hipLaunchKernelGGL(bn_rt_bwd_stats<false>, dim3(static_cast<unsigned>(ceil_div(C, kRowTileWaves))),
-                           dim3(kRowTileThreads), 0, st, C, cs, h, p.slabs, part, epsilon, training, use_var, scale,
-                           dscale, dbias, dmean, dvar);
+      const int mode = bn_rt_stats_mode(cs, p.slabs);
+      const dim3 sgrid(bn_rt_stats_grid(mode, C));
+#define X(MODE)                                                                                          \
+  if (mode == MODE)                                                                                      \
+    hipLaunchKernelGGL(bn_rt_bwd_stats<MODE>, sgrid, dim3(kRowTileThreads), 0, st, C, cs, h, p.slabs, part, \
+                       epsilon, training, use_var, scale, dscale, dbias, dmean, dvar);
+      X(kBnRtWave) X(kBnRtWide) X(kBnRtThin)
+#undef X
       bn_rt_launch_apply<S, true>(st, p, a);
       return launch_status();
     }

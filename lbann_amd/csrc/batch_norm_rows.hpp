@@ -162,19 +162,76 @@ __device__ __forceinline__ float2 bn_rt_channel_total_wide(const float2* part, i
   return t;
 }
 
-// One wave per channel (4 channels per workgroup); WIDE: one workgroup per channel.
-template <typename S, bool WIDE>
+// Channels of a few rows (batch norm behind a fully connected layer: 16384 channels of one row):
+// one thread per channel adds its rows x slabs partials, instead of a wave per channel with one
+// busy lane (16384 channels x 512 columns: 8 us of a 29 us forward pass that way).
+constexpr int64_t kBnRtThinChannel = 8;  // rows x slabs up to which a channel takes one thread
+
+__device__ __forceinline__ float2 bn_rt_channel_total_thin(const float2* part, int64_t h, int slabs, int64_t cs,
+                                                           int64_t c)
+{
+  double a = 0., b = 0.;
+  for (int s = 0; s < slabs; ++s) {
+    const float2* row = part + static_cast<int64_t>(s) * h + c * cs;
+    for (int64_t i = 0; i < cs; ++i) {
+      a += static_cast<double>(row[i].x);
+      b += static_cast<double>(row[i].y);
+    }
+  }
+  return make_float2(static_cast<float>(a), static_cast<float>(b));
+}
+
+// How a channel's partials are added up: by one wave (4 channels per workgroup), by a whole
+// workgroup, or by one thread (256 channels per workgroup).
+constexpr int kBnRtWave = 0, kBnRtWide = 1, kBnRtThin = 2;
+
+inline int bn_rt_stats_mode(int64_t cs, int slabs)
+{
+  const int64_t parts = cs * slabs;
+  return parts >= kBnRtWideChannel ? kBnRtWide : parts <= kBnRtThinChannel ? kBnRtThin : kBnRtWave;
+}
+
+inline unsigned bn_rt_stats_grid(int mode, int64_t C)
+{
+  const int64_t per = mode == kBnRtWide ? 1 : mode == kBnRtThin ? kRowTileThreads : kRowTileWaves;
+  return static_cast<unsigned>((C + per - 1) / per);
+}
+
+template <int MODE>
+__device__ __forceinline__ bool bn_rt_stats_channel(int64_t C, int64_t& c)
+{
+  c = MODE == kBnRtWide   ? static_cast<int64_t>(blockIdx.x)
+      : MODE == kBnRtThin ? static_cast<int64_t>(blockIdx.x) * kRowTileThreads + threadIdx.x
+                          : static_cast<int64_t>(blockIdx.x) * kRowTileWaves + wave_index();
+  return c < C;
+}
+
+// The thread that holds a channel's totals and writes its results.
+template <int MODE>
+__device__ __forceinline__ bool bn_rt_stats_writer()
+{
+  return MODE == kBnRtWide ? threadIdx.x == 0 : MODE == kBnRtThin ? true : (threadIdx.x & (kWave - 1)) == 0;
+}
+
+template <int MODE>
+__device__ __forceinline__ float2 bn_rt_stats_total(const float2* part, int64_t h, int slabs, int64_t cs, int64_t c)
+{
+  if constexpr (MODE == kBnRtWide) return bn_rt_channel_total_wide(part, h, slabs, cs, c);
+  else if constexpr (MODE == kBnRtThin) return bn_rt_channel_total_thin(part, h, slabs, cs, c);
+  else return bn_rt_channel_total(part, h, slabs, cs, c);
+}
+
+template <typename S, int MODE>
 __global__ void __launch_bounds__(kRowTileThreads)
 bn_rt_fwd_stats(int64_t C, int64_t cs, int64_t w, int64_t h, int slabs, const float2* __restrict__ part,
                 const S* __restrict__ x, int use_pivot, int bessel, float eps, float decay,
                 float* __restrict__ mean, float* __restrict__ var, float* __restrict__ rmean,
                 float* __restrict__ rvar)
 {
-  const int64_t c = WIDE ? static_cast<int64_t>(blockIdx.x)
-                         : static_cast<int64_t>(blockIdx.x) * kRowTileWaves + wave_index();
-  if (c >= C) return;
-  const float2 t = WIDE ? bn_rt_channel_total_wide(part, h, slabs, cs, c) : bn_rt_channel_total(part, h, slabs, cs, c);
-  if (WIDE ? threadIdx.x != 0 : (threadIdx.x & (kWave - 1)) != 0) return;
+  int64_t c;
+  if (!bn_rt_stats_channel<MODE>(C, c)) return;  // (whole workgroups or waves in the modes that use barriers or wave sums)
+  const float2 t = bn_rt_stats_total<MODE>(part, h, slabs, cs, c);
+  if (!bn_rt_stats_writer<MODE>()) return;
   const int64_t n = cs * w;
   if (n <= 1) {  // batch_normalization.cpp:118-120: the mean holds x, the variance is 1
     mean[c] = Vec16<S>::load1(x + c * cs);
@@ -190,18 +247,17 @@ bn_rt_fwd_stats(int64_t C, int64_t cs, int64_t w, int64_t h, int slabs, const fl
   rvar[c] = decay * rvar[c] + (1.f - decay) * v;
 }
 
-template <bool WIDE>
+template <int MODE>
 __global__ void __launch_bounds__(kRowTileThreads)
 bn_rt_bwd_stats(int64_t C, int64_t cs, int64_t h, int slabs, const float2* __restrict__ part, float eps,
                 int training, const float* __restrict__ var, const float* __restrict__ scale,
                 float* __restrict__ dscale, float* __restrict__ dbias, float* __restrict__ dmean,
                 float* __restrict__ dvar)
 {
-  const int64_t c = WIDE ? static_cast<int64_t>(blockIdx.x)
-                         : static_cast<int64_t>(blockIdx.x) * kRowTileWaves + wave_index();
-  if (c >= C) return;
-  const float2 t = WIDE ? bn_rt_channel_total_wide(part, h, slabs, cs, c) : bn_rt_channel_total(part, h, slabs, cs, c);
-  if (WIDE ? threadIdx.x != 0 : (threadIdx.x & (kWave - 1)) != 0) return;
+  int64_t c;
+  if (!bn_rt_stats_channel<MODE>(C, c)) return;  // (whole workgroups or waves in the modes that use barriers or wave sums)
+  const float2 t = bn_rt_stats_total<MODE>(part, h, slabs, cs, c);
+  if (!bn_rt_stats_writer<MODE>()) return;
   const float inv_stdev = 1.0f / sqrtf(var[c] + eps);
   float ds, db, dm, dv;
   grads_from_sums(t.x, t.y, scale[c], inv_stdev, ds, db, dm, dv);
