@@ -62,7 +62,32 @@ __device__ __forceinline__ void ce_store_partial(const CeArgs<S>& a, float sum, 
   }
 }
 
-template <bool VEC, int T, typename S>
+// How a column is accessed: entry by entry, in aligned 16-byte vectors (columns of whole vectors
+// on the 16-byte grid), or in 16-byte vectors at the alignment of one entry with the last
+// h % VE entries apart (columns of odd height: 1001 classes x 16384 forward 22 us entry by entry).
+constexpr int kCeScalar = 0, kCeVec = 1, kCeUnaligned = 2;
+
+template <typename S> struct CeUnaligned;
+template <> struct CeUnaligned<float> { using type = f32u; };
+template <> struct CeUnaligned<__half> { using type = f16u; };
+
+template <int VEC, typename S>
+struct CeIO {
+  using U = typename CeUnaligned<S>::type;
+  static constexpr int N = Vec16<S>::N;
+  static __device__ __forceinline__ void load(const S* p, float (&v)[N])
+  {
+    if constexpr (VEC == kCeUnaligned) Vec16<U>::load(reinterpret_cast<const U*>(p), v);
+    else Vec16<S>::load(p, v);
+  }
+  static __device__ __forceinline__ void store(S* p, const float (&v)[N])
+  {
+    if constexpr (VEC == kCeUnaligned) Vec16<U>::store(reinterpret_cast<U*>(p), v);
+    else Vec16<S>::store(p, v);
+  }
+};
+
+template <int VEC, int T, typename S>
 __global__ void __launch_bounds__(T)
 ce_fwd_dense(CeArgs<S> a)
 {
@@ -77,14 +102,18 @@ ce_fwd_dense(CeArgs<S> a)
   for (int64_t j = static_cast<int64_t>(blockIdx.y) * T + threadIdx.x; j < n; j += step) {
     if (VEC) {
       float v[VE], t[VE];
-      Vec16<S>::load(xc + VE * j, v);
-      Vec16<S>::load(tc + VE * j, t);
+      CeIO<VEC, S>::load(xc + VE * j, v);
+      CeIO<VEC, S>::load(tc + VE * j, t);
 #pragma unroll
       for (int k = 0; k < VE; ++k) sum += ce_term(t[k], v[k]);
     }
     else {
       sum += ce_term(Vec16<S>::load1(tc + j), Vec16<S>::load1(xc + j));
     }
+  }
+  if (VEC == kCeUnaligned && blockIdx.y == 0) {  // the entries behind the last whole vector
+    const int64_t j = VE * n + threadIdx.x;
+    if (j < a.h) sum += ce_term(Vec16<S>::load1(tc + j), Vec16<S>::load1(xc + j));
   }
   ce_store_partial<T>(a, sum, red);
 }
@@ -171,7 +200,7 @@ ce_merge_parts(int P, const float* __restrict__ part, S* __restrict__ loss, int6
   if (lane == 0) Vec16<S>::store1(loss + c * ld_loss, v);
 }
 
-template <bool VEC, typename S>
+template <int VEC, typename S>
 __global__ void __launch_bounds__(kCeThreads)
 ce_bwd_dense(CeArgs<S> a)
 {
@@ -187,17 +216,25 @@ ce_bwd_dense(CeArgs<S> a)
   for (int64_t j = static_cast<int64_t>(blockIdx.y) * kCeThreads + threadIdx.x; j < n; j += step) {
     if (VEC) {
       float v[VE], t[VE], d[VE], dt[VE];
-      Vec16<S>::load(xc + VE * j, v);
-      Vec16<S>::load(tc + VE * j, t);
+      CeIO<VEC, S>::load(xc + VE * j, v);
+      CeIO<VEC, S>::load(tc + VE * j, t);
 #pragma unroll
       for (int k = 0; k < VE; ++k) {
         dt[k] = -g * logf(v[k]);
         d[k] = t[k] > 0.f ? -g * t[k] / v[k] : 0.f;
       }
-      Vec16<S>::store(dxc + VE * j, d);
-      if (a.dtruth) Vec16<S>::store(dtc + VE * j, dt);
+      CeIO<VEC, S>::store(dxc + VE * j, d);
+      if (a.dtruth) CeIO<VEC, S>::store(dtc + VE * j, dt);
     }
     else {
+      const float v = Vec16<S>::load1(xc + j), t = Vec16<S>::load1(tc + j);
+      if (a.dtruth) Vec16<S>::store1(dtc + j, -g * logf(v));
+      Vec16<S>::store1(dxc + j, t > 0.f ? -g * t / v : 0.f);
+    }
+  }
+  if (VEC == kCeUnaligned && blockIdx.y == 0) {  // the entries behind the last whole vector
+    const int64_t j = VE * n + threadIdx.x;
+    if (j < a.h) {
       const float v = Vec16<S>::load1(xc + j), t = Vec16<S>::load1(tc + j);
       if (a.dtruth) Vec16<S>::store1(dtc + j, -g * logf(v));
       Vec16<S>::store1(dxc + j, t > 0.f ? -g * t / v : 0.f);
@@ -307,7 +344,10 @@ static int ce_fwd_impl(lbn_stream_t stream, int64_t height, int64_t width, int u
   }
   const bool vec = !use_labels && ce_vec_ok(height, width, prediction, ld_prediction, VE) &&
                    ce_vec_ok(height, width, ground_truth, ld_ground_truth, VE);
-  const int64_t units = use_labels ? (spatial_size < height ? spatial_size : height) : (vec ? height / VE : height);
+  // columns off the 16-byte grid: 16-byte accesses at the alignment of one entry
+  const bool unal = !use_labels && !vec && height >= 4 * VE;
+  const int64_t units = use_labels ? (spatial_size < height ? spatial_size : height)
+                                   : ((vec || unal) ? height / VE : height);
   // 1024-thread workgroups when that fills the device with one workgroup per column: no
   // partial sums to merge, so no second kernel
   const bool big = !use_labels && units >= 4 * 1024 && width >= 256;
@@ -317,10 +357,12 @@ static int ce_fwd_impl(lbn_stream_t stream, int64_t height, int64_t width, int u
     return LBN_ERR_WORKSPACE;
   const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
   if (use_labels) hipLaunchKernelGGL((ce_fwd_labels<S>), grid, dim3(kCeThreads), 0, st, a);
-  else if (vec && big) hipLaunchKernelGGL((ce_fwd_dense<true, 1024, S>), grid, dim3(1024), 0, st, a);
-  else if (vec) hipLaunchKernelGGL((ce_fwd_dense<true, kCeThreads, S>), grid, dim3(kCeThreads), 0, st, a);
-  else if (big) hipLaunchKernelGGL((ce_fwd_dense<false, 1024, S>), grid, dim3(1024), 0, st, a);
-  else hipLaunchKernelGGL((ce_fwd_dense<false, kCeThreads, S>), grid, dim3(kCeThreads), 0, st, a);
+  else if (vec && big) hipLaunchKernelGGL((ce_fwd_dense<kCeVec, 1024, S>), grid, dim3(1024), 0, st, a);
+  else if (vec) hipLaunchKernelGGL((ce_fwd_dense<kCeVec, kCeThreads, S>), grid, dim3(kCeThreads), 0, st, a);
+  else if (unal && big) hipLaunchKernelGGL((ce_fwd_dense<kCeUnaligned, 1024, S>), grid, dim3(1024), 0, st, a);
+  else if (unal) hipLaunchKernelGGL((ce_fwd_dense<kCeUnaligned, kCeThreads, S>), grid, dim3(kCeThreads), 0, st, a);
+  else if (big) hipLaunchKernelGGL((ce_fwd_dense<kCeScalar, 1024, S>), grid, dim3(1024), 0, st, a);
+  else hipLaunchKernelGGL((ce_fwd_dense<kCeScalar, kCeThreads, S>), grid, dim3(kCeThreads), 0, st, a);
   if (P > 1)
     hipLaunchKernelGGL((ce_merge_parts<S>), dim3(static_cast<unsigned>(width)), dim3(kWave), 0, st, P, a.part, loss,
                        ld_loss);
@@ -357,15 +399,17 @@ static int ce_bwd_impl(lbn_stream_t stream, int64_t height, int64_t width, int u
   else
     vec = vec && ce_vec_ok(height, width, ground_truth, ld_ground_truth, VE) &&
           ce_vec_ok(height, width, dground_truth, ld_dground_truth, VE);
-  const int P = ce_parts(width, vec ? height / VE : height, kCeThreads, kCeMaxPartsBwd);
+  const bool unal = !use_labels && !vec && height >= 4 * VE;
+  const int P = ce_parts(width, (vec || unal) ? height / VE : height, kCeThreads, kCeMaxPartsBwd);
   const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
   if (use_labels) {
     if (vec) hipLaunchKernelGGL((ce_bwd_labels<true, S>), grid, dim3(kCeThreads), 0, st, a);
     else hipLaunchKernelGGL((ce_bwd_labels<false, S>), grid, dim3(kCeThreads), 0, st, a);
   }
   else {
-    if (vec) hipLaunchKernelGGL((ce_bwd_dense<true, S>), grid, dim3(kCeThreads), 0, st, a);
-    else hipLaunchKernelGGL((ce_bwd_dense<false, S>), grid, dim3(kCeThreads), 0, st, a);
+    if (vec) hipLaunchKernelGGL((ce_bwd_dense<kCeVec, S>), grid, dim3(kCeThreads), 0, st, a);
+    else if (unal) hipLaunchKernelGGL((ce_bwd_dense<kCeUnaligned, S>), grid, dim3(kCeThreads), 0, st, a);
+    else hipLaunchKernelGGL((ce_bwd_dense<kCeScalar, S>), grid, dim3(kCeThreads), 0, st, a);
   }
   return launch_status();
 }

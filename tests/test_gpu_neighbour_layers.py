@@ -46,6 +46,8 @@ CE_DENSE = [
     (16384, 256, 0), (4101, 257, 0),   # one 1024-thread workgroup per column, vector and scalar
     (10, 5000, 0), (21, 70000, 0), (64, 4099, 3), (1, 6000, 0), (3, 100000, 0), (17, 4096, 0),   # 16-lane teams
     (2000000, 1, 0), (600000, 2, 0),   # a column or two: many workgroups per column
+    # columns off the 16-byte grid: unaligned vectors and the h % 4 entries behind them
+    (17, 40, 0), (19, 300, 0), (1003, 70, 0), (50257, 5, 0), (2048, 9, 1), (4099, 300, 2), (600001, 2, 0), (16, 33, 3),
 ]
 
 
@@ -104,6 +106,8 @@ CE_F16 = [
     (16, 128, 0), (1000, 64, 0), (192, 23, 0), (4096, 33, 0), (7, 5, 0), (1001, 3, 0), (136, 4, 8), (130, 4, 2),
     (16384, 256, 0), (4101, 257, 0), (65536, 40, 0), (300000, 3, 0), (1, 6, 0),
     (10, 5000, 0), (33, 4500, 8), (64, 4100, 0),   # 16-lane teams
+    # columns off the 16-byte grid: unaligned vectors and the h % 8 entries behind them
+    (33, 40, 0), (39, 300, 0), (1003, 70, 0), (50257, 5, 0), (2048, 9, 1), (4103, 300, 2), (600001, 2, 0), (32, 33, 3),
 ]
 
 
