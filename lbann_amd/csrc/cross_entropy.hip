@@ -286,6 +286,86 @@ ce_bwd_labels(CeArgs<S> a)
   }
 }
 
+// Labels with one position per sample (plain classification: a column of `classes` entries and
+// one label): every entry of dx is zero but the label's, so the column goes out in 16-byte
+// stores at the alignment of one entry and x is read at the label only.  1000 classes x 65536:
+// 100 us entry by entry.
+template <typename S>
+__global__ void __launch_bounds__(kCeThreads)
+ce_bwd_one_label(CeArgs<S> a)
+{
+  using U = typename CeUnaligned<S>::type;
+  constexpr int VE = Vec16<S>::N;
+  const int64_t c = blockIdx.x;
+  const float g = Vec16<S>::load1(a.dy + c * a.lddy);
+  const S* xc = a.x + c * a.ldx;
+  S* dxc = a.dx + c * a.lddx;
+  const int64_t label = ce_label(Vec16<S>::load1(a.truth + c * a.ldt));
+  const float hit = (label >= 0 && label < a.h) ? -g / Vec16<S>::load1(xc + label) : 0.f;
+  const int64_t n = a.h / VE;
+  const int64_t step = static_cast<int64_t>(gridDim.y) * kCeThreads;
+  for (int64_t j = static_cast<int64_t>(blockIdx.y) * kCeThreads + threadIdx.x; j < n; j += step) {
+    float d[VE];
+#pragma unroll
+    for (int k = 0; k < VE; ++k) d[k] = (VE * j + k == label) ? hit : 0.f;
+    Vec16<U>::store(reinterpret_cast<U*>(dxc + VE * j), d);
+  }
+  if (blockIdx.y == 0) {  // the entries behind the last whole vector
+    const int64_t j = VE * n + threadIdx.x;
+    if (j < a.h) Vec16<S>::store1(dxc + j, j == label ? hit : 0.f);
+  }
+}
+
+// The same for many short columns: a workgroup takes eight of them, so that the chain of loads
+// that ends in x[label] is waited for once per eight columns (one workgroup per column of 1000
+// classes x 65536: 80 us, bound by that wait).
+constexpr int kCeOneLabelColumns = 8;
+
+template <typename S>
+__global__ void __launch_bounds__(kCeThreads)
+ce_bwd_one_label_columns(CeArgs<S> a)
+{
+  using U = typename CeUnaligned<S>::type;
+  constexpr int VE = Vec16<S>::N;
+  __shared__ float s_hit[kCeOneLabelColumns];
+  __shared__ int64_t s_label[kCeOneLabelColumns];
+  const int64_t c0 = static_cast<int64_t>(blockIdx.x) * kCeOneLabelColumns;
+  if (threadIdx.x < kCeOneLabelColumns) {
+    const int64_t c = c0 + threadIdx.x;
+    int64_t label = -1;
+    float hit = 0.f;
+    if (c < a.w) {
+      const float g = Vec16<S>::load1(a.dy + c * a.lddy);
+      label = ce_label(Vec16<S>::load1(a.truth + c * a.ldt));
+      if (label >= 0 && label < a.h) hit = -g / Vec16<S>::load1(a.x + c * a.ldx + label);
+      else label = -1;
+    }
+    s_hit[threadIdx.x] = hit;
+    s_label[threadIdx.x] = label;
+  }
+  __syncthreads();
+  const int64_t n = a.h / VE;
+  const int tail = static_cast<int>(a.h - VE * n);
+#pragma unroll
+  for (int k = 0; k < kCeOneLabelColumns; ++k) {
+    const int64_t c = c0 + k;
+    if (c >= a.w) break;  // block-uniform
+    const int64_t label = s_label[k];
+    const float hit = s_hit[k];
+    S* dxc = a.dx + c * a.lddx;
+    for (int64_t j = threadIdx.x; j < n; j += kCeThreads) {
+      float d[VE];
+#pragma unroll
+      for (int e = 0; e < VE; ++e) d[e] = (VE * j + e == label) ? hit : 0.f;
+      Vec16<U>::store(reinterpret_cast<U*>(dxc + VE * j), d);
+    }
+    if (static_cast<int>(threadIdx.x) < tail) {
+      const int64_t j = VE * n + threadIdx.x;
+      Vec16<S>::store1(dxc + j, j == label ? hit : 0.f);
+    }
+  }
+}
+
 // Workgroups of `threads` threads per column: about 2048 * 256 threads in total, each
 // thread with at least four units.  (A single column of a segmentation map, 19 classes x
 // 1024 x 2048 positions, had been held to 64 workgroups: 426 us backward.)
@@ -402,7 +482,16 @@ static int ce_bwd_impl(lbn_stream_t stream, int64_t height, int64_t width, int u
   const bool unal = !use_labels && !vec && height >= 4 * VE;
   const int P = ce_parts(width, (vec || unal) ? height / VE : height, kCeThreads, kCeMaxPartsBwd);
   const dim3 grid(static_cast<unsigned>(width), static_cast<unsigned>(P));
-  if (use_labels) {
+  if (use_labels && spatial_size == 1 && height >= 4 * VE) {
+    const int P1 = ce_parts(width, height / VE, kCeThreads, kCeMaxPartsBwd);
+    if (P1 == 1 && width >= 4096)
+      hipLaunchKernelGGL((ce_bwd_one_label_columns<S>), dim3(static_cast<unsigned>(ceil_div(width, kCeOneLabelColumns))),
+                         dim3(kCeThreads), 0, st, a);
+    else
+      hipLaunchKernelGGL((ce_bwd_one_label<S>), dim3(static_cast<unsigned>(width), static_cast<unsigned>(P1)),
+                         dim3(kCeThreads), 0, st, a);
+  }
+  else if (use_labels) {
     if (vec) hipLaunchKernelGGL((ce_bwd_labels<true, S>), grid, dim3(kCeThreads), 0, st, a);
     else hipLaunchKernelGGL((ce_bwd_labels<false, S>), grid, dim3(kCeThreads), 0, st, a);
   }

@@ -76,6 +76,7 @@ CE_LABELS = [
     (3, (8, 8), 23, 0), (3, (4, 4, 4), 11, 0), (10, (1,), 64, 0), (5, (7, 3), 9, 0), (4, (6,), 5, 3),
     (21, (64, 64), 6, 0), (2, (300, 300), 3, 0), (1000, (1,), 128, 0), (19, (128, 130), 2, 0),
     (19, (512, 1024), 1, 0),   # one column of a large map: many workgroups per column
+    (1000, (1,), 300, 0), (1003, (1,), 70, 3), (17, (1,), 5000, 1), (50257, (1,), 9, 0),   # one label per sample
 ]
 
 
@@ -89,6 +90,9 @@ def test_cross_entropy_labels(L, classes, spatial, w, pad):
     if sp > 2:
         labels[1, 0] = classes      # a label no class matches contributes nothing
         labels[2, 0] = -3.0
+    elif w > 3:
+        labels[0, 1] = classes
+        labels[0, 2] = -3.0
     dy = rng.standard_normal(w).astype(np.float32)
     layer = L.cross_entropy_layer((classes,) + tuple(spatial), use_labels=True)
     loss = layer.forward(L.DeviceMatrix.from_numpy(x, ldim=h + pad),
@@ -139,7 +143,7 @@ def test_cross_entropy_dense_f16(L, h, w, pad):
 
 @pytest.mark.parametrize("classes,spatial,w,pad", [(3, (8, 8), 23, 0), (10, (1,), 64, 0), (5, (7, 3), 9, 0),
                                                   (4, (6,), 5, 3), (21, (64, 64), 6, 0), (1000, (1,), 128, 0),
-                                                  (2048, (1,), 16, 0)])
+                                                  (2048, (1,), 16, 0), (1003, (1,), 70, 3), (37, (1,), 5000, 1)])
 def test_cross_entropy_labels_f16(L, classes, spatial, w, pad):
     """Class indices stored as binary16 (exact up to 2048)."""
     rng = np.random.default_rng(classes * 101 + w)
@@ -150,6 +154,9 @@ def test_cross_entropy_labels_f16(L, classes, spatial, w, pad):
     if sp > 2:
         labels[1, 0] = classes      # a label no class matches contributes nothing
         labels[2, 0] = -3.0
+    elif w > 3:
+        labels[0, 1] = classes
+        labels[0, 2] = -3.0
     dy = rng.standard_normal(w).astype(np.float16)
     half = torch.float16
     layer = L.cross_entropy_layer((classes,) + tuple(spatial), use_labels=True)
