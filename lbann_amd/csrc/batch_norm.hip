@@ -1196,7 +1196,7 @@ static int bn_fwd_apply_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, f
   if (!x || !y || !mean || !var || !scale || !bias) return LBN_ERR_INVALID_ARGUMENT;
   if constexpr (Vec16<S>::N == 4) {  // float or fp16 in fours: the row-tile kernels
     if (bn_rt_usable<S>(C, cs, w, x, ldx) && bn_rt_usable<S>(C, cs, w, y, ldy)) {
-      const RowTilePlan p = row_tile_plan(C * cs, w);
+      const RowTilePlan p = row_tile_plan(C * cs, w, sizeof(S) == 2 ? 2 : 4);
       BnRtArgs<S> a{};
       a.h = C * cs, a.w = w, a.cs = cs, a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy;
       a.slab_width = p.slab_width, a.eps = epsilon, a.mean = mean, a.var = var, a.scale = scale, a.bias = bias;
@@ -1258,7 +1258,7 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
         t.scale = scale, t.bias = bias, t.rmean = running_mean, t.rvar = running_var;
         if (bn_rt_try_tile<S, false>(st, t)) return launch_status();
       }
-      const RowTilePlan p = row_tile_plan(h, w);
+      const RowTilePlan p = row_tile_plan(h, w, sizeof(S) == 2 ? 2 : 4);
       BnRtArgs<S> a{};
       a.h = h, a.w = w, a.cs = cs, a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy;
       a.slab_width = p.slab_width, a.part = part, a.use_pivot = pivot, a.eps = epsilon;
@@ -1342,7 +1342,7 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
         t.dscale = dscale, t.dbias = dbias, t.dmean = dmean, t.dvar = dvar;
         if (bn_rt_try_tile<S, true>(st, t)) return launch_status();
       }
-      const RowTilePlan p = row_tile_plan(h, w);
+      const RowTilePlan p = row_tile_plan(h, w, sizeof(S) == 2 ? 2 : 4);
       BnRtArgs<S> a{};
       a.h = h, a.w = w, a.cs = cs, a.x = x, a.dy = dy, a.out = dx, a.ldx = ldx, a.lddy = lddy, a.ldo = lddx;
       a.slab_width = p.slab_width, a.part = part, a.eps = epsilon;

@@ -577,8 +577,9 @@ inline int bn_rt_tile_rows(int64_t cs, int rows)
 
 inline size_t bn_rt_workspace_bytes(int64_t h, int64_t w)
 {
-  const RowTilePlan p = row_tile_plan(h, w);
-  return static_cast<size_t>(p.slabs) * static_cast<size_t>(h) * sizeof(float2);
+  // (the query does not know the storage type: the larger of the two plans)
+  const int a = row_tile_plan(h, w, 4).slabs, b = row_tile_plan(h, w, 2).slabs;
+  return static_cast<size_t>(a > b ? a : b) * static_cast<size_t>(h) * sizeof(float2);
 }
 
 }  // namespace lbn

@@ -85,10 +85,16 @@ struct RowTilePlan {
   int64_t slab_width;
 };
 
-inline RowTilePlan row_tile_plan(int64_t h, int64_t w)
+// 16-bit storage (a row quad is 8 bytes): with GW = 4 a wave's access touches four columns, 128
+// bytes in each; tall matrices take GW = 1 there, 512 contiguous bytes of one column (batch norm
+// on 64 x 111 x 111, w = 32: 65 / 68 -> 47 / 57 us; 96 x 55 x 55, w = 64: 37 / 49 -> 34 / 41), while
+// 16384 rows x 512 columns have too few tiles of 256 rows for that (24 / 24 -> 33 / 37 us).
+constexpr int64_t kRowTileTallRows = 65536;
+
+inline RowTilePlan row_tile_plan(int64_t h, int64_t w, int elem_bytes = 4)
 {
   RowTilePlan p;
-  p.gw = w >= 16 ? 4 : 1;
+  p.gw = (w >= 16 && !(elem_bytes == 2 && h >= kRowTileTallRows)) ? 4 : 1;
   p.tiles = ceil_div(h, p.gw == 1 ? RowTilePos<1>::kRows : RowTilePos<4>::kRows);
   const int64_t min_width = 4 * kRowTileWaves * p.gw;
   const int64_t want = ceil_div(1024, p.tiles);
