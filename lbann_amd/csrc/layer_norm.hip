@@ -1239,7 +1239,7 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
   if constexpr (std::is_same<T, float>::value) {
     // longer fp32 rows off the 16-byte grid: 16-byte accesses at 4-byte alignment, the last n % 4
     // entries in a vector that overlaps its neighbour; first the register kernels, then two passes
-    if (!ln_no_unaligned_rows()) {
+    if (n >= 4 && !ln_no_unaligned_rows()) {  // (the partial vector reaches back four entries from the row's end)
       if (int r = ln_fwd_rows_launch<f32u>(st, reinterpret_cast<const f32u*>(x), reinterpret_cast<f32u*>(y), ldx, ldy,
                                            map, rows, ceil_div(n, 4), inv_n, eps, stats, lds, gamma, beta, sumsq,
                                            static_cast<int>(n % 4)))
@@ -1446,7 +1446,7 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
       }
     }
     if constexpr (std::is_same<T, float>::value) {
-      if (!ln_no_unaligned_rows()) {
+      if (n >= 4 && !ln_no_unaligned_rows()) {
         if (int r = ln_bwd_rows_launch<f32u>(st, wgrad, reinterpret_cast<const f32u*>(x),
                                              reinterpret_cast<const f32u*>(dy), reinterpret_cast<f32u*>(dx), ldx,
                                              lddy, lddx, map, rows, ceil_div(n, 4), n, 4, eps, stats, lds, sgrad, ldsg,
