@@ -89,6 +89,7 @@ def test_softmax_family(L, kind, h, w, pad):
     (32768, 300, 0, True), (20480, 513, 0, False), (24584, 260, 8, False),    # more rows than compute units: walked
     (128256, 40, 0, True), (65544, 5, 8, False), (65540, 3, 0, False),        # long rows: two packed passes,
     (50257, 9, 0, True), (40001, 5, 16, False), (33001, 7, 0, False), (32770, 4, 3, False),  # cut at 16-byte boundaries per row
+    (1003, 33, 0, True), (4099, 9, 1, True), (259, 5000, 0, True),   # unaligned vectors, in place
 ])
 def test_softmax_family_f16_storage(L, kind, h, w, pad, in_place):
     """fp16 storage, fp32 arithmetic (softmax.cpp:236-243 instantiates the layers for half):
@@ -350,12 +351,12 @@ def test_matrices_that_start_off_the_16_byte_grid(L, h, offsets):
 
 
 @pytest.mark.parametrize("kind", ["softmax", "log_softmax", "channelwise"])
-@pytest.mark.parametrize("h,w", [(4096, 6), (777, 5), (70000, 2)])
+@pytest.mark.parametrize("h,w", [(4096, 6), (777, 5), (70000, 2), (3003, 7)])
 def test_softmax_family_in_place(L, kind, h, w):
     rng = np.random.default_rng(h + w)
     x, dy = rand(rng, h, w, 0, 2), rand(rng, h, w)
     if kind == "channelwise":
-        C = 7 if h == 777 else 4
+        C = 7 if h % 7 == 0 else 4
         layer = L.channelwise_softmax_layer((C, h // C))
         fwd = lambda a: orc.channelwise_softmax_fwd(a, C, h // C, h // C)
         bwd = lambda y, g: orc.channelwise_softmax_bwd(y, g, C, h // C, h // C)
