@@ -369,7 +369,9 @@ static bool sm_bwd_unaligned_rows(hipStream_t st, int64_t n, int64_t rows, const
   }
   else {
     constexpr int W = 16 / sizeof(S);
-    if (!unaligned_rows_serve<S>(n, kUnalignedRowMaxBwd)) return false;
+    // (softmax backward gains up to the forward limit: 30522 x 2048 fp16 82 -> 72 us; log-softmax,
+    // whose exponentials sit between the loads and the stores, loses there: 64 -> 74 us)
+    if (!unaligned_rows_serve<S>(n, KIND == kLogSoftmax ? kUnalignedRowMaxBwd : kUnalignedRowMaxFwd)) return false;
     const RowConfig c = pick_sm_row_config(ceil_div(n, W), rows);
     if (!c.tpr) return false;
 #define X(TPR, V)                                                                                       \
