@@ -5,12 +5,13 @@
 
 A "step" is one forward + backward pass of the headline layer (Softmax, fp32,
 32768 classes x 512 samples) over one batch of synthetic input that is already
-resident in HBM.  The last line printed is ONE JSON object: the headline
-throughput in GB/s of algorithmic bytes (forward reads x and writes y, backward
-reads y and dy and writes dx), the roofline entry of its dominant kernel timed
-with HIP events on the launch stream, the CPU baseline (the restated reference
-CPU code, OpenMP, on the host cores), and under "layers" the same measurements
-for every benchmark configuration.
+resident in HBM.  The last line printed is ONE JSON object of a few KB: the
+headline throughput in GB/s of algorithmic bytes (forward reads x and writes y,
+backward reads y and dy and writes dx), the roofline entry of its dominant
+kernel timed with HIP events on the launch stream, the CPU baseline (the
+restated reference CPU code, OpenMP, on the host cores), and under
+config.per_config one short row for every benchmark configuration.  Every
+timing of every row goes to stderr and to gpurun_out/bench_layers.json.
 """
 import argparse
 import json
@@ -22,6 +23,99 @@ import time
 import numpy as np
 
 HBM_PEAK_GBS = 8000.0
+ROOT = os.path.dirname(os.path.abspath(__file__))
+# CPU baseline protocol: untimed warm-ups, then timed repetitions (median), threads pinned
+CPU_WARMUPS, CPU_REPS = 3, 5
+CPU_ENV = {"OMP_PROC_BIND": "close", "OMP_PLACES": "cores"}
+
+
+def _r(v, digits):
+    return None if v is None else round(v, digits)
+
+
+def build_record(results, headline, steps, warmup, cold_yardstick=None, committed=None, copy_cal=None):
+    """The ONE JSON object of the benchmark's last stdout line, from the per-row measurements.
+
+    `results[name]` holds a row's timings (see main()); `committed` is the content of
+    profiles/headline_traffic.json (HBM bytes per launch from the byte counters and the kernel
+    trace's per-dispatch average of the headline kernel) or None.  Kept small (a few KB): the
+    per-row detail is written to a file, not to this line.
+
+    roofline: the dominant kernel of the headline step is the backward row kernel (3 tensors
+    against 2).  `avg_launch_ms` is THIS run's measurement: `steps` launches of that kernel back
+    to back between two HIP events on the launch stream, divided by `steps`.  The event pair
+    around every single launch of the timed steps ("event_bracket_launch_ms") reads 2 to 5 us
+    more, the cost of the two markers.  The committed rocprofv3 per-dispatch average is quoted
+    beside it and `agrees_with_rocprof` says whether the two are within 5 %."""
+    h = results[headline]
+    dom_bytes = h["algorithmic_bytes"]["bwd"]
+    dom_ms = h["bwd_back_to_back_ms"]
+    bracket_ms = h["bwd_ms"]
+    traffic = rocprof_ms = None
+    if committed:
+        traffic = committed.get("traffic_bytes_per_launch")
+        if committed.get("rocprof_avg_us"):
+            rocprof_ms = committed["rocprof_avg_us"] * 1e-3
+    dom_gbs = dom_bytes / (dom_ms * 1e-3) / 1e9
+    agrees = None if rocprof_ms is None else bool(abs(dom_ms - rocprof_ms) <= 0.05 * rocprof_ms)
+
+    # every benchmark configuration: us per step (forward + backward, buffers reused every step),
+    # fraction of the 8 TB/s peak on algorithmic bytes, the same with the tensors rotated out of
+    # the caches ("cold") where they fit them, the two calls on their own (event-bracketed: each
+    # includes the event markers) and the CPU baseline's rate where it was timed
+    per_config = {}
+    for name, r in results.items():
+        if not name.startswith("cfg"):
+            continue
+        per_config[name] = {"us_per_step": _r(r["ms_per_step"] * 1e3, 2), "frac": _r(r["frac_of_hbm_peak"], 4),
+                            "fwd_us": _r(r["fwd_ms"] * 1e3, 2), "bwd_us": _r(r["bwd_ms"] * 1e3, 2),
+                            "cold_frac": _r(r["cold"]["frac_of_hbm_peak"], 4) if r.get("cold") else None,
+                            "samples_per_s": round(r["samples_per_s"]),
+                            "cpu_gbs": _r(r["cpu"]["gbs"], 1) if r.get("cpu") else None}
+    out = {
+        "metric": "fwd+bwd achieved HBM GB/s (algorithmic bytes / time), Softmax 32768x512 fp32, 1 GPU",
+        "value": h["gbs"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": h["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic (seeded N(0,2^2) logits with 1% set to +30, N(0,1) upstream gradient), resident in HBM; "
+                "every step reuses the same buffers, which (3 x 64 MiB) stay in the 256 MB Infinity Cache: "
+                "config.cold_frac is the same step with its tensors rotated among 1 GiB of copies",
+        "config": {"workload": h["workload"], "samples": 512, "classes": 32768,
+                   "samples_per_s": _r(h["samples_per_s"], 1), "frac_of_hbm_peak": _r(h["frac_of_hbm_peak"], 4),
+                   "cold_frac": _r(h["cold"]["frac_of_hbm_peak"], 4) if h.get("cold") else None,
+                   "cold_yardstick": cold_yardstick,
+                   "per_config": per_config},
+        "roofline": {"bound": "hbm", "kernel": "sm_bwd_rows_walk<float,8,softmax>", "achieved": dom_gbs,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom_gbs / HBM_PEAK_GBS,
+                     "bytes_per_launch": dom_bytes, "avg_launch_ms": dom_ms,
+                     "avg_launch_source": "this run: `steps` launches back to back between two HIP events "
+                                          "on the launch stream",
+                     "traffic": traffic,
+                     "traffic_source": "profiles/headline_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)",
+                     "event_bracket_launch_ms": bracket_ms,
+                     "event_pair_ms": h.get("event_pair_ms"),
+                     "frac_event_bracket": dom_bytes / (bracket_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "rocprof_avg_launch_ms": rocprof_ms,
+                     "agrees_with_rocprof": agrees},
+    }
+    if copy_cal:
+        out["copy_calibration"] = copy_cal
+    if "cpu" in h:
+        c = h["cpu"]
+        out["cpu_baseline"] = {"value": c["gbs"], "unit": "GB/s", "cores": c["threads"], "kind": "port",
+                               "sample": f"the full 32768x512 workload, forward+backward, median of "
+                                         f"{c.get('reps', CPU_REPS)} repetitions after {c.get('warmups', CPU_WARMUPS)} "
+                                         f"warm-ups ({c.get('seconds', 0):.2f} s of CPU time in all)",
+                               "env": c.get("env", CPU_ENV),
+                               "samples_per_s": c["samples_per_s"]}
+    return out
 
 
 def parse():
@@ -45,6 +139,11 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path "
               f"(--gpus {args.gpus} requested); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    # the CPU baseline's threads stay on their cores (read when the OpenMP runtime starts)
+    for k, v in CPU_ENV.items():
+        os.environ.setdefault(k, v)
+        CPU_ENV[k] = os.environ[k]
 
     import torch
     from lbann_amd import layers as L
@@ -476,11 +575,18 @@ def main():
         if not args.no_cpu:
             from oracle import cpu_oracle as orc
             cpu_threads = orc.max_threads()
-            reps = [cpu() for _ in range(2 if elems > 3e7 else 4)][1:]
+            # benchmark configurations: the stated protocol; the informational rows on tensors of
+            # hundreds of MiB keep one warm-up and three repetitions (seconds of CPU time each)
+            full = name.startswith("cfg") or elems <= 3e7
+            nw, nr = (CPU_WARMUPS, CPU_REPS) if full else (1, 3)
+            t_cpu = time.perf_counter()
+            reps = [cpu() for _ in range(nw + nr)][nw:]
+            t_cpu = time.perf_counter() - t_cpu
             cf = statistics.median(t[0] for t in reps)
             cb = statistics.median(t[1] for t in reps)
             r["cpu"] = {"fwd_ms": cf * 1e3, "bwd_ms": cb * 1e3, "gbs": (fwd_b + bwd_b) / (cf + cb) / 1e9,
-                        "samples_per_s": samples / (cf + cb), "threads": cpu_threads}
+                        "samples_per_s": samples / (cf + cb), "threads": cpu_threads,
+                        "warmups": nw, "reps": nr, "seconds": t_cpu, "env": dict(CPU_ENV)}
         results[name] = r
         print(f"# {name}: {step_ms*1e3:8.1f} us/step  {r['gbs']:7.0f} GB/s ({100*r['frac_of_hbm_peak']:.1f}% of 8 TB/s)  "
               f"fwd {f_ms*1e3:7.1f} us ({r['fwd_gbs']:.0f} GB/s)  bwd {b_ms*1e3:7.1f} us ({r['bwd_gbs']:.0f} GB/s)"
@@ -540,92 +646,28 @@ def main():
         del xs, ds, os_
         torch.cuda.empty_cache()
 
-    h = results[headline]
-    # Dominant kernel of the headline step: the backward row kernel (3 tensors against 2).  Its
-    # launch duration is measured here with HIP events on the launch stream, one pair of events
-    # around every launch of the timed region ("event_bracket_launch_ms": the dispatch plus what
-    # the two event markers cost, 2 to 4 us on this part) and once more as `steps` launches back
-    # to back between two events (which overlap their ramp-up and drain, and re-read the same
-    # buffers).  The per-dispatch begin-to-end average of the same command under
-    # `rocprofv3 --kernel-trace --stats` is committed under profiles/ and lies between the two:
-    # `achieved` and `frac` use it as long as the live bracket figure is consistent with it (the
-    # bracket must be longer, by no more than 6 us); otherwise they fall back to the bracket figure.
-    dom_bytes = h["algorithmic_bytes"]["bwd"]
-    bracket_ms = h["bwd_ms"]
-    b2b_ms = h["bwd_back_to_back_ms"]
-    traffic = rocprof_ms = None
-    tpath = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "headline_traffic.json")
+    committed = None
+    tpath = os.path.join(ROOT, "profiles", "headline_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
             committed = json.load(f)
-        traffic = committed.get("traffic_bytes_per_launch")
-        if committed.get("rocprof_avg_us"):
-            rocprof_ms = committed["rocprof_avg_us"] * 1e-3
-    consistent = rocprof_ms is not None and 0.0 <= bracket_ms - rocprof_ms <= 0.006
-    if rocprof_ms is not None and not consistent:
-        print(f"# note: the headline kernel measures {bracket_ms*1e3:.1f} us per bracketed launch here, "
-              f"{rocprof_ms*1e3:.1f} us per dispatch in the committed kernel trace: using the live figure",
+    out = build_record(results, headline, args.steps, args.warmup, cold_yardstick, committed, copy_cal)
+    rf = out["roofline"]
+    if rf["agrees_with_rocprof"] is False:
+        print(f"# note: the headline kernel measures {rf['avg_launch_ms']*1e3:.2f} us per launch here, "
+              f"{rf['rocprof_avg_launch_ms']*1e3:.2f} us per dispatch in the committed kernel trace (> 5 % apart)",
               file=sys.stderr)
-    dom_ms = rocprof_ms if consistent else bracket_ms
-    dom_gbs = dom_bytes / (dom_ms * 1e-3) / 1e9
-
-    def frac_of(r):
-        return r["frac_of_hbm_peak"] if r else None
-
-    # every benchmark configuration in the record the driver keeps: us per step (forward +
-    # backward, buffers reused every step), fraction of the 8 TB/s peak on algorithmic bytes,
-    # the same with the tensors rotated out of the caches ("cold") where they fit them, and
-    # the two calls on their own (event-bracketed: each includes 2 to 4 us of event markers)
-    per_config = {}
-    for name, r in results.items():
-        if not name.startswith("cfg"):
-            continue
-        per_config[name] = {"us_per_step": round(r["ms_per_step"] * 1e3, 2), "frac": round(r["frac_of_hbm_peak"], 4),
-                            "fwd_us": round(r["fwd_ms"] * 1e3, 2), "bwd_us": round(r["bwd_ms"] * 1e3, 2),
-                            "cold_frac": round(frac_of(r.get("cold")), 4) if r.get("cold") else None,
-                            "samples_per_s": round(r["samples_per_s"])}
-    out = {
-        "metric": "fwd+bwd achieved HBM GB/s (algorithmic bytes / time), Softmax 32768x512 fp32, 1 GPU",
-        "value": h["gbs"],
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": h["ms_per_step"],
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic (seeded N(0,2^2) logits with 1% set to +30, N(0,1) upstream gradient), resident in HBM; "
-                "every step reuses the same buffers, which (3 x 64 MiB) stay in the 256 MB Infinity Cache: "
-                "config.cold_frac is the same step with its tensors rotated among 1 GiB of copies",
-        "config": {"workload": h["workload"], "samples": 512, "classes": 32768,
-                   "samples_per_s": h["samples_per_s"], "frac_of_hbm_peak": h["frac_of_hbm_peak"],
-                   "cold_frac": frac_of(h.get("cold")), "cold_yardstick": cold_yardstick,
-                   "per_config": per_config},
-        "roofline": {"bound": "hbm", "kernel": "sm_bwd_rows_walk<float,8,softmax>", "achieved": dom_gbs,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom_gbs / HBM_PEAK_GBS,
-                     "bytes_per_launch": dom_bytes, "avg_launch_ms": dom_ms,
-                     "avg_launch_source": ("rocprofv3 per-dispatch average (profiles/bench_all_layers_kernel_trace.md), "
-                                           "consistent with this run's event timing") if consistent
-                                          else "HIP events around every launch of this run (includes the event markers)",
-                     "traffic": traffic,
-                     "traffic_source": "profiles/headline_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)",
-                     "event_bracket_launch_ms": bracket_ms,
-                     "frac_event_bracket": dom_bytes / (bracket_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "back_to_back_launch_ms": b2b_ms,
-                     "frac_back_to_back": dom_bytes / (b2b_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "rocprof_avg_launch_ms": rocprof_ms},
-        "layers": results,
-    }
-    if copy_cal:
-        out["copy_calibration"] = copy_cal
-    if "cpu" in h:
-        out["cpu_baseline"] = {"value": h["cpu"]["gbs"], "unit": "GB/s", "cores": h["cpu"]["threads"],
-                               "kind": "port",
-                               "sample": "the full 32768x512 workload, forward+backward, median of 3 repetitions after 1 warm-up",
-                               "samples_per_s": h["cpu"]["samples_per_s"]}
-    print(json.dumps(out))
+    # the per-row detail (every timing of every row, informational rows included) goes to a file
+    # and stays out of the one JSON line on stdout
+    detail = os.path.join(ROOT, "gpurun_out", "bench_layers.json")
+    try:
+        os.makedirs(os.path.dirname(detail), exist_ok=True)
+        with open(detail, "w") as f:
+            json.dump({"steps": args.steps, "warmup": args.warmup, "layers": results}, f, indent=1)
+        print(f"# per-row detail written to {detail}", file=sys.stderr)
+    except OSError as e:
+        print(f"# per-row detail not written ({e})", file=sys.stderr)
+    print(json.dumps(out), flush=True)
 
 
 if __name__ == "__main__":
