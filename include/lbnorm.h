@@ -3,8 +3,10 @@
  * Each entry point is the device compute of one LBANN layer's fp_compute() or
  * bp_compute() on LOCAL matrices: column-major, element (r,c) at buf[r + c*ld],
  * one column per mini-batch sample (El::Matrix<T,Device>: Height/Width/LDim/Buffer).
- * A call only enqueues work on `stream`: it never synchronises the device,
- * allocates or frees memory, or reads results back.  All pointers are device
+ * A call only enqueues work on `stream`: it allocates and frees no memory, reads
+ * no results back, and does not wait for the device (one exception, described under
+ * "Waits across workgroups": a cluster kernel that follows one enqueued on another
+ * host thread's hipStreamPerThread waits for the device once).  All pointers are device
  * pointers that must stay valid until the stream work completes.  Every output
  * element is overwritten (outputs may be uninitialised on entry); nothing is
  * accumulated into.  Calls with width == 0 or an empty sample return LBN_OK
@@ -12,6 +14,10 @@
  *
  * Return value: LBN_OK, a negative LBN_ERR_* code for a rejected argument, or a
  * positive hipError_t from the launch.  No C++ exception crosses this boundary.
+ * An entry point clears the calling thread's pending HIP error (hipGetLastError)
+ * when it starts, so that the status it returns reports its own launches only: a
+ * caller that wants to see an error left by its own earlier HIP calls reads it
+ * before calling in.
  *
  * Scratch memory ("workspace") is always caller-provided.  The matching
  * *_workspace_bytes() function returns the size needed for a given shape
@@ -38,8 +44,12 @@
  * not share the device: each could hold part of it and wait for workgroups that cannot
  * start.  The library sees to that for eager calls itself: a cluster kernel whose
  * predecessor went to another stream is made to wait for it with an event (processes that
- * use one stream for these calls pay nothing; the first call from a second stream waits
- * for the device once), and launches from several host threads queue up behind a mutex.
+ * use one stream for these calls pay nothing; the first call from a second stream records
+ * the event behind its predecessor, and only when that predecessor went to another host
+ * thread's hipStreamPerThread, a stream this thread cannot name, does it wait for the device,
+ * once), and launches from several host threads queue up behind a mutex.  Should the order
+ * not be established at all (event and device wait both refused, e.g. while another thread
+ * records a graph in global capture mode), the call runs its multi-kernel path instead.
  * What it cannot order are replays of HIP graphs that contain cluster kernels: do not
  * replay two such graphs, or one next to eager cluster calls of another stream, at the same
  * time (or set LBN_NO_CLUSTER=1 in the environment, which selects the multi-kernel paths
@@ -101,7 +111,10 @@ int lbn_workspace_timed_out(lbn_stream_t stream, const void* workspace, int* tim
  * raises the error word of `workspace` (at least 128 bytes, 16-byte aligned) and the
  * kernel ends like any other.  out4 (4 floats, device) receives member 0's pair and the
  * stand-in (-1, -1) of the absent member.  Afterwards lbn_workspace_timed_out() reports 1
- * for this workspace until its header is cleared.  No counterpart in the reference. */
+ * for this workspace until its header is cleared.  workspace == NULL (workspace_bytes
+ * ignored) runs the same on the library-owned array of lbn_softmax_fwd_static_scratch_f32,
+ * whose word lbn_softmax_fwd_static_scratch_timed_out() reads.  No counterpart in the
+ * reference. */
 int lbn_selftest_cluster_wait_gives_up(lbn_stream_t stream, void* workspace, size_t workspace_bytes,
                                        int max_polls, float* out4);
 
@@ -365,10 +378,22 @@ int lbn_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
  * size are rejected with LBN_ERR_UNSUPPORTED before anything is launched.  All calls on
  * one GPU share the array: two such calls that overlap in time on one GPU (different
  * streams, or concurrent graph replays) race on it and are not supported; calls on one
- * stream are ordered and safe.  Nothing in the array has to start at zero. */
+ * stream are ordered and safe.  Nothing in the array has to start at zero.
+ *
+ * The first call on a device looks up the array's address and creates the event that
+ * orders cluster kernels across streams; neither may happen while a stream is recording
+ * a graph, so callers that record call lbn_softmax_fwd_static_scratch_prepare() once per
+ * device beforehand, with that device current (it launches nothing; calling it again is
+ * harmless).  The array's first 64 bytes hold the sticky word of the bounded waits like any
+ * workspace's; the caller never sees the array, so
+ * lbn_softmax_fwd_static_scratch_timed_out() reads that word for the current device
+ * (waits for `stream`, stores 0 or 1 in *timed_out) and clears it when it was raised.
+ * lbn_selftest_cluster_wait_gives_up() with a NULL workspace raises it on purpose. */
 size_t lbn_softmax_fwd_static_scratch_max_bytes(void);
+int lbn_softmax_fwd_static_scratch_prepare(void);
 int lbn_softmax_fwd_static_scratch_f32(lbn_stream_t stream, int64_t height, int64_t width,
                                        const float* x, int64_t ldx, float* y, int64_t ldy);
+int lbn_softmax_fwd_static_scratch_timed_out(lbn_stream_t stream, int* timed_out);
 
 /* ----------------------------------------------------------------- log-softmax
  * Replaces log_softmax_layer::fp_compute / bp_compute

@@ -64,6 +64,8 @@ PROTOTYPES = {
     "lbn_softmax_bwd_f32": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_softmax_fwd_static_scratch_max_bytes": (sz, []),
     "lbn_softmax_fwd_static_scratch_f32": (cint, [vp, i64, i64, vp, i64, vp, i64]),
+    "lbn_softmax_fwd_static_scratch_prepare": (cint, []),
+    "lbn_softmax_fwd_static_scratch_timed_out": (cint, [vp, ctypes.POINTER(ctypes.c_int)]),
     "lbn_log_softmax_fwd_f32": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_log_softmax_bwd_f32": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_softmax_fwd_f16": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, sz]),

@@ -733,7 +733,7 @@ __device__ __forceinline__ void bn_fwd_finish_ws(const BnFwdArgs<S>& a, const Bn
     wave_merge_broadcast(stage_f, use, ts, tq);
   }
   else {
-    wave_merge_wait(stage_f, use, ts, tq);
+    wave_merge_wait(stage_f, use, a.cw.error, ts, tq);
   }
   float mean, var;
   stats_from_sums(ts, tq, t.K, a.n, a.bessel, a.eps, mean, var);
@@ -842,7 +842,7 @@ __device__ __forceinline__ void bn_bwd_finish_ws(const BnBwdArgs<S>& a, const Bn
     wave_merge_broadcast(stage_f, use, ta, tb);
   }
   else {
-    wave_merge_wait(stage_f, use, ta, tb);
+    wave_merge_wait(stage_f, use, a.cw.error, ta, tb);
   }
   float ds, db, dmean, dvar;
   grads_from_sums(ta, tb, scale, inv_stdev, ds, db, dmean, dvar);
@@ -1029,6 +1029,7 @@ static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   const BnClusterShape p = bn_cluster_shape(E, 4, 256);
   if (!p.T) return false;
   ClusterLaunchGuard guard(st);
+  if (guard.failed()) return false;
   const BnFwdArgs<S> a{x, y, ldx, ldy, cs, static_cast<int>(C), p.M, pivot, bessel, eps, decay, cs * w,
                        cluster_workspace(ws), cluster_call_tag(st, cluster_workspace(ws)), mean, var, scale, bias, rmean, rvar};
   const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(E);
@@ -1053,6 +1054,7 @@ static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   const BnClusterShape p = bn_cluster_shape(E, kShortVectors ? 4 : 2, 256);
   if (!p.T) return false;
   ClusterLaunchGuard guard(st);
+  if (guard.failed()) return false;
   const BnBwdArgs<S> a{x, dy, dx, ldx, lddy, lddx, cs, static_cast<int>(C), p.M, bessel, eps, cs * w,
                        cluster_workspace(ws), cluster_call_tag(st, cluster_workspace(ws)), mean, var, scale, dscale, dbias, dmean, dvar};
   const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(E);
@@ -1088,6 +1090,7 @@ static bool bn_try_stream(hipStream_t st, BnStreamArgs<S> a, int64_t C, int64_t 
   a.seg = static_cast<unsigned>(cs / VE), a.E = static_cast<unsigned>(E), a.share = static_cast<unsigned>(share);
   a.cw = cluster_workspace(ws);
   ClusterLaunchGuard guard(st);
+  if (guard.failed()) return false;
   a.tag = cluster_call_tag(st, a.cw);
   const dim3 grid(static_cast<unsigned>(nc * M));
   if (BWD) hipLaunchKernelGGL(bn_bwd_stream<S>, grid, dim3(kBnStreamThreads), 0, st, a);

@@ -59,7 +59,12 @@ int lbn_workspace_timed_out(lbn_stream_t stream, const void* workspace, int* tim
 int lbn_selftest_cluster_wait_gives_up(lbn_stream_t stream, void* workspace, size_t workspace_bytes,
                                        int max_polls, float* out4)
 {
-  if (!workspace || !out4 || max_polls < 1 || max_polls > (1 << 16)) return LBN_ERR_INVALID_ARGUMENT;
+  if (!out4 || max_polls < 1 || max_polls > (1 << 16)) return LBN_ERR_INVALID_ARGUMENT;
+  if (!workspace) {  // the library-owned array of the entry point that allocates nothing
+    const int status = lbn::static_scratch_address(&workspace);
+    if (status != LBN_OK) return status;
+    workspace_bytes = lbn::static_scratch_bytes();
+  }
   if (workspace_bytes < lbn::cluster_workspace_bytes(1, 2) || !lbn::aligned16(workspace)) return LBN_ERR_WORKSPACE;
   hipStream_t st = lbn::as_stream(stream);
   const lbn::ClusterWorkspace cw = lbn::cluster_workspace(workspace);

@@ -264,12 +264,20 @@ __device__ __forceinline__ void wave_merge_broadcast(WaveMerge<NW>& st, unsigned
 }
 
 template <int NW>
-__device__ __forceinline__ void wave_merge_wait(WaveMerge<NW>& st, unsigned use, float& a, float& b)
+__device__ __forceinline__ void wave_merge_wait(WaveMerge<NW>& st, unsigned use, int* error_word, float& a, float& b)
 {
-  // bounded like the cluster polls: the polling wave gives up after kClusterMaxPolls rounds
-  // and still broadcasts, so this loop ends as well
-  while (__hip_atomic_load(&st.ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != use + 1)
+  // The polling wave gives up after kClusterMaxPolls rounds and still broadcasts, so this loop
+  // ends with it; it also has a bound of its own (the polling wave's budget and as much again,
+  // an LDS poll being shorter than a device-scope one) and raises the error word past it.
+  int polls = 0;
+  while (__hip_atomic_load(&st.ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != use + 1) {
+    if (++polls > 2 * kClusterMaxPolls) {
+      if ((threadIdx.x & (kWave - 1)) == 0)
+        __hip_atomic_store(error_word, kClusterTimedOut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      break;
+    }
     __builtin_amdgcn_s_sleep(1);
+  }
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   a = st.total[0];
   b = st.total[1];
@@ -453,11 +461,18 @@ inline ClusterTag cluster_call_tag(hipStream_t st, const ClusterWorkspace& cw)
 // mutex, so that launches from several host threads queue up one at a time.
 //
 // A process that only ever uses one stream for these calls pays nothing: events are recorded
-// only from the moment a second stream shows up (that launch waits for the device once, the
-// earlier launch having left no event).  Recording one after every launch from the start was
-// measured: about 3 us per kernel (262144 x 16 softmax 26.6 against 20.9 us per step).  Streams that are being recorded into a HIP graph are
-// left alone: keeping graphs that contain cluster kernels from replaying side by side is up to
-// the caller.
+// only from the moment a second stream shows up.  That launch records the event behind the
+// earlier launch on the earlier launch's stream (which the guard remembers) and waits for it;
+// nothing waits for the device.  The one exception: when the earlier stream was another host
+// thread's hipStreamPerThread, which this thread cannot name, the launch waits for the device
+// once.  Recording an event after every launch from the start was measured: about 3 us per kernel
+// (262144 x 16 softmax 26.6 against 20.9 us per step).  Streams that are being recorded into a
+// HIP graph are left alone: keeping graphs that contain cluster kernels from replaying side by
+// side is up to the caller.
+//
+// failed(): the order could not be established (the event calls and the device-wide wait all
+// returned errors, e.g. while another thread records a graph in global capture mode).  The
+// caller then does not launch its cluster kernel and takes its multi-kernel path instead.
 class ClusterLaunchGuard {
  public:
   explicit ClusterLaunchGuard(hipStream_t st) : st_(st), capturing_(stream_is_capturing(st))
@@ -470,25 +485,33 @@ class ClusterLaunchGuard {
     if (!state_->several) {
       state_->several = true;
       make_event(*state_);
-      (void)hipDeviceSynchronize();
+      // the earlier launch left no event: put one behind it now, on its own stream
+      const bool nameable = state_->last != hipStreamPerThread || state_->last_thread == std::this_thread::get_id();
+      if (state_->done && nameable && hipEventRecord(state_->done, state_->last) == hipSuccess &&
+          hipStreamWaitEvent(st, state_->done, 0) == hipSuccess)
+        return;
+      wait_for_device();
     }
-    else if (state_->done) {
-      (void)hipStreamWaitEvent(st, state_->done, 0);
-    }
-    else {
-      (void)hipDeviceSynchronize();  // no event could be created: order the launches the slow way
+    else if (!state_->done || hipStreamWaitEvent(st, state_->done, 0) != hipSuccess) {
+      wait_for_device();  // no event: order the launches the slow way
     }
   }
   ~ClusterLaunchGuard()
   {
-    if (!capturing_) {
-      if (state_->several && state_->done) (void)hipEventRecord(state_->done, st_);
+    if (!capturing_ && !failed_) {
+      if (state_->several && state_->done && hipEventRecord(state_->done, st_) != hipSuccess) {
+        // the next launch from another stream must not trust a stale event
+        (void)hipGetLastError();
+        (void)hipEventDestroy(state_->done);
+        state_->done = nullptr;
+      }
       state_->last = st_;
       state_->have_last = true;
       if (st_ == hipStreamPerThread) state_->last_thread = std::this_thread::get_id();
     }
     state_->mu.unlock();
   }
+  bool failed() const { return failed_; }
   ClusterLaunchGuard(const ClusterLaunchGuard&) = delete;
   ClusterLaunchGuard& operator=(const ClusterLaunchGuard&) = delete;
 
@@ -524,6 +547,14 @@ class ClusterLaunchGuard {
     static State s[kMaxDevices];
     return s;
   }
+  void wait_for_device()
+  {
+    (void)hipGetLastError();  // whatever the event calls left behind
+    if (hipDeviceSynchronize() != hipSuccess) {
+      (void)hipGetLastError();
+      failed_ = true;
+    }
+  }
   static void make_event(State& s)
   {
     if (!s.done && hipEventCreateWithFlags(&s.done, hipEventDisableTiming) != hipSuccess) {
@@ -533,6 +564,7 @@ class ClusterLaunchGuard {
   }
   hipStream_t st_;
   bool capturing_;
+  bool failed_ = false;
   State* state_;
 };
 

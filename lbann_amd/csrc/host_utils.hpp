@@ -17,7 +17,8 @@ namespace lbn {
 
 // Every entry point converts its stream argument first: that is also where an error left
 // behind by an earlier, unrelated HIP call of this thread is dropped, so that
-// launch_status() below reports this call's launches only.
+// launch_status() below reports this call's launches only (the header of the C ABI tells
+// callers that their pending error is cleared).
 inline hipStream_t as_stream(lbn_stream_t s)
 {
   (void)hipGetLastError();
@@ -43,6 +44,11 @@ inline bool stream_is_capturing(hipStream_t st)
   }
   return status != hipStreamCaptureStatusNone;
 }
+
+// Device address (current device) and size of the library-owned scratch array of the entry
+// point that allocates nothing (defined in softmax.hip); *out stays null on failure.
+int static_scratch_address(void** out);
+size_t static_scratch_bytes();
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -1086,6 +1086,7 @@ static int ln_fwd_cluster_launch(hipStream_t st, const T* x, T* y, int64_t ldx, 
     a.nvec = static_cast<unsigned>(n / VE), a.per_wg = l.per_wg, a.M = l.M, a.sumsq = sumsq;         \
     a.inv_n = 1.0f / static_cast<float>(n), a.eps = eps, a.stats = stats, a.ld_stats = lds;          \
     ClusterLaunchGuard guard(st);                                                                    \
+    if (guard.failed()) return 0;                                                                    \
     a.gamma = gamma, a.beta = beta, a.cw = cw, a.tag = cluster_call_tag(st, cw);                     \
     const dim3 grid(static_cast<unsigned>(l.clusters * l.M));                                        \
     if (affine) hipLaunchKernelGGL((ln_fwd_cluster<T, VV, true>), grid, dim3(kLnClThreads), 0, st, a); \
@@ -1125,6 +1126,7 @@ static int ln_bwd_cluster_launch(hipStream_t st, bool wgrad, const T* x, const T
     a.inv_n = 1.0f / static_cast<float>(n), a.eps = eps, a.stats = const_cast<float*>(stats);        \
     a.ld_stats = lds, a.sgrad = sgrad, a.ld_sgrad = ldsg, a.gamma = gamma, a.wpart = wpart;          \
     ClusterLaunchGuard guard(st);                                                                    \
+    if (guard.failed()) return 0;                                                                    \
     a.cw = cw, a.tag = cluster_call_tag(st, cw);                                                     \
     const dim3 grid(static_cast<unsigned>(nc * l.M));                                                \
     if (wgrad) {                                                                                     \
@@ -1168,6 +1170,7 @@ static int ln_stream_launch(hipStream_t st, LnClArgs<T> a, int64_t rows, int64_t
   a.M = static_cast<int>(M), a.inv_n = 1.0f / static_cast<float>(n);
   a.cw = cluster_workspace(ws);
   ClusterLaunchGuard guard(st);
+  if (guard.failed()) return 0;
   a.tag = cluster_call_tag(st, a.cw);
   const dim3 grid(static_cast<unsigned>(nc * M));
   if (BWD && affine) hipLaunchKernelGGL((ln_bwd_stream<T, true>), grid, dim3(kLnStreamThreads), 0, st, a);

@@ -202,6 +202,7 @@ static int sm_fwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, 
     if (ncl < 1) return -1;                                                                      \
     ncl = cluster_count(rows, ncl, cp.M);                                                        \
     ClusterLaunchGuard guard(st);                                                                \
+    if (guard.failed()) return -1;                                                               \
     const SmClusterArgs a{x, nullptr, y, ldx, 0, ldy, map, rows, static_cast<unsigned>(units),   \
                           n, cp.M, cw, cluster_call_tag(st, cw)};                                \
     hipLaunchKernelGGL((sm_fwd_cluster<VV, KIND, W, FR>), dim3(static_cast<unsigned>(ncl * cp.M)), \
@@ -229,6 +230,7 @@ static int sm_bwd_cluster_launch(hipStream_t st, ClusterPlan cp, int64_t units, 
     if (ncl < 1) return -1;                                                                      \
     ncl = cluster_count(rows, ncl, cp.M);                                                        \
     ClusterLaunchGuard guard(st);                                                                \
+    if (guard.failed()) return -1;                                                               \
     const SmClusterArgs a{y, dy, dx, ldy, lddy, lddx, map, rows, static_cast<unsigned>(units),   \
                           n, cp.M, cw, cluster_call_tag(st, cw)};                                \
     hipLaunchKernelGGL((sm_bwd_cluster<VV, KIND, W, FR>), dim3(static_cast<unsigned>(ncl * cp.M)), \
@@ -776,8 +778,10 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxDevices = 64;
 
+size_t static_scratch_bytes() { return kStaticScratchBytes; }
+
 // Device address of `scratch` on the current device; *out stays null on failure.
-static int static_scratch_address(void** out)
+int static_scratch_address(void** out)
 {
   static std::mutex mu;
   static void* address[kMaxDevices] = {};
@@ -843,6 +847,33 @@ int lbn_softmax_fwd_static_scratch_f32(lbn_stream_t stream, int64_t height, int6
   const int status = static_scratch_address(&ptr);
   if (status != LBN_OK) return status;
   return sm_fwd<kSoftmax>(as_stream(stream), 1, height, height, width, x, ldx, y, ldy, ptr, kStaticScratchBytes);
+}
+
+int lbn_softmax_fwd_static_scratch_prepare(void)
+{
+  void* ptr = nullptr;
+  return static_scratch_address(&ptr);
+}
+
+int lbn_softmax_fwd_static_scratch_timed_out(lbn_stream_t stream, int* timed_out)
+{
+  if (!timed_out) return LBN_ERR_INVALID_ARGUMENT;
+  *timed_out = 0;
+  void* ptr = nullptr;
+  const int status = static_scratch_address(&ptr);
+  if (status != LBN_OK) return status;
+  hipStream_t st = as_stream(stream);
+  int word = 0;
+  hipError_t e = hipMemcpyAsync(&word, ptr, sizeof(int), hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (word == kClusterTimedOut) {
+    *timed_out = 1;
+    e = hipMemsetAsync(ptr, 0, sizeof(int), st);  // read and cleared: the next call starts afresh
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return static_cast<int>(e);
+  }
+  return LBN_OK;
 }
 
 int lbn_log_softmax_fwd_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* x,

@@ -43,7 +43,8 @@ def test_wait_gives_up_sets_the_flag_and_the_kernel_ends(L):
     ws[:64].zero_()
     assert _flag(L, ws) == 0
     # rejected arguments launch nothing
-    assert lib.lbn_selftest_cluster_wait_gives_up(L._stream(), None, 4096, 64, L.capi.vp(out.data_ptr())) == L.capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_selftest_cluster_wait_gives_up(L._stream(), L.capi.vp(ws.data_ptr()), 4096, 64, None) == L.capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_selftest_cluster_wait_gives_up(L._stream(), L.capi.vp(ws.data_ptr()), 4096, 0, L.capi.vp(out.data_ptr())) == L.capi.LBN_ERR_INVALID_ARGUMENT
     assert lib.lbn_selftest_cluster_wait_gives_up(L._stream(), L.capi.vp(ws.data_ptr()), 64, 64, L.capi.vp(out.data_ptr())) == L.capi.LBN_ERR_WORKSPACE
 
 

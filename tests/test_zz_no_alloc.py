@@ -3,6 +3,8 @@ the library's code object) against lbn_softmax_fwd_f32 with a caller-provided wo
 the same kernels on the same inputs, so the outputs must agree bit for bit.  Two calls in
 a row on one GPU share the array, the second with a smaller input; both shapes take the
 paths that use scratch (partial sums of the split kernels, cluster slots)."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -69,3 +71,33 @@ def test_static_scratch_softmax_rejects_what_does_not_fit(L):
     xd, yd = L.DeviceMatrix.from_numpy(x), L.DeviceMatrix(1024, 7)
     L.call("lbn_softmax_fwd_static_scratch_f32", L._stream(), 1024, 7, xd.Buffer(), xd.ldim, yd.Buffer(), yd.ldim)
     check("static scratch softmax 1024x7", yd.to_numpy(), orc.softmax_fwd(x))
+
+
+def _static_flag(L):
+    flag = ctypes.c_int(-1)
+    L.call("lbn_softmax_fwd_static_scratch_timed_out", L._stream(), flag)
+    return flag.value
+
+
+def test_static_scratch_wait_that_gives_up_is_seen_and_cleared(L):
+    """The bounded waits' sticky word lives in the library-owned array on this path: the
+    host-driven give-up (one member of a cluster of two, a budget of a few polls; the kernel
+    exits normally) raises it there, the dedicated call reads and clears it, and the entry
+    point works as before afterwards."""
+    lib = L.capi.lib()
+    assert lib.lbn_softmax_fwd_static_scratch_prepare() == 0
+    assert lib.lbn_softmax_fwd_static_scratch_prepare() == 0     # again: harmless
+    assert _static_flag(L) == 0
+    out = torch.full((4,), float("nan"), device="cuda")
+    # NULL workspace = the library's own array
+    L.call("lbn_selftest_cluster_wait_gives_up", L._stream(), None, 0, 32, L.capi.vp(out.data_ptr()))
+    torch.cuda.synchronize()
+    assert out.cpu().tolist() == [1.0, 2.0, -1.0, -1.0]
+    assert _static_flag(L) == 1      # seen ...
+    assert _static_flag(L) == 0      # ... and cleared by that read
+    assert lib.lbn_softmax_fwd_static_scratch_timed_out(L._stream(), None) == L.capi.LBN_ERR_INVALID_ARGUMENT
+    rng = np.random.default_rng(0x4C42000C)
+    x = np.asfortranarray((2.0 * rng.standard_normal((8, 100000), dtype=np.float32)).T)
+    got, ref = _pair(L, x)
+    assert got.tobytes() == ref.tobytes()
+    assert _static_flag(L) == 0
