@@ -92,6 +92,19 @@ typedef void* lbn_stream_t; /* a hipStream_t; NULL is the default stream */
  * cancellation error. */
 #define LBN_STATS_TWO_PASS 0
 #define LBN_STATS_SUMSQ 1
+/* LBN_STATS_REFERENCE_ORDER: for parity tests only, never a default.  The statistics are
+ * formed as the reference CPU code forms them: ONE sequential fp32 sum of x and of x*x
+ * per row (layer norm, layer_norm.cpp:77-88) or per channel (batch norm, columns outer,
+ * rows inner, batch_normalization.cpp:70-85), separate multiplications and additions,
+ * then the reference's expression for mean and variance operation for operation.  Mean
+ * and variance then equal the CPU code's bit for bit, which shows that the order of
+ * summation is all that separates the default modes from it.  One lane per row or
+ * channel does the adding: thousands of times slower than the default, and rejected with
+ * LBN_ERR_UNSUPPORTED for tensors of more than 2^27 entries.  The layer-norm output is
+ * written with the reference's operations as well; batch norm applies the statistics
+ * with the kernel that inference uses.  lbn_batch_norm_bwd_reference_order_f32 is the
+ * matching backward. */
+#define LBN_STATS_REFERENCE_ORDER 2
 
 int lbn_version(void);
 const char* lbn_status_string(int status);
@@ -300,6 +313,21 @@ int lbn_batch_norm_bwd_f32(lbn_stream_t stream, int64_t channels, int64_t channe
                            const float* scale, float* dscale, float* dbias,
                            float* dmean, float* dvar,
                            void* workspace, size_t workspace_bytes);
+/* For parity tests only: lbn_batch_norm_bwd_f32 with the four per-channel gradients
+ * accumulated as the reference CPU code does (batch_normalization.cpp:211-245: one
+ * sequential fp32 sum each per channel, columns outer, rows inner, the reference's
+ * per-entry expressions without fused multiply-adds), then the ordinary dx kernel on
+ * those values.  With the statistics of an LBN_STATS_REFERENCE_ORDER forward, dscale,
+ * dbias, dmean and dvar equal the CPU code's bit for bit.  Same arguments, workspace and
+ * size limit (2^27 entries) as described for that flag. */
+int lbn_batch_norm_bwd_reference_order_f32(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                           int64_t width, int bessel, float epsilon, int training,
+                                           const float* x, int64_t ldx, const float* dy, int64_t lddy,
+                                           float* dx, int64_t lddx, const float* mean, const float* var,
+                                           const float* running_mean, const float* running_var,
+                                           const float* scale, float* dscale, float* dbias,
+                                           float* dmean, float* dvar,
+                                           void* workspace, size_t workspace_bytes);
 int lbn_batch_norm_fwd_f16(lbn_stream_t stream, int64_t channels, int64_t channel_size,
                            int64_t width, int bessel, float epsilon, float decay,
                            int training, const void* x, int64_t ldx, void* y, int64_t ldy,

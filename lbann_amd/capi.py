@@ -20,6 +20,7 @@ LBN_ERR_WORKSPACE = -2
 LBN_ERR_UNSUPPORTED = -3
 LBN_STATS_TWO_PASS = 0
 LBN_STATS_SUMSQ = 1
+LBN_STATS_REFERENCE_ORDER = 2
 
 # name -> (restype, argtypes); mirrors include/lbnorm.h declaration by declaration
 PROTOTYPES = {
@@ -48,6 +49,8 @@ PROTOTYPES = {
                                       vp, vp, vp, vp, vp, sz, cint]),
     "lbn_batch_norm_bwd_f32": (cint, [vp, i64, i64, i64, cint, f32, cint, vp, i64, vp, i64, vp, i64, vp,
                                       vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]),
+    "lbn_batch_norm_bwd_reference_order_f32": (cint, [vp, i64, i64, i64, cint, f32, cint, vp, i64, vp, i64, vp, i64, vp,
+                                                      vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]),
     "lbn_batch_norm_fwd_f16": (cint, [vp, i64, i64, i64, cint, f32, f32, cint, vp, i64, vp, i64, vp, vp,
                                       vp, vp, vp, vp, vp, sz, cint]),
     "lbn_batch_norm_bwd_f16": (cint, [vp, i64, i64, i64, cint, f32, cint, vp, i64, vp, i64, vp, i64, vp,

@@ -28,6 +28,7 @@
 #include "batch_norm_math.hpp"
 #include "batch_norm_rows.hpp"
 #include "batch_norm_stream.hpp"
+#include "reference_order.hpp"
 
 namespace lbn {
 
@@ -1241,6 +1242,23 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   const dim3 grid(static_cast<unsigned>(C), P);
   const int pivot = (flags & LBN_STATS_SUMSQ) ? 0 : 1;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, y, ldy);
+  if (flags & LBN_STATS_REFERENCE_ORDER) {
+    // parity tests only: the statistics as one sequential fp32 sum per channel, then the apply
+    // kernel that inference uses, on those statistics
+    if (C * cs > kRefOrderMaxEntries / w || C > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+    if constexpr (std::is_same<S, f16x4>::value) return LBN_ERR_UNSUPPORTED;  // callers pass plain halves
+    else {
+      hipLaunchKernelGGL(bn_ref_order_fwd_stats<S>, dim3(static_cast<unsigned>(C)), dim3(kWave), 0, st, x, ldx, cs, w,
+                         bessel, epsilon, decay, mean, var, running_mean, running_var);
+      if (vec)
+        hipLaunchKernelGGL((bn_fwd_apply<S, true, false>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs, w, 0,
+                           bessel, epsilon, decay, part, mean, var, scale, bias, running_mean, running_var);
+      else
+        hipLaunchKernelGGL((bn_fwd_apply<S, false, false>), grid, dim3(kBnThreads), 0, st, x, y, ldx, ldy, cs, w, 0,
+                           bessel, epsilon, decay, part, mean, var, scale, bias, running_mean, running_var);
+      return launch_status();
+    }
+  }
   if constexpr (Vec16<S>::N == 4) {  // float or fp16 in fours: the row-tile kernels
     // channels of three or four vectors: the register tile when the mini-batch fits it
     // (1024 x 16, w = 256: 19 us per step against 25 us for clusters), else clusters
@@ -1309,7 +1327,8 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
                        int training, const S* x, int64_t ldx, const S* dy, int64_t lddy, S* dx,
                        int64_t lddx, const float* mean, const float* var, const float* running_mean,
                        const float* running_var, const float* scale, float* dscale, float* dbias,
-                       float* dmean, float* dvar, void* workspace, size_t workspace_bytes)
+                       float* dmean, float* dvar, void* workspace, size_t workspace_bytes,
+                       bool reference_order = false)
 {
   const int64_t lds[3] = {ldx, lddy, lddx};
   if (int e = bn_check(C, cs, w, lds, 3)) return e;
@@ -1324,6 +1343,25 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
   const dim3 grid(static_cast<unsigned>(C), P);
   const int64_t n = cs * w;
   const bool vec = bn_vec_ok<S>(cs, w, x, ldx) && bn_vec_ok<S>(cs, w, dy, lddy) && bn_vec_ok<S>(cs, w, dx, lddx);
+  if (reference_order) {
+    // parity tests only: the four gradients as sequential fp32 sums per channel, then the apply
+    // kernel of the several-rank cut, which takes dmean and dvar as inputs
+    if (C * cs > kRefOrderMaxEntries / w || C > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+    if constexpr (std::is_same<S, f16x4>::value) return LBN_ERR_UNSUPPORTED;
+    else {
+      hipLaunchKernelGGL(bn_ref_order_bwd_sums<S>, dim3(static_cast<unsigned>(C)), dim3(kWave), 0, st, x, dy, ldx, lddy,
+                         cs, w, epsilon, training, use_mean, use_var, scale, dscale, dbias, dmean, dvar);
+      if (vec)
+        hipLaunchKernelGGL((bn_bwd_apply<S, true, false>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy, lddx,
+                           cs, w, n, bessel, epsilon, training, part, use_mean, use_var, scale, dscale, dbias, dmean,
+                           dvar);
+      else
+        hipLaunchKernelGGL((bn_bwd_apply<S, false, false>), grid, dim3(kBnThreads), 0, st, x, dy, dx, ldx, lddy, lddx,
+                           cs, w, n, bessel, epsilon, training, part, use_mean, use_var, scale, dscale, dbias, dmean,
+                           dvar);
+      return launch_status();
+    }
+  }
   if constexpr (Vec16<S>::N == 4) {  // float or fp16 in fours: the row-tile kernels
     if (!bn_rt_shape(cs) && cs <= kBnTileMaxCs && row_quads_ok(C * cs, w, x, ldx, sizeof(S)) && row_quads_ok(C * cs, w, dy, lddy, sizeof(S)) &&
         row_quads_ok(C * cs, w, dx, lddx, sizeof(S))) {
@@ -1473,7 +1511,7 @@ int lbn_batch_norm_fwd_f16(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
                            const float* bias, float* running_mean, float* running_var,
                            void* workspace, size_t workspace_bytes, int flags)
 {
-  if (C > 0 && cs > 0 && w > 0 && bn_f16_in_fours(C, cs, w, {{x, ldx}, {y, ldy}}))
+  if (C > 0 && cs > 0 && w > 0 && !(flags & LBN_STATS_REFERENCE_ORDER) && bn_f16_in_fours(C, cs, w, {{x, ldx}, {y, ldy}}))
     return bn_fwd_host<f16x4>(as_stream(stream), C, cs, w, bessel, epsilon, decay, training,
                               static_cast<const f16x4*>(x), ldx, static_cast<f16x4*>(y), ldy, mean, var,
                               scale, bias, running_mean, running_var, workspace, workspace_bytes, flags);
@@ -1544,6 +1582,19 @@ int lbn_batch_norm_bwd_f32(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
   return bn_bwd_host<float>(as_stream(stream), C, cs, w, bessel, epsilon, training, x, ldx, dy, lddy, dx, lddx,
                             mean, var, running_mean, running_var, scale, dscale, dbias, dmean, dvar, workspace,
                             workspace_bytes);
+}
+
+int lbn_batch_norm_bwd_reference_order_f32(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w, int bessel,
+                                           float epsilon, int training, const float* x, int64_t ldx,
+                                           const float* dy, int64_t lddy, float* dx, int64_t lddx,
+                                           const float* mean, const float* var, const float* running_mean,
+                                           const float* running_var, const float* scale, float* dscale,
+                                           float* dbias, float* dmean, float* dvar, void* workspace,
+                                           size_t workspace_bytes)
+{
+  return bn_bwd_host<float>(as_stream(stream), C, cs, w, bessel, epsilon, training, x, ldx, dy, lddy, dx, lddx,
+                            mean, var, running_mean, running_var, scale, dscale, dbias, dmean, dvar, workspace,
+                            workspace_bytes, true);
 }
 
 int lbn_batch_norm_bwd_f16(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w, int bessel,

@@ -30,6 +30,7 @@
 #include "host_utils.hpp"
 #include "layer_norm_cluster.hpp"
 #include "layer_norm_long.hpp"
+#include "reference_order.hpp"
 
 namespace lbn {
 
@@ -1199,6 +1200,13 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                    rows_aligned16(y, stride, ldy, G, w, sizeof(T)) &&
                    (!gamma || aligned16(gamma)) && (!beta || aligned16(beta));
   const float inv_n = 1.0f / static_cast<float>(n);
+  if (flags & LBN_STATS_REFERENCE_ORDER) {
+    // parity tests only: one sequential fp32 sum per row, in the reference's order
+    if (rows > kRefOrderMaxEntries / n) return LBN_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((ln_ref_order_fwd<T, RowMap>), dim3(static_cast<unsigned>(rows)), dim3(kWave), 0, st, x, y, ldx,
+                       ldy, map, n, eps, stats, lds, gamma, beta);
+    return launch_status();
+  }
   if (n == 1) {
     const int64_t want = ceil_div(rows, 256);
     hipLaunchKernelGGL((ln_fwd_single<T>), dim3(static_cast<unsigned>(want > 8192 ? 8192 : want)), dim3(256), 0, st, x,

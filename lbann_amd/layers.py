@@ -20,7 +20,7 @@ import numpy as np
 import torch
 
 from . import capi
-from .capi import LBN_STATS_SUMSQ, LBN_STATS_TWO_PASS, LbnError, call  # noqa: F401
+from .capi import LBN_STATS_REFERENCE_ORDER, LBN_STATS_SUMSQ, LBN_STATS_TWO_PASS, LbnError, call  # noqa: F401
 
 
 def _prod(xs):
@@ -451,7 +451,10 @@ class batch_normalization_layer(_Layer):
         x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
         C, cs = self.num_channels, self.channel_size
         ws, nb = self._ws.get(capi.lib().lbn_batch_norm_workspace_bytes(C, cs, x.width), self.device)
-        return (f"lbn_batch_norm_bwd_{'f16' if x.dtype == torch.float16 else 'f32'}",
+        name = f"lbn_batch_norm_bwd_{'f16' if x.dtype == torch.float16 else 'f32'}"
+        if self.stats_mode & LBN_STATS_REFERENCE_ORDER:  # parity tests: the reference's order of summation
+            name = "lbn_batch_norm_bwd_reference_order_f32"
+        return (name,
                 (_stream(), C, cs, x.width, int(self.m_bessel_correction),
                  self.m_epsilon, int(self.training), x.Buffer(), x.ldim, dy.Buffer(), dy.ldim, dx.Buffer(),
                  dx.ldim, self._col(self.m_mean_and_var, 0), self._col(self.m_mean_and_var, 1),

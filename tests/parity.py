@@ -42,8 +42,10 @@ def rel_err(a, b):
 REPORT = []
 
 
-def check(name, got, ref32, exact64=None, tol=TOL_F32, slack=1.0):
+def check(name, got, ref32, exact64=None, tol=TOL_F32, slack=1.0, strict=False):
     """Returns the dict of measured errors; raises AssertionError when the gate fails.
+
+    strict: only the fp32-reference leg counts (the float64 distances are still recorded).
 
     The dict names the leg that passed: "fp32 reference" (within `tol` of the restated
     reference) or "float64" (at least as close to the float64 evaluation as the fp32
@@ -57,7 +59,7 @@ def check(name, got, ref32, exact64=None, tol=TOL_F32, slack=1.0):
     REPORT.append(out)
     if e_ref <= tol:
         return out
-    assert exact64 is not None, f"{name}: err vs fp32 reference {e_ref:.3e} > {tol:.1e}"
+    assert exact64 is not None and not strict, f"{name}: err vs fp32 reference {e_ref:.3e} > {tol:.1e}"
     e_exact, e_ref_exact = out["vs_exact"], out["ref_vs_exact"]
     assert e_exact <= max(tol, slack * e_ref_exact), (
         f"{name}: err vs fp32 reference {e_ref:.3e} > {tol:.1e} and err vs float64 "

@@ -119,6 +119,100 @@ def test_cfg3_batch_norm_64x256x56x56(L, W, bessel):
     assert np.abs(ym - d["bias"]).max() < 1e-5
 
 
+@pytest.mark.parametrize("bessel", [True, False])
+def test_cfg3_batch_norm_reference_order_meets_the_strict_gate(L, W, bessel):
+    """cfg3 with the statistics and the four per-channel gradients summed in the reference's
+    order (one sequential fp32 sum per channel): what the tree-summing default is judged
+    through float64 for, agrees here with the fp32 reference itself.  The per-channel values
+    bit for bit, the tensors within 1e-5 through the fp32 leg alone."""
+    d = W.cfg3_batch_norm()
+    x, dy = f32(d["x"]), f32(d["dy"])
+    C, cs = 256, 56 * 56
+    bn = L.batch_normalization_layer(d["dims"], d["decay"], d["eps"], bessel, d["scale"], d["bias"],
+                                     stats_mode=L.LBN_STATS_REFERENCE_ORDER)
+    y = bn.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    dx = bn.backward(L.DeviceMatrix.from_numpy(dy)).to_numpy()
+    mv, mvg = bn.m_mean_and_var.to_numpy(), bn.m_mean_and_var_gradient.to_numpy()
+    out = dict(y=y, dx=dx, mean=mv[:, 0], var=mv[:, 1], dmean=mvg[:, 0], dvar=mvg[:, 1],
+               dscale=bn.m_scale_gradient.to_numpy(), dbias=bn.m_bias_gradient.to_numpy(),
+               rmean=bn.weights[2].to_numpy(), rvar=bn.weights[3].to_numpy())
+    del bn
+    torch.cuda.empty_cache()
+    res = {}
+    for tag, conv in (("ref", f32), ("ex", f64)):
+        rm, rv = conv(np.zeros(C)), conv(np.ones(C))
+        r = {}
+        r["y"], r["mean"], r["var"] = orc.batch_norm_fwd(conv(x), C, cs, 1e-5, 0.9, conv(d["scale"]), conv(d["bias"]), rm, rv, bessel)
+        r["rmean"], r["rvar"] = rm, rv
+        r["dx"], r["dscale"], r["dbias"], r["dmean"], r["dvar"] = orc.batch_norm_bwd(
+            conv(x), conv(dy), C, cs, 1e-5, r["mean"], r["var"], conv(d["scale"]), bessel=bessel)
+        res[tag] = r
+    tagb = "bessel" if bessel else "no bessel"
+    for k in out:
+        check(f"cfg3 ({tagb}) reference-order {k}", out[k], res["ref"][k], res["ex"][k], strict=True)
+    for k in ("mean", "var", "rmean", "rvar", "dscale", "dbias", "dmean", "dvar"):
+        assert np.asarray(out[k], np.float32).tobytes() == np.asarray(res["ref"][k], np.float32).tobytes(), \
+            f"{k}: not bit-equal to the fp32 reference"
+
+
+def test_cfg4_layer_norm_reference_order_meets_the_strict_gate(L, W):
+    """cfg4 with each row's sums formed sequentially in fp32 as the reference forms them: the
+    statistics (E[x^2] - mean^2 with its cancellation for |mean| >> stdev rows included) equal
+    the fp32 reference's bit for bit, y and every backward tensor computed from those
+    statistics agree with the fp32 reference through the fp32 leg alone."""
+    d = W.cfg4_layer_norm_f16()
+    x16, dy16 = d["x"], d["dy"]
+    x, dy = f32(x16), f32(dy16)
+    n = 4096
+    ln = L.layer_norm_layer(d["dims"], d["eps"], True, True, 0, d["scale"], d["bias"],
+                            stats_mode=L.LBN_STATS_REFERENCE_ORDER)
+    y = ln.forward(L.DeviceMatrix.from_numpy(x16)).to_numpy()
+    dx = ln.backward(L.DeviceMatrix.from_numpy(dy16)).to_numpy()
+    stats, sgrad = ln.m_statistics.to_numpy(), ln.m_statistics_gradient.to_numpy()
+    dg, db = ln.m_scale_gradient.to_numpy(), ln.m_bias_gradient.to_numpy()
+    y_ref, st = orc.layer_norm_fwd(x, 1, n, n, 1e-5, d["scale"], d["bias"])
+    assert stats.tobytes() == st.tobytes(), "statistics are not bit-equal to the fp32 reference"
+    check("cfg4 reference-order mean", stats[0], st[0], strict=True)
+    check("cfg4 reference-order var", stats[1], st[1], strict=True)
+    check("cfg4 reference-order y", y, y_ref, tol=TOL_F16, strict=True)
+    dx_own, sg_own, dg_own, db_own = orc.layer_norm_bwd(x, dy, st, 1, n, n, 1e-5, d["scale"], True, True)
+    # the reference's variance is 0 (clamped) for rows with |mean| >> stdev, so 1/stdev = 316 and
+    # some gradients exceed binary16's range: the GPU stores them as infinities, which is what
+    # the reference's value becomes in that storage type as well
+    with np.errstate(over="ignore"):
+        dx_own16 = f32(dx_own.astype(np.float16))
+    assert np.isinf(dx_own16).sum() < dx_own16.size // 100
+    check("cfg4 reference-order dx", dx, dx_own16, tol=TOL_F16, strict=True)
+    check("cfg4 reference-order stats grad", sgrad, sg_own, tol=TOL_F16, strict=True)
+    check("cfg4 reference-order dscale", dg, dg_own, tol=TOL_F16, strict=True)
+    check("cfg4 reference-order dbias", db, db_own, tol=TOL_F16, strict=True)
+
+
+def test_reference_order_mode_rejects_large_tensors(L):
+    """The mode is for parity tests: above 2^27 entries it is refused before any launch (the
+    small buffers passed here are never touched)."""
+    lib = L.capi.lib()
+    small = L.DeviceMatrix(16, 1)
+    ws = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    p, wp = small.Buffer(), L.capi.vp(ws.data_ptr())
+    st = L._stream()
+    limit = 1 << 27
+    rows = limit // 4096 + 1
+    assert 4096 * rows > limit   # the calls below must be refused: their buffers are tiny
+    assert lib.lbn_layer_norm_fwd_f32(st, 1, 4096, 4096, rows, 1e-5, p, 4096, p, 4096, p, 2, None, None,
+                                      None, 0, L.LBN_STATS_REFERENCE_ORDER) == L.capi.LBN_ERR_UNSUPPORTED
+    h = 64 * 4096
+    wb = limit // h + 1
+    assert h * wb > limit
+    need = lib.lbn_batch_norm_workspace_bytes(64, 4096, wb)
+    ws = torch.zeros(max(need, 64), dtype=torch.uint8, device="cuda")
+    wp = L.capi.vp(ws.data_ptr())
+    assert lib.lbn_batch_norm_fwd_f32(st, 64, 4096, wb, 1, 1e-5, 0.9, 1, p, h, p, h, p, p, p, p, p, p, wp,
+                                      ws.numel(), L.LBN_STATS_REFERENCE_ORDER) == L.capi.LBN_ERR_UNSUPPORTED
+    assert lib.lbn_batch_norm_bwd_reference_order_f32(st, 64, 4096, wb, 1, 1e-5, 1, p, h, p, h, p, h, p, p, p,
+                                                      p, p, p, p, p, p, wp, ws.numel()) == L.capi.LBN_ERR_UNSUPPORTED
+
+
 def test_cfg4_layer_norm_f16_4096x8192(L, W):
     d = W.cfg4_layer_norm_f16()
     x16, dy16 = d["x"], d["dy"]

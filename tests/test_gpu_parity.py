@@ -1207,3 +1207,81 @@ def test_cluster_kernels_from_two_host_threads_on_the_per_thread_stream(L, monke
         assert np.array_equal(y.to_numpy(), sm_ref)
     for y in yb:
         assert np.array_equal(y.to_numpy(), bn_ref)
+
+
+# ---------------------------------------------------------------- the reference's summation order
+def _bits_equal(name, a, b):
+    a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)
+    assert a.shape == b.shape and a.tobytes() == b.tobytes(), \
+        f"{name}: not bit-equal to the fp32 reference (max abs difference {np.abs(a - b).max():.3e})"
+
+
+@pytest.mark.parametrize("dims,w,bessel,pad,half", [
+    ((8, 16, 16), 12, True, 0, False), ((7, 5, 3), 14, False, 0, False), ((5, 24), 10, True, 8, False),
+    ((3, 1001), 7, True, 3, False), ((4, 1), 1, True, 0, False), ((6, 1), 33, True, 0, False),
+    ((16, 14, 14), 9, True, 0, True), ((5, 7, 7), 20, False, 1, True)])
+def test_batch_norm_reference_order_is_bit_equal(L, dims, w, bessel, pad, half):
+    """LBN_STATS_REFERENCE_ORDER: statistics and the four per-channel gradients equal the
+    restated CPU code's bit for bit (any alignment, channel size, fp16 storage; a channel of
+    one entry in all keeps the reference's special case)."""
+    rng = np.random.default_rng(int(np.prod(dims)) * 31 + w)
+    h = int(np.prod(dims))
+    x, dy = rand(rng, h, w, 2.0, 3.0), rand(rng, h, w)
+    if half:
+        x, dy = f32(x.astype(np.float16)), f32(dy.astype(np.float16))
+    C = dims[0]
+    scale = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    cs = h // C
+    layer = L.batch_normalization_layer(dims, 0.9, 1e-5, bessel, scale, bias, stats_mode=L.LBN_STATS_REFERENCE_ORDER)
+    tdt = torch.float16 if half else torch.float32
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, dtype=tdt, ldim=h + pad)).to_numpy()
+    mv = layer.m_mean_and_var.to_numpy()
+    rm, rv = np.zeros(C, np.float32), np.ones(C, np.float32)
+    y_ref, m_ref, v_ref = orc.batch_norm_fwd(x, C, cs, 1e-5, 0.9, scale, bias, rm, rv, bessel)
+    _bits_equal("mean", mv[:, 0], m_ref)
+    _bits_equal("var", mv[:, 1], v_ref)
+    _bits_equal("running mean", layer.weights[2].to_numpy(), rm)
+    _bits_equal("running var", layer.weights[3].to_numpy(), rv)
+    check(f"batch_norm reference-order y dims={dims}", y, y_ref, tol=TOL_F16 if half else TOL_F32)
+    if half:
+        return  # the backward of this mode is fp32 only
+    dx = layer.backward(L.DeviceMatrix.from_numpy(dy, ldim=h + pad)).to_numpy()
+    mvg = layer.m_mean_and_var_gradient.to_numpy()
+    dx_ref, dg_ref, db_ref, dm_ref, dv_ref = orc.batch_norm_bwd(x, dy, C, cs, 1e-5, m_ref, v_ref, scale, bessel=bessel)
+    _bits_equal("dscale", layer.m_scale_gradient.to_numpy(), dg_ref)
+    _bits_equal("dbias", layer.m_bias_gradient.to_numpy(), db_ref)
+    _bits_equal("dmean", mvg[:, 0], dm_ref)
+    _bits_equal("dvar", mvg[:, 1], dv_ref)
+    check(f"batch_norm reference-order dx dims={dims}", dx, dx_ref)
+
+
+@pytest.mark.parametrize("dims,start_dim,w,affine,pad,half", [
+    ((1024,), 0, 64, True, 0, False), ((31,), 0, 15, False, 0, False), ((8, 512), -1, 9, True, 5, False),
+    ((1,), 0, 6, True, 0, False), ((3, 777), 1, 11, True, 1, False), ((2, 4096), 1, 33, True, 0, True),
+    ((1001,), 0, 17, False, 3, True)])
+def test_layer_norm_reference_order_is_bit_equal(L, dims, start_dim, w, affine, pad, half):
+    """LBN_STATS_REFERENCE_ORDER: mean, variance and y equal the restated CPU code's bit for
+    bit (fp16 storage: y equal after rounding to binary16); columns with |mean| >> stdev keep
+    the reference's cancellation."""
+    rng = np.random.default_rng(int(np.prod(dims)) * 17 + w)
+    h = int(np.prod(dims))
+    x = rand(rng, h, w, 0.3, 1.5)
+    x[:, ::3] += 300.0   # E[x^2] - mean^2 cancels in fp32 here
+    x = np.asfortranarray(x)
+    if half:
+        x = f32(x.astype(np.float16))
+    n = int(np.prod(dims[(start_dim if start_dim >= 0 else len(dims) + start_dim):]))
+    scale = (1 + 0.3 * rng.standard_normal(n)).astype(np.float32)
+    bias = (0.3 * rng.standard_normal(n)).astype(np.float32)
+    kw = dict(scale_values=scale, bias_values=bias) if affine else {}
+    layer = L.layer_norm_layer(dims, 1e-5, affine, affine, start_dim, stats_mode=L.LBN_STATS_REFERENCE_ORDER, **kw)
+    G = layer.num_normalized
+    tdt = torch.float16 if half else torch.float32
+    y = layer.forward(L.DeviceMatrix.from_numpy(x, dtype=tdt, ldim=h + pad)).to_numpy()
+    y_ref, st_ref = orc.layer_norm_fwd(x, G, n, n, 1e-5, scale if affine else None, bias if affine else None)
+    _bits_equal("statistics", layer.m_statistics.to_numpy(), st_ref)
+    if half:
+        _bits_equal("y", f32(y), f32(y_ref.astype(np.float16)))
+    else:
+        _bits_equal("y", y, y_ref)
