@@ -3,6 +3,7 @@
     python3 -m lbann_amd.rocprof_summary trace STATS.db [--fetch FETCH.db --write WRITE.db]
                                                [--headline-json OUT.json] [--command "..."]...
     python3 -m lbann_amd.rocprof_summary counters PMC.db [PMC2.db ...] [--match SUBSTR]... [--command "..."]...
+    python3 -m lbann_amd.rocprof_summary sequence STATS.db --match SUBSTR [--match SUBSTR]... [--command "..."]...
 
 `trace` prints one markdown table row per (kernel, grid) of a `rocprofv3 --kernel-trace --stats`
 database: calls, average and minimum duration, and, for the kernels of the benchmark
@@ -11,7 +12,9 @@ databases of two counter runs (`--pmc FETCH_SIZE`, `--pmc WRITE_SIZE`) it adds t
 crossed the fabric per launch, each counter scaled by what it reads for the plain 256 MiB copy
 kernel that `bench.py --copy-calibration` runs in the same process.  `counters` prints the average
 per dispatch of every collected counter for the kernels whose name contains one of the --match
-strings.  Both write to stdout; `--command` lines are quoted at the top so that a summary names
+strings.  `sequence` splits the dispatches of the matching kernels by the kernel that ran on the
+device immediately before them (what a kernel finds in the caches depends on its predecessor).
+All write to stdout; `--command` lines are quoted at the top so that a summary names
 the commands that produced it.
 """
 import argparse
@@ -221,6 +224,30 @@ def counters(args):
             print(f"* `{_short(kernel)}`: " + "; ".join(notes))
 
 
+def sequence(args):
+    rows = _rows(args.db, "select name, grid_x / workgroup_x, start, end from kernels order by start")
+    print("# rocprofv3 kernel trace, dispatches split by the kernel that ran before them\n")
+    if args.command:
+        print("Commands (from /tmp with TMPDIR=/tmp on the MI355X box; $R is the repository):\n")
+        for c in args.command:
+            print(f"    {c}")
+        print()
+    groups = {}
+    for i, (name, wgs, start, end) in enumerate(rows):
+        if not any(m in name for m in args.match):
+            continue
+        prev = _short(rows[i - 1][0]) if i else "(first kernel of the process)"
+        gap = (start - rows[i - 1][3]) / 1e3 if i else 0.0
+        groups.setdefault((_short(name), int(wgs), prev), []).append(((end - start) / 1e3, gap))
+    print("| kernel | workgroups | ran after | calls | avg us | median us | min us | max us | median gap to predecessor us |")
+    print("|---|---|---|---|---|---|---|---|---|")
+    for (name, wgs, prev), v in sorted(groups.items(), key=lambda kv: (kv[0][0], -len(kv[1]))):
+        d = sorted(x[0] for x in v)
+        g = sorted(x[1] for x in v)
+        print(f"| `{name}` | {wgs} | `{prev}` | {len(d)} | {sum(d) / len(d):.2f} | {d[len(d) // 2]:.2f} | {d[0]:.2f} | "
+              f"{d[-1]:.2f} | {g[len(g) // 2]:.2f} |")
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="mode", required=True)
@@ -236,6 +263,11 @@ def main():
     c.add_argument("--match", action="append", default=[])
     c.add_argument("--command", action="append", default=[])
     c.set_defaults(fn=counters)
+    q = sub.add_parser("sequence")
+    q.add_argument("db")
+    q.add_argument("--match", action="append", required=True)
+    q.add_argument("--command", action="append", default=[])
+    q.set_defaults(fn=sequence)
     args = ap.parse_args()
     args.fn(args)
 
