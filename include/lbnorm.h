@@ -615,6 +615,66 @@ int lbn_gradient_sink_f32(lbn_stream_t stream, int64_t height, int64_t width, fl
                           float in_scale, const float* contribution, int64_t ld_contribution,
                           float* gradient, int64_t ld_gradient);
 
+/* ------------------------------------------- the five layers for double precision
+ * The reference instantiates its layers for TensorDataType = double when it is built with
+ * LBANN_HAS_DOUBLE (include/lbann/macros/instantiate.hpp:28-30,
+ * src/layers/regularizers/layer_norm_builder.cpp:48-54, batch_normalization_builder.cpp,
+ * softmax.cpp / log_softmax.cpp / channelwise_softmax.cpp instantiations).  These entry points
+ * are the _f32 ones with every matrix, statistic, weight and epsilon in binary64 and all
+ * arithmetic in binary64; arguments mean what they mean there (sizes, leading dimensions in
+ * elements, NULL rules, in-place rules, LBN_STATS_TWO_PASS / LBN_STATS_SUMSQ).  Differences:
+ * the softmax family and the layer-norm forward use no scratch (no workspace arguments);
+ * layer-norm backward needs lbn_layer_norm_bwd_workspace_bytes_f64() only for weight
+ * gradients; batch norm always needs lbn_batch_norm_workspace_bytes_f64() in training mode
+ * and in backward.  Workspaces are 16-byte aligned.  No kernel here waits across workgroups.
+ * Batch norm channels are limited to 2^31 - 1 entries (channel_size * width). */
+int lbn_softmax_fwd_f64(lbn_stream_t stream, int64_t height, int64_t width,
+                        const double* x, int64_t ldx, double* y, int64_t ldy);
+int lbn_softmax_bwd_f64(lbn_stream_t stream, int64_t height, int64_t width,
+                        const double* y, int64_t ldy, const double* dy, int64_t lddy,
+                        double* dx, int64_t lddx);
+int lbn_log_softmax_fwd_f64(lbn_stream_t stream, int64_t height, int64_t width,
+                            const double* x, int64_t ldx, double* y, int64_t ldy);
+int lbn_log_softmax_bwd_f64(lbn_stream_t stream, int64_t height, int64_t width,
+                            const double* y, int64_t ldy, const double* dy, int64_t lddy,
+                            double* dx, int64_t lddx);
+int lbn_channelwise_softmax_fwd_f64(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                    int64_t channel_stride, int64_t width,
+                                    const double* x, int64_t ldx, double* y, int64_t ldy);
+int lbn_channelwise_softmax_bwd_f64(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                    int64_t channel_stride, int64_t width,
+                                    const double* y, int64_t ldy, const double* dy, int64_t lddy,
+                                    double* dx, int64_t lddx);
+int lbn_layer_norm_fwd_f64(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
+                           int64_t norm_stride, int64_t width, double epsilon,
+                           const double* x, int64_t ldx, double* y, int64_t ldy,
+                           double* stats, int64_t ld_stats,
+                           const double* scale, const double* bias, int flags);
+size_t lbn_layer_norm_bwd_workspace_bytes_f64(int64_t num_groups, int64_t norm_size,
+                                              int64_t width, int has_weight_grads);
+int lbn_layer_norm_bwd_f64(lbn_stream_t stream, int64_t num_groups, int64_t norm_size,
+                           int64_t norm_stride, int64_t width, double epsilon,
+                           const double* x, int64_t ldx, const double* dy, int64_t lddy,
+                           double* dx, int64_t lddx, const double* stats, int64_t ld_stats,
+                           double* stats_grad, int64_t ld_stats_grad,
+                           const double* scale, double* dscale, double* dbias,
+                           void* workspace, size_t workspace_bytes);
+size_t lbn_batch_norm_workspace_bytes_f64(int64_t channels, int64_t channel_size, int64_t width);
+int lbn_batch_norm_fwd_f64(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                           int64_t width, int bessel, double epsilon, double decay,
+                           int training, const double* x, int64_t ldx, double* y, int64_t ldy,
+                           double* mean, double* var, const double* scale, const double* bias,
+                           double* running_mean, double* running_var,
+                           void* workspace, size_t workspace_bytes, int flags);
+int lbn_batch_norm_bwd_f64(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                           int64_t width, int bessel, double epsilon, int training,
+                           const double* x, int64_t ldx, const double* dy, int64_t lddy,
+                           double* dx, int64_t lddx, const double* mean, const double* var,
+                           const double* running_mean, const double* running_var,
+                           const double* scale, double* dscale, double* dbias,
+                           double* dmean, double* dvar,
+                           void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -213,13 +213,16 @@ using element_t = std::remove_cv_t<std::remove_pointer_t<decltype(std::declval<M
 }  // namespace detail
 
 // ------------------------------------------------------------------ layer norm
-/// include/lbann/layers/regularizers/layer_norm.hpp:53-143.  T is float, or a 16-bit
-/// storage type (any 2-byte IEEE binary16 type) for the fp16-storage kernels.
+/// include/lbann/layers/regularizers/layer_norm.hpp:53-143.  T is float, a 16-bit
+/// storage type (any 2-byte IEEE binary16 type) for the fp16-storage kernels, or double
+/// (TensorDataType = double: statistics, weights and their gradients are doubles too).
 template <typename T, typename Mat = device_matrix<T>>
 class layer_norm_layer {
 public:
+  /// Type of statistics, weights and weight gradients: float unless the layer is one of doubles.
+  using weight_t = std::conditional_t<sizeof(T) == 8, double, float>;
   layer_norm_layer(double epsilon = 1e-5, bool scale = false, bool bias = false, int start_dim = 0)
-    : m_epsilon(static_cast<float>(epsilon)), m_scale(scale), m_bias(bias), m_start_dim(start_dim) {}
+    : m_epsilon(epsilon), m_scale(scale), m_bias(bias), m_start_dim(start_dim) {}
 
   /// setup_dims + setup_data: fixes the normalised dimensions (layer_norm.hpp:259-290).
   void setup(const std::vector<int64_t>& dims)
@@ -242,12 +245,12 @@ public:
     global_normalization_size = normalization_size;
   }
   /// Weight values (weights_values(i).LockedMatrix().LockedBuffer()) and gradient sinks.
-  void set_weights(const float* scale, const float* bias) { m_scale_w = scale; m_bias_w = bias; }
-  void set_weight_gradients(float* dscale, float* dbias) { m_scale_grad = dscale; m_bias_grad = dbias; }
+  void set_weights(const weight_t* scale, const weight_t* bias) { m_scale_w = scale; m_bias_w = bias; }
+  void set_weight_gradients(weight_t* dscale, weight_t* dbias) { m_scale_grad = dscale; m_bias_grad = dbias; }
 
   layer_io<Mat> io;
-  device_matrix<float> m_statistics;           // 2*num_normalized x width: means, then variances
-  device_matrix<float> m_statistics_gradient;  // same shape: dL/dmean, dL/dvar
+  device_matrix<weight_t> m_statistics;           // 2*num_normalized x width: means, then variances
+  device_matrix<weight_t> m_statistics_gradient;  // same shape: dL/dmean, dL/dvar
   int stats_mode = LBN_STATS_TWO_PASS;
 
   /// layer_norm.cpp:263-290 / layer_norm.cu fp_compute.
@@ -258,21 +261,30 @@ public:
     int64_t n, gn, G, stride;
     get_normdims(n, gn, G, stride);
     m_statistics.Resize(2 * G, x.Width());
-    const float* sw = m_scale ? m_scale_w : nullptr;
-    const float* bw = m_bias ? m_bias_w : nullptr;
-    // scratch is only needed (and only non-zero) for groups of tens of thousands of entries
-    const size_t bytes = lbn_layer_norm_fwd_workspace_bytes(G, n, x.Width(), static_cast<int>(sizeof(T)));
-    void* ws = m_ws.reserve(bytes, io.stream);
+    const weight_t* sw = m_scale ? m_scale_w : nullptr;
+    const weight_t* bw = m_bias ? m_bias_w : nullptr;
     int st;
-    if (sizeof(T) == 2)
-      st = lbn_layer_norm_fwd_f16(io.stream, G, n, stride, x.Width(), m_epsilon, x.LockedBuffer(), x.LDim(),
-                                  y.Buffer(), y.LDim(), m_statistics.Buffer(), m_statistics.LDim(), sw, bw,
-                                  ws, bytes, stats_mode);
-    else
-      st = lbn_layer_norm_fwd_f32(io.stream, G, n, stride, x.Width(), m_epsilon,
-                                  reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
-                                  reinterpret_cast<float*>(y.Buffer()), y.LDim(), m_statistics.Buffer(),
-                                  m_statistics.LDim(), sw, bw, ws, bytes, stats_mode);
+    if constexpr (sizeof(T) == 8) {
+      st = lbn_layer_norm_fwd_f64(io.stream, G, n, stride, x.Width(), m_epsilon,
+                                  reinterpret_cast<const double*>(x.LockedBuffer()), x.LDim(),
+                                  reinterpret_cast<double*>(y.Buffer()), y.LDim(), m_statistics.Buffer(),
+                                  m_statistics.LDim(), sw, bw, stats_mode);
+    }
+    else {
+      // scratch is only needed (and only non-zero) for groups of tens of thousands of entries
+      const size_t bytes = lbn_layer_norm_fwd_workspace_bytes(G, n, x.Width(), static_cast<int>(sizeof(T)));
+      void* ws = m_ws.reserve(bytes, io.stream);
+      const float eps = static_cast<float>(m_epsilon);
+      if constexpr (sizeof(T) == 2)
+        st = lbn_layer_norm_fwd_f16(io.stream, G, n, stride, x.Width(), eps, x.LockedBuffer(), x.LDim(),
+                                    y.Buffer(), y.LDim(), m_statistics.Buffer(), m_statistics.LDim(), sw, bw,
+                                    ws, bytes, stats_mode);
+      else
+        st = lbn_layer_norm_fwd_f32(io.stream, G, n, stride, x.Width(), eps,
+                                    reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
+                                    reinterpret_cast<float*>(y.Buffer()), y.LDim(), m_statistics.Buffer(),
+                                    m_statistics.LDim(), sw, bw, ws, bytes, stats_mode);
+    }
     check_status(st, "layer_norm_layer::fp_compute");
     m_ws.after_call(io.stream, "layer_norm_layer::fp_compute");
   }
@@ -288,27 +300,41 @@ public:
     int64_t n, gn, G, stride;
     get_normdims(n, gn, G, stride);
     m_statistics_gradient.Resize(2 * G, x.Width());
-    const float* sw = m_scale ? m_scale_w : nullptr;
-    float* dsw = m_scale ? m_scale_grad : nullptr;
-    float* dbw = m_bias ? m_bias_grad : nullptr;
-    const size_t bytes = lbn_layer_norm_bwd_workspace_bytes(G, n, x.Width(), (dsw || dbw) ? 1 : 0,
-                                                            static_cast<int>(sizeof(T)));
-    void* ws = m_ws.reserve(bytes, io.stream);
+    const weight_t* sw = m_scale ? m_scale_w : nullptr;
+    weight_t* dsw = m_scale ? m_scale_grad : nullptr;
+    weight_t* dbw = m_bias ? m_bias_grad : nullptr;
     int st;
-    if (sizeof(T) == 2)
-      st = lbn_layer_norm_bwd_f16(io.stream, G, n, stride, x.Width(), m_epsilon, x.LockedBuffer(), x.LDim(),
-                                  dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+    if constexpr (sizeof(T) == 8) {
+      const size_t bytes = lbn_layer_norm_bwd_workspace_bytes_f64(G, n, x.Width(), (dsw || dbw) ? 1 : 0);
+      void* ws = m_ws.reserve(bytes, io.stream);
+      st = lbn_layer_norm_bwd_f64(io.stream, G, n, stride, x.Width(), m_epsilon,
+                                  reinterpret_cast<const double*>(x.LockedBuffer()), x.LDim(),
+                                  reinterpret_cast<const double*>(dy.LockedBuffer()), dy.LDim(),
+                                  reinterpret_cast<double*>(dx.Buffer()), dx.LDim(),
                                   m_statistics.LockedBuffer(), m_statistics.LDim(),
                                   m_statistics_gradient.Buffer(), m_statistics_gradient.LDim(), sw, dsw, dbw,
                                   ws, bytes);
-    else
-      st = lbn_layer_norm_bwd_f32(io.stream, G, n, stride, x.Width(), m_epsilon,
-                                  reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
-                                  reinterpret_cast<const float*>(dy.LockedBuffer()), dy.LDim(),
-                                  reinterpret_cast<float*>(dx.Buffer()), dx.LDim(),
-                                  m_statistics.LockedBuffer(), m_statistics.LDim(),
-                                  m_statistics_gradient.Buffer(), m_statistics_gradient.LDim(), sw, dsw, dbw,
-                                  ws, bytes);
+    }
+    else {
+      const size_t bytes = lbn_layer_norm_bwd_workspace_bytes(G, n, x.Width(), (dsw || dbw) ? 1 : 0,
+                                                              static_cast<int>(sizeof(T)));
+      void* ws = m_ws.reserve(bytes, io.stream);
+      const float eps = static_cast<float>(m_epsilon);
+      if constexpr (sizeof(T) == 2)
+        st = lbn_layer_norm_bwd_f16(io.stream, G, n, stride, x.Width(), eps, x.LockedBuffer(), x.LDim(),
+                                    dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+                                    m_statistics.LockedBuffer(), m_statistics.LDim(),
+                                    m_statistics_gradient.Buffer(), m_statistics_gradient.LDim(), sw, dsw, dbw,
+                                    ws, bytes);
+      else
+        st = lbn_layer_norm_bwd_f32(io.stream, G, n, stride, x.Width(), eps,
+                                    reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
+                                    reinterpret_cast<const float*>(dy.LockedBuffer()), dy.LDim(),
+                                    reinterpret_cast<float*>(dx.Buffer()), dx.LDim(),
+                                    m_statistics.LockedBuffer(), m_statistics.LDim(),
+                                    m_statistics_gradient.Buffer(), m_statistics_gradient.LDim(), sw, dsw, dbw,
+                                    ws, bytes);
+    }
     check_status(st, "layer_norm_layer::bp_compute");
     m_ws.after_call(io.stream, "layer_norm_layer::bp_compute");
   }
@@ -323,29 +349,30 @@ public:
   }
 
 private:
-  float m_epsilon;
+  double m_epsilon;
   bool m_scale, m_bias;
   int m_start_dim, m_sd = 0;
   std::vector<int64_t> m_dims;
-  const float* m_scale_w = nullptr;
-  const float* m_bias_w = nullptr;
-  float* m_scale_grad = nullptr;
-  float* m_bias_grad = nullptr;
+  const weight_t* m_scale_w = nullptr;
+  const weight_t* m_bias_w = nullptr;
+  weight_t* m_scale_grad = nullptr;
+  weight_t* m_bias_grad = nullptr;
   workspace m_ws;
 };
 
 // ------------------------------------------------------------------ batch norm
 /// include/lbann/layers/regularizers/batch_normalization.hpp:130-199 with local
 /// statistics (statistics_group_size == 1).  T is the storage type of the activations
-/// and error signals: float, or a 2-byte type holding IEEE binary16; statistics and
-/// weights are float either way.
+/// and error signals: float, or a 2-byte type holding IEEE binary16 (statistics and
+/// weights are float for both), or double (statistics and weights are doubles as well).
 template <typename T = float, typename Mat = device_matrix<T>>
 class batch_normalization_layer {
-  static_assert(sizeof(T) == 4 || sizeof(T) == 2, "fp32 or fp16 storage");
+  static_assert(sizeof(T) == 8 || sizeof(T) == 4 || sizeof(T) == 2, "fp64, fp32 or fp16 storage");
 public:
+  using weight_t = std::conditional_t<sizeof(T) == 8, double, float>;
   batch_normalization_layer(double decay = 0.9, double epsilon = 1e-5, int statistics_group_size = 1,
                             bool bessel_correction = true)
-    : m_decay(static_cast<float>(decay)), m_epsilon(static_cast<float>(epsilon)),
+    : m_decay(decay), m_epsilon(epsilon),
       m_statistics_group_size(statistics_group_size), m_bessel_correction(bessel_correction)
   {
     if (statistics_group_size != 1)
@@ -361,40 +388,51 @@ public:
     m_mean_and_var_gradient.Resize(m_num_channels, 2);
   }
   /// weights 0..3: scale, bias, running mean, running variance (all device pointers).
-  void set_weights(const float* scale, const float* bias, float* running_mean, float* running_var)
+  void set_weights(const weight_t* scale, const weight_t* bias, weight_t* running_mean, weight_t* running_var)
   {
-    m_w[0] = const_cast<float*>(scale); m_w[1] = const_cast<float*>(bias);
+    m_w[0] = const_cast<weight_t*>(scale); m_w[1] = const_cast<weight_t*>(bias);
     m_w[2] = running_mean; m_w[3] = running_var;
   }
-  void set_weight_gradients(float* dscale, float* dbias) { m_scale_grad = dscale; m_bias_grad = dbias; }
+  void set_weight_gradients(weight_t* dscale, weight_t* dbias) { m_scale_grad = dscale; m_bias_grad = dbias; }
 
   layer_io<Mat> io;
-  bool is_training = true;                        // execution_mode::training
-  device_matrix<float> m_mean_and_var;            // C x 2: column 0 mean, column 1 variance
-  device_matrix<float> m_mean_and_var_gradient;   // C x 2
+  bool is_training = true;                           // execution_mode::training
+  device_matrix<weight_t> m_mean_and_var;            // C x 2: column 0 mean, column 1 variance
+  device_matrix<weight_t> m_mean_and_var_gradient;   // C x 2
   int stats_mode = LBN_STATS_TWO_PASS;
 
   void fp_compute()
   {
     const Mat& x = *io.prev_activations;
     Mat& y = *io.activations;
-    const size_t bytes = lbn_batch_norm_workspace_bytes(m_num_channels, m_channel_size, x.Width());
+    const size_t bytes = workspace_bytes(x.Width());
     void* ws = m_ws.reserve(bytes, io.stream);
-    float* mv = m_mean_and_var.Buffer();
+    weight_t* mv = m_mean_and_var.Buffer();
     int st;
-    if (sizeof(T) == 2)
-      st = lbn_batch_norm_fwd_f16(io.stream, m_num_channels, m_channel_size, x.Width(),
+    if constexpr (sizeof(T) == 8) {
+      st = lbn_batch_norm_fwd_f64(io.stream, m_num_channels, m_channel_size, x.Width(),
                                   m_bessel_correction ? 1 : 0, m_epsilon, m_decay, is_training ? 1 : 0,
-                                  x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(), mv,
+                                  reinterpret_cast<const double*>(x.LockedBuffer()), x.LDim(),
+                                  reinterpret_cast<double*>(y.Buffer()), y.LDim(), mv,
                                   mv + m_mean_and_var.LDim(), m_w[0], m_w[1], m_w[2], m_w[3], ws, bytes,
                                   stats_mode);
-    else
-      st = lbn_batch_norm_fwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
-                                  m_bessel_correction ? 1 : 0, m_epsilon, m_decay, is_training ? 1 : 0,
-                                  reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
-                                  reinterpret_cast<float*>(y.Buffer()), y.LDim(), mv,
-                                  mv + m_mean_and_var.LDim(), m_w[0], m_w[1], m_w[2], m_w[3], ws, bytes,
-                                  stats_mode);
+    }
+    else {
+      const float eps = static_cast<float>(m_epsilon), decay = static_cast<float>(m_decay);
+      if constexpr (sizeof(T) == 2)
+        st = lbn_batch_norm_fwd_f16(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                    m_bessel_correction ? 1 : 0, eps, decay, is_training ? 1 : 0,
+                                    x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(), mv,
+                                    mv + m_mean_and_var.LDim(), m_w[0], m_w[1], m_w[2], m_w[3], ws, bytes,
+                                    stats_mode);
+      else
+        st = lbn_batch_norm_fwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                    m_bessel_correction ? 1 : 0, eps, decay, is_training ? 1 : 0,
+                                    reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
+                                    reinterpret_cast<float*>(y.Buffer()), y.LDim(), mv,
+                                    mv + m_mean_and_var.LDim(), m_w[0], m_w[1], m_w[2], m_w[3], ws, bytes,
+                                    stats_mode);
+    }
     check_status(st, "batch_normalization_layer::fp_compute");
     m_ws.after_call(io.stream, "batch_normalization_layer::fp_compute");
   }
@@ -403,26 +441,38 @@ public:
     const Mat& x = *io.prev_activations;
     const Mat& dy = *io.prev_error_signals;
     Mat& dx = *io.error_signals;
-    const size_t bytes = lbn_batch_norm_workspace_bytes(m_num_channels, m_channel_size, x.Width());
+    const size_t bytes = workspace_bytes(x.Width());
     void* ws = m_ws.reserve(bytes, io.stream);
-    const float* mv = m_mean_and_var.LockedBuffer();
-    float* mvg = m_mean_and_var_gradient.Buffer();
+    const weight_t* mv = m_mean_and_var.LockedBuffer();
+    weight_t* mvg = m_mean_and_var_gradient.Buffer();
     int st;
-    if (sizeof(T) == 2)
-      st = lbn_batch_norm_bwd_f16(io.stream, m_num_channels, m_channel_size, x.Width(),
+    if constexpr (sizeof(T) == 8) {
+      st = lbn_batch_norm_bwd_f64(io.stream, m_num_channels, m_channel_size, x.Width(),
                                   m_bessel_correction ? 1 : 0, m_epsilon, is_training ? 1 : 0,
-                                  x.LockedBuffer(), x.LDim(), dy.LockedBuffer(), dy.LDim(), dx.Buffer(),
-                                  dx.LDim(), mv, mv + m_mean_and_var.LDim(), m_w[2], m_w[3], m_w[0],
-                                  m_scale_grad, m_bias_grad, mvg, mvg + m_mean_and_var_gradient.LDim(), ws,
-                                  bytes);
-    else
-      st = lbn_batch_norm_bwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
-                                  m_bessel_correction ? 1 : 0, m_epsilon, is_training ? 1 : 0,
-                                  reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
-                                  reinterpret_cast<const float*>(dy.LockedBuffer()), dy.LDim(),
-                                  reinterpret_cast<float*>(dx.Buffer()), dx.LDim(), mv,
+                                  reinterpret_cast<const double*>(x.LockedBuffer()), x.LDim(),
+                                  reinterpret_cast<const double*>(dy.LockedBuffer()), dy.LDim(),
+                                  reinterpret_cast<double*>(dx.Buffer()), dx.LDim(), mv,
                                   mv + m_mean_and_var.LDim(), m_w[2], m_w[3], m_w[0], m_scale_grad,
                                   m_bias_grad, mvg, mvg + m_mean_and_var_gradient.LDim(), ws, bytes);
+    }
+    else {
+      const float eps = static_cast<float>(m_epsilon);
+      if constexpr (sizeof(T) == 2)
+        st = lbn_batch_norm_bwd_f16(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                    m_bessel_correction ? 1 : 0, eps, is_training ? 1 : 0,
+                                    x.LockedBuffer(), x.LDim(), dy.LockedBuffer(), dy.LDim(), dx.Buffer(),
+                                    dx.LDim(), mv, mv + m_mean_and_var.LDim(), m_w[2], m_w[3], m_w[0],
+                                    m_scale_grad, m_bias_grad, mvg, mvg + m_mean_and_var_gradient.LDim(), ws,
+                                    bytes);
+      else
+        st = lbn_batch_norm_bwd_f32(io.stream, m_num_channels, m_channel_size, x.Width(),
+                                    m_bessel_correction ? 1 : 0, eps, is_training ? 1 : 0,
+                                    reinterpret_cast<const float*>(x.LockedBuffer()), x.LDim(),
+                                    reinterpret_cast<const float*>(dy.LockedBuffer()), dy.LDim(),
+                                    reinterpret_cast<float*>(dx.Buffer()), dx.LDim(), mv,
+                                    mv + m_mean_and_var.LDim(), m_w[2], m_w[3], m_w[0], m_scale_grad,
+                                    m_bias_grad, mvg, mvg + m_mean_and_var_gradient.LDim(), ws, bytes);
+    }
     check_status(st, "batch_normalization_layer::bp_compute");
     m_ws.after_call(io.stream, "batch_normalization_layer::bp_compute");
   }
@@ -437,14 +487,19 @@ public:
   }
 
 private:
-  float m_decay, m_epsilon;
+  size_t workspace_bytes(int64_t width) const
+  {
+    return sizeof(T) == 8 ? lbn_batch_norm_workspace_bytes_f64(m_num_channels, m_channel_size, width)
+                          : lbn_batch_norm_workspace_bytes(m_num_channels, m_channel_size, width);
+  }
+  double m_decay, m_epsilon;
   int m_statistics_group_size;
   bool m_bessel_correction;
   std::vector<int64_t> m_dims;
   int64_t m_num_channels = 0, m_channel_size = 0;
-  float* m_w[4] = {nullptr, nullptr, nullptr, nullptr};
-  float* m_scale_grad = nullptr;
-  float* m_bias_grad = nullptr;
+  weight_t* m_w[4] = {nullptr, nullptr, nullptr, nullptr};
+  weight_t* m_scale_grad = nullptr;
+  weight_t* m_bias_grad = nullptr;
   workspace m_ws;
 };
 
@@ -465,6 +520,13 @@ public:
   {
     const Mat& x = *io.prev_activations;
     Mat& y = *io.activations;
+    if constexpr (sizeof(detail::element_t<Mat>) == 8) {  // TensorDataType = double: no scratch
+      check_status(lbn_softmax_fwd_f64(io.stream, x.Height(), x.Width(),
+                                       reinterpret_cast<const double*>(x.LockedBuffer()), x.LDim(),
+                                       reinterpret_cast<double*>(y.Buffer()), y.LDim()),
+                   "softmax_layer::fp_compute");
+      return;
+    }
     const size_t bytes = lbn_softmax_workspace_bytes(x.Height(), x.Width());
     const auto fwd = sizeof(detail::element_t<Mat>) == 2 ? &lbn_softmax_fwd_f16 : &call_f32_fwd;
     check_status(fwd(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(),
@@ -477,6 +539,14 @@ public:
     const Mat& y = *io.activations;
     const Mat& dy = *io.prev_error_signals;
     Mat& dx = *io.error_signals;
+    if constexpr (sizeof(detail::element_t<Mat>) == 8) {
+      check_status(lbn_softmax_bwd_f64(io.stream, y.Height(), y.Width(),
+                                       reinterpret_cast<const double*>(y.LockedBuffer()), y.LDim(),
+                                       reinterpret_cast<const double*>(dy.LockedBuffer()), dy.LDim(),
+                                       reinterpret_cast<double*>(dx.Buffer()), dx.LDim()),
+                   "softmax_layer::bp_compute");
+      return;
+    }
     const size_t bytes = lbn_softmax_workspace_bytes(y.Height(), y.Width());
     const auto bwd = sizeof(detail::element_t<Mat>) == 2 ? &lbn_softmax_bwd_f16 : &call_f32_bwd;
     check_status(bwd(io.stream, y.Height(), y.Width(), y.LockedBuffer(), y.LDim(), dy.LockedBuffer(), dy.LDim(),
@@ -519,6 +589,13 @@ public:
   {
     const Mat& x = *io.prev_activations;
     Mat& y = *io.activations;
+    if constexpr (sizeof(detail::element_t<Mat>) == 8) {  // TensorDataType = double: no scratch
+      check_status(lbn_log_softmax_fwd_f64(io.stream, x.Height(), x.Width(),
+                                       reinterpret_cast<const double*>(x.LockedBuffer()), x.LDim(),
+                                       reinterpret_cast<double*>(y.Buffer()), y.LDim()),
+                   "log_softmax_layer::fp_compute");
+      return;
+    }
     const size_t bytes = lbn_softmax_workspace_bytes(x.Height(), x.Width());
     const auto fwd = sizeof(detail::element_t<Mat>) == 2 ? &lbn_log_softmax_fwd_f16 : &call_f32_fwd;
     check_status(fwd(io.stream, x.Height(), x.Width(), x.LockedBuffer(), x.LDim(), y.Buffer(), y.LDim(),
@@ -531,6 +608,14 @@ public:
     const Mat& y = *io.activations;
     const Mat& dy = *io.prev_error_signals;
     Mat& dx = *io.error_signals;
+    if constexpr (sizeof(detail::element_t<Mat>) == 8) {
+      check_status(lbn_log_softmax_bwd_f64(io.stream, y.Height(), y.Width(),
+                                       reinterpret_cast<const double*>(y.LockedBuffer()), y.LDim(),
+                                       reinterpret_cast<const double*>(dy.LockedBuffer()), dy.LDim(),
+                                       reinterpret_cast<double*>(dx.Buffer()), dx.LDim()),
+                   "log_softmax_layer::bp_compute");
+      return;
+    }
     const size_t bytes = lbn_softmax_workspace_bytes(y.Height(), y.Width());
     const auto bwd = sizeof(detail::element_t<Mat>) == 2 ? &lbn_log_softmax_bwd_f16 : &call_f32_bwd;
     check_status(bwd(io.stream, y.Height(), y.Width(), y.LockedBuffer(), y.LDim(), dy.LockedBuffer(), dy.LDim(),
@@ -606,10 +691,18 @@ public:
     Mat& y = *io.activations;
     int64_t cs, stride, C;
     get_channel_size_and_stride(cs, stride, C);
-    const size_t bytes = lbn_channelwise_softmax_workspace_bytes(C, cs, x.Width());
-    check_status(lbn_channelwise_softmax_fwd_f32(io.stream, C, cs, stride, x.Width(), x.LockedBuffer(), x.LDim(),
-                                                 y.Buffer(), y.LDim(), m_ws.reserve(bytes, io.stream), bytes),
-                 "channelwise_softmax_layer::fp_compute");
+    if constexpr (sizeof(detail::element_t<Mat>) == 8) {  // TensorDataType = double: no scratch
+      check_status(lbn_channelwise_softmax_fwd_f64(io.stream, C, cs, stride, x.Width(), x.LockedBuffer(), x.LDim(),
+                                                   y.Buffer(), y.LDim()),
+                   "channelwise_softmax_layer::fp_compute");
+      return;
+    }
+    else {
+      const size_t bytes = lbn_channelwise_softmax_workspace_bytes(C, cs, x.Width());
+      check_status(lbn_channelwise_softmax_fwd_f32(io.stream, C, cs, stride, x.Width(), x.LockedBuffer(), x.LDim(),
+                                                   y.Buffer(), y.LDim(), m_ws.reserve(bytes, io.stream), bytes),
+                   "channelwise_softmax_layer::fp_compute");
+    }
     m_ws.after_call(io.stream, "channelwise_softmax_layer::fp_compute");
   }
   void bp_compute()
@@ -619,11 +712,19 @@ public:
     Mat& dx = *io.error_signals;
     int64_t cs, stride, C;
     get_channel_size_and_stride(cs, stride, C);
-    const size_t bytes = lbn_channelwise_softmax_workspace_bytes(C, cs, y.Width());
-    check_status(lbn_channelwise_softmax_bwd_f32(io.stream, C, cs, stride, y.Width(), y.LockedBuffer(), y.LDim(),
-                                                 dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
-                                                 m_ws.reserve(bytes, io.stream), bytes),
-                 "channelwise_softmax_layer::bp_compute");
+    if constexpr (sizeof(detail::element_t<Mat>) == 8) {
+      check_status(lbn_channelwise_softmax_bwd_f64(io.stream, C, cs, stride, y.Width(), y.LockedBuffer(), y.LDim(),
+                                                   dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim()),
+                   "channelwise_softmax_layer::bp_compute");
+      return;
+    }
+    else {
+      const size_t bytes = lbn_channelwise_softmax_workspace_bytes(C, cs, y.Width());
+      check_status(lbn_channelwise_softmax_bwd_f32(io.stream, C, cs, stride, y.Width(), y.LockedBuffer(), y.LDim(),
+                                                   dy.LockedBuffer(), dy.LDim(), dx.Buffer(), dx.LDim(),
+                                                   m_ws.reserve(bytes, io.stream), bytes),
+                   "channelwise_softmax_layer::bp_compute");
+    }
     m_ws.after_call(io.stream, "channelwise_softmax_layer::bp_compute");
   }
   /// The layer's scratch buffer (reserve it up front to keep the hooks free of allocation).

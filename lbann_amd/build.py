@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "liblbnorm.so")
 SOURCES = ["capi_common.hip", "softmax.hip", "layer_norm.hip", "batch_norm.hip", "entrywise_batch_norm.hip",
-           "entrywise_batch_norm_split.hip", "cross_entropy.hip", "scale_bias.hip", "gradient_sink.hip"]
+           "entrywise_batch_norm_split.hip", "cross_entropy.hip", "scale_bias.hip", "gradient_sink.hip", "f64_layers.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -10,6 +10,7 @@ LIB_PATH = os.environ.get("LBN_LIB") or os.path.join(_HERE, "liblbnorm.so")
 
 i64 = ctypes.c_int64
 f32 = ctypes.c_float
+f64 = ctypes.c_double
 cint = ctypes.c_int
 vp = ctypes.c_void_p
 sz = ctypes.c_size_t
@@ -100,6 +101,21 @@ PROTOTYPES = {
     "lbn_entrywise_batch_norm_bwd_apply_f32": (cint, [vp, i64, i64, i64, f32, vp, i64, vp, i64, vp, i64, vp, i64,
                                                       vp, i64]),
     "lbn_gradient_sink_f32": (cint, [vp, i64, i64, f32, f32, vp, i64, vp, i64]),
+    "lbn_softmax_fwd_f64": (cint, [vp, i64, i64, vp, i64, vp, i64]),
+    "lbn_softmax_bwd_f64": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64]),
+    "lbn_log_softmax_fwd_f64": (cint, [vp, i64, i64, vp, i64, vp, i64]),
+    "lbn_log_softmax_bwd_f64": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64]),
+    "lbn_channelwise_softmax_fwd_f64": (cint, [vp, i64, i64, i64, i64, vp, i64, vp, i64]),
+    "lbn_channelwise_softmax_bwd_f64": (cint, [vp, i64, i64, i64, i64, vp, i64, vp, i64, vp, i64]),
+    "lbn_layer_norm_fwd_f64": (cint, [vp, i64, i64, i64, i64, f64, vp, i64, vp, i64, vp, i64, vp, vp, cint]),
+    "lbn_layer_norm_bwd_workspace_bytes_f64": (sz, [i64, i64, i64, cint]),
+    "lbn_layer_norm_bwd_f64": (cint, [vp, i64, i64, i64, i64, f64, vp, i64, vp, i64, vp, i64, vp, i64,
+                                      vp, i64, vp, vp, vp, vp, sz]),
+    "lbn_batch_norm_workspace_bytes_f64": (sz, [i64, i64, i64]),
+    "lbn_batch_norm_fwd_f64": (cint, [vp, i64, i64, i64, cint, f64, f64, cint, vp, i64, vp, i64, vp, vp,
+                                      vp, vp, vp, vp, vp, sz, cint]),
+    "lbn_batch_norm_bwd_f64": (cint, [vp, i64, i64, i64, cint, f64, cint, vp, i64, vp, i64, vp, i64, vp,
+                                      vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]),
 }
 
 _lib = None

@@ -1,0 +1,1139 @@
+// The five layers for TensorDataType = double (the reference instantiates its layers for double
+// under LBANN_HAS_DOUBLE: include/lbann/macros/instantiate.hpp:28-30,
+// src/layers/regularizers/layer_norm_builder.cpp:48-54).  Storage, statistics, weights and all
+// arithmetic are binary64; every kernel is bound by HBM bandwidth at 8 bytes per entry.
+//
+// One family of row kernels serves layer norm, softmax, log-softmax and channelwise softmax: a
+// team of 64, 256 or 1024 threads owns a row and keeps it in registers (V accesses of W = 2
+// doubles, 16 bytes, per thread; W = 1 for rows off the 16-byte grid), so a tensor is read once
+// and written once.  Teams walk rows b, b + grid, ... (the launch is a few workgroups per compute
+// unit).  Rows beyond 32768 entries (16384 for W = 1) are streamed by one 1024-thread workgroup
+// each, twice (the second pass re-reads what the first one left in the caches).  Layer-norm weight
+// gradients are accumulated in registers across a team's rows and leave one partial row per team,
+// added in a fixed order by a second kernel.  Batch norm reduces a channel (width segments of
+// channel_size entries) over P workgroups into partial pairs and merges them, in a fixed order, in
+// the prologue of the apply kernel.  No atomics: results are bitwise reproducible.
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+#include <cmath>
+#include <cstdint>
+
+#include "device_utils.hpp"
+#include "host_utils.hpp"
+
+namespace lbn {
+namespace f64 {
+
+constexpr int kMaxV = 16;
+constexpr int kStreamThreads = 1024;
+constexpr int kBnThreads = 256;
+constexpr int kBnMaxSplit = 64;
+
+enum { kSoftmax = 0, kLogSoftmax = 1, kChannelwise = 2 };
+
+// ------------------------------------------------------------------ reductions
+__device__ __forceinline__ double wave_sum_d(double v)
+{
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+__device__ __forceinline__ double wave_max_d(double v)
+{
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmax(v, __shfl_xor(v, o));
+  return v;
+}
+
+// Sum / maximum over a team of NW waves.  `slot` points to NW doubles of LDS private to the team
+// and to this reduction; all threads of the workgroup call when NW > 1 (a team is then the whole
+// workgroup).  Fixed order.
+template <int NW>
+__device__ __forceinline__ double team_sum_d(double v, double* slot)
+{
+  v = wave_sum_d(v);
+  if constexpr (NW == 1) return v;
+  if ((threadIdx.x & (kWave - 1)) == 0) slot[(threadIdx.x / kWave) % NW] = v;
+  __syncthreads();
+  double r = slot[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) r += slot[i];
+  return r;
+}
+template <int NW>
+__device__ __forceinline__ double team_max_d(double v, double* slot)
+{
+  v = wave_max_d(v);
+  if constexpr (NW == 1) return v;
+  if ((threadIdx.x & (kWave - 1)) == 0) slot[(threadIdx.x / kWave) % NW] = v;
+  __syncthreads();
+  double r = slot[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) r = fmax(r, slot[i]);
+  return r;
+}
+
+// ------------------------------------------------------------------ access
+template <int W>
+__device__ __forceinline__ void load_w(const double* p, double (&v)[W])
+{
+  if constexpr (W == 2) {
+    const double2 t = *reinterpret_cast<const double2*>(p);
+    v[0] = t.x;
+    v[1] = t.y;
+  }
+  else {
+    v[0] = *p;
+  }
+}
+template <int W>
+__device__ __forceinline__ void store_w(double* p, const double (&v)[W])
+{
+  if constexpr (W == 2) {
+    typedef double v2d __attribute__((ext_vector_type(2)));
+    v2d t;
+    t.x = v[0];
+    t.y = v[1];
+    __builtin_nontemporal_store(t, reinterpret_cast<v2d*>(p));
+  }
+  else {
+    __builtin_nontemporal_store(v[0], p);
+  }
+}
+
+// A team's place in the launch: TPR threads per row, 256-thread workgroups hold 256 / TPR teams.
+template <int TPR>
+struct Team {
+  static constexpr int kThreads = TPR < 256 ? 256 : TPR;
+  static constexpr int kTeams = kThreads / TPR;
+  static constexpr int kNW = TPR / kWave;
+};
+
+// Shapes of the register kernels.
+struct RowShape {
+  int tpr, v;
+};
+inline RowShape pick_shape(int64_t units, int64_t rows)
+{
+  const int tprs[3] = {64, 256, 1024};
+  for (int i = 0; i < 3; ++i) {
+    const int64_t per = ceil_div(units, tprs[i]);
+    const int max_v = i == 2 ? kMaxV : 8;
+    if (per > max_v) continue;
+    int v = 1;
+    while (v < per) v *= 2;
+    // few rows: a wider team keeps more of the device busy
+    if (i < 2 && v > 1 && rows * (tprs[i] / kWave) < 2048 && ceil_div(units, tprs[i + 1]) >= 1) continue;
+    return {tprs[i], v};
+  }
+  return {0, 0};
+}
+
+// Every register kernel: rows map to (column, group) as in the fp32 kernels.
+struct RowArgs {
+  const double* a;   // x (forward) or y / x (backward)
+  const double* g;   // dy
+  double* out;
+  int64_t lda, ldg, ldo;
+  RowMap map;
+  int64_t rows;
+  int units;         // accesses per row
+  int n;             // entries per row
+  double eps;
+  double* stats;     // layer norm: (2G x w)
+  int64_t ld_stats;
+  double* sgrad;
+  int64_t ld_sgrad;
+  const double* gamma;
+  const double* beta;
+  double* part;      // layer norm backward: one partial (dscale | dbias) row of 2n per team
+  int sumsq;
+};
+
+#define LBN_F64_ROW_PROLOGUE                                                         \
+  using TM = Team<TPR>;                                                              \
+  constexpr int NW = TM::kNW;                                                        \
+  __shared__ double red[4][TM::kTeams][NW > 1 ? NW : 1];                             \
+  const int team = threadIdx.x / TPR;                                                \
+  const int t = threadIdx.x - team * TPR;                                            \
+  const int64_t teams_total = static_cast<int64_t>(gridDim.x) * TM::kTeams;          \
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * TM::kTeams + team;        \
+  const int64_t iters = (a.rows + teams_total - 1) / teams_total;                    \
+  bool ok[V];                                                                        \
+  _Pragma("unroll") for (int i = 0; i < V; ++i) ok[i] = t + i * TPR < a.units;
+
+// ------------------------------------------------------------------ softmax family
+template <int KIND, int TPR, int V, int W>
+__global__ void __launch_bounds__(Team<TPR>::kThreads)
+sm_fwd_rows_f64(RowArgs a)
+{
+  LBN_F64_ROW_PROLOGUE
+  for (int64_t it = 0; it < iters; ++it) {
+    const int64_t row = first + it * teams_total;
+    const bool live = row < a.rows;  // teams of a workgroup run the same number of iterations
+    const int64_t r = live ? row : a.rows - 1;
+    const double* xr = a.a + a.map.offset(r, a.lda);
+    double v[V][W];
+    double m = -DBL_MAX;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      if (ok[i]) {
+        load_w<W>(xr + W * static_cast<int64_t>(t + i * TPR), v[i]);
+#pragma unroll
+        for (int j = 0; j < W; ++j) m = fmax(m, v[i][j]);
+      }
+    }
+    m = team_max_d<NW>(m, red[2 * (it & 1)][team]);
+    double s = 0.0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      if (ok[i]) {
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+          const double d = v[i][j] - m;
+          const double e = exp(d);
+          s += e;
+          v[i][j] = KIND == kLogSoftmax ? d : e;
+        }
+      }
+    }
+    s = team_sum_d<NW>(s, red[2 * (it & 1) + 1][team]);
+    if (!live) continue;
+    double* yr = a.out + a.map.offset(row, a.ldo);
+    const double scale = 1.0 / s;
+    const double lse = KIND == kLogSoftmax ? log(s) : 0.0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      if (!ok[i]) continue;
+#pragma unroll
+      for (int j = 0; j < W; ++j) {
+        if (KIND == kSoftmax) {
+          const double r2 = scale * v[i][j];
+          v[i][j] = __builtin_isnormal(r2) ? r2 : 0.0;  // openmp/softmax.hpp:108-113
+        }
+        else if (KIND == kLogSoftmax) {
+          v[i][j] -= lse;
+        }
+        else {
+          v[i][j] /= s;  // channelwise_softmax.cpp:88-97: a division, denormals kept
+        }
+      }
+      store_w<W>(yr + W * static_cast<int64_t>(t + i * TPR), v[i]);
+    }
+  }
+}
+
+template <int KIND, int TPR, int V, int W>
+__global__ void __launch_bounds__(Team<TPR>::kThreads)
+sm_bwd_rows_f64(RowArgs a)
+{
+  LBN_F64_ROW_PROLOGUE
+  for (int64_t it = 0; it < iters; ++it) {
+    const int64_t row = first + it * teams_total;
+    const bool live = row < a.rows;
+    const int64_t r = live ? row : a.rows - 1;
+    const double* yr = a.a + a.map.offset(r, a.lda);
+    const double* gr = a.g + a.map.offset(r, a.ldg);
+    double y[V][W], g[V][W];
+    double s = 0.0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      if (ok[i]) {
+        load_w<W>(yr + W * static_cast<int64_t>(t + i * TPR), y[i]);
+        load_w<W>(gr + W * static_cast<int64_t>(t + i * TPR), g[i]);
+#pragma unroll
+        for (int j = 0; j < W; ++j) s += KIND == kLogSoftmax ? g[i][j] : y[i][j] * g[i][j];
+      }
+    }
+    s = team_sum_d<NW>(s, red[it & 3][team]);
+    if (!live) continue;
+    double* dr = a.out + a.map.offset(row, a.ldo);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      if (!ok[i]) continue;
+#pragma unroll
+      for (int j = 0; j < W; ++j)
+        g[i][j] = KIND == kLogSoftmax ? g[i][j] - exp(y[i][j]) * s : y[i][j] * (g[i][j] - s);
+      store_w<W>(dr + W * static_cast<int64_t>(t + i * TPR), g[i]);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ layer norm
+template <int TPR, int V, int W>
+__global__ void __launch_bounds__(Team<TPR>::kThreads)
+ln_fwd_rows_f64(RowArgs a)
+{
+  LBN_F64_ROW_PROLOGUE
+  const double inv_n = 1.0 / static_cast<double>(a.n);
+  for (int64_t it = 0; it < iters; ++it) {
+    const int64_t row = first + it * teams_total;
+    const bool live = row < a.rows;
+    const int64_t r = live ? row : a.rows - 1;
+    const double* xr = a.a + a.map.offset(r, a.lda);
+    double v[V][W];
+    double s = 0.0, q = 0.0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+#pragma unroll
+      for (int j = 0; j < W; ++j) v[i][j] = 0.0;
+      if (ok[i]) {
+        load_w<W>(xr + W * static_cast<int64_t>(t + i * TPR), v[i]);
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+          s += v[i][j];
+          q += v[i][j] * v[i][j];
+        }
+      }
+    }
+    s = team_sum_d<NW>(s, red[2 * (it & 1)][team]);
+    const double mean = s * inv_n;
+    double var;
+    if (a.sumsq) {  // the reference's expression (layer_norm.cpp:99-112)
+      q = team_sum_d<NW>(q, red[2 * (it & 1) + 1][team]);
+      const double nn = static_cast<double>(a.n);
+      const double m2 = s / nn;
+      var = fmax(q / nn - m2 * m2, 0.0);
+    }
+    else {
+      double c = 0.0;
+#pragma unroll
+      for (int i = 0; i < V; ++i)
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+          const double d = ok[i] ? v[i][j] - mean : 0.0;
+          c += d * d;
+        }
+      var = team_sum_d<NW>(c, red[2 * (it & 1) + 1][team]) * inv_n;
+    }
+    if (!live) continue;
+    int64_t col, g;
+    a.map.split(row, col, g);
+    if (t == 0) {
+      a.stats[g + col * a.ld_stats] = a.sumsq ? s / static_cast<double>(a.n) : mean;
+      a.stats[a.map.groups + g + col * a.ld_stats] = var;
+    }
+    const double mu = a.sumsq ? s / static_cast<double>(a.n) : mean;
+    const double inv_stdev = 1.0 / sqrt(var + a.eps);
+    double* yr = a.out + g * a.map.stride + col * a.ldo;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      if (!ok[i]) continue;
+      const int64_t e0 = W * static_cast<int64_t>(t + i * TPR);
+#pragma unroll
+      for (int j = 0; j < W; ++j) {
+        double y = (v[i][j] - mu) * inv_stdev;
+        if (a.gamma) y *= a.gamma[e0 + j];
+        if (a.beta) y += a.beta[e0 + j];
+        v[i][j] = y;
+      }
+      store_w<W>(yr + e0, v[i]);
+    }
+  }
+}
+
+// WGRAD: dscale / dbias accumulate in registers across the team's rows (a thread always owns the
+// same entries) and leave one partial row per team.
+template <int TPR, int V, int W, bool WGRAD>
+__global__ void __launch_bounds__(Team<TPR>::kThreads)
+ln_bwd_rows_f64(RowArgs a)
+{
+  LBN_F64_ROW_PROLOGUE
+  const double nn = static_cast<double>(a.n);
+  double gam[V][W];
+  double dg[WGRAD ? V : 1][W], db[WGRAD ? V : 1][W];
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      gam[i][j] = (a.gamma && ok[i]) ? a.gamma[W * static_cast<int64_t>(t + i * TPR) + j] : 1.0;
+      if (WGRAD) dg[i][j] = db[i][j] = 0.0;
+    }
+  for (int64_t it = 0; it < iters; ++it) {
+    const int64_t row = first + it * teams_total;
+    const bool live = row < a.rows;
+    const int64_t r = live ? row : a.rows - 1;
+    int64_t col, g;
+    a.map.split(r, col, g);
+    const double* xr = a.a + g * a.map.stride + col * a.lda;
+    const double* gr = a.g + g * a.map.stride + col * a.ldg;
+    const double mean = a.stats[g + col * a.ld_stats];
+    const double var = a.stats[a.map.groups + g + col * a.ld_stats];
+    const double inv_stdev = 1.0 / sqrt(var + a.eps);
+    double d[V][W], gs[V][W];
+    double A = 0.0, B = 0.0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+#pragma unroll
+      for (int j = 0; j < W; ++j) d[i][j] = gs[i][j] = 0.0;
+      if (ok[i]) {
+        load_w<W>(xr + W * static_cast<int64_t>(t + i * TPR), d[i]);
+        load_w<W>(gr + W * static_cast<int64_t>(t + i * TPR), gs[i]);
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+          d[i][j] -= mean;
+          if (WGRAD && live) {
+            db[i][j] += gs[i][j];
+            dg[i][j] += gs[i][j] * d[i][j] * inv_stdev;
+          }
+          gs[i][j] *= gam[i][j];
+          A += gs[i][j];
+          B += gs[i][j] * d[i][j];
+        }
+      }
+    }
+    A = team_sum_d<NW>(A, red[2 * (it & 1)][team]);
+    B = team_sum_d<NW>(B, red[2 * (it & 1) + 1][team]);
+    if (!live) continue;
+    const double dmean = -A * inv_stdev;
+    const double dvar = -B * inv_stdev * inv_stdev * inv_stdev / 2;
+    if (t == 0) {
+      a.sgrad[g + col * a.ld_sgrad] = dmean;
+      a.sgrad[a.map.groups + g + col * a.ld_sgrad] = dvar;
+    }
+    double* dr = a.out + g * a.map.stride + col * a.ldo;
+    const double c0 = dmean / nn, c1 = dvar * 2 / nn;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      if (!ok[i]) continue;
+#pragma unroll
+      for (int j = 0; j < W; ++j) gs[i][j] = gs[i][j] * inv_stdev + c0 + c1 * d[i][j];
+      store_w<W>(dr + W * static_cast<int64_t>(t + i * TPR), gs[i]);
+    }
+  }
+  if (WGRAD) {
+    double* out = a.part + first * 2 * a.n;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      if (!ok[i]) continue;
+#pragma unroll
+      for (int j = 0; j < W; ++j) {
+        const int64_t e = W * static_cast<int64_t>(t + i * TPR) + j;
+        out[e] = dg[i][j];
+        out[a.n + e] = db[i][j];
+      }
+    }
+  }
+}
+
+// Adds P partial rows of 2n entries; thread per entry, fixed order.
+__global__ void __launch_bounds__(256)
+ln_wgrad_reduce_f64(const double* __restrict__ part, int64_t P, int64_t n, double* dscale, double* dbias)
+{
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= 2 * n) return;
+  double acc = 0.0;
+  for (int64_t p = 0; p < P; ++p) acc += part[p * 2 * n + e];
+  double* out = e < n ? dscale : dbias;
+  if (out) out[e < n ? e : e - n] = acc;
+}
+
+// ------------------------------------------------------------------ long rows
+// One 1024-thread workgroup per row, one double per access (512 contiguous bytes per wave), two
+// passes; the second finds the row in the caches.  OP: 0 softmax family forward (KIND), 1 softmax
+// family backward, 2 layer norm forward, 3 layer norm backward (weight gradients by the column
+// kernel below).
+template <int OP, int KIND>
+__global__ void __launch_bounds__(kStreamThreads)
+rows_stream_f64(RowArgs a)
+{
+  constexpr int NW = kStreamThreads / kWave;
+  __shared__ double red[3][NW];
+  const int64_t row = blockIdx.x;
+  int64_t col, g;
+  a.map.split(row, col, g);
+  const int64_t off_a = g * a.map.stride + col * a.lda;
+  const int64_t off_g = g * a.map.stride + col * a.ldg;
+  const int64_t off_o = g * a.map.stride + col * a.ldo;
+  const int t = threadIdx.x;
+  const int64_t n = a.n;
+  if (OP == 0) {
+    const double* xr = a.a + off_a;
+    double m = -DBL_MAX, s = 0.0;  // online: s = sum exp(x - m) over the thread's entries
+    for (int64_t k = t; k < n; k += kStreamThreads) {
+      const double x = xr[k];
+      if (x > m) {
+        s = s * exp(m - x) + 1.0;
+        m = x;
+      }
+      else {
+        s += exp(x - m);
+      }
+    }
+    const double gm = team_max_d<NW>(m, red[0]);
+    s = team_sum_d<NW>(s * exp(m - gm), red[1]);
+    const double scale = 1.0 / s, lse = log(s);
+    double* yr = a.out + off_o;
+    for (int64_t k = t; k < n; k += kStreamThreads) {
+      const double d = xr[k] - gm;
+      double y;
+      if (KIND == kLogSoftmax) y = d - lse;
+      else if (KIND == kSoftmax) {
+        y = scale * exp(d);
+        y = __builtin_isnormal(y) ? y : 0.0;
+      }
+      else y = exp(d) / s;
+      yr[k] = y;
+    }
+  }
+  else if (OP == 1) {
+    const double* yr = a.a + off_a;
+    const double* gr = a.g + off_g;
+    double s = 0.0;
+    for (int64_t k = t; k < n; k += kStreamThreads) s += KIND == kLogSoftmax ? gr[k] : yr[k] * gr[k];
+    s = team_sum_d<NW>(s, red[0]);
+    double* dr = a.out + off_o;
+    for (int64_t k = t; k < n; k += kStreamThreads) {
+      const double y = yr[k], gg = gr[k];
+      dr[k] = KIND == kLogSoftmax ? gg - exp(y) * s : y * (gg - s);
+    }
+  }
+  else if (OP == 2) {
+    const double* xr = a.a + off_a;
+    const double K = a.sumsq ? 0.0 : xr[0];  // sums about the row's first entry: no cancellation
+    double s = 0.0, q = 0.0;
+    for (int64_t k = t; k < n; k += kStreamThreads) {
+      const double d = xr[k] - K;
+      s += d;
+      q += d * d;
+    }
+    s = team_sum_d<NW>(s, red[0]);
+    q = team_sum_d<NW>(q, red[1]);
+    const double nn = static_cast<double>(n);
+    const double dm = s / nn;
+    const double mean = K + dm;
+    const double var = n <= 1 ? 1.0 : fmax(q / nn - dm * dm, 0.0);
+    if (t == 0) {
+      a.stats[g + col * a.ld_stats] = mean;
+      a.stats[a.map.groups + g + col * a.ld_stats] = var;
+    }
+    const double inv_stdev = 1.0 / sqrt(var + a.eps);
+    double* yr = a.out + off_o;
+    for (int64_t k = t; k < n; k += kStreamThreads) {
+      double y = (xr[k] - mean) * inv_stdev;
+      if (a.gamma) y *= a.gamma[k];
+      if (a.beta) y += a.beta[k];
+      yr[k] = y;
+    }
+  }
+  else {
+    const double* xr = a.a + off_a;
+    const double* gr = a.g + off_g;
+    const double mean = a.stats[g + col * a.ld_stats];
+    const double var = a.stats[a.map.groups + g + col * a.ld_stats];
+    const double inv_stdev = 1.0 / sqrt(var + a.eps);
+    double A = 0.0, B = 0.0;
+    for (int64_t k = t; k < n; k += kStreamThreads) {
+      const double gg = a.gamma ? gr[k] * a.gamma[k] : gr[k];
+      A += gg;
+      B += gg * (xr[k] - mean);
+    }
+    A = team_sum_d<NW>(A, red[0]);
+    B = team_sum_d<NW>(B, red[1]);
+    const double dmean = -A * inv_stdev;
+    const double dvar = -B * inv_stdev * inv_stdev * inv_stdev / 2;
+    if (t == 0) {
+      a.sgrad[g + col * a.ld_sgrad] = dmean;
+      a.sgrad[a.map.groups + g + col * a.ld_sgrad] = dvar;
+    }
+    const double nn = static_cast<double>(n);
+    const double c0 = dmean / nn, c1 = dvar * 2 / nn;
+    double* dr = a.out + off_o;
+    for (int64_t k = t; k < n; k += kStreamThreads) {
+      const double gg = a.gamma ? gr[k] * a.gamma[k] : gr[k];
+      dr[k] = gg * inv_stdev + c0 + c1 * (xr[k] - mean);
+    }
+  }
+}
+
+// Weight gradients of long rows: thread per entry k walks a slab of rows; grid (ceil(n/256), slabs);
+// partial rows [slab][2n], added by ln_wgrad_reduce_f64.
+__global__ void __launch_bounds__(256)
+ln_wgrad_columns_f64(RowArgs a, int64_t rows_per_slab)
+{
+  const int64_t k = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (k >= a.n) return;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * rows_per_slab;
+  const int64_t r1 = r0 + rows_per_slab < a.rows ? r0 + rows_per_slab : a.rows;
+  double dg = 0.0, db = 0.0;
+  for (int64_t row = r0; row < r1; ++row) {
+    int64_t col, g;
+    a.map.split(row, col, g);
+    const double mean = a.stats[g + col * a.ld_stats];
+    const double inv_stdev = 1.0 / sqrt(a.stats[a.map.groups + g + col * a.ld_stats] + a.eps);
+    const double gg = a.g[g * a.map.stride + col * a.ldg + k];
+    db += gg;
+    dg += gg * (a.a[g * a.map.stride + col * a.lda + k] - mean) * inv_stdev;
+  }
+  double* out = a.part + static_cast<int64_t>(blockIdx.y) * 2 * a.n;
+  out[k] = dg;
+  out[a.n + k] = db;
+}
+
+__global__ void __launch_bounds__(256)
+fill_f64(double* p, int64_t h, int64_t w, int64_t ld, double value)
+{
+  const int64_t total = h * w;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += static_cast<int64_t>(gridDim.x) * 256)
+    p[i % h + (i / h) * ld] = value;
+}
+
+// n == 1 (layer norm): mean = x, variance 1 (layer_norm.cpp:92-95), y from those.
+__global__ void __launch_bounds__(256)
+ln_fwd_single_f64(RowArgs a)
+{
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (row >= a.rows) return;
+  int64_t col, g;
+  a.map.split(row, col, g);
+  const double x = a.a[g * a.map.stride + col * a.lda];
+  a.stats[g + col * a.ld_stats] = x;
+  a.stats[a.map.groups + g + col * a.ld_stats] = 1.0;
+  double y = (x - x) * (1.0 / sqrt(1.0 + a.eps));
+  if (a.gamma) y *= a.gamma[0];
+  if (a.beta) y += a.beta[0];
+  a.out[g * a.map.stride + col * a.ldo] = y;
+}
+
+// ------------------------------------------------------------------ batch norm
+struct BnArgs {
+  const double* x;
+  const double* dy;
+  double* out;
+  int64_t ldx, lddy, ldo, cs, w;
+  int bessel, training, use_pivot;
+  double eps, decay;
+  double2* part;  // [C][P]
+  double* mean;
+  double* var;
+  const double* gamma;
+  const double* beta;
+  double* rmean;
+  double* rvar;
+  double* dscale;
+  double* dbias;
+  double* dmean;
+  double* dvar;
+};
+
+// Entry j of channel c: column j / seg, position j % seg (seg = accesses per column segment).
+template <int W, typename F>
+__device__ __forceinline__ void bn_walk(int64_t seg, int64_t w, int p, int P, F f)
+{
+  // seg * w < 2^31 (host check): 32-bit division
+  const unsigned total = static_cast<unsigned>(seg * w), useg = static_cast<unsigned>(seg);
+  for (unsigned j = static_cast<unsigned>(p) * kBnThreads + threadIdx.x; j < total; j += static_cast<unsigned>(P) * kBnThreads) {
+    const unsigned col = j / useg;
+    f(static_cast<int64_t>(col), static_cast<int64_t>(W) * (j - col * useg));
+  }
+}
+
+template <int W, bool BWD>
+__global__ void __launch_bounds__(kBnThreads)
+bn_sums_f64(BnArgs a)
+{
+  __shared__ double red[2][kBnThreads / kWave];
+  const int64_t c = blockIdx.x;
+  const int P = gridDim.y, p = blockIdx.y;
+  const double* xc = a.x + c * a.cs;
+  const double* gc = BWD ? a.dy + c * a.cs : nullptr;
+  const double K = BWD ? a.mean[c] : (a.use_pivot ? xc[0] : 0.0);
+  double s = 0.0, q = 0.0;
+  bn_walk<W>(a.cs / W, a.w, p, P, [&](int64_t col, int64_t pos) {
+    double v[W], g[W];
+    load_w<W>(xc + col * a.ldx + pos, v);
+    if (BWD) load_w<W>(gc + col * a.lddy + pos, g);
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      const double d = v[j] - K;
+      if (BWD) {
+        s += g[j];
+        q += g[j] * d;
+      }
+      else {
+        s += d;
+        q += d * d;
+      }
+    }
+  });
+  s = team_sum_d<kBnThreads / kWave>(s, red[0]);
+  q = team_sum_d<kBnThreads / kWave>(q, red[1]);
+  if (threadIdx.x == 0) a.part[c * P + p] = make_double2(s, q);
+}
+
+// The P partial pairs of channel c, added in order by every thread (P <= 64, cached reads).
+__device__ __forceinline__ double2 bn_merge(const double2* part, int64_t c, int P)
+{
+  double s = 0.0, q = 0.0;
+  for (int p = 0; p < P; ++p) {
+    const double2 v = part[c * P + p];
+    s += v.x;
+    q += v.y;
+  }
+  return make_double2(s, q);
+}
+
+// FROM_PART: training (statistics from the partial sums, published by workgroup 0 of the channel);
+// otherwise mean / var are inputs (inference: the running statistics).
+template <int W, bool FROM_PART>
+__global__ void __launch_bounds__(kBnThreads)
+bn_fwd_apply_f64(BnArgs a)
+{
+  const int64_t c = blockIdx.x;
+  const int P = gridDim.y, p = blockIdx.y;
+  const double* xc = a.x + c * a.cs;
+  double* yc = a.out + c * a.cs;
+  double mean, var;
+  if (FROM_PART) {
+    const int64_t n = a.cs * a.w;
+    if (n <= 1) {
+      mean = xc[0];
+      var = 1.0;
+      if (p == 0 && threadIdx.x == 0) {
+        a.mean[c] = mean;
+        a.var[c] = var;
+      }
+    }
+    else {
+      const double K = a.use_pivot ? xc[0] : 0.0;
+      const double2 r = bn_merge(a.part, c, P);
+      const double nn = static_cast<double>(n);
+      const double dm = r.x / nn;
+      mean = K + dm;
+      var = fmax(nn * (r.y / nn - dm * dm) / (nn - (a.bessel ? 1 : 0)), a.eps);
+      if (p == 0 && threadIdx.x == 0) {
+        a.mean[c] = mean;
+        a.var[c] = var;
+        a.rmean[c] = a.decay * a.rmean[c] + (1.0 - a.decay) * mean;
+        a.rvar[c] = a.decay * a.rvar[c] + (1.0 - a.decay) * var;
+      }
+    }
+  }
+  else {
+    mean = a.mean[c];
+    var = a.var[c];
+  }
+  const double inv_stdev = 1.0 / sqrt(var + a.eps);
+  const double scale = a.gamma[c], bias = a.beta[c];
+  bn_walk<W>(a.cs / W, a.w, p, P, [&](int64_t col, int64_t pos) {
+    double v[W];
+    load_w<W>(xc + col * a.ldx + pos, v);
+#pragma unroll
+    for (int j = 0; j < W; ++j) v[j] = scale * ((v[j] - mean) * inv_stdev) + bias;
+    store_w<W>(yc + col * a.ldo + pos, v);
+  });
+}
+
+template <int W>
+__global__ void __launch_bounds__(kBnThreads)
+bn_bwd_apply_f64(BnArgs a)
+{
+  const int64_t c = blockIdx.x;
+  const int P = gridDim.y, p = blockIdx.y;
+  const double* xc = a.x + c * a.cs;
+  const double* gc = a.dy + c * a.cs;
+  double* dc = a.out + c * a.cs;
+  const int64_t n = a.cs * a.w;
+  const double mean = a.mean[c];
+  const double inv_stdev = 1.0 / sqrt(a.var[c] + a.eps);
+  const double scale = a.gamma[c];
+  const double2 r = bn_merge(a.part, c, P);  // A = sum dy, B = sum dy (x - mean)
+  double dmean = -(scale * inv_stdev) * r.x;
+  double dvar = -scale * r.y * (inv_stdev * inv_stdev * inv_stdev / 2);
+  if (!a.training) dmean = dvar = 0.0;  // statistics are constants outside training
+  if (p == 0 && threadIdx.x == 0) {
+    a.dscale[c] = r.y * inv_stdev;
+    a.dbias[c] = r.x;
+    a.dmean[c] = dmean;
+    a.dvar[c] = dvar;
+  }
+  const bool zero = n <= 1;
+  const double k0 = scale * inv_stdev;
+  const double c0 = dmean / static_cast<double>(n);
+  const double c1 = dvar * 2 / static_cast<double>(n - (a.bessel ? 1 : 0));
+  bn_walk<W>(a.cs / W, a.w, p, P, [&](int64_t col, int64_t pos) {
+    double v[W], g[W];
+    load_w<W>(xc + col * a.ldx + pos, v);
+    load_w<W>(gc + col * a.lddy + pos, g);
+#pragma unroll
+    for (int j = 0; j < W; ++j) g[j] = zero ? 0.0 : g[j] * k0 + c0 + c1 * (v[j] - mean);
+    store_w<W>(dc + col * a.ldo + pos, g);
+  });
+}
+
+// ================================================================== host side
+static bool aligned_rows(const void* p, int64_t stride, int64_t ld, int64_t groups, int64_t w)
+{
+  return aligned16(p) && (groups <= 1 || stride % 2 == 0) && (w <= 1 || ld % 2 == 0);
+}
+
+// Workgroups of a row launch: a few per compute unit.  With weight gradients every team leaves a
+// partial row of 2n doubles, so the launch is held to kWgradMaxGroups workgroups (at most
+// 4 * kWgradMaxGroups partial rows, which is what the workspace is sized for).
+constexpr int64_t kWgradMaxGroups = 512;
+
+static int64_t row_grid(int64_t rows, int teams, bool wgrad = false)
+{
+  int cus = compute_units();
+  if (cus < 1) cus = 256;
+  const int64_t want = ceil_div(rows, teams);
+  int64_t cap = static_cast<int64_t>(cus) * 8;
+  if (wgrad && cap > kWgradMaxGroups) cap = kWgradMaxGroups;
+  return want < cap ? want : cap;
+}
+
+#define LBN_F64_SHAPES(X, W)                                                                          \
+  X(64, 1, W) X(64, 2, W) X(64, 4, W) X(64, 8, W) X(256, 1, W) X(256, 2, W) X(256, 4, W) X(256, 8, W) \
+  X(1024, 1, W) X(1024, 2, W) X(1024, 4, W) X(1024, 8, W) X(1024, 16, W)
+
+static int sm_check(int64_t G, int64_t n, int64_t stride, int64_t w, const int64_t* lds, int nld)
+{
+  if (G < 0 || n < 0 || w < 0 || stride < 0) return LBN_ERR_INVALID_ARGUMENT;
+  const int64_t height = G > 0 ? (G - 1) * stride + n : 0;
+  for (int i = 0; i < nld; ++i)
+    if (w > 1 && lds[i] < height) return LBN_ERR_INVALID_ARGUMENT;
+  if (G * w > (int64_t(1) << 30) || n > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+  return LBN_OK;
+}
+
+template <int KIND>
+static int sm_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t w, const double* x, int64_t ldx,
+                  double* y, int64_t ldy)
+{
+  const int64_t lds[2] = {ldx, ldy};
+  if (int e = sm_check(G, n, stride, w, lds, 2)) return e;
+  if (G == 0 || n == 0 || w == 0) return LBN_OK;
+  if (!x || !y) return LBN_ERR_INVALID_ARGUMENT;
+  RowArgs a{};
+  a.a = x, a.out = y, a.lda = ldx, a.ldo = ldy, a.map = RowMap{G, stride}, a.rows = G * w, a.n = static_cast<int>(n);
+  const bool vec = n % 2 == 0 && aligned_rows(x, stride, ldx, G, w) && aligned_rows(y, stride, ldy, G, w);
+  const int W = vec ? 2 : 1;
+  a.units = static_cast<int>(n / W);
+  const RowShape s = pick_shape(a.units, a.rows);
+#define X(TPR, V, WW)                                                                                   \
+  if (s.tpr == TPR && s.v == V && W == WW) {                                                            \
+    hipLaunchKernelGGL((sm_fwd_rows_f64<KIND, TPR, V, WW>), dim3(static_cast<unsigned>(row_grid(a.rows, Team<TPR>::kTeams))), \
+                       dim3(Team<TPR>::kThreads), 0, st, a);                                            \
+    return launch_status();                                                                             \
+  }
+  LBN_F64_SHAPES(X, 1) LBN_F64_SHAPES(X, 2)
+#undef X
+  hipLaunchKernelGGL((rows_stream_f64<0, KIND>), dim3(static_cast<unsigned>(a.rows)), dim3(kStreamThreads), 0, st, a);
+  return launch_status();
+}
+
+template <int KIND>
+static int sm_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t w, const double* y, int64_t ldy,
+                  const double* dy, int64_t lddy, double* dx, int64_t lddx)
+{
+  const int64_t lds[3] = {ldy, lddy, lddx};
+  if (int e = sm_check(G, n, stride, w, lds, 3)) return e;
+  if (G == 0 || n == 0 || w == 0) return LBN_OK;
+  if (!y || !dy || !dx) return LBN_ERR_INVALID_ARGUMENT;
+  RowArgs a{};
+  a.a = y, a.g = dy, a.out = dx, a.lda = ldy, a.ldg = lddy, a.ldo = lddx, a.map = RowMap{G, stride};
+  a.rows = G * w, a.n = static_cast<int>(n);
+  const bool vec = n % 2 == 0 && aligned_rows(y, stride, ldy, G, w) && aligned_rows(dy, stride, lddy, G, w) &&
+                   aligned_rows(dx, stride, lddx, G, w);
+  const int W = vec ? 2 : 1;
+  a.units = static_cast<int>(n / W);
+  RowShape s = pick_shape(a.units, a.rows);
+  if (s.v > 8) s = RowShape{0, 0};  // two tensors in registers: at most 8 accesses each
+#define X(TPR, V, WW)                                                                                   \
+  if (V <= 8 && s.tpr == TPR && s.v == V && W == WW) {                                                  \
+    hipLaunchKernelGGL((sm_bwd_rows_f64<KIND, TPR, (V <= 8 ? V : 8), WW>),                              \
+                       dim3(static_cast<unsigned>(row_grid(a.rows, Team<TPR>::kTeams))),                \
+                       dim3(Team<TPR>::kThreads), 0, st, a);                                            \
+    return launch_status();                                                                             \
+  }
+  LBN_F64_SHAPES(X, 1) LBN_F64_SHAPES(X, 2)
+#undef X
+  hipLaunchKernelGGL((rows_stream_f64<1, KIND>), dim3(static_cast<unsigned>(a.rows)), dim3(kStreamThreads), 0, st, a);
+  return launch_status();
+}
+
+static size_t ln_bwd_workspace(int64_t n, int64_t rows)
+{
+  if (n <= 0 || rows <= 0) return 0;
+  const int64_t teams = kWgradMaxGroups * 4;  // the largest launch: four teams per workgroup
+  const int64_t parts = rows < teams ? rows : teams;
+  return static_cast<size_t>(parts) * 2 * n * sizeof(double);
+}
+
+static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t w, double eps, const double* x,
+                  int64_t ldx, double* y, int64_t ldy, double* stats, int64_t ld_stats, const double* gamma,
+                  const double* beta, int flags)
+{
+  const int64_t lds[2] = {ldx, ldy};
+  if (int e = sm_check(G, n, stride, w, lds, 2)) return e;
+  if (G == 0 || n == 0 || w == 0) return LBN_OK;
+  if (!x || !y || !stats || (w > 1 && ld_stats < 2 * G)) return LBN_ERR_INVALID_ARGUMENT;
+  RowArgs a{};
+  a.a = x, a.out = y, a.lda = ldx, a.ldo = ldy, a.map = RowMap{G, stride}, a.rows = G * w, a.n = static_cast<int>(n);
+  a.eps = eps, a.stats = stats, a.ld_stats = ld_stats, a.gamma = gamma, a.beta = beta;
+  a.sumsq = (flags & LBN_STATS_SUMSQ) ? 1 : 0;
+  if (n == 1) {
+    hipLaunchKernelGGL(ln_fwd_single_f64, dim3(static_cast<unsigned>(ceil_div(a.rows, 256))), dim3(256), 0, st, a);
+    return launch_status();
+  }
+  const bool vec = n % 2 == 0 && aligned_rows(x, stride, ldx, G, w) && aligned_rows(y, stride, ldy, G, w);
+  const int W = vec ? 2 : 1;
+  a.units = static_cast<int>(n / W);
+  const RowShape s = pick_shape(a.units, a.rows);
+#define X(TPR, V, WW)                                                                                   \
+  if (s.tpr == TPR && s.v == V && W == WW) {                                                            \
+    hipLaunchKernelGGL((ln_fwd_rows_f64<TPR, V, WW>), dim3(static_cast<unsigned>(row_grid(a.rows, Team<TPR>::kTeams))), \
+                       dim3(Team<TPR>::kThreads), 0, st, a);                                            \
+    return launch_status();                                                                             \
+  }
+  LBN_F64_SHAPES(X, 1) LBN_F64_SHAPES(X, 2)
+#undef X
+  hipLaunchKernelGGL((rows_stream_f64<2, 0>), dim3(static_cast<unsigned>(a.rows)), dim3(kStreamThreads), 0, st, a);
+  return launch_status();
+}
+
+static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t w, double eps, const double* x,
+                  int64_t ldx, const double* dy, int64_t lddy, double* dx, int64_t lddx, const double* stats,
+                  int64_t ld_stats, double* sgrad, int64_t ld_sgrad, const double* gamma, double* dgamma,
+                  double* dbeta, void* ws, size_t ws_bytes)
+{
+  const int64_t lds[3] = {ldx, lddy, lddx};
+  if (int e = sm_check(G, n, stride, w, lds, 3)) return e;
+  if (G == 0 || n == 0 || w == 0) return LBN_OK;
+  if (!x || !dy || !dx || !stats || !sgrad || (w > 1 && (ld_stats < 2 * G || ld_sgrad < 2 * G)))
+    return LBN_ERR_INVALID_ARGUMENT;
+  if (dgamma && !gamma) return LBN_ERR_INVALID_ARGUMENT;
+  const bool wgrad = dgamma || dbeta;
+  const int64_t rows = G * w;
+  if (n <= 1) {
+    // a single entry per group: the output is constant and every gradient zero
+    // (layer_norm.cpp:189-192; the weight-gradient buffers were zeroed at :300-309)
+    const int64_t height = (G - 1) * stride + n;
+    const int64_t want = ceil_div(height * w, 256);
+    hipLaunchKernelGGL(fill_f64, dim3(static_cast<unsigned>(want > 4096 ? 4096 : want)), dim3(256), 0, st, dx, height,
+                       w, lddx, 0.0);
+    if (dgamma) hipLaunchKernelGGL(fill_f64, dim3(1), dim3(256), 0, st, dgamma, n, int64_t(1), n, 0.0);
+    if (dbeta) hipLaunchKernelGGL(fill_f64, dim3(1), dim3(256), 0, st, dbeta, n, int64_t(1), n, 0.0);
+    return launch_status();
+  }
+  RowArgs a{};
+  a.a = x, a.g = dy, a.out = dx, a.lda = ldx, a.ldg = lddy, a.ldo = lddx, a.map = RowMap{G, stride};
+  a.rows = rows, a.n = static_cast<int>(n), a.eps = eps, a.stats = const_cast<double*>(stats), a.ld_stats = ld_stats;
+  a.sgrad = sgrad, a.ld_sgrad = ld_sgrad, a.gamma = gamma, a.part = static_cast<double*>(ws);
+  if (wgrad && (!ws || ws_bytes < ln_bwd_workspace(n, rows) || !aligned16(ws))) return LBN_ERR_WORKSPACE;
+  const bool vec = n % 2 == 0 && aligned_rows(x, stride, ldx, G, w) && aligned_rows(dy, stride, lddy, G, w) &&
+                   aligned_rows(dx, stride, lddx, G, w);
+  const int W = vec ? 2 : 1;
+  a.units = static_cast<int>(n / W);
+  RowShape s = pick_shape(a.units, rows);
+  if (s.v > 8) s = RowShape{0, 0};
+#define X(TPR, V, WW)                                                                                   \
+  if (V <= 8 && s.tpr == TPR && s.v == V && W == WW) {                                                  \
+    constexpr int VV = V <= 8 ? V : 8;                                                                  \
+    const int64_t grid = row_grid(rows, Team<TPR>::kTeams, wgrad);                                      \
+    if (wgrad) {                                                                                        \
+      hipLaunchKernelGGL((ln_bwd_rows_f64<TPR, VV, WW, true>), dim3(static_cast<unsigned>(grid)),       \
+                         dim3(Team<TPR>::kThreads), 0, st, a);                                          \
+      hipLaunchKernelGGL(ln_wgrad_reduce_f64, dim3(static_cast<unsigned>(ceil_div(2 * n, 256))), dim3(256), 0, st, \
+                         a.part, grid * Team<TPR>::kTeams, n, dgamma, dbeta);                           \
+    }                                                                                                   \
+    else {                                                                                              \
+      hipLaunchKernelGGL((ln_bwd_rows_f64<TPR, VV, WW, false>), dim3(static_cast<unsigned>(grid)),      \
+                         dim3(Team<TPR>::kThreads), 0, st, a);                                          \
+    }                                                                                                   \
+    return launch_status();                                                                             \
+  }
+  LBN_F64_SHAPES(X, 1) LBN_F64_SHAPES(X, 2)
+#undef X
+  hipLaunchKernelGGL((rows_stream_f64<3, 0>), dim3(static_cast<unsigned>(rows)), dim3(kStreamThreads), 0, st, a);
+  if (wgrad) {
+    int64_t slabs = ceil_div(2048, ceil_div(n, 256));
+    if (slabs > rows) slabs = rows;
+    if (slabs > 256) slabs = 256;
+    const int64_t per = ceil_div(rows, slabs);
+    slabs = ceil_div(rows, per);
+    hipLaunchKernelGGL(ln_wgrad_columns_f64, dim3(static_cast<unsigned>(ceil_div(n, 256)), static_cast<unsigned>(slabs)),
+                       dim3(256), 0, st, a, per);
+    hipLaunchKernelGGL(ln_wgrad_reduce_f64, dim3(static_cast<unsigned>(ceil_div(2 * n, 256))), dim3(256), 0, st, a.part,
+                       slabs, n, dgamma, dbeta);
+  }
+  return launch_status();
+}
+
+static int bn_split(int64_t C, int64_t cs, int64_t w)
+{
+  int64_t P = ceil_div(2048, C);
+  const int64_t most = ceil_div(cs * w, 2 * kBnThreads);
+  if (P > most) P = most;
+  if (P > kBnMaxSplit) P = kBnMaxSplit;
+  return static_cast<int>(P < 1 ? 1 : P);
+}
+
+static int bn_check(int64_t C, int64_t cs, int64_t w, const int64_t* lds, int nld)
+{
+  if (C < 0 || cs < 0 || w < 0) return LBN_ERR_INVALID_ARGUMENT;
+  for (int i = 0; i < nld; ++i)
+    if (w > 1 && lds[i] < C * cs) return LBN_ERR_INVALID_ARGUMENT;
+  if (C > (int64_t(1) << 30) || cs * w >= (int64_t(1) << 31)) return LBN_ERR_UNSUPPORTED;
+  return LBN_OK;
+}
+
+static bool bn_vec(int64_t cs, int64_t w, const void* p, int64_t ld)
+{
+  return cs % 2 == 0 && aligned16(p) && (w <= 1 || ld % 2 == 0);
+}
+
+}  // namespace f64
+}  // namespace lbn
+
+using namespace lbn;
+using namespace lbn::f64;
+
+extern "C" {
+
+int lbn_softmax_fwd_f64(lbn_stream_t stream, int64_t height, int64_t width, const double* x, int64_t ldx,
+                        double* y, int64_t ldy)
+{
+  return f64::sm_fwd<kSoftmax>(as_stream(stream), 1, height, height, width, x, ldx, y, ldy);
+}
+
+int lbn_softmax_bwd_f64(lbn_stream_t stream, int64_t height, int64_t width, const double* y, int64_t ldy,
+                        const double* dy, int64_t lddy, double* dx, int64_t lddx)
+{
+  return f64::sm_bwd<kSoftmax>(as_stream(stream), 1, height, height, width, y, ldy, dy, lddy, dx, lddx);
+}
+
+int lbn_log_softmax_fwd_f64(lbn_stream_t stream, int64_t height, int64_t width, const double* x, int64_t ldx,
+                            double* y, int64_t ldy)
+{
+  return f64::sm_fwd<kLogSoftmax>(as_stream(stream), 1, height, height, width, x, ldx, y, ldy);
+}
+
+int lbn_log_softmax_bwd_f64(lbn_stream_t stream, int64_t height, int64_t width, const double* y, int64_t ldy,
+                            const double* dy, int64_t lddy, double* dx, int64_t lddx)
+{
+  return f64::sm_bwd<kLogSoftmax>(as_stream(stream), 1, height, height, width, y, ldy, dy, lddy, dx, lddx);
+}
+
+int lbn_channelwise_softmax_fwd_f64(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                    int64_t channel_stride, int64_t width, const double* x, int64_t ldx,
+                                    double* y, int64_t ldy)
+{
+  return f64::sm_fwd<kChannelwise>(as_stream(stream), channels, channel_size, channel_stride, width, x, ldx, y, ldy);
+}
+
+int lbn_channelwise_softmax_bwd_f64(lbn_stream_t stream, int64_t channels, int64_t channel_size,
+                                    int64_t channel_stride, int64_t width, const double* y, int64_t ldy,
+                                    const double* dy, int64_t lddy, double* dx, int64_t lddx)
+{
+  return f64::sm_bwd<kChannelwise>(as_stream(stream), channels, channel_size, channel_stride, width, y, ldy, dy, lddy,
+                                   dx, lddx);
+}
+
+int lbn_layer_norm_fwd_f64(lbn_stream_t stream, int64_t num_groups, int64_t norm_size, int64_t norm_stride,
+                           int64_t width, double epsilon, const double* x, int64_t ldx, double* y, int64_t ldy,
+                           double* stats, int64_t ld_stats, const double* scale, const double* bias, int flags)
+{
+  return f64::ln_fwd(as_stream(stream), num_groups, norm_size, norm_stride, width, epsilon, x, ldx, y, ldy, stats,
+                     ld_stats, scale, bias, flags);
+}
+
+size_t lbn_layer_norm_bwd_workspace_bytes_f64(int64_t num_groups, int64_t norm_size, int64_t width,
+                                              int has_weight_grads)
+{
+  if (!has_weight_grads || num_groups <= 0 || width <= 0) return 0;
+  return f64::ln_bwd_workspace(norm_size, num_groups * width);
+}
+
+int lbn_layer_norm_bwd_f64(lbn_stream_t stream, int64_t num_groups, int64_t norm_size, int64_t norm_stride,
+                           int64_t width, double epsilon, const double* x, int64_t ldx, const double* dy,
+                           int64_t lddy, double* dx, int64_t lddx, const double* stats, int64_t ld_stats,
+                           double* stats_grad, int64_t ld_stats_grad, const double* scale, double* dscale,
+                           double* dbias, void* workspace, size_t workspace_bytes)
+{
+  return f64::ln_bwd(as_stream(stream), num_groups, norm_size, norm_stride, width, epsilon, x, ldx, dy, lddy, dx, lddx,
+                     stats, ld_stats, stats_grad, ld_stats_grad, scale, dscale, dbias, workspace, workspace_bytes);
+}
+
+size_t lbn_batch_norm_workspace_bytes_f64(int64_t channels, int64_t channel_size, int64_t width)
+{
+  if (channels <= 0 || channel_size <= 0 || width <= 0) return 0;
+  return static_cast<size_t>(channels) * f64::kBnMaxSplit * sizeof(double2);
+}
+
+int lbn_batch_norm_fwd_f64(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w, int bessel, double epsilon,
+                           double decay, int training, const double* x, int64_t ldx, double* y, int64_t ldy,
+                           double* mean, double* var, const double* scale, const double* bias,
+                           double* running_mean, double* running_var, void* workspace, size_t workspace_bytes,
+                           int flags)
+{
+  const int64_t lds[2] = {ldx, ldy};
+  if (int e = f64::bn_check(C, cs, w, lds, 2)) return e;
+  if (C == 0 || cs == 0 || w == 0) return LBN_OK;
+  if (!x || !y || !scale || !bias || !running_mean || !running_var) return LBN_ERR_INVALID_ARGUMENT;
+  if (training && (!mean || !var)) return LBN_ERR_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  f64::BnArgs a{};
+  a.x = x, a.out = y, a.ldx = ldx, a.ldo = ldy, a.cs = cs, a.w = w, a.bessel = bessel, a.training = training;
+  a.use_pivot = (flags & LBN_STATS_SUMSQ) ? 0 : 1, a.eps = epsilon, a.decay = decay;
+  a.gamma = scale, a.beta = bias, a.rmean = running_mean, a.rvar = running_var;
+  const int P = f64::bn_split(C, cs, w);
+  const dim3 grid(static_cast<unsigned>(C), P);
+  const bool vec = f64::bn_vec(cs, w, x, ldx) && f64::bn_vec(cs, w, y, ldy);
+  if (!training) {
+    a.mean = running_mean, a.var = running_var;
+    if (vec) hipLaunchKernelGGL((bn_fwd_apply_f64<2, false>), grid, dim3(f64::kBnThreads), 0, st, a);
+    else hipLaunchKernelGGL((bn_fwd_apply_f64<1, false>), grid, dim3(f64::kBnThreads), 0, st, a);
+    return launch_status();
+  }
+  if (!workspace || workspace_bytes < lbn_batch_norm_workspace_bytes_f64(C, cs, w) || !aligned16(workspace))
+    return LBN_ERR_WORKSPACE;
+  a.part = static_cast<double2*>(workspace), a.mean = mean, a.var = var;
+  if (vec) {
+    hipLaunchKernelGGL((bn_sums_f64<2, false>), grid, dim3(f64::kBnThreads), 0, st, a);
+    hipLaunchKernelGGL((bn_fwd_apply_f64<2, true>), grid, dim3(f64::kBnThreads), 0, st, a);
+  }
+  else {
+    hipLaunchKernelGGL((bn_sums_f64<1, false>), grid, dim3(f64::kBnThreads), 0, st, a);
+    hipLaunchKernelGGL((bn_fwd_apply_f64<1, true>), grid, dim3(f64::kBnThreads), 0, st, a);
+  }
+  return launch_status();
+}
+
+int lbn_batch_norm_bwd_f64(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w, int bessel, double epsilon,
+                           int training, const double* x, int64_t ldx, const double* dy, int64_t lddy, double* dx,
+                           int64_t lddx, const double* mean, const double* var, const double* running_mean,
+                           const double* running_var, const double* scale, double* dscale, double* dbias,
+                           double* dmean, double* dvar, void* workspace, size_t workspace_bytes)
+{
+  const int64_t lds[3] = {ldx, lddy, lddx};
+  if (int e = f64::bn_check(C, cs, w, lds, 3)) return e;
+  if (C == 0 || cs == 0 || w == 0) return LBN_OK;
+  const double* use_mean = training ? mean : running_mean;
+  const double* use_var = training ? var : running_var;
+  if (!x || !dy || !dx || !use_mean || !use_var || !scale || !dscale || !dbias || !dmean || !dvar)
+    return LBN_ERR_INVALID_ARGUMENT;
+  if (!workspace || workspace_bytes < lbn_batch_norm_workspace_bytes_f64(C, cs, w) || !aligned16(workspace))
+    return LBN_ERR_WORKSPACE;
+  hipStream_t st = as_stream(stream);
+  f64::BnArgs a{};
+  a.x = x, a.dy = dy, a.out = dx, a.ldx = ldx, a.lddy = lddy, a.ldo = lddx, a.cs = cs, a.w = w, a.bessel = bessel;
+  a.training = training, a.eps = epsilon, a.part = static_cast<double2*>(workspace);
+  a.mean = const_cast<double*>(use_mean), a.var = const_cast<double*>(use_var), a.gamma = scale;
+  a.dscale = dscale, a.dbias = dbias, a.dmean = dmean, a.dvar = dvar;
+  const int P = f64::bn_split(C, cs, w);
+  const dim3 grid(static_cast<unsigned>(C), P);
+  const bool vec = f64::bn_vec(cs, w, x, ldx) && f64::bn_vec(cs, w, dy, lddy) && f64::bn_vec(cs, w, dx, lddx);
+  if (vec) {
+    hipLaunchKernelGGL((bn_sums_f64<2, true>), grid, dim3(f64::kBnThreads), 0, st, a);
+    hipLaunchKernelGGL((bn_bwd_apply_f64<2>), grid, dim3(f64::kBnThreads), 0, st, a);
+  }
+  else {
+    hipLaunchKernelGGL((bn_sums_f64<1, true>), grid, dim3(f64::kBnThreads), 0, st, a);
+    hipLaunchKernelGGL((bn_bwd_apply_f64<1>), grid, dim3(f64::kBnThreads), 0, st, a);
+  }
+  return launch_status();
+}
+
+}  // extern "C"

@@ -85,13 +85,14 @@ class DeviceMatrix:
 
 
 class _Vector:
-    """Weights / gradient vector in device memory (fp32)."""
+    """Weights / gradient vector in device memory (fp32; binary64 for a layer of doubles)."""
 
-    def __init__(self, n, device="cuda", values=None):
+    def __init__(self, n, device="cuda", values=None, dtype=torch.float32):
         if values is None:
-            self.tensor = torch.empty(max(int(n), 1), dtype=torch.float32, device=device)
+            self.tensor = torch.empty(max(int(n), 1), dtype=dtype, device=device)
         else:
-            self.tensor = torch.as_tensor(np.asarray(values, dtype=np.float32)).to(device).contiguous()
+            npdt = np.float64 if dtype == torch.float64 else np.float32
+            self.tensor = torch.as_tensor(np.asarray(values, dtype=npdt)).to(device).contiguous()
         self.n = int(n)
 
     def Buffer(self):
@@ -227,8 +228,12 @@ class layer_norm_layer(_Layer):
     """lbann::layer_norm_layer (include/lbann/layers/regularizers/layer_norm.hpp:53-143)."""
 
     def __init__(self, dims, epsilon=1e-5, scale=False, bias=False, start_dim=0,
-                 scale_values=None, bias_values=None, stats_mode=LBN_STATS_TWO_PASS, device="cuda"):
+                 scale_values=None, bias_values=None, stats_mode=LBN_STATS_TWO_PASS, device="cuda",
+                 datatype=torch.float32):
+        """datatype: the reference's TensorDataType; torch.float64 selects the _f64 entry points
+        (weights, statistics and their gradients are then doubles as well)."""
         super().__init__(device)
+        self.datatype = wt = torch.float64 if datatype == torch.float64 else torch.float32
         self.dims = tuple(int(d) for d in dims)
         self.m_epsilon, self.m_scale, self.m_bias, self.m_start_dim = float(epsilon), bool(scale), bool(bias), int(start_dim)
         sd = self.m_start_dim if self.m_start_dim >= 0 else len(self.dims) + self.m_start_dim
@@ -241,16 +246,18 @@ class layer_norm_layer(_Layer):
         n = self.normalization_size
         self.weights = []
         if self.m_scale:
-            self.weights.append(_Vector(n, device, scale_values if scale_values is not None else np.ones(n)))
+            self.weights.append(_Vector(n, device, scale_values if scale_values is not None else np.ones(n), wt))
         if self.m_bias:
-            self.weights.append(_Vector(n, device, bias_values if bias_values is not None else np.zeros(n)))
-        self.m_scale_gradient = _Vector(n, device) if self.m_scale else None
-        self.m_bias_gradient = _Vector(n, device) if self.m_bias else None
+            self.weights.append(_Vector(n, device, bias_values if bias_values is not None else np.zeros(n), wt))
+        self.m_scale_gradient = _Vector(n, device, dtype=wt) if self.m_scale else None
+        self.m_bias_gradient = _Vector(n, device, dtype=wt) if self.m_bias else None
         self.m_statistics = None
         self.m_statistics_gradient = None
         self.stats_mode = stats_mode
 
     def _suffix(self):
+        if self.datatype == torch.float64:
+            return "f64"
         return "f16" if self.prev_activations.dtype == torch.float16 else "f32"
 
     def _scratch(self):
@@ -260,6 +267,10 @@ class layer_norm_layer(_Layer):
         G, n = self.num_normalized, self.normalization_size
         esize = 2 if x.dtype == torch.float16 else 4
         lib = capi.lib()
+        if self.datatype == torch.float64:
+            self._ws.header = False
+            return self._ws.get(lib.lbn_layer_norm_bwd_workspace_bytes_f64(G, n, x.width, int(self.m_scale or self.m_bias)),
+                                self.device)
         need = max(lib.lbn_layer_norm_fwd_workspace_bytes(G, n, x.width, esize),
                    lib.lbn_layer_norm_bwd_workspace_bytes(G, n, x.width, int(self.m_scale or self.m_bias), esize))
         return self._ws.get(need, self.device)
@@ -268,10 +279,15 @@ class layer_norm_layer(_Layer):
         x, y = self.prev_activations, self.activations
         G, n = self.num_normalized, self.normalization_size
         if self.m_statistics is None or self.m_statistics.width != x.width:
-            self.m_statistics = DeviceMatrix(2 * G, x.width, device=self.device)
+            self.m_statistics = DeviceMatrix(2 * G, x.width, dtype=self.datatype, device=self.device)
         scale = self.weights[0].Buffer() if self.m_scale else _null()
         bias = self.weights[-1].Buffer() if self.m_bias else _null()
         ws, nb = self._scratch()
+        if self.datatype == torch.float64:  # no forward scratch
+            return ("lbn_layer_norm_fwd_f64",
+                    (_stream(), G, n, self.normalization_stride, x.width,
+                     self.m_epsilon, x.Buffer(), x.ldim, y.Buffer(), y.ldim, self.m_statistics.Buffer(),
+                     self.m_statistics.ldim, scale, bias, self.stats_mode))
         return (f"lbn_layer_norm_fwd_{self._suffix()}",
                 (_stream(), G, n, self.normalization_stride, x.width,
                  self.m_epsilon, x.Buffer(), x.ldim, y.Buffer(), y.ldim, self.m_statistics.Buffer(),
@@ -281,7 +297,7 @@ class layer_norm_layer(_Layer):
         x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
         G, n = self.num_normalized, self.normalization_size
         if self.m_statistics_gradient is None or self.m_statistics_gradient.width != x.width:
-            self.m_statistics_gradient = DeviceMatrix(2 * G, x.width, device=self.device)
+            self.m_statistics_gradient = DeviceMatrix(2 * G, x.width, dtype=self.datatype, device=self.device)
         scale = self.weights[0].Buffer() if self.m_scale else _null()
         dscale = self.m_scale_gradient.Buffer() if self.m_scale else _null()
         dbias = self.m_bias_gradient.Buffer() if self.m_bias else _null()
@@ -411,8 +427,9 @@ class batch_normalization_layer(_Layer):
     local statistics (statistics_group_size == 1)."""
 
     def __init__(self, dims, decay=0.9, epsilon=1e-5, bessel_correction=True, scale_values=None,
-                 bias_values=None, stats_mode=LBN_STATS_TWO_PASS, device="cuda"):
+                 bias_values=None, stats_mode=LBN_STATS_TWO_PASS, device="cuda", datatype=torch.float32):
         super().__init__(device)
+        self.datatype = wt = torch.float64 if datatype == torch.float64 else torch.float32
         self.dims = tuple(int(d) for d in dims)
         self.m_decay, self.m_epsilon, self.m_bessel_correction = float(decay), float(epsilon), bool(bessel_correction)
         self.num_channels = self.dims[0]
@@ -420,27 +437,39 @@ class batch_normalization_layer(_Layer):
         C = self.num_channels
         # weights 0..3: scale, bias, running mean, running variance (defaults 1, 0, 0, 1)
         self.weights = [
-            _Vector(C, device, scale_values if scale_values is not None else np.ones(C)),
-            _Vector(C, device, bias_values if bias_values is not None else np.zeros(C)),
-            _Vector(C, device, np.zeros(C)),
-            _Vector(C, device, np.ones(C)),
+            _Vector(C, device, scale_values if scale_values is not None else np.ones(C), wt),
+            _Vector(C, device, bias_values if bias_values is not None else np.zeros(C), wt),
+            _Vector(C, device, np.zeros(C), wt),
+            _Vector(C, device, np.ones(C), wt),
         ]
         # m_mean_and_var / m_mean_and_var_gradient: C x 2, column 0 mean, column 1 variance
-        self.m_mean_and_var = DeviceMatrix(C, 2, device=device)
-        self.m_mean_and_var_gradient = DeviceMatrix(C, 2, device=device)
-        self.m_scale_gradient = _Vector(C, device)
-        self.m_bias_gradient = _Vector(C, device)
+        self.m_mean_and_var = DeviceMatrix(C, 2, dtype=wt, device=device)
+        self.m_mean_and_var_gradient = DeviceMatrix(C, 2, dtype=wt, device=device)
+        self.m_scale_gradient = _Vector(C, device, dtype=wt)
+        self.m_bias_gradient = _Vector(C, device, dtype=wt)
         self.training = True
         self.stats_mode = stats_mode
 
     def _col(self, m, j):
-        return capi.vp(m.tensor.data_ptr() + 4 * j * m.ldim)
+        return capi.vp(m.tensor.data_ptr() + m.tensor.element_size() * j * m.ldim)
+
+    def _scratch(self, width):
+        C, cs = self.num_channels, self.channel_size
+        if self.datatype == torch.float64:
+            self._ws.header = False
+            return self._ws.get(capi.lib().lbn_batch_norm_workspace_bytes_f64(C, cs, width), self.device)
+        return self._ws.get(capi.lib().lbn_batch_norm_workspace_bytes(C, cs, width), self.device)
+
+    def _suffix(self, x):
+        if self.datatype == torch.float64:
+            return "f64"
+        return "f16" if x.dtype == torch.float16 else "f32"
 
     def fp_call(self):
         x, y = self.prev_activations, self.activations
         C, cs = self.num_channels, self.channel_size
-        ws, nb = self._ws.get(capi.lib().lbn_batch_norm_workspace_bytes(C, cs, x.width), self.device)
-        return (f"lbn_batch_norm_fwd_{'f16' if x.dtype == torch.float16 else 'f32'}",
+        ws, nb = self._scratch(x.width)
+        return (f"lbn_batch_norm_fwd_{self._suffix(x)}",
                 (_stream(), C, cs, x.width, int(self.m_bessel_correction),
                  self.m_epsilon, self.m_decay, int(self.training), x.Buffer(), x.ldim, y.Buffer(), y.ldim,
                  self._col(self.m_mean_and_var, 0), self._col(self.m_mean_and_var, 1),
@@ -450,9 +479,9 @@ class batch_normalization_layer(_Layer):
     def bp_call(self):
         x, dy, dx = self.prev_activations, self.prev_error_signals, self.error_signals
         C, cs = self.num_channels, self.channel_size
-        ws, nb = self._ws.get(capi.lib().lbn_batch_norm_workspace_bytes(C, cs, x.width), self.device)
-        name = f"lbn_batch_norm_bwd_{'f16' if x.dtype == torch.float16 else 'f32'}"
-        if self.stats_mode & LBN_STATS_REFERENCE_ORDER:  # parity tests: the reference's order of summation
+        ws, nb = self._scratch(x.width)
+        name = f"lbn_batch_norm_bwd_{self._suffix(x)}"
+        if self.stats_mode & LBN_STATS_REFERENCE_ORDER and self.datatype != torch.float64:  # parity tests: the reference's order of summation
             name = "lbn_batch_norm_bwd_reference_order_f32"
         return (name,
                 (_stream(), C, cs, x.width, int(self.m_bessel_correction),
@@ -468,16 +497,21 @@ class _softmax_like(_Layer):
 
     @staticmethod
     def _suffix(m):
-        return "f16" if m.dtype == torch.float16 else "f32"
+        return {torch.float16: "f16", torch.float64: "f64"}.get(m.dtype, "f32")
 
     def fp_call(self):
         x, y = self.prev_activations, self.activations
+        if x.dtype == torch.float64:  # TensorDataType = double: no scratch
+            return (f"lbn_{self._name}_fwd_f64", (_stream(), x.height, x.width, x.Buffer(), x.ldim, y.Buffer(), y.ldim))
         ws, nb = self._ws.get(capi.lib().lbn_softmax_workspace_bytes(x.height, x.width), self.device)
         return (f"lbn_{self._name}_fwd_{self._suffix(x)}",
                 (_stream(), x.height, x.width, x.Buffer(), x.ldim, y.Buffer(), y.ldim, ws, nb))
 
     def bp_call(self):
         y, dy, dx = self.activations, self.prev_error_signals, self.error_signals
+        if y.dtype == torch.float64:
+            return (f"lbn_{self._name}_bwd_f64",
+                    (_stream(), y.height, y.width, y.Buffer(), y.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim))
         ws, nb = self._ws.get(capi.lib().lbn_softmax_workspace_bytes(y.height, y.width), self.device)
         return (f"lbn_{self._name}_bwd_{self._suffix(y)}",
                 (_stream(), y.height, y.width, y.Buffer(), y.ldim, dy.Buffer(), dy.ldim, dx.Buffer(),
@@ -528,6 +562,9 @@ class channelwise_softmax_layer(_Layer):
     def fp_call(self):
         x, y = self.prev_activations, self.activations
         cs, stride, C = self.get_channel_size_and_stride()
+        if x.dtype == torch.float64:
+            return ("lbn_channelwise_softmax_fwd_f64",
+                    (_stream(), C, cs, stride, x.width, x.Buffer(), x.ldim, y.Buffer(), y.ldim))
         ws, nb = self._ws.get(capi.lib().lbn_channelwise_softmax_workspace_bytes(C, cs, x.width), self.device)
         return ("lbn_channelwise_softmax_fwd_f32",
                 (_stream(), C, cs, stride, x.width, x.Buffer(), x.ldim, y.Buffer(), y.ldim, ws, nb))
@@ -535,6 +572,9 @@ class channelwise_softmax_layer(_Layer):
     def bp_call(self):
         y, dy, dx = self.activations, self.prev_error_signals, self.error_signals
         cs, stride, C = self.get_channel_size_and_stride()
+        if y.dtype == torch.float64:
+            return ("lbn_channelwise_softmax_bwd_f64",
+                    (_stream(), C, cs, stride, y.width, y.Buffer(), y.ldim, dy.Buffer(), dy.ldim, dx.Buffer(), dx.ldim))
         ws, nb = self._ws.get(capi.lib().lbn_channelwise_softmax_workspace_bytes(C, cs, y.width), self.device)
         return ("lbn_channelwise_softmax_bwd_f32",
                 (_stream(), C, cs, stride, y.width, y.Buffer(), y.ldim, dy.Buffer(), dy.ldim, dx.Buffer(),

@@ -27,20 +27,22 @@ void attach(device_matrix<T>& m, int64_t h, int64_t w, void* p, int64_t ld)
   m.Attach(h, w, static_cast<T*>(p), ld);
 }
 
-void copy_out(float* dst, const device_matrix<float>& src, hipStream_t st)
+template <typename W>
+void copy_out(void* dst, const device_matrix<W>& src, hipStream_t st)
 {
   if (!dst || src.IsEmpty()) return;
-  check_hip(hipMemcpy2DAsync(dst, static_cast<size_t>(src.Height()) * 4, src.LockedBuffer(),
-                             static_cast<size_t>(src.LDim()) * 4, static_cast<size_t>(src.Height()) * 4,
+  check_hip(hipMemcpy2DAsync(dst, static_cast<size_t>(src.Height()) * sizeof(W), src.LockedBuffer(),
+                             static_cast<size_t>(src.LDim()) * sizeof(W), static_cast<size_t>(src.Height()) * sizeof(W),
                              static_cast<size_t>(src.Width()), hipMemcpyDeviceToDevice, st),
             "copy_out");
 }
 
 template <typename T>
 int run_layer_norm(const int64_t* dims, int nd, int start_dim, int scale, int bias, double eps, int64_t h,
-                   int64_t w, int64_t ld, void* x, void* y, void* dy, void* dx, const float* gw,
-                   const float* bw, float* dg, float* db, float* stats_out, float* sgrad_out, void* stream)
+                   int64_t w, int64_t ld, void* x, void* y, void* dy, void* dx, const void* gw,
+                   const void* bw, void* dg, void* db, void* stats_out, void* sgrad_out, void* stream)
 {
+  using W = typename layer_norm_layer<T>::weight_t;  // float, or double for a layer of doubles
   layer_norm_layer<T> layer(eps, scale != 0, bias != 0, start_dim);
   layer.setup(std::vector<int64_t>(dims, dims + nd));
   device_matrix<T> mx, my, mdy, mdx;
@@ -48,8 +50,8 @@ int run_layer_norm(const int64_t* dims, int nd, int start_dim, int scale, int bi
   layer.io.prev_activations = &mx; layer.io.activations = &my;
   layer.io.prev_error_signals = &mdy; layer.io.error_signals = &mdx;
   layer.io.stream = static_cast<hipStream_t>(stream);
-  layer.set_weights(gw, bw);
-  layer.set_weight_gradients(dg, db);
+  layer.set_weights(static_cast<const W*>(gw), static_cast<const W*>(bw));
+  layer.set_weight_gradients(static_cast<W*>(dg), static_cast<W*>(db));
   layer.fp_compute();
   layer.bp_compute();
   copy_out(stats_out, layer.m_statistics, layer.io.stream);
@@ -63,9 +65,10 @@ int run_layer_norm(const int64_t* dims, int nd, int start_dim, int scale, int bi
 template <typename T>
 static int run_batch_norm(const int64_t* dims, int nd, double decay, double eps, int bessel, int training,
                           int64_t h, int64_t w, int64_t ld, void* x, void* y, void* dy, void* dx,
-                          const float* gw, const float* bw, float* rmean, float* rvar, float* dg, float* db,
-                          float* mean_var_out, float* mean_var_grad_out, void* stream)
+                          const void* gw, const void* bw, void* rmean, void* rvar, void* dg, void* db,
+                          void* mean_var_out, void* mean_var_grad_out, void* stream)
 {
+  using W = typename batch_normalization_layer<T>::weight_t;
   batch_normalization_layer<T> layer(decay, eps, 1, bessel != 0);
   layer.setup(std::vector<int64_t>(dims, dims + nd));
   layer.is_training = training != 0;
@@ -75,8 +78,8 @@ static int run_batch_norm(const int64_t* dims, int nd, double decay, double eps,
   layer.io.prev_activations = &mx; layer.io.activations = &my;
   layer.io.prev_error_signals = &mdy; layer.io.error_signals = &mdx;
   layer.io.stream = static_cast<hipStream_t>(stream);
-  layer.set_weights(gw, bw, rmean, rvar);
-  layer.set_weight_gradients(dg, db);
+  layer.set_weights(static_cast<const W*>(gw), static_cast<const W*>(bw), static_cast<W*>(rmean), static_cast<W*>(rvar));
+  layer.set_weight_gradients(static_cast<W*>(dg), static_cast<W*>(db));
   layer.fp_compute();
   layer.bp_compute();
   copy_out(mean_var_out, layer.m_mean_and_var, layer.io.stream);
@@ -87,12 +90,16 @@ static int run_batch_norm(const int64_t* dims, int nd, double decay, double eps,
 
 extern "C" {
 
+// half: 0 fp32, 1 fp16 storage, 2 double (weights, statistics and gradients are doubles then)
 int drv_layer_norm(int half, const int64_t* dims, int nd, int start_dim, int scale, int bias, double eps,
-                   int64_t h, int64_t w, int64_t ld, void* x, void* y, void* dy, void* dx, const float* gw,
-                   const float* bw, float* dg, float* db, float* stats_out, float* sgrad_out, void* stream,
+                   int64_t h, int64_t w, int64_t ld, void* x, void* y, void* dy, void* dx, const void* gw,
+                   const void* bw, void* dg, void* db, void* stats_out, void* sgrad_out, void* stream,
                    char* err, int errlen)
 {
   try {
+    if (half == 2)
+      return run_layer_norm<double>(dims, nd, start_dim, scale, bias, eps, h, w, ld, x, y, dy, dx, gw, bw,
+                                    dg, db, stats_out, sgrad_out, stream);
     if (half)
       return run_layer_norm<uint16_t>(dims, nd, start_dim, scale, bias, eps, h, w, ld, x, y, dy, dx, gw, bw,
                                       dg, db, stats_out, sgrad_out, stream);
@@ -105,11 +112,14 @@ int drv_layer_norm(int half, const int64_t* dims, int nd, int start_dim, int sca
 }
 
 int drv_batch_norm(int half, const int64_t* dims, int nd, double decay, double eps, int bessel, int training,
-                   int64_t h, int64_t w, int64_t ld, void* x, void* y, void* dy, void* dx, const float* gw,
-                   const float* bw, float* rmean, float* rvar, float* dg, float* db, float* mean_var_out,
-                   float* mean_var_grad_out, void* stream, char* err, int errlen)
+                   int64_t h, int64_t w, int64_t ld, void* x, void* y, void* dy, void* dx, const void* gw,
+                   const void* bw, void* rmean, void* rvar, void* dg, void* db, void* mean_var_out,
+                   void* mean_var_grad_out, void* stream, char* err, int errlen)
 {
   try {
+    if (half == 2)
+      return run_batch_norm<double>(dims, nd, decay, eps, bessel, training, h, w, ld, x, y, dy, dx, gw, bw,
+                                    rmean, rvar, dg, db, mean_var_out, mean_var_grad_out, stream);
     if (half)
       return run_batch_norm<uint16_t>(dims, nd, decay, eps, bessel, training, h, w, ld, x, y, dy, dx, gw, bw,
                                       rmean, rvar, dg, db, mean_var_out, mean_var_grad_out, stream);
@@ -141,6 +151,37 @@ int drv_softmax_family(int kind, const int64_t* dims, int nd, int64_t dim, int s
     else if (kind == 1) { log_softmax_layer<> l; bind(l); }
     else {
       channelwise_softmax_layer<> l(dim, single_dim_mode != 0);
+      l.setup(std::vector<int64_t>(dims, dims + nd));
+      bind(l);
+    }
+    return 0;
+  }
+  catch (const std::exception& e) {
+    return fail(e, err, errlen);
+  }
+}
+
+// The softmax family on matrices of doubles (kind as above).
+int drv_softmax_family_f64(int kind, const int64_t* dims, int nd, int64_t dim, int single_dim_mode, int64_t h,
+                           int64_t w, int64_t ld, double* x, double* y, double* dy, double* dx, void* stream,
+                           char* err, int errlen)
+{
+  try {
+    using M = device_matrix<double>;
+    M mx, my, mdy, mdx;
+    attach(mx, h, w, x, ld); attach(my, h, w, y, ld); attach(mdy, h, w, dy, ld); attach(mdx, h, w, dx, ld);
+    auto bind = [&](auto& layer) {
+      layer.io.prev_activations = &mx; layer.io.activations = &my;
+      layer.io.prev_error_signals = &mdy; layer.io.error_signals = &mdx;
+      layer.io.stream = static_cast<hipStream_t>(stream);
+      layer.fp_compute();
+      layer.bp_compute();
+      check_hip(hipStreamSynchronize(layer.io.stream), "sync");
+    };
+    if (kind == 0) { softmax_layer<M> l; bind(l); }
+    else if (kind == 1) { log_softmax_layer<M> l; bind(l); }
+    else {
+      channelwise_softmax_layer<M> l(dim, single_dim_mode != 0);
       l.setup(std::vector<int64_t>(dims, dims + nd));
       bind(l);
     }

@@ -15,6 +15,7 @@ import numpy as np
 
 TOL_F32 = 1e-5   # fp32 storage and arithmetic
 TOL_F16 = 2e-3   # fp16 storage, fp32 accumulation
+TOL_F64 = 1e-10  # binary64 storage and arithmetic, against the float64 evaluation of the reference code
 
 
 def rel_err(a, b):

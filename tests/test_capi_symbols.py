@@ -18,6 +18,9 @@ def test_header_declares_the_expected_surface():
     for layer in ("layer_norm", "batch_norm", "softmax", "log_softmax", "channelwise_softmax"):
         assert f"lbn_{layer}_fwd_f32" in names and f"lbn_{layer}_bwd_f32" in names
     assert "lbn_layer_norm_fwd_f16" in names and "lbn_layer_norm_bwd_f16" in names
+    # the five layers also exist for TensorDataType = double
+    for layer in ("layer_norm", "batch_norm", "softmax", "log_softmax", "channelwise_softmax"):
+        assert f"lbn_{layer}_fwd_f64" in names and f"lbn_{layer}_bwd_f64" in names
 
 
 def test_library_exports_every_declared_symbol():

@@ -328,3 +328,88 @@ def test_adapter_layers_match_oracle():
     for k in range(2):
         check("adapter two-rank running mean", rm2[k * h:(k + 1) * h].cpu().numpy(), rm0)
         check("adapter two-rank running var", rv2[k * h:(k + 1) * h].cpu().numpy(), rv0)
+
+
+@pytest.mark.gpu
+def test_adapter_layers_of_doubles_match_oracle():
+    """TensorDataType = double through the C++ adapter: layer_norm_layer<double>,
+    batch_normalization_layer<double> and the softmax family on device_matrix<double>."""
+    import torch
+    from oracle import cpu_oracle as orc
+    from tests.parity import TOL_F64, check
+    from lbann_amd.layers import DeviceMatrix
+    d = driver()
+    err = ctypes.create_string_buffer(512)
+    st = vp(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(31)
+    F64 = torch.float64
+    mk = lambda h, w, m=0.0, s=1.0: np.asfortranarray((rng.standard_normal((w, h)) * s + m).T)
+    dev = lambda a: torch.from_numpy(np.asarray(a, np.float64)).cuda()
+    p = lambda t: vp(t.data_ptr())
+    new = lambda h, w: DeviceMatrix(h, w, dtype=F64)
+
+    dims, w = (6, 512), 20
+    h = 6 * 512
+    g, b = 1 + 0.2 * rng.standard_normal(512), 0.2 * rng.standard_normal(512)
+    x, dy = mk(h, w, 0.3, 1.5), mk(h, w)
+    mx, mdy, my, mdx = DeviceMatrix.from_numpy(x), DeviceMatrix.from_numpy(dy), new(h, w), new(h, w)
+    gw, bw = dev(g), dev(b)
+    dg, db = torch.empty(512, dtype=F64).cuda(), torch.empty(512, dtype=F64).cuda()
+    stats, sgrad = new(12, w), new(12, w)
+    da, nd = _dims(dims)
+    rc = d.drv_layer_norm(cint(2), da, cint(nd), cint(-1), cint(1), cint(1), dbl(1e-5), i64(h), i64(w), i64(h),
+                          mx.Buffer(), my.Buffer(), mdy.Buffer(), mdx.Buffer(), p(gw), p(bw), p(dg), p(db),
+                          stats.Buffer(), sgrad.Buffer(), st, err, cint(512))
+    assert rc == 0, err.value
+    y_ref, st_ref = orc.layer_norm_fwd(x, 6, 512, 512, 1e-5, g, b)
+    dx_ref, sg_ref, dg_ref, db_ref = orc.layer_norm_bwd(x, dy, st_ref, 6, 512, 512, 1e-5, g, True, True)
+    for name, got, ref in (("y", my.to_numpy(), y_ref), ("dx", mdx.to_numpy(), dx_ref), ("stats", stats.to_numpy(), st_ref),
+                           ("sgrad", sgrad.to_numpy(), sg_ref), ("dscale", dg.cpu().numpy(), dg_ref),
+                           ("dbias", db.cpu().numpy(), db_ref)):
+        assert got.dtype == np.float64
+        check(f"adapter f64 ln {name}", got, ref, tol=TOL_F64)
+
+    dims, w = (8, 12, 12), 10
+    h = 8 * 144
+    g, b = rng.uniform(0.5, 1.5, 8), 0.1 * rng.standard_normal(8)
+    x, dy = mk(h, w, 2.0, 3.0), mk(h, w)
+    mx, mdy, my, mdx = DeviceMatrix.from_numpy(x), DeviceMatrix.from_numpy(dy), new(h, w), new(h, w)
+    gw, bw, rm, rv = dev(g), dev(b), torch.zeros(8, dtype=F64).cuda(), torch.ones(8, dtype=F64).cuda()
+    dg, db = torch.empty(8, dtype=F64).cuda(), torch.empty(8, dtype=F64).cuda()
+    mv, mvg = new(8, 2), new(8, 2)
+    da, nd = _dims(dims)
+    rc = d.drv_batch_norm(cint(2), da, cint(nd), dbl(0.9), dbl(1e-5), cint(1), cint(1), i64(h), i64(w),
+                          i64(h), mx.Buffer(), my.Buffer(), mdy.Buffer(), mdx.Buffer(), p(gw), p(bw), p(rm),
+                          p(rv), p(dg), p(db), mv.Buffer(), mvg.Buffer(), st, err, cint(512))
+    assert rc == 0, err.value
+    rm0, rv0 = np.zeros(8), np.ones(8)
+    y_ref, m_ref, v_ref = orc.batch_norm_fwd(x, 8, 144, 1e-5, 0.9, g, b, rm0, rv0)
+    dx_ref, dg_ref, db_ref, dm_ref, dv_ref = orc.batch_norm_bwd(x, dy, 8, 144, 1e-5, m_ref, v_ref, g)
+    for name, got, ref in (("y", my.to_numpy(), y_ref), ("dx", mdx.to_numpy(), dx_ref),
+                           ("mean/var", mv.to_numpy(), np.stack([m_ref, v_ref], axis=1)),
+                           ("dmean/dvar", mvg.to_numpy(), np.stack([dm_ref, dv_ref], axis=1)),
+                           ("dscale", dg.cpu().numpy(), dg_ref), ("dbias", db.cpu().numpy(), db_ref),
+                           ("running mean", rm.cpu().numpy(), rm0), ("running var", rv.cpu().numpy(), rv0)):
+        check(f"adapter f64 bn {name}", got, ref, tol=TOL_F64)
+
+    for kind, h, w, dims, dim, single in ((0, 4096, 9, (4096,), 0, 0), (1, 1000, 7, (1000,), 0, 0),
+                                          (0, 70000, 2, (70000,), 0, 0), (2, 5 * 2 * 8, 11, (5, 2, 8), -1, 1),
+                                          (2, 16 * 256, 6, (16, 256), 0, 0)):
+        x, dy = mk(h, w, 0.0, 2.0), mk(h, w)
+        mx, mdy, my, mdx = DeviceMatrix.from_numpy(x), DeviceMatrix.from_numpy(dy), new(h, w), new(h, w)
+        da, nd = _dims(dims)
+        rc = d.drv_softmax_family_f64(cint(kind), da, cint(nd), i64(dim), cint(single), i64(h), i64(w), i64(h),
+                                      mx.Buffer(), my.Buffer(), mdy.Buffer(), mdx.Buffer(), st, err, cint(512))
+        assert rc == 0, err.value
+        if kind == 0:
+            fwd, bwd = orc.softmax_fwd, orc.softmax_bwd
+        elif kind == 1:
+            fwd, bwd = orc.log_softmax_fwd, orc.log_softmax_bwd
+        else:
+            cs = dims[-1] if single else h // dims[0]
+            C = h // cs
+            fwd = lambda a: orc.channelwise_softmax_fwd(a, C, cs, cs)
+            bwd = lambda yy, gg: orc.channelwise_softmax_bwd(yy, gg, C, cs, cs)
+        y = my.to_numpy()
+        check(f"adapter f64 softmax kind {kind} y", y, fwd(x), tol=TOL_F64)
+        check(f"adapter f64 softmax kind {kind} dx", mdx.to_numpy(), bwd(y, dy), tol=TOL_F64)
