@@ -162,6 +162,11 @@ def main():
         return L.DeviceMatrix.from_numpy(a, dtype=torch.float16 if half else None,
                                          ldim=a.shape[0] + ld_pad if ld_pad else None)
 
+    def as_f64(data):
+        """The workload with every tensor and weight vector in binary64 (TensorDataType = double)."""
+        return {k: (np.asfortranarray(v.astype(np.float64)) if isinstance(v, np.ndarray) and v.dtype.kind == "f" else v)
+                for k, v in data.items()}
+
     # ---- workload table: name -> builder returning (fwd, bwd, elements, elem_size, samples, cpu_fn)
     def build_softmax(kind, data, half=False):
         if half:  # fp16 storage: both sides see the rounded values
@@ -179,7 +184,7 @@ def main():
             t0 = time.perf_counter(); y = f(data["x"]); t1 = time.perf_counter()
             b(y, data["dy"]); t2 = time.perf_counter()
             return t1 - t0, t2 - t1
-        return layer, data["x"].size, 2 if half else 4, data["x"].shape[1], cpu
+        return layer, data["x"].size, 8 if data["x"].dtype == np.float64 else (2 if half else 4), data["x"].shape[1], cpu
 
     def build_cws(data):
         x, dy = upload(data["x"]), upload(data["dy"])
@@ -197,19 +202,22 @@ def main():
 
     def build_ln(data, half):
         x, dy = upload(data["x"], half), upload(data["dy"], half)
-        layer = L.layer_norm_layer(data["dims"], data["eps"], True, True, 0, data["scale"], data["bias"])
+        dbl = data["x"].dtype == np.float64
+        layer = L.layer_norm_layer(data["dims"], data["eps"], True, True, 0, data["scale"], data["bias"],
+                                   datatype=torch.float64 if dbl else torch.float32)
         layer.bind_forward(x)
         layer.bind_backward(dy)
         n = data["dims"][0]
 
         def cpu():
             from oracle import cpu_oracle as orc
-            xs = np.asfortranarray(data["x"].astype(np.float32))
-            gs = np.asfortranarray(data["dy"].astype(np.float32))
+            cdt = np.float64 if dbl else np.float32
+            xs = np.asfortranarray(data["x"].astype(cdt))
+            gs = np.asfortranarray(data["dy"].astype(cdt))
             t0 = time.perf_counter(); _, st = orc.layer_norm_fwd(xs, 1, n, n, data["eps"], data["scale"], data["bias"]); t1 = time.perf_counter()
             orc.layer_norm_bwd(xs, gs, st, 1, n, n, data["eps"], data["scale"], True, True); t2 = time.perf_counter()
             return t1 - t0, t2 - t1
-        return layer, data["x"].size, 2 if half else 4, data["x"].shape[1], cpu
+        return layer, data["x"].size, 8 if dbl else (2 if half else 4), data["x"].shape[1], cpu
 
     def volume_in():
         # 16 channels of 160^3 voxels, 2 samples: 32 rows of 4.1 M entries (501 MiB per tensor)
@@ -231,7 +239,9 @@ def main():
             data = dict(data, x=np.asfortranarray(data["x"].astype(np.float16).astype(np.float32)),
                         dy=np.asfortranarray(data["dy"].astype(np.float16).astype(np.float32)))
         x, dy = upload(data["x"], half), upload(data["dy"], half)
-        layer = L.batch_normalization_layer(data["dims"], data["decay"], data["eps"], True, data["scale"], data["bias"])
+        dbl = data["x"].dtype == np.float64
+        layer = L.batch_normalization_layer(data["dims"], data["decay"], data["eps"], True, data["scale"], data["bias"],
+                                            datatype=torch.float64 if dbl else torch.float32)
         layer.bind_forward(x)
         layer.bind_backward(dy)
         C = data["dims"][0]
@@ -239,11 +249,11 @@ def main():
 
         def cpu():
             from oracle import cpu_oracle as orc
-            rm, rv = np.zeros(C, np.float32), np.ones(C, np.float32)
+            rm, rv = np.zeros(C, data["x"].dtype), np.ones(C, data["x"].dtype)
             t0 = time.perf_counter(); _, m, v = orc.batch_norm_fwd(data["x"], C, cs, data["eps"], data["decay"], data["scale"], data["bias"], rm, rv); t1 = time.perf_counter()
             orc.batch_norm_bwd(data["x"], data["dy"], C, cs, data["eps"], m, v, data["scale"]); t2 = time.perf_counter()
             return t1 - t0, t2 - t1
-        return layer, data["x"].size, 2 if half else 4, data["x"].shape[1], cpu
+        return layer, data["x"].size, 8 if dbl else (2 if half else 4), data["x"].shape[1], cpu
 
     def build_in(data):
         x, dy = upload(data["x"]), upload(data["dy"])
@@ -419,6 +429,13 @@ def main():
                               lambda: build_softmax("softmax", W.cfg2_softmax(), True)),
         "extra_softmax_vocab_50257": ("Softmax fwd+bwd fp32 50257x1024, rows 4-byte aligned (informational)",
                                       lambda: build_softmax("softmax", W.cfg5b_wide_softmax(h=50257, w=1024))),
+        # not baseline configurations: the layers for TensorDataType = double (8 bytes per entry)
+        "extra_softmax_f64": ("Softmax fwd+bwd fp64 32768x512 (informational)",
+                              lambda: build_softmax("softmax", as_f64(W.cfg2_softmax()))),
+        "extra_layer_norm_f64": ("LayerNorm fwd+bwd fp64 4096x8192 (informational)",
+                                 lambda: build_ln(as_f64(W.cfg4_layer_norm_f16()), False)),
+        "extra_batch_norm_f64": ("BatchNorm train fwd+bwd fp64 NCHW 64x256x28x28 (informational)",
+                                 lambda: build_bn(as_f64(W.cfg3_batch_norm(H=28, W=28)))),
         # not a baseline configuration: where weight gradients go next (a 4096 x 4096 weight matrix)
         "extra_gradient_sink": ("Gradient buffer overwrite+accumulate fp32 4096x4096 (informational)",
                                 lambda: build_sink(4096, 4096)),

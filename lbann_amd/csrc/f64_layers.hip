@@ -33,28 +33,56 @@ constexpr int kBnMaxSplit = 64;
 enum { kSoftmax = 0, kLogSoftmax = 1, kChannelwise = 2 };
 
 // ------------------------------------------------------------------ reductions
-__device__ __forceinline__ double wave_sum_d(double v)
+// Wave reductions of doubles on the DPP data path (the two halves of a double move with the same
+// control; see the fp32 versions in device_utils.hpp): the wave's result is valid in lane 63.
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ double dpp_move_d(double v, double old = 0.0)
 {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+  const unsigned long long o = __builtin_bit_cast(unsigned long long, old);
+  const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_update_dpp(static_cast<int>(o), static_cast<int>(b), CTRL,
+                                                                        ROW_MASK, 0xF, false));
+  const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_update_dpp(static_cast<int>(o >> 32), static_cast<int>(b >> 32),
+                                                                        CTRL, ROW_MASK, 0xF, false));
+  return __builtin_bit_cast(double, (static_cast<unsigned long long>(hi) << 32) | lo);
+}
+__device__ __forceinline__ double read_lane_d(double v, int lane)
+{
+  const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+  const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b), lane));
+  const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b >> 32), lane));
+  return __builtin_bit_cast(double, (static_cast<unsigned long long>(hi) << 32) | lo);
+}
+__device__ __forceinline__ double wave_sum_in_last_d(double v)
+{
+  v += dpp_move_d<kDppQuadSwap1>(v);
+  v += dpp_move_d<kDppQuadSwap2>(v);
+  v += dpp_move_d<kDppHalfMirror>(v);
+  v += dpp_move_d<kDppRowMirror>(v);
+  v += dpp_move_d<kDppRowBcast15, 0xA>(v);  // rows 1 and 3 add rows 0 and 2; the others add 0
+  v += dpp_move_d<kDppRowBcast31, 0xC>(v);  // row 3 adds rows 0 + 1
   return v;
 }
-__device__ __forceinline__ double wave_max_d(double v)
+__device__ __forceinline__ double wave_max_in_last_d(double v)
 {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmax(v, __shfl_xor(v, o));
+  v = fmax(v, dpp_move_d<kDppQuadSwap1>(v));
+  v = fmax(v, dpp_move_d<kDppQuadSwap2>(v));
+  v = fmax(v, dpp_move_d<kDppHalfMirror>(v));
+  v = fmax(v, dpp_move_d<kDppRowMirror>(v));
+  v = fmax(v, dpp_move_d<kDppRowBcast15, 0xA>(v, v));  // disabled rows keep their own value
+  v = fmax(v, dpp_move_d<kDppRowBcast31, 0xC>(v, v));
   return v;
 }
 
-// Sum / maximum over a team of NW waves.  `slot` points to NW doubles of LDS private to the team
-// and to this reduction; all threads of the workgroup call when NW > 1 (a team is then the whole
-// workgroup).  Fixed order.
+// Sum / maximum over a team of NW waves; every thread gets the result.  `slot` points to NW
+// doubles of LDS private to the team and to this reduction; all threads of the workgroup call
+// when NW > 1 (a team is then the whole workgroup).  Fixed order.
 template <int NW>
 __device__ __forceinline__ double team_sum_d(double v, double* slot)
 {
-  v = wave_sum_d(v);
-  if constexpr (NW == 1) return v;
-  if ((threadIdx.x & (kWave - 1)) == 0) slot[(threadIdx.x / kWave) % NW] = v;
+  v = wave_sum_in_last_d(v);
+  if constexpr (NW == 1) return read_lane_d(v, kWave - 1);
+  if ((threadIdx.x & (kWave - 1)) == kWave - 1) slot[(threadIdx.x / kWave) % NW] = v;
   __syncthreads();
   double r = slot[0];
 #pragma unroll
@@ -64,9 +92,9 @@ __device__ __forceinline__ double team_sum_d(double v, double* slot)
 template <int NW>
 __device__ __forceinline__ double team_max_d(double v, double* slot)
 {
-  v = wave_max_d(v);
-  if constexpr (NW == 1) return v;
-  if ((threadIdx.x & (kWave - 1)) == 0) slot[(threadIdx.x / kWave) % NW] = v;
+  v = wave_max_in_last_d(v);
+  if constexpr (NW == 1) return read_lane_d(v, kWave - 1);
+  if ((threadIdx.x & (kWave - 1)) == kWave - 1) slot[(threadIdx.x / kWave) % NW] = v;
   __syncthreads();
   double r = slot[0];
 #pragma unroll
@@ -114,17 +142,19 @@ struct Team {
 struct RowShape {
   int tpr, v;
 };
+// The narrowest team whose threads own at most two accesses each (a thread's entries are doubles:
+// registers run out quickly, and several small workgroups per compute unit overlap better than one
+// large one); rows beyond 2048 accesses take 1024 threads with up to 16 accesses each.
 inline RowShape pick_shape(int64_t units, int64_t rows)
 {
   const int tprs[3] = {64, 256, 1024};
   for (int i = 0; i < 3; ++i) {
     const int64_t per = ceil_div(units, tprs[i]);
-    const int max_v = i == 2 ? kMaxV : 8;
-    if (per > max_v) continue;
+    if (per > (i == 2 ? kMaxV : 2)) continue;
     int v = 1;
     while (v < per) v *= 2;
     // few rows: a wider team keeps more of the device busy
-    if (i < 2 && v > 1 && rows * (tprs[i] / kWave) < 2048 && ceil_div(units, tprs[i + 1]) >= 1) continue;
+    if (i < 2 && v > 1 && rows * (tprs[i] / kWave) < 2048) continue;
     return {tprs[i], v};
   }
   return {0, 0};
@@ -161,51 +191,61 @@ struct RowArgs {
   const int64_t first = static_cast<int64_t>(blockIdx.x) * TM::kTeams + team;        \
   const int64_t iters = (a.rows + teams_total - 1) / teams_total;                    \
   bool ok[V];                                                                        \
-  _Pragma("unroll") for (int i = 0; i < V; ++i) ok[i] = t + i * TPR < a.units;
+  int off[V]; /* entry offset of access i; accesses past the row's end re-read access 0 */ \
+  _Pragma("unroll") for (int i = 0; i < V; ++i) {                                    \
+    ok[i] = t + i * TPR < a.units;                                                   \
+    off[i] = ok[i] ? W * (t + i * TPR) : 0;                                          \
+  }                                                                                  \
+  /* row of iteration `it` (clamped to the last row: its loads are harmless, its stores skipped) */ \
+  auto row_of = [&](int64_t it) {                                                    \
+    const int64_t r = first + it * teams_total;                                      \
+    return r < a.rows ? r : a.rows - 1;                                              \
+  };
 
 // ------------------------------------------------------------------ softmax family
+// All of a row's loads are issued together, unconditionally; the row that a team takes next is
+// requested while the current one is stored: every access is reloaded right behind its store, into
+// the registers the store has just freed, so loads and stores of a compute unit overlap even
+// when a row fills its registers (32768 doubles in a 1024-thread workgroup).
 template <int KIND, int TPR, int V, int W>
 __global__ void __launch_bounds__(Team<TPR>::kThreads)
 sm_fwd_rows_f64(RowArgs a)
 {
   LBN_F64_ROW_PROLOGUE
+  double v[V][W];
+  {
+    const double* xr = a.a + a.map.offset(row_of(0), a.lda);
+#pragma unroll
+    for (int i = 0; i < V; ++i) load_w<W>(xr + off[i], v[i]);
+  }
   for (int64_t it = 0; it < iters; ++it) {
     const int64_t row = first + it * teams_total;
     const bool live = row < a.rows;  // teams of a workgroup run the same number of iterations
-    const int64_t r = live ? row : a.rows - 1;
-    const double* xr = a.a + a.map.offset(r, a.lda);
-    double v[V][W];
     double m = -DBL_MAX;
 #pragma unroll
-    for (int i = 0; i < V; ++i) {
-      if (ok[i]) {
-        load_w<W>(xr + W * static_cast<int64_t>(t + i * TPR), v[i]);
+    for (int i = 0; i < V; ++i)
 #pragma unroll
-        for (int j = 0; j < W; ++j) m = fmax(m, v[i][j]);
-      }
-    }
+      for (int j = 0; j < W; ++j) m = fmax(m, ok[i] ? v[i][j] : -DBL_MAX);
     m = team_max_d<NW>(m, red[2 * (it & 1)][team]);
     double s = 0.0;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      if (ok[i]) {
 #pragma unroll
-        for (int j = 0; j < W; ++j) {
-          const double d = v[i][j] - m;
-          const double e = exp(d);
-          s += e;
-          v[i][j] = KIND == kLogSoftmax ? d : e;
-        }
+      for (int j = 0; j < W; ++j) {
+        const double d = v[i][j] - m;
+        const double e = exp(d);
+        s += ok[i] ? e : 0.0;
+        v[i][j] = KIND == kLogSoftmax ? d : e;
       }
     }
     s = team_sum_d<NW>(s, red[2 * (it & 1) + 1][team]);
-    if (!live) continue;
-    double* yr = a.out + a.map.offset(row, a.ldo);
+    double* yr = a.out + a.map.offset(live ? row : a.rows - 1, a.ldo);
+    const double* xn = a.a + a.map.offset(row_of(it + 1), a.lda);
+    const bool more = it + 1 < iters;
     const double scale = 1.0 / s;
     const double lse = KIND == kLogSoftmax ? log(s) : 0.0;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      if (!ok[i]) continue;
 #pragma unroll
       for (int j = 0; j < W; ++j) {
         if (KIND == kSoftmax) {
@@ -219,7 +259,8 @@ sm_fwd_rows_f64(RowArgs a)
           v[i][j] /= s;  // channelwise_softmax.cpp:88-97: a division, denormals kept
         }
       }
-      store_w<W>(yr + W * static_cast<int64_t>(t + i * TPR), v[i]);
+      if (live && ok[i]) store_w<W>(yr + off[i], v[i]);
+      if (more) load_w<W>(xn + off[i], v[i]);
     }
   }
 }
@@ -229,33 +270,41 @@ __global__ void __launch_bounds__(Team<TPR>::kThreads)
 sm_bwd_rows_f64(RowArgs a)
 {
   LBN_F64_ROW_PROLOGUE
+  double y[V][W], g[V][W];
+  {
+    const int64_t r = row_of(0);
+    const double* yr = a.a + a.map.offset(r, a.lda);
+    const double* gr = a.g + a.map.offset(r, a.ldg);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      load_w<W>(yr + off[i], y[i]);
+      load_w<W>(gr + off[i], g[i]);
+    }
+  }
   for (int64_t it = 0; it < iters; ++it) {
     const int64_t row = first + it * teams_total;
     const bool live = row < a.rows;
-    const int64_t r = live ? row : a.rows - 1;
-    const double* yr = a.a + a.map.offset(r, a.lda);
-    const double* gr = a.g + a.map.offset(r, a.ldg);
-    double y[V][W], g[V][W];
     double s = 0.0;
 #pragma unroll
-    for (int i = 0; i < V; ++i) {
-      if (ok[i]) {
-        load_w<W>(yr + W * static_cast<int64_t>(t + i * TPR), y[i]);
-        load_w<W>(gr + W * static_cast<int64_t>(t + i * TPR), g[i]);
+    for (int i = 0; i < V; ++i)
 #pragma unroll
-        for (int j = 0; j < W; ++j) s += KIND == kLogSoftmax ? g[i][j] : y[i][j] * g[i][j];
-      }
-    }
+      for (int j = 0; j < W; ++j) s += ok[i] ? (KIND == kLogSoftmax ? g[i][j] : y[i][j] * g[i][j]) : 0.0;
     s = team_sum_d<NW>(s, red[it & 3][team]);
-    if (!live) continue;
-    double* dr = a.out + a.map.offset(row, a.ldo);
+    double* dr = a.out + a.map.offset(live ? row : a.rows - 1, a.ldo);
+    const int64_t rn = row_of(it + 1);
+    const double* yn = a.a + a.map.offset(rn, a.lda);
+    const double* gn = a.g + a.map.offset(rn, a.ldg);
+    const bool more = it + 1 < iters;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      if (!ok[i]) continue;
 #pragma unroll
       for (int j = 0; j < W; ++j)
         g[i][j] = KIND == kLogSoftmax ? g[i][j] - exp(y[i][j]) * s : y[i][j] * (g[i][j] - s);
-      store_w<W>(dr + W * static_cast<int64_t>(t + i * TPR), g[i]);
+      if (live && ok[i]) store_w<W>(dr + off[i], g[i]);
+      if (more) {
+        load_w<W>(yn + off[i], y[i]);
+        load_w<W>(gn + off[i], g[i]);
+      }
     }
   }
 }
@@ -267,34 +316,44 @@ ln_fwd_rows_f64(RowArgs a)
 {
   LBN_F64_ROW_PROLOGUE
   const double inv_n = 1.0 / static_cast<double>(a.n);
+  // threads that own at most 8 entries keep their scale and bias in registers across rows
+  constexpr bool kWeightsInRegs = V * W <= 8;
+  double gam[kWeightsInRegs ? V : 1][W], bet[kWeightsInRegs ? V : 1][W];
+  if constexpr (kWeightsInRegs) {
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+#pragma unroll
+      for (int j = 0; j < W; ++j) {
+        gam[i][j] = (a.gamma && ok[i]) ? a.gamma[off[i] + j] : 1.0;
+        bet[i][j] = (a.beta && ok[i]) ? a.beta[off[i] + j] : 0.0;
+      }
+  }
+  double v[V][W];
+  {
+    const double* xr = a.a + a.map.offset(row_of(0), a.lda);
+#pragma unroll
+    for (int i = 0; i < V; ++i) load_w<W>(xr + off[i], v[i]);
+  }
   for (int64_t it = 0; it < iters; ++it) {
     const int64_t row = first + it * teams_total;
     const bool live = row < a.rows;
-    const int64_t r = live ? row : a.rows - 1;
-    const double* xr = a.a + a.map.offset(r, a.lda);
-    double v[V][W];
     double s = 0.0, q = 0.0;
 #pragma unroll
-    for (int i = 0; i < V; ++i) {
+    for (int i = 0; i < V; ++i)
 #pragma unroll
-      for (int j = 0; j < W; ++j) v[i][j] = 0.0;
-      if (ok[i]) {
-        load_w<W>(xr + W * static_cast<int64_t>(t + i * TPR), v[i]);
-#pragma unroll
-        for (int j = 0; j < W; ++j) {
-          s += v[i][j];
-          q += v[i][j] * v[i][j];
-        }
+      for (int j = 0; j < W; ++j) {
+        if (!ok[i]) v[i][j] = 0.0;
+        s += v[i][j];
+        q += v[i][j] * v[i][j];
       }
-    }
     s = team_sum_d<NW>(s, red[2 * (it & 1)][team]);
-    const double mean = s * inv_n;
+    double mean = s * inv_n;
     double var;
     if (a.sumsq) {  // the reference's expression (layer_norm.cpp:99-112)
       q = team_sum_d<NW>(q, red[2 * (it & 1) + 1][team]);
       const double nn = static_cast<double>(a.n);
-      const double m2 = s / nn;
-      var = fmax(q / nn - m2 * m2, 0.0);
+      mean = s / nn;
+      var = fmax(q / nn - mean * mean, 0.0);
     }
     else {
       double c = 0.0;
@@ -307,28 +366,32 @@ ln_fwd_rows_f64(RowArgs a)
         }
       var = team_sum_d<NW>(c, red[2 * (it & 1) + 1][team]) * inv_n;
     }
-    if (!live) continue;
     int64_t col, g;
-    a.map.split(row, col, g);
-    if (t == 0) {
-      a.stats[g + col * a.ld_stats] = a.sumsq ? s / static_cast<double>(a.n) : mean;
+    a.map.split(live ? row : a.rows - 1, col, g);
+    if (live && t == 0) {
+      a.stats[g + col * a.ld_stats] = mean;
       a.stats[a.map.groups + g + col * a.ld_stats] = var;
     }
-    const double mu = a.sumsq ? s / static_cast<double>(a.n) : mean;
     const double inv_stdev = 1.0 / sqrt(var + a.eps);
     double* yr = a.out + g * a.map.stride + col * a.ldo;
+    const double* xn = a.a + a.map.offset(row_of(it + 1), a.lda);
+    const bool more = it + 1 < iters;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      if (!ok[i]) continue;
-      const int64_t e0 = W * static_cast<int64_t>(t + i * TPR);
 #pragma unroll
       for (int j = 0; j < W; ++j) {
-        double y = (v[i][j] - mu) * inv_stdev;
-        if (a.gamma) y *= a.gamma[e0 + j];
-        if (a.beta) y += a.beta[e0 + j];
+        double y = (v[i][j] - mean) * inv_stdev;
+        if constexpr (kWeightsInRegs) {
+          y = y * gam[i][j] + bet[i][j];
+        }
+        else {
+          if (a.gamma) y *= a.gamma[off[i] + j];
+          if (a.beta) y += a.beta[off[i] + j];
+        }
         v[i][j] = y;
       }
-      store_w<W>(yr + e0, v[i]);
+      if (live && ok[i]) store_w<W>(yr + off[i], v[i]);
+      if (more) load_w<W>(xn + off[i], v[i]);
     }
   }
 }
@@ -347,48 +410,54 @@ ln_bwd_rows_f64(RowArgs a)
   for (int i = 0; i < V; ++i)
 #pragma unroll
     for (int j = 0; j < W; ++j) {
-      gam[i][j] = (a.gamma && ok[i]) ? a.gamma[W * static_cast<int64_t>(t + i * TPR) + j] : 1.0;
+      gam[i][j] = (a.gamma && ok[i]) ? a.gamma[off[i] + j] : 1.0;
       if (WGRAD) dg[i][j] = db[i][j] = 0.0;
     }
+  double d[V][W], gs[V][W];
+  double mean, var;
+  auto issue = [&](int64_t it) {
+    int64_t col, g;
+    a.map.split(row_of(it), col, g);
+    const double* xr = a.a + g * a.map.stride + col * a.lda;
+    const double* gr = a.g + g * a.map.stride + col * a.ldg;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      load_w<W>(xr + off[i], d[i]);
+      load_w<W>(gr + off[i], gs[i]);
+    }
+    mean = a.stats[g + col * a.ld_stats];
+    var = a.stats[a.map.groups + g + col * a.ld_stats];
+  };
+  issue(0);
   for (int64_t it = 0; it < iters; ++it) {
     const int64_t row = first + it * teams_total;
     const bool live = row < a.rows;
-    const int64_t r = live ? row : a.rows - 1;
-    int64_t col, g;
-    a.map.split(r, col, g);
-    const double* xr = a.a + g * a.map.stride + col * a.lda;
-    const double* gr = a.g + g * a.map.stride + col * a.ldg;
-    const double mean = a.stats[g + col * a.ld_stats];
-    const double var = a.stats[a.map.groups + g + col * a.ld_stats];
+    const double mu = mean;
     const double inv_stdev = 1.0 / sqrt(var + a.eps);
-    double d[V][W], gs[V][W];
     double A = 0.0, B = 0.0;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
 #pragma unroll
-      for (int j = 0; j < W; ++j) d[i][j] = gs[i][j] = 0.0;
-      if (ok[i]) {
-        load_w<W>(xr + W * static_cast<int64_t>(t + i * TPR), d[i]);
-        load_w<W>(gr + W * static_cast<int64_t>(t + i * TPR), gs[i]);
-#pragma unroll
-        for (int j = 0; j < W; ++j) {
-          d[i][j] -= mean;
-          if (WGRAD && live) {
-            db[i][j] += gs[i][j];
-            dg[i][j] += gs[i][j] * d[i][j] * inv_stdev;
-          }
-          gs[i][j] *= gam[i][j];
-          A += gs[i][j];
-          B += gs[i][j] * d[i][j];
+      for (int j = 0; j < W; ++j) {
+        const bool use = ok[i] && live;
+        const double gv = use ? gs[i][j] : 0.0;
+        d[i][j] = use ? d[i][j] - mu : 0.0;
+        if (WGRAD) {
+          db[i][j] += gv;
+          dg[i][j] += gv * d[i][j] * inv_stdev;
         }
+        gs[i][j] = gv * gam[i][j];
+        A += gs[i][j];
+        B += gs[i][j] * d[i][j];
       }
     }
     A = team_sum_d<NW>(A, red[2 * (it & 1)][team]);
     B = team_sum_d<NW>(B, red[2 * (it & 1) + 1][team]);
-    if (!live) continue;
+    int64_t col, g;
+    a.map.split(live ? row : a.rows - 1, col, g);
     const double dmean = -A * inv_stdev;
     const double dvar = -B * inv_stdev * inv_stdev * inv_stdev / 2;
-    if (t == 0) {
+    if (live && t == 0) {
       a.sgrad[g + col * a.ld_sgrad] = dmean;
       a.sgrad[a.map.groups + g + col * a.ld_sgrad] = dvar;
     }
@@ -396,11 +465,11 @@ ln_bwd_rows_f64(RowArgs a)
     const double c0 = dmean / nn, c1 = dvar * 2 / nn;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      if (!ok[i]) continue;
 #pragma unroll
       for (int j = 0; j < W; ++j) gs[i][j] = gs[i][j] * inv_stdev + c0 + c1 * d[i][j];
-      store_w<W>(dr + W * static_cast<int64_t>(t + i * TPR), gs[i]);
+      if (live && ok[i]) store_w<W>(dr + off[i], gs[i]);
     }
+    if (it + 1 < iters) issue(it + 1);
   }
   if (WGRAD) {
     double* out = a.part + first * 2 * a.n;
@@ -409,24 +478,43 @@ ln_bwd_rows_f64(RowArgs a)
       if (!ok[i]) continue;
 #pragma unroll
       for (int j = 0; j < W; ++j) {
-        const int64_t e = W * static_cast<int64_t>(t + i * TPR) + j;
-        out[e] = dg[i][j];
-        out[a.n + e] = db[i][j];
+        out[off[i] + j] = dg[i][j];
+        out[a.n + off[i] + j] = db[i][j];
       }
     }
   }
 }
 
-// Adds P partial rows of 2n entries; thread per entry, fixed order.
+// Adds P partial rows of 2n entries in a fixed order.  A workgroup takes 16 consecutive entries
+// (128 contiguous bytes of every partial row); its 256 threads are 16 row groups x 16 entries, a
+// thread adds rows g, g + 16, ... eight loads at a time, the groups are added through LDS.
 __global__ void __launch_bounds__(256)
 ln_wgrad_reduce_f64(const double* __restrict__ part, int64_t P, int64_t n, double* dscale, double* dbias)
 {
-  const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (e >= 2 * n) return;
+  __shared__ double sm[16][17];
+  const int e_in = threadIdx.x & 15, g = threadIdx.x >> 4;
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * 16 + e_in;
   double acc = 0.0;
-  for (int64_t p = 0; p < P; ++p) acc += part[p * 2 * n + e];
-  double* out = e < n ? dscale : dbias;
-  if (out) out[e < n ? e : e - n] = acc;
+  if (e < 2 * n) {
+    for (int64_t p0 = g; p0 < P; p0 += 16 * 8) {
+      double w[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int64_t p = p0 + 16 * j;
+        w[j] = p < P ? part[p * 2 * n + e] : 0.0;
+      }
+      acc += ((w[0] + w[1]) + (w[2] + w[3])) + ((w[4] + w[5]) + (w[6] + w[7]));
+    }
+  }
+  sm[g][e_in] = acc;
+  __syncthreads();
+  if (threadIdx.x < 16 && e < 2 * n) {
+    double r = 0.0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) r += sm[k][threadIdx.x];
+    double* out = e < n ? dscale : dbias;
+    if (out) out[e < n ? e : e - n] = r;
+  }
 }
 
 // ------------------------------------------------------------------ long rows
@@ -450,21 +538,28 @@ rows_stream_f64(RowArgs a)
   const int64_t n = a.n;
   if (OP == 0) {
     const double* xr = a.a + off_a;
-    double m = -DBL_MAX, s = 0.0;  // online: s = sum exp(x - m) over the thread's entries
-    for (int64_t k = t; k < n; k += kStreamThreads) {
-      const double x = xr[k];
-      if (x > m) {
-        s = s * exp(m - x) + 1.0;
-        m = x;
+    // online, four entries at a time (their loads go out together, no data-dependent branch):
+    // s = sum exp(x - m) over the thread's entries so far
+    double m = -DBL_MAX, s = 0.0;
+    for (int64_t k = t; k < n; k += 4 * kStreamThreads) {
+      double x[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t kk = k + u * kStreamThreads;
+        x[u] = xr[kk < n ? kk : k];
       }
-      else {
-        s += exp(x - m);
-      }
+      const double mn = fmax(fmax(m, fmax(x[0], x[1])), fmax(x[2], x[3]));
+      double add = 0.0;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) add += k + u * kStreamThreads < n ? exp(x[u] - mn) : 0.0;
+      s = s * exp(m - mn) + add;
+      m = mn;
     }
     const double gm = team_max_d<NW>(m, red[0]);
     s = team_sum_d<NW>(s * exp(m - gm), red[1]);
     const double scale = 1.0 / s, lse = log(s);
     double* yr = a.out + off_o;
+#pragma unroll 4
     for (int64_t k = t; k < n; k += kStreamThreads) {
       const double d = xr[k] - gm;
       double y;
@@ -481,9 +576,11 @@ rows_stream_f64(RowArgs a)
     const double* yr = a.a + off_a;
     const double* gr = a.g + off_g;
     double s = 0.0;
+#pragma unroll 4
     for (int64_t k = t; k < n; k += kStreamThreads) s += KIND == kLogSoftmax ? gr[k] : yr[k] * gr[k];
     s = team_sum_d<NW>(s, red[0]);
     double* dr = a.out + off_o;
+#pragma unroll 4
     for (int64_t k = t; k < n; k += kStreamThreads) {
       const double y = yr[k], gg = gr[k];
       dr[k] = KIND == kLogSoftmax ? gg - exp(y) * s : y * (gg - s);
@@ -493,6 +590,7 @@ rows_stream_f64(RowArgs a)
     const double* xr = a.a + off_a;
     const double K = a.sumsq ? 0.0 : xr[0];  // sums about the row's first entry: no cancellation
     double s = 0.0, q = 0.0;
+#pragma unroll 4
     for (int64_t k = t; k < n; k += kStreamThreads) {
       const double d = xr[k] - K;
       s += d;
@@ -510,6 +608,7 @@ rows_stream_f64(RowArgs a)
     }
     const double inv_stdev = 1.0 / sqrt(var + a.eps);
     double* yr = a.out + off_o;
+#pragma unroll 4
     for (int64_t k = t; k < n; k += kStreamThreads) {
       double y = (xr[k] - mean) * inv_stdev;
       if (a.gamma) y *= a.gamma[k];
@@ -524,6 +623,7 @@ rows_stream_f64(RowArgs a)
     const double var = a.stats[a.map.groups + g + col * a.ld_stats];
     const double inv_stdev = 1.0 / sqrt(var + a.eps);
     double A = 0.0, B = 0.0;
+#pragma unroll 4
     for (int64_t k = t; k < n; k += kStreamThreads) {
       const double gg = a.gamma ? gr[k] * a.gamma[k] : gr[k];
       A += gg;
@@ -540,6 +640,7 @@ rows_stream_f64(RowArgs a)
     const double nn = static_cast<double>(n);
     const double c0 = dmean / nn, c1 = dvar * 2 / nn;
     double* dr = a.out + off_o;
+#pragma unroll 4
     for (int64_t k = t; k < n; k += kStreamThreads) {
       const double gg = a.gamma ? gr[k] * a.gamma[k] : gr[k];
       dr[k] = gg * inv_stdev + c0 + c1 * (xr[k] - mean);
@@ -618,14 +719,32 @@ struct BnArgs {
 };
 
 // Entry j of channel c: column j / seg, position j % seg (seg = accesses per column segment).
-template <int W, typename F>
-__device__ __forceinline__ void bn_walk(int64_t seg, int64_t w, int p, int P, F f)
+// A thread's accesses are taken four at a time: load(u, column, position) for all four first, then
+// use(u, column, position), so that four requests are in flight per thread.
+constexpr int kBnUnroll = 4;
+
+template <int W, typename Load, typename Use>
+__device__ __forceinline__ void bn_walk(int64_t seg, int64_t w, int p, int P, Load load, Use use)
 {
   // seg * w < 2^31 (host check): 32-bit division
   const unsigned total = static_cast<unsigned>(seg * w), useg = static_cast<unsigned>(seg);
-  for (unsigned j = static_cast<unsigned>(p) * kBnThreads + threadIdx.x; j < total; j += static_cast<unsigned>(P) * kBnThreads) {
-    const unsigned col = j / useg;
-    f(static_cast<int64_t>(col), static_cast<int64_t>(W) * (j - col * useg));
+  const unsigned step = static_cast<unsigned>(P) * kBnThreads;
+  for (unsigned j0 = static_cast<unsigned>(p) * kBnThreads + threadIdx.x; j0 < total; j0 += kBnUnroll * step) {
+    int64_t col[kBnUnroll], pos[kBnUnroll];
+    bool in[kBnUnroll];
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u) {
+      const unsigned j = j0 + u * step;
+      in[u] = j < total && j >= j0;  // (the second test: no wrap-around near 2^32)
+      const unsigned jj = in[u] ? j : j0;
+      const unsigned c = jj / useg;
+      col[u] = c;
+      pos[u] = static_cast<int64_t>(W) * (jj - c * useg);
+      load(u, col[u], pos[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u)
+      if (in[u]) use(u, col[u], pos[u]);
   }
 }
 
@@ -640,23 +759,27 @@ bn_sums_f64(BnArgs a)
   const double* gc = BWD ? a.dy + c * a.cs : nullptr;
   const double K = BWD ? a.mean[c] : (a.use_pivot ? xc[0] : 0.0);
   double s = 0.0, q = 0.0;
-  bn_walk<W>(a.cs / W, a.w, p, P, [&](int64_t col, int64_t pos) {
-    double v[W], g[W];
-    load_w<W>(xc + col * a.ldx + pos, v);
-    if (BWD) load_w<W>(gc + col * a.lddy + pos, g);
+  double v[kBnUnroll][W], g[kBnUnroll][W];
+  bn_walk<W>(
+    a.cs / W, a.w, p, P,
+    [&](int u, int64_t col, int64_t pos) {
+      load_w<W>(xc + col * a.ldx + pos, v[u]);
+      if (BWD) load_w<W>(gc + col * a.lddy + pos, g[u]);
+    },
+    [&](int u, int64_t, int64_t) {
 #pragma unroll
-    for (int j = 0; j < W; ++j) {
-      const double d = v[j] - K;
-      if (BWD) {
-        s += g[j];
-        q += g[j] * d;
+      for (int j = 0; j < W; ++j) {
+        const double d = v[u][j] - K;
+        if (BWD) {
+          s += g[u][j];
+          q += g[u][j] * d;
+        }
+        else {
+          s += d;
+          q += d * d;
+        }
       }
-      else {
-        s += d;
-        q += d * d;
-      }
-    }
-  });
+    });
   s = team_sum_d<kBnThreads / kWave>(s, red[0]);
   q = team_sum_d<kBnThreads / kWave>(q, red[1]);
   if (threadIdx.x == 0) a.part[c * P + p] = make_double2(s, q);
@@ -716,13 +839,14 @@ bn_fwd_apply_f64(BnArgs a)
   }
   const double inv_stdev = 1.0 / sqrt(var + a.eps);
   const double scale = a.gamma[c], bias = a.beta[c];
-  bn_walk<W>(a.cs / W, a.w, p, P, [&](int64_t col, int64_t pos) {
-    double v[W];
-    load_w<W>(xc + col * a.ldx + pos, v);
+  double v[kBnUnroll][W];
+  bn_walk<W>(
+    a.cs / W, a.w, p, P, [&](int u, int64_t col, int64_t pos) { load_w<W>(xc + col * a.ldx + pos, v[u]); },
+    [&](int u, int64_t col, int64_t pos) {
 #pragma unroll
-    for (int j = 0; j < W; ++j) v[j] = scale * ((v[j] - mean) * inv_stdev) + bias;
-    store_w<W>(yc + col * a.ldo + pos, v);
-  });
+      for (int j = 0; j < W; ++j) v[u][j] = scale * ((v[u][j] - mean) * inv_stdev) + bias;
+      store_w<W>(yc + col * a.ldo + pos, v[u]);
+    });
 }
 
 template <int W>
@@ -752,14 +876,18 @@ bn_bwd_apply_f64(BnArgs a)
   const double k0 = scale * inv_stdev;
   const double c0 = dmean / static_cast<double>(n);
   const double c1 = dvar * 2 / static_cast<double>(n - (a.bessel ? 1 : 0));
-  bn_walk<W>(a.cs / W, a.w, p, P, [&](int64_t col, int64_t pos) {
-    double v[W], g[W];
-    load_w<W>(xc + col * a.ldx + pos, v);
-    load_w<W>(gc + col * a.lddy + pos, g);
+  double v[kBnUnroll][W], g[kBnUnroll][W];
+  bn_walk<W>(
+    a.cs / W, a.w, p, P,
+    [&](int u, int64_t col, int64_t pos) {
+      load_w<W>(xc + col * a.ldx + pos, v[u]);
+      load_w<W>(gc + col * a.lddy + pos, g[u]);
+    },
+    [&](int u, int64_t col, int64_t pos) {
 #pragma unroll
-    for (int j = 0; j < W; ++j) g[j] = zero ? 0.0 : g[j] * k0 + c0 + c1 * (v[j] - mean);
-    store_w<W>(dc + col * a.ldo + pos, g);
-  });
+      for (int j = 0; j < W; ++j) g[u][j] = zero ? 0.0 : g[u][j] * k0 + c0 + c1 * (v[u][j] - mean);
+      store_w<W>(dc + col * a.ldo + pos, g[u]);
+    });
 }
 
 // ================================================================== host side
@@ -784,7 +912,7 @@ static int64_t row_grid(int64_t rows, int teams, bool wgrad = false)
 }
 
 #define LBN_F64_SHAPES(X, W)                                                                          \
-  X(64, 1, W) X(64, 2, W) X(64, 4, W) X(64, 8, W) X(256, 1, W) X(256, 2, W) X(256, 4, W) X(256, 8, W) \
+  X(64, 1, W) X(64, 2, W) X(256, 1, W) X(256, 2, W)                                                   \
   X(1024, 1, W) X(1024, 2, W) X(1024, 4, W) X(1024, 8, W) X(1024, 16, W)
 
 static int sm_check(int64_t G, int64_t n, int64_t stride, int64_t w, const int64_t* lds, int nld)
@@ -935,7 +1063,7 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     if (wgrad) {                                                                                        \
       hipLaunchKernelGGL((ln_bwd_rows_f64<TPR, VV, WW, true>), dim3(static_cast<unsigned>(grid)),       \
                          dim3(Team<TPR>::kThreads), 0, st, a);                                          \
-      hipLaunchKernelGGL(ln_wgrad_reduce_f64, dim3(static_cast<unsigned>(ceil_div(2 * n, 256))), dim3(256), 0, st, \
+      hipLaunchKernelGGL(ln_wgrad_reduce_f64, dim3(static_cast<unsigned>(ceil_div(2 * n, 16))), dim3(256), 0, st, \
                          a.part, grid * Team<TPR>::kTeams, n, dgamma, dbeta);                           \
     }                                                                                                   \
     else {                                                                                              \
@@ -955,7 +1083,7 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     slabs = ceil_div(rows, per);
     hipLaunchKernelGGL(ln_wgrad_columns_f64, dim3(static_cast<unsigned>(ceil_div(n, 256)), static_cast<unsigned>(slabs)),
                        dim3(256), 0, st, a, per);
-    hipLaunchKernelGGL(ln_wgrad_reduce_f64, dim3(static_cast<unsigned>(ceil_div(2 * n, 256))), dim3(256), 0, st, a.part,
+    hipLaunchKernelGGL(ln_wgrad_reduce_f64, dim3(static_cast<unsigned>(ceil_div(2 * n, 16))), dim3(256), 0, st, a.part,
                        slabs, n, dgamma, dbeta);
   }
   return launch_status();
