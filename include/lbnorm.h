@@ -396,6 +396,20 @@ int lbn_softmax_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
                         const float* y, int64_t ldy, const float* dy, int64_t lddy,
                         float* dx, int64_t lddx, void* workspace, size_t workspace_bytes);
 
+/* For parity tests only (see LBN_STATS_REFERENCE_ORDER): softmax forward with the column's
+ * denominator formed as the reference CPU code forms it (openmp/softmax.hpp:75-95: ONE
+ * sequential fp32 sum of exp(x - max) in row order), and log-softmax backward with the
+ * column's sum of dy formed likewise (log_softmax.cpp:108-118).  What the default kernels
+ * add as trees then agrees with the CPU code to the last bits (the log-softmax sum bit for
+ * bit; the softmax denominator up to the 1-ulp difference between two accurate exponential
+ * functions).  One wave per column, one lane adding: rejected with LBN_ERR_UNSUPPORTED
+ * above 2^27 entries.  No workspace. */
+int lbn_softmax_fwd_reference_order_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                        const float* x, int64_t ldx, float* y, int64_t ldy);
+int lbn_log_softmax_bwd_reference_order_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                            const float* y, int64_t ldy, const float* dy, int64_t lddy,
+                                            float* dx, int64_t lddx);
+
 /* Softmax forward for callers that cannot allocate device memory or hand over a
  * workspace: code running under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, results

@@ -66,6 +66,8 @@ PROTOTYPES = {
     "lbn_softmax_workspace_bytes": (sz, [i64, i64]),
     "lbn_softmax_fwd_f32": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_softmax_bwd_f32": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
+    "lbn_softmax_fwd_reference_order_f32": (cint, [vp, i64, i64, vp, i64, vp, i64]),
+    "lbn_log_softmax_bwd_reference_order_f32": (cint, [vp, i64, i64, vp, i64, vp, i64, vp, i64]),
     "lbn_softmax_fwd_static_scratch_max_bytes": (sz, []),
     "lbn_softmax_fwd_static_scratch_f32": (cint, [vp, i64, i64, vp, i64, vp, i64]),
     "lbn_softmax_fwd_static_scratch_prepare": (cint, []),

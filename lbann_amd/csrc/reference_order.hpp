@@ -17,6 +17,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cfloat>
 #include <cstdint>
 
 #include "device_utils.hpp"
@@ -226,6 +227,59 @@ ln_ref_order_fwd(const T* __restrict__ x, T* __restrict__ y, int64_t ldx, int64_
     if (beta) r = ref_add(r, beta[k]);
     Vec16<T>::store1(yr + k, r);
   }
+}
+
+// ------------------------------------------------------------------- softmax family
+// Softmax forward of column blockIdx.x as openmp/softmax.hpp:39-117 computes it: the column's
+// maximum, then ONE sequential fp32 sum of exp(x - max) in row order (the exponentials themselves
+// are evaluated by all lanes, with the accurate library exponential), then y = (1 / sum) * exp,
+// non-normal results flushed to zero.
+static __global__ void __launch_bounds__(kWave)
+sm_ref_order_fwd(const float* __restrict__ x, float* __restrict__ y, int64_t ldx, int64_t ldy, int64_t h)
+{
+  __shared__ float buf[1][kRefChunk];
+  __shared__ float result;
+  const float* xc = x + static_cast<int64_t>(blockIdx.x) * ldx;
+  float* yc = y + static_cast<int64_t>(blockIdx.x) * ldy;
+  float m = -FLT_MAX;
+  for (int64_t r = threadIdx.x; r < h; r += kWave) m = fmaxf(m, xc[r]);
+  m = wave_max(m);
+  float sum = 0.f;
+  ref_order_walk<1>(
+    h, buf,
+    [&](int64_t idx, float (&v)[1]) {
+      v[0] = expf(ref_sub(xc[idx], m));
+      yc[idx] = v[0];  // in place safe: x[idx] is not read again
+    },
+    [&](const float (&v)[1]) { sum = ref_add(sum, v[0]); });
+  if (threadIdx.x == 0) result = ref_div(1.f, sum);
+  __syncthreads();
+  const float scale = result;
+  for (int64_t r = threadIdx.x; r < h; r += kWave) {
+    const float t = ref_mul(scale, yc[r]);
+    yc[r] = __builtin_isnormal(t) ? t : 0.f;
+  }
+}
+
+// Log-softmax backward of column blockIdx.x as log_softmax.cpp:95-136 computes it: ONE sequential
+// fp32 sum of dy in row order, then dx = dy - exp(y) * sum.
+static __global__ void __launch_bounds__(kWave)
+lsm_ref_order_bwd(const float* __restrict__ y, const float* __restrict__ dy, float* __restrict__ dx, int64_t ldy,
+                  int64_t lddy, int64_t lddx, int64_t h)
+{
+  __shared__ float buf[1][kRefChunk];
+  __shared__ float result;
+  const float* yc = y + static_cast<int64_t>(blockIdx.x) * ldy;
+  const float* gc = dy + static_cast<int64_t>(blockIdx.x) * lddy;
+  float* dc = dx + static_cast<int64_t>(blockIdx.x) * lddx;
+  float sum = 0.f;
+  ref_order_walk<1>(
+    h, buf, [&](int64_t idx, float (&v)[1]) { v[0] = gc[idx]; },
+    [&](const float (&v)[1]) { sum = ref_add(sum, v[0]); });
+  if (threadIdx.x == 0) result = sum;
+  __syncthreads();
+  const float s = result;
+  for (int64_t r = threadIdx.x; r < h; r += kWave) dc[r] = ref_sub(gc[r], ref_mul(expf(yc[r]), s));
 }
 
 }  // namespace lbn

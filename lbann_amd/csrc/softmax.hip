@@ -29,6 +29,7 @@
 #include "cluster_sync.hpp"
 #include "device_utils.hpp"
 #include "host_utils.hpp"
+#include "reference_order.hpp"
 #include "softmax_cluster.hpp"
 #include "softmax_rows.hpp"
 #include "softmax_split.hpp"
@@ -847,6 +848,32 @@ int lbn_softmax_fwd_static_scratch_f32(lbn_stream_t stream, int64_t height, int6
   const int status = static_scratch_address(&ptr);
   if (status != LBN_OK) return status;
   return sm_fwd<kSoftmax>(as_stream(stream), 1, height, height, width, x, ldx, y, ldy, ptr, kStaticScratchBytes);
+}
+
+// Parity tests only: the reference's order of summation (reference_order.hpp).
+int lbn_softmax_fwd_reference_order_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* x,
+                                        int64_t ldx, float* y, int64_t ldy)
+{
+  if (height < 0 || width < 0 || (width > 1 && (ldx < height || ldy < height))) return LBN_ERR_INVALID_ARGUMENT;
+  if (height == 0 || width == 0) return LBN_OK;
+  if (!x || !y) return LBN_ERR_INVALID_ARGUMENT;
+  if (height > kRefOrderMaxEntries / width || width > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(sm_ref_order_fwd, dim3(static_cast<unsigned>(width)), dim3(kWave), 0, as_stream(stream), x, y, ldx,
+                     ldy, height);
+  return launch_status();
+}
+
+int lbn_log_softmax_bwd_reference_order_f32(lbn_stream_t stream, int64_t height, int64_t width, const float* y,
+                                            int64_t ldy, const float* dy, int64_t lddy, float* dx, int64_t lddx)
+{
+  if (height < 0 || width < 0 || (width > 1 && (ldy < height || lddy < height || lddx < height)))
+    return LBN_ERR_INVALID_ARGUMENT;
+  if (height == 0 || width == 0) return LBN_OK;
+  if (!y || !dy || !dx) return LBN_ERR_INVALID_ARGUMENT;
+  if (height > kRefOrderMaxEntries / width || width > (int64_t(1) << 30)) return LBN_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(lsm_ref_order_bwd, dim3(static_cast<unsigned>(width)), dim3(kWave), 0, as_stream(stream), y, dy,
+                     dx, ldy, lddy, lddx, height);
+  return launch_status();
 }
 
 int lbn_softmax_fwd_static_scratch_prepare(void)

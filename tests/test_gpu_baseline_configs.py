@@ -188,6 +188,49 @@ def test_cfg4_layer_norm_reference_order_meets_the_strict_gate(L, W):
     check("cfg4 reference-order dbias", db, db_own, tol=TOL_F16, strict=True)
 
 
+def test_cfg2_cfg5b_softmax_reference_order_meets_the_strict_gate(L, W):
+    """The two softmax-family tensors of the benchmark that the default kernels pass through the
+    float64 leg (cfg5b y: 262144 sequential fp32 additions per column in the reference; cfg2
+    log-softmax dx: 32768), with the column sums formed in the reference's order: within 1e-5 of
+    the fp32 reference itself."""
+    d = W.cfg5b_wide_softmax()
+    x = f32(d["x"])
+    h, w = x.shape
+    xm, ym = L.DeviceMatrix.from_numpy(x), L.DeviceMatrix(h, w)
+    L.call("lbn_softmax_fwd_reference_order_f32", L._stream(), h, w, xm.Buffer(), xm.ldim, ym.Buffer(), ym.ldim)
+    check("cfg5b reference-order y", ym.to_numpy(), orc.softmax_fwd(x), orc.softmax_fwd(f64(x)), strict=True)
+    d = W.cfg2_softmax()
+    x, dy = f32(d["x"]), f32(d["dy"])
+    h, w = x.shape
+    layer = L.log_softmax_layer()
+    y = layer.forward(L.DeviceMatrix.from_numpy(x)).to_numpy()
+    ym, gm, dm = L.DeviceMatrix.from_numpy(y), L.DeviceMatrix.from_numpy(dy), L.DeviceMatrix(h, w)
+    L.call("lbn_log_softmax_bwd_reference_order_f32", L._stream(), h, w, ym.Buffer(), ym.ldim, gm.Buffer(), gm.ldim,
+           dm.Buffer(), dm.ldim)
+    check("cfg2 log_softmax reference-order dx", dm.to_numpy(), orc.log_softmax_bwd(y, dy),
+          orc.log_softmax_bwd(f64(y), f64(dy)), strict=True)
+    # small and ragged shapes, in place, and the size limit
+    rng = np.random.default_rng(77)
+    for hh, ww, pad in ((1, 3, 0), (255, 4, 0), (256, 2, 1), (1001, 5, 3)):
+        xs = np.asfortranarray((2 * rng.standard_normal((ww, hh))).astype(np.float32).T)
+        gs = np.asfortranarray(rng.standard_normal((ww, hh)).astype(np.float32).T)
+        xm = L.DeviceMatrix.from_numpy(xs, ldim=hh + pad)
+        L.call("lbn_softmax_fwd_reference_order_f32", L._stream(), hh, ww, xm.Buffer(), xm.ldim, xm.Buffer(), xm.ldim)
+        check(f"reference-order softmax {hh}x{ww}", xm.to_numpy(), orc.softmax_fwd(xs), strict=True)
+        ys = orc.log_softmax_fwd(xs)
+        ym, gm = L.DeviceMatrix.from_numpy(ys, ldim=hh + pad), L.DeviceMatrix.from_numpy(gs, ldim=hh + pad)
+        L.call("lbn_log_softmax_bwd_reference_order_f32", L._stream(), hh, ww, ym.Buffer(), ym.ldim, gm.Buffer(),
+               gm.ldim, gm.Buffer(), gm.ldim)
+        check(f"reference-order log_softmax bwd {hh}x{ww}", gm.to_numpy(), orc.log_softmax_bwd(ys, gs), strict=True)
+    lib = L.capi.lib()
+    small = L.DeviceMatrix(16, 1)
+    p = small.Buffer()
+    big_h = (1 << 27) // 4 + 1
+    assert lib.lbn_softmax_fwd_reference_order_f32(L._stream(), big_h, 4, p, big_h, p, big_h) == L.capi.LBN_ERR_UNSUPPORTED
+    assert lib.lbn_log_softmax_bwd_reference_order_f32(L._stream(), big_h, 4, p, big_h, p, big_h, p,
+                                                       big_h) == L.capi.LBN_ERR_UNSUPPORTED
+
+
 def test_reference_order_mode_rejects_large_tensors(L):
     """The mode is for parity tests: above 2^27 entries it is refused before any launch (the
     small buffers passed here are never touched)."""
