@@ -81,6 +81,14 @@ WORKLOADS = [
     ("esb_bwd_tile", None, "extra: entry-wise scale/bias bwd", 3 * 67108864 * 4),
     ("csb_fwd", None, "extra: channel-wise scale/bias fwd 64x256x56x56", 2 * _E3 * 4),
     ("csb_bwd", None, "extra: channel-wise scale/bias bwd", 3 * _E3 * 4),
+    ("f64::sm_fwd_rows_f64<0, 1024, 16", None, "extra: softmax fp64 fwd 32768x512", 2 * _E2 * 8),
+    ("f64::rows_stream_f64<1, 0>", None, "extra: softmax fp64 bwd (one workgroup per row, two passes)", 3 * _E2 * 8),
+    ("f64::ln_fwd_rows_f64", None, "extra: layer norm fp64 fwd 4096x8192", 2 * _E4 * 8),
+    ("f64::ln_bwd_rows_f64", None, "extra: layer norm fp64 bwd (followed by ln_wgrad_reduce_f64)", 3 * _E4 * 8),
+    ("f64::bn_sums_f64<2, false>", None, "extra: batch norm fp64 64x256x28x28 fwd, kernel 1 of 2 (reads x)", 12845056 * 8),
+    ("f64::bn_fwd_apply_f64", None, "extra: batch norm fp64 fwd, kernel 2 of 2 (reads x, writes y)", 2 * 12845056 * 8),
+    ("f64::bn_sums_f64<2, true>", None, "extra: batch norm fp64 bwd, kernel 1 of 2 (reads x, dy)", 2 * 12845056 * 8),
+    ("f64::bn_bwd_apply_f64", None, "extra: batch norm fp64 bwd, kernel 2 of 2 (reads x, dy, writes dx)", 3 * 12845056 * 8),
     ("grad_sink_quads<true>", None, "extra: gradient buffer, cleared: overwrite 4096x4096", 2 * _E2 * 4),
     ("grad_sink_quads<false>", None, "extra: gradient buffer, ready: accumulate 4096x4096", 3 * _E2 * 4),
 ]
