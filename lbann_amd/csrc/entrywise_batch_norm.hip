@@ -114,7 +114,8 @@ __device__ __forceinline__ void ebn_merge(float (&a)[4], float (&b)[4],
   }
 }
 
-template <int CPT, int GW>
+// ST: inputs through streaming loads (calls that move more than the last-level cache holds).
+template <int CPT, int GW, bool ST>
 __global__ void __launch_bounds__(kEbnThreads)
 ebn_fwd_tile(EbnArgs a)
 {
@@ -132,7 +133,8 @@ ebn_fwd_tile(EbnArgs a)
   for (int j = 0; j < CPT; ++j) {
     const int64_t c = p.g + P::kGroups * j;
     if (c < a.w) {
-      Vec16<float>::load(a.x + rr + c * a.ldx, v[j]);
+      if constexpr (ST) Vec16<float>::load_stream(a.x + rr + c * a.ldx, v[j]);
+      else Vec16<float>::load(a.x + rr + c * a.ldx, v[j]);
     }
     else {
 #pragma unroll
@@ -183,7 +185,7 @@ ebn_fwd_tile(EbnArgs a)
   }
 }
 
-template <int CPT, int GW>
+template <int CPT, int GW, bool ST>
 __global__ void __launch_bounds__(kEbnThreads)
 ebn_bwd_tile(EbnArgs a)
 {
@@ -202,8 +204,14 @@ ebn_bwd_tile(EbnArgs a)
   for (int j = 0; j < CPT; ++j) {
     const int64_t c = p.g + P::kGroups * j;
     if (c < a.w) {
-      Vec16<float>::load(a.x + rr + c * a.ldx, xc[j]);
-      Vec16<float>::load(a.dy + rr + c * a.lddy, gv[j]);
+      if constexpr (ST) {
+        Vec16<float>::load_stream(a.x + rr + c * a.ldx, xc[j]);
+        Vec16<float>::load_stream(a.dy + rr + c * a.lddy, gv[j]);
+      }
+      else {
+        Vec16<float>::load(a.x + rr + c * a.ldx, xc[j]);
+        Vec16<float>::load(a.dy + rr + c * a.lddy, gv[j]);
+      }
     }
     else {
 #pragma unroll
@@ -538,10 +546,12 @@ int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_
                    aligned16(stats) && ld_stats % 4 == 0 && aligned16(running_mean) &&
                    aligned16(running_var);
   if (training && vec && width <= kEbnMaxTileWidth) {
+    const bool stream = stream_call_inputs(2 * height * width * 4);
 #define X(C, G)                                                                                  \
   if (width <= 4 * G * C) {                                                                      \
     const dim3 grid(static_cast<unsigned>(ceil_div(height, EbnPos<G>::kRows)));                  \
-    hipLaunchKernelGGL((ebn_fwd_tile<C, G>), grid, dim3(kEbnThreads), 0, st, a);                 \
+    if (stream) hipLaunchKernelGGL((ebn_fwd_tile<C, G, true>), grid, dim3(kEbnThreads), 0, st, a); \
+    else hipLaunchKernelGGL((ebn_fwd_tile<C, G, false>), grid, dim3(kEbnThreads), 0, st, a);     \
     return launch_status();                                                                      \
   }
     LBN_EBN_TILE_CASES(X)
@@ -591,10 +601,12 @@ int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_
                    ebn_vec_ok(height, width, dx, lddx) && aligned16(stats) && ld_stats % 4 == 0 &&
                    aligned16(stats_grad) && ld_stats_grad % 4 == 0;
   if (vec && width <= kEbnMaxTileWidth) {
+    const bool stream = stream_call_inputs(3 * height * width * 4);
 #define X(C, G)                                                                                  \
   if (width <= 4 * G * C) {                                                                      \
     const dim3 grid(static_cast<unsigned>(ceil_div(height, EbnPos<G>::kRows)));                  \
-    hipLaunchKernelGGL((ebn_bwd_tile<C, G>), grid, dim3(kEbnThreads), 0, st, a);                 \
+    if (stream) hipLaunchKernelGGL((ebn_bwd_tile<C, G, true>), grid, dim3(kEbnThreads), 0, st, a); \
+    else hipLaunchKernelGGL((ebn_bwd_tile<C, G, false>), grid, dim3(kEbnThreads), 0, st, a);     \
     return launch_status();                                                                      \
   }
     LBN_EBN_TILE_CASES(X)

@@ -45,6 +45,19 @@ inline bool stream_is_capturing(hipStream_t st)
   return status != hipStreamCaptureStatusNone;
 }
 
+// Calls that move more than the 256 MB last-level cache holds read their inputs with streaming
+// (non-temporal) loads: nothing they read is found there, and lines that are read once then do
+// not displace each other.  Smaller calls keep ordinary loads, which find what the neighbouring
+// layers have just written.  LBN_STREAM_LOADS=0|1 overrides, for experiments.
+constexpr int64_t kStreamLoadMinBytes = int64_t(384) << 20;
+
+inline bool stream_call_inputs(int64_t bytes_moved)
+{
+  static const int forced = std::getenv("LBN_STREAM_LOADS") ? std::atoi(std::getenv("LBN_STREAM_LOADS")) : -1;
+  if (forced >= 0) return forced != 0;
+  return bytes_moved >= kStreamLoadMinBytes;
+}
+
 // Device address (current device) and size of the library-owned scratch array of the entry
 // point that allocates nothing (defined in softmax.hip); *out stays null on failure.
 int static_scratch_address(void** out);

@@ -1214,9 +1214,16 @@ static int ln_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
     return launch_status();
   }
   if (vec) {
-    if (int r = ln_fwd_rows_launch<T>(st, x, y, ldx, ldy, map, rows, n / VE, inv_n, eps, stats, lds, gamma,
-                                      beta, sumsq))
-      return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
+    int r;
+    if (stream_call_inputs(2 * rows * n * static_cast<int64_t>(sizeof(T)))) {
+      using S = typename Streamed<T>::type;  // the same kernels with streaming loads of x
+      r = ln_fwd_rows_launch<S>(st, reinterpret_cast<const S*>(x), reinterpret_cast<S*>(y), ldx, ldy, map, rows,
+                                n / VE, inv_n, eps, stats, lds, gamma, beta, sumsq);
+    }
+    else {
+      r = ln_fwd_rows_launch<T>(st, x, y, ldx, ldy, map, rows, n / VE, inv_n, eps, stats, lds, gamma, beta, sumsq);
+    }
+    if (r) return r < 0 ? LBN_ERR_UNSUPPORTED : launch_status();
     // longer than the register kernels hold: clusters when the caller gave scratch, else two passes
     if (ln_fwd_cluster_launch<T>(st, x, y, ldx, ldy, map, rows, n, eps, stats, lds, gamma, beta, sumsq, ws, ws_bytes))
       return launch_status();
@@ -1408,9 +1415,18 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                    rows_aligned16(dx, stride, lddx, G, w, sizeof(T)) &&
                    (!gamma || aligned16(gamma));
   if (vec) {
-    if (int r = ln_bwd_rows_launch<T>(st, wgrad, x, dy, dx, ldx, lddy, lddx, map, rows, n / VE, n, sizeof(T), eps,
-                                      stats, lds, sgrad, ldsg, gamma, dgamma, dbeta, ws, ws_bytes))
-      return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
+    int r;
+    if (stream_call_inputs(3 * rows * n * static_cast<int64_t>(sizeof(T)))) {
+      using S = typename Streamed<T>::type;  // the same kernels with streaming loads of x and dy
+      r = ln_bwd_rows_launch<S>(st, wgrad, reinterpret_cast<const S*>(x), reinterpret_cast<const S*>(dy),
+                                reinterpret_cast<S*>(dx), ldx, lddy, lddx, map, rows, n / VE, n, sizeof(T), eps,
+                                stats, lds, sgrad, ldsg, gamma, dgamma, dbeta, ws, ws_bytes);
+    }
+    else {
+      r = ln_bwd_rows_launch<T>(st, wgrad, x, dy, dx, ldx, lddy, lddx, map, rows, n / VE, n, sizeof(T), eps,
+                                stats, lds, sgrad, ldsg, gamma, dgamma, dbeta, ws, ws_bytes);
+    }
+    if (r) return r < 0 ? LBN_ERR_WORKSPACE : launch_status();
     // longer than the register kernels hold: clusters (weight gradients included), else two passes
     if (ln_bwd_cluster_launch<T>(st, wgrad, x, dy, dx, ldx, lddy, lddx, map, rows, n, eps, stats, lds, sgrad, ldsg,
                                  gamma, dgamma, dbeta, ws, ws_bytes))

@@ -51,7 +51,8 @@ using EsbPos = RowTilePos<GW>;
 
 // CH: one (scale, bias) pair per channel of a.cs rows instead of one per row (channel-wise
 // scale/bias on channels too small for the channel walk further down).
-template <int GW, bool CH = false>
+// ST: inputs through streaming loads (calls that move more than the last-level cache holds).
+template <int GW, bool CH = false, bool ST = false>
 __global__ void __launch_bounds__(kSbThreads)
 esb_fwd_tile(EsbArgs a)
 {
@@ -78,7 +79,10 @@ esb_fwd_tile(EsbArgs a)
   for (; c + 3 * P::kGroups < c1; c += 4 * P::kGroups) {
     float v[4][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) Vec16<float>::load(a.x + r0 + (c + j * P::kGroups) * a.ldx, v[j]);
+    for (int j = 0; j < 4; ++j) {
+      if constexpr (ST) Vec16<float>::load_stream(a.x + r0 + (c + j * P::kGroups) * a.ldx, v[j]);
+      else Vec16<float>::load(a.x + r0 + (c + j * P::kGroups) * a.ldx, v[j]);
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -95,7 +99,7 @@ esb_fwd_tile(EsbArgs a)
   }
 }
 
-template <int GW, bool CH = false>
+template <int GW, bool CH = false, bool ST = false>
 __global__ void __launch_bounds__(kSbThreads)
 esb_bwd_tile(EsbArgs a)
 {
@@ -121,8 +125,14 @@ esb_bwd_tile(EsbArgs a)
     float v[2][4], g[2][4];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      Vec16<float>::load(a.x + rr + (c + j * P::kGroups) * a.ldx, v[j]);
-      Vec16<float>::load(a.dy + rr + (c + j * P::kGroups) * a.lddy, g[j]);
+      if constexpr (ST) {
+        Vec16<float>::load_stream(a.x + rr + (c + j * P::kGroups) * a.ldx, v[j]);
+        Vec16<float>::load_stream(a.dy + rr + (c + j * P::kGroups) * a.lddy, g[j]);
+      }
+      else {
+        Vec16<float>::load(a.x + rr + (c + j * P::kGroups) * a.ldx, v[j]);
+        Vec16<float>::load(a.dy + rr + (c + j * P::kGroups) * a.lddy, g[j]);
+      }
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -469,6 +479,8 @@ int lbn_entrywise_scale_bias_fwd_f32(lbn_stream_t stream, int64_t height, int64_
     a.slab_width = p.slab_width;
     const dim3 grid(static_cast<unsigned>(p.tiles), static_cast<unsigned>(p.slabs));
     if (p.gw == 1) hipLaunchKernelGGL((esb_fwd_tile<1>), grid, dim3(kSbThreads), 0, st, a);
+    else if (stream_call_inputs(2 * height * width * 4))
+      hipLaunchKernelGGL((esb_fwd_tile<4, false, true>), grid, dim3(kSbThreads), 0, st, a);
     else hipLaunchKernelGGL((esb_fwd_tile<4>), grid, dim3(kSbThreads), 0, st, a);
     return launch_status();
   }
@@ -514,6 +526,8 @@ int lbn_entrywise_scale_bias_bwd_f32(lbn_stream_t stream, int64_t height, int64_
       return LBN_ERR_WORKSPACE;
     const dim3 grid(static_cast<unsigned>(p.tiles), static_cast<unsigned>(slabs));
     if (p.gw == 1) hipLaunchKernelGGL((esb_bwd_tile<1>), grid, dim3(kSbThreads), 0, st, a);
+    else if (stream_call_inputs(3 * height * width * 4))
+      hipLaunchKernelGGL((esb_bwd_tile<4, false, true>), grid, dim3(kSbThreads), 0, st, a);
     else hipLaunchKernelGGL((esb_bwd_tile<4>), grid, dim3(kSbThreads), 0, st, a);
     if (slabs > 1)
       hipLaunchKernelGGL(esb_merge_slabs, dim3(static_cast<unsigned>(ceil_div(height, 256))), dim3(256), 0,

@@ -104,15 +104,12 @@ constexpr int64_t kClusterMinBytes = int64_t(48) << 20;
 // the neighbouring layers and sit in the 256 MB Infinity Cache, while y was written a whole
 // forward and backward sweep ago: y is streamed once a call moves more than a third of
 // that cache, which costs nothing when the others are resident and helps when they are not.
-// Calls that move more than the cache holds stream everything.
-constexpr int64_t kStreamLoadMinBytes = int64_t(384) << 20;
+// Calls that move more than the cache holds stream everything (stream_call_inputs).
 constexpr int64_t kStreamOldInputMinBytes = int64_t(96) << 20;
 
 static int stream_loads(int64_t rows, int64_t n, int tensors)
 {
-  static const int forced = std::getenv("LBN_STREAM_LOADS") ? std::atoi(std::getenv("LBN_STREAM_LOADS")) : -1;
-  if (forced >= 0) return forced;
-  return rows * n * 4 * tensors >= kStreamLoadMinBytes ? 1 : 0;
+  return stream_call_inputs(rows * n * 4 * tensors) ? 1 : 0;
 }
 
 // A few very long rows whose tensors fit the caches (262144 x 16): one cluster kernel

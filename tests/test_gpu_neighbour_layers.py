@@ -219,6 +219,7 @@ ESB_SHAPES = [
     # (h, w, ld_pad)   tile kernels with 64 and 256 rows per workgroup, column slabs, scalar fallback
     (105, 29, 0), (4096, 64, 0), (64, 1024, 0), (1024, 4096, 0), (256 * 512, 24, 0), (256 * 512 + 8, 5, 0),
     (2048, 17, 4), (1001, 7, 0), (130, 3, 3), (4, 300, 0), (1, 9, 0), (8192, 1, 0), (300000, 16, 0),
+    (786432, 64, 0),   # a call that moves more than the last-level cache holds: streaming loads
 ]
 
 

@@ -451,6 +451,8 @@ LN_CASES = [
     # many short rows: teams of 16 lanes, four rows per wave
     ((1024, 64), -1, 8, True, 0), ((512, 128), -1, 16, True, 0), ((64, 256), -1, 70, True, 0), ((4099, 16), -1, 3, False, 0),
     ((49,), 0, 5000, True, 0), ((600, 20), -1, 9, True, 0), ((4096, 8), -1, 1, True, 0), ((2048, 12), -1, 2, True, 4),
+    # calls that move more than the last-level cache holds (192 MiB tensors): streaming loads
+    ((4096,), 0, 12288, True, 0), ((12288, 64), -1, 64, False, 0),
 ]
 
 
@@ -522,7 +524,8 @@ def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
                                                    ((50003,), 0, 3, 0), ((20002,), 0, 4, 1), ((301,), 0, 20, 0),
                                                    # long rows shared by clusters of workgroups
                                                    ((802816,), 0, 4, 0), ((65536,), 0, 150, 0), ((2, 100000), -1, 20, 8),
-                                                   ((1048576,), 0, 2, 0), ((5000000,), 0, 2, 0)])
+                                                   ((1048576,), 0, 2, 0), ((5000000,), 0, 2, 0),
+                                                   ((8192,), 0, 12288, 0)])   # 192 MiB tensors: streaming loads
 def test_layer_norm_f16(L, dims, start_dim, w, pad):
     rng = np.random.default_rng(int(np.prod(dims)) * 3 + w)
     h = int(np.prod(dims))
@@ -606,7 +609,8 @@ def test_instance_norm(L, dims, w, pad):
 @pytest.mark.parametrize("h,w,pad", [(105, 14, 0), (105, 29, 0), (4096, 64, 0), (4096, 256, 0), (1024, 300, 0),
                                      (200000, 16, 0), (64, 1, 0), (260, 7, 4), (258, 9, 0), (100000, 33, 0),
                                      (2048, 1000, 0), (8196, 257, 4), (60, 513, 0),   # wider than the register tiles
-                                     (4096, 1024, 0), (512, 4100, 0), (64, 5000, 4), (1000, 1777, 0), (4, 2000, 0), (4096, 1023, 0)])   # column slabs from 1024 columns
+                                     (4096, 1024, 0), (512, 4100, 0), (64, 5000, 4), (1000, 1777, 0), (4, 2000, 0), (4096, 1023, 0),   # column slabs from 1024 columns
+                                     (786432, 64, 0)])   # 192 MiB tensors: streaming loads
 def test_entrywise_batch_norm(L, h, w, pad):
     rng = np.random.default_rng(h + 3 * w)
     x, dy = rand(rng, h, w, 0.5, 2.0), rand(rng, h, w)
