@@ -416,6 +416,24 @@ struct Streamed<__half> {
   using type = f16s;
 };
 
+// Storage type for a tensor beside streamed data that goes through ordinary loads (the upstream
+// gradient in a backward call: the next layer has just written it).
+template <typename T>
+struct FreshInput {
+  using type = T;
+};
+template <>
+struct FreshInput<f32s> {
+  using type = float;
+};
+template <>
+struct FreshInput<f16s> {
+  using type = __half;
+};
+
+template <typename T>
+struct StreamedVec : std::integral_constant<bool, std::is_same<T, f16s>::value || std::is_same<T, f32s>::value> {};
+
 // Storage types whose 16-byte accesses need no alignment beyond that of one entry.
 template <typename T>
 struct UnalignedVec : std::integral_constant<bool, std::is_same<T, f16u>::value || std::is_same<T, f32u>::value> {};

@@ -51,11 +51,11 @@ inline bool stream_is_capturing(hipStream_t st)
 // layers have just written.  LBN_STREAM_LOADS=0|1 overrides, for experiments.
 constexpr int64_t kStreamLoadMinBytes = int64_t(384) << 20;
 
-inline bool stream_call_inputs(int64_t bytes_moved)
+inline bool stream_call_inputs(int64_t bytes_moved, int64_t min_bytes = kStreamLoadMinBytes)
 {
   static const int forced = std::getenv("LBN_STREAM_LOADS") ? std::atoi(std::getenv("LBN_STREAM_LOADS")) : -1;
   if (forced >= 0) return forced != 0;
-  return bytes_moved >= kStreamLoadMinBytes;
+  return bytes_moved >= min_bytes;
 }
 
 // Device address (current device) and size of the library-owned scratch array of the entry

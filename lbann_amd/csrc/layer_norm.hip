@@ -506,7 +506,8 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       s.x[i] = IO::load_raw(xr + voff[i]);
-      s.g[i] = IO::load_raw(gr + voff[i]);
+      using F = typename FreshInput<T>::type;  // dy through ordinary loads also beside a streamed x
+      s.g[i] = Vec16<F>::load_raw(reinterpret_cast<const F*>(gr + voff[i]));
     }
     s.mean = stats[g + col * ld_stats];
     s.var = stats[map.groups + g + col * ld_stats];
@@ -1329,7 +1330,7 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
   constexpr int VE = Vec16<ST>::N;
   const LnBwdPlan p = plan_ln_bwd(units, rows, VE, elem_bytes, wgrad);
   if (!p.tpr) return 0;
-  if constexpr (VE >= 4 && !UnalignedVec<ST>::value) {
+  if constexpr (VE >= 4 && !UnalignedVec<ST>::value && !StreamedVec<ST>::value) {  // (small calls never stream)
     if (wgrad && ln_bwd_small(rows, n, elem_bytes)) {
       // tensors that fit the caches: weight gradients from column slices, in the same kernel
       const int nvec_s = static_cast<int>(units);
@@ -1379,6 +1380,17 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
   return 1;
 }
 
+// Backward reads x a whole forward and backward sweep after the forward call did, and dy right
+// after the next layer wrote it: from 160 MiB per call x goes through streaming loads and dy through
+// ordinary ones.  Measured with the tensors of every call rotated out of the caches, rows of 4096
+// floats, % of 8 TB/s with ordinary loads / with x streamed: 96 MiB per call 78 / 66, 120 MiB 74 / 70,
+// 144 MiB 73 / 72, 168 MiB 71 / 74, 192 MiB 70 / 75, 384 MiB 70 / 74, 768 MiB 68 / 74 (dy streamed as
+// well: 76 at both; not worth a third set of kernels).  A loop over the same buffers, where x is
+// still cached from the forward call 30 us earlier, loses 9 % at 192 MiB.  Calls that also form
+// weight gradients gain next to nothing below the general limit (fp16 4096 x 8192, 192 MiB per call,
+// rotated: 67.5 -> 66.8 us per step; same buffers 59.8 -> 65.2) and keep it.
+constexpr int64_t kLnStreamOldInputMinBytes = int64_t(160) << 20;
+
 template <typename T>
 static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t w, float eps,
                   const T* x, int64_t ldx, const T* dy, int64_t lddy, T* dx, int64_t lddx,
@@ -1416,8 +1428,9 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
                    (!gamma || aligned16(gamma));
   if (vec) {
     int r;
-    if (stream_call_inputs(3 * rows * n * static_cast<int64_t>(sizeof(T)))) {
-      using S = typename Streamed<T>::type;  // the same kernels with streaming loads of x and dy
+    if (stream_call_inputs(3 * rows * n * static_cast<int64_t>(sizeof(T)),
+                           wgrad ? kStreamLoadMinBytes : kLnStreamOldInputMinBytes)) {
+      using S = typename Streamed<T>::type;  // the same kernels with streaming loads of x
       r = ln_bwd_rows_launch<S>(st, wgrad, reinterpret_cast<const S*>(x), reinterpret_cast<const S*>(dy),
                                 reinterpret_cast<S*>(dx), ldx, lddy, lddx, map, rows, n / VE, n, sizeof(T), eps,
                                 stats, lds, sgrad, ldsg, gamma, dgamma, dbeta, ws, ws_bytes);
