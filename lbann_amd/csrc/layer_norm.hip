@@ -1015,6 +1015,22 @@ static size_t ln_bwd_workspace(int64_t n, int64_t rows, int ve)
   return need;
 }
 
+// Workgroups of the row kernels that form no weight gradients, for `work` rows per team slot and
+// `resident` workgroups that the device holds at once.  One resident wave of workgroups, each
+// walking the same number of rows with the next row in flight, was the first design; workgroups
+// that live for two rows only, far more than are resident, measure faster wherever that differs
+// (forward, % of 8 TB/s with every call's tensors out of the caches, persistent -> two rows: rows of
+// 64 / 256 / 1024 / 4096 floats at 64 MiB per tensor 74 / 79 / 78 / 80 -> 80 / 81 / 81 / 80, at
+// 256 MiB 66 / 74 / 73 / 74 -> 74 / 76 / 76 / 75; fp16 4096 x 8192 on the same buffers 25.0 -> 24.0 us).
+// Backward only gains on rows of up to 2 KiB (128- and 512-float rows at 196 MiB per tensor: 68 / 66
+// -> 75 / 75) and loses on longer ones (3136 floats: 77 -> 64), which keep the resident wave.
+static int64_t ln_row_grid(int64_t work, int64_t resident, bool short_lived)
+{
+  const int64_t rounds = ceil_div(work, resident);
+  if (short_lived && rounds > 2) return ceil_div(work, 2);
+  return ceil_div(work, rounds);
+}
+
 // Register-resident forward over rows of `units` access units (16-byte vectors, or single
 // floats for ST = f32x1).  Returns 1 when launched, 0 when no configuration holds the row,
 // -1 when the occupancy query fails.
@@ -1048,8 +1064,7 @@ static int ln_fwd_rows_launch(hipStream_t st, const ST* x, ST* y, int64_t ldx, i
     const int64_t work = ceil_div(rows, B::kTeams);                                            \
     const int64_t resident = resident_blocks(ln_fwd_rows<ST, TPR, V>, B::kThreads);            \
     if (resident <= 0) return -1;                                                              \
-    /* one wave of blocks, each walking the same number of rows */                             \
-    const int64_t grid = ceil_div(work, ceil_div(work, resident));                             \
+    const int64_t grid = ln_row_grid(work, resident, true);                                    \
     hipLaunchKernelGGL((ln_fwd_rows<ST, TPR, V>), dim3(static_cast<unsigned>(grid)),           \
                        dim3(B::kThreads), 0, st, x, y, ldx, ldy, map, rows, nvec, inv_n, eps,  \
                        stats, lds, gamma, beta, sumsq, tail);                                  \
@@ -1309,7 +1324,8 @@ static void launch_ln_bwd_rows(hipStream_t st, bool wgrad, int64_t blocks, const
     const int64_t units = ceil_div(rows, TEAMS);
     int64_t resident = resident_blocks(ln_bwd_rows<T, TPR, TEAMS, V, false>, B::kThreads);
     if (resident < 1) resident = 1;
-    const dim3 all(static_cast<unsigned>(ceil_div(units, ceil_div(units, resident))));
+    // (rows of up to 2 KiB: short-lived workgroups, see ln_row_grid)
+    const dim3 all(static_cast<unsigned>(ln_row_grid(units, resident, static_cast<size_t>(n) * sizeof(T) <= 2048)));
     hipLaunchKernelGGL((ln_bwd_rows<T, TPR, TEAMS, V, false>), all, block, 0, st, x, dy, dx, ldx,
                        lddy, lddx, map, rows, nvec, n, eps, stats, lds, sgrad, ldsg, gamma, part, nullptr, nullptr,
                        tail);
@@ -1386,9 +1402,10 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
 // floats, % of 8 TB/s with ordinary loads / with x streamed: 96 MiB per call 78 / 66, 120 MiB 74 / 70,
 // 144 MiB 73 / 72, 168 MiB 71 / 74, 192 MiB 70 / 75, 384 MiB 70 / 74, 768 MiB 68 / 74 (dy streamed as
 // well: 76 at both; not worth a third set of kernels).  A loop over the same buffers, where x is
-// still cached from the forward call 30 us earlier, loses 9 % at 192 MiB.  Calls that also form
-// weight gradients gain next to nothing below the general limit (fp16 4096 x 8192, 192 MiB per call,
-// rotated: 67.5 -> 66.8 us per step; same buffers 59.8 -> 65.2) and keep it.
+// still cached from the forward call 30 us earlier, loses 9 % at 192 MiB.  With weight gradients
+// fp32 calls gain as much (192 MiB per call, rows of 256 / 1024 / 4096 floats, rotated: 46.0 / 42.6 /
+// 43.4 -> 41.9 / 37.9 / 39.5 us), 16-bit ones next to nothing below the general limit (4096 x 8192,
+// 192 MiB per call, rotated: 67.5 -> 66.8 us per step; same buffers 59.8 -> 65.2), which they keep.
 constexpr int64_t kLnStreamOldInputMinBytes = int64_t(160) << 20;
 
 template <typename T>
@@ -1429,7 +1446,7 @@ static int ln_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
   if (vec) {
     int r;
     if (stream_call_inputs(3 * rows * n * static_cast<int64_t>(sizeof(T)),
-                           wgrad ? kStreamLoadMinBytes : kLnStreamOldInputMinBytes)) {
+                           (wgrad && sizeof(T) == 2) ? kStreamLoadMinBytes : kLnStreamOldInputMinBytes)) {
       using S = typename Streamed<T>::type;  // the same kernels with streaming loads of x
       r = ln_bwd_rows_launch<S>(st, wgrad, reinterpret_cast<const S*>(x), reinterpret_cast<const S*>(dy),
                                 reinterpret_cast<S*>(dx), ldx, lddy, lddx, map, rows, n / VE, n, sizeof(T), eps,
