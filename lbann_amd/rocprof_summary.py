@@ -59,6 +59,9 @@ WORKLOADS = [
     ("ln_bwd_rows<float, 64, 4, 4, true", None, "cfg1 layer norm bwd (followed by ln_wgrad_reduce)", 3 * 131072 * 4),
     ("ln_fwd_rows<float, 256, 4>", None, "extra: instance norm fwd 64x256x56x56", 2 * _E3 * 4),
     ("ln_bwd_rows<float, 256, 2, 4, false", None, "extra: instance norm bwd", 3 * _E3 * 4),
+    # the same kernels on the storage type whose loads stream (calls beyond the last-level cache)
+    ("ln_fwd_rows<lbn::f32s, 256, 4>", None, "extra: instance norm fwd 64x256x56x56 (streaming loads)", 2 * _E3 * 4),
+    ("ln_bwd_rows<lbn::f32s, 256, 2, 4, false", None, "extra: instance norm bwd (x through streaming loads)", 3 * _E3 * 4),
     ("sm_fwd_cluster<4, 0, 4, false>", None, "extra: softmax 262144x256 fwd (row clusters)", 2 * 67108864 * 4),
     ("sm_bwd_cluster<4, 0, 4, false>", None, "extra: softmax 262144x256 bwd (row clusters)", 3 * 67108864 * 4),
     ("sm_fwd_cluster<4, 0, 4, true>", None, "extra: softmax 50257x1024 fwd (row clusters, framed 16-byte access)", 2 * 50257 * 1024 * 4),
