@@ -127,6 +127,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay leg")
     ap.add_argument("--no-cold", action="store_true", help="skip the cold-cache leg")
+    ap.add_argument("--pattern-yardstick", action="store_true",
+                    help="time the library's copy pipeline (no arithmetic, no exchange between workgroups) "
+                         "on cfg3's tensor in batch norm's order of accesses and in contiguous order")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also time a plain elementwise copy of 256 MiB (torch kernel): the practical "
                          "streaming ceiling, and the known-size kernel that scales the rocprof byte counters")
@@ -663,6 +666,49 @@ def main():
               f"({100*cold_yardstick['copy_frac']:.1f}%), add {cold_yardstick['add_gbs']:.0f} GB/s "
               f"({100*cold_yardstick['add_frac']:.1f}%)", file=sys.stderr)
         del xs, ds, os_
+        torch.cuda.empty_cache()
+
+    # Yardstick for the batch-norm kernels that share a channel among workgroups: the same register
+    # pipeline copying cfg3's tensor in their order of accesses (and in contiguous order), with
+    # nothing computed and nothing exchanged: what the memory system gives that order.
+    pattern = None
+    if args.pattern_yardstick:
+        C, cs, w = 256, 56 * 56, 64
+        h = C * cs
+        lib = L.capi.lib()
+        sets = [(L.DeviceMatrix(h, w), L.DeviceMatrix(h, w)) for _ in range(4)]
+        for xm, _ in sets:
+            xm.tensor.normal_()
+        nbytes = 2 * h * w * 4
+
+        def copy_us(channel_major, rotate, n=20):
+            def go(i):
+                xm, ym = sets[i % len(sets) if rotate else 0]
+                if lib.lbn_selftest_copy_pipeline_f32(L._stream(), C, cs, w, xm.Buffer(), xm.ldim, ym.Buffer(),
+                                                      ym.ldim, channel_major):
+                    raise RuntimeError("copy pipeline failed")
+            for i in range(4):
+                go(i)
+            torch.cuda.synchronize()
+            a, b = ev(), ev()
+            a.record()
+            for i in range(n):
+                go(i)
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / n * 1e3
+
+        pattern = {"tensor": "64x256x56x56 fp32", "bytes": nbytes}
+        for name, cm in (("contiguous", 0), ("channel_major", 1)):
+            for regime, rot in (("same_buffers", False), ("rotated", True)):
+                us = copy_us(cm, rot)
+                pattern[f"{name}_{regime}_us"] = us
+                pattern[f"{name}_{regime}_frac"] = nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS
+        print("# copy pipeline on cfg3's tensor (2 tensors of traffic, % of 8 TB/s): "
+              + ", ".join(f"{k[:-3].replace('_', ' ')} {pattern[k]:.1f} us ({100*pattern[k[:-2] + 'frac']:.1f}%)"
+                          for k in pattern if k.endswith("_us")), file=sys.stderr)
+        results["pattern_yardstick"] = pattern
+        del sets
         torch.cuda.empty_cache()
 
     committed = None

@@ -131,6 +131,19 @@ int lbn_workspace_timed_out(lbn_stream_t stream, const void* workspace, int* tim
 int lbn_selftest_cluster_wait_gives_up(lbn_stream_t stream, void* workspace, size_t workspace_bytes,
                                        int max_polls, float* out4);
 
+/* Diagnostic, no counterpart in the reference: copies x to y (num_channels channels of
+ * channel_size entries per column, `width` columns; channel_size a multiple of 4, buffers and
+ * leading dimensions on the 16-byte grid, else LBN_ERR_UNSUPPORTED) through the register
+ * pipeline of the batch-norm kernels in which workgroups share a channel (persistent workgroups
+ * of 512 threads, three tiles of four 16-byte vectors per thread in rotation, non-temporal
+ * stores) without any arithmetic and without any exchange between workgroups.  channel_major
+ * != 0 walks the matrix in the order of those kernels, channel after channel with every
+ * channel's `width` segments cut into the workgroups' shares; 0 walks contiguous tiles.
+ * The time of this call is what the memory system gives that order of accesses; bench.py
+ * --pattern-yardstick reports it beside the batch-norm figures. */
+int lbn_selftest_copy_pipeline_f32(lbn_stream_t stream, int64_t num_channels, int64_t channel_size, int64_t width,
+                                   const float* x, int64_t ldx, float* y, int64_t ldy, int channel_major);
+
 /* ------------------------------------------------------------------ layer norm
  * Replaces layer_norm_layer::fp_compute / bp_compute
  * (src/layers/regularizers/layer_norm.cpp:263-290, :292-348; math :41-136, :139-258).

@@ -29,6 +29,7 @@ PROTOTYPES = {
     "lbn_status_string": (ctypes.c_char_p, [cint]),
     "lbn_workspace_timed_out": (cint, [vp, vp, ctypes.POINTER(cint)]),
     "lbn_selftest_cluster_wait_gives_up": (cint, [vp, vp, sz, cint, vp]),
+    "lbn_selftest_copy_pipeline_f32": (cint, [vp, i64, i64, i64, vp, i64, vp, i64, cint]),
     "lbn_layer_norm_fwd_workspace_bytes": (sz, [i64, i64, i64, cint]),
     "lbn_layer_norm_fwd_f32": (cint, [vp, i64, i64, i64, i64, f32, vp, i64, vp, i64, vp, i64, vp, vp, vp, sz, cint]),
     "lbn_layer_norm_fwd_f16": (cint, [vp, i64, i64, i64, i64, f32, vp, i64, vp, i64, vp, i64, vp, vp, vp, sz, cint]),

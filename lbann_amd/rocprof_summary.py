@@ -54,6 +54,8 @@ WORKLOADS = [
     ("sm_fwd_apply", None, "cfg5b fwd, split path, kernel 2 of 2", 2 * _E5B * 4),
     ("sm_bwd_partial", None, "cfg5b bwd, split path, kernel 1 of 2", 2 * _E5B * 4),
     ("sm_bwd_apply", None, "cfg5b bwd, split path, kernel 2 of 2", 3 * _E5B * 4),
+    ("selftest_copy_pipeline<true>", None, "copy pipeline on cfg3's tensor, batch norm's order of accesses (bench.py --pattern-yardstick)", 2 * _E3 * 4),
+    ("selftest_copy_pipeline<false>", None, "copy pipeline on cfg3's tensor, contiguous tiles", 2 * _E3 * 4),
     ("ln_fwd_rows<float, 256, 1>", None, "cfg1 layer norm fwd 1024x128", 2 * 131072 * 4),
     ("ln_bwd_rows<float, 64, 4, 4, false, true>", None, "cfg1 layer norm bwd (weight gradients in the same kernel)", 3 * 131072 * 4),
     ("ln_bwd_rows<float, 64, 4, 4, true", None, "cfg1 layer norm bwd (followed by ln_wgrad_reduce)", 3 * 131072 * 4),

@@ -1289,3 +1289,34 @@ def test_layer_norm_reference_order_is_bit_equal(L, dims, start_dim, w, affine, 
         _bits_equal("y", f32(y), f32(y_ref.astype(np.float16)))
     else:
         _bits_equal("y", y, y_ref)
+
+
+# ===================================================================== diagnostics
+@pytest.mark.parametrize("C,cs,w,pad", [(5, 12, 7, 4), (1, 4, 1, 0), (3, 100000, 2, 0), (40, 3136, 16, 0),
+                                        (256, 3136, 64, 0), (700, 8, 300, 8), (2, 2048 * 4 * 3, 5, 0)])
+@pytest.mark.parametrize("channel_major", [0, 1])
+def test_selftest_copy_pipeline_copies_bit_for_bit(L, C, cs, w, pad, channel_major):
+    """The copy that stands for the batch-norm cluster kernels' order of accesses moves every
+    entry once and touches nothing else."""
+    h = C * cs
+    ld = h + pad
+    x = L.DeviceMatrix(h, w, ldim=ld)
+    x.tensor.normal_()
+    y = L.DeviceMatrix(h, w, ldim=ld, fill=-7.0)
+    L.call("lbn_selftest_copy_pipeline_f32", L._stream(), C, cs, w, x.Buffer(), x.ldim, y.Buffer(), y.ldim,
+           channel_major)
+    torch.cuda.synchronize()
+    assert torch.equal(y.tensor[:, :h], x.tensor[:, :h])
+    if pad:
+        assert bool((y.tensor[:, h:] == -7.0).all())
+
+
+def test_selftest_copy_pipeline_rejects_what_it_cannot_copy(L):
+    x = L.DeviceMatrix(24, 3)
+    y = L.DeviceMatrix(24, 3)
+    lib = L.capi.lib()
+    st = L._stream()
+    assert lib.lbn_selftest_copy_pipeline_f32(st, 4, 6, 3, x.Buffer(), 24, y.Buffer(), 24, 1) == L.capi.LBN_ERR_UNSUPPORTED
+    assert lib.lbn_selftest_copy_pipeline_f32(st, 2, 12, 3, x.Buffer(), 20, y.Buffer(), 24, 0) == L.capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_selftest_copy_pipeline_f32(st, 2, 12, 3, None, 24, y.Buffer(), 24, 0) == L.capi.LBN_ERR_INVALID_ARGUMENT
+    assert lib.lbn_selftest_copy_pipeline_f32(st, 0, 12, 3, None, 0, None, 0, 1) == L.capi.LBN_OK
