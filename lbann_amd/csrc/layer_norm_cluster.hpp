@@ -535,11 +535,29 @@ namespace lbn {
 constexpr int kLnStreamThreads = 512;
 constexpr int kLnStreamWaves = kLnStreamThreads / kWave;
 constexpr int kLnStreamUnroll = 4;
-// Vectors per thread at the head of a workgroup's share that stay in registers between the
+// Vectors per thread at the head of a workgroup's share that stay in the workgroup between the
 // two passes (16.8 M-entry rows over 128 workgroups are 64 vectors per thread, 4.1 M-entry rows
-// 16: the latter are then read once).
-constexpr int kLnStreamKeepFwd = 16;
-constexpr int kLnStreamKeepBwd = 8;
+// 16: the latter are then read once).  Forward: half of them in registers, half parked in LDS by
+// the thread that fetches them again (no barrier), 64 KiB per workgroup, so that two workgroups
+// share a compute unit (all sixteen in registers took 136 of them: one workgroup per unit).
+#ifndef LBN_LN_STREAM_KEEP_FWD
+#define LBN_LN_STREAM_KEEP_FWD 8
+#endif
+constexpr int kLnStreamKeepFwd = LBN_LN_STREAM_KEEP_FWD;
+constexpr int kLnStreamLdsFwd = 16 - kLnStreamKeepFwd;
+#ifndef LBN_LN_STREAM_KEEP_BWD
+#define LBN_LN_STREAM_KEEP_BWD 8
+#endif
+constexpr int kLnStreamKeepBwd = LBN_LN_STREAM_KEEP_BWD;
+// Backward: eight vectors per thread and tensor in registers, the next eight parked in LDS by the
+// thread that fetches them again (no barrier), 128 KiB per workgroup; the kernel's registers allow
+// one workgroup per compute unit anyway.  4.1 M-entry rows over 128 workgroups (15.6 vectors per
+// thread and tensor) are then read once: 346 -> 313 us (half as much parked: the same 313 us; two
+// workgroups per unit with eight vectors per tensor kept in all: 339 us).
+#ifndef LBN_LN_STREAM_LDS_BWD
+#define LBN_LN_STREAM_LDS_BWD 8
+#endif
+constexpr int kLnStreamLdsBwd = LBN_LN_STREAM_LDS_BWD;
 
 template <int U, typename F>
 __device__ __forceinline__ void ln_stream_walk(unsigned begin, unsigned end, F&& f)
@@ -567,8 +585,10 @@ ln_fwd_stream(LnClArgs<T> a)
   constexpr int VE = IO::N;
   // with weights the second pass also holds their loads: half the cache keeps it off the stack
   constexpr int KEEP = AFFINE ? kLnStreamKeepFwd / 2 : kLnStreamKeepFwd;
+  constexpr int LK = kLnStreamLdsFwd;
   __shared__ float red[2 * kLnStreamWaves];
   __shared__ float bc[2];
+  __shared__ typename IO::raw_t parked[LK > 0 ? LK : 1][kLnStreamThreads];
   const int64_t nc = gridDim.x / a.M;
   const int64_t cl = blockIdx.x / a.M;
   const int k = blockIdx.x - static_cast<int>(cl) * a.M;
@@ -576,7 +596,8 @@ ln_fwd_stream(LnClArgs<T> a)
   cluster_resolve_tag(a.tag);
   const unsigned begin = static_cast<unsigned>(k) * a.per_wg;
   const unsigned end = begin + a.per_wg < a.nvec ? begin + a.per_wg : a.nvec;
-  const unsigned rest_fwd = begin + KEEP * kLnStreamThreads;  // where streaming takes over
+  const unsigned parked_begin = begin + KEEP * kLnStreamThreads;
+  const unsigned rest_fwd = parked_begin + LK * kLnStreamThreads;  // where streaming takes over
   for (int64_t row = cl; row < a.rows; row += nc) {
     const T* xr = a.x + a.map.offset(row, a.ldx);
     T* yr = a.out + a.map.offset(row, a.ldo);
@@ -600,6 +621,29 @@ ln_fwd_stream(LnClArgs<T> a)
           const float d = v[j] - K;
           s += d;
           q = __builtin_fmaf(d, d, q);
+        }
+      }
+    }
+    if constexpr (LK > 0) {  // the next vectors of the share: summed now, parked in LDS for the second pass
+      typename IO::raw_t pv[LK];
+#pragma unroll
+      for (int i = 0; i < LK; ++i) {
+        const unsigned e = parked_begin + threadIdx.x + i * kLnStreamThreads;
+        pv[i] = typename IO::raw_t{};
+        if (e < end) pv[i] = IO::load_raw(xr + VE * static_cast<int64_t>(e));
+      }
+#pragma unroll
+      for (int i = 0; i < LK; ++i) {
+        if (parked_begin + threadIdx.x + i * kLnStreamThreads < end) {
+          parked[i][threadIdx.x] = pv[i];
+          float v[VE];
+          IO::unpack(pv[i], v);
+#pragma unroll
+          for (int j = 0; j < VE; ++j) {
+            const float d = v[j] - K;
+            s += d;
+            q = __builtin_fmaf(d, d, q);
+          }
         }
       }
     }
@@ -656,6 +700,21 @@ ln_fwd_stream(LnClArgs<T> a)
         IO::store(yr + VE * static_cast<int64_t>(e), v);
       }
     }
+    if constexpr (LK > 0) {
+#pragma unroll
+      for (int i = 0; i < LK; ++i) {
+        const unsigned e = parked_begin + threadIdx.x + i * kLnStreamThreads;
+        if (e < end) {
+          float v[VE], ga[VE], be[VE];
+          IO::unpack(parked[i][threadIdx.x], v);
+          ln_stream_weights<T, AFFINE>(a.gamma, e, 1.f, ga);
+          ln_stream_weights<T, AFFINE>(a.beta, e, 0.f, be);
+#pragma unroll
+          for (int j = 0; j < VE; ++j) v[j] = __builtin_fmaf((v[j] - mean) * inv_stdev, ga[j], be[j]);
+          IO::store(yr + VE * static_cast<int64_t>(e), v);
+        }
+      }
+    }
     ln_stream_walk<kLnStreamUnroll>(rest_fwd, end, [&](unsigned e, auto count) {
       constexpr int N = decltype(count)::value;
       float v[N][VE];
@@ -685,6 +744,8 @@ ln_bwd_stream(LnClArgs<T> a)
   constexpr int U = kLnStreamUnroll / 2;  // two tensors per step
   __shared__ float red[2 * kLnStreamWaves];
   __shared__ float bc[2];
+  __shared__ typename IO::raw_t parked_x[kLnStreamLdsBwd][kLnStreamThreads];
+  __shared__ typename IO::raw_t parked_g[kLnStreamLdsBwd][kLnStreamThreads];
   const int64_t nc = gridDim.x / a.M;
   const int64_t cl = blockIdx.x / a.M;
   const int k = blockIdx.x - static_cast<int>(cl) * a.M;
@@ -692,7 +753,8 @@ ln_bwd_stream(LnClArgs<T> a)
   cluster_resolve_tag(a.tag);
   const unsigned begin = static_cast<unsigned>(k) * a.per_wg;
   const unsigned end = begin + a.per_wg < a.nvec ? begin + a.per_wg : a.nvec;
-  const unsigned rest_bwd = begin + kLnStreamKeepBwd * kLnStreamThreads;
+  const unsigned parked_begin = begin + kLnStreamKeepBwd * kLnStreamThreads;
+  const unsigned rest_bwd = parked_begin + kLnStreamLdsBwd * kLnStreamThreads;
   for (int64_t row = cl; row < a.rows; row += nc) {
     int64_t col, g;
     a.map.split(row, col, g);
@@ -726,6 +788,39 @@ ln_bwd_stream(LnClArgs<T> a)
           const float gs = d[j] * ga[j];
           sa += gs;
           sb = __builtin_fmaf(gs, (x[j] - mean) * inv_stdev, sb);
+        }
+      }
+    }
+    // the next vectors of the share: summed now, parked in LDS for the second pass
+#pragma unroll
+    for (int i0 = 0; i0 < kLnStreamLdsBwd; i0 += 2) {  // two vectors of each tensor at a time
+      typename IO::raw_t px[2], pg[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const unsigned e = parked_begin + threadIdx.x + (i0 + i) * kLnStreamThreads;
+        px[i] = typename IO::raw_t{};
+        pg[i] = typename IO::raw_t{};
+        if (i0 + i < kLnStreamLdsBwd && e < end) {
+          px[i] = IO::load_raw(xr + VE * static_cast<int64_t>(e));
+          pg[i] = IO::load_raw(gr + VE * static_cast<int64_t>(e));
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const unsigned e = parked_begin + threadIdx.x + (i0 + i) * kLnStreamThreads;
+        if (i0 + i < kLnStreamLdsBwd && e < end) {
+          parked_x[i0 + i][threadIdx.x] = px[i];
+          parked_g[i0 + i][threadIdx.x] = pg[i];
+          float x[VE], d[VE], ga[VE];
+          IO::unpack(px[i], x);
+          IO::unpack(pg[i], d);
+          ln_stream_weights<T, AFFINE>(a.gamma, e, 1.f, ga);
+#pragma unroll
+          for (int j = 0; j < VE; ++j) {
+            const float gs = d[j] * ga[j];
+            sa += gs;
+            sb = __builtin_fmaf(gs, (x[j] - mean) * inv_stdev, sb);
+          }
         }
       }
     }
@@ -775,6 +870,22 @@ ln_bwd_stream(LnClArgs<T> a)
         float x[VE], d[VE], ga[VE];
         IO::unpack(kept_x[i], x);
         IO::unpack(kept_g[i], d);
+        ln_stream_weights<T, AFFINE>(a.gamma, e, 1.f, ga);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          const float xh = (x[j] - mean) * inv_stdev;
+          d[j] = __builtin_fmaf(d[j] * ga[j], inv_stdev, __builtin_fmaf(c1, xh, c0));
+        }
+        IO::store(dr + VE * static_cast<int64_t>(e), d);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kLnStreamLdsBwd; ++i) {
+      const unsigned e = parked_begin + threadIdx.x + i * kLnStreamThreads;
+      if (e < end) {
+        float x[VE], d[VE], ga[VE];
+        IO::unpack(parked_x[i][threadIdx.x], x);
+        IO::unpack(parked_g[i][threadIdx.x], d);
         ln_stream_weights<T, AFFINE>(a.gamma, e, 1.f, ga);
 #pragma unroll
         for (int j = 0; j < VE; ++j) {
