@@ -11,7 +11,7 @@ backward reads y and dy and writes dx), the roofline entry of its dominant
 kernel timed with HIP events on the launch stream, the CPU baseline (the
 restated reference CPU code, OpenMP, on the host cores), and under
 config.per_config one short row for every benchmark configuration.  Every
-timing of every row goes to stderr and to gpurun_out/bench_layers.json.
+timing of every row goes to stderr and to a JSON file whose path the last stderr line names.
 """
 import argparse
 import json
