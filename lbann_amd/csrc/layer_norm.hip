@@ -429,7 +429,7 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
             int64_t lddy, int64_t lddx, RowMap map, int64_t rows, int nvec, int n, float eps,
             const float* __restrict__ stats, int64_t ld_stats, float* __restrict__ sgrad,
             int64_t ld_sgrad, const float* __restrict__ gamma, float* __restrict__ part,
-            float* __restrict__ dscale, float* __restrict__ dbias, int tail = 0)
+            float* __restrict__ dscale, float* __restrict__ dbias, int tail = 0, int col_blocks = 0)
 {
   static_assert(!(WGRAD && COLS), "one way of forming the weight gradients");
   using B = RowBlock<TPR, TEAMS>;
@@ -454,10 +454,20 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   const int lane = tid & (kWave - 1);
   const int wv = t / kWave;
 
+  // COLS: the last col_blocks workgroups of the grid form the weight gradients from column slices
+  // and nothing else, the others walk rows and nothing else: neither waits for the other, since
+  // both read inputs of the call only (col_blocks == 0: every workgroup does both, in turn).
+  const int row_grid = COLS ? static_cast<int>(gridDim.x) - col_blocks : static_cast<int>(gridDim.x);
+  const bool col_block = COLS && col_blocks > 0 && static_cast<int>(blockIdx.x) >= row_grid;
+  const bool row_block = !col_block;
+  const int64_t first_slice = col_block ? static_cast<int64_t>(blockIdx.x) - row_grid : blockIdx.x;
+  const int64_t slice_step = (COLS && col_blocks > 0) ? col_blocks : gridDim.x;
   LnColLoads<T> cols;
   const int64_t col_slices = (n + 8 * VE - 1) / (8 * VE);
-  if constexpr (COLS)
-    ln_cols_issue<T, B::kThreads>(cols, x, dy, ldx, lddy, map, rows, n, stats, ld_stats, blockIdx.x, 0);
+  if constexpr (COLS) {
+    if (col_block || col_blocks == 0)
+      ln_cols_issue<T, B::kThreads>(cols, x, dy, ldx, lddy, map, rows, n, stats, ld_stats, first_slice, 0);
+  }
 
   // Loads are issued unconditionally: a row past the end re-reads the last row, a
   // vector past the end of a row re-reads vector 0.
@@ -514,8 +524,8 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   };
 
   const float inv_n = 1.0f / static_cast<float>(n);
-  const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * TEAMS;
-  const int64_t iters = (rows + rows_per_iter - 1) / rows_per_iter;
+  const int64_t rows_per_iter = static_cast<int64_t>(row_grid) * TEAMS;
+  const int64_t iters = row_block ? (rows + rows_per_iter - 1) / rows_per_iter : 0;
   const int64_t first_row = static_cast<int64_t>(blockIdx.x) * TEAMS + team;
 
   // One row: s holds it on entry and, after its registers are unpacked, is refilled
@@ -598,8 +608,10 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
   // The main loop covers the iterations in which every team has a row; the last,
   // partly filled iteration is masked.
   Slot q;
-  if constexpr (kPrefetch) issue(q, first_row);
-  const int64_t full_iters = rows / rows_per_iter;
+  if constexpr (kPrefetch) {
+    if (row_block) issue(q, first_row);
+  }
+  const int64_t full_iters = row_block ? rows / rows_per_iter : 0;
   int64_t it = 0;
   if (nvec == TPR * V && !(kTail && tail)) {
     for (; it < full_iters; ++it) process(q, it, std::true_type{}, std::true_type{});
@@ -611,12 +623,12 @@ ln_bwd_rows(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ d
 
   if constexpr (COLS) {
     constexpr int64_t kRowsPerPass = 4 * (B::kThreads / 8);
-    for (int64_t slice = blockIdx.x; slice < col_slices; slice += gridDim.x) {
+    for (int64_t slice = first_slice; (col_block || col_blocks == 0) && slice < col_slices; slice += slice_step) {
       float cg[VE], cb[VE];
 #pragma unroll
       for (int e = 0; e < VE; ++e) cg[e] = cb[e] = 0.f;
       for (int64_t row0 = 0; row0 < rows; row0 += kRowsPerPass) {
-        if (slice != blockIdx.x || row0 != 0)
+        if (slice != first_slice || row0 != 0)
           ln_cols_issue<T, B::kThreads>(cols, x, dy, ldx, lddy, map, rows, n, stats, ld_stats, slice, row0);
         ln_cols_accumulate<T, B::kThreads>(cols, rows, n, eps, slice, row0, cg, cb);
       }
@@ -1348,14 +1360,19 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
   if (!p.tpr) return 0;
   if constexpr (VE >= 4 && !UnalignedVec<ST>::value && !StreamedVec<ST>::value) {  // (small calls never stream)
     if (wgrad && ln_bwd_small(rows, n, elem_bytes)) {
-      // tensors that fit the caches: weight gradients from column slices, in the same kernel
+      // tensors that fit the caches: weight gradients from column slices, in the same kernel, by
+      // workgroups of their own beside those that walk the rows (1024 x 128: the kernel takes 3.x us
+      // where one set of workgroups doing both in turn took 5.0)
       const int nvec_s = static_cast<int>(units);
+      const int64_t slices = ceil_div(n, 8 * VE);
+      const int col_blocks = static_cast<int>(slices < 256 ? slices : 256);
 #define X(TPR, TEAMS, V)                                                                              \
   if (p.tpr == TPR && p.teams == TEAMS && p.v == V) {                                                 \
     using B = RowBlock<TPR, TEAMS>;                                                                   \
-    hipLaunchKernelGGL((ln_bwd_rows<ST, TPR, TEAMS, V, false, true>), dim3(static_cast<unsigned>(p.blocks)), \
-                       dim3(B::kThreads), 0, st, x, dy, dx, ldx, lddy, lddx, map, rows, nvec_s,       \
-                       static_cast<int>(n), eps, stats, lds, sgrad, ldsg, gamma, nullptr, dgamma, dbeta); \
+    hipLaunchKernelGGL((ln_bwd_rows<ST, TPR, TEAMS, V, false, true>),                                 \
+                       dim3(static_cast<unsigned>(p.blocks + col_blocks)), dim3(B::kThreads), 0, st, x, dy, dx, ldx, \
+                       lddy, lddx, map, rows, nvec_s, static_cast<int>(n), eps, stats, lds, sgrad, ldsg, gamma,  \
+                       nullptr, dgamma, dbeta, 0, col_blocks);                                        \
     return 1;                                                                                         \
   }
       X(64, 4, 1) X(64, 4, 2) X(64, 4, 4) X(256, 2, 1) X(256, 2, 2) X(256, 1, 1) X(256, 1, 2)
