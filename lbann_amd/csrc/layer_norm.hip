@@ -1378,7 +1378,8 @@ static int ln_bwd_rows_launch(hipStream_t st, bool wgrad, const ST* x, const ST*
     return 1;                                                                                         \
   }
       X(64, 4, 1) X(64, 4, 2) X(64, 4, 4) X(256, 2, 1) X(256, 2, 2) X(256, 1, 1) X(256, 1, 2)
-      if constexpr (VE == 4) { X(256, 2, 4) X(256, 1, 4) }
+      X(512, 1, 1) X(512, 1, 2)
+      if constexpr (VE == 4) { X(256, 2, 4) X(256, 1, 4) X(512, 1, 4) }
 #undef X
     }
   }
