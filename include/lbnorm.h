@@ -251,6 +251,18 @@ int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_
                                      float* stats, int64_t ld_stats,
                                      float* running_mean, float* running_var,
                                      void* workspace, size_t workspace_bytes);
+/* Parity tests only (compare LBN_STATS_REFERENCE_ORDER): the training-mode forward with the CPU
+ * code's own arithmetic (entrywise_batch_normalization.cpp:77-124, :136-163): per entry ONE
+ * sequential fp32 sum of x and of x * x over the columns in order, variance = (sqsum / n -
+ * mean * mean) * n / (n - 1) with no clamp, so that a negative value gives NaN outputs as it does
+ * there.  Results equal the CPU layer's bit for bit.  No workspace; tensors of more than 2^27
+ * entries are refused with LBN_ERR_UNSUPPORTED.  No counterpart of its own in the reference: it
+ * is the reference's arithmetic on the GPU. */
+int lbn_entrywise_batch_norm_fwd_reference_order_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                                     float decay, float epsilon,
+                                                     const float* x, int64_t ldx, float* y, int64_t ldy,
+                                                     float* stats, int64_t ld_stats,
+                                                     float* running_mean, float* running_var);
 int lbn_entrywise_batch_norm_bwd_f32(lbn_stream_t stream, int64_t height, int64_t width,
                                      float epsilon, int training,
                                      const float* x, int64_t ldx, const float* dy, int64_t lddy,

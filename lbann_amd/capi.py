@@ -44,6 +44,7 @@ PROTOTYPES = {
     "lbn_instance_norm_bwd_f32": (cint, [vp, i64, i64, i64, f32, vp, i64, vp, i64, vp, i64, vp, i64, vp, sz]),
     "lbn_entrywise_batch_norm_workspace_bytes": (sz, [i64, i64]),
     "lbn_entrywise_batch_norm_fwd_f32": (cint, [vp, i64, i64, f32, f32, cint, vp, i64, vp, i64, vp, i64, vp, vp, vp, sz]),
+    "lbn_entrywise_batch_norm_fwd_reference_order_f32": (cint, [vp, i64, i64, f32, f32, vp, i64, vp, i64, vp, i64, vp, vp]),
     "lbn_entrywise_batch_norm_bwd_f32": (cint, [vp, i64, i64, f32, cint, vp, i64, vp, i64, vp, i64, vp, i64,
                                                 vp, i64, vp, vp, sz]),
     "lbn_batch_norm_workspace_bytes": (sz, [i64, i64, i64]),

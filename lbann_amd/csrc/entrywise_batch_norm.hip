@@ -26,6 +26,7 @@
 #include "device_utils.hpp"
 #include "entrywise_batch_norm_slabs.hpp"
 #include "host_utils.hpp"
+#include "reference_order.hpp"
 
 namespace lbn {
 
@@ -569,6 +570,22 @@ int lbn_entrywise_batch_norm_fwd_f32(lbn_stream_t stream, int64_t height, int64_
   const dim3 grid(static_cast<unsigned>(ceil_div(height, 256))), block(256);
   if (training) hipLaunchKernelGGL(ebn_fwd_generic, grid, block, 0, st, a);
   else ebn_inference_fwd(st, height, width, epsilon, x, ldx, y, ldy, running_mean, running_var);
+  return launch_status();
+}
+
+int lbn_entrywise_batch_norm_fwd_reference_order_f32(lbn_stream_t stream, int64_t height, int64_t width,
+                                                     float decay, float epsilon, const float* x, int64_t ldx,
+                                                     float* y, int64_t ldy, float* stats, int64_t ld_stats,
+                                                     float* running_mean, float* running_var)
+{
+  const int64_t lds[2] = {ldx, ldy};
+  if (int e = ebn_check(height, width, lds, 2)) return e;
+  if (height == 0 || width == 0) return LBN_OK;
+  if (!x || !y || !running_mean || !running_var || !stats || ld_stats < height) return LBN_ERR_INVALID_ARGUMENT;
+  if (height > kRefOrderMaxEntries / width) return LBN_ERR_UNSUPPORTED;
+  hipStream_t st = as_stream(stream);
+  hipLaunchKernelGGL(ebn_ref_order_fwd, dim3(static_cast<unsigned>(ceil_div(height, 256))), dim3(256), 0, st, height,
+                     width, decay, epsilon, x, ldx, y, ldy, stats, ld_stats, running_mean, running_var);
   return launch_status();
 }
 

@@ -282,4 +282,39 @@ lsm_ref_order_bwd(const float* __restrict__ y, const float* __restrict__ dy, flo
   for (int64_t r = threadIdx.x; r < h; r += kWave) dc[r] = ref_sub(gc[r], ref_mul(expf(yc[r]), s));
 }
 
+// Entry-wise batch norm forward (training) as the CPU code computes it
+// (entrywise_batch_normalization.cpp:77-124, :136-163): per entry one sequential sum of x and of
+// x * x over the columns in order, mean = sum / w, variance = (sqsum / w - mean * mean) * w / (w - 1)
+// WITHOUT a clamp (a negative value then gives NaN outputs, as it does there), running statistics,
+// y = (x - mean) * (1 / sqrt(var + eps)).  One thread per entry: consecutive lanes read consecutive
+// rows of a column.
+static __global__ void __launch_bounds__(256)
+ebn_ref_order_fwd(int64_t h, int64_t w, float decay, float eps, const float* __restrict__ x, int64_t ldx,
+                  float* __restrict__ y, int64_t ldy, float* __restrict__ stats, int64_t ld_stats,
+                  float* __restrict__ rmean, float* __restrict__ rvar)
+{
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (r >= h) return;
+  float sum = 0.f, sqsum = 0.f;
+  for (int64_t c = 0; c < w; ++c) {
+    const float v = x[r + c * ldx];
+    sum = ref_add(sum, v);
+    sqsum = ref_add(sqsum, ref_mul(v, v));
+  }
+  float mean = sum, var = 1.f;
+  if (w > 1) {
+    const float wf = static_cast<float>(w);
+    mean = ref_div(sum, wf);
+    const float sqmean = ref_div(sqsum, wf);
+    var = ref_div(ref_mul(ref_sub(sqmean, ref_mul(mean, mean)), wf), ref_sub(wf, 1.f));
+    const float keep = ref_sub(1.f, decay);
+    rmean[r] = ref_add(ref_mul(decay, rmean[r]), ref_mul(keep, mean));
+    rvar[r] = ref_add(ref_mul(decay, rvar[r]), ref_mul(keep, var));
+  }
+  stats[r] = mean;
+  stats[r + ld_stats] = var;
+  const float inv_stdev = ref_inv_stdev(var, eps);
+  for (int64_t c = 0; c < w; ++c) y[r + c * ldy] = ref_mul(ref_sub(x[r + c * ldx], mean), inv_stdev);
+}
+
 }  // namespace lbn

@@ -1320,3 +1320,44 @@ def test_selftest_copy_pipeline_rejects_what_it_cannot_copy(L):
     assert lib.lbn_selftest_copy_pipeline_f32(st, 2, 12, 3, x.Buffer(), 20, y.Buffer(), 24, 0) == L.capi.LBN_ERR_INVALID_ARGUMENT
     assert lib.lbn_selftest_copy_pipeline_f32(st, 2, 12, 3, None, 24, y.Buffer(), 24, 0) == L.capi.LBN_ERR_INVALID_ARGUMENT
     assert lib.lbn_selftest_copy_pipeline_f32(st, 0, 12, 3, None, 0, None, 0, 1) == L.capi.LBN_OK
+
+
+@pytest.mark.parametrize("h,w,pad", [(105, 29, 0), (4096, 64, 4), (1000, 1, 0), (260, 300, 0), (100000, 33, 0),
+                                     (7, 2, 1)])
+def test_entrywise_batch_norm_reference_order_is_bit_equal(L, h, w, pad):
+    """The test-only forward that adds in the CPU code's order and applies its unclamped variance
+    gives the CPU code's bits: the default kernels differ from it by summation order and the clamp."""
+    rng = np.random.default_rng(11 * h + w)
+    x = rand(rng, h, w, 3.0, 0.5)   # |mean| >> sigma: E[x^2] - mean^2 cancels
+    rm0 = rng.normal(size=h).astype(np.float32)
+    rv0 = rng.uniform(0.5, 2.0, size=h).astype(np.float32)
+    rm, rv = rm0.copy(), rv0.copy()
+    y_ref, st_ref = orc.entrywise_batch_norm_fwd(f32(x), 0.9, 1e-5, rm, rv, True)
+    xd = L.DeviceMatrix.from_numpy(x, ldim=h + pad)
+    yd = L.DeviceMatrix(h, w, ldim=h + pad)
+    st = L.DeviceMatrix(h, 2)
+    rmd, rvd = L._Vector(h, "cuda", rm0), L._Vector(h, "cuda", rv0)
+    L.call("lbn_entrywise_batch_norm_fwd_reference_order_f32", L._stream(), h, w, 0.9, 1e-5, xd.Buffer(), xd.ldim,
+           yd.Buffer(), yd.ldim, st.Buffer(), st.ldim, rmd.Buffer(), rvd.Buffer())
+    _bits_equal("entrywise_bn reference-order stats", st.to_numpy(), st_ref)
+    _bits_equal("entrywise_bn reference-order y", yd.to_numpy(), y_ref)
+    _bits_equal("entrywise_bn reference-order running mean", rmd.to_numpy(), rm)
+    _bits_equal("entrywise_bn reference-order running var", rvd.to_numpy(), rv)
+
+
+def test_entrywise_batch_norm_reference_order_keeps_the_negative_variance(L):
+    """Where the default kernels clamp E[x^2] - mean^2 at zero, the reference-order forward returns what
+    the CPU code returns: the negative variance and NaN outputs for that entry."""
+    x = f32(np.array([[3198.374755859375, 3198.375], [1.0, 3.0], [0.5, -0.5], [2.0, 2.0]], dtype=np.float32))
+    rm, rv = np.zeros(4, np.float32), np.ones(4, np.float32)
+    y_ref, st_ref = orc.entrywise_batch_norm_fwd(f32(x), 0.9, 1e-5, rm, rv, True)
+    assert st_ref[0, 1] < 0 and np.isnan(y_ref[0]).all()
+    xd, yd, st = L.DeviceMatrix.from_numpy(x), L.DeviceMatrix(4, 2), L.DeviceMatrix(4, 2)
+    rmd, rvd = L._Vector(4, "cuda", np.zeros(4)), L._Vector(4, "cuda", np.ones(4))
+    L.call("lbn_entrywise_batch_norm_fwd_reference_order_f32", L._stream(), 4, 2, 0.9, 1e-5, xd.Buffer(), xd.ldim,
+           yd.Buffer(), yd.ldim, st.Buffer(), st.ldim, rmd.Buffer(), rvd.Buffer())
+    _bits_equal("stats", st.to_numpy(), st_ref)
+    y = yd.to_numpy()
+    assert np.isnan(y[0]).all()
+    _bits_equal("y of the other entries", y[1:], y_ref[1:])
+    _bits_equal("running var", rvd.to_numpy(), rv)
