@@ -32,16 +32,10 @@ constexpr int kBnStreamUnroll = 4;
 // registers and four in LDS (its registers allow one workgroup per unit either way).  Measured,
 // forward / backward us before -> after: 16 x 128 x 128 x 64 volumes (w = 4) 112 / 196 -> 103 / 176;
 // 8 x 160^3 (w = 1) 56 / 80 -> 51 / 71; 64 x 112 x 112 (w = 256) 434 / 546 -> 402 / 546.
-#ifndef LBN_BNS_KF
-#define LBN_BNS_KF 2
-#define LBN_BNS_LF 8
-#define LBN_BNS_KB 8
-#define LBN_BNS_LB 4
-#endif
-template <typename S> constexpr int kBnStreamKeepFwd = Vec16<S>::N > 4 ? LBN_BNS_KF / 2 : LBN_BNS_KF;
-template <typename S> constexpr int kBnStreamKeepBwd = Vec16<S>::N > 4 ? LBN_BNS_KB / 2 : LBN_BNS_KB;
-constexpr int kBnStreamLdsFwd = LBN_BNS_LF;
-constexpr int kBnStreamLdsBwd = LBN_BNS_LB;
+template <typename S> constexpr int kBnStreamKeepFwd = Vec16<S>::N > 4 ? 1 : 2;
+template <typename S> constexpr int kBnStreamKeepBwd = Vec16<S>::N > 4 ? 4 : 8;
+constexpr int kBnStreamLdsFwd = 8;
+constexpr int kBnStreamLdsBwd = 4;
 
 template <typename S>
 struct BnStreamArgs {

@@ -540,24 +540,15 @@ constexpr int kLnStreamUnroll = 4;
 // 16: the latter are then read once).  Forward: half of them in registers, half parked in LDS by
 // the thread that fetches them again (no barrier), 64 KiB per workgroup, so that two workgroups
 // share a compute unit (all sixteen in registers took 136 of them: one workgroup per unit).
-#ifndef LBN_LN_STREAM_KEEP_FWD
-#define LBN_LN_STREAM_KEEP_FWD 8
-#endif
-constexpr int kLnStreamKeepFwd = LBN_LN_STREAM_KEEP_FWD;
+constexpr int kLnStreamKeepFwd = 8;
 constexpr int kLnStreamLdsFwd = 16 - kLnStreamKeepFwd;
-#ifndef LBN_LN_STREAM_KEEP_BWD
-#define LBN_LN_STREAM_KEEP_BWD 8
-#endif
-constexpr int kLnStreamKeepBwd = LBN_LN_STREAM_KEEP_BWD;
+constexpr int kLnStreamKeepBwd = 8;
 // Backward: eight vectors per thread and tensor in registers, the next eight parked in LDS by the
 // thread that fetches them again (no barrier), 128 KiB per workgroup; the kernel's registers allow
 // one workgroup per compute unit anyway.  4.1 M-entry rows over 128 workgroups (15.6 vectors per
 // thread and tensor) are then read once: 346 -> 313 us (half as much parked: the same 313 us; two
 // workgroups per unit with eight vectors per tensor kept in all: 339 us).
-#ifndef LBN_LN_STREAM_LDS_BWD
-#define LBN_LN_STREAM_LDS_BWD 8
-#endif
-constexpr int kLnStreamLdsBwd = LBN_LN_STREAM_LDS_BWD;
+constexpr int kLnStreamLdsBwd = 8;
 
 template <int U, typename F>
 __device__ __forceinline__ void ln_stream_walk(unsigned begin, unsigned end, F&& f)
