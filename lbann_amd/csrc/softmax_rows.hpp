@@ -680,6 +680,9 @@ sm_bwd_rows(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t l
 // 54.8).  The same walk in the forward kernel, whose rows need half the registers so that two
 // workgroups share a compute unit anyway, loses (53.0 against 51.2 us per step), and so does the
 // walk over fp16 rows of this length (backward 19.9 against 18.8 us): fp32 rows of 8 vectors only.
+// The fused softmax -> cross-entropy kernels, which hold two tensors each way, lose with it too: the
+// division and the logarithms leave no registers for a second row (forward 47.8 against 35.8 us
+// with 43 registers spilled, backward 38.8 against 37.0 us).
 template <typename S, int V, int KIND, int STREAM>
 __global__ void __launch_bounds__(1024)
 sm_bwd_rows_walk(const S* y, const S* dy, S* dx, int64_t ldy, int64_t lddy, int64_t lddx,
