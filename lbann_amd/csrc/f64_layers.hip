@@ -309,6 +309,110 @@ sm_bwd_rows_f64(RowArgs a)
   }
 }
 
+// Backward for rows of 16384 to 32768 doubles, whose y and dy are more than the registers of a
+// 1024-thread workgroup hold (2 x 64 of 128 per thread): y stays in registers, of dy the first KR
+// accesses per thread do and the other V - KR go from memory straight into LDS
+// (global_load_lds_dwordx4: lane l of a wave fills the 16 bytes at the wave's base + 16 l, no
+// registers in between), where each thread reads the slots that its own wave requested (no
+// barrier).  Every entry is read once.  One workgroup per compute unit walks rows b, b + grid,
+// ...; each access of the next row is requested right behind the store that frees its registers or
+// its slot, so a compute unit's loads overlap its stores.
+template <int KIND, int V, int KR>
+__global__ void __launch_bounds__(1024)
+sm_bwd_rows_parked_f64(RowArgs a)
+{
+  constexpr int TPR = 1024, NW = TPR / kWave, LK = V - KR;
+  typedef double v2d __attribute__((ext_vector_type(2)));
+  __shared__ v2d parked[LK][TPR];
+  __shared__ double red[2][NW];
+  const int t = threadIdx.x;
+  auto live = [&](int i) { return t + i * TPR < a.units; };
+  // Byte offset of access i in a row; accesses past the row's end repeat access 0 (every load is
+  // unconditional, their values are left out of the sum and never stored).  A row's address is the
+  // same for every thread: scalar registers, and one 32-bit offset per access.
+  auto at = [&](const double* p, int i) {
+    unsigned tv = t;
+    asm volatile("" : "+v"(tv));  // formed anew at every use: sixteen offsets kept across the loop cost sixteen registers
+    const unsigned off = tv + i * TPR < unsigned(a.units) ? 16u * (tv + i * TPR) : 16u * tv;
+    return reinterpret_cast<const v2d*>(reinterpret_cast<const char*>(p) + off);
+  };
+  // access KR + j of a row of dy into slot j
+  auto park = [&](const double* p, int j) {
+    unsigned first = t;
+    asm volatile("" : "+v"(first));  // as in at(): nine slot addresses would wait in registers otherwise
+    first &= ~unsigned(kWave - 1);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)at(p, KR + j),
+                                     (__attribute__((address_space(3))) void*)&parked[j][first], 16, 0, 0);
+  };
+  int64_t row = blockIdx.x;
+  if (row >= a.rows) return;
+  v2d y[V], g[KR];
+  {
+    const double* yr = a.a + a.map.offset(row, a.lda);
+    const double* gr = a.g + a.map.offset(row, a.ldg);
+#pragma unroll
+    for (int j = 0; j < LK; ++j) park(gr, j);
+#pragma unroll
+    for (int i = 0; i < V; ++i) y[i] = *at(yr, i);
+#pragma unroll
+    for (int i = 0; i < KR; ++i) g[i] = *at(gr, i);
+  }
+  for (int it = 0; row < a.rows; row += gridDim.x, ++it) {
+    // the slots are written by the memory system: everything this thread requested has arrived
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    double s = 0.0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const v2d gi = i < KR ? g[i < KR ? i : 0] : parked[i < KR ? 0 : i - KR][t];
+      const double part = KIND == kLogSoftmax ? gi.x + gi.y : y[i].x * gi.x + y[i].y * gi.y;
+      s += live(i) ? part : 0.0;
+      if (KIND == kLogSoftmax) {
+        // exp(y) now, while no load is outstanding, and in place: its temporaries do not fit beside
+        // the next row's requests in the loop of stores
+        y[i].x = exp(y[i].x);
+        y[i].y = exp(y[i].y);
+      }
+      if (i >= KR || KIND == kLogSoftmax) __builtin_amdgcn_sched_barrier(0);  // one access at a time: the registers are full
+    }
+    // team_sum_d with the partial sums fetched four at a time (it would hold all 16 at once)
+    s = wave_sum_in_last_d(s);
+    if ((t & (kWave - 1)) == kWave - 1) red[it & 1][t / kWave] = s;
+    __syncthreads();
+    s = 0.0;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      s += red[it & 1][i];
+      if (i % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+    }
+    double* dr = a.out + a.map.offset(row, a.ldo);
+    const int64_t next = row + gridDim.x;
+    const bool more = next < a.rows;
+    const double* yn = a.a + a.map.offset(more ? next : row, a.lda);
+    const double* gn = a.g + a.map.offset(more ? next : row, a.ldg);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const v2d gi = i < KR ? g[i < KR ? i : 0] : parked[i < KR ? 0 : i - KR][t];
+      v2d d;
+      if (KIND == kLogSoftmax) {
+        d.x = gi.x - y[i].x * s;
+        d.y = gi.y - y[i].y * s;
+      }
+      else {
+        d.x = y[i].x * (gi.x - s);
+        d.y = y[i].y * (gi.y - s);
+      }
+      if (live(i)) __builtin_nontemporal_store(d, const_cast<v2d*>(at(dr, i)));
+      asm volatile("" ::: "memory");  // the slot has been read before the next row's request overwrites it
+      if (more) {
+        y[i] = *at(yn, i);
+        if (i < KR) g[i < KR ? i : 0] = *at(gn, i);
+        else park(gn, i - KR);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // one access at a time
+    }
+  }
+}
+
 // ------------------------------------------------------------------ layer norm
 template <int TPR, int V, int W>
 __global__ void __launch_bounds__(Team<TPR>::kThreads)
@@ -977,6 +1081,14 @@ static int sm_bwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
   }
   LBN_F64_SHAPES(X, 1) LBN_F64_SHAPES(X, 2)
 #undef X
+  if (W == 2 && a.units <= 16 * 1024) {
+    // up to 32768 doubles: y in registers, dy in registers and LDS, one workgroup per compute unit
+    int cus = compute_units();
+    if (cus < 1) cus = 256;
+    const int64_t grid = a.rows < cus ? a.rows : cus;
+    hipLaunchKernelGGL((sm_bwd_rows_parked_f64<KIND, 16, 7>), dim3(static_cast<unsigned>(grid)), dim3(1024), 0, st, a);
+    return launch_status();
+  }
   hipLaunchKernelGGL((rows_stream_f64<1, KIND>), dim3(static_cast<unsigned>(a.rows)), dim3(kStreamThreads), 0, st, a);
   return launch_status();
 }

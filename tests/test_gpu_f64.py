@@ -31,7 +31,9 @@ def up(L, a, pad=0):
 # (height, width, padding of the leading dimension)
 SM_CASES = [(1, 5, 0), (2, 3, 0), (7, 9, 0), (64, 33, 0), (100, 17, 2), (1001, 40, 0), (1001, 40, 1), (4096, 64, 0),
             (32768, 40, 0), (30522, 24, 0), (50257, 6, 1), (70000, 5, 0), (262144, 3, 0), (16, 4096, 0),
-            (128, 2048, 0), (10, 20000, 0)]
+            (128, 2048, 0), (10, 20000, 0),
+            # backward with dy partly in LDS (16386 to 32768 entries), more rows than compute units
+            (20000, 300, 2), (32766, 520, 0), (16386, 257, 0)]
 
 
 @pytest.mark.parametrize("kind", ["softmax", "log_softmax"])
