@@ -191,11 +191,23 @@ struct RowArgs {
   const int64_t first = static_cast<int64_t>(blockIdx.x) * TM::kTeams + team;        \
   const int64_t iters = (a.rows + teams_total - 1) / teams_total;                    \
   bool ok[V];                                                                        \
-  int off[V]; /* entry offset of access i; accesses past the row's end re-read access 0 */ \
+  int offs[V]; /* entry offset of access i; accesses past the row's end re-read access 0 */ \
   _Pragma("unroll") for (int i = 0; i < V; ++i) {                                    \
     ok[i] = t + i * TPR < a.units;                                                   \
-    off[i] = ok[i] ? W * (t + i * TPR) : 0;                                          \
+    offs[i] = ok[i] ? W * (t + i * TPR) : 0;                                         \
   }                                                                                  \
+  /* threads with many accesses form the offset anew at every use: held across the row loop the */ \
+  /* offsets take V registers, and a spilled one is reloaded behind every load in flight */ \
+  auto off_at = [&](int i) -> int {                                                  \
+    if constexpr (V >= 8) {                                                          \
+      int tv = t;                                                                    \
+      asm volatile("" : "+v"(tv));                                                   \
+      return tv + i * TPR < a.units ? W * (tv + i * TPR) : 0;                        \
+    }                                                                                \
+    else {                                                                           \
+      return offs[i];                                                                \
+    }                                                                                \
+  };                                                                                 \
   /* row of iteration `it` (clamped to the last row: its loads are harmless, its stores skipped) */ \
   auto row_of = [&](int64_t it) {                                                    \
     const int64_t r = first + it * teams_total;                                      \
@@ -216,7 +228,7 @@ sm_fwd_rows_f64(RowArgs a)
   {
     const double* xr = a.a + a.map.offset(row_of(0), a.lda);
 #pragma unroll
-    for (int i = 0; i < V; ++i) load_w<W>(xr + off[i], v[i]);
+    for (int i = 0; i < V; ++i) load_w<W>(xr + off_at(i), v[i]);
   }
   for (int64_t it = 0; it < iters; ++it) {
     const int64_t row = first + it * teams_total;
@@ -259,8 +271,8 @@ sm_fwd_rows_f64(RowArgs a)
           v[i][j] /= s;  // channelwise_softmax.cpp:88-97: a division, denormals kept
         }
       }
-      if (live && ok[i]) store_w<W>(yr + off[i], v[i]);
-      if (more) load_w<W>(xn + off[i], v[i]);
+      if (live && ok[i]) store_w<W>(yr + off_at(i), v[i]);
+      if (more) load_w<W>(xn + off_at(i), v[i]);
     }
   }
 }
@@ -277,8 +289,8 @@ sm_bwd_rows_f64(RowArgs a)
     const double* gr = a.g + a.map.offset(r, a.ldg);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      load_w<W>(yr + off[i], y[i]);
-      load_w<W>(gr + off[i], g[i]);
+      load_w<W>(yr + off_at(i), y[i]);
+      load_w<W>(gr + off_at(i), g[i]);
     }
   }
   for (int64_t it = 0; it < iters; ++it) {
@@ -300,10 +312,10 @@ sm_bwd_rows_f64(RowArgs a)
 #pragma unroll
       for (int j = 0; j < W; ++j)
         g[i][j] = KIND == kLogSoftmax ? g[i][j] - exp(y[i][j]) * s : y[i][j] * (g[i][j] - s);
-      if (live && ok[i]) store_w<W>(dr + off[i], g[i]);
+      if (live && ok[i]) store_w<W>(dr + off_at(i), g[i]);
       if (more) {
-        load_w<W>(yn + off[i], y[i]);
-        load_w<W>(gn + off[i], g[i]);
+        load_w<W>(yn + off_at(i), y[i]);
+        load_w<W>(gn + off_at(i), g[i]);
       }
     }
   }
@@ -428,15 +440,15 @@ ln_fwd_rows_f64(RowArgs a)
     for (int i = 0; i < V; ++i)
 #pragma unroll
       for (int j = 0; j < W; ++j) {
-        gam[i][j] = (a.gamma && ok[i]) ? a.gamma[off[i] + j] : 1.0;
-        bet[i][j] = (a.beta && ok[i]) ? a.beta[off[i] + j] : 0.0;
+        gam[i][j] = (a.gamma && ok[i]) ? a.gamma[off_at(i) + j] : 1.0;
+        bet[i][j] = (a.beta && ok[i]) ? a.beta[off_at(i) + j] : 0.0;
       }
   }
   double v[V][W];
   {
     const double* xr = a.a + a.map.offset(row_of(0), a.lda);
 #pragma unroll
-    for (int i = 0; i < V; ++i) load_w<W>(xr + off[i], v[i]);
+    for (int i = 0; i < V; ++i) load_w<W>(xr + off_at(i), v[i]);
   }
   for (int64_t it = 0; it < iters; ++it) {
     const int64_t row = first + it * teams_total;
@@ -489,13 +501,13 @@ ln_fwd_rows_f64(RowArgs a)
           y = y * gam[i][j] + bet[i][j];
         }
         else {
-          if (a.gamma) y *= a.gamma[off[i] + j];
-          if (a.beta) y += a.beta[off[i] + j];
+          if (a.gamma) y *= a.gamma[off_at(i) + j];
+          if (a.beta) y += a.beta[off_at(i) + j];
         }
         v[i][j] = y;
       }
-      if (live && ok[i]) store_w<W>(yr + off[i], v[i]);
-      if (more) load_w<W>(xn + off[i], v[i]);
+      if (live && ok[i]) store_w<W>(yr + off_at(i), v[i]);
+      if (more) load_w<W>(xn + off_at(i), v[i]);
     }
   }
 }
@@ -514,7 +526,7 @@ ln_bwd_rows_f64(RowArgs a)
   for (int i = 0; i < V; ++i)
 #pragma unroll
     for (int j = 0; j < W; ++j) {
-      gam[i][j] = (a.gamma && ok[i]) ? a.gamma[off[i] + j] : 1.0;
+      gam[i][j] = (a.gamma && ok[i]) ? a.gamma[off_at(i) + j] : 1.0;
       if (WGRAD) dg[i][j] = db[i][j] = 0.0;
     }
   double d[V][W], gs[V][W];
@@ -526,8 +538,8 @@ ln_bwd_rows_f64(RowArgs a)
     const double* gr = a.g + g * a.map.stride + col * a.ldg;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      load_w<W>(xr + off[i], d[i]);
-      load_w<W>(gr + off[i], gs[i]);
+      load_w<W>(xr + off_at(i), d[i]);
+      load_w<W>(gr + off_at(i), gs[i]);
     }
     mean = a.stats[g + col * a.ld_stats];
     var = a.stats[a.map.groups + g + col * a.ld_stats];
@@ -571,7 +583,7 @@ ln_bwd_rows_f64(RowArgs a)
     for (int i = 0; i < V; ++i) {
 #pragma unroll
       for (int j = 0; j < W; ++j) gs[i][j] = gs[i][j] * inv_stdev + c0 + c1 * d[i][j];
-      if (live && ok[i]) store_w<W>(dr + off[i], gs[i]);
+      if (live && ok[i]) store_w<W>(dr + off_at(i), gs[i]);
     }
     if (it + 1 < iters) issue(it + 1);
   }
@@ -582,8 +594,8 @@ ln_bwd_rows_f64(RowArgs a)
       if (!ok[i]) continue;
 #pragma unroll
       for (int j = 0; j < W; ++j) {
-        out[off[i] + j] = dg[i][j];
-        out[a.n + off[i] + j] = db[i][j];
+        out[off_at(i) + j] = dg[i][j];
+        out[a.n + off_at(i) + j] = db[i][j];
       }
     }
   }
@@ -1045,7 +1057,15 @@ static int sm_fwd(hipStream_t st, int64_t G, int64_t n, int64_t stride, int64_t 
   const RowShape s = pick_shape(a.units, a.rows);
 #define X(TPR, V, WW)                                                                                   \
   if (s.tpr == TPR && s.v == V && W == WW) {                                                            \
-    hipLaunchKernelGGL((sm_fwd_rows_f64<KIND, TPR, V, WW>), dim3(static_cast<unsigned>(row_grid(a.rows, Team<TPR>::kTeams))), \
+    int64_t grid = row_grid(a.rows, Team<TPR>::kTeams);                                                 \
+    if (TPR == 1024 && V >= 16) {                                                                       \
+      /* a row fills a compute unit's registers (one workgroup per unit): one resident wave of */       \
+      /* workgroups, each walking its rows with the next row's loads behind the stores, instead of */   \
+      /* one workgroup after another */                                                                 \
+      const int cap = resident_blocks(sm_fwd_rows_f64<KIND, TPR, V, WW>, Team<TPR>::kThreads);          \
+      if (cap >= 1 && cap <= compute_units() && grid > cap) grid = cap;                                 \
+    }                                                                                                   \
+    hipLaunchKernelGGL((sm_fwd_rows_f64<KIND, TPR, V, WW>), dim3(static_cast<unsigned>(grid)),          \
                        dim3(Team<TPR>::kThreads), 0, st, a);                                            \
     return launch_status();                                                                             \
   }
