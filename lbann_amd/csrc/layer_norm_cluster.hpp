@@ -548,6 +548,11 @@ constexpr int kLnStreamKeepBwd = 8;
 // one workgroup per compute unit anyway.  4.1 M-entry rows over 128 workgroups (15.6 vectors per
 // thread and tensor) are then read once: 346 -> 313 us (half as much parked: the same 313 us; two
 // workgroups per unit with eight vectors per tensor kept in all: 339 us).
+// Requesting the next row's head behind the stores that free its registers and slots (the slots
+// filled from memory directly, global_load_lds_dwordx4) loses in both directions (16 x 160^3 x 2:
+// forward 202 -> 223 us, backward 311 -> 351 us): the rendezvous keeps the workgroups of the device
+// in step, so memory sees a phase of loads and then a phase of stores, and reads mixed into the
+// stores cost more than the overlap returns.
 constexpr int kLnStreamLdsBwd = 8;
 
 template <int U, typename F>

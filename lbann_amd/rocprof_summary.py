@@ -87,6 +87,7 @@ WORKLOADS = [
     ("csb_fwd", None, "extra: channel-wise scale/bias fwd 64x256x56x56", 2 * _E3 * 4),
     ("csb_bwd", None, "extra: channel-wise scale/bias bwd", 3 * _E3 * 4),
     ("f64::sm_fwd_rows_f64<0, 1024, 16", None, "extra: softmax fp64 fwd 32768x512", 2 * _E2 * 8),
+    ("f64::sm_bwd_rows_parked_f64<0", None, "extra: softmax fp64 bwd (y in registers, dy in registers and LDS)", 3 * _E2 * 8),
     ("f64::rows_stream_f64<1, 0>", None, "extra: softmax fp64 bwd (one workgroup per row, two passes)", 3 * _E2 * 8),
     ("f64::ln_fwd_rows_f64", None, "extra: layer norm fp64 fwd 4096x8192", 2 * _E4 * 8),
     ("f64::ln_bwd_rows_f64", None, "extra: layer norm fp64 bwd (followed by ln_wgrad_reduce_f64)", 3 * _E4 * 8),
