@@ -73,9 +73,25 @@ def test_softmax_f64_in_place_and_special_values(L):
     check("f64 softmax special dx", dx, orc.softmax_bwd(y, dy), tol=TOL_F64)
 
 
+def test_softmax_f64_long_rows_in_place(L):
+    """Rows of 24000 doubles, more rows than compute units: the backward kernel that walks rows with
+    dy partly in LDS writes dx over dy."""
+    rng = np.random.default_rng(77)
+    h, w = 24000, 300
+    x, dy = rand(rng, h, w, 0.0, 2.0), rand(rng, h, w)
+    for kind, fwd, bwd in (("softmax", orc.softmax_fwd, orc.softmax_bwd),
+                           ("log_softmax", orc.log_softmax_fwd, orc.log_softmax_bwd)):
+        layer = L.softmax_layer() if kind == "softmax" else L.log_softmax_layer()
+        y = layer.forward(up(L, x)).to_numpy()
+        dx = layer.backward(up(L, dy), in_place=True).to_numpy()
+        check(f"f64 {kind} dx in place {h}x{w}", dx, bwd(y, dy), tol=TOL_F64)
+
+
 @pytest.mark.parametrize("dims,dim,single,w,pad", [((8, 256), 0, False, 24, 0), ((5, 7, 3), 0, False, 9, 0),
                                                   ((64, 4096), 0, False, 4, 0), ((3, 40001), 0, False, 5, 1),
-                                                  ((12, 16, 10), -1, True, 6, 0), ((6, 50), -1, True, 33, 0)])
+                                                  ((12, 16, 10), -1, True, 6, 0), ((6, 50), -1, True, 33, 0),
+                                                  # channels of 16386 to 32768 entries: backward with dy partly in LDS
+                                                  ((3, 20000), 0, False, 100, 0), ((2, 32768), 0, False, 3, 2)])
 def test_channelwise_softmax_f64(L, dims, dim, single, w, pad):
     h = int(np.prod(dims))
     rng = np.random.default_rng(h + w)
