@@ -515,8 +515,10 @@ ln_fwd_rows_f64(RowArgs a)
 // WGRAD: dscale / dbias accumulate in registers across the team's rows (a thread always owns the
 // same entries) and leave one partial row per team.  Measured and rejected for rows of 4096 doubles
 // with weight gradients (8192 rows, 158 us): 512 threads with twice the entries each so that two
-// workgroups share a compute unit (178 us: 18 registers spilled within 128), and a second row
-// requested ahead in 1024 threads (32 spilled).
+// workgroups share a compute unit (178 us: 18 registers spilled within 128), a second row
+// requested ahead in 1024 threads (32 spilled), and 256 threads with eight accesses each, two
+// workgroups per unit (157 us, no spill: the same time, so the kernel's shape is not what
+// limits a call that moves 805 MB).
 template <int TPR, int V, int W, bool WGRAD>
 __global__ void __launch_bounds__(Team<TPR>::kThreads)
 ln_bwd_rows_f64(RowArgs a)
