@@ -827,6 +827,7 @@ struct BnArgs {
   int bessel, training, use_pivot;
   double eps, decay;
   double2* part;  // [C][P]
+  int64_t part_channels;  // C, for the kernels that walk channels
   double* mean;
   double* var;
   const double* gamma;
@@ -1009,6 +1010,129 @@ bn_bwd_apply_f64(BnArgs a)
       for (int j = 0; j < W; ++j) g[u][j] = zero ? 0.0 : g[u][j] * k0 + c0 + c1 * (v[u][j] - mean);
       store_w<W>(dc + col * a.ldo + pos, g[u]);
     });
+}
+
+// Training forward for channels of 128 KB to 400 KB (late convolution stages: many channels of few
+// entries), one 1024-thread workgroup per channel: the channel waits in the workgroup between the
+// statistics and the output (VR accesses of two doubles per thread in registers, LK more in LDS,
+// filled from memory directly), so x crosses HBM once where bn_sums_f64 + bn_fwd_apply_f64 read it
+// twice.  A workgroup walks channels c, c + grid, ...; each access of the next channel is
+// requested behind the store that frees its registers or its slot.  Accesses past the channel's
+// end repeat the thread's first access (every load is unconditional); they are left out of the
+// sums and never stored.
+constexpr int kBnChanRegs = 16;
+constexpr int kBnChanLds = 9;
+constexpr int kBnChanThreads = 1024;
+
+__global__ void __launch_bounds__(kBnChanThreads)
+bn_fwd_channel_f64(BnArgs a)
+{
+  constexpr int TPR = kBnChanThreads, NW = TPR / kWave, VR = kBnChanRegs, LK = kBnChanLds, V = VR + LK;
+  typedef double v2d __attribute__((ext_vector_type(2)));
+  __shared__ v2d parked[LK][TPR];
+  __shared__ double red[2][NW];
+  __shared__ double bc[2];
+  const unsigned t = threadIdx.x;
+  const unsigned seg = static_cast<unsigned>(a.cs / 2);             // accesses per column of the channel
+  const unsigned total = seg * static_cast<unsigned>(a.w);
+  const unsigned step_col = TPR / seg, step_pos = TPR % seg;        // access i + 1 from access i
+  const unsigned col_first = t / seg, pos_first = t - col_first * seg;
+  // f(i, column, position in the column in accesses, inside the channel) for the thread's accesses
+  // in order; the chain of columns and positions is formed anew on every pass (kept across the
+  // passes it would take two registers per access)
+  auto for_each = [&](auto&& f) {
+    unsigned col = col_first, pos = pos_first;
+    asm volatile("" : "+v"(col), "+v"(pos));
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const bool in = t + i * TPR < total;
+      f(i, in ? col : col_first, in ? pos : pos_first, in);
+      col += step_col;
+      pos += step_pos;
+      if (pos >= seg) {
+        pos -= seg;
+        ++col;
+      }
+    }
+  };
+  auto slot = [&](int j) {
+    unsigned first = t;
+    asm volatile("" : "+v"(first));
+    first &= ~unsigned(kWave - 1);
+    return (__attribute__((address_space(3))) void*)&parked[j][first];
+  };
+  v2d xr[VR];
+  auto request = [&](const double* xc) {
+    for_each([&](int i, unsigned col, unsigned pos, bool) {
+      const double* p = xc + col * a.ldx + 2 * pos;
+      if (i < VR) xr[i < VR ? i : 0] = *reinterpret_cast<const v2d*>(p);
+      else __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p, slot(i < VR ? 0 : i - VR), 16, 0, 0);
+    });
+  };
+  int64_t c = blockIdx.x;
+  if (c >= a.part_channels) return;
+  request(a.x + c * a.cs);
+  const double nn = static_cast<double>(a.cs * a.w);
+  for (; c < a.part_channels; c += gridDim.x) {
+    const double* xc = a.x + c * a.cs;
+    double* yc = a.out + c * a.cs;
+    const double K = a.use_pivot ? xc[0] : 0.0;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the slots in LDS are written by the memory system
+    double s = 0.0, q = 0.0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const v2d v = i < VR ? xr[i < VR ? i : 0] : parked[i < VR ? 0 : i - VR][t];
+      const bool in = t + i * TPR < total;
+      const double d0 = v.x - K, d1 = v.y - K;
+      s += in ? d0 + d1 : 0.0;
+      q += in ? d0 * d0 + d1 * d1 : 0.0;
+      if (i >= VR) __builtin_amdgcn_sched_barrier(0);  // one slot at a time: the registers are full
+    }
+    s = wave_sum_in_last_d(s);
+    q = wave_sum_in_last_d(q);
+    if ((t & (kWave - 1)) == kWave - 1) {
+      red[0][t / kWave] = s;
+      red[1][t / kWave] = q;
+    }
+    __syncthreads();
+    if (t == 0) {
+      double ts = 0.0, tq = 0.0;
+      for (int i = 0; i < NW; ++i) {
+        ts += red[0][i];
+        tq += red[1][i];
+      }
+      const double dm = ts / nn;
+      const double mean = K + dm;
+      const double var = fmax(nn * (tq / nn - dm * dm) / (nn - (a.bessel ? 1 : 0)), a.eps);
+      bc[0] = mean;
+      bc[1] = var;
+      a.mean[c] = mean;
+      a.var[c] = var;
+      a.rmean[c] = a.decay * a.rmean[c] + (1.0 - a.decay) * mean;
+      a.rvar[c] = a.decay * a.rvar[c] + (1.0 - a.decay) * var;
+    }
+    __syncthreads();
+    const double mean = bc[0];
+    const double inv_stdev = 1.0 / sqrt(bc[1] + a.eps);
+    const double scale = a.gamma[c], bias = a.beta[c];
+    const int64_t cn = c + gridDim.x;
+    const bool more = cn < a.part_channels;
+    const double* xn = a.x + (more ? cn : c) * a.cs;
+    for_each([&](int i, unsigned col, unsigned pos, bool in) {
+      v2d v = i < VR ? xr[i < VR ? i : 0] : parked[i < VR ? 0 : i - VR][t];
+      v.x = scale * ((v.x - mean) * inv_stdev) + bias;
+      v.y = scale * ((v.y - mean) * inv_stdev) + bias;
+      if (in) __builtin_nontemporal_store(v, reinterpret_cast<v2d*>(yc + col * a.ldo + 2 * pos));
+      asm volatile("" ::: "memory");  // the slot has been read before the next channel's request overwrites it
+      if (more) {
+        const double* p = xn + col * a.ldx + 2 * pos;
+        if (i < VR) xr[i < VR ? i : 0] = *reinterpret_cast<const v2d*>(p);
+        else __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p, slot(i < VR ? 0 : i - VR), 16, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // one access at a time
+    });
+    // bc and red are written again only after the next channel's first barrier
+  }
 }
 
 // ================================================================== host side
@@ -1355,6 +1479,18 @@ int lbn_batch_norm_fwd_f64(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
   if (!workspace || workspace_bytes < lbn_batch_norm_workspace_bytes_f64(C, cs, w) || !aligned16(workspace))
     return LBN_ERR_WORKSPACE;
   a.part = static_cast<double2*>(workspace), a.mean = mean, a.var = var;
+  a.part_channels = C;
+  {
+    // channels that fit a compute unit's registers and LDS, at least one per unit: x is read once
+    const int64_t accesses = cs / 2 * w;
+    const int cus = compute_units();
+    if (vec && cs * w > 1 && accesses >= 8 * f64::kBnChanThreads &&
+        accesses <= (f64::kBnChanRegs + f64::kBnChanLds) * f64::kBnChanThreads && cus > 0 && C >= cus &&
+        !std::getenv("LBN_F64_BN_TWO_PASS")) {
+      hipLaunchKernelGGL(f64::bn_fwd_channel_f64, dim3(static_cast<unsigned>(cus)), dim3(f64::kBnChanThreads), 0, st, a);
+      return launch_status();
+    }
+  }
   if (vec) {
     hipLaunchKernelGGL((bn_sums_f64<2, false>), grid, dim3(f64::kBnThreads), 0, st, a);
     hipLaunchKernelGGL((bn_fwd_apply_f64<2, true>), grid, dim3(f64::kBnThreads), 0, st, a);

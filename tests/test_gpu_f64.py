@@ -141,7 +141,10 @@ def test_layer_norm_f64(L, dims, start_dim, w, affine, pad, mode):
 BN_CASES = [((8, 16, 16), 12, True, 0, True), ((7, 5, 3), 14, False, 0, True), ((5, 24), 10, True, 8, True),
             ((3, 1001), 7, True, 3, True), ((4, 1), 1, True, 0, True), ((6, 1), 33, True, 0, True),
             ((64, 28, 28), 16, True, 0, True), ((3, 56, 56), 16, True, 0, False), ((256, 14, 14), 32, False, 0, True),
-            ((2, 100000), 3, True, 0, True), ((1024, 2, 2), 64, True, 0, True)]
+            ((2, 100000), 3, True, 0, True), ((1024, 2, 2), 64, True, 0, True),
+            # channels of 128 KB to 400 KB, at least one per compute unit: one workgroup keeps a channel
+            ((256, 28, 28), 64, True, 0, True), ((300, 14, 14), 100, False, 2, True), ((257, 10, 10), 201, True, 0, True),
+            ((600, 6, 14), 196, True, 0, True)]
 
 
 @pytest.mark.parametrize("dims,w,bessel,pad,training", BN_CASES)
