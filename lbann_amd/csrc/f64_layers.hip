@@ -1135,6 +1135,151 @@ bn_fwd_channel_f64(BnArgs a)
   }
 }
 
+// Backward for the same channels: dy waits in the workgroup (registers and LDS as x does in
+// bn_fwd_channel_f64) while x streams through the registers twice, five accesses at a time: once
+// for the two sums, once for dx.  Four passes over HBM (x, dy, x, dx) where bn_sums_f64 +
+// bn_bwd_apply_f64 make five.  The next channel's dy is requested behind the stores of dx.
+__global__ void __launch_bounds__(kBnChanThreads)
+bn_bwd_channel_f64(BnArgs a)
+{
+  constexpr int TPR = kBnChanThreads, NW = TPR / kWave, VR = kBnChanRegs, LK = kBnChanLds, V = VR + LK, CH = 5;
+  static_assert(V % CH == 0, "x streams through the registers CH accesses at a time");
+  typedef double v2d __attribute__((ext_vector_type(2)));
+  __shared__ v2d parked[LK][TPR];
+  __shared__ double red[2][NW];
+  __shared__ double bc[2];
+  const unsigned t = threadIdx.x;
+  const unsigned seg = static_cast<unsigned>(a.cs / 2);
+  const unsigned total = seg * static_cast<unsigned>(a.w);
+  const unsigned step_col = TPR / seg, step_pos = TPR % seg;
+  const unsigned col_first = t / seg, pos_first = t - col_first * seg;
+  auto advance = [&](unsigned& col, unsigned& pos) {
+    col += step_col;
+    pos += step_pos;
+    if (pos >= seg) {
+      pos -= seg;
+      ++col;
+    }
+  };
+  auto slot = [&](int j) {
+    unsigned first = t;
+    asm volatile("" : "+v"(first));
+    first &= ~unsigned(kWave - 1);
+    return (__attribute__((address_space(3))) void*)&parked[j][first];
+  };
+  v2d gr[VR];
+  auto request_one = [&](const double* gc, int i, unsigned col, unsigned pos) {
+    const double* p = gc + col * a.lddy + 2 * pos;
+    if (i < VR) gr[i < VR ? i : 0] = *reinterpret_cast<const v2d*>(p);
+    else __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p, slot(i < VR ? 0 : i - VR), 16, 0, 0);
+  };
+  int64_t c = blockIdx.x;
+  if (c >= a.part_channels) return;
+  {
+    unsigned col = col_first, pos = pos_first;
+    asm volatile("" : "+v"(col), "+v"(pos));
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const bool in = t + i * TPR < total;
+      request_one(a.dy + c * a.cs, i, in ? col : col_first, in ? pos : pos_first);
+      advance(col, pos);
+    }
+  }
+  const int64_t n = a.cs * a.w;
+  for (; c < a.part_channels; c += gridDim.x) {
+    const double* xc = a.x + c * a.cs;
+    double* dc = a.out + c * a.cs;
+    const double mean = a.mean[c];
+    const double inv_stdev = 1.0 / sqrt(a.var[c] + a.eps);
+    const double scale = a.gamma[c];
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the slots in LDS are written by the memory system
+    double A = 0.0, B = 0.0;
+    {
+      unsigned col = col_first, pos = pos_first;
+      asm volatile("" : "+v"(col), "+v"(pos));
+#pragma unroll
+      for (int i0 = 0; i0 < V; i0 += CH) {
+        v2d xv[CH];
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+          const bool in = t + (i0 + k) * TPR < total;
+          xv[k] = *reinterpret_cast<const v2d*>(xc + (in ? col : col_first) * a.ldx + 2 * (in ? pos : pos_first));
+          advance(col, pos);
+        }
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+          const int i = i0 + k;
+          const v2d g = i < VR ? gr[i < VR ? i : 0] : parked[i < VR ? 0 : i - VR][t];
+          const bool in = t + i * TPR < total;
+          A += in ? g.x + g.y : 0.0;
+          B += in ? g.x * (xv[k].x - mean) + g.y * (xv[k].y - mean) : 0.0;
+        }
+        __builtin_amdgcn_sched_barrier(0);  // one group of accesses at a time: the registers are full
+      }
+    }
+    A = wave_sum_in_last_d(A);
+    B = wave_sum_in_last_d(B);
+    if ((t & (kWave - 1)) == kWave - 1) {
+      red[0][t / kWave] = A;
+      red[1][t / kWave] = B;
+    }
+    __syncthreads();
+    if (t == 0) {
+      double ta = 0.0, tb = 0.0;
+      for (int i = 0; i < NW; ++i) {
+        ta += red[0][i];
+        tb += red[1][i];
+      }
+      double dmean = -(scale * inv_stdev) * ta;
+      double dvar = -scale * tb * (inv_stdev * inv_stdev * inv_stdev / 2);
+      if (!a.training) dmean = dvar = 0.0;  // statistics are constants outside training
+      a.dscale[c] = tb * inv_stdev;
+      a.dbias[c] = ta;
+      a.dmean[c] = dmean;
+      a.dvar[c] = dvar;
+      bc[0] = dmean / static_cast<double>(n);
+      bc[1] = dvar * 2 / static_cast<double>(n - (a.bessel ? 1 : 0));
+    }
+    __syncthreads();
+    const double k0 = scale * inv_stdev, c0 = bc[0], c1 = bc[1];
+    const int64_t cn = c + gridDim.x;
+    const bool more = cn < a.part_channels;
+    const double* gn = a.dy + (more ? cn : c) * a.cs;
+    {
+      unsigned col = col_first, pos = pos_first;
+      asm volatile("" : "+v"(col), "+v"(pos));
+#pragma unroll
+      for (int i0 = 0; i0 < V; i0 += CH) {
+        v2d xv[CH];
+        unsigned ccol[CH], cpos[CH];
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+          const bool in = t + (i0 + k) * TPR < total;
+          ccol[k] = in ? col : col_first;
+          cpos[k] = in ? pos : pos_first;
+          xv[k] = *reinterpret_cast<const v2d*>(xc + ccol[k] * a.ldx + 2 * cpos[k]);
+          advance(col, pos);
+        }
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+          const int i = i0 + k;
+          const v2d g = i < VR ? gr[i < VR ? i : 0] : parked[i < VR ? 0 : i - VR][t];
+          v2d d;
+          d.x = g.x * k0 + c0 + c1 * (xv[k].x - mean);
+          d.y = g.y * k0 + c0 + c1 * (xv[k].y - mean);
+          if (t + i * TPR < total) __builtin_nontemporal_store(d, reinterpret_cast<v2d*>(dc + ccol[k] * a.ldo + 2 * cpos[k]));
+        }
+        asm volatile("" ::: "memory");  // the slots have been read before the next channel's requests overwrite them
+        if (more) {
+#pragma unroll
+          for (int k = 0; k < CH; ++k) request_one(gn, i0 + k, ccol[k], cpos[k]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+}
+
 // ================================================================== host side
 static bool aligned_rows(const void* p, int64_t stride, int64_t ld, int64_t groups, int64_t w)
 {
@@ -1526,6 +1671,18 @@ int lbn_batch_norm_bwd_f64(lbn_stream_t stream, int64_t C, int64_t cs, int64_t w
   const int P = f64::bn_split(C, cs, w);
   const dim3 grid(static_cast<unsigned>(C), P);
   const bool vec = f64::bn_vec(cs, w, x, ldx) && f64::bn_vec(cs, w, dy, lddy) && f64::bn_vec(cs, w, dx, lddx);
+  a.part_channels = C;
+  {
+    // channels that fit a compute unit's registers and LDS, at least one per unit: dy is read once
+    const int64_t accesses = cs / 2 * w;
+    const int cus = compute_units();
+    if (vec && cs * w > 1 && accesses >= 8 * f64::kBnChanThreads &&
+        accesses <= (f64::kBnChanRegs + f64::kBnChanLds) * f64::kBnChanThreads && cus > 0 && C >= cus &&
+        !std::getenv("LBN_F64_BN_TWO_PASS")) {
+      hipLaunchKernelGGL(f64::bn_bwd_channel_f64, dim3(static_cast<unsigned>(cus)), dim3(f64::kBnChanThreads), 0, st, a);
+      return launch_status();
+    }
+  }
   if (vec) {
     hipLaunchKernelGGL((bn_sums_f64<2, true>), grid, dim3(f64::kBnThreads), 0, st, a);
     hipLaunchKernelGGL((bn_bwd_apply_f64<2>), grid, dim3(f64::kBnThreads), 0, st, a);
