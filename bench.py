@@ -428,6 +428,11 @@ def main():
         # not baseline configurations: fp16 storage for batch norm, and softmax rows off the 16-byte grid
         "extra_batch_norm_f16": ("BatchNorm train fwd+bwd fp16 storage NCHW 64x256x56x56 (informational)",
                                  lambda: build_bn(W.cfg3_batch_norm(), True)),
+        # a late convolution stage: many channels of small maps, one workgroup per channel
+        "extra_batch_norm_14x14": ("BatchNorm train fwd+bwd fp32 NCHW 128x1024x14x14 (informational)",
+                                   lambda: build_bn(W.cfg3_batch_norm(N=128, C=1024, H=14, W=14))),
+        "extra_batch_norm_14x14_f16": ("BatchNorm train fwd+bwd fp16 storage NCHW 128x1024x14x14 (informational)",
+                                       lambda: build_bn(W.cfg3_batch_norm(N=128, C=1024, H=14, W=14), True)),
         "extra_softmax_f16": ("Softmax fwd+bwd fp16 storage 32768x512 (informational)",
                               lambda: build_softmax("softmax", W.cfg2_softmax(), True)),
         "extra_softmax_vocab_50257": ("Softmax fwd+bwd fp32 50257x1024, rows 4-byte aligned (informational)",

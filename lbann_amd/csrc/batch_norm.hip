@@ -681,6 +681,110 @@ bn_bwd_cluster(BnBwdArgs<S> a, unsigned seg, unsigned E)
   }
 }
 
+// ---------------------------------------------- a channel in one workgroup's registers
+// Channels of up to 8192 vectors (late convolution stages: 14 x 14 or 28 x 28 maps), at least
+// as many of them as fill the device: one short-lived workgroup per channel keeps the channel in
+// registers between the sums and the output.  Nothing is exchanged between workgroups, so there
+// is no rendezvous, no workspace and no tag; workgroups of different channels on a compute unit
+// are in different phases, which is what overlaps loads, sums and stores.  Every thread forms the
+// statistics from the workgroup's sums itself (one barrier per channel).
+template <typename S, int T, int V>
+__global__ void __launch_bounds__(T)
+bn_fwd_channel(BnFwdArgs<S> a, unsigned seg, unsigned E)
+{
+  __shared__ float red[2 * (T / kWave)];
+  const unsigned tid = threadIdx.x;
+  // neighbouring channels, whose segments share cache lines, on one die
+  const int ch = static_cast<int>(item_of_block_by_die(blockIdx.x, gridDim.x));
+  const BnIndex<V> ix = bn_make_index<T, V>(0, seg, E);
+  BnFwdTile<S, V> t;
+  bn_fwd_load<S, V>(t, a, ch, ix);
+  const float K = t.K;
+  float s = 0.f, q = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    float v[Vec16<S>::N];
+    Vec16<S>::unpack(t.v[i], v);
+#pragma unroll
+    for (int j = 0; j < Vec16<S>::N; ++j) {
+      const float d = ix.ok[i] ? v[j] - K : 0.f;
+      s += d;
+      q += d * d;
+    }
+  }
+  team_sum2<T / kWave>(s, q, red, tid / kWave, tid & (kWave - 1));
+  float mean, var;
+  stats_from_sums(s, q, K, a.n, a.bessel, a.eps, mean, var);
+  if (tid == 0) {
+    a.mean_out[ch] = mean;
+    a.var_out[ch] = var;
+    a.rmean[ch] = a.decay * a.rmean[ch] + (1.f - a.decay) * mean;
+    a.rvar[ch] = a.decay * a.rvar[ch] + (1.f - a.decay) * var;
+  }
+  const float inv_stdev = 1.0f / sqrtf(var + a.eps);
+  S* yc = a.y + static_cast<int64_t>(ch) * a.cs;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    if (!ix.ok[i]) continue;
+    float v[Vec16<S>::N];
+    Vec16<S>::unpack(t.v[i], v);
+#pragma unroll
+    for (int j = 0; j < Vec16<S>::N; ++j) v[j] = t.scale * ((v[j] - mean) * inv_stdev) + t.bias;
+    Vec16<S>::store(bn_tile_address<S, V>(yc, a.ldy, ix, i), v);
+  }
+}
+
+template <typename S, int T, int V>
+__global__ void __launch_bounds__(T)
+bn_bwd_channel(BnBwdArgs<S> a, unsigned seg, unsigned E)
+{
+  __shared__ float red[2 * (T / kWave)];
+  const unsigned tid = threadIdx.x;
+  // neighbouring channels, whose segments share cache lines, on one die
+  const int ch = static_cast<int>(item_of_block_by_die(blockIdx.x, gridDim.x));
+  const BnIndex<V> ix = bn_make_index<T, V>(0, seg, E);
+  BnBwdTile<S, V> t;
+  bn_bwd_load<S, V>(t, a, ch, ix);
+  const float mean = t.mean;
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {  // vectors past the end hold zeros in dy
+    float x[Vec16<S>::N], g[Vec16<S>::N];
+    Vec16<S>::unpack(t.x[i], x);
+    Vec16<S>::unpack(t.g[i], g);
+#pragma unroll
+    for (int j = 0; j < Vec16<S>::N; ++j) {
+      sa += g[j];
+      sb += g[j] * (x[j] - mean);
+    }
+  }
+  team_sum2<T / kWave>(sa, sb, red, tid / kWave, tid & (kWave - 1));
+  const float inv_stdev = 1.0f / sqrtf(t.var + a.eps);
+  const float scale = t.scale;
+  float ds, db, dmean, dvar;
+  grads_from_sums(sa, sb, scale, inv_stdev, ds, db, dmean, dvar);
+  if (tid == 0) {
+    a.dscale[ch] = ds;
+    a.dbias[ch] = db;
+    a.dmean_out[ch] = dmean;
+    a.dvar_out[ch] = dvar;
+  }
+  const float dmean_term = dmean / static_cast<float>(a.n);
+  const float dvar_term = dvar * 2.f / static_cast<float>(a.n - (a.bessel ? 1 : 0));
+  const float k0 = scale * inv_stdev;
+  S* dxc = a.dx + static_cast<int64_t>(ch) * a.cs;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    if (!ix.ok[i]) continue;
+    float x[Vec16<S>::N], g[Vec16<S>::N];
+    Vec16<S>::unpack(t.x[i], x);
+    Vec16<S>::unpack(t.g[i], g);
+#pragma unroll
+    for (int j = 0; j < Vec16<S>::N; ++j) g[j] = g[j] * k0 + dmean_term + dvar_term * (x[j] - mean);
+    Vec16<S>::store(bn_tile_address<S, V>(dxc, a.lddx, ix, i), g);
+  }
+}
+
 // ------------------------------------------------ the same rotation without barriers
 // Variant of the cluster kernels above in which the waves of a workgroup never meet at a
 // barrier after the start-up (WaveMerge in cluster_sync.hpp): a wave adds its share, leaves
@@ -937,6 +1041,24 @@ static BnClusterShape bn_cluster_shape(int64_t E, int max_v, int first_t)
   return {0, 0, 0};
 }
 
+// Workgroup size and vectors per thread for a channel of E vectors held by one workgroup: the
+// smallest workgroup whose threads hold at most eight vectors (of each tensor); T = 0 when the
+// channel is too large or too small, or when C channels of that size leave compute units idle.
+static BnClusterShape bn_channel_shape(int64_t E, int64_t C, int64_t max_e = 8192)
+{
+  static const bool disabled = std::getenv("LBN_BN_NO_CHANNEL") != nullptr;
+  if (disabled || E < 512 || E > max_e) return {0, 0, 0};
+  const int T = E <= 2048 ? 256 : E <= 4096 ? 512 : 1024;
+  const int64_t per = ceil_div(E, T);
+  const int V = per <= 2 ? 2 : per <= 4 ? 4 : 8;
+  int cus = compute_units();
+  if (cus < 1) cus = 256;
+  // measured against the clusters on 14 x 14 to 32 x 32 maps: ahead by 5 to 40 % from 128 channels
+  // on (256 of them when 256 threads hold a channel), level or behind with 64
+  if (C * T < static_cast<int64_t>(cus) * 256 || 2 * C < cus) return {0, 0, 0};
+  return {T, V, 1};
+}
+
 // 16-bit storage runs the barrier-free variant of the cluster kernels, fp32 the one with
 // barriers; LBN_BN_WAVE_SYNC=0|1 in the environment forces one of them for every type.
 template <typename S>
@@ -1025,6 +1147,21 @@ static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
                                float* rmean, float* rvar, void* ws)
 {
   constexpr int VE = Vec16<S>::N;
+  if (cs * w > 1 && C <= (1 << 24)) {
+    const BnClusterShape q = bn_channel_shape(cs / VE * w, C);
+    if (q.T) {  // a channel per workgroup: no cluster, no workspace
+      const BnFwdArgs<S> a{x, y, ldx, ldy, cs, static_cast<int>(C), 1, pivot, bessel, eps, decay, cs * w,
+                           ClusterWorkspace{}, ClusterTag{}, mean, var, scale, bias, rmean, rvar};
+      const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(cs / VE * w);
+#define X(TT, VV)                                                                                        \
+  if (q.T == TT && q.V == VV) {                                                                          \
+    hipLaunchKernelGGL((bn_fwd_channel<S, TT, VV>), dim3(static_cast<unsigned>(C)), dim3(TT), 0, st, a, seg, Eu); \
+    return true;                                                                                         \
+  }
+      X(256, 2) X(256, 4) X(256, 8) X(512, 8) X(1024, 8)
+#undef X
+    }
+  }
   if (!bn_cluster_usable<S>(C, cs, w, ws)) return false;
   const int64_t E = cs / VE * w;
   const BnClusterShape p = bn_cluster_shape(E, 4, 256);
@@ -1049,6 +1186,24 @@ static bool bn_try_bwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
                                float* dbias, float* dmean, float* dvar, void* ws)
 {
   constexpr int VE = Vec16<S>::N;
+  if (cs * w > 1 && C <= (1 << 24)) {
+    // (two tensors of eight halves per vector, widened to fp32 where they are used: 1024 threads
+    // with eight vectors of each would spill)
+    const BnClusterShape q = bn_channel_shape(cs / VE * w, C, VE == 8 ? 4096 : 8192);
+    if (q.T) {
+      const BnBwdArgs<S> a{x, dy, dx, ldx, lddy, lddx, cs, static_cast<int>(C), 1, bessel, eps, cs * w,
+                           ClusterWorkspace{}, ClusterTag{}, mean, var, scale, dscale, dbias, dmean, dvar};
+      const unsigned seg = static_cast<unsigned>(cs / VE), Eu = static_cast<unsigned>(cs / VE * w);
+#define X(TT, VV)                                                                                        \
+  if (q.T == TT && q.V == VV) {                                                                          \
+    hipLaunchKernelGGL((bn_bwd_channel<S, TT, VV>), dim3(static_cast<unsigned>(C)), dim3(TT), 0, st, a, seg, Eu); \
+    return true;                                                                                         \
+  }
+      X(256, 2) X(256, 4) X(256, 8) X(512, 8)
+      if constexpr (VE < 8) { X(1024, 8) }
+#undef X
+    }
+  }
   if (!bn_cluster_usable<S>(C, cs, w, ws)) return false;
   const int64_t E = cs / VE * w;
   constexpr bool kShortVectors = sizeof(typename Vec16<S>::raw_t) == 8;

@@ -588,6 +588,19 @@ __device__ __forceinline__ float team_max(float v, float* slot, int wave_in_team
   return r;
 }
 
+// Workgroups are handed to the eight accelerator dies (each with an L2 of its own) in turn: block b
+// runs on die b % 8.  Where neighbouring work items share cache lines (channels whose segments
+// are not whole lines), this gives die x the items [start(x), start(x + 1)) in the order in which
+// its blocks start, so that neighbours meet in one L2 instead of being fetched into two.  A
+// bijection of [0, blocks) for any number of blocks.
+constexpr unsigned kDies = 8;
+__device__ __forceinline__ unsigned item_of_block_by_die(unsigned b, unsigned blocks)
+{
+  const unsigned die = b % kDies, turn = b / kDies;
+  const unsigned q = blocks / kDies, r = blocks % kDies;
+  return die * q + (die < r ? die : r) + turn;
+}
+
 template <int NW>
 __device__ __forceinline__ void team_sum2(float& a, float& b, float* slot, int wave_in_team,
                                           int lane)

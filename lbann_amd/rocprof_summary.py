@@ -92,6 +92,10 @@ WORKLOADS = [
     ("f64::ln_fwd_rows_f64", None, "extra: layer norm fp64 fwd 4096x8192", 2 * _E4 * 8),
     ("f64::ln_bwd_rows_f64", None, "extra: layer norm fp64 bwd (followed by ln_wgrad_reduce_f64)", 3 * _E4 * 8),
     ("f64::bn_fwd_channel_f64", None, "extra: batch norm fp64 64x256x28x28 fwd (one workgroup keeps a channel: x read once)", 2 * 12845056 * 8),
+    ("bn_fwd_channel<float, 1024, 8>", None, "extra: batch norm 128x1024x14x14 fwd (one workgroup per channel)", 2 * 25690112 * 4),
+    ("bn_bwd_channel<float, 1024, 8>", None, "extra: batch norm 128x1024x14x14 bwd (one workgroup per channel)", 3 * 25690112 * 4),
+    ("bn_fwd_channel<lbn::f16x4, 1024, 8>", None, "extra: batch norm fp16 storage 128x1024x14x14 fwd (one workgroup per channel)", 2 * 25690112 * 2),
+    ("bn_bwd_channel<lbn::f16x4, 1024, 8>", None, "extra: batch norm fp16 storage 128x1024x14x14 bwd (one workgroup per channel)", 3 * 25690112 * 2),
     ("f64::bn_bwd_channel_f64", None, "extra: batch norm fp64 bwd (one workgroup keeps a channel's dy: x read twice, dy once)", 3 * 12845056 * 8),
     ("f64::bn_sums_f64<2, false>", None, "extra: batch norm fp64 64x256x28x28 fwd, kernel 1 of 2 (reads x)", 12845056 * 8),
     ("f64::bn_fwd_apply_f64", None, "extra: batch norm fp64 fwd, kernel 2 of 2 (reads x, writes y)", 2 * 12845056 * 8),

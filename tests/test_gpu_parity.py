@@ -841,6 +841,9 @@ BN_CASES = [
     ((256, 4, 4), 200, True, 0), ((100, 12), 64, True, 0),
     # more channels than resident clusters: some clusters take two or three channels in turn, others one
     ((478, 16), 577, True, 0), ((1500, 4, 4), 600, False, 0), ((900, 64), 300, True, 0),
+    # many channels of 512 to 8192 vectors: one workgroup keeps a channel (256, 512 and 1024 threads)
+    ((1024, 14, 14), 32, True, 0), ((600, 8, 8), 100, False, 4), ((300, 28, 28), 40, True, 0), ((2048, 4, 4), 130, True, 0),
+    ((1100, 8), 300, False, 0), ((520, 14, 14), 72, True, 0),
     # channels of up to a million entries: clusters of more than 64 workgroups (two slots per polling lane)
     ((3, 56, 56), 256, True, 0), ((2, 802816), 1, True, 0), ((2, 1000000), 1, False, 0), ((1, 1100000), 1, True, 0),
     # beyond that: clusters that stream their share twice (backward from 1 M entries, forward from 2 M)
@@ -903,6 +906,9 @@ def test_batch_norm(L, dims, w, bessel, pad):
     ((12, 3, 3), 20, True, 0, True), ((1024, 1), 2048, True, 0, True), ((128, 7, 7), 10, True, 0, False),
     ((32, 7, 7), 64, True, 4, True), ((2000, 2), 200, False, 0, True), ((100, 12), 64, True, 0, True),
     ((8, 55, 55), 300, True, 0, True), ((4, 111, 111), 20, False, 0, True),
+    # many channels of 512 to 8192 vectors: one workgroup keeps a channel (backward up to 4096 vectors of eight)
+    ((512, 16, 16), 100, True, 0, True), ((300, 28, 28), 64, False, 0, True), ((1024, 14, 14), 128, True, 0, True),
+    ((1100, 8), 600, True, 0, True),
     ((3, 56, 56), 512, True, 0, True), ((2, 2000000), 1, True, 0, True),   # clusters of more than 64 workgroups
     ((3, 112, 112), 512, True, 0, True), ((2, 2500000), 2, False, 0, True)])   # streaming clusters
 def test_batch_norm_f16(L, dims, w, bessel, pad, training):
