@@ -1059,6 +1059,22 @@ static BnClusterShape bn_channel_shape(int64_t E, int64_t C, int64_t max_e = 819
   return {T, V, 1};
 }
 
+// The same for fp32 channels that are not a whole number of 16-byte vectors (7 x 7 maps), held as
+// single floats, up to sixteen per thread: consecutive lanes take consecutive floats, so a wave
+// instruction reads 256 contiguous bytes wherever it does not cross from one sample to the next.
+static BnClusterShape bn_scalar_channel_shape(int64_t E, int64_t C)
+{
+  static const bool disabled = std::getenv("LBN_BN_NO_CHANNEL") != nullptr;
+  if (disabled || E < 1024 || E > 16384) return {0, 0, 0};
+  const int T = E <= 4096 ? 256 : E <= 8192 ? 512 : 1024;
+  const int64_t per = ceil_div(E, T);
+  const int V = per <= 4 ? 4 : per <= 8 ? 8 : 16;
+  int cus = compute_units();
+  if (cus < 1) cus = 256;
+  if (C * T < static_cast<int64_t>(cus) * 256 || 2 * C < cus) return {0, 0, 0};
+  return {T, V, 1};
+}
+
 // 16-bit storage runs the barrier-free variant of the cluster kernels, fp32 the one with
 // barriers; LBN_BN_WAVE_SYNC=0|1 in the environment forces one of them for every type.
 template <typename S>
@@ -1415,6 +1431,24 @@ static int bn_fwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
       return launch_status();
     }
   }
+  if constexpr (std::is_same<S, float>::value) {
+    if (!vec && cs * w > 1 && C <= (1 << 24)) {
+      const BnClusterShape q = bn_scalar_channel_shape(cs * w, C);
+      if (q.T) {  // a channel of single floats per workgroup
+        const BnFwdArgs<f32x1> a{reinterpret_cast<const f32x1*>(x), reinterpret_cast<f32x1*>(y), ldx, ldy, cs,
+                                 static_cast<int>(C), 1, pivot, bessel, epsilon, decay, cs * w, ClusterWorkspace{},
+                                 ClusterTag{}, mean, var, scale, bias, running_mean, running_var};
+        const unsigned seg = static_cast<unsigned>(cs), Eu = static_cast<unsigned>(cs * w);
+#define X(TT, VV)                                                                                        \
+  if (q.T == TT && q.V == VV) {                                                                          \
+    hipLaunchKernelGGL((bn_fwd_channel<f32x1, TT, VV>), dim3(static_cast<unsigned>(C)), dim3(TT), 0, st, a, seg, Eu); \
+    return launch_status();                                                                              \
+  }
+        X(256, 4) X(256, 8) X(256, 16) X(512, 16) X(1024, 16)
+#undef X
+      }
+    }
+  }
   if constexpr (Vec16<S>::N == 4) {  // float or fp16 in fours: the row-tile kernels
     // channels of three or four vectors: the register tile when the mini-batch fits it
     // (1024 x 16, w = 256: 19 us per step against 25 us for clusters), else clusters
@@ -1516,6 +1550,25 @@ static int bn_bwd_host(hipStream_t st, int64_t C, int64_t cs, int64_t w, int bes
                            cs, w, n, bessel, epsilon, training, part, use_mean, use_var, scale, dscale, dbias, dmean,
                            dvar);
       return launch_status();
+    }
+  }
+  if constexpr (std::is_same<S, float>::value) {
+    if (!vec && training && n > 1 && C <= (1 << 24)) {
+      const BnClusterShape q = bn_scalar_channel_shape(n, C);
+      if (q.T) {
+        const BnBwdArgs<f32x1> a{reinterpret_cast<const f32x1*>(x), reinterpret_cast<const f32x1*>(dy),
+                                 reinterpret_cast<f32x1*>(dx), ldx, lddy, lddx, cs, static_cast<int>(C), 1, bessel,
+                                 epsilon, n, ClusterWorkspace{}, ClusterTag{}, use_mean, use_var, scale, dscale, dbias,
+                                 dmean, dvar};
+        const unsigned seg = static_cast<unsigned>(cs), Eu = static_cast<unsigned>(n);
+#define X(TT, VV)                                                                                        \
+  if (q.T == TT && q.V == VV) {                                                                          \
+    hipLaunchKernelGGL((bn_bwd_channel<f32x1, TT, VV>), dim3(static_cast<unsigned>(C)), dim3(TT), 0, st, a, seg, Eu); \
+    return launch_status();                                                                              \
+  }
+        X(256, 4) X(256, 8) X(256, 16) X(512, 16) X(1024, 16)
+#undef X
+      }
     }
   }
   if constexpr (Vec16<S>::N == 4) {  // float or fp16 in fours: the row-tile kernels

@@ -844,6 +844,9 @@ BN_CASES = [
     # many channels of 512 to 8192 vectors: one workgroup keeps a channel (256, 512 and 1024 threads)
     ((1024, 14, 14), 32, True, 0), ((600, 8, 8), 100, False, 4), ((300, 28, 28), 40, True, 0), ((2048, 4, 4), 130, True, 0),
     ((1100, 8), 300, False, 0), ((520, 14, 14), 72, True, 0),
+    # the same for channels that are not whole 16-byte vectors (7 x 7 maps): single floats, up to 16 per thread
+    ((2048, 7, 7), 128, True, 0), ((512, 7, 7), 256, False, 0), ((300, 5, 5), 100, True, 0), ((256, 3, 3), 200, True, 3),
+    ((1024, 1), 1100, True, 1), ((130, 7, 7), 300, True, 0),
     # channels of up to a million entries: clusters of more than 64 workgroups (two slots per polling lane)
     ((3, 56, 56), 256, True, 0), ((2, 802816), 1, True, 0), ((2, 1000000), 1, False, 0), ((1, 1100000), 1, True, 0),
     # beyond that: clusters that stream their share twice (backward from 1 M entries, forward from 2 M)
