@@ -196,6 +196,42 @@ struct Vec16<f16x2> {
   }
 };
 
+// fp16 storage accessed one value at a time: channels of odd sizes (7 x 7 maps) held by one
+// workgroup.  Consecutive lanes take consecutive halves.  Sized like one half.
+struct f16x1 {
+  unsigned short bits;
+};
+
+template <>
+struct Vec16<f16x1> {
+  static constexpr int N = 1;
+  using raw_t = unsigned short;
+  static __device__ __forceinline__ raw_t load_raw(const f16x1* p) { return p->bits; }
+  static __device__ __forceinline__ void unpack(const raw_t& r, float (&v)[1])
+  {
+    __half h;
+    __builtin_memcpy(&h, &r, 2);
+    v[0] = __half2float(h);
+  }
+  static __device__ __forceinline__ void load(const f16x1* p, float (&v)[1]) { unpack(load_raw(p), v); }
+  static __device__ __forceinline__ void store(f16x1* p, const float (&v)[1])
+  {
+    const __half h = __float2half_rn(v[0]);
+    __builtin_memcpy(&p->bits, &h, 2);
+  }
+  static __device__ __forceinline__ float load1(const f16x1* p)
+  {
+    float v[1];
+    load(p, v);
+    return v[0];
+  }
+  static __device__ __forceinline__ void store1(f16x1* p, float v)
+  {
+    const float a[1] = {v};
+    store(p, a);
+  }
+};
+
 // fp16 storage accessed four values (8 bytes) at a time: for channels and rows whose length
 // is a multiple of 4 but not of 8 (14 x 14 feature maps: 196 entries).  Sized like one half,
 // so pointer offsets count halves.

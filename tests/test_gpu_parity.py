@@ -912,6 +912,9 @@ def test_batch_norm(L, dims, w, bessel, pad):
     # many channels of 512 to 8192 vectors: one workgroup keeps a channel (backward up to 4096 vectors of eight)
     ((512, 16, 16), 100, True, 0, True), ((300, 28, 28), 64, False, 0, True), ((1024, 14, 14), 128, True, 0, True),
     ((1100, 8), 600, True, 0, True),
+    # odd maps, many channels: single halves in one workgroup's registers
+    ((512, 7, 7), 100, True, 0, True), ((1024, 7, 7), 32, False, 0, True), ((300, 5, 5), 100, True, 0, True),
+    ((256, 3, 3), 200, True, 1, True), ((130, 7, 7), 300, True, 0, True),
     ((3, 56, 56), 512, True, 0, True), ((2, 2000000), 1, True, 0, True),   # clusters of more than 64 workgroups
     ((3, 112, 112), 512, True, 0, True), ((2, 2500000), 2, False, 0, True)])   # streaming clusters
 def test_batch_norm_f16(L, dims, w, bessel, pad, training):
