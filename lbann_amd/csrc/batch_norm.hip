@@ -1170,7 +1170,11 @@ static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   if (cs * w > 1 && C <= (1 << 24)) {
     // (vectors of eight halves, widened to fp32 where they are used: up to 4096 of them, which 512
     // threads hold; 64x512x28x28 in 1024 threads measured 3 % behind the clusters)
-    const BnClusterShape q = bn_channel_shape(cs / VE * w, C, VE == 8 ? 4096 : 8192);
+    BnClusterShape q = bn_channel_shape(cs / VE * w, C, VE == 8 ? 4096 : 8192);
+    // forward, 4097 to 8192 vectors of 8 bytes: 512 threads with sixteen each, so that two workgroups
+    // share a compute unit (128x1024x14x14 fp16: 55.0 -> 52.3 us per step; 16-byte vectors of fp32
+    // then need 130 registers and lose, 93.0 -> 97.1 us)
+    if (q.T == 1024 && sizeof(typename Vec16<S>::raw_t) == 8) q = BnClusterShape{512, 16, 1};
     if (q.T) {  // a channel per workgroup: no cluster, no workspace
       const BnFwdArgs<S> a{x, y, ldx, ldy, cs, static_cast<int>(C), 1, pivot, bessel, eps, decay, cs * w,
                            ClusterWorkspace{}, ClusterTag{}, mean, var, scale, bias, rmean, rvar};
@@ -1182,6 +1186,7 @@ static bool bn_try_fwd_cluster(hipStream_t st, int64_t C, int64_t cs, int64_t w,
   }
       X(256, 2) X(256, 4) X(256, 8) X(512, 8)
       if constexpr (VE < 8) { X(1024, 8) }
+      if constexpr (sizeof(typename Vec16<S>::raw_t) == 8) { X(512, 16) }
 #undef X
     }
   }

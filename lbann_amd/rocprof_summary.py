@@ -94,6 +94,7 @@ WORKLOADS = [
     ("f64::bn_fwd_channel_f64", None, "extra: batch norm fp64 64x256x28x28 fwd (one workgroup keeps a channel: x read once)", 2 * 12845056 * 8),
     ("bn_fwd_channel<float, 1024, 8>", None, "extra: batch norm 128x1024x14x14 fwd (one workgroup per channel)", 2 * 25690112 * 4),
     ("bn_bwd_channel<float, 1024, 8>", None, "extra: batch norm 128x1024x14x14 bwd (one workgroup per channel)", 3 * 25690112 * 4),
+    ("bn_fwd_channel<lbn::f16x4, 512, 16>", None, "extra: batch norm fp16 storage 128x1024x14x14 fwd (one workgroup per channel)", 2 * 25690112 * 2),
     ("bn_fwd_channel<lbn::f16x4, 1024, 8>", None, "extra: batch norm fp16 storage 128x1024x14x14 fwd (one workgroup per channel)", 2 * 25690112 * 2),
     ("bn_bwd_channel<lbn::f16x4, 1024, 8>", None, "extra: batch norm fp16 storage 128x1024x14x14 bwd (one workgroup per channel)", 3 * 25690112 * 2),
     ("f64::bn_bwd_channel_f64", None, "extra: batch norm fp64 bwd (one workgroup keeps a channel's dy: x read twice, dy once)", 3 * 12845056 * 8),
