@@ -369,12 +369,12 @@ struct BnIndex {
 };
 
 template <int T, int V>
-__device__ __forceinline__ BnIndex<V> bn_make_index(int k, unsigned seg, unsigned E)
+__device__ __forceinline__ BnIndex<V> bn_make_index(int k, unsigned seg, unsigned E, unsigned tid = threadIdx.x)
 {
   BnIndex<V> ix;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    const unsigned e = static_cast<unsigned>(k) * (T * V) + i * T + threadIdx.x;
+    const unsigned e = static_cast<unsigned>(k) * (T * V) + i * T + tid;
     ix.ok[i] = e < E;
     ix.col[i] = e / seg;
     ix.pos[i] = e - ix.col[i] * seg;
@@ -696,18 +696,26 @@ bn_fwd_channel(BnFwdArgs<S> a, unsigned seg, unsigned E)
   const unsigned tid = threadIdx.x;
   // neighbouring channels, whose segments share cache lines, on one die
   const int ch = static_cast<int>(item_of_block_by_die(blockIdx.x, gridDim.x));
-  const BnIndex<V> ix = bn_make_index<T, V>(0, seg, E);
+  // The columns and positions of a thread's vectors are formed once for the loads and once more
+  // for the stores (kLeanIndex: from a copy of the thread index that the compiler cannot see
+  // through): kept across the sums they take two registers per vector, which is what stands
+  // between sixteen waves with eight 16-byte vectors each and two workgroups per compute unit.
+  constexpr bool kLeanIndex = T == 1024 && V >= 8;
   BnFwdTile<S, V> t;
-  bn_fwd_load<S, V>(t, a, ch, ix);
+  {
+    const BnIndex<V> ix = bn_make_index<T, V>(0, seg, E);
+    bn_fwd_load<S, V>(t, a, ch, ix);
+  }
   const float K = t.K;
   float s = 0.f, q = 0.f;
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     float v[Vec16<S>::N];
     Vec16<S>::unpack(t.v[i], v);
+    const bool in = i * T + tid < E;
 #pragma unroll
     for (int j = 0; j < Vec16<S>::N; ++j) {
-      const float d = ix.ok[i] ? v[j] - K : 0.f;
+      const float d = in ? v[j] - K : 0.f;
       s += d;
       q += d * d;
     }
@@ -723,6 +731,9 @@ bn_fwd_channel(BnFwdArgs<S> a, unsigned seg, unsigned E)
   }
   const float inv_stdev = 1.0f / sqrtf(var + a.eps);
   S* yc = a.y + static_cast<int64_t>(ch) * a.cs;
+  unsigned tid2 = tid;
+  if (kLeanIndex) asm volatile("" : "+v"(tid2));
+  const BnIndex<V> ix = bn_make_index<T, V>(0, seg, E, tid2);
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     if (!ix.ok[i]) continue;
