@@ -514,7 +514,7 @@ def test_layer_norm_reference_formula_mode(L, dims, start_dim, w):
 @pytest.mark.parametrize("dims,start_dim,w,pad", [((4096,), 0, 64, 0), ((512,), 0, 100, 0), ((64,), 0, 9, 0),
                                                    ((8, 1024), -1, 5, 0), ((100,), 0, 7, 0), ((2048,), 0, 600, 8),
                                                    ((16384,), 0, 3, 0), ((16384,), 0, 40, 0), ((8192,), 0, 300, 0),
-                                                   ((768,), 0, 1000, 0), ((12288,), 0, 9, 0),
+                                                   ((768,), 0, 1000, 0), ((12288,), 0, 9, 0), ((12288,), 0, 600, 0), ((10248,), 0, 520, 8),
                                                    ((32768,), 0, 20, 0), ((150528,), 0, 3, 0), ((20000,), 0, 5, 8),
                                                    ((1024, 256), -1, 8, 0), ((512, 64), -1, 16, 0), ((128, 512), -1, 40, 0),
                                                    # even lengths that are not a multiple of 8: one pair per access
