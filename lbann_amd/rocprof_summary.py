@@ -35,6 +35,11 @@ WORKLOADS = [
     ("sm_bwd_rows<float, 1024, 8, 0", None, "cfg2 softmax bwd, one row per workgroup (LBN_NO_BWD_WALK)", 3 * _E2 * 4),
     ("sm_fwd_rows<float, 1024, 8, 1", None, "cfg2 log-softmax fwd", 2 * _E2 * 4),
     ("sm_bwd_rows_walk<float, 8, 1", None, "cfg2 log-softmax bwd", 3 * _E2 * 4),
+    # clusters on the 14 x 14 shape (LBN_BN_NO_CHANNEL): 256-thread workgroups, cfg3 takes 512
+    ("bn_fwd_cluster<float, 256, 4>", None, "extra: batch norm 128x1024x14x14 fwd, clusters share a channel (LBN_BN_NO_CHANNEL)", 2 * 25690112 * 4),
+    ("bn_bwd_cluster<float, 256, 2>", None, "extra: batch norm 128x1024x14x14 bwd, clusters share a channel (LBN_BN_NO_CHANNEL)", 3 * 25690112 * 4),
+    ("bn_fwd_cluster_ws<lbn::f16x4, 256, 4>", None, "extra: batch norm fp16 storage 128x1024x14x14 fwd, clusters share a channel (LBN_BN_NO_CHANNEL)", 2 * 25690112 * 2),
+    ("bn_bwd_cluster_ws<lbn::f16x4, 256, 4>", None, "extra: batch norm fp16 storage 128x1024x14x14 bwd, clusters share a channel (LBN_BN_NO_CHANNEL)", 3 * 25690112 * 2),
     ("bn_fwd_cluster<float", None, "cfg3 batch norm fwd 64x256x56x56", 2 * _E3 * 4),
     ("bn_bwd_cluster<float", None, "cfg3 batch norm bwd", 3 * _E3 * 4),
     ("bn_fwd_cluster_ws<__half", None, "extra: batch norm fp16 storage fwd 64x256x56x56", 2 * _E3 * 2),
