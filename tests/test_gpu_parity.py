@@ -886,6 +886,23 @@ def _bn_run(L, x, dy, dims, bessel, pad, scale, bias, mode=None, training=True, 
     return {k: check(f"batch_norm {k} dims={dims} w={w} half={half}", out[k], ref[k], ex[k], tol=tol) for k in out}
 
 
+@pytest.mark.parametrize("w", [127, 128, 512, 513, 1024, 1025, 2048, 2049])
+@pytest.mark.parametrize("half", [False, True])
+def test_batch_norm_channel_per_workgroup_boundaries(L, w, half):
+    """256 channels of 4 x 4 (fp16: 8 x 4) entries: the mini-batch sizes either side of every switch
+    between 256, 512 and 1024 threads per channel, and between one workgroup per channel and the
+    paths around it (fewer than 512 vectors, more than 8192; fp16 backward more than 4096)."""
+    dims = (256, 8, 4) if half else (256, 4, 4)
+    rng = np.random.default_rng(900 + w)
+    h = int(np.prod(dims))
+    x, dy = rand(rng, h, w, 2.0, 3.0), rand(rng, h, w)
+    if half:
+        x, dy = x.astype(np.float16).astype(np.float32), dy.astype(np.float16).astype(np.float32)
+    scale = rng.uniform(0.5, 1.5, dims[0]).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(dims[0])).astype(np.float32)
+    _bn_run(L, x, dy, dims, bool(w % 2), 0, scale, bias, half=half)
+
+
 @pytest.mark.parametrize("dims,w,bessel,pad", BN_CASES)
 def test_batch_norm(L, dims, w, bessel, pad):
     rng = np.random.default_rng(int(np.prod(dims)) + w)
